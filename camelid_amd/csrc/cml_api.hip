@@ -1,0 +1,515 @@
+// C ABI of libcamelid_hip (declared in include/camelid_hip.h): lifecycle,
+// device-resident weights, and dispatch to the per-format kernels.
+//
+// The conventions follow the reference's device seam (src/cuda.rs:167-236 for
+// gating, :691-699 for the process-global backend, :1044-1218 for the
+// "handled / not handled" contract): nothing here throws or aborts; every
+// failure becomes a status code plus a thread-local message.
+#include <stdarg.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <atomic>
+#include <mutex>
+#include <unordered_map>
+
+#include "cml_host.hpp"
+
+namespace cml {
+
+static thread_local char g_error[512] = "";
+static std::atomic<int> g_device{-1};
+static std::atomic<uint64_t> g_runs{0};
+static std::mutex g_mutex;
+
+int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+void clear_error() { g_error[0] = '\0'; }
+
+bool ready() { return g_device.load(std::memory_order_acquire) >= 0; }
+
+int env_int(const char *name, int dflt) {
+    const char *v = getenv(name);
+    if (!v || !*v) return dflt;
+    return atoi(v);
+}
+
+// Environment masking is checked before any driver call (reference
+// devices_masked_by_env, src/cuda.rs:206-218).
+static bool masked_by_env() {
+    const char *off = getenv("CAMELID_HIP");
+    if (off && (!strcmp(off, "0") || !strcasecmp(off, "off") || !strcasecmp(off, "false"))) return true;
+    const char *names[] = {"HIP_VISIBLE_DEVICES", "ROCR_VISIBLE_DEVICES"};
+    for (const char *n : names) {
+        const char *v = getenv(n);
+        if (v && (!*v || !strcmp(v, "-1"))) return true;
+    }
+    return false;
+}
+
+static int check_ready() {
+    if (!ready()) return fail(CML_ERR_UNAVAILABLE, "cml_init has not succeeded");
+    return CML_OK;
+}
+
+}  // namespace cml
+
+using namespace cml;
+
+extern "C" {
+
+int cml_block_values(int fmt) { return geometry(fmt).block_values; }
+int cml_block_bytes(int fmt) { return geometry(fmt).block_bytes; }
+
+int cml_available(void) {
+    if (masked_by_env()) return 0;
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess || n <= 0) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    for (int i = 0; i < n; i++) {
+        hipDeviceProp_t prop;
+        if (hipGetDeviceProperties(&prop, i) == hipSuccess && strncmp(prop.gcnArchName, "gfx950", 6) == 0) return 1;
+    }
+    return 0;
+}
+
+int cml_init(int device) {
+    clear_error();
+    if (masked_by_env()) return fail(CML_ERR_UNAVAILABLE, "GPU use is masked by the environment");
+    std::lock_guard<std::mutex> lock(g_mutex);
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess || n <= 0) {
+        (void)hipGetLastError();
+        return fail(CML_ERR_UNAVAILABLE, "no HIP device");
+    }
+    if (device < 0) device = env_int("CAMELID_HIP_DEVICE", 0);
+    if (device >= n) return fail(CML_ERR_INVALID, "device %d out of range (%d present)", device, n);
+    hipDeviceProp_t prop;
+    CML_HIP_TRY(hipGetDeviceProperties(&prop, device));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(CML_ERR_UNAVAILABLE, "device %d is %s; this library carries gfx950 code only", device, prop.gcnArchName);
+    CML_HIP_TRY(hipSetDevice(device));
+    g_device.store(device, std::memory_order_release);
+    return CML_OK;
+}
+
+void cml_shutdown(void) {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    g_device.store(-1, std::memory_order_release);
+}
+
+const char *cml_last_error(void) { return g_error; }
+uint64_t cml_run_count(void) { return g_runs.load(std::memory_order_relaxed); }
+
+// ---- device memory plumbing ------------------------------------------------------------------------
+
+int cml_dev_alloc(size_t nbytes, void **out_dev) {
+    if (!out_dev) return fail(CML_ERR_INVALID, "null out pointer");
+    *out_dev = nullptr;
+    if (int rc = check_ready()) return rc;
+    if (nbytes == 0) nbytes = 16;
+    CML_HIP_TRY(hipMalloc(out_dev, nbytes));
+    return CML_OK;
+}
+
+int cml_dev_free(void *ptr_dev) {
+    if (!ptr_dev) return CML_OK;
+    if (int rc = check_ready()) return rc;
+    CML_HIP_TRY(hipFree(ptr_dev));
+    return CML_OK;
+}
+
+int cml_memcpy_h2d(void *dst_dev, const void *src_host, size_t nbytes, cml_stream_t stream) {
+    if (int rc = check_ready()) return rc;
+    if (nbytes == 0) return CML_OK;
+    if (!dst_dev || !src_host) return fail(CML_ERR_INVALID, "null pointer");
+    CML_HIP_TRY(hipMemcpyAsync(dst_dev, src_host, nbytes, hipMemcpyHostToDevice, as_stream(stream)));
+    CML_HIP_TRY(hipStreamSynchronize(as_stream(stream)));
+    return CML_OK;
+}
+
+int cml_memcpy_d2h(void *dst_host, const void *src_dev, size_t nbytes, cml_stream_t stream) {
+    if (int rc = check_ready()) return rc;
+    if (nbytes == 0) return CML_OK;
+    if (!dst_host || !src_dev) return fail(CML_ERR_INVALID, "null pointer");
+    CML_HIP_TRY(hipMemcpyAsync(dst_host, src_dev, nbytes, hipMemcpyDeviceToHost, as_stream(stream)));
+    CML_HIP_TRY(hipStreamSynchronize(as_stream(stream)));
+    return CML_OK;
+}
+
+int cml_memset_dev(void *dst_dev, int value, size_t nbytes, cml_stream_t stream) {
+    if (int rc = check_ready()) return rc;
+    if (nbytes == 0) return CML_OK;
+    if (!dst_dev) return fail(CML_ERR_INVALID, "null pointer");
+    CML_HIP_TRY(hipMemsetAsync(dst_dev, value, nbytes, as_stream(stream)));
+    return CML_OK;
+}
+
+int cml_stream_sync(cml_stream_t stream) {
+    if (int rc = check_ready()) return rc;
+    CML_HIP_TRY(hipStreamSynchronize(as_stream(stream)));
+    return CML_OK;
+}
+
+// ---- weights ---------------------------------------------------------------------------------------
+
+static int check_weight_shape(int fmt, int64_t rows, int64_t cols, size_t nbytes, int64_t *nb_out) {
+    const Geometry g = geometry(fmt);
+    if (g.block_values == 0) return fail(CML_ERR_INVALID, "unknown weight format %d", fmt);
+    if (rows < 0 || cols <= 0) return fail(CML_ERR_SHAPE, "bad shape %lld x %lld", (long long)rows, (long long)cols);
+    if (cols % g.block_values != 0)
+        return fail(CML_ERR_SHAPE, "cols %lld is not a multiple of the %d-value block", (long long)cols, g.block_values);
+    if (rows > INT32_MAX / 2 || cols > (int64_t)1 << 24) return fail(CML_ERR_SHAPE, "shape too large");
+    const int64_t nb = cols / g.block_values;
+    const size_t want = static_cast<size_t>(rows) * static_cast<size_t>(nb) * g.block_bytes;
+    if (nbytes != want)
+        return fail(CML_ERR_SHAPE, "%zu wire bytes given, %zu expected for %lld x %lld", nbytes, want, (long long)rows, (long long)cols);
+    *nb_out = nb;
+    return CML_OK;
+}
+
+static int make_weight(int fmt, int64_t rows, int64_t cols, int64_t nb, cml_weight **out) {
+    cml_weight *w = new (std::nothrow) cml_weight();
+    if (!w) return fail(CML_ERR_OOM, "host allocation failed");
+    w->fmt = fmt;
+    w->rows = rows;
+    w->cols = cols;
+    w->nb = nb;
+    size_t offset[4], total = 0;
+    int64_t stride[4];
+    plane_layout(fmt, rows, nb, stride, offset, &total);
+    void *base = nullptr;
+    hipError_t e = hipMalloc(&base, total ? total : 256);
+    if (e != hipSuccess) {
+        delete w;
+        return fail(e == hipErrorOutOfMemory ? CML_ERR_OOM : CML_ERR_HIP, "hipMalloc(%zu) failed: %s", total, hipGetErrorString(e));
+    }
+    w->allocation = base;
+    w->allocation_bytes = total;
+    for (int i = 0; i < 4; i++) {
+        w->planes.p[i] = static_cast<uint8_t *>(base) + offset[i];
+        w->planes.row_stride[i] = stride[i];
+    }
+    *out = w;
+    return CML_OK;
+}
+
+int cml_weight_upload_dev(int fmt, int64_t rows, int64_t cols, const void *wire_dev, size_t nbytes,
+                          cml_stream_t stream, cml_weight **out) {
+    if (!out) return fail(CML_ERR_INVALID, "null out pointer");
+    *out = nullptr;
+    if (int rc = check_ready()) return rc;
+    int64_t nb = 0;
+    if (int rc = check_weight_shape(fmt, rows, cols, nbytes, &nb)) return rc;
+    if (!wire_dev && nbytes) return fail(CML_ERR_INVALID, "null wire pointer");
+    cml_weight *w = nullptr;
+    if (int rc = make_weight(fmt, rows, cols, nb, &w)) return rc;
+    int rc = launch_wire_to_planes(fmt, static_cast<const uint8_t *>(wire_dev), rows, nb, w->planes, as_stream(stream));
+    if (rc != CML_OK) {
+        cml_weight_free(w);
+        return rc;
+    }
+    *out = w;
+    return CML_OK;
+}
+
+int cml_weight_upload(int fmt, int64_t rows, int64_t cols, const void *wire_host, size_t nbytes, cml_weight **out) {
+    if (!out) return fail(CML_ERR_INVALID, "null out pointer");
+    *out = nullptr;
+    if (int rc = check_ready()) return rc;
+    int64_t nb = 0;
+    if (int rc = check_weight_shape(fmt, rows, cols, nbytes, &nb)) return rc;
+    if (!wire_host && nbytes) return fail(CML_ERR_INVALID, "null wire pointer");
+    if (fmt == CML_Q4_K) {  // device layout == wire layout: copy straight in
+        cml_weight *w = nullptr;
+        if (int rc = make_weight(fmt, rows, cols, nb, &w)) return rc;
+        if (nbytes) {
+            hipError_t e = hipMemcpy(const_cast<uint8_t *>(w->planes.p[0]), wire_host, nbytes, hipMemcpyHostToDevice);
+            if (e != hipSuccess) {
+                cml_weight_free(w);
+                return fail(CML_ERR_HIP, "hipMemcpy failed: %s", hipGetErrorString(e));
+            }
+        }
+        *out = w;
+        return CML_OK;
+    }
+    void *staging = nullptr;
+    CML_HIP_TRY(hipMalloc(&staging, nbytes ? nbytes : 16));
+    hipError_t e = nbytes ? hipMemcpy(staging, wire_host, nbytes, hipMemcpyHostToDevice) : hipSuccess;
+    int rc = CML_OK;
+    if (e != hipSuccess) rc = fail(CML_ERR_HIP, "hipMemcpy failed: %s", hipGetErrorString(e));
+    if (rc == CML_OK) rc = cml_weight_upload_dev(fmt, rows, cols, staging, nbytes, nullptr, out);
+    if (rc == CML_OK) {
+        e = hipStreamSynchronize(nullptr);
+        if (e != hipSuccess) rc = fail(CML_ERR_HIP, "re-layout failed: %s", hipGetErrorString(e));
+    }
+    (void)hipFree(staging);
+    if (rc != CML_OK && *out) {
+        cml_weight_free(*out);
+        *out = nullptr;
+    }
+    return rc;
+}
+
+int cml_weight_slice(const cml_weight *parent, int64_t row_start, int64_t rows, cml_weight **out) {
+    if (!out) return fail(CML_ERR_INVALID, "null out pointer");
+    *out = nullptr;
+    if (!parent) return fail(CML_ERR_INVALID, "null weight");
+    if (row_start < 0 || rows < 0 || row_start + rows > parent->rows)
+        return fail(CML_ERR_SHAPE, "rows [%lld, %lld) outside 0..%lld", (long long)row_start, (long long)(row_start + rows), (long long)parent->rows);
+    cml_weight *w = new (std::nothrow) cml_weight(*parent);
+    if (!w) return fail(CML_ERR_OOM, "host allocation failed");
+    w->allocation = nullptr;
+    w->allocation_bytes = 0;
+    w->rows = rows;
+    for (int i = 0; i < 4; i++)
+        if (w->planes.p[i]) w->planes.p[i] += row_start * w->planes.row_stride[i];
+    *out = w;
+    return CML_OK;
+}
+
+int cml_weight_info(const cml_weight *w, int *fmt, int64_t *rows, int64_t *cols, size_t *wire_bytes) {
+    if (!w) return fail(CML_ERR_INVALID, "null weight");
+    if (fmt) *fmt = w->fmt;
+    if (rows) *rows = w->rows;
+    if (cols) *cols = w->cols;
+    if (wire_bytes) *wire_bytes = static_cast<size_t>(w->rows) * w->nb * geometry(w->fmt).block_bytes;
+    return CML_OK;
+}
+
+int cml_weight_download(const cml_weight *w, void *wire_host, size_t nbytes) {
+    if (!w) return fail(CML_ERR_INVALID, "null weight");
+    if (int rc = check_ready()) return rc;
+    const size_t want = static_cast<size_t>(w->rows) * w->nb * geometry(w->fmt).block_bytes;
+    if (nbytes != want) return fail(CML_ERR_SHAPE, "%zu bytes given, %zu expected", nbytes, want);
+    if (want == 0) return CML_OK;
+    if (!wire_host) return fail(CML_ERR_INVALID, "null pointer");
+    void *staging = nullptr;
+    CML_HIP_TRY(hipMalloc(&staging, want));
+    int rc = launch_planes_to_wire(w->fmt, w->planes, w->rows, w->nb, static_cast<uint8_t *>(staging), nullptr);
+    if (rc == CML_OK) {
+        hipError_t e = hipMemcpy(wire_host, staging, want, hipMemcpyDeviceToHost);
+        if (e != hipSuccess) rc = fail(CML_ERR_HIP, "hipMemcpy failed: %s", hipGetErrorString(e));
+    }
+    (void)hipFree(staging);
+    return rc;
+}
+
+void cml_weight_free(cml_weight *w) {
+    if (!w) return;
+    if (w->allocation) (void)hipFree(w->allocation);
+    delete w;
+}
+
+static bool misaligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) != 0; }
+
+// ---- activation quantizers ------------------------------------------------------------------------
+
+int cml_quantize_q8_0(const float *x_dev, int64_t n_tokens, int64_t cols, int8_t *q_dev, float *scales_dev,
+                      cml_stream_t stream) {
+    if (int rc = check_ready()) return rc;
+    if (n_tokens < 0 || cols < 0 || cols % 32 != 0) return fail(CML_ERR_SHAPE, "cols %lld is not a multiple of 32", (long long)cols);
+    if (n_tokens == 0 || cols == 0) return CML_OK;
+    if (!x_dev || !q_dev || !scales_dev) return fail(CML_ERR_INVALID, "null pointer");
+    if (misaligned16(x_dev) || (reinterpret_cast<uintptr_t>(q_dev) & 3u)) return fail(CML_ERR_INVALID, "x must be 16-byte and q 4-byte aligned");
+    return launch_quantize_q8_0(x_dev, n_tokens, cols, q_dev, scales_dev, as_stream(stream));
+}
+
+int cml_quantize_q8_k(const float *x_dev, int64_t n_tokens, int64_t cols, int8_t *q_dev, float *d_dev,
+                      cml_stream_t stream) {
+    if (int rc = check_ready()) return rc;
+    if (n_tokens < 0 || cols < 0 || cols % 256 != 0) return fail(CML_ERR_SHAPE, "cols %lld is not a multiple of 256", (long long)cols);
+    if (n_tokens == 0 || cols == 0) return CML_OK;
+    if (!x_dev || !q_dev || !d_dev) return fail(CML_ERR_INVALID, "null pointer");
+    if (misaligned16(x_dev) || (reinterpret_cast<uintptr_t>(q_dev) & 3u)) return fail(CML_ERR_INVALID, "x must be 16-byte and q 4-byte aligned");
+    return launch_quantize_q8_k(x_dev, n_tokens, cols, q_dev, d_dev, as_stream(stream));
+}
+
+int cml_dequantize(const cml_weight *w, float *out_dev, cml_stream_t stream) {
+    if (!w) return fail(CML_ERR_INVALID, "null weight");
+    if (int rc = check_ready()) return rc;
+    if (w->rows == 0) return CML_OK;
+    if (!out_dev) return fail(CML_ERR_INVALID, "null pointer");
+    return launch_dequantize(w, out_dev, as_stream(stream));
+}
+
+// ---- matvec / matmul --------------------------------------------------------------------------------
+
+static int dispatch(const MatArgs &a, hipStream_t st) {
+    int rc;
+    switch (a.w->fmt) {
+        case CML_Q4_K: rc = launch_gemv_q4k(a, st); break;
+        case CML_Q8_0: rc = launch_gemv_q8_0(a, st); break;
+        case CML_Q4_0: rc = launch_gemv_q4_0(a, st); break;
+        case CML_Q6_K: rc = launch_gemv_q6k(a, st); break;
+        default: return fail(CML_ERR_INVALID, "unknown weight format %d", a.w->fmt);
+    }
+    if (rc == CML_OK) g_runs.fetch_add(1, std::memory_order_relaxed);
+    return rc;
+}
+
+static MatArgs plain_args(const cml_weight *w, const int8_t *q, const float *s, int64_t n_tokens, float *out) {
+    MatArgs a;
+    a.w = w;
+    a.q = q;
+    a.scales = s;
+    a.n_tokens = n_tokens;
+    a.out = out;
+    a.residual = nullptr;
+    a.ints = nullptr;
+    a.band_ids = nullptr;
+    a.n_bands = 1;
+    a.band_rows = 0;
+    a.act_per_slot = false;
+    return a;
+}
+
+int cml_gemv(const cml_weight *w, const int8_t *q_dev, const float *scales_dev, float *out_dev,
+             const float *residual_dev, cml_stream_t stream) {
+    if (!w) return fail(CML_ERR_INVALID, "null weight");
+    if (int rc = check_ready()) return rc;
+    if (w->rows == 0) return CML_OK;
+    if (!q_dev || !scales_dev || !out_dev) return fail(CML_ERR_INVALID, "null pointer");
+    if (misaligned16(q_dev)) return fail(CML_ERR_INVALID, "activation quants must be 16-byte aligned");
+    MatArgs a = plain_args(w, q_dev, scales_dev, 1, out_dev);
+    a.residual = residual_dev;
+    return dispatch(a, as_stream(stream));
+}
+
+int cml_gemm(const cml_weight *w, const int8_t *q_dev, const float *scales_dev, int64_t n_tokens, float *out_dev,
+             cml_stream_t stream) {
+    if (!w) return fail(CML_ERR_INVALID, "null weight");
+    if (int rc = check_ready()) return rc;
+    if (n_tokens < 0) return fail(CML_ERR_SHAPE, "negative token count");
+    if (w->rows == 0 || n_tokens == 0) return CML_OK;
+    if (!q_dev || !scales_dev || !out_dev) return fail(CML_ERR_INVALID, "null pointer");
+    if (misaligned16(q_dev)) return fail(CML_ERR_INVALID, "activation quants must be 16-byte aligned");
+    return dispatch(plain_args(w, q_dev, scales_dev, n_tokens, out_dev), as_stream(stream));
+}
+
+int cml_block_dots(const cml_weight *w, const int8_t *q_dev, int32_t *ints_dev, cml_stream_t stream) {
+    if (!w) return fail(CML_ERR_INVALID, "null weight");
+    if (int rc = check_ready()) return rc;
+    if (w->rows == 0) return CML_OK;
+    if (!q_dev || !ints_dev) return fail(CML_ERR_INVALID, "null pointer");
+    if (misaligned16(q_dev)) return fail(CML_ERR_INVALID, "activation quants must be 16-byte aligned");
+    // The integers do not depend on the activation scales; run the real gemv
+    // kernel with zero scales into a scratch output and keep its integers.
+    float *scratch = nullptr;
+    const size_t n_scales = static_cast<size_t>(w->nb);
+    CML_HIP_TRY(hipMalloc(reinterpret_cast<void **>(&scratch), (n_scales + static_cast<size_t>(w->rows)) * sizeof(float)));
+    hipStream_t st = as_stream(stream);
+    int rc = CML_OK;
+    hipError_t e = hipMemsetAsync(scratch, 0, n_scales * sizeof(float), st);
+    if (e != hipSuccess) rc = fail(CML_ERR_HIP, "hipMemsetAsync failed: %s", hipGetErrorString(e));
+    if (rc == CML_OK) {
+        MatArgs a = plain_args(w, q_dev, scratch, 1, scratch + n_scales);
+        a.ints = ints_dev;
+        rc = dispatch(a, st);
+    }
+    if (rc == CML_OK) {
+        e = hipStreamSynchronize(st);
+        if (e != hipSuccess) rc = fail(CML_ERR_HIP, "block-dot kernel failed: %s", hipGetErrorString(e));
+    }
+    (void)hipFree(scratch);
+    return rc;
+}
+
+size_t cml_matmul_workspace_bytes(int fmt, int64_t cols, int64_t n_tokens) {
+    const Geometry g = geometry(fmt);
+    if (g.block_values == 0 || cols <= 0 || n_tokens <= 0) return 0;
+    const int64_t per = is_k_family(fmt) ? 256 : 32;
+    const size_t q = (static_cast<size_t>(n_tokens) * cols + 255) & ~size_t(255);
+    const size_t s = (static_cast<size_t>(n_tokens) * (cols / per) * 4 + 255) & ~size_t(255);
+    return q + s;
+}
+
+int cml_matmul_f32(const cml_weight *w, const float *x_dev, int64_t n_tokens, float *out_dev, void *workspace_dev,
+                   size_t workspace_bytes, cml_stream_t stream) {
+    if (!w) return fail(CML_ERR_INVALID, "null weight");
+    if (int rc = check_ready()) return rc;
+    if (n_tokens < 0) return fail(CML_ERR_SHAPE, "negative token count");
+    if (w->rows == 0 || n_tokens == 0) return CML_OK;
+    if (!x_dev || !out_dev || !workspace_dev) return fail(CML_ERR_INVALID, "null pointer");
+    if (misaligned16(x_dev) || misaligned16(workspace_dev)) return fail(CML_ERR_INVALID, "activations and workspace must be 16-byte aligned");
+    const size_t need = cml_matmul_workspace_bytes(w->fmt, w->cols, n_tokens);
+    if (workspace_bytes < need) return fail(CML_ERR_SHAPE, "workspace of %zu bytes given, %zu needed", workspace_bytes, need);
+    int8_t *q = static_cast<int8_t *>(workspace_dev);
+    float *s = reinterpret_cast<float *>(static_cast<uint8_t *>(workspace_dev) +
+                                         ((static_cast<size_t>(n_tokens) * w->cols + 255) & ~size_t(255)));
+    hipStream_t st = as_stream(stream);
+    int rc = is_k_family(w->fmt) ? launch_quantize_q8_k(x_dev, n_tokens, w->cols, q, s, st)
+                                 : launch_quantize_q8_0(x_dev, n_tokens, w->cols, q, s, st);
+    if (rc != CML_OK) return rc;
+    return dispatch(plain_args(w, q, s, n_tokens, out_dev), st);
+}
+
+// ---- host-slice seam ----------------------------------------------------------------------------------
+
+namespace {
+struct CacheKey {
+    const void *ptr;
+    size_t len;
+    int fmt;
+    bool operator==(const CacheKey &o) const { return ptr == o.ptr && len == o.len && fmt == o.fmt; }
+};
+struct CacheHash {
+    size_t operator()(const CacheKey &k) const {
+        return std::hash<const void *>()(k.ptr) ^ (std::hash<size_t>()(k.len) * 1315423911u) ^ static_cast<size_t>(k.fmt);
+    }
+};
+std::unordered_map<CacheKey, cml_weight *, CacheHash> g_weight_cache;
+}  // namespace
+
+int cml_try_linear_rows(int fmt, const float *input_scales, const int8_t *input_quants, const uint8_t *weight_wire,
+                        size_t weight_nbytes, int64_t input_rows, int64_t weight_rows, int64_t cols, float *output) {
+    if (!ready()) {
+        if (cml_init(-1) != CML_OK) return CML_ERR_UNAVAILABLE;
+    }
+    if (!input_scales || !input_quants || !weight_wire || !output) return fail(CML_ERR_INVALID, "null pointer");
+    if (input_rows <= 0 || weight_rows <= 0) return fail(CML_ERR_SHAPE, "empty shape");
+    const Geometry g = geometry(fmt);
+    if (g.block_values == 0) return fail(CML_ERR_INVALID, "unknown weight format %d", fmt);
+    std::lock_guard<std::mutex> lock(g_mutex);
+    cml_weight *w = nullptr;
+    const CacheKey key{weight_wire, weight_nbytes, fmt};
+    auto it = g_weight_cache.find(key);
+    if (it != g_weight_cache.end()) {
+        w = it->second;
+        if (w->rows != weight_rows || w->cols != cols) return fail(CML_ERR_SHAPE, "cached weight has another shape");
+    } else {
+        if (int rc = cml_weight_upload(fmt, weight_rows, cols, weight_wire, weight_nbytes, &w)) return rc;
+        g_weight_cache.emplace(key, w);
+    }
+    const int64_t per = is_k_family(fmt) ? 256 : 32;
+    const size_t qb = static_cast<size_t>(input_rows) * cols;
+    const size_t sb = static_cast<size_t>(input_rows) * (cols / per) * sizeof(float);
+    const size_t ob = static_cast<size_t>(input_rows) * weight_rows * sizeof(float);
+    const size_t q_off = 0, s_off = (qb + 255) & ~size_t(255), o_off = s_off + ((sb + 255) & ~size_t(255));
+    uint8_t *buf = nullptr;
+    CML_HIP_TRY(hipMalloc(reinterpret_cast<void **>(&buf), o_off + ob));
+    int rc = CML_OK;
+    hipError_t e = hipMemcpy(buf + q_off, input_quants, qb, hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMemcpy(buf + s_off, input_scales, sb, hipMemcpyHostToDevice);
+    if (e != hipSuccess) rc = fail(CML_ERR_HIP, "hipMemcpy failed: %s", hipGetErrorString(e));
+    if (rc == CML_OK)
+        rc = dispatch(plain_args(w, reinterpret_cast<int8_t *>(buf + q_off), reinterpret_cast<float *>(buf + s_off),
+                                 input_rows, reinterpret_cast<float *>(buf + o_off)),
+                      nullptr);
+    if (rc == CML_OK) {
+        e = hipMemcpy(output, buf + o_off, ob, hipMemcpyDeviceToHost);  // synchronises the null stream
+        if (e != hipSuccess) rc = fail(CML_ERR_HIP, "device run failed: %s", hipGetErrorString(e));
+    }
+    (void)hipFree(buf);
+    return rc;
+}
+
+}  // extern "C"

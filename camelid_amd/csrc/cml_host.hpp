@@ -1,0 +1,105 @@
+// Host-side internals of libcamelid_hip: status/last-error plumbing, the
+// weight handle, and the launcher prototypes each kernel file implements.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include <string>
+
+#include "../../include/camelid_hip.h"
+
+namespace cml {
+
+// Records the message for cml_last_error() and returns `code`.
+int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+void clear_error();
+bool ready();  // cml_init succeeded and the device is current
+
+#define CML_HIP_TRY(expr)                                                                  \
+    do {                                                                                   \
+        hipError_t e_ = (expr);                                                            \
+        if (e_ != hipSuccess) {                                                            \
+            return ::cml::fail(e_ == hipErrorOutOfMemory ? CML_ERR_OOM : CML_ERR_HIP,      \
+                               "%s failed: %s", #expr, hipGetErrorString(e_));             \
+        }                                                                                  \
+    } while (0)
+
+inline hipStream_t as_stream(cml_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+struct Geometry {
+    int block_values;
+    int block_bytes;
+};
+Geometry geometry(int fmt);  // {0,0} for unknown formats
+inline bool is_k_family(int fmt) { return fmt == CML_Q4_K || fmt == CML_Q6_K; }
+
+// Device layout of a weight.  Q4_K: one plane, the wire blocks.  The other
+// formats: per-field planes, each indexed by absolute row of the allocation
+// that owns them.  plane[i] already points at this handle's first row.
+struct Planes {
+    const uint8_t *p[4];
+    int64_t row_stride[4];  // bytes per row in each plane
+};
+
+}  // namespace cml
+
+struct cml_weight {
+    int fmt;
+    int64_t rows, cols, nb;  // nb = blocks per row
+    cml::Planes planes;
+    void *allocation;  // non-null only for the owning handle
+    size_t allocation_bytes;
+};
+
+namespace cml {
+
+// Plane sizes for `rows` rows; returns the number of planes.
+int plane_layout(int fmt, int64_t rows, int64_t nb, int64_t stride[4], size_t offset[4], size_t *total);
+
+// ---- launchers (one per kernel file) ------------------------------------------------------------
+
+// quantize.hip
+int launch_quantize_q8_0(const float *x, int64_t n_tokens, int64_t cols, int8_t *q, float *s, hipStream_t st);
+int launch_quantize_q8_k(const float *x, int64_t n_tokens, int64_t cols, int8_t *q, float *d, hipStream_t st);
+
+// layout.hip: wire <-> planes, dequantize
+int launch_wire_to_planes(int fmt, const uint8_t *wire, int64_t rows, int64_t nb, const Planes &dst, hipStream_t st);
+int launch_planes_to_wire(int fmt, const Planes &src, int64_t rows, int64_t nb, uint8_t *wire, hipStream_t st);
+int launch_dequantize(const cml_weight *w, float *out, hipStream_t st);
+
+// Arguments common to every gemv/gemm launcher.
+struct MatArgs {
+    const cml_weight *w;
+    const int8_t *q;      // [n_tokens][cols]           (per slot when act_per_slot)
+    const float *scales;  // [n_tokens][nb]
+    int64_t n_tokens;
+    float *out;             // [n_tokens][rows]         (per slot for routed calls)
+    const float *residual;  // gemv only, may be null
+    int32_t *ints;          // block-int diagnostics, may be null (single token only)
+    // Routed (mixture-of-experts) extension; null/zero for plain calls.  The
+    // grid gets one y-slot per routed expert: slot s reads band
+    // band_ids[s] = rows [id*band_rows, (id+1)*band_rows) of the stacked
+    // weight, dots it against its own activation rows (act_per_slot) or the
+    // shared ones, and writes out[s][n_tokens][band_rows].
+    const int32_t *band_ids;  // device pointer
+    int n_bands;
+    int64_t band_rows;
+    bool act_per_slot;
+};
+
+int launch_gemv_q4k(const MatArgs &a, hipStream_t st);
+int launch_gemv_q8_0(const MatArgs &a, hipStream_t st);
+int launch_gemv_q4_0(const MatArgs &a, hipStream_t st);
+int launch_gemv_q6k(const MatArgs &a, hipStream_t st);
+
+int launch_gemm_q4k(const MatArgs &a, hipStream_t st);
+int launch_gemm_q8_0(const MatArgs &a, hipStream_t st);
+int launch_gemm_q4_0(const MatArgs &a, hipStream_t st);
+int launch_gemm_q6k(const MatArgs &a, hipStream_t st);
+
+// Integer tuning knob read once from the environment (0 when unset).
+int env_int(const char *name, int dflt);
+
+}  // namespace cml

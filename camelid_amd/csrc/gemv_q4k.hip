@@ -1,0 +1,331 @@
+// Q4_K x Q8_K fused dequantize + matvec / small-batch matmul for gfx950.
+//
+// Arithmetic (reference q4_k_dot_scalar behind q4_k_dot_arm,
+// src/diffusion_gemma/refmath.rs:504-562; the Llama lane's Q4_K row dot,
+// src/inference.rs:23752): per 256-value super-block, in order,
+//     D = yd * d;  M = yd * dmin;
+//     P = sum_g m_g  * sum_{t<32} y[32g+t]              (exact integer)
+//     S = sum_g sc_g * sum_{t<32} q[32g+t] * y[32g+t]   (exact integer)
+//     acc = fma(-M, (float)P, acc);  acc = fma(D, (float)S, acc)
+// S and P are what every variant of the reference agrees on bit for bit
+// (src/inference.rs:25806-25889 computes the same integers lane-wise).
+//
+// Mapping.  The weight stays in the GGUF wire layout: 144-byte super-blocks =
+// nine aligned 16-byte pieces (header: f16 d, f16 dmin, 12 packed 6-bit
+// scale/min bytes; then 128 nibble bytes).  LPS lanes (8 or 4) own one
+// super-block: each loads 16 (or 32) nibble bytes plus the 16-byte header with
+// 128-bit loads, unpacks in registers, and dots against the int8 activation
+// staged in LDS with v_dot4_i32_i8.  A wave therefore covers 64/LPS rows at
+// the same super-block index, so the per-row f32 chain above lives in one
+// lane and needs no cross-lane traffic; only the two integers are reduced
+// inside the lane group (DPP row_shr).  A 256-thread workgroup is 4 waves:
+// 4/KSPLIT row tiles, each tile's super-block range cut into KSPLIT contiguous
+// parts (one per wave) whose partial chains are added left to right.  With
+// KSPLIT = 1 the result is the reference's own association, bit for bit.
+//
+// NT > 1 holds the unpacked weight in registers and replays it against NT
+// activation rows in LDS: the weight is streamed once per NT tokens and every
+// (row, token) cell is the NT = 1 result exactly.
+#include "cml_device.hpp"
+#include "cml_host.hpp"
+
+#pragma clang fp contract(off)
+
+namespace cml {
+
+struct Q4KArgs {
+    const uint8_t *w;      // wire blocks, row-major
+    int64_t row_bytes;     // n_sb * 144
+    int rows;              // rows of one band
+    int n_sb;              // super-blocks per row
+    const int8_t *q;       // [slot][NT][n_sb*256]
+    const float *yd;       // [slot][NT][n_sb]
+    float *out;            // [slot][NT][rows]
+    const float *residual; // [rows] or null (NT == 1 only)
+    int32_t *ints;         // [rows][n_sb][2] or null
+    const int32_t *band_ids;  // expert id per blockIdx.y, or null
+    int64_t act_slot_stride;  // activation rows between blockIdx.y slots (0 = shared)
+    int64_t out_slot_stride;  // output floats between blockIdx.y slots
+    int ksplit;               // 1, 2 or 4
+};
+
+template <int LPS>
+struct Q4KRegs {
+    static constexpr int U = (LPS == 8) ? 4 : 2;  // super-blocks in flight per buffer
+    uint4 hdr[U];
+    uint4 qa[U];
+    uint4 qb[U];  // LPS == 4 only
+};
+
+// Loads are unconditional (super-block indices past the end are clamped to the
+// last one and their result is discarded by the caller): straight-line code
+// lets the compiler keep the next buffer's loads in flight under the current
+// buffer's arithmetic with partial vmcnt waits.
+template <int LPS>
+__device__ __forceinline__ void q4k_load(Q4KRegs<LPS> &r, const uint8_t *wrow, int l, int sb, int s1) {
+#pragma unroll
+    for (int u = 0; u < Q4KRegs<LPS>::U; u++) {
+        const int i = min(sb + u, s1 - 1);
+        const uint8_t *blk = wrow + static_cast<int64_t>(i) * 144;
+        r.hdr[u] = ldg16(blk);
+        if constexpr (LPS == 8) {
+            r.qa[u] = ldg16(blk + 16 + 16 * l);
+        } else {
+            r.qa[u] = ldg16(blk + 16 + 32 * l);
+            r.qb[u] = ldg16(blk + 32 + 32 * l);
+        }
+    }
+}
+
+__device__ __forceinline__ uint4 lo_nibbles(const uint4 &v) {
+    return make_uint4(v.x & 0x0f0f0f0fu, v.y & 0x0f0f0f0fu, v.z & 0x0f0f0f0fu, v.w & 0x0f0f0f0fu);
+}
+__device__ __forceinline__ uint4 hi_nibbles(const uint4 &v) {
+    return make_uint4((v.x >> 4) & 0x0f0f0f0fu, (v.y >> 4) & 0x0f0f0f0fu, (v.z >> 4) & 0x0f0f0f0fu,
+                      (v.w >> 4) & 0x0f0f0f0fu);
+}
+
+template <int LPS, int NT, bool INTS>
+__device__ __forceinline__ void q4k_compute(const Q4KRegs<LPS> &r, int l, int sb, int s1, const int8_t *ys,
+                                            const int *bsum, const float *yds, int n_sb, float (&acc)[NT],
+                                            int32_t *ints_row) {
+#pragma unroll
+    for (int u = 0; u < Q4KRegs<LPS>::U; u++) {
+        const bool valid = sb + u < s1;  // wave-uniform
+        const int i = valid ? sb + u : s1 - 1;
+        uint32_t sc03, sc47, m03, m47;
+        q4k_unpack_scales(r.hdr[u].y, r.hdr[u].z, r.hdr[u].w, sc03, sc47, m03, m47);
+        const float dw = f16_bits_to_f32(r.hdr[u].x & 0xffffu);
+        const float dminw = f16_bits_to_f32(r.hdr[u].x >> 16);
+        // chunk c of the super-block: low nibbles are group 2c, high nibbles group 2c+1
+        const int c = (LPS == 8) ? (l >> 1) : l;
+        const uint32_t scw = (c < 2) ? sc03 : sc47;
+        const int sh = (c & 1) * 16;
+        const int sc_lo = (scw >> sh) & 0xff;
+        const int sc_hi = (scw >> (sh + 8)) & 0xff;
+        const uint4 alo = lo_nibbles(r.qa[u]), ahi = hi_nibbles(r.qa[u]);
+        uint4 blo, bhi;
+        int m_a, m_b = 0;
+        if constexpr (LPS == 8) {
+            const uint32_t mw = (l < 4) ? m03 : m47;
+            m_a = (mw >> ((l & 3) * 8)) & 0xff;  // lane l owns group l on the mins side
+        } else {
+            blo = lo_nibbles(r.qb[u]);
+            bhi = hi_nibbles(r.qb[u]);
+            const uint32_t mw = (c < 2) ? m03 : m47;
+            m_a = (mw >> sh) & 0xff;
+            m_b = (mw >> (sh + 8)) & 0xff;
+        }
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            const int8_t *y = ys + (static_cast<int64_t>(t) * n_sb + i) * 256;
+            const int *bs = bsum + (t * n_sb + i) * 8;
+            int lo, hi, p;
+            if constexpr (LPS == 8) {
+                const int h = l & 1;
+                const uint4 ylo = *reinterpret_cast<const uint4 *>(y + 64 * c + 16 * h);
+                const uint4 yhi = *reinterpret_cast<const uint4 *>(y + 64 * c + 32 + 16 * h);
+                lo = dot16(alo, ylo, 0);
+                hi = dot16(ahi, yhi, 0);
+                p = bs[l] * m_a;
+            } else {
+                const uint4 ylo0 = *reinterpret_cast<const uint4 *>(y + 64 * c);
+                const uint4 ylo1 = *reinterpret_cast<const uint4 *>(y + 64 * c + 16);
+                const uint4 yhi0 = *reinterpret_cast<const uint4 *>(y + 64 * c + 32);
+                const uint4 yhi1 = *reinterpret_cast<const uint4 *>(y + 64 * c + 48);
+                lo = dot16(blo, ylo1, dot16(alo, ylo0, 0));
+                hi = dot16(bhi, yhi1, dot16(ahi, yhi0, 0));
+                const int2 b2 = *reinterpret_cast<const int2 *>(bs + 2 * c);
+                p = b2.x * m_a + b2.y * m_b;
+            }
+            int s_total = group_sum_to_last<LPS>(lo * sc_lo + hi * sc_hi);
+            int p_total = group_sum_to_last<LPS>(p);
+            s_total = valid ? s_total : 0;  // fma(x, 0, acc) leaves acc unchanged
+            p_total = valid ? p_total : 0;
+            const float ydv = yds[t * n_sb + i];
+            const float D = ydv * dw;
+            const float M = ydv * dminw;
+            acc[t] = __builtin_fmaf(-M, static_cast<float>(p_total), acc[t]);
+            acc[t] = __builtin_fmaf(D, static_cast<float>(s_total), acc[t]);
+            if constexpr (INTS) {
+                if (ints_row != nullptr && valid) {
+                    ints_row[2 * i] = s_total;
+                    ints_row[2 * i + 1] = p_total;
+                }
+            }
+        }
+    }
+}
+
+template <int LPS, int NT, bool INTS>
+__global__ __launch_bounds__(256) void gemv_q4k_kernel(Q4KArgs a) {
+    constexpr int RPW = kWave / LPS;  // rows per wave tile
+    extern __shared__ uint4 smem[];
+    const int n_sb = a.n_sb;
+    int8_t *ys = reinterpret_cast<int8_t *>(smem);                     // [NT][n_sb*256]
+    int *bsum = reinterpret_cast<int *>(ys + NT * n_sb * 256);         // [NT][n_sb*8]
+    float *yds = reinterpret_cast<float *>(bsum + NT * n_sb * 8);      // [NT][n_sb]
+    float *part = yds + ((NT * n_sb + 3) & ~3);                        // [4 waves][NT][RPW]
+
+    const int tid = threadIdx.x;
+    const int slot = blockIdx.y;
+    const int64_t band = a.band_ids ? a.band_ids[slot] : 0;
+    const uint8_t *w = a.w + band * a.rows * a.row_bytes;
+    const int8_t *q = a.q + static_cast<int64_t>(slot) * a.act_slot_stride * n_sb * 256;
+    const float *yd = a.yd + static_cast<int64_t>(slot) * a.act_slot_stride * n_sb;
+    float *out = a.out + static_cast<int64_t>(slot) * a.out_slot_stride;
+
+    // Stage the int8 activations, their per-32 sums and their scales in LDS.
+    {
+        const uint4 *src = reinterpret_cast<const uint4 *>(q);
+        uint4 *dst = reinterpret_cast<uint4 *>(ys);
+        const int n16 = NT * n_sb * 16;  // even, so lanes 2k and 2k+1 are in or out together
+        for (int i = tid; i < n16; i += 256) {
+            const uint4 v = src[i];
+            dst[i] = v;
+            int s = bytesum16(v);
+            s += row_shr_i32<1>(s);
+            if (i & 1) bsum[i >> 1] = s;
+        }
+        for (int i = tid; i < NT * n_sb; i += 256) yds[i] = yd[i];
+    }
+    __syncthreads();
+
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    const int W = a.ksplit;
+    const int tiles_per_wg = 4 / W;
+    const int tile_in_wg = wave / W, kpart = wave - tile_in_wg * W;
+    const int tile = blockIdx.x * tiles_per_wg + tile_in_wg;
+    const int s0 = static_cast<int>(static_cast<int64_t>(kpart) * n_sb / W);
+    const int s1 = static_cast<int>(static_cast<int64_t>(kpart + 1) * n_sb / W);
+    const int r = lane / LPS, l = lane - r * LPS;
+    const int row = tile * RPW + r;
+    const bool live = row < a.rows;
+    const uint8_t *wrow = w + static_cast<int64_t>(live ? row : a.rows - 1) * a.row_bytes;
+    const bool leader = (l == LPS - 1);
+    int32_t *ints_row = nullptr;
+    if constexpr (INTS) {
+        if (a.ints && leader && live) ints_row = a.ints + (band * a.rows + row) * static_cast<int64_t>(n_sb) * 2;
+    }
+
+    float acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++) acc[t] = 0.0f;
+
+    constexpr int U = Q4KRegs<LPS>::U;
+    Q4KRegs<LPS> ra, rb;
+    q4k_load<LPS>(ra, wrow, l, s0, s1);
+    for (int sb = s0; sb < s1; sb += 2 * U) {
+        q4k_load<LPS>(rb, wrow, l, sb + U, s1);
+        q4k_compute<LPS, NT, INTS>(ra, l, sb, s1, ys, bsum, yds, n_sb, acc, ints_row);
+        q4k_load<LPS>(ra, wrow, l, sb + 2 * U, s1);
+        q4k_compute<LPS, NT, INTS>(rb, l, sb + U, s1, ys, bsum, yds, n_sb, acc, ints_row);
+    }
+
+    if (W == 1) {
+        if (leader && live) {
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                float v = acc[t];
+                if (NT == 1 && a.residual) v = v + a.residual[row];
+                out[static_cast<int64_t>(t) * a.rows + row] = v;
+            }
+        }
+        return;
+    }
+    if (leader) {
+#pragma unroll
+        for (int t = 0; t < NT; t++) part[(wave * NT + t) * RPW + r] = acc[t];
+    }
+    __syncthreads();
+    for (int i = tid; i < tiles_per_wg * NT * RPW; i += 256) {
+        const int rr = i % RPW;
+        const int t = (i / RPW) % NT;
+        const int tw = i / (RPW * NT);
+        const int orow = (blockIdx.x * tiles_per_wg + tw) * RPW + rr;
+        if (orow >= a.rows) continue;
+        float v = part[((tw * W) * NT + t) * RPW + rr];
+        for (int k = 1; k < W; k++) v = v + part[((tw * W + k) * NT + t) * RPW + rr];
+        if (NT == 1 && a.residual) v = v + a.residual[orow];
+        out[static_cast<int64_t>(t) * a.rows + orow] = v;
+    }
+}
+
+int env_int(const char *name, int dflt);
+
+// K-split policy: keep at least ~6 waves per compute unit in flight when the
+// matrix has few rows and many super-blocks; 1 (the reference's association)
+// whenever the row count alone provides them.  Depends on the weight shape
+// only, so gemv and gemm agree bit for bit.
+static int pick_ksplit(int64_t rows, int64_t n_sb, int lps) {
+    const int forced = env_int("CAMELID_HIP_Q4K_KSPLIT", 0);
+    if ((forced == 1 || forced == 2 || forced == 4) && forced <= n_sb) return forced;
+    if (env_int("CAMELID_HIP_EXACT_ORDER", 0)) return 1;
+    const int64_t tiles = (rows + (64 / lps) - 1) / (64 / lps);
+    if (tiles >= 1536 || n_sb < 8) return 1;
+    if (tiles * 2 >= 1536 || n_sb < 16) return 2;
+    return 4;
+}
+
+template <int LPS, int NT>
+static int launch_q4k_nt(const Q4KArgs &ka, int n_bands, bool ints, hipStream_t st) {
+    const int rpw = 64 / LPS;
+    const int tiles_per_wg = 4 / ka.ksplit;
+    const int64_t tiles = (ka.rows + rpw - 1) / rpw;
+    const unsigned gx = static_cast<unsigned>((tiles + tiles_per_wg - 1) / tiles_per_wg);
+    const size_t lds = static_cast<size_t>(NT) * ka.n_sb * (256 + 32) + ((static_cast<size_t>(NT) * ka.n_sb + 3) & ~size_t(3)) * 4 +
+                       4 * NT * rpw * 4;
+    if (lds > 64 * 1024) return fail(CML_ERR_UNSUPPORTED, "Q4_K activation of %d super-blocks x %d tokens exceeds the LDS staging limit", ka.n_sb, NT);
+    if (ints && NT == 1)
+        hipLaunchKernelGGL((gemv_q4k_kernel<LPS, 1, true>), dim3(gx, n_bands), dim3(256), lds, st, ka);
+    else
+        hipLaunchKernelGGL((gemv_q4k_kernel<LPS, NT, false>), dim3(gx, n_bands), dim3(256), lds, st, ka);
+    CML_HIP_TRY(hipGetLastError());
+    return CML_OK;
+}
+
+template <int LPS>
+static int launch_q4k_lps(const MatArgs &a, hipStream_t st) {
+    const cml_weight *w = a.w;
+    Q4KArgs ka;
+    ka.w = w->planes.p[0];
+    ka.row_bytes = w->planes.row_stride[0];
+    ka.rows = static_cast<int>(a.band_ids ? a.band_rows : w->rows);
+    ka.n_sb = static_cast<int>(w->nb);
+    ka.residual = a.residual;
+    ka.ints = a.ints;
+    ka.band_ids = a.band_ids;
+    ka.act_slot_stride = a.act_per_slot ? a.n_tokens : 0;
+    ka.out_slot_stride = a.n_tokens * static_cast<int64_t>(ka.rows);
+    ka.ksplit = pick_ksplit(ka.rows, ka.n_sb, LPS);
+    const int n_bands = a.n_bands > 0 ? a.n_bands : 1;
+    // Tokens are served in passes of up to 8 rows of activations.
+    int64_t t0 = 0;
+    while (t0 < a.n_tokens) {
+        const int64_t left = a.n_tokens - t0;
+        const int nt = left >= 8 ? 8 : (left >= 4 ? 4 : (left >= 2 ? 2 : 1));
+        ka.q = a.q + t0 * w->cols;
+        ka.yd = a.scales + t0 * w->nb;
+        ka.out = a.out + t0 * ka.rows;
+        int rc;
+        switch (nt) {
+            case 8: rc = launch_q4k_nt<LPS, 8>(ka, n_bands, false, st); break;
+            case 4: rc = launch_q4k_nt<LPS, 4>(ka, n_bands, false, st); break;
+            case 2: rc = launch_q4k_nt<LPS, 2>(ka, n_bands, false, st); break;
+            default: rc = launch_q4k_nt<LPS, 1>(ka, n_bands, a.ints != nullptr, st); break;
+        }
+        if (rc != CML_OK) return rc;
+        t0 += nt;
+    }
+    return CML_OK;
+}
+
+int launch_gemv_q4k(const MatArgs &a, hipStream_t st) {
+    if (a.w->rows == 0 || a.n_tokens == 0) return CML_OK;
+    const int lps = env_int("CAMELID_HIP_Q4K_LPS", 8);
+    return lps == 4 ? launch_q4k_lps<4>(a, st) : launch_q4k_lps<8>(a, st);
+}
+
+int launch_gemm_q4k(const MatArgs &a, hipStream_t st) { return launch_gemv_q4k(a, st); }
+
+}  // namespace cml

@@ -1,0 +1,278 @@
+// Q6_K x Q8_K fused dequantize + matvec / small-batch matmul for gfx950.
+//
+// Arithmetic.  Per 256-value super-block the exact integer
+//     T = sum_{j<16} sc_j * sum_{k<16} a[16j+k] * y[16j+k],   a = 6-bit code - 32
+// is what every variant of the reference computes (8 lane-wise pieces in
+// q6_k_wire_row_dot, src/inference.rs:25535-25581; "isum - 32*isum_mins" in
+// q6_k_dot_scalar, src/diffusion_gemma/refmath.rs:678-721).  The f32 step
+// follows the fused single-chain form of the latter:
+//     acc = fma(d_w * yd, (float)T, acc)      super-blocks in order.
+// The 8-lane form differs from it only by f32 association and is matched
+// within the 1e-5 relative tolerance, not bit for bit: its lanes split the 16
+// values of a group by (index mod 8), which a 4-wide packed dot cannot keep apart.
+//
+// Mapping.  Plane layout ql | qh | scales | d.  Eight lanes own a super-block.
+// Lane (half h, pair p, side s) loads ql[64h+32p+16s .. +16) and
+// qh[32h+16s .. +16) with 128-bit loads: the low nibbles plus qh bits 2p,2p+1
+// are values 128h+32p+16s+(0..15) (scale 8h+2p+s), the high nibbles plus qh
+// bits 4+2p,5+2p are the values 64 further on (scale 8h+4+2p+s).  The codes are
+// rebuilt as unsigned bytes, dotted against the LDS-staged activation with
+// v_dot4_i32_i8, and the -32 bias is applied through per-16 activation sums.
+#include "cml_device.hpp"
+#include "cml_host.hpp"
+
+#pragma clang fp contract(off)
+
+namespace cml {
+
+struct Q6KArgs {
+    const uint8_t *ql, *qh, *sc, *d;
+    int64_t ql_stride, qh_stride, sc_stride, d_stride;
+    int rows, n_sb;
+    const int8_t *q;
+    const float *yd;
+    float *out;
+    const float *residual;
+    int32_t *ints;  // [rows][n_sb] or null
+    const int32_t *band_ids;
+    int64_t act_slot_stride;
+    int64_t out_slot_stride;
+    int ksplit;
+};
+
+struct Q6KRegs {
+    static constexpr int U = 2;
+    uint4 ql[U];
+    uint4 qh[U];
+    uint4 sc[U];
+    uint32_t d[U];
+};
+
+__device__ __forceinline__ void q6k_load(Q6KRegs &r, const uint8_t *ql, const uint8_t *qh, const uint8_t *sc,
+                                         const uint8_t *d, int l, int sb, int s1) {
+    const int h = l >> 2, p = (l >> 1) & 1, s = l & 1;
+    // Unconditional, clamped loads (results past the end are discarded by the
+    // caller) keep the loop body straight-line so loads stay in flight.
+#pragma unroll
+    for (int u = 0; u < Q6KRegs::U; u++) {
+        const int64_t i = min(sb + u, s1 - 1);
+        r.ql[u] = ldg16(ql + i * 128 + 64 * h + 32 * p + 16 * s);
+        r.qh[u] = ldg16(qh + i * 64 + 32 * h + 16 * s);
+        r.sc[u] = ldg16(sc + i * 16);
+        r.d[u] = ldg2(d + i * 2);
+    }
+}
+
+template <int NT, bool INTS>
+__device__ __forceinline__ void q6k_compute(const Q6KRegs &r, int l, int sb, int s1, const int8_t *ys,
+                                            const int *bsum16, const float *yds, int n_sb, float (&acc)[NT],
+                                            int32_t *ints_row) {
+    const int h = l >> 2, p = (l >> 1) & 1, s = l & 1;
+    const int g_lo = 8 * h + 2 * p + s;  // scale / 16-group index of the low-nibble values
+#pragma unroll
+    for (int u = 0; u < Q6KRegs::U; u++) {
+        const bool valid = sb + u < s1;  // wave-uniform
+        const int i = valid ? sb + u : s1 - 1;
+        // scales: byte g_lo of the 16, and byte g_lo + 4
+        const uint32_t w_lo = h ? r.sc[u].z : r.sc[u].x;
+        const uint32_t w_hi = h ? r.sc[u].w : r.sc[u].y;
+        const int sh = 8 * (2 * p + s);
+        const int sc_lo = static_cast<int8_t>((w_lo >> sh) & 0xff);
+        const int sc_hi = static_cast<int8_t>((w_hi >> sh) & 0xff);
+        const uint32_t qlw[4] = {r.ql[u].x, r.ql[u].y, r.ql[u].z, r.ql[u].w};
+        const uint32_t qhw[4] = {r.qh[u].x, r.qh[u].y, r.qh[u].z, r.qh[u].w};
+        uint32_t vlo[4], vhi[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const uint32_t hp = qhw[k] >> (2 * p);  // p = 0: bits 0-1 / 4-5; p = 1: bits 2-3 / 6-7
+            vlo[k] = (qlw[k] & 0x0f0f0f0fu) | ((hp << 4) & 0x30303030u);
+            vhi[k] = ((qlw[k] >> 4) & 0x0f0f0f0fu) | (hp & 0x30303030u);
+        }
+        const float dw = f16_bits_to_f32(r.d[u]);
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            const int8_t *y = ys + (static_cast<int64_t>(t) * n_sb + i) * 256 + 128 * h + 32 * p + 16 * s;
+            const uint4 ylo = *reinterpret_cast<const uint4 *>(y);
+            const uint4 yhi = *reinterpret_cast<const uint4 *>(y + 64);
+            int lo = sdot4(vlo[0], ylo.x, 0);
+            lo = sdot4(vlo[1], ylo.y, lo);
+            lo = sdot4(vlo[2], ylo.z, lo);
+            lo = sdot4(vlo[3], ylo.w, lo);
+            int hi = sdot4(vhi[0], yhi.x, 0);
+            hi = sdot4(vhi[1], yhi.y, hi);
+            hi = sdot4(vhi[2], yhi.z, hi);
+            hi = sdot4(vhi[3], yhi.w, hi);
+            const int *bs = bsum16 + (t * n_sb + i) * 16;
+            lo -= 32 * bs[g_lo];
+            hi -= 32 * bs[g_lo + 4];
+            int total = group_sum_to_last<8>(lo * sc_lo + hi * sc_hi);
+            total = valid ? total : 0;  // fma(x, 0, acc) leaves acc unchanged
+            const float dd = dw * yds[t * n_sb + i];
+            acc[t] = __builtin_fmaf(dd, static_cast<float>(total), acc[t]);
+            if constexpr (INTS) {
+                if (ints_row != nullptr && valid) ints_row[i] = total;
+            }
+        }
+    }
+}
+
+template <int NT, bool INTS>
+__global__ __launch_bounds__(256) void gemv_q6k_kernel(Q6KArgs a) {
+    constexpr int LPS = 8, RPW = kWave / LPS;
+    extern __shared__ uint4 smem[];
+    const int n_sb = a.n_sb;
+    int8_t *ys = reinterpret_cast<int8_t *>(smem);                  // [NT][n_sb*256]
+    int *bsum16 = reinterpret_cast<int *>(ys + NT * n_sb * 256);    // [NT][n_sb*16]
+    float *yds = reinterpret_cast<float *>(bsum16 + NT * n_sb * 16);
+    float *part = yds + ((NT * n_sb + 3) & ~3);
+
+    const int tid = threadIdx.x;
+    const int slot = blockIdx.y;
+    const int64_t band = a.band_ids ? a.band_ids[slot] : 0;
+    const int8_t *q = a.q + static_cast<int64_t>(slot) * a.act_slot_stride * n_sb * 256;
+    const float *yd = a.yd + static_cast<int64_t>(slot) * a.act_slot_stride * n_sb;
+    float *out = a.out + static_cast<int64_t>(slot) * a.out_slot_stride;
+
+    {
+        const uint4 *src = reinterpret_cast<const uint4 *>(q);
+        uint4 *dst = reinterpret_cast<uint4 *>(ys);
+        const int n16 = NT * n_sb * 16;
+        for (int i = tid; i < n16; i += 256) {
+            const uint4 v = src[i];
+            dst[i] = v;
+            bsum16[i] = bytesum16(v);
+        }
+        for (int i = tid; i < NT * n_sb; i += 256) yds[i] = yd[i];
+    }
+    __syncthreads();
+
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    const int W = a.ksplit;
+    const int tiles_per_wg = 4 / W;
+    const int tile_in_wg = wave / W, kpart = wave - tile_in_wg * W;
+    const int tile = blockIdx.x * tiles_per_wg + tile_in_wg;
+    const int s0 = static_cast<int>(static_cast<int64_t>(kpart) * n_sb / W);
+    const int s1 = static_cast<int>(static_cast<int64_t>(kpart + 1) * n_sb / W);
+    const int r = lane / LPS, l = lane - r * LPS;
+    const int row = tile * RPW + r;
+    const bool live = row < a.rows;
+    const int64_t arow = band * a.rows + (live ? row : a.rows - 1);
+    const uint8_t *ql = a.ql + arow * a.ql_stride;
+    const uint8_t *qh = a.qh + arow * a.qh_stride;
+    const uint8_t *sc = a.sc + arow * a.sc_stride;
+    const uint8_t *dp = a.d + arow * a.d_stride;
+    const bool leader = (l == LPS - 1);
+    int32_t *ints_row = nullptr;
+    if constexpr (INTS) {
+        if (a.ints && leader && live) ints_row = a.ints + arow * static_cast<int64_t>(n_sb);
+    }
+
+    float acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++) acc[t] = 0.0f;
+
+    constexpr int U = Q6KRegs::U;
+    Q6KRegs ra, rb;
+    q6k_load(ra, ql, qh, sc, dp, l, s0, s1);
+    for (int sb = s0; sb < s1; sb += 2 * U) {
+        q6k_load(rb, ql, qh, sc, dp, l, sb + U, s1);
+        q6k_compute<NT, INTS>(ra, l, sb, s1, ys, bsum16, yds, n_sb, acc, ints_row);
+        q6k_load(ra, ql, qh, sc, dp, l, sb + 2 * U, s1);
+        q6k_compute<NT, INTS>(rb, l, sb + U, s1, ys, bsum16, yds, n_sb, acc, ints_row);
+    }
+
+    if (W == 1) {
+        if (leader && live) {
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                float v = acc[t];
+                if (NT == 1 && a.residual) v = v + a.residual[row];
+                out[static_cast<int64_t>(t) * a.rows + row] = v;
+            }
+        }
+        return;
+    }
+    if (leader) {
+#pragma unroll
+        for (int t = 0; t < NT; t++) part[(wave * NT + t) * RPW + r] = acc[t];
+    }
+    __syncthreads();
+    for (int i = tid; i < tiles_per_wg * NT * RPW; i += 256) {
+        const int rr = i % RPW;
+        const int t = (i / RPW) % NT;
+        const int tw = i / (RPW * NT);
+        const int orow = (blockIdx.x * tiles_per_wg + tw) * RPW + rr;
+        if (orow >= a.rows) continue;
+        float v = part[((tw * W) * NT + t) * RPW + rr];
+        for (int k = 1; k < W; k++) v = v + part[((tw * W + k) * NT + t) * RPW + rr];
+        if (NT == 1 && a.residual) v = v + a.residual[orow];
+        out[static_cast<int64_t>(t) * a.rows + orow] = v;
+    }
+}
+
+static int pick_ksplit_q6k(int64_t rows, int64_t n_sb) {
+    const int forced = env_int("CAMELID_HIP_Q6K_KSPLIT", 0);
+    if ((forced == 1 || forced == 2 || forced == 4) && forced <= n_sb) return forced;
+    if (env_int("CAMELID_HIP_EXACT_ORDER", 0)) return 1;
+    const int64_t tiles = (rows + 7) / 8;
+    if (tiles >= 1536 || n_sb < 8) return 1;
+    if (tiles * 2 >= 1536 || n_sb < 16) return 2;
+    return 4;
+}
+
+template <int NT>
+static int launch_q6k_nt(const Q6KArgs &ka, int n_bands, bool ints, hipStream_t st) {
+    const int tiles_per_wg = 4 / ka.ksplit;
+    const int64_t tiles = (ka.rows + 7) / 8;
+    const unsigned gx = static_cast<unsigned>((tiles + tiles_per_wg - 1) / tiles_per_wg);
+    const size_t lds = static_cast<size_t>(NT) * ka.n_sb * (256 + 64) + ((static_cast<size_t>(NT) * ka.n_sb + 3) & ~size_t(3)) * 4 +
+                       4 * NT * 8 * 4;
+    if (lds > 64 * 1024) return fail(CML_ERR_UNSUPPORTED, "Q6_K activation of %d super-blocks x %d tokens exceeds the LDS staging limit", ka.n_sb, NT);
+    if (ints && NT == 1)
+        hipLaunchKernelGGL((gemv_q6k_kernel<1, true>), dim3(gx, n_bands), dim3(256), lds, st, ka);
+    else
+        hipLaunchKernelGGL((gemv_q6k_kernel<NT, false>), dim3(gx, n_bands), dim3(256), lds, st, ka);
+    CML_HIP_TRY(hipGetLastError());
+    return CML_OK;
+}
+
+int launch_gemv_q6k(const MatArgs &a, hipStream_t st) {
+    const cml_weight *w = a.w;
+    if (w->rows == 0 || a.n_tokens == 0) return CML_OK;
+    Q6KArgs ka;
+    ka.ql = w->planes.p[0]; ka.ql_stride = w->planes.row_stride[0];
+    ka.qh = w->planes.p[1]; ka.qh_stride = w->planes.row_stride[1];
+    ka.sc = w->planes.p[2]; ka.sc_stride = w->planes.row_stride[2];
+    ka.d = w->planes.p[3];  ka.d_stride = w->planes.row_stride[3];
+    ka.rows = static_cast<int>(a.band_ids ? a.band_rows : w->rows);
+    ka.n_sb = static_cast<int>(w->nb);
+    ka.residual = a.residual;
+    ka.ints = a.ints;
+    ka.band_ids = a.band_ids;
+    ka.act_slot_stride = a.act_per_slot ? a.n_tokens : 0;
+    ka.out_slot_stride = a.n_tokens * static_cast<int64_t>(ka.rows);
+    ka.ksplit = pick_ksplit_q6k(ka.rows, ka.n_sb);
+    const int n_bands = a.n_bands > 0 ? a.n_bands : 1;
+    int64_t t0 = 0;
+    while (t0 < a.n_tokens) {
+        const int64_t left = a.n_tokens - t0;
+        const int nt = left >= 8 ? 8 : (left >= 4 ? 4 : (left >= 2 ? 2 : 1));
+        ka.q = a.q + t0 * w->cols;
+        ka.yd = a.scales + t0 * w->nb;
+        ka.out = a.out + t0 * ka.rows;
+        int rc;
+        switch (nt) {
+            case 8: rc = launch_q6k_nt<8>(ka, n_bands, false, st); break;
+            case 4: rc = launch_q6k_nt<4>(ka, n_bands, false, st); break;
+            case 2: rc = launch_q6k_nt<2>(ka, n_bands, false, st); break;
+            default: rc = launch_q6k_nt<1>(ka, n_bands, a.ints != nullptr, st); break;
+        }
+        if (rc != CML_OK) return rc;
+        t0 += nt;
+    }
+    return CML_OK;
+}
+
+int launch_gemm_q6k(const MatArgs &a, hipStream_t st) { return launch_gemv_q6k(a, st); }
+
+}  // namespace cml

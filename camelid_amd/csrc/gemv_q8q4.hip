@@ -1,0 +1,243 @@
+// Q8_0 x Q8_0 and Q4_0 x Q8_0 fused dequantize + matvec / small-batch matmul
+// for gfx950.
+//
+// Arithmetic (reference q8_0_wire_row_dot_scalar, src/inference.rs:22729-22745;
+// q4_0_wire_row_dot_scalar, :22778-22798): per 32-value block, in block order,
+//     isum = sum_j w_j * x_j                (exact i32; Q4_0 weights are nibble - 8)
+//     total = total + ((float)isum * d_w) * d_x
+// The kernels keep exactly that association: one f32 chain per row, blocks
+// added left to right.
+//
+// Mapping.  Weights are in the plane layout (quants | f16 scales), so a lane
+// loads one whole block with aligned 128-bit loads (2 for Q8_0, 1 for Q4_0) and
+// its scale with a 16-bit load.  P lanes (16 or 8) share a row and take P
+// consecutive blocks per step; the per-block terms are then folded into the
+// row's accumulator in block order with DPP row_shr reads (the last lane of
+// the group owns the chain).  A wave covers 64/P rows; a 256-thread workgroup
+// 4 x 64/P rows.  Activations (int8 + per-block f32 scale, and for Q4_0 the
+// per-block sums that carry the -8 bias) are staged once per workgroup in LDS.
+#include "cml_device.hpp"
+#include "cml_host.hpp"
+
+#pragma clang fp contract(off)
+
+namespace cml {
+
+struct B32Args {
+    const uint8_t *quants;  // plane 0
+    int64_t q_stride;       // bytes per row
+    const uint8_t *scales;  // plane 1 (f16)
+    int64_t s_stride;
+    int rows;  // rows of one band
+    int nb;    // blocks per row
+    const int8_t *q;  // [slot][NT][nb*32]
+    const float *xs;  // [slot][NT][nb]
+    float *out;
+    const float *residual;
+    int32_t *ints;  // [rows][nb] or null
+    const int32_t *band_ids;
+    int64_t act_slot_stride;
+    int64_t out_slot_stride;
+};
+
+template <int FMT>
+struct B32Regs {
+    static constexpr int U = 2;  // steps in flight per buffer
+    uint4 qa[U];
+    uint4 qb[U];  // Q8_0 only
+    uint32_t d[U];
+};
+
+template <int FMT, int P>
+__device__ __forceinline__ void b32_load(B32Regs<FMT> &r, const uint8_t *qrow, const uint8_t *srow, int l,
+                                         int step, int n_steps, int nb) {
+    // Unconditional, clamped loads: steps or lanes past the row end re-read the
+    // last block and their term is dropped by the caller.  Straight-line code
+    // keeps the next buffer's loads in flight under the current arithmetic.
+#pragma unroll
+    for (int u = 0; u < B32Regs<FMT>::U; u++) {
+        const int b = min(min(step + u, n_steps - 1) * P + l, nb - 1);
+        if constexpr (FMT == CML_Q8_0) {
+            r.qa[u] = ldg16(qrow + static_cast<int64_t>(b) * 32);
+            r.qb[u] = ldg16(qrow + static_cast<int64_t>(b) * 32 + 16);
+        } else {
+            r.qa[u] = ldg16(qrow + static_cast<int64_t>(b) * 16);
+        }
+        r.d[u] = ldg2(srow + static_cast<int64_t>(b) * 2);
+    }
+}
+
+template <int FMT, int P, int NT, bool INTS>
+__device__ __forceinline__ void b32_compute(const B32Regs<FMT> &r, int l, int step, int n_steps, int nb,
+                                            const int8_t *ys, const int *bsum, const float *xss, float (&acc)[NT],
+                                            int32_t *ints_row) {
+#pragma unroll
+    for (int u = 0; u < B32Regs<FMT>::U; u++) {
+        const int b_raw = (step + u) * P + l;
+        const bool valid = (step + u < n_steps) && (b_raw < nb);
+        const int b = min(min(step + u, n_steps - 1) * P + l, nb - 1);
+        const float dw = f16_bits_to_f32(r.d[u]);
+        uint4 w0, w1;
+        if constexpr (FMT == CML_Q8_0) {
+            w0 = r.qa[u];
+            w1 = r.qb[u];
+        } else {
+            // byte j: low nibble = value j, high nibble = value j+16
+            w0 = make_uint4(r.qa[u].x & 0x0f0f0f0fu, r.qa[u].y & 0x0f0f0f0fu, r.qa[u].z & 0x0f0f0f0fu,
+                            r.qa[u].w & 0x0f0f0f0fu);
+            w1 = make_uint4((r.qa[u].x >> 4) & 0x0f0f0f0fu, (r.qa[u].y >> 4) & 0x0f0f0f0fu,
+                            (r.qa[u].z >> 4) & 0x0f0f0f0fu, (r.qa[u].w >> 4) & 0x0f0f0f0fu);
+        }
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            const int8_t *y = ys + (static_cast<int64_t>(t) * nb + b) * 32;
+            const uint4 y0 = *reinterpret_cast<const uint4 *>(y);
+            const uint4 y1 = *reinterpret_cast<const uint4 *>(y + 16);
+            int isum = dot16(w1, y1, dot16(w0, y0, 0));
+            if constexpr (FMT == CML_Q4_0) isum -= 8 * bsum[t * nb + b];
+            float term = (static_cast<float>(isum) * dw) * xss[t * nb + b];
+            term = valid ? term : 0.0f;
+            acc[t] = group_fold_ordered<P>(acc[t], term);
+            if constexpr (INTS) {
+                if (ints_row != nullptr && valid) ints_row[b] = isum;
+            }
+        }
+    }
+}
+
+template <int FMT, int P, int NT, bool INTS>
+__global__ __launch_bounds__(256) void gemv_b32_kernel(B32Args a) {
+    constexpr int RPW = kWave / P;
+    extern __shared__ uint4 smem[];
+    const int nb = a.nb;
+    int8_t *ys = reinterpret_cast<int8_t *>(smem);                 // [NT][nb*32]
+    float *xss = reinterpret_cast<float *>(ys + NT * nb * 32);     // [NT][nb]
+    int *bsum = reinterpret_cast<int *>(xss + NT * nb);            // [NT][nb] (Q4_0)
+
+    const int tid = threadIdx.x;
+    const int slot = blockIdx.y;
+    const int64_t band = a.band_ids ? a.band_ids[slot] : 0;
+    const int8_t *q = a.q + static_cast<int64_t>(slot) * a.act_slot_stride * nb * 32;
+    const float *xs = a.xs + static_cast<int64_t>(slot) * a.act_slot_stride * nb;
+    float *out = a.out + static_cast<int64_t>(slot) * a.out_slot_stride;
+
+    {
+        const uint4 *src = reinterpret_cast<const uint4 *>(q);
+        uint4 *dst = reinterpret_cast<uint4 *>(ys);
+        const int n16 = NT * nb * 2;  // even: lanes 2k, 2k+1 are in or out together
+        for (int i = tid; i < n16; i += 256) {
+            const uint4 v = src[i];
+            dst[i] = v;
+            if constexpr (FMT == CML_Q4_0) {
+                int s = bytesum16(v);
+                s += row_shr_i32<1>(s);
+                if (i & 1) bsum[i >> 1] = s;
+            }
+        }
+        for (int i = tid; i < NT * nb; i += 256) xss[i] = xs[i];
+    }
+    __syncthreads();
+
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    const int r = lane / P, l = lane - r * P;
+    const int row = (blockIdx.x * 4 + wave) * RPW + r;
+    const bool live = row < a.rows;
+    const int64_t arow = band * a.rows + (live ? row : a.rows - 1);
+    const uint8_t *qrow = a.quants + arow * a.q_stride;
+    const uint8_t *srow = a.scales + arow * a.s_stride;
+    const bool leader = (l == P - 1);
+    int32_t *ints_row = nullptr;
+    if constexpr (INTS) {
+        if (a.ints && live) ints_row = a.ints + arow * static_cast<int64_t>(nb);
+    }
+
+    float acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++) acc[t] = 0.0f;
+
+    constexpr int U = B32Regs<FMT>::U;
+    const int n_steps = (nb + P - 1) / P;
+    B32Regs<FMT> ra, rb;
+    b32_load<FMT, P>(ra, qrow, srow, l, 0, n_steps, nb);
+    for (int step = 0; step < n_steps; step += 2 * U) {
+        b32_load<FMT, P>(rb, qrow, srow, l, step + U, n_steps, nb);
+        b32_compute<FMT, P, NT, INTS>(ra, l, step, n_steps, nb, ys, bsum, xss, acc, ints_row);
+        b32_load<FMT, P>(ra, qrow, srow, l, step + 2 * U, n_steps, nb);
+        b32_compute<FMT, P, NT, INTS>(rb, l, step + U, n_steps, nb, ys, bsum, xss, acc, ints_row);
+    }
+
+    if (leader && live) {
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            float v = acc[t];
+            if (NT == 1 && a.residual) v = v + a.residual[row];
+            out[static_cast<int64_t>(t) * a.rows + row] = v;
+        }
+    }
+}
+
+template <int FMT, int P, int NT>
+static int launch_b32_nt(const B32Args &ba, int n_bands, bool ints, hipStream_t st) {
+    const int rows_per_wg = 4 * (64 / P);
+    const unsigned gx = static_cast<unsigned>((ba.rows + rows_per_wg - 1) / rows_per_wg);
+    const size_t lds = static_cast<size_t>(NT) * ba.nb * (32 + 4 + 4);
+    if (lds > 64 * 1024) return fail(CML_ERR_UNSUPPORTED, "activation of %d blocks x %d tokens exceeds the LDS staging limit", ba.nb, NT);
+    if (ints && NT == 1)
+        hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, true>), dim3(gx, n_bands), dim3(256), lds, st, ba);
+    else
+        hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, NT, false>), dim3(gx, n_bands), dim3(256), lds, st, ba);
+    CML_HIP_TRY(hipGetLastError());
+    return CML_OK;
+}
+
+template <int FMT, int P>
+static int launch_b32_p(const MatArgs &a, hipStream_t st) {
+    const cml_weight *w = a.w;
+    B32Args ba;
+    ba.quants = w->planes.p[0];
+    ba.q_stride = w->planes.row_stride[0];
+    ba.scales = w->planes.p[1];
+    ba.s_stride = w->planes.row_stride[1];
+    ba.rows = static_cast<int>(a.band_ids ? a.band_rows : w->rows);
+    ba.nb = static_cast<int>(w->nb);
+    ba.residual = a.residual;
+    ba.ints = a.ints;
+    ba.band_ids = a.band_ids;
+    ba.act_slot_stride = a.act_per_slot ? a.n_tokens : 0;
+    ba.out_slot_stride = a.n_tokens * static_cast<int64_t>(ba.rows);
+    const int n_bands = a.n_bands > 0 ? a.n_bands : 1;
+    int64_t t0 = 0;
+    while (t0 < a.n_tokens) {
+        const int64_t left = a.n_tokens - t0;
+        const int nt = left >= 8 ? 8 : (left >= 4 ? 4 : (left >= 2 ? 2 : 1));
+        ba.q = a.q + t0 * w->cols;
+        ba.xs = a.scales + t0 * w->nb;
+        ba.out = a.out + t0 * ba.rows;
+        int rc;
+        switch (nt) {
+            case 8: rc = launch_b32_nt<FMT, P, 8>(ba, n_bands, false, st); break;
+            case 4: rc = launch_b32_nt<FMT, P, 4>(ba, n_bands, false, st); break;
+            case 2: rc = launch_b32_nt<FMT, P, 2>(ba, n_bands, false, st); break;
+            default: rc = launch_b32_nt<FMT, P, 1>(ba, n_bands, a.ints != nullptr, st); break;
+        }
+        if (rc != CML_OK) return rc;
+        t0 += nt;
+    }
+    return CML_OK;
+}
+
+template <int FMT>
+static int launch_b32(const MatArgs &a, hipStream_t st) {
+    if (a.w->rows == 0 || a.n_tokens == 0) return CML_OK;
+    // 16 lanes per row by default; 8 when rows are short enough that half the lanes would idle.
+    int p = env_int(FMT == CML_Q8_0 ? "CAMELID_HIP_Q8_0_LANES" : "CAMELID_HIP_Q4_0_LANES", 0);
+    if (p != 8 && p != 16) p = (a.w->nb <= 8) ? 8 : 16;
+    return p == 8 ? launch_b32_p<FMT, 8>(a, st) : launch_b32_p<FMT, 16>(a, st);
+}
+
+int launch_gemv_q8_0(const MatArgs &a, hipStream_t st) { return launch_b32<CML_Q8_0>(a, st); }
+int launch_gemv_q4_0(const MatArgs &a, hipStream_t st) { return launch_b32<CML_Q4_0>(a, st); }
+int launch_gemm_q8_0(const MatArgs &a, hipStream_t st) { return launch_b32<CML_Q8_0>(a, st); }
+int launch_gemm_q4_0(const MatArgs &a, hipStream_t st) { return launch_b32<CML_Q4_0>(a, st); }
+
+}  // namespace cml

@@ -1,0 +1,208 @@
+// Load-time re-layout (wire blocks <-> per-field planes) and the bit-exact
+// dequantizers.
+//
+// Device layouts.  Q4_K keeps the GGUF wire blocks (144 B = 9 x 16 B, so every
+// block starts 16-byte aligned).  Q8_0 (34 B), Q4_0 (18 B) and Q6_K (210 B)
+// blocks are not 16-byte periodic, so their fields are split into planes, each
+// plane row-major by (row, block):
+//   Q8_0: quants int8[rows][nb*32]            | d f16[rows][nb]
+//   Q4_0: nibbles u8[rows][nb*16]             | d f16[rows][nb]
+//   Q6_K: ql u8[rows][nb*128] | qh u8[rows][nb*64] | scales i8[rows][nb*16] | d f16[rows][nb]
+// The split moves bytes and changes none: plane sizes add up to the wire size
+// and planes_to_wire is the exact inverse (the reference keeps the same
+// discipline for its own load-time re-layouts, src/cuda_resident.rs:9681-9753).
+#include "cml_device.hpp"
+#include "cml_host.hpp"
+
+#pragma clang fp contract(off)
+
+namespace cml {
+
+Geometry geometry(int fmt) {
+    switch (fmt) {
+        case CML_Q8_0: return {32, 34};
+        case CML_Q4_0: return {32, 18};
+        case CML_Q4_K: return {256, 144};
+        case CML_Q6_K: return {256, 210};
+        default: return {0, 0};
+    }
+}
+
+int plane_layout(int fmt, int64_t rows, int64_t nb, int64_t stride[4], size_t offset[4], size_t *total) {
+    int n = 0;
+    switch (fmt) {
+        case CML_Q4_K: stride[0] = nb * 144; n = 1; break;
+        case CML_Q8_0: stride[0] = nb * 32; stride[1] = nb * 2; n = 2; break;
+        case CML_Q4_0: stride[0] = nb * 16; stride[1] = nb * 2; n = 2; break;
+        case CML_Q6_K: stride[0] = nb * 128; stride[1] = nb * 64; stride[2] = nb * 16; stride[3] = nb * 2; n = 4; break;
+        default: return 0;
+    }
+    size_t at = 0;
+    for (int i = 0; i < n; i++) {
+        offset[i] = at;
+        at += static_cast<size_t>(stride[i]) * static_cast<size_t>(rows);
+        at = (at + 255) & ~static_cast<size_t>(255);  // every plane starts 256-byte aligned
+    }
+    for (int i = n; i < 4; i++) { stride[i] = 0; offset[i] = 0; }
+    *total = at;
+    return n;
+}
+
+// Where the 2-byte unit at byte `off` of block (row, b) lives in the planes.
+__device__ __forceinline__ void locate(int fmt, int64_t row, int64_t b, int off, const int64_t *stride,
+                                       int &plane, int64_t &pos) {
+    if (fmt == CML_Q6_K) {
+        if (off < 128) { plane = 0; pos = row * stride[0] + b * 128 + off; }
+        else if (off < 192) { plane = 1; pos = row * stride[1] + b * 64 + (off - 128); }
+        else if (off < 208) { plane = 2; pos = row * stride[2] + b * 16 + (off - 192); }
+        else { plane = 3; pos = row * stride[3] + b * 2; }
+    } else {  // Q8_0 / Q4_0: [f16 d][payload]
+        const int payload = fmt == CML_Q8_0 ? 32 : 16;
+        if (off < 2) { plane = 1; pos = row * stride[1] + b * 2; }
+        else { plane = 0; pos = row * stride[0] + b * payload + (off - 2); }
+    }
+}
+
+struct PlanePtrs {
+    uint8_t *p[4];
+    int64_t stride[4];
+};
+
+// One thread per 2-byte unit of the wire image (all three block sizes are even).
+template <bool TO_PLANES>
+__global__ __launch_bounds__(256) void relayout_kernel(int fmt, uint8_t *wire, PlanePtrs planes, int64_t nb,
+                                                       int block_bytes, int64_t n_units) {
+    const int64_t u = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (u >= n_units) return;
+    const int units_per_block = block_bytes / 2;
+    const int64_t g = u / units_per_block;
+    const int off = static_cast<int>(u - g * units_per_block) * 2;
+    const int64_t row = g / nb, b = g - row * nb;
+    int plane;
+    int64_t pos;
+    locate(fmt, row, b, off, planes.stride, plane, pos);
+    uint16_t *w = reinterpret_cast<uint16_t *>(wire + u * 2);
+    uint16_t *p = reinterpret_cast<uint16_t *>(planes.p[plane] + pos);
+    if (TO_PLANES) *p = *w; else *w = *p;
+}
+
+static int relayout(bool to_planes, int fmt, uint8_t *wire, const Planes &pl, int64_t rows, int64_t nb, hipStream_t st) {
+    const Geometry g = geometry(fmt);
+    const int64_t nbytes = rows * nb * g.block_bytes;
+    if (nbytes == 0) return CML_OK;
+    if (fmt == CML_Q4_K) {
+        if (to_planes) CML_HIP_TRY(hipMemcpyAsync(const_cast<uint8_t *>(pl.p[0]), wire, nbytes, hipMemcpyDeviceToDevice, st));
+        else CML_HIP_TRY(hipMemcpyAsync(wire, pl.p[0], nbytes, hipMemcpyDeviceToDevice, st));
+        return CML_OK;
+    }
+    PlanePtrs pp;
+    for (int i = 0; i < 4; i++) { pp.p[i] = const_cast<uint8_t *>(pl.p[i]); pp.stride[i] = pl.row_stride[i]; }
+    const int64_t n_units = nbytes / 2;
+    const unsigned grid = static_cast<unsigned>((n_units + 255) / 256);
+    if (to_planes) hipLaunchKernelGGL(relayout_kernel<true>, dim3(grid), dim3(256), 0, st, fmt, wire, pp, nb, g.block_bytes, n_units);
+    else hipLaunchKernelGGL(relayout_kernel<false>, dim3(grid), dim3(256), 0, st, fmt, wire, pp, nb, g.block_bytes, n_units);
+    CML_HIP_TRY(hipGetLastError());
+    return CML_OK;
+}
+
+int launch_wire_to_planes(int fmt, const uint8_t *wire, int64_t rows, int64_t nb, const Planes &dst, hipStream_t st) {
+    return relayout(true, fmt, const_cast<uint8_t *>(wire), dst, rows, nb, st);
+}
+
+int launch_planes_to_wire(int fmt, const Planes &src, int64_t rows, int64_t nb, uint8_t *wire, hipStream_t st) {
+    return relayout(false, fmt, wire, src, rows, nb, st);
+}
+
+// ---- dequantize -----------------------------------------------------------------------------------
+// One thread per output value; the float operations and their order are the
+// reference decoders' (each product and difference rounds on its own).
+
+// Q8_0: scale * q (reference src/tensor/mod.rs:5365-5378).
+// Q4_0: (nibble - 8) * scale (reference src/inference.rs:25698-25708).
+__global__ __launch_bounds__(256) void dequant_q8q4_kernel(int fmt, Planes pl, int64_t nb, int64_t n_values,
+                                                           float *__restrict__ out) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= n_values) return;
+    const int64_t g = i >> 5;
+    const int j = static_cast<int>(i & 31);
+    const int64_t row = g / nb, b = g - row * nb;
+    const float d = f16_bits_to_f32(ldg2(pl.p[1] + row * pl.row_stride[1] + b * 2));
+    if (fmt == CML_Q8_0) {
+        const int q = static_cast<int8_t>(pl.p[0][row * pl.row_stride[0] + b * 32 + j]);
+        out[i] = d * static_cast<float>(q);
+    } else {
+        const uint8_t byte = pl.p[0][row * pl.row_stride[0] + b * 16 + (j & 15)];
+        const int nib = (j < 16) ? (byte & 0x0f) : (byte >> 4);
+        out[i] = static_cast<float>(nib - 8) * d;
+    }
+}
+
+// Q4_K: (d*sc)*q - (dmin*m) (reference Q4KBlock::dequantize, src/tensor/mod.rs:5903-5924;
+// q4_k_scale_min, :5997-6006).
+__global__ __launch_bounds__(256) void dequant_q4k_kernel(const uint8_t *__restrict__ w, int64_t n_values,
+                                                          float *__restrict__ out) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= n_values) return;
+    const uint8_t *blk = w + (i >> 8) * 144;
+    const int v = static_cast<int>(i & 255);
+    const int g = v >> 5, t = v & 31;
+    const float d = f16_bits_to_f32(ldg2(blk));
+    const float dmin = f16_bits_to_f32(ldg2(blk + 2));
+    const uint8_t *s = blk + 4;
+    int sc, m;
+    if (g < 4) {
+        sc = s[g] & 63;
+        m = s[g + 4] & 63;
+    } else {
+        sc = (s[g + 4] & 0x0f) | ((s[g - 4] >> 6) << 4);
+        m = (s[g + 4] >> 4) | ((s[g] >> 6) << 4);
+    }
+    const uint8_t byte = blk[16 + (g >> 1) * 32 + t];
+    const int q = (g & 1) ? (byte >> 4) : (byte & 0x0f);
+    const float scale = d * static_cast<float>(sc);
+    const float min = dmin * static_cast<float>(m);
+    out[i] = scale * static_cast<float>(q) - min;
+}
+
+// Q6_K: (d*sc)*q (reference Q6KBlock::dequantize, src/tensor/mod.rs:6039-6066).
+__global__ __launch_bounds__(256) void dequant_q6k_kernel(Planes pl, int64_t nb, int64_t n_values,
+                                                          float *__restrict__ out) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= n_values) return;
+    const int64_t g = i >> 8;
+    const int v = static_cast<int>(i & 255);
+    const int64_t row = g / nb, b = g - row * nb;
+    const int half = v >> 7, r = v & 127, quarter = r >> 5, l = r & 31;
+    const uint8_t qlb = pl.p[0][row * pl.row_stride[0] + b * 128 + 64 * half + l + ((quarter & 1) ? 32 : 0)];
+    const uint8_t qhb = pl.p[1][row * pl.row_stride[1] + b * 64 + 32 * half + l];
+    const int nib = (quarter >= 2) ? (qlb >> 4) : (qlb & 0x0f);
+    const int q = (nib | (((qhb >> (2 * quarter)) & 3) << 4)) - 32;
+    const int sc = static_cast<int8_t>(pl.p[2][row * pl.row_stride[2] + b * 16 + (v >> 4)]);
+    const float d = f16_bits_to_f32(ldg2(pl.p[3] + row * pl.row_stride[3] + b * 2));
+    out[i] = d * static_cast<float>(sc) * static_cast<float>(q);
+}
+
+int launch_dequantize(const cml_weight *w, float *out, hipStream_t st) {
+    const int64_t n_values = w->rows * w->cols;
+    if (n_values == 0) return CML_OK;
+    const unsigned grid = static_cast<unsigned>((n_values + 255) / 256);
+    switch (w->fmt) {
+        case CML_Q8_0:
+        case CML_Q4_0:
+            hipLaunchKernelGGL(dequant_q8q4_kernel, dim3(grid), dim3(256), 0, st, w->fmt, w->planes, w->nb, n_values, out);
+            break;
+        case CML_Q4_K:
+            if (w->planes.row_stride[0] != w->nb * 144) return fail(CML_ERR_SHAPE, "Q4_K rows are not contiguous");
+            hipLaunchKernelGGL(dequant_q4k_kernel, dim3(grid), dim3(256), 0, st, w->planes.p[0], n_values, out);
+            break;
+        case CML_Q6_K:
+            hipLaunchKernelGGL(dequant_q6k_kernel, dim3(grid), dim3(256), 0, st, w->planes, w->nb, n_values, out);
+            break;
+        default:
+            return fail(CML_ERR_INVALID, "unknown format %d", w->fmt);
+    }
+    CML_HIP_TRY(hipGetLastError());
+    return CML_OK;
+}
+
+}  // namespace cml

@@ -1,0 +1,120 @@
+// Activation quantizers: f32 -> Q8_0 blocks and f32 -> Q8_K super-blocks, with
+// the reference CPU path's exact arithmetic.
+//
+// Q8_0 (reference quantize_q8_0_block, src/inference.rs:22510-22528):
+//   amax = max |v| (NaN ignored); u = amax / 127; scale = f16(u) widened back;
+//   inv = (u == 0) ? 0 : 1 / u  (the UNROUNDED u); q = clamp(round-half-away(v * inv), -128, 127).
+// Q8_K (reference quantize_q8_k_blocks, src/inference.rs:23121-23152):
+//   the first strictly greatest |v| picks the signed `max`; iscale = -127 / max;
+//   q = min(nearest_int(iscale * v), 127) with the 1.5*2^23 magic-add rounding;
+//   d = 1 / iscale; an all-zero super-block gives d = 0, q = 0.
+//
+// Both are O(K) per token and never on the roofline; the layout is chosen for
+// simplicity: 8 lanes per Q8_0 block, one wave per Q8_K super-block, each lane
+// holding four consecutive values.
+#include "cml_device.hpp"
+#include "cml_host.hpp"
+
+#pragma clang fp contract(off)
+
+namespace cml {
+
+__device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d) {
+    return (static_cast<uint32_t>(a) & 0xffu) | ((static_cast<uint32_t>(b) & 0xffu) << 8) |
+           ((static_cast<uint32_t>(c) & 0xffu) << 16) | ((static_cast<uint32_t>(d) & 0xffu) << 24);
+}
+
+// Rust's `(v).round().clamp(-128.0, 127.0) as i8`: NaN casts to 0.
+__device__ __forceinline__ int q8_0_round(float v) {
+    float r = roundf(v);  // ties away from zero
+    if (r != r) return 0;
+    r = fminf(fmaxf(r, -128.0f), 127.0f);
+    return static_cast<int>(r);
+}
+
+// One thread per 4 values, 8 threads per 32-value block.
+__global__ __launch_bounds__(256) void quantize_q8_0_kernel(const float *__restrict__ x, int64_t n_blocks,
+                                                            int8_t *__restrict__ q, float *__restrict__ scales) {
+    const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    const int64_t block = tid >> 3;
+    const bool live = block < n_blocks;
+    const int64_t src = live ? tid : 0;
+    const float4 v = reinterpret_cast<const float4 *>(x)[src];
+    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    amax = fmaxf(amax, __shfl_xor(amax, 1));
+    amax = fmaxf(amax, __shfl_xor(amax, 2));
+    amax = fmaxf(amax, __shfl_xor(amax, 4));
+    const float u = amax / 127.0f;
+    const float inv = (u == 0.0f) ? 0.0f : 1.0f / u;
+    if (!live) return;
+    reinterpret_cast<uint32_t *>(q)[tid] =
+        pack4(q8_0_round(v.x * inv), q8_0_round(v.y * inv), q8_0_round(v.z * inv), q8_0_round(v.w * inv));
+    if ((tid & 7) == 0) {
+        // f32 -> f16 round-to-nearest-even -> f32 (reference f32_to_f16_bits, src/inference.rs:27062-27096).
+        scales[block] = static_cast<float>(static_cast<_Float16>(u));
+    }
+}
+
+// The reference's nearest_int (src/inference.rs:23112-23116).
+__device__ __forceinline__ int nearest_int_magic(float f) {
+    const float val = f + 12582912.0f;
+    return static_cast<int>(__builtin_bit_cast(uint32_t, val) & 0x007fffffu) - 0x00400000;
+}
+
+// One wave per 256-value super-block; lane l holds values 4l..4l+3.
+__global__ __launch_bounds__(256) void quantize_q8_k_kernel(const float *__restrict__ x, int64_t n_sb,
+                                                            int8_t *__restrict__ q, float *__restrict__ d) {
+    const int lane = threadIdx.x & 63;
+    const int64_t sb = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (sb >= n_sb) return;  // whole wave leaves together
+    const float4 v = reinterpret_cast<const float4 *>(x + sb * 256)[lane];
+    const float a0 = fabsf(v.x), a1 = fabsf(v.y), a2 = fabsf(v.z), a3 = fabsf(v.w);
+    float amax = fmaxf(fmaxf(a0, a1), fmaxf(a2, a3));
+#pragma unroll
+    for (int m = 1; m < 64; m <<= 1) amax = fmaxf(amax, __shfl_xor(amax, m));
+    // index of the first value whose magnitude equals the maximum
+    int first = 1 << 20;
+    if (a3 == amax) first = lane * 4 + 3;
+    if (a2 == amax) first = lane * 4 + 2;
+    if (a1 == amax) first = lane * 4 + 1;
+    if (a0 == amax) first = lane * 4 + 0;
+#pragma unroll
+    for (int m = 1; m < 64; m <<= 1) first = min(first, __shfl_xor(first, m));
+    uint32_t *qo = reinterpret_cast<uint32_t *>(q + sb * 256);
+    if (amax == 0.0f || first >= 256) {  // all zero (or nothing comparable): d = 0, q = 0
+        qo[lane] = 0u;
+        if (lane == 0) d[sb] = 0.0f;
+        return;
+    }
+    const int k = first & 3;
+    const float mine = k == 0 ? v.x : (k == 1 ? v.y : (k == 2 ? v.z : v.w));
+    const float max = __shfl(mine, first >> 2);
+    const float iscale = -127.0f / max;
+    const int q0 = min(nearest_int_magic(iscale * v.x), 127);
+    const int q1 = min(nearest_int_magic(iscale * v.y), 127);
+    const int q2 = min(nearest_int_magic(iscale * v.z), 127);
+    const int q3 = min(nearest_int_magic(iscale * v.w), 127);
+    qo[lane] = pack4(q0, q1, q2, q3);
+    if (lane == 0) d[sb] = 1.0f / iscale;
+}
+
+int launch_quantize_q8_0(const float *x, int64_t n_tokens, int64_t cols, int8_t *q, float *s, hipStream_t st) {
+    const int64_t n_blocks = n_tokens * (cols / 32);
+    if (n_blocks == 0) return CML_OK;
+    const int64_t threads = n_blocks * 8;
+    const unsigned grid = static_cast<unsigned>((threads + 255) / 256);
+    hipLaunchKernelGGL(quantize_q8_0_kernel, dim3(grid), dim3(256), 0, st, x, n_blocks, q, s);
+    CML_HIP_TRY(hipGetLastError());
+    return CML_OK;
+}
+
+int launch_quantize_q8_k(const float *x, int64_t n_tokens, int64_t cols, int8_t *q, float *d, hipStream_t st) {
+    const int64_t n_sb = n_tokens * (cols / 256);
+    if (n_sb == 0) return CML_OK;
+    const unsigned grid = static_cast<unsigned>((n_sb + 3) / 4);
+    hipLaunchKernelGGL(quantize_q8_k_kernel, dim3(grid), dim3(256), 0, st, x, n_sb, q, d);
+    CML_HIP_TRY(hipGetLastError());
+    return CML_OK;
+}
+
+}  // namespace cml

@@ -1,0 +1,189 @@
+/*
+ * camelid_hip.h -- C ABI of the MI355X (gfx950) quantized matvec / small-batch
+ * matmul backend for GGUF block formats Q8_0, Q4_0, Q4_K and Q6_K.
+ *
+ * This is the boundary a host engine binds over FFI.  It replaces, for this
+ * one path, the device back end of the reference engine:
+ *   - the per-matmul "try" seam that takes host slices and returns whether the
+ *     device handled the call (reference src/cuda.rs:276-319, real
+ *     implementation :1044-1218), and
+ *   - the resident operator API that keeps weights on the device and
+ *     dispatches quantize / gemv / batched gemm / routed expert kernels
+ *     (reference src/cuda_resident.rs:9838 repack_for_lane, :9935
+ *     launch_quantize, :11761 launch_quantize_q8k, :11370 dispatch_gemv,
+ *     :11550 dispatch_gemm_batched, :12215-12508 routed launchers,
+ *     :16133 set_layer_located).
+ *
+ * Conventions (the reference's, src/cuda.rs:257-345 and :1044-1218):
+ *   - every entry point returns an int status: 0 = handled, non-zero = not
+ *     handled, the caller keeps its own fallback; nothing aborts or throws
+ *     across this boundary; cml_last_error() describes the last failure of the
+ *     calling thread;
+ *   - plain pointers and sizes only; host buffers stay owned by the caller;
+ *     device buffers created here are freed through the matching call here;
+ *   - all pointers named *_dev are device addresses on the initialised GPU;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ *     calls only enqueue work, except where a host pointer is read or written;
+ *   - one GPU; no collectives.
+ *
+ * Tensor conventions (reference src/tensor/mod.rs:79-89, src/inference.rs:
+ * 23728-23749): a weight is `rows` output rows of `cols` contraction values,
+ * row-major in whole blocks; row o occupies wire bytes
+ * [o*row_bytes, (o+1)*row_bytes) with row_bytes = cols/block_values*block_bytes.
+ * Activations: int8 quants q[n_tokens*cols], f32 scales s[n_tokens*cols/32]
+ * (Q8_0 family) or s[n_tokens*cols/256] (Q8_K, for Q4_K/Q6_K weights), token
+ * major.  Outputs: f32 out[t*rows + row] (reference src/cuda_resident.rs:4442).
+ */
+#ifndef CAMELID_HIP_H
+#define CAMELID_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Weight formats: the GGUF tensor type ids (reference src/gguf/reader.rs:94-127). */
+#define CML_Q4_0 2
+#define CML_Q8_0 8
+#define CML_Q4_K 12
+#define CML_Q6_K 14
+
+/* Status codes. */
+#define CML_OK 0
+#define CML_ERR_UNAVAILABLE 1 /* no usable GPU / not initialised / masked by env */
+#define CML_ERR_INVALID 2     /* null pointer, bad format id, bad flag */
+#define CML_ERR_SHAPE 3       /* sizes do not fit the format or each other */
+#define CML_ERR_HIP 4         /* a HIP runtime call failed */
+#define CML_ERR_OOM 5         /* device allocation failed */
+#define CML_ERR_UNSUPPORTED 6 /* valid request this build does not serve */
+
+typedef struct cml_weight cml_weight; /* opaque device-resident weight */
+typedef void *cml_stream_t;           /* hipStream_t */
+
+/* ---- lifecycle (reference src/cuda.rs:167-236, :691-699, :350-358) ------- */
+
+/* 1 when a gfx950 device can be used.  Honours HIP_VISIBLE_DEVICES /
+ * ROCR_VISIBLE_DEVICES / CAMELID_HIP=0 masking before touching the driver
+ * (reference devices_masked_by_env, src/cuda.rs:206-218). */
+int cml_available(void);
+/* Select the device (CAMELID_HIP_DEVICE overrides when device < 0). Idempotent. */
+int cml_init(int device);
+void cml_shutdown(void);
+/* Message for the last non-zero status returned to this thread ("" if none). */
+const char *cml_last_error(void);
+/* Number of gemv/gemm launches completed by this process: proves the device
+ * lane ran (reference cuda_q8_run_count, src/cuda.rs:350-358). */
+uint64_t cml_run_count(void);
+/* Block geometry helpers: 0 for an unknown format. */
+int cml_block_values(int fmt);
+int cml_block_bytes(int fmt);
+
+/* ---- device memory plumbing for hosts without their own HIP bindings ----- */
+int cml_dev_alloc(size_t nbytes, void **out_dev);
+int cml_dev_free(void *ptr_dev);
+int cml_memcpy_h2d(void *dst_dev, const void *src_host, size_t nbytes, cml_stream_t stream);
+int cml_memcpy_d2h(void *dst_host, const void *src_dev, size_t nbytes, cml_stream_t stream);
+int cml_memset_dev(void *dst_dev, int value, size_t nbytes, cml_stream_t stream);
+int cml_stream_sync(cml_stream_t stream);
+
+/* ---- weights (reference repack_for_lane + set_layer_located,
+ *      src/cuda_resident.rs:9838, :16133-16253) ---------------------------- */
+
+/* Copy `nbytes` of GGUF wire bytes (host memory) to the device.  Q4_K keeps
+ * the on-disk block layout; Q8_0, Q4_0 and Q6_K are re-laid at load time into
+ * per-field planes of exactly the same total size (quants | scales, or
+ * ql | qh | scales | d) so that every device load is a naturally aligned
+ * 128-bit load.  The re-layout is a pure permutation of bytes:
+ * cml_weight_download returns the original wire bytes. */
+int cml_weight_upload(int fmt, int64_t rows, int64_t cols, const void *wire_host, size_t nbytes,
+                      cml_weight **out);
+/* Same, from wire bytes that already live in device memory. */
+int cml_weight_upload_dev(int fmt, int64_t rows, int64_t cols, const void *wire_dev, size_t nbytes,
+                          cml_stream_t stream, cml_weight **out);
+/* A view of rows [row_start, row_start+rows) of `parent`: the expert band of a
+ * stacked expert tensor (reference matvec_q8k_rows, src/gemma4_runtime.rs:
+ * 1084-1110).  The parent must outlive the view. */
+int cml_weight_slice(const cml_weight *parent, int64_t row_start, int64_t rows, cml_weight **out);
+int cml_weight_info(const cml_weight *w, int *fmt, int64_t *rows, int64_t *cols, size_t *wire_bytes);
+/* Reconstruct the GGUF wire bytes of `w` (a view yields its rows only). */
+int cml_weight_download(const cml_weight *w, void *wire_host, size_t nbytes);
+void cml_weight_free(cml_weight *w);
+
+/* ---- activation quantizers (reference quantize_q8_0_block,
+ *      src/inference.rs:22510-22528; quantize_q8_k_blocks, :23121-23152;
+ *      device lane launch_quantize / launch_quantize_q8k,
+ *      src/cuda_resident.rs:9935, :11761) ---------------------------------- */
+int cml_quantize_q8_0(const float *x_dev, int64_t n_tokens, int64_t cols, int8_t *q_dev,
+                      float *scales_dev, cml_stream_t stream);
+int cml_quantize_q8_k(const float *x_dev, int64_t n_tokens, int64_t cols, int8_t *q_dev,
+                      float *d_dev, cml_stream_t stream);
+
+/* ---- dequantize (reference Q4KBlock::dequantize & siblings,
+ *      src/tensor/mod.rs:5365-5409, :5547-5572, :5903-5924, :6039-6066) ----- */
+/* out_dev: f32[rows*cols], bit-identical to the reference decoders. */
+int cml_dequantize(const cml_weight *w, float *out_dev, cml_stream_t stream);
+
+/* ---- matvec / small-batch matmul (reference dispatch_gemv,
+ *      src/cuda_resident.rs:11370; dispatch_gemm_batched, :11550; CPU
+ *      semantics WireQuant::matvec_q / matvec_q8k / matmul_q / matmul_q8k,
+ *      src/gemma4_runtime.rs:922-1150) ------------------------------------- */
+/* One activation row.  residual_dev may be NULL; when given,
+ * out[row] = dot + residual[row] (reference q8_gemv fused residual,
+ * src/cuda_resident.rs:334-413). */
+int cml_gemv(const cml_weight *w, const int8_t *q_dev, const float *scales_dev, float *out_dev,
+             const float *residual_dev, cml_stream_t stream);
+/* n_tokens activation rows against one pass over the weight;
+ * out_dev[t*rows + row].  Every cell equals the cml_gemv result for that
+ * token bit for bit. */
+int cml_gemm(const cml_weight *w, const int8_t *q_dev, const float *scales_dev, int64_t n_tokens,
+             float *out_dev, cml_stream_t stream);
+/* The exact per-block integer dot products of cml_gemv, for parity checks:
+ * Q8_0/Q4_0 int32[rows][cols/32]; Q4_K int32[rows][cols/256][2] =
+ * {sum_g sc_g*dot_g, sum_g m_g*bsum_g}; Q6_K int32[rows][cols/256]. */
+int cml_block_dots(const cml_weight *w, const int8_t *q_dev, int32_t *ints_dev, cml_stream_t stream);
+
+/* f32 activations in, f32 out: quantize (Q8_0 or Q8_K by weight family) into
+ * the caller's workspace, then gemv/gemm (reference WireQuant::matvec,
+ * src/gemma4_runtime.rs:826-856).  workspace_dev needs
+ * cml_matmul_workspace_bytes(fmt, cols, n_tokens) bytes. */
+size_t cml_matmul_workspace_bytes(int fmt, int64_t cols, int64_t n_tokens);
+int cml_matmul_f32(const cml_weight *w, const float *x_dev, int64_t n_tokens, float *out_dev,
+                   void *workspace_dev, size_t workspace_bytes, cml_stream_t stream);
+
+/* ---- mixture of experts (reference softmax_top_k, src/inference.rs:
+ *      13940-13991; mixtral_moe_ffn, :14142-14280; routed launchers,
+ *      src/cuda_resident.rs:12215-12508; moe_weighted_sum_*, :6347-6389) ---- */
+/* Mixtral routing on the device: for each token the top-k experts by logit
+ * (ties to the lower index), softmax over the selected, renormalised, sorted
+ * by weight.  idx_dev int32[n_tokens*k], weight_dev f32[n_tokens*k]. */
+int cml_moe_route_top_k(const float *logits_dev, int64_t n_tokens, int n_experts, int k,
+                        int32_t *idx_dev, float *weight_dev, cml_stream_t stream);
+/* Whole expert FFN for quantized stacked experts: gate/up hold n_experts*ff
+ * rows of `hidden` values, down holds n_experts*hidden rows of `ff` values.
+ * For every token, in routed order: y = down_e(silu(gate_e x) * up_e x),
+ * out += y * weight.  Tokens that share an expert are grouped so each touched
+ * expert matrix is streamed once.  x_dev/out_dev: f32[n_tokens*hidden];
+ * idx/weight as produced by cml_moe_route_top_k.  workspace_dev needs
+ * cml_moe_workspace_bytes(...) bytes. */
+size_t cml_moe_workspace_bytes(int fmt, int64_t hidden, int64_t ff, int64_t n_tokens, int k,
+                               int n_experts);
+int cml_moe_ffn(const cml_weight *gate, const cml_weight *up, const cml_weight *down, int n_experts,
+                int k, const int32_t *idx_dev, const float *weight_dev, const float *x_dev,
+                int64_t n_tokens, float *out_dev, void *workspace_dev, size_t workspace_bytes,
+                cml_stream_t stream);
+
+/* ---- host-slice seam (reference try_q8_0_encoded_linear_rows,
+ *      src/cuda.rs:1044-1218): everything in host memory, synchronous.
+ *      Returns 0 when the device produced `output`, non-zero when the caller
+ *      must run its CPU path.  Weights are cached on the device keyed by
+ *      (pointer, length), so they must stay alive and unchanged. ------------ */
+int cml_try_linear_rows(int fmt, const float *input_scales, const int8_t *input_quants,
+                        const uint8_t *weight_wire, size_t weight_nbytes, int64_t input_rows,
+                        int64_t weight_rows, int64_t cols, float *output);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,290 @@
+"""GPU parity: the HIP path against the CPU oracle on the same seeded inputs,
+through the C ABI.
+
+Bars: activation quantization, per-block integer dots and dequantized weights
+bit-exact; final f32 within max-relative error 1e-5 (|x-y| / max(|y|, 1), the
+reference's own metric) of every accumulation order the reference has, and
+bit-exact against the order each kernel follows when no K-split is in play.
+"""
+import ctypes as C
+import json
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from camelid_amd import binding as B
+from camelid_amd.binding import DeviceBuffer, Weight, check, lib
+from tests import gpu_util as G
+
+pytestmark = pytest.mark.gpu
+
+FMTS = [("Q8_0", B.CML_Q8_0), ("Q4_0", B.CML_Q4_0), ("Q4_K", B.CML_Q4_K), ("Q6_K", B.CML_Q6_K)]
+TOL = 1e-5
+
+# The accumulation order a kernel follows bit for bit (when it does not split K).
+EXACT_ORDER = {B.CML_Q8_0: oracle.ORDER_PRIMARY, B.CML_Q4_0: oracle.ORDER_PRIMARY,
+               B.CML_Q4_K: oracle.ORDER_PRIMARY, B.CML_Q6_K: oracle.ORDER_ALT}
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _init():
+    assert lib().cml_available() == 1, "a GPU node is present but libcamelid_hip cannot use it"
+    B.init(0)
+    yield
+
+
+def check_outputs(fmt, wire, cols, x_scales, x_q, got, row_start=0, rows=None, expect_exact=True):
+    for order in (oracle.ORDER_PRIMARY, oracle.ORDER_ALT):
+        if order == oracle.ORDER_ALT and not G.is_k(fmt):
+            continue
+        want = oracle.matmul_q(fmt, wire, cols, x_scales, x_q, order=order, row_start=row_start, rows=rows, threads=8)
+        err = G.max_rel(got, want)
+        assert err <= TOL, f"order {order}: max rel err {err}"
+        if expect_exact and order == EXACT_ORDER[fmt]:
+            assert G.same_bits(got, want), f"not bit-identical to reference order {order}"
+
+
+# ----------------------------------------------------------- quantizers ----
+
+def _activation_cases(cols, rng):
+    x = rng.standard_normal((6, cols)).astype(np.float32)
+    x[1] *= 1e-3
+    x[2] *= 50.0
+    x[3, :cols // 2] = 0.0          # all-zero blocks
+    x[4] = np.round(x[4] * 4) / 4   # many exact ties after scaling
+    x[5, ::7] = -x[5, ::7]
+    return x
+
+
+def test_quantize_q8_0_bit_exact():
+    rng = np.random.default_rng(100)
+    for cols in (32, 2048, 3072, 4096 + 32):
+        G.say(f"quantize_q8_0 cols={cols}")
+        x = _activation_cases(cols, rng)
+        # exact .5 ties: amax = 127 makes the inverse scale 1.0
+        x[0, :32] = 0.0
+        x[0, 0] = 127.0
+        x[0, 1:7] = [2.5, 0.5, -0.5, -2.5, 1.5, -1.5]
+        s, q = G.gpu_quantize(False, x)
+        so, qo = oracle.quantize_q8_0(x)
+        assert np.array_equal(s.view(np.uint32), so.view(np.uint32))
+        assert np.array_equal(q, qo)
+    assert list(q[0, :7]) == [127, 3, 1, -1, -3, 2, -2]
+
+
+def test_quantize_q8_k_bit_exact():
+    rng = np.random.default_rng(101)
+    for cols in (256, 3072, 4096, 14336):
+        G.say(f"quantize_q8_k cols={cols}")
+        x = _activation_cases(cols, rng)
+        x[0, :256] = 0.0
+        x[0, 5], x[0, 9] = 3.0, -3.0   # equal magnitudes: the first one sets the sign
+        x[0, 17:21] = [1.5 * 3 / 127, 2.5 * 3 / 127, -0.5 * 3 / 127, 0.5 * 3 / 127]
+        d, q = G.gpu_quantize(True, x)
+        do, qo = oracle.quantize_q8_k(x)
+        assert np.array_equal(d.view(np.uint32), do.view(np.uint32))
+        assert np.array_equal(q, qo)
+    assert q[0, 5] == -127 and q[0, 9] == 127
+
+
+# ------------------------------------------------- layout and dequantize ----
+
+@pytest.mark.parametrize("name,fmt", FMTS)
+def test_relayout_is_a_pure_permutation(name, fmt):
+    rng = np.random.default_rng(110 + fmt)
+    bv = oracle.block_values(fmt)
+    for rows, cols in ((1, bv), (7, 3 * bv), (33, 8 * bv), (130, 5 * bv)):
+        G.say(f"relayout {name} {rows}x{cols}")
+        wire = rng.integers(0, 256, size=rows * oracle.row_bytes(fmt, cols), dtype=np.uint8)
+        w = Weight.upload(fmt, rows, cols, wire)
+        assert np.array_equal(w.download(), wire)
+        if rows > 4:
+            band = w.slice(2, rows - 3)
+            rb = oracle.row_bytes(fmt, cols)
+            assert np.array_equal(band.download(), wire[2 * rb:(rows - 1) * rb])
+
+
+@pytest.mark.parametrize("name,fmt", FMTS)
+def test_dequantize_bit_exact_golden_and_random(name, fmt):
+    gold = os.path.join(os.path.dirname(__file__), "golden", "dequant", f"{name}.json")
+    fx = json.load(open(gold))
+    wire = np.frombuffer(bytes.fromhex(fx["quant_hex"]), dtype=np.uint8)
+    ref = np.array([int(v, 16) if isinstance(v, str) else int(v) for v in fx["ref_f32_bits"]], dtype=np.uint32)
+    G.say(f"dequantize golden {name}")
+    w = Weight.upload(fmt, 1, fx["n_elements"], wire)
+    assert np.array_equal(G.gpu_dequant(w).view(np.uint32), ref)
+    rng = np.random.default_rng(120 + fmt)
+    rows, cols = 37, 4 * oracle.block_values(fmt)
+    wire = G.synth_weight(fmt, rows, cols, seed=120 + fmt)
+    # also arbitrary scale/min bytes, not only what the quantizer emits
+    wire2 = rng.integers(0, 256, size=wire.size, dtype=np.uint8)
+    bb = oracle.block_bytes(fmt)
+    d_off = {B.CML_Q8_0: [0], B.CML_Q4_0: [0], B.CML_Q4_K: [0, 2], B.CML_Q6_K: [208]}[fmt]
+    w2 = wire2.reshape(-1, bb)
+    w1 = wire.reshape(-1, bb)
+    for off in d_off:
+        w2[:, off:off + 2] = w1[:, off:off + 2]  # keep finite f16 scales
+    for wr in (wire, wire2):
+        G.say(f"dequantize random {name}")
+        w = Weight.upload(fmt, rows, cols, wr)
+        got = G.gpu_dequant(w)
+        assert np.array_equal(got.view(np.uint32), oracle.dequant(fmt, wr).view(np.uint32))
+
+
+# ------------------------------------------------------- integer block dots ----
+
+@pytest.mark.parametrize("name,fmt", FMTS)
+def test_block_dots_bit_exact(name, fmt):
+    rng = np.random.default_rng(130 + fmt)
+    bv = oracle.block_values(fmt)
+    for rows, cols in ((5, bv), (67, 6 * bv), (129, 16 * bv)):
+        G.say(f"block_dots {name} {rows}x{cols}")
+        wire = rng.integers(0, 256, size=rows * oracle.row_bytes(fmt, cols), dtype=np.uint8)
+        q = rng.integers(-128, 128, size=cols).astype(np.int8)
+        w = Weight.upload(fmt, rows, cols, wire)
+        got = G.gpu_block_dots(w, q)
+        want = oracle.block_ints(fmt, wire, cols, q)
+        assert np.array_equal(got, want)
+
+
+# ------------------------------------------------------------------- gemv ----
+
+SMALL_SHAPES = {
+    B.CML_Q8_0: [(1, 32), (9, 64), (130, 2048), (2049, 57 * 32), (513, 96 * 32)],
+    B.CML_Q4_0: [(1, 32), (9, 64), (130, 2048), (2049, 57 * 32), (513, 96 * 32)],
+    B.CML_Q4_K: [(1, 256), (9, 512), (130, 4096), (2049, 5 * 256), (300, 56 * 256)],
+    B.CML_Q6_K: [(1, 256), (9, 512), (130, 3072), (2049, 5 * 256), (300, 56 * 256)],
+}
+
+
+@pytest.mark.parametrize("name,fmt", FMTS)
+def test_gemv_matches_oracle_small_and_ragged(name, fmt):
+    rng = np.random.default_rng(140 + fmt)
+    for rows, cols in SMALL_SHAPES[fmt]:
+        G.say(f"gemv {name} {rows}x{cols}")
+        wire = G.synth_weight(fmt, rows, cols, seed=rows * 7 + cols)
+        x = rng.standard_normal(cols).astype(np.float32)
+        s, q = oracle.quantize_activation(fmt, x)
+        w = Weight.upload(fmt, rows, cols, wire)
+        with G.env(CAMELID_HIP_EXACT_ORDER="1"):
+            got = G.gpu_gemm(w, s, q)
+        check_outputs(fmt, wire, cols, s, q, got, expect_exact=True)
+        got = G.gpu_gemm(w, s, q)  # default K-split policy: tolerance only
+        check_outputs(fmt, wire, cols, s, q, got, expect_exact=False)
+
+
+def test_q4k_gemv_every_configuration_agrees():
+    rng = np.random.default_rng(150)
+    rows, cols = 301, 56 * 256
+    wire = G.synth_weight(B.CML_Q4_K, rows, cols, seed=150)
+    x = rng.standard_normal(cols).astype(np.float32)
+    s, q = oracle.quantize_activation(B.CML_Q4_K, x)
+    w = Weight.upload(B.CML_Q4_K, rows, cols, wire)
+    for lps in (8, 4):
+        for ks in (1, 2, 4):
+            G.say(f"gemv Q4_K lanes={lps} ksplit={ks}")
+            with G.env(CAMELID_HIP_Q4K_LPS=lps, CAMELID_HIP_Q4K_KSPLIT=ks):
+                got = G.gpu_gemm(w, s, q)
+                ints = G.gpu_block_dots(w, q)
+            check_outputs(B.CML_Q4_K, wire, cols, s, q, got, expect_exact=(ks == 1))
+            assert np.array_equal(ints, oracle.block_ints(B.CML_Q4_K, wire, cols, q))
+
+
+@pytest.mark.parametrize("name,fmt", FMTS)
+def test_gemv_residual_and_band_view(name, fmt):
+    rng = np.random.default_rng(160 + fmt)
+    rows, cols = 96, 4 * oracle.block_values(fmt) * (2 if not G.is_k(fmt) else 1)
+    wire = G.synth_weight(fmt, rows, cols, seed=160 + fmt)
+    x = rng.standard_normal(cols).astype(np.float32)
+    s, q = oracle.quantize_activation(fmt, x)
+    w = Weight.upload(fmt, rows, cols, wire)
+    G.say(f"gemv residual {name}")
+    res = rng.standard_normal(rows).astype(np.float32)
+    with G.env(CAMELID_HIP_EXACT_ORDER="1"):
+        base = G.gpu_gemm(w, s, q)
+        got = G.gpu_gemm(w, s, q, residual=res)
+        assert G.same_bits(got, (base + res).astype(np.float32))
+        G.say(f"gemv band view {name}")
+        band = w.slice(24, 40)   # rows 24..63: an expert band of a stacked tensor
+        got = G.gpu_gemm(band, s, q)
+    assert G.same_bits(got, base[24:64])
+    check_outputs(fmt, wire, cols, s, q, got, row_start=24, rows=40, expect_exact=True)
+
+
+# ------------------------------------------------------------- batched ----
+
+@pytest.mark.parametrize("name,fmt", FMTS)
+def test_gemm_cells_are_bitwise_the_gemv(name, fmt):
+    rng = np.random.default_rng(170 + fmt)
+    rows, cols = 257, (4096 if G.is_k(fmt) else 2048)
+    wire = G.synth_weight(fmt, rows, cols, seed=170 + fmt)
+    w = Weight.upload(fmt, rows, cols, wire)
+    for n in (2, 3, 4, 7, 8, 13, 16):
+        G.say(f"gemm {name} n={n}")
+        x = rng.standard_normal((n, cols)).astype(np.float32)
+        s, q = oracle.quantize_activation(fmt, x)
+        got = G.gpu_gemm(w, s, q)   # default K-split policy (a function of the weight shape only)
+        for t in range(n):
+            assert G.same_bits(got[t], G.gpu_gemm(w, s[t], q[t])), f"token {t}"
+        check_outputs(fmt, wire, cols, s, q, got, expect_exact=False)
+        with G.env(CAMELID_HIP_EXACT_ORDER="1"):
+            got = G.gpu_gemm(w, s, q)
+        check_outputs(fmt, wire, cols, s, q, got, expect_exact=True)
+
+
+@pytest.mark.parametrize("name,fmt", FMTS)
+def test_matmul_f32_is_quantize_then_gemm(name, fmt):
+    rng = np.random.default_rng(180 + fmt)
+    rows, cols = 190, (3072 if G.is_k(fmt) else 2048)
+    wire = G.synth_weight(fmt, rows, cols, seed=180 + fmt)
+    w = Weight.upload(fmt, rows, cols, wire)
+    for n in (1, 4):
+        G.say(f"matmul_f32 {name} n={n}")
+        x = rng.standard_normal((n, cols)).astype(np.float32)
+        with G.env(CAMELID_HIP_EXACT_ORDER="1"):
+            got = G.gpu_matmul_f32(w, x)
+        want = oracle.matmul(fmt, wire, cols, x, order=EXACT_ORDER[fmt], threads=8)
+        assert G.same_bits(got, want)
+
+
+# ----------------------------------------------------- errors and the seam ----
+
+def test_error_paths_return_status_codes():
+    L = lib()
+    h = C.c_void_p()
+    wire = np.zeros(144 * 3, np.uint8)
+    assert L.cml_weight_upload(12, 3, 256, wire.ctypes.data, 100, C.byref(h)) == 3     # wrong byte count
+    assert b"expected" in L.cml_last_error()
+    assert L.cml_weight_upload(12, 3, 250, wire.ctypes.data, wire.nbytes, C.byref(h)) == 3  # cols not whole blocks
+    assert L.cml_weight_upload(7, 3, 256, wire.ctypes.data, wire.nbytes, C.byref(h)) == 2   # unknown format
+    w = Weight.upload(12, 3, 256, wire)
+    assert L.cml_weight_slice(w.handle, 2, 5, C.byref(h)) == 3
+    assert L.cml_gemv(w.handle, None, None, None, None, None) == 2
+    empty = Weight.upload(12, 0, 256, np.zeros(0, np.uint8))   # zero rows: accepted, nothing to do
+    assert L.cml_gemv(empty.handle, None, None, None, None, None) == 0
+    d = DeviceBuffer(64)
+    assert L.cml_quantize_q8_k(d.ptr, 1, 100, d.ptr, d.ptr, None) == 3
+
+
+@pytest.mark.parametrize("name,fmt", FMTS)
+def test_host_slice_seam(name, fmt):
+    rng = np.random.default_rng(190 + fmt)
+    rows, cols, n = 77, (1024 if G.is_k(fmt) else 512), 3
+    wire = G.synth_weight(fmt, rows, cols, seed=190 + fmt)
+    x = rng.standard_normal((n, cols)).astype(np.float32)
+    s, q = oracle.quantize_activation(fmt, x)
+    out = np.full((n, rows), np.nan, np.float32)
+    before = lib().cml_run_count()
+    G.say(f"try_linear_rows {name}")
+    for _ in range(2):  # second call hits the device weight cache
+        with G.env(CAMELID_HIP_EXACT_ORDER="1"):
+            rc = lib().cml_try_linear_rows(fmt, s.ctypes.data, q.ctypes.data, wire.ctypes.data, wire.nbytes, n, rows,
+                                           cols, out.ctypes.data)
+        assert rc == 0, lib().cml_last_error()
+        assert G.same_bits(out, oracle.matmul_q(fmt, wire, cols, s, q, order=EXACT_ORDER[fmt]))
+    assert lib().cml_run_count() >= before + 2
+    bad = lib().cml_try_linear_rows(fmt, s.ctypes.data, q.ctypes.data, wire.ctypes.data, wire.nbytes - 1, n, rows,
+                                    cols, out.ctypes.data)
+    assert bad != 0
