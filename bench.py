@@ -1,0 +1,232 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized matvec hot path on one MI355X.
+
+A "step" is one call of the f32-in / f32-out operator (cml_matmul_f32:
+activation quantize + fused dequantize-matvec) on a device-resident weight.
+Inputs are synthetic: seeded N(0, 0.02) weights quantized with the host
+quantizer, seeded N(0, 1) activations.  Consecutive steps rotate over enough
+distinct copies of the weight that neither L2 nor the 256 MB Infinity Cache can
+serve it, so the weight really streams from HBM (decode over a whole model
+behaves that way); a cache-warm figure is reported beside it.
+
+Prints one JSON line (see --help for the knobs).  The timed regions are HIP
+events recorded on the stream the kernels run on; steps are replayed from a
+captured graph so the GPU, not the Python launch loop, sets the pace.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+from camelid_amd import binding as B  # noqa: E402
+from camelid_amd.binding import DeviceBuffer, Weight, check, lib  # noqa: E402
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+# name -> (format, rows, cols, tokens): BASELINE.json's configurations.
+CONFIGS = {
+    "q4k_14336x4096_n1": ("Q4_K", 14336, 4096, 1),   # the metric's configuration (Llama-3-8B FFN gate/up)
+    "q4k_4096x14336_n1": ("Q4_K", 4096, 14336, 1),   # FFN down
+    "q8_0_8192x2048_n1": ("Q8_0", 8192, 2048, 1),
+    "q6k_128256x3072_n1": ("Q6_K", 128256, 3072, 1),
+    "q4_0_128256x3072_n1": ("Q4_0", 128256, 3072, 1),
+    "q4k_14336x4096_n4": ("Q4_K", 14336, 4096, 4),
+    "q4k_14336x4096_n8": ("Q4_K", 14336, 4096, 8),
+    "q4k_14336x4096_n16": ("Q4_K", 14336, 4096, 16),
+    "q4k_14336x4096_n64": ("Q4_K", 14336, 4096, 64),
+}
+
+
+def synth_weight(fmt: int, rows: int, cols: int, seed: int) -> np.ndarray:
+    L = lib()
+    rb = cols // L.cml_block_values(fmt) * L.cml_block_bytes(fmt)
+    out = np.empty(rows * rb, np.uint8)
+    rng = np.random.default_rng(seed)
+    step = max(1, (1 << 24) // cols)
+    threads = min(16, os.cpu_count() or 1)
+    for r0 in range(0, rows, step):
+        r1 = min(rows, r0 + step)
+        w = rng.standard_normal((r1 - r0, cols), dtype=np.float32) * np.float32(0.02)
+        out[r0 * rb:r1 * rb] = B.quantize_weights(fmt, w, threads=threads)
+    return out
+
+
+class Timer:
+    def __init__(self, stream):
+        self.stream = stream
+        self.e0, self.e1 = C.c_void_p(), C.c_void_p()
+        check(lib().cml_event_create(C.byref(self.e0)))
+        check(lib().cml_event_create(C.byref(self.e1)))
+
+    def start(self):
+        check(lib().cml_event_record(self.e0, self.stream))
+
+    def stop_ms(self) -> float:
+        check(lib().cml_event_record(self.e1, self.stream))
+        ms = C.c_float()
+        check(lib().cml_event_elapsed_ms(self.e0, self.e1, C.byref(ms)))
+        return float(ms.value)
+
+
+def capture(stream, fn, count: int):
+    """Capture `count` calls of fn(i) on `stream` into one replayable graph."""
+    L = lib()
+    check(L.cml_graph_begin_capture(stream), "begin capture")
+    for i in range(count):
+        fn(i)
+    g = C.c_void_p()
+    check(L.cml_graph_end_capture(stream, C.byref(g)), "end capture")
+    return g
+
+
+def time_graph(stream, graph, timer: Timer, replays: int = 1) -> float:
+    L = lib()
+    check(L.cml_stream_sync(stream))
+    timer.start()
+    for _ in range(replays):
+        check(L.cml_graph_launch(graph, stream))
+    return timer.stop_ms()
+
+
+def cpu_baseline(fmt: int, wire: np.ndarray, rows: int, cols: int, x: np.ndarray, alg_bytes: int, budget_s: float):
+    """The CPU path, restated (oracle/): same weight, same activation, on the host cores."""
+    import oracle  # test infrastructure; used here only as the timed CPU baseline
+    threads = min(16, os.cpu_count() or 1)
+    order = oracle.ORDER_PRIMARY
+    oracle.matmul(fmt, wire, cols, x, order=order, threads=threads)  # warm-up
+    times = []
+    t_end = time.perf_counter() + budget_s
+    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 200):
+        t0 = time.perf_counter()
+        oracle.matmul(fmt, wire, cols, x, order=order, threads=threads)
+        times.append(time.perf_counter() - t0)
+    med = float(np.median(times))
+    return {
+        "value": round(alg_bytes / med / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+        "us_per_call": round(med * 1e6, 1),
+        "sample": f"{len(times)} full calls of the same {rows}x{cols} matvec (quantize + row dots), median",
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--config", default="q4k_14336x4096_n1", choices=sorted(CONFIGS))
+    ap.add_argument("--copies", type=int, default=0, help="distinct weight copies to rotate over (0 = enough for ~600 MB)")
+    ap.add_argument("--cpu-seconds", type=float, default=10.0, help="time budget of the CPU baseline leg (0 = skip)")
+    ap.add_argument("--seed", type=int, default=1234)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this path has no collectives and every box here has one GPU; "
+              f"--gpus {args.gpus} is not supported", file=sys.stderr)
+        return 2
+
+    L = lib()
+    if L.cml_available() != 1:
+        print("no usable gfx950 device: " + L.cml_last_error().decode(), file=sys.stderr)
+        return 3
+    B.init(0)
+    fmt_name, rows, cols, n = CONFIGS[args.config]
+    fmt = B.FORMATS[fmt_name]
+    K, W = max(1, args.steps), max(0, args.warmup)
+
+    wire = synth_weight(fmt, rows, cols, args.seed)
+    x = np.random.default_rng(args.seed + 1).standard_normal((n, cols)).astype(np.float32)
+    copies = args.copies or max(2, min(32, -(-600_000_000 // wire.nbytes)))
+    weights = [Weight.upload(fmt, rows, cols, wire) for _ in range(copies)]
+    alg_bytes = wire.nbytes + 4 * cols * n + 4 * rows * n
+
+    stream = C.c_void_p()
+    check(L.cml_stream_create(C.byref(stream)))
+    xd = DeviceBuffer.from_numpy(x)
+    ws_bytes = L.cml_matmul_workspace_bytes(fmt, cols, n)
+    ws = DeviceBuffer(ws_bytes)
+    out = DeviceBuffer(n * rows * 4)
+    timer = Timer(stream)
+
+    def step(i):
+        check(L.cml_matmul_f32(weights[i % copies].handle, xd.ptr, n, out.ptr, ws.ptr, ws_bytes, stream), "cml_matmul_f32")
+
+    # warm-up (eager), then the timed region: exactly K steps replayed from one graph
+    for i in range(W):
+        step(i)
+    check(L.cml_stream_sync(stream))
+    g_steps = capture(stream, step, K)
+    time_graph(stream, g_steps, timer)  # one untimed replay settles clocks and code caches
+    ms_total = min(time_graph(stream, g_steps, timer) for _ in range(3))
+    ms_per_step = ms_total / K
+    # the same K steps launched one by one from Python, for the record
+    check(L.cml_stream_sync(stream))
+    t0 = time.perf_counter()
+    for i in range(K):
+        step(i)
+    check(L.cml_stream_sync(stream))
+    eager_us = (time.perf_counter() - t0) / K * 1e6
+
+    # dominant kernel alone: the gemv/gemm on already quantized activations
+    per = 256 if fmt_name in ("Q4_K", "Q6_K") else 32
+    qd = DeviceBuffer(n * cols)
+    sd = DeviceBuffer(n * (cols // per) * 4)
+    quant = L.cml_quantize_q8_k if per == 256 else L.cml_quantize_q8_0
+    check(quant(xd.ptr, n, cols, qd.ptr, sd.ptr, stream))
+
+    def gemv_cold(i):
+        check(L.cml_gemm(weights[i % copies].handle, qd.ptr, sd.ptr, n, out.ptr, stream), "cml_gemm")
+
+    def gemv_warm(i):
+        check(L.cml_gemm(weights[0].handle, qd.ptr, sd.ptr, n, out.ptr, stream), "cml_gemm")
+
+    g_cold = capture(stream, gemv_cold, K)
+    g_warm = capture(stream, gemv_warm, K)
+    time_graph(stream, g_cold, timer)
+    kern_ms = min(time_graph(stream, g_cold, timer) for _ in range(3)) / K
+    time_graph(stream, g_warm, timer)
+    warm_ms = min(time_graph(stream, g_warm, timer) for _ in range(3)) / K
+    check(L.cml_stream_sync(stream))
+    result = out.to_numpy(np.float32, (n, rows))
+    if not np.all(np.isfinite(result)):
+        print("non-finite output", file=sys.stderr)
+        return 4
+
+    achieved = alg_bytes / (kern_ms * 1e-3) / 1e9
+    line = {
+        "metric": "Q4_K matvec µs + achieved HBM GB/s (% of peak), 14336x4096, batch 1"
+                  if args.config == "q4k_14336x4096_n1" else f"{fmt_name} matvec µs + achieved HBM GB/s, {rows}x{cols}, batch {n}",
+        "value": round(alg_bytes / (ms_per_step * 1e-3) / 1e9, 2),
+        "unit": "GB/s",
+        "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": round(ms_per_step, 6),
+        "us_per_call": round(ms_per_step * 1e3, 3),
+        "pct_of_hbm_peak": round(100.0 * alg_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8 dot, f32 accumulate", "data": "synthetic",
+        "config": {"workload": args.config, "format": fmt_name, "rows": rows, "cols": cols, "tokens": n,
+                   "algorithmic_bytes_per_call": alg_bytes, "weight_copies_rotated": copies,
+                   "step": "quantize activation + fused dequantize-matvec (cml_matmul_f32), graph replay",
+                   "eager_python_us_per_call": round(eager_us, 3)},
+        "roofline": {"bound": "hbm", "kernel": f"gemv_{fmt_name.lower()} (cml_gemm on quantized activations)",
+                     "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "us_per_launch": round(kern_ms * 1e3, 3),
+                     "cache_warm_us_per_launch": round(warm_ms * 1e3, 3),
+                     "cache_warm_gbs": round(alg_bytes / (warm_ms * 1e-3) / 1e9, 2)},
+    }
+    if args.cpu_seconds > 0:
+        line["cpu_baseline"] = cpu_baseline(fmt, wire, rows, cols, x, alg_bytes, args.cpu_seconds)
+    print(json.dumps(line, ensure_ascii=False))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -19,12 +19,14 @@ EXPORTS = [
     "cml_available", "cml_init", "cml_shutdown", "cml_last_error", "cml_run_count",
     "cml_block_values", "cml_block_bytes",
     "cml_dev_alloc", "cml_dev_free", "cml_memcpy_h2d", "cml_memcpy_d2h", "cml_memset_dev", "cml_stream_sync",
+    "cml_stream_create", "cml_stream_destroy", "cml_event_create", "cml_event_record", "cml_event_elapsed_ms",
+    "cml_event_destroy", "cml_graph_begin_capture", "cml_graph_end_capture", "cml_graph_launch", "cml_graph_destroy",
     "cml_weight_upload", "cml_weight_upload_dev", "cml_weight_slice", "cml_weight_info",
     "cml_weight_download", "cml_weight_free",
     "cml_quantize_q8_0", "cml_quantize_q8_k", "cml_dequantize",
     "cml_gemv", "cml_gemm", "cml_block_dots", "cml_matmul_workspace_bytes", "cml_matmul_f32",
     "cml_moe_route_top_k", "cml_moe_workspace_bytes", "cml_moe_ffn",
-    "cml_try_linear_rows",
+    "cml_quantize_weights_host", "cml_try_linear_rows",
 ]
 
 
@@ -64,6 +66,16 @@ def lib() -> C.CDLL:
     L.cml_memcpy_d2h.argtypes = [vp, vp, sz, vp]
     L.cml_memset_dev.argtypes = [vp, i32, sz, vp]
     L.cml_stream_sync.argtypes = [vp]
+    L.cml_stream_create.argtypes = [pp]
+    L.cml_stream_destroy.argtypes = [vp]
+    L.cml_event_create.argtypes = [pp]
+    L.cml_event_record.argtypes = [vp, vp]
+    L.cml_event_elapsed_ms.argtypes = [vp, vp, C.POINTER(C.c_float)]
+    L.cml_event_destroy.argtypes = [vp]
+    L.cml_graph_begin_capture.argtypes = [vp]
+    L.cml_graph_end_capture.argtypes = [vp, pp]
+    L.cml_graph_launch.argtypes = [vp, vp]
+    L.cml_graph_destroy.argtypes = [vp]
     L.cml_weight_upload.argtypes = [i32, i64, i64, vp, sz, pp]
     L.cml_weight_upload_dev.argtypes = [i32, i64, i64, vp, sz, vp, pp]
     L.cml_weight_slice.argtypes = [vp, i64, i64, pp]
@@ -84,6 +96,7 @@ def lib() -> C.CDLL:
     L.cml_moe_workspace_bytes.argtypes = [i32, i64, i64, i64, i32, i32]
     L.cml_moe_workspace_bytes.restype = sz
     L.cml_moe_ffn.argtypes = [vp, vp, vp, i32, i32, vp, vp, vp, i64, vp, vp, sz, vp]
+    L.cml_quantize_weights_host.argtypes = [i32, vp, sz, vp, i32]
     L.cml_try_linear_rows.argtypes = [i32, vp, vp, vp, sz, i64, i64, i64, vp]
     _lib = L
     return L
@@ -186,3 +199,13 @@ class Weight:
             self.free()
         except Exception:
             pass
+
+
+def quantize_weights(fmt: int, values: np.ndarray, threads: int = 8) -> np.ndarray:
+    """f32 values (rows of whole blocks) -> GGUF wire bytes, on the host (cml_quantize_weights_host)."""
+    L = lib()
+    values = np.ascontiguousarray(values, np.float32)
+    out = np.empty(values.size // L.cml_block_values(fmt) * L.cml_block_bytes(fmt), np.uint8)
+    check(L.cml_quantize_weights_host(fmt, values.ctypes.data, values.size, out.ctypes.data, threads),
+          "cml_quantize_weights_host")
+    return out

@@ -23,6 +23,7 @@ SOURCES = [
     "gemv_q8q4.hip",
     "gemv_q6k.hip",
     "moe.hip",
+    "weight_quantize.cpp",
 ]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")

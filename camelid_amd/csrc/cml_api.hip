@@ -159,6 +159,83 @@ int cml_stream_sync(cml_stream_t stream) {
     return CML_OK;
 }
 
+int cml_stream_create(cml_stream_t *out) {
+    if (!out) return fail(CML_ERR_INVALID, "null out pointer");
+    *out = nullptr;
+    if (int rc = check_ready()) return rc;
+    hipStream_t s;
+    CML_HIP_TRY(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    *out = s;
+    return CML_OK;
+}
+
+int cml_stream_destroy(cml_stream_t stream) {
+    if (!stream) return CML_OK;
+    CML_HIP_TRY(hipStreamDestroy(as_stream(stream)));
+    return CML_OK;
+}
+
+int cml_event_create(cml_event_t *out) {
+    if (!out) return fail(CML_ERR_INVALID, "null out pointer");
+    *out = nullptr;
+    if (int rc = check_ready()) return rc;
+    hipEvent_t e;
+    CML_HIP_TRY(hipEventCreate(&e));
+    *out = e;
+    return CML_OK;
+}
+
+int cml_event_record(cml_event_t event, cml_stream_t stream) {
+    if (!event) return fail(CML_ERR_INVALID, "null event");
+    CML_HIP_TRY(hipEventRecord(static_cast<hipEvent_t>(event), as_stream(stream)));
+    return CML_OK;
+}
+
+int cml_event_elapsed_ms(cml_event_t start, cml_event_t stop, float *ms) {
+    if (!start || !stop || !ms) return fail(CML_ERR_INVALID, "null pointer");
+    CML_HIP_TRY(hipEventSynchronize(static_cast<hipEvent_t>(stop)));
+    CML_HIP_TRY(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)));
+    return CML_OK;
+}
+
+int cml_event_destroy(cml_event_t event) {
+    if (!event) return CML_OK;
+    CML_HIP_TRY(hipEventDestroy(static_cast<hipEvent_t>(event)));
+    return CML_OK;
+}
+
+int cml_graph_begin_capture(cml_stream_t stream) {
+    if (int rc = check_ready()) return rc;
+    if (!stream) return fail(CML_ERR_INVALID, "capture needs a stream created with cml_stream_create");
+    CML_HIP_TRY(hipStreamBeginCapture(as_stream(stream), hipStreamCaptureModeThreadLocal));
+    return CML_OK;
+}
+
+int cml_graph_end_capture(cml_stream_t stream, cml_graph_t *out) {
+    if (!out) return fail(CML_ERR_INVALID, "null out pointer");
+    *out = nullptr;
+    hipGraph_t graph = nullptr;
+    CML_HIP_TRY(hipStreamEndCapture(as_stream(stream), &graph));
+    hipGraphExec_t exec = nullptr;
+    hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    if (e != hipSuccess) return fail(CML_ERR_HIP, "hipGraphInstantiate failed: %s", hipGetErrorString(e));
+    *out = exec;
+    return CML_OK;
+}
+
+int cml_graph_launch(cml_graph_t graph, cml_stream_t stream) {
+    if (!graph) return fail(CML_ERR_INVALID, "null graph");
+    CML_HIP_TRY(hipGraphLaunch(static_cast<hipGraphExec_t>(graph), as_stream(stream)));
+    return CML_OK;
+}
+
+int cml_graph_destroy(cml_graph_t graph) {
+    if (!graph) return CML_OK;
+    CML_HIP_TRY(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph)));
+    return CML_OK;
+}
+
 // ---- weights ---------------------------------------------------------------------------------------
 
 static int check_weight_shape(int fmt, int64_t rows, int64_t cols, size_t nbytes, int64_t *nb_out) {

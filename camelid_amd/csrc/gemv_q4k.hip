@@ -12,16 +12,21 @@
 //
 // Mapping.  The weight stays in the GGUF wire layout: 144-byte super-blocks =
 // nine aligned 16-byte pieces (header: f16 d, f16 dmin, 12 packed 6-bit
-// scale/min bytes; then 128 nibble bytes).  LPS lanes (8 or 4) own one
-// super-block: each loads 16 (or 32) nibble bytes plus the 16-byte header with
+// scale/min bytes; then 128 nibble bytes).  LPS lanes (4 or 8) own one
+// super-block: each loads 32 (or 16) nibble bytes plus the 16-byte header with
 // 128-bit loads, unpacks in registers, and dots against the int8 activation
 // staged in LDS with v_dot4_i32_i8.  A wave therefore covers 64/LPS rows at
 // the same super-block index, so the per-row f32 chain above lives in one
 // lane and needs no cross-lane traffic; only the two integers are reduced
-// inside the lane group (DPP row_shr).  A 256-thread workgroup is 4 waves:
-// 4/KSPLIT row tiles, each tile's super-block range cut into KSPLIT contiguous
-// parts (one per wave) whose partial chains are added left to right.  With
+// inside the lane group (DPP row_shr).  A workgroup is TPW row tiles x KSPLIT
+// waves: each tile's super-block range is cut into KSPLIT contiguous parts
+// (one per wave) whose partial chains are added left to right.  With
 // KSPLIT = 1 the result is the reference's own association, bit for bit.
+//
+// The kernel is short (a 33 MB matrix streams in a few microseconds), so the
+// prologue is ordered to keep HBM busy from the first cycle: the activation
+// loads are issued first, the first weight buffer right behind them, and only
+// then is the activation written to LDS.
 //
 // NT > 1 holds the unpacked weight in registers and replays it against NT
 // activation rows in LDS: the weight is streamed once per NT tokens and every
@@ -46,12 +51,15 @@ struct Q4KArgs {
     const int32_t *band_ids;  // expert id per blockIdx.y, or null
     int64_t act_slot_stride;  // activation rows between blockIdx.y slots (0 = shared)
     int64_t out_slot_stride;  // output floats between blockIdx.y slots
-    int ksplit;               // 1, 2 or 4
+    int ksplit;               // waves sharing one row tile (1, 2, 4 or 8)
+    int tiles_per_wg;         // row tiles per workgroup; blockDim.x = 64 * ksplit * tiles_per_wg
 };
+
+constexpr int kQ4KStageRegs = 4;  // activation chunks a thread holds in registers during the prologue
 
 template <int LPS>
 struct Q4KRegs {
-    static constexpr int U = (LPS == 8) ? 4 : 2;  // super-blocks in flight per buffer
+    static constexpr int U = 4;  // super-blocks in flight per buffer
     uint4 hdr[U];
     uint4 qa[U];
     uint4 qb[U];  // LPS == 4 only
@@ -85,36 +93,56 @@ __device__ __forceinline__ uint4 hi_nibbles(const uint4 &v) {
                       (v.w >> 4) & 0x0f0f0f0fu);
 }
 
+// Per-lane constants of the scale/min extraction.  A lane works on chunk c of
+// the super-block (values 64c..64c+63: scale groups 2c and 2c+1).  With
+// sh = 16*(c&1), the pair (sc[2c], sc[2c+1]) sits in bytes 0,1 of
+//   c < 2 :  (u0 >> sh) & 0x3f3f
+//   c >= 2:  ((u2 >> sh) & 0x0f0f) | (((u0 >> sh) >> 2) & 0x3030)
+// and the pair of mins in
+//   c < 2 :  (u1 >> sh) & 0x3f3f
+//   c >= 2:  (((u2 >> sh) >> 4) & 0x0f0f) | (((u1 >> sh) >> 2) & 0x3030)
+// (u0,u1,u2 = the 12 scale bytes as little-endian words; this is the 6-bit
+// packing of reference q4_k_scale_min, src/tensor/mod.rs:5997-6006.)
+struct Q4KLane {
+    int c;       // chunk
+    int sh;      // 16 * (c & 1)
+    bool upper;  // c >= 2
+};
+
+__device__ __forceinline__ void q4k_scale_pairs(const Q4KLane &ln, const uint4 &hdr, uint32_t &sc_pair,
+                                                uint32_t &m_pair) {
+    const uint32_t a0 = hdr.y >> ln.sh, a1 = hdr.z >> ln.sh, a2 = hdr.w >> ln.sh;
+    const uint32_t sc_lo = a0 & 0x3f3fu, m_lo = a1 & 0x3f3fu;
+    const uint32_t sc_up = (a2 & 0x0f0fu) | ((a0 >> 2) & 0x3030u);
+    const uint32_t m_up = ((a2 >> 4) & 0x0f0fu) | ((a1 >> 2) & 0x3030u);
+    sc_pair = ln.upper ? sc_up : sc_lo;
+    m_pair = ln.upper ? m_up : m_lo;
+}
+
 template <int LPS, int NT, bool INTS>
-__device__ __forceinline__ void q4k_compute(const Q4KRegs<LPS> &r, int l, int sb, int s1, const int8_t *ys,
-                                            const int *bsum, const float *yds, int n_sb, float (&acc)[NT],
-                                            int32_t *ints_row) {
+__device__ __forceinline__ void q4k_compute(const Q4KRegs<LPS> &r, const Q4KLane &ln, int l, int sb, int s1,
+                                            const int8_t *ys, const int *bsum, const float *yds, int n_sb,
+                                            float (&acc)[NT], int32_t *ints_row) {
 #pragma unroll
     for (int u = 0; u < Q4KRegs<LPS>::U; u++) {
         const bool valid = sb + u < s1;  // wave-uniform
         const int i = valid ? sb + u : s1 - 1;
-        uint32_t sc03, sc47, m03, m47;
-        q4k_unpack_scales(r.hdr[u].y, r.hdr[u].z, r.hdr[u].w, sc03, sc47, m03, m47);
+        uint32_t sc_pair, m_pair;
+        q4k_scale_pairs(ln, r.hdr[u], sc_pair, m_pair);
+        const int sc_lo = sc_pair & 0xff, sc_hi = sc_pair >> 8;
         const float dw = f16_bits_to_f32(r.hdr[u].x & 0xffffu);
         const float dminw = f16_bits_to_f32(r.hdr[u].x >> 16);
-        // chunk c of the super-block: low nibbles are group 2c, high nibbles group 2c+1
-        const int c = (LPS == 8) ? (l >> 1) : l;
-        const uint32_t scw = (c < 2) ? sc03 : sc47;
-        const int sh = (c & 1) * 16;
-        const int sc_lo = (scw >> sh) & 0xff;
-        const int sc_hi = (scw >> (sh + 8)) & 0xff;
+        const int c = ln.c;
         const uint4 alo = lo_nibbles(r.qa[u]), ahi = hi_nibbles(r.qa[u]);
         uint4 blo, bhi;
         int m_a, m_b = 0;
         if constexpr (LPS == 8) {
-            const uint32_t mw = (l < 4) ? m03 : m47;
-            m_a = (mw >> ((l & 3) * 8)) & 0xff;  // lane l owns group l on the mins side
+            m_a = (l & 1) ? (m_pair >> 8) : (m_pair & 0xff);  // lane l owns group l on the mins side
         } else {
             blo = lo_nibbles(r.qb[u]);
             bhi = hi_nibbles(r.qb[u]);
-            const uint32_t mw = (c < 2) ? m03 : m47;
-            m_a = (mw >> sh) & 0xff;
-            m_b = (mw >> (sh + 8)) & 0xff;
+            m_a = m_pair & 0xff;
+            m_b = m_pair >> 8;
         }
 #pragma unroll
         for (int t = 0; t < NT; t++) {
@@ -127,7 +155,7 @@ __device__ __forceinline__ void q4k_compute(const Q4KRegs<LPS> &r, int l, int sb
                 const uint4 yhi = *reinterpret_cast<const uint4 *>(y + 64 * c + 32 + 16 * h);
                 lo = dot16(alo, ylo, 0);
                 hi = dot16(ahi, yhi, 0);
-                p = bs[l] * m_a;
+                p = __mul24(bs[l], m_a);
             } else {
                 const uint4 ylo0 = *reinterpret_cast<const uint4 *>(y + 64 * c);
                 const uint4 ylo1 = *reinterpret_cast<const uint4 *>(y + 64 * c + 16);
@@ -136,9 +164,10 @@ __device__ __forceinline__ void q4k_compute(const Q4KRegs<LPS> &r, int l, int sb
                 lo = dot16(blo, ylo1, dot16(alo, ylo0, 0));
                 hi = dot16(bhi, yhi1, dot16(ahi, yhi0, 0));
                 const int2 b2 = *reinterpret_cast<const int2 *>(bs + 2 * c);
-                p = b2.x * m_a + b2.y * m_b;
+                p = __mul24(b2.x, m_a) + __mul24(b2.y, m_b);
             }
-            int s_total = group_sum_to_last<LPS>(lo * sc_lo + hi * sc_hi);
+            // |lo|, |hi| <= 32*15*128 and the 6-bit scales keep every product inside 24 bits.
+            int s_total = group_sum_to_last<LPS>(__mul24(lo, sc_lo) + __mul24(hi, sc_hi));
             int p_total = group_sum_to_last<LPS>(p);
             s_total = valid ? s_total : 0;  // fma(x, 0, acc) leaves acc unchanged
             p_total = valid ? p_total : 0;
@@ -158,16 +187,17 @@ __device__ __forceinline__ void q4k_compute(const Q4KRegs<LPS> &r, int l, int sb
 }
 
 template <int LPS, int NT, bool INTS>
-__global__ __launch_bounds__(256) void gemv_q4k_kernel(Q4KArgs a) {
+__global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
     constexpr int RPW = kWave / LPS;  // rows per wave tile
     extern __shared__ uint4 smem[];
     const int n_sb = a.n_sb;
     int8_t *ys = reinterpret_cast<int8_t *>(smem);                     // [NT][n_sb*256]
     int *bsum = reinterpret_cast<int *>(ys + NT * n_sb * 256);         // [NT][n_sb*8]
     float *yds = reinterpret_cast<float *>(bsum + NT * n_sb * 8);      // [NT][n_sb]
-    float *part = yds + ((NT * n_sb + 3) & ~3);                        // [4 waves][NT][RPW]
+    float *part = yds + ((NT * n_sb + 3) & ~3);                        // [waves][NT][RPW]
 
     const int tid = threadIdx.x;
+    const int nthreads = blockDim.x;
     const int slot = blockIdx.y;
     const int64_t band = a.band_ids ? a.band_ids[slot] : 0;
     const uint8_t *w = a.w + band * a.rows * a.row_bytes;
@@ -175,27 +205,10 @@ __global__ __launch_bounds__(256) void gemv_q4k_kernel(Q4KArgs a) {
     const float *yd = a.yd + static_cast<int64_t>(slot) * a.act_slot_stride * n_sb;
     float *out = a.out + static_cast<int64_t>(slot) * a.out_slot_stride;
 
-    // Stage the int8 activations, their per-32 sums and their scales in LDS.
-    {
-        const uint4 *src = reinterpret_cast<const uint4 *>(q);
-        uint4 *dst = reinterpret_cast<uint4 *>(ys);
-        const int n16 = NT * n_sb * 16;  // even, so lanes 2k and 2k+1 are in or out together
-        for (int i = tid; i < n16; i += 256) {
-            const uint4 v = src[i];
-            dst[i] = v;
-            int s = bytesum16(v);
-            s += row_shr_i32<1>(s);
-            if (i & 1) bsum[i >> 1] = s;
-        }
-        for (int i = tid; i < NT * n_sb; i += 256) yds[i] = yd[i];
-    }
-    __syncthreads();
-
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int W = a.ksplit;
-    const int tiles_per_wg = 4 / W;
     const int tile_in_wg = wave / W, kpart = wave - tile_in_wg * W;
-    const int tile = blockIdx.x * tiles_per_wg + tile_in_wg;
+    const int tile = blockIdx.x * a.tiles_per_wg + tile_in_wg;
     const int s0 = static_cast<int>(static_cast<int64_t>(kpart) * n_sb / W);
     const int s1 = static_cast<int>(static_cast<int64_t>(kpart + 1) * n_sb / W);
     const int r = lane / LPS, l = lane - r * LPS;
@@ -203,6 +216,49 @@ __global__ __launch_bounds__(256) void gemv_q4k_kernel(Q4KArgs a) {
     const bool live = row < a.rows;
     const uint8_t *wrow = w + static_cast<int64_t>(live ? row : a.rows - 1) * a.row_bytes;
     const bool leader = (l == LPS - 1);
+    Q4KLane ln;
+    ln.c = (LPS == 8) ? (l >> 1) : l;
+    ln.sh = (ln.c & 1) * 16;
+    ln.upper = ln.c >= 2;
+
+    // Prologue: activation loads first, the first weight buffer right behind
+    // them, then the LDS writes -- so HBM requests are in flight while the
+    // activation is staged.
+    const uint4 *src = reinterpret_cast<const uint4 *>(q);
+    uint4 *dst = reinterpret_cast<uint4 *>(ys);
+    const int n16 = NT * n_sb * 16;  // even; blockDim is even: lanes 2k, 2k+1 are in or out together
+    uint4 sv[kQ4KStageRegs];
+#pragma unroll
+    for (int k = 0; k < kQ4KStageRegs; k++) sv[k] = src[min(tid + k * nthreads, n16 - 1)];
+    const float yd0 = yd[min(tid, NT * n_sb - 1)];
+
+    constexpr int U = Q4KRegs<LPS>::U;
+    Q4KRegs<LPS> ra, rb;
+    __builtin_amdgcn_sched_barrier(0);
+    q4k_load<LPS>(ra, wrow, l, s0, s1);
+    __builtin_amdgcn_sched_barrier(0);
+
+#pragma unroll
+    for (int k = 0; k < kQ4KStageRegs; k++) {
+        const int i = tid + k * nthreads;
+        int s = bytesum16(sv[k]);
+        s += row_shr_i32<1>(s);
+        if (i < n16) {
+            dst[i] = sv[k];
+            if (i & 1) bsum[i >> 1] = s;
+        }
+    }
+    for (int i = tid + kQ4KStageRegs * nthreads; i < n16; i += nthreads) {
+        const uint4 v = src[i];
+        dst[i] = v;
+        int s = bytesum16(v);
+        s += row_shr_i32<1>(s);
+        if (i & 1) bsum[i >> 1] = s;
+    }
+    if (tid < NT * n_sb) yds[tid] = yd0;
+    for (int i = tid + nthreads; i < NT * n_sb; i += nthreads) yds[i] = yd[i];
+    __syncthreads();
+
     int32_t *ints_row = nullptr;
     if constexpr (INTS) {
         if (a.ints && leader && live) ints_row = a.ints + (band * a.rows + row) * static_cast<int64_t>(n_sb) * 2;
@@ -212,14 +268,17 @@ __global__ __launch_bounds__(256) void gemv_q4k_kernel(Q4KArgs a) {
 #pragma unroll
     for (int t = 0; t < NT; t++) acc[t] = 0.0f;
 
-    constexpr int U = Q4KRegs<LPS>::U;
-    Q4KRegs<LPS> ra, rb;
-    q4k_load<LPS>(ra, wrow, l, s0, s1);
+    // sched_barrier keeps each buffer's loads ahead of the other buffer's
+    // arithmetic, so one buffer is always in flight under the compute.
     for (int sb = s0; sb < s1; sb += 2 * U) {
         q4k_load<LPS>(rb, wrow, l, sb + U, s1);
-        q4k_compute<LPS, NT, INTS>(ra, l, sb, s1, ys, bsum, yds, n_sb, acc, ints_row);
+        __builtin_amdgcn_sched_barrier(0);
+        q4k_compute<LPS, NT, INTS>(ra, ln, l, sb, s1, ys, bsum, yds, n_sb, acc, ints_row);
+        __builtin_amdgcn_sched_barrier(0);
         q4k_load<LPS>(ra, wrow, l, sb + 2 * U, s1);
-        q4k_compute<LPS, NT, INTS>(rb, l, sb + U, s1, ys, bsum, yds, n_sb, acc, ints_row);
+        __builtin_amdgcn_sched_barrier(0);
+        q4k_compute<LPS, NT, INTS>(rb, ln, l, sb + U, s1, ys, bsum, yds, n_sb, acc, ints_row);
+        __builtin_amdgcn_sched_barrier(0);
     }
 
     if (W == 1) {
@@ -238,11 +297,11 @@ __global__ __launch_bounds__(256) void gemv_q4k_kernel(Q4KArgs a) {
         for (int t = 0; t < NT; t++) part[(wave * NT + t) * RPW + r] = acc[t];
     }
     __syncthreads();
-    for (int i = tid; i < tiles_per_wg * NT * RPW; i += 256) {
+    for (int i = tid; i < a.tiles_per_wg * NT * RPW; i += nthreads) {
         const int rr = i % RPW;
         const int t = (i / RPW) % NT;
         const int tw = i / (RPW * NT);
-        const int orow = (blockIdx.x * tiles_per_wg + tw) * RPW + rr;
+        const int orow = (blockIdx.x * a.tiles_per_wg + tw) * RPW + rr;
         if (orow >= a.rows) continue;
         float v = part[((tw * W) * NT + t) * RPW + rr];
         for (int k = 1; k < W; k++) v = v + part[((tw * W + k) * NT + t) * RPW + rr];
@@ -251,41 +310,55 @@ __global__ __launch_bounds__(256) void gemv_q4k_kernel(Q4KArgs a) {
     }
 }
 
-int env_int(const char *name, int dflt);
+// Launch shape.  `ksplit` depends on the weight shape only, so gemv and gemm
+// give every cell the same association; 1 (the reference's own) whenever the
+// row count alone yields about one wave per SIMD (1024 on this chip).
+struct Q4KShape {
+    int lps, ksplit, tiles_per_wg;
+};
 
-// K-split policy: keep at least ~6 waves per compute unit in flight when the
-// matrix has few rows and many super-blocks; 1 (the reference's association)
-// whenever the row count alone provides them.  Depends on the weight shape
-// only, so gemv and gemm agree bit for bit.
-static int pick_ksplit(int64_t rows, int64_t n_sb, int lps) {
+static Q4KShape pick_shape(int64_t rows, int64_t n_sb) {
+    Q4KShape s;
+    s.lps = env_int("CAMELID_HIP_Q4K_LPS", 4) == 8 ? 8 : 4;
+    const int64_t tiles = (rows + (64 / s.lps) - 1) / (64 / s.lps);
+    int ks = 1;
     const int forced = env_int("CAMELID_HIP_Q4K_KSPLIT", 0);
-    if ((forced == 1 || forced == 2 || forced == 4) && forced <= n_sb) return forced;
-    if (env_int("CAMELID_HIP_EXACT_ORDER", 0)) return 1;
-    const int64_t tiles = (rows + (64 / lps) - 1) / (64 / lps);
-    if (tiles >= 1536 || n_sb < 8) return 1;
-    if (tiles * 2 >= 1536 || n_sb < 16) return 2;
-    return 4;
+    if ((forced == 1 || forced == 2 || forced == 4 || forced == 8) && forced <= n_sb) {
+        ks = forced;
+    } else if (!env_int("CAMELID_HIP_EXACT_ORDER", 0)) {
+        while (ks < 8 && tiles * ks < 768 && n_sb / (ks * 2) >= 4) ks *= 2;
+    }
+    s.ksplit = ks;
+    int tpw = env_int("CAMELID_HIP_Q4K_TILES_PER_WG", 0);
+    if (tpw < 1 || tpw * ks > 8) {
+        tpw = 1;
+        while (tpw < 4 && tpw * 2 * ks <= 8 && tiles >= 2048 * tpw) tpw *= 2;
+    }
+    s.tiles_per_wg = tpw;
+    return s;
 }
 
 template <int LPS, int NT>
-static int launch_q4k_nt(const Q4KArgs &ka, int n_bands, bool ints, hipStream_t st) {
+static int launch_q4k_nt(Q4KArgs ka, const Q4KShape &shape, int n_bands, bool ints, hipStream_t st) {
     const int rpw = 64 / LPS;
-    const int tiles_per_wg = 4 / ka.ksplit;
+    const int waves = shape.ksplit * shape.tiles_per_wg;
     const int64_t tiles = (ka.rows + rpw - 1) / rpw;
-    const unsigned gx = static_cast<unsigned>((tiles + tiles_per_wg - 1) / tiles_per_wg);
+    const unsigned gx = static_cast<unsigned>((tiles + shape.tiles_per_wg - 1) / shape.tiles_per_wg);
     const size_t lds = static_cast<size_t>(NT) * ka.n_sb * (256 + 32) + ((static_cast<size_t>(NT) * ka.n_sb + 3) & ~size_t(3)) * 4 +
-                       4 * NT * rpw * 4;
+                       static_cast<size_t>(waves) * NT * rpw * 4;
     if (lds > 64 * 1024) return fail(CML_ERR_UNSUPPORTED, "Q4_K activation of %d super-blocks x %d tokens exceeds the LDS staging limit", ka.n_sb, NT);
+    ka.ksplit = shape.ksplit;
+    ka.tiles_per_wg = shape.tiles_per_wg;
     if (ints && NT == 1)
-        hipLaunchKernelGGL((gemv_q4k_kernel<LPS, 1, true>), dim3(gx, n_bands), dim3(256), lds, st, ka);
+        hipLaunchKernelGGL((gemv_q4k_kernel<LPS, 1, true>), dim3(gx, n_bands), dim3(64 * waves), lds, st, ka);
     else
-        hipLaunchKernelGGL((gemv_q4k_kernel<LPS, NT, false>), dim3(gx, n_bands), dim3(256), lds, st, ka);
+        hipLaunchKernelGGL((gemv_q4k_kernel<LPS, NT, false>), dim3(gx, n_bands), dim3(64 * waves), lds, st, ka);
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }
 
 template <int LPS>
-static int launch_q4k_lps(const MatArgs &a, hipStream_t st) {
+static int launch_q4k_lps(const MatArgs &a, const Q4KShape &shape, hipStream_t st) {
     const cml_weight *w = a.w;
     Q4KArgs ka;
     ka.w = w->planes.p[0];
@@ -297,7 +370,6 @@ static int launch_q4k_lps(const MatArgs &a, hipStream_t st) {
     ka.band_ids = a.band_ids;
     ka.act_slot_stride = a.act_per_slot ? a.n_tokens : 0;
     ka.out_slot_stride = a.n_tokens * static_cast<int64_t>(ka.rows);
-    ka.ksplit = pick_ksplit(ka.rows, ka.n_sb, LPS);
     const int n_bands = a.n_bands > 0 ? a.n_bands : 1;
     // Tokens are served in passes of up to 8 rows of activations.
     int64_t t0 = 0;
@@ -309,10 +381,10 @@ static int launch_q4k_lps(const MatArgs &a, hipStream_t st) {
         ka.out = a.out + t0 * ka.rows;
         int rc;
         switch (nt) {
-            case 8: rc = launch_q4k_nt<LPS, 8>(ka, n_bands, false, st); break;
-            case 4: rc = launch_q4k_nt<LPS, 4>(ka, n_bands, false, st); break;
-            case 2: rc = launch_q4k_nt<LPS, 2>(ka, n_bands, false, st); break;
-            default: rc = launch_q4k_nt<LPS, 1>(ka, n_bands, a.ints != nullptr, st); break;
+            case 8: rc = launch_q4k_nt<LPS, 8>(ka, shape, n_bands, false, st); break;
+            case 4: rc = launch_q4k_nt<LPS, 4>(ka, shape, n_bands, false, st); break;
+            case 2: rc = launch_q4k_nt<LPS, 2>(ka, shape, n_bands, false, st); break;
+            default: rc = launch_q4k_nt<LPS, 1>(ka, shape, n_bands, a.ints != nullptr, st); break;
         }
         if (rc != CML_OK) return rc;
         t0 += nt;
@@ -322,8 +394,9 @@ static int launch_q4k_lps(const MatArgs &a, hipStream_t st) {
 
 int launch_gemv_q4k(const MatArgs &a, hipStream_t st) {
     if (a.w->rows == 0 || a.n_tokens == 0) return CML_OK;
-    const int lps = env_int("CAMELID_HIP_Q4K_LPS", 8);
-    return lps == 4 ? launch_q4k_lps<4>(a, st) : launch_q4k_lps<8>(a, st);
+    const int64_t rows = a.band_ids ? a.band_rows : a.w->rows;
+    const Q4KShape shape = pick_shape(rows, a.w->nb);
+    return shape.lps == 4 ? launch_q4k_lps<4>(a, shape, st) : launch_q4k_lps<8>(a, shape, st);
 }
 
 int launch_gemm_q4k(const MatArgs &a, hipStream_t st) { return launch_gemv_q4k(a, st); }

@@ -61,6 +61,8 @@ extern "C" {
 
 typedef struct cml_weight cml_weight; /* opaque device-resident weight */
 typedef void *cml_stream_t;           /* hipStream_t */
+typedef void *cml_event_t;            /* hipEvent_t */
+typedef void *cml_graph_t;            /* an instantiated hipGraphExec_t */
 
 /* ---- lifecycle (reference src/cuda.rs:167-236, :691-699, :350-358) ------- */
 
@@ -87,6 +89,23 @@ int cml_memcpy_h2d(void *dst_dev, const void *src_host, size_t nbytes, cml_strea
 int cml_memcpy_d2h(void *dst_host, const void *src_dev, size_t nbytes, cml_stream_t stream);
 int cml_memset_dev(void *dst_dev, int value, size_t nbytes, cml_stream_t stream);
 int cml_stream_sync(cml_stream_t stream);
+/* Streams (default priority), timing events and captured launch sequences, for
+ * hosts that drive a decode loop through this library alone.  The reference's
+ * resident engine owns one stream, syncs once per token and may replay a
+ * captured graph (src/cuda_resident.rs:15195-15205); these are the pieces for
+ * the same pattern.  Every matvec / matmul / quantize / mixture-of-experts entry
+ * point may be captured; uploads, downloads and cml_block_dots may not. */
+int cml_stream_create(cml_stream_t *out);
+int cml_stream_destroy(cml_stream_t stream);
+int cml_event_create(cml_event_t *out);
+int cml_event_record(cml_event_t event, cml_stream_t stream);
+/* Waits for `stop`, then returns the milliseconds between the two events. */
+int cml_event_elapsed_ms(cml_event_t start, cml_event_t stop, float *ms);
+int cml_event_destroy(cml_event_t event);
+int cml_graph_begin_capture(cml_stream_t stream);
+int cml_graph_end_capture(cml_stream_t stream, cml_graph_t *out);
+int cml_graph_launch(cml_graph_t graph, cml_stream_t stream);
+int cml_graph_destroy(cml_graph_t graph);
 
 /* ---- weights (reference repack_for_lane + set_layer_located,
  *      src/cuda_resident.rs:9838, :16133-16253) ---------------------------- */
@@ -173,6 +192,12 @@ int cml_moe_ffn(const cml_weight *gate, const cml_weight *up, const cml_weight *
                 int k, const int32_t *idx_dev, const float *weight_dev, const float *x_dev,
                 int64_t n_tokens, float *out_dev, void *workspace_dev, size_t workspace_bytes,
                 cml_stream_t stream);
+
+/* ---- weight quantizer tool (reference quantize_block_q8_0 / q4_0 / q4_k,
+ *      src/quantize.rs:98-244): f32 values -> GGUF wire bytes on the host, in
+ *      whole blocks, on `threads` threads.  Q6_K has no counterpart in the
+ *      reference; its encoder here only produces valid super-blocks. -------- */
+int cml_quantize_weights_host(int fmt, const float *src, size_t n_values, uint8_t *dst, int threads);
 
 /* ---- host-slice seam (reference try_q8_0_encoded_linear_rows,
  *      src/cuda.rs:1044-1218): everything in host memory, synchronous.

@@ -64,3 +64,13 @@ def test_env_masking_is_honoured_before_the_driver():
             "print(L.cml_available(), L.cml_init(0))")
     r = subprocess.run([sys.executable, "-c", code], cwd=ROOT, capture_output=True, text=True, timeout=120)
     assert r.stdout.split() == ["0", "1"], r.stderr
+
+
+def test_host_weight_quantizer_matches_the_oracle_restatement():
+    import oracle
+    rng = np.random.default_rng(7)
+    for fmt in (2, 8, 12, 14):
+        w = (rng.standard_normal((48, 2048)) * 0.02).astype(np.float32)
+        w[3, :512] = 0.0
+        assert np.array_equal(B.quantize_weights(fmt, w, threads=3), oracle.quantize_weights(fmt, w, threads=1))
+    assert B.lib().cml_quantize_weights_host(12, None, 100, None, 1) == 3

@@ -183,9 +183,9 @@ def test_q4k_gemv_every_configuration_agrees():
     s, q = oracle.quantize_activation(B.CML_Q4_K, x)
     w = Weight.upload(B.CML_Q4_K, rows, cols, wire)
     for lps in (8, 4):
-        for ks in (1, 2, 4):
-            G.say(f"gemv Q4_K lanes={lps} ksplit={ks}")
-            with G.env(CAMELID_HIP_Q4K_LPS=lps, CAMELID_HIP_Q4K_KSPLIT=ks):
+        for ks, tpw in ((1, 1), (1, 2), (1, 4), (2, 1), (2, 4), (4, 1), (4, 2), (8, 1)):
+            G.say(f"gemv Q4_K lanes={lps} ksplit={ks} tiles_per_wg={tpw}")
+            with G.env(CAMELID_HIP_Q4K_LPS=lps, CAMELID_HIP_Q4K_KSPLIT=ks, CAMELID_HIP_Q4K_TILES_PER_WG=tpw):
                 got = G.gpu_gemm(w, s, q)
                 ints = G.gpu_block_dots(w, q)
             check_outputs(B.CML_Q4_K, wire, cols, s, q, got, expect_exact=(ks == 1))
