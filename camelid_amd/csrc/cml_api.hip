@@ -305,19 +305,6 @@ int cml_weight_upload(int fmt, int64_t rows, int64_t cols, const void *wire_host
     int64_t nb = 0;
     if (int rc = check_weight_shape(fmt, rows, cols, nbytes, &nb)) return rc;
     if (!wire_host && nbytes) return fail(CML_ERR_INVALID, "null wire pointer");
-    if (fmt == CML_Q4_K) {  // device layout == wire layout: copy straight in
-        cml_weight *w = nullptr;
-        if (int rc = make_weight(fmt, rows, cols, nb, &w)) return rc;
-        if (nbytes) {
-            hipError_t e = hipMemcpy(const_cast<uint8_t *>(w->planes.p[0]), wire_host, nbytes, hipMemcpyHostToDevice);
-            if (e != hipSuccess) {
-                cml_weight_free(w);
-                return fail(CML_ERR_HIP, "hipMemcpy failed: %s", hipGetErrorString(e));
-            }
-        }
-        *out = w;
-        return CML_OK;
-    }
     void *staging = nullptr;
     CML_HIP_TRY(hipMalloc(&staging, nbytes ? nbytes : 16));
     hipError_t e = nbytes ? hipMemcpy(staging, wire_host, nbytes, hipMemcpyHostToDevice) : hipSuccess;
@@ -347,8 +334,16 @@ int cml_weight_slice(const cml_weight *parent, int64_t row_start, int64_t rows, 
     w->allocation = nullptr;
     w->allocation_bytes = 0;
     w->rows = rows;
-    for (int i = 0; i < 4; i++)
-        if (w->planes.p[i]) w->planes.p[i] += row_start * w->planes.row_stride[i];
+    if (parent->fmt == CML_Q4_K) {
+        if (row_start % 16 != 0) {
+            delete w;
+            return fail(CML_ERR_UNSUPPORTED, "a Q4_K band must start on a 16-row tile boundary (row %lld)", (long long)row_start);
+        }
+        w->planes.p[0] += (row_start / 16) * 2304;  // tiles are 2304-byte chunks inside each super-block slab
+    } else {
+        for (int i = 0; i < 4; i++)
+            if (w->planes.p[i]) w->planes.p[i] += row_start * w->planes.row_stride[i];
+    }
     *out = w;
     return CML_OK;
 }

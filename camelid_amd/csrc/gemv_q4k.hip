@@ -10,18 +10,26 @@
 // S and P are what every variant of the reference agrees on bit for bit
 // (src/inference.rs:25806-25889 computes the same integers lane-wise).
 //
-// Mapping.  The weight stays in the GGUF wire layout: 144-byte super-blocks =
-// nine aligned 16-byte pieces (header: f16 d, f16 dmin, 12 packed 6-bit
-// scale/min bytes; then 128 nibble bytes).  LPS lanes (4 or 8) own one
-// super-block: each loads 32 (or 16) nibble bytes plus the 16-byte header with
-// 128-bit loads, unpacks in registers, and dots against the int8 activation
-// staged in LDS with v_dot4_i32_i8.  A wave therefore covers 64/LPS rows at
-// the same super-block index, so the per-row f32 chain above lives in one
-// lane and needs no cross-lane traffic; only the two integers are reduced
-// inside the lane group (DPP row_shr).  A workgroup is TPW row tiles x KSPLIT
-// waves: each tile's super-block range is cut into KSPLIT contiguous parts
-// (one per wave) whose partial chains are added left to right.  With
-// KSPLIT = 1 the result is the reference's own association, bit for bit.
+// Mapping.  At load time the 144-byte wire super-blocks are re-laid, losslessly
+// and at the same density, into a tile-interleaved layout (layout.hip): for a
+// tile of 16 consecutive rows and one super-block index there is one contiguous
+// 2304-byte chunk, chunks ordered [super-block][tile] so that waves working on
+// neighbouring tiles at the same super-block read neighbouring memory (a
+// contiguous front sweeps the matrix, as in a grid-stride copy):
+//     [16 headers x 16 B][16 rows x 4 x 16 B "a" pieces][16 rows x 4 x 16 B "b" pieces]
+// (header = f16 d, f16 dmin, 12 packed 6-bit scale/min bytes; piece a/b of lane
+// c = nibble bytes [32c, 32c+16) / [32c+16, 32c+32) of the block).  Four lanes
+// own one super-block of one row, a wave owns a 16-row tile: each of its three
+// 128-bit load instructions reads whole, consecutive 128-byte lines (256 B of
+// headers, 1 KB, 1 KB) -- the same shape as a plain streaming copy.  The lane
+// unpacks its 64 values in registers and dots them against the int8 activation
+// staged in LDS with v_dot4_i32_i8.  All lanes of a group work on the same
+// row, so the per-row f32 chain above lives in one lane and needs no
+// cross-lane traffic; only the two integers are reduced inside the group (DPP
+// row_shr).  A workgroup is TPW row tiles x KSPLIT waves: each tile's
+// super-block range is cut into KSPLIT contiguous parts (one per wave) whose
+// partial chains are added left to right.  With KSPLIT = 1 the result is the
+// reference's own association, bit for bit.
 //
 // The kernel is short (a 33 MB matrix streams in a few microseconds), so the
 // prologue is ordered to keep HBM busy from the first cycle: the activation
@@ -39,9 +47,9 @@
 namespace cml {
 
 struct Q4KArgs {
-    const uint8_t *w;      // wire blocks, row-major
-    int64_t row_bytes;     // n_sb * 144
-    int rows;              // rows of one band
+    const uint8_t *w;      // tiled layout: [super-block][tile][2304 B]
+    int64_t sb_stride;     // bytes between consecutive super-blocks of one tile (= all tiles * 2304)
+    int rows;              // rows of one band (a multiple of 16 when bands are used)
     int n_sb;              // super-blocks per row
     const int8_t *q;       // [slot][NT][n_sb*256]
     const float *yd;       // [slot][NT][n_sb]
@@ -57,31 +65,30 @@ struct Q4KArgs {
 
 constexpr int kQ4KStageRegs = 4;  // activation chunks a thread holds in registers during the prologue
 
-template <int LPS>
+constexpr int kQ4KChunk = 2304;  // bytes of one (tile, super-block) chunk
+constexpr int LPS = 4;           // lanes per super-block
+
 struct Q4KRegs {
     static constexpr int U = 4;  // super-blocks in flight per buffer
     uint4 hdr[U];
     uint4 qa[U];
-    uint4 qb[U];  // LPS == 4 only
+    uint4 qb[U];
 };
 
 // Loads are unconditional (super-block indices past the end are clamped to the
 // last one and their result is discarded by the caller): straight-line code
 // lets the compiler keep the next buffer's loads in flight under the current
-// buffer's arithmetic with partial vmcnt waits.
-template <int LPS>
-__device__ __forceinline__ void q4k_load(Q4KRegs<LPS> &r, const uint8_t *wrow, int l, int sb, int s1) {
+// buffer's arithmetic with partial vmcnt waits.  `tile` points at the tile's
+// first chunk; r = row in tile, lane = 4r + c.
+__device__ __forceinline__ void q4k_load(Q4KRegs &r, const uint8_t *tile, int64_t sb_stride, int row_in_tile, int lane,
+                                         int sb, int s1) {
 #pragma unroll
-    for (int u = 0; u < Q4KRegs<LPS>::U; u++) {
+    for (int u = 0; u < Q4KRegs::U; u++) {
         const int i = min(sb + u, s1 - 1);
-        const uint8_t *blk = wrow + static_cast<int64_t>(i) * 144;
-        r.hdr[u] = ldg16(blk);
-        if constexpr (LPS == 8) {
-            r.qa[u] = ldg16(blk + 16 + 16 * l);
-        } else {
-            r.qa[u] = ldg16(blk + 16 + 32 * l);
-            r.qb[u] = ldg16(blk + 32 + 32 * l);
-        }
+        const uint8_t *chunk = tile + static_cast<int64_t>(i) * sb_stride;
+        r.hdr[u] = ldg16(chunk + row_in_tile * 16);
+        r.qa[u] = ldg16(chunk + 256 + lane * 16);
+        r.qb[u] = ldg16(chunk + 1280 + lane * 16);
     }
 }
 
@@ -119,12 +126,12 @@ __device__ __forceinline__ void q4k_scale_pairs(const Q4KLane &ln, const uint4 &
     m_pair = ln.upper ? m_up : m_lo;
 }
 
-template <int LPS, int NT, bool INTS>
-__device__ __forceinline__ void q4k_compute(const Q4KRegs<LPS> &r, const Q4KLane &ln, int l, int sb, int s1,
+template <int NT, bool INTS>
+__device__ __forceinline__ void q4k_compute(const Q4KRegs &r, const Q4KLane &ln, int sb, int s1,
                                             const int8_t *ys, const int *bsum, const float *yds, int n_sb,
                                             float (&acc)[NT], int32_t *ints_row) {
 #pragma unroll
-    for (int u = 0; u < Q4KRegs<LPS>::U; u++) {
+    for (int u = 0; u < Q4KRegs::U; u++) {
         const bool valid = sb + u < s1;  // wave-uniform
         const int i = valid ? sb + u : s1 - 1;
         uint32_t sc_pair, m_pair;
@@ -134,38 +141,20 @@ __device__ __forceinline__ void q4k_compute(const Q4KRegs<LPS> &r, const Q4KLane
         const float dminw = f16_bits_to_f32(r.hdr[u].x >> 16);
         const int c = ln.c;
         const uint4 alo = lo_nibbles(r.qa[u]), ahi = hi_nibbles(r.qa[u]);
-        uint4 blo, bhi;
-        int m_a, m_b = 0;
-        if constexpr (LPS == 8) {
-            m_a = (l & 1) ? (m_pair >> 8) : (m_pair & 0xff);  // lane l owns group l on the mins side
-        } else {
-            blo = lo_nibbles(r.qb[u]);
-            bhi = hi_nibbles(r.qb[u]);
-            m_a = m_pair & 0xff;
-            m_b = m_pair >> 8;
-        }
+        const uint4 blo = lo_nibbles(r.qb[u]), bhi = hi_nibbles(r.qb[u]);
+        const int m_a = m_pair & 0xff, m_b = m_pair >> 8;
 #pragma unroll
         for (int t = 0; t < NT; t++) {
             const int8_t *y = ys + (static_cast<int64_t>(t) * n_sb + i) * 256;
             const int *bs = bsum + (t * n_sb + i) * 8;
-            int lo, hi, p;
-            if constexpr (LPS == 8) {
-                const int h = l & 1;
-                const uint4 ylo = *reinterpret_cast<const uint4 *>(y + 64 * c + 16 * h);
-                const uint4 yhi = *reinterpret_cast<const uint4 *>(y + 64 * c + 32 + 16 * h);
-                lo = dot16(alo, ylo, 0);
-                hi = dot16(ahi, yhi, 0);
-                p = __mul24(bs[l], m_a);
-            } else {
-                const uint4 ylo0 = *reinterpret_cast<const uint4 *>(y + 64 * c);
-                const uint4 ylo1 = *reinterpret_cast<const uint4 *>(y + 64 * c + 16);
-                const uint4 yhi0 = *reinterpret_cast<const uint4 *>(y + 64 * c + 32);
-                const uint4 yhi1 = *reinterpret_cast<const uint4 *>(y + 64 * c + 48);
-                lo = dot16(blo, ylo1, dot16(alo, ylo0, 0));
-                hi = dot16(bhi, yhi1, dot16(ahi, yhi0, 0));
-                const int2 b2 = *reinterpret_cast<const int2 *>(bs + 2 * c);
-                p = __mul24(b2.x, m_a) + __mul24(b2.y, m_b);
-            }
+            const uint4 ylo0 = *reinterpret_cast<const uint4 *>(y + 64 * c);
+            const uint4 ylo1 = *reinterpret_cast<const uint4 *>(y + 64 * c + 16);
+            const uint4 yhi0 = *reinterpret_cast<const uint4 *>(y + 64 * c + 32);
+            const uint4 yhi1 = *reinterpret_cast<const uint4 *>(y + 64 * c + 48);
+            const int lo = dot16(blo, ylo1, dot16(alo, ylo0, 0));
+            const int hi = dot16(bhi, yhi1, dot16(ahi, yhi0, 0));
+            const int2 b2 = *reinterpret_cast<const int2 *>(bs + 2 * c);
+            const int p = __mul24(b2.x, m_a) + __mul24(b2.y, m_b);
             // |lo|, |hi| <= 32*15*128 and the 6-bit scales keep every product inside 24 bits.
             int s_total = group_sum_to_last<LPS>(__mul24(lo, sc_lo) + __mul24(hi, sc_hi));
             int p_total = group_sum_to_last<LPS>(p);
@@ -186,7 +175,7 @@ __device__ __forceinline__ void q4k_compute(const Q4KRegs<LPS> &r, const Q4KLane
     }
 }
 
-template <int LPS, int NT, bool INTS>
+template <int NT, bool INTS>
 __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
     constexpr int RPW = kWave / LPS;  // rows per wave tile
     extern __shared__ uint4 smem[];
@@ -200,7 +189,7 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
     const int nthreads = blockDim.x;
     const int slot = blockIdx.y;
     const int64_t band = a.band_ids ? a.band_ids[slot] : 0;
-    const uint8_t *w = a.w + band * a.rows * a.row_bytes;
+    const uint8_t *w = a.w + band * (a.rows / 16) * kQ4KChunk;
     const int8_t *q = a.q + static_cast<int64_t>(slot) * a.act_slot_stride * n_sb * 256;
     const float *yd = a.yd + static_cast<int64_t>(slot) * a.act_slot_stride * n_sb;
     float *out = a.out + static_cast<int64_t>(slot) * a.out_slot_stride;
@@ -214,10 +203,11 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
     const int r = lane / LPS, l = lane - r * LPS;
     const int row = tile * RPW + r;
     const bool live = row < a.rows;
-    const uint8_t *wrow = w + static_cast<int64_t>(live ? row : a.rows - 1) * a.row_bytes;
+    // the last tile is padded to 16 rows; tiles past the end (grid rounding) re-read it and store nothing
+    const uint8_t *wtile = w + static_cast<int64_t>(min(tile, (a.rows + 15) / 16 - 1)) * kQ4KChunk;
     const bool leader = (l == LPS - 1);
     Q4KLane ln;
-    ln.c = (LPS == 8) ? (l >> 1) : l;
+    ln.c = l;
     ln.sh = (ln.c & 1) * 16;
     ln.upper = ln.c >= 2;
 
@@ -232,10 +222,10 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
     for (int k = 0; k < kQ4KStageRegs; k++) sv[k] = src[min(tid + k * nthreads, n16 - 1)];
     const float yd0 = yd[min(tid, NT * n_sb - 1)];
 
-    constexpr int U = Q4KRegs<LPS>::U;
-    Q4KRegs<LPS> ra, rb;
+    constexpr int U = Q4KRegs::U;
+    Q4KRegs ra, rb;
     __builtin_amdgcn_sched_barrier(0);
-    q4k_load<LPS>(ra, wrow, l, s0, s1);
+    q4k_load(ra, wtile, a.sb_stride, r, lane, s0, s1);
     __builtin_amdgcn_sched_barrier(0);
 
 #pragma unroll
@@ -268,17 +258,29 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
 #pragma unroll
     for (int t = 0; t < NT; t++) acc[t] = 0.0f;
 
-    // sched_barrier keeps each buffer's loads ahead of the other buffer's
-    // arithmetic, so one buffer is always in flight under the compute.
-    for (int sb = s0; sb < s1; sb += 2 * U) {
-        q4k_load<LPS>(rb, wrow, l, sb + U, s1);
+    // Two register buffers alternate: the next buffer's loads are issued, then
+    // the current one is consumed.  The last buffer is consumed without issuing
+    // anything, so no load is wasted; sched_barrier keeps the loads ahead of
+    // the arithmetic they overlap with.
+    for (int sb = s0;;) {
+        if (sb + U >= s1) {
+            q4k_compute<NT, INTS>(ra, ln, sb, s1, ys, bsum, yds, n_sb, acc, ints_row);
+            break;
+        }
+        q4k_load(rb, wtile, a.sb_stride, r, lane, sb + U, s1);
         __builtin_amdgcn_sched_barrier(0);
-        q4k_compute<LPS, NT, INTS>(ra, ln, l, sb, s1, ys, bsum, yds, n_sb, acc, ints_row);
+        q4k_compute<NT, INTS>(ra, ln, sb, s1, ys, bsum, yds, n_sb, acc, ints_row);
         __builtin_amdgcn_sched_barrier(0);
-        q4k_load<LPS>(ra, wrow, l, sb + 2 * U, s1);
+        sb += U;
+        if (sb + U >= s1) {
+            q4k_compute<NT, INTS>(rb, ln, sb, s1, ys, bsum, yds, n_sb, acc, ints_row);
+            break;
+        }
+        q4k_load(ra, wtile, a.sb_stride, r, lane, sb + U, s1);
         __builtin_amdgcn_sched_barrier(0);
-        q4k_compute<LPS, NT, INTS>(rb, ln, l, sb + U, s1, ys, bsum, yds, n_sb, acc, ints_row);
+        q4k_compute<NT, INTS>(rb, ln, sb, s1, ys, bsum, yds, n_sb, acc, ints_row);
         __builtin_amdgcn_sched_barrier(0);
+        sb += U;
     }
 
     if (W == 1) {
@@ -314,13 +316,12 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
 // give every cell the same association; 1 (the reference's own) whenever the
 // row count alone yields about one wave per SIMD (1024 on this chip).
 struct Q4KShape {
-    int lps, ksplit, tiles_per_wg;
+    int ksplit, tiles_per_wg;
 };
 
 static Q4KShape pick_shape(int64_t rows, int64_t n_sb) {
     Q4KShape s;
-    s.lps = env_int("CAMELID_HIP_Q4K_LPS", 4) == 8 ? 8 : 4;
-    const int64_t tiles = (rows + (64 / s.lps) - 1) / (64 / s.lps);
+    const int64_t tiles = (rows + 15) / 16;
     int ks = 1;
     const int forced = env_int("CAMELID_HIP_Q4K_KSPLIT", 0);
     if ((forced == 1 || forced == 2 || forced == 4 || forced == 8) && forced <= n_sb) {
@@ -338,38 +339,39 @@ static Q4KShape pick_shape(int64_t rows, int64_t n_sb) {
     return s;
 }
 
-template <int LPS, int NT>
+template <int NT>
 static int launch_q4k_nt(Q4KArgs ka, const Q4KShape &shape, int n_bands, bool ints, hipStream_t st) {
-    const int rpw = 64 / LPS;
     const int waves = shape.ksplit * shape.tiles_per_wg;
-    const int64_t tiles = (ka.rows + rpw - 1) / rpw;
+    const int64_t tiles = (ka.rows + 15) / 16;
     const unsigned gx = static_cast<unsigned>((tiles + shape.tiles_per_wg - 1) / shape.tiles_per_wg);
     const size_t lds = static_cast<size_t>(NT) * ka.n_sb * (256 + 32) + ((static_cast<size_t>(NT) * ka.n_sb + 3) & ~size_t(3)) * 4 +
-                       static_cast<size_t>(waves) * NT * rpw * 4;
+                       static_cast<size_t>(waves) * NT * 16 * 4;
     if (lds > 64 * 1024) return fail(CML_ERR_UNSUPPORTED, "Q4_K activation of %d super-blocks x %d tokens exceeds the LDS staging limit", ka.n_sb, NT);
     ka.ksplit = shape.ksplit;
     ka.tiles_per_wg = shape.tiles_per_wg;
     if (ints && NT == 1)
-        hipLaunchKernelGGL((gemv_q4k_kernel<LPS, 1, true>), dim3(gx, n_bands), dim3(64 * waves), lds, st, ka);
+        hipLaunchKernelGGL((gemv_q4k_kernel<1, true>), dim3(gx, n_bands), dim3(64 * waves), lds, st, ka);
     else
-        hipLaunchKernelGGL((gemv_q4k_kernel<LPS, NT, false>), dim3(gx, n_bands), dim3(64 * waves), lds, st, ka);
+        hipLaunchKernelGGL((gemv_q4k_kernel<NT, false>), dim3(gx, n_bands), dim3(64 * waves), lds, st, ka);
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }
 
-template <int LPS>
-static int launch_q4k_lps(const MatArgs &a, const Q4KShape &shape, hipStream_t st) {
+int launch_gemv_q4k(const MatArgs &a, hipStream_t st) {
     const cml_weight *w = a.w;
+    if (w->rows == 0 || a.n_tokens == 0) return CML_OK;
     Q4KArgs ka;
     ka.w = w->planes.p[0];
-    ka.row_bytes = w->planes.row_stride[0];
+    ka.sb_stride = w->planes.row_stride[0];
     ka.rows = static_cast<int>(a.band_ids ? a.band_rows : w->rows);
+    if (a.band_ids && (ka.rows % 16) != 0) return fail(CML_ERR_UNSUPPORTED, "Q4_K expert bands must be whole 16-row tiles (%d rows)", ka.rows);
     ka.n_sb = static_cast<int>(w->nb);
     ka.residual = a.residual;
     ka.ints = a.ints;
     ka.band_ids = a.band_ids;
     ka.act_slot_stride = a.act_per_slot ? a.n_tokens : 0;
     ka.out_slot_stride = a.n_tokens * static_cast<int64_t>(ka.rows);
+    const Q4KShape shape = pick_shape(ka.rows, ka.n_sb);
     const int n_bands = a.n_bands > 0 ? a.n_bands : 1;
     // Tokens are served in passes of up to 8 rows of activations.
     int64_t t0 = 0;
@@ -381,22 +383,15 @@ static int launch_q4k_lps(const MatArgs &a, const Q4KShape &shape, hipStream_t s
         ka.out = a.out + t0 * ka.rows;
         int rc;
         switch (nt) {
-            case 8: rc = launch_q4k_nt<LPS, 8>(ka, shape, n_bands, false, st); break;
-            case 4: rc = launch_q4k_nt<LPS, 4>(ka, shape, n_bands, false, st); break;
-            case 2: rc = launch_q4k_nt<LPS, 2>(ka, shape, n_bands, false, st); break;
-            default: rc = launch_q4k_nt<LPS, 1>(ka, shape, n_bands, a.ints != nullptr, st); break;
+            case 8: rc = launch_q4k_nt<8>(ka, shape, n_bands, false, st); break;
+            case 4: rc = launch_q4k_nt<4>(ka, shape, n_bands, false, st); break;
+            case 2: rc = launch_q4k_nt<2>(ka, shape, n_bands, false, st); break;
+            default: rc = launch_q4k_nt<1>(ka, shape, n_bands, a.ints != nullptr, st); break;
         }
         if (rc != CML_OK) return rc;
         t0 += nt;
     }
     return CML_OK;
-}
-
-int launch_gemv_q4k(const MatArgs &a, hipStream_t st) {
-    if (a.w->rows == 0 || a.n_tokens == 0) return CML_OK;
-    const int64_t rows = a.band_ids ? a.band_rows : a.w->rows;
-    const Q4KShape shape = pick_shape(rows, a.w->nb);
-    return shape.lps == 4 ? launch_q4k_lps<4>(a, shape, st) : launch_q4k_lps<8>(a, shape, st);
 }
 
 int launch_gemm_q4k(const MatArgs &a, hipStream_t st) { return launch_gemv_q4k(a, st); }

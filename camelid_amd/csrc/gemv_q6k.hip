@@ -174,11 +174,28 @@ __global__ __launch_bounds__(256) void gemv_q6k_kernel(Q6KArgs a) {
     constexpr int U = Q6KRegs::U;
     Q6KRegs ra, rb;
     q6k_load(ra, ql, qh, sc, dp, l, s0, s1);
-    for (int sb = s0; sb < s1; sb += 2 * U) {
+    __builtin_amdgcn_sched_barrier(0);
+    // Two register buffers alternate; the last one is consumed without issuing
+    // further loads.
+    for (int sb = s0;;) {
+        if (sb + U >= s1) {
+            q6k_compute<NT, INTS>(ra, l, sb, s1, ys, bsum16, yds, n_sb, acc, ints_row);
+            break;
+        }
         q6k_load(rb, ql, qh, sc, dp, l, sb + U, s1);
+        __builtin_amdgcn_sched_barrier(0);
         q6k_compute<NT, INTS>(ra, l, sb, s1, ys, bsum16, yds, n_sb, acc, ints_row);
-        q6k_load(ra, ql, qh, sc, dp, l, sb + 2 * U, s1);
-        q6k_compute<NT, INTS>(rb, l, sb + U, s1, ys, bsum16, yds, n_sb, acc, ints_row);
+        __builtin_amdgcn_sched_barrier(0);
+        sb += U;
+        if (sb + U >= s1) {
+            q6k_compute<NT, INTS>(rb, l, sb, s1, ys, bsum16, yds, n_sb, acc, ints_row);
+            break;
+        }
+        q6k_load(ra, ql, qh, sc, dp, l, sb + U, s1);
+        __builtin_amdgcn_sched_barrier(0);
+        q6k_compute<NT, INTS>(rb, l, sb, s1, ys, bsum16, yds, n_sb, acc, ints_row);
+        __builtin_amdgcn_sched_barrier(0);
+        sb += U;
     }
 
     if (W == 1) {

@@ -159,11 +159,28 @@ __global__ __launch_bounds__(256) void gemv_b32_kernel(B32Args a) {
     const int n_steps = (nb + P - 1) / P;
     B32Regs<FMT> ra, rb;
     b32_load<FMT, P>(ra, qrow, srow, l, 0, n_steps, nb);
-    for (int step = 0; step < n_steps; step += 2 * U) {
+    __builtin_amdgcn_sched_barrier(0);
+    // Two register buffers alternate; the last one is consumed without issuing
+    // further loads.
+    for (int step = 0;;) {
+        if (step + U >= n_steps) {
+            b32_compute<FMT, P, NT, INTS>(ra, l, step, n_steps, nb, ys, bsum, xss, acc, ints_row);
+            break;
+        }
         b32_load<FMT, P>(rb, qrow, srow, l, step + U, n_steps, nb);
+        __builtin_amdgcn_sched_barrier(0);
         b32_compute<FMT, P, NT, INTS>(ra, l, step, n_steps, nb, ys, bsum, xss, acc, ints_row);
-        b32_load<FMT, P>(ra, qrow, srow, l, step + 2 * U, n_steps, nb);
-        b32_compute<FMT, P, NT, INTS>(rb, l, step + U, n_steps, nb, ys, bsum, xss, acc, ints_row);
+        __builtin_amdgcn_sched_barrier(0);
+        step += U;
+        if (step + U >= n_steps) {
+            b32_compute<FMT, P, NT, INTS>(rb, l, step, n_steps, nb, ys, bsum, xss, acc, ints_row);
+            break;
+        }
+        b32_load<FMT, P>(ra, qrow, srow, l, step + U, n_steps, nb);
+        __builtin_amdgcn_sched_barrier(0);
+        b32_compute<FMT, P, NT, INTS>(rb, l, step, n_steps, nb, ys, bsum, xss, acc, ints_row);
+        __builtin_amdgcn_sched_barrier(0);
+        step += U;
     }
 
     if (leader && live) {

@@ -1,10 +1,16 @@
 // Load-time re-layout (wire blocks <-> per-field planes) and the bit-exact
 // dequantizers.
 //
-// Device layouts.  Q4_K keeps the GGUF wire blocks (144 B = 9 x 16 B, so every
-// block starts 16-byte aligned).  Q8_0 (34 B), Q4_0 (18 B) and Q6_K (210 B)
-// blocks are not 16-byte periodic, so their fields are split into planes, each
-// plane row-major by (row, block):
+// Device layouts.  Q4_K (144 B = 9 x 16 B pieces per super-block) is
+// tile-interleaved: rows are grouped in tiles of 16 (the last tile zero-padded)
+// and for every (super-block, tile) -- in that order, super-block major --
+// there is one contiguous 2304-byte chunk
+//     [16 rows x 16 B header][16 rows x 4 x 16 B piece a][16 rows x 4 x 16 B piece b]
+// where piece a / b of lane c holds nibble bytes [32c, 32c+16) / [32c+16, 32c+32)
+// of that row's block -- so the three 128-bit loads of a wave that owns the
+// tile each read whole consecutive cache lines.  Q8_0 (34 B), Q4_0 (18 B) and
+// Q6_K (210 B) blocks are not 16-byte periodic; their fields are split into
+// planes, each plane row-major by (row, block):
 //   Q8_0: quants int8[rows][nb*32]            | d f16[rows][nb]
 //   Q4_0: nibbles u8[rows][nb*16]             | d f16[rows][nb]
 //   Q6_K: ql u8[rows][nb*128] | qh u8[rows][nb*64] | scales i8[rows][nb*16] | d f16[rows][nb]
@@ -31,7 +37,7 @@ Geometry geometry(int fmt) {
 int plane_layout(int fmt, int64_t rows, int64_t nb, int64_t stride[4], size_t offset[4], size_t *total) {
     int n = 0;
     switch (fmt) {
-        case CML_Q4_K: stride[0] = nb * 144; n = 1; break;
+        case CML_Q4_K: stride[0] = ((rows + 15) / 16) * 2304; n = 1; break;  // bytes between super-blocks (all tiles)
         case CML_Q8_0: stride[0] = nb * 32; stride[1] = nb * 2; n = 2; break;
         case CML_Q4_0: stride[0] = nb * 16; stride[1] = nb * 2; n = 2; break;
         case CML_Q6_K: stride[0] = nb * 128; stride[1] = nb * 64; stride[2] = nb * 16; stride[3] = nb * 2; n = 4; break;
@@ -40,7 +46,8 @@ int plane_layout(int fmt, int64_t rows, int64_t nb, int64_t stride[4], size_t of
     size_t at = 0;
     for (int i = 0; i < n; i++) {
         offset[i] = at;
-        at += static_cast<size_t>(stride[i]) * static_cast<size_t>(rows);
+        const size_t units = fmt == CML_Q4_K ? static_cast<size_t>(nb) : static_cast<size_t>(rows);
+        at += static_cast<size_t>(stride[i]) * units;
         at = (at + 255) & ~static_cast<size_t>(255);  // every plane starts 256-byte aligned
     }
     for (int i = n; i < 4; i++) { stride[i] = 0; offset[i] = 0; }
@@ -86,13 +93,46 @@ __global__ __launch_bounds__(256) void relayout_kernel(int fmt, uint8_t *wire, P
     if (TO_PLANES) *p = *w; else *w = *p;
 }
 
+// Q4_K: one thread per 16-byte piece of the wire image (9 per super-block).
+template <bool TO_TILED>
+__global__ __launch_bounds__(256) void q4k_tile_kernel(uint4 *wire, uint8_t *tiled, int64_t sb_stride, int64_t nb,
+                                                       int64_t n_pieces) {
+    const int64_t g = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (g >= n_pieces) return;
+    const int64_t blk = g / 9;
+    const int piece = static_cast<int>(g - blk * 9);
+    const int64_t row = blk / nb, sb = blk - row * nb;
+    const int r = static_cast<int>(row & 15);
+    uint8_t *chunk = tiled + sb * sb_stride + (row >> 4) * 2304;
+    uint8_t *p;
+    if (piece == 0) {
+        p = chunk + r * 16;
+    } else {
+        const int c = (piece - 1) >> 1, half = (piece - 1) & 1;
+        p = chunk + (half ? 1280 : 256) + (4 * r + c) * 16;
+    }
+    if (TO_TILED) *reinterpret_cast<uint4 *>(p) = wire[g]; else wire[g] = *reinterpret_cast<const uint4 *>(p);
+}
+
 static int relayout(bool to_planes, int fmt, uint8_t *wire, const Planes &pl, int64_t rows, int64_t nb, hipStream_t st) {
     const Geometry g = geometry(fmt);
     const int64_t nbytes = rows * nb * g.block_bytes;
     if (nbytes == 0) return CML_OK;
     if (fmt == CML_Q4_K) {
-        if (to_planes) CML_HIP_TRY(hipMemcpyAsync(const_cast<uint8_t *>(pl.p[0]), wire, nbytes, hipMemcpyDeviceToDevice, st));
-        else CML_HIP_TRY(hipMemcpyAsync(wire, pl.p[0], nbytes, hipMemcpyDeviceToDevice, st));
+        if (reinterpret_cast<uintptr_t>(wire) & 15u) return fail(CML_ERR_INVALID, "Q4_K wire bytes must be 16-byte aligned on the device");
+        const int64_t n_pieces = rows * nb * 9;
+        const unsigned grid = static_cast<unsigned>((n_pieces + 255) / 256);
+        uint8_t *tiled = const_cast<uint8_t *>(pl.p[0]);
+        if (to_planes) {
+            if (rows % 16) {  // zero the padding rows of the last tile (one chunk per super-block)
+                const int64_t last = rows / 16;
+                CML_HIP_TRY(hipMemset2DAsync(tiled + last * 2304, static_cast<size_t>(pl.row_stride[0]), 0, 2304, static_cast<size_t>(nb), st));
+            }
+            hipLaunchKernelGGL(q4k_tile_kernel<true>, dim3(grid), dim3(256), 0, st, reinterpret_cast<uint4 *>(wire), tiled, pl.row_stride[0], nb, n_pieces);
+        } else {
+            hipLaunchKernelGGL(q4k_tile_kernel<false>, dim3(grid), dim3(256), 0, st, reinterpret_cast<uint4 *>(wire), tiled, pl.row_stride[0], nb, n_pieces);
+        }
+        CML_HIP_TRY(hipGetLastError());
         return CML_OK;
     }
     PlanePtrs pp;
@@ -139,16 +179,20 @@ __global__ __launch_bounds__(256) void dequant_q8q4_kernel(int fmt, Planes pl, i
 
 // Q4_K: (d*sc)*q - (dmin*m) (reference Q4KBlock::dequantize, src/tensor/mod.rs:5903-5924;
 // q4_k_scale_min, :5997-6006).
-__global__ __launch_bounds__(256) void dequant_q4k_kernel(const uint8_t *__restrict__ w, int64_t n_values,
-                                                          float *__restrict__ out) {
+__global__ __launch_bounds__(256) void dequant_q4k_kernel(const uint8_t *__restrict__ tiled, int64_t sb_stride,
+                                                          int64_t nb, int64_t n_values, float *__restrict__ out) {
     const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i >= n_values) return;
-    const uint8_t *blk = w + (i >> 8) * 144;
+    const int64_t blk = i >> 8;
+    const int64_t row = blk / nb, sb = blk - row * nb;
+    const int rr = static_cast<int>(row & 15);
+    const uint8_t *chunk = tiled + sb * sb_stride + (row >> 4) * 2304;
+    const uint8_t *hdr = chunk + rr * 16;
     const int v = static_cast<int>(i & 255);
     const int g = v >> 5, t = v & 31;
-    const float d = f16_bits_to_f32(ldg2(blk));
-    const float dmin = f16_bits_to_f32(ldg2(blk + 2));
-    const uint8_t *s = blk + 4;
+    const float d = f16_bits_to_f32(ldg2(hdr));
+    const float dmin = f16_bits_to_f32(ldg2(hdr + 2));
+    const uint8_t *s = hdr + 4;
     int sc, m;
     if (g < 4) {
         sc = s[g] & 63;
@@ -157,7 +201,8 @@ __global__ __launch_bounds__(256) void dequant_q4k_kernel(const uint8_t *__restr
         sc = (s[g + 4] & 0x0f) | ((s[g - 4] >> 6) << 4);
         m = (s[g + 4] >> 4) | ((s[g] >> 6) << 4);
     }
-    const uint8_t byte = blk[16 + (g >> 1) * 32 + t];
+    // nibble byte t of chunk c = g/2: piece a holds bytes 0..15, piece b bytes 16..31
+    const uint8_t byte = chunk[((t & 16) ? 1280 : 256) + (4 * rr + (g >> 1)) * 16 + (t & 15)];
     const int q = (g & 1) ? (byte >> 4) : (byte & 0x0f);
     const float scale = d * static_cast<float>(sc);
     const float min = dmin * static_cast<float>(m);
@@ -192,8 +237,7 @@ int launch_dequantize(const cml_weight *w, float *out, hipStream_t st) {
             hipLaunchKernelGGL(dequant_q8q4_kernel, dim3(grid), dim3(256), 0, st, w->fmt, w->planes, w->nb, n_values, out);
             break;
         case CML_Q4_K:
-            if (w->planes.row_stride[0] != w->nb * 144) return fail(CML_ERR_SHAPE, "Q4_K rows are not contiguous");
-            hipLaunchKernelGGL(dequant_q4k_kernel, dim3(grid), dim3(256), 0, st, w->planes.p[0], n_values, out);
+            hipLaunchKernelGGL(dequant_q4k_kernel, dim3(grid), dim3(256), 0, st, w->planes.p[0], w->planes.row_stride[0], w->nb, n_values, out);
             break;
         case CML_Q6_K:
             hipLaunchKernelGGL(dequant_q6k_kernel, dim3(grid), dim3(256), 0, st, w->planes, w->nb, n_values, out);

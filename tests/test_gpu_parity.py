@@ -100,10 +100,10 @@ def test_relayout_is_a_pure_permutation(name, fmt):
         wire = rng.integers(0, 256, size=rows * oracle.row_bytes(fmt, cols), dtype=np.uint8)
         w = Weight.upload(fmt, rows, cols, wire)
         assert np.array_equal(w.download(), wire)
-        if rows > 4:
-            band = w.slice(2, rows - 3)
+        if rows > 20:
+            band = w.slice(16, rows - 19)   # Q4_K bands start on 16-row tile boundaries
             rb = oracle.row_bytes(fmt, cols)
-            assert np.array_equal(band.download(), wire[2 * rb:(rows - 1) * rb])
+            assert np.array_equal(band.download(), wire[16 * rb:(rows - 3) * rb])
 
 
 @pytest.mark.parametrize("name,fmt", FMTS)
@@ -182,14 +182,13 @@ def test_q4k_gemv_every_configuration_agrees():
     x = rng.standard_normal(cols).astype(np.float32)
     s, q = oracle.quantize_activation(B.CML_Q4_K, x)
     w = Weight.upload(B.CML_Q4_K, rows, cols, wire)
-    for lps in (8, 4):
-        for ks, tpw in ((1, 1), (1, 2), (1, 4), (2, 1), (2, 4), (4, 1), (4, 2), (8, 1)):
-            G.say(f"gemv Q4_K lanes={lps} ksplit={ks} tiles_per_wg={tpw}")
-            with G.env(CAMELID_HIP_Q4K_LPS=lps, CAMELID_HIP_Q4K_KSPLIT=ks, CAMELID_HIP_Q4K_TILES_PER_WG=tpw):
-                got = G.gpu_gemm(w, s, q)
-                ints = G.gpu_block_dots(w, q)
-            check_outputs(B.CML_Q4_K, wire, cols, s, q, got, expect_exact=(ks == 1))
-            assert np.array_equal(ints, oracle.block_ints(B.CML_Q4_K, wire, cols, q))
+    for ks, tpw in ((1, 1), (1, 2), (1, 4), (1, 8), (2, 1), (2, 4), (4, 1), (4, 2), (8, 1)):
+        G.say(f"gemv Q4_K ksplit={ks} tiles_per_wg={tpw}")
+        with G.env(CAMELID_HIP_Q4K_KSPLIT=ks, CAMELID_HIP_Q4K_TILES_PER_WG=tpw):
+            got = G.gpu_gemm(w, s, q)
+            ints = G.gpu_block_dots(w, q)
+        check_outputs(B.CML_Q4_K, wire, cols, s, q, got, expect_exact=(ks == 1))
+        assert np.array_equal(ints, oracle.block_ints(B.CML_Q4_K, wire, cols, q))
 
 
 @pytest.mark.parametrize("name,fmt", FMTS)
@@ -207,10 +206,10 @@ def test_gemv_residual_and_band_view(name, fmt):
         got = G.gpu_gemm(w, s, q, residual=res)
         assert G.same_bits(got, (base + res).astype(np.float32))
         G.say(f"gemv band view {name}")
-        band = w.slice(24, 40)   # rows 24..63: an expert band of a stacked tensor
+        band = w.slice(32, 40)   # rows 32..71: an expert band of a stacked tensor
         got = G.gpu_gemm(band, s, q)
-    assert G.same_bits(got, base[24:64])
-    check_outputs(fmt, wire, cols, s, q, got, row_start=24, rows=40, expect_exact=True)
+    assert G.same_bits(got, base[32:72])
+    check_outputs(fmt, wire, cols, s, q, got, row_start=32, rows=40, expect_exact=True)
 
 
 # ------------------------------------------------------------- batched ----
@@ -261,6 +260,8 @@ def test_error_paths_return_status_codes():
     assert L.cml_weight_upload(7, 3, 256, wire.ctypes.data, wire.nbytes, C.byref(h)) == 2   # unknown format
     w = Weight.upload(12, 3, 256, wire)
     assert L.cml_weight_slice(w.handle, 2, 5, C.byref(h)) == 3
+    w20 = Weight.upload(12, 20, 256, np.zeros(144 * 20, np.uint8))
+    assert L.cml_weight_slice(w20.handle, 3, 5, C.byref(h)) == 6   # Q4_K bands start on a tile boundary
     assert L.cml_gemv(w.handle, None, None, None, None, None) == 2
     empty = Weight.upload(12, 0, 256, np.zeros(0, np.uint8))   # zero rows: accepted, nothing to do
     assert L.cml_gemv(empty.handle, None, None, None, None, None) == 0
