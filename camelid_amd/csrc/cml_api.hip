@@ -437,10 +437,10 @@ static MatArgs plain_args(const cml_weight *w, const int8_t *q, const float *s, 
     a.out = out;
     a.residual = nullptr;
     a.ints = nullptr;
-    a.band_ids = nullptr;
-    a.n_bands = 1;
+    a.group_offsets = nullptr;
+    a.group_rows = nullptr;
+    a.n_groups = 1;
     a.band_rows = 0;
-    a.act_per_slot = false;
     return a;
 }
 

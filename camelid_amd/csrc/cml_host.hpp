@@ -72,21 +72,21 @@ int launch_dequantize(const cml_weight *w, float *out, hipStream_t st);
 // Arguments common to every gemv/gemm launcher.
 struct MatArgs {
     const cml_weight *w;
-    const int8_t *q;      // [n_tokens][cols]           (per slot when act_per_slot)
-    const float *scales;  // [n_tokens][nb]
-    int64_t n_tokens;
-    float *out;             // [n_tokens][rows]         (per slot for routed calls)
-    const float *residual;  // gemv only, may be null
-    int32_t *ints;          // block-int diagnostics, may be null (single token only)
-    // Routed (mixture-of-experts) extension; null/zero for plain calls.  The
-    // grid gets one y-slot per routed expert: slot s reads band
-    // band_ids[s] = rows [id*band_rows, (id+1)*band_rows) of the stacked
-    // weight, dots it against its own activation rows (act_per_slot) or the
-    // shared ones, and writes out[s][n_tokens][band_rows].
-    const int32_t *band_ids;  // device pointer
-    int n_bands;
+    const int8_t *q;      // activation rows [*][cols]
+    const float *scales;  // [*][nb]
+    int64_t n_tokens;     // plain: activation rows; grouped: the most assignments one group can hold
+    float *out;           // [*][rows]
+    const float *residual;  // plain single-token calls only, may be null
+    int32_t *ints;          // block-int diagnostics, may be null (plain single token only)
+    // Grouped (mixture-of-experts) extension; null/zero for plain calls.  The
+    // grid gets one y-slot per group (expert) e, which owns the band of rows
+    // [e*band_rows, (e+1)*band_rows) of the stacked weight and the
+    // assignments [group_offsets[e], group_offsets[e+1]); assignment j dots
+    // activation row group_rows[j] (j itself when null) and writes out[j][band_rows].
+    const int32_t *group_offsets;  // device, [n_groups + 1]
+    const int32_t *group_rows;     // device, [assignments] or null
+    int n_groups;
     int64_t band_rows;
-    bool act_per_slot;
 };
 
 int launch_gemv_q4k(const MatArgs &a, hipStream_t st);

@@ -49,18 +49,23 @@ namespace cml {
 struct Q4KArgs {
     const uint8_t *w;      // tiled layout: [super-block][tile][2304 B]
     int64_t sb_stride;     // bytes between consecutive super-blocks of one tile (= all tiles * 2304)
-    int rows;              // rows of one band (a multiple of 16 when bands are used)
+    int rows;              // rows of one band (a multiple of 16 when groups are used)
     int n_sb;              // super-blocks per row
-    const int8_t *q;       // [slot][NT][n_sb*256]
-    const float *yd;       // [slot][NT][n_sb]
-    float *out;            // [slot][NT][rows]
-    const float *residual; // [rows] or null (NT == 1 only)
+    const int8_t *q;       // activation rows [*][n_sb*256]
+    const float *yd;       // activation scales [*][n_sb]
+    float *out;            // [*][rows]
+    const float *residual; // [rows] or null (plain single-token calls only)
     int32_t *ints;         // [rows][n_sb][2] or null
-    const int32_t *band_ids;  // expert id per blockIdx.y, or null
-    int64_t act_slot_stride;  // activation rows between blockIdx.y slots (0 = shared)
-    int64_t out_slot_stride;  // output floats between blockIdx.y slots
-    int ksplit;               // waves sharing one row tile (1, 2, 4 or 8)
-    int tiles_per_wg;         // row tiles per workgroup; blockDim.x = 64 * ksplit * tiles_per_wg
+    // Plain call: blockIdx.y = 0, the NT activation rows 0..NT-1 go to output rows 0..NT-1.
+    // Grouped call (mixture of experts): blockIdx.y = group e, which owns the
+    // weight band of rows [e*rows, (e+1)*rows) and the assignments
+    // [group_offsets[e], group_offsets[e+1]); assignment j reads activation row
+    // group_rows[j] (j itself when null) and writes output row j.  A group
+    // serves its assignments in passes of NT.
+    const int32_t *group_offsets;
+    const int32_t *group_rows;
+    int ksplit;        // waves sharing one row tile (1, 2, 4 or 8)
+    int tiles_per_wg;  // row tiles per workgroup; blockDim.x = 64 * ksplit * tiles_per_wg
 };
 
 constexpr int kQ4KStageRegs = 4;  // activation chunks a thread holds in registers during the prologue
@@ -187,12 +192,12 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
 
     const int tid = threadIdx.x;
     const int nthreads = blockDim.x;
-    const int slot = blockIdx.y;
-    const int64_t band = a.band_ids ? a.band_ids[slot] : 0;
+    const bool grouped = a.group_offsets != nullptr;
+    const int64_t band = grouped ? blockIdx.y : 0;
+    const int a0 = grouped ? a.group_offsets[band] : 0;               // first assignment of this group
+    const int n_assign = grouped ? a.group_offsets[band + 1] - a0 : NT;
+    if (n_assign <= 0) return;  // an expert nobody routed to: the whole workgroup leaves
     const uint8_t *w = a.w + band * (a.rows / 16) * kQ4KChunk;
-    const int8_t *q = a.q + static_cast<int64_t>(slot) * a.act_slot_stride * n_sb * 256;
-    const float *yd = a.yd + static_cast<int64_t>(slot) * a.act_slot_stride * n_sb;
-    float *out = a.out + static_cast<int64_t>(slot) * a.out_slot_stride;
 
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int W = a.ksplit;
@@ -210,105 +215,130 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
     ln.c = l;
     ln.sh = (ln.c & 1) * 16;
     ln.upper = ln.c >= 2;
-
-    // Prologue: activation loads first, the first weight buffer right behind
-    // them, then the LDS writes -- so HBM requests are in flight while the
-    // activation is staged.
-    const uint4 *src = reinterpret_cast<const uint4 *>(q);
-    uint4 *dst = reinterpret_cast<uint4 *>(ys);
-    const int n16 = NT * n_sb * 16;  // even; blockDim is even: lanes 2k, 2k+1 are in or out together
-    uint4 sv[kQ4KStageRegs];
-#pragma unroll
-    for (int k = 0; k < kQ4KStageRegs; k++) sv[k] = src[min(tid + k * nthreads, n16 - 1)];
-    const float yd0 = yd[min(tid, NT * n_sb - 1)];
-
+    const int c16 = n_sb * 16;       // 16-byte chunks per activation row
+    const int n16 = NT * c16;        // even; blockDim is even: lanes 2k, 2k+1 are in or out together
     constexpr int U = Q4KRegs::U;
-    Q4KRegs ra, rb;
-    __builtin_amdgcn_sched_barrier(0);
-    q4k_load(ra, wtile, a.sb_stride, r, lane, s0, s1);
-    __builtin_amdgcn_sched_barrier(0);
+
+    for (int p0 = 0; p0 < n_assign; p0 += NT) {
+        // Activation row of local token t (clamped to the group's last assignment; extra tokens store nothing).
+        auto act_row = [&](int t) -> int64_t {
+            const int j = a0 + min(p0 + t, n_assign - 1);
+            return a.group_rows ? a.group_rows[j] : j;
+        };
+        // Prologue: activation loads first, the first weight buffer right behind
+        // them, then the LDS writes -- so HBM requests are in flight while the
+        // activation is staged.
+        uint4 *dst = reinterpret_cast<uint4 *>(ys);
+        uint4 sv[kQ4KStageRegs];
+#pragma unroll
+        for (int k = 0; k < kQ4KStageRegs; k++) {
+            const int i = min(tid + k * nthreads, n16 - 1);
+            const int t = NT == 1 ? 0 : i / c16;
+            sv[k] = reinterpret_cast<const uint4 *>(a.q + act_row(t) * n_sb * 256)[i - t * c16];
+        }
+        float yd0;
+        {
+            const int i = min(tid, NT * n_sb - 1);
+            const int t = NT == 1 ? 0 : i / n_sb;
+            yd0 = a.yd[act_row(t) * n_sb + (i - t * n_sb)];
+        }
+
+        Q4KRegs ra, rb;
+        __builtin_amdgcn_sched_barrier(0);
+        q4k_load(ra, wtile, a.sb_stride, r, lane, s0, s1);
+        __builtin_amdgcn_sched_barrier(0);
 
 #pragma unroll
-    for (int k = 0; k < kQ4KStageRegs; k++) {
-        const int i = tid + k * nthreads;
-        int s = bytesum16(sv[k]);
-        s += row_shr_i32<1>(s);
-        if (i < n16) {
-            dst[i] = sv[k];
-            if (i & 1) bsum[i >> 1] = s;
-        }
-    }
-    for (int i = tid + kQ4KStageRegs * nthreads; i < n16; i += nthreads) {
-        const uint4 v = src[i];
-        dst[i] = v;
-        int s = bytesum16(v);
-        s += row_shr_i32<1>(s);
-        if (i & 1) bsum[i >> 1] = s;
-    }
-    if (tid < NT * n_sb) yds[tid] = yd0;
-    for (int i = tid + nthreads; i < NT * n_sb; i += nthreads) yds[i] = yd[i];
-    __syncthreads();
-
-    int32_t *ints_row = nullptr;
-    if constexpr (INTS) {
-        if (a.ints && leader && live) ints_row = a.ints + (band * a.rows + row) * static_cast<int64_t>(n_sb) * 2;
-    }
-
-    float acc[NT];
-#pragma unroll
-    for (int t = 0; t < NT; t++) acc[t] = 0.0f;
-
-    // Two register buffers alternate: the next buffer's loads are issued, then
-    // the current one is consumed.  The last buffer is consumed without issuing
-    // anything, so no load is wasted; sched_barrier keeps the loads ahead of
-    // the arithmetic they overlap with.
-    for (int sb = s0;;) {
-        if (sb + U >= s1) {
-            q4k_compute<NT, INTS>(ra, ln, sb, s1, ys, bsum, yds, n_sb, acc, ints_row);
-            break;
-        }
-        q4k_load(rb, wtile, a.sb_stride, r, lane, sb + U, s1);
-        __builtin_amdgcn_sched_barrier(0);
-        q4k_compute<NT, INTS>(ra, ln, sb, s1, ys, bsum, yds, n_sb, acc, ints_row);
-        __builtin_amdgcn_sched_barrier(0);
-        sb += U;
-        if (sb + U >= s1) {
-            q4k_compute<NT, INTS>(rb, ln, sb, s1, ys, bsum, yds, n_sb, acc, ints_row);
-            break;
-        }
-        q4k_load(ra, wtile, a.sb_stride, r, lane, sb + U, s1);
-        __builtin_amdgcn_sched_barrier(0);
-        q4k_compute<NT, INTS>(rb, ln, sb, s1, ys, bsum, yds, n_sb, acc, ints_row);
-        __builtin_amdgcn_sched_barrier(0);
-        sb += U;
-    }
-
-    if (W == 1) {
-        if (leader && live) {
-#pragma unroll
-            for (int t = 0; t < NT; t++) {
-                float v = acc[t];
-                if (NT == 1 && a.residual) v = v + a.residual[row];
-                out[static_cast<int64_t>(t) * a.rows + row] = v;
+        for (int k = 0; k < kQ4KStageRegs; k++) {
+            const int i = tid + k * nthreads;
+            int s = bytesum16(sv[k]);
+            s += row_shr_i32<1>(s);
+            if (i < n16) {
+                dst[i] = sv[k];
+                if (i & 1) bsum[i >> 1] = s;
             }
         }
-        return;
-    }
-    if (leader) {
+        for (int i = tid + kQ4KStageRegs * nthreads; i < n16; i += nthreads) {
+            const int t = NT == 1 ? 0 : i / c16;
+            const uint4 v = reinterpret_cast<const uint4 *>(a.q + act_row(t) * n_sb * 256)[i - t * c16];
+            dst[i] = v;
+            int s = bytesum16(v);
+            s += row_shr_i32<1>(s);
+            if (i & 1) bsum[i >> 1] = s;
+        }
+        if (tid < NT * n_sb) yds[tid] = yd0;
+        for (int i = tid + nthreads; i < NT * n_sb; i += nthreads) {
+            const int t = NT == 1 ? 0 : i / n_sb;
+            yds[i] = a.yd[act_row(t) * n_sb + (i - t * n_sb)];
+        }
+        __syncthreads();
+
+        int32_t *ints_row = nullptr;
+        if constexpr (INTS) {
+            if (a.ints && leader && live) ints_row = a.ints + (band * a.rows + row) * static_cast<int64_t>(n_sb) * 2;
+        }
+
+        float acc[NT];
 #pragma unroll
-        for (int t = 0; t < NT; t++) part[(wave * NT + t) * RPW + r] = acc[t];
-    }
-    __syncthreads();
-    for (int i = tid; i < a.tiles_per_wg * NT * RPW; i += nthreads) {
-        const int rr = i % RPW;
-        const int t = (i / RPW) % NT;
-        const int tw = i / (RPW * NT);
-        const int orow = (blockIdx.x * a.tiles_per_wg + tw) * RPW + rr;
-        if (orow >= a.rows) continue;
-        float v = part[((tw * W) * NT + t) * RPW + rr];
-        for (int k = 1; k < W; k++) v = v + part[((tw * W + k) * NT + t) * RPW + rr];
-        if (NT == 1 && a.residual) v = v + a.residual[orow];
-        out[static_cast<int64_t>(t) * a.rows + orow] = v;
+        for (int t = 0; t < NT; t++) acc[t] = 0.0f;
+
+        // Two register buffers alternate: the next buffer's loads are issued, then
+        // the current one is consumed.  The last buffer is consumed without issuing
+        // anything, so no load is wasted; sched_barrier keeps the loads ahead of
+        // the arithmetic they overlap with.
+        for (int sb = s0;;) {
+            if (sb + U >= s1) {
+                q4k_compute<NT, INTS>(ra, ln, sb, s1, ys, bsum, yds, n_sb, acc, ints_row);
+                break;
+            }
+            q4k_load(rb, wtile, a.sb_stride, r, lane, sb + U, s1);
+            __builtin_amdgcn_sched_barrier(0);
+            q4k_compute<NT, INTS>(ra, ln, sb, s1, ys, bsum, yds, n_sb, acc, ints_row);
+            __builtin_amdgcn_sched_barrier(0);
+            sb += U;
+            if (sb + U >= s1) {
+                q4k_compute<NT, INTS>(rb, ln, sb, s1, ys, bsum, yds, n_sb, acc, ints_row);
+                break;
+            }
+            q4k_load(ra, wtile, a.sb_stride, r, lane, sb + U, s1);
+            __builtin_amdgcn_sched_barrier(0);
+            q4k_compute<NT, INTS>(rb, ln, sb, s1, ys, bsum, yds, n_sb, acc, ints_row);
+            __builtin_amdgcn_sched_barrier(0);
+            sb += U;
+        }
+
+        float *out = a.out + static_cast<int64_t>(a0 + p0) * a.rows;  // output row of local token 0
+        const int n_here = min(NT, n_assign - p0);
+        if (W == 1) {
+            if (leader && live) {
+#pragma unroll
+                for (int t = 0; t < NT; t++) {
+                    if (t < n_here) {
+                        float v = acc[t];
+                        if (NT == 1 && a.residual) v = v + a.residual[row];
+                        out[static_cast<int64_t>(t) * a.rows + row] = v;
+                    }
+                }
+            }
+        } else {
+            if (leader) {
+#pragma unroll
+                for (int t = 0; t < NT; t++) part[(wave * NT + t) * RPW + r] = acc[t];
+            }
+            __syncthreads();
+            for (int i = tid; i < a.tiles_per_wg * NT * RPW; i += nthreads) {
+                const int rr = i % RPW;
+                const int t = (i / RPW) % NT;
+                const int tw = i / (RPW * NT);
+                const int orow = (blockIdx.x * a.tiles_per_wg + tw) * RPW + rr;
+                if (orow >= a.rows || t >= n_here) continue;
+                float v = part[((tw * W) * NT + t) * RPW + rr];
+                for (int k = 1; k < W; k++) v = v + part[((tw * W + k) * NT + t) * RPW + rr];
+                if (NT == 1 && a.residual) v = v + a.residual[orow];
+                out[static_cast<int64_t>(t) * a.rows + orow] = v;
+            }
+        }
+        if (p0 + NT < n_assign) __syncthreads();  // the next pass overwrites the staged activation
     }
 }
 
@@ -340,7 +370,7 @@ static Q4KShape pick_shape(int64_t rows, int64_t n_sb) {
 }
 
 template <int NT>
-static int launch_q4k_nt(Q4KArgs ka, const Q4KShape &shape, int n_bands, bool ints, hipStream_t st) {
+static int launch_q4k_nt(Q4KArgs ka, const Q4KShape &shape, int n_groups, bool ints, hipStream_t st) {
     const int waves = shape.ksplit * shape.tiles_per_wg;
     const int64_t tiles = (ka.rows + 15) / 16;
     const unsigned gx = static_cast<unsigned>((tiles + shape.tiles_per_wg - 1) / shape.tiles_per_wg);
@@ -350,45 +380,63 @@ static int launch_q4k_nt(Q4KArgs ka, const Q4KShape &shape, int n_bands, bool in
     ka.ksplit = shape.ksplit;
     ka.tiles_per_wg = shape.tiles_per_wg;
     if (ints && NT == 1)
-        hipLaunchKernelGGL((gemv_q4k_kernel<1, true>), dim3(gx, n_bands), dim3(64 * waves), lds, st, ka);
+        hipLaunchKernelGGL((gemv_q4k_kernel<1, true>), dim3(gx, n_groups), dim3(64 * waves), lds, st, ka);
     else
-        hipLaunchKernelGGL((gemv_q4k_kernel<NT, false>), dim3(gx, n_bands), dim3(64 * waves), lds, st, ka);
+        hipLaunchKernelGGL((gemv_q4k_kernel<NT, false>), dim3(gx, n_groups), dim3(64 * waves), lds, st, ka);
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
+}
+
+// Largest token count per pass (8, 4, 2 or 1) whose LDS staging fits 64 KB.
+static int cap_nt(int64_t want, int n_sb, int waves) {
+    int nt = want >= 8 ? 8 : (want >= 4 ? 4 : (want >= 2 ? 2 : 1));
+    while (nt > 1 && static_cast<size_t>(nt) * n_sb * (256 + 32) + ((static_cast<size_t>(nt) * n_sb + 3) & ~size_t(3)) * 4 +
+                             static_cast<size_t>(waves) * nt * 16 * 4 > 64 * 1024)
+        nt >>= 1;
+    return nt;
+}
+
+static int launch_q4k_pick_nt(const Q4KArgs &ka, const Q4KShape &shape, int n_groups, int nt, bool ints, hipStream_t st) {
+    switch (nt) {
+        case 8: return launch_q4k_nt<8>(ka, shape, n_groups, false, st);
+        case 4: return launch_q4k_nt<4>(ka, shape, n_groups, false, st);
+        case 2: return launch_q4k_nt<2>(ka, shape, n_groups, false, st);
+        default: return launch_q4k_nt<1>(ka, shape, n_groups, ints, st);
+    }
 }
 
 int launch_gemv_q4k(const MatArgs &a, hipStream_t st) {
     const cml_weight *w = a.w;
     if (w->rows == 0 || a.n_tokens == 0) return CML_OK;
+    const bool grouped = a.group_offsets != nullptr;
     Q4KArgs ka;
     ka.w = w->planes.p[0];
     ka.sb_stride = w->planes.row_stride[0];
-    ka.rows = static_cast<int>(a.band_ids ? a.band_rows : w->rows);
-    if (a.band_ids && (ka.rows % 16) != 0) return fail(CML_ERR_UNSUPPORTED, "Q4_K expert bands must be whole 16-row tiles (%d rows)", ka.rows);
+    ka.rows = static_cast<int>(grouped ? a.band_rows : w->rows);
+    if (grouped && (ka.rows % 16) != 0) return fail(CML_ERR_UNSUPPORTED, "Q4_K expert bands must be whole 16-row tiles (%d rows)", ka.rows);
     ka.n_sb = static_cast<int>(w->nb);
     ka.residual = a.residual;
     ka.ints = a.ints;
-    ka.band_ids = a.band_ids;
-    ka.act_slot_stride = a.act_per_slot ? a.n_tokens : 0;
-    ka.out_slot_stride = a.n_tokens * static_cast<int64_t>(ka.rows);
+    ka.group_offsets = a.group_offsets;
+    ka.group_rows = a.group_rows;
     const Q4KShape shape = pick_shape(ka.rows, ka.n_sb);
-    const int n_bands = a.n_bands > 0 ? a.n_bands : 1;
-    // Tokens are served in passes of up to 8 rows of activations.
+    if (grouped) {
+        // One launch: every group walks its own assignments in passes of NT
+        // (NT sized for the most a single group can hold).
+        ka.q = a.q;
+        ka.yd = a.scales;
+        ka.out = a.out;
+        const int nt = cap_nt(a.n_tokens, ka.n_sb, shape.ksplit * shape.tiles_per_wg);
+        return launch_q4k_pick_nt(ka, shape, a.n_groups, nt, false, st);
+    }
+    // Plain call: tokens are served in launches of up to 8 activation rows.
     int64_t t0 = 0;
     while (t0 < a.n_tokens) {
-        const int64_t left = a.n_tokens - t0;
-        const int nt = left >= 8 ? 8 : (left >= 4 ? 4 : (left >= 2 ? 2 : 1));
+        const int nt = cap_nt(a.n_tokens - t0, ka.n_sb, shape.ksplit * shape.tiles_per_wg);
         ka.q = a.q + t0 * w->cols;
         ka.yd = a.scales + t0 * w->nb;
         ka.out = a.out + t0 * ka.rows;
-        int rc;
-        switch (nt) {
-            case 8: rc = launch_q4k_nt<8>(ka, shape, n_bands, false, st); break;
-            case 4: rc = launch_q4k_nt<4>(ka, shape, n_bands, false, st); break;
-            case 2: rc = launch_q4k_nt<2>(ka, shape, n_bands, false, st); break;
-            default: rc = launch_q4k_nt<1>(ka, shape, n_bands, a.ints != nullptr, st); break;
-        }
-        if (rc != CML_OK) return rc;
+        if (int rc = launch_q4k_pick_nt(ka, shape, 1, nt, a.ints != nullptr, st)) return rc;
         t0 += nt;
     }
     return CML_OK;

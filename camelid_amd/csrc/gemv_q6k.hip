@@ -256,20 +256,21 @@ static int launch_q6k_nt(const Q6KArgs &ka, int n_bands, bool ints, hipStream_t 
 int launch_gemv_q6k(const MatArgs &a, hipStream_t st) {
     const cml_weight *w = a.w;
     if (w->rows == 0 || a.n_tokens == 0) return CML_OK;
+    if (a.group_offsets) return fail(CML_ERR_UNSUPPORTED, "grouped (mixture-of-experts) dispatch is built for Q4_K weights only");
     Q6KArgs ka;
     ka.ql = w->planes.p[0]; ka.ql_stride = w->planes.row_stride[0];
     ka.qh = w->planes.p[1]; ka.qh_stride = w->planes.row_stride[1];
     ka.sc = w->planes.p[2]; ka.sc_stride = w->planes.row_stride[2];
     ka.d = w->planes.p[3];  ka.d_stride = w->planes.row_stride[3];
-    ka.rows = static_cast<int>(a.band_ids ? a.band_rows : w->rows);
+    ka.rows = static_cast<int>(w->rows);
     ka.n_sb = static_cast<int>(w->nb);
     ka.residual = a.residual;
     ka.ints = a.ints;
-    ka.band_ids = a.band_ids;
-    ka.act_slot_stride = a.act_per_slot ? a.n_tokens : 0;
+    ka.band_ids = nullptr;
+    ka.act_slot_stride = 0;
     ka.out_slot_stride = a.n_tokens * static_cast<int64_t>(ka.rows);
     ka.ksplit = pick_ksplit_q6k(ka.rows, ka.n_sb);
-    const int n_bands = a.n_bands > 0 ? a.n_bands : 1;
+    const int n_bands = 1;
     int64_t t0 = 0;
     while (t0 < a.n_tokens) {
         const int64_t left = a.n_tokens - t0;

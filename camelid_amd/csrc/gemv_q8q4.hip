@@ -215,14 +215,14 @@ static int launch_b32_p(const MatArgs &a, hipStream_t st) {
     ba.q_stride = w->planes.row_stride[0];
     ba.scales = w->planes.p[1];
     ba.s_stride = w->planes.row_stride[1];
-    ba.rows = static_cast<int>(a.band_ids ? a.band_rows : w->rows);
+    ba.rows = static_cast<int>(w->rows);
     ba.nb = static_cast<int>(w->nb);
     ba.residual = a.residual;
     ba.ints = a.ints;
-    ba.band_ids = a.band_ids;
-    ba.act_slot_stride = a.act_per_slot ? a.n_tokens : 0;
+    ba.band_ids = nullptr;
+    ba.act_slot_stride = 0;
     ba.out_slot_stride = a.n_tokens * static_cast<int64_t>(ba.rows);
-    const int n_bands = a.n_bands > 0 ? a.n_bands : 1;
+    const int n_bands = 1;
     int64_t t0 = 0;
     while (t0 < a.n_tokens) {
         const int64_t left = a.n_tokens - t0;
@@ -246,6 +246,7 @@ static int launch_b32_p(const MatArgs &a, hipStream_t st) {
 template <int FMT>
 static int launch_b32(const MatArgs &a, hipStream_t st) {
     if (a.w->rows == 0 || a.n_tokens == 0) return CML_OK;
+    if (a.group_offsets) return fail(CML_ERR_UNSUPPORTED, "grouped (mixture-of-experts) dispatch is built for Q4_K weights only");
     // 16 lanes per row by default; 8 when rows are short enough that half the lanes would idle.
     int p = env_int(FMT == CML_Q8_0 ? "CAMELID_HIP_Q8_0_LANES" : "CAMELID_HIP_Q4_0_LANES", 0);
     if (p != 8 && p != 16) p = (a.w->nb <= 8) ? 8 : 16;

@@ -1,19 +1,309 @@
-// Mixture-of-experts dispatch (placeholder until the routed kernels land).
+// Mixture-of-experts dispatch for quantized stacked experts.
+//
+// What the reference does per token (mixtral_moe_ffn, src/inference.rs:14142-14280):
+// route (softmax_top_k, :13940-13991), then for every selected expert in routed
+// order  y = down_e( silu(gate_e x) * up_e x )  and  out += y * weight.
+// The device version keeps that arithmetic per (token, expert) cell and only
+// changes the schedule: assignments are grouped by expert (the reference's
+// expert-grouped plan for K-token batches, Gemma4RouteUnionPlan,
+// src/gemma4_runtime.rs:12309-12424), so each touched expert matrix is streamed
+// once for all the tokens routed to it, and the weighted sum walks each token's
+// experts in router order (moe_weighted_sum_batched, src/cuda_resident.rs:6369-6389).
+// Nothing here synchronises with the host: the grouping is built on the device
+// and the expert kernels are launched over all experts, idle ones exiting at once.
+#include "cml_device.hpp"
 #include "cml_host.hpp"
+
+#pragma clang fp contract(off)
+
+namespace cml {
+
+constexpr int kMaxExperts = 64;
+
+// f32::total_cmp as an integer key (larger key = greater value).
+__device__ __forceinline__ int total_key(float v) {
+    const int b = __builtin_bit_cast(int, v);
+    return b ^ static_cast<int>(static_cast<unsigned>(b >> 31) >> 1);
+}
+
+// One thread per token.  reference softmax_top_k, src/inference.rs:13940-13991.
+__global__ __launch_bounds__(64) void moe_route_kernel(const float *__restrict__ logits, int64_t n_tokens, int n_experts,
+                                                       int k, int32_t *__restrict__ idx_out, float *__restrict__ w_out) {
+    const int64_t t = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (t >= n_tokens) return;
+    const float *lg = logits + t * n_experts;
+    int sel_idx[kMaxExperts];
+    float sel_w[kMaxExperts];
+    unsigned long long taken = 0;
+    // top-k by logit (total order, descending), ties to the lower index
+    for (int s = 0; s < k; s++) {
+        int best = -1, best_key = 0;
+        for (int e = 0; e < n_experts; e++) {
+            if ((taken >> e) & 1ull) continue;
+            const int key = total_key(lg[e]);
+            if (best < 0 || key > best_key) {
+                best = e;
+                best_key = key;
+            }
+        }
+        taken |= 1ull << best;
+        sel_idx[s] = best;
+        sel_w[s] = lg[best];
+    }
+    float mx = -INFINITY;
+    for (int s = 0; s < k; s++) mx = fmaxf(mx, sel_w[s]);
+    float sum = 0.0f;
+    for (int s = 0; s < k; s++) {
+        const float v = sel_w[s];
+        const float wv = (fabsf(v) < INFINITY) ? expf(v - mx) : 0.0f;  // is_finite: NaN and inf give 0
+        sel_w[s] = wv;
+        sum = sum + wv;
+    }
+    if (sum > 0.0f) {
+        for (int s = 0; s < k; s++) sel_w[s] = sel_w[s] / sum;
+    } else {
+        const float uniform = 1.0f / static_cast<float>(k);
+        for (int s = 0; s < k; s++) sel_w[s] = uniform;
+    }
+    // re-sort by weight (descending), ties to the lower index: insertion sort, stable
+    for (int i = 1; i < k; i++) {
+        const int ci = sel_idx[i];
+        const float cw = sel_w[i];
+        const int ck = total_key(cw);
+        int j = i - 1;
+        while (j >= 0) {
+            const int kj = total_key(sel_w[j]);
+            const bool before = (ck > kj) || (ck == kj && ci < sel_idx[j]);
+            if (!before) break;
+            sel_idx[j + 1] = sel_idx[j];
+            sel_w[j + 1] = sel_w[j];
+            j--;
+        }
+        sel_idx[j + 1] = ci;
+        sel_w[j + 1] = cw;
+    }
+    for (int s = 0; s < k; s++) {
+        idx_out[t * k + s] = sel_idx[s];
+        w_out[t * k + s] = sel_w[s];
+    }
+}
+
+// Group the n_tokens*k assignments by expert, keeping (token, rank) order
+// inside each group.  One workgroup; thread e builds group e.
+//   offsets[e..e+1)   assignment range of expert e
+//   assign_token[j]   token whose activation assignment j reads
+//   slot_to_assign[t*k+s]  where (token t, rank s) landed
+__global__ __launch_bounds__(64) void moe_plan_kernel(const int32_t *__restrict__ idx, int n_slots, int n_experts, int k,
+                                                      int32_t *__restrict__ offsets, int32_t *__restrict__ assign_token,
+                                                      int32_t *__restrict__ slot_to_assign) {
+    __shared__ int count[kMaxExperts + 1];
+    const int e = threadIdx.x;
+    int mine = 0;
+    if (e < n_experts) {
+        for (int i = 0; i < n_slots; i++) mine += (idx[i] == e);
+        count[e] = mine;
+    }
+    __syncthreads();
+    if (e < n_experts) {
+        int start = 0;
+        for (int j = 0; j < e; j++) start += count[j];
+        offsets[e] = start;
+        if (e == n_experts - 1) offsets[n_experts] = start + mine;
+        int at = start;
+        for (int i = 0; i < n_slots; i++) {
+            if (idx[i] == e) {
+                assign_token[at] = i / k;
+                slot_to_assign[i] = at;
+                at++;
+            }
+        }
+    }
+}
+
+__device__ __forceinline__ int nearest_int_magic_(float f) {
+    const float val = f + 12582912.0f;
+    return static_cast<int>(__builtin_bit_cast(uint32_t, val) & 0x007fffffu) - 0x00400000;
+}
+
+// h = silu(g) * u (reference CpuTensor::silu_mul, src/tensor/mod.rs:2610-2634:
+// (a / (1 + exp(-a))) * b), quantized to Q8_K on the fly (reference
+// quantize_q8_k_blocks, src/inference.rs:23121-23152).  One wave per 256-value
+// super-block, lane l holds values 4l..4l+3 -- the layout of quantize_q8_k_kernel.
+__global__ __launch_bounds__(256) void silu_mul_quantize_q8k_kernel(const float *__restrict__ g, const float *__restrict__ u,
+                                                                    int64_t n_sb, int8_t *__restrict__ q, float *__restrict__ d) {
+    const int lane = threadIdx.x & 63;
+    const int64_t sb = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (sb >= n_sb) return;
+    const float4 gv = reinterpret_cast<const float4 *>(g + sb * 256)[lane];
+    const float4 uv = reinterpret_cast<const float4 *>(u + sb * 256)[lane];
+    float4 v;
+    v.x = (gv.x / (1.0f + expf(-gv.x))) * uv.x;
+    v.y = (gv.y / (1.0f + expf(-gv.y))) * uv.y;
+    v.z = (gv.z / (1.0f + expf(-gv.z))) * uv.z;
+    v.w = (gv.w / (1.0f + expf(-gv.w))) * uv.w;
+    const float a0 = fabsf(v.x), a1 = fabsf(v.y), a2 = fabsf(v.z), a3 = fabsf(v.w);
+    float amax = fmaxf(fmaxf(a0, a1), fmaxf(a2, a3));
+#pragma unroll
+    for (int m = 1; m < 64; m <<= 1) amax = fmaxf(amax, __shfl_xor(amax, m));
+    int first = 1 << 20;
+    if (a3 == amax) first = lane * 4 + 3;
+    if (a2 == amax) first = lane * 4 + 2;
+    if (a1 == amax) first = lane * 4 + 1;
+    if (a0 == amax) first = lane * 4 + 0;
+#pragma unroll
+    for (int m = 1; m < 64; m <<= 1) first = min(first, __shfl_xor(first, m));
+    uint32_t *qo = reinterpret_cast<uint32_t *>(q + sb * 256);
+    if (amax == 0.0f || first >= 256) {
+        qo[lane] = 0u;
+        if (lane == 0) d[sb] = 0.0f;
+        return;
+    }
+    const int kk = first & 3;
+    const float mine = kk == 0 ? v.x : (kk == 1 ? v.y : (kk == 2 ? v.z : v.w));
+    const float mx = __shfl(mine, first >> 2);
+    const float iscale = -127.0f / mx;
+    const int q0 = min(nearest_int_magic_(iscale * v.x), 127);
+    const int q1 = min(nearest_int_magic_(iscale * v.y), 127);
+    const int q2 = min(nearest_int_magic_(iscale * v.z), 127);
+    const int q3 = min(nearest_int_magic_(iscale * v.w), 127);
+    qo[lane] = (static_cast<uint32_t>(q0) & 0xffu) | ((static_cast<uint32_t>(q1) & 0xffu) << 8) |
+               ((static_cast<uint32_t>(q2) & 0xffu) << 16) | ((static_cast<uint32_t>(q3) & 0xffu) << 24);
+    if (lane == 0) d[sb] = 1.0f / iscale;
+}
+
+// out[t][c] = ((0 + y[a(t,0)][c]*w[t][0]) + y[a(t,1)][c]*w[t][1]) + ...  (reference
+// src/inference.rs:14255-14257: `output += expert_out * weight`, routed order,
+// multiply and add rounded separately).
+__global__ __launch_bounds__(256) void moe_weighted_sum_kernel(const float *__restrict__ y, const int32_t *__restrict__ slot_to_assign,
+                                                               const float *__restrict__ weight, int k, int64_t hidden,
+                                                               float *__restrict__ out) {
+    const int64_t c = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    const int64_t t = blockIdx.y;
+    if (c >= hidden) return;
+    float acc = 0.0f;
+    for (int s = 0; s < k; s++) {
+        const int64_t a = slot_to_assign[t * k + s];
+        acc = acc + y[a * hidden + c] * weight[t * k + s];
+    }
+    out[t * hidden + c] = acc;
+}
+
+struct MoeWorkspace {
+    int8_t *xq;
+    float *xd;
+    int32_t *offsets, *assign_token, *slot_to_assign;
+    float *g, *u, *y, *hd;
+    int8_t *hq;
+    size_t total;
+};
+
+static MoeWorkspace carve(void *base, int64_t hidden, int64_t ff, int64_t n_tokens, int k, int n_experts) {
+    MoeWorkspace w;
+    size_t at = 0;
+    auto take = [&](size_t bytes) {
+        const size_t here = at;
+        at += (bytes + 255) & ~size_t(255);
+        return base ? static_cast<uint8_t *>(base) + here : nullptr;
+    };
+    const size_t T = static_cast<size_t>(n_tokens), A = T * static_cast<size_t>(k);
+    w.xq = reinterpret_cast<int8_t *>(take(T * hidden));
+    w.xd = reinterpret_cast<float *>(take(T * (hidden / 256) * 4));
+    w.offsets = reinterpret_cast<int32_t *>(take((static_cast<size_t>(n_experts) + 1) * 4));
+    w.assign_token = reinterpret_cast<int32_t *>(take(A * 4));
+    w.slot_to_assign = reinterpret_cast<int32_t *>(take(A * 4));
+    w.g = reinterpret_cast<float *>(take(A * ff * 4));
+    w.u = reinterpret_cast<float *>(take(A * ff * 4));
+    w.hq = reinterpret_cast<int8_t *>(take(A * ff));
+    w.hd = reinterpret_cast<float *>(take(A * (ff / 256) * 4));
+    w.y = reinterpret_cast<float *>(take(A * hidden * 4));
+    w.total = at;
+    return w;
+}
+
+}  // namespace cml
 
 using namespace cml;
 
 extern "C" {
 
-int cml_moe_route_top_k(const float *, int64_t, int, int, int32_t *, float *, cml_stream_t) {
-    return fail(CML_ERR_UNSUPPORTED, "cml_moe_route_top_k is not built yet");
+int cml_moe_route_top_k(const float *logits_dev, int64_t n_tokens, int n_experts, int k, int32_t *idx_dev,
+                        float *weight_dev, cml_stream_t stream) {
+    if (!ready()) return fail(CML_ERR_UNAVAILABLE, "cml_init has not succeeded");
+    if (n_tokens < 0 || n_experts <= 0 || k <= 0) return fail(CML_ERR_SHAPE, "bad routing shape");
+    if (n_experts > kMaxExperts) return fail(CML_ERR_UNSUPPORTED, "at most %d experts", kMaxExperts);
+    if (k > n_experts) return fail(CML_ERR_SHAPE, "top-%d of %d experts", k, n_experts);
+    if (n_tokens == 0) return CML_OK;
+    if (!logits_dev || !idx_dev || !weight_dev) return fail(CML_ERR_INVALID, "null pointer");
+    const unsigned grid = static_cast<unsigned>((n_tokens + 63) / 64);
+    hipLaunchKernelGGL(moe_route_kernel, dim3(grid), dim3(64), 0, as_stream(stream), logits_dev, n_tokens, n_experts, k, idx_dev, weight_dev);
+    CML_HIP_TRY(hipGetLastError());
+    return CML_OK;
 }
 
-size_t cml_moe_workspace_bytes(int, int64_t, int64_t, int64_t, int, int) { return 0; }
+size_t cml_moe_workspace_bytes(int fmt, int64_t hidden, int64_t ff, int64_t n_tokens, int k, int n_experts) {
+    if (fmt != CML_Q4_K || hidden <= 0 || ff <= 0 || n_tokens <= 0 || k <= 0 || n_experts <= 0) return 0;
+    return carve(nullptr, hidden, ff, n_tokens, k, n_experts).total;
+}
 
-int cml_moe_ffn(const cml_weight *, const cml_weight *, const cml_weight *, int, int, const int32_t *, const float *,
-                const float *, int64_t, float *, void *, size_t, cml_stream_t) {
-    return fail(CML_ERR_UNSUPPORTED, "cml_moe_ffn is not built yet");
+int cml_moe_ffn(const cml_weight *gate, const cml_weight *up, const cml_weight *down, int n_experts, int k,
+                const int32_t *idx_dev, const float *weight_dev, const float *x_dev, int64_t n_tokens, float *out_dev,
+                void *workspace_dev, size_t workspace_bytes, cml_stream_t stream) {
+    if (!ready()) return fail(CML_ERR_UNAVAILABLE, "cml_init has not succeeded");
+    if (!gate || !up || !down) return fail(CML_ERR_INVALID, "null weight");
+    if (gate->fmt != CML_Q4_K || up->fmt != CML_Q4_K || down->fmt != CML_Q4_K)
+        return fail(CML_ERR_UNSUPPORTED, "mixture-of-experts dispatch is built for Q4_K expert matrices only");
+    if (n_experts <= 0 || n_experts > kMaxExperts || k <= 0 || k > n_experts || n_tokens < 0)
+        return fail(CML_ERR_SHAPE, "bad routing shape (%d experts, top-%d)", n_experts, k);
+    const int64_t hidden = gate->cols, ff = down->cols;
+    if (up->cols != hidden || gate->rows != up->rows || gate->rows != ff * n_experts || down->rows != hidden * n_experts)
+        return fail(CML_ERR_SHAPE, "expert matrices do not stack to %d experts of %lld x %lld", n_experts, (long long)ff, (long long)hidden);
+    if (hidden % 256 || ff % 256) return fail(CML_ERR_SHAPE, "hidden and ff must be multiples of 256");
+    if (n_tokens == 0) return CML_OK;
+    if (!idx_dev || !weight_dev || !x_dev || !out_dev || !workspace_dev) return fail(CML_ERR_INVALID, "null pointer");
+    if ((reinterpret_cast<uintptr_t>(x_dev) & 15u) || (reinterpret_cast<uintptr_t>(workspace_dev) & 255u))
+        return fail(CML_ERR_INVALID, "x must be 16-byte and the workspace 256-byte aligned");
+    const MoeWorkspace ws = carve(workspace_dev, hidden, ff, n_tokens, k, n_experts);
+    if (workspace_bytes < ws.total) return fail(CML_ERR_SHAPE, "workspace of %zu bytes given, %zu needed", workspace_bytes, ws.total);
+    hipStream_t st = as_stream(stream);
+    const int n_slots = static_cast<int>(n_tokens * k);
+
+    if (int rc = launch_quantize_q8_k(x_dev, n_tokens, hidden, ws.xq, ws.xd, st)) return rc;
+    hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(64), 0, st, idx_dev, n_slots, n_experts, k, ws.offsets, ws.assign_token, ws.slot_to_assign);
+    CML_HIP_TRY(hipGetLastError());
+
+    MatArgs a;
+    a.residual = nullptr;
+    a.ints = nullptr;
+    a.group_offsets = ws.offsets;
+    a.n_groups = n_experts;
+    a.n_tokens = n_tokens;  // the most assignments one expert can receive
+    // gate and up: every assignment reads its token's activation
+    a.q = ws.xq;
+    a.scales = ws.xd;
+    a.group_rows = ws.assign_token;
+    a.band_rows = ff;
+    a.w = gate;
+    a.out = ws.g;
+    if (int rc = launch_gemv_q4k(a, st)) return rc;
+    a.w = up;
+    a.out = ws.u;
+    if (int rc = launch_gemv_q4k(a, st)) return rc;
+    // h = silu(g) * u, quantized per assignment
+    const int64_t h_sb = static_cast<int64_t>(n_slots) * (ff / 256);
+    hipLaunchKernelGGL(silu_mul_quantize_q8k_kernel, dim3(static_cast<unsigned>((h_sb + 3) / 4)), dim3(256), 0, st, ws.g, ws.u, h_sb, ws.hq, ws.hd);
+    CML_HIP_TRY(hipGetLastError());
+    // down: assignment j reads its own h
+    a.q = ws.hq;
+    a.scales = ws.hd;
+    a.group_rows = nullptr;
+    a.band_rows = hidden;
+    a.w = down;
+    a.out = ws.y;
+    if (int rc = launch_gemv_q4k(a, st)) return rc;
+    hipLaunchKernelGGL(moe_weighted_sum_kernel, dim3(static_cast<unsigned>((hidden + 255) / 256), static_cast<unsigned>(n_tokens)), dim3(256), 0, st,
+                       ws.y, ws.slot_to_assign, weight_dev, k, hidden, out_dev);
+    CML_HIP_TRY(hipGetLastError());
+    return CML_OK;
 }
 
 }  // extern "C"
