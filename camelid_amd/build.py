@@ -20,6 +20,7 @@ SOURCES = [
     "quantize.hip",
     "layout.hip",
     "gemv_q4k.hip",
+    "gemm_q4k_mfma.hip",
     "gemv_q8q4.hip",
     "gemv_q6k.hip",
     "moe.hip",
@@ -38,6 +39,8 @@ FLAGS = [
     "-fPIC",
     "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # MFMA results straight into VGPRs: the integer epilogue reads every one of them
+    "-mllvm", "-amdgpu-mfma-vgpr-form=1",
     "-Wall",
     "-Wno-unused-function",
     "-Wno-unknown-warning-option",

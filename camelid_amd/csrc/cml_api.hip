@@ -418,7 +418,15 @@ int cml_dequantize(const cml_weight *w, float *out_dev, cml_stream_t stream) {
 static int dispatch(const MatArgs &a, hipStream_t st) {
     int rc;
     switch (a.w->fmt) {
-        case CML_Q4_K: rc = launch_gemv_q4k(a, st); break;
+        case CML_Q4_K:
+            // int8 matrix cores for the batched shapes (speculative-verify / prefill); packed dot below.
+            // The measured crossover on MI355X is between 4 and 8 tokens (14336x4096: 8 tokens take
+            // 32 us on the packed-dot kernel, 19.5 us here), hence 8 and not 16.
+            if (!a.group_offsets && !a.ints && a.n_tokens >= env_int("CAMELID_HIP_Q4K_MFMA_MIN_TOKENS", 8))
+                rc = launch_gemm_q4k_mfma(a, st);
+            else
+                rc = launch_gemv_q4k(a, st);
+            break;
         case CML_Q8_0: rc = launch_gemv_q8_0(a, st); break;
         case CML_Q4_0: rc = launch_gemv_q4_0(a, st); break;
         case CML_Q6_K: rc = launch_gemv_q6k(a, st); break;

@@ -95,6 +95,7 @@ int launch_gemv_q4_0(const MatArgs &a, hipStream_t st);
 int launch_gemv_q6k(const MatArgs &a, hipStream_t st);
 
 int launch_gemm_q4k(const MatArgs &a, hipStream_t st);
+int launch_gemm_q4k_mfma(const MatArgs &a, hipStream_t st);  // plain calls, n_tokens >= 16
 int launch_gemm_q8_0(const MatArgs &a, hipStream_t st);
 int launch_gemm_q4_0(const MatArgs &a, hipStream_t st);
 int launch_gemm_q6k(const MatArgs &a, hipStream_t st);

@@ -369,6 +369,10 @@ static Q4KShape pick_shape(int64_t rows, int64_t n_sb) {
     return s;
 }
 
+// The K-split the matvec kernel applies to a weight of this shape (the
+// matrix-core kernel reproduces the same association).
+int q4k_ksplit_for(int64_t rows, int64_t n_sb) { return pick_shape(rows, n_sb).ksplit; }
+
 template <int NT>
 static int launch_q4k_nt(Q4KArgs ka, const Q4KShape &shape, int n_groups, bool ints, hipStream_t st) {
     const int waves = shape.ksplit * shape.tiles_per_wg;

@@ -289,3 +289,27 @@ def test_host_slice_seam(name, fmt):
     bad = lib().cml_try_linear_rows(fmt, s.ctypes.data, q.ctypes.data, wire.ctypes.data, wire.nbytes - 1, n, rows,
                                     cols, out.ctypes.data)
     assert bad != 0
+
+
+# ------------------------------------------------- matrix-core path (n >= 16) ----
+
+@pytest.mark.parametrize("rows,cols", [(130, 1024), (2049, 5 * 256), (300, 56 * 256), (16, 256)])
+def test_q4k_matrix_core_cells_are_bitwise_the_gemv(rows, cols):
+    fmt = B.CML_Q4_K
+    rng = np.random.default_rng(rows + cols)
+    wire = G.synth_weight(fmt, rows, cols, seed=rows * 3 + cols)
+    w = Weight.upload(fmt, rows, cols, wire)
+    for n in (8, 16, 17, 33, 50, 64, 70):
+        x = rng.standard_normal((n, cols)).astype(np.float32)
+        s, q = oracle.quantize_activation(fmt, x)
+        for shape in (0, 1, 2, 3, 4, 5, 6, 7):   # 0 = the default workgroup shape, 1..7 = every other one
+            G.say(f"Q4_K matrix-core {rows}x{cols} n={n} shape={shape}")
+            with G.env(CAMELID_HIP_Q4K_MFMA_SHAPE=shape):
+                got = G.gpu_gemm(w, s, q)                      # default K-split policy, reproduced in-lane
+            with G.env(CAMELID_HIP_Q4K_MFMA_MIN_TOKENS=1 << 30):
+                ref = G.gpu_gemm(w, s, q)                      # the packed-dot kernel on the same inputs
+            assert G.same_bits(got, ref)
+            check_outputs(fmt, wire, cols, s, q, got, expect_exact=False)
+        with G.env(CAMELID_HIP_EXACT_ORDER="1"):
+            got = G.gpu_gemm(w, s, q)
+        check_outputs(fmt, wire, cols, s, q, got, expect_exact=True)
