@@ -30,7 +30,14 @@ sys.path.insert(0, ROOT)
 from camelid_amd import binding as B  # noqa: E402
 from camelid_amd.binding import DeviceBuffer, Weight, check, lib  # noqa: E402
 
-HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+HBM_PEAK_GBS = 8000.0    # MI355X published HBM3E bandwidth
+INT8_PEAK_TOPS = 5000.0  # MI355X published dense int8 matrix-core rate
+
+# HBM bytes per launch of the dominant kernel, from hardware counters: FETCH_SIZE + WRITE_SIZE of
+# `rocprofv3 --pmc` runs of this file, each scaled by what the same counter reads for
+# `--calibrate-copy` (a plain copy of known size).  Counters cannot be read from inside the timed
+# run, so the figures measured for the committed kernels are carried here; null where not measured.
+MEASURED_TRAFFIC_BYTES: dict = {}
 
 # name -> (format, rows, cols, tokens): BASELINE.json's configurations.
 CONFIGS = {
@@ -117,6 +124,35 @@ def cpu_baseline(fmt: int, wire: np.ndarray, rows: int, cols: int, x: np.ndarray
     }
 
 
+def calibrate_copy(nbytes: int, K: int, W: int) -> int:
+    """Plain copy kernel over rotating buffers: what this box's HBM gives a kernel with no arithmetic."""
+    L = lib()
+    nbytes = max(16, nbytes // 16 * 16)
+    pairs = max(2, min(16, -(-600_000_000 // (2 * nbytes))))
+    src = [DeviceBuffer(nbytes) for _ in range(pairs)]
+    dst = [DeviceBuffer(nbytes) for _ in range(pairs)]
+    for b in src:
+        b.fill(1)
+    stream = C.c_void_p()
+    check(L.cml_stream_create(C.byref(stream)))
+    timer = Timer(stream)
+
+    def step(i):
+        check(L.cml_copy_dev(dst[i % pairs].ptr, src[i % pairs].ptr, nbytes, stream), "cml_copy_dev")
+
+    for i in range(W):
+        step(i)
+    g = capture(stream, step, K)
+    time_graph(stream, g, timer)
+    ms = min(time_graph(stream, g, timer) for _ in range(3)) / K
+    check(L.cml_stream_sync(stream))
+    gbs = 2 * nbytes / (ms * 1e-3) / 1e9
+    print(json.dumps({"metric": "plain device copy (read + write)", "value": round(gbs, 2), "unit": "GB/s",
+                      "bytes_copied": nbytes, "bytes_moved": 2 * nbytes, "us_per_launch": round(ms * 1e3, 3),
+                      "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4), "steps": K, "warmup": W, "n_gpus": 1}))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
@@ -126,6 +162,11 @@ def main() -> int:
     ap.add_argument("--copies", type=int, default=0, help="distinct weight copies to rotate over (0 = enough for ~600 MB)")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="time budget of the CPU baseline leg (0 = skip)")
     ap.add_argument("--seed", type=int, default=1234)
+    ap.add_argument("--cold-only", action="store_true",
+                    help="skip the cache-warm leg and the eager loop (every launch of the dominant kernel is then "
+                         "cache-cold, so a profiler's average duration is comparable with roofline.us_per_launch)")
+    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="BYTES",
+                    help="instead of a matvec, time a plain device copy of BYTES (the yardstick for byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no collectives and every box here has one GPU; "
@@ -137,6 +178,8 @@ def main() -> int:
         print("no usable gfx950 device: " + L.cml_last_error().decode(), file=sys.stderr)
         return 3
     B.init(0)
+    if args.calibrate_copy:
+        return calibrate_copy(args.calibrate_copy, max(1, args.steps), max(0, args.warmup))
     fmt_name, rows, cols, n = CONFIGS[args.config]
     fmt = B.FORMATS[fmt_name]
     K, W = max(1, args.steps), max(0, args.warmup)
@@ -168,11 +211,13 @@ def main() -> int:
     ms_per_step = ms_total / K
     # the same K steps launched one by one from Python, for the record
     check(L.cml_stream_sync(stream))
-    t0 = time.perf_counter()
-    for i in range(K):
-        step(i)
-    check(L.cml_stream_sync(stream))
-    eager_us = (time.perf_counter() - t0) / K * 1e6
+    eager_us = None
+    if not args.cold_only:
+        t0 = time.perf_counter()
+        for i in range(K):
+            step(i)
+        check(L.cml_stream_sync(stream))
+        eager_us = (time.perf_counter() - t0) / K * 1e6
 
     # dominant kernel alone: the gemv/gemm on already quantized activations
     per = 256 if fmt_name in ("Q4_K", "Q6_K") else 32
@@ -191,8 +236,10 @@ def main() -> int:
     g_warm = capture(stream, gemv_warm, K)
     time_graph(stream, g_cold, timer)
     kern_ms = min(time_graph(stream, g_cold, timer) for _ in range(3)) / K
-    time_graph(stream, g_warm, timer)
-    warm_ms = min(time_graph(stream, g_warm, timer) for _ in range(3)) / K
+    warm_ms = None
+    if not args.cold_only:
+        time_graph(stream, g_warm, timer)
+        warm_ms = min(time_graph(stream, g_warm, timer) for _ in range(3)) / K
     check(L.cml_stream_sync(stream))
     result = out.to_numpy(np.float32, (n, rows))
     if not np.all(np.isfinite(result)):
@@ -210,18 +257,23 @@ def main() -> int:
         "us_per_call": round(ms_per_step * 1e3, 3),
         "pct_of_hbm_peak": round(100.0 * alg_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "int8 dot, f32 accumulate", "data": "synthetic",
+        "dtype": "int8", "data": "synthetic",
         "config": {"workload": args.config, "format": fmt_name, "rows": rows, "cols": cols, "tokens": n,
                    "algorithmic_bytes_per_call": alg_bytes, "weight_copies_rotated": copies,
                    "step": "quantize activation + fused dequantize-matvec (cml_matmul_f32), graph replay",
-                   "eager_python_us_per_call": round(eager_us, 3)},
+                   "eager_python_us_per_call": None if eager_us is None else round(eager_us, 3)},
         "roofline": {"bound": "hbm", "kernel": f"gemv_{fmt_name.lower()} (cml_gemm on quantized activations)",
                      "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.config),
                      "us_per_launch": round(kern_ms * 1e3, 3),
-                     "cache_warm_us_per_launch": round(warm_ms * 1e3, 3),
-                     "cache_warm_gbs": round(alg_bytes / (warm_ms * 1e-3) / 1e9, 2)},
+                     "cache_warm_us_per_launch": None if warm_ms is None else round(warm_ms * 1e3, 3),
+                     "cache_warm_gbs": None if warm_ms is None else round(alg_bytes / (warm_ms * 1e-3) / 1e9, 2)},
     }
+    if n >= 8:
+        # the batched shapes also have a matrix-core side: 2*rows*cols*tokens integer operations
+        tops = 2.0 * rows * cols * n / (kern_ms * 1e-3) / 1e12
+        line["roofline"]["mfma"] = {"achieved": round(tops, 2), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
+                                    "frac": round(tops / INT8_PEAK_TOPS, 4)}
     if args.cpu_seconds > 0:
         line["cpu_baseline"] = cpu_baseline(fmt, wire, rows, cols, x, alg_bytes, args.cpu_seconds)
     print(json.dumps(line, ensure_ascii=False))

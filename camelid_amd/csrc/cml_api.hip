@@ -153,6 +153,25 @@ int cml_memset_dev(void *dst_dev, int value, size_t nbytes, cml_stream_t stream)
     return CML_OK;
 }
 
+// Plain streaming copy, 16 bytes per lane per trip: the yardstick the byte counters and the matvec
+// kernels are read against (it moves nbytes in and nbytes out and nothing else).
+__global__ void __launch_bounds__(256) copy_kernel(uint4 *__restrict__ dst, const uint4 *__restrict__ src, size_t n16) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
+}
+
+int cml_copy_dev(void *dst_dev, const void *src_dev, size_t nbytes, cml_stream_t stream) {
+    if (int rc = check_ready()) return rc;
+    if (nbytes == 0) return CML_OK;
+    if (!dst_dev || !src_dev) return fail(CML_ERR_INVALID, "null pointer");
+    if ((nbytes | (uintptr_t)dst_dev | (uintptr_t)src_dev) & 15) return fail(CML_ERR_INVALID, "cml_copy_dev needs 16-byte aligned pointers and size");
+    const size_t n16 = nbytes / 16;
+    const unsigned blocks = (unsigned)std::min<size_t>((n16 + 255) / 256, 256u * 32u);
+    hipLaunchKernelGGL(copy_kernel, dim3(blocks), dim3(256), 0, as_stream(stream), (uint4 *)dst_dev, (const uint4 *)src_dev, n16);
+    CML_HIP_TRY(hipGetLastError());
+    return CML_OK;
+}
+
 int cml_stream_sync(cml_stream_t stream) {
     if (int rc = check_ready()) return rc;
     CML_HIP_TRY(hipStreamSynchronize(as_stream(stream)));

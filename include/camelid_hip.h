@@ -88,13 +88,17 @@ int cml_dev_free(void *ptr_dev);
 int cml_memcpy_h2d(void *dst_dev, const void *src_host, size_t nbytes, cml_stream_t stream);
 int cml_memcpy_d2h(void *dst_host, const void *src_dev, size_t nbytes, cml_stream_t stream);
 int cml_memset_dev(void *dst_dev, int value, size_t nbytes, cml_stream_t stream);
+/* Device-to-device streaming copy by a plain kernel (16-byte aligned pointers and
+ * size; may be captured).  Also the yardstick bench.py reads byte counters and
+ * matvec bandwidth against: it moves nbytes in, nbytes out and nothing else. */
+int cml_copy_dev(void *dst_dev, const void *src_dev, size_t nbytes, cml_stream_t stream);
 int cml_stream_sync(cml_stream_t stream);
 /* Streams (default priority), timing events and captured launch sequences, for
  * hosts that drive a decode loop through this library alone.  The reference's
  * resident engine owns one stream, syncs once per token and may replay a
  * captured graph (src/cuda_resident.rs:15195-15205); these are the pieces for
  * the same pattern.  Every matvec / matmul / quantize / mixture-of-experts entry
- * point may be captured; uploads, downloads and cml_block_dots may not. */
+ * point may be captured; uploads, downloads, cml_memset_dev and cml_block_dots may not. */
 int cml_stream_create(cml_stream_t *out);
 int cml_stream_destroy(cml_stream_t stream);
 int cml_event_create(cml_event_t *out);
@@ -110,12 +114,19 @@ int cml_graph_destroy(cml_graph_t graph);
 /* ---- weights (reference repack_for_lane + set_layer_located,
  *      src/cuda_resident.rs:9838, :16133-16253) ---------------------------- */
 
-/* Copy `nbytes` of GGUF wire bytes (host memory) to the device.  Q4_K keeps
- * the on-disk block layout; Q8_0, Q4_0 and Q6_K are re-laid at load time into
- * per-field planes of exactly the same total size (quants | scales, or
- * ql | qh | scales | d) so that every device load is a naturally aligned
- * 128-bit load.  The re-layout is a pure permutation of bytes:
- * cml_weight_download returns the original wire bytes. */
+/* Copy `nbytes` of GGUF wire bytes (host memory) to the device, re-laid at load
+ * time so that every device load is a naturally aligned 128-bit load:
+ *  - Q8_0, Q4_0, Q6_K: per-field planes of exactly the wire size
+ *    (quants | scales, or ql | qh | scales | d);
+ *  - Q4_K: super-block major, tiles of 16 rows; a tile is 2304 bytes =
+ *    16 x 16 header bytes (d, dmin, scales) then the 16 rows' nibbles
+ *    interleaved in 16-byte pieces, so one wave reads whole 1 KB runs.  The
+ *    last tile of a weight whose row count is not a multiple of 16 is padded
+ *    with zero blocks (device size = ceil(rows/16)*16 rows).
+ * Both are pure permutations of the wire bytes: cml_weight_download returns the
+ * original bytes (cf. the reference's lossless repacks,
+ * src/cuda_resident.rs:9741-9753, :9878-9911).  Views (cml_weight_slice) of a
+ * Q4_K weight must start on a multiple of 16 rows. */
 int cml_weight_upload(int fmt, int64_t rows, int64_t cols, const void *wire_host, size_t nbytes,
                       cml_weight **out);
 /* Same, from wire bytes that already live in device memory. */
