@@ -105,6 +105,128 @@ __device__ __forceinline__ float group_fold_ordered(float acc, float term) {
     }
 }
 
+// ---- Q8_K activation quantizer, one wave per super-block ------------------------
+
+__device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d) {
+    return (static_cast<uint32_t>(a) & 0xffu) | ((static_cast<uint32_t>(b) & 0xffu) << 8) |
+           ((static_cast<uint32_t>(c) & 0xffu) << 16) | ((static_cast<uint32_t>(d) & 0xffu) << 24);
+}
+
+// The reference's nearest_int (src/inference.rs:23112-23116).
+__device__ __forceinline__ int nearest_int_magic(float f) {
+    const float val = f + 12582912.0f;
+    return static_cast<int>(__builtin_bit_cast(uint32_t, val) & 0x007fffffu) - 0x00400000;
+}
+
+// Quantizes one 256-value super-block held by a whole wave, lane l holding
+// values 4l..4l+3 (reference quantize_q8_k_blocks, src/inference.rs:23121-23152):
+// the first strictly greatest |v| picks the signed `max`; iscale = -127 / max;
+// q = min(nearest_int(iscale * v), 127); d = 1 / iscale; an all-zero (or all-NaN)
+// super-block gives d = 0, q = 0.  Returns the lane's four quants packed; `d` is
+// the same in every lane; lanes with (lane & 7) == 7 get in `bsum` the sum of the
+// 32 quants of group lane / 8 (other lanes hold partial sums).
+// Must be called by all 64 lanes.
+__device__ __forceinline__ uint32_t q8k_quantize_wave(const float4 v, float &d, int &bsum) {
+    const float a0 = fabsf(v.x), a1 = fabsf(v.y), a2 = fabsf(v.z), a3 = fabsf(v.w);
+    // fmaxf drops NaNs; the trailing 0 turns an all-NaN lane into 0
+    const float lmax = fmaxf(fmaxf(fmaxf(a0, a1), fmaxf(a2, a3)), 0.0f);
+    float m = lmax;  // row maxima gather in lanes 15, 31, 47, 63 (values are >= 0, so the 0 fill is neutral)
+    m = fmaxf(m, row_shr_f32<1>(m));
+    m = fmaxf(m, row_shr_f32<2>(m));
+    m = fmaxf(m, row_shr_f32<4>(m));
+    m = fmaxf(m, row_shr_f32<8>(m));
+    const int mi = __builtin_bit_cast(int, m);  // non-negative floats order like their bit patterns
+    const int r0 = __builtin_amdgcn_readlane(mi, 15), r1 = __builtin_amdgcn_readlane(mi, 31);
+    const int r2 = __builtin_amdgcn_readlane(mi, 47), r3 = __builtin_amdgcn_readlane(mi, 63);
+    const int amax_bits = max(max(r0, r1), max(r2, r3));
+    // Straight-line on purpose (several super-blocks interleave in one wave): an all-zero or
+    // all-NaN super-block runs through with iscale = inf or NaN and is forced to d = 0, q = 0 at the end.
+    const bool empty = amax_bits == 0;  // wave-uniform
+    const float amax = __builtin_bit_cast(float, amax_bits);
+    const unsigned long long holders = __builtin_amdgcn_ballot_w64(lmax == amax);
+    const int first_lane = holders ? __builtin_ctzll(holders) : 0;
+    const float mine = (a0 == amax) ? v.x : ((a1 == amax) ? v.y : ((a2 == amax) ? v.z : v.w));
+    const float vmax = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine), first_lane));
+    const float iscale = -127.0f / vmax;
+    const int q0 = min(nearest_int_magic(iscale * v.x), 127);
+    const int q1 = min(nearest_int_magic(iscale * v.y), 127);
+    const int q2 = min(nearest_int_magic(iscale * v.z), 127);
+    const int q3 = min(nearest_int_magic(iscale * v.w), 127);
+    const uint32_t packed = empty ? 0u : pack4(q0, q1, q2, q3);
+    d = empty ? 0.0f : 1.0f / iscale;
+    bsum = group_sum_to_last<8>(sdot4(packed, 0x01010101u, 0));
+    return packed;
+}
+
+// row_ror:N -- lane i reads lane (i - N) mod 16 of its 16-lane row.  Four of
+// them (1, 2, 4, 8) leave every lane of a row with the row's reduction.
+template <int N>
+__device__ __forceinline__ int row_ror_i32(int v) {
+    static_assert(N >= 1 && N <= 15, "row_ror distance");
+    return __builtin_amdgcn_update_dpp(0, v, 0x120 + N, 0xf, 0xf, false);
+}
+__device__ __forceinline__ float row_allmax_nonneg(float m) {
+    m = fmaxf(m, __builtin_bit_cast(float, row_ror_i32<1>(__builtin_bit_cast(int, m))));
+    m = fmaxf(m, __builtin_bit_cast(float, row_ror_i32<2>(__builtin_bit_cast(int, m))));
+    m = fmaxf(m, __builtin_bit_cast(float, row_ror_i32<4>(__builtin_bit_cast(int, m))));
+    m = fmaxf(m, __builtin_bit_cast(float, row_ror_i32<8>(__builtin_bit_cast(int, m))));
+    return m;
+}
+__device__ __forceinline__ int row_allor(int v) {
+    v |= row_ror_i32<1>(v);
+    v |= row_ror_i32<2>(v);
+    v |= row_ror_i32<4>(v);
+    v |= row_ror_i32<8>(v);
+    return v;
+}
+
+// The same quantizer with a 16-lane row per super-block, so that one wave does
+// four super-blocks in one pass and one dependency chain: lane l of a row holds
+// values 16l..16l+15 (v[0..3]).  Returns the 16 quants packed in value order;
+// `d` is the same in every lane of the row; odd lanes get in `bsum` the sum of
+// the 32 quants of group l / 2.  Same arithmetic, value for value, as
+// q8k_quantize_wave.  Must be called by all 64 lanes.
+__device__ __forceinline__ uint4 q8k_quantize_row16(const float4 (&v)[4], int lane, float &d, int &bsum) {
+    float a[16];
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        a[4 * k + 0] = fabsf(v[k].x);
+        a[4 * k + 1] = fabsf(v[k].y);
+        a[4 * k + 2] = fabsf(v[k].z);
+        a[4 * k + 3] = fabsf(v[k].w);
+    }
+    float lmax = 0.0f;  // fmaxf drops NaNs
+#pragma unroll
+    for (int j = 0; j < 16; j++) lmax = fmaxf(lmax, a[j]);
+    const float amax = row_allmax_nonneg(lmax);
+    const bool empty = amax == 0.0f;
+    // first holder of the maximum: lowest lane of the row, lowest value in the lane
+    const unsigned long long holders = __builtin_amdgcn_ballot_w64(lmax == amax);
+    const uint32_t row_holders = static_cast<uint32_t>(holders >> (lane & 48)) & 0xffffu;
+    const bool first = row_holders != 0u && (lane & 15) == __builtin_ctz(row_holders);
+    const float vals[16] = {v[0].x, v[0].y, v[0].z, v[0].w, v[1].x, v[1].y, v[1].z, v[1].w,
+                            v[2].x, v[2].y, v[2].z, v[2].w, v[3].x, v[3].y, v[3].z, v[3].w};
+    float mine = vals[15];
+#pragma unroll
+    for (int j = 14; j >= 0; j--) mine = (a[j] == amax) ? vals[j] : mine;
+    const float vmax = __builtin_bit_cast(float, row_allor(first ? __builtin_bit_cast(int, mine) : 0));
+    const float iscale = -127.0f / vmax;
+    uint32_t pk[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const int q0 = min(nearest_int_magic(iscale * vals[4 * k + 0]), 127);
+        const int q1 = min(nearest_int_magic(iscale * vals[4 * k + 1]), 127);
+        const int q2 = min(nearest_int_magic(iscale * vals[4 * k + 2]), 127);
+        const int q3 = min(nearest_int_magic(iscale * vals[4 * k + 3]), 127);
+        pk[k] = empty ? 0u : pack4(q0, q1, q2, q3);
+    }
+    d = empty ? 0.0f : 1.0f / iscale;
+    const uint4 packed = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+    const int s = bytesum16(packed);
+    bsum = s + row_shr_i32<1>(s);
+    return packed;
+}
+
 // ---- GGUF Q4_K scale/min words ------------------------------------------------
 
 // The 12 scale bytes of a Q4_K super-block as three little-endian words

@@ -90,6 +90,7 @@ struct MatArgs {
 };
 
 int launch_gemv_q4k(const MatArgs &a, hipStream_t st);
+int launch_gemv_q4k_f32(const cml_weight *w, const float *x, float *out, hipStream_t st);  // quantize + matvec, one token
 int launch_gemv_q8_0(const MatArgs &a, hipStream_t st);
 int launch_gemv_q4_0(const MatArgs &a, hipStream_t st);
 int launch_gemv_q6k(const MatArgs &a, hipStream_t st);

@@ -39,6 +39,8 @@
 // NT > 1 holds the unpacked weight in registers and replays it against NT
 // activation rows in LDS: the weight is streamed once per NT tokens and every
 // (row, token) cell is the NT = 1 result exactly.
+#include <algorithm>
+
 #include "cml_device.hpp"
 #include "cml_host.hpp"
 
@@ -53,6 +55,7 @@ struct Q4KArgs {
     int n_sb;              // super-blocks per row
     const int8_t *q;       // activation rows [*][n_sb*256]
     const float *yd;       // activation scales [*][n_sb]
+    const float *x;        // f32 activation row [n_sb*256]: only for the kernel that quantizes it itself
     float *out;            // [*][rows]
     const float *residual; // [rows] or null (plain single-token calls only)
     int32_t *ints;         // [rows][n_sb][2] or null
@@ -180,8 +183,13 @@ __device__ __forceinline__ void q4k_compute(const Q4KRegs &r, const Q4KLane &ln,
     }
 }
 
-template <int NT, bool INTS>
+// FUSEQ (single token, plain call): the activation arrives as f32 and every
+// workgroup quantizes it to Q8_K itself, wave w taking super-blocks w, w+waves, ...,
+// straight into the LDS staging area -- the arithmetic of quantize_q8_k_kernel,
+// without the launch and the round trip through memory.
+template <int NT, bool INTS, bool FUSEQ = false>
 __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
+    static_assert(!FUSEQ || (NT == 1 && !INTS), "the fused quantizer serves single-token calls");
     constexpr int RPW = kWave / LPS;  // rows per wave tile
     extern __shared__ uint4 smem[];
     const int n_sb = a.n_sb;
@@ -225,53 +233,98 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
             const int j = a0 + min(p0 + t, n_assign - 1);
             return a.group_rows ? a.group_rows[j] : j;
         };
-        // Prologue: activation loads first, the first weight buffer right behind
-        // them, then the LDS writes -- so HBM requests are in flight while the
-        // activation is staged.
-        uint4 *dst = reinterpret_cast<uint4 *>(ys);
-        uint4 sv[kQ4KStageRegs];
-#pragma unroll
-        for (int k = 0; k < kQ4KStageRegs; k++) {
-            const int i = min(tid + k * nthreads, n16 - 1);
-            const int t = NT == 1 ? 0 : i / c16;
-            sv[k] = reinterpret_cast<const uint4 *>(a.q + act_row(t) * n_sb * 256)[i - t * c16];
-        }
-        float yd0;
-        {
-            const int i = min(tid, NT * n_sb - 1);
-            const int t = NT == 1 ? 0 : i / n_sb;
-            yd0 = a.yd[act_row(t) * n_sb + (i - t * n_sb)];
-        }
-
         Q4KRegs ra, rb;
-        __builtin_amdgcn_sched_barrier(0);
-        q4k_load(ra, wtile, a.sb_stride, r, lane, s0, s1);
-        __builtin_amdgcn_sched_barrier(0);
-
+        if constexpr (FUSEQ) {
+            // f32 loads of the first batch, the first weight buffer right behind
+            // them, then the quantizer: HBM requests are in flight while it runs.
+            // A 16-lane row per super-block: a wave quantizes four at a time (pass p of wave w
+            // takes super-blocks 4*(w + p*waves) ..+3), lane l of a row holding values 16l..16l+15.
+            const int nw = nthreads >> 6;
+            const int qrow = lane >> 4, ql = lane & 15;
+            const float4 *x4 = reinterpret_cast<const float4 *>(a.x);
+            auto load_pass = [&](float4 (&xv)[4], int base) {
+                const int sbk = min(base + qrow, n_sb - 1);
 #pragma unroll
-        for (int k = 0; k < kQ4KStageRegs; k++) {
-            const int i = tid + k * nthreads;
-            int s = bytesum16(sv[k]);
-            s += row_shr_i32<1>(s);
-            if (i < n16) {
-                dst[i] = sv[k];
+                for (int k = 0; k < 4; k++) xv[k] = x4[sbk * 64 + ql * 4 + k];
+            };
+            auto quantize_pass = [&](const float4 (&xv)[4], int base) {
+                const int sbk = base + qrow;
+                float dv;
+                int bs;
+                const uint4 packed = q8k_quantize_row16(xv, lane, dv, bs);
+                if (sbk < n_sb) {
+                    reinterpret_cast<uint4 *>(ys)[sbk * 16 + ql] = packed;
+                    if (ql & 1) bsum[sbk * 8 + (ql >> 1)] = bs;
+                    if (ql == 0) yds[sbk] = dv;
+                }
+            };
+            float4 xa[4], xb[4];
+            load_pass(xa, 4 * wave);
+            __builtin_amdgcn_sched_barrier(0);
+            q4k_load(ra, wtile, a.sb_stride, r, lane, s0, s1);
+            __builtin_amdgcn_sched_barrier(0);
+            for (int base = 4 * wave;;) {
+                const int next = base + 4 * nw;
+                if (next >= n_sb) {
+                    quantize_pass(xa, base);
+                    break;
+                }
+                load_pass(xb, next);
+                quantize_pass(xa, base);
+#pragma unroll
+                for (int k = 0; k < 4; k++) xa[k] = xb[k];
+                base = next;
+            }
+            __syncthreads();
+        } else {
+            // Prologue: activation loads first, the first weight buffer right behind
+            // them, then the LDS writes -- so HBM requests are in flight while the
+            // activation is staged.
+            uint4 *dst = reinterpret_cast<uint4 *>(ys);
+            uint4 sv[kQ4KStageRegs];
+    #pragma unroll
+            for (int k = 0; k < kQ4KStageRegs; k++) {
+                const int i = min(tid + k * nthreads, n16 - 1);
+                const int t = NT == 1 ? 0 : i / c16;
+                sv[k] = reinterpret_cast<const uint4 *>(a.q + act_row(t) * n_sb * 256)[i - t * c16];
+            }
+            float yd0;
+            {
+                const int i = min(tid, NT * n_sb - 1);
+                const int t = NT == 1 ? 0 : i / n_sb;
+                yd0 = a.yd[act_row(t) * n_sb + (i - t * n_sb)];
+            }
+
+            __builtin_amdgcn_sched_barrier(0);
+            q4k_load(ra, wtile, a.sb_stride, r, lane, s0, s1);
+            __builtin_amdgcn_sched_barrier(0);
+
+    #pragma unroll
+            for (int k = 0; k < kQ4KStageRegs; k++) {
+                const int i = tid + k * nthreads;
+                int s = bytesum16(sv[k]);
+                s += row_shr_i32<1>(s);
+                if (i < n16) {
+                    dst[i] = sv[k];
+                    if (i & 1) bsum[i >> 1] = s;
+                }
+            }
+            for (int i = tid + kQ4KStageRegs * nthreads; i < n16; i += nthreads) {
+                const int t = NT == 1 ? 0 : i / c16;
+                const uint4 v = reinterpret_cast<const uint4 *>(a.q + act_row(t) * n_sb * 256)[i - t * c16];
+                dst[i] = v;
+                int s = bytesum16(v);
+                s += row_shr_i32<1>(s);
                 if (i & 1) bsum[i >> 1] = s;
             }
+            if (tid < NT * n_sb) yds[tid] = yd0;
+            for (int i = tid + nthreads; i < NT * n_sb; i += nthreads) {
+                const int t = NT == 1 ? 0 : i / n_sb;
+                yds[i] = a.yd[act_row(t) * n_sb + (i - t * n_sb)];
+            }
+            __syncthreads();
+
         }
-        for (int i = tid + kQ4KStageRegs * nthreads; i < n16; i += nthreads) {
-            const int t = NT == 1 ? 0 : i / c16;
-            const uint4 v = reinterpret_cast<const uint4 *>(a.q + act_row(t) * n_sb * 256)[i - t * c16];
-            dst[i] = v;
-            int s = bytesum16(v);
-            s += row_shr_i32<1>(s);
-            if (i & 1) bsum[i >> 1] = s;
-        }
-        if (tid < NT * n_sb) yds[tid] = yd0;
-        for (int i = tid + nthreads; i < NT * n_sb; i += nthreads) {
-            const int t = NT == 1 ? 0 : i / n_sb;
-            yds[i] = a.yd[act_row(t) * n_sb + (i - t * n_sb)];
-        }
-        __syncthreads();
 
         int32_t *ints_row = nullptr;
         if constexpr (INTS) {
@@ -407,6 +460,35 @@ static int launch_q4k_pick_nt(const Q4KArgs &ka, const Q4KShape &shape, int n_gr
         case 2: return launch_q4k_nt<2>(ka, shape, n_groups, false, st);
         default: return launch_q4k_nt<1>(ka, shape, n_groups, ints, st);
     }
+}
+
+// Single token, f32 activation in: quantize + matvec in one launch.  The K-split
+// is the matvec's own (same association); waves of a workgroup share the
+// quantizing, so a workgroup holds 4 waves where the split alone gives fewer.
+int launch_gemv_q4k_f32(const cml_weight *w, const float *x, float *out, hipStream_t st) {
+    if (w->rows == 0) return CML_OK;
+    Q4KArgs ka{};
+    ka.w = w->planes.p[0];
+    ka.sb_stride = w->planes.row_stride[0];
+    ka.rows = static_cast<int>(w->rows);
+    ka.n_sb = static_cast<int>(w->nb);
+    ka.x = x;
+    ka.out = out;
+    Q4KShape shape = pick_shape(ka.rows, ka.n_sb);
+    int tpw = env_int("CAMELID_HIP_Q4K_FUSED_TILES_PER_WG", 0);
+    if (tpw < 1 || tpw * shape.ksplit > 8) tpw = std::max(1, 4 / shape.ksplit);
+    shape.tiles_per_wg = tpw;
+    const int waves = shape.ksplit * shape.tiles_per_wg;
+    const int64_t tiles = (ka.rows + 15) / 16;
+    const unsigned gx = static_cast<unsigned>((tiles + shape.tiles_per_wg - 1) / shape.tiles_per_wg);
+    const size_t lds = static_cast<size_t>(ka.n_sb) * (256 + 32) + ((static_cast<size_t>(ka.n_sb) + 3) & ~size_t(3)) * 4 +
+                       static_cast<size_t>(waves) * 16 * 4;
+    if (lds > 64 * 1024) return fail(CML_ERR_UNSUPPORTED, "Q4_K activation of %d super-blocks exceeds the LDS staging limit", ka.n_sb);
+    ka.ksplit = shape.ksplit;
+    ka.tiles_per_wg = shape.tiles_per_wg;
+    hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true>), dim3(gx, 1), dim3(64 * waves), lds, st, ka);
+    CML_HIP_TRY(hipGetLastError());
+    return CML_OK;
 }
 
 int launch_gemv_q4k(const MatArgs &a, hipStream_t st) {

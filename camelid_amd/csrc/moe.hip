@@ -120,11 +120,6 @@ __global__ __launch_bounds__(64) void moe_plan_kernel(const int32_t *__restrict_
     }
 }
 
-__device__ __forceinline__ int nearest_int_magic_(float f) {
-    const float val = f + 12582912.0f;
-    return static_cast<int>(__builtin_bit_cast(uint32_t, val) & 0x007fffffu) - 0x00400000;
-}
-
 // h = silu(g) * u (reference CpuTensor::silu_mul, src/tensor/mod.rs:2610-2634:
 // (a / (1 + exp(-a))) * b), quantized to Q8_K on the fly (reference
 // quantize_q8_k_blocks, src/inference.rs:23121-23152).  One wave per 256-value
@@ -141,34 +136,11 @@ __global__ __launch_bounds__(256) void silu_mul_quantize_q8k_kernel(const float 
     v.y = (gv.y / (1.0f + expf(-gv.y))) * uv.y;
     v.z = (gv.z / (1.0f + expf(-gv.z))) * uv.z;
     v.w = (gv.w / (1.0f + expf(-gv.w))) * uv.w;
-    const float a0 = fabsf(v.x), a1 = fabsf(v.y), a2 = fabsf(v.z), a3 = fabsf(v.w);
-    float amax = fmaxf(fmaxf(a0, a1), fmaxf(a2, a3));
-#pragma unroll
-    for (int m = 1; m < 64; m <<= 1) amax = fmaxf(amax, __shfl_xor(amax, m));
-    int first = 1 << 20;
-    if (a3 == amax) first = lane * 4 + 3;
-    if (a2 == amax) first = lane * 4 + 2;
-    if (a1 == amax) first = lane * 4 + 1;
-    if (a0 == amax) first = lane * 4 + 0;
-#pragma unroll
-    for (int m = 1; m < 64; m <<= 1) first = min(first, __shfl_xor(first, m));
-    uint32_t *qo = reinterpret_cast<uint32_t *>(q + sb * 256);
-    if (amax == 0.0f || first >= 256) {
-        qo[lane] = 0u;
-        if (lane == 0) d[sb] = 0.0f;
-        return;
-    }
-    const int kk = first & 3;
-    const float mine = kk == 0 ? v.x : (kk == 1 ? v.y : (kk == 2 ? v.z : v.w));
-    const float mx = __shfl(mine, first >> 2);
-    const float iscale = -127.0f / mx;
-    const int q0 = min(nearest_int_magic_(iscale * v.x), 127);
-    const int q1 = min(nearest_int_magic_(iscale * v.y), 127);
-    const int q2 = min(nearest_int_magic_(iscale * v.z), 127);
-    const int q3 = min(nearest_int_magic_(iscale * v.w), 127);
-    qo[lane] = (static_cast<uint32_t>(q0) & 0xffu) | ((static_cast<uint32_t>(q1) & 0xffu) << 8) |
-               ((static_cast<uint32_t>(q2) & 0xffu) << 16) | ((static_cast<uint32_t>(q3) & 0xffu) << 24);
-    if (lane == 0) d[sb] = 1.0f / iscale;
+    float dv;
+    int bsum;
+    const uint32_t packed = q8k_quantize_wave(v, dv, bsum);
+    reinterpret_cast<uint32_t *>(q + sb * 256)[lane] = packed;
+    if (lane == 0) d[sb] = dv;
 }
 
 // out[t][c] = ((0 + y[a(t,0)][c]*w[t][0]) + y[a(t,1)][c]*w[t][1]) + ...  (reference

@@ -19,11 +19,6 @@
 
 namespace cml {
 
-__device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d) {
-    return (static_cast<uint32_t>(a) & 0xffu) | ((static_cast<uint32_t>(b) & 0xffu) << 8) |
-           ((static_cast<uint32_t>(c) & 0xffu) << 16) | ((static_cast<uint32_t>(d) & 0xffu) << 24);
-}
-
 // Rust's `(v).round().clamp(-128.0, 127.0) as i8`: NaN casts to 0.
 __device__ __forceinline__ int q8_0_round(float v) {
     float r = roundf(v);  // ties away from zero
@@ -55,12 +50,6 @@ __global__ __launch_bounds__(256) void quantize_q8_0_kernel(const float *__restr
     }
 }
 
-// The reference's nearest_int (src/inference.rs:23112-23116).
-__device__ __forceinline__ int nearest_int_magic(float f) {
-    const float val = f + 12582912.0f;
-    return static_cast<int>(__builtin_bit_cast(uint32_t, val) & 0x007fffffu) - 0x00400000;
-}
-
 // One wave per 256-value super-block; lane l holds values 4l..4l+3.
 __global__ __launch_bounds__(256) void quantize_q8_k_kernel(const float *__restrict__ x, int64_t n_sb,
                                                             int8_t *__restrict__ q, float *__restrict__ d) {
@@ -68,34 +57,11 @@ __global__ __launch_bounds__(256) void quantize_q8_k_kernel(const float *__restr
     const int64_t sb = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (sb >= n_sb) return;  // whole wave leaves together
     const float4 v = reinterpret_cast<const float4 *>(x + sb * 256)[lane];
-    const float a0 = fabsf(v.x), a1 = fabsf(v.y), a2 = fabsf(v.z), a3 = fabsf(v.w);
-    float amax = fmaxf(fmaxf(a0, a1), fmaxf(a2, a3));
-#pragma unroll
-    for (int m = 1; m < 64; m <<= 1) amax = fmaxf(amax, __shfl_xor(amax, m));
-    // index of the first value whose magnitude equals the maximum
-    int first = 1 << 20;
-    if (a3 == amax) first = lane * 4 + 3;
-    if (a2 == amax) first = lane * 4 + 2;
-    if (a1 == amax) first = lane * 4 + 1;
-    if (a0 == amax) first = lane * 4 + 0;
-#pragma unroll
-    for (int m = 1; m < 64; m <<= 1) first = min(first, __shfl_xor(first, m));
-    uint32_t *qo = reinterpret_cast<uint32_t *>(q + sb * 256);
-    if (amax == 0.0f || first >= 256) {  // all zero (or nothing comparable): d = 0, q = 0
-        qo[lane] = 0u;
-        if (lane == 0) d[sb] = 0.0f;
-        return;
-    }
-    const int k = first & 3;
-    const float mine = k == 0 ? v.x : (k == 1 ? v.y : (k == 2 ? v.z : v.w));
-    const float max = __shfl(mine, first >> 2);
-    const float iscale = -127.0f / max;
-    const int q0 = min(nearest_int_magic(iscale * v.x), 127);
-    const int q1 = min(nearest_int_magic(iscale * v.y), 127);
-    const int q2 = min(nearest_int_magic(iscale * v.z), 127);
-    const int q3 = min(nearest_int_magic(iscale * v.w), 127);
-    qo[lane] = pack4(q0, q1, q2, q3);
-    if (lane == 0) d[sb] = 1.0f / iscale;
+    float dv;
+    int bsum;
+    const uint32_t packed = q8k_quantize_wave(v, dv, bsum);
+    reinterpret_cast<uint32_t *>(q + sb * 256)[lane] = packed;
+    if (lane == 0) d[sb] = dv;
 }
 
 int launch_quantize_q8_0(const float *x, int64_t n_tokens, int64_t cols, int8_t *q, float *s, hipStream_t st) {

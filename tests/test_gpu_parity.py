@@ -248,6 +248,40 @@ def test_matmul_f32_is_quantize_then_gemm(name, fmt):
         assert G.same_bits(got, want)
 
 
+@pytest.mark.parametrize("rows,cols", [(190, 3072), (64, 256), (333, 4096), (48, 14336)])
+def test_q4k_fused_quantize_matvec_is_the_two_step_path(rows, cols):
+    """Single-token cml_matmul_f32 on Q4_K quantizes inside the matvec kernel: same bits as
+    quantize_q8_k followed by the matvec, for every workgroup shape, on activations with zero
+    super-blocks, equal magnitudes of both signs, exact rounding ties and NaNs."""
+    fmt = oracle.Q4_K
+    rng = np.random.default_rng(7000 + rows)
+    wire = G.synth_weight(fmt, rows, cols, seed=7100 + rows)
+    w = Weight.upload(fmt, rows, cols, wire)
+    acts = _activation_cases(cols, rng)
+    acts[0, :256] = 0.0
+    acts[0, 5], acts[0, 9] = 3.0, -3.0
+    acts[0, 17:21] = [1.5 * 3 / 127, 2.5 * 3 / 127, -0.5 * 3 / 127, 0.5 * 3 / 127]
+    acts[1, 3] = np.nan
+    acts[2, -256:] = 0.0
+    for i, x in enumerate(acts):
+        for tpw in (0, 1, 2, 4, 8):
+            for ks in (0, 1, 2):
+                if ks > cols // 256:
+                    continue
+                G.say(f"Q4_K fused quantize+matvec {rows}x{cols} act={i} tiles_per_wg={tpw} ksplit={ks}")
+                with G.env(CAMELID_HIP_Q4K_FUSED_TILES_PER_WG=tpw, CAMELID_HIP_Q4K_KSPLIT=ks):
+                    with G.env(CAMELID_HIP_FUSED_QUANT=2):   # also where the shape policy would not fuse
+                        fused = G.gpu_matmul_f32(w, x)
+                    with G.env(CAMELID_HIP_FUSED_QUANT=0):
+                        two_step = G.gpu_matmul_f32(w, x)
+                assert G.same_bits(fused, two_step)
+        if i != 1:  # the oracle's f64 criterion has no meaning for a NaN input; bits above cover it
+            with G.env(CAMELID_HIP_EXACT_ORDER="1"):
+                got = G.gpu_matmul_f32(w, x)
+            want = oracle.matmul(fmt, wire, cols, x[None, :], order=EXACT_ORDER[fmt], threads=8)[0]
+            assert G.same_bits(got, want)
+
+
 # ----------------------------------------------------- errors and the seam ----
 
 def test_error_paths_return_status_codes():
