@@ -126,16 +126,18 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
     }
 
     // Staging: each thread owns kPer fixed (token, piece) pairs; only the super-block moves.
-    const uint4 *stage_src[kPer];
+    // (native vector type on purpose: assigning the HIP uint4 struct between address spaces
+    // becomes a memcpy that pins the staging array in scratch memory)
+    const v4i *stage_src[kPer];
     int stage_dst[kPer];
 #pragma unroll
     for (int k = 0; k < kPer; k++) {
         const int i = tid + k * nthreads;
         const int t = i >> 4, piece = i & 15;
-        stage_src[k] = reinterpret_cast<const uint4 *>(q + static_cast<int64_t>(min(t, n_here - 1)) * n_sb * 256) + piece;
+        stage_src[k] = reinterpret_cast<const v4i *>(q + static_cast<int64_t>(min(t, n_here - 1)) * n_sb * 256) + piece;
         stage_dst[k] = t * kSlabRow + piece * 16;
     }
-    uint4 sreg[KC][kPer];
+    v4i sreg[KC][kPer];
     auto stage_load = [&](int p0) {  // the KC super-blocks starting at p0
 #pragma unroll
         for (int s = 0; s < KC; s++) {
@@ -148,7 +150,7 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
 #pragma unroll
         for (int s = 0; s < KC; s++)
 #pragma unroll
-            for (int k = 0; k < kPer; k++) *reinterpret_cast<uint4 *>(buf + s * (NTOK * kSlabRow) + stage_dst[k]) = sreg[s][k];
+            for (int k = 0; k < kPer; k++) *reinterpret_cast<v4i *>(buf + s * (NTOK * kSlabRow) + stage_dst[k]) = sreg[s][k];
     };
 
     // Lane constants.
@@ -257,8 +259,9 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
     for (int p0 = 0, ph = 0; p0 < n_sb; p0 += KC, ph++) {
         uint8_t *cur = (ph & 1) ? buf1 : buf0;
         uint8_t *nxt = (ph & 1) ? buf0 : buf1;
-        const bool more = p0 + KC < n_sb;
-        if (more) stage_load(p0 + KC);
+        // unconditional (the last phase re-reads clamped super-blocks into the idle buffer): keeps
+        // the staging values in registers and the loads in straight-line code
+        stage_load(p0 + KC);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int s0 = 0; s0 < KC; s0 += 2 * U) {
@@ -277,7 +280,7 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
                     if (p0 + s0 + U + u < n_sb) step(wb[u], p0 + s0 + U + u, cur + (s0 + U + u) * (NTOK * kSlabRow));
             }
         }
-        if (more) stage_store(nxt);
+        stage_store(nxt);
         __syncthreads();  // next phase complete in `nxt`, everyone done with `cur`
     }
 
