@@ -336,7 +336,7 @@ def test_q4k_matrix_core_cells_are_bitwise_the_gemv(rows, cols):
     for n in (8, 16, 17, 33, 50, 64, 70):
         x = rng.standard_normal((n, cols)).astype(np.float32)
         s, q = oracle.quantize_activation(fmt, x)
-        for shape in (0, 1, 2, 3, 4, 5, 6, 7):   # 0 = the default workgroup shape, 1..7 = every other one
+        for shape in (0, 1, 2, 3, 4, 5, 6):   # 0 = the default workgroup shape, 1..6 = every other one
             G.say(f"Q4_K matrix-core {rows}x{cols} n={n} shape={shape}")
             with G.env(CAMELID_HIP_Q4K_MFMA_SHAPE=shape):
                 got = G.gpu_gemm(w, s, q)                      # default K-split policy, reproduced in-lane
