@@ -354,11 +354,11 @@ int cml_weight_slice(const cml_weight *parent, int64_t row_start, int64_t rows, 
     w->allocation_bytes = 0;
     w->rows = rows;
     if (parent->fmt == CML_Q4_K) {
-        if (row_start % 16 != 0) {
-            delete w;
-            return fail(CML_ERR_UNSUPPORTED, "a Q4_K band must start on a 16-row tile boundary (row %lld)", (long long)row_start);
-        }
-        w->planes.p[0] += (row_start / 16) * 2304;  // tiles are 2304-byte chunks inside each super-block slab
+        // tiles are 2304-byte chunks inside each super-block slab; a band that starts inside a
+        // tile keeps the tile and skips its leading rows
+        const int64_t first = parent->row_skip + row_start;
+        w->planes.p[0] += (first / 16) * 2304;
+        w->row_skip = static_cast<int>(first % 16);
     } else {
         for (int i = 0; i < 4; i++)
             if (w->planes.p[i]) w->planes.p[i] += row_start * w->planes.row_stride[i];
@@ -385,7 +385,7 @@ int cml_weight_download(const cml_weight *w, void *wire_host, size_t nbytes) {
     if (!wire_host) return fail(CML_ERR_INVALID, "null pointer");
     void *staging = nullptr;
     CML_HIP_TRY(hipMalloc(&staging, want));
-    int rc = launch_planes_to_wire(w->fmt, w->planes, w->rows, w->nb, static_cast<uint8_t *>(staging), nullptr);
+    int rc = launch_planes_to_wire(w->fmt, w->planes, w->rows, w->nb, w->row_skip, static_cast<uint8_t *>(staging), nullptr);
     if (rc == CML_OK) {
         hipError_t e = hipMemcpy(wire_host, staging, want, hipMemcpyDeviceToHost);
         if (e != hipSuccess) rc = fail(CML_ERR_HIP, "hipMemcpy failed: %s", hipGetErrorString(e));

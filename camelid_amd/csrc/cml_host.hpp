@@ -49,6 +49,7 @@ struct cml_weight {
     int fmt;
     int64_t rows, cols, nb;  // nb = blocks per row
     cml::Planes planes;
+    int row_skip;      // Q4_K views that start inside a 16-row tile: rows of the first tile that precede the view (else 0)
     void *allocation;  // non-null only for the owning handle
     size_t allocation_bytes;
 };
@@ -66,7 +67,7 @@ int launch_quantize_q8_k(const float *x, int64_t n_tokens, int64_t cols, int8_t 
 
 // layout.hip: wire <-> planes, dequantize
 int launch_wire_to_planes(int fmt, const uint8_t *wire, int64_t rows, int64_t nb, const Planes &dst, hipStream_t st);
-int launch_planes_to_wire(int fmt, const Planes &src, int64_t rows, int64_t nb, uint8_t *wire, hipStream_t st);
+int launch_planes_to_wire(int fmt, const Planes &src, int64_t rows, int64_t nb, int row_skip, uint8_t *wire, hipStream_t st);
 int launch_dequantize(const cml_weight *w, float *out, hipStream_t st);
 
 // Arguments common to every gemv/gemm launcher.

@@ -56,6 +56,7 @@ struct Q4KMfmaArgs {
     const uint8_t *w;   // tiled layout [super-block][tile][2304 B]
     int64_t sb_stride;
     int rows, n_sb;
+    int row_skip;       // leading rows of the first tile that precede this weight view (0..15)
     const int8_t *q;    // [n_tokens][n_sb*256]
     const float *yd;    // [n_tokens][n_sb]
     float *out;         // [n_tokens][rows]
@@ -113,9 +114,9 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
     const int n = lane & 15, kq = lane >> 4;         // B/D column (weight row in tile) and k-quarter / A-row quad
     const int half = kq >> 1;                        // which sub-block of a chunk this lane's B bytes belong to
     const int rt = wave / TB, tb = wave - rt * TB;
-    const int n_tiles = (a.rows + 15) / 16;
+    const int n_tiles = (a.rows + a.row_skip + 15) / 16;
     const int tile = blockIdx.x * RT + rt;
-    const int row = tile * 16 + n;
+    const int row = tile * 16 + n - a.row_skip;
     const uint8_t *wtile = a.w + static_cast<int64_t>(min(tile, n_tiles - 1)) * 2304;
     const int tok0 = blockIdx.y * NTOK;                    // first token of this workgroup
     const int n_here = min(NTOK, a.n_tokens - tok0);       // >= 1 by construction of the grid
@@ -283,7 +284,7 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
     for (; sb0 + RING < n_sb; sb0 += RING) round(sb0, std::true_type{});
     round(sb0, std::false_type{});
 
-    if (tile < n_tiles && row < a.rows) {
+    if (tile < n_tiles && row >= 0 && row < a.rows) {
 #pragma unroll
         for (int g = 0; g < GPW; g++)
 #pragma unroll
@@ -302,7 +303,7 @@ int q4k_ksplit_for(int64_t rows, int64_t n_sb);  // gemv_q4k.hip: the matvec ker
 template <int GPW, int TB, bool SPLIT>
 static int launch_mfma_split(const Q4KMfmaArgs &ka, hipStream_t st) {
     constexpr int NTOK = 16 * GPW * TB, RT = 4 / TB;
-    const int n_tiles = (ka.rows + 15) / 16;
+    const int n_tiles = (ka.rows + ka.row_skip + 15) / 16;
     const unsigned gx = static_cast<unsigned>((n_tiles + RT - 1) / RT);
     const unsigned gy = static_cast<unsigned>((ka.n_tokens + NTOK - 1) / NTOK);
     const size_t lds = 2 * static_cast<size_t>(128) * kSlabRow + static_cast<size_t>(ka.n_sb) * NTOK * 4;
@@ -332,6 +333,7 @@ int launch_gemm_q4k_mfma(const MatArgs &a, hipStream_t st) {
     ka.w = w->planes.p[0];
     ka.sb_stride = w->planes.row_stride[0];
     ka.rows = static_cast<int>(w->rows);
+    ka.row_skip = w->row_skip;
     ka.n_sb = static_cast<int>(w->nb);
     ka.ksplit = q4k_ksplit_for(w->rows, w->nb);
     ka.q = a.q;

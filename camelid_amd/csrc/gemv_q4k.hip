@@ -52,6 +52,7 @@ struct Q4KArgs {
     const uint8_t *w;      // tiled layout: [super-block][tile][2304 B]
     int64_t sb_stride;     // bytes between consecutive super-blocks of one tile (= all tiles * 2304)
     int rows;              // rows of one band (a multiple of 16 when groups are used)
+    int row_skip;          // leading rows of the first tile that are not part of this weight view (0..15; plain calls only)
     int n_sb;              // super-blocks per row
     const int8_t *q;       // activation rows [*][n_sb*256]
     const float *yd;       // activation scales [*][n_sb]
@@ -214,10 +215,10 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
     const int s0 = static_cast<int>(static_cast<int64_t>(kpart) * n_sb / W);
     const int s1 = static_cast<int>(static_cast<int64_t>(kpart + 1) * n_sb / W);
     const int r = lane / LPS, l = lane - r * LPS;
-    const int row = tile * RPW + r;
-    const bool live = row < a.rows;
+    const int row = tile * RPW + r - a.row_skip;  // output row; negative for the skipped head of a view's first tile
+    const bool live = row >= 0 && row < a.rows;
     // the last tile is padded to 16 rows; tiles past the end (grid rounding) re-read it and store nothing
-    const uint8_t *wtile = w + static_cast<int64_t>(min(tile, (a.rows + 15) / 16 - 1)) * kQ4KChunk;
+    const uint8_t *wtile = w + static_cast<int64_t>(min(tile, (a.rows + a.row_skip + 15) / 16 - 1)) * kQ4KChunk;
     const bool leader = (l == LPS - 1);
     Q4KLane ln;
     ln.c = l;
@@ -383,8 +384,8 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
                 const int rr = i % RPW;
                 const int t = (i / RPW) % NT;
                 const int tw = i / (RPW * NT);
-                const int orow = (blockIdx.x * a.tiles_per_wg + tw) * RPW + rr;
-                if (orow >= a.rows || t >= n_here) continue;
+                const int orow = (blockIdx.x * a.tiles_per_wg + tw) * RPW + rr - a.row_skip;
+                if (orow < 0 || orow >= a.rows || t >= n_here) continue;
                 float v = part[((tw * W) * NT + t) * RPW + rr];
                 for (int k = 1; k < W; k++) v = v + part[((tw * W + k) * NT + t) * RPW + rr];
                 if (NT == 1 && a.residual) v = v + a.residual[orow];
@@ -429,7 +430,7 @@ int q4k_ksplit_for(int64_t rows, int64_t n_sb) { return pick_shape(rows, n_sb).k
 template <int NT>
 static int launch_q4k_nt(Q4KArgs ka, const Q4KShape &shape, int n_groups, bool ints, hipStream_t st) {
     const int waves = shape.ksplit * shape.tiles_per_wg;
-    const int64_t tiles = (ka.rows + 15) / 16;
+    const int64_t tiles = (ka.rows + ka.row_skip + 15) / 16;
     const unsigned gx = static_cast<unsigned>((tiles + shape.tiles_per_wg - 1) / shape.tiles_per_wg);
     const size_t lds = static_cast<size_t>(NT) * ka.n_sb * (256 + 32) + ((static_cast<size_t>(NT) * ka.n_sb + 3) & ~size_t(3)) * 4 +
                        static_cast<size_t>(waves) * NT * 16 * 4;
@@ -471,6 +472,7 @@ int launch_gemv_q4k_f32(const cml_weight *w, const float *x, float *out, hipStre
     ka.w = w->planes.p[0];
     ka.sb_stride = w->planes.row_stride[0];
     ka.rows = static_cast<int>(w->rows);
+    ka.row_skip = w->row_skip;
     ka.n_sb = static_cast<int>(w->nb);
     ka.x = x;
     ka.out = out;
@@ -479,7 +481,7 @@ int launch_gemv_q4k_f32(const cml_weight *w, const float *x, float *out, hipStre
     if (tpw < 1 || tpw * shape.ksplit > 8) tpw = std::max(1, 4 / shape.ksplit);
     shape.tiles_per_wg = tpw;
     const int waves = shape.ksplit * shape.tiles_per_wg;
-    const int64_t tiles = (ka.rows + 15) / 16;
+    const int64_t tiles = (ka.rows + ka.row_skip + 15) / 16;
     const unsigned gx = static_cast<unsigned>((tiles + shape.tiles_per_wg - 1) / shape.tiles_per_wg);
     const size_t lds = static_cast<size_t>(ka.n_sb) * (256 + 32) + ((static_cast<size_t>(ka.n_sb) + 3) & ~size_t(3)) * 4 +
                        static_cast<size_t>(waves) * 16 * 4;
@@ -495,11 +497,13 @@ int launch_gemv_q4k(const MatArgs &a, hipStream_t st) {
     const cml_weight *w = a.w;
     if (w->rows == 0 || a.n_tokens == 0) return CML_OK;
     const bool grouped = a.group_offsets != nullptr;
-    Q4KArgs ka;
+    Q4KArgs ka{};
     ka.w = w->planes.p[0];
     ka.sb_stride = w->planes.row_stride[0];
     ka.rows = static_cast<int>(grouped ? a.band_rows : w->rows);
-    if (grouped && (ka.rows % 16) != 0) return fail(CML_ERR_UNSUPPORTED, "Q4_K expert bands must be whole 16-row tiles (%d rows)", ka.rows);
+    if (grouped && ((ka.rows % 16) != 0 || w->row_skip != 0))
+        return fail(CML_ERR_UNSUPPORTED, "Q4_K expert bands must be whole 16-row tiles (%d rows, first tile offset %d)", ka.rows, w->row_skip);
+    ka.row_skip = grouped ? 0 : w->row_skip;
     ka.n_sb = static_cast<int>(w->nb);
     ka.residual = a.residual;
     ka.ints = a.ints;

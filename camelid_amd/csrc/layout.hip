@@ -96,12 +96,13 @@ __global__ __launch_bounds__(256) void relayout_kernel(int fmt, uint8_t *wire, P
 // Q4_K: one thread per 16-byte piece of the wire image (9 per super-block).
 template <bool TO_TILED>
 __global__ __launch_bounds__(256) void q4k_tile_kernel(uint4 *wire, uint8_t *tiled, int64_t sb_stride, int64_t nb,
-                                                       int64_t n_pieces) {
+                                                       int64_t n_pieces, int row_skip) {
     const int64_t g = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (g >= n_pieces) return;
     const int64_t blk = g / 9;
     const int piece = static_cast<int>(g - blk * 9);
-    const int64_t row = blk / nb, sb = blk - row * nb;
+    const int64_t wire_row = blk / nb, sb = blk - wire_row * nb;
+    const int64_t row = wire_row + row_skip;  // position in the tiled image (`tiled` points at the view's first tile)
     const int r = static_cast<int>(row & 15);
     uint8_t *chunk = tiled + sb * sb_stride + (row >> 4) * 2304;
     uint8_t *p;
@@ -114,7 +115,7 @@ __global__ __launch_bounds__(256) void q4k_tile_kernel(uint4 *wire, uint8_t *til
     if (TO_TILED) *reinterpret_cast<uint4 *>(p) = wire[g]; else wire[g] = *reinterpret_cast<const uint4 *>(p);
 }
 
-static int relayout(bool to_planes, int fmt, uint8_t *wire, const Planes &pl, int64_t rows, int64_t nb, hipStream_t st) {
+static int relayout(bool to_planes, int fmt, uint8_t *wire, const Planes &pl, int64_t rows, int64_t nb, int row_skip, hipStream_t st) {
     const Geometry g = geometry(fmt);
     const int64_t nbytes = rows * nb * g.block_bytes;
     if (nbytes == 0) return CML_OK;
@@ -128,9 +129,9 @@ static int relayout(bool to_planes, int fmt, uint8_t *wire, const Planes &pl, in
                 const int64_t last = rows / 16;
                 CML_HIP_TRY(hipMemset2DAsync(tiled + last * 2304, static_cast<size_t>(pl.row_stride[0]), 0, 2304, static_cast<size_t>(nb), st));
             }
-            hipLaunchKernelGGL(q4k_tile_kernel<true>, dim3(grid), dim3(256), 0, st, reinterpret_cast<uint4 *>(wire), tiled, pl.row_stride[0], nb, n_pieces);
+            hipLaunchKernelGGL(q4k_tile_kernel<true>, dim3(grid), dim3(256), 0, st, reinterpret_cast<uint4 *>(wire), tiled, pl.row_stride[0], nb, n_pieces, 0);
         } else {
-            hipLaunchKernelGGL(q4k_tile_kernel<false>, dim3(grid), dim3(256), 0, st, reinterpret_cast<uint4 *>(wire), tiled, pl.row_stride[0], nb, n_pieces);
+            hipLaunchKernelGGL(q4k_tile_kernel<false>, dim3(grid), dim3(256), 0, st, reinterpret_cast<uint4 *>(wire), tiled, pl.row_stride[0], nb, n_pieces, row_skip);
         }
         CML_HIP_TRY(hipGetLastError());
         return CML_OK;
@@ -146,11 +147,11 @@ static int relayout(bool to_planes, int fmt, uint8_t *wire, const Planes &pl, in
 }
 
 int launch_wire_to_planes(int fmt, const uint8_t *wire, int64_t rows, int64_t nb, const Planes &dst, hipStream_t st) {
-    return relayout(true, fmt, const_cast<uint8_t *>(wire), dst, rows, nb, st);
+    return relayout(true, fmt, const_cast<uint8_t *>(wire), dst, rows, nb, 0, st);
 }
 
-int launch_planes_to_wire(int fmt, const Planes &src, int64_t rows, int64_t nb, uint8_t *wire, hipStream_t st) {
-    return relayout(false, fmt, wire, src, rows, nb, st);
+int launch_planes_to_wire(int fmt, const Planes &src, int64_t rows, int64_t nb, int row_skip, uint8_t *wire, hipStream_t st) {
+    return relayout(false, fmt, wire, src, rows, nb, row_skip, st);
 }
 
 // ---- dequantize -----------------------------------------------------------------------------------
@@ -180,11 +181,12 @@ __global__ __launch_bounds__(256) void dequant_q8q4_kernel(int fmt, Planes pl, i
 // Q4_K: (d*sc)*q - (dmin*m) (reference Q4KBlock::dequantize, src/tensor/mod.rs:5903-5924;
 // q4_k_scale_min, :5997-6006).
 __global__ __launch_bounds__(256) void dequant_q4k_kernel(const uint8_t *__restrict__ tiled, int64_t sb_stride,
-                                                          int64_t nb, int64_t n_values, float *__restrict__ out) {
+                                                          int64_t nb, int64_t n_values, int row_skip, float *__restrict__ out) {
     const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i >= n_values) return;
     const int64_t blk = i >> 8;
-    const int64_t row = blk / nb, sb = blk - row * nb;
+    const int64_t out_row = blk / nb, sb = blk - out_row * nb;
+    const int64_t row = out_row + row_skip;
     const int rr = static_cast<int>(row & 15);
     const uint8_t *chunk = tiled + sb * sb_stride + (row >> 4) * 2304;
     const uint8_t *hdr = chunk + rr * 16;
@@ -237,7 +239,7 @@ int launch_dequantize(const cml_weight *w, float *out, hipStream_t st) {
             hipLaunchKernelGGL(dequant_q8q4_kernel, dim3(grid), dim3(256), 0, st, w->fmt, w->planes, w->nb, n_values, out);
             break;
         case CML_Q4_K:
-            hipLaunchKernelGGL(dequant_q4k_kernel, dim3(grid), dim3(256), 0, st, w->planes.p[0], w->planes.row_stride[0], w->nb, n_values, out);
+            hipLaunchKernelGGL(dequant_q4k_kernel, dim3(grid), dim3(256), 0, st, w->planes.p[0], w->planes.row_stride[0], w->nb, n_values, w->row_skip, out);
             break;
         case CML_Q6_K:
             hipLaunchKernelGGL(dequant_q6k_kernel, dim3(grid), dim3(256), 0, st, w->planes, w->nb, n_values, out);

@@ -125,8 +125,7 @@ int cml_graph_destroy(cml_graph_t graph);
  *    with zero blocks (device size = ceil(rows/16)*16 rows).
  * Both are pure permutations of the wire bytes: cml_weight_download returns the
  * original bytes (cf. the reference's lossless repacks,
- * src/cuda_resident.rs:9741-9753, :9878-9911).  Views (cml_weight_slice) of a
- * Q4_K weight must start on a multiple of 16 rows. */
+ * src/cuda_resident.rs:9741-9753, :9878-9911). */
 int cml_weight_upload(int fmt, int64_t rows, int64_t cols, const void *wire_host, size_t nbytes,
                       cml_weight **out);
 /* Same, from wire bytes that already live in device memory. */
@@ -134,7 +133,9 @@ int cml_weight_upload_dev(int fmt, int64_t rows, int64_t cols, const void *wire_
                           cml_stream_t stream, cml_weight **out);
 /* A view of rows [row_start, row_start+rows) of `parent`: the expert band of a
  * stacked expert tensor (reference matvec_q8k_rows, src/gemma4_runtime.rs:
- * 1084-1110).  The parent must outlive the view. */
+ * 1084-1110).  Any row range is accepted; the mixture-of-experts entry points
+ * additionally need Q4_K bands that are whole 16-row tiles.  The parent must
+ * outlive the view. */
 int cml_weight_slice(const cml_weight *parent, int64_t row_start, int64_t rows, cml_weight **out);
 int cml_weight_info(const cml_weight *w, int *fmt, int64_t *rows, int64_t *cols, size_t *wire_bytes);
 /* Reconstruct the GGUF wire bytes of `w` (a view yields its rows only). */
