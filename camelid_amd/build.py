@@ -1,7 +1,8 @@
-"""Builds libcamelid_hip.so (gfx950) in-tree with hipcc.
+"""Builds libcamelid_hip.so (gfx950) in-tree with hipcc, the C++ host layer
+libcamelid_host.so above it with g++, and the host layer's test programs.
 
 hipcc cross-compiles without a GPU, so this runs in the build container; the
-shared library then travels with the tree to the GPU box.
+shared libraries then travel with the tree to the GPU box.
 """
 from __future__ import annotations
 
@@ -72,5 +73,43 @@ def build(extra_flags: list[str] | None = None, jobs: int = 8) -> str:
     return LIB
 
 
+HOST_DIR = os.path.join(HERE, "host")
+HOST_LIB = os.path.join(HERE, "libcamelid_host.so")
+HOST_SOURCES = ["gguf_reader.cpp", "wire_quant.cpp"]
+CXX = os.environ.get("CXX", "g++")
+CXXFLAGS = ["-O2", "-std=c++17", "-fPIC", "-Wall", "-Wextra"]
+
+
+def build_host() -> str:
+    """libcamelid_host.so: GGUF reader + WireQuant over the C ABI (plain C++, no HIP headers)."""
+    cmd = [CXX, *CXXFLAGS, "-shared", *[os.path.join(HOST_DIR, s) for s in HOST_SOURCES],
+           "-L" + HERE, "-lcamelid_hip", "-Wl,-rpath,$ORIGIN", "-o", HOST_LIB]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"host library build failed:\n{r.stdout}\n{r.stderr}")
+    return HOST_LIB
+
+
+def build_host_tests() -> list[str]:
+    """The host layer's test programs (tests/host/*.cpp -> tests/host/bin/), run by pytest as
+    subprocesses.  They link the CPU oracle as their checker, so it must be built first."""
+    root = os.path.dirname(HERE)
+    tdir = os.path.join(root, "tests", "host")
+    bindir = os.path.join(tdir, "bin")
+    os.makedirs(bindir, exist_ok=True)
+    oracle_dir = os.path.join(root, "oracle")
+    out = []
+    for name, libs in (("test_gguf_reader", []), ("test_wire_quant", ["-L" + oracle_dir, "-loracle"])):
+        exe = os.path.join(bindir, name)
+        cmd = [CXX, *CXXFLAGS, os.path.join(tdir, name + ".cpp"), "-L" + HERE, "-lcamelid_host", "-lcamelid_hip", *libs,
+               "-Wl,-rpath,$ORIGIN/../../../camelid_amd", "-Wl,-rpath,$ORIGIN/../../../oracle", "-o", exe]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError(f"{name} build failed:\n{r.stdout}\n{r.stderr}")
+        out.append(exe)
+    return out
+
+
 if __name__ == "__main__":
     print(build(sys.argv[1:]))
+    print(build_host())
