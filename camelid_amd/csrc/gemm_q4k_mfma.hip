@@ -60,8 +60,13 @@ struct Q4KMfmaArgs {
     const int8_t *q;    // [n_tokens][n_sb*256]
     const float *yd;    // [n_tokens][n_sb]
     float *out;         // [n_tokens][rows]
-    int n_tokens;
+    int n_tokens;       // plain: activation rows; grouped: the most assignments one group can hold
     int ksplit;         // association to reproduce (see gemv_q4k.hip)
+    // Grouped call (mixture of experts): blockIdx.z = group e, which owns the weight band of rows
+    // [e*rows, (e+1)*rows) and the assignments [group_offsets[e], group_offsets[e+1]); assignment j
+    // reads activation row group_rows[j] (j itself when null) and writes output row j.
+    const int32_t *group_offsets;
+    const int32_t *group_rows;
 };
 
 struct MfmaWeights {
@@ -117,16 +122,24 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
     const int n_tiles = (a.rows + a.row_skip + 15) / 16;
     const int tile = blockIdx.x * RT + rt;
     const int row = tile * 16 + n - a.row_skip;
-    const uint8_t *wtile = a.w + static_cast<int64_t>(min(tile, n_tiles - 1)) * 2304;
-    const int tok0 = blockIdx.y * NTOK;                    // first token of this workgroup
-    const int n_here = min(NTOK, a.n_tokens - tok0);       // >= 1 by construction of the grid
-    const int8_t *q = a.q + static_cast<int64_t>(tok0) * n_sb * 256;
-    const float *yd = a.yd + static_cast<int64_t>(tok0) * n_sb;
+    const bool grouped = a.group_offsets != nullptr;
+    const int64_t band = grouped ? blockIdx.z : 0;
+    const int a0 = grouped ? a.group_offsets[band] : 0;                      // first assignment of this group
+    const int n_assign = grouped ? a.group_offsets[band + 1] - a0 : a.n_tokens;
+    const int tok0 = blockIdx.y * NTOK;                    // first token (assignment of the group) of this workgroup
+    if (tok0 >= n_assign) return;                          // nothing routed here: the whole workgroup leaves
+    const int n_here = min(NTOK, n_assign - tok0);
+    const uint8_t *wtile = a.w + (band * (a.rows / 16) + min(tile, n_tiles - 1)) * 2304;
+    // activation row of local token t (tokens past the end repeat the last one; their cells are not stored)
+    auto act_row = [&](int t) -> int64_t {
+        const int j = a0 + tok0 + min(t, n_here - 1);
+        return a.group_rows ? a.group_rows[j] : j;
+    };
 
     // activation scales: yds[sb][token] (tokens past the end repeat the last one; their cells are not stored)
     for (int i = tid; i < n_sb * NTOK; i += nthreads) {
         const int sb = i / NTOK, t = i - sb * NTOK;
-        yds[i] = yd[min(t, n_here - 1) * n_sb + sb];
+        yds[i] = a.yd[act_row(t) * n_sb + sb];
     }
 
     // Staging: each thread owns kPer fixed (token, piece) pairs; only the super-block moves.
@@ -138,7 +151,7 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
     for (int k = 0; k < kPer; k++) {
         const int i = tid + k * nthreads;
         const int t = i >> 4, piece = i & 15;
-        stage_src[k] = reinterpret_cast<const v4i *>(q + static_cast<int64_t>(min(t, n_here - 1)) * n_sb * 256) + piece;
+        stage_src[k] = reinterpret_cast<const v4i *>(a.q + act_row(t) * n_sb * 256) + piece;
         stage_dst[k] = t * kSlabRow + piece * 16;
     }
     v4i sreg[KC][kPer];
@@ -292,7 +305,7 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
                 const int t = tb * (16 * GPW) + 16 * g + cell_tok + j;
                 if (t < n_here) {
                     const float v = (part == 0) ? acc[g][j] : total[g][j] + acc[g][j];
-                    a.out[static_cast<int64_t>(tok0 + t) * a.rows + row] = v;
+                    a.out[static_cast<int64_t>(a0 + tok0 + t) * a.rows + row] = v;
                 }
             }
     }
@@ -301,7 +314,7 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
 int q4k_ksplit_for(int64_t rows, int64_t n_sb);  // gemv_q4k.hip: the matvec kernel's K-split policy
 
 template <int GPW, int TB, bool SPLIT>
-static int launch_mfma_split(const Q4KMfmaArgs &ka, hipStream_t st) {
+static int launch_mfma_split(const Q4KMfmaArgs &ka, int n_groups, hipStream_t st) {
     constexpr int NTOK = 16 * GPW * TB, RT = 4 / TB;
     const int n_tiles = (ka.rows + ka.row_skip + 15) / 16;
     const unsigned gx = static_cast<unsigned>((n_tiles + RT - 1) / RT);
@@ -314,7 +327,7 @@ static int launch_mfma_split(const Q4KMfmaArgs &ka, hipStream_t st) {
                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
         raised = true;
     }
-    hipLaunchKernelGGL((gemm_q4k_mfma_kernel<GPW, TB, SPLIT>), dim3(gx, gy), dim3(256), lds, st, ka);
+    hipLaunchKernelGGL((gemm_q4k_mfma_kernel<GPW, TB, SPLIT>), dim3(gx, gy, n_groups), dim3(256), lds, st, ka);
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }
@@ -322,41 +335,49 @@ static int launch_mfma_split(const Q4KMfmaArgs &ka, hipStream_t st) {
 // The K-split bookkeeping costs a branch per super-block, so it is compiled in only where the
 // matvec kernel splits K for this weight shape.
 template <int GPW, int TB>
-static int launch_mfma(const Q4KMfmaArgs &ka, hipStream_t st) {
-    return ka.ksplit > 1 ? launch_mfma_split<GPW, TB, true>(ka, st) : launch_mfma_split<GPW, TB, false>(ka, st);
+static int launch_mfma(const Q4KMfmaArgs &ka, int n_groups, hipStream_t st) {
+    return ka.ksplit > 1 ? launch_mfma_split<GPW, TB, true>(ka, n_groups, st) : launch_mfma_split<GPW, TB, false>(ka, n_groups, st);
 }
 
-// Plain (ungrouped) Q4_K matmul on the matrix cores.
+// Q4_K matmul on the matrix cores: plain calls, or grouped by expert (mixture of experts).
 int launch_gemm_q4k_mfma(const MatArgs &a, hipStream_t st) {
     const cml_weight *w = a.w;
-    Q4KMfmaArgs ka;
+    const bool grouped = a.group_offsets != nullptr;
+    if (w->rows == 0 || a.n_tokens == 0) return CML_OK;
+    Q4KMfmaArgs ka{};
     ka.w = w->planes.p[0];
     ka.sb_stride = w->planes.row_stride[0];
-    ka.rows = static_cast<int>(w->rows);
-    ka.row_skip = w->row_skip;
+    ka.rows = static_cast<int>(grouped ? a.band_rows : w->rows);
+    if (grouped && ((ka.rows % 16) != 0 || w->row_skip != 0))
+        return fail(CML_ERR_UNSUPPORTED, "Q4_K expert bands must be whole 16-row tiles (%d rows, first tile offset %d)", ka.rows, w->row_skip);
+    ka.row_skip = grouped ? 0 : w->row_skip;
     ka.n_sb = static_cast<int>(w->nb);
-    ka.ksplit = q4k_ksplit_for(w->rows, w->nb);
+    ka.ksplit = q4k_ksplit_for(ka.rows, w->nb);
     ka.q = a.q;
     ka.yd = a.scales;
     ka.out = a.out;
     ka.n_tokens = static_cast<int>(a.n_tokens);
-    // Workgroup shape: tokens staged per workgroup x how they are split over waves.
-    // Default: 16 tokens (n <= 16) or 32 tokens per workgroup, one wave per row tile; more
-    // tokens = more workgroup columns (grid.y), each a pass over the weight.  The other
-    // shapes stay selectable for tuning.
+    ka.group_offsets = a.group_offsets;
+    ka.group_rows = a.group_rows;
+    const int ng = grouped ? a.n_groups : 1;
+    // Workgroup shape: tokens staged per workgroup x how they are split over waves.  Default: one
+    // wave per row tile, 16 / 32 / 64 tokens per workgroup by batch size; more tokens = more
+    // workgroup columns (grid.y), each a pass over the weight.  The other shapes stay selectable
+    // for tuning.
     const int shape = env_int("CAMELID_HIP_Q4K_MFMA_SHAPE", 0);
     switch (shape) {
-        case 1: return launch_mfma<1, 1>(ka, st);   // 16 tokens, 1 wave per row tile
-        case 2: return launch_mfma<2, 1>(ka, st);   // 32 tokens, 1 wave per row tile
-        case 3: return launch_mfma<4, 1>(ka, st);   // 64 tokens, 1 wave per row tile
-        case 4: return launch_mfma<1, 2>(ka, st);   // 32 tokens, 2 waves per row tile
-        case 5: return launch_mfma<2, 2>(ka, st);   // 64 tokens, 2 waves per row tile
-        case 6: return launch_mfma<1, 4>(ka, st);   // 64 tokens, 4 waves per row tile
+        case 1: return launch_mfma<1, 1>(ka, ng, st);   // 16 tokens, 1 wave per row tile
+        case 2: return launch_mfma<2, 1>(ka, ng, st);   // 32 tokens, 1 wave per row tile
+        case 3: return launch_mfma<4, 1>(ka, ng, st);   // 64 tokens, 1 wave per row tile
+        case 4: return launch_mfma<1, 2>(ka, ng, st);   // 32 tokens, 2 waves per row tile
+        case 5: return launch_mfma<2, 2>(ka, ng, st);   // 64 tokens, 2 waves per row tile
+        case 6: return launch_mfma<1, 4>(ka, ng, st);   // 64 tokens, 4 waves per row tile
         default: break;
     }
-    if (a.n_tokens > 32) return launch_mfma<4, 1>(ka, st);
-    if (a.n_tokens > 16) return launch_mfma<2, 1>(ka, st);
-    return launch_mfma<1, 1>(ka, st);
+    if (grouped) return launch_mfma<1, 1>(ka, ng, st);  // assignments per expert are few and uneven: the smallest tile wastes least
+    if (a.n_tokens > 32) return launch_mfma<4, 1>(ka, ng, st);
+    if (a.n_tokens > 16) return launch_mfma<2, 1>(ka, ng, st);
+    return launch_mfma<1, 1>(ka, ng, st);
 }
 
 }  // namespace cml

@@ -120,6 +120,13 @@ __global__ __launch_bounds__(64) void moe_plan_kernel(const int32_t *__restrict_
     }
 }
 
+// Expert-grouped matmul: the packed-dot kernel for a few tokens, the matrix cores from 8 tokens
+// up (an expert can then hold 8 or more assignments).  Both produce the same bits per cell.
+static int launch_expert_matmul(const MatArgs &a, hipStream_t st) {
+    if (a.n_tokens >= env_int("CAMELID_HIP_Q4K_MFMA_MIN_TOKENS", 8)) return launch_gemm_q4k_mfma(a, st);
+    return launch_gemv_q4k(a, st);
+}
+
 // h = silu(g) * u (reference CpuTensor::silu_mul, src/tensor/mod.rs:2610-2634:
 // (a / (1 + exp(-a))) * b), quantized to Q8_K on the fly (reference
 // quantize_q8_k_blocks, src/inference.rs:23121-23152).  One wave per 256-value
@@ -256,10 +263,10 @@ int cml_moe_ffn(const cml_weight *gate, const cml_weight *up, const cml_weight *
     a.band_rows = ff;
     a.w = gate;
     a.out = ws.g;
-    if (int rc = launch_gemv_q4k(a, st)) return rc;
+    if (int rc = launch_expert_matmul(a, st)) return rc;
     a.w = up;
     a.out = ws.u;
-    if (int rc = launch_gemv_q4k(a, st)) return rc;
+    if (int rc = launch_expert_matmul(a, st)) return rc;
     // h = silu(g) * u, quantized per assignment
     const int64_t h_sb = static_cast<int64_t>(n_slots) * (ff / 256);
     hipLaunchKernelGGL(silu_mul_quantize_q8k_kernel, dim3(static_cast<unsigned>((h_sb + 3) / 4)), dim3(256), 0, st, ws.g, ws.u, h_sb, ws.hq, ws.hd);
@@ -271,7 +278,7 @@ int cml_moe_ffn(const cml_weight *gate, const cml_weight *up, const cml_weight *
     a.band_rows = hidden;
     a.w = down;
     a.out = ws.y;
-    if (int rc = launch_gemv_q4k(a, st)) return rc;
+    if (int rc = launch_expert_matmul(a, st)) return rc;
     hipLaunchKernelGGL(moe_weighted_sum_kernel, dim3(static_cast<unsigned>((hidden + 255) / 256), static_cast<unsigned>(n_tokens)), dim3(256), 0, st,
                        ws.y, ws.slot_to_assign, weight_dev, k, hidden, out_dev);
     CML_HIP_TRY(hipGetLastError());
