@@ -46,6 +46,7 @@ CONFIGS = {
     "q8_0_8192x2048_n1": ("Q8_0", 8192, 2048, 1),
     "q6k_128256x3072_n1": ("Q6_K", 128256, 3072, 1),
     "q4_0_128256x3072_n1": ("Q4_0", 128256, 3072, 1),
+    "q4k_14336x4096_n2": ("Q4_K", 14336, 4096, 2),
     "q4k_14336x4096_n4": ("Q4_K", 14336, 4096, 4),
     "q4k_14336x4096_n8": ("Q4_K", 14336, 4096, 8),
     "q4k_14336x4096_n16": ("Q4_K", 14336, 4096, 16),

@@ -439,9 +439,9 @@ static int dispatch(const MatArgs &a, hipStream_t st) {
     switch (a.w->fmt) {
         case CML_Q4_K:
             // int8 matrix cores for the batched shapes (speculative-verify / prefill); packed dot below.
-            // The measured crossover on MI355X is between 4 and 8 tokens (14336x4096: 8 tokens take
-            // 32 us on the packed-dot kernel, 19.5 us here), hence 8 and not 16.
-            if (!a.group_offsets && !a.ints && a.n_tokens >= env_int("CAMELID_HIP_Q4K_MFMA_MIN_TOKENS", 8))
+            // Measured on MI355X at 14336x4096: the matrix-core kernel takes 11.5-12 us for any batch
+            // up to 16 tokens, the packed-dot kernel 8.9 / 12.1 / 18.9 us for 1 / 2 / 4 tokens.
+            if (!a.group_offsets && !a.ints && a.n_tokens >= env_int("CAMELID_HIP_Q4K_MFMA_MIN_TOKENS", 4))
                 rc = launch_gemm_q4k_mfma(a, st);
             else
                 rc = launch_gemv_q4k(a, st);

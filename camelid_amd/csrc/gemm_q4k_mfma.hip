@@ -1,5 +1,5 @@
 // Q4_K x Q8_K small-batch matmul on the int8 matrix cores (gfx950), for
-// batches of 8 tokens and more: speculative-verify chunks and short prefill.
+// batches of 4 tokens and more: speculative-verify chunks and short prefill.
 //
 // Arithmetic: identical, cell by cell, to the matvec kernel (gemv_q4k.hip;
 // reference q4_k_dot_scalar, src/diffusion_gemma/refmath.rs:504-562):

@@ -120,10 +120,10 @@ __global__ __launch_bounds__(64) void moe_plan_kernel(const int32_t *__restrict_
     }
 }
 
-// Expert-grouped matmul: the packed-dot kernel for a few tokens, the matrix cores from 8 tokens
-// up (an expert can then hold 8 or more assignments).  Both produce the same bits per cell.
+// Expert-grouped matmul: the packed-dot kernel for a few tokens, the matrix cores from 4 tokens
+// up (the same crossover as for plain calls).  Both produce the same bits per cell.
 static int launch_expert_matmul(const MatArgs &a, hipStream_t st) {
-    if (a.n_tokens >= env_int("CAMELID_HIP_Q4K_MFMA_MIN_TOKENS", 8)) return launch_gemm_q4k_mfma(a, st);
+    if (a.n_tokens >= env_int("CAMELID_HIP_Q4K_MFMA_MIN_TOKENS", 4)) return launch_gemm_q4k_mfma(a, st);
     return launch_gemv_q4k(a, st);
 }
 

@@ -348,7 +348,7 @@ def test_q4k_matrix_core_cells_are_bitwise_the_gemv(rows, cols):
     rng = np.random.default_rng(rows + cols)
     wire = G.synth_weight(fmt, rows, cols, seed=rows * 3 + cols)
     w = Weight.upload(fmt, rows, cols, wire)
-    for n in (8, 16, 17, 33, 50, 64, 70):
+    for n in (4, 5, 8, 16, 17, 33, 50, 64, 70):
         x = rng.standard_normal((n, cols)).astype(np.float32)
         s, q = oracle.quantize_activation(fmt, x)
         for shape in (0, 1, 2, 3, 4, 5, 6):   # 0 = the default workgroup shape, 1..6 = every other one
