@@ -19,6 +19,7 @@ LIB = os.path.join(HERE, "libcamelid_hip.so")
 SOURCES = [
     "cml_api.hip",
     "quantize.hip",
+    "producers.hip",
     "layout.hip",
     "gemv_q4k.hip",
     "gemm_q4k_mfma.hip",

@@ -424,6 +424,34 @@ int cml_quantize_q8_k(const float *x_dev, int64_t n_tokens, int64_t cols, int8_t
     return launch_quantize_q8_k(x_dev, n_tokens, cols, q_dev, d_dev, as_stream(stream));
 }
 
+int cml_rms_norm_quantize(int act, const float *x_dev, const float *weight_dev, float eps, int64_t n_tokens, int64_t cols,
+                          float *normed_dev, int8_t *q_dev, float *scales_dev, cml_stream_t stream) {
+    if (int rc = check_ready()) return rc;
+    if (act != CML_ACT_F32 && act != CML_ACT_Q8_0 && act != CML_ACT_Q8_K) return fail(CML_ERR_INVALID, "unknown activation format %d", act);
+    const int64_t unit = act == CML_ACT_Q8_K ? 256 : (act == CML_ACT_Q8_0 ? 32 : 4);
+    if (n_tokens < 0 || cols < 0 || cols % unit != 0) return fail(CML_ERR_SHAPE, "cols %lld is not a multiple of %lld", (long long)cols, (long long)unit);
+    if (n_tokens == 0 || cols == 0) return CML_OK;
+    if (!x_dev || !weight_dev) return fail(CML_ERR_INVALID, "null pointer");
+    if (act == CML_ACT_F32 ? !normed_dev : (!q_dev || !scales_dev)) return fail(CML_ERR_INVALID, "null output pointer");
+    if (misaligned16(x_dev) || misaligned16(weight_dev) || (normed_dev && misaligned16(normed_dev)) ||
+        (act != CML_ACT_F32 && (reinterpret_cast<uintptr_t>(q_dev) & 3u)))
+        return fail(CML_ERR_INVALID, "x, weight and normed must be 16-byte and q 4-byte aligned");
+    return launch_rms_norm_quantize(act, x_dev, weight_dev, eps, n_tokens, cols, normed_dev, q_dev, scales_dev, as_stream(stream));
+}
+
+int cml_silu_mul_quantize(int act, const float *gate_dev, const float *up_dev, int64_t n_tokens, int64_t cols, int8_t *q_dev,
+                          float *scales_dev, cml_stream_t stream) {
+    if (int rc = check_ready()) return rc;
+    if (act != CML_ACT_Q8_0 && act != CML_ACT_Q8_K) return fail(CML_ERR_INVALID, "activation format %d is not a quantized one", act);
+    const int64_t unit = act == CML_ACT_Q8_K ? 256 : 32;
+    if (n_tokens < 0 || cols < 0 || cols % unit != 0) return fail(CML_ERR_SHAPE, "cols %lld is not a multiple of %lld", (long long)cols, (long long)unit);
+    if (n_tokens == 0 || cols == 0) return CML_OK;
+    if (!gate_dev || !up_dev || !q_dev || !scales_dev) return fail(CML_ERR_INVALID, "null pointer");
+    if (misaligned16(gate_dev) || misaligned16(up_dev) || (reinterpret_cast<uintptr_t>(q_dev) & 3u))
+        return fail(CML_ERR_INVALID, "gate and up must be 16-byte and q 4-byte aligned");
+    return launch_silu_mul_quantize(act, gate_dev, up_dev, n_tokens, cols, q_dev, scales_dev, as_stream(stream));
+}
+
 int cml_dequantize(const cml_weight *w, float *out_dev, cml_stream_t stream) {
     if (!w) return fail(CML_ERR_INVALID, "null weight");
     if (int rc = check_ready()) return rc;

@@ -105,12 +105,39 @@ __device__ __forceinline__ float group_fold_ordered(float acc, float term) {
     }
 }
 
-// ---- Q8_K activation quantizer, one wave per super-block ------------------------
-
 __device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d) {
     return (static_cast<uint32_t>(a) & 0xffu) | ((static_cast<uint32_t>(b) & 0xffu) << 8) |
            ((static_cast<uint32_t>(c) & 0xffu) << 16) | ((static_cast<uint32_t>(d) & 0xffu) << 24);
 }
+
+// ---- Q8_0 activation quantizer, eight lanes per block ---------------------------
+
+// Rust's `(v).round().clamp(-128.0, 127.0) as i8`: NaN casts to 0.
+__device__ __forceinline__ int q8_0_round(float v) {
+    float r = roundf(v);  // ties away from zero
+    if (r != r) return 0;
+    r = fminf(fmaxf(r, -128.0f), 127.0f);
+    return static_cast<int>(r);
+}
+
+// Quantizes one 32-value block held by eight consecutive lanes (lane l of the group holds
+// values 4l..4l+3): reference quantize_q8_0_block, src/inference.rs:22510-22528 -- amax = max |v|
+// (NaN ignored); u = amax / 127; scale = f16(u) widened back; inv = (u == 0) ? 0 : 1 / u (the
+// UNROUNDED u); q = clamp(round-half-away(v * inv), -128, 127).  Returns the lane's four quants
+// packed; `scale` is the same in all eight lanes.  All eight lanes of a group must call it together.
+__device__ __forceinline__ uint32_t q8_0_quantize_lane8(const float4 v, float &scale) {
+    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    amax = fmaxf(amax, __shfl_xor(amax, 1));
+    amax = fmaxf(amax, __shfl_xor(amax, 2));
+    amax = fmaxf(amax, __shfl_xor(amax, 4));
+    const float u = amax / 127.0f;
+    const float inv = (u == 0.0f) ? 0.0f : 1.0f / u;
+    // f32 -> f16 round-to-nearest-even -> f32 (reference f32_to_f16_bits, src/inference.rs:27062-27096)
+    scale = static_cast<float>(static_cast<_Float16>(u));
+    return pack4(q8_0_round(v.x * inv), q8_0_round(v.y * inv), q8_0_round(v.z * inv), q8_0_round(v.w * inv));
+}
+
+// ---- Q8_K activation quantizer, one wave per super-block ------------------------
 
 // The reference's nearest_int (src/inference.rs:23112-23116).
 __device__ __forceinline__ int nearest_int_magic(float f) {

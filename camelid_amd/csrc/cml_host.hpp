@@ -65,6 +65,12 @@ int plane_layout(int fmt, int64_t rows, int64_t nb, int64_t stride[4], size_t of
 int launch_quantize_q8_0(const float *x, int64_t n_tokens, int64_t cols, int8_t *q, float *s, hipStream_t st);
 int launch_quantize_q8_k(const float *x, int64_t n_tokens, int64_t cols, int8_t *q, float *d, hipStream_t st);
 
+// producers.hip: act = 0 (f32 only), 1 (Q8_0), 2 (Q8_K)
+int launch_rms_norm_quantize(int act, const float *x, const float *weight, float eps, int64_t n_tokens, int64_t cols,
+                             float *normed, int8_t *q, float *scales, hipStream_t st);
+int launch_silu_mul_quantize(int act, const float *g, const float *u, int64_t n_tokens, int64_t cols, int8_t *q, float *scales,
+                             hipStream_t st);
+
 // layout.hip: wire <-> planes, dequantize
 int launch_wire_to_planes(int fmt, const uint8_t *wire, int64_t rows, int64_t nb, const Planes &dst, hipStream_t st);
 int launch_planes_to_wire(int fmt, const Planes &src, int64_t rows, int64_t nb, int row_skip, uint8_t *wire, hipStream_t st);

@@ -127,29 +127,6 @@ static int launch_expert_matmul(const MatArgs &a, hipStream_t st) {
     return launch_gemv_q4k(a, st);
 }
 
-// h = silu(g) * u (reference CpuTensor::silu_mul, src/tensor/mod.rs:2610-2634:
-// (a / (1 + exp(-a))) * b), quantized to Q8_K on the fly (reference
-// quantize_q8_k_blocks, src/inference.rs:23121-23152).  One wave per 256-value
-// super-block, lane l holds values 4l..4l+3 -- the layout of quantize_q8_k_kernel.
-__global__ __launch_bounds__(256) void silu_mul_quantize_q8k_kernel(const float *__restrict__ g, const float *__restrict__ u,
-                                                                    int64_t n_sb, int8_t *__restrict__ q, float *__restrict__ d) {
-    const int lane = threadIdx.x & 63;
-    const int64_t sb = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6);
-    if (sb >= n_sb) return;
-    const float4 gv = reinterpret_cast<const float4 *>(g + sb * 256)[lane];
-    const float4 uv = reinterpret_cast<const float4 *>(u + sb * 256)[lane];
-    float4 v;
-    v.x = (gv.x / (1.0f + expf(-gv.x))) * uv.x;
-    v.y = (gv.y / (1.0f + expf(-gv.y))) * uv.y;
-    v.z = (gv.z / (1.0f + expf(-gv.z))) * uv.z;
-    v.w = (gv.w / (1.0f + expf(-gv.w))) * uv.w;
-    float dv;
-    int bsum;
-    const uint32_t packed = q8k_quantize_wave(v, dv, bsum);
-    reinterpret_cast<uint32_t *>(q + sb * 256)[lane] = packed;
-    if (lane == 0) d[sb] = dv;
-}
-
 // out[t][c] = ((0 + y[a(t,0)][c]*w[t][0]) + y[a(t,1)][c]*w[t][1]) + ...  (reference
 // src/inference.rs:14255-14257: `output += expert_out * weight`, routed order,
 // multiply and add rounded separately).
@@ -268,9 +245,7 @@ int cml_moe_ffn(const cml_weight *gate, const cml_weight *up, const cml_weight *
     a.out = ws.u;
     if (int rc = launch_expert_matmul(a, st)) return rc;
     // h = silu(g) * u, quantized per assignment
-    const int64_t h_sb = static_cast<int64_t>(n_slots) * (ff / 256);
-    hipLaunchKernelGGL(silu_mul_quantize_q8k_kernel, dim3(static_cast<unsigned>((h_sb + 3) / 4)), dim3(256), 0, st, ws.g, ws.u, h_sb, ws.hq, ws.hd);
-    CML_HIP_TRY(hipGetLastError());
+    if (int rc = launch_silu_mul_quantize(2, ws.g, ws.u, n_slots, ff, ws.hq, ws.hd, st)) return rc;
     // down: assignment j reads its own h
     a.q = ws.hq;
     a.scales = ws.hd;

@@ -1,0 +1,162 @@
+// The steps immediately upstream of a quantized projection, fused with the
+// activation quantizer so that the f32 intermediate never leaves the chip:
+//   rms_norm -> Q8_0 / Q8_K      reference rms_norm_quantize, rms_norm_quantize_q8k
+//                                (src/cuda_resident.rs:236-270, :4152-4177), CPU
+//                                arithmetic CpuTensor::rms_norm_into, src/tensor/mod.rs:2707-2760
+//   silu(gate) * up -> Q8_0/Q8_K reference silu_mul_quantize[_q8k] (src/cuda_resident.rs:
+//                                4289-4341), CPU arithmetic CpuTensor::silu_mul,
+//                                src/tensor/mod.rs:2610-2634
+// The quantizers are the ones of quantize.hip (same device functions), so the
+// fused result equals the composed one bit for bit.
+//
+// rms_norm keeps the reference's arithmetic exactly, including the part that
+// cannot be spread over lanes: the squares are summed left to right in f32 (a
+// tree sum reassociates and changes greedy tokens, as the reference's device
+// lane notes at src/cuda_resident.rs:124-131).  The row is staged in LDS, one
+// lane walks it in order -- about 4 cycles per element, ~7 us for 4096 values,
+// the price of that contract -- and every lane then applies (x * scale) * weight.
+// Rows are independent: one workgroup per token.
+#include "cml_device.hpp"
+#include "cml_host.hpp"
+
+#pragma clang fp contract(off)
+
+namespace cml {
+
+// ACT: 0 = f32 output only, 1 = Q8_0, 2 = Q8_K (normed may be written as well).
+template <int ACT>
+__global__ __launch_bounds__(256) void rms_norm_quantize_kernel(const float *__restrict__ x, const float *__restrict__ weight,
+                                                                float eps, int cols, float *__restrict__ normed,
+                                                                int8_t *__restrict__ q, float *__restrict__ scales) {
+    extern __shared__ float4 xs4[];  // the row: cols floats
+    __shared__ float s_scale;
+    float *xs = reinterpret_cast<float *>(xs4);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t token = blockIdx.x;
+    const int n4 = cols >> 2;
+    const float4 *x4 = reinterpret_cast<const float4 *>(x + token * cols);
+    for (int i = tid; i < n4; i += 256) xs4[i] = x4[i];
+    __syncthreads();
+    if (tid == 0) {
+        float sum = 0.0f;
+        for (int i = 0; i < n4; i++) {  // in order, every product and every sum rounded on its own
+            const float4 v = xs4[i];
+            sum = sum + v.x * v.x;
+            sum = sum + v.y * v.y;
+            sum = sum + v.z * v.z;
+            sum = sum + v.w * v.w;
+        }
+        const float mean_square = sum / static_cast<float>(cols);
+        s_scale = 1.0f / sqrtf(mean_square + eps);
+    }
+    __syncthreads();
+    const float scale = s_scale;
+    const float4 *w4 = reinterpret_cast<const float4 *>(weight);
+    float4 *n4out = normed ? reinterpret_cast<float4 *>(normed + token * cols) : nullptr;
+    for (int i = tid; i < n4; i += 256) {
+        const float4 v = xs4[i], w = w4[i];
+        float4 y;
+        y.x = (v.x * scale) * w.x;
+        y.y = (v.y * scale) * w.y;
+        y.z = (v.z * scale) * w.z;
+        y.w = (v.w * scale) * w.w;
+        if (ACT != 0) xs4[i] = y;
+        if (n4out) n4out[i] = y;
+    }
+    if constexpr (ACT == 0) return;
+    __syncthreads();
+    uint32_t *q32 = reinterpret_cast<uint32_t *>(q + token * cols);
+    if constexpr (ACT == 1) {
+        // eight lanes per 32-value block; cols/4 is a multiple of 8, so groups enter and leave together
+        float *sc = scales + token * (cols / 32);
+        for (int i = tid; i < n4; i += 256) {
+            float s;
+            const uint32_t packed = q8_0_quantize_lane8(xs4[i], s);
+            q32[i] = packed;
+            if ((i & 7) == 0) sc[i >> 3] = s;
+        }
+    } else {
+        // one wave per 256-value super-block
+        float *d = scales + token * (cols / 256);
+        for (int sb = wave; sb < cols / 256; sb += 4) {
+            float dv;
+            int bsum;
+            const uint32_t packed = q8k_quantize_wave(xs4[sb * 64 + lane], dv, bsum);
+            q32[sb * 64 + lane] = packed;
+            if (lane == 0) d[sb] = dv;
+        }
+    }
+    (void)xs;
+}
+
+int launch_rms_norm_quantize(int act, const float *x, const float *weight, float eps, int64_t n_tokens, int64_t cols,
+                             float *normed, int8_t *q, float *scales, hipStream_t st) {
+    if (n_tokens == 0 || cols == 0) return CML_OK;
+    const size_t lds = static_cast<size_t>(cols) * sizeof(float);
+    if (lds > 64 * 1024 - 64) return fail(CML_ERR_UNSUPPORTED, "rms_norm row of %lld values exceeds the LDS staging limit", (long long)cols);
+    const dim3 grid(static_cast<unsigned>(n_tokens)), block(256);
+    const int c = static_cast<int>(cols);
+    switch (act) {
+        case 0: hipLaunchKernelGGL(rms_norm_quantize_kernel<0>, grid, block, lds, st, x, weight, eps, c, normed, q, scales); break;
+        case 1: hipLaunchKernelGGL(rms_norm_quantize_kernel<1>, grid, block, lds, st, x, weight, eps, c, normed, q, scales); break;
+        default: hipLaunchKernelGGL(rms_norm_quantize_kernel<2>, grid, block, lds, st, x, weight, eps, c, normed, q, scales); break;
+    }
+    CML_HIP_TRY(hipGetLastError());
+    return CML_OK;
+}
+
+// h = silu(g) * u = (g / (1 + exp(-g))) * u, quantized on the fly.  Q8_K: one wave per
+// 256-value super-block, lane l holding values 4l..4l+3 (the layout of quantize_q8_k_kernel).
+__device__ __forceinline__ float4 silu_mul4(const float4 gv, const float4 uv) {
+    float4 v;
+    v.x = (gv.x / (1.0f + expf(-gv.x))) * uv.x;
+    v.y = (gv.y / (1.0f + expf(-gv.y))) * uv.y;
+    v.z = (gv.z / (1.0f + expf(-gv.z))) * uv.z;
+    v.w = (gv.w / (1.0f + expf(-gv.w))) * uv.w;
+    return v;
+}
+
+__global__ __launch_bounds__(256) void silu_mul_quantize_q8k_kernel(const float *__restrict__ g, const float *__restrict__ u,
+                                                                    int64_t n_sb, int8_t *__restrict__ q, float *__restrict__ d) {
+    const int lane = threadIdx.x & 63;
+    const int64_t sb = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (sb >= n_sb) return;
+    const float4 v = silu_mul4(reinterpret_cast<const float4 *>(g + sb * 256)[lane], reinterpret_cast<const float4 *>(u + sb * 256)[lane]);
+    float dv;
+    int bsum;
+    const uint32_t packed = q8k_quantize_wave(v, dv, bsum);
+    reinterpret_cast<uint32_t *>(q + sb * 256)[lane] = packed;
+    if (lane == 0) d[sb] = dv;
+}
+
+// Q8_0: one thread per 4 values, 8 threads per 32-value block (the layout of quantize_q8_0_kernel).
+__global__ __launch_bounds__(256) void silu_mul_quantize_q8_0_kernel(const float *__restrict__ g, const float *__restrict__ u,
+                                                                     int64_t n_blocks, int8_t *__restrict__ q, float *__restrict__ scales) {
+    const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    const int64_t block = tid >> 3;
+    const bool live = block < n_blocks;
+    const int64_t src = live ? tid : 0;
+    const float4 v = silu_mul4(reinterpret_cast<const float4 *>(g)[src], reinterpret_cast<const float4 *>(u)[src]);
+    float scale;
+    const uint32_t packed = q8_0_quantize_lane8(v, scale);
+    if (!live) return;
+    reinterpret_cast<uint32_t *>(q)[tid] = packed;
+    if ((tid & 7) == 0) scales[block] = scale;
+}
+
+int launch_silu_mul_quantize(int act, const float *g, const float *u, int64_t n_tokens, int64_t cols, int8_t *q, float *scales,
+                             hipStream_t st) {
+    if (n_tokens == 0 || cols == 0) return CML_OK;
+    if (act == 1) {
+        const int64_t n_blocks = n_tokens * (cols / 32);
+        const unsigned grid = static_cast<unsigned>((n_blocks * 8 + 255) / 256);
+        hipLaunchKernelGGL(silu_mul_quantize_q8_0_kernel, dim3(grid), dim3(256), 0, st, g, u, n_blocks, q, scales);
+    } else {
+        const int64_t n_sb = n_tokens * (cols / 256);
+        hipLaunchKernelGGL(silu_mul_quantize_q8k_kernel, dim3(static_cast<unsigned>((n_sb + 3) / 4)), dim3(256), 0, st, g, u, n_sb, q, scales);
+    }
+    CML_HIP_TRY(hipGetLastError());
+    return CML_OK;
+}
+
+}  // namespace cml

@@ -19,14 +19,6 @@
 
 namespace cml {
 
-// Rust's `(v).round().clamp(-128.0, 127.0) as i8`: NaN casts to 0.
-__device__ __forceinline__ int q8_0_round(float v) {
-    float r = roundf(v);  // ties away from zero
-    if (r != r) return 0;
-    r = fminf(fmaxf(r, -128.0f), 127.0f);
-    return static_cast<int>(r);
-}
-
 // One thread per 4 values, 8 threads per 32-value block.
 __global__ __launch_bounds__(256) void quantize_q8_0_kernel(const float *__restrict__ x, int64_t n_blocks,
                                                             int8_t *__restrict__ q, float *__restrict__ scales) {
@@ -35,19 +27,11 @@ __global__ __launch_bounds__(256) void quantize_q8_0_kernel(const float *__restr
     const bool live = block < n_blocks;
     const int64_t src = live ? tid : 0;
     const float4 v = reinterpret_cast<const float4 *>(x)[src];
-    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-    amax = fmaxf(amax, __shfl_xor(amax, 1));
-    amax = fmaxf(amax, __shfl_xor(amax, 2));
-    amax = fmaxf(amax, __shfl_xor(amax, 4));
-    const float u = amax / 127.0f;
-    const float inv = (u == 0.0f) ? 0.0f : 1.0f / u;
+    float scale;
+    const uint32_t packed = q8_0_quantize_lane8(v, scale);
     if (!live) return;
-    reinterpret_cast<uint32_t *>(q)[tid] =
-        pack4(q8_0_round(v.x * inv), q8_0_round(v.y * inv), q8_0_round(v.z * inv), q8_0_round(v.w * inv));
-    if ((tid & 7) == 0) {
-        // f32 -> f16 round-to-nearest-even -> f32 (reference f32_to_f16_bits, src/inference.rs:27062-27096).
-        scales[block] = static_cast<float>(static_cast<_Float16>(u));
-    }
+    reinterpret_cast<uint32_t *>(q)[tid] = packed;
+    if ((tid & 7) == 0) scales[block] = scale;
 }
 
 // One wave per 256-value super-block; lane l holds values 4l..4l+3.

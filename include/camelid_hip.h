@@ -151,6 +151,27 @@ int cml_quantize_q8_0(const float *x_dev, int64_t n_tokens, int64_t cols, int8_t
 int cml_quantize_q8_k(const float *x_dev, int64_t n_tokens, int64_t cols, int8_t *q_dev,
                       float *d_dev, cml_stream_t stream);
 
+/* ---- fused producers: the step upstream of a projection, quantizing as it goes.
+ *      act selects the activation format: CML_ACT_F32 (no quantized output),
+ *      CML_ACT_Q8_0 (scales per 32 values) or CML_ACT_Q8_K (per 256). -------- */
+enum { CML_ACT_F32 = 0, CML_ACT_Q8_0 = 1, CML_ACT_Q8_K = 2 };
+/* RMS norm of every row (reference CpuTensor::rms_norm_into, src/tensor/mod.rs:
+ * 2707-2760: squares summed left to right in f32, scale = 1/sqrt(mean + eps),
+ * out = (x*scale)*weight), then the quantizer above on the normalised row
+ * (reference rms_norm_quantize / rms_norm_quantize_q8k, src/cuda_resident.rs:
+ * 236-270, :4152-4177).  normed_dev (f32[n_tokens*cols]) may be null when only
+ * the quantized form is wanted; q_dev/scales_dev are ignored for CML_ACT_F32.
+ * Rows of up to 16368 values. */
+int cml_rms_norm_quantize(int act, const float *x_dev, const float *weight_dev, float eps,
+                          int64_t n_tokens, int64_t cols, float *normed_dev, int8_t *q_dev,
+                          float *scales_dev, cml_stream_t stream);
+/* silu(gate) * up = (g / (1 + exp(-g))) * u per element (reference
+ * CpuTensor::silu_mul, src/tensor/mod.rs:2610-2634), quantized (reference
+ * silu_mul_quantize / _q8k, src/cuda_resident.rs:4289-4341).  act must be
+ * CML_ACT_Q8_0 or CML_ACT_Q8_K. */
+int cml_silu_mul_quantize(int act, const float *gate_dev, const float *up_dev, int64_t n_tokens,
+                          int64_t cols, int8_t *q_dev, float *scales_dev, cml_stream_t stream);
+
 /* ---- dequantize (reference Q4KBlock::dequantize & siblings,
  *      src/tensor/mod.rs:5365-5409, :5547-5572, :5903-5924, :6039-6066) ----- */
 /* out_dev: f32[rows*cols], bit-identical to the reference decoders. */

@@ -64,6 +64,8 @@ def lib() -> C.CDLL:
         L.orc_softmax_top_k.argtypes = [vp, i32, i32, vp, vp]
         L.orc_softmax_top_k.restype = i32
         L.orc_silu_mul.argtypes = [vp, vp, sz, vp]
+        L.orc_rms_norm.argtypes = [vp, vp, C.c_float, sz, sz, vp]
+        L.orc_rms_norm.restype = None
         L.orc_moe_ffn.argtypes = [i32, vp, vp, vp, i32, i32, sz, sz, vp, vp, sz, vp, i32]
         L.orc_moe_ffn.restype = i32
         L.orc_quantize_weights.argtypes = [i32, vp, sz, vp, i32]
@@ -231,6 +233,16 @@ def softmax_top_k(logits, k: int):
     w = np.empty(max(kk, 1), np.float32)
     n = lib().orc_softmax_top_k(_p(logits), logits.size, k, _p(idx), _p(w))
     return idx[:n].copy(), w[:n].copy()
+
+
+def rms_norm(x, weight, eps: float) -> np.ndarray:
+    """Rows of x normalised as the reference does (sequential f32 sum of squares)."""
+    x = _c(x, np.float32)
+    weight = _c(weight, np.float32)
+    x2 = x.reshape(-1, weight.size)
+    out = np.empty_like(x2)
+    lib().orc_rms_norm(_p(x2), _p(weight), C.c_float(eps), x2.shape[0], x2.shape[1], _p(out))
+    return out.reshape(x.shape)
 
 
 def silu_mul(a, b) -> np.ndarray:

@@ -761,6 +761,22 @@ void orc_silu_mul(const float *a, const float *b, size_t n, float *out) {
         out[i] = (a[i] / (1.0f + expf(-a[i]))) * b[i];
 }
 
+/* src/tensor/mod.rs:2707-2760 (the portable branch): per row, the squares are summed
+ * left to right in f32, mean = sum / cols, scale = 1 / sqrt(mean + eps),
+ * out = (x * scale) * weight. */
+void orc_rms_norm(const float *x, const float *weight, float eps, size_t rows, size_t cols, float *out) {
+    for (size_t r = 0; r < rows; r++) {
+        const float *in = x + r * cols;
+        float sum = 0.0f;
+        for (size_t c = 0; c < cols; c++)
+            sum = sum + in[c] * in[c];
+        float mean_square = sum / (float)cols;
+        float scale = 1.0f / sqrtf(mean_square + eps);
+        for (size_t c = 0; c < cols; c++)
+            out[r * cols + c] = (in[c] * scale) * weight[c];
+    }
+}
+
 /* src/inference.rs:14142-14280 with quantized expert bands
  * (src/gemma4_runtime.rs:1084-1110 for the band matvec). */
 int orc_moe_ffn(int fmt, const uint8_t *gate, const uint8_t *up, const uint8_t *down,

@@ -31,6 +31,10 @@
  *                                ("parity unpinned" for the last-ulp value).
  *   softmax_top_k              : closed forms and brute force on small inputs;
  *                                libm expf may differ from Rust's by 1 ulp.
+ *   rms_norm                   : the reference's known vector (tests/
+ *                                tensor_primitives.rs:83-93), exact power-of-two
+ *                                cases, an order-sensitive input checked against
+ *                                an independent sequential sum, f64 within 1e-6.
  *   weight quantizers          : reconstruction-error bounds on the reference's
  *                                ramps; they only generate inputs.
  */
@@ -114,6 +118,10 @@ int orc_matmul_q(int fmt, int order, const uint8_t *wire, size_t cols,
 /* Mixtral routing: src/inference.rs:13940-13991.  Writes min(k, n) pairs,
  * returns the count. */
 int orc_softmax_top_k(const float *logits, int n, int k, int32_t *idx, float *w);
+
+/* RMS norm, the step upstream of the activation quantizers:
+ * src/tensor/mod.rs:2707-2760 (sequential f32 sum of squares). */
+void orc_rms_norm(const float *x, const float *weight, float eps, size_t rows, size_t cols, float *out);
 
 /* Expert activation: src/tensor/mod.rs:2610-2634. */
 void orc_silu_mul(const float *a, const float *b, size_t n, float *out);

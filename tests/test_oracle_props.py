@@ -432,3 +432,47 @@ def test_q6_k_input_generator_round_trips_within_a_step():
     assert not rec[256:512].any()
     step = np.abs(w.reshape(-1, 16)).max(axis=1) / 31.0
     assert np.all(np.abs(rec - w).reshape(-1, 16) <= step[:, None] * 1.05 + 1e-6)
+
+
+# ------------------------------------------------------------------ rms_norm ----
+
+def test_rms_norm_known_vector_of_the_reference():
+    """tests/tensor_primitives.rs:83-93 of the reference: x = [3, 4], w = [1, 2], eps = 0."""
+    out = oracle.rms_norm(np.array([[3.0, 4.0]], np.float32), np.array([1.0, 2.0], np.float32), 0.0)
+    rms = np.sqrt(np.float32((9.0 + 16.0) / 2.0))
+    assert abs(out[0, 0] - 3.0 / rms) < 1e-5 and abs(out[0, 1] - 4.0 / rms * 2.0) < 1e-5
+
+
+def test_rms_norm_exact_cases_and_summation_order():
+    # powers of two make every step exact: 256 values of 0.5 -> mean 0.25 -> scale 2 -> out = w
+    w = np.linspace(-3, 3, 256, dtype=np.float32)
+    out = oracle.rms_norm(np.full((1, 256), 0.5, np.float32), w, 0.0)
+    assert np.array_equal(out[0].view(np.uint32), w.view(np.uint32))
+    # eps enters under the root: x = 0 -> scale = 1/sqrt(eps), out = 0 * scale * w = 0
+    assert np.all(oracle.rms_norm(np.zeros((1, 64), np.float32), np.ones(64, np.float32), 1e-5) == 0)
+    # left-to-right f32 sum: 1 followed by 2^24 .. the small squares after a huge one vanish one by one,
+    # whereas a pairwise sum would keep them
+    x = np.zeros((1, 4096), np.float32)
+    x[0, 0] = 4096.0                      # square 2^24
+    x[0, 1:] = 1.0                        # 4095 squares of 1: sequentially each is absorbed (2^24 + 1 rounds to 2^24)
+    out = oracle.rms_norm(x, np.ones(4096, np.float32), 0.0)
+    seq_scale = np.float32(1.0) / np.sqrt(np.float32(2.0 ** 24) / np.float32(4096))
+    assert out[0, 1].view(np.uint32) == np.float32(np.float32(1.0) * seq_scale).view(np.uint32)
+    tree_scale = np.float32(1.0) / np.sqrt(np.float32(2.0 ** 24 + 4095) / np.float32(4096))
+    assert out[0, 1] != np.float32(tree_scale)   # a reassociated sum would have given this
+    # reversed order: the ones add up first (exactly 4095), then 2^24 + 4095 rounds to even
+    out_r = oracle.rms_norm(x[:, ::-1].copy(), np.ones(4096, np.float32), 0.0)
+    rev_scale = np.float32(1.0) / np.sqrt(np.float32(np.float32(4095.0) + np.float32(2.0 ** 24)) / np.float32(4096))
+    assert out_r[0, 0].view(np.uint32) == np.float32(np.float32(1.0) * rev_scale).view(np.uint32)
+
+
+def test_rms_norm_against_float64_and_rows_are_independent():
+    rng = np.random.default_rng(77)
+    x = rng.standard_normal((5, 3072)).astype(np.float32)
+    w = (rng.standard_normal(3072) * 0.5 + 1.0).astype(np.float32)
+    out = oracle.rms_norm(x, w, 1e-6)
+    x64 = x.astype(np.float64)
+    ref = x64 / np.sqrt((x64 ** 2).mean(axis=1, keepdims=True) + 1e-6) * w.astype(np.float64)
+    assert np.max(np.abs(out - ref) / np.maximum(np.abs(ref), 1.0)) < 1e-6
+    for r in range(5):
+        assert np.array_equal(oracle.rms_norm(x[r:r + 1], w, 1e-6)[0].view(np.uint32), out[r].view(np.uint32))
