@@ -215,6 +215,44 @@ def bench_moe(name: str, K: int, W: int, seed: int, cpu_seconds: float) -> int:
     return 0
 
 
+PRODUCER_CONFIGS = {
+    # name -> (cols, tokens): rms_norm fused with the Q8_K quantizer, the step upstream of a projection
+    "rmsnorm_q8k_4096_t1": (4096, 1),
+    "rmsnorm_q8k_4096_t32": (4096, 32),
+}
+
+
+def bench_producer(name: str, K: int, W: int, seed: int) -> int:
+    """rms_norm + Q8_K quantize of `tokens` rows.  Latency-bound by construction: the reference's
+    left-to-right sum of squares runs in one lane per row."""
+    L = lib()
+    cols, T = PRODUCER_CONFIGS[name]
+    rng = np.random.default_rng(seed)
+    xd = DeviceBuffer.from_numpy(rng.standard_normal((T, cols)).astype(np.float32))
+    wd = DeviceBuffer.from_numpy((rng.standard_normal(cols) * 0.5 + 1).astype(np.float32))
+    qd, sd = DeviceBuffer(T * cols), DeviceBuffer(T * (cols // 256) * 4)
+    stream = C.c_void_p()
+    check(L.cml_stream_create(C.byref(stream)))
+    timer = Timer(stream)
+
+    def step(i):
+        check(L.cml_rms_norm_quantize(2, xd.ptr, wd.ptr, 1e-6, T, cols, None, qd.ptr, sd.ptr, stream), "cml_rms_norm_quantize")
+
+    for i in range(W):
+        step(i)
+    g = capture(stream, step, K)
+    time_graph(stream, g, timer)
+    ms = min(time_graph(stream, g, timer) for _ in range(3)) / K
+    alg = T * cols * 5 + cols * 4 + T * (cols // 256) * 4
+    print(json.dumps({"metric": f"rms_norm + Q8_K quantize µs, {cols} values x {T} token(s)", "value": round(ms * 1e3, 3), "unit": "us",
+                      "higher_is_better": False, "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": round(ms, 6),
+                      "dtype": "f32", "data": "synthetic", "config": {"workload": name, "algorithmic_bytes_per_call": alg},
+                      "roofline": {"bound": "hbm", "achieved": round(alg / (ms * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                   "frac": round(alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 6), "traffic": None,
+                                   "note": "latency-bound: one lane sums the squares in the reference's order"}}, ensure_ascii=False))
+    return 0
+
+
 def calibrate_copy(nbytes: int, K: int, W: int) -> int:
     """Plain copy kernel over rotating buffers: what this box's HBM gives a kernel with no arithmetic."""
     L = lib()
@@ -249,7 +287,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--config", default="q4k_14336x4096_n1", choices=sorted(CONFIGS) + sorted(MOE_CONFIGS))
+    ap.add_argument("--config", default="q4k_14336x4096_n1", choices=sorted(CONFIGS) + sorted(MOE_CONFIGS) + sorted(PRODUCER_CONFIGS))
     ap.add_argument("--copies", type=int, default=0, help="distinct weight copies to rotate over (0 = enough for ~600 MB)")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="time budget of the CPU baseline leg (0 = skip)")
     ap.add_argument("--seed", type=int, default=1234)
@@ -271,6 +309,8 @@ def main() -> int:
     B.init(0)
     if args.calibrate_copy:
         return calibrate_copy(args.calibrate_copy, max(1, args.steps), max(0, args.warmup))
+    if args.config in PRODUCER_CONFIGS:
+        return bench_producer(args.config, max(1, args.steps), max(0, args.warmup), args.seed)
     if args.config in MOE_CONFIGS:
         return bench_moe(args.config, max(1, args.steps), max(0, args.warmup), args.seed, args.cpu_seconds)
     fmt_name, rows, cols, n = CONFIGS[args.config]

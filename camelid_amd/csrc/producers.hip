@@ -13,8 +13,9 @@
 // cannot be spread over lanes: the squares are summed left to right in f32 (a
 // tree sum reassociates and changes greedy tokens, as the reference's device
 // lane notes at src/cuda_resident.rs:124-131).  The row is staged in LDS, one
-// lane walks it in order -- about 4 cycles per element, ~7 us for 4096 values,
-// the price of that contract -- and every lane then applies (x * scale) * weight.
+// wave walks it in order -- one dependent addition per element, a few microseconds
+// for 4096 values, the price of that contract -- and every lane then applies
+// (x * scale) * weight.
 // Rows are independent: one workgroup per token.
 #include "cml_device.hpp"
 #include "cml_host.hpp"
@@ -24,44 +25,91 @@
 namespace cml {
 
 // ACT: 0 = f32 output only, 1 = Q8_0, 2 = Q8_K (normed may be written as well).
+// Every thread keeps its share of the row in registers (up to kRmsRegs float4) and puts the
+// squares into LDS; wave 0 then adds them up in order, reading ahead in batches so that the
+// only thing on its critical path is the chain of additions; the LDS row is reused for the
+// normalised values the quantizers read.
+constexpr int kRmsRegs = 16;  // float4 per thread: rows of up to 16 * 256 * 4 = 16384 values
+
 template <int ACT>
 __global__ __launch_bounds__(256) void rms_norm_quantize_kernel(const float *__restrict__ x, const float *__restrict__ weight,
                                                                 float eps, int cols, float *__restrict__ normed,
                                                                 int8_t *__restrict__ q, float *__restrict__ scales) {
-    extern __shared__ float4 xs4[];  // the row: cols floats
+    extern __shared__ float4 xs4[];  // the row, padded to whole batches: squares first, then the normalised values
     __shared__ float s_scale;
-    float *xs = reinterpret_cast<float *>(xs4);
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int64_t token = blockIdx.x;
     const int n4 = cols >> 2;
     const float4 *x4 = reinterpret_cast<const float4 *>(x + token * cols);
-    for (int i = tid; i < n4; i += 256) xs4[i] = x4[i];
+    float4 xv[kRmsRegs];
+#pragma unroll
+    for (int k = 0; k < kRmsRegs; k++) {
+        const int i = tid + k * 256;
+        if (i < n4) {
+            const float4 v = x4[i];
+            xv[k] = v;
+            xs4[i] = make_float4(v.x * v.x, v.y * v.y, v.z * v.z, v.w * v.w);
+        }
+    }
+    // zeros from the end of the row up to the next multiple of 16 float4 and one more batch pair:
+    // the walk below runs in whole batches and reads one batch ahead, and sum + 0 == sum exactly
+    // (the sum of squares is never negative)
+    const int n4p = (n4 + 15) & ~15;
+    if (tid < n4p + 16 - n4) xs4[n4 + tid] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     __syncthreads();
-    if (tid == 0) {
+    if (wave == 0) {
+        // Left to right, every sum rounded on its own (the products were rounded above).  All lanes
+        // of the wave run the same chain on the same (broadcast) reads.  Two register batches
+        // alternate so that nothing but the additions sits between consecutive LDS reads.
+        constexpr int B = 8;
+        float4 ra[B], rb[B];
+#pragma unroll
+        for (int j = 0; j < B; j++) ra[j] = xs4[j];
         float sum = 0.0f;
-        for (int i = 0; i < n4; i++) {  // in order, every product and every sum rounded on its own
-            const float4 v = xs4[i];
-            sum = sum + v.x * v.x;
-            sum = sum + v.y * v.y;
-            sum = sum + v.z * v.z;
-            sum = sum + v.w * v.w;
+        for (int i = 0; i < n4p; i += 2 * B) {
+#pragma unroll
+            for (int j = 0; j < B; j++) rb[j] = xs4[i + B + j];
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < B; j++) {
+                sum = sum + ra[j].x;
+                sum = sum + ra[j].y;
+                sum = sum + ra[j].z;
+                sum = sum + ra[j].w;
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < B; j++) ra[j] = xs4[i + 2 * B + j];
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < B; j++) {
+                sum = sum + rb[j].x;
+                sum = sum + rb[j].y;
+                sum = sum + rb[j].z;
+                sum = sum + rb[j].w;
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
         const float mean_square = sum / static_cast<float>(cols);
-        s_scale = 1.0f / sqrtf(mean_square + eps);
+        if (lane == 0) s_scale = 1.0f / sqrtf(mean_square + eps);
     }
     __syncthreads();
     const float scale = s_scale;
     const float4 *w4 = reinterpret_cast<const float4 *>(weight);
     float4 *n4out = normed ? reinterpret_cast<float4 *>(normed + token * cols) : nullptr;
-    for (int i = tid; i < n4; i += 256) {
-        const float4 v = xs4[i], w = w4[i];
-        float4 y;
-        y.x = (v.x * scale) * w.x;
-        y.y = (v.y * scale) * w.y;
-        y.z = (v.z * scale) * w.z;
-        y.w = (v.w * scale) * w.w;
-        if (ACT != 0) xs4[i] = y;
-        if (n4out) n4out[i] = y;
+#pragma unroll
+    for (int k = 0; k < kRmsRegs; k++) {
+        const int i = tid + k * 256;
+        if (i < n4) {
+            const float4 v = xv[k], w = w4[i];
+            float4 y;
+            y.x = (v.x * scale) * w.x;
+            y.y = (v.y * scale) * w.y;
+            y.z = (v.z * scale) * w.z;
+            y.w = (v.w * scale) * w.w;
+            if (ACT != 0) xs4[i] = y;
+            if (n4out) n4out[i] = y;
+        }
     }
     if constexpr (ACT == 0) return;
     __syncthreads();
@@ -86,14 +134,14 @@ __global__ __launch_bounds__(256) void rms_norm_quantize_kernel(const float *__r
             if (lane == 0) d[sb] = dv;
         }
     }
-    (void)xs;
 }
 
 int launch_rms_norm_quantize(int act, const float *x, const float *weight, float eps, int64_t n_tokens, int64_t cols,
                              float *normed, int8_t *q, float *scales, hipStream_t st) {
     if (n_tokens == 0 || cols == 0) return CML_OK;
-    const size_t lds = static_cast<size_t>(cols) * sizeof(float);
-    if (lds > 64 * 1024 - 64) return fail(CML_ERR_UNSUPPORTED, "rms_norm row of %lld values exceeds the LDS staging limit", (long long)cols);
+    if (cols > static_cast<int64_t>(kRmsRegs) * 1024 - 32)
+        return fail(CML_ERR_UNSUPPORTED, "rms_norm row of %lld values exceeds the staging limit of %d", (long long)cols, kRmsRegs * 1024 - 32);
+    const size_t lds = (((static_cast<size_t>(cols) / 4 + 15) & ~size_t(15)) + 16) * sizeof(float4);
     const dim3 grid(static_cast<unsigned>(n_tokens)), block(256);
     const int c = static_cast<int>(cols);
     switch (act) {

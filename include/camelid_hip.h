@@ -161,7 +161,7 @@ enum { CML_ACT_F32 = 0, CML_ACT_Q8_0 = 1, CML_ACT_Q8_K = 2 };
  * (reference rms_norm_quantize / rms_norm_quantize_q8k, src/cuda_resident.rs:
  * 236-270, :4152-4177).  normed_dev (f32[n_tokens*cols]) may be null when only
  * the quantized form is wanted; q_dev/scales_dev are ignored for CML_ACT_F32.
- * Rows of up to 16368 values. */
+ * Rows of up to 16352 values. */
 int cml_rms_norm_quantize(int act, const float *x_dev, const float *weight_dev, float eps,
                           int64_t n_tokens, int64_t cols, float *normed_dev, int8_t *q_dev,
                           float *scales_dev, cml_stream_t stream);
