@@ -460,6 +460,23 @@ int cml_dequantize(const cml_weight *w, float *out_dev, cml_stream_t stream) {
     return launch_dequantize(w, out_dev, as_stream(stream));
 }
 
+int cml_embed_gather(const cml_weight *table, const uint32_t *token_ids_dev, int64_t n_tokens, float *out_dev, cml_stream_t stream) {
+    if (!table) return fail(CML_ERR_INVALID, "null weight");
+    if (int rc = check_ready()) return rc;
+    if (n_tokens < 0) return fail(CML_ERR_SHAPE, "negative token count");
+    if (n_tokens == 0 || table->cols == 0) return CML_OK;
+    if (!token_ids_dev || !out_dev) return fail(CML_ERR_INVALID, "null pointer");
+    return launch_embed_gather(table, token_ids_dev, n_tokens, out_dev, as_stream(stream));
+}
+
+int cml_argmax_f32(const float *logits_dev, int64_t n_rows, int64_t n, uint32_t *out_idx_dev, cml_stream_t stream) {
+    if (int rc = check_ready()) return rc;
+    if (n_rows < 0 || n <= 0 || n > INT32_MAX) return fail(CML_ERR_SHAPE, "argmax over %lld rows of %lld values", (long long)n_rows, (long long)n);
+    if (n_rows == 0) return CML_OK;
+    if (!logits_dev || !out_idx_dev) return fail(CML_ERR_INVALID, "null pointer");
+    return launch_argmax_f32(logits_dev, n_rows, n, out_idx_dev, as_stream(stream));
+}
+
 // ---- matvec / matmul --------------------------------------------------------------------------------
 
 static int dispatch(const MatArgs &a, hipStream_t st) {

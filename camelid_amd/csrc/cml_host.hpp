@@ -75,6 +75,8 @@ int launch_silu_mul_quantize(int act, const float *g, const float *u, int64_t n_
 int launch_wire_to_planes(int fmt, const uint8_t *wire, int64_t rows, int64_t nb, const Planes &dst, hipStream_t st);
 int launch_planes_to_wire(int fmt, const Planes &src, int64_t rows, int64_t nb, int row_skip, uint8_t *wire, hipStream_t st);
 int launch_dequantize(const cml_weight *w, float *out, hipStream_t st);
+int launch_embed_gather(const cml_weight *table, const uint32_t *token_ids, int64_t n_tokens, float *out, hipStream_t st);
+int launch_argmax_f32(const float *logits, int64_t n_rows, int64_t n, uint32_t *out_idx, hipStream_t st);
 
 // Arguments common to every gemv/gemm launcher.
 struct MatArgs {

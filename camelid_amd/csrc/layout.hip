@@ -158,15 +158,33 @@ int launch_planes_to_wire(int fmt, const Planes &src, int64_t rows, int64_t nb, 
 // One thread per output value; the float operations and their order are the
 // reference decoders' (each product and difference rounds on its own).
 
+// Output row -> weight row.  With `row_ids` (embedding gather) output row r decodes weight row
+// row_ids[r]; an id outside the table yields -1 and the caller writes NaN instead of reading.
+struct RowMap {
+    const uint32_t *row_ids;  // device, or null: identity
+    int64_t table_rows;
+};
+__device__ __forceinline__ int64_t map_row(const RowMap &m, int64_t out_row) {
+    if (!m.row_ids) return out_row;
+    const uint32_t id = m.row_ids[out_row];
+    return id < static_cast<uint64_t>(m.table_rows) ? static_cast<int64_t>(id) : -1;
+}
+__device__ __forceinline__ float quiet_nan() { return __builtin_bit_cast(float, 0x7fc00000u); }
+
 // Q8_0: scale * q (reference src/tensor/mod.rs:5365-5378).
 // Q4_0: (nibble - 8) * scale (reference src/inference.rs:25698-25708).
-__global__ __launch_bounds__(256) void dequant_q8q4_kernel(int fmt, Planes pl, int64_t nb, int64_t n_values,
+__global__ __launch_bounds__(256) void dequant_q8q4_kernel(int fmt, Planes pl, int64_t nb, int64_t n_values, RowMap rm,
                                                            float *__restrict__ out) {
     const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i >= n_values) return;
     const int64_t g = i >> 5;
     const int j = static_cast<int>(i & 31);
-    const int64_t row = g / nb, b = g - row * nb;
+    const int64_t out_row = g / nb, b = g - out_row * nb;
+    const int64_t row = map_row(rm, out_row);
+    if (row < 0) {
+        out[i] = quiet_nan();
+        return;
+    }
     const float d = f16_bits_to_f32(ldg2(pl.p[1] + row * pl.row_stride[1] + b * 2));
     if (fmt == CML_Q8_0) {
         const int q = static_cast<int8_t>(pl.p[0][row * pl.row_stride[0] + b * 32 + j]);
@@ -181,12 +199,18 @@ __global__ __launch_bounds__(256) void dequant_q8q4_kernel(int fmt, Planes pl, i
 // Q4_K: (d*sc)*q - (dmin*m) (reference Q4KBlock::dequantize, src/tensor/mod.rs:5903-5924;
 // q4_k_scale_min, :5997-6006).
 __global__ __launch_bounds__(256) void dequant_q4k_kernel(const uint8_t *__restrict__ tiled, int64_t sb_stride,
-                                                          int64_t nb, int64_t n_values, int row_skip, float *__restrict__ out) {
+                                                          int64_t nb, int64_t n_values, int row_skip, RowMap rm,
+                                                          float *__restrict__ out) {
     const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i >= n_values) return;
     const int64_t blk = i >> 8;
     const int64_t out_row = blk / nb, sb = blk - out_row * nb;
-    const int64_t row = out_row + row_skip;
+    const int64_t mapped = map_row(rm, out_row);
+    if (mapped < 0) {
+        out[i] = quiet_nan();
+        return;
+    }
+    const int64_t row = mapped + row_skip;
     const int rr = static_cast<int>(row & 15);
     const uint8_t *chunk = tiled + sb * sb_stride + (row >> 4) * 2304;
     const uint8_t *hdr = chunk + rr * 16;
@@ -212,13 +236,18 @@ __global__ __launch_bounds__(256) void dequant_q4k_kernel(const uint8_t *__restr
 }
 
 // Q6_K: (d*sc)*q (reference Q6KBlock::dequantize, src/tensor/mod.rs:6039-6066).
-__global__ __launch_bounds__(256) void dequant_q6k_kernel(Planes pl, int64_t nb, int64_t n_values,
+__global__ __launch_bounds__(256) void dequant_q6k_kernel(Planes pl, int64_t nb, int64_t n_values, RowMap rm,
                                                           float *__restrict__ out) {
     const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i >= n_values) return;
     const int64_t g = i >> 8;
     const int v = static_cast<int>(i & 255);
-    const int64_t row = g / nb, b = g - row * nb;
+    const int64_t out_row = g / nb, b = g - out_row * nb;
+    const int64_t row = map_row(rm, out_row);
+    if (row < 0) {
+        out[i] = quiet_nan();
+        return;
+    }
     const int half = v >> 7, r = v & 127, quarter = r >> 5, l = r & 31;
     const uint8_t qlb = pl.p[0][row * pl.row_stride[0] + b * 128 + 64 * half + l + ((quarter & 1) ? 32 : 0)];
     const uint8_t qhb = pl.p[1][row * pl.row_stride[1] + b * 64 + 32 * half + l];
@@ -229,24 +258,76 @@ __global__ __launch_bounds__(256) void dequant_q6k_kernel(Planes pl, int64_t nb,
     out[i] = d * static_cast<float>(sc) * static_cast<float>(q);
 }
 
-int launch_dequantize(const cml_weight *w, float *out, hipStream_t st) {
-    const int64_t n_values = w->rows * w->cols;
+// Decodes `n_rows` rows: the weight's own rows in order (row_ids null), or the rows row_ids[0..n_rows).
+static int dequantize_rows(const cml_weight *w, const uint32_t *row_ids, int64_t n_rows, float *out, hipStream_t st) {
+    const int64_t n_values = n_rows * w->cols;
     if (n_values == 0) return CML_OK;
     const unsigned grid = static_cast<unsigned>((n_values + 255) / 256);
+    const RowMap rm{row_ids, w->rows};
     switch (w->fmt) {
         case CML_Q8_0:
         case CML_Q4_0:
-            hipLaunchKernelGGL(dequant_q8q4_kernel, dim3(grid), dim3(256), 0, st, w->fmt, w->planes, w->nb, n_values, out);
+            hipLaunchKernelGGL(dequant_q8q4_kernel, dim3(grid), dim3(256), 0, st, w->fmt, w->planes, w->nb, n_values, rm, out);
             break;
         case CML_Q4_K:
-            hipLaunchKernelGGL(dequant_q4k_kernel, dim3(grid), dim3(256), 0, st, w->planes.p[0], w->planes.row_stride[0], w->nb, n_values, w->row_skip, out);
+            hipLaunchKernelGGL(dequant_q4k_kernel, dim3(grid), dim3(256), 0, st, w->planes.p[0], w->planes.row_stride[0], w->nb, n_values, w->row_skip, rm, out);
             break;
         case CML_Q6_K:
-            hipLaunchKernelGGL(dequant_q6k_kernel, dim3(grid), dim3(256), 0, st, w->planes, w->nb, n_values, out);
+            hipLaunchKernelGGL(dequant_q6k_kernel, dim3(grid), dim3(256), 0, st, w->planes, w->nb, n_values, rm, out);
             break;
         default:
             return fail(CML_ERR_INVALID, "unknown format %d", w->fmt);
     }
+    CML_HIP_TRY(hipGetLastError());
+    return CML_OK;
+}
+
+int launch_dequantize(const cml_weight *w, float *out, hipStream_t st) { return dequantize_rows(w, nullptr, w->rows, out, st); }
+
+int launch_embed_gather(const cml_weight *table, const uint32_t *token_ids, int64_t n_tokens, float *out, hipStream_t st) {
+    return dequantize_rows(table, token_ids, n_tokens, out, st);
+}
+
+// Greedy argmax of each row: strict >, the first index wins ties, starting from (-3.4e38, index 0)
+// like the reference's scan (argmax_f32, src/cuda_resident.rs:6391-6417) -- values that are not
+// greater than -3.4e38 (and NaNs) never win.  One workgroup of 1024 threads per row.
+__global__ __launch_bounds__(1024) void argmax_f32_kernel(const float *__restrict__ logits, int64_t n, uint32_t *__restrict__ out_idx) {
+    __shared__ float sval[16];
+    __shared__ int sidx[16];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const float *row = logits + static_cast<int64_t>(blockIdx.x) * n;
+    float best = -3.4e38f;
+    int besti = 0;
+    // every thread scans ascending indices, so within a thread the first maximum is kept
+    for (int64_t i = tid; i < n; i += 1024) {
+        const float v = row[i];
+        if (v > best) {
+            best = v;
+            besti = static_cast<int>(i);
+        }
+    }
+    // pairs meet keeping the greater value, the lower index on equal values
+    auto meet = [](float &bv, int &bi, float ov, int oi) {
+        if (ov > bv || (ov == bv && oi < bi)) {
+            bv = ov;
+            bi = oi;
+        }
+    };
+    for (int m = 1; m < 64; m <<= 1) meet(best, besti, __shfl_xor(best, m), __shfl_xor(besti, m));
+    if (lane == 0) {
+        sval[wave] = best;
+        sidx[wave] = besti;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        for (int k = 1; k < 16; k++) meet(best, besti, sval[k], sidx[k]);
+        out_idx[blockIdx.x] = static_cast<uint32_t>(besti);
+    }
+}
+
+int launch_argmax_f32(const float *logits, int64_t n_rows, int64_t n, uint32_t *out_idx, hipStream_t st) {
+    if (n_rows == 0) return CML_OK;
+    hipLaunchKernelGGL(argmax_f32_kernel, dim3(static_cast<unsigned>(n_rows)), dim3(1024), 0, st, logits, n, out_idx);
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }

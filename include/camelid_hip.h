@@ -177,6 +177,20 @@ int cml_silu_mul_quantize(int act, const float *gate_dev, const float *up_dev, i
 /* out_dev: f32[rows*cols], bit-identical to the reference decoders. */
 int cml_dequantize(const cml_weight *w, float *out_dev, cml_stream_t stream);
 
+/* ---- either side of the largest matvec (the output projection) ------------- */
+/* Dequantizes rows token_ids[0..n_tokens) of an embedding table into
+ * out_dev f32[n_tokens*cols]; the ids are read on the device, e.g. straight
+ * from cml_argmax_f32 (reference embed_gather_q4k / _q6k / _q8_0,
+ * src/cuda_resident.rs:8248-8383: element for element the block decode of
+ * cml_dequantize).  An id outside the table yields a row of NaNs. */
+int cml_embed_gather(const cml_weight *table, const uint32_t *token_ids_dev, int64_t n_tokens,
+                     float *out_dev, cml_stream_t stream);
+/* Greedy pick per row of logits_dev f32[n_rows*n]: strict >, the first index
+ * wins ties, scanning from (-3.4e38, index 0) (reference argmax_f32,
+ * src/cuda_resident.rs:6391-6417).  out_idx_dev u32[n_rows]. */
+int cml_argmax_f32(const float *logits_dev, int64_t n_rows, int64_t n, uint32_t *out_idx_dev,
+                   cml_stream_t stream);
+
 /* ---- matvec / small-batch matmul (reference dispatch_gemv,
  *      src/cuda_resident.rs:11370; dispatch_gemm_batched, :11550; CPU
  *      semantics WireQuant::matvec_q / matvec_q8k / matmul_q / matmul_q8k,

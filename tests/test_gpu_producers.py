@@ -113,3 +113,73 @@ def test_producer_error_paths():
     assert L.cml_rms_norm_quantize(ACT_F32, d.ptr, d.ptr, 1e-6, 1, 32768, d.ptr, None, None, None) == 6   # row too long to stage
     assert L.cml_silu_mul_quantize(ACT_F32, d.ptr, d.ptr, 1, 256, d.ptr, d.ptr, None) == 2
     assert L.cml_rms_norm_quantize(ACT_F32, d.ptr, d.ptr, 1e-6, 0, 256, d.ptr, None, None, None) == 0
+
+
+# ------------------------------------------------- either side of the LM head ----
+
+@pytest.mark.parametrize("name,fmt", [("Q8_0", oracle.Q8_0), ("Q4_0", oracle.Q4_0), ("Q4_K", oracle.Q4_K), ("Q6_K", oracle.Q6_K)])
+def test_embed_gather_rows_are_the_block_decode(name, fmt):
+    rows, cols = 77, 1024
+    wire = G.synth_weight(fmt, rows, cols, seed=1200 + fmt)
+    w = B.Weight.upload(fmt, rows, cols, wire)
+    ref = oracle.dequant(fmt, wire).reshape(rows, cols)
+    ids = np.array([0, 76, 5, 5, 33, 16, 15, 1000, 17], np.uint32)   # 1000 is outside the table
+    G.say(f"embed_gather {name}")
+    idd = DeviceBuffer.from_numpy(ids)
+    out = DeviceBuffer(ids.size * cols * 4)
+    out.fill(0)
+    check(lib().cml_embed_gather(w.handle, idd.ptr, ids.size, out.ptr, None), "cml_embed_gather")
+    check(lib().cml_stream_sync(None))
+    got = out.to_numpy(np.float32, (ids.size, cols))
+    for k, t in enumerate(ids):
+        if t < rows:
+            assert G.same_bits(got[k], ref[t]), (k, t)
+        else:
+            assert np.all(np.isnan(got[k]))
+    # a band view gathers relative to the band
+    band = w.slice(21, 40)
+    check(lib().cml_embed_gather(band.handle, idd.ptr, 3, out.ptr, None), "cml_embed_gather")
+    check(lib().cml_stream_sync(None))
+    got = out.to_numpy(np.float32, (ids.size, cols))
+    assert G.same_bits(got[0], ref[21]) and np.all(np.isnan(got[1])) and G.same_bits(got[2], ref[26])
+
+
+def test_argmax_first_maximum_wins():
+    rng = np.random.default_rng(1300)
+    for n in (1, 63, 1024, 1025, 128256):
+        logits = rng.standard_normal((6, n)).astype(np.float32)
+        if n > 3:
+            logits[1, n // 2] = logits[1, 1] = 9.0          # equal maxima: the lower index
+            logits[2, :] = -np.inf                          # nothing beats the starting value: index 0
+            logits[3, 0] = np.nan
+            logits[3, n - 1] = 50.0
+            logits[4, :] = 2.5                              # all equal
+            logits[5, n - 1] = 100.0                        # the very last element
+        G.say(f"argmax n={n}")
+        ld = DeviceBuffer.from_numpy(logits)
+        od = DeviceBuffer(6 * 4)
+        check(lib().cml_argmax_f32(ld.ptr, 6, n, od.ptr, None), "cml_argmax_f32")
+        check(lib().cml_stream_sync(None))
+        got = od.to_numpy(np.uint32, (6,))
+        for r in range(6):
+            best, besti = np.float32(-3.4e38), 0            # the reference's scan, spelled out
+            for i, v in enumerate(logits[r]) if n <= 2048 else ():
+                if v > best:
+                    best, besti = v, i
+            if n > 2048:
+                row = np.where(np.isnan(logits[r]), -np.inf, logits[r])
+                besti = int(np.argmax(row)) if row.max() > -3.4e38 else 0
+            assert got[r] == besti, (n, r, got[r], besti)
+    # argmax feeds embed_gather without leaving the device
+    rows, cols = 300, 512
+    wire = G.synth_weight(oracle.Q6_K, rows, cols, seed=1301)
+    w = B.Weight.upload(oracle.Q6_K, rows, cols, wire)
+    logits = rng.standard_normal((2, rows)).astype(np.float32)
+    ld, od, out = DeviceBuffer.from_numpy(logits), DeviceBuffer(8), DeviceBuffer(2 * cols * 4)
+    check(lib().cml_argmax_f32(ld.ptr, 2, rows, od.ptr, None), "cml_argmax_f32")
+    check(lib().cml_embed_gather(w.handle, od.ptr, 2, out.ptr, None), "cml_embed_gather")
+    check(lib().cml_stream_sync(None))
+    ref = oracle.dequant(oracle.Q6_K, wire).reshape(rows, cols)
+    got = out.to_numpy(np.float32, (2, cols))
+    for r in range(2):
+        assert G.same_bits(got[r], ref[int(np.argmax(logits[r]))])
