@@ -192,9 +192,10 @@ def bench_moe(name: str, K: int, W: int, seed: int, cpu_seconds: float) -> int:
         "config": {"workload": name, "format": "Q4_K", "experts": E, "top_k": k, "hidden": hidden, "ff": ff, "tokens": T,
                    "algorithmic_bytes_per_call": int(alg_bytes), "mean_experts_touched": float(np.mean(touched)),
                    "step": "route + gate/up matvecs + silu*up->Q8_K + down matvec + weighted sum, graph replay",
-                   "launches_per_step": 7},
-        # the step is seven launches; the three expert matvec launches carry the bytes
-        "roofline": {"bound": "hbm", "kernel": "gemv_q4k_kernel grouped by expert (3 launches of the step)",
+                   # route, plan, [quantize,] gate, up (one launch at 1 token), silu*up->Q8_K, down, weighted sum
+                   "launches_per_step": 6 if T == 1 else 8},
+        # the expert matvec launches carry the bytes; the figure is for the whole step
+        "roofline": {"bound": "hbm", "kernel": "gemv_q4k_kernel / gemm_q4k_mfma_kernel grouped by expert (2-3 launches of the step)",
                      "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
                      "traffic": None, "us_per_launch": round(ms * 1e3, 3), "note": "whole step, all launches"},
     }

@@ -68,6 +68,10 @@ struct Q4KArgs {
     // serves its assignments in passes of NT.
     const int32_t *group_offsets;
     const int32_t *group_rows;
+    // Pair launch (gridDim.z == 2): blockIdx.z = 1 works on a second weight of the same shape
+    // against the same activations and writes out2 (gate and up projections in one launch).
+    const uint8_t *w2;
+    float *out2;
     int ksplit;        // waves sharing one row tile (1, 2, 4 or 8)
     int tiles_per_wg;  // row tiles per workgroup; blockDim.x = 64 * ksplit * tiles_per_wg
 };
@@ -206,7 +210,8 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
     const int a0 = grouped ? a.group_offsets[band] : 0;               // first assignment of this group
     const int n_assign = grouped ? a.group_offsets[band + 1] - a0 : NT;
     if (n_assign <= 0) return;  // an expert nobody routed to: the whole workgroup leaves
-    const uint8_t *w = a.w + band * (a.rows / 16) * kQ4KChunk;
+    const bool second = gridDim.z > 1 && blockIdx.z == 1;
+    const uint8_t *w = (second ? a.w2 : a.w) + band * (a.rows / 16) * kQ4KChunk;
 
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int W = a.ksplit;
@@ -242,7 +247,7 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
             // takes super-blocks 4*(w + p*waves) ..+3), lane l of a row holding values 16l..16l+15.
             const int nw = nthreads >> 6;
             const int qrow = lane >> 4, ql = lane & 15;
-            const float4 *x4 = reinterpret_cast<const float4 *>(a.x);
+            const float4 *x4 = reinterpret_cast<const float4 *>(a.x + act_row(0) * n_sb * 256);
             auto load_pass = [&](float4 (&xv)[4], int base) {
                 const int sbk = min(base + qrow, n_sb - 1);
 #pragma unroll
@@ -361,7 +366,7 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
             sb += U;
         }
 
-        float *out = a.out + static_cast<int64_t>(a0 + p0) * a.rows;  // output row of local token 0
+        float *out = (second ? a.out2 : a.out) + static_cast<int64_t>(a0 + p0) * a.rows;  // output row of local token 0
         const int n_here = min(NT, n_assign - p0);
         if (W == 1) {
             if (leader && live) {
@@ -463,19 +468,35 @@ static int launch_q4k_pick_nt(const Q4KArgs &ka, const Q4KShape &shape, int n_gr
     }
 }
 
-// Single token, f32 activation in: quantize + matvec in one launch.  The K-split
-// is the matvec's own (same association); waves of a workgroup share the
-// quantizing, so a workgroup holds 4 waves where the split alone gives fewer.
-int launch_gemv_q4k_f32(const cml_weight *w, const float *x, float *out, hipStream_t st) {
+// Single token per group, f32 activation in: quantize + matvec in one launch.  The K-split is
+// the matvec's own (same association); waves of a workgroup share the quantizing, so a workgroup
+// holds 4 waves where the split alone gives fewer.  Plain call: `a.w` against activation row 0.
+// Grouped call (group_offsets set): every group dots its assignments' activation rows
+// (group_rows) one at a time.  `w2`/`out2` non-null: a second weight of the same shape in the
+// same launch (grid.z = 2).
+static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, const float *x, hipStream_t st) {
+    const cml_weight *w = a.w;
+    const bool grouped = a.group_offsets != nullptr;
     if (w->rows == 0) return CML_OK;
     Q4KArgs ka{};
     ka.w = w->planes.p[0];
     ka.sb_stride = w->planes.row_stride[0];
-    ka.rows = static_cast<int>(w->rows);
-    ka.row_skip = w->row_skip;
+    ka.rows = static_cast<int>(grouped ? a.band_rows : w->rows);
+    if (grouped && ((ka.rows % 16) != 0 || w->row_skip != 0))
+        return fail(CML_ERR_UNSUPPORTED, "Q4_K expert bands must be whole 16-row tiles (%d rows, first tile offset %d)", ka.rows, w->row_skip);
+    ka.row_skip = grouped ? 0 : w->row_skip;
     ka.n_sb = static_cast<int>(w->nb);
     ka.x = x;
-    ka.out = out;
+    ka.out = a.out;
+    ka.group_offsets = a.group_offsets;
+    ka.group_rows = a.group_rows;
+    if (w2) {
+        if (w2->fmt != w->fmt || w2->rows != w->rows || w2->nb != w->nb || w2->row_skip != w->row_skip ||
+            w2->planes.row_stride[0] != w->planes.row_stride[0])
+            return fail(CML_ERR_SHAPE, "the two weights of a pair launch differ in shape");
+        ka.w2 = w2->planes.p[0];
+        ka.out2 = out2;
+    }
     Q4KShape shape = pick_shape(ka.rows, ka.n_sb);
     int tpw = env_int("CAMELID_HIP_Q4K_FUSED_TILES_PER_WG", 0);
     if (tpw < 1 || tpw * shape.ksplit > 8) tpw = std::max(1, 4 / shape.ksplit);
@@ -488,9 +509,24 @@ int launch_gemv_q4k_f32(const cml_weight *w, const float *x, float *out, hipStre
     if (lds > 64 * 1024) return fail(CML_ERR_UNSUPPORTED, "Q4_K activation of %d super-blocks exceeds the LDS staging limit", ka.n_sb);
     ka.ksplit = shape.ksplit;
     ka.tiles_per_wg = shape.tiles_per_wg;
-    hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true>), dim3(gx, 1), dim3(64 * waves), lds, st, ka);
+    const dim3 grid(gx, grouped ? a.n_groups : 1, w2 ? 2 : 1);
+    hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true>), grid, dim3(64 * waves), lds, st, ka);
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
+}
+
+int launch_gemv_q4k_f32(const cml_weight *w, const float *x, float *out, hipStream_t st) {
+    MatArgs a{};
+    a.w = w;
+    a.out = out;
+    a.n_tokens = 1;
+    a.n_groups = 1;
+    return launch_q4k_f32(a, nullptr, nullptr, x, st);
+}
+
+// Expert-grouped pair (gate and up of a mixture-of-experts layer), one assignment at a time.
+int launch_gemv_q4k_f32_grouped_pair(const MatArgs &a, const cml_weight *w2, float *out2, const float *x, hipStream_t st) {
+    return launch_q4k_f32(a, w2, out2, x, st);
 }
 
 int launch_gemv_q4k(const MatArgs &a, hipStream_t st) {

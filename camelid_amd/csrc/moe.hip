@@ -223,7 +223,12 @@ int cml_moe_ffn(const cml_weight *gate, const cml_weight *up, const cml_weight *
     hipStream_t st = as_stream(stream);
     const int n_slots = static_cast<int>(n_tokens * k);
 
-    if (int rc = launch_quantize_q8_k(x_dev, n_tokens, hidden, ws.xq, ws.xd, st)) return rc;
+    // Decode (one token, rows of up to 4096 values): gate and up run as ONE launch that quantizes
+    // the token inside every workgroup -- two launches and the quantized round trip fewer.
+    const bool fused_decode = n_tokens == 1 && hidden / 256 <= 16 && env_int("CAMELID_HIP_FUSED_QUANT", 1) != 0;
+    if (!fused_decode) {
+        if (int rc = launch_quantize_q8_k(x_dev, n_tokens, hidden, ws.xq, ws.xd, st)) return rc;
+    }
     hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(64), 0, st, idx_dev, n_slots, n_experts, k, ws.offsets, ws.assign_token, ws.slot_to_assign);
     CML_HIP_TRY(hipGetLastError());
 
@@ -240,10 +245,14 @@ int cml_moe_ffn(const cml_weight *gate, const cml_weight *up, const cml_weight *
     a.band_rows = ff;
     a.w = gate;
     a.out = ws.g;
-    if (int rc = launch_expert_matmul(a, st)) return rc;
-    a.w = up;
-    a.out = ws.u;
-    if (int rc = launch_expert_matmul(a, st)) return rc;
+    if (fused_decode) {
+        if (int rc = launch_gemv_q4k_f32_grouped_pair(a, up, ws.u, x_dev, st)) return rc;
+    } else {
+        if (int rc = launch_expert_matmul(a, st)) return rc;
+        a.w = up;
+        a.out = ws.u;
+        if (int rc = launch_expert_matmul(a, st)) return rc;
+    }
     // h = silu(g) * u, quantized per assignment
     if (int rc = launch_silu_mul_quantize(2, ws.g, ws.u, n_slots, ff, ws.hq, ws.hd, st)) return rc;
     // down: assignment j reads its own h
