@@ -360,9 +360,11 @@ def main() -> int:
     quant = L.cml_quantize_q8_k if per == 256 else L.cml_quantize_q8_0
     check(quant(xd.ptr, n, cols, qd.ptr, sd.ptr, stream))
 
-    # Q4_K decode at hidden sizes up to 4096 runs quantize + matvec as ONE kernel: there the step
-    # itself is the dominant kernel's launch.  Elsewhere it is the matvec on quantized activations.
-    fused = fmt_name == "Q4_K" and n == 1 and cols <= 4096 and os.environ.get("CAMELID_HIP_FUSED_QUANT", "1") != "0"
+    # Decode at the usual hidden sizes runs quantize + matvec as ONE kernel (Q4_K up to 4096 values
+    # per row, Q8_0 / Q4_0 up to 8192 values and 32768 rows): there the step itself is the dominant kernel's launch.
+    # Elsewhere it is the matvec on quantized activations.
+    fused = n == 1 and os.environ.get("CAMELID_HIP_FUSED_QUANT", "1") != "0" and (
+        (fmt_name == "Q4_K" and cols <= 4096) or (fmt_name in ("Q8_0", "Q4_0") and cols <= 8192 and rows <= 32768))
 
     def gemv_cold(i):
         if fused:
@@ -408,7 +410,7 @@ def main() -> int:
                    "launches_per_step": 1 if fused else 2,
                    "eager_python_us_per_call": None if eager_us is None else round(eager_us, 3)},
         "roofline": {"bound": "hbm",
-                     "kernel": "gemv_q4k_kernel<1,false,true> (cml_matmul_f32: activation quantizer fused into the matvec)" if fused
+                     "kernel": f"gemv_{fmt_name.lower()} with the activation quantizer fused in (cml_matmul_f32, one launch)" if fused
                      else f"gemv_{fmt_name.lower()} (cml_gemm on quantized activations)",
                      "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.config),

@@ -103,6 +103,7 @@ int launch_gemv_q4k(const MatArgs &a, hipStream_t st);
 int launch_gemv_q4k_f32_grouped_pair(const MatArgs &a, const cml_weight *w2, float *out2, const float *x, hipStream_t st);
 
 int launch_gemv_q4k_f32(const cml_weight *w, const float *x, float *out, hipStream_t st);  // quantize + matvec, one token
+int launch_gemv_b32_f32(const cml_weight *w, const float *x, float *out, hipStream_t st);  // Q8_0 / Q4_0: quantize + matvec, one token
 int launch_gemv_q8_0(const MatArgs &a, hipStream_t st);
 int launch_gemv_q4_0(const MatArgs &a, hipStream_t st);
 int launch_gemv_q6k(const MatArgs &a, hipStream_t st);

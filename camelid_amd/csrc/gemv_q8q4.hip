@@ -32,6 +32,7 @@ struct B32Args {
     int nb;    // blocks per row
     const int8_t *q;  // [slot][NT][nb*32]
     const float *xs;  // [slot][NT][nb]
+    const float *x;   // f32 activation row [nb*32]: only for the kernel that quantizes it itself
     float *out;
     const float *residual;
     int32_t *ints;  // [rows][nb] or null
@@ -105,8 +106,12 @@ __device__ __forceinline__ void b32_compute(const B32Regs<FMT> &r, int l, int st
     }
 }
 
-template <int FMT, int P, int NT, bool INTS>
+// FUSEQ (single token): the activation arrives as f32 and every workgroup quantizes it to Q8_0
+// itself, eight lanes per block, straight into the LDS staging area -- the arithmetic of
+// quantize_q8_0_kernel without the launch and the round trip through memory.
+template <int FMT, int P, int NT, bool INTS, bool FUSEQ = false>
 __global__ __launch_bounds__(256) void gemv_b32_kernel(B32Args a) {
+    static_assert(!FUSEQ || (NT == 1 && !INTS), "the fused quantizer serves single-token calls");
     constexpr int RPW = kWave / P;
     extern __shared__ uint4 smem[];
     const int nb = a.nb;
@@ -121,7 +126,21 @@ __global__ __launch_bounds__(256) void gemv_b32_kernel(B32Args a) {
     const float *xs = a.xs + static_cast<int64_t>(slot) * a.act_slot_stride * nb;
     float *out = a.out + static_cast<int64_t>(slot) * a.out_slot_stride;
 
-    {
+    if constexpr (FUSEQ) {
+        const float4 *x4 = reinterpret_cast<const float4 *>(a.x);
+        uint32_t *ys32 = reinterpret_cast<uint32_t *>(ys);
+        const int n4 = nb * 8;  // a multiple of 8: the eight lanes of a block enter and leave together
+        for (int i = tid; i < n4; i += 256) {
+            float scale;
+            const uint32_t packed = q8_0_quantize_lane8(x4[i], scale);
+            ys32[i] = packed;
+            if ((i & 7) == 0) xss[i >> 3] = scale;
+            if constexpr (FMT == CML_Q4_0) {
+                const int s = group_sum_to_last<8>(sdot4(packed, 0x01010101u, 0));
+                if ((i & 7) == 7) bsum[i >> 3] = s;
+            }
+        }
+    } else {
         const uint4 *src = reinterpret_cast<const uint4 *>(q);
         uint4 *dst = reinterpret_cast<uint4 *>(ys);
         const int n16 = NT * nb * 2;  // even: lanes 2k, 2k+1 are in or out together
@@ -241,6 +260,36 @@ static int launch_b32_p(const MatArgs &a, hipStream_t st) {
         t0 += nt;
     }
     return CML_OK;
+}
+
+// Single token, f32 activation in: quantize + matvec in one launch.
+template <int FMT, int P>
+static int launch_b32_f32_p(const cml_weight *w, const float *x, float *out, hipStream_t st) {
+    B32Args ba{};
+    ba.quants = w->planes.p[0];
+    ba.q_stride = w->planes.row_stride[0];
+    ba.scales = w->planes.p[1];
+    ba.s_stride = w->planes.row_stride[1];
+    ba.rows = static_cast<int>(w->rows);
+    ba.nb = static_cast<int>(w->nb);
+    ba.x = x;
+    ba.out = out;
+    const int rows_per_wg = 4 * (64 / P);
+    const unsigned gx = static_cast<unsigned>((ba.rows + rows_per_wg - 1) / rows_per_wg);
+    const size_t lds = static_cast<size_t>(ba.nb) * (32 + 4 + 4);
+    if (lds > 64 * 1024) return fail(CML_ERR_UNSUPPORTED, "activation of %d blocks exceeds the LDS staging limit", ba.nb);
+    hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, true>), dim3(gx, 1), dim3(256), lds, st, ba);
+    CML_HIP_TRY(hipGetLastError());
+    return CML_OK;
+}
+
+int launch_gemv_b32_f32(const cml_weight *w, const float *x, float *out, hipStream_t st) {
+    if (w->rows == 0) return CML_OK;
+    const bool q8 = w->fmt == CML_Q8_0;
+    int p = env_int(q8 ? "CAMELID_HIP_Q8_0_LANES" : "CAMELID_HIP_Q4_0_LANES", 0);
+    if (p != 8 && p != 16) p = (w->nb <= 8) ? 8 : 16;
+    if (q8) return p == 8 ? launch_b32_f32_p<CML_Q8_0, 8>(w, x, out, st) : launch_b32_f32_p<CML_Q8_0, 16>(w, x, out, st);
+    return p == 8 ? launch_b32_f32_p<CML_Q4_0, 8>(w, x, out, st) : launch_b32_f32_p<CML_Q4_0, 16>(w, x, out, st);
 }
 
 template <int FMT>

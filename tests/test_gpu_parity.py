@@ -299,6 +299,35 @@ def test_q4k_fused_quantize_matvec_is_the_two_step_path(rows, cols):
             assert G.same_bits(got, want)
 
 
+@pytest.mark.parametrize("name,fmt", [("Q8_0", oracle.Q8_0), ("Q4_0", oracle.Q4_0)])
+@pytest.mark.parametrize("rows,cols", [(190, 2048), (33, 32), (70, 3072 + 32), (16, 14336)])
+def test_b32_fused_quantize_matvec_is_the_two_step_path(name, fmt, rows, cols):
+    """Single-token cml_matmul_f32 on Q8_0 / Q4_0 weights quantizes inside the matvec kernel: same
+    bits as quantize_q8_0 followed by the matvec, on activations with zero blocks, exact .5 ties
+    (rounded away from zero) and NaNs, for both lane mappings."""
+    rng = np.random.default_rng(7300 + rows + fmt)
+    wire = G.synth_weight(fmt, rows, cols, seed=7400 + rows + fmt)
+    w = Weight.upload(fmt, rows, cols, wire)
+    acts = _activation_cases(cols, rng)
+    acts[0, :32] = 0.0
+    acts[0, 0] = 127.0
+    acts[0, 1:7] = [2.5, 0.5, -0.5, -2.5, 1.5, -1.5]
+    acts[1, 3] = np.nan
+    lanes_env = "CAMELID_HIP_Q8_0_LANES" if fmt == oracle.Q8_0 else "CAMELID_HIP_Q4_0_LANES"
+    for i, x in enumerate(acts):
+        for lanes in (0, 8, 16):
+            G.say(f"{name} fused quantize+matvec {rows}x{cols} act={i} lanes={lanes}")
+            with G.env(**{lanes_env: lanes}):
+                with G.env(CAMELID_HIP_FUSED_QUANT=2):
+                    fused = G.gpu_matmul_f32(w, x)
+                with G.env(CAMELID_HIP_FUSED_QUANT=0):
+                    two_step = G.gpu_matmul_f32(w, x)
+            assert G.same_bits(fused, two_step)
+        if i != 1:
+            want = oracle.matmul(fmt, wire, cols, x[None, :], order=EXACT_ORDER[fmt], threads=8)[0]
+            assert G.same_bits(fused, want)
+
+
 # ----------------------------------------------------- errors and the seam ----
 
 def test_error_paths_return_status_codes():
