@@ -441,7 +441,13 @@ int cml_rms_norm_quantize(int act, const float *x_dev, const float *weight_dev, 
 
 int cml_silu_mul_quantize(int act, const float *gate_dev, const float *up_dev, int64_t n_tokens, int64_t cols, int8_t *q_dev,
                           float *scales_dev, cml_stream_t stream) {
+    return cml_glu_quantize(CML_GLU_SILU, act, gate_dev, up_dev, n_tokens, cols, q_dev, scales_dev, stream);
+}
+
+int cml_glu_quantize(int glu, int act, const float *gate_dev, const float *up_dev, int64_t n_tokens, int64_t cols, int8_t *q_dev,
+                     float *scales_dev, cml_stream_t stream) {
     if (int rc = check_ready()) return rc;
+    if (glu != CML_GLU_SILU && glu != CML_GLU_GELU_TANH) return fail(CML_ERR_INVALID, "unknown activation %d", glu);
     if (act != CML_ACT_Q8_0 && act != CML_ACT_Q8_K) return fail(CML_ERR_INVALID, "activation format %d is not a quantized one", act);
     const int64_t unit = act == CML_ACT_Q8_K ? 256 : 32;
     if (n_tokens < 0 || cols < 0 || cols % unit != 0) return fail(CML_ERR_SHAPE, "cols %lld is not a multiple of %lld", (long long)cols, (long long)unit);
@@ -449,7 +455,7 @@ int cml_silu_mul_quantize(int act, const float *gate_dev, const float *up_dev, i
     if (!gate_dev || !up_dev || !q_dev || !scales_dev) return fail(CML_ERR_INVALID, "null pointer");
     if (misaligned16(gate_dev) || misaligned16(up_dev) || (reinterpret_cast<uintptr_t>(q_dev) & 3u))
         return fail(CML_ERR_INVALID, "gate and up must be 16-byte and q 4-byte aligned");
-    return launch_silu_mul_quantize(act, gate_dev, up_dev, n_tokens, cols, q_dev, scales_dev, as_stream(stream));
+    return launch_glu_quantize(glu, act, gate_dev, up_dev, n_tokens, cols, cols, q_dev, scales_dev, as_stream(stream));
 }
 
 int cml_dequantize(const cml_weight *w, float *out_dev, cml_stream_t stream) {

@@ -68,6 +68,8 @@ int launch_quantize_q8_k(const float *x, int64_t n_tokens, int64_t cols, int8_t 
 // producers.hip: act = 0 (f32 only), 1 (Q8_0), 2 (Q8_K)
 int launch_rms_norm_quantize(int act, const float *x, const float *weight, float eps, int64_t n_tokens, int64_t cols,
                              float *normed, int8_t *q, float *scales, hipStream_t st);
+int launch_glu_quantize(int glu, int act, const float *g, const float *u, int64_t n_tokens, int64_t cols, int64_t in_stride,
+                        int8_t *q, float *scales, hipStream_t st);  // glu: 0 = silu, 1 = gelu_tanh
 int launch_silu_mul_quantize(int act, const float *g, const float *u, int64_t n_tokens, int64_t cols, int8_t *q, float *scales,
                              hipStream_t st);
 
@@ -104,6 +106,8 @@ int launch_gemv_q4k_f32_grouped_pair(const MatArgs &a, const cml_weight *w2, flo
 
 int launch_gemv_q4k_f32(const cml_weight *w, const float *x, float *out, hipStream_t st);  // quantize + matvec, one token
 int launch_gemv_b32_f32(const cml_weight *w, const float *x, float *out, hipStream_t st);  // Q8_0 / Q4_0: quantize + matvec, one token
+// Q8_0 / Q4_0 grouped (mixture-of-experts) matvec; x non-null = one f32 token quantized in the kernel
+int launch_gemv_b32_grouped(const MatArgs &a, const float *x, hipStream_t st);
 int launch_gemv_q8_0(const MatArgs &a, hipStream_t st);
 int launch_gemv_q4_0(const MatArgs &a, hipStream_t st);
 int launch_gemv_q6k(const MatArgs &a, hipStream_t st);

@@ -19,6 +19,8 @@
 #include "cml_device.hpp"
 #include "cml_host.hpp"
 
+#include <type_traits>
+
 #pragma clang fp contract(off)
 
 namespace cml {
@@ -106,6 +108,57 @@ __device__ __forceinline__ void b32_compute(const B32Regs<FMT> &r, int l, int st
     }
 }
 
+// One pass over a row's blocks for NT staged activation rows: two register buffers alternate,
+// the last one is consumed without issuing further loads.
+template <int FMT, int P, int NT, bool INTS>
+__device__ __forceinline__ void b32_row_pass(const uint8_t *qrow, const uint8_t *srow, int l, int nb, const int8_t *ys,
+                                             const int *bsum, const float *xss, float (&acc)[NT], int32_t *ints_row) {
+    constexpr int U = B32Regs<FMT>::U;
+    const int n_steps = (nb + P - 1) / P;
+    B32Regs<FMT> ra, rb;
+    b32_load<FMT, P>(ra, qrow, srow, l, 0, n_steps, nb);
+    __builtin_amdgcn_sched_barrier(0);
+    for (int step = 0;;) {
+        if (step + U >= n_steps) {
+            b32_compute<FMT, P, NT, INTS>(ra, l, step, n_steps, nb, ys, bsum, xss, acc, ints_row);
+            break;
+        }
+        b32_load<FMT, P>(rb, qrow, srow, l, step + U, n_steps, nb);
+        __builtin_amdgcn_sched_barrier(0);
+        b32_compute<FMT, P, NT, INTS>(ra, l, step, n_steps, nb, ys, bsum, xss, acc, ints_row);
+        __builtin_amdgcn_sched_barrier(0);
+        step += U;
+        if (step + U >= n_steps) {
+            b32_compute<FMT, P, NT, INTS>(rb, l, step, n_steps, nb, ys, bsum, xss, acc, ints_row);
+            break;
+        }
+        b32_load<FMT, P>(ra, qrow, srow, l, step + U, n_steps, nb);
+        __builtin_amdgcn_sched_barrier(0);
+        b32_compute<FMT, P, NT, INTS>(rb, l, step, n_steps, nb, ys, bsum, xss, acc, ints_row);
+        __builtin_amdgcn_sched_barrier(0);
+        step += U;
+    }
+}
+
+// Quantize one f32 row of nb blocks to Q8_0 straight into the LDS staging area, eight lanes per
+// block: the arithmetic of quantize_q8_0_kernel without the launch and the round trip.
+template <int FMT>
+__device__ __forceinline__ void b32_stage_quantized(const float *x, int nb, int tid, int8_t *ys, float *xss, int *bsum) {
+    const float4 *x4 = reinterpret_cast<const float4 *>(x);
+    uint32_t *ys32 = reinterpret_cast<uint32_t *>(ys);
+    const int n4 = nb * 8;  // a multiple of 8: the eight lanes of a block enter and leave together
+    for (int i = tid; i < n4; i += 256) {
+        float scale;
+        const uint32_t packed = q8_0_quantize_lane8(x4[i], scale);
+        ys32[i] = packed;
+        if ((i & 7) == 0) xss[i >> 3] = scale;
+        if constexpr (FMT == CML_Q4_0) {
+            const int s = group_sum_to_last<8>(sdot4(packed, 0x01010101u, 0));
+            if ((i & 7) == 7) bsum[i >> 3] = s;
+        }
+    }
+}
+
 // FUSEQ (single token): the activation arrives as f32 and every workgroup quantizes it to Q8_0
 // itself, eight lanes per block, straight into the LDS staging area -- the arithmetic of
 // quantize_q8_0_kernel without the launch and the round trip through memory.
@@ -127,19 +180,7 @@ __global__ __launch_bounds__(256) void gemv_b32_kernel(B32Args a) {
     float *out = a.out + static_cast<int64_t>(slot) * a.out_slot_stride;
 
     if constexpr (FUSEQ) {
-        const float4 *x4 = reinterpret_cast<const float4 *>(a.x);
-        uint32_t *ys32 = reinterpret_cast<uint32_t *>(ys);
-        const int n4 = nb * 8;  // a multiple of 8: the eight lanes of a block enter and leave together
-        for (int i = tid; i < n4; i += 256) {
-            float scale;
-            const uint32_t packed = q8_0_quantize_lane8(x4[i], scale);
-            ys32[i] = packed;
-            if ((i & 7) == 0) xss[i >> 3] = scale;
-            if constexpr (FMT == CML_Q4_0) {
-                const int s = group_sum_to_last<8>(sdot4(packed, 0x01010101u, 0));
-                if ((i & 7) == 7) bsum[i >> 3] = s;
-            }
-        }
+        b32_stage_quantized<FMT>(a.x, nb, tid, ys, xss, bsum);
     } else {
         const uint4 *src = reinterpret_cast<const uint4 *>(q);
         uint4 *dst = reinterpret_cast<uint4 *>(ys);
@@ -174,33 +215,7 @@ __global__ __launch_bounds__(256) void gemv_b32_kernel(B32Args a) {
 #pragma unroll
     for (int t = 0; t < NT; t++) acc[t] = 0.0f;
 
-    constexpr int U = B32Regs<FMT>::U;
-    const int n_steps = (nb + P - 1) / P;
-    B32Regs<FMT> ra, rb;
-    b32_load<FMT, P>(ra, qrow, srow, l, 0, n_steps, nb);
-    __builtin_amdgcn_sched_barrier(0);
-    // Two register buffers alternate; the last one is consumed without issuing
-    // further loads.
-    for (int step = 0;;) {
-        if (step + U >= n_steps) {
-            b32_compute<FMT, P, NT, INTS>(ra, l, step, n_steps, nb, ys, bsum, xss, acc, ints_row);
-            break;
-        }
-        b32_load<FMT, P>(rb, qrow, srow, l, step + U, n_steps, nb);
-        __builtin_amdgcn_sched_barrier(0);
-        b32_compute<FMT, P, NT, INTS>(ra, l, step, n_steps, nb, ys, bsum, xss, acc, ints_row);
-        __builtin_amdgcn_sched_barrier(0);
-        step += U;
-        if (step + U >= n_steps) {
-            b32_compute<FMT, P, NT, INTS>(rb, l, step, n_steps, nb, ys, bsum, xss, acc, ints_row);
-            break;
-        }
-        b32_load<FMT, P>(ra, qrow, srow, l, step + U, n_steps, nb);
-        __builtin_amdgcn_sched_barrier(0);
-        b32_compute<FMT, P, NT, INTS>(rb, l, step, n_steps, nb, ys, bsum, xss, acc, ints_row);
-        __builtin_amdgcn_sched_barrier(0);
-        step += U;
-    }
+    b32_row_pass<FMT, P, NT, INTS>(qrow, srow, l, nb, ys, bsum, xss, acc, ints_row);
 
     if (leader && live) {
 #pragma unroll
@@ -292,10 +307,155 @@ int launch_gemv_b32_f32(const cml_weight *w, const float *x, float *out, hipStre
     return p == 8 ? launch_b32_f32_p<CML_Q4_0, 8>(w, x, out, st) : launch_b32_f32_p<CML_Q4_0, 16>(w, x, out, st);
 }
 
+// ---- grouped (mixture-of-experts) dispatch ------------------------------------------------------
+// blockIdx.y = group (expert) e: the band of rows [e*rows, (e+1)*rows) of the stacked weight dotted
+// with the activation rows of the assignments [group_offsets[e], group_offsets[e+1]).  The group's
+// assignments are staged NTMAX at a time; a chunk of 1, 2, 3-4 or 5-8 runs the 1-, 2-, 4- or
+// 8-token row pass (slots past the chunk repeat its last row and are not written).  Every cell is
+// the single-row chain of the plain kernel: bit-identical to it.
+// FUSEQ: one token, f32, quantized inside every workgroup; every assignment reads it.
+struct B32GroupArgs {
+    const uint8_t *quants;
+    int64_t q_stride;
+    const uint8_t *scales;
+    int64_t s_stride;
+    int rows;  // rows of one band
+    int nb;
+    const int8_t *q;  // [activation rows][nb*32]
+    const float *xs;  // [activation rows][nb]
+    const float *x;   // FUSEQ: the f32 token
+    float *out;       // [assignments][rows]
+    const int32_t *group_offsets;
+    const int32_t *group_rows;  // assignment -> activation row, or null (the assignment itself)
+};
+
+template <int FMT, int P, int NTMAX, bool FUSEQ>
+__global__ __launch_bounds__(256) void gemv_b32_grouped_kernel(B32GroupArgs a) {
+    static_assert(!FUSEQ || NTMAX == 1, "the fused quantizer serves single-token calls");
+    constexpr int RPW = kWave / P;
+    extern __shared__ uint4 smem[];
+    const int nb = a.nb;
+    int8_t *ys = reinterpret_cast<int8_t *>(smem);                 // [NTMAX][nb*32]
+    float *xss = reinterpret_cast<float *>(ys + NTMAX * nb * 32);  // [NTMAX][nb]
+    int *bsum = reinterpret_cast<int *>(xss + NTMAX * nb);         // [NTMAX][nb] (Q4_0)
+
+    const int tid = threadIdx.x;
+    const int g = blockIdx.y;
+    const int a0 = a.group_offsets[g];
+    const int cnt = a.group_offsets[g + 1] - a0;
+    if (cnt <= 0) return;  // the whole workgroup leaves together
+
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    const int r = lane / P, l = lane - r * P;
+    const int row = (blockIdx.x * 4 + wave) * RPW + r;
+    const bool live = row < a.rows;
+    const int64_t arow = static_cast<int64_t>(g) * a.rows + (live ? row : a.rows - 1);
+    const uint8_t *qrow = a.quants + arow * a.q_stride;
+    const uint8_t *srow = a.scales + arow * a.s_stride;
+    const bool leader = (l == P - 1);
+
+    for (int c0 = 0; c0 < cnt; c0 += NTMAX) {
+        const int nt = min(NTMAX, cnt - c0);
+        if constexpr (FUSEQ) {
+            if (c0 == 0) b32_stage_quantized<FMT>(a.x, nb, tid, ys, xss, bsum);
+        } else {
+            if (c0 > 0) __syncthreads();  // the previous chunk's readers are done
+            const int per_t = nb * 2;     // 16-byte pieces per activation row (even)
+            const int staged = (nt <= 1 ? 1 : nt <= 2 ? 2 : nt <= 4 ? 4 : 8);
+            uint4 *dst = reinterpret_cast<uint4 *>(ys);
+            for (int i = tid; i < staged * per_t; i += 256) {
+                const int t = i / per_t, j = i - t * per_t;
+                const int slot = a0 + c0 + min(t, nt - 1);
+                const int64_t src_row = a.group_rows ? a.group_rows[slot] : slot;
+                const uint4 v = reinterpret_cast<const uint4 *>(a.q + src_row * nb * 32)[j];
+                dst[i] = v;
+                if constexpr (FMT == CML_Q4_0) {
+                    int s = bytesum16(v);
+                    s += row_shr_i32<1>(s);
+                    if (i & 1) bsum[i >> 1] = s;
+                }
+            }
+            for (int i = tid; i < staged * nb; i += 256) {
+                const int t = i / nb, j = i - t * nb;
+                const int slot = a0 + c0 + min(t, nt - 1);
+                const int64_t src_row = a.group_rows ? a.group_rows[slot] : slot;
+                xss[i] = a.xs[src_row * nb + j];
+            }
+        }
+        __syncthreads();
+        float *out = a.out + static_cast<int64_t>(a0 + c0) * a.rows + row;
+        auto run = [&](auto nt_tag) {
+            constexpr int NT = decltype(nt_tag)::value;
+            float acc[NT];
+#pragma unroll
+            for (int t = 0; t < NT; t++) acc[t] = 0.0f;
+            b32_row_pass<FMT, P, NT, false>(qrow, srow, l, nb, ys, bsum, xss, acc, nullptr);
+            if (leader && live) {
+#pragma unroll
+                for (int t = 0; t < NT; t++)
+                    if (t < nt) out[static_cast<int64_t>(t) * a.rows] = acc[t];
+            }
+        };
+        if constexpr (NTMAX == 1) {
+            run(std::integral_constant<int, 1>{});
+        } else {
+            if (nt <= 1) run(std::integral_constant<int, 1>{});
+            else if (nt <= 2) run(std::integral_constant<int, 2>{});
+            else if (nt <= 4) run(std::integral_constant<int, 4>{});
+            else run(std::integral_constant<int, 8>{});
+        }
+    }
+}
+
+template <int FMT, int P>
+static int launch_b32_grouped_p(const MatArgs &a, const float *x, hipStream_t st) {
+    const cml_weight *w = a.w;
+    B32GroupArgs ga{};
+    ga.quants = w->planes.p[0];
+    ga.q_stride = w->planes.row_stride[0];
+    ga.scales = w->planes.p[1];
+    ga.s_stride = w->planes.row_stride[1];
+    ga.rows = static_cast<int>(a.band_rows);
+    ga.nb = static_cast<int>(w->nb);
+    ga.q = a.q;
+    ga.xs = a.scales;
+    ga.x = x;
+    ga.out = a.out;
+    ga.group_offsets = a.group_offsets;
+    ga.group_rows = a.group_rows;
+    const int rows_per_wg = 4 * (64 / P);
+    const dim3 grid(static_cast<unsigned>((ga.rows + rows_per_wg - 1) / rows_per_wg), static_cast<unsigned>(a.n_groups));
+    const bool one = x != nullptr || a.n_tokens <= 1;
+    const size_t lds = static_cast<size_t>(one ? 1 : 8) * ga.nb * (32 + 4 + 4);
+    if (lds > 64 * 1024) return fail(CML_ERR_UNSUPPORTED, "activation of %d blocks exceeds the LDS staging limit", ga.nb);
+    if (x)
+        hipLaunchKernelGGL((gemv_b32_grouped_kernel<FMT, P, 1, true>), grid, dim3(256), lds, st, ga);
+    else if (one)
+        hipLaunchKernelGGL((gemv_b32_grouped_kernel<FMT, P, 1, false>), grid, dim3(256), lds, st, ga);
+    else
+        hipLaunchKernelGGL((gemv_b32_grouped_kernel<FMT, P, 8, false>), grid, dim3(256), lds, st, ga);
+    CML_HIP_TRY(hipGetLastError());
+    return CML_OK;
+}
+
+// x non-null: one f32 token that every assignment reads, quantized inside the kernel (a.q and
+// a.scales unused).
+int launch_gemv_b32_grouped(const MatArgs &a, const float *x, hipStream_t st) {
+    const cml_weight *w = a.w;
+    if (a.band_rows <= 0 || a.n_groups <= 0 || a.n_tokens <= 0) return CML_OK;
+    if (w->fmt != CML_Q8_0 && w->fmt != CML_Q4_0) return fail(CML_ERR_UNSUPPORTED, "not a 32-value block format");
+    if (a.band_rows * a.n_groups != w->rows) return fail(CML_ERR_SHAPE, "%d bands of %lld rows do not cover %lld rows", a.n_groups, (long long)a.band_rows, (long long)w->rows);
+    const bool q8 = w->fmt == CML_Q8_0;
+    int p = env_int(q8 ? "CAMELID_HIP_Q8_0_LANES" : "CAMELID_HIP_Q4_0_LANES", 0);
+    if (p != 8 && p != 16) p = (w->nb <= 8) ? 8 : 16;
+    if (q8) return p == 8 ? launch_b32_grouped_p<CML_Q8_0, 8>(a, x, st) : launch_b32_grouped_p<CML_Q8_0, 16>(a, x, st);
+    return p == 8 ? launch_b32_grouped_p<CML_Q4_0, 8>(a, x, st) : launch_b32_grouped_p<CML_Q4_0, 16>(a, x, st);
+}
+
 template <int FMT>
 static int launch_b32(const MatArgs &a, hipStream_t st) {
     if (a.w->rows == 0 || a.n_tokens == 0) return CML_OK;
-    if (a.group_offsets) return fail(CML_ERR_UNSUPPORTED, "grouped (mixture-of-experts) dispatch is built for Q4_K weights only");
+    if (a.group_offsets) return launch_gemv_b32_grouped(a, nullptr, st);
     // 16 lanes per row by default; 8 when rows are short enough that half the lanes would idle.
     int p = env_int(FMT == CML_Q8_0 ? "CAMELID_HIP_Q8_0_LANES" : "CAMELID_HIP_Q4_0_LANES", 0);
     if (p != 8 && p != 16) p = (a.w->nb <= 8) ? 8 : 16;

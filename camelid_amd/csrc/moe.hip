@@ -18,7 +18,7 @@
 
 namespace cml {
 
-constexpr int kMaxExperts = 64;
+constexpr int kMaxExperts = 128;
 
 // f32::total_cmp as an integer key (larger key = greater value).
 __device__ __forceinline__ int total_key(float v) {
@@ -34,19 +34,19 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const float *__restrict__
     const float *lg = logits + t * n_experts;
     int sel_idx[kMaxExperts];
     float sel_w[kMaxExperts];
-    unsigned long long taken = 0;
+    unsigned long long taken[2] = {0, 0};
     // top-k by logit (total order, descending), ties to the lower index
     for (int s = 0; s < k; s++) {
         int best = -1, best_key = 0;
         for (int e = 0; e < n_experts; e++) {
-            if ((taken >> e) & 1ull) continue;
+            if ((taken[e >> 6] >> (e & 63)) & 1ull) continue;
             const int key = total_key(lg[e]);
             if (best < 0 || key > best_key) {
                 best = e;
                 best_key = key;
             }
         }
-        taken |= 1ull << best;
+        taken[best >> 6] |= 1ull << (best & 63);
         sel_idx[s] = best;
         sel_w[s] = lg[best];
     }
@@ -88,12 +88,62 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const float *__restrict__
     }
 }
 
+// One thread per token.  Gemma-4 routing (reference moe_layer_ffn, src/gemma4_runtime.rs:5567-5610;
+// router_top_k, :61-84): softmax over ALL experts (max folded from f32::MIN, exp(v - max), sum in
+// index order, p /= sum), top-k by probability (descending, ties to the lower index), then
+// scale[s] = down_scale[e] * (p[e] / max(sum of the selected p in selection order, 6.103515e-5)).
+__global__ __launch_bounds__(64) void moe_route_softmax_kernel(const float *__restrict__ logits, int64_t n_tokens, int n_experts,
+                                                               int k, const float *__restrict__ down_scale,
+                                                               int32_t *__restrict__ idx_out, float *__restrict__ w_out) {
+    const int64_t t = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (t >= n_tokens) return;
+    const float *lg = logits + t * n_experts;
+    float p[kMaxExperts];
+    int sel[kMaxExperts];
+    float maxl = -3.4028235e38f;
+    for (int e = 0; e < n_experts; e++) maxl = fmaxf(maxl, lg[e]);
+    float sum = 0.0f;
+    for (int e = 0; e < n_experts; e++) {
+        p[e] = expf(lg[e] - maxl);
+        sum = sum + p[e];
+    }
+    for (int e = 0; e < n_experts; e++) p[e] = p[e] / sum;
+    int len = 0;
+    for (int c = 0; c < n_experts; c++) {
+        int at = -1;
+        for (int j = 0; j < len; j++) {
+            const int cur = sel[j];
+            if (p[cur] < p[c] || (p[cur] == p[c] && c < cur)) {
+                at = j;
+                break;
+            }
+        }
+        if (at >= 0) {
+            const int last = len < k ? len : k - 1;
+            for (int j = last; j > at; j--) sel[j] = sel[j - 1];
+            sel[at] = c;
+            if (len < k) len++;
+        } else if (len < k) {
+            sel[len++] = c;
+        }
+    }
+    float wsum = 0.0f;
+    for (int s = 0; s < k; s++) wsum = wsum + p[sel[s]];
+    wsum = fmaxf(wsum, 6.103515e-5f);
+    for (int s = 0; s < k; s++) {
+        const int e = sel[s];
+        const float ds = down_scale ? down_scale[e] : 1.0f;
+        idx_out[t * k + s] = e;
+        w_out[t * k + s] = ds * (p[e] / wsum);
+    }
+}
+
 // Group the n_tokens*k assignments by expert, keeping (token, rank) order
 // inside each group.  One workgroup; thread e builds group e.
 //   offsets[e..e+1)   assignment range of expert e
 //   assign_token[j]   token whose activation assignment j reads
 //   slot_to_assign[t*k+s]  where (token t, rank s) landed
-__global__ __launch_bounds__(64) void moe_plan_kernel(const int32_t *__restrict__ idx, int n_slots, int n_experts, int k,
+__global__ __launch_bounds__(kMaxExperts) void moe_plan_kernel(const int32_t *__restrict__ idx, int n_slots, int n_experts, int k,
                                                       int32_t *__restrict__ offsets, int32_t *__restrict__ assign_token,
                                                       int32_t *__restrict__ slot_to_assign) {
     __shared__ int count[kMaxExperts + 1];
@@ -123,8 +173,16 @@ __global__ __launch_bounds__(64) void moe_plan_kernel(const int32_t *__restrict_
 // Expert-grouped matmul: the packed-dot kernel for a few tokens, the matrix cores from 4 tokens
 // up (the same crossover as for plain calls).  Both produce the same bits per cell.
 static int launch_expert_matmul(const MatArgs &a, hipStream_t st) {
+    if (a.w->fmt != CML_Q4_K) return launch_gemv_b32_grouped(a, nullptr, st);
     if (a.n_tokens >= env_int("CAMELID_HIP_Q4K_MFMA_MIN_TOKENS", 4)) return launch_gemm_q4k_mfma(a, st);
     return launch_gemv_q4k(a, st);
+}
+
+static bool expert_format(int fmt) { return fmt == CML_Q4_K || fmt == CML_Q8_0 || fmt == CML_Q4_0; }
+// Activation quantization an expert matrix of this format is dotted with: 2 = Q8_K, 1 = Q8_0.
+static int act_of(int fmt) { return fmt == CML_Q4_K ? 2 : 1; }
+static int launch_quantize_act(int act, const float *x, int64_t n, int64_t cols, int8_t *q, float *s, hipStream_t st) {
+    return act == 2 ? launch_quantize_q8_k(x, n, cols, q, s, st) : launch_quantize_q8_0(x, n, cols, q, s, st);
 }
 
 // out[t][c] = ((0 + y[a(t,0)][c]*w[t][0]) + y[a(t,1)][c]*w[t][1]) + ...  (reference
@@ -163,14 +221,15 @@ static MoeWorkspace carve(void *base, int64_t hidden, int64_t ff, int64_t n_toke
     };
     const size_t T = static_cast<size_t>(n_tokens), A = T * static_cast<size_t>(k);
     w.xq = reinterpret_cast<int8_t *>(take(T * hidden));
-    w.xd = reinterpret_cast<float *>(take(T * (hidden / 256) * 4));
+    // scale arrays are sized for 32-value blocks, the finest any expert format uses
+    w.xd = reinterpret_cast<float *>(take(T * ((hidden + 31) / 32) * 4));
     w.offsets = reinterpret_cast<int32_t *>(take((static_cast<size_t>(n_experts) + 1) * 4));
     w.assign_token = reinterpret_cast<int32_t *>(take(A * 4));
     w.slot_to_assign = reinterpret_cast<int32_t *>(take(A * 4));
     w.g = reinterpret_cast<float *>(take(A * ff * 4));
     w.u = reinterpret_cast<float *>(take(A * ff * 4));
     w.hq = reinterpret_cast<int8_t *>(take(A * ff));
-    w.hd = reinterpret_cast<float *>(take(A * (ff / 256) * 4));
+    w.hd = reinterpret_cast<float *>(take(A * ((ff + 31) / 32) * 4));
     w.y = reinterpret_cast<float *>(take(A * hidden * 4));
     w.total = at;
     return w;
@@ -196,24 +255,52 @@ int cml_moe_route_top_k(const float *logits_dev, int64_t n_tokens, int n_experts
     return CML_OK;
 }
 
+int cml_moe_route_softmax_top_k(const float *logits_dev, int64_t n_tokens, int n_experts, int k, const float *down_scale_dev,
+                                int32_t *idx_dev, float *weight_dev, cml_stream_t stream) {
+    if (!ready()) return fail(CML_ERR_UNAVAILABLE, "cml_init has not succeeded");
+    if (n_tokens < 0 || n_experts <= 0 || k <= 0) return fail(CML_ERR_SHAPE, "bad routing shape");
+    if (n_experts > kMaxExperts) return fail(CML_ERR_UNSUPPORTED, "at most %d experts", kMaxExperts);
+    if (k > n_experts) return fail(CML_ERR_SHAPE, "top-%d of %d experts", k, n_experts);
+    if (n_tokens == 0) return CML_OK;
+    if (!logits_dev || !idx_dev || !weight_dev) return fail(CML_ERR_INVALID, "null pointer");
+    const unsigned grid = static_cast<unsigned>((n_tokens + 63) / 64);
+    hipLaunchKernelGGL(moe_route_softmax_kernel, dim3(grid), dim3(64), 0, as_stream(stream), logits_dev, n_tokens, n_experts, k,
+                       down_scale_dev, idx_dev, weight_dev);
+    CML_HIP_TRY(hipGetLastError());
+    return CML_OK;
+}
+
 size_t cml_moe_workspace_bytes(int fmt, int64_t hidden, int64_t ff, int64_t n_tokens, int k, int n_experts) {
-    if (fmt != CML_Q4_K || hidden <= 0 || ff <= 0 || n_tokens <= 0 || k <= 0 || n_experts <= 0) return 0;
+    if (!expert_format(fmt) || hidden <= 0 || ff <= 0 || n_tokens <= 0 || k <= 0 || n_experts <= 0) return 0;
     return carve(nullptr, hidden, ff, n_tokens, k, n_experts).total;
 }
 
 int cml_moe_ffn(const cml_weight *gate, const cml_weight *up, const cml_weight *down, int n_experts, int k,
                 const int32_t *idx_dev, const float *weight_dev, const float *x_dev, int64_t n_tokens, float *out_dev,
                 void *workspace_dev, size_t workspace_bytes, cml_stream_t stream) {
+    if (!up) return fail(CML_ERR_INVALID, "null weight");
+    return cml_moe_ffn_ex(gate, up, down, n_experts, k, idx_dev, weight_dev, x_dev, n_tokens, out_dev, workspace_dev, workspace_bytes,
+                          CML_GLU_SILU, stream);
+}
+
+int cml_moe_ffn_ex(const cml_weight *gate, const cml_weight *up, const cml_weight *down, int n_experts, int k,
+                   const int32_t *idx_dev, const float *weight_dev, const float *x_dev, int64_t n_tokens, float *out_dev,
+                   void *workspace_dev, size_t workspace_bytes, int glu, cml_stream_t stream) {
     if (!ready()) return fail(CML_ERR_UNAVAILABLE, "cml_init has not succeeded");
-    if (!gate || !up || !down) return fail(CML_ERR_INVALID, "null weight");
-    if (gate->fmt != CML_Q4_K || up->fmt != CML_Q4_K || down->fmt != CML_Q4_K)
-        return fail(CML_ERR_UNSUPPORTED, "mixture-of-experts dispatch is built for Q4_K expert matrices only");
+    if (!gate || !down) return fail(CML_ERR_INVALID, "null weight");
+    if (glu != CML_GLU_SILU && glu != CML_GLU_GELU_TANH) return fail(CML_ERR_INVALID, "unknown expert activation %d", glu);
+    const bool fused_gate_up = up == nullptr;  // `gate` holds gate|up experts of 2*ff rows each
+    if (!expert_format(gate->fmt) || (up && up->fmt != gate->fmt) || !expert_format(down->fmt))
+        return fail(CML_ERR_UNSUPPORTED, "mixture-of-experts dispatch is built for Q4_K, Q8_0 and Q4_0 expert matrices (gate and up alike)");
     if (n_experts <= 0 || n_experts > kMaxExperts || k <= 0 || k > n_experts || n_tokens < 0)
         return fail(CML_ERR_SHAPE, "bad routing shape (%d experts, top-%d)", n_experts, k);
     const int64_t hidden = gate->cols, ff = down->cols;
-    if (up->cols != hidden || gate->rows != up->rows || gate->rows != ff * n_experts || down->rows != hidden * n_experts)
+    if ((up && (up->cols != hidden || gate->rows != up->rows)) || gate->rows != (fused_gate_up ? 2 : 1) * ff * n_experts ||
+        down->rows != hidden * n_experts)
         return fail(CML_ERR_SHAPE, "expert matrices do not stack to %d experts of %lld x %lld", n_experts, (long long)ff, (long long)hidden);
-    if (hidden % 256 || ff % 256) return fail(CML_ERR_SHAPE, "hidden and ff must be multiples of 256");
+    const int act_in = act_of(gate->fmt), act_mid = act_of(down->fmt);
+    if (hidden % (act_in == 2 ? 256 : 32) || ff % (act_mid == 2 ? 256 : 32))
+        return fail(CML_ERR_SHAPE, "hidden and ff must be whole blocks of the expert formats");
     if (n_tokens == 0) return CML_OK;
     if (!idx_dev || !weight_dev || !x_dev || !out_dev || !workspace_dev) return fail(CML_ERR_INVALID, "null pointer");
     if ((reinterpret_cast<uintptr_t>(x_dev) & 15u) || (reinterpret_cast<uintptr_t>(workspace_dev) & 255u))
@@ -225,11 +312,13 @@ int cml_moe_ffn(const cml_weight *gate, const cml_weight *up, const cml_weight *
 
     // Decode (one token, rows of up to 4096 values): gate and up run as ONE launch that quantizes
     // the token inside every workgroup -- two launches and the quantized round trip fewer.
-    const bool fused_decode = n_tokens == 1 && hidden / 256 <= 16 && env_int("CAMELID_HIP_FUSED_QUANT", 1) != 0;
+    const bool fused_decode = n_tokens == 1 && (act_in == 1 || hidden / 256 <= 16) && env_int("CAMELID_HIP_FUSED_QUANT", 1) != 0;
+    // ws.g and ws.u are adjacent: a fused gate|up projection writes rows of 2*ff values across both
+    const int64_t glu_stride = fused_gate_up ? 2 * ff : ff;
     if (!fused_decode) {
-        if (int rc = launch_quantize_q8_k(x_dev, n_tokens, hidden, ws.xq, ws.xd, st)) return rc;
+        if (int rc = launch_quantize_act(act_in, x_dev, n_tokens, hidden, ws.xq, ws.xd, st)) return rc;
     }
-    hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(64), 0, st, idx_dev, n_slots, n_experts, k, ws.offsets, ws.assign_token, ws.slot_to_assign);
+    hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(kMaxExperts), 0, st, idx_dev, n_slots, n_experts, k, ws.offsets, ws.assign_token, ws.slot_to_assign);
     CML_HIP_TRY(hipGetLastError());
 
     MatArgs a;
@@ -242,19 +331,28 @@ int cml_moe_ffn(const cml_weight *gate, const cml_weight *up, const cml_weight *
     a.q = ws.xq;
     a.scales = ws.xd;
     a.group_rows = ws.assign_token;
-    a.band_rows = ff;
+    a.band_rows = fused_gate_up ? 2 * ff : ff;
     a.w = gate;
     a.out = ws.g;
-    if (fused_decode) {
-        if (int rc = launch_gemv_q4k_f32_grouped_pair(a, up, ws.u, x_dev, st)) return rc;
+    if (fused_decode && act_in == 1) {
+        if (int rc = launch_gemv_b32_grouped(a, x_dev, st)) return rc;
+        if (up) {
+            a.w = up;
+            a.out = ws.u;
+            if (int rc = launch_gemv_b32_grouped(a, x_dev, st)) return rc;
+        }
+    } else if (fused_decode) {
+        if (int rc = launch_gemv_q4k_f32_grouped_pair(a, up, up ? ws.u : nullptr, x_dev, st)) return rc;
+    } else if (fused_gate_up) {
+        if (int rc = launch_expert_matmul(a, st)) return rc;
     } else {
         if (int rc = launch_expert_matmul(a, st)) return rc;
         a.w = up;
         a.out = ws.u;
         if (int rc = launch_expert_matmul(a, st)) return rc;
     }
-    // h = silu(g) * u, quantized per assignment
-    if (int rc = launch_silu_mul_quantize(2, ws.g, ws.u, n_slots, ff, ws.hq, ws.hd, st)) return rc;
+    // h = act(g) * u, quantized per assignment
+    if (int rc = launch_glu_quantize(glu, act_mid, ws.g, fused_gate_up ? ws.g + ff : ws.u, n_slots, ff, glu_stride, ws.hq, ws.hd, st)) return rc;
     // down: assignment j reads its own h
     a.q = ws.hq;
     a.scales = ws.hd;

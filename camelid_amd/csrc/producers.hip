@@ -6,6 +6,8 @@
 //   silu(gate) * up -> Q8_0/Q8_K reference silu_mul_quantize[_q8k] (src/cuda_resident.rs:
 //                                4289-4341), CPU arithmetic CpuTensor::silu_mul,
 //                                src/tensor/mod.rs:2610-2634
+//   gelu_tanh(gate) * up -> ...  reference geglu_quantize_routed (src/cuda_resident.rs:6301-6343),
+//                                CPU arithmetic src/gemma4_runtime.rs:5689-5691
 // The quantizers are the ones of quantize.hip (same device functions), so the
 // fused result equals the composed one bit for bit.
 //
@@ -155,21 +157,36 @@ int launch_rms_norm_quantize(int act, const float *x, const float *weight, float
 
 // h = silu(g) * u = (g / (1 + exp(-g))) * u, quantized on the fly.  Q8_K: one wave per
 // 256-value super-block, lane l holding values 4l..4l+3 (the layout of quantize_q8_k_kernel).
-__device__ __forceinline__ float4 silu_mul4(const float4 gv, const float4 uv) {
-    float4 v;
-    v.x = (gv.x / (1.0f + expf(-gv.x))) * uv.x;
-    v.y = (gv.y / (1.0f + expf(-gv.y))) * uv.y;
-    v.z = (gv.z / (1.0f + expf(-gv.z))) * uv.z;
-    v.w = (gv.w / (1.0f + expf(-gv.w))) * uv.w;
-    return v;
+// GLU 0: silu(g) * u = (g / (1 + exp(-g))) * u (reference CpuTensor::silu_mul).
+// GLU 1: gelu_pytorch_tanh(g) * u = (0.5 * g * (1 + tanh(C * (g + 0.044715 * g * g * g)))) * u,
+//        evaluated left to right (reference gelu_tanh, src/gemma4_mtp.rs:172-175; the expert
+//        activation of the Gemma-4 lane, src/gemma4_runtime.rs:5689-5691).
+template <int GLU>
+__device__ __forceinline__ float glu1(float g, float u) {
+    if constexpr (GLU == 0) {
+        return (g / (1.0f + expf(-g))) * u;
+    } else {
+        const float cube = ((0.044715f * g) * g) * g;
+        return ((0.5f * g) * (1.0f + tanhf(0.7978846f * (g + cube)))) * u;
+    }
+}
+template <int GLU>
+__device__ __forceinline__ float4 glu4(const float4 gv, const float4 uv) {
+    return make_float4(glu1<GLU>(gv.x, uv.x), glu1<GLU>(gv.y, uv.y), glu1<GLU>(gv.z, uv.z), glu1<GLU>(gv.w, uv.w));
 }
 
-__global__ __launch_bounds__(256) void silu_mul_quantize_q8k_kernel(const float *__restrict__ g, const float *__restrict__ u,
-                                                                    int64_t n_sb, int8_t *__restrict__ q, float *__restrict__ d) {
+// Row r of g / u starts at g + r * in_stride / u + r * in_stride (in_stride = cols for separate
+// buffers; 2 * cols with u = g + cols when a fused gate|up projection wrote both halves of a row).
+template <int GLU>
+__global__ __launch_bounds__(256) void glu_quantize_q8k_kernel(const float *__restrict__ g, const float *__restrict__ u,
+                                                               int64_t n_sb, int sb_per_row, int64_t in_stride,
+                                                               int8_t *__restrict__ q, float *__restrict__ d) {
     const int lane = threadIdx.x & 63;
     const int64_t sb = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (sb >= n_sb) return;
-    const float4 v = silu_mul4(reinterpret_cast<const float4 *>(g + sb * 256)[lane], reinterpret_cast<const float4 *>(u + sb * 256)[lane]);
+    const int64_t r = sb / sb_per_row, c = (sb - r * sb_per_row) * 256;
+    const float4 v = glu4<GLU>(reinterpret_cast<const float4 *>(g + r * in_stride + c)[lane],
+                               reinterpret_cast<const float4 *>(u + r * in_stride + c)[lane]);
     float dv;
     int bsum;
     const uint32_t packed = q8k_quantize_wave(v, dv, bsum);
@@ -178,13 +195,16 @@ __global__ __launch_bounds__(256) void silu_mul_quantize_q8k_kernel(const float 
 }
 
 // Q8_0: one thread per 4 values, 8 threads per 32-value block (the layout of quantize_q8_0_kernel).
-__global__ __launch_bounds__(256) void silu_mul_quantize_q8_0_kernel(const float *__restrict__ g, const float *__restrict__ u,
-                                                                     int64_t n_blocks, int8_t *__restrict__ q, float *__restrict__ scales) {
+template <int GLU>
+__global__ __launch_bounds__(256) void glu_quantize_q8_0_kernel(const float *__restrict__ g, const float *__restrict__ u,
+                                                                int64_t n_blocks, int blocks_per_row, int64_t in_stride,
+                                                                int8_t *__restrict__ q, float *__restrict__ scales) {
     const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     const int64_t block = tid >> 3;
     const bool live = block < n_blocks;
-    const int64_t src = live ? tid : 0;
-    const float4 v = silu_mul4(reinterpret_cast<const float4 *>(g)[src], reinterpret_cast<const float4 *>(u)[src]);
+    const int64_t bsafe = live ? block : 0;
+    const int64_t r = bsafe / blocks_per_row, c = (bsafe - r * blocks_per_row) * 32 + (tid & 7) * 4;
+    const float4 v = glu4<GLU>(*reinterpret_cast<const float4 *>(g + r * in_stride + c), *reinterpret_cast<const float4 *>(u + r * in_stride + c));
     float scale;
     const uint32_t packed = q8_0_quantize_lane8(v, scale);
     if (!live) return;
@@ -192,19 +212,30 @@ __global__ __launch_bounds__(256) void silu_mul_quantize_q8_0_kernel(const float
     if ((tid & 7) == 0) scales[block] = scale;
 }
 
-int launch_silu_mul_quantize(int act, const float *g, const float *u, int64_t n_tokens, int64_t cols, int8_t *q, float *scales,
-                             hipStream_t st) {
+// glu: 0 = silu, 1 = gelu_tanh; act: 1 = Q8_0, 2 = Q8_K.
+int launch_glu_quantize(int glu, int act, const float *g, const float *u, int64_t n_tokens, int64_t cols, int64_t in_stride,
+                        int8_t *q, float *scales, hipStream_t st) {
     if (n_tokens == 0 || cols == 0) return CML_OK;
     if (act == 1) {
         const int64_t n_blocks = n_tokens * (cols / 32);
-        const unsigned grid = static_cast<unsigned>((n_blocks * 8 + 255) / 256);
-        hipLaunchKernelGGL(silu_mul_quantize_q8_0_kernel, dim3(grid), dim3(256), 0, st, g, u, n_blocks, q, scales);
+        const dim3 grid(static_cast<unsigned>((n_blocks * 8 + 255) / 256));
+        const int bpr = static_cast<int>(cols / 32);
+        if (glu == 0) hipLaunchKernelGGL(glu_quantize_q8_0_kernel<0>, grid, dim3(256), 0, st, g, u, n_blocks, bpr, in_stride, q, scales);
+        else hipLaunchKernelGGL(glu_quantize_q8_0_kernel<1>, grid, dim3(256), 0, st, g, u, n_blocks, bpr, in_stride, q, scales);
     } else {
         const int64_t n_sb = n_tokens * (cols / 256);
-        hipLaunchKernelGGL(silu_mul_quantize_q8k_kernel, dim3(static_cast<unsigned>((n_sb + 3) / 4)), dim3(256), 0, st, g, u, n_sb, q, scales);
+        const dim3 grid(static_cast<unsigned>((n_sb + 3) / 4));
+        const int spr = static_cast<int>(cols / 256);
+        if (glu == 0) hipLaunchKernelGGL(glu_quantize_q8k_kernel<0>, grid, dim3(256), 0, st, g, u, n_sb, spr, in_stride, q, scales);
+        else hipLaunchKernelGGL(glu_quantize_q8k_kernel<1>, grid, dim3(256), 0, st, g, u, n_sb, spr, in_stride, q, scales);
     }
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
+}
+
+int launch_silu_mul_quantize(int act, const float *g, const float *u, int64_t n_tokens, int64_t cols, int8_t *q, float *scales,
+                             hipStream_t st) {
+    return launch_glu_quantize(0, act, g, u, n_tokens, cols, cols, q, scales, st);
 }
 
 }  // namespace cml

@@ -171,6 +171,14 @@ int cml_rms_norm_quantize(int act, const float *x_dev, const float *weight_dev, 
  * CML_ACT_Q8_0 or CML_ACT_Q8_K. */
 int cml_silu_mul_quantize(int act, const float *gate_dev, const float *up_dev, int64_t n_tokens,
                           int64_t cols, int8_t *q_dev, float *scales_dev, cml_stream_t stream);
+/* The same with the expert activation named: CML_GLU_SILU as above, or
+ * CML_GLU_GELU_TANH: (0.5*g*(1 + tanh(0.7978846*(g + 0.044715*g*g*g)))) * u,
+ * evaluated left to right (reference gelu_tanh, src/gemma4_mtp.rs:172-175; the
+ * Gemma-4 expert activation, src/gemma4_runtime.rs:5689-5691; device lane
+ * geglu_quantize_routed, src/cuda_resident.rs:6301-6343). */
+enum { CML_GLU_SILU = 0, CML_GLU_GELU_TANH = 1 };
+int cml_glu_quantize(int glu, int act, const float *gate_dev, const float *up_dev, int64_t n_tokens,
+                     int64_t cols, int8_t *q_dev, float *scales_dev, cml_stream_t stream);
 
 /* ---- dequantize (reference Q4KBlock::dequantize & siblings,
  *      src/tensor/mod.rs:5365-5409, :5547-5572, :5903-5924, :6039-6066) ----- */
@@ -226,6 +234,14 @@ int cml_matmul_f32(const cml_weight *w, const float *x_dev, int64_t n_tokens, fl
  * by weight.  idx_dev int32[n_tokens*k], weight_dev f32[n_tokens*k]. */
 int cml_moe_route_top_k(const float *logits_dev, int64_t n_tokens, int n_experts, int k,
                         int32_t *idx_dev, float *weight_dev, cml_stream_t stream);
+/* Gemma-4 routing on the device (reference moe_layer_ffn, src/gemma4_runtime.rs:
+ * 5567-5610; router_top_k, :61-84): softmax over ALL experts, the k most
+ * probable (ties to the lower index), weight = down_scale[e] * (p[e] /
+ * max(sum of the selected p, 6.103515e-5)) in selection order.  down_scale_dev
+ * f32[n_experts] may be null (= 1).  Up to 128 experts. */
+int cml_moe_route_softmax_top_k(const float *logits_dev, int64_t n_tokens, int n_experts, int k,
+                                const float *down_scale_dev, int32_t *idx_dev, float *weight_dev,
+                                cml_stream_t stream);
 /* Whole expert FFN for quantized stacked experts: gate/up hold n_experts*ff
  * rows of `hidden` values, down holds n_experts*hidden rows of `ff` values.
  * For every token, in routed order: y = down_e(silu(gate_e x) * up_e x),
@@ -239,6 +255,15 @@ int cml_moe_ffn(const cml_weight *gate, const cml_weight *up, const cml_weight *
                 int k, const int32_t *idx_dev, const float *weight_dev, const float *x_dev,
                 int64_t n_tokens, float *out_dev, void *workspace_dev, size_t workspace_bytes,
                 cml_stream_t stream);
+
+/* The same with the expert activation named (CML_GLU_SILU / CML_GLU_GELU_TANH)
+ * and, when up == NULL, with `gate` holding fused gate|up experts of 2*ff rows
+ * each, gate rows first (the Gemma-4 lane's gate_up_exps, reference
+ * src/gemma4_runtime.rs:5676-5691): one projection launch instead of two. */
+int cml_moe_ffn_ex(const cml_weight *gate, const cml_weight *up, const cml_weight *down, int n_experts,
+                   int k, const int32_t *idx_dev, const float *weight_dev, const float *x_dev,
+                   int64_t n_tokens, float *out_dev, void *workspace_dev, size_t workspace_bytes,
+                   int glu, cml_stream_t stream);
 
 /* ---- weight quantizer tool (reference quantize_block_q8_0 / q4_0 / q4_k,
  *      src/quantize.rs:98-244): f32 values -> GGUF wire bytes on the host, in

@@ -64,6 +64,11 @@ def lib() -> C.CDLL:
         L.orc_softmax_top_k.argtypes = [vp, i32, i32, vp, vp]
         L.orc_softmax_top_k.restype = i32
         L.orc_silu_mul.argtypes = [vp, vp, sz, vp]
+        L.orc_gelu_tanh_mul.argtypes = [vp, vp, sz, vp]
+        L.orc_router_softmax_top_k.argtypes = [vp, i32, i32, vp, vp, vp]
+        L.orc_router_softmax_top_k.restype = i32
+        L.orc_moe_ffn_ex.argtypes = [i32, i32, vp, vp, vp, i32, i32, sz, sz, vp, vp, sz, vp, i32, i32, vp]
+        L.orc_moe_ffn_ex.restype = i32
         L.orc_rms_norm.argtypes = [vp, vp, C.c_float, sz, sz, vp]
         L.orc_rms_norm.restype = None
         L.orc_moe_ffn.argtypes = [i32, vp, vp, vp, i32, i32, sz, sz, vp, vp, sz, vp, i32]
@@ -250,6 +255,41 @@ def silu_mul(a, b) -> np.ndarray:
     b = _c(b, np.float32)
     out = np.empty_like(a)
     lib().orc_silu_mul(_p(a), _p(b), a.size, _p(out))
+    return out
+
+
+def gelu_tanh_mul(a, b) -> np.ndarray:
+    a = _c(a, np.float32)
+    b = _c(b, np.float32)
+    out = np.empty_like(a)
+    lib().orc_gelu_tanh_mul(_p(a), _p(b), a.size, _p(out))
+    return out
+
+
+def router_softmax_top_k(logits, k: int, down_scale=None):
+    """Gemma-4 routing of one token: (idx int32[k'], scale f32[k'])."""
+    logits = _c(logits, np.float32).reshape(-1)
+    idx = np.zeros(k, np.int32)
+    w = np.zeros(k, np.float32)
+    ds = None if down_scale is None else _c(down_scale, np.float32)
+    n = lib().orc_router_softmax_top_k(_p(logits), logits.size, k, None if ds is None else _p(ds), _p(idx), _p(w))
+    return idx[:n], w[:n]
+
+
+def moe_ffn_ex(fmt: int, gate, up, down, n_experts: int, top_k: int, hidden: int, ff: int, logits, x,
+               variant: int = 0, down_scale=None, threads: int = 1, fmt_down: int | None = None) -> np.ndarray:
+    """variant 0 = Mixtral, 1 = Gemma-4; up=None: `gate` holds fused gate|up experts;
+    fmt_down: format of `down` when it differs from that of gate / up."""
+    gate, down = (_c(a, np.uint8).reshape(-1) for a in (gate, down))
+    upc = None if up is None else _c(up, np.uint8).reshape(-1)
+    logits = _c(logits, np.float32).reshape(-1, n_experts)
+    x = _c(x, np.float32).reshape(-1, hidden)
+    ds = None if down_scale is None else _c(down_scale, np.float32)
+    out = np.empty_like(x)
+    rc = lib().orc_moe_ffn_ex(fmt, fmt if fmt_down is None else fmt_down, _p(gate), None if upc is None else _p(upc), _p(down), n_experts, top_k, hidden, ff,
+                              _p(logits), _p(x), x.shape[0], _p(out), threads, variant, None if ds is None else _p(ds))
+    if rc != 0:
+        raise ValueError(f"orc_moe_ffn_ex failed: {rc}")
     return out
 
 

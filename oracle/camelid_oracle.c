@@ -8,6 +8,7 @@
  */
 #include "camelid_oracle.h"
 
+#include <float.h>
 #include <math.h>
 #include <pthread.h>
 #include <stdlib.h>
@@ -755,6 +756,72 @@ int orc_softmax_top_k(const float *logits, int n, int k, int32_t *idx, float *w)
     return kk;
 }
 
+/* Gemma-4 routing: src/gemma4_runtime.rs:5567-5580 (softmax over ALL experts: max folded
+ * from f32::MIN, exp(v - max), sequential sum, p /= sum), router_top_k :61-84 (top-k by
+ * probability, descending, ties to the lower index), route scale = down_scale[e] *
+ * (p[e] / max(sum of the selected p in selection order, 6.103515e-5)) (:5580-5610). */
+int orc_router_softmax_top_k(const float *logits, int n, int k, const float *down_scale, int32_t *idx, float *scale) {
+    if (n <= 0 || k <= 0)
+        return 0;
+    float *p = (float *)malloc(sizeof(float) * (size_t)n);
+    if (!p)
+        return 0;
+    float maxl = -FLT_MAX;
+    for (int i = 0; i < n; i++)
+        maxl = fmaxf(maxl, logits[i]);
+    float sum = 0.0f;
+    for (int i = 0; i < n; i++) {
+        p[i] = expf(logits[i] - maxl);
+        sum += p[i];
+    }
+    for (int i = 0; i < n; i++)
+        p[i] /= sum;
+    int keep = k < n ? k : n, len = 0;
+    for (int c = 0; c < n; c++) {
+        /* first position whose occupant ranks after the candidate: lower probability, or equal and a higher index */
+        int at = -1;
+        for (int j = 0; j < len; j++) {
+            int cur = idx[j];
+            if (p[cur] < p[c] || (p[cur] == p[c] && c < cur)) {
+                at = j;
+                break;
+            }
+        }
+        if (at >= 0 && at < keep) {
+            int last = len < keep ? len : keep - 1;
+            for (int j = last; j > at; j--)
+                idx[j] = idx[j - 1];
+            idx[at] = c;
+            if (len < keep)
+                len++;
+        } else if (at < 0 && len < keep) {
+            idx[len++] = c;
+        }
+    }
+    float wsum = 0.0f;
+    for (int s = 0; s < len; s++)
+        wsum += p[idx[s]];
+    wsum = fmaxf(wsum, 6.103515e-5f);
+    for (int s = 0; s < len; s++) {
+        float ds = down_scale ? down_scale[idx[s]] : 1.0f;
+        scale[s] = ds * (p[idx[s]] / wsum);
+    }
+    free(p);
+    return len;
+}
+
+/* gelu_pytorch_tanh(g) * u: src/gemma4_mtp.rs:172-175 and src/gemma4_runtime.rs:5689-5691:
+ * 0.5 * x * (1 + tanh(C * (x + 0.044715 * x * x * x))), C = 0.7978846, evaluated left to right. */
+void orc_gelu_tanh_mul(const float *a, const float *b, size_t n, float *out) {
+    const float C = 0.7978846f;
+    for (size_t i = 0; i < n; i++) {
+        float x = a[i];
+        float cube = ((0.044715f * x) * x) * x;
+        float g = (0.5f * x) * (1.0f + tanhf(C * (x + cube)));
+        out[i] = g * b[i];
+    }
+}
+
 /* src/tensor/mod.rs:2624: (a / (1.0 + (-a).exp())) * b. */
 void orc_silu_mul(const float *a, const float *b, size_t n, float *out) {
     for (size_t i = 0; i < n; i++)
@@ -783,6 +850,18 @@ int orc_moe_ffn(int fmt, const uint8_t *gate, const uint8_t *up, const uint8_t *
                 int n_experts, int top_k, size_t hidden, size_t ff,
                 const float *logits, const float *x, size_t n_tokens,
                 float *out, int threads) {
+    return orc_moe_ffn_ex(fmt, fmt, gate, up, down, n_experts, top_k, hidden, ff, logits, x, n_tokens, out, threads, 0, NULL);
+}
+
+/* variant 0: Mixtral (softmax_top_k routing, silu).  variant 1: Gemma-4 (softmax over all experts,
+ * route scales with down_scale, gelu_tanh; src/gemma4_runtime.rs:5550-5710).  up == NULL: `gate`
+ * holds fused gate|up experts, 2*ff rows each (gate rows first), as the Gemma-4 lane stores them.
+ * fmt is the format of gate / up, fmt_down that of down (each projection quantizes its activation
+ * for its own format, as SharedActivation does). */
+int orc_moe_ffn_ex(int fmt, int fmt_down, const uint8_t *gate, const uint8_t *up, const uint8_t *down,
+                   int n_experts, int top_k, size_t hidden, size_t ff,
+                   const float *logits, const float *x, size_t n_tokens,
+                   float *out, int threads, int variant, const float *down_scale) {
     if (n_experts <= 0 || top_k <= 0)
         return -1;
     float *g = (float *)malloc(sizeof(float) * ff);
@@ -800,13 +879,22 @@ int orc_moe_ffn(int fmt, const uint8_t *gate, const uint8_t *up, const uint8_t *
         float *o = out + t * hidden;
         for (size_t c = 0; c < hidden; c++)
             o[c] = 0.0f;
-        int kk = orc_softmax_top_k(logits + t * (size_t)n_experts, n_experts, top_k, idx, wt);
+        int kk = variant == 1 ? orc_router_softmax_top_k(logits + t * (size_t)n_experts, n_experts, top_k, down_scale, idx, wt)
+                              : orc_softmax_top_k(logits + t * (size_t)n_experts, n_experts, top_k, idx, wt);
         for (int s = 0; s < kk; s++) {
             size_t e = (size_t)idx[s];
-            rc |= orc_matmul(fmt, ORC_ORDER_PRIMARY, gate, hidden, e * ff, ff, x + t * hidden, 1, g, threads);
-            rc |= orc_matmul(fmt, ORC_ORDER_PRIMARY, up, hidden, e * ff, ff, x + t * hidden, 1, u, threads);
-            orc_silu_mul(g, u, ff, h);
-            rc |= orc_matmul(fmt, ORC_ORDER_PRIMARY, down, ff, e * hidden, hidden, h, 1, y, threads);
+            if (up) {
+                rc |= orc_matmul(fmt, ORC_ORDER_PRIMARY, gate, hidden, e * ff, ff, x + t * hidden, 1, g, threads);
+                rc |= orc_matmul(fmt, ORC_ORDER_PRIMARY, up, hidden, e * ff, ff, x + t * hidden, 1, u, threads);
+            } else {
+                rc |= orc_matmul(fmt, ORC_ORDER_PRIMARY, gate, hidden, e * 2 * ff, ff, x + t * hidden, 1, g, threads);
+                rc |= orc_matmul(fmt, ORC_ORDER_PRIMARY, gate, hidden, e * 2 * ff + ff, ff, x + t * hidden, 1, u, threads);
+            }
+            if (variant == 1)
+                orc_gelu_tanh_mul(g, u, ff, h);
+            else
+                orc_silu_mul(g, u, ff, h);
+            rc |= orc_matmul(fmt_down, ORC_ORDER_PRIMARY, down, ff, e * hidden, hidden, h, 1, y, threads);
             for (size_t c = 0; c < hidden; c++)
                 o[c] += y[c] * wt[s];
         }

@@ -29,8 +29,10 @@
  *                                stored vector in the reference: the order of
  *                                operations is transcribed, not pinned
  *                                ("parity unpinned" for the last-ulp value).
- *   softmax_top_k              : closed forms and brute force on small inputs;
- *                                libm expf may differ from Rust's by 1 ulp.
+ *   softmax_top_k, router_     : closed forms and brute force on small inputs;
+ *   softmax_top_k                libm expf may differ from Rust's by 1 ulp.
+ *   gelu_tanh_mul, silu_mul    : f64 evaluation of the formula within 1e-6; libm
+ *                                tanhf / expf vs Rust's: last ulp unpinned.
  *   rms_norm                   : the reference's known vector (tests/
  *                                tensor_primitives.rs:83-93), exact power-of-two
  *                                cases, an order-sensitive input checked against
@@ -119,6 +121,14 @@ int orc_matmul_q(int fmt, int order, const uint8_t *wire, size_t cols,
  * returns the count. */
 int orc_softmax_top_k(const float *logits, int n, int k, int32_t *idx, float *w);
 
+/* Gemma-4 routing (src/gemma4_runtime.rs:61-84, :5567-5610): softmax over all experts, top-k by
+ * probability (ties to the lower index), scale[s] = down_scale[e] * (p[e] / max(sum selected, 6.103515e-5));
+ * down_scale may be NULL (= 1).  Returns the count written. */
+int orc_router_softmax_top_k(const float *logits, int n, int k, const float *down_scale, int32_t *idx, float *scale);
+
+/* gelu_pytorch_tanh(a) * b: src/gemma4_mtp.rs:172-175, src/gemma4_runtime.rs:5689-5691. */
+void orc_gelu_tanh_mul(const float *a, const float *b, size_t n, float *out);
+
 /* RMS norm, the step upstream of the activation quantizers:
  * src/tensor/mod.rs:2707-2760 (sequential f32 sum of squares). */
 void orc_rms_norm(const float *x, const float *weight, float eps, size_t rows, size_t cols, float *out);
@@ -138,6 +148,14 @@ int orc_moe_ffn(int fmt, const uint8_t *gate, const uint8_t *up, const uint8_t *
                 int n_experts, int top_k, size_t hidden, size_t ff,
                 const float *logits, const float *x, size_t n_tokens,
                 float *out, int threads);
+
+/* The same with the routing / activation variant spelled out: variant 0 = Mixtral as above,
+ * 1 = Gemma-4 (orc_router_softmax_top_k with down_scale, gelu_tanh).  up == NULL: `gate` holds
+ * fused gate|up experts of 2*ff rows each. */
+int orc_moe_ffn_ex(int fmt, int fmt_down, const uint8_t *gate, const uint8_t *up, const uint8_t *down,
+                   int n_experts, int top_k, size_t hidden, size_t ff,
+                   const float *logits, const float *x, size_t n_tokens,
+                   float *out, int threads, int variant, const float *down_scale);
 
 /* Weight quantizers used to make synthetic inputs: src/quantize.rs:98-244.
  * Q6_K has no quantizer in the reference; orc_quantize_weights builds Q6_K

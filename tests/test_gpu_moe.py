@@ -33,17 +33,35 @@ def gpu_route(logits, k):
     return idx, w, idx.to_numpy(np.int32, (T, k)), w.to_numpy(np.float32, (T, k))
 
 
-def gpu_moe(gate, up, down, E, k, idx_dev, w_dev, x):
+def gpu_route_softmax(logits, k, down_scale=None):
+    logits = np.ascontiguousarray(logits, np.float32)
+    T, E = logits.shape
+    ld = DeviceBuffer.from_numpy(logits)
+    ds = None if down_scale is None else DeviceBuffer.from_numpy(np.ascontiguousarray(down_scale, np.float32))
+    idx = DeviceBuffer(T * k * 4)
+    w = DeviceBuffer(T * k * 4)
+    check(lib().cml_moe_route_softmax_top_k(ld.ptr, T, E, k, None if ds is None else ds.ptr, idx.ptr, w.ptr, None),
+          "cml_moe_route_softmax_top_k")
+    check(lib().cml_stream_sync(None))
+    return idx, w, idx.to_numpy(np.int32, (T, k)), w.to_numpy(np.float32, (T, k))
+
+
+def gpu_moe(gate, up, down, E, k, idx_dev, w_dev, x, glu=None):
+    """glu None: cml_moe_ffn; else cml_moe_ffn_ex with that activation (up may be None: fused gate|up)."""
     T, hidden = x.shape
     ff = down.cols
     xd = DeviceBuffer.from_numpy(x)
     out = DeviceBuffer(T * hidden * 4)
     out.fill(0xFF)
-    ws_bytes = lib().cml_moe_workspace_bytes(B.CML_Q4_K, hidden, ff, T, k, E)
+    ws_bytes = lib().cml_moe_workspace_bytes(gate.fmt, hidden, ff, T, k, E)
     assert ws_bytes > 0
     ws = DeviceBuffer(ws_bytes)
-    check(lib().cml_moe_ffn(gate.handle, up.handle, down.handle, E, k, idx_dev.ptr, w_dev.ptr, xd.ptr, T, out.ptr,
-                            ws.ptr, ws_bytes, None), "cml_moe_ffn")
+    if glu is None:
+        check(lib().cml_moe_ffn(gate.handle, up.handle, down.handle, E, k, idx_dev.ptr, w_dev.ptr, xd.ptr, T, out.ptr,
+                                ws.ptr, ws_bytes, None), "cml_moe_ffn")
+    else:
+        check(lib().cml_moe_ffn_ex(gate.handle, None if up is None else up.handle, down.handle, E, k, idx_dev.ptr, w_dev.ptr,
+                                   xd.ptr, T, out.ptr, ws.ptr, ws_bytes, glu, None), "cml_moe_ffn_ex")
     check(lib().cml_stream_sync(None))
     return out.to_numpy(np.float32, (T, hidden))
 
@@ -147,3 +165,167 @@ def test_c5_mixtral_shaped_moe(T):
     if T > tt:   # the rest of the batch: same cells as single-token calls of the same entry point
         one = gpu_moe(wg, wu, wd, E, k, *gpu_route(logits[T - 1:T], k)[:2], x[T - 1:T])
         assert G.max_rel(got[T - 1:T], one) <= 1e-6
+
+
+# ---------------------------------------------------------------- Gemma-4 variant ----
+
+GLU_SILU, GLU_GELU_TANH = 0, 1
+
+
+def test_route_softmax_top_k_matches_oracle():
+    """Softmax over all experts, top-k by probability, scales renormalised over the selection and
+    multiplied by down_scale (reference src/gemma4_runtime.rs:5567-5610): indices exact, scales
+    within the last bits expf may differ in."""
+    rng = np.random.default_rng(340)
+    logits = (rng.standard_normal((130, 128)) * 3).astype(np.float32)
+    logits[0] = 0.0                                   # all tied: the lowest indices, scale 1/k each
+    logits[1, 7] = logits[1, 99] = logits[1].max() + 1  # tie for first place: 7 before 99
+    logits[2] = [((e * 37 + 11) % 17) / 17.0 for e in range(128)]   # the reference's own tie vector
+    ds = rng.uniform(0.5, 2.0, 128).astype(np.float32)
+    for k, scale in ((8, ds), (1, None), (128, ds)):
+        G.say(f"moe route softmax 130x128 top-{k}")
+        # full ranking (k = 128) on a few rows only: two random logits a few ulps apart would rank
+        # by the last bit of expf, which the device and the host libm need not share
+        lg = logits[:4] if k == 128 else logits
+        _, _, idx, w = gpu_route_softmax(lg, k, scale)
+        for t in range(lg.shape[0]):
+            oi, ow = oracle.router_softmax_top_k(lg[t], k, down_scale=scale)
+            assert list(idx[t]) == list(oi), (k, t)
+            assert np.allclose(w[t], ow, rtol=1e-6, atol=1e-12), (k, t)
+    _, _, idx, w = gpu_route_softmax(logits[:1], 8)
+    assert list(idx[0]) == list(range(8)) and list(w[0]) == [0.125] * 8
+    G.say("moe route softmax 5x16 top-3")
+    logits = rng.standard_normal((5, 16)).astype(np.float32)
+    _, _, idx, w = gpu_route_softmax(logits, 3)
+    for t in range(5):
+        oi, ow = oracle.router_softmax_top_k(logits[t], 3)
+        assert list(idx[t]) == list(oi) and np.allclose(w[t], ow, rtol=1e-6)
+
+
+def test_route_softmax_rejects_bad_shapes():
+    d = DeviceBuffer(4096)
+    L = lib()
+    assert L.cml_moe_route_softmax_top_k(d.ptr, 1, 129, 2, None, d.ptr, d.ptr, None) == 6   # more than 128 experts
+    assert L.cml_moe_route_softmax_top_k(d.ptr, 1, 8, 9, None, d.ptr, d.ptr, None) == 3     # k > experts
+    assert L.cml_moe_route_softmax_top_k(None, 1, 8, 2, None, d.ptr, d.ptr, None) == 2
+    assert L.cml_moe_route_softmax_top_k(None, 0, 8, 2, None, None, None, None) == 0        # empty batch
+
+
+def _experts_fused(fmt, fmt_down, E, hidden, ff, seed):
+    gate_up = G.synth_weight(fmt, E * 2 * ff, hidden, seed)
+    down = G.synth_weight(fmt_down, E * hidden, ff, seed + 2)
+    return gate_up, down
+
+
+def _split_gate_up(gate_up, fmt, E, hidden, ff):
+    rb = oracle.row_bytes(fmt, hidden)
+    gu = np.asarray(gate_up, np.uint8).reshape(E, 2, ff * rb)
+    return np.ascontiguousarray(gu[:, 0]).reshape(-1), np.ascontiguousarray(gu[:, 1]).reshape(-1)
+
+
+GEMMA_SMALL = [
+    # (gate/up format, down format, hidden, ff): whole blocks of each format; 352 = 11 and 96 = 3
+    # blocks of 32, so rows end inside a 16-lane step
+    (B.CML_Q4_K, B.CML_Q4_K, 512, 256),
+    (B.CML_Q4_0, B.CML_Q4_0, 352, 96),
+    (B.CML_Q8_0, B.CML_Q8_0, 352, 96),
+    (B.CML_Q4_0, B.CML_Q8_0, 512, 704),
+    (B.CML_Q4_K, B.CML_Q4_0, 256, 96),
+]
+
+
+@pytest.mark.parametrize("T", [1, 2, 5, 40])
+@pytest.mark.parametrize("fmt,fmt_down,hidden,ff", GEMMA_SMALL)
+def test_moe_ffn_ex_gemma4_small_matches_oracle(fmt, fmt_down, hidden, ff, T):
+    E, k = 16, 4
+    gate_up, down = _experts_fused(fmt, fmt_down, E, hidden, ff, 350)
+    gate, up = _split_gate_up(gate_up, fmt, E, hidden, ff)
+    rng = np.random.default_rng(351 + T)
+    x = rng.standard_normal((T, hidden)).astype(np.float32)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    if T >= 5:
+        logits[:, 3] += 4.0   # crowd one expert: more than 8 assignments in one group at T = 40
+    ds = rng.uniform(0.5, 2.0, E).astype(np.float32)
+    G.say(f"moe ffn_ex gemma4 small fmt={fmt}/{fmt_down} {hidden}x{ff} T={T}")
+    wgu = Weight.upload(fmt, E * 2 * ff, hidden, gate_up)
+    wg = Weight.upload(fmt, E * ff, hidden, gate)
+    wu = Weight.upload(fmt, E * ff, hidden, up)
+    wd = Weight.upload(fmt_down, E * hidden, ff, down)
+    idx_dev, w_dev, idx, w = gpu_route_softmax(logits, k, ds)
+    want = oracle.moe_ffn_ex(fmt, gate_up, None, down, E, k, hidden, ff, logits, x, variant=1, down_scale=ds, threads=8,
+                             fmt_down=fmt_down)
+    with G.env(CAMELID_HIP_EXACT_ORDER="1"):
+        fused = gpu_moe(wgu, None, wd, E, k, idx_dev, w_dev, x, glu=GLU_GELU_TANH)
+        split = gpu_moe(wg, wu, wd, E, k, idx_dev, w_dev, x, glu=GLU_GELU_TANH)
+    assert G.max_rel(fused, want) <= 1e-5
+    assert G.same_bits(fused, split)      # one projection over gate|up or two: the same cells
+    got2 = gpu_moe(wgu, None, wd, E, k, idx_dev, w_dev, x, glu=GLU_GELU_TANH)   # default K-split policy
+    assert G.max_rel(got2, want) <= 1e-5
+
+
+@pytest.mark.parametrize("fmt,fmt_down", [(B.CML_Q4_0, B.CML_Q4_0), (B.CML_Q8_0, B.CML_Q4_0), (B.CML_Q4_0, B.CML_Q4_K)])
+def test_moe_ffn_ex_is_the_sum_of_single_expert_calls(fmt, fmt_down):
+    """Grouping must not change any (token, expert) cell, for the 32-value formats too: compare
+    with per-token, per-expert matvecs through the plain entry points, mixed on the host."""
+    E, k, hidden, ff, T = 6, 3, 256, 256, 7
+    gate_up, down = _experts_fused(fmt, fmt_down, E, hidden, ff, 360)
+    rng = np.random.default_rng(361)
+    x = rng.standard_normal((T, hidden)).astype(np.float32)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    wgu = Weight.upload(fmt, E * 2 * ff, hidden, gate_up)
+    wd = Weight.upload(fmt_down, E * hidden, ff, down)
+    idx_dev, w_dev, idx, w = gpu_route_softmax(logits, k)
+    G.say(f"moe ffn_ex vs single-expert calls fmt={fmt}/{fmt_down}")
+    with G.env(CAMELID_HIP_EXACT_ORDER="1"):
+        got = gpu_moe(wgu, None, wd, E, k, idx_dev, w_dev, x, glu=GLU_GELU_TANH)
+        want = np.zeros((T, hidden), np.float32)
+        for t in range(T):
+            for s in range(k):
+                e = int(idx[t, s])
+                gu = G.gpu_matmul_f32(wgu.slice(e * 2 * ff, 2 * ff), x[t]).reshape(-1)
+                h = oracle.gelu_tanh_mul(gu[:ff], gu[ff:])
+                y = G.gpu_matmul_f32(wd.slice(e * hidden, hidden), h).reshape(-1)
+                want[t] = (want[t] + (y * w[t, s]).astype(np.float32)).astype(np.float32)
+    assert G.max_rel(got, want) <= 2e-6   # gelu's tanhf is the only difference
+
+
+def test_moe_ffn_ex_rejects_bad_arguments():
+    E, k, hidden, ff = 4, 2, 256, 256
+    gate_up, down = _experts_fused(B.CML_Q4_0, B.CML_Q4_0, E, hidden, ff, 370)
+    wgu = Weight.upload(B.CML_Q4_0, E * 2 * ff, hidden, gate_up)
+    wd = Weight.upload(B.CML_Q4_0, E * hidden, ff, down)
+    w6 = Weight.upload(B.CML_Q6_K, 256, 256, G.synth_weight(B.CML_Q6_K, 256, 256, 371))
+    d = DeviceBuffer(1 << 20)
+    L = lib()
+    args = (E, k, d.ptr, d.ptr, d.ptr, 1, d.ptr, d.ptr, 1 << 20)
+    assert L.cml_moe_ffn_ex(wgu.handle, None, wd.handle, *args, 7, None) == 2        # unknown activation
+    assert L.cml_moe_ffn_ex(w6.handle, None, wd.handle, *args, 1, None) == 6         # Q6_K experts
+    assert L.cml_moe_ffn_ex(wgu.handle, wd.handle, wd.handle, *args, 1, None) == 3   # up of another shape
+    assert L.cml_moe_ffn_ex(wgu.handle, None, wd.handle, E, k, d.ptr, d.ptr, d.ptr, 1, d.ptr, d.ptr, 16, 1, None) == 3  # workspace
+    assert L.cml_moe_ffn(wgu.handle, None, wd.handle, *args, None) == 2              # the plain entry needs up
+
+
+@pytest.mark.parametrize("T", [1, 32])
+def test_gemma4_26b_shaped_moe(T):
+    """The geometry the reference admits for its Gemma-4 26B expert lane (src/gemma4_runtime.rs:
+    3389-3397, 4068-4079): 128 experts, top-8, hidden 2816, expert width 704, Q4_0, fused gate|up."""
+    E, k, hidden, ff = 128, 8, 2816, 704
+    G.say(f"Gemma-4 26B-shaped MoE T={T}: building 128 experts")
+    gate_up, down = _experts_fused(B.CML_Q4_0, B.CML_Q4_0, E, hidden, ff, 380)
+    rng = np.random.default_rng(381 + T)
+    x = rng.standard_normal((T, hidden)).astype(np.float32)
+    logits = (rng.standard_normal((T, E)) * 2).astype(np.float32)
+    ds = rng.uniform(0.5, 2.0, E).astype(np.float32)
+    wgu = Weight.upload(B.CML_Q4_0, E * 2 * ff, hidden, gate_up)
+    wd = Weight.upload(B.CML_Q4_0, E * hidden, ff, down)
+    idx_dev, w_dev, idx, w = gpu_route_softmax(logits, k, ds)
+    G.say(f"Gemma-4 26B-shaped MoE T={T}: device run")
+    got = gpu_moe(wgu, None, wd, E, k, idx_dev, w_dev, x, glu=GLU_GELU_TANH)
+    tt = min(T, 4)
+    want = oracle.moe_ffn_ex(B.CML_Q4_0, gate_up, None, down, E, k, hidden, ff, logits[:tt], x[:tt], variant=1,
+                             down_scale=ds, threads=16)
+    assert G.max_rel(got[:tt], want) <= 1e-5
+    assert np.all(np.isfinite(got))
+    if T > tt:   # the rest of the batch: the same cells as a single-token call (bit for bit: one chain per cell)
+        one = gpu_moe(wgu, None, wd, E, k, *gpu_route_softmax(logits[T - 1:T], k, ds)[:2], x[T - 1:T], glu=GLU_GELU_TANH)
+        assert G.same_bits(got[T - 1:T], one)

@@ -104,6 +104,48 @@ def test_silu_mul_quantize():
             assert np.max(np.abs(deq.reshape(n, cols) - h)) <= np.max(np.abs(s)) * 1.01 + 1e-12
 
 
+def test_gelu_tanh_mul_quantize():
+    """The Gemma-4 expert activation fused with the quantizer (reference geglu_quantize_routed,
+    src/cuda_resident.rs:6301-6343).  tanhf on the device vs the host libm: h may differ in its
+    last bits, hence at most one quantization step; all-zero blocks stay exact."""
+    rng = np.random.default_rng(991)
+    for n, cols in ((1, 704), (3, 2048), (8, 256)):
+        g = (rng.standard_normal((n, cols)) * 2).astype(np.float32)
+        u = rng.standard_normal((n, cols)).astype(np.float32)
+        g[0, :256] = 0.0
+        h = oracle.gelu_tanh_mul(g, u)
+        gd, ud = DeviceBuffer.from_numpy(g), DeviceBuffer.from_numpy(u)
+        for act, per in ((ACT_Q8_0, 32), (ACT_Q8_K, 256)):
+            if cols % per:
+                continue
+            G.say(f"glu_quantize gelu_tanh {n}x{cols} act={act}")
+            qd, sd = DeviceBuffer(n * cols), DeviceBuffer(n * (cols // per) * 4)
+            check(lib().cml_glu_quantize(1, act, gd.ptr, ud.ptr, n, cols, qd.ptr, sd.ptr, None), "cml_glu_quantize")
+            check(lib().cml_stream_sync(None))
+            q = qd.to_numpy(np.int8, (n, cols)).astype(np.int32)
+            s = sd.to_numpy(np.float32, (n, cols // per))
+            so, qo = (oracle.quantize_q8_0 if act == ACT_Q8_0 else oracle.quantize_q8_k)(h)
+            assert np.max(np.abs(q - qo.astype(np.int32))) <= 1
+            assert np.allclose(s, so, rtol=2e-6, atol=0)
+            assert not q[0, :256].any() and not s[0, :256 // per].any()
+            deq = q.reshape(n, cols // per, per) * s[:, :, None]
+            assert np.max(np.abs(deq.reshape(n, cols) - h)) <= np.max(np.abs(s)) * 1.01 + 1e-12
+    # the selector 0 is cml_silu_mul_quantize, bit for bit
+    g = (rng.standard_normal((2, 512)) * 2).astype(np.float32)
+    u = rng.standard_normal((2, 512)).astype(np.float32)
+    gd, ud = DeviceBuffer.from_numpy(g), DeviceBuffer.from_numpy(u)
+    outs = []
+    for call in (lambda q, s: lib().cml_glu_quantize(0, ACT_Q8_K, gd.ptr, ud.ptr, 2, 512, q, s, None),
+                 lambda q, s: lib().cml_silu_mul_quantize(ACT_Q8_K, gd.ptr, ud.ptr, 2, 512, q, s, None)):
+        qd, sd = DeviceBuffer(1024), DeviceBuffer(16)
+        check(call(qd.ptr, sd.ptr))
+        check(lib().cml_stream_sync(None))
+        outs.append((qd.to_numpy(np.int8, (1024,)), sd.to_numpy(np.float32, (4,))))
+    assert np.array_equal(outs[0][0], outs[1][0]) and np.array_equal(outs[0][1], outs[1][1])
+    d = DeviceBuffer(4096)
+    assert lib().cml_glu_quantize(2, ACT_Q8_0, d.ptr, d.ptr, 1, 256, d.ptr, d.ptr, None) == 2   # unknown activation
+
+
 def test_producer_error_paths():
     L = lib()
     d = DeviceBuffer(4096)

@@ -403,6 +403,114 @@ def test_moe_ffn_is_the_composition_of_its_pieces():
         assert np.array_equal(acc.view(np.uint32), out[t].view(np.uint32))
 
 
+def test_router_softmax_top_k_reference_tie_vector():
+    """The reference's own selection test (src/gemma4_runtime.rs:21548-21561): 128 values
+    ((e*37+11)%17)/17 with many repeats, top-k must equal a full sort by (descending value,
+    ascending index).  Fed as logits: exp is monotone and equal logits give equal probabilities,
+    so the selection over probabilities is the selection over these values."""
+    vals = np.array([((e * 37 + 11) % 17) / 17.0 for e in range(128)], np.float32)
+    full = sorted(range(128), key=lambda i: (-float(vals[i]), i))
+    for k in [1, 8, 17, 127, 128, 256]:
+        idx, _ = oracle.router_softmax_top_k(vals, k)
+        assert list(idx) == full[:min(k, 128)], k
+
+
+def test_router_softmax_top_k_closed_forms():
+    # all equal: p = 1/n each, the first k win, scale = (1/n) / (k/n) = 1/k
+    idx, sc = oracle.router_softmax_top_k(np.zeros(8, np.float32), 4)
+    assert list(idx) == [0, 1, 2, 3] and list(sc) == [0.25] * 4
+    # softmax over ALL experts, renormalised over the selected ones: the ratio of two scales is
+    # exp(logit difference) and they sum to 1, whatever the unselected logits are
+    for rest in (-30.0, 0.5):
+        idx, sc = oracle.router_softmax_top_k([1.0, rest, 3.0, 2.0, rest], 2)
+        e = np.exp(-1.0)
+        assert list(idx) == [2, 3]
+        assert np.allclose(sc, [1 / (1 + e), e / (1 + e)], rtol=3e-7)
+    # down_scale multiplies per selected expert after the renormalisation
+    ds = np.array([2.0, 1.0, 0.5, 4.0, 1.0], np.float32)
+    idx, sc2 = oracle.router_softmax_top_k([1.0, 0.5, 3.0, 2.0, 0.5], 2, down_scale=ds)
+    assert list(idx) == [2, 3]
+    assert np.array_equal(sc2, sc * np.array([0.5, 4.0], np.float32))
+    # k = n: every expert, in descending order; the scales are the plain softmax
+    lg = np.array([0.3, -1.0, 2.0, 0.3], np.float32)
+    idx, sc = oracle.router_softmax_top_k(lg, 4)
+    assert list(idx) == [2, 0, 3, 1]
+    p = np.exp(lg.astype(np.float64) - 2.0)
+    assert np.allclose(sc, (p / p.sum())[[2, 0, 3, 1]], rtol=5e-7)
+
+
+def test_router_softmax_top_k_brute_force():
+    rng = np.random.default_rng(63)
+    for trial in range(200):
+        n, k = (128, 8) if trial % 2 else (16, 3)
+        logits = (rng.standard_normal(n) * 3).astype(np.float32)
+        ds = rng.uniform(0.5, 2.0, n).astype(np.float32)
+        idx, sc = oracle.router_softmax_top_k(logits, k, down_scale=ds)
+        order = sorted(range(n), key=lambda i: (-float(logits[i]), i))[:k]
+        assert list(idx) == order
+        p = np.exp(logits.astype(np.float64) - float(logits.max()))
+        want = ds[order] * (p[order] / p[order].sum())
+        assert np.allclose(sc, want, rtol=2e-6)
+
+
+def test_gelu_tanh_mul_reference_values_and_f64():
+    """Known answers of the reference's unit tests (src/inference/gemma4.rs:90-111), then the
+    formula in float64 (the libm tanhf's last bit is not pinned by anything the reference holds)."""
+    one = np.ones(1, np.float32)
+    for x, want, tol in [(0.0, 0.0, 1e-6), (1.0, 0.841192, 1e-4), (-1.0, -0.158808, 1e-4), (2.0, 1.954598, 1e-4),
+                         (8.0, 8.0, 1e-3), (-8.0, 0.0, 1e-3)]:
+        assert abs(float(oracle.gelu_tanh_mul(np.float32([x]), one)[0]) - want) <= tol, x
+    got = oracle.gelu_tanh_mul(np.float32([0.0, 1.0, 2.0]), np.float32([3.0, 4.0, 5.0]))
+    assert got[0] == 0.0
+    assert got[1] == np.float32(oracle.gelu_tanh_mul(np.float32([1.0]), one)[0] * np.float32(4.0))
+    assert got[2] == np.float32(oracle.gelu_tanh_mul(np.float32([2.0]), one)[0] * np.float32(5.0))
+    rng = np.random.default_rng(64)
+    a = (rng.standard_normal(8192) * 3).astype(np.float32)
+    b = rng.standard_normal(8192).astype(np.float32)
+    a64 = a.astype(np.float64)
+    want = 0.5 * a64 * (1 + np.tanh(np.sqrt(2 / np.pi) * (a64 + 0.044715 * a64 ** 3))) * b
+    got = oracle.gelu_tanh_mul(a, b)
+    # 1 + tanh cancels for negative inputs: absolute error there is a few ulp of 1 times |0.5 a b|
+    assert np.all(np.abs(got - want) <= 2e-6 * np.abs(want) + 4e-7 * np.abs(0.5 * a64 * b))
+    # odd-part identity gelu(x) - gelu(-x) = x holds to rounding: pins the sign of the cubic term
+    gp = oracle.gelu_tanh_mul(a, np.ones_like(a))
+    gm = oracle.gelu_tanh_mul(-a, np.ones_like(a))
+    assert np.allclose(gp - gm, a, rtol=1e-6, atol=1e-6)
+
+
+def test_moe_ffn_ex_gemma4_is_the_composition_of_its_pieces():
+    """Gemma-4 expert mix (reference moe_layer_ffn, src/gemma4_runtime.rs:5567-5708): route over
+    the full softmax, fused gate|up band of 2*ff rows per expert, gelu_tanh(g)*u, down band,
+    acc += y * (down_scale[e] * p[e]/wsum) in selection order.  Also: the separate-gate/up call on
+    the de-interleaved halves gives the same bits."""
+    rng = np.random.default_rng(65)
+    n_exp, hidden, ff, k = 6, 256, 512, 3
+    gate_up = oracle.quantize_weights(Q4_K, rng.standard_normal((n_exp * 2 * ff, hidden)).astype(np.float32) * 0.05)
+    down = oracle.quantize_weights(Q4_K, rng.standard_normal((n_exp * hidden, ff)).astype(np.float32) * 0.05)
+    ds = rng.uniform(0.5, 2.0, n_exp).astype(np.float32)
+    x = rng.standard_normal((3, hidden)).astype(np.float32)
+    logits = rng.standard_normal((3, n_exp)).astype(np.float32)
+    out = oracle.moe_ffn_ex(Q4_K, gate_up, None, down, n_exp, k, hidden, ff, logits, x, variant=1, down_scale=ds)
+    for t in range(3):
+        acc = np.zeros(hidden, np.float32)
+        idx, sc = oracle.router_softmax_top_k(logits[t], k, down_scale=ds)
+        for e, wt in zip(idx, sc):
+            gu = oracle.matmul(Q4_K, gate_up, hidden, x[t], row_start=e * 2 * ff, rows=2 * ff).reshape(-1)
+            h = oracle.gelu_tanh_mul(gu[:ff], gu[ff:])
+            y = oracle.matmul(Q4_K, down, ff, h, row_start=e * hidden, rows=hidden)
+            acc = (acc + (y * wt).astype(np.float32)).astype(np.float32)
+        assert np.array_equal(acc.view(np.uint32), out[t].view(np.uint32))
+    rb = oracle.row_bytes(Q4_K, hidden)
+    gu3 = gate_up.reshape(n_exp, 2, ff * rb)
+    out2 = oracle.moe_ffn_ex(Q4_K, gu3[:, 0].copy(), gu3[:, 1].copy(), down, n_exp, k, hidden, ff, logits, x, variant=1,
+                             down_scale=ds)
+    assert np.array_equal(out.view(np.uint32), out2.view(np.uint32))
+    # variant 0 through the extended entry is the plain entry
+    a = oracle.moe_ffn_ex(Q4_K, gu3[:, 0].copy(), gu3[:, 1].copy(), down, n_exp, 2, hidden, ff, logits, x)
+    b = oracle.moe_ffn(Q4_K, gu3[:, 0].copy(), gu3[:, 1].copy(), down, n_exp, 2, hidden, ff, logits, x)
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
 # ----------------------------------------------------- weight quantizers ---
 
 def test_weight_quantizer_error_bounds_on_reference_ramps():
