@@ -132,32 +132,46 @@ def cpu_baseline(fmt: int, wire: np.ndarray, rows: int, cols: int, x: np.ndarray
 
 
 MOE_CONFIGS = {
-    # name -> (experts, top_k, hidden, ff, tokens): Mixtral-8x7B-shaped expert FFN in Q4_K
-    "moe_q4k_8x14336x4096_t1": (8, 2, 4096, 14336, 1),
-    "moe_q4k_8x14336x4096_t32": (8, 2, 4096, 14336, 32),
+    # name -> (variant, format, experts, top_k, hidden, ff, tokens)
+    # Mixtral-8x7B-shaped expert FFN in Q4_K: separate gate / up tensors, top-k softmax routing, silu
+    "moe_q4k_8x14336x4096_t1": ("mixtral", "Q4_K", 8, 2, 4096, 14336, 1),
+    "moe_q4k_8x14336x4096_t32": ("mixtral", "Q4_K", 8, 2, 4096, 14336, 32),
+    # Gemma-4 26B-shaped expert lane in Q4_0: fused gate|up tensor, full-softmax routing with
+    # per-expert down scales, gelu_tanh
+    "moe_q4_0_128x704x2816_t1": ("gemma4", "Q4_0", 128, 8, 2816, 704, 1),
+    "moe_q4_0_128x704x2816_t32": ("gemma4", "Q4_0", 128, 8, 2816, 704, 32),
 }
 
 
 def bench_moe(name: str, K: int, W: int, seed: int, cpu_seconds: float) -> int:
-    """One step = route (top-k softmax) + the whole expert FFN (gate, up, silu*up -> Q8_K, down,
-    weighted sum) for all tokens, on stacked expert tensors resident in HBM.  Steps rotate over
-    several routing inputs and two copies of the layer, so different experts are touched and
-    nothing is served from cache."""
+    """One step = route + the whole expert FFN (gate and up projections, activation * up ->
+    quantize, down projection, weighted sum) for all tokens, on stacked expert tensors resident
+    in HBM.  Steps rotate over several routing inputs and several copies of the layer, so different
+    experts are touched and nothing is served from cache."""
     L = lib()
-    E, k, hidden, ff, T = MOE_CONFIGS[name]
-    fmt = B.FORMATS["Q4_K"]
+    variant, fmt_name, E, k, hidden, ff, T = MOE_CONFIGS[name]
+    gemma = variant == "gemma4"
+    fmt = B.FORMATS[fmt_name]
     # values do not matter for timing: one expert's worth of seeded weights, repeated for every expert
     g1 = synth_weight(fmt, ff, hidden, seed)
     u1 = synth_weight(fmt, ff, hidden, seed + 1)
     d1 = synth_weight(fmt, hidden, ff, seed + 2)
-    gate_w, up_w, down_w = np.tile(g1, E), np.tile(u1, E), np.tile(d1, E)
-    layers = [(Weight.upload(fmt, E * ff, hidden, gate_w), Weight.upload(fmt, E * ff, hidden, up_w),
-               Weight.upload(fmt, E * hidden, ff, down_w)) for _ in range(2)]
+    expert_bytes = g1.nbytes + u1.nbytes + d1.nbytes
+    down_w = np.tile(d1, E)
+    n_layers = max(2, min(16, -(-600_000_000 // (E * expert_bytes))))
+    if gemma:
+        gate_w, up_w = np.tile(np.concatenate([g1, u1]), E), None
+        layers = [(Weight.upload(fmt, E * 2 * ff, hidden, gate_w), None, Weight.upload(fmt, E * hidden, ff, down_w))
+                  for _ in range(n_layers)]
+    else:
+        gate_w, up_w = np.tile(g1, E), np.tile(u1, E)
+        layers = [(Weight.upload(fmt, E * ff, hidden, gate_w), Weight.upload(fmt, E * ff, hidden, up_w),
+                   Weight.upload(fmt, E * hidden, ff, down_w)) for _ in range(n_layers)]
     rng = np.random.default_rng(seed + 3)
     n_sets = 8
     logits = rng.standard_normal((n_sets, T, E)).astype(np.float32)
     x = rng.standard_normal((T, hidden)).astype(np.float32)
-    expert_bytes = g1.nbytes + u1.nbytes + d1.nbytes
+    down_scale = rng.uniform(0.5, 2.0, E).astype(np.float32)
     touched = [len(set(np.argsort(-logits[s], axis=1, kind="stable")[:, :k].reshape(-1))) for s in range(n_sets)]
     alg_bytes = float(np.mean(touched)) * expert_bytes + 2 * 4 * T * hidden + 4 * T * E
 
@@ -165,6 +179,7 @@ def bench_moe(name: str, K: int, W: int, seed: int, cpu_seconds: float) -> int:
     check(L.cml_stream_create(C.byref(stream)))
     ld = [DeviceBuffer.from_numpy(logits[s]) for s in range(n_sets)]
     xd = DeviceBuffer.from_numpy(x)
+    dsd = DeviceBuffer.from_numpy(down_scale)
     idx = DeviceBuffer(T * k * 4)
     wts = DeviceBuffer(T * k * 4)
     out = DeviceBuffer(T * hidden * 4)
@@ -173,10 +188,16 @@ def bench_moe(name: str, K: int, W: int, seed: int, cpu_seconds: float) -> int:
     timer = Timer(stream)
 
     def step(i):
-        gate, up, down = layers[i % 2]
-        check(L.cml_moe_route_top_k(ld[i % n_sets].ptr, T, E, k, idx.ptr, wts.ptr, stream), "cml_moe_route_top_k")
-        check(L.cml_moe_ffn(gate.handle, up.handle, down.handle, E, k, idx.ptr, wts.ptr, xd.ptr, T, out.ptr,
-                            ws.ptr, ws_bytes, stream), "cml_moe_ffn")
+        gate, up, down = layers[i % n_layers]
+        if gemma:
+            check(L.cml_moe_route_softmax_top_k(ld[i % n_sets].ptr, T, E, k, dsd.ptr, idx.ptr, wts.ptr, stream),
+                  "cml_moe_route_softmax_top_k")
+            check(L.cml_moe_ffn_ex(gate.handle, None, down.handle, E, k, idx.ptr, wts.ptr, xd.ptr, T, out.ptr,
+                                   ws.ptr, ws_bytes, 1, stream), "cml_moe_ffn_ex")
+        else:
+            check(L.cml_moe_route_top_k(ld[i % n_sets].ptr, T, E, k, idx.ptr, wts.ptr, stream), "cml_moe_route_top_k")
+            check(L.cml_moe_ffn(gate.handle, up.handle, down.handle, E, k, idx.ptr, wts.ptr, xd.ptr, T, out.ptr,
+                                ws.ptr, ws_bytes, stream), "cml_moe_ffn")
 
     for i in range(W):
         step(i)
@@ -189,19 +210,25 @@ def bench_moe(name: str, K: int, W: int, seed: int, cpu_seconds: float) -> int:
         print("non-finite output", file=sys.stderr)
         return 4
     gbs = alg_bytes / (ms * 1e-3) / 1e9
+    if gemma:
+        # route, plan, [quantize,] gate|up, gelu*up->Q8_0, down, weighted sum
+        launches, kernel = (6 if T == 1 else 7), "gemv_b32_grouped_kernel (2 launches of the step)"
+        what = "route (full softmax) + fused gate|up matvec + gelu_tanh*up->Q8_0 + down matvec + weighted sum, graph replay"
+    else:
+        # route, plan, [quantize,] gate, up (one launch at 1 token), silu*up->Q8_K, down, weighted sum
+        launches, kernel = (6 if T == 1 else 8), "gemv_q4k_kernel / gemm_q4k_mfma_kernel grouped by expert (2-3 launches of the step)"
+        what = "route + gate/up matvecs + silu*up->Q8_K + down matvec + weighted sum, graph replay"
     line = {
-        "metric": f"Q4_K mixture-of-experts FFN µs + achieved HBM GB/s, {E} experts top-{k}, {ff}x{hidden}, {T} token(s)",
+        "metric": f"{fmt_name} mixture-of-experts FFN µs + achieved HBM GB/s, {E} experts top-{k}, {ff}x{hidden}, {T} token(s)",
         "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": W,
         "ms_per_step": round(ms, 6), "us_per_call": round(ms * 1e3, 3),
         "pct_of_hbm_peak": round(100.0 * gbs / HBM_PEAK_GBS, 2),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
-        "config": {"workload": name, "format": "Q4_K", "experts": E, "top_k": k, "hidden": hidden, "ff": ff, "tokens": T,
-                   "algorithmic_bytes_per_call": int(alg_bytes), "mean_experts_touched": float(np.mean(touched)),
-                   "step": "route + gate/up matvecs + silu*up->Q8_K + down matvec + weighted sum, graph replay",
-                   # route, plan, [quantize,] gate, up (one launch at 1 token), silu*up->Q8_K, down, weighted sum
-                   "launches_per_step": 6 if T == 1 else 8},
+        "config": {"workload": name, "variant": variant, "format": fmt_name, "experts": E, "top_k": k, "hidden": hidden, "ff": ff,
+                   "tokens": T, "algorithmic_bytes_per_call": int(alg_bytes), "mean_experts_touched": float(np.mean(touched)),
+                   "layer_copies": n_layers, "step": what, "launches_per_step": launches},
         # the expert matvec launches carry the bytes; the figure is for the whole step
-        "roofline": {"bound": "hbm", "kernel": "gemv_q4k_kernel / gemm_q4k_mfma_kernel grouped by expert (2-3 launches of the step)",
+        "roofline": {"bound": "hbm", "kernel": kernel,
                      "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
                      "traffic": None, "us_per_launch": round(ms * 1e3, 3), "note": "whole step, all launches"},
     }
@@ -212,7 +239,8 @@ def bench_moe(name: str, K: int, W: int, seed: int, cpu_seconds: float) -> int:
         t_end = time.perf_counter() + cpu_seconds
         while len(times) < 2 or (time.perf_counter() < t_end and len(times) < 50):
             t0 = time.perf_counter()
-            oracle.moe_ffn(fmt, gate_w, up_w, down_w, E, k, hidden, ff, logits[len(times) % n_sets], x, threads=threads)
+            oracle.moe_ffn_ex(fmt, gate_w, up_w, down_w, E, k, hidden, ff, logits[len(times) % n_sets], x,
+                              variant=1 if gemma else 0, down_scale=down_scale if gemma else None, threads=threads)
             times.append(time.perf_counter() - t0)
         med = float(np.median(times))
         line["cpu_baseline"] = {"value": round(alg_bytes / med / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",

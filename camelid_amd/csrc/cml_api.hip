@@ -507,7 +507,7 @@ static int dispatch(const MatArgs &a, hipStream_t st) {
 }
 
 static MatArgs plain_args(const cml_weight *w, const int8_t *q, const float *s, int64_t n_tokens, float *out) {
-    MatArgs a;
+    MatArgs a{};
     a.w = w;
     a.q = q;
     a.scales = s;

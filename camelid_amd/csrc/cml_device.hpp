@@ -207,6 +207,25 @@ __device__ __forceinline__ int row_allor(int v) {
     return v;
 }
 
+// ---- gated activations ------------------------------------------------------------------------
+// GLU 0: silu(g) * u = (g / (1 + exp(-g))) * u (reference CpuTensor::silu_mul).
+// GLU 1: gelu_pytorch_tanh(g) * u = (0.5 * g * (1 + tanh(C * (g + 0.044715 * g * g * g)))) * u,
+//        evaluated left to right (reference gelu_tanh, src/gemma4_mtp.rs:172-175; the expert
+//        activation of the Gemma-4 lane, src/gemma4_runtime.rs:5689-5691).
+template <int GLU>
+__device__ __forceinline__ float glu1(float g, float u) {
+    if constexpr (GLU == 0) {
+        return (g / (1.0f + expf(-g))) * u;
+    } else {
+        const float cube = ((0.044715f * g) * g) * g;
+        return ((0.5f * g) * (1.0f + tanhf(0.7978846f * (g + cube)))) * u;
+    }
+}
+template <int GLU>
+__device__ __forceinline__ float4 glu4(const float4 gv, const float4 uv) {
+    return make_float4(glu1<GLU>(gv.x, uv.x), glu1<GLU>(gv.y, uv.y), glu1<GLU>(gv.z, uv.z), glu1<GLU>(gv.w, uv.w));
+}
+
 // The same quantizer with a 16-lane row per super-block, so that one wave does
 // four super-blocks in one pass and one dependency chain: lane l of a row holds
 // values 16l..16l+15 (v[0..3]).  Returns the 16 quants packed in value order;

@@ -96,6 +96,11 @@ struct MatArgs {
     // activation row group_rows[j] (j itself when null) and writes out[j][band_rows].
     const int32_t *group_offsets;  // device, [n_groups + 1]
     const int32_t *group_rows;     // device, [assignments] or null
+    // Optional compaction of the grid: group_ids[y] is the group that y-slot y serves, the groups
+    // that hold assignments first, -1 in the slots after them; the grid then has max_active
+    // y-slots (at least the number of groups that can be non-empty) instead of n_groups.
+    const int32_t *group_ids;      // device, [n_groups] or null
+    int max_active;
     int n_groups;
     int64_t band_rows;
 };
@@ -106,8 +111,17 @@ int launch_gemv_q4k_f32_grouped_pair(const MatArgs &a, const cml_weight *w2, flo
 
 int launch_gemv_q4k_f32(const cml_weight *w, const float *x, float *out, hipStream_t st);  // quantize + matvec, one token
 int launch_gemv_b32_f32(const cml_weight *w, const float *x, float *out, hipStream_t st);  // Q8_0 / Q4_0: quantize + matvec, one token
-// Q8_0 / Q4_0 grouped (mixture-of-experts) matvec; x non-null = one f32 token quantized in the kernel
-int launch_gemv_b32_grouped(const MatArgs &a, const float *x, hipStream_t st);
+// Where a grouped matvec takes its activation rows from instead of MatArgs::q / scales:
+//   kind 1: ONE f32 token x, quantized inside the kernel, read by every assignment
+//   kind 2 / 3: assignment j's row is silu / gelu_tanh of x[j] times u[j] (f32 rows `stride` apart), quantized in the kernel
+struct GroupedPrologue {
+    int kind = 0;
+    const float *x = nullptr;
+    const float *u = nullptr;
+    int64_t stride = 0;
+};
+// Q8_0 / Q4_0 grouped (mixture-of-experts) matvec
+int launch_gemv_b32_grouped(const MatArgs &a, const GroupedPrologue &pro, hipStream_t st);
 int launch_gemv_q8_0(const MatArgs &a, hipStream_t st);
 int launch_gemv_q4_0(const MatArgs &a, hipStream_t st);
 int launch_gemv_q6k(const MatArgs &a, hipStream_t st);

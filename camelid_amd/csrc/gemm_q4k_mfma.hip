@@ -67,6 +67,7 @@ struct Q4KMfmaArgs {
     // reads activation row group_rows[j] (j itself when null) and writes output row j.
     const int32_t *group_offsets;
     const int32_t *group_rows;
+    const int32_t *group_ids;  // z-slot -> group (-1: unused slot), or null (the z-slot is the group)
 };
 
 struct MfmaWeights {
@@ -123,7 +124,8 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
     const int tile = blockIdx.x * RT + rt;
     const int row = tile * 16 + n - a.row_skip;
     const bool grouped = a.group_offsets != nullptr;
-    const int64_t band = grouped ? blockIdx.z : 0;
+    const int64_t band = grouped ? (a.group_ids ? a.group_ids[blockIdx.z] : static_cast<int>(blockIdx.z)) : 0;
+    if (band < 0) return;  // a z-slot past the groups in use
     const int a0 = grouped ? a.group_offsets[band] : 0;                      // first assignment of this group
     const int n_assign = grouped ? a.group_offsets[band + 1] - a0 : a.n_tokens;
     const int tok0 = blockIdx.y * NTOK;                    // first token (assignment of the group) of this workgroup
@@ -359,7 +361,8 @@ int launch_gemm_q4k_mfma(const MatArgs &a, hipStream_t st) {
     ka.n_tokens = static_cast<int>(a.n_tokens);
     ka.group_offsets = a.group_offsets;
     ka.group_rows = a.group_rows;
-    const int ng = grouped ? a.n_groups : 1;
+    ka.group_ids = a.group_ids;
+    const int ng = grouped ? (a.group_ids ? a.max_active : a.n_groups) : 1;
     // Workgroup shape: tokens staged per workgroup x how they are split over waves.  Default: one
     // wave per row tile, 16 / 32 / 64 tokens per workgroup by batch size; more tokens = more
     // workgroup columns (grid.y), each a pass over the weight.  The other shapes stay selectable

@@ -68,6 +68,7 @@ struct Q4KArgs {
     // serves its assignments in passes of NT.
     const int32_t *group_offsets;
     const int32_t *group_rows;
+    const int32_t *group_ids;  // y-slot -> group (-1: unused slot), or null (the y-slot is the group)
     // Pair launch (gridDim.z == 2): blockIdx.z = 1 works on a second weight of the same shape
     // against the same activations and writes out2 (gate and up projections in one launch).
     const uint8_t *w2;
@@ -206,7 +207,8 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
     const int tid = threadIdx.x;
     const int nthreads = blockDim.x;
     const bool grouped = a.group_offsets != nullptr;
-    const int64_t band = grouped ? blockIdx.y : 0;
+    const int64_t band = grouped ? (a.group_ids ? a.group_ids[blockIdx.y] : static_cast<int>(blockIdx.y)) : 0;
+    if (band < 0) return;  // a y-slot past the groups in use
     const int a0 = grouped ? a.group_offsets[band] : 0;               // first assignment of this group
     const int n_assign = grouped ? a.group_offsets[band + 1] - a0 : NT;
     if (n_assign <= 0) return;  // an expert nobody routed to: the whole workgroup leaves
@@ -490,6 +492,7 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
     ka.out = a.out;
     ka.group_offsets = a.group_offsets;
     ka.group_rows = a.group_rows;
+    ka.group_ids = a.group_ids;
     if (w2) {
         if (w2->fmt != w->fmt || w2->rows != w->rows || w2->nb != w->nb || w2->row_skip != w->row_skip ||
             w2->planes.row_stride[0] != w->planes.row_stride[0])
@@ -509,7 +512,7 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
     if (lds > 64 * 1024) return fail(CML_ERR_UNSUPPORTED, "Q4_K activation of %d super-blocks exceeds the LDS staging limit", ka.n_sb);
     ka.ksplit = shape.ksplit;
     ka.tiles_per_wg = shape.tiles_per_wg;
-    const dim3 grid(gx, grouped ? a.n_groups : 1, w2 ? 2 : 1);
+    const dim3 grid(gx, grouped ? (a.group_ids ? a.max_active : a.n_groups) : 1, w2 ? 2 : 1);
     hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true>), grid, dim3(64 * waves), lds, st, ka);
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
@@ -545,6 +548,7 @@ int launch_gemv_q4k(const MatArgs &a, hipStream_t st) {
     ka.ints = a.ints;
     ka.group_offsets = a.group_offsets;
     ka.group_rows = a.group_rows;
+    ka.group_ids = a.group_ids;
     const Q4KShape shape = pick_shape(ka.rows, ka.n_sb);
     if (grouped) {
         // One launch: every group walks its own assignments in passes of NT
@@ -553,7 +557,7 @@ int launch_gemv_q4k(const MatArgs &a, hipStream_t st) {
         ka.yd = a.scales;
         ka.out = a.out;
         const int nt = cap_nt(a.n_tokens, ka.n_sb, shape.ksplit * shape.tiles_per_wg);
-        return launch_q4k_pick_nt(ka, shape, a.n_groups, nt, false, st);
+        return launch_q4k_pick_nt(ka, shape, a.group_ids ? a.max_active : a.n_groups, nt, false, st);
     }
     // Plain call: tokens are served in launches of up to 8 activation rows.
     int64_t t0 = 0;

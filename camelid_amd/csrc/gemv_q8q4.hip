@@ -19,6 +19,7 @@
 #include "cml_device.hpp"
 #include "cml_host.hpp"
 
+#include <algorithm>
 #include <type_traits>
 
 #pragma clang fp contract(off)
@@ -43,22 +44,22 @@ struct B32Args {
     int64_t out_slot_stride;
 };
 
-template <int FMT>
+template <int FMT, int UU = 2>
 struct B32Regs {
-    static constexpr int U = 2;  // steps in flight per buffer
+    static constexpr int U = UU;  // steps in flight per buffer
     uint4 qa[U];
     uint4 qb[U];  // Q8_0 only
     uint32_t d[U];
 };
 
-template <int FMT, int P>
-__device__ __forceinline__ void b32_load(B32Regs<FMT> &r, const uint8_t *qrow, const uint8_t *srow, int l,
+template <int FMT, int P, int U>
+__device__ __forceinline__ void b32_load(B32Regs<FMT, U> &r, const uint8_t *qrow, const uint8_t *srow, int l,
                                          int step, int n_steps, int nb) {
     // Unconditional, clamped loads: steps or lanes past the row end re-read the
     // last block and their term is dropped by the caller.  Straight-line code
     // keeps the next buffer's loads in flight under the current arithmetic.
 #pragma unroll
-    for (int u = 0; u < B32Regs<FMT>::U; u++) {
+    for (int u = 0; u < U; u++) {
         const int b = min(min(step + u, n_steps - 1) * P + l, nb - 1);
         if constexpr (FMT == CML_Q8_0) {
             r.qa[u] = ldg16(qrow + static_cast<int64_t>(b) * 32);
@@ -70,12 +71,12 @@ __device__ __forceinline__ void b32_load(B32Regs<FMT> &r, const uint8_t *qrow, c
     }
 }
 
-template <int FMT, int P, int NT, bool INTS>
-__device__ __forceinline__ void b32_compute(const B32Regs<FMT> &r, int l, int step, int n_steps, int nb,
+template <int FMT, int P, int NT, bool INTS, int U>
+__device__ __forceinline__ void b32_compute(const B32Regs<FMT, U> &r, int l, int step, int n_steps, int nb,
                                             const int8_t *ys, const int *bsum, const float *xss, float (&acc)[NT],
                                             int32_t *ints_row) {
 #pragma unroll
-    for (int u = 0; u < B32Regs<FMT>::U; u++) {
+    for (int u = 0; u < U; u++) {
         const int b_raw = (step + u) * P + l;
         const bool valid = (step + u < n_steps) && (b_raw < nb);
         const int b = min(min(step + u, n_steps - 1) * P + l, nb - 1);
@@ -110,52 +111,32 @@ __device__ __forceinline__ void b32_compute(const B32Regs<FMT> &r, int l, int st
 
 // One pass over a row's blocks for NT staged activation rows: two register buffers alternate,
 // the last one is consumed without issuing further loads.
-template <int FMT, int P, int NT, bool INTS>
+template <int FMT, int P, int NT, bool INTS, int U = 2>
 __device__ __forceinline__ void b32_row_pass(const uint8_t *qrow, const uint8_t *srow, int l, int nb, const int8_t *ys,
                                              const int *bsum, const float *xss, float (&acc)[NT], int32_t *ints_row) {
-    constexpr int U = B32Regs<FMT>::U;
     const int n_steps = (nb + P - 1) / P;
-    B32Regs<FMT> ra, rb;
-    b32_load<FMT, P>(ra, qrow, srow, l, 0, n_steps, nb);
+    B32Regs<FMT, U> ra, rb;
+    b32_load<FMT, P, U>(ra, qrow, srow, l, 0, n_steps, nb);
     __builtin_amdgcn_sched_barrier(0);
     for (int step = 0;;) {
         if (step + U >= n_steps) {
-            b32_compute<FMT, P, NT, INTS>(ra, l, step, n_steps, nb, ys, bsum, xss, acc, ints_row);
+            b32_compute<FMT, P, NT, INTS, U>(ra, l, step, n_steps, nb, ys, bsum, xss, acc, ints_row);
             break;
         }
-        b32_load<FMT, P>(rb, qrow, srow, l, step + U, n_steps, nb);
+        b32_load<FMT, P, U>(rb, qrow, srow, l, step + U, n_steps, nb);
         __builtin_amdgcn_sched_barrier(0);
-        b32_compute<FMT, P, NT, INTS>(ra, l, step, n_steps, nb, ys, bsum, xss, acc, ints_row);
+        b32_compute<FMT, P, NT, INTS, U>(ra, l, step, n_steps, nb, ys, bsum, xss, acc, ints_row);
         __builtin_amdgcn_sched_barrier(0);
         step += U;
         if (step + U >= n_steps) {
-            b32_compute<FMT, P, NT, INTS>(rb, l, step, n_steps, nb, ys, bsum, xss, acc, ints_row);
+            b32_compute<FMT, P, NT, INTS, U>(rb, l, step, n_steps, nb, ys, bsum, xss, acc, ints_row);
             break;
         }
-        b32_load<FMT, P>(ra, qrow, srow, l, step + U, n_steps, nb);
+        b32_load<FMT, P, U>(ra, qrow, srow, l, step + U, n_steps, nb);
         __builtin_amdgcn_sched_barrier(0);
-        b32_compute<FMT, P, NT, INTS>(rb, l, step, n_steps, nb, ys, bsum, xss, acc, ints_row);
+        b32_compute<FMT, P, NT, INTS, U>(rb, l, step, n_steps, nb, ys, bsum, xss, acc, ints_row);
         __builtin_amdgcn_sched_barrier(0);
         step += U;
-    }
-}
-
-// Quantize one f32 row of nb blocks to Q8_0 straight into the LDS staging area, eight lanes per
-// block: the arithmetic of quantize_q8_0_kernel without the launch and the round trip.
-template <int FMT>
-__device__ __forceinline__ void b32_stage_quantized(const float *x, int nb, int tid, int8_t *ys, float *xss, int *bsum) {
-    const float4 *x4 = reinterpret_cast<const float4 *>(x);
-    uint32_t *ys32 = reinterpret_cast<uint32_t *>(ys);
-    const int n4 = nb * 8;  // a multiple of 8: the eight lanes of a block enter and leave together
-    for (int i = tid; i < n4; i += 256) {
-        float scale;
-        const uint32_t packed = q8_0_quantize_lane8(x4[i], scale);
-        ys32[i] = packed;
-        if ((i & 7) == 0) xss[i >> 3] = scale;
-        if constexpr (FMT == CML_Q4_0) {
-            const int s = group_sum_to_last<8>(sdot4(packed, 0x01010101u, 0));
-            if ((i & 7) == 7) bsum[i >> 3] = s;
-        }
     }
 }
 
@@ -180,7 +161,8 @@ __global__ __launch_bounds__(256) void gemv_b32_kernel(B32Args a) {
     float *out = a.out + static_cast<int64_t>(slot) * a.out_slot_stride;
 
     if constexpr (FUSEQ) {
-        b32_stage_quantized<FMT>(a.x, nb, tid, ys, xss, bsum);
+        const float4 *x4 = reinterpret_cast<const float4 *>(a.x);
+        b32_stage_quantized_from<FMT>([&](int i) { return x4[i]; }, nb, tid, ys, xss, bsum);
     } else {
         const uint4 *src = reinterpret_cast<const uint4 *>(q);
         uint4 *dst = reinterpret_cast<uint4 *>(ys);
@@ -308,12 +290,19 @@ int launch_gemv_b32_f32(const cml_weight *w, const float *x, float *out, hipStre
 }
 
 // ---- grouped (mixture-of-experts) dispatch ------------------------------------------------------
-// blockIdx.y = group (expert) e: the band of rows [e*rows, (e+1)*rows) of the stacked weight dotted
-// with the activation rows of the assignments [group_offsets[e], group_offsets[e+1]).  The group's
-// assignments are staged NTMAX at a time; a chunk of 1, 2, 3-4 or 5-8 runs the 1-, 2-, 4- or
-// 8-token row pass (slots past the chunk repeat its last row and are not written).  Every cell is
+// blockIdx.y = y-slot.  With group_offsets: the slot serves group (expert) e = group_ids[y] (y
+// itself when group_ids is null; -1 = unused slot): the band of rows [e*rows, (e+1)*rows) of the
+// stacked weight dotted with the activation rows of the assignments [group_offsets[e],
+// group_offsets[e+1]).  Without group_offsets (single-token decode): y-slot y IS assignment y and
+// group_ids[y] its expert; ids outside [0, n_groups) are skipped.
+// A group's assignments are staged NTMAX at a time; a chunk of 1, 2 or 3-4 runs the 1-, 2- or
+// 4-token row pass (slots past the chunk repeat its last row and are not written).  Every cell is
 // the single-row chain of the plain kernel: bit-identical to it.
-// FUSEQ: one token, f32, quantized inside every workgroup; every assignment reads it.
+// PRO selects where the staged activation comes from:
+//   0  quantized rows q / xs (row group_rows[j], or j)
+//   1  ONE f32 token x, quantized to Q8_0 inside every workgroup; every assignment reads it
+//   2  assignment j's row is silu(x[j]) * u[j] (f32 rows x_stride apart), quantized in the workgroup
+//   3  the same with gelu_tanh
 struct B32GroupArgs {
     const uint8_t *quants;
     int64_t q_stride;
@@ -321,17 +310,39 @@ struct B32GroupArgs {
     int64_t s_stride;
     int rows;  // rows of one band
     int nb;
+    int n_groups;
     const int8_t *q;  // [activation rows][nb*32]
     const float *xs;  // [activation rows][nb]
-    const float *x;   // FUSEQ: the f32 token
+    const float *x;   // PRO 1: the f32 token; PRO 2, 3: gate rows
+    const float *u;   // PRO 2, 3: up rows
+    int64_t x_stride;
     float *out;       // [assignments][rows]
     const int32_t *group_offsets;
     const int32_t *group_rows;  // assignment -> activation row, or null (the assignment itself)
+    const int32_t *group_ids;
 };
 
-template <int FMT, int P, int NTMAX, bool FUSEQ>
+// Quantize one row of nb blocks to Q8_0 straight into the LDS staging area, eight lanes per block;
+// value4(i) yields the row's i-th float4.
+template <int FMT, typename F>
+__device__ __forceinline__ void b32_stage_quantized_from(F value4, int nb, int tid, int8_t *ys, float *xss, int *bsum) {
+    uint32_t *ys32 = reinterpret_cast<uint32_t *>(ys);
+    const int n4 = nb * 8;  // a multiple of 8: the eight lanes of a block enter and leave together
+    for (int i = tid; i < n4; i += 256) {
+        float scale;
+        const uint32_t packed = q8_0_quantize_lane8(value4(i), scale);
+        ys32[i] = packed;
+        if ((i & 7) == 0) xss[i >> 3] = scale;
+        if constexpr (FMT == CML_Q4_0) {
+            const int s = group_sum_to_last<8>(sdot4(packed, 0x01010101u, 0));
+            if ((i & 7) == 7) bsum[i >> 3] = s;
+        }
+    }
+}
+
+template <int FMT, int P, int NTMAX, int PRO, int U>
 __global__ __launch_bounds__(256) void gemv_b32_grouped_kernel(B32GroupArgs a) {
-    static_assert(!FUSEQ || NTMAX == 1, "the fused quantizer serves single-token calls");
+    static_assert(PRO == 0 || NTMAX == 1, "the fused prologues stage one activation row at a time");
     constexpr int RPW = kWave / P;
     extern __shared__ uint4 smem[];
     const int nb = a.nb;
@@ -340,10 +351,18 @@ __global__ __launch_bounds__(256) void gemv_b32_grouped_kernel(B32GroupArgs a) {
     int *bsum = reinterpret_cast<int *>(xss + NTMAX * nb);         // [NTMAX][nb] (Q4_0)
 
     const int tid = threadIdx.x;
-    const int g = blockIdx.y;
-    const int a0 = a.group_offsets[g];
-    const int cnt = a.group_offsets[g + 1] - a0;
-    if (cnt <= 0) return;  // the whole workgroup leaves together
+    int g, a0, cnt;
+    if (a.group_offsets) {
+        g = a.group_ids ? a.group_ids[blockIdx.y] : static_cast<int>(blockIdx.y);
+        if (g < 0 || g >= a.n_groups) return;  // the whole workgroup leaves together
+        a0 = a.group_offsets[g];
+        cnt = a.group_offsets[g + 1] - a0;
+    } else {
+        g = a.group_ids[blockIdx.y];
+        a0 = blockIdx.y;
+        cnt = 1;
+    }
+    if (g < 0 || g >= a.n_groups || cnt <= 0) return;
 
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int r = lane / P, l = lane - r * P;
@@ -353,15 +372,21 @@ __global__ __launch_bounds__(256) void gemv_b32_grouped_kernel(B32GroupArgs a) {
     const uint8_t *qrow = a.quants + arow * a.q_stride;
     const uint8_t *srow = a.scales + arow * a.s_stride;
     const bool leader = (l == P - 1);
+    const int n_steps = (nb + P - 1) / P;
 
-    for (int c0 = 0; c0 < cnt; c0 += NTMAX) {
-        const int nt = min(NTMAX, cnt - c0);
-        if constexpr (FUSEQ) {
-            if (c0 == 0) b32_stage_quantized<FMT>(a.x, nb, tid, ys, xss, bsum);
+    // Stage the activation rows of assignments a0+c0 .. (nt of them, `staged` slots filled).
+    auto stage = [&](int c0, int nt, int staged) {
+        if constexpr (PRO == 1) {
+            if (c0 == 0) {
+                const float4 *x4 = reinterpret_cast<const float4 *>(a.x);
+                b32_stage_quantized_from<FMT>([&](int i) { return x4[i]; }, nb, tid, ys, xss, bsum);
+            }
+        } else if constexpr (PRO >= 2) {
+            const float4 *g4 = reinterpret_cast<const float4 *>(a.x + static_cast<int64_t>(a0 + c0) * a.x_stride);
+            const float4 *u4 = reinterpret_cast<const float4 *>(a.u + static_cast<int64_t>(a0 + c0) * a.x_stride);
+            b32_stage_quantized_from<FMT>([&](int i) { return glu4<PRO - 2>(g4[i], u4[i]); }, nb, tid, ys, xss, bsum);
         } else {
-            if (c0 > 0) __syncthreads();  // the previous chunk's readers are done
-            const int per_t = nb * 2;     // 16-byte pieces per activation row (even)
-            const int staged = (nt <= 1 ? 1 : nt <= 2 ? 2 : nt <= 4 ? 4 : 8);
+            const int per_t = nb * 2;  // 16-byte pieces per activation row (even)
             uint4 *dst = reinterpret_cast<uint4 *>(ys);
             for (int i = tid; i < staged * per_t; i += 256) {
                 const int t = i / per_t, j = i - t * per_t;
@@ -382,6 +407,12 @@ __global__ __launch_bounds__(256) void gemv_b32_grouped_kernel(B32GroupArgs a) {
                 xss[i] = a.xs[src_row * nb + j];
             }
         }
+    };
+
+    for (int c0 = 0; c0 < cnt; c0 += NTMAX) {
+        const int nt = min(NTMAX, cnt - c0);
+        if (c0 > 0 && PRO != 1) __syncthreads();  // the previous chunk's readers are done
+        stage(c0, nt, nt <= 1 ? 1 : (nt <= 2 ? 2 : 4));
         __syncthreads();
         float *out = a.out + static_cast<int64_t>(a0 + c0) * a.rows + row;
         auto run = [&](auto nt_tag) {
@@ -389,7 +420,7 @@ __global__ __launch_bounds__(256) void gemv_b32_grouped_kernel(B32GroupArgs a) {
             float acc[NT];
 #pragma unroll
             for (int t = 0; t < NT; t++) acc[t] = 0.0f;
-            b32_row_pass<FMT, P, NT, false>(qrow, srow, l, nb, ys, bsum, xss, acc, nullptr);
+            b32_row_pass<FMT, P, NT, false, U>(qrow, srow, l, nb, ys, bsum, xss, acc, nullptr);
             if (leader && live) {
 #pragma unroll
                 for (int t = 0; t < NT; t++)
@@ -399,16 +430,16 @@ __global__ __launch_bounds__(256) void gemv_b32_grouped_kernel(B32GroupArgs a) {
         if constexpr (NTMAX == 1) {
             run(std::integral_constant<int, 1>{});
         } else {
+            static_assert(NTMAX == 4, "chunk sizes 1, 2, 4");
             if (nt <= 1) run(std::integral_constant<int, 1>{});
             else if (nt <= 2) run(std::integral_constant<int, 2>{});
-            else if (nt <= 4) run(std::integral_constant<int, 4>{});
-            else run(std::integral_constant<int, 8>{});
+            else run(std::integral_constant<int, 4>{});
         }
     }
 }
 
-template <int FMT, int P>
-static int launch_b32_grouped_p(const MatArgs &a, const float *x, hipStream_t st) {
+template <int FMT, int P, int U>
+static int launch_b32_grouped_u(const MatArgs &a, const GroupedPrologue &pro, hipStream_t st) {
     const cml_weight *w = a.w;
     B32GroupArgs ga{};
     ga.quants = w->planes.p[0];
@@ -417,45 +448,67 @@ static int launch_b32_grouped_p(const MatArgs &a, const float *x, hipStream_t st
     ga.s_stride = w->planes.row_stride[1];
     ga.rows = static_cast<int>(a.band_rows);
     ga.nb = static_cast<int>(w->nb);
+    ga.n_groups = a.n_groups;
     ga.q = a.q;
     ga.xs = a.scales;
-    ga.x = x;
+    ga.x = pro.x;
+    ga.u = pro.u;
+    ga.x_stride = pro.stride;
     ga.out = a.out;
     ga.group_offsets = a.group_offsets;
     ga.group_rows = a.group_rows;
+    ga.group_ids = a.group_ids;
     const int rows_per_wg = 4 * (64 / P);
-    const dim3 grid(static_cast<unsigned>((ga.rows + rows_per_wg - 1) / rows_per_wg), static_cast<unsigned>(a.n_groups));
-    const bool one = x != nullptr || a.n_tokens <= 1;
-    const size_t lds = static_cast<size_t>(one ? 1 : 8) * ga.nb * (32 + 4 + 4);
+    const int slots = a.group_ids ? a.max_active : a.n_groups;
+    const dim3 grid(static_cast<unsigned>((ga.rows + rows_per_wg - 1) / rows_per_wg), static_cast<unsigned>(slots));
+    const bool one = pro.kind != 0 || a.n_tokens <= 1;
+    const size_t lds = static_cast<size_t>(one ? 1 : 4) * ga.nb * (32 + 4 + 4);
     if (lds > 64 * 1024) return fail(CML_ERR_UNSUPPORTED, "activation of %d blocks exceeds the LDS staging limit", ga.nb);
-    if (x)
-        hipLaunchKernelGGL((gemv_b32_grouped_kernel<FMT, P, 1, true>), grid, dim3(256), lds, st, ga);
-    else if (one)
-        hipLaunchKernelGGL((gemv_b32_grouped_kernel<FMT, P, 1, false>), grid, dim3(256), lds, st, ga);
-    else
-        hipLaunchKernelGGL((gemv_b32_grouped_kernel<FMT, P, 8, false>), grid, dim3(256), lds, st, ga);
+    switch (pro.kind) {
+        case 1: hipLaunchKernelGGL((gemv_b32_grouped_kernel<FMT, P, 1, 1, U>), grid, dim3(256), lds, st, ga); break;
+        case 2: hipLaunchKernelGGL((gemv_b32_grouped_kernel<FMT, P, 1, 2, U>), grid, dim3(256), lds, st, ga); break;
+        case 3: hipLaunchKernelGGL((gemv_b32_grouped_kernel<FMT, P, 1, 3, U>), grid, dim3(256), lds, st, ga); break;
+        default:
+            if (one) hipLaunchKernelGGL((gemv_b32_grouped_kernel<FMT, P, 1, 0, U>), grid, dim3(256), lds, st, ga);
+            else hipLaunchKernelGGL((gemv_b32_grouped_kernel<FMT, P, 4, 0, U>), grid, dim3(256), lds, st, ga);
+            break;
+    }
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }
 
-// x non-null: one f32 token that every assignment reads, quantized inside the kernel (a.q and
-// a.scales unused).
-int launch_gemv_b32_grouped(const MatArgs &a, const float *x, hipStream_t st) {
+template <int FMT, int P>
+static int launch_b32_grouped_p(const MatArgs &a, const GroupedPrologue &pro, hipStream_t st) {
+    return launch_b32_grouped_u<FMT, P, 2>(a, pro, st);  // 2 steps in flight per register buffer (4 measured slower)
+}
+
+int launch_gemv_b32_grouped(const MatArgs &a, const GroupedPrologue &pro, hipStream_t st) {
     const cml_weight *w = a.w;
     if (a.band_rows <= 0 || a.n_groups <= 0 || a.n_tokens <= 0) return CML_OK;
     if (w->fmt != CML_Q8_0 && w->fmt != CML_Q4_0) return fail(CML_ERR_UNSUPPORTED, "not a 32-value block format");
     if (a.band_rows * a.n_groups != w->rows) return fail(CML_ERR_SHAPE, "%d bands of %lld rows do not cover %lld rows", a.n_groups, (long long)a.band_rows, (long long)w->rows);
+    if (!a.group_offsets && !a.group_ids) return fail(CML_ERR_INVALID, "grouped call without groups");
+    if (pro.kind < 0 || pro.kind > 3 || (pro.kind != 0 && !pro.x) || (pro.kind >= 2 && !pro.u)) return fail(CML_ERR_INVALID, "bad prologue");
     const bool q8 = w->fmt == CML_Q8_0;
-    int p = env_int(q8 ? "CAMELID_HIP_Q8_0_LANES" : "CAMELID_HIP_Q4_0_LANES", 0);
-    if (p != 8 && p != 16) p = (w->nb <= 8) ? 8 : 16;
-    if (q8) return p == 8 ? launch_b32_grouped_p<CML_Q8_0, 8>(a, x, st) : launch_b32_grouped_p<CML_Q8_0, 16>(a, x, st);
-    return p == 8 ? launch_b32_grouped_p<CML_Q4_0, 8>(a, x, st) : launch_b32_grouped_p<CML_Q4_0, 16>(a, x, st);
+    // Lanes per row.  Batched calls: 4, so that a workgroup covers 64 rows -- the per-workgroup
+    // chain (group lookup, activation staging, barrier) is then paid once per 64 rows instead of
+    // once per 16, which is what bounds many small expert bands.  Single-token calls: 16, or 8 for
+    // rows of up to 32 blocks so that a step's lanes are not mostly idle.
+    int p = env_int(q8 ? "CAMELID_HIP_Q8_0_GROUPED_LANES" : "CAMELID_HIP_Q4_0_GROUPED_LANES", 0);
+    const bool single = pro.kind != 0 || a.n_tokens <= 1;
+    if (p != 4 && p != 8 && p != 16) p = !single ? 4 : (w->nb <= 8 ? 4 : (w->nb <= 32 ? 8 : 16));
+    if (q8) {
+        if (p == 4) return launch_b32_grouped_p<CML_Q8_0, 4>(a, pro, st);
+        return p == 8 ? launch_b32_grouped_p<CML_Q8_0, 8>(a, pro, st) : launch_b32_grouped_p<CML_Q8_0, 16>(a, pro, st);
+    }
+    if (p == 4) return launch_b32_grouped_p<CML_Q4_0, 4>(a, pro, st);
+    return p == 8 ? launch_b32_grouped_p<CML_Q4_0, 8>(a, pro, st) : launch_b32_grouped_p<CML_Q4_0, 16>(a, pro, st);
 }
 
 template <int FMT>
 static int launch_b32(const MatArgs &a, hipStream_t st) {
     if (a.w->rows == 0 || a.n_tokens == 0) return CML_OK;
-    if (a.group_offsets) return launch_gemv_b32_grouped(a, nullptr, st);
+    if (a.group_offsets) return launch_gemv_b32_grouped(a, GroupedPrologue{}, st);
     // 16 lanes per row by default; 8 when rows are short enough that half the lanes would idle.
     int p = env_int(FMT == CML_Q8_0 ? "CAMELID_HIP_Q8_0_LANES" : "CAMELID_HIP_Q4_0_LANES", 0);
     if (p != 8 && p != 16) p = (a.w->nb <= 8) ? 8 : 16;

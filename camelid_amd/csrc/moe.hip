@@ -14,6 +14,8 @@
 #include "cml_device.hpp"
 #include "cml_host.hpp"
 
+#include <algorithm>
+
 #pragma clang fp contract(off)
 
 namespace cml {
@@ -88,84 +90,155 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const float *__restrict__
     }
 }
 
-// One thread per token.  Gemma-4 routing (reference moe_layer_ffn, src/gemma4_runtime.rs:5567-5610;
-// router_top_k, :61-84): softmax over ALL experts (max folded from f32::MIN, exp(v - max), sum in
-// index order, p /= sum), top-k by probability (descending, ties to the lower index), then
+// Maximum over the 64 lanes of a wave, returned in every lane (all lanes must be active).
+__device__ __forceinline__ int wave_allmax_i32(int v) {
+    v = max(v, row_ror_i32<1>(v));
+    v = max(v, row_ror_i32<2>(v));
+    v = max(v, row_ror_i32<4>(v));
+    v = max(v, row_ror_i32<8>(v));
+    return max(max(__builtin_amdgcn_readlane(v, 0), __builtin_amdgcn_readlane(v, 16)),
+               max(__builtin_amdgcn_readlane(v, 32), __builtin_amdgcn_readlane(v, 48)));
+}
+
+// One wave per token, lane l holding experts l and l + 64.  Gemma-4 routing (reference
+// moe_layer_ffn, src/gemma4_runtime.rs:5567-5610; router_top_k, :61-84): softmax over ALL experts
+// (max folded from f32::MIN, exp(v - max), sum left to right in index order, p /= sum), top-k by
+// probability (descending, ties to the lower index), then
 // scale[s] = down_scale[e] * (p[e] / max(sum of the selected p in selection order, 6.103515e-5)).
-__global__ __launch_bounds__(64) void moe_route_softmax_kernel(const float *__restrict__ logits, int64_t n_tokens, int n_experts,
-                                                               int k, const float *__restrict__ down_scale,
-                                                               int32_t *__restrict__ idx_out, float *__restrict__ w_out) {
-    const int64_t t = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-    if (t >= n_tokens) return;
+// The two sums are sequential chains, run redundantly in every lane; the rest is per lane plus
+// one wave-wide maximum per selected expert.
+__global__ __launch_bounds__(256) void moe_route_softmax_kernel(const float *__restrict__ logits, int64_t n_tokens, int n_experts,
+                                                                int k, const float *__restrict__ down_scale,
+                                                                int32_t *__restrict__ idx_out, float *__restrict__ w_out) {
+    __shared__ float ps[4][kMaxExperts];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int64_t t_raw = static_cast<int64_t>(blockIdx.x) * 4 + wave;
+    const bool live = t_raw < n_tokens;
+    const int64_t t = live ? t_raw : n_tokens - 1;  // spare waves repeat the last token and store nothing
     const float *lg = logits + t * n_experts;
-    float p[kMaxExperts];
-    int sel[kMaxExperts];
-    float maxl = -3.4028235e38f;
-    for (int e = 0; e < n_experts; e++) maxl = fmaxf(maxl, lg[e]);
+    const bool has0 = lane < n_experts, has1 = lane + 64 < n_experts;
+    const float kLowest = -3.4028235e38f;
+    const float l0 = has0 ? lg[lane] : kLowest, l1 = has1 ? lg[lane + 64] : kLowest;
+    // The maximum does not depend on the order.  fmaxf drops NaNs as f32::max does; total_key
+    // orders floats like the floats and is its own inverse.
+    const int mkey = wave_allmax_i32(total_key(fmaxf(fmaxf(l0, l1), kLowest)));
+    const float maxl = __builtin_bit_cast(float, mkey ^ static_cast<int>(static_cast<unsigned>(mkey >> 31) >> 1));
+    float p0 = has0 ? expf(l0 - maxl) : 0.0f, p1 = has1 ? expf(l1 - maxl) : 0.0f;
+    ps[wave][lane] = p0;
+    ps[wave][lane + 64] = p1;
+    __syncthreads();
     float sum = 0.0f;
-    for (int e = 0; e < n_experts; e++) {
-        p[e] = expf(lg[e] - maxl);
-        sum = sum + p[e];
-    }
-    for (int e = 0; e < n_experts; e++) p[e] = p[e] / sum;
-    int len = 0;
-    for (int c = 0; c < n_experts; c++) {
-        int at = -1;
-        for (int j = 0; j < len; j++) {
-            const int cur = sel[j];
-            if (p[cur] < p[c] || (p[cur] == p[c] && c < cur)) {
-                at = j;
-                break;
+#pragma unroll 8
+    for (int e = 0; e < n_experts; e++) sum = sum + ps[wave][e];
+    p0 = p0 / sum;
+    p1 = p1 / sum;
+    // selection: probabilities are >= 0, so their bit patterns order like the values; -1 = not a candidate
+    int c0 = has0 ? __builtin_bit_cast(int, p0) : -1, c1 = has1 ? __builtin_bit_cast(int, p1) : -1;
+    int se0 = 0, se1 = 0;       // lane s holds the s-th selected expert (se1: the (s + 64)-th)
+    float sp0 = 0.0f, sp1 = 0.0f;
+    float wsum = 0.0f;
+    for (int s = 0; s < k; s++) {
+        const int m = wave_allmax_i32(max(c0, c1));
+        const unsigned long long b0 = __builtin_amdgcn_ballot_w64(c0 == m), b1 = __builtin_amdgcn_ballot_w64(c1 == m);
+        const int e = b0 ? __builtin_ctzll(b0) : (b1 ? 64 + __builtin_ctzll(b1) : 0);
+        const float pm = __builtin_bit_cast(float, m);
+        if (e == lane) c0 = -1;
+        if (e == lane + 64) c1 = -1;
+        if (lane == (s & 63)) {
+            if (s < 64) {
+                se0 = e;
+                sp0 = pm;
+            } else {
+                se1 = e;
+                sp1 = pm;
             }
         }
-        if (at >= 0) {
-            const int last = len < k ? len : k - 1;
-            for (int j = last; j > at; j--) sel[j] = sel[j - 1];
-            sel[at] = c;
-            if (len < k) len++;
-        } else if (len < k) {
-            sel[len++] = c;
-        }
+        wsum = wsum + pm;
     }
-    float wsum = 0.0f;
-    for (int s = 0; s < k; s++) wsum = wsum + p[sel[s]];
     wsum = fmaxf(wsum, 6.103515e-5f);
-    for (int s = 0; s < k; s++) {
-        const int e = sel[s];
-        const float ds = down_scale ? down_scale[e] : 1.0f;
-        idx_out[t * k + s] = e;
-        w_out[t * k + s] = ds * (p[e] / wsum);
+    if (live && lane < k) {
+        const float ds = down_scale ? down_scale[se0] : 1.0f;
+        idx_out[t * k + lane] = se0;
+        w_out[t * k + lane] = ds * (sp0 / wsum);
+    }
+    if (live && lane + 64 < k) {
+        const float ds = down_scale ? down_scale[se1] : 1.0f;
+        idx_out[t * k + lane + 64] = se1;
+        w_out[t * k + lane + 64] = ds * (sp1 / wsum);
     }
 }
 
-// Group the n_tokens*k assignments by expert, keeping (token, rank) order
-// inside each group.  One workgroup; thread e builds group e.
+// Group the n_tokens*k assignments by expert, keeping (token, rank) order inside each group (a
+// stable counting sort).  One workgroup of 256 threads, one routed slot per thread and pass:
 //   offsets[e..e+1)   assignment range of expert e
 //   assign_token[j]   token whose activation assignment j reads
-//   slot_to_assign[t*k+s]  where (token t, rank s) landed
-__global__ __launch_bounds__(kMaxExperts) void moe_plan_kernel(const int32_t *__restrict__ idx, int n_slots, int n_experts, int k,
-                                                      int32_t *__restrict__ offsets, int32_t *__restrict__ assign_token,
-                                                      int32_t *__restrict__ slot_to_assign) {
-    __shared__ int count[kMaxExperts + 1];
-    const int e = threadIdx.x;
-    int mine = 0;
-    if (e < n_experts) {
-        for (int i = 0; i < n_slots; i++) mine += (idx[i] == e);
-        count[e] = mine;
+//   slot_to_assign[t*k+s]  where (token t, rank s) landed (-1: expert id out of range, slot dropped)
+//   group_ids[y]      the experts that received assignments, ascending, then -1
+// A slot's place = start of its expert's range + the slots of that expert before it: those of
+// earlier passes (base), of earlier waves of this pass (wave_cnt), and of lower lanes of its own
+// wave (a match mask built from 64 lane reads).
+constexpr int kPlanThreads = 256;
+__global__ __launch_bounds__(kPlanThreads) void moe_plan_kernel(const int32_t *__restrict__ idx, int n_slots, int n_experts, int k,
+                                                                int32_t *__restrict__ offsets, int32_t *__restrict__ assign_token,
+                                                                int32_t *__restrict__ slot_to_assign, int32_t *__restrict__ group_ids) {
+    __shared__ int total[kMaxExperts];
+    __shared__ int first[kMaxExperts];
+    __shared__ int base[kMaxExperts];
+    __shared__ int wave_cnt[kPlanThreads / 64][kMaxExperts];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    if (tid < kMaxExperts) {
+        total[tid] = 0;
+        base[tid] = 0;
     }
     __syncthreads();
-    if (e < n_experts) {
-        int start = 0;
-        for (int j = 0; j < e; j++) start += count[j];
+    for (int i = tid; i < n_slots; i += kPlanThreads) {
+        const int e = idx[i];
+        if (e >= 0 && e < n_experts) atomicAdd(&total[e], 1);
+    }
+    __syncthreads();
+    if (tid < n_experts) {
+        const int e = tid, mine = total[e];
+        int start = 0, rank = 0, n_active = 0;
+        for (int j = 0; j < n_experts; j++) {
+            const int c = total[j];
+            start += j < e ? c : 0;
+            rank += (j < e && c > 0) ? 1 : 0;
+            n_active += c > 0 ? 1 : 0;
+        }
+        first[e] = start;
         offsets[e] = start;
         if (e == n_experts - 1) offsets[n_experts] = start + mine;
-        int at = start;
-        for (int i = 0; i < n_slots; i++) {
-            if (idx[i] == e) {
-                assign_token[at] = i / k;
-                slot_to_assign[i] = at;
-                at++;
+        if (mine > 0) group_ids[rank] = e;
+        else group_ids[n_active + (e - rank)] = -1;
+    }
+    for (int c0 = 0; c0 < n_slots; c0 += kPlanThreads) {
+        const int i = c0 + tid;
+        int e = i < n_slots ? idx[i] : -1;
+        if (e >= n_experts) e = -1;
+        wave_cnt[wave][lane] = 0;
+        wave_cnt[wave][lane + 64] = 0;
+        unsigned long long same = 0;  // lanes of this wave routed to the same expert
+#pragma unroll
+        for (int j = 0; j < 64; j++) same |= (__builtin_amdgcn_readlane(e, j) == e) ? (1ull << j) : 0ull;
+        const int before = __builtin_popcountll(same & ((1ull << lane) - 1ull));
+        if (e >= 0 && lane == 63 - __builtin_clzll(same)) wave_cnt[wave][e] = __builtin_popcountll(same);
+        __syncthreads();  // also orders `first` / `base` before their first use
+        if (e >= 0) {
+            int at = first[e] + base[e] + before;
+            for (int w = 0; w < wave; w++) at += wave_cnt[w][e];
+            assign_token[at] = i / k;
+            slot_to_assign[i] = at;
+        } else if (i < n_slots) {
+            slot_to_assign[i] = -1;
+        }
+        __syncthreads();
+        if (c0 + kPlanThreads < n_slots) {
+            if (tid < kMaxExperts) {
+                int add = 0;
+                for (int w = 0; w < kPlanThreads / 64; w++) add += wave_cnt[w][tid];
+                base[tid] += add;
             }
+            __syncthreads();
         }
     }
 }
@@ -173,7 +246,7 @@ __global__ __launch_bounds__(kMaxExperts) void moe_plan_kernel(const int32_t *__
 // Expert-grouped matmul: the packed-dot kernel for a few tokens, the matrix cores from 4 tokens
 // up (the same crossover as for plain calls).  Both produce the same bits per cell.
 static int launch_expert_matmul(const MatArgs &a, hipStream_t st) {
-    if (a.w->fmt != CML_Q4_K) return launch_gemv_b32_grouped(a, nullptr, st);
+    if (a.w->fmt != CML_Q4_K) return launch_gemv_b32_grouped(a, GroupedPrologue{}, st);
     if (a.n_tokens >= env_int("CAMELID_HIP_Q4K_MFMA_MIN_TOKENS", 4)) return launch_gemm_q4k_mfma(a, st);
     return launch_gemv_q4k(a, st);
 }
@@ -196,7 +269,8 @@ __global__ __launch_bounds__(256) void moe_weighted_sum_kernel(const float *__re
     if (c >= hidden) return;
     float acc = 0.0f;
     for (int s = 0; s < k; s++) {
-        const int64_t a = slot_to_assign[t * k + s];
+        const int64_t a = slot_to_assign ? slot_to_assign[t * k + s] : t * k + s;
+        if (a < 0) continue;  // a slot whose expert id was out of range
         acc = acc + y[a * hidden + c] * weight[t * k + s];
     }
     out[t * hidden + c] = acc;
@@ -205,7 +279,7 @@ __global__ __launch_bounds__(256) void moe_weighted_sum_kernel(const float *__re
 struct MoeWorkspace {
     int8_t *xq;
     float *xd;
-    int32_t *offsets, *assign_token, *slot_to_assign;
+    int32_t *offsets, *assign_token, *slot_to_assign, *group_ids;
     float *g, *u, *y, *hd;
     int8_t *hq;
     size_t total;
@@ -224,6 +298,7 @@ static MoeWorkspace carve(void *base, int64_t hidden, int64_t ff, int64_t n_toke
     // scale arrays are sized for 32-value blocks, the finest any expert format uses
     w.xd = reinterpret_cast<float *>(take(T * ((hidden + 31) / 32) * 4));
     w.offsets = reinterpret_cast<int32_t *>(take((static_cast<size_t>(n_experts) + 1) * 4));
+    w.group_ids = reinterpret_cast<int32_t *>(take(static_cast<size_t>(n_experts) * 4));
     w.assign_token = reinterpret_cast<int32_t *>(take(A * 4));
     w.slot_to_assign = reinterpret_cast<int32_t *>(take(A * 4));
     w.g = reinterpret_cast<float *>(take(A * ff * 4));
@@ -263,8 +338,8 @@ int cml_moe_route_softmax_top_k(const float *logits_dev, int64_t n_tokens, int n
     if (k > n_experts) return fail(CML_ERR_SHAPE, "top-%d of %d experts", k, n_experts);
     if (n_tokens == 0) return CML_OK;
     if (!logits_dev || !idx_dev || !weight_dev) return fail(CML_ERR_INVALID, "null pointer");
-    const unsigned grid = static_cast<unsigned>((n_tokens + 63) / 64);
-    hipLaunchKernelGGL(moe_route_softmax_kernel, dim3(grid), dim3(64), 0, as_stream(stream), logits_dev, n_tokens, n_experts, k,
+    const unsigned grid = static_cast<unsigned>((n_tokens + 3) / 4);
+    hipLaunchKernelGGL(moe_route_softmax_kernel, dim3(grid), dim3(256), 0, as_stream(stream), logits_dev, n_tokens, n_experts, k,
                        down_scale_dev, idx_dev, weight_dev);
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
@@ -315,31 +390,42 @@ int cml_moe_ffn_ex(const cml_weight *gate, const cml_weight *up, const cml_weigh
     const bool fused_decode = n_tokens == 1 && (act_in == 1 || hidden / 256 <= 16) && env_int("CAMELID_HIP_FUSED_QUANT", 1) != 0;
     // ws.g and ws.u are adjacent: a fused gate|up projection writes rows of 2*ff values across both
     const int64_t glu_stride = fused_gate_up ? 2 * ff : ff;
+    const float *u_rows = fused_gate_up ? ws.g + ff : ws.u;
+    // Decode with 32-value-block experts on both sides: the k routed slots ARE the assignments, so
+    // no grouping pass runs (y-slot s of the grid serves expert idx[s]), and the down projection
+    // computes act(g) * u and quantizes it in its own prologue: 4 launches after routing.
+    const bool direct = fused_decode && act_in == 1 && act_mid == 1 && ff <= 8192;
     if (!fused_decode) {
         if (int rc = launch_quantize_act(act_in, x_dev, n_tokens, hidden, ws.xq, ws.xd, st)) return rc;
     }
-    hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(kMaxExperts), 0, st, idx_dev, n_slots, n_experts, k, ws.offsets, ws.assign_token, ws.slot_to_assign);
-    CML_HIP_TRY(hipGetLastError());
+    if (!direct) {
+        hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(kPlanThreads), 0, st, idx_dev, n_slots, n_experts, k, ws.offsets, ws.assign_token,
+                           ws.slot_to_assign, ws.group_ids);
+        CML_HIP_TRY(hipGetLastError());
+    }
 
-    MatArgs a;
-    a.residual = nullptr;
-    a.ints = nullptr;
-    a.group_offsets = ws.offsets;
+    MatArgs a{};
+    a.group_offsets = direct ? nullptr : ws.offsets;
+    a.group_ids = direct ? idx_dev : ws.group_ids;
+    a.max_active = direct ? n_slots : static_cast<int>(std::min<int64_t>(n_experts, n_slots));
     a.n_groups = n_experts;
     a.n_tokens = n_tokens;  // the most assignments one expert can receive
     // gate and up: every assignment reads its token's activation
     a.q = ws.xq;
     a.scales = ws.xd;
-    a.group_rows = ws.assign_token;
+    a.group_rows = direct ? nullptr : ws.assign_token;
     a.band_rows = fused_gate_up ? 2 * ff : ff;
     a.w = gate;
     a.out = ws.g;
     if (fused_decode && act_in == 1) {
-        if (int rc = launch_gemv_b32_grouped(a, x_dev, st)) return rc;
+        GroupedPrologue token;
+        token.kind = 1;
+        token.x = x_dev;
+        if (int rc = launch_gemv_b32_grouped(a, token, st)) return rc;
         if (up) {
             a.w = up;
             a.out = ws.u;
-            if (int rc = launch_gemv_b32_grouped(a, x_dev, st)) return rc;
+            if (int rc = launch_gemv_b32_grouped(a, token, st)) return rc;
         }
     } else if (fused_decode) {
         if (int rc = launch_gemv_q4k_f32_grouped_pair(a, up, up ? ws.u : nullptr, x_dev, st)) return rc;
@@ -351,18 +437,26 @@ int cml_moe_ffn_ex(const cml_weight *gate, const cml_weight *up, const cml_weigh
         a.out = ws.u;
         if (int rc = launch_expert_matmul(a, st)) return rc;
     }
-    // h = act(g) * u, quantized per assignment
-    if (int rc = launch_glu_quantize(glu, act_mid, ws.g, fused_gate_up ? ws.g + ff : ws.u, n_slots, ff, glu_stride, ws.hq, ws.hd, st)) return rc;
-    // down: assignment j reads its own h
+    // down: assignment j reads its own h = act(g) * u, quantized per assignment
     a.q = ws.hq;
     a.scales = ws.hd;
     a.group_rows = nullptr;
     a.band_rows = hidden;
     a.w = down;
     a.out = ws.y;
-    if (int rc = launch_expert_matmul(a, st)) return rc;
+    if (direct) {
+        GroupedPrologue gated;
+        gated.kind = 2 + glu;
+        gated.x = ws.g;
+        gated.u = u_rows;
+        gated.stride = glu_stride;
+        if (int rc = launch_gemv_b32_grouped(a, gated, st)) return rc;
+    } else {
+        if (int rc = launch_glu_quantize(glu, act_mid, ws.g, u_rows, n_slots, ff, glu_stride, ws.hq, ws.hd, st)) return rc;
+        if (int rc = launch_expert_matmul(a, st)) return rc;
+    }
     hipLaunchKernelGGL(moe_weighted_sum_kernel, dim3(static_cast<unsigned>((hidden + 255) / 256), static_cast<unsigned>(n_tokens)), dim3(256), 0, st,
-                       ws.y, ws.slot_to_assign, weight_dev, k, hidden, out_dev);
+                       ws.y, direct ? nullptr : ws.slot_to_assign, weight_dev, k, hidden, out_dev);
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }

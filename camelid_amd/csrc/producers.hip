@@ -157,24 +157,6 @@ int launch_rms_norm_quantize(int act, const float *x, const float *weight, float
 
 // h = silu(g) * u = (g / (1 + exp(-g))) * u, quantized on the fly.  Q8_K: one wave per
 // 256-value super-block, lane l holding values 4l..4l+3 (the layout of quantize_q8_k_kernel).
-// GLU 0: silu(g) * u = (g / (1 + exp(-g))) * u (reference CpuTensor::silu_mul).
-// GLU 1: gelu_pytorch_tanh(g) * u = (0.5 * g * (1 + tanh(C * (g + 0.044715 * g * g * g)))) * u,
-//        evaluated left to right (reference gelu_tanh, src/gemma4_mtp.rs:172-175; the expert
-//        activation of the Gemma-4 lane, src/gemma4_runtime.rs:5689-5691).
-template <int GLU>
-__device__ __forceinline__ float glu1(float g, float u) {
-    if constexpr (GLU == 0) {
-        return (g / (1.0f + expf(-g))) * u;
-    } else {
-        const float cube = ((0.044715f * g) * g) * g;
-        return ((0.5f * g) * (1.0f + tanhf(0.7978846f * (g + cube)))) * u;
-    }
-}
-template <int GLU>
-__device__ __forceinline__ float4 glu4(const float4 gv, const float4 uv) {
-    return make_float4(glu1<GLU>(gv.x, uv.x), glu1<GLU>(gv.y, uv.y), glu1<GLU>(gv.z, uv.z), glu1<GLU>(gv.w, uv.w));
-}
-
 // Row r of g / u starts at g + r * in_stride / u + r * in_stride (in_stride = cols for separate
 // buffers; 2 * cols with u = g + cols when a fused gate|up projection wrote both halves of a row).
 template <int GLU>
