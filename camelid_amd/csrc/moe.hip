@@ -345,6 +345,59 @@ int cml_moe_route_softmax_top_k(const float *logits_dev, int64_t n_tokens, int n
     return CML_OK;
 }
 
+int cml_moe_plan(const int32_t *idx_dev, int64_t n_tokens, int k, int n_experts, int32_t *token_offsets_dev,
+                 int32_t *token_ids_dev, int32_t *route_to_assignment_dev, int32_t *union_experts_dev, cml_stream_t stream) {
+    if (!ready()) return fail(CML_ERR_UNAVAILABLE, "cml_init has not succeeded");
+    if (n_tokens < 0 || k <= 0 || n_experts <= 0 || n_tokens * k > INT32_MAX) return fail(CML_ERR_SHAPE, "bad routing shape");
+    if (n_experts > kMaxExperts) return fail(CML_ERR_UNSUPPORTED, "at most %d experts", kMaxExperts);
+    if (!token_offsets_dev || !union_experts_dev) return fail(CML_ERR_INVALID, "null pointer");
+    if (n_tokens > 0 && (!idx_dev || !token_ids_dev || !route_to_assignment_dev)) return fail(CML_ERR_INVALID, "null pointer");
+    hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(kPlanThreads), 0, as_stream(stream), idx_dev, static_cast<int>(n_tokens * k), n_experts, k,
+                       token_offsets_dev, token_ids_dev, route_to_assignment_dev, union_experts_dev);
+    CML_HIP_TRY(hipGetLastError());
+    return CML_OK;
+}
+
+int cml_moe_gemv_routed(const cml_weight *experts, int n_experts, const int8_t *q_dev, const float *scales_dev,
+                        const int32_t *token_offsets_dev, const int32_t *token_ids_dev, const int32_t *union_experts_dev,
+                        int max_union, int64_t max_assignments_per_expert, float *out_dev, cml_stream_t stream) {
+    if (!ready()) return fail(CML_ERR_UNAVAILABLE, "cml_init has not succeeded");
+    if (!experts) return fail(CML_ERR_INVALID, "null weight");
+    if (!expert_format(experts->fmt)) return fail(CML_ERR_UNSUPPORTED, "routed matvec is built for Q4_K, Q8_0 and Q4_0 expert matrices");
+    if (n_experts <= 0 || n_experts > kMaxExperts || experts->rows % n_experts != 0)
+        return fail(CML_ERR_SHAPE, "%lld rows do not stack to %d experts", (long long)experts->rows, n_experts);
+    if (max_assignments_per_expert < 0 || (union_experts_dev && (max_union <= 0 || max_union > n_experts)))
+        return fail(CML_ERR_SHAPE, "bad routed shape");
+    if (max_assignments_per_expert == 0) return CML_OK;
+    if (!q_dev || !scales_dev || !token_offsets_dev || !out_dev) return fail(CML_ERR_INVALID, "null pointer");
+    if ((reinterpret_cast<uintptr_t>(q_dev) & 15u) != 0) return fail(CML_ERR_INVALID, "quantized activations must be 16-byte aligned");
+    MatArgs a{};
+    a.w = experts;
+    a.q = q_dev;
+    a.scales = scales_dev;
+    a.n_tokens = max_assignments_per_expert;
+    a.out = out_dev;
+    a.group_offsets = token_offsets_dev;
+    a.group_rows = token_ids_dev;
+    a.group_ids = union_experts_dev;
+    a.max_active = max_union;
+    a.n_groups = n_experts;
+    a.band_rows = experts->rows / n_experts;
+    return launch_expert_matmul(a, as_stream(stream));
+}
+
+int cml_moe_weighted_sum(const float *y_dev, const int32_t *route_to_assignment_dev, const float *weight_dev, int64_t n_tokens, int k,
+                         int64_t hidden, float *out_dev, cml_stream_t stream) {
+    if (!ready()) return fail(CML_ERR_UNAVAILABLE, "cml_init has not succeeded");
+    if (n_tokens < 0 || k <= 0 || hidden <= 0 || n_tokens > 65535) return fail(CML_ERR_SHAPE, "bad shape");
+    if (n_tokens == 0) return CML_OK;
+    if (!y_dev || !weight_dev || !out_dev) return fail(CML_ERR_INVALID, "null pointer");
+    hipLaunchKernelGGL(moe_weighted_sum_kernel, dim3(static_cast<unsigned>((hidden + 255) / 256), static_cast<unsigned>(n_tokens)), dim3(256), 0,
+                       as_stream(stream), y_dev, route_to_assignment_dev, weight_dev, k, hidden, out_dev);
+    CML_HIP_TRY(hipGetLastError());
+    return CML_OK;
+}
+
 size_t cml_moe_workspace_bytes(int fmt, int64_t hidden, int64_t ff, int64_t n_tokens, int k, int n_experts) {
     if (!expert_format(fmt) || hidden <= 0 || ff <= 0 || n_tokens <= 0 || k <= 0 || n_experts <= 0) return 0;
     return carve(nullptr, hidden, ff, n_tokens, k, n_experts).total;

@@ -265,6 +265,38 @@ int cml_moe_ffn_ex(const cml_weight *gate, const cml_weight *up, const cml_weigh
                    int64_t n_tokens, float *out_dev, void *workspace_dev, size_t workspace_bytes,
                    int glu, cml_stream_t stream);
 
+/* The pieces cml_moe_ffn is made of, for callers that schedule the expert
+ * lane themselves.
+ * cml_moe_plan groups the n_tokens*k routed slots by expert, keeping (token,
+ * rank) order inside each group (reference gemma4_plan_route_union,
+ * src/gemma4_runtime.rs:12309-12424): token_offsets_dev int32[n_experts+1]
+ * (CSR over expert ids), token_ids_dev int32[n_tokens*k] (assignment -> token),
+ * route_to_assignment_dev int32[n_tokens*k] (slot t*k+s -> assignment; -1 for
+ * an expert id out of range), union_experts_dev int32[n_experts] (the experts
+ * in use, ascending, then -1). */
+int cml_moe_plan(const int32_t *idx_dev, int64_t n_tokens, int k, int n_experts,
+                 int32_t *token_offsets_dev, int32_t *token_ids_dev,
+                 int32_t *route_to_assignment_dev, int32_t *union_experts_dev, cml_stream_t stream);
+/* Expert-grouped matvec on quantized activations (reference
+ * launch_q4_wire_gemm_routed, src/cuda_resident.rs:12215-12313): `experts`
+ * stacks n_experts bands of rows/n_experts rows; assignment j of expert e (j in
+ * [token_offsets[e], token_offsets[e+1])) dots band e with activation row
+ * token_ids[j] (j itself when token_ids_dev is null) and writes
+ * out_dev[j][band rows].  Activations are Q8_K for Q4_K experts, Q8_0 for Q8_0 /
+ * Q4_0 (cml_quantize_*).  union_experts_dev (nullable) compacts the launch to
+ * max_union grid slots; max_assignments_per_expert bounds any one group. */
+int cml_moe_gemv_routed(const cml_weight *experts, int n_experts, const int8_t *q_dev,
+                        const float *scales_dev, const int32_t *token_offsets_dev,
+                        const int32_t *token_ids_dev, const int32_t *union_experts_dev, int max_union,
+                        int64_t max_assignments_per_expert, float *out_dev, cml_stream_t stream);
+/* out[t][c] = sum over s in routed order of y[route_to_assignment[t*k+s]][c] *
+ * weight[t*k+s], multiply and add rounded separately (reference
+ * moe_weighted_sum_batched, src/cuda_resident.rs:6369-6389; CPU accumulate,
+ * src/inference.rs:14255-14257).  route_to_assignment_dev null = identity. */
+int cml_moe_weighted_sum(const float *y_dev, const int32_t *route_to_assignment_dev,
+                         const float *weight_dev, int64_t n_tokens, int k, int64_t hidden,
+                         float *out_dev, cml_stream_t stream);
+
 /* ---- weight quantizer tool (reference quantize_block_q8_0 / q4_0 / q4_k,
  *      src/quantize.rs:98-244): f32 values -> GGUF wire bytes on the host, in
  *      whole blocks, on `threads` threads.  Q6_K has no counterpart in the

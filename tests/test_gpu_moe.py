@@ -170,6 +170,7 @@ def test_c5_mixtral_shaped_moe(T):
 # ---------------------------------------------------------------- Gemma-4 variant ----
 
 GLU_SILU, GLU_GELU_TANH = 0, 1
+ACT_Q8_0, ACT_Q8_K = 1, 2
 
 
 def test_route_softmax_top_k_matches_oracle():
@@ -329,3 +330,104 @@ def test_gemma4_26b_shaped_moe(T):
     if T > tt:   # the rest of the batch: the same cells as a single-token call (bit for bit: one chain per cell)
         one = gpu_moe(wgu, None, wd, E, k, *gpu_route_softmax(logits[T - 1:T], k, ds)[:2], x[T - 1:T], glu=GLU_GELU_TANH)
         assert G.same_bits(got[T - 1:T], one)
+
+
+# ---------------------------------------------------------------- the pieces ----
+
+def gpu_plan(idx, E):
+    idx = np.ascontiguousarray(idx, np.int32)
+    T, k = idx.shape
+    d_idx = DeviceBuffer.from_numpy(idx)
+    off, tok = DeviceBuffer((E + 1) * 4), DeviceBuffer(max(1, T * k) * 4)
+    r2a, uni = DeviceBuffer(max(1, T * k) * 4), DeviceBuffer(E * 4)
+    for b in (off, tok, r2a, uni):
+        b.fill(0x7F)
+    check(lib().cml_moe_plan(d_idx.ptr, T, k, E, off.ptr, tok.ptr, r2a.ptr, uni.ptr, None), "cml_moe_plan")
+    check(lib().cml_stream_sync(None))
+    return (off, tok, r2a, uni), (off.to_numpy(np.int32, (E + 1,)), tok.to_numpy(np.int32, (T * k,)),
+                                  r2a.to_numpy(np.int32, (T * k,)), uni.to_numpy(np.int32, (E,)))
+
+
+@pytest.mark.parametrize("T,k,E", [(1, 2, 8), (7, 3, 6), (32, 8, 128), (100, 8, 128), (600, 8, 128), (300, 1, 5)])
+def test_moe_plan_is_a_stable_grouping(T, k, E):
+    """The route-union plan (reference gemma4_plan_route_union, src/gemma4_runtime.rs:12309-12424):
+    a stable sort of the routed slots by expert, checked against numpy's stable argsort."""
+    rng = np.random.default_rng(390 + T)
+    idx = np.stack([rng.permutation(E)[:k] for _ in range(T)]).astype(np.int32)
+    if T >= 7:
+        idx[:, 0] = 3 % E          # crowd one expert across waves and passes
+        idx[2, k - 1] = E + 5      # ids out of range are dropped
+        idx[5, k - 1] = -1
+    G.say(f"moe plan T={T} k={k} E={E}")
+    _, (off, tok, r2a, uni) = gpu_plan(idx, E)
+    flat = idx.reshape(-1)
+    valid = (flat >= 0) & (flat < E)
+    order = np.flatnonzero(valid)[np.argsort(flat[valid], kind="stable")]
+    counts = np.bincount(flat[valid], minlength=E)
+    assert list(off) == [0] + list(np.cumsum(counts))
+    assert list(tok[:order.size]) == list(order // k)
+    want_r2a = np.full(T * k, -1, np.int32)
+    want_r2a[order] = np.arange(order.size)
+    assert list(r2a) == list(want_r2a)
+    used = np.flatnonzero(counts)
+    assert list(uni) == list(used) + [-1] * (E - used.size)
+
+
+@pytest.mark.parametrize("fmt,fmt_down,hidden,ff", [(B.CML_Q4_K, B.CML_Q4_K, 512, 256), (B.CML_Q4_0, B.CML_Q8_0, 352, 96)])
+@pytest.mark.parametrize("T", [1, 9])
+def test_moe_pieces_compose_to_the_whole(fmt, fmt_down, hidden, ff, T):
+    """plan + quantize + routed matvec (gate|up) + gated activation + routed matvec (down) +
+    weighted sum through the separate entry points = cml_moe_ffn_ex, bit for bit."""
+    E, k = 16, 4
+    L = lib()
+    gate_up, down = _experts_fused(fmt, fmt_down, E, hidden, ff, 400)
+    rng = np.random.default_rng(401 + T)
+    x = rng.standard_normal((T, hidden)).astype(np.float32)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    logits[:, 2] += 3.0
+    wgu = Weight.upload(fmt, E * 2 * ff, hidden, gate_up)
+    wd = Weight.upload(fmt_down, E * hidden, ff, down)
+    idx_dev, w_dev, idx, w = gpu_route_softmax(logits, k)
+    G.say(f"moe pieces vs whole fmt={fmt}/{fmt_down} T={T}")
+    with G.env(CAMELID_HIP_EXACT_ORDER="1"):
+        whole = gpu_moe(wgu, None, wd, E, k, idx_dev, w_dev, x, glu=GLU_GELU_TANH)
+        (off, tok, r2a, uni), _ = gpu_plan(idx, E)
+        A = T * k
+        act_in = ACT_Q8_K if fmt == B.CML_Q4_K else ACT_Q8_0
+        act_mid = ACT_Q8_K if fmt_down == B.CML_Q4_K else ACT_Q8_0
+        per_in, per_mid = (256 if act_in == ACT_Q8_K else 32), (256 if act_mid == ACT_Q8_K else 32)
+        xd = DeviceBuffer.from_numpy(x)
+        xq, xs = DeviceBuffer(T * hidden), DeviceBuffer(T * (hidden // per_in) * 4)
+        quant = L.cml_quantize_q8_k if act_in == ACT_Q8_K else L.cml_quantize_q8_0
+        check(quant(xd.ptr, T, hidden, xq.ptr, xs.ptr, None))
+        gu = DeviceBuffer(A * 2 * ff * 4)
+        check(L.cml_moe_gemv_routed(wgu.handle, E, xq.ptr, xs.ptr, off.ptr, tok.ptr, uni.ptr, min(E, A), T, gu.ptr, None),
+              "cml_moe_gemv_routed gate|up")
+        check(L.cml_stream_sync(None))
+        g_u = gu.to_numpy(np.float32, (A, 2, ff))
+        gd = DeviceBuffer.from_numpy(np.ascontiguousarray(g_u[:, 0]))
+        ud = DeviceBuffer.from_numpy(np.ascontiguousarray(g_u[:, 1]))
+        hq, hs = DeviceBuffer(A * ff), DeviceBuffer(A * (ff // per_mid) * 4)
+        check(L.cml_glu_quantize(GLU_GELU_TANH, act_mid, gd.ptr, ud.ptr, A, ff, hq.ptr, hs.ptr, None), "cml_glu_quantize")
+        y = DeviceBuffer(A * hidden * 4)
+        check(L.cml_moe_gemv_routed(wd.handle, E, hq.ptr, hs.ptr, off.ptr, None, None, 0, T, y.ptr, None), "cml_moe_gemv_routed down")
+        out = DeviceBuffer(T * hidden * 4)
+        check(L.cml_moe_weighted_sum(y.ptr, r2a.ptr, w_dev.ptr, T, k, hidden, out.ptr, None), "cml_moe_weighted_sum")
+        check(L.cml_stream_sync(None))
+    assert G.same_bits(out.to_numpy(np.float32, (T, hidden)), whole)
+
+
+def test_moe_pieces_reject_bad_arguments():
+    L = lib()
+    d = DeviceBuffer(1 << 16)
+    w6 = Weight.upload(B.CML_Q6_K, 256, 256, G.synth_weight(B.CML_Q6_K, 256, 256, 410))
+    w4 = Weight.upload(B.CML_Q4_0, 96, 64, G.synth_weight(B.CML_Q4_0, 96, 64, 411))
+    assert L.cml_moe_plan(d.ptr, 4, 2, 129, d.ptr, d.ptr, d.ptr, d.ptr, None) == 6
+    assert L.cml_moe_plan(d.ptr, 4, 0, 8, d.ptr, d.ptr, d.ptr, d.ptr, None) == 3
+    assert L.cml_moe_plan(None, 4, 2, 8, d.ptr, d.ptr, d.ptr, d.ptr, None) == 2
+    assert L.cml_moe_gemv_routed(w6.handle, 2, d.ptr, d.ptr, d.ptr, None, None, 0, 1, d.ptr, None) == 6
+    assert L.cml_moe_gemv_routed(w4.handle, 5, d.ptr, d.ptr, d.ptr, None, None, 0, 1, d.ptr, None) == 3   # 96 rows, 5 experts
+    assert L.cml_moe_gemv_routed(w4.handle, 4, None, d.ptr, d.ptr, None, None, 0, 1, d.ptr, None) == 2
+    assert L.cml_moe_gemv_routed(w4.handle, 4, d.ptr, d.ptr, d.ptr, None, None, 0, 0, d.ptr, None) == 0   # nothing routed
+    assert L.cml_moe_weighted_sum(None, None, d.ptr, 1, 2, 64, d.ptr, None) == 2
+    assert L.cml_moe_weighted_sum(d.ptr, None, d.ptr, 0, 2, 64, d.ptr, None) == 0
