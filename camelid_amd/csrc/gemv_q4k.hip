@@ -69,6 +69,11 @@ struct Q4KArgs {
     const int32_t *group_offsets;
     const int32_t *group_rows;
     const int32_t *group_ids;  // y-slot -> group (-1: unused slot), or null (the y-slot is the group)
+    // Direct call (single-token decode; group_offsets null, group_ids set): y-slot y IS assignment y
+    // and group_ids[y] its expert (ids outside [0, n_groups) are skipped); its activation row is
+    // row 0 (shared_act: every assignment reads the one token) or row y.
+    int n_groups;
+    int shared_act;
     // Pair launch (gridDim.z == 2): blockIdx.z = 1 works on a second weight of the same shape
     // against the same activations and writes out2 (gate and up projections in one launch).
     const uint8_t *w2;
@@ -206,11 +211,12 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
 
     const int tid = threadIdx.x;
     const int nthreads = blockDim.x;
+    const bool direct = a.group_offsets == nullptr && a.group_ids != nullptr;
     const bool grouped = a.group_offsets != nullptr;
-    const int64_t band = grouped ? (a.group_ids ? a.group_ids[blockIdx.y] : static_cast<int>(blockIdx.y)) : 0;
-    if (band < 0) return;  // a y-slot past the groups in use
-    const int a0 = grouped ? a.group_offsets[band] : 0;               // first assignment of this group
-    const int n_assign = grouped ? a.group_offsets[band + 1] - a0 : NT;
+    const int64_t band = (grouped || direct) ? (a.group_ids ? a.group_ids[blockIdx.y] : static_cast<int>(blockIdx.y)) : 0;
+    if (band < 0 || (direct && band >= a.n_groups)) return;  // a y-slot past the groups in use, or an id out of range
+    const int a0 = grouped ? a.group_offsets[band] : (direct ? static_cast<int>(blockIdx.y) : 0);  // first assignment of this group
+    const int n_assign = grouped ? a.group_offsets[band + 1] - a0 : (direct ? 1 : NT);
     if (n_assign <= 0) return;  // an expert nobody routed to: the whole workgroup leaves
     const bool second = gridDim.z > 1 && blockIdx.z == 1;
     const uint8_t *w = (second ? a.w2 : a.w) + band * (a.rows / 16) * kQ4KChunk;
@@ -239,6 +245,7 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
         // Activation row of local token t (clamped to the group's last assignment; extra tokens store nothing).
         auto act_row = [&](int t) -> int64_t {
             const int j = a0 + min(p0 + t, n_assign - 1);
+            if (a.shared_act) return 0;
             return a.group_rows ? a.group_rows[j] : j;
         };
         Q4KRegs ra, rb;
@@ -478,7 +485,7 @@ static int launch_q4k_pick_nt(const Q4KArgs &ka, const Q4KShape &shape, int n_gr
 // same launch (grid.z = 2).
 static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, const float *x, hipStream_t st) {
     const cml_weight *w = a.w;
-    const bool grouped = a.group_offsets != nullptr;
+    const bool grouped = a.group_offsets != nullptr || a.group_ids != nullptr;
     if (w->rows == 0) return CML_OK;
     Q4KArgs ka{};
     ka.w = w->planes.p[0];
@@ -493,6 +500,8 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
     ka.group_offsets = a.group_offsets;
     ka.group_rows = a.group_rows;
     ka.group_ids = a.group_ids;
+    ka.n_groups = a.n_groups;
+    ka.shared_act = grouped && !a.group_offsets;  // direct call: the one f32 token
     if (w2) {
         if (w2->fmt != w->fmt || w2->rows != w->rows || w2->nb != w->nb || w2->row_skip != w->row_skip ||
             w2->planes.row_stride[0] != w->planes.row_stride[0])
@@ -535,7 +544,7 @@ int launch_gemv_q4k_f32_grouped_pair(const MatArgs &a, const cml_weight *w2, flo
 int launch_gemv_q4k(const MatArgs &a, hipStream_t st) {
     const cml_weight *w = a.w;
     if (w->rows == 0 || a.n_tokens == 0) return CML_OK;
-    const bool grouped = a.group_offsets != nullptr;
+    const bool grouped = a.group_offsets != nullptr || a.group_ids != nullptr;
     Q4KArgs ka{};
     ka.w = w->planes.p[0];
     ka.sb_stride = w->planes.row_stride[0];
@@ -549,6 +558,7 @@ int launch_gemv_q4k(const MatArgs &a, hipStream_t st) {
     ka.group_offsets = a.group_offsets;
     ka.group_rows = a.group_rows;
     ka.group_ids = a.group_ids;
+    ka.n_groups = a.n_groups;
     const Q4KShape shape = pick_shape(ka.rows, ka.n_sb);
     if (grouped) {
         // One launch: every group walks its own assignments in passes of NT

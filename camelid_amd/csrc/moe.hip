@@ -247,7 +247,7 @@ __global__ __launch_bounds__(kPlanThreads) void moe_plan_kernel(const int32_t *_
 // up (the same crossover as for plain calls).  Both produce the same bits per cell.
 static int launch_expert_matmul(const MatArgs &a, hipStream_t st) {
     if (a.w->fmt != CML_Q4_K) return launch_gemv_b32_grouped(a, GroupedPrologue{}, st);
-    if (a.n_tokens >= env_int("CAMELID_HIP_Q4K_MFMA_MIN_TOKENS", 4)) return launch_gemm_q4k_mfma(a, st);
+    if (a.group_offsets && a.n_tokens >= env_int("CAMELID_HIP_Q4K_MFMA_MIN_TOKENS", 4)) return launch_gemm_q4k_mfma(a, st);
     return launch_gemv_q4k(a, st);
 }
 
@@ -447,7 +447,11 @@ int cml_moe_ffn_ex(const cml_weight *gate, const cml_weight *up, const cml_weigh
     // Decode with 32-value-block experts on both sides: the k routed slots ARE the assignments, so
     // no grouping pass runs (y-slot s of the grid serves expert idx[s]), and the down projection
     // computes act(g) * u and quantizes it in its own prologue: 4 launches after routing.
-    const bool direct = fused_decode && act_in == 1 && act_mid == 1 && ff <= 8192;
+    const bool b32_direct = fused_decode && act_in == 1 && act_mid == 1 && ff <= 8192;
+    // Q4_K on both sides: the same without the fused down prologue (a 56-super-block row is too
+    // much to re-quantize in every workgroup).
+    const bool q4k_direct = fused_decode && act_in == 2 && act_mid == 2;
+    const bool direct = b32_direct || q4k_direct;
     if (!fused_decode) {
         if (int rc = launch_quantize_act(act_in, x_dev, n_tokens, hidden, ws.xq, ws.xd, st)) return rc;
     }
@@ -497,7 +501,7 @@ int cml_moe_ffn_ex(const cml_weight *gate, const cml_weight *up, const cml_weigh
     a.band_rows = hidden;
     a.w = down;
     a.out = ws.y;
-    if (direct) {
+    if (b32_direct) {
         GroupedPrologue gated;
         gated.kind = 2 + glu;
         gated.x = ws.g;
