@@ -34,9 +34,17 @@ struct Q6KArgs {
     float *out;
     const float *residual;
     int32_t *ints;  // [rows][n_sb] or null
-    const int32_t *band_ids;
-    int64_t act_slot_stride;
-    int64_t out_slot_stride;
+    // Plain call: blockIdx.y = 0, the NT activation rows 0..NT-1 go to output rows 0..NT-1.
+    // Grouped call (mixture of experts): y-slot -> group e = group_ids[y] (y itself when null; -1 =
+    // unused slot), which owns the band of rows [e*rows, (e+1)*rows) and the assignments
+    // [group_offsets[e], group_offsets[e+1]); assignment j reads activation row group_rows[j] (j
+    // itself when null) and writes output row j, NT assignments per pass.
+    // Direct call (single-token decode; group_offsets null, group_ids set): y-slot y IS assignment
+    // y and group_ids[y] its expert; ids outside [0, n_groups) are skipped.
+    const int32_t *group_offsets;
+    const int32_t *group_rows;
+    const int32_t *group_ids;
+    int n_groups;
     int ksplit;
 };
 
@@ -116,8 +124,9 @@ __device__ __forceinline__ void q6k_compute(const Q6KRegs &r, int l, int sb, int
     }
 }
 
-template <int NT, bool INTS>
+template <int NT, bool INTS, bool GROUPED = false>
 __global__ __launch_bounds__(256) void gemv_q6k_kernel(Q6KArgs a) {
+    static_assert(!(GROUPED && INTS), "block-int diagnostics are for plain calls");
     constexpr int LPS = 8, RPW = kWave / LPS;
     extern __shared__ uint4 smem[];
     const int n_sb = a.n_sb;
@@ -127,24 +136,16 @@ __global__ __launch_bounds__(256) void gemv_q6k_kernel(Q6KArgs a) {
     float *part = yds + ((NT * n_sb + 3) & ~3);
 
     const int tid = threadIdx.x;
-    const int slot = blockIdx.y;
-    const int64_t band = a.band_ids ? a.band_ids[slot] : 0;
-    const int8_t *q = a.q + static_cast<int64_t>(slot) * a.act_slot_stride * n_sb * 256;
-    const float *yd = a.yd + static_cast<int64_t>(slot) * a.act_slot_stride * n_sb;
-    float *out = a.out + static_cast<int64_t>(slot) * a.out_slot_stride;
-
-    {
-        const uint4 *src = reinterpret_cast<const uint4 *>(q);
-        uint4 *dst = reinterpret_cast<uint4 *>(ys);
-        const int n16 = NT * n_sb * 16;
-        for (int i = tid; i < n16; i += 256) {
-            const uint4 v = src[i];
-            dst[i] = v;
-            bsum16[i] = bytesum16(v);
-        }
-        for (int i = tid; i < NT * n_sb; i += 256) yds[i] = yd[i];
+    int64_t band = 0;
+    int a0 = 0, n_assign = NT;
+    if constexpr (GROUPED) {
+        const bool direct = a.group_offsets == nullptr;
+        band = a.group_ids ? a.group_ids[blockIdx.y] : static_cast<int>(blockIdx.y);
+        if (band < 0 || band >= a.n_groups) return;  // an unused y-slot or an id out of range: the workgroup leaves together
+        a0 = direct ? static_cast<int>(blockIdx.y) : a.group_offsets[band];
+        n_assign = direct ? 1 : a.group_offsets[band + 1] - a0;
+        if (n_assign <= 0) return;
     }
-    __syncthreads();
 
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int W = a.ksplit;
@@ -167,63 +168,100 @@ __global__ __launch_bounds__(256) void gemv_q6k_kernel(Q6KArgs a) {
         if (a.ints && leader && live) ints_row = a.ints + arow * static_cast<int64_t>(n_sb);
     }
 
-    float acc[NT];
-#pragma unroll
-    for (int t = 0; t < NT; t++) acc[t] = 0.0f;
-
-    constexpr int U = Q6KRegs::U;
-    Q6KRegs ra, rb;
-    q6k_load(ra, ql, qh, sc, dp, l, s0, s1);
-    __builtin_amdgcn_sched_barrier(0);
-    // Two register buffers alternate; the last one is consumed without issuing
-    // further loads.
-    for (int sb = s0;;) {
-        if (sb + U >= s1) {
-            q6k_compute<NT, INTS>(ra, l, sb, s1, ys, bsum16, yds, n_sb, acc, ints_row);
-            break;
-        }
-        q6k_load(rb, ql, qh, sc, dp, l, sb + U, s1);
-        __builtin_amdgcn_sched_barrier(0);
-        q6k_compute<NT, INTS>(ra, l, sb, s1, ys, bsum16, yds, n_sb, acc, ints_row);
-        __builtin_amdgcn_sched_barrier(0);
-        sb += U;
-        if (sb + U >= s1) {
-            q6k_compute<NT, INTS>(rb, l, sb, s1, ys, bsum16, yds, n_sb, acc, ints_row);
-            break;
-        }
-        q6k_load(ra, ql, qh, sc, dp, l, sb + U, s1);
-        __builtin_amdgcn_sched_barrier(0);
-        q6k_compute<NT, INTS>(rb, l, sb, s1, ys, bsum16, yds, n_sb, acc, ints_row);
-        __builtin_amdgcn_sched_barrier(0);
-        sb += U;
-    }
-
-    if (W == 1) {
-        if (leader && live) {
-#pragma unroll
-            for (int t = 0; t < NT; t++) {
-                float v = acc[t];
-                if (NT == 1 && a.residual) v = v + a.residual[row];
-                out[static_cast<int64_t>(t) * a.rows + row] = v;
+    for (int p0 = 0; p0 < n_assign; p0 += NT) {
+        // activation row of local token t (clamped to the group's last assignment; extra tokens store nothing)
+        auto act_row = [&](int t) -> int64_t {
+            const int j = a0 + min(p0 + t, n_assign - 1);
+            return a.group_rows ? a.group_rows[j] : j;
+        };
+        if (p0 > 0) __syncthreads();  // the previous pass's readers are done
+        if constexpr (!GROUPED) {
+            const uint4 *src = reinterpret_cast<const uint4 *>(a.q);
+            uint4 *dst = reinterpret_cast<uint4 *>(ys);
+            const int n16 = NT * n_sb * 16;
+            for (int i = tid; i < n16; i += 256) {
+                const uint4 v = src[i];
+                dst[i] = v;
+                bsum16[i] = bytesum16(v);
+            }
+            for (int i = tid; i < NT * n_sb; i += 256) yds[i] = a.yd[i];
+        } else {
+            uint4 *dst = reinterpret_cast<uint4 *>(ys);
+            const int c16 = n_sb * 16;
+            for (int i = tid; i < NT * c16; i += 256) {
+                const int t = i / c16;
+                const uint4 v = reinterpret_cast<const uint4 *>(a.q + act_row(t) * n_sb * 256)[i - t * c16];
+                dst[i] = v;
+                bsum16[i] = bytesum16(v);
+            }
+            for (int i = tid; i < NT * n_sb; i += 256) {
+                const int t = i / n_sb;
+                yds[i] = a.yd[act_row(t) * n_sb + (i - t * n_sb)];
             }
         }
-        return;
-    }
-    if (leader) {
+        __syncthreads();
+        float *out = a.out + static_cast<int64_t>(a0 + p0) * a.rows;
+        const int n_here = GROUPED ? min(NT, n_assign - p0) : NT;
+
+        float acc[NT];
 #pragma unroll
-        for (int t = 0; t < NT; t++) part[(wave * NT + t) * RPW + r] = acc[t];
-    }
-    __syncthreads();
-    for (int i = tid; i < tiles_per_wg * NT * RPW; i += 256) {
-        const int rr = i % RPW;
-        const int t = (i / RPW) % NT;
-        const int tw = i / (RPW * NT);
-        const int orow = (blockIdx.x * tiles_per_wg + tw) * RPW + rr;
-        if (orow >= a.rows) continue;
-        float v = part[((tw * W) * NT + t) * RPW + rr];
-        for (int k = 1; k < W; k++) v = v + part[((tw * W + k) * NT + t) * RPW + rr];
-        if (NT == 1 && a.residual) v = v + a.residual[orow];
-        out[static_cast<int64_t>(t) * a.rows + orow] = v;
+        for (int t = 0; t < NT; t++) acc[t] = 0.0f;
+
+        constexpr int U = Q6KRegs::U;
+        Q6KRegs ra, rb;
+        q6k_load(ra, ql, qh, sc, dp, l, s0, s1);
+        __builtin_amdgcn_sched_barrier(0);
+        // Two register buffers alternate; the last one is consumed without issuing
+        // further loads.
+        for (int sb = s0;;) {
+            if (sb + U >= s1) {
+                q6k_compute<NT, INTS>(ra, l, sb, s1, ys, bsum16, yds, n_sb, acc, ints_row);
+                break;
+            }
+            q6k_load(rb, ql, qh, sc, dp, l, sb + U, s1);
+            __builtin_amdgcn_sched_barrier(0);
+            q6k_compute<NT, INTS>(ra, l, sb, s1, ys, bsum16, yds, n_sb, acc, ints_row);
+            __builtin_amdgcn_sched_barrier(0);
+            sb += U;
+            if (sb + U >= s1) {
+                q6k_compute<NT, INTS>(rb, l, sb, s1, ys, bsum16, yds, n_sb, acc, ints_row);
+                break;
+            }
+            q6k_load(ra, ql, qh, sc, dp, l, sb + U, s1);
+            __builtin_amdgcn_sched_barrier(0);
+            q6k_compute<NT, INTS>(rb, l, sb, s1, ys, bsum16, yds, n_sb, acc, ints_row);
+            __builtin_amdgcn_sched_barrier(0);
+            sb += U;
+        }
+
+        if (W == 1) {
+            if (leader && live) {
+#pragma unroll
+                for (int t = 0; t < NT; t++) {
+                    if (t >= n_here) break;
+                    float v = acc[t];
+                    if (NT == 1 && a.residual) v = v + a.residual[row];
+                    out[static_cast<int64_t>(t) * a.rows + row] = v;
+                }
+            }
+            continue;
+        }
+        if (leader) {
+#pragma unroll
+            for (int t = 0; t < NT; t++) part[(wave * NT + t) * RPW + r] = acc[t];
+        }
+        __syncthreads();
+        for (int i = tid; i < tiles_per_wg * NT * RPW; i += 256) {
+            const int rr = i % RPW;
+            const int t = (i / RPW) % NT;
+            const int tw = i / (RPW * NT);
+            const int orow = (blockIdx.x * tiles_per_wg + tw) * RPW + rr;
+            if (orow >= a.rows || t >= n_here) continue;
+            float v = part[((tw * W) * NT + t) * RPW + rr];
+            for (int k = 1; k < W; k++) v = v + part[((tw * W + k) * NT + t) * RPW + rr];
+            if (NT == 1 && a.residual) v = v + a.residual[orow];
+            out[static_cast<int64_t>(t) * a.rows + orow] = v;
+        }
     }
 }
 
@@ -237,15 +275,20 @@ static int pick_ksplit_q6k(int64_t rows, int64_t n_sb) {
     return 4;
 }
 
+static size_t q6k_lds_bytes(int nt, int n_sb) {
+    return static_cast<size_t>(nt) * n_sb * (256 + 64) + ((static_cast<size_t>(nt) * n_sb + 3) & ~size_t(3)) * 4 + 4 * nt * 8 * 4;
+}
+
 template <int NT>
-static int launch_q6k_nt(const Q6KArgs &ka, int n_bands, bool ints, hipStream_t st) {
+static int launch_q6k_nt(const Q6KArgs &ka, int n_bands, bool ints, bool grouped, hipStream_t st) {
     const int tiles_per_wg = 4 / ka.ksplit;
     const int64_t tiles = (ka.rows + 7) / 8;
     const unsigned gx = static_cast<unsigned>((tiles + tiles_per_wg - 1) / tiles_per_wg);
-    const size_t lds = static_cast<size_t>(NT) * ka.n_sb * (256 + 64) + ((static_cast<size_t>(NT) * ka.n_sb + 3) & ~size_t(3)) * 4 +
-                       4 * NT * 8 * 4;
+    const size_t lds = q6k_lds_bytes(NT, ka.n_sb);
     if (lds > 64 * 1024) return fail(CML_ERR_UNSUPPORTED, "Q6_K activation of %d super-blocks x %d tokens exceeds the LDS staging limit", ka.n_sb, NT);
-    if (ints && NT == 1)
+    if (grouped)
+        hipLaunchKernelGGL((gemv_q6k_kernel<NT, false, true>), dim3(gx, n_bands), dim3(256), lds, st, ka);
+    else if (ints && NT == 1)
         hipLaunchKernelGGL((gemv_q6k_kernel<1, true>), dim3(gx, n_bands), dim3(256), lds, st, ka);
     else
         hipLaunchKernelGGL((gemv_q6k_kernel<NT, false>), dim3(gx, n_bands), dim3(256), lds, st, ka);
@@ -256,20 +299,39 @@ static int launch_q6k_nt(const Q6KArgs &ka, int n_bands, bool ints, hipStream_t 
 int launch_gemv_q6k(const MatArgs &a, hipStream_t st) {
     const cml_weight *w = a.w;
     if (w->rows == 0 || a.n_tokens == 0) return CML_OK;
-    if (a.group_offsets) return fail(CML_ERR_UNSUPPORTED, "grouped (mixture-of-experts) dispatch is built for Q4_K weights only");
-    Q6KArgs ka;
+    const bool grouped = a.group_offsets != nullptr || a.group_ids != nullptr;
+    Q6KArgs ka{};
     ka.ql = w->planes.p[0]; ka.ql_stride = w->planes.row_stride[0];
     ka.qh = w->planes.p[1]; ka.qh_stride = w->planes.row_stride[1];
     ka.sc = w->planes.p[2]; ka.sc_stride = w->planes.row_stride[2];
     ka.d = w->planes.p[3];  ka.d_stride = w->planes.row_stride[3];
-    ka.rows = static_cast<int>(w->rows);
+    ka.rows = static_cast<int>(grouped ? a.band_rows : w->rows);
     ka.n_sb = static_cast<int>(w->nb);
     ka.residual = a.residual;
     ka.ints = a.ints;
-    ka.band_ids = nullptr;
-    ka.act_slot_stride = 0;
-    ka.out_slot_stride = a.n_tokens * static_cast<int64_t>(ka.rows);
+    ka.group_offsets = a.group_offsets;
+    ka.group_rows = a.group_rows;
+    ka.group_ids = a.group_ids;
+    ka.n_groups = a.n_groups;
     ka.ksplit = pick_ksplit_q6k(ka.rows, ka.n_sb);
+    if (grouped) {
+        if (a.band_rows <= 0 || a.band_rows * a.n_groups != w->rows)
+            return fail(CML_ERR_SHAPE, "%d bands of %lld rows do not cover %lld rows", a.n_groups, (long long)a.band_rows, (long long)w->rows);
+        // One launch: every group walks its own assignments in passes of NT, NT sized for the most
+        // a single group can hold and for the LDS staging limit.
+        ka.q = a.q;
+        ka.yd = a.scales;
+        ka.out = a.out;
+        int nt = a.n_tokens >= 8 ? 8 : (a.n_tokens >= 4 ? 4 : (a.n_tokens >= 2 ? 2 : 1));
+        while (nt > 1 && q6k_lds_bytes(nt, ka.n_sb) > 64 * 1024) nt /= 2;
+        const int slots = a.group_ids ? a.max_active : a.n_groups;
+        switch (nt) {
+            case 8: return launch_q6k_nt<8>(ka, slots, false, true, st);
+            case 4: return launch_q6k_nt<4>(ka, slots, false, true, st);
+            case 2: return launch_q6k_nt<2>(ka, slots, false, true, st);
+            default: return launch_q6k_nt<1>(ka, slots, false, true, st);
+        }
+    }
     const int n_bands = 1;
     int64_t t0 = 0;
     while (t0 < a.n_tokens) {
@@ -280,10 +342,10 @@ int launch_gemv_q6k(const MatArgs &a, hipStream_t st) {
         ka.out = a.out + t0 * ka.rows;
         int rc;
         switch (nt) {
-            case 8: rc = launch_q6k_nt<8>(ka, n_bands, false, st); break;
-            case 4: rc = launch_q6k_nt<4>(ka, n_bands, false, st); break;
-            case 2: rc = launch_q6k_nt<2>(ka, n_bands, false, st); break;
-            default: rc = launch_q6k_nt<1>(ka, n_bands, a.ints != nullptr, st); break;
+            case 8: rc = launch_q6k_nt<8>(ka, n_bands, false, false, st); break;
+            case 4: rc = launch_q6k_nt<4>(ka, n_bands, false, false, st); break;
+            case 2: rc = launch_q6k_nt<2>(ka, n_bands, false, false, st); break;
+            default: rc = launch_q6k_nt<1>(ka, n_bands, a.ints != nullptr, false, st); break;
         }
         if (rc != CML_OK) return rc;
         t0 += nt;

@@ -246,14 +246,15 @@ __global__ __launch_bounds__(kPlanThreads) void moe_plan_kernel(const int32_t *_
 // Expert-grouped matmul: the packed-dot kernel for a few tokens, the matrix cores from 4 tokens
 // up (the same crossover as for plain calls).  Both produce the same bits per cell.
 static int launch_expert_matmul(const MatArgs &a, hipStream_t st) {
+    if (a.w->fmt == CML_Q6_K) return launch_gemv_q6k(a, st);
     if (a.w->fmt != CML_Q4_K) return launch_gemv_b32_grouped(a, GroupedPrologue{}, st);
     if (a.group_offsets && a.n_tokens >= env_int("CAMELID_HIP_Q4K_MFMA_MIN_TOKENS", 4)) return launch_gemm_q4k_mfma(a, st);
     return launch_gemv_q4k(a, st);
 }
 
-static bool expert_format(int fmt) { return fmt == CML_Q4_K || fmt == CML_Q8_0 || fmt == CML_Q4_0; }
+static bool expert_format(int fmt) { return fmt == CML_Q4_K || fmt == CML_Q6_K || fmt == CML_Q8_0 || fmt == CML_Q4_0; }
 // Activation quantization an expert matrix of this format is dotted with: 2 = Q8_K, 1 = Q8_0.
-static int act_of(int fmt) { return fmt == CML_Q4_K ? 2 : 1; }
+static int act_of(int fmt) { return is_k_family(fmt) ? 2 : 1; }
 static int launch_quantize_act(int act, const float *x, int64_t n, int64_t cols, int8_t *q, float *s, hipStream_t st) {
     return act == 2 ? launch_quantize_q8_k(x, n, cols, q, s, st) : launch_quantize_q8_0(x, n, cols, q, s, st);
 }
@@ -363,7 +364,7 @@ int cml_moe_gemv_routed(const cml_weight *experts, int n_experts, const int8_t *
                         int max_union, int64_t max_assignments_per_expert, float *out_dev, cml_stream_t stream) {
     if (!ready()) return fail(CML_ERR_UNAVAILABLE, "cml_init has not succeeded");
     if (!experts) return fail(CML_ERR_INVALID, "null weight");
-    if (!expert_format(experts->fmt)) return fail(CML_ERR_UNSUPPORTED, "routed matvec is built for Q4_K, Q8_0 and Q4_0 expert matrices");
+    if (!expert_format(experts->fmt)) return fail(CML_ERR_UNSUPPORTED, "routed matvec is built for Q4_K, Q6_K, Q8_0 and Q4_0 expert matrices");
     if (n_experts <= 0 || n_experts > kMaxExperts || experts->rows % n_experts != 0)
         return fail(CML_ERR_SHAPE, "%lld rows do not stack to %d experts", (long long)experts->rows, n_experts);
     if (max_assignments_per_expert < 0 || (union_experts_dev && (max_union <= 0 || max_union > n_experts)))
@@ -419,7 +420,7 @@ int cml_moe_ffn_ex(const cml_weight *gate, const cml_weight *up, const cml_weigh
     if (glu != CML_GLU_SILU && glu != CML_GLU_GELU_TANH) return fail(CML_ERR_INVALID, "unknown expert activation %d", glu);
     const bool fused_gate_up = up == nullptr;  // `gate` holds gate|up experts of 2*ff rows each
     if (!expert_format(gate->fmt) || (up && up->fmt != gate->fmt) || !expert_format(down->fmt))
-        return fail(CML_ERR_UNSUPPORTED, "mixture-of-experts dispatch is built for Q4_K, Q8_0 and Q4_0 expert matrices (gate and up alike)");
+        return fail(CML_ERR_UNSUPPORTED, "mixture-of-experts dispatch is built for Q4_K, Q6_K, Q8_0 and Q4_0 expert matrices (gate and up alike)");
     if (n_experts <= 0 || n_experts > kMaxExperts || k <= 0 || k > n_experts || n_tokens < 0)
         return fail(CML_ERR_SHAPE, "bad routing shape (%d experts, top-%d)", n_experts, k);
     const int64_t hidden = gate->cols, ff = down->cols;
@@ -440,7 +441,8 @@ int cml_moe_ffn_ex(const cml_weight *gate, const cml_weight *up, const cml_weigh
 
     // Decode (one token, rows of up to 4096 values): gate and up run as ONE launch that quantizes
     // the token inside every workgroup -- two launches and the quantized round trip fewer.
-    const bool fused_decode = n_tokens == 1 && (act_in == 1 || hidden / 256 <= 16) && env_int("CAMELID_HIP_FUSED_QUANT", 1) != 0;
+    const bool fused_decode = n_tokens == 1 && (act_in == 1 || (gate->fmt == CML_Q4_K && hidden / 256 <= 16)) &&
+                              env_int("CAMELID_HIP_FUSED_QUANT", 1) != 0;
     // ws.g and ws.u are adjacent: a fused gate|up projection writes rows of 2*ff values across both
     const int64_t glu_stride = fused_gate_up ? 2 * ff : ff;
     const float *u_rows = fused_gate_up ? ws.g + ff : ws.u;

@@ -116,6 +116,31 @@ def test_moe_ffn_small_matches_oracle(T):
     assert G.max_rel(got2, want) <= 1e-5
 
 
+@pytest.mark.parametrize("T", [1, 2, 5, 32])
+def test_moe_ffn_mixtral_with_q6k_down_matches_oracle(T):
+    """Q4_K_M-style files keep some expert down projections in Q6_K: gate / up Q4_K, down Q6_K."""
+    E, k, hidden, ff = 8, 2, 512, 1024
+    gate = G.synth_weight(B.CML_Q4_K, E * ff, hidden, 312)
+    up = G.synth_weight(B.CML_Q4_K, E * ff, hidden, 313)
+    down = G.synth_weight(B.CML_Q6_K, E * hidden, ff, 314)
+    rng = np.random.default_rng(315 + T)
+    x = rng.standard_normal((T, hidden)).astype(np.float32)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    if T >= 5:
+        logits[:, 3] += 4.0
+    G.say(f"moe ffn Q4_K gate/up + Q6_K down T={T}")
+    wg = Weight.upload(B.CML_Q4_K, E * ff, hidden, gate)
+    wu = Weight.upload(B.CML_Q4_K, E * ff, hidden, up)
+    wd = Weight.upload(B.CML_Q6_K, E * hidden, ff, down)
+    idx_dev, w_dev, idx, w = gpu_route(logits, k)
+    want = oracle.moe_ffn_ex(B.CML_Q4_K, gate, up, down, E, k, hidden, ff, logits, x, threads=8, fmt_down=B.CML_Q6_K)
+    with G.env(CAMELID_HIP_EXACT_ORDER="1"):
+        got = gpu_moe(wg, wu, wd, E, k, idx_dev, w_dev, x)
+    assert G.max_rel(got, want) <= 1e-5
+    got2 = gpu_moe(wg, wu, wd, E, k, idx_dev, w_dev, x)   # default K-split policy
+    assert G.max_rel(got2, want) <= 1e-5
+
+
 def test_moe_ffn_is_the_sum_of_single_expert_calls():
     """Grouping must not change any (token, expert) cell: compare with per-token, per-expert
     matvecs through the plain entry points, mixed on the host in routed order."""
@@ -232,6 +257,9 @@ GEMMA_SMALL = [
     (B.CML_Q8_0, B.CML_Q8_0, 352, 96),
     (B.CML_Q4_0, B.CML_Q8_0, 512, 704),
     (B.CML_Q4_K, B.CML_Q4_0, 256, 96),
+    (B.CML_Q4_K, B.CML_Q6_K, 256, 512),
+    (B.CML_Q6_K, B.CML_Q6_K, 512, 256),
+    (B.CML_Q8_0, B.CML_Q6_K, 96, 256),
 ]
 
 
@@ -264,7 +292,8 @@ def test_moe_ffn_ex_gemma4_small_matches_oracle(fmt, fmt_down, hidden, ff, T):
     assert G.max_rel(got2, want) <= 1e-5
 
 
-@pytest.mark.parametrize("fmt,fmt_down", [(B.CML_Q4_0, B.CML_Q4_0), (B.CML_Q8_0, B.CML_Q4_0), (B.CML_Q4_0, B.CML_Q4_K)])
+@pytest.mark.parametrize("fmt,fmt_down", [(B.CML_Q4_0, B.CML_Q4_0), (B.CML_Q8_0, B.CML_Q4_0), (B.CML_Q4_0, B.CML_Q4_K),
+                                          (B.CML_Q4_K, B.CML_Q6_K), (B.CML_Q6_K, B.CML_Q8_0)])
 def test_moe_ffn_ex_is_the_sum_of_single_expert_calls(fmt, fmt_down):
     """Grouping must not change any (token, expert) cell, for the 32-value formats too: compare
     with per-token, per-expert matvecs through the plain entry points, mixed on the host."""
@@ -300,7 +329,7 @@ def test_moe_ffn_ex_rejects_bad_arguments():
     L = lib()
     args = (E, k, d.ptr, d.ptr, d.ptr, 1, d.ptr, d.ptr, 1 << 20)
     assert L.cml_moe_ffn_ex(wgu.handle, None, wd.handle, *args, 7, None) == 2        # unknown activation
-    assert L.cml_moe_ffn_ex(w6.handle, None, wd.handle, *args, 1, None) == 6         # Q6_K experts
+    assert L.cml_moe_ffn_ex(w6.handle, None, wd.handle, *args, 1, None) == 3         # a 256-row Q6_K tensor is not 4 x 512 rows
     assert L.cml_moe_ffn_ex(wgu.handle, wd.handle, wd.handle, *args, 1, None) == 3   # up of another shape
     assert L.cml_moe_ffn_ex(wgu.handle, None, wd.handle, E, k, d.ptr, d.ptr, d.ptr, 1, d.ptr, d.ptr, 16, 1, None) == 3  # workspace
     assert L.cml_moe_ffn(wgu.handle, None, wd.handle, *args, None) == 2              # the plain entry needs up
@@ -425,7 +454,7 @@ def test_moe_pieces_reject_bad_arguments():
     assert L.cml_moe_plan(d.ptr, 4, 2, 129, d.ptr, d.ptr, d.ptr, d.ptr, None) == 6
     assert L.cml_moe_plan(d.ptr, 4, 0, 8, d.ptr, d.ptr, d.ptr, d.ptr, None) == 3
     assert L.cml_moe_plan(None, 4, 2, 8, d.ptr, d.ptr, d.ptr, d.ptr, None) == 2
-    assert L.cml_moe_gemv_routed(w6.handle, 2, d.ptr, d.ptr, d.ptr, None, None, 0, 1, d.ptr, None) == 6
+    assert L.cml_moe_gemv_routed(w6.handle, 3, d.ptr, d.ptr, d.ptr, None, None, 0, 1, d.ptr, None) == 3   # 256 rows, 3 experts
     assert L.cml_moe_gemv_routed(w4.handle, 5, d.ptr, d.ptr, d.ptr, None, None, 0, 1, d.ptr, None) == 3   # 96 rows, 5 experts
     assert L.cml_moe_gemv_routed(w4.handle, 4, None, d.ptr, d.ptr, None, None, 0, 1, d.ptr, None) == 2
     assert L.cml_moe_gemv_routed(w4.handle, 4, d.ptr, d.ptr, d.ptr, None, None, 0, 0, d.ptr, None) == 0   # nothing routed
