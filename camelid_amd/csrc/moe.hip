@@ -264,14 +264,14 @@ static int launch_quantize_act(int act, const float *x, int64_t n, int64_t cols,
 // multiply and add rounded separately).
 __global__ __launch_bounds__(256) void moe_weighted_sum_kernel(const float *__restrict__ y, const int32_t *__restrict__ slot_to_assign,
                                                                const float *__restrict__ weight, int k, int64_t hidden,
-                                                               float *__restrict__ out) {
+                                                               int64_t n_assign, float *__restrict__ out) {
     const int64_t c = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     const int64_t t = blockIdx.y;
     if (c >= hidden) return;
     float acc = 0.0f;
     for (int s = 0; s < k; s++) {
         const int64_t a = slot_to_assign ? slot_to_assign[t * k + s] : t * k + s;
-        if (a < 0) continue;  // a slot whose expert id was out of range
+        if (a < 0 || a >= n_assign) continue;  // a dropped slot (expert id out of range) or a malformed map
         acc = acc + y[a * hidden + c] * weight[t * k + s];
     }
     out[t * hidden + c] = acc;
@@ -394,7 +394,7 @@ int cml_moe_weighted_sum(const float *y_dev, const int32_t *route_to_assignment_
     if (n_tokens == 0) return CML_OK;
     if (!y_dev || !weight_dev || !out_dev) return fail(CML_ERR_INVALID, "null pointer");
     hipLaunchKernelGGL(moe_weighted_sum_kernel, dim3(static_cast<unsigned>((hidden + 255) / 256), static_cast<unsigned>(n_tokens)), dim3(256), 0,
-                       as_stream(stream), y_dev, route_to_assignment_dev, weight_dev, k, hidden, out_dev);
+                       as_stream(stream), y_dev, route_to_assignment_dev, weight_dev, k, hidden, n_tokens * k, out_dev);
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }
@@ -515,7 +515,7 @@ int cml_moe_ffn_ex(const cml_weight *gate, const cml_weight *up, const cml_weigh
         if (int rc = launch_expert_matmul(a, st)) return rc;
     }
     hipLaunchKernelGGL(moe_weighted_sum_kernel, dim3(static_cast<unsigned>((hidden + 255) / 256), static_cast<unsigned>(n_tokens)), dim3(256), 0, st,
-                       ws.y, direct ? nullptr : ws.slot_to_assign, weight_dev, k, hidden, out_dev);
+                       ws.y, direct ? nullptr : ws.slot_to_assign, weight_dev, k, hidden, static_cast<int64_t>(n_slots), out_dev);
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }

@@ -460,3 +460,52 @@ def test_moe_pieces_reject_bad_arguments():
     assert L.cml_moe_gemv_routed(w4.handle, 4, d.ptr, d.ptr, d.ptr, None, None, 0, 0, d.ptr, None) == 0   # nothing routed
     assert L.cml_moe_weighted_sum(None, None, d.ptr, 1, 2, 64, d.ptr, None) == 2
     assert L.cml_moe_weighted_sum(d.ptr, None, d.ptr, 0, 2, 64, d.ptr, None) == 0
+
+
+def test_weighted_sum_maps_grouped_assignments_in_router_order_bitwise():
+    """The reference's own fixture for the routed weighted sum (moe_weighted_sum_batched_maps_csr_
+    assignments_in_router_order_bitwise, src/cuda_resident/tests.rs:12603-12735): 15 tokens x 8
+    routes over 32 experts, expert of (token, route) = (7*route + 3*token) % 32, experts reused
+    across tokens, so the grouped order is not router order.  The plan built on the device must be
+    the expert-major map the fixture constructs, and the sum must walk ranks 0..7 with a separately
+    rounded multiply and add."""
+    T, R, E, hidden = 15, 8, 32, 2816
+    experts = np.array([[(r * 7 + t * 3) % E for r in range(R)] for t in range(T)], np.int32)
+    assert all(len(set(row)) == R for row in experts)
+    want_map = np.full(T * R, -1, np.int32)
+    n = 0
+    for e in range(E):
+        for t in range(T):
+            for r in range(R):
+                if experts[t, r] == e:
+                    want_map[t * R + r] = n
+                    n += 1
+    assert n == T * R and list(want_map) != list(range(T * R))
+    G.say("moe weighted sum: reference fixture 15x8 over 32 experts")
+    (off, tok, r2a, uni), (_, _, got_map, _) = gpu_plan(experts, E)
+    assert list(got_map) == list(want_map)
+    rng = np.random.default_rng(420)
+    y = (rng.standard_normal((T * R, hidden)) * (1 + np.arange(T * R)[:, None] / 64.0)).astype(np.float32)
+    scales = (0.0125 + (np.arange(T * R) % R) * 0.017 + rng.uniform(0, 0.01, T * R)).astype(np.float32)
+    yd, sd = DeviceBuffer.from_numpy(y), DeviceBuffer.from_numpy(scales)
+    out = DeviceBuffer(T * hidden * 4)
+    check(lib().cml_moe_weighted_sum(yd.ptr, r2a.ptr, sd.ptr, T, R, hidden, out.ptr, None), "cml_moe_weighted_sum")
+    check(lib().cml_stream_sync(None))
+    got = out.to_numpy(np.float32, (T, hidden))
+    want = np.zeros((T, hidden), np.float32)
+    for t in range(T):
+        for r in range(R):
+            want[t] = want[t] + (y[want_map[t * R + r]] * scales[t * R + r]).astype(np.float32)
+    assert G.same_bits(got, want) and np.any(got != 0)
+    # a malformed map entry is skipped, not read
+    bad = want_map.copy()
+    bad[5] = T * R + 7
+    bd = DeviceBuffer.from_numpy(bad)
+    check(lib().cml_moe_weighted_sum(yd.ptr, bd.ptr, sd.ptr, T, R, hidden, out.ptr, None))
+    check(lib().cml_stream_sync(None))
+    got = out.to_numpy(np.float32, (T, hidden))
+    want0 = np.zeros(hidden, np.float32)
+    for r in range(R):
+        if r != 5:
+            want0 = want0 + (y[want_map[r]] * scales[r]).astype(np.float32)
+    assert G.same_bits(got[0], want0)
