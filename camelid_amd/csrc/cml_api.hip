@@ -497,8 +497,14 @@ static int dispatch(const MatArgs &a, hipStream_t st) {
             else
                 rc = launch_gemv_q4k(a, st);
             break;
-        case CML_Q8_0: rc = launch_gemv_q8_0(a, st); break;
-        case CML_Q4_0: rc = launch_gemv_q4_0(a, st); break;
+        case CML_Q8_0:
+        case CML_Q4_0:
+            // the same split for the 32-value-block formats (rows of whole 256-value slabs)
+            if (!a.group_offsets && !a.ints && a.n_tokens >= b32_mfma_min_tokens(a.w->rows) && b32_mfma_usable(a.w))
+                rc = launch_gemm_b32_mfma(a, st);
+            else
+                rc = a.w->fmt == CML_Q8_0 ? launch_gemv_q8_0(a, st) : launch_gemv_q4_0(a, st);
+            break;
         case CML_Q6_K: rc = launch_gemv_q6k(a, st); break;
         default: return fail(CML_ERR_INVALID, "unknown weight format %d", a.w->fmt);
     }

@@ -101,6 +101,7 @@ struct MatArgs {
     // y-slots (at least the number of groups that can be non-empty) instead of n_groups.
     const int32_t *group_ids;      // device, [n_groups] or null
     int max_active;
+    int64_t n_assign_total;        // all assignments of a grouped call (0 = unknown): sizes the expected group
     int n_groups;
     int64_t band_rows;
 };
@@ -128,6 +129,9 @@ int launch_gemv_q6k(const MatArgs &a, hipStream_t st);
 
 int launch_gemm_q4k(const MatArgs &a, hipStream_t st);
 int launch_gemm_q4k_mfma(const MatArgs &a, hipStream_t st);  // plain calls, n_tokens >= 16
+int launch_gemm_b32_mfma(const MatArgs &a, hipStream_t st);  // Q8_0 / Q4_0 on the matrix cores; plain or grouped
+bool b32_mfma_usable(const cml_weight *w);                   // rows of whole 256-value slabs
+int b32_mfma_min_tokens(int64_t rows);                       // batch size from which it pays
 int launch_gemm_q8_0(const MatArgs &a, hipStream_t st);
 int launch_gemm_q4_0(const MatArgs &a, hipStream_t st);
 int launch_gemm_q6k(const MatArgs &a, hipStream_t st);

@@ -1,0 +1,433 @@
+// Q8_0 x Q8_0 and Q4_0 x Q8_0 small-batch matmul on the int8 matrix cores
+// (gfx950), for batches of several tokens: speculative-verify chunks and short
+// prefill on the 32-value-block formats.
+//
+// Arithmetic: identical, cell by cell, to the matvec kernel (gemv_q8q4.hip;
+// reference q8_0_wire_row_dot_scalar, src/inference.rs:22729-22745;
+// q4_0_wire_row_dot_scalar, :22778-22798): per 32-value block, in block order,
+//     isum = sum_j w_j * x_j                  (exact i32; Q4_0 weights are nibble - 8)
+//     acc  = acc + ((float)isum * d_w) * d_x
+// Every block has its own f32 step, so one matrix instruction covers exactly one
+// block: v_mfma_i32_16x16x32_i8, K = 32.
+//     A[t][k]  = x_t[32b + k]          16 tokens, from LDS
+//     B[k][n]  = w_n[32b + k]          16 rows, straight from the weight plane
+//     D[t][n]  = isum                  (Q4_0: C[t][n] = -8 * sum_k x_t[32b+k] carries the bias)
+// Lane L supplies A-row t = L%16 and B-column n = L%16 at k-octet L/16, and
+// receives D[4*(L/16)+v][L%16], v < 4: four tokens of one weight row, whose f32
+// chains live in that lane, in block order.  The contraction index inside a
+// block may be permuted freely (the sum is an exact integer), which is what makes
+// the plain row-major weight plane usable without a re-layout.  The four lanes of
+// a weight row load 64 contiguous bytes (16 each; narrower loads per lane were
+// measured at a fraction of the bandwidth) and trade pieces with lane-swap
+// instructions so that each ends up with its k-octet of every block:
+//   Q8_0: 64 bytes = 2 blocks.  v_permlane32_swap hands each lane one 8-byte
+//         octet of either block; lane octet kq supplies bytes 8*p..8*p+7 of a
+//         block, p = {0, 2, 1, 3}[kq].
+//   Q4_0: 64 bytes = 4 blocks, one per lane.  A 4x4 transpose (v_permlane32_swap,
+//         v_permlane16_swap) leaves lane kq with bytes 4kq..4kq+3 of each block:
+//         its low nibbles are values 4kq..4kq+3, its high nibbles 16+4kq..16+4kq+3.
+// The activations are staged in LDS in the matching order, the two octets a lane
+// needs of a pair of blocks side by side (one 16-byte LDS read per pair).
+//
+// A workgroup is 4 waves: 4/TB consecutive 16-row tiles x TB token blocks of
+// 16*GPW tokens, sharing the staged activations of NTOK = 16*GPW*TB tokens.  K is
+// walked in slabs of 256 values (8 blocks; rows must be whole slabs -- other
+// lengths take the packed-dot kernel), phases of KC slabs double-buffered in LDS
+// as in the Q4_K matrix-core kernel; weights stream through a register ring of
+// RING slabs per wave.
+#include <type_traits>
+
+#include "cml_device.hpp"
+#include "cml_host.hpp"
+
+#pragma clang fp contract(off)
+
+namespace cml {
+
+typedef int v4i_b32 __attribute__((ext_vector_type(4)));
+typedef int v2i_b32 __attribute__((ext_vector_type(2)));
+
+constexpr int kB32SlabRow = 256 + 16;  // bytes of one token's 256-value slab in LDS (padded)
+
+struct B32MfmaArgs {
+    const uint8_t *quants;  // plane 0, row-major
+    int64_t q_stride;
+    const uint8_t *scales;  // plane 1: f16 per block, row-major
+    int64_t s_stride;
+    int rows, n_slabs;      // rows of one band; 256-value slabs per row
+    const int8_t *q;        // [n_tokens][n_slabs*256]
+    const float *xs;        // [n_tokens][n_slabs*8]
+    float *out;             // [n_tokens][rows]
+    int n_tokens;           // plain: activation rows; grouped: the most assignments one group can hold
+    // Grouped call (mixture of experts): blockIdx.z -> group e (through group_ids when set; -1 =
+    // unused slot), which owns the band of rows [e*rows, (e+1)*rows) and the assignments
+    // [group_offsets[e], group_offsets[e+1]); assignment j reads activation row group_rows[j] (j
+    // itself when null) and writes output row j.
+    const int32_t *group_offsets;
+    const int32_t *group_rows;
+    const int32_t *group_ids;
+};
+
+template <int FMT>
+struct B32SlabWeights {
+    static constexpr int kPieces = FMT == CML_Q8_0 ? 4 : 2;  // 16-byte loads per slab and lane
+    uint4 piece[kPieces];
+    uint4 d;  // the slab's eight f16 block scales
+};
+
+// qlane already includes the lane's 16 * kq.
+template <int FMT>
+__device__ __forceinline__ void b32_mfma_load(B32SlabWeights<FMT> &r, const uint8_t *qlane, const uint8_t *srow, int64_t slab) {
+    constexpr int slab_bytes = FMT == CML_Q8_0 ? 256 : 128;
+#pragma unroll
+    for (int i = 0; i < B32SlabWeights<FMT>::kPieces; i++) r.piece[i] = ldg16(qlane + slab * slab_bytes + i * 64);
+    r.d = ldg16(srow + slab * 16);
+}
+
+typedef unsigned v2u_b32 __attribute__((ext_vector_type(2)));
+// vdst's lanes 32..63 trade places with src's lanes 0..31
+__device__ __forceinline__ void swap32(uint32_t &vdst, uint32_t &src) {
+    const v2u_b32 r = __builtin_amdgcn_permlane32_swap(vdst, src, false, false);
+    vdst = r.x;
+    src = r.y;
+}
+// vdst's odd 16-lane rows trade places with src's even rows
+__device__ __forceinline__ void swap16(uint32_t &vdst, uint32_t &src) {
+    const v2u_b32 r = __builtin_amdgcn_permlane16_swap(vdst, src, false, false);
+    vdst = r.x;
+    src = r.y;
+}
+
+// The eight B operands (one per block of the slab) of this lane.
+template <int FMT>
+__device__ __forceinline__ void b32_mfma_operands(const B32SlabWeights<FMT> &r, long (&bw)[8]) {
+    auto pack = [](uint32_t lo, uint32_t hi) __attribute__((always_inline)) {
+        return static_cast<long>(static_cast<unsigned long long>(lo) | (static_cast<unsigned long long>(hi) << 32));
+    };
+    if constexpr (FMT == CML_Q8_0) {
+        // piece i: lanes kq = 0, 1 hold block 2i (its halves), lanes 2, 3 block 2i+1
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            uint32_t a0 = r.piece[i].x, a1 = r.piece[i].y, b0 = r.piece[i].z, b1 = r.piece[i].w;
+            swap32(a0, b0);
+            swap32(a1, b1);
+            bw[2 * i] = pack(a0, a1);      // an octet of block 2i
+            bw[2 * i + 1] = pack(b0, b1);  // an octet of block 2i+1
+        }
+    } else {
+        // piece i: lane kq holds block 4i + kq; transpose so that it holds word kq of blocks 4i..4i+3
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            uint32_t r0 = r.piece[i].x, r1 = r.piece[i].y, r2 = r.piece[i].z, r3 = r.piece[i].w;
+            swap32(r0, r2);
+            swap32(r1, r3);
+            swap16(r0, r1);
+            swap16(r2, r3);
+            const uint32_t w[4] = {r0, r1, r2, r3};
+#pragma unroll
+            for (int j = 0; j < 4; j++) bw[4 * i + j] = pack(w[j] & 0x0f0f0f0fu, (w[j] >> 4) & 0x0f0f0f0fu);
+        }
+    }
+}
+
+// KC = slabs per phase (LDS holds two phases of NTOK tokens), RING = weight slabs a wave keeps in
+// flight in registers.
+// A workgroup's 4 waves are 4/TB consecutive row tiles x TB token blocks of 16*GPW tokens.
+template <int FMT, int GPW, int TB, int KC, int RING>
+__global__ __launch_bounds__(256) void gemm_b32_mfma_kernel(B32MfmaArgs a) {
+    constexpr int NTOK = 16 * GPW * TB;              // tokens staged per workgroup
+    constexpr int RT = 4 / TB;                       // row tiles per workgroup
+    constexpr int kBufBytes = KC * NTOK * kB32SlabRow;
+    constexpr int kBsInts = KC * 8 * NTOK;           // per buffer: -8 * block sums, [slab][block][token]
+    constexpr int nthreads = 256;
+    constexpr int kPer = NTOK * 16 / nthreads;       // 16-byte pieces of one slab of all tokens, per thread
+    static_assert(RING % KC == 0 && kPer >= 1, "phase / staging shape");
+    extern __shared__ uint4 smem[];
+    uint8_t *buf0 = reinterpret_cast<uint8_t *>(smem);  // [KC][NTOK][kB32SlabRow]
+    uint8_t *buf1 = buf0 + kBufBytes;
+    int *bs0 = reinterpret_cast<int *>(buf1 + kBufBytes);  // Q4_0 only
+    int *bs1 = bs0 + (FMT == CML_Q4_0 ? kBsInts : 0);
+    float *xss = reinterpret_cast<float *>(bs1 + (FMT == CML_Q4_0 ? kBsInts : 0));  // [n_slabs*8][NTOK]
+
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    const int n_slabs = a.n_slabs;
+    const int n = lane & 15, kq = lane >> 4;  // B/D column (weight row in tile) and k-octet / A-row quad
+    const int n_tiles = (a.rows + 15) / 16;
+    const int rt = wave / TB, tb = wave - rt * TB;
+    const int tile = blockIdx.x * RT + rt;
+    const int row = tile * 16 + n;
+    const bool grouped = a.group_offsets != nullptr;
+    const int64_t band = grouped ? (a.group_ids ? a.group_ids[blockIdx.z] : static_cast<int>(blockIdx.z)) : 0;
+    if (band < 0) return;  // a z-slot past the groups in use
+    const int a0 = grouped ? a.group_offsets[band] : 0;  // first assignment of this group
+    const int n_assign = grouped ? a.group_offsets[band + 1] - a0 : a.n_tokens;
+    const int tok0 = blockIdx.y * NTOK;  // first token (assignment of the group) of this workgroup
+    if (tok0 >= n_assign) return;        // nothing routed here: the whole workgroup leaves
+    const int n_here = min(NTOK, n_assign - tok0);
+    // activation row of local token t (tokens past the end repeat the last one; their cells are not stored)
+    auto act_row = [&](int t) __attribute__((always_inline)) -> int64_t {
+        const int j = a0 + tok0 + min(t, n_here - 1);
+        return a.group_rows ? a.group_rows[j] : j;
+    };
+
+    // activation scales: xss[block][token]
+    const int nb = n_slabs * 8;
+    for (int i = tid; i < nb * NTOK; i += nthreads) {
+        const int b = i / NTOK, t = i - b * NTOK;
+        xss[i] = a.xs[act_row(t) * nb + b];
+    }
+
+    // Staging: each thread owns kPer fixed (token, piece) pairs; only the slab moves.  Piece pc =
+    // half h = pc & 1 of block pc >> 1.  Destination order inside a slab: [pair of blocks][octet
+    // lane 0..3][block of the pair][8 bytes], so that a lane reads its octets of both blocks of a
+    // pair with one 16-byte load.
+    const v4i_b32 *stage_src[kPer];
+    int stage_dst[kPer], stage_tok[kPer], stage_blk[kPer];
+#pragma unroll
+    for (int k = 0; k < kPer; k++) {
+        const int i = tid + k * nthreads;
+        const int t = i >> 4, pc = i & 15;
+        const int blk = pc >> 1, h = pc & 1;
+        stage_src[k] = reinterpret_cast<const v4i_b32 *>(a.q + act_row(t) * n_slabs * 256) + pc;
+        stage_tok[k] = t;
+        stage_blk[k] = blk;
+        if constexpr (FMT == CML_Q8_0)  // bytes 16h..16h+15 = octets 2h and 2h+1, which go to lane octets h and h + 2
+            stage_dst[k] = t * kB32SlabRow + (blk >> 1) * 64 + h * 16 + (blk & 1) * 8;
+        else  // values 16h..16h+15: dword o of the piece joins octet o at byte 4h
+            stage_dst[k] = t * kB32SlabRow + (blk >> 1) * 64 + (blk & 1) * 8 + h * 4;
+    }
+    v4i_b32 sreg[KC][kPer];
+    auto stage_load = [&](int p0) __attribute__((always_inline)) {  // the KC slabs starting at p0
+#pragma unroll
+        for (int s = 0; s < KC; s++) {
+            const int off = min(p0 + s, n_slabs - 1) * 16;  // in 16-byte units
+#pragma unroll
+            for (int k = 0; k < kPer; k++) sreg[s][k] = stage_src[k][off];
+        }
+    };
+    auto stage_store = [&](uint8_t *buf, int *bs) __attribute__((always_inline)) {
+#pragma unroll
+        for (int s = 0; s < KC; s++)
+#pragma unroll
+            for (int k = 0; k < kPer; k++) {
+                uint8_t *dst = buf + s * (NTOK * kB32SlabRow) + stage_dst[k];
+                const v4i_b32 v = sreg[s][k];
+                if constexpr (FMT == CML_Q8_0) {
+                    *reinterpret_cast<v2i_b32 *>(dst) = v2i_b32{v.x, v.y};
+                    *reinterpret_cast<v2i_b32 *>(dst + 32) = v2i_b32{v.z, v.w};
+                } else {
+                    *reinterpret_cast<int *>(dst) = v.x;
+                    *reinterpret_cast<int *>(dst + 16) = v.y;
+                    *reinterpret_cast<int *>(dst + 32) = v.z;
+                    *reinterpret_cast<int *>(dst + 48) = v.w;
+                    // the block's -8 * sum of activations: the two halves sit in adjacent lanes, which
+                    // swap partial sums and both store the total (a store under a lane condition here
+                    // breaks the straight-line schedule and spills)
+                    int sum = sdot4(static_cast<uint32_t>(v.x), 0x01010101u, 0);
+                    sum = sdot4(static_cast<uint32_t>(v.y), 0x01010101u, sum);
+                    sum = sdot4(static_cast<uint32_t>(v.z), 0x01010101u, sum);
+                    sum = sdot4(static_cast<uint32_t>(v.w), 0x01010101u, sum);
+                    sum += __builtin_amdgcn_update_dpp(0, sum, 0xB1 /* quad_perm [1,0,3,2] */, 0xf, 0xf, false);
+                    bs[(s * 8 + stage_blk[k]) * NTOK + stage_tok[k]] = -8 * sum;
+                }
+            }
+    };
+
+    // Lane constants.
+    const int64_t arow = band * a.rows + min(row, a.rows - 1);
+    const uint8_t *qlane = a.quants + arow * a.q_stride + 16 * kq;
+    const uint8_t *srow = a.scales + arow * a.s_stride;
+    // A operand: this lane is token (lane & 15) of a group, octet kq: 16 bytes per pair of blocks.
+    const int a_off = (lane & 15) * kB32SlabRow + 16 * kq;
+    const int cell_tok = 4 * kq;  // D values v = 0..3 of this lane: tokens 4*kq + v of the group, weight row n
+
+    B32SlabWeights<FMT> ring[RING];
+    auto load_slot = [&](B32SlabWeights<FMT> &r, int slab) __attribute__((always_inline)) { b32_mfma_load<FMT>(r, qlane, srow, min(slab, n_slabs - 1)); };
+
+    stage_load(0);
+#pragma unroll
+    for (int i = 0; i < RING; i++) load_slot(ring[i], i);
+    stage_store(buf0, bs0);
+    __syncthreads();
+
+    float acc[GPW][4];
+#pragma unroll
+    for (int g = 0; g < GPW; g++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[g][j] = 0.0f;
+
+    // One slab (8 blocks) of this wave's tile against its tokens.
+    auto step = [&](const B32SlabWeights<FMT> &w0, int slab, const uint8_t *act, const int *bs) __attribute__((always_inline)) {
+        const uint32_t dwords[4] = {w0.d.x, w0.d.y, w0.d.z, w0.d.w};
+        long bw8[8];
+        b32_mfma_operands<FMT>(w0, bw8);
+#pragma unroll
+        for (int pr = 0; pr < 4; pr++) {
+            const long bw[2] = {bw8[2 * pr], bw8[2 * pr + 1]};
+            const float dw[2] = {f16_bits_to_f32(dwords[pr] & 0xffffu), f16_bits_to_f32(dwords[pr] >> 16)};
+#pragma unroll
+            for (int g = 0; g < GPW; g++) {
+                const v4i_b32 av = *reinterpret_cast<const v4i_b32 *>(act + (tb * GPW + g) * (16 * kB32SlabRow) + a_off + 64 * pr);
+                const long a2[2] = {
+                    static_cast<long>(static_cast<unsigned long long>(static_cast<uint32_t>(av.x)) | (static_cast<unsigned long long>(static_cast<uint32_t>(av.y)) << 32)),
+                    static_cast<long>(static_cast<unsigned long long>(static_cast<uint32_t>(av.z)) | (static_cast<unsigned long long>(static_cast<uint32_t>(av.w)) << 32))};
+#pragma unroll
+                for (int e = 0; e < 2; e++) {
+                    const int b = 2 * pr + e;
+                    v4i_b32 c = {0, 0, 0, 0};
+                    if constexpr (FMT == CML_Q4_0) c = *reinterpret_cast<const v4i_b32 *>(bs + b * NTOK + 16 * (tb * GPW + g) + cell_tok);
+                    const v4i_b32 d = __builtin_amdgcn_mfma_i32_16x16x32_i8(a2[e], bw[e], c, 0, 0, 0);
+                    const float4 xv = *reinterpret_cast<const float4 *>(xss + (slab * 8 + b) * NTOK + 16 * (tb * GPW + g) + cell_tok);
+                    acc[g][0] = acc[g][0] + (static_cast<float>(d[0]) * dw[e]) * xv.x;
+                    acc[g][1] = acc[g][1] + (static_cast<float>(d[1]) * dw[e]) * xv.y;
+                    acc[g][2] = acc[g][2] + (static_cast<float>(d[2]) * dw[e]) * xv.z;
+                    acc[g][3] = acc[g][3] + (static_cast<float>(d[3]) * dw[e]) * xv.w;
+                }
+            }
+        }
+    };
+
+    // Rounds of RING slabs, phases of KC inside them (the schedule of the Q4_K matrix-core
+    // kernel): the next phase's activation loads are issued at a phase start, ahead of younger
+    // weight loads, and stored at its end; the only barriers are the phase boundaries.
+    uint8_t *cur = buf0, *nxt = buf1;
+    int *bcur = bs0, *bnxt = bs1;
+    auto round = [&](int s0, auto refill) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < RING; i++) {
+            const int slab = s0 + i;
+            if (i % KC == 0) {
+                stage_load(slab + KC);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (slab < n_slabs) step(ring[i], slab, cur + (i % KC) * (NTOK * kB32SlabRow), bcur + (i % KC) * (8 * NTOK));
+            if constexpr (GPW > 1) __builtin_amdgcn_sched_barrier(0);
+            if constexpr (decltype(refill)::value) load_slot(ring[i], slab + RING);
+            if (i % KC == KC - 1) {
+                stage_store(nxt, bnxt);
+                __syncthreads();  // next phase complete in `nxt`, everyone done with `cur`
+                uint8_t *t = cur;
+                cur = nxt;
+                nxt = t;
+                int *tb = bcur;
+                bcur = bnxt;
+                bnxt = tb;
+            }
+        }
+    };
+    int s0 = 0;
+    for (; s0 + RING < n_slabs; s0 += RING) round(s0, std::true_type{});
+    round(s0, std::false_type{});
+
+    if (tile < n_tiles && row < a.rows) {
+#pragma unroll
+        for (int g = 0; g < GPW; g++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int t = 16 * (tb * GPW + g) + cell_tok + j;
+                if (t < n_here) a.out[static_cast<int64_t>(a0 + tok0 + t) * a.rows + row] = acc[g][j];
+            }
+    }
+}
+
+template <int FMT, int GPW, int TB, int KC, int RING>
+static int launch_b32_mfma_g(const B32MfmaArgs &ka, int n_groups, hipStream_t st) {
+    constexpr int NTOK = 16 * GPW * TB, RT = 4 / TB;
+    const int n_tiles = (ka.rows + 15) / 16;
+    const unsigned gx = static_cast<unsigned>((n_tiles + RT - 1) / RT);
+    const unsigned gy = static_cast<unsigned>((ka.n_tokens + NTOK - 1) / NTOK);
+    const size_t lds = 2 * static_cast<size_t>(KC * NTOK) * kB32SlabRow + (FMT == CML_Q4_0 ? 2 * static_cast<size_t>(KC * NTOK) * 8 * 4 : 0) +
+                       static_cast<size_t>(ka.n_slabs) * 8 * NTOK * 4;
+    if (lds > 160 * 1024) return fail(CML_ERR_UNSUPPORTED, "matrix-core path: %d blocks per row exceed the LDS budget", ka.n_slabs * 8);
+    static bool raised = false;  // per instantiation: allow more than 64 KB of dynamic LDS once
+    if (!raised) {
+        CML_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_b32_mfma_kernel<FMT, GPW, TB, KC, RING>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        raised = true;
+    }
+    hipLaunchKernelGGL((gemm_b32_mfma_kernel<FMT, GPW, TB, KC, RING>), dim3(gx, gy, n_groups), dim3(256), lds, st, ka);
+    CML_HIP_TRY(hipGetLastError());
+    return CML_OK;
+}
+
+// Phase length and ring depth.  Short phases keep the LDS footprint small, so that several
+// workgroups share a compute unit and cover each other's barriers and load latency: what a large
+// matrix wants (measured at 128256x3072, 8 tokens: 130 us with 128 token-slabs per phase, 60 us with
+// 32).  A matrix with fewer workgroups than compute units gains nothing from that and prefers the
+// deep ring.
+template <int FMT, int GPW, int TB>
+static int launch_b32_mfma_p(const B32MfmaArgs &ka, int n_groups, hipStream_t st) {
+    constexpr int NTOK = 16 * GPW * TB;
+    int deep = env_int("CAMELID_HIP_B32_MFMA_DEEP", -1);
+    if (deep != 0 && deep != 1) deep = (ka.rows + 15) / 16 < 2048 ? 1 : 0;
+    if constexpr (NTOK == 16) {
+        return deep ? launch_b32_mfma_g<FMT, GPW, TB, 8, 8>(ka, n_groups, st) : launch_b32_mfma_g<FMT, GPW, TB, 2, 2>(ka, n_groups, st);
+    } else if constexpr (NTOK == 32) {
+        return deep ? launch_b32_mfma_g<FMT, GPW, TB, 4, 4>(ka, n_groups, st) : launch_b32_mfma_g<FMT, GPW, TB, 2, 2>(ka, n_groups, st);
+    } else {  // 64 tokens: one slab per phase either way, so that two or three workgroups fit a compute unit
+        return deep ? launch_b32_mfma_g<FMT, GPW, TB, 1, 4>(ka, n_groups, st) : launch_b32_mfma_g<FMT, GPW, TB, 1, 2>(ka, n_groups, st);
+    }
+}
+
+template <int FMT>
+static int launch_b32_mfma_fmt(const B32MfmaArgs &ka, int n_groups, bool grouped, hipStream_t st) {
+    // Workgroup shape: token groups per wave x token blocks across waves.  Default: one wave per
+    // row tile with 16 / 32 / 64 tokens; a matrix with fewer row tiles than the chip has SIMDs
+    // spreads the tokens of a tile over 2 or 4 waves instead.
+    switch (env_int("CAMELID_HIP_B32_MFMA_SHAPE", 0)) {
+        case 1: return launch_b32_mfma_p<FMT, 1, 1>(ka, n_groups, st);   // 16 tokens, 1 wave per row tile
+        case 2: return launch_b32_mfma_p<FMT, 2, 1>(ka, n_groups, st);   // 32 tokens, 1 wave per row tile
+        case 3: return launch_b32_mfma_p<FMT, 4, 1>(ka, n_groups, st);   // 64 tokens, 1 wave per row tile
+        case 4: return launch_b32_mfma_p<FMT, 1, 2>(ka, n_groups, st);   // 32 tokens, 2 waves per row tile
+        case 5: return launch_b32_mfma_p<FMT, 2, 2>(ka, n_groups, st);   // 64 tokens, 2 waves per row tile
+        case 6: return launch_b32_mfma_p<FMT, 1, 4>(ka, n_groups, st);   // 64 tokens, 4 waves per row tile
+        default: break;
+    }
+    if (grouped || ka.n_tokens <= 16) return launch_b32_mfma_p<FMT, 1, 1>(ka, n_groups, st);
+    const bool few_tiles = (ka.rows + 15) / 16 < 1024;
+    if (ka.n_tokens <= 32) return few_tiles ? launch_b32_mfma_p<FMT, 1, 2>(ka, n_groups, st) : launch_b32_mfma_p<FMT, 2, 1>(ka, n_groups, st);
+    return few_tiles ? launch_b32_mfma_p<FMT, 1, 4>(ka, n_groups, st) : launch_b32_mfma_p<FMT, 4, 1>(ka, n_groups, st);
+}
+
+// Rows must be whole 256-value slabs whose scale octets can be read with one aligned 16-byte load.
+bool b32_mfma_usable(const cml_weight *w) {
+    return (w->fmt == CML_Q8_0 || w->fmt == CML_Q4_0) && w->nb > 0 && w->nb % 8 == 0 &&
+           (reinterpret_cast<uintptr_t>(w->planes.p[1]) % 16 == 0) && (w->planes.row_stride[1] % 16 == 0);
+}
+
+// Batch size from which the matrix-core kernel beats the packed-dot kernel (which serves up to 8
+// tokens per pass over the weight).  Measured on MI355X: 8192x2048 Q8_0, 4 / 8 tokens: 7.0 / 10.0 us
+// packed dot against 10.9 us; 128256x3072 Q4_0: 62 / 105 us against 59 / 61 us.
+int b32_mfma_min_tokens(int64_t rows) {
+    const int forced = env_int("CAMELID_HIP_B32_MFMA_MIN_TOKENS", 0);
+    if (forced > 0) return forced;
+    return (rows + 15) / 16 >= 2048 ? 5 : 9;
+}
+
+// Q8_0 / Q4_0 matmul on the matrix cores: plain calls, or grouped by expert (mixture of experts).
+int launch_gemm_b32_mfma(const MatArgs &a, hipStream_t st) {
+    const cml_weight *w = a.w;
+    const bool grouped = a.group_offsets != nullptr;
+    if (w->rows == 0 || a.n_tokens == 0) return CML_OK;
+    if (!b32_mfma_usable(w)) return fail(CML_ERR_UNSUPPORTED, "matrix-core path needs rows of whole 256-value slabs");
+    B32MfmaArgs ka{};
+    ka.quants = w->planes.p[0];
+    ka.q_stride = w->planes.row_stride[0];
+    ka.scales = w->planes.p[1];
+    ka.s_stride = w->planes.row_stride[1];
+    ka.rows = static_cast<int>(grouped ? a.band_rows : w->rows);
+    ka.n_slabs = static_cast<int>(w->nb / 8);
+    ka.q = a.q;
+    ka.xs = a.scales;
+    ka.out = a.out;
+    ka.n_tokens = static_cast<int>(a.n_tokens);
+    ka.group_offsets = a.group_offsets;
+    ka.group_rows = a.group_rows;
+    ka.group_ids = a.group_ids;
+    const int ng = grouped ? (a.group_ids ? a.max_active : a.n_groups) : 1;
+    if (w->fmt == CML_Q8_0) return launch_b32_mfma_fmt<CML_Q8_0>(ka, ng, grouped, st);
+    return launch_b32_mfma_fmt<CML_Q4_0>(ka, ng, grouped, st);
+}
+
+}  // namespace cml

@@ -247,7 +247,13 @@ __global__ __launch_bounds__(kPlanThreads) void moe_plan_kernel(const int32_t *_
 // up (the same crossover as for plain calls).  Both produce the same bits per cell.
 static int launch_expert_matmul(const MatArgs &a, hipStream_t st) {
     if (a.w->fmt == CML_Q6_K) return launch_gemv_q6k(a, st);
-    if (a.w->fmt != CML_Q4_K) return launch_gemv_b32_grouped(a, GroupedPrologue{}, st);
+    if (a.w->fmt != CML_Q4_K) {
+        // matrix cores once the groups in use hold enough assignments on average to fill a 16-token tile reasonably
+        const int64_t groups = a.group_ids ? a.max_active : a.n_groups;
+        if (a.group_offsets && b32_mfma_usable(a.w) && a.n_assign_total >= groups * env_int("CAMELID_HIP_B32_MFMA_MIN_GROUP", 6))
+            return launch_gemm_b32_mfma(a, st);
+        return launch_gemv_b32_grouped(a, GroupedPrologue{}, st);
+    }
     if (a.group_offsets && a.n_tokens >= env_int("CAMELID_HIP_Q4K_MFMA_MIN_TOKENS", 4)) return launch_gemm_q4k_mfma(a, st);
     return launch_gemv_q4k(a, st);
 }
@@ -467,6 +473,7 @@ int cml_moe_ffn_ex(const cml_weight *gate, const cml_weight *up, const cml_weigh
     a.group_offsets = direct ? nullptr : ws.offsets;
     a.group_ids = direct ? idx_dev : ws.group_ids;
     a.max_active = direct ? n_slots : static_cast<int>(std::min<int64_t>(n_experts, n_slots));
+    a.n_assign_total = n_slots;
     a.n_groups = n_experts;
     a.n_tokens = n_tokens;  // the most assignments one expert can receive
     // gate and up: every assignment reads its token's activation

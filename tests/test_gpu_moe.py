@@ -509,3 +509,29 @@ def test_weighted_sum_maps_grouped_assignments_in_router_order_bitwise():
         if r != 5:
             want0 = want0 + (y[want_map[r]] * scales[r]).astype(np.float32)
     assert G.same_bits(got[0], want0)
+
+
+@pytest.mark.parametrize("fmt", [B.CML_Q4_0, B.CML_Q8_0])
+def test_moe_batches_on_the_matrix_cores_are_bitwise_the_packed_dot_path(fmt):
+    """Enough assignments per expert send the Q8_0 / Q4_0 expert projections to the matrix-core
+    kernel (grouped mode): the same cells as the packed-dot grouped kernel, bit for bit."""
+    E, k, hidden, ff, T = 8, 2, 512, 256, 70
+    gate_up, down = _experts_fused(fmt, fmt, E, hidden, ff, 430)
+    rng = np.random.default_rng(431)
+    x = rng.standard_normal((T, hidden)).astype(np.float32)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    logits[:, 5] += 2.0       # one crowded expert: several 16-token blocks in its group
+    logits[:, 1] -= 50.0      # and one that nobody picks
+    wgu = Weight.upload(fmt, E * 2 * ff, hidden, gate_up)
+    wd = Weight.upload(fmt, E * hidden, ff, down)
+    idx_dev, w_dev, idx, w = gpu_route_softmax(logits, k)
+    assert 1 not in idx
+    G.say(f"moe matrix-core grouped fmt={fmt} T={T}")
+    with G.env(CAMELID_HIP_B32_MFMA_MIN_GROUP=1 << 30):
+        packed = gpu_moe(wgu, None, wd, E, k, idx_dev, w_dev, x, glu=GLU_GELU_TANH)
+    for min_group in (1, 6):
+        with G.env(CAMELID_HIP_B32_MFMA_MIN_GROUP=min_group):
+            got = gpu_moe(wgu, None, wd, E, k, idx_dev, w_dev, x, glu=GLU_GELU_TANH)
+        assert G.same_bits(got, packed)
+    want = oracle.moe_ffn_ex(fmt, gate_up, None, down, E, k, hidden, ff, logits[:6], x[:6], variant=1, threads=8)
+    assert G.max_rel(packed[:6], want) <= 1e-5

@@ -391,3 +391,40 @@ def test_q4k_matrix_core_cells_are_bitwise_the_gemv(rows, cols):
         with G.env(CAMELID_HIP_EXACT_ORDER="1"):
             got = G.gpu_gemm(w, s, q)
         check_outputs(fmt, wire, cols, s, q, got, expect_exact=True)
+
+
+@pytest.mark.parametrize("name,fmt", [("Q8_0", oracle.Q8_0), ("Q4_0", oracle.Q4_0)])
+@pytest.mark.parametrize("rows,cols", [(130, 1024), (2049, 5 * 256), (77, 12 * 256), (16, 256)])
+def test_b32_matrix_core_cells_are_bitwise_the_gemv(name, fmt, rows, cols):
+    """Q8_0 / Q4_0 batches on the matrix cores: every cell is the matvec kernel's block-ordered
+    chain, bit for bit, and the oracle's (these formats have one accumulation order)."""
+    rng = np.random.default_rng(rows + cols + fmt)
+    wire = G.synth_weight(fmt, rows, cols, seed=rows * 5 + cols + fmt)
+    w = Weight.upload(fmt, rows, cols, wire)
+    for n in (4, 5, 8, 16, 17, 33, 50, 64, 70):
+        x = rng.standard_normal((n, cols)).astype(np.float32)
+        if n == 5:
+            x[1] = 0.0              # an all-zero token: scale 0, sums 0
+            x[2, :32] = -x[2, :32].max() * 4   # a block at the negative extreme
+        s, q = oracle.quantize_activation(fmt, x)
+        with G.env(CAMELID_HIP_B32_MFMA_MIN_TOKENS=1 << 30):
+            ref = G.gpu_gemm(w, s, q)                      # the packed-dot kernel on the same inputs
+        for shape in (0, 1, 2, 3, 4, 5, 6):   # 0 = the default workgroup shape, 1..6 = every other one
+            G.say(f"{name} matrix-core {rows}x{cols} n={n} shape={shape}")
+            for deep in (0, 1):          # short phases / shallow ring, long phases / deep ring
+                with G.env(CAMELID_HIP_B32_MFMA_SHAPE=shape, CAMELID_HIP_B32_MFMA_DEEP=deep):
+                    got = G.gpu_gemm(w, s, q)
+                assert G.same_bits(got, ref)
+        check_outputs(fmt, wire, cols, s, q, got, expect_exact=True)
+
+
+@pytest.mark.parametrize("name,fmt", [("Q8_0", oracle.Q8_0), ("Q4_0", oracle.Q4_0)])
+def test_b32_rows_that_are_not_whole_slabs_take_the_packed_dot_kernel(name, fmt):
+    rows, cols, n = 40, 352, 9     # 11 blocks: not a multiple of 8
+    wire = G.synth_weight(fmt, rows, cols, seed=77 + fmt)
+    w = Weight.upload(fmt, rows, cols, wire)
+    x = np.random.default_rng(78).standard_normal((n, cols)).astype(np.float32)
+    s, q = oracle.quantize_activation(fmt, x)
+    G.say(f"{name} 11-block rows, 9 tokens")
+    got = G.gpu_gemm(w, s, q)
+    check_outputs(fmt, wire, cols, s, q, got, expect_exact=True)
