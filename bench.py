@@ -57,6 +57,8 @@ CONFIGS = {
     "q4k_14336x4096_n8": ("Q4_K", 14336, 4096, 8),
     "q4k_14336x4096_n16": ("Q4_K", 14336, 4096, 16),
     "q4k_14336x4096_n64": ("Q4_K", 14336, 4096, 64),
+    "q4k_4096x14336_n16": ("Q4_K", 4096, 14336, 16),
+    "q4k_4096x14336_n64": ("Q4_K", 4096, 14336, 64),
     # batches on the other formats (speculative verify / prefill widths); not BASELINE configurations
     "q8_0_8192x2048_n4": ("Q8_0", 8192, 2048, 4),
     "q8_0_8192x2048_n8": ("Q8_0", 8192, 2048, 8),
@@ -67,7 +69,13 @@ CONFIGS = {
     "q4_0_128256x3072_n8": ("Q4_0", 128256, 3072, 8),
     "q4_0_128256x3072_n16": ("Q4_0", 128256, 3072, 16),
     "q4_0_128256x3072_n64": ("Q4_0", 128256, 3072, 64),
+    "q6k_128256x3072_n4": ("Q6_K", 128256, 3072, 4),
     "q6k_128256x3072_n8": ("Q6_K", 128256, 3072, 8),
+    "q6k_128256x3072_n64": ("Q6_K", 128256, 3072, 64),
+    "q6k_4096x14336_n4": ("Q6_K", 4096, 14336, 4),
+    "q6k_4096x14336_n8": ("Q6_K", 4096, 14336, 8),
+    "q6k_4096x14336_n16": ("Q6_K", 4096, 14336, 16),
+    "q6k_4096x14336_n64": ("Q6_K", 4096, 14336, 64),
     "q6k_128256x3072_n16": ("Q6_K", 128256, 3072, 16),
 }
 

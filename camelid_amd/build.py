@@ -22,7 +22,7 @@ SOURCES = [
     "producers.hip",
     "layout.hip",
     "gemv_q4k.hip",
-    "gemm_q4k_mfma.hip", "gemm_b32_mfma.hip",
+    "gemm_q4k_mfma.hip", "gemm_b32_mfma.hip", "gemm_q6k_mfma.hip",
     "gemv_q8q4.hip",
     "gemv_q6k.hip",
     "moe.hip",

@@ -505,7 +505,12 @@ static int dispatch(const MatArgs &a, hipStream_t st) {
             else
                 rc = a.w->fmt == CML_Q8_0 ? launch_gemv_q8_0(a, st) : launch_gemv_q4_0(a, st);
             break;
-        case CML_Q6_K: rc = launch_gemv_q6k(a, st); break;
+        case CML_Q6_K:
+            if (!a.group_offsets && !a.ints && a.n_tokens >= q6k_mfma_min_tokens(a.w->rows, a.w->nb))
+                rc = launch_gemm_q6k_mfma(a, st);
+            else
+                rc = launch_gemv_q6k(a, st);
+            break;
         default: return fail(CML_ERR_INVALID, "unknown weight format %d", a.w->fmt);
     }
     if (rc == CML_OK) g_runs.fetch_add(1, std::memory_order_relaxed);

@@ -135,6 +135,8 @@ int b32_mfma_min_tokens(int64_t rows);                       // batch size from 
 int launch_gemm_q8_0(const MatArgs &a, hipStream_t st);
 int launch_gemm_q4_0(const MatArgs &a, hipStream_t st);
 int launch_gemm_q6k(const MatArgs &a, hipStream_t st);
+int launch_gemm_q6k_mfma(const MatArgs &a, hipStream_t st);  // Q6_K on the matrix cores; plain or grouped
+int q6k_mfma_min_tokens(int64_t rows, int64_t n_sb);         // batch size from which it pays
 
 // Integer tuning knob read once from the environment (0 when unset).
 int env_int(const char *name, int dflt);

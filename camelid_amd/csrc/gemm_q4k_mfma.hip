@@ -35,10 +35,13 @@
 // phase's loads are issued at the start of the current phase, ahead of the
 // weight loads, and stored at its end, so the only barriers are the phase
 // boundaries.  Weights (tile-interleaved layout, layout.hip) are double-buffered
-// in registers.  When the matvec kernel would split K for this weight shape, the
-// same split is reproduced inside the lane (the chain restarts at the split
-// points and the partial chains are added left to right), so every cell equals
-// the matvec result bit for bit.
+// in registers.  When the matvec kernel would split K for this weight shape (few
+// row tiles, long rows: an FFN down projection), the same split is reproduced, so
+// every cell equals the matvec result bit for bit: with KS = 2 or 4 waves per row
+// tile, each walking one part of K and the partial chains added left to right
+// through LDS at the end -- which is also what fills the chip when there are
+// fewer row tiles than SIMDs -- or, for other split factors, inside the lane (the
+// chain restarts at the split points).
 #include <type_traits>
 
 #include "cml_device.hpp"
@@ -96,19 +99,21 @@ __device__ __forceinline__ int scale_bytes(uint32_t bytes, uint32_t digit2) {
     return __builtin_bit_cast(int, p);
 }
 
-template <int GPW, int TB, bool SPLIT>
+template <int GPW, int TB, bool SPLIT, int KS = 1>
 __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
+    static_assert(!(SPLIT && KS > 1), "K is split across waves or inside the lane, not both");
     constexpr int NTOK = 16 * GPW * TB;              // tokens staged per workgroup
-    constexpr int KC = 128 / NTOK;                   // super-blocks per phase (a buffer is always 128 token-super-blocks)
-    constexpr int RT = 4 / TB;                       // row tiles per workgroup
-    constexpr int kBufBytes = KC * NTOK * kSlabRow;
+    // super-blocks per phase and K part (a buffer holds up to 128 token-super-blocks)
+    constexpr int KC = (128 / (NTOK * KS)) > 0 ? 128 / (NTOK * KS) : 1;
+    constexpr int RT = 4 / (TB * KS);                // row tiles per workgroup
+    constexpr int kBufBytes = KS * KC * NTOK * kSlabRow;
     constexpr int nthreads = 256;
     constexpr int kPieces = NTOK * 16;               // 16-byte pieces of one super-block of all tokens
     constexpr int kPer = kPieces / nthreads;         // 1, 2 or 4
     // weight super-blocks a wave keeps in flight (register ring): a 16-token step is short, so it
     // takes 8 to cover the HBM latency; steps over more tokens are longer and 4 are enough
-    constexpr int RING = GPW == 1 ? 8 : 4;
-    static_assert(RING % KC == 0 && kPer >= 1, "phase / staging shape");
+    constexpr int RING = (GPW == 1 && KS == 1) ? 8 : 4;
+    static_assert(RING % KC == 0 && kPer >= 1 && RT >= 1, "phase / staging shape");
     extern __shared__ uint4 smem[];
     uint8_t *buf0 = reinterpret_cast<uint8_t *>(smem);  // [KC][NTOK][kSlabRow]
     uint8_t *buf1 = buf0 + kBufBytes;
@@ -119,7 +124,11 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
     const int n_sb = a.n_sb;
     const int n = lane & 15, kq = lane >> 4;         // B/D column (weight row in tile) and k-quarter / A-row quad
     const int half = kq >> 1;                        // which sub-block of a chunk this lane's B bytes belong to
-    const int rt = wave / TB, tb = wave - rt * TB;
+    const int ks = wave % KS, w2 = wave / KS;        // K part of this wave; its (row tile, token block)
+    const int rt = w2 / TB, tb = w2 - rt * TB;
+    // this wave's part of K (the matvec kernel's split points) and the longest part
+    const int s_begin = KS > 1 ? ks * n_sb / KS : 0, s_end = KS > 1 ? (ks + 1) * n_sb / KS : n_sb;
+    const int n_loc = s_end - s_begin, n_max = (n_sb + KS - 1) / KS;
     const int n_tiles = (a.rows + a.row_skip + 15) / 16;
     const int tile = blockIdx.x * RT + rt;
     const int row = tile * 16 + n - a.row_skip;
@@ -133,7 +142,7 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
     const int n_here = min(NTOK, n_assign - tok0);
     const uint8_t *wtile = a.w + (band * (a.rows / 16) + min(tile, n_tiles - 1)) * 2304;
     // activation row of local token t (tokens past the end repeat the last one; their cells are not stored)
-    auto act_row = [&](int t) -> int64_t {
+    auto act_row = [&](int t) __attribute__((always_inline)) -> int64_t {
         const int j = a0 + tok0 + min(t, n_here - 1);
         return a.group_rows ? a.group_rows[j] : j;
     };
@@ -156,18 +165,20 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
         stage_src[k] = reinterpret_cast<const v4i *>(a.q + act_row(t) * n_sb * 256) + piece;
         stage_dst[k] = t * kSlabRow + piece * 16;
     }
-    v4i sreg[KC][kPer];
-    auto stage_load = [&](int p0) {  // the KC super-blocks starting at p0
+    v4i sreg[KS * KC][kPer];
+    auto stage_load = [&](int p0) __attribute__((always_inline)) {  // of every K part, the KC super-blocks starting at its p0-th
 #pragma unroll
-        for (int s = 0; s < KC; s++) {
-            const int off = min(p0 + s, n_sb - 1) * 16;  // in uint4 units
+        for (int kp = 0; kp < KS; kp++)
 #pragma unroll
-            for (int k = 0; k < kPer; k++) sreg[s][k] = stage_src[k][off];
-        }
+            for (int s = 0; s < KC; s++) {
+                const int off = min((KS > 1 ? kp * n_sb / KS : 0) + p0 + s, n_sb - 1) * 16;  // in uint4 units
+#pragma unroll
+                for (int k = 0; k < kPer; k++) sreg[kp * KC + s][k] = stage_src[k][off];
+            }
     };
-    auto stage_store = [&](uint8_t *buf) {
+    auto stage_store = [&](uint8_t *buf) __attribute__((always_inline)) {
 #pragma unroll
-        for (int s = 0; s < KC; s++)
+        for (int s = 0; s < KS * KC; s++)
 #pragma unroll
             for (int k = 0; k < kPer; k++) *reinterpret_cast<v4i *>(buf + s * (NTOK * kSlabRow) + stage_dst[k]) = sreg[s][k];
     };
@@ -188,7 +199,10 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
     // flight under the arithmetic -- with one wave per SIMD that depth, not the
     // occupancy, is what covers the HBM latency.
     MfmaWeights ring[RING];
-    auto load_slot = [&](MfmaWeights &r, int sb) { mfma_load_weights(r, w_hdr, w_piece, min(sb, n_sb - 1) * a.sb_stride); };
+    // `loc` counts super-blocks inside this wave's part of K
+    auto load_slot = [&](MfmaWeights &r, int loc) __attribute__((always_inline)) {
+        mfma_load_weights(r, w_hdr, w_piece, min(s_begin + loc, s_end - 1) * a.sb_stride);
+    };
 
     stage_load(0);
 #pragma unroll
@@ -205,7 +219,7 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
     int next_cut = a.ksplit <= 1 ? n_sb : n_sb / a.ksplit;  // first super-block of part 1
 
     // One super-block of this wave's tile against its token block.
-    auto step = [&](const MfmaWeights &w0, int sb, const uint8_t *slot) {
+    auto step = [&](const MfmaWeights &w0, int sb, const uint8_t *slot) __attribute__((always_inline)) {
         if (SPLIT && sb == next_cut) {  // the matvec kernel's K-split point: close the partial chain
 #pragma unroll
             for (int g = 0; g < GPW; g++)
@@ -273,19 +287,19 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
     // Every round but the last refills the ring; the last one only drains it, so
     // no weight is fetched twice when the row length is a multiple of RING.
     uint8_t *cur = buf0, *nxt = buf1;
-    auto round = [&](int sb0, auto refill) {
+    auto round = [&](int l0, auto refill) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < RING; i++) {
-            const int sb = sb0 + i;
+            const int loc = l0 + i;
             if (i % KC == 0) {
-                stage_load(sb + KC);
+                stage_load(loc + KC);
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if (sb < n_sb) step(ring[i], sb, cur + (i % KC) * (NTOK * kSlabRow));
+            if (loc < n_loc) step(ring[i], s_begin + loc, cur + (ks * KC + i % KC) * (NTOK * kSlabRow));
             // many-token steps fill the register file on their own: keep the scheduler from
             // overlapping two of them (measured: it spills and loses more than it hides)
             if constexpr (GPW > 1) __builtin_amdgcn_sched_barrier(0);
-            if constexpr (decltype(refill)::value) load_slot(ring[i], sb + RING);
+            if constexpr (decltype(refill)::value) load_slot(ring[i], loc + RING);
             if (i % KC == KC - 1) {
                 stage_store(nxt);
                 __syncthreads();  // next phase complete in `nxt`, everyone done with `cur`
@@ -295,9 +309,30 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
             }
         }
     };
-    int sb0 = 0;
-    for (; sb0 + RING < n_sb; sb0 += RING) round(sb0, std::true_type{});
-    round(sb0, std::false_type{});
+    int l0 = 0;
+    for (; l0 + RING < n_max; l0 += RING) round(l0, std::true_type{});
+    round(l0, std::false_type{});
+
+    if constexpr (KS > 1) {
+        // The partial chains of a tile's KS waves, added left to right as the matvec kernel adds
+        // them.  Every wave has passed the barrier that closed the last phase: the buffers are free.
+        float *red = reinterpret_cast<float *>(buf0);  // [wave][g][j][lane]
+#pragma unroll
+        for (int g = 0; g < GPW; g++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) red[((wave * GPW + g) * 4 + j) * 64 + lane] = acc[g][j];
+        __syncthreads();
+        if (ks != 0) return;
+#pragma unroll
+        for (int g = 0; g < GPW; g++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                float v = acc[g][j];
+#pragma unroll
+                for (int kp = 1; kp < KS; kp++) v = v + red[(((wave + kp) * GPW + g) * 4 + j) * 64 + lane];
+                acc[g][j] = v;
+            }
+    }
 
     if (tile < n_tiles && row >= 0 && row < a.rows) {
 #pragma unroll
@@ -315,27 +350,29 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
 
 int q4k_ksplit_for(int64_t rows, int64_t n_sb);  // gemv_q4k.hip: the matvec kernel's K-split policy
 
-template <int GPW, int TB, bool SPLIT>
+template <int GPW, int TB, bool SPLIT, int KS = 1>
 static int launch_mfma_split(const Q4KMfmaArgs &ka, int n_groups, hipStream_t st) {
-    constexpr int NTOK = 16 * GPW * TB, RT = 4 / TB;
+    constexpr int NTOK = 16 * GPW * TB, RT = 4 / (TB * KS);
+    constexpr int KC = (128 / (NTOK * KS)) > 0 ? 128 / (NTOK * KS) : 1;
     const int n_tiles = (ka.rows + ka.row_skip + 15) / 16;
     const unsigned gx = static_cast<unsigned>((n_tiles + RT - 1) / RT);
     const unsigned gy = static_cast<unsigned>((ka.n_tokens + NTOK - 1) / NTOK);
-    const size_t lds = 2 * static_cast<size_t>(128) * kSlabRow + static_cast<size_t>(ka.n_sb) * NTOK * 4;
+    const size_t lds = 2 * static_cast<size_t>(KS * KC * NTOK) * kSlabRow + static_cast<size_t>(ka.n_sb) * NTOK * 4;
     if (lds > 160 * 1024) return fail(CML_ERR_UNSUPPORTED, "Q4_K matrix-core path: %d super-blocks exceed the LDS budget", ka.n_sb);
     static bool raised = false;  // per instantiation: allow more than 64 KB of dynamic LDS once
     if (!raised) {
-        CML_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_mfma_kernel<GPW, TB, SPLIT>),
+        CML_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_mfma_kernel<GPW, TB, SPLIT, KS>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
         raised = true;
     }
-    hipLaunchKernelGGL((gemm_q4k_mfma_kernel<GPW, TB, SPLIT>), dim3(gx, gy, n_groups), dim3(256), lds, st, ka);
+    hipLaunchKernelGGL((gemm_q4k_mfma_kernel<GPW, TB, SPLIT, KS>), dim3(gx, gy, n_groups), dim3(256), lds, st, ka);
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }
 
-// The K-split bookkeeping costs a branch per super-block, so it is compiled in only where the
-// matvec kernel splits K for this weight shape.
+// The K-split bookkeeping inside the lane costs a branch per super-block, so it is compiled in
+// only where the matvec kernel splits K for this weight shape and the split is not 2 or 4 (those
+// run as 2 or 4 waves per row tile).
 template <int GPW, int TB>
 static int launch_mfma(const Q4KMfmaArgs &ka, int n_groups, hipStream_t st) {
     return ka.ksplit > 1 ? launch_mfma_split<GPW, TB, true>(ka, n_groups, st) : launch_mfma_split<GPW, TB, false>(ka, n_groups, st);
@@ -368,6 +405,14 @@ int launch_gemm_q4k_mfma(const MatArgs &a, hipStream_t st) {
     // workgroup columns (grid.y), each a pass over the weight.  The other shapes stay selectable
     // for tuning.
     const int shape = env_int("CAMELID_HIP_Q4K_MFMA_SHAPE", 0);
+    // K split across waves: 16 or 32 tokens per workgroup, more tokens = more workgroup columns
+    // (worth it when the launch has fewer row tiles than the chip has SIMDs; a grouped call with
+    // many experts in use fills the chip without it)
+    const int64_t launch_tiles = static_cast<int64_t>((ka.rows + ka.row_skip + 15) / 16) * ng;
+    if (shape == 0 && launch_tiles < 1024 && !env_int("CAMELID_HIP_Q4K_MFMA_SERIAL_SPLIT", 0)) {
+        if (ka.ksplit == 4) return (grouped || a.n_tokens <= 16) ? launch_mfma_split<1, 1, false, 4>(ka, ng, st) : launch_mfma_split<2, 1, false, 4>(ka, ng, st);
+        if (ka.ksplit == 2) return (grouped || a.n_tokens <= 16) ? launch_mfma_split<1, 1, false, 2>(ka, ng, st) : launch_mfma_split<2, 1, false, 2>(ka, ng, st);
+    }
     switch (shape) {
         case 1: return launch_mfma<1, 1>(ka, ng, st);   // 16 tokens, 1 wave per row tile
         case 2: return launch_mfma<2, 1>(ka, ng, st);   // 32 tokens, 1 wave per row tile

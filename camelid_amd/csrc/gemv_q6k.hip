@@ -275,6 +275,8 @@ static int pick_ksplit_q6k(int64_t rows, int64_t n_sb) {
     return 4;
 }
 
+int q6k_ksplit_for(int64_t rows, int64_t n_sb) { return pick_ksplit_q6k(rows, n_sb); }
+
 static size_t q6k_lds_bytes(int nt, int n_sb) {
     return static_cast<size_t>(nt) * n_sb * (256 + 64) + ((static_cast<size_t>(nt) * n_sb + 3) & ~size_t(3)) * 4 + 4 * nt * 8 * 4;
 }
@@ -336,7 +338,8 @@ int launch_gemv_q6k(const MatArgs &a, hipStream_t st) {
     int64_t t0 = 0;
     while (t0 < a.n_tokens) {
         const int64_t left = a.n_tokens - t0;
-        const int nt = left >= 8 ? 8 : (left >= 4 ? 4 : (left >= 2 ? 2 : 1));
+        int nt = left >= 8 ? 8 : (left >= 4 ? 4 : (left >= 2 ? 2 : 1));
+        while (nt > 1 && q6k_lds_bytes(nt, ka.n_sb) > 64 * 1024) nt /= 2;  // long rows: fewer tokens per pass
         ka.q = a.q + t0 * w->cols;
         ka.yd = a.scales + t0 * w->nb;
         ka.out = a.out + t0 * ka.rows;

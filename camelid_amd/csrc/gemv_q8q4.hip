@@ -242,7 +242,8 @@ static int launch_b32_p(const MatArgs &a, hipStream_t st) {
     int64_t t0 = 0;
     while (t0 < a.n_tokens) {
         const int64_t left = a.n_tokens - t0;
-        const int nt = left >= 8 ? 8 : (left >= 4 ? 4 : (left >= 2 ? 2 : 1));
+        int nt = left >= 8 ? 8 : (left >= 4 ? 4 : (left >= 2 ? 2 : 1));
+        while (nt > 1 && static_cast<size_t>(nt) * ba.nb * (32 + 4 + 4) > 64 * 1024) nt /= 2;  // long rows: fewer tokens per pass
         ba.q = a.q + t0 * w->cols;
         ba.xs = a.scales + t0 * w->nb;
         ba.out = a.out + t0 * ba.rows;
@@ -461,7 +462,8 @@ static int launch_b32_grouped_u(const MatArgs &a, const GroupedPrologue &pro, hi
     const int rows_per_wg = 4 * (64 / P);
     const int slots = a.group_ids ? a.max_active : a.n_groups;
     const dim3 grid(static_cast<unsigned>((ga.rows + rows_per_wg - 1) / rows_per_wg), static_cast<unsigned>(slots));
-    const bool one = pro.kind != 0 || a.n_tokens <= 1;
+    // one activation row per pass: single-token calls, and rows too long to stage four at a time
+    const bool one = pro.kind != 0 || a.n_tokens <= 1 || static_cast<size_t>(4) * ga.nb * (32 + 4 + 4) > 64 * 1024;
     const size_t lds = static_cast<size_t>(one ? 1 : 4) * ga.nb * (32 + 4 + 4);
     if (lds > 64 * 1024) return fail(CML_ERR_UNSUPPORTED, "activation of %d blocks exceeds the LDS staging limit", ga.nb);
     switch (pro.kind) {

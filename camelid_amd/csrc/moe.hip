@@ -246,7 +246,11 @@ __global__ __launch_bounds__(kPlanThreads) void moe_plan_kernel(const int32_t *_
 // Expert-grouped matmul: the packed-dot kernel for a few tokens, the matrix cores from 4 tokens
 // up (the same crossover as for plain calls).  Both produce the same bits per cell.
 static int launch_expert_matmul(const MatArgs &a, hipStream_t st) {
-    if (a.w->fmt == CML_Q6_K) return launch_gemv_q6k(a, st);
+    if (a.w->fmt == CML_Q6_K) {
+        const int64_t groups = a.group_ids ? a.max_active : a.n_groups;
+        if (a.group_offsets && a.n_assign_total >= groups * env_int("CAMELID_HIP_Q6K_MFMA_MIN_GROUP", 6)) return launch_gemm_q6k_mfma(a, st);
+        return launch_gemv_q6k(a, st);
+    }
     if (a.w->fmt != CML_Q4_K) {
         // matrix cores once the groups in use hold enough assignments on average to fill a 16-token tile reasonably
         const int64_t groups = a.group_ids ? a.max_active : a.n_groups;

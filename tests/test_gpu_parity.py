@@ -371,7 +371,10 @@ def test_host_slice_seam(name, fmt):
 
 # ------------------------------------------------- matrix-core path (n >= 16) ----
 
-@pytest.mark.parametrize("rows,cols", [(130, 1024), (2049, 5 * 256), (300, 56 * 256), (16, 256)])
+# (4096, 4096) and (2000, 18*256): the matvec kernel splits K four ways (even and uneven parts);
+# (1600, 9*256) and (6400, 8*256): two ways; (300, 56*256): eight ways (reproduced inside the lane)
+@pytest.mark.parametrize("rows,cols", [(130, 1024), (2049, 5 * 256), (300, 56 * 256), (16, 256), (4096, 4096), (2000, 18 * 256),
+                                       (1600, 9 * 256), (6400, 8 * 256)])
 def test_q4k_matrix_core_cells_are_bitwise_the_gemv(rows, cols):
     fmt = B.CML_Q4_K
     rng = np.random.default_rng(rows + cols)
@@ -383,7 +386,10 @@ def test_q4k_matrix_core_cells_are_bitwise_the_gemv(rows, cols):
         for shape in (0, 1, 2, 3, 4, 5, 6):   # 0 = the default workgroup shape, 1..6 = every other one
             G.say(f"Q4_K matrix-core {rows}x{cols} n={n} shape={shape}")
             with G.env(CAMELID_HIP_Q4K_MFMA_SHAPE=shape):
-                got = G.gpu_gemm(w, s, q)                      # default K-split policy, reproduced in-lane
+                got = G.gpu_gemm(w, s, q)                      # default K-split policy, reproduced across waves or in-lane
+            if shape == 0:
+                with G.env(CAMELID_HIP_Q4K_MFMA_SERIAL_SPLIT=1):
+                    assert G.same_bits(got, G.gpu_gemm(w, s, q))
             with G.env(CAMELID_HIP_Q4K_MFMA_MIN_TOKENS=1 << 30):
                 ref = G.gpu_gemm(w, s, q)                      # the packed-dot kernel on the same inputs
             assert G.same_bits(got, ref)
@@ -428,3 +434,54 @@ def test_b32_rows_that_are_not_whole_slabs_take_the_packed_dot_kernel(name, fmt)
     G.say(f"{name} 11-block rows, 9 tokens")
     got = G.gpu_gemm(w, s, q)
     check_outputs(fmt, wire, cols, s, q, got, expect_exact=True)
+
+
+# K split by the matvec kernel: (300, 12*256) and (300, 13*256) two ways, (4000, 16*256) and
+# (1000, 18*256) four ways (even and uneven parts); the others not at all
+@pytest.mark.parametrize("rows,cols", [(130, 1024), (2049, 5 * 256), (300, 12 * 256), (16, 256), (4000, 16 * 256), (300, 13 * 256),
+                                       (1000, 18 * 256)])
+def test_q6k_matrix_core_cells_are_bitwise_the_gemv(rows, cols):
+    """Q6_K batches on the matrix cores: every cell is the matvec kernel's chain (K-split policy
+    included), bit for bit; with the split off it is the oracle's fused order."""
+    fmt = B.CML_Q6_K
+    rng = np.random.default_rng(rows + cols + 6)
+    wire = G.synth_weight(fmt, rows, cols, seed=rows * 7 + cols)
+    w = Weight.upload(fmt, rows, cols, wire)
+    for n in (5, 8, 16, 17, 33, 50, 64, 70):
+        x = rng.standard_normal((n, cols)).astype(np.float32)
+        if n == 5:
+            x[1] = 0.0
+            x[2, :256] = -np.abs(x[2, :256]).max() * 4   # a super-block at the negative extreme
+        s, q = oracle.quantize_activation(fmt, x)
+        with G.env(CAMELID_HIP_Q6K_MFMA_MIN_TOKENS=1 << 30):
+            ref = G.gpu_gemm(w, s, q)                      # the packed-dot kernel on the same inputs
+        for shape in (0, 1, 2, 3, 4, 6):
+            for deep in (0, 1):
+                G.say(f"Q6_K matrix-core {rows}x{cols} n={n} shape={shape} deep={deep}")
+                with G.env(CAMELID_HIP_Q6K_MFMA_SHAPE=shape, CAMELID_HIP_Q6K_MFMA_DEEP=deep, CAMELID_HIP_Q6K_MFMA_MIN_TOKENS=1):
+                    got = G.gpu_gemm(w, s, q)
+                assert G.same_bits(got, ref)
+        with G.env(CAMELID_HIP_Q6K_MFMA_SERIAL_SPLIT=1, CAMELID_HIP_Q6K_MFMA_MIN_TOKENS=1):   # the split inside the lane
+            assert G.same_bits(G.gpu_gemm(w, s, q), ref)
+        check_outputs(fmt, wire, cols, s, q, got, expect_exact=False)
+        with G.env(CAMELID_HIP_EXACT_ORDER="1", CAMELID_HIP_Q6K_MFMA_MIN_TOKENS=1):
+            got = G.gpu_gemm(w, s, q)
+        check_outputs(fmt, wire, cols, s, q, got, expect_exact=True)
+
+
+@pytest.mark.parametrize("name,fmt", FMTS)
+def test_long_rows_in_small_batches_fit_the_staging_limit(name, fmt):
+    """14336-value rows (an FFN down projection) with 2..8 tokens: the packed-dot kernels stage
+    fewer tokens per pass instead of refusing the call."""
+    rows, cols = 40, 14336
+    wire = G.synth_weight(fmt, rows, cols, seed=900 + fmt)
+    w = Weight.upload(fmt, rows, cols, wire)
+    rng = np.random.default_rng(901)
+    for n in (2, 4, 8):
+        x = rng.standard_normal((n, cols)).astype(np.float32)
+        s, q = oracle.quantize_activation(fmt, x)
+        G.say(f"{name} {rows}x{cols} n={n} packed-dot")
+        with G.env(CAMELID_HIP_Q4K_MFMA_MIN_TOKENS=1 << 30, CAMELID_HIP_B32_MFMA_MIN_TOKENS=1 << 30,
+                   CAMELID_HIP_Q6K_MFMA_MIN_TOKENS=1 << 30, CAMELID_HIP_EXACT_ORDER="1"):
+            got = G.gpu_gemm(w, s, q)
+        check_outputs(fmt, wire, cols, s, q, got, expect_exact=True)
