@@ -27,7 +27,7 @@ EXPORTS = [
     "cml_gemv", "cml_gemm", "cml_block_dots", "cml_matmul_workspace_bytes", "cml_matmul_f32",
     "cml_moe_route_top_k", "cml_moe_route_softmax_top_k", "cml_moe_workspace_bytes", "cml_moe_ffn", "cml_moe_ffn_ex",
     "cml_moe_plan", "cml_moe_gemv_routed", "cml_moe_weighted_sum",
-    "cml_quantize_weights_host", "cml_try_linear_rows",
+    "cml_quantize_weights_host", "cml_try_linear_rows", "cml_try_q8_0_block_linear_row",
 ]
 
 
@@ -110,6 +110,7 @@ def lib() -> C.CDLL:
     L.cml_glu_quantize.argtypes = [i32, i32, vp, vp, i64, i64, vp, vp, vp]
     L.cml_quantize_weights_host.argtypes = [i32, vp, sz, vp, i32]
     L.cml_try_linear_rows.argtypes = [i32, vp, vp, vp, sz, i64, i64, i64, vp]
+    L.cml_try_q8_0_block_linear_row.argtypes = [vp, vp, vp, sz, i64, i64, vp]
     _lib = L
     return L
 

@@ -11,6 +11,7 @@
 
 #include <atomic>
 #include <mutex>
+#include <vector>
 #include <unordered_map>
 
 #include "cml_host.hpp"
@@ -648,6 +649,31 @@ struct CacheHash {
 std::unordered_map<CacheKey, cml_weight *, CacheHash> g_weight_cache;
 }  // namespace
 
+// Activations down, one dispatch, outputs up; synchronous.  g_mutex is held by the caller.
+static int run_host_seam(const cml_weight *w, const float *input_scales, const int8_t *input_quants, int64_t input_rows, float *output) {
+    const int64_t per = is_k_family(w->fmt) ? 256 : 32;
+    const size_t qb = static_cast<size_t>(input_rows) * w->cols;
+    const size_t sb = static_cast<size_t>(input_rows) * (w->cols / per) * sizeof(float);
+    const size_t ob = static_cast<size_t>(input_rows) * w->rows * sizeof(float);
+    const size_t q_off = 0, s_off = (qb + 255) & ~size_t(255), o_off = s_off + ((sb + 255) & ~size_t(255));
+    uint8_t *buf = nullptr;
+    CML_HIP_TRY(hipMalloc(reinterpret_cast<void **>(&buf), o_off + ob));
+    int rc = CML_OK;
+    hipError_t e = hipMemcpy(buf + q_off, input_quants, qb, hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMemcpy(buf + s_off, input_scales, sb, hipMemcpyHostToDevice);
+    if (e != hipSuccess) rc = fail(CML_ERR_HIP, "hipMemcpy failed: %s", hipGetErrorString(e));
+    if (rc == CML_OK)
+        rc = dispatch(plain_args(w, reinterpret_cast<int8_t *>(buf + q_off), reinterpret_cast<float *>(buf + s_off),
+                                 input_rows, reinterpret_cast<float *>(buf + o_off)),
+                      nullptr);
+    if (rc == CML_OK) {
+        e = hipMemcpy(output, buf + o_off, ob, hipMemcpyDeviceToHost);  // synchronises the null stream
+        if (e != hipSuccess) rc = fail(CML_ERR_HIP, "device run failed: %s", hipGetErrorString(e));
+    }
+    (void)hipFree(buf);
+    return rc;
+}
+
 int cml_try_linear_rows(int fmt, const float *input_scales, const int8_t *input_quants, const uint8_t *weight_wire,
                         size_t weight_nbytes, int64_t input_rows, int64_t weight_rows, int64_t cols, float *output) {
     if (!ready()) {
@@ -668,27 +694,33 @@ int cml_try_linear_rows(int fmt, const float *input_scales, const int8_t *input_
         if (int rc = cml_weight_upload(fmt, weight_rows, cols, weight_wire, weight_nbytes, &w)) return rc;
         g_weight_cache.emplace(key, w);
     }
-    const int64_t per = is_k_family(fmt) ? 256 : 32;
-    const size_t qb = static_cast<size_t>(input_rows) * cols;
-    const size_t sb = static_cast<size_t>(input_rows) * (cols / per) * sizeof(float);
-    const size_t ob = static_cast<size_t>(input_rows) * weight_rows * sizeof(float);
-    const size_t q_off = 0, s_off = (qb + 255) & ~size_t(255), o_off = s_off + ((sb + 255) & ~size_t(255));
-    uint8_t *buf = nullptr;
-    CML_HIP_TRY(hipMalloc(reinterpret_cast<void **>(&buf), o_off + ob));
-    int rc = CML_OK;
-    hipError_t e = hipMemcpy(buf + q_off, input_quants, qb, hipMemcpyHostToDevice);
-    if (e == hipSuccess) e = hipMemcpy(buf + s_off, input_scales, sb, hipMemcpyHostToDevice);
-    if (e != hipSuccess) rc = fail(CML_ERR_HIP, "hipMemcpy failed: %s", hipGetErrorString(e));
-    if (rc == CML_OK)
-        rc = dispatch(plain_args(w, reinterpret_cast<int8_t *>(buf + q_off), reinterpret_cast<float *>(buf + s_off),
-                                 input_rows, reinterpret_cast<float *>(buf + o_off)),
-                      nullptr);
-    if (rc == CML_OK) {
-        e = hipMemcpy(output, buf + o_off, ob, hipMemcpyDeviceToHost);  // synchronises the null stream
-        if (e != hipSuccess) rc = fail(CML_ERR_HIP, "device run failed: %s", hipGetErrorString(e));
+    return run_host_seam(w, input_scales, input_quants, input_rows, output);
+}
+
+int cml_try_q8_0_block_linear_row(const float *input_scales, const int8_t *input_quants, const uint8_t *weight_block_bytes,
+                                  size_t weight_nbytes, int64_t rows, int64_t blocks_per_row, float *output) {
+    if (!ready()) {
+        if (cml_init(-1) != CML_OK) return CML_ERR_UNAVAILABLE;
     }
-    (void)hipFree(buf);
-    return rc;
+    if (!input_scales || !input_quants || !weight_block_bytes || !output) return fail(CML_ERR_INVALID, "null pointer");
+    if (rows <= 0 || blocks_per_row <= 0) return fail(CML_ERR_SHAPE, "empty shape");
+    const size_t n_blocks = static_cast<size_t>(rows) * static_cast<size_t>(blocks_per_row);
+    if (weight_nbytes != n_blocks * 36) return fail(CML_ERR_SHAPE, "%zu bytes are not %lld x %lld blocks of 36", weight_nbytes, (long long)rows, (long long)blocks_per_row);
+    std::lock_guard<std::mutex> lock(g_mutex);
+    cml_weight *w = nullptr;
+    const CacheKey key{weight_block_bytes, weight_nbytes, -36};  // the in-memory block layout, not a wire format
+    auto it = g_weight_cache.find(key);
+    if (it != g_weight_cache.end()) {
+        w = it->second;
+        if (w->rows != rows || w->nb != blocks_per_row) return fail(CML_ERR_SHAPE, "cached weight has another shape");
+    } else {
+        std::vector<uint8_t> wire(n_blocks * 34);
+        if (!q8_0_blocks_to_wire(weight_block_bytes, n_blocks, wire.data()))
+            return fail(CML_ERR_UNSUPPORTED, "a block scale is not an f16 value: these blocks did not come from Q8_0 wire bytes");
+        if (int rc = cml_weight_upload(CML_Q8_0, rows, blocks_per_row * 32, wire.data(), wire.size(), &w)) return rc;
+        g_weight_cache.emplace(key, w);
+    }
+    return run_host_seam(w, input_scales, input_quants, 1, output);
 }
 
 }  // extern "C"

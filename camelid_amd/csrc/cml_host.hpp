@@ -59,6 +59,9 @@ namespace cml {
 // Plane sizes for `rows` rows; returns the number of planes.
 int plane_layout(int fmt, int64_t rows, int64_t nb, int64_t stride[4], size_t offset[4], size_t *total);
 
+// weight_quantize.cpp: 36-byte in-memory Q8_0 blocks (f32 scale + 32 int8) -> 34-byte wire blocks; false if a scale is not an f16 value
+bool q8_0_blocks_to_wire(const uint8_t *blocks, size_t n_blocks, uint8_t *wire);
+
 // ---- launchers (one per kernel file) ------------------------------------------------------------
 
 // quantize.hip

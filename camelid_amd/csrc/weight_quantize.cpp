@@ -197,6 +197,28 @@ void block_q6_k(const float *src, uint8_t *dst) {
 
 }  // namespace
 
+namespace cml {
+
+// In-memory Q8_0 blocks (36 bytes: f32 scale + 32 int8; reference Q8_0Block, src/tensor/mod.rs:
+// 105-110) -> 34-byte wire blocks.  The scale must be a value an f16 holds exactly (it is whenever
+// the blocks were decoded from a GGUF file); returns false at the first one that is not.
+bool q8_0_blocks_to_wire(const uint8_t *blocks, size_t n_blocks, uint8_t *wire) {
+    for (size_t i = 0; i < n_blocks; i++) {
+        float scale;
+        memcpy(&scale, blocks + i * 36, 4);
+        const uint16_t h = f16_bits(scale);
+        const float back = f16_value(h);
+        if (memcmp(&back, &scale, 4) != 0 && !(back == 0.0f && scale == 0.0f)) return false;
+        uint8_t *dst = wire + i * 34;
+        dst[0] = static_cast<uint8_t>(h & 0xff);
+        dst[1] = static_cast<uint8_t>(h >> 8);
+        memcpy(dst + 2, blocks + i * 36 + 4, 32);
+    }
+    return true;
+}
+
+}  // namespace cml
+
 extern "C" int cml_quantize_weights_host(int fmt, const float *src, size_t n_values, uint8_t *dst, int threads) {
     const int bv = cml_block_values(fmt), bb = cml_block_bytes(fmt);
     if (bv == 0) return CML_ERR_INVALID;

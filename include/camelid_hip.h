@@ -311,6 +311,17 @@ int cml_quantize_weights_host(int fmt, const float *src, size_t n_values, uint8_
 int cml_try_linear_rows(int fmt, const float *input_scales, const int8_t *input_quants,
                         const uint8_t *weight_wire, size_t weight_nbytes, int64_t input_rows,
                         int64_t weight_rows, int64_t cols, float *output);
+/* The seam the reference's CPU linear consults on its decode path (reference
+ * try_q8_0_block_linear_row, src/cuda.rs:1089-1222; call site
+ * src/inference.rs:27939-27955): one input row against `rows` weight rows held
+ * as in-memory Q8_0Block values, 36 bytes each = f32 scale + 32 int8
+ * (src/tensor/mod.rs:105-110); weight_nbytes must be rows*blocks_per_row*36.
+ * The blocks are converted to wire form once per (pointer, length) and cached
+ * on the device; a scale that is not an f16 value (blocks that were not decoded
+ * from Q8_0 wire bytes) makes the call decline.  Same return convention. */
+int cml_try_q8_0_block_linear_row(const float *input_scales, const int8_t *input_quants,
+                                  const uint8_t *weight_block_bytes, size_t weight_nbytes,
+                                  int64_t rows, int64_t blocks_per_row, float *output);
 
 #ifdef __cplusplus
 }

@@ -369,6 +369,35 @@ def test_host_slice_seam(name, fmt):
     assert bad != 0
 
 
+def test_q8_0_block_seam_takes_in_memory_blocks():
+    """The seam the reference's CPU linear calls on its decode path (try_q8_0_block_linear_row,
+    src/cuda.rs:1089-1222, called at src/inference.rs:27944): weights as 36-byte in-memory blocks
+    (f32 scale + 32 int8).  Same bits as the wire-format matvec; blocks whose scale is not an f16
+    value, and wrong lengths, make the call decline."""
+    rng = np.random.default_rng(195)
+    rows, cols = 70, 2048
+    nb = cols // 32
+    wire = G.synth_weight(B.CML_Q8_0, rows, cols, seed=195).reshape(rows * nb, 34)
+    blocks = np.zeros((rows * nb, 36), np.uint8)
+    blocks[:, :4] = np.ascontiguousarray(wire[:, :2]).view(np.float16).astype(np.float32).view(np.uint8).reshape(-1, 4)
+    blocks[:, 4:] = wire[:, 2:]
+    x = rng.standard_normal((1, cols)).astype(np.float32)
+    s, q = oracle.quantize_activation(B.CML_Q8_0, x)
+    out = np.full(rows, np.nan, np.float32)
+    G.say("try_q8_0_block_linear_row")
+    L = lib()
+    before = L.cml_run_count()
+    for _ in range(2):   # second call hits the device weight cache
+        rc = L.cml_try_q8_0_block_linear_row(s.ctypes.data, q.ctypes.data, blocks.ctypes.data, blocks.nbytes, rows, nb, out.ctypes.data)
+        assert rc == 0, L.cml_last_error()
+        assert G.same_bits(out, oracle.matmul_q(B.CML_Q8_0, wire.reshape(-1), cols, s, q)[0])
+    assert L.cml_run_count() >= before + 2
+    assert L.cml_try_q8_0_block_linear_row(s.ctypes.data, q.ctypes.data, blocks.ctypes.data, blocks.nbytes - 36, rows, nb, out.ctypes.data) != 0
+    odd = blocks.copy()
+    odd[5, :4] = np.float32([0.1]).view(np.uint8)          # 0.1 is not an f16 value
+    assert L.cml_try_q8_0_block_linear_row(s.ctypes.data, q.ctypes.data, odd.ctypes.data, odd.nbytes, rows, nb, out.ctypes.data) == 6
+
+
 # ------------------------------------------------- matrix-core path (n >= 16) ----
 
 # (4096, 4096) and (2000, 18*256): the matvec kernel splits K four ways (even and uneven parts);
