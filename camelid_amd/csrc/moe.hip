@@ -433,6 +433,7 @@ int cml_moe_ffn_ex(const cml_weight *gate, const cml_weight *up, const cml_weigh
         return fail(CML_ERR_UNSUPPORTED, "mixture-of-experts dispatch is built for Q4_K, Q6_K, Q8_0 and Q4_0 expert matrices (gate and up alike)");
     if (n_experts <= 0 || n_experts > kMaxExperts || k <= 0 || k > n_experts || n_tokens < 0)
         return fail(CML_ERR_SHAPE, "bad routing shape (%d experts, top-%d)", n_experts, k);
+    if (n_tokens > 65535) return fail(CML_ERR_SHAPE, "at most 65535 tokens per call (%lld given)", (long long)n_tokens);
     const int64_t hidden = gate->cols, ff = down->cols;
     if ((up && (up->cols != hidden || gate->rows != up->rows)) || gate->rows != (fused_gate_up ? 2 : 1) * ff * n_experts ||
         down->rows != hidden * n_experts)
