@@ -208,9 +208,11 @@ int cml_argmax_f32(const float *logits_dev, int64_t n_rows, int64_t n, uint32_t 
  * src/cuda_resident.rs:334-413). */
 int cml_gemv(const cml_weight *w, const int8_t *q_dev, const float *scales_dev, float *out_dev,
              const float *residual_dev, cml_stream_t stream);
-/* n_tokens activation rows against one pass over the weight;
- * out_dev[t*rows + row].  Every cell equals the cml_gemv result for that
- * token bit for bit. */
+/* n_tokens activation rows; out_dev[t*rows + row].  A few tokens run on the
+ * packed-dot kernel (up to 8 per pass over the weight), larger batches on the
+ * int8 matrix cores (all four formats; Q8_0 / Q4_0 rows must be whole multiples
+ * of 256 values for that, other lengths stay on the packed-dot kernel).  Every
+ * cell equals the cml_gemv result for that token bit for bit. */
 int cml_gemm(const cml_weight *w, const int8_t *q_dev, const float *scales_dev, int64_t n_tokens,
              float *out_dev, cml_stream_t stream);
 /* The exact per-block integer dot products of cml_gemv, for parity checks:
