@@ -42,6 +42,7 @@ struct B32Args {
     const int32_t *band_ids;
     int64_t act_slot_stride;
     int64_t out_slot_stride;
+    int early_loads;  // issue the first weight loads ahead of the fused quantizer
 };
 
 template <int FMT, int UU = 2>
@@ -109,15 +110,14 @@ __device__ __forceinline__ void b32_compute(const B32Regs<FMT, U> &r, int l, int
     }
 }
 
-// One pass over a row's blocks for NT staged activation rows: two register buffers alternate,
-// the last one is consumed without issuing further loads.
+// `ra` arrives loaded with steps 0..U-1 (b32_load) -- the caller may have issued those loads well
+// before, e.g. ahead of its prologue.
 template <int FMT, int P, int NT, bool INTS, int U = 2>
-__device__ __forceinline__ void b32_row_pass(const uint8_t *qrow, const uint8_t *srow, int l, int nb, const int8_t *ys,
-                                             const int *bsum, const float *xss, float (&acc)[NT], int32_t *ints_row) {
+__device__ __forceinline__ void b32_row_pass_from(B32Regs<FMT, U> &ra, const uint8_t *qrow, const uint8_t *srow, int l, int nb,
+                                                  const int8_t *ys, const int *bsum, const float *xss, float (&acc)[NT],
+                                                  int32_t *ints_row) {
     const int n_steps = (nb + P - 1) / P;
-    B32Regs<FMT, U> ra, rb;
-    b32_load<FMT, P, U>(ra, qrow, srow, l, 0, n_steps, nb);
-    __builtin_amdgcn_sched_barrier(0);
+    B32Regs<FMT, U> rb;
     for (int step = 0;;) {
         if (step + U >= n_steps) {
             b32_compute<FMT, P, NT, INTS, U>(ra, l, step, n_steps, nb, ys, bsum, xss, acc, ints_row);
@@ -140,6 +140,18 @@ __device__ __forceinline__ void b32_row_pass(const uint8_t *qrow, const uint8_t 
     }
 }
 
+// One pass over a row's blocks for NT staged activation rows: two register buffers alternate,
+// the last one is consumed without issuing further loads.
+template <int FMT, int P, int NT, bool INTS, int U = 2>
+__device__ __forceinline__ void b32_row_pass(const uint8_t *qrow, const uint8_t *srow, int l, int nb, const int8_t *ys,
+                                             const int *bsum, const float *xss, float (&acc)[NT], int32_t *ints_row) {
+    const int n_steps = (nb + P - 1) / P;
+    B32Regs<FMT, U> ra;
+    b32_load<FMT, P, U>(ra, qrow, srow, l, 0, n_steps, nb);
+    __builtin_amdgcn_sched_barrier(0);
+    b32_row_pass_from<FMT, P, NT, INTS, U>(ra, qrow, srow, l, nb, ys, bsum, xss, acc, ints_row);
+}
+
 // FUSEQ (single token): the activation arrives as f32 and every workgroup quantizes it to Q8_0
 // itself, eight lanes per block, straight into the LDS staging area -- the arithmetic of
 // quantize_q8_0_kernel without the launch and the round trip through memory.
@@ -160,26 +172,6 @@ __global__ __launch_bounds__(256) void gemv_b32_kernel(B32Args a) {
     const float *xs = a.xs + static_cast<int64_t>(slot) * a.act_slot_stride * nb;
     float *out = a.out + static_cast<int64_t>(slot) * a.out_slot_stride;
 
-    if constexpr (FUSEQ) {
-        const float4 *x4 = reinterpret_cast<const float4 *>(a.x);
-        b32_stage_quantized_from<FMT>([&](int i) { return x4[i]; }, nb, tid, ys, xss, bsum);
-    } else {
-        const uint4 *src = reinterpret_cast<const uint4 *>(q);
-        uint4 *dst = reinterpret_cast<uint4 *>(ys);
-        const int n16 = NT * nb * 2;  // even: lanes 2k, 2k+1 are in or out together
-        for (int i = tid; i < n16; i += 256) {
-            const uint4 v = src[i];
-            dst[i] = v;
-            if constexpr (FMT == CML_Q4_0) {
-                int s = bytesum16(v);
-                s += row_shr_i32<1>(s);
-                if (i & 1) bsum[i >> 1] = s;
-            }
-        }
-        for (int i = tid; i < NT * nb; i += 256) xss[i] = xs[i];
-    }
-    __syncthreads();
-
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int r = lane / P, l = lane - r * P;
     const int row = (blockIdx.x * 4 + wave) * RPW + r;
@@ -188,6 +180,79 @@ __global__ __launch_bounds__(256) void gemv_b32_kernel(B32Args a) {
     const uint8_t *qrow = a.quants + arow * a.q_stride;
     const uint8_t *srow = a.scales + arow * a.s_stride;
     const bool leader = (l == P - 1);
+    const int n_steps = (nb + P - 1) / P;
+    constexpr int UE = 2;  // steps loaded ahead of the fused quantizer (4 measured slower)
+    B32Regs<FMT, UE> ra;
+    bool preloaded = false;
+
+    if constexpr (FUSEQ) {
+        const float4 *x4 = reinterpret_cast<const float4 *>(a.x);
+        constexpr int NX = 4;  // float4 per thread held in registers: rows of up to 128 blocks
+        if (nb <= NX * 32 && a.early_loads) {  // uniform
+            // The token's f32 loads go out first, the row's first weight steps right behind them, and
+            // the quantizer then waits for the f32 values only (a wave's loads return in order).
+            const int n4 = nb * 8;
+            float4 xv[NX];
+#pragma unroll
+            for (int j = 0; j < NX; j++) xv[j] = x4[min(tid + 256 * j, n4 - 1)];
+            __builtin_amdgcn_sched_barrier(0);
+            b32_load<FMT, P, UE>(ra, qrow, srow, l, 0, n_steps, nb);
+            preloaded = true;
+            __builtin_amdgcn_sched_barrier(0);
+            uint32_t *ys32 = reinterpret_cast<uint32_t *>(ys);
+#pragma unroll
+            for (int j = 0; j < NX; j++) {
+                const int i = tid + 256 * j;
+                if (i < n4) {  // whole blocks of eight lanes enter and leave together
+                    float scale;
+                    const uint32_t packed = q8_0_quantize_lane8(xv[j], scale);
+                    ys32[i] = packed;
+                    if ((i & 7) == 0) xss[i >> 3] = scale;
+                    if constexpr (FMT == CML_Q4_0) {
+                        const int sum = group_sum_to_last<8>(sdot4(packed, 0x01010101u, 0));
+                        if ((i & 7) == 7) bsum[i >> 3] = sum;
+                    }
+                }
+            }
+        } else {
+            b32_stage_quantized_from<FMT>([&](int i) { return x4[i]; }, nb, tid, ys, xss, bsum);
+        }
+    } else {
+        const uint4 *src = reinterpret_cast<const uint4 *>(q);
+        uint4 *dst = reinterpret_cast<uint4 *>(ys);
+        const int n16 = NT * nb * 2;  // even: lanes 2k, 2k+1 are in or out together
+        if (NT == 1 && n16 <= 256 && a.early_loads) {  // uniform: one 16-byte piece and one scale per thread at most
+            // the same order of issue for a quantized activation: its loads, the first weight steps, then the staging
+            const uint4 v = src[min(tid, n16 - 1)];
+            const float sc = xs[min(tid, nb - 1)];
+            __builtin_amdgcn_sched_barrier(0);
+            b32_load<FMT, P, UE>(ra, qrow, srow, l, 0, n_steps, nb);
+            preloaded = true;
+            __builtin_amdgcn_sched_barrier(0);
+            if (tid < n16) {
+                dst[tid] = v;
+                if constexpr (FMT == CML_Q4_0) {
+                    int s = bytesum16(v);
+                    s += row_shr_i32<1>(s);
+                    if (tid & 1) bsum[tid >> 1] = s;
+                }
+            }
+            if (tid < nb) xss[tid] = sc;
+        } else {
+            for (int i = tid; i < n16; i += 256) {
+                const uint4 v = src[i];
+                dst[i] = v;
+                if constexpr (FMT == CML_Q4_0) {
+                    int s = bytesum16(v);
+                    s += row_shr_i32<1>(s);
+                    if (i & 1) bsum[i >> 1] = s;
+                }
+            }
+            for (int i = tid; i < NT * nb; i += 256) xss[i] = xs[i];
+        }
+    }
+    __syncthreads();
+
     int32_t *ints_row = nullptr;
     if constexpr (INTS) {
         if (a.ints && live) ints_row = a.ints + arow * static_cast<int64_t>(nb);
@@ -197,7 +262,11 @@ __global__ __launch_bounds__(256) void gemv_b32_kernel(B32Args a) {
 #pragma unroll
     for (int t = 0; t < NT; t++) acc[t] = 0.0f;
 
-    b32_row_pass<FMT, P, NT, INTS>(qrow, srow, l, nb, ys, bsum, xss, acc, ints_row);
+    if (preloaded) {
+        b32_row_pass_from<FMT, P, NT, INTS, UE>(ra, qrow, srow, l, nb, ys, bsum, xss, acc, ints_row);
+    } else {
+        b32_row_pass<FMT, P, NT, INTS>(qrow, srow, l, nb, ys, bsum, xss, acc, ints_row);
+    }
 
     if (leader && live) {
 #pragma unroll
@@ -236,6 +305,7 @@ static int launch_b32_p(const MatArgs &a, hipStream_t st) {
     ba.residual = a.residual;
     ba.ints = a.ints;
     ba.band_ids = nullptr;
+    ba.early_loads = env_int("CAMELID_HIP_B32_EARLY_LOADS", 1);
     ba.act_slot_stride = 0;
     ba.out_slot_stride = a.n_tokens * static_cast<int64_t>(ba.rows);
     const int n_bands = 1;
@@ -272,6 +342,7 @@ static int launch_b32_f32_p(const cml_weight *w, const float *x, float *out, hip
     ba.nb = static_cast<int>(w->nb);
     ba.x = x;
     ba.out = out;
+    ba.early_loads = env_int("CAMELID_HIP_B32_EARLY_LOADS", 1);
     const int rows_per_wg = 4 * (64 / P);
     const unsigned gx = static_cast<unsigned>((ba.rows + rows_per_wg - 1) / rows_per_wg);
     const size_t lds = static_cast<size_t>(ba.nb) * (32 + 4 + 4);
