@@ -100,6 +100,54 @@ __device__ __forceinline__ int wave_allmax_i32(int v) {
                max(__builtin_amdgcn_readlane(v, 32), __builtin_amdgcn_readlane(v, 48)));
 }
 
+// The same routing with one wave per token (k <= 64), lane l holding experts l and l + 64 during the
+// selection and the l-th selected expert afterwards; the short sequential parts (maximum and sum over
+// the k selected, in selection order) run redundantly in every lane.  Same arithmetic, value for
+// value, as moe_route_kernel.
+__global__ __launch_bounds__(256) void moe_route_wave_kernel(const float *__restrict__ logits, int64_t n_tokens, int n_experts, int k,
+                                                             int32_t *__restrict__ idx_out, float *__restrict__ w_out) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int64_t t_raw = static_cast<int64_t>(blockIdx.x) * 4 + wave;
+    const bool live = t_raw < n_tokens;
+    const int64_t t = live ? t_raw : n_tokens - 1;  // spare waves repeat the last token and store nothing
+    const float *lg = logits + t * n_experts;
+    bool v0 = lane < n_experts, v1 = lane + 64 < n_experts;
+    const float l0 = v0 ? lg[lane] : 0.0f, l1 = v1 ? lg[lane + 64] : 0.0f;
+    const int k0 = total_key(l0), k1 = total_key(l1);
+    int sel_e = 0;
+    float sel_v = 0.0f;
+    for (int s = 0; s < k; s++) {  // top-k by logit (total order, descending), ties to the lower index
+        const int m = wave_allmax_i32(max(v0 ? k0 : INT32_MIN, v1 ? k1 : INT32_MIN));
+        const unsigned long long b0 = __builtin_amdgcn_ballot_w64(v0 && k0 == m), b1 = __builtin_amdgcn_ballot_w64(v1 && k1 == m);
+        const int e = b0 ? __builtin_ctzll(b0) : (b1 ? 64 + __builtin_ctzll(b1) : 0);
+        const int from = __builtin_amdgcn_readlane(__builtin_bit_cast(int, e < 64 ? l0 : l1), e & 63);
+        if (e == lane) v0 = false;
+        if (e == lane + 64) v1 = false;
+        if (lane == s) {
+            sel_e = e;
+            sel_v = __builtin_bit_cast(float, from);
+        }
+    }
+    float mx = -INFINITY;
+    for (int s = 0; s < k; s++) mx = fmaxf(mx, __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sel_v), s)));
+    const float wv = (lane < k && fabsf(sel_v) < INFINITY) ? expf(sel_v - mx) : 0.0f;  // is_finite: NaN and inf give 0
+    float sum = 0.0f;
+    for (int s = 0; s < k; s++) sum = sum + __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wv), s));
+    const float w = sum > 0.0f ? wv / sum : 1.0f / static_cast<float>(k);
+    // re-sort by weight (descending), ties to the lower index: the rank of (w, index) in that total order
+    const int wk = total_key(w);
+    int rank = 0;
+    for (int s = 0; s < k; s++) {
+        const int ok = total_key(__builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, w), s)));
+        const int oe = __builtin_amdgcn_readlane(sel_e, s);
+        rank += (ok > wk || (ok == wk && oe < sel_e)) ? 1 : 0;
+    }
+    if (live && lane < k) {
+        idx_out[t * k + rank] = sel_e;
+        w_out[t * k + rank] = w;
+    }
+}
+
 // One wave per token, lane l holding experts l and l + 64.  Gemma-4 routing (reference
 // moe_layer_ffn, src/gemma4_runtime.rs:5567-5610; router_top_k, :61-84): softmax over ALL experts
 // (max folded from f32::MIN, exp(v - max), sum left to right in index order, p /= sum), top-k by
@@ -335,8 +383,13 @@ int cml_moe_route_top_k(const float *logits_dev, int64_t n_tokens, int n_experts
     if (k > n_experts) return fail(CML_ERR_SHAPE, "top-%d of %d experts", k, n_experts);
     if (n_tokens == 0) return CML_OK;
     if (!logits_dev || !idx_dev || !weight_dev) return fail(CML_ERR_INVALID, "null pointer");
-    const unsigned grid = static_cast<unsigned>((n_tokens + 63) / 64);
-    hipLaunchKernelGGL(moe_route_kernel, dim3(grid), dim3(64), 0, as_stream(stream), logits_dev, n_tokens, n_experts, k, idx_dev, weight_dev);
+    if (k <= 64) {
+        hipLaunchKernelGGL(moe_route_wave_kernel, dim3(static_cast<unsigned>((n_tokens + 3) / 4)), dim3(256), 0, as_stream(stream), logits_dev,
+                           n_tokens, n_experts, k, idx_dev, weight_dev);
+    } else {
+        hipLaunchKernelGGL(moe_route_kernel, dim3(static_cast<unsigned>((n_tokens + 63) / 64)), dim3(64), 0, as_stream(stream), logits_dev,
+                           n_tokens, n_experts, k, idx_dev, weight_dev);
+    }
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }

@@ -87,6 +87,22 @@ def test_route_top_k_matches_oracle():
         assert list(idx[t]) == list(oi) and np.allclose(w[t], ow, rtol=3e-7)
 
 
+def test_route_top_k_many_experts_both_kernels():
+    """128 experts: k <= 64 takes the wave-per-token kernel, larger k the thread-per-token one."""
+    rng = np.random.default_rng(302)
+    logits = (rng.standard_normal((9, 128)) * 2).astype(np.float32)
+    logits[0] = 1.5                         # all tied
+    logits[1, 100] = np.inf                 # an infinite logit is selected first and gets weight 0
+    logits[2, 5] = np.nan
+    for k in (1, 8, 64, 70, 128):
+        G.say(f"moe route 9x128 top-{k}")
+        _, _, idx, w = gpu_route(logits, k)
+        for t in range(logits.shape[0]):
+            oi, ow = oracle.softmax_top_k(logits[t], k)
+            assert list(idx[t]) == list(oi), (k, t)
+            assert np.allclose(w[t], ow, rtol=1e-6, atol=1e-12, equal_nan=True), (k, t)
+
+
 def _experts(E, hidden, ff, seed):
     gate = G.synth_weight(B.CML_Q4_K, E * ff, hidden, seed)
     up = G.synth_weight(B.CML_Q4_K, E * ff, hidden, seed + 1)
