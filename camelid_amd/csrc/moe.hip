@@ -327,10 +327,22 @@ __global__ __launch_bounds__(256) void moe_weighted_sum_kernel(const float *__re
     const int64_t t = blockIdx.y;
     if (c >= hidden) return;
     float acc = 0.0f;
-    for (int s = 0; s < k; s++) {
-        const int64_t a = slot_to_assign ? slot_to_assign[t * k + s] : t * k + s;
-        if (a < 0 || a >= n_assign) continue;  // a dropped slot (expert id out of range) or a malformed map
-        acc = acc + y[a * hidden + c] * weight[t * k + s];
+    // eight routed slots at a time: their loads go out together, the sum stays in routed order
+    for (int s0 = 0; s0 < k; s0 += 8) {
+        float yv[8], wv[8];
+        bool ok[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int s = s0 + j;
+            const int64_t slot = t * k + min(s, k - 1);
+            const int64_t a = slot_to_assign ? slot_to_assign[slot] : slot;
+            ok[j] = s < k && a >= 0 && a < n_assign;  // a dropped slot (expert id out of range) or a malformed map is skipped
+            yv[j] = y[(ok[j] ? a : 0) * hidden + c];
+            wv[j] = weight[slot];
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+            if (ok[j]) acc = acc + yv[j] * wv[j];
     }
     out[t * hidden + c] = acc;
 }
