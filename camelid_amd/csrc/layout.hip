@@ -298,21 +298,38 @@ __global__ __launch_bounds__(1024) void argmax_f32_kernel(const float *__restric
     const float *row = logits + static_cast<int64_t>(blockIdx.x) * n;
     float best = -3.4e38f;
     int besti = 0;
-    // every thread scans ascending indices, so within a thread the first maximum is kept
-    for (int64_t i = tid; i < n; i += 1024) {
-        const float v = row[i];
-        if (v > best) {
-            best = v;
-            besti = static_cast<int>(i);
-        }
-    }
     // pairs meet keeping the greater value, the lower index on equal values
-    auto meet = [](float &bv, int &bi, float ov, int oi) {
+    auto meet = [](float &bv, int &bi, float ov, int oi) __attribute__((always_inline)) {
         if (ov > bv || (ov == bv && oi < bi)) {
             bv = ov;
             bi = oi;
         }
     };
+    // The row is read as 16-byte pieces, four of them in flight per thread: up to three leading
+    // values before the first aligned address and the values after the last whole piece are taken
+    // one by one.  Every thread meets ascending indices in the body, so strict > keeps its first
+    // maximum; the odd ends go through meet(), which orders equal values by index.
+    const int64_t head = min<int64_t>(n, static_cast<int64_t>((16 - (reinterpret_cast<uintptr_t>(row) & 15)) & 15) >> 2);
+    const int64_t n4 = (n - head) >> 2;
+    const float4 *row4 = reinterpret_cast<const float4 *>(row + head);
+    if (tid < head) meet(best, besti, row[tid], tid);
+    auto take4 = [&](const float4 &v, int64_t p) __attribute__((always_inline)) {
+        const int i0 = static_cast<int>(head + 4 * p);
+        if (v.x > best) { best = v.x; besti = i0; }
+        if (v.y > best) { best = v.y; besti = i0 + 1; }
+        if (v.z > best) { best = v.z; besti = i0 + 2; }
+        if (v.w > best) { best = v.w; besti = i0 + 3; }
+    };
+    int64_t p = tid;
+    for (; p + 3 * 1024 < n4; p += 4 * 1024) {
+        const float4 a = row4[p], b = row4[p + 1024], c = row4[p + 2048], d = row4[p + 3072];
+        take4(a, p);
+        take4(b, p + 1024);
+        take4(c, p + 2048);
+        take4(d, p + 3072);
+    }
+    for (; p < n4; p += 1024) take4(row4[p], p);
+    for (int64_t i = head + 4 * n4 + tid; i < n; i += 1024) meet(best, besti, row[i], static_cast<int>(i));
     for (int m = 1; m < 64; m <<= 1) meet(best, besti, __shfl_xor(best, m), __shfl_xor(besti, m));
     if (lane == 0) {
         sval[wave] = best;

@@ -188,7 +188,7 @@ def test_embed_gather_rows_are_the_block_decode(name, fmt):
 
 def test_argmax_first_maximum_wins():
     rng = np.random.default_rng(1300)
-    for n in (1, 63, 1024, 1025, 128256):
+    for n in (1, 3, 63, 1024, 1025, 4099, 20483, 128256):
         logits = rng.standard_normal((6, n)).astype(np.float32)
         if n > 3:
             logits[1, n // 2] = logits[1, 1] = 9.0          # equal maxima: the lower index
