@@ -146,11 +146,35 @@ def cpu_baseline(fmt: int, wire: np.ndarray, rows: int, cols: int, x: np.ndarray
         oracle.matmul(fmt, wire, cols, x, order=order, threads=threads)
         times.append(time.perf_counter() - t0)
     med = float(np.median(times))
+    # the same call at 1 and 4 threads (the reference's own characterisation found 4 of 8 cores
+    # best on its box): a few calls each, so the default run stays short
+    other = {}
+    for nthr in (1, 4):
+        if nthr >= threads:
+            continue
+        ts = []
+        t_stop = time.perf_counter() + min(2.0, budget_s / 4)
+        while len(ts) < 2 or (time.perf_counter() < t_stop and len(ts) < 20):
+            t0 = time.perf_counter()
+            oracle.matmul(fmt, wire, cols, x, order=order, threads=nthr)
+            ts.append(time.perf_counter() - t0)
+        other[f"us_per_call_{nthr}_threads"] = round(float(np.median(ts)) * 1e6, 1)
     return {
         "value": round(alg_bytes / med / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
-        "us_per_call": round(med * 1e6, 1),
+        "us_per_call": round(med * 1e6, 1), **other, "cpu_model": cpu_model(),
         "sample": f"{len(times)} full calls of the same {rows}x{cols} matvec (quantize + row dots), median",
     }
+
+
+def cpu_model() -> str:
+    try:
+        with open("/proc/cpuinfo") as f:
+            for ln in f:
+                if ln.startswith("model name"):
+                    return ln.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
 
 
 MOE_CONFIGS = {

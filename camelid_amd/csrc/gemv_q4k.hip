@@ -87,8 +87,9 @@ constexpr int kQ4KStageRegs = 4;  // activation chunks a thread holds in registe
 constexpr int kQ4KChunk = 2304;  // bytes of one (tile, super-block) chunk
 constexpr int LPS = 4;           // lanes per super-block
 
+template <int U_>
 struct Q4KRegs {
-    static constexpr int U = 4;  // super-blocks in flight per buffer
+    static constexpr int U = U_;  // super-blocks in flight per buffer and 4-lane group
     uint4 hdr[U];
     uint4 qa[U];
     uint4 qb[U];
@@ -98,16 +99,19 @@ struct Q4KRegs {
 // last one and their result is discarded by the caller): straight-line code
 // lets the compiler keep the next buffer's loads in flight under the current
 // buffer's arithmetic with partial vmcnt waits.  `tile` points at the tile's
-// first chunk; r = row in tile, lane = 4r + c.
-__device__ __forceinline__ void q4k_load(Q4KRegs &r, const uint8_t *tile, int64_t sb_stride, int row_in_tile, int lane,
+// first chunk; row_in_tile = row in the 16-row layout tile, piece = 4*row_in_tile + c.  With SPR
+// groups per row the group's own first super-block comes in `sb` and consecutive buffer entries
+// are SPR super-blocks apart.
+template <int U, int SPR>
+__device__ __forceinline__ void q4k_load(Q4KRegs<U> &r, const uint8_t *tile, int64_t sb_stride, int row_in_tile, int piece,
                                          int sb, int s1) {
 #pragma unroll
-    for (int u = 0; u < Q4KRegs::U; u++) {
-        const int i = min(sb + u, s1 - 1);
+    for (int u = 0; u < U; u++) {
+        const int i = min(sb + u * SPR, s1 - 1);
         const uint8_t *chunk = tile + static_cast<int64_t>(i) * sb_stride;
         r.hdr[u] = ldg16(chunk + row_in_tile * 16);
-        r.qa[u] = ldg16(chunk + 256 + lane * 16);
-        r.qb[u] = ldg16(chunk + 1280 + lane * 16);
+        r.qa[u] = ldg16(chunk + 256 + piece * 16);
+        r.qb[u] = ldg16(chunk + 1280 + piece * 16);
     }
 }
 
@@ -145,14 +149,14 @@ __device__ __forceinline__ void q4k_scale_pairs(const Q4KLane &ln, const uint4 &
     m_pair = ln.upper ? m_up : m_lo;
 }
 
-template <int NT, bool INTS>
-__device__ __forceinline__ void q4k_compute(const Q4KRegs &r, const Q4KLane &ln, int sb, int s1,
+template <int NT, bool INTS, int U, int SPR>
+__device__ __forceinline__ void q4k_compute(const Q4KRegs<U> &r, const Q4KLane &ln, int sb, int s1,
                                             const int8_t *ys, const int *bsum, const float *yds, int n_sb,
                                             float (&acc)[NT], int32_t *ints_row) {
 #pragma unroll
-    for (int u = 0; u < Q4KRegs::U; u++) {
-        const bool valid = sb + u < s1;  // wave-uniform
-        const int i = valid ? sb + u : s1 - 1;
+    for (int u = 0; u < U; u++) {
+        const bool valid = sb + u * SPR < s1;  // wave-uniform when SPR == 1
+        const int i = valid ? sb + u * SPR : s1 - 1;
         uint32_t sc_pair, m_pair;
         q4k_scale_pairs(ln, r.hdr[u], sc_pair, m_pair);
         const int sc_lo = sc_pair & 0xff, sc_hi = sc_pair >> 8;
@@ -182,6 +186,14 @@ __device__ __forceinline__ void q4k_compute(const Q4KRegs &r, const Q4KLane &ln,
             const float ydv = yds[t * n_sb + i];
             const float D = ydv * dw;
             const float M = ydv * dminw;
+            if constexpr (SPR == 2) {
+                // the row's first group hands its terms four lanes up: the second group's last lane
+                // runs the chain in super-block order
+                const float Mp = row_shr_f32<4>(M), Dp = row_shr_f32<4>(D);
+                const float pp = row_shr_f32<4>(static_cast<float>(p_total)), sp = row_shr_f32<4>(static_cast<float>(s_total));
+                acc[t] = __builtin_fmaf(-Mp, pp, acc[t]);
+                acc[t] = __builtin_fmaf(Dp, sp, acc[t]);
+            }
             acc[t] = __builtin_fmaf(-M, static_cast<float>(p_total), acc[t]);
             acc[t] = __builtin_fmaf(D, static_cast<float>(s_total), acc[t]);
             if constexpr (INTS) {
@@ -198,10 +210,18 @@ __device__ __forceinline__ void q4k_compute(const Q4KRegs &r, const Q4KLane &ln,
 // workgroup quantizes it to Q8_K itself, wave w taking super-blocks w, w+waves, ...,
 // straight into the LDS staging area -- the arithmetic of quantize_q8_k_kernel,
 // without the launch and the round trip through memory.
-template <int NT, bool INTS, bool FUSEQ = false>
+//
+// SPR = 2: a wave owns 8 rows and two 4-lane groups per row work on neighbouring super-blocks
+// (lane = 8*row + 4*h + c).  Twice the waves with half the steps each, for weights whose 16-row
+// tiles alone leave one wave per SIMD; every sum keeps its order, so the results are the same bits.
+template <int NT, bool INTS, bool FUSEQ = false, int SPR = 1>
 __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
     static_assert(!FUSEQ || (NT == 1 && !INTS), "the fused quantizer serves single-token calls");
-    constexpr int RPW = kWave / LPS;  // rows per wave tile
+    static_assert(SPR == 1 || SPR == 2, "groups per row");
+    constexpr int RPW = kWave / (LPS * SPR);  // rows per wave tile
+    constexpr int U = 4 / SPR;                // buffer entries per group: a buffer always holds 4 super-blocks of a row
+    constexpr int UB = U * SPR;
+    using Regs = Q4KRegs<U>;
     extern __shared__ uint4 smem[];
     const int n_sb = a.n_sb;
     int8_t *ys = reinterpret_cast<int8_t *>(smem);                     // [NT][n_sb*256]
@@ -227,19 +247,22 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
     const int tile = blockIdx.x * a.tiles_per_wg + tile_in_wg;
     const int s0 = static_cast<int>(static_cast<int64_t>(kpart) * n_sb / W);
     const int s1 = static_cast<int>(static_cast<int64_t>(kpart + 1) * n_sb / W);
-    const int r = lane / LPS, l = lane - r * LPS;
+    const int g = lane / LPS, l = lane - g * LPS;
+    const int r = g / SPR, h = g - r * SPR;
     const int row = tile * RPW + r - a.row_skip;  // output row; negative for the skipped head of a view's first tile
     const bool live = row >= 0 && row < a.rows;
     // the last tile is padded to 16 rows; tiles past the end (grid rounding) re-read it and store nothing
-    const uint8_t *wtile = w + static_cast<int64_t>(min(tile, (a.rows + a.row_skip + 15) / 16 - 1)) * kQ4KChunk;
-    const bool leader = (l == LPS - 1);
+    const int rl = (tile % SPR) * RPW + r;  // row in the 16-row layout tile
+    const uint8_t *wtile = w + static_cast<int64_t>(min(tile / SPR, (a.rows + a.row_skip + 15) / 16 - 1)) * kQ4KChunk;
+    const int piece = rl * LPS + l;
+    const bool gleader = (l == LPS - 1);          // holds its group's integers
+    const bool leader = gleader && h == SPR - 1;  // runs the row's f32 chain
     Q4KLane ln;
     ln.c = l;
     ln.sh = (ln.c & 1) * 16;
     ln.upper = ln.c >= 2;
     const int c16 = n_sb * 16;       // 16-byte chunks per activation row
     const int n16 = NT * c16;        // even; blockDim is even: lanes 2k, 2k+1 are in or out together
-    constexpr int U = Q4KRegs::U;
 
     for (int p0 = 0; p0 < n_assign; p0 += NT) {
         // Activation row of local token t (clamped to the group's last assignment; extra tokens store nothing).
@@ -248,7 +271,7 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
             if (a.shared_act) return 0;
             return a.group_rows ? a.group_rows[j] : j;
         };
-        Q4KRegs ra, rb;
+        Regs ra, rb;
         if constexpr (FUSEQ) {
             // f32 loads of the first batch, the first weight buffer right behind
             // them, then the quantizer: HBM requests are in flight while it runs.
@@ -276,7 +299,7 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
             float4 xa[4], xb[4];
             load_pass(xa, 4 * wave);
             __builtin_amdgcn_sched_barrier(0);
-            q4k_load(ra, wtile, a.sb_stride, r, lane, s0, s1);
+            q4k_load<U, SPR>(ra, wtile, a.sb_stride, rl, piece, s0 + h, s1);
             __builtin_amdgcn_sched_barrier(0);
             for (int base = 4 * wave;;) {
                 const int next = base + 4 * nw;
@@ -311,7 +334,7 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
             }
 
             __builtin_amdgcn_sched_barrier(0);
-            q4k_load(ra, wtile, a.sb_stride, r, lane, s0, s1);
+            q4k_load<U, SPR>(ra, wtile, a.sb_stride, rl, piece, s0 + h, s1);
             __builtin_amdgcn_sched_barrier(0);
 
     #pragma unroll
@@ -343,7 +366,7 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
 
         int32_t *ints_row = nullptr;
         if constexpr (INTS) {
-            if (a.ints && leader && live) ints_row = a.ints + (band * a.rows + row) * static_cast<int64_t>(n_sb) * 2;
+            if (a.ints && gleader && live) ints_row = a.ints + (band * a.rows + row) * static_cast<int64_t>(n_sb) * 2;
         }
 
         float acc[NT];
@@ -355,24 +378,24 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
         // anything, so no load is wasted; sched_barrier keeps the loads ahead of
         // the arithmetic they overlap with.
         for (int sb = s0;;) {
-            if (sb + U >= s1) {
-                q4k_compute<NT, INTS>(ra, ln, sb, s1, ys, bsum, yds, n_sb, acc, ints_row);
+            if (sb + UB >= s1) {
+                q4k_compute<NT, INTS, U, SPR>(ra, ln, sb + h, s1, ys, bsum, yds, n_sb, acc, ints_row);
                 break;
             }
-            q4k_load(rb, wtile, a.sb_stride, r, lane, sb + U, s1);
+            q4k_load<U, SPR>(rb, wtile, a.sb_stride, rl, piece, sb + UB + h, s1);
             __builtin_amdgcn_sched_barrier(0);
-            q4k_compute<NT, INTS>(ra, ln, sb, s1, ys, bsum, yds, n_sb, acc, ints_row);
+            q4k_compute<NT, INTS, U, SPR>(ra, ln, sb + h, s1, ys, bsum, yds, n_sb, acc, ints_row);
             __builtin_amdgcn_sched_barrier(0);
-            sb += U;
-            if (sb + U >= s1) {
-                q4k_compute<NT, INTS>(rb, ln, sb, s1, ys, bsum, yds, n_sb, acc, ints_row);
+            sb += UB;
+            if (sb + UB >= s1) {
+                q4k_compute<NT, INTS, U, SPR>(rb, ln, sb + h, s1, ys, bsum, yds, n_sb, acc, ints_row);
                 break;
             }
-            q4k_load(ra, wtile, a.sb_stride, r, lane, sb + U, s1);
+            q4k_load<U, SPR>(ra, wtile, a.sb_stride, rl, piece, sb + UB + h, s1);
             __builtin_amdgcn_sched_barrier(0);
-            q4k_compute<NT, INTS>(rb, ln, sb, s1, ys, bsum, yds, n_sb, acc, ints_row);
+            q4k_compute<NT, INTS, U, SPR>(rb, ln, sb + h, s1, ys, bsum, yds, n_sb, acc, ints_row);
             __builtin_amdgcn_sched_barrier(0);
-            sb += U;
+            sb += UB;
         }
 
         float *out = (second ? a.out2 : a.out) + static_cast<int64_t>(a0 + p0) * a.rows;  // output row of local token 0
@@ -441,10 +464,23 @@ static Q4KShape pick_shape(int64_t rows, int64_t n_sb) {
 // matrix-core kernel reproduces the same association).
 int q4k_ksplit_for(int64_t rows, int64_t n_sb) { return pick_shape(rows, n_sb).ksplit; }
 
+// Rows per wave of a single-token launch: 8 (two groups per row) when 16-row tiles would leave at
+// most one wave per SIMD of the 256 compute units -- measured on the 14336 x 4096 matvec: twice
+// the waves hide each other's instruction latency as long as the bytes in flight stay the same
+// (8.7 against 9.1 us cache-cold, 6.7 against 7.5 us cache-warm; 4096 x 14336: 9.2 against 9.5).
+// The choice never changes a result bit.
+static int q4k_rows_per_wave(int64_t tiles16, int ksplit, int64_t slots) {
+    const int forced = env_int("CAMELID_HIP_Q4K_ROWS_PER_WAVE", 0);
+    if (forced == 8 || forced == 16) return forced;
+    return tiles16 * ksplit * slots <= 1024 ? 8 : 16;
+}
+
 template <int NT>
 static int launch_q4k_nt(Q4KArgs ka, const Q4KShape &shape, int n_groups, bool ints, hipStream_t st) {
     const int waves = shape.ksplit * shape.tiles_per_wg;
-    const int64_t tiles = (ka.rows + ka.row_skip + 15) / 16;
+    const int64_t tiles16 = (ka.rows + ka.row_skip + 15) / 16;
+    const bool half_tiles = NT == 1 && !ints && q4k_rows_per_wave(tiles16, shape.ksplit, n_groups) == 8;
+    const int64_t tiles = half_tiles ? 2 * tiles16 : tiles16;
     const unsigned gx = static_cast<unsigned>((tiles + shape.tiles_per_wg - 1) / shape.tiles_per_wg);
     const size_t lds = static_cast<size_t>(NT) * ka.n_sb * (256 + 32) + ((static_cast<size_t>(NT) * ka.n_sb + 3) & ~size_t(3)) * 4 +
                        static_cast<size_t>(waves) * NT * 16 * 4;
@@ -453,6 +489,8 @@ static int launch_q4k_nt(Q4KArgs ka, const Q4KShape &shape, int n_groups, bool i
     ka.tiles_per_wg = shape.tiles_per_wg;
     if (ints && NT == 1)
         hipLaunchKernelGGL((gemv_q4k_kernel<1, true>), dim3(gx, n_groups), dim3(64 * waves), lds, st, ka);
+    else if (half_tiles)
+        hipLaunchKernelGGL((gemv_q4k_kernel<1, false, false, 2>), dim3(gx, n_groups), dim3(64 * waves), lds, st, ka);
     else
         hipLaunchKernelGGL((gemv_q4k_kernel<NT, false>), dim3(gx, n_groups), dim3(64 * waves), lds, st, ka);
     CML_HIP_TRY(hipGetLastError());
@@ -510,11 +548,17 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
         ka.out2 = out2;
     }
     Q4KShape shape = pick_shape(ka.rows, ka.n_sb);
+    const int64_t tiles16 = (ka.rows + ka.row_skip + 15) / 16;
+    const int64_t slots = static_cast<int64_t>(grouped ? (a.group_ids ? a.max_active : a.n_groups) : 1) * (w2 ? 2 : 1);
+    const bool half_tiles = q4k_rows_per_wave(tiles16, shape.ksplit, slots) == 8;
+    const int64_t tiles = half_tiles ? 2 * tiles16 : tiles16;
     int tpw = env_int("CAMELID_HIP_Q4K_FUSED_TILES_PER_WG", 0);
+    // 4 waves share the quantizing.  Measured with 8-row tiles at 14336 x 4096 (1792 tiles): 2 waves
+    // 9.6 us, 4 waves 8.7, 8 waves 9.1; 7 waves -- one workgroup for each of the 256 compute units
+    // on paper -- 9.1, and 5 or 6 waves 12.7 / 13.2: workgroups do not land one per unit.
     if (tpw < 1 || tpw * shape.ksplit > 8) tpw = std::max(1, 4 / shape.ksplit);
     shape.tiles_per_wg = tpw;
     const int waves = shape.ksplit * shape.tiles_per_wg;
-    const int64_t tiles = (ka.rows + ka.row_skip + 15) / 16;
     const unsigned gx = static_cast<unsigned>((tiles + shape.tiles_per_wg - 1) / shape.tiles_per_wg);
     const size_t lds = static_cast<size_t>(ka.n_sb) * (256 + 32) + ((static_cast<size_t>(ka.n_sb) + 3) & ~size_t(3)) * 4 +
                        static_cast<size_t>(waves) * 16 * 4;
@@ -522,7 +566,10 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
     ka.ksplit = shape.ksplit;
     ka.tiles_per_wg = shape.tiles_per_wg;
     const dim3 grid(gx, grouped ? (a.group_ids ? a.max_active : a.n_groups) : 1, w2 ? 2 : 1);
-    hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true>), grid, dim3(64 * waves), lds, st, ka);
+    if (half_tiles)
+        hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, 2>), grid, dim3(64 * waves), lds, st, ka);
+    else
+        hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true>), grid, dim3(64 * waves), lds, st, ka);
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }

@@ -188,12 +188,16 @@ def test_q4k_gemv_every_configuration_agrees():
     s, q = oracle.quantize_activation(B.CML_Q4_K, x)
     w = Weight.upload(B.CML_Q4_K, rows, cols, wire)
     for ks, tpw in ((1, 1), (1, 2), (1, 4), (1, 8), (2, 1), (2, 4), (4, 1), (4, 2), (8, 1)):
-        G.say(f"gemv Q4_K ksplit={ks} tiles_per_wg={tpw}")
-        with G.env(CAMELID_HIP_Q4K_KSPLIT=ks, CAMELID_HIP_Q4K_TILES_PER_WG=tpw):
-            got = G.gpu_gemm(w, s, q)
-            ints = G.gpu_block_dots(w, q)
-        check_outputs(B.CML_Q4_K, wire, cols, s, q, got, expect_exact=(ks == 1))
-        assert np.array_equal(ints, oracle.block_ints(B.CML_Q4_K, wire, cols, q))
+        per_rpw = []
+        for rpw in (16, 8):   # rows per wave: 8 = two lane groups per row on neighbouring super-blocks
+            G.say(f"gemv Q4_K ksplit={ks} tiles_per_wg={tpw} rows_per_wave={rpw}")
+            with G.env(CAMELID_HIP_Q4K_KSPLIT=ks, CAMELID_HIP_Q4K_TILES_PER_WG=tpw, CAMELID_HIP_Q4K_ROWS_PER_WAVE=rpw):
+                got = G.gpu_gemm(w, s, q)
+                ints = G.gpu_block_dots(w, q)
+            check_outputs(B.CML_Q4_K, wire, cols, s, q, got, expect_exact=(ks == 1))
+            assert np.array_equal(ints, oracle.block_ints(B.CML_Q4_K, wire, cols, q))
+            per_rpw.append(got)
+        assert G.same_bits(per_rpw[0], per_rpw[1])
 
 
 @pytest.mark.parametrize("name,fmt", FMTS)
@@ -204,8 +208,16 @@ def test_gemv_residual_and_band_view(name, fmt):
     x = rng.standard_normal(cols).astype(np.float32)
     s, q = oracle.quantize_activation(fmt, x)
     w = Weight.upload(fmt, rows, cols, wire)
-    G.say(f"gemv residual {name}")
     res = rng.standard_normal(rows).astype(np.float32)
+    for rpw in (16, 8):
+        G.say(f"gemv residual {name} rows_per_wave={rpw}")
+        with G.env(CAMELID_HIP_Q4K_ROWS_PER_WAVE=rpw):
+            _residual_and_band_view(name, fmt, rows, cols, wire, w, x, s, q, res, rng)
+        if fmt != oracle.Q4_K:
+            break
+
+
+def _residual_and_band_view(name, fmt, rows, cols, wire, w, x, s, q, res, rng):
     with G.env(CAMELID_HIP_EXACT_ORDER="1"):
         base = G.gpu_gemm(w, s, q)
         got = G.gpu_gemm(w, s, q, residual=res)
@@ -265,7 +277,7 @@ def test_matmul_f32_is_quantize_then_gemm(name, fmt):
         assert G.same_bits(got, want)
 
 
-@pytest.mark.parametrize("rows,cols", [(190, 3072), (64, 256), (333, 4096), (48, 14336)])
+@pytest.mark.parametrize("rows,cols", [(190, 3072), (64, 256), (333, 4096), (48, 14336), (77, 1280)])
 def test_q4k_fused_quantize_matvec_is_the_two_step_path(rows, cols):
     """Single-token cml_matmul_f32 on Q4_K quantizes inside the matvec kernel: same bits as
     quantize_q8_k followed by the matvec, for every workgroup shape, on activations with zero
@@ -281,17 +293,18 @@ def test_q4k_fused_quantize_matvec_is_the_two_step_path(rows, cols):
     acts[1, 3] = np.nan
     acts[2, -256:] = 0.0
     for i, x in enumerate(acts):
-        for tpw in (0, 1, 2, 4, 8):
+        for tpw in (0, 1, 2, 3, 4, 7, 8):
             for ks in (0, 1, 2):
                 if ks > cols // 256:
                     continue
-                G.say(f"Q4_K fused quantize+matvec {rows}x{cols} act={i} tiles_per_wg={tpw} ksplit={ks}")
-                with G.env(CAMELID_HIP_Q4K_FUSED_TILES_PER_WG=tpw, CAMELID_HIP_Q4K_KSPLIT=ks):
-                    with G.env(CAMELID_HIP_FUSED_QUANT=2):   # also where the shape policy would not fuse
-                        fused = G.gpu_matmul_f32(w, x)
-                    with G.env(CAMELID_HIP_FUSED_QUANT=0):
-                        two_step = G.gpu_matmul_f32(w, x)
-                assert G.same_bits(fused, two_step)
+                for rpw in (16, 8):
+                    G.say(f"Q4_K fused quantize+matvec {rows}x{cols} act={i} tiles_per_wg={tpw} ksplit={ks} rows_per_wave={rpw}")
+                    with G.env(CAMELID_HIP_Q4K_FUSED_TILES_PER_WG=tpw, CAMELID_HIP_Q4K_KSPLIT=ks, CAMELID_HIP_Q4K_ROWS_PER_WAVE=rpw):
+                        with G.env(CAMELID_HIP_FUSED_QUANT=2):   # also where the shape policy would not fuse
+                            fused = G.gpu_matmul_f32(w, x)
+                        with G.env(CAMELID_HIP_FUSED_QUANT=0, CAMELID_HIP_Q4K_ROWS_PER_WAVE=16):
+                            two_step = G.gpu_matmul_f32(w, x)
+                    assert G.same_bits(fused, two_step)
         if i != 1:  # the oracle's f64 criterion has no meaning for a NaN input; bits above cover it
             with G.env(CAMELID_HIP_EXACT_ORDER="1"):
                 got = G.gpu_matmul_f32(w, x)
