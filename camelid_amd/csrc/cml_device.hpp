@@ -20,6 +20,18 @@ constexpr int kWave = 64;
 __device__ __forceinline__ uint4 ldg16(const void *p) {
     return *reinterpret_cast<const uint4 *>(p);
 }
+// The bulk of a weight is read once per launch: the non-temporal hint keeps it from displacing
+// what is reused (activations, scale planes) on its way through the caches.  Measured on the
+// 14336 x 4096 Q4_K matvec, cache-cold: 8.7 -> 8.1 us.
+__device__ __forceinline__ uint4 ldg16_stream(const void *p) {
+#ifdef CML_PLAIN_WEIGHT_LOADS
+    return ldg16(p);
+#else
+    typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+    const v4u v = __builtin_nontemporal_load(reinterpret_cast<const v4u *>(p));
+    return make_uint4(v.x, v.y, v.z, v.w);
+#endif
+}
 __device__ __forceinline__ uint2 ldg8(const void *p) {
     return *reinterpret_cast<const uint2 *>(p);
 }

@@ -109,9 +109,25 @@ __device__ __forceinline__ void q4k_load(Q4KRegs<U> &r, const uint8_t *tile, int
     for (int u = 0; u < U; u++) {
         const int i = min(sb + u * SPR, s1 - 1);
         const uint8_t *chunk = tile + static_cast<int64_t>(i) * sb_stride;
-        r.hdr[u] = ldg16(chunk + row_in_tile * 16);
-        r.qa[u] = ldg16(chunk + 256 + piece * 16);
-        r.qb[u] = ldg16(chunk + 1280 + piece * 16);
+        r.hdr[u] = ldg16_stream(chunk + row_in_tile * 16);
+        r.qa[u] = ldg16_stream(chunk + 256 + piece * 16);
+        r.qb[u] = ldg16_stream(chunk + 1280 + piece * 16);
+    }
+}
+
+// The same loads for a buffer that lies wholly inside the part (no clamping): a wave-uniform
+// 64-bit base per entry plus two 32-bit lane constants.  The clamped form multiplies a per-lane
+// index by the 64-bit stride for every entry -- quarter-rate instructions that were about a
+// seventh of the loop's vector time.  `ubase` = the tile's chunk of super-block `sb` (uniform);
+// hdr_off / q_off = the lane's own offsets inside a chunk plus h * stride.
+template <int U, int SPR>
+__device__ __forceinline__ void q4k_load_whole(Q4KRegs<U> &r, const uint8_t *ubase, int64_t sb_stride, uint32_t hdr_off, uint32_t q_off) {
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const uint8_t *chunk = ubase + static_cast<int64_t>(u * SPR) * sb_stride;
+        r.hdr[u] = ldg16_stream(chunk + hdr_off);
+        r.qa[u] = ldg16_stream(chunk + 256 + q_off);
+        r.qb[u] = ldg16_stream(chunk + 1280 + q_off);
     }
 }
 
@@ -149,13 +165,13 @@ __device__ __forceinline__ void q4k_scale_pairs(const Q4KLane &ln, const uint4 &
     m_pair = ln.upper ? m_up : m_lo;
 }
 
-template <int NT, bool INTS, int U, int SPR>
+template <int NT, bool INTS, int U, int SPR, bool WHOLE = false>
 __device__ __forceinline__ void q4k_compute(const Q4KRegs<U> &r, const Q4KLane &ln, int sb, int s1,
                                             const int8_t *ys, const int *bsum, const float *yds, int n_sb,
                                             float (&acc)[NT], int32_t *ints_row) {
 #pragma unroll
     for (int u = 0; u < U; u++) {
-        const bool valid = sb + u * SPR < s1;  // wave-uniform when SPR == 1
+        const bool valid = WHOLE || sb + u * SPR < s1;  // wave-uniform when SPR == 1
         const int i = valid ? sb + u * SPR : s1 - 1;
         uint32_t sc_pair, m_pair;
         q4k_scale_pairs(ln, r.hdr[u], sc_pair, m_pair);
@@ -214,7 +230,7 @@ __device__ __forceinline__ void q4k_compute(const Q4KRegs<U> &r, const Q4KLane &
 // SPR = 2: a wave owns 8 rows and two 4-lane groups per row work on neighbouring super-blocks
 // (lane = 8*row + 4*h + c).  Twice the waves with half the steps each, for weights whose 16-row
 // tiles alone leave one wave per SIMD; every sum keeps its order, so the results are the same bits.
-template <int NT, bool INTS, bool FUSEQ = false, int SPR = 1>
+template <int NT, bool INTS, bool FUSEQ = false, int SPR = 1, bool WHOLE = false>
 __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
     static_assert(!FUSEQ || (NT == 1 && !INTS), "the fused quantizer serves single-token calls");
     static_assert(SPR == 1 || SPR == 2, "groups per row");
@@ -255,6 +271,16 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
     const int rl = (tile % SPR) * RPW + r;  // row in the 16-row layout tile
     const uint8_t *wtile = w + static_cast<int64_t>(min(tile / SPR, (a.rows + a.row_skip + 15) / 16 - 1)) * kQ4KChunk;
     const int piece = rl * LPS + l;
+    // lane constants of the unclamped loads (WHOLE: every part is a whole number of buffers and
+    // the stride fits 31 bits -- the launcher checks both)
+    const uint32_t hoff = WHOLE ? static_cast<uint32_t>(h) * static_cast<uint32_t>(a.sb_stride) : 0u;
+    const uint32_t hdr_off = hoff + rl * 16, q_off = hoff + piece * 16;
+    auto load_buffer = [&](Regs &dst, int sb) __attribute__((always_inline)) {  // super-blocks sb .. sb+UB-1 of the row
+        if constexpr (WHOLE)
+            q4k_load_whole<U, SPR>(dst, wtile + static_cast<int64_t>(sb) * a.sb_stride, a.sb_stride, hdr_off, q_off);
+        else
+            q4k_load<U, SPR>(dst, wtile, a.sb_stride, rl, piece, sb + h, s1);
+    };
     const bool gleader = (l == LPS - 1);          // holds its group's integers
     const bool leader = gleader && h == SPR - 1;  // runs the row's f32 chain
     Q4KLane ln;
@@ -299,7 +325,7 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
             float4 xa[4], xb[4];
             load_pass(xa, 4 * wave);
             __builtin_amdgcn_sched_barrier(0);
-            q4k_load<U, SPR>(ra, wtile, a.sb_stride, rl, piece, s0 + h, s1);
+            load_buffer(ra, s0);
             __builtin_amdgcn_sched_barrier(0);
             for (int base = 4 * wave;;) {
                 const int next = base + 4 * nw;
@@ -334,7 +360,7 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
             }
 
             __builtin_amdgcn_sched_barrier(0);
-            q4k_load<U, SPR>(ra, wtile, a.sb_stride, rl, piece, s0 + h, s1);
+            load_buffer(ra, s0);
             __builtin_amdgcn_sched_barrier(0);
 
     #pragma unroll
@@ -379,21 +405,21 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
         // the arithmetic they overlap with.
         for (int sb = s0;;) {
             if (sb + UB >= s1) {
-                q4k_compute<NT, INTS, U, SPR>(ra, ln, sb + h, s1, ys, bsum, yds, n_sb, acc, ints_row);
+                q4k_compute<NT, INTS, U, SPR, WHOLE>(ra, ln, sb + h, s1, ys, bsum, yds, n_sb, acc, ints_row);
                 break;
             }
-            q4k_load<U, SPR>(rb, wtile, a.sb_stride, rl, piece, sb + UB + h, s1);
+            load_buffer(rb, sb + UB);
             __builtin_amdgcn_sched_barrier(0);
-            q4k_compute<NT, INTS, U, SPR>(ra, ln, sb + h, s1, ys, bsum, yds, n_sb, acc, ints_row);
+            q4k_compute<NT, INTS, U, SPR, WHOLE>(ra, ln, sb + h, s1, ys, bsum, yds, n_sb, acc, ints_row);
             __builtin_amdgcn_sched_barrier(0);
             sb += UB;
             if (sb + UB >= s1) {
-                q4k_compute<NT, INTS, U, SPR>(rb, ln, sb + h, s1, ys, bsum, yds, n_sb, acc, ints_row);
+                q4k_compute<NT, INTS, U, SPR, WHOLE>(rb, ln, sb + h, s1, ys, bsum, yds, n_sb, acc, ints_row);
                 break;
             }
-            q4k_load<U, SPR>(ra, wtile, a.sb_stride, rl, piece, sb + UB + h, s1);
+            load_buffer(ra, sb + UB);
             __builtin_amdgcn_sched_barrier(0);
-            q4k_compute<NT, INTS, U, SPR>(rb, ln, sb + h, s1, ys, bsum, yds, n_sb, acc, ints_row);
+            q4k_compute<NT, INTS, U, SPR, WHOLE>(rb, ln, sb + h, s1, ys, bsum, yds, n_sb, acc, ints_row);
             __builtin_amdgcn_sched_barrier(0);
             sb += UB;
         }
@@ -475,6 +501,13 @@ static int q4k_rows_per_wave(int64_t tiles16, int ksplit, int64_t slots) {
     return tiles16 * ksplit * slots <= 1024 ? 8 : 16;
 }
 
+// Every K part a whole number of 4-super-block buffers and a stride of less than 2 GiB: the
+// kernel variant whose loads need no clamping applies.
+static bool q4k_whole_buffers(const Q4KArgs &ka, int ksplit) {
+    if (env_int("CAMELID_HIP_Q4K_CLAMPED_LOADS", 0)) return false;
+    return ka.n_sb % (4 * ksplit) == 0 && ka.sb_stride < (int64_t(1) << 31);
+}
+
 template <int NT>
 static int launch_q4k_nt(Q4KArgs ka, const Q4KShape &shape, int n_groups, bool ints, hipStream_t st) {
     const int waves = shape.ksplit * shape.tiles_per_wg;
@@ -489,7 +522,12 @@ static int launch_q4k_nt(Q4KArgs ka, const Q4KShape &shape, int n_groups, bool i
     ka.tiles_per_wg = shape.tiles_per_wg;
     if (ints && NT == 1)
         hipLaunchKernelGGL((gemv_q4k_kernel<1, true>), dim3(gx, n_groups), dim3(64 * waves), lds, st, ka);
-    else if (half_tiles)
+    else if (NT == 1 && q4k_whole_buffers(ka, shape.ksplit)) {
+        if (half_tiles)
+            hipLaunchKernelGGL((gemv_q4k_kernel<1, false, false, 2, true>), dim3(gx, n_groups), dim3(64 * waves), lds, st, ka);
+        else
+            hipLaunchKernelGGL((gemv_q4k_kernel<1, false, false, 1, true>), dim3(gx, n_groups), dim3(64 * waves), lds, st, ka);
+    } else if (half_tiles)
         hipLaunchKernelGGL((gemv_q4k_kernel<1, false, false, 2>), dim3(gx, n_groups), dim3(64 * waves), lds, st, ka);
     else
         hipLaunchKernelGGL((gemv_q4k_kernel<NT, false>), dim3(gx, n_groups), dim3(64 * waves), lds, st, ka);
@@ -566,7 +604,12 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
     ka.ksplit = shape.ksplit;
     ka.tiles_per_wg = shape.tiles_per_wg;
     const dim3 grid(gx, grouped ? (a.group_ids ? a.max_active : a.n_groups) : 1, w2 ? 2 : 1);
-    if (half_tiles)
+    if (q4k_whole_buffers(ka, shape.ksplit)) {
+        if (half_tiles)
+            hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, 2, true>), grid, dim3(64 * waves), lds, st, ka);
+        else
+            hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, 1, true>), grid, dim3(64 * waves), lds, st, ka);
+    } else if (half_tiles)
         hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, 2>), grid, dim3(64 * waves), lds, st, ka);
     else
         hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true>), grid, dim3(64 * waves), lds, st, ka);

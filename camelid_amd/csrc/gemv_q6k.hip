@@ -64,8 +64,8 @@ __device__ __forceinline__ void q6k_load(Q6KRegs &r, const uint8_t *ql, const ui
 #pragma unroll
     for (int u = 0; u < Q6KRegs::U; u++) {
         const int64_t i = min(sb + u, s1 - 1);
-        r.ql[u] = ldg16(ql + i * 128 + 64 * h + 32 * p + 16 * s);
-        r.qh[u] = ldg16(qh + i * 64 + 32 * h + 16 * s);
+        r.ql[u] = ldg16_stream(ql + i * 128 + 64 * h + 32 * p + 16 * s);
+        r.qh[u] = ldg16_stream(qh + i * 64 + 32 * h + 16 * s);
         r.sc[u] = ldg16(sc + i * 16);
         r.d[u] = ldg2(d + i * 2);
     }

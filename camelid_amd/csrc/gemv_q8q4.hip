@@ -63,10 +63,16 @@ __device__ __forceinline__ void b32_load(B32Regs<FMT, U> &r, const uint8_t *qrow
     for (int u = 0; u < U; u++) {
         const int b = min(min(step + u, n_steps - 1) * P + l, nb - 1);
         if constexpr (FMT == CML_Q8_0) {
+            // two loads per 32-byte block: each touches half of every line, so the lines must
+            // stay cached between them (the streaming hint cost 0.25 us at 8192 x 2048)
             r.qa[u] = ldg16(qrow + static_cast<int64_t>(b) * 32);
             r.qb[u] = ldg16(qrow + static_cast<int64_t>(b) * 32 + 16);
+        } else if constexpr (P >= 8) {
+            // a row's lanes read whole 128-byte lines per step: read-once data
+            // (128256 x 3072: 36.9 -> 32.8 us)
+            r.qa[u] = ldg16_stream(qrow + static_cast<int64_t>(b) * 16);
         } else {
-            r.qa[u] = ldg16(qrow + static_cast<int64_t>(b) * 16);
+            r.qa[u] = ldg16(qrow + static_cast<int64_t>(b) * 16);  // 4 lanes: a line lasts two steps
         }
         r.d[u] = ldg2(srow + static_cast<int64_t>(b) * 2);
     }
