@@ -74,6 +74,7 @@ CONFIGS = {
     "q6k_128256x3072_n4": ("Q6_K", 128256, 3072, 4),
     "q6k_128256x3072_n8": ("Q6_K", 128256, 3072, 8),
     "q6k_128256x3072_n64": ("Q6_K", 128256, 3072, 64),
+    "q6k_4096x14336_n1": ("Q6_K", 4096, 14336, 1),
     "q6k_4096x14336_n4": ("Q6_K", 4096, 14336, 4),
     "q6k_4096x14336_n8": ("Q6_K", 4096, 14336, 8),
     "q6k_4096x14336_n16": ("Q6_K", 4096, 14336, 16),

@@ -48,37 +48,41 @@ struct Q6KArgs {
     int ksplit;
 };
 
+template <int U_>
 struct Q6KRegs {
-    static constexpr int U = 2;
+    static constexpr int U = U_;  // super-blocks in flight per buffer
     uint4 ql[U];
     uint4 qh[U];
     uint4 sc[U];
     uint32_t d[U];
 };
 
-__device__ __forceinline__ void q6k_load(Q6KRegs &r, const uint8_t *ql, const uint8_t *qh, const uint8_t *sc,
+template <int U>
+__device__ __forceinline__ void q6k_load(Q6KRegs<U> &r, const uint8_t *ql, const uint8_t *qh, const uint8_t *sc,
                                          const uint8_t *d, int l, int sb, int s1) {
     const int h = l >> 2, p = (l >> 1) & 1, s = l & 1;
     // Unconditional, clamped loads (results past the end are discarded by the
     // caller) keep the loop body straight-line so loads stay in flight.
 #pragma unroll
-    for (int u = 0; u < Q6KRegs::U; u++) {
+    for (int u = 0; u < U; u++) {
         const int64_t i = min(sb + u, s1 - 1);
         r.ql[u] = ldg16_stream(ql + i * 128 + 64 * h + 32 * p + 16 * s);
-        r.qh[u] = ldg16_stream(qh + i * 64 + 32 * h + 16 * s);
+        // half a line per instruction (the other half belongs to the next super-block): the line
+        // must stay cached in between, so no streaming hint here (128256 x 3072: 55.1 -> 49.7 us)
+        r.qh[u] = ldg16(qh + i * 64 + 32 * h + 16 * s);
         r.sc[u] = ldg16(sc + i * 16);
         r.d[u] = ldg2(d + i * 2);
     }
 }
 
-template <int NT, bool INTS>
-__device__ __forceinline__ void q6k_compute(const Q6KRegs &r, int l, int sb, int s1, const int8_t *ys,
+template <int NT, bool INTS, int U>
+__device__ __forceinline__ void q6k_compute(const Q6KRegs<U> &r, int l, int sb, int s1, const int8_t *ys,
                                             const int *bsum16, const float *yds, int n_sb, float (&acc)[NT],
                                             int32_t *ints_row) {
     const int h = l >> 2, p = (l >> 1) & 1, s = l & 1;
     const int g_lo = 8 * h + 2 * p + s;  // scale / 16-group index of the low-nibble values
 #pragma unroll
-    for (int u = 0; u < Q6KRegs::U; u++) {
+    for (int u = 0; u < U; u++) {
         const bool valid = sb + u < s1;  // wave-uniform
         const int i = valid ? sb + u : s1 - 1;
         // scales: byte g_lo of the 16, and byte g_lo + 4
@@ -124,7 +128,10 @@ __device__ __forceinline__ void q6k_compute(const Q6KRegs &r, int l, int sb, int
     }
 }
 
-template <int NT, bool INTS, bool GROUPED = false>
+// U = super-blocks per register buffer: 2, or 4 for weights with thousands of row tiles (an LM
+// head), where the deeper queue per wave pays (128256 x 3072: 49.3 -> 47.1 us; at 4096 x 14336 it
+// costs 1 us).
+template <int NT, bool INTS, bool GROUPED = false, int U = 2>
 __global__ __launch_bounds__(256) void gemv_q6k_kernel(Q6KArgs a) {
     static_assert(!(GROUPED && INTS), "block-int diagnostics are for plain calls");
     constexpr int LPS = 8, RPW = kWave / LPS;
@@ -207,29 +214,28 @@ __global__ __launch_bounds__(256) void gemv_q6k_kernel(Q6KArgs a) {
 #pragma unroll
         for (int t = 0; t < NT; t++) acc[t] = 0.0f;
 
-        constexpr int U = Q6KRegs::U;
-        Q6KRegs ra, rb;
+        Q6KRegs<U> ra, rb;
         q6k_load(ra, ql, qh, sc, dp, l, s0, s1);
         __builtin_amdgcn_sched_barrier(0);
         // Two register buffers alternate; the last one is consumed without issuing
         // further loads.
         for (int sb = s0;;) {
             if (sb + U >= s1) {
-                q6k_compute<NT, INTS>(ra, l, sb, s1, ys, bsum16, yds, n_sb, acc, ints_row);
+                q6k_compute<NT, INTS, U>(ra, l, sb, s1, ys, bsum16, yds, n_sb, acc, ints_row);
                 break;
             }
             q6k_load(rb, ql, qh, sc, dp, l, sb + U, s1);
             __builtin_amdgcn_sched_barrier(0);
-            q6k_compute<NT, INTS>(ra, l, sb, s1, ys, bsum16, yds, n_sb, acc, ints_row);
+            q6k_compute<NT, INTS, U>(ra, l, sb, s1, ys, bsum16, yds, n_sb, acc, ints_row);
             __builtin_amdgcn_sched_barrier(0);
             sb += U;
             if (sb + U >= s1) {
-                q6k_compute<NT, INTS>(rb, l, sb, s1, ys, bsum16, yds, n_sb, acc, ints_row);
+                q6k_compute<NT, INTS, U>(rb, l, sb, s1, ys, bsum16, yds, n_sb, acc, ints_row);
                 break;
             }
             q6k_load(ra, ql, qh, sc, dp, l, sb + U, s1);
             __builtin_amdgcn_sched_barrier(0);
-            q6k_compute<NT, INTS>(rb, l, sb, s1, ys, bsum16, yds, n_sb, acc, ints_row);
+            q6k_compute<NT, INTS, U>(rb, l, sb, s1, ys, bsum16, yds, n_sb, acc, ints_row);
             __builtin_amdgcn_sched_barrier(0);
             sb += U;
         }
@@ -292,6 +298,8 @@ static int launch_q6k_nt(const Q6KArgs &ka, int n_bands, bool ints, bool grouped
         hipLaunchKernelGGL((gemv_q6k_kernel<NT, false, true>), dim3(gx, n_bands), dim3(256), lds, st, ka);
     else if (ints && NT == 1)
         hipLaunchKernelGGL((gemv_q6k_kernel<1, true>), dim3(gx, n_bands), dim3(256), lds, st, ka);
+    else if (NT == 1 && tiles >= env_int("CAMELID_HIP_Q6K_DEEP_MIN_TILES", 2048))
+        hipLaunchKernelGGL((gemv_q6k_kernel<1, false, false, 4>), dim3(gx, n_bands), dim3(256), lds, st, ka);
     else
         hipLaunchKernelGGL((gemv_q6k_kernel<NT, false>), dim3(gx, n_bands), dim3(256), lds, st, ka);
     CML_HIP_TRY(hipGetLastError());

@@ -178,6 +178,13 @@ def test_gemv_matches_oracle_small_and_ragged(name, fmt):
         check_outputs(fmt, wire, cols, s, q, got, expect_exact=True)
         got = G.gpu_gemm(w, s, q)  # default K-split policy: tolerance only
         check_outputs(fmt, wire, cols, s, q, got, expect_exact=False)
+        if fmt == B.CML_Q6_K:
+            # the deeper register buffers taken for weights with thousands of row tiles: same bits
+            with G.env(CAMELID_HIP_Q6K_DEEP_MIN_TILES=1):
+                assert G.same_bits(G.gpu_gemm(w, s, q), got)
+                assert G.same_bits(G.gpu_matmul_f32(w, x), G.gpu_matmul_f32(w, x))
+            with G.env(CAMELID_HIP_Q6K_DEEP_MIN_TILES=1, CAMELID_HIP_EXACT_ORDER="1"):
+                check_outputs(fmt, wire, cols, s, q, G.gpu_gemm(w, s, q), expect_exact=True)
 
 
 def test_q4k_gemv_every_configuration_agrees():
