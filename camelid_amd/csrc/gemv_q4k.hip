@@ -522,14 +522,16 @@ static int launch_q4k_nt(Q4KArgs ka, const Q4KShape &shape, int n_groups, bool i
     ka.tiles_per_wg = shape.tiles_per_wg;
     if (ints && NT == 1)
         hipLaunchKernelGGL((gemv_q4k_kernel<1, true>), dim3(gx, n_groups), dim3(64 * waves), lds, st, ka);
-    else if (NT == 1 && q4k_whole_buffers(ka, shape.ksplit)) {
+    else if (NT <= 2 && q4k_whole_buffers(ka, shape.ksplit)) {
+        constexpr int NTS = NT <= 2 ? NT : 1;
         if (half_tiles)
-            hipLaunchKernelGGL((gemv_q4k_kernel<1, false, false, 2, true>), dim3(gx, n_groups), dim3(64 * waves), lds, st, ka);
+            hipLaunchKernelGGL((gemv_q4k_kernel<NTS, false, false, 2, true>), dim3(gx, n_groups), dim3(64 * waves), lds, st, ka);
         else
-            hipLaunchKernelGGL((gemv_q4k_kernel<1, false, false, 1, true>), dim3(gx, n_groups), dim3(64 * waves), lds, st, ka);
-    } else if (half_tiles)
-        hipLaunchKernelGGL((gemv_q4k_kernel<1, false, false, 2>), dim3(gx, n_groups), dim3(64 * waves), lds, st, ka);
-    else
+            hipLaunchKernelGGL((gemv_q4k_kernel<NTS, false, false, 1, true>), dim3(gx, n_groups), dim3(64 * waves), lds, st, ka);
+    } else if (half_tiles) {
+        constexpr int NTS = NT <= 2 ? NT : 1;
+        hipLaunchKernelGGL((gemv_q4k_kernel<NTS, false, false, 2>), dim3(gx, n_groups), dim3(64 * waves), lds, st, ka);
+    } else
         hipLaunchKernelGGL((gemv_q4k_kernel<NT, false>), dim3(gx, n_groups), dim3(64 * waves), lds, st, ka);
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;

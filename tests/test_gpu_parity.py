@@ -194,6 +194,8 @@ def test_q4k_gemv_every_configuration_agrees():
     x = rng.standard_normal(cols).astype(np.float32)
     s, q = oracle.quantize_activation(B.CML_Q4_K, x)
     w = Weight.upload(B.CML_Q4_K, rows, cols, wire)
+    x2 = np.stack([x, rng.standard_normal(cols).astype(np.float32)])
+    s2, q2 = oracle.quantize_activation(B.CML_Q4_K, x2)
     for ks, tpw in ((1, 1), (1, 2), (1, 4), (1, 8), (2, 1), (2, 4), (4, 1), (4, 2), (8, 1)):
         per_rpw = []
         for rpw in (16, 8):   # rows per wave: 8 = two lane groups per row on neighbouring super-blocks
@@ -204,6 +206,15 @@ def test_q4k_gemv_every_configuration_agrees():
             check_outputs(B.CML_Q4_K, wire, cols, s, q, got, expect_exact=(ks == 1))
             assert np.array_equal(ints, oracle.block_ints(B.CML_Q4_K, wire, cols, q))
             per_rpw.append(got)
+            # the load form with per-lane clamping (taken when a K part is not whole buffers) and
+            # the one without: same bits, one and two tokens
+            with G.env(CAMELID_HIP_Q4K_KSPLIT=ks, CAMELID_HIP_Q4K_TILES_PER_WG=tpw, CAMELID_HIP_Q4K_ROWS_PER_WAVE=rpw,
+                       CAMELID_HIP_Q4K_MFMA_MIN_TOKENS=1 << 30):
+                two = G.gpu_gemm(w, s2, q2)
+                with G.env(CAMELID_HIP_Q4K_CLAMPED_LOADS=1):
+                    assert G.same_bits(G.gpu_gemm(w, s, q), got)
+                    assert G.same_bits(G.gpu_gemm(w, s2, q2), two)
+            assert G.same_bits(two[0], got) and not G.same_bits(two[1], got)
         assert G.same_bits(per_rpw[0], per_rpw[1])
 
 
