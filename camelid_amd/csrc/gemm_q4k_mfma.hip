@@ -246,7 +246,7 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
             const uint32_t lo = scale & 7u, hi = scale >> 3;
             const uint32_t lo2 = lo | (lo << 16), hi2 = hi | (hi << 16);
             const uint32_t m = (mw >> sh) & 0xff;
-            const int m4 = static_cast<int>(__umul24(m, 0x010101u) | (m << 24));  // m < 64 in all four bytes
+            const int m4 = static_cast<int>(__builtin_amdgcn_perm(m, m, 0u));  // byte 0 (m < 64) in all four bytes
             bm[c] = v4i{m4, m4, m4, m4};
             const uint4 &pc = w0.piece[c];
             const uint32_t n0 = (pc.x >> nib_shift) & 0x0f0f0f0fu, n1 = (pc.y >> nib_shift) & 0x0f0f0f0fu;

@@ -117,7 +117,8 @@ __device__ __forceinline__ void q6k_compute(const Q6KRegs<U> &r, int l, int sb, 
             const int *bs = bsum16 + (t * n_sb + i) * 16;
             lo -= 32 * bs[g_lo];
             hi -= 32 * bs[g_lo + 4];
-            int total = group_sum_to_last<8>(lo * sc_lo + hi * sc_hi);
+            // |lo|, |hi| <= 16*63*127 + 32*16*127 and int8 scales: every product fits 24 bits (full-rate multiplies)
+            int total = group_sum_to_last<8>(__mul24(lo, sc_lo) + __mul24(hi, sc_hi));
             total = valid ? total : 0;  // fma(x, 0, acc) leaves acc unchanged
             const float dd = dw * yds[t * n_sb + i];
             acc[t] = __builtin_fmaf(dd, static_cast<float>(total), acc[t]);
