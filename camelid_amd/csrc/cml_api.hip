@@ -440,6 +440,16 @@ int cml_rms_norm_quantize(int act, const float *x_dev, const float *weight_dev, 
     return launch_rms_norm_quantize(act, x_dev, weight_dev, eps, n_tokens, cols, normed_dev, q_dev, scales_dev, as_stream(stream));
 }
 
+int cml_sum_squares_f32(const float *x_dev, int64_t n_rows, int64_t cols, float *out_dev, cml_stream_t stream) {
+    if (int rc = check_ready()) return rc;
+    if (n_rows < 0 || cols < 0 || cols % 4 != 0) return fail(CML_ERR_SHAPE, "cols %lld is not a multiple of 4", (long long)cols);
+    if (n_rows == 0) return CML_OK;
+    if (!x_dev || !out_dev) return fail(CML_ERR_INVALID, "null pointer");
+    if (misaligned16(x_dev)) return fail(CML_ERR_INVALID, "x must be 16-byte aligned");
+    if (cols == 0) return cml_memset_dev(out_dev, 0, static_cast<size_t>(n_rows) * 4, stream);
+    return launch_rms_norm_quantize(3, x_dev, nullptr, 0.0f, n_rows, cols, out_dev, nullptr, nullptr, as_stream(stream));
+}
+
 int cml_silu_mul_quantize(int act, const float *gate_dev, const float *up_dev, int64_t n_tokens, int64_t cols, int8_t *q_dev,
                           float *scales_dev, cml_stream_t stream) {
     return cml_glu_quantize(CML_GLU_SILU, act, gate_dev, up_dev, n_tokens, cols, q_dev, scales_dev, stream);

@@ -161,10 +161,17 @@ enum { CML_ACT_F32 = 0, CML_ACT_Q8_0 = 1, CML_ACT_Q8_K = 2 };
  * (reference rms_norm_quantize / rms_norm_quantize_q8k, src/cuda_resident.rs:
  * 236-270, :4152-4177).  normed_dev (f32[n_tokens*cols]) may be null when only
  * the quantized form is wanted; q_dev/scales_dev are ignored for CML_ACT_F32.
- * Rows of up to 16352 values. */
+ * Rows of up to 16384 values. */
 int cml_rms_norm_quantize(int act, const float *x_dev, const float *weight_dev, float eps,
                           int64_t n_tokens, int64_t cols, float *normed_dev, int8_t *q_dev,
                           float *scales_dev, cml_stream_t stream);
+/* The first pass of the norm on its own: out_dev[r] = (((0 + x[r][0]^2) + x[r][1]^2) + ...) in f32,
+ * every product and every sum rounded, in index order -- the bits of the scalar
+ * loop (reference rms_norm's ordered sum, src/cuda_resident.rs:124-131;
+ * src/tensor/mod.rs:2707-2760), computed in parallel.  cols a multiple of 4, up
+ * to 16384. */
+int cml_sum_squares_f32(const float *x_dev, int64_t n_rows, int64_t cols, float *out_dev,
+                        cml_stream_t stream);
 /* silu(gate) * up = (g / (1 + exp(-g))) * u per element (reference
  * CpuTensor::silu_mul, src/tensor/mod.rs:2610-2634), quantized (reference
  * silu_mul_quantize / _q8k, src/cuda_resident.rs:4289-4341).  act must be

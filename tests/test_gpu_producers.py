@@ -52,6 +52,62 @@ def _rows(n, cols, seed):
     return x, w
 
 
+def _ordered_sum_rows(cols, rng):
+    """Rows that stress the in-order f32 sum of squares: plain, wide dynamic range, exact rounding
+    ties, squares that underflow to subnormals, sums that overflow, sparse rows, constant rows with
+    a few outliers, descending magnitudes, a large head (every later term is a fraction of an ulp),
+    non-finite values."""
+    n = cols
+    rows = [
+        rng.standard_normal(n),
+        rng.standard_normal(n) * np.exp(rng.standard_normal(n) * 3),
+        np.round(rng.standard_normal(n) * 8) / 8,
+        np.round(rng.standard_normal(n) * 2) / 2 * 1024.0,
+        rng.standard_normal(n) * 1e-20,
+        rng.standard_normal(n) * 1e-23,
+        rng.standard_normal(n) * 1e18,
+        np.where(rng.random(n) < 0.9, 0.0, rng.standard_normal(n)),
+        np.full(n, 1.5) * (1 + (rng.random(n) < 0.01)),
+        np.full(n, 1.0),
+        np.sort(np.abs(rng.standard_normal(n)))[::-1] * 1000.0,
+        np.sort(np.abs(rng.standard_normal(n))) * 0.001,
+        np.concatenate([[4096.0], np.ones(n - 1)]),
+        np.concatenate([[1e10], rng.standard_normal(n - 1)]),
+        np.zeros(n),
+        np.concatenate([np.zeros(n - 1), [3.0]]),
+    ]
+    x = np.stack(rows).astype(np.float32)
+    extra = rng.standard_normal((3, n)).astype(np.float32)
+    extra[0, n // 3] = np.inf
+    extra[1, n // 2] = np.nan
+    extra[2, min(5, n - 1)], extra[2, max(n - 7, 0)] = np.inf, np.nan
+    return np.concatenate([x, extra])
+
+
+@pytest.mark.parametrize("cols", [4, 64, 256, 1000, 2048, 2816, 4096, 5120, 8192, 14336, 16384])
+def test_sum_of_squares_is_the_scalar_loop(cols):
+    """cml_sum_squares_f32 adds the squares in parallel and must return the bits of the
+    left-to-right scalar loop (the first pass of the reference's rms_norm)."""
+    rng = np.random.default_rng(4200 + cols)
+    for rep in range(3):
+        x = _ordered_sum_rows(cols, rng)
+        n = x.shape[0]
+        G.say(f"sum of squares cols={cols} rep={rep}")
+        xd, od = DeviceBuffer.from_numpy(x), DeviceBuffer(n * 4)
+        check(lib().cml_sum_squares_f32(xd.ptr, n, cols, od.ptr, None), "cml_sum_squares_f32")
+        check(lib().cml_stream_sync(None))
+        got = od.to_numpy(np.float32, (n,))
+        with np.errstate(over="ignore", invalid="ignore"):
+            sq = (x * x).astype(np.float32)
+            want = np.zeros(n, np.float32)
+            for c in range(cols):                      # the scalar loop, all rows at once
+                want = (want + sq[:, c]).astype(np.float32)
+        finite = np.isfinite(want)
+        assert np.array_equal(np.isnan(got), np.isnan(want))
+        assert G.same_bits(got[~np.isnan(want)], want[~np.isnan(want)]), (cols, rep, np.nonzero(got.view(np.uint32) != want.view(np.uint32))[0][:8])
+        assert finite.sum() >= 12
+
+
 @pytest.mark.parametrize("cols", [256, 2048, 2816, 4096, 14336])
 def test_rms_norm_rows_are_bit_exact(cols):
     x, w = _rows(5, cols, 900 + cols)
