@@ -45,20 +45,66 @@ namespace cml {
 
 constexpr uint32_t kRunBig = 1u << 26;  // saturation of run increments: anything >= 2^24 leaves the binade
 
-// Terms xs[0 .. 1024*c4) (non-negative f32, zero padded) in LDS, thread t owning the contiguous
+__device__ __forceinline__ float readlane_f32(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+
+// A run of terms as a function of the parity of the sum that enters it.
+struct RunPair {
+    uint32_t d0, d1;
+};
+// `left` runs first, then `right`
+__device__ __forceinline__ RunPair run_then(const RunPair &left, const RunPair &right) {
+    RunPair r;
+    r.d0 = min(left.d0 + ((left.d0 & 1u) ? right.d1 : right.d0), kRunBig);
+    r.d1 = min(left.d1 + ((left.d1 & 1u) ? right.d0 : right.d1), kRunBig);
+    return r;
+}
+
+// Segmented inclusive scan over the 64 lanes of a wave: every lane ends up with the composition
+// of the runs from its group's first lane to itself, and with that first lane's `first`.
+// `seen` enters as 1 in the lanes that start a group.  Rows of 16 lanes by DPP, then row by row
+// through lane reads.
+__device__ __forceinline__ void run_scan64(RunPair &me, int &first, int &seen, int lane) {
+    const int rl = lane & 15, row = lane >> 4;
+    auto absorb = [&](uint32_t o0, uint32_t o1, int ofirst, int oseen, bool reach) __attribute__((always_inline)) {
+        if (reach && !seen) {
+            me = run_then(RunPair{o0, o1}, me);
+            first = ofirst;
+            seen = oseen;
+        }
+    };
+    absorb(row_shr_i32<1>(me.d0), row_shr_i32<1>(me.d1), row_shr_i32<1>(first), row_shr_i32<1>(seen), rl >= 1);
+    absorb(row_shr_i32<2>(me.d0), row_shr_i32<2>(me.d1), row_shr_i32<2>(first), row_shr_i32<2>(seen), rl >= 2);
+    absorb(row_shr_i32<4>(me.d0), row_shr_i32<4>(me.d1), row_shr_i32<4>(first), row_shr_i32<4>(seen), rl >= 4);
+    absorb(row_shr_i32<8>(me.d0), row_shr_i32<8>(me.d1), row_shr_i32<8>(first), row_shr_i32<8>(seen), rl >= 8);
+#pragma unroll
+    for (int r = 1; r < 4; r++) {  // the (by now complete) last lane of row r-1 into row r
+        const int src = 16 * r - 1;
+        absorb(__builtin_amdgcn_readlane(me.d0, src), __builtin_amdgcn_readlane(me.d1, src), __builtin_amdgcn_readlane(first, src),
+               __builtin_amdgcn_readlane(seen, src), row == r);
+    }
+}
+
+constexpr int kSumThreads = 1024, kSumWaves = kSumThreads / 64;
+
+// Terms xs[0 .. 4*1024*c4) (non-negative f32, zero padded) in LDS, thread t owning the contiguous
 // chunk of c4 float4 starting at t*c4.  Returns, in every lane of wave 0, the f32 sum
-// (((0 + xs[0]) + xs[1]) + ...) exactly as a scalar loop produces it.  256 threads; n = number of
-// real terms (sets the width of the binade guard).
+// (((0 + xs[0]) + xs[1]) + ...) exactly as a scalar loop produces it.  1024 threads (short
+// chunks: the terms of a chunk that straddles a power of two are added one by one); n = number
+// of real terms (sets the width of the binade guard).
 __device__ __forceinline__ float ordered_sum_nonneg(const float4 *xs4, int c4, int n, int tid) {
-    __shared__ float s_wave_total[4];
-    __shared__ int s_E[256];         // binade of the group ending at thread t (0: add in order)
-    __shared__ uint32_t s_D0[256], s_D1[256];
-    __shared__ int s_head[256];      // first thread of the group ending at thread t
-    __shared__ unsigned long long s_tail[4];
-    const int lane = tid & 63, wave = tid >> 6;
+    __shared__ float s_wave_total[kSumWaves];
+    __shared__ int s_E[kSumThreads];         // binade of the group ending at thread t (0: add in order)
+    __shared__ uint32_t s_D0[kSumThreads], s_D1[kSumThreads];
+    __shared__ int s_head[kSumThreads];      // first thread of the group ending at thread t
+    __shared__ int s_count[kSumWaves];       // groups per wave
+    __shared__ uint16_t s_list[kSumWaves][64];  // the last threads of a wave's groups, in order
+    const int lane = tid & 63, wave = tid >> 6, rl = lane & 15, row = lane >> 4;
     const float4 *mine = xs4 + tid * c4;
 
-    // 1. chunk sums and their exclusive scan (the association of this approximation is free)
+    // 1. chunk sums and their exclusive scan (the association of this approximation is free):
+    //    rows of 16 lanes by DPP, the three row totals by lane reads
     float local = 0.0f;
     for (int j = 0; j < c4; j++) {
         const float4 v = mine[j];
@@ -68,15 +114,22 @@ __device__ __forceinline__ float ordered_sum_nonneg(const float4 *xs4, int c4, i
         local = local + v.w;
     }
     float incl = local;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        const float o = __shfl_up(incl, d);
-        if (lane >= d) incl = incl + o;
-    }
+    incl = incl + row_shr_f32<1>(incl);  // lanes at the start of a row receive 0
+    incl = incl + row_shr_f32<2>(incl);
+    incl = incl + row_shr_f32<4>(incl);
+    incl = incl + row_shr_f32<8>(incl);
+    const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, incl), 15));
+    const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, incl), 31));
+    const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, incl), 47));
+    incl = incl + (row == 0 ? 0.0f : (row == 1 ? r0 : (row == 2 ? r0 + r1 : (r0 + r1) + r2)));
     if (lane == 63) s_wave_total[wave] = incl;
     __syncthreads();
     float before = 0.0f;
-    for (int w = 0; w < wave; w++) before = before + s_wave_total[w];
+#pragma unroll
+    for (int w = 0; w < kSumWaves - 1; w++) {  // all reads at once, then the additions
+        const float tw = s_wave_total[w];
+        before = before + (w < wave ? tw : 0.0f);
+    }
     const float base = before + (incl - local), after = before + incl;
 
     // 2. same binade on both sides, with room for the difference between summation orders?
@@ -84,97 +137,133 @@ __device__ __forceinline__ float ordered_sum_nonneg(const float4 *xs4, int c4, i
     const uint32_t e_lo = __float_as_uint(base * (1.0f - delta)) >> 23, e_hi = __float_as_uint(after * (1.0f + delta)) >> 23;
     const bool run = e_lo == e_hi && e_lo >= 1 && e_lo < 255;
     const int E = run ? static_cast<int>(e_lo) : 0;
-    uint32_t D0 = 0, D1 = 0;
+    RunPair me{0u, 0u};
     if (run) {
         for (int j = 0; j < c4; j++) {
             const float4 v = mine[j];
             const float t4[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
             for (int k = 0; k < 4; k++) {
+                // branch-free: a right shift by 1..31 covers every term below the sum's binade
+                // (25 and more leave nothing: no increment, no tie), a left shift the others
                 const uint32_t bits = __float_as_uint(t4[k]);
                 const int Ea = static_cast<int>(bits >> 23);
                 const uint32_t ma = (bits & 0x7fffffu) | (Ea ? 0x800000u : 0u);
                 const int sh = E - max(Ea, 1);
-                uint32_t inc, tie = 0, floor_part;
-                if (sh <= 0) {
-                    floor_part = inc = -sh > 7 ? (ma ? kRunBig : 0u) : min(ma << (-sh), kRunBig);
-                } else if (sh >= 25) {
-                    floor_part = inc = 0;
-                } else {
-                    floor_part = ma >> sh;
-                    const uint32_t rem = ma & ((1u << sh) - 1u), half = 1u << (sh - 1);
-                    inc = floor_part + (rem > half ? 1u : 0u);
-                    tie = rem == half ? 1u : 0u;
-                }
+                const int rs = min(max(sh, 1), 31);
+                const uint32_t floor_r = ma >> rs, rem = ma & ((1u << rs) - 1u), half = 1u << (rs - 1);
+                const uint32_t inc_r = floor_r + (rem > half ? 1u : 0u), tie_r = rem == half ? 1u : 0u;
+                const int ls = min(-sh, 8);
+                const uint32_t inc_l = ls == 8 ? (ma ? kRunBig : 0u) : min(ma << (ls & 7), kRunBig);
+                const bool right = sh >= 1;
+                const uint32_t inc = right ? inc_r : inc_l, floor_part = right ? floor_r : inc_l, tie = right ? tie_r : 0u;
                 // a tie goes to the even neighbour: up exactly when S + floor is odd
-                D0 = min(D0 + inc + (tie & (D0 ^ floor_part) & 1u), kRunBig);
-                D1 = min(D1 + inc + (tie & (D1 ^ floor_part ^ 1u) & 1u), kRunBig);
+                me.d0 = min(me.d0 + inc + (tie & (me.d0 ^ floor_part) & 1u), kRunBig);
+                me.d1 = min(me.d1 + inc + (tie & (me.d1 ^ floor_part ^ 1u) & 1u), kRunBig);
             }
         }
     }
 
-    // 3. compose neighbouring runs of one binade (segmented inclusive scan inside each wave; a
-    //    wave boundary ends a group, the walk below simply meets one more group there)
+    // 3. compose neighbouring runs of one binade: a segmented inclusive scan, rows of 16 lanes by
+    //    DPP, then row by row through lane reads (a wave boundary ends a group; the walk below
+    //    simply meets one more group there)
     const int E_prev = __shfl_up(E, 1);
-    bool head = lane == 0 || E == 0 || E_prev != E;  // in-order chunks stand alone
+    const bool head = lane == 0 || E_prev != E;  // neighbouring in-order chunks (E = 0) form one range
     int first = tid;
-    bool seen = head;  // a group head lies inside the span composed so far
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        const uint32_t o0 = __shfl_up(D0, d), o1 = __shfl_up(D1, d);
-        const int ofirst = __shfl_up(first, d);
-        const bool oseen = __shfl_up(static_cast<int>(seen), d) != 0;
-        if (lane >= d && !seen) {
-            // the span to the left (o0, o1) runs first, then this one
-            const uint32_t n0 = min(o0 + ((o0 & 1u) ? D1 : D0), kRunBig);
-            const uint32_t n1 = min(o1 + ((o1 & 1u) ? D0 : D1), kRunBig);
-            D0 = n0;
-            D1 = n1;
-            first = ofirst;
-            seen = oseen;
-        }
-    }
+    int seen = head ? 1 : 0;  // a group head lies inside the span composed so far
+    run_scan64(me, first, seen, lane);
+    // the zero padding behind the last real chunk is not walked at all
+    const int n_chunks = (n + 4 * c4 - 1) / (4 * c4);
     const int next_head = __shfl_down(static_cast<int>(head), 1);
-    const bool tail = lane == 63 || next_head != 0;
+    const bool tail = tid < n_chunks && (lane == 63 || next_head != 0 || tid == n_chunks - 1);
     s_E[tid] = E;
-    s_D0[tid] = D0;
-    s_D1[tid] = D1;
+    s_D0[tid] = me.d0;
+    s_D1[tid] = me.d1;
     s_head[tid] = first;
     const unsigned long long tails = __ballot(tail);
-    if (lane == 0) s_tail[wave] = tails;
+    if (lane == 0) s_count[wave] = __builtin_popcountll(tails);
+    if (tail) s_list[wave][__builtin_popcountll(tails & ((1ull << lane) - 1ull))] = static_cast<uint16_t>(tid);
     __syncthreads();
     if (wave != 0) return 0.0f;
 
-    // 4. the walk, every lane of wave 0 alike (all reads are broadcasts)
+    // 4. the walk, every lane of wave 0 alike.  Lane g first fetches the g-th group of a batch of
+    //    up to 64 (its last thread from the tail masks, then the group's record), so that the
+    //    chain through the running sum reads lanes, not memory.
     float s = 0.0f;
-    auto add_in_order = [&](int t0, int t1) __attribute__((always_inline)) {  // chunks t0..t1
-        const float4 *p = xs4 + t0 * c4;
-        const int cnt = (t1 - t0 + 1) * c4;
+    auto add_in_order = [&](const float4 *p, int cnt) __attribute__((always_inline)) {  // cnt float4, the next one read ahead
+        float4 v = p[0];
         for (int j = 0; j < cnt; j++) {
-            const float4 v = p[j];
+            const float4 nx = p[min(j + 1, cnt - 1)];
             s = s + v.x;
             s = s + v.y;
             s = s + v.z;
             s = s + v.w;
+            v = nx;
         }
     };
-    for (int w = 0; w < 4; w++) {
-        unsigned long long m = s_tail[w];
-        while (m) {
-            const int t = w * 64 + __builtin_ctzll(m);
-            m &= m - 1;
-            const int Eg = s_E[t];
+    int cnt_w[kSumWaves];
+#pragma unroll
+    for (int w = 0; w < kSumWaves; w++) cnt_w[w] = s_count[w];
+    int n_groups = 0;
+#pragma unroll
+    for (int w = 0; w < kSumWaves; w++) n_groups += cnt_w[w];
+    for (int g0 = 0; g0 < n_groups; g0 += 64) {
+        // the (g0 + lane)-th group: which wave's list, which entry
+        int k = g0 + lane, w_mine = 0;
+        bool found = false;
+#pragma unroll
+        for (int w = 0; w < kSumWaves; w++) {
+            if (!found) {
+                if (k < cnt_w[w]) {
+                    found = true;
+                    w_mine = w;
+                } else {
+                    k -= cnt_w[w];
+                }
+            }
+        }
+        const int t_mine = found ? s_list[w_mine][k] : kSumThreads - 1;
+        // Groups that a wave boundary cut apart are put together again here, in parallel: the same
+        // scan over the batch's records (lanes past the last group form groups of their own).
+        const int gE = g0 + lane < n_groups ? s_E[t_mine] : -1 - lane;
+        const int gE_prev = __shfl_up(gE, 1);
+        RunPair gD{s_D0[t_mine], s_D1[t_mine]};
+        int gH = s_head[t_mine];
+        int gSeen = (lane == 0 || gE_prev != gE) ? 1 : 0;
+        const int gE_next = __shfl_down(gE, 1);
+        const bool gTail = g0 + lane < n_groups && (lane == 63 || gE_next != gE);
+        run_scan64(gD, gH, gSeen, lane);
+        // an in-order range usually is one or two float4 long: fetch those with the record
+        const int gCnt = (t_mine - gH + 1) * c4;
+        const float4 gV0 = xs4[gH * c4], gV1 = xs4[gH * c4 + (gCnt > 1 ? 1 : 0)];
+        unsigned long long todo = __ballot(gTail);
+        while (todo) {
+            const int g = __builtin_ctzll(todo);
+            todo &= todo - 1;
+            const int Eg = __builtin_amdgcn_readlane(gE, g);
             if (Eg == 0) {
-                add_in_order(t, t);
+                const int cnt = __builtin_amdgcn_readlane(gCnt, g);
+                s = s + readlane_f32(gV0.x, g);
+                s = s + readlane_f32(gV0.y, g);
+                s = s + readlane_f32(gV0.z, g);
+                s = s + readlane_f32(gV0.w, g);
+                if (cnt > 1) {
+                    s = s + readlane_f32(gV1.x, g);
+                    s = s + readlane_f32(gV1.y, g);
+                    s = s + readlane_f32(gV1.z, g);
+                    s = s + readlane_f32(gV1.w, g);
+                    if (cnt > 2) add_in_order(xs4 + __builtin_amdgcn_readlane(gH, g) * c4 + 2, cnt - 2);
+                }
                 continue;
             }
+            const uint32_t D0 = __builtin_amdgcn_readlane(gD.d0, g), D1 = __builtin_amdgcn_readlane(gD.d1, g);
             const uint32_t sb = __float_as_uint(s);
             const uint32_t S = (sb & 0x7fffffu) | 0x800000u;
-            const uint32_t D = (S & 1u) ? s_D1[t] : s_D0[t];
+            const uint32_t D = (S & 1u) ? D1 : D0;
             if (static_cast<int>(sb >> 23) == Eg && S + D < (1u << 24)) {
                 s = __uint_as_float((static_cast<uint32_t>(Eg) << 23) | ((S + D) & 0x7fffffu));
-            } else {
-                add_in_order(s_head[t], t);  // the guard was too narrow for this data: still exact
+            } else {  // the guard was too narrow for this data: still exact
+                add_in_order(xs4 + __builtin_amdgcn_readlane(gH, g) * c4, __builtin_amdgcn_readlane(gCnt, g));
             }
         }
     }
@@ -186,10 +275,10 @@ __device__ __forceinline__ float ordered_sum_nonneg(const float4 *xs4, int c4, i
 // Every thread keeps its share of the row in registers (up to kRmsRegs float4) and puts the
 // squares into LDS, where ordered_sum_nonneg adds them up; the LDS row is reused for the
 // normalised values the quantizers read.
-constexpr int kRmsRegs = 16;  // float4 per thread: rows of up to 16 * 256 * 4 = 16384 values
+constexpr int kRmsRegs = 4;  // float4 per thread: rows of up to 4 * 1024 * 4 = 16384 values
 
 template <int ACT>
-__global__ __launch_bounds__(256) void rms_norm_quantize_kernel(const float *__restrict__ x, const float *__restrict__ weight,
+__global__ __launch_bounds__(kSumThreads) void rms_norm_quantize_kernel(const float *__restrict__ x, const float *__restrict__ weight,
                                                                 float eps, int cols, float *__restrict__ normed,
                                                                 int8_t *__restrict__ q, float *__restrict__ scales) {
     extern __shared__ float4 xs4[];  // the row, padded to whole batches: squares first, then the normalised values
@@ -201,17 +290,17 @@ __global__ __launch_bounds__(256) void rms_norm_quantize_kernel(const float *__r
     float4 xv[kRmsRegs];
 #pragma unroll
     for (int k = 0; k < kRmsRegs; k++) {
-        const int i = tid + k * 256;
+        const int i = tid + k * kSumThreads;
         if (i < n4) {
             const float4 v = x4[i];
             xv[k] = v;
             xs4[i] = make_float4(v.x * v.x, v.y * v.y, v.z * v.z, v.w * v.w);
         }
     }
-    // zeros from the end of the row up to 256 whole chunks: sum + 0 == sum exactly (the sum of
+    // zeros from the end of the row up to 1024 whole chunks: sum + 0 == sum exactly (the sum of
     // squares is never negative) and a zero term has increment 0
-    const int c4 = (n4 + 255) >> 8;  // float4 per thread chunk
-    for (int i = n4 + tid; i < 256 * c4; i += 256) xs4[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    const int c4 = (n4 + kSumThreads - 1) / kSumThreads;  // float4 per thread chunk
+    for (int i = n4 + tid; i < kSumThreads * c4; i += kSumThreads) xs4[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     __syncthreads();
     const float sum = ordered_sum_nonneg(xs4, c4, cols, tid);  // valid in wave 0
     if constexpr (ACT == 3) {
@@ -228,7 +317,7 @@ __global__ __launch_bounds__(256) void rms_norm_quantize_kernel(const float *__r
     float4 *n4out = normed ? reinterpret_cast<float4 *>(normed + token * cols) : nullptr;
 #pragma unroll
     for (int k = 0; k < kRmsRegs; k++) {
-        const int i = tid + k * 256;
+        const int i = tid + k * kSumThreads;
         if (i < n4) {
             const float4 v = xv[k], w = w4[i];
             float4 y;
@@ -246,7 +335,7 @@ __global__ __launch_bounds__(256) void rms_norm_quantize_kernel(const float *__r
     if constexpr (ACT == 1) {
         // eight lanes per 32-value block; cols/4 is a multiple of 8, so groups enter and leave together
         float *sc = scales + token * (cols / 32);
-        for (int i = tid; i < n4; i += 256) {
+        for (int i = tid; i < n4; i += kSumThreads) {
             float s;
             const uint32_t packed = q8_0_quantize_lane8(xs4[i], s);
             q32[i] = packed;
@@ -255,7 +344,7 @@ __global__ __launch_bounds__(256) void rms_norm_quantize_kernel(const float *__r
     } else {
         // one wave per 256-value super-block
         float *d = scales + token * (cols / 256);
-        for (int sb = wave; sb < cols / 256; sb += 4) {
+        for (int sb = wave; sb < cols / 256; sb += kSumWaves) {
             float dv;
             int bsum;
             const uint32_t packed = q8k_quantize_wave(xs4[sb * 64 + lane], dv, bsum);
@@ -268,10 +357,10 @@ __global__ __launch_bounds__(256) void rms_norm_quantize_kernel(const float *__r
 int launch_rms_norm_quantize(int act, const float *x, const float *weight, float eps, int64_t n_tokens, int64_t cols,
                              float *normed, int8_t *q, float *scales, hipStream_t st) {
     if (n_tokens == 0 || cols == 0) return CML_OK;
-    if (cols > static_cast<int64_t>(kRmsRegs) * 1024)
-        return fail(CML_ERR_UNSUPPORTED, "rms_norm row of %lld values exceeds the staging limit of %d", (long long)cols, kRmsRegs * 1024);
-    // the row in 256 whole chunks (zero padded); rows past 64 KB need the larger dynamic LDS window
-    const size_t lds = static_cast<size_t>((cols / 4 + 255) / 256) * 256 * sizeof(float4);
+    if (cols > static_cast<int64_t>(kRmsRegs) * kSumThreads * 4)
+        return fail(CML_ERR_UNSUPPORTED, "rms_norm row of %lld values exceeds the staging limit of %d", (long long)cols, kRmsRegs * kSumThreads * 4);
+    // the row in 1024 whole chunks (zero padded)
+    const size_t lds = static_cast<size_t>((cols / 4 + kSumThreads - 1) / kSumThreads) * kSumThreads * sizeof(float4);
     static bool raised = false;
     if (!raised) {
         CML_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&rms_norm_quantize_kernel<0>), hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
@@ -280,7 +369,7 @@ int launch_rms_norm_quantize(int act, const float *x, const float *weight, float
         CML_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&rms_norm_quantize_kernel<3>), hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
         raised = true;
     }
-    const dim3 grid(static_cast<unsigned>(n_tokens)), block(256);
+    const dim3 grid(static_cast<unsigned>(n_tokens)), block(kSumThreads);
     const int c = static_cast<int>(cols);
     switch (act) {
         case 0: hipLaunchKernelGGL(rms_norm_quantize_kernel<0>, grid, block, lds, st, x, weight, eps, c, normed, q, scales); break;

@@ -75,6 +75,10 @@ def _ordered_sum_rows(cols, rng):
         np.concatenate([[1e10], rng.standard_normal(n - 1)]),
         np.zeros(n),
         np.concatenate([np.zeros(n - 1), [3.0]]),
+        # sums that sit on or next to a power of two over a long stretch of small or zero terms
+        np.concatenate([np.ones(n // 2), np.zeros(n - n // 2)]),
+        np.concatenate([np.ones(n // 2) * 1.0001, np.full(n - n // 2, 1e-4)]),
+        np.concatenate([np.ones(n // 2) * 0.9999, np.full(n - n // 2, 3e-3)]),
     ]
     x = np.stack(rows).astype(np.float32)
     extra = rng.standard_normal((3, n)).astype(np.float32)
