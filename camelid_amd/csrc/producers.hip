@@ -256,12 +256,15 @@ __device__ __forceinline__ float ordered_sum_nonneg(const float4 *xs4, int c4, i
                 }
                 continue;
             }
+            // The run enters with S even or odd; adding its increment to the BITS of s is adding it
+            // to S as long as no carry reaches the exponent field -- which is also the test that
+            // the sum stays in the binade.  D1 - D0 is a handful of ties: a 24-bit multiply.
             const uint32_t D0 = __builtin_amdgcn_readlane(gD.d0, g), D1 = __builtin_amdgcn_readlane(gD.d1, g);
             const uint32_t sb = __float_as_uint(s);
-            const uint32_t S = (sb & 0x7fffffu) | 0x800000u;
-            const uint32_t D = (S & 1u) ? D1 : D0;
-            if (static_cast<int>(sb >> 23) == Eg && S + D < (1u << 24)) {
-                s = __uint_as_float((static_cast<uint32_t>(Eg) << 23) | ((S + D) & 0x7fffffu));
+            const uint32_t after = sb + D0 + static_cast<uint32_t>(__mul24(static_cast<int>(sb & 1u), static_cast<int>(D1 - D0)));
+            const uint32_t e_bits = static_cast<uint32_t>(Eg) << 23;
+            if (((sb ^ e_bits) | (after ^ e_bits)) < (1u << 23) && D0 < (1u << 24)) {
+                s = __uint_as_float(after);
             } else {  // the guard was too narrow for this data: still exact
                 add_in_order(xs4 + __builtin_amdgcn_readlane(gH, g) * c4, __builtin_amdgcn_readlane(gCnt, g));
             }
