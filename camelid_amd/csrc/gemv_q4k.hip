@@ -79,6 +79,7 @@ struct Q4KArgs {
     const uint8_t *w2;
     float *out2;
     int ksplit;        // waves sharing one row tile (1, 2, 4 or 8)
+    int ksplit_log2;
     int tiles_per_wg;  // row tiles per workgroup; blockDim.x = 64 * ksplit * tiles_per_wg
 };
 
@@ -230,7 +231,13 @@ __device__ __forceinline__ void q4k_compute(const Q4KRegs<U> &r, const Q4KLane &
 // SPR = 2: a wave owns 8 rows and two 4-lane groups per row work on neighbouring super-blocks
 // (lane = 8*row + 4*h + c).  Twice the waves with half the steps each, for weights whose 16-row
 // tiles alone leave one wave per SIMD; every sum keeps its order, so the results are the same bits.
-template <int NT, bool INTS, bool FUSEQ = false, int SPR = 1, bool WHOLE = false>
+//
+// PLAIN: a plain call (no groups, no second weight).  The general entry reads its arguments in
+// several dependent rounds (group tables, then what they point to): with the split factors'
+// integer divisions that was about 600 instructions and four scalar-load round trips before the
+// first weight request -- 0.8 us of a kernel that lives for eight (14336 x 4096: 8.05 -> 7.25 us).
+// The plain entry has none of it, and the K split (a power of two) is shifts.
+template <int NT, bool INTS, bool FUSEQ = false, int SPR = 1, bool WHOLE = false, bool PLAIN = false>
 __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
     static_assert(!FUSEQ || (NT == 1 && !INTS), "the fused quantizer serves single-token calls");
     static_assert(SPR == 1 || SPR == 2, "groups per row");
@@ -247,22 +254,22 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
 
     const int tid = threadIdx.x;
     const int nthreads = blockDim.x;
-    const bool direct = a.group_offsets == nullptr && a.group_ids != nullptr;
-    const bool grouped = a.group_offsets != nullptr;
+    const bool direct = !PLAIN && a.group_offsets == nullptr && a.group_ids != nullptr;
+    const bool grouped = !PLAIN && a.group_offsets != nullptr;
     const int64_t band = (grouped || direct) ? (a.group_ids ? a.group_ids[blockIdx.y] : static_cast<int>(blockIdx.y)) : 0;
     if (band < 0 || (direct && band >= a.n_groups)) return;  // a y-slot past the groups in use, or an id out of range
     const int a0 = grouped ? a.group_offsets[band] : (direct ? static_cast<int>(blockIdx.y) : 0);  // first assignment of this group
     const int n_assign = grouped ? a.group_offsets[band + 1] - a0 : (direct ? 1 : NT);
     if (n_assign <= 0) return;  // an expert nobody routed to: the whole workgroup leaves
-    const bool second = gridDim.z > 1 && blockIdx.z == 1;
+    const bool second = !PLAIN && gridDim.z > 1 && blockIdx.z == 1;
     const uint8_t *w = (second ? a.w2 : a.w) + band * (a.rows / 16) * kQ4KChunk;
 
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
-    const int W = a.ksplit;
-    const int tile_in_wg = wave / W, kpart = wave - tile_in_wg * W;
+    const int W = a.ksplit;  // 1, 2, 4 or 8
+    const int tile_in_wg = wave >> a.ksplit_log2, kpart = wave & (W - 1);
     const int tile = blockIdx.x * a.tiles_per_wg + tile_in_wg;
-    const int s0 = static_cast<int>(static_cast<int64_t>(kpart) * n_sb / W);
-    const int s1 = static_cast<int>(static_cast<int64_t>(kpart + 1) * n_sb / W);
+    const int s0 = (kpart * n_sb) >> a.ksplit_log2;  // == kpart * n_sb / W
+    const int s1 = ((kpart + 1) * n_sb) >> a.ksplit_log2;
     const int g = lane / LPS, l = lane - g * LPS;
     const int r = g / SPR, h = g - r * SPR;
     const int row = tile * RPW + r - a.row_skip;  // output row; negative for the skipped head of a view's first tile
@@ -294,6 +301,7 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
         // Activation row of local token t (clamped to the group's last assignment; extra tokens store nothing).
         auto act_row = [&](int t) -> int64_t {
             const int j = a0 + min(p0 + t, n_assign - 1);
+            if (PLAIN) return j;
             if (a.shared_act) return 0;
             return a.group_rows ? a.group_rows[j] : j;
         };
@@ -519,20 +527,27 @@ static int launch_q4k_nt(Q4KArgs ka, const Q4KShape &shape, int n_groups, bool i
                        static_cast<size_t>(waves) * NT * 16 * 4;
     if (lds > 64 * 1024) return fail(CML_ERR_UNSUPPORTED, "Q4_K activation of %d super-blocks x %d tokens exceeds the LDS staging limit", ka.n_sb, NT);
     ka.ksplit = shape.ksplit;
+    ka.ksplit_log2 = shape.ksplit >= 8 ? 3 : (shape.ksplit >= 4 ? 2 : (shape.ksplit >= 2 ? 1 : 0));
     ka.tiles_per_wg = shape.tiles_per_wg;
+    const bool plain = !ka.group_offsets && !ka.group_ids && !env_int("CAMELID_HIP_Q4K_GENERAL_ENTRY", 0);
+    const dim3 grid(gx, n_groups), block(64 * waves);
     if (ints && NT == 1)
-        hipLaunchKernelGGL((gemv_q4k_kernel<1, true>), dim3(gx, n_groups), dim3(64 * waves), lds, st, ka);
-    else if (NT <= 2 && q4k_whole_buffers(ka, shape.ksplit)) {
+        hipLaunchKernelGGL((gemv_q4k_kernel<1, true>), grid, block, lds, st, ka);
+    else if (NT <= 2) {
+        // one or two tokens: 8-row waves, unclamped loads and the short entry where they apply
         constexpr int NTS = NT <= 2 ? NT : 1;
-        if (half_tiles)
-            hipLaunchKernelGGL((gemv_q4k_kernel<NTS, false, false, 2, true>), dim3(gx, n_groups), dim3(64 * waves), lds, st, ka);
-        else
-            hipLaunchKernelGGL((gemv_q4k_kernel<NTS, false, false, 1, true>), dim3(gx, n_groups), dim3(64 * waves), lds, st, ka);
-    } else if (half_tiles) {
-        constexpr int NTS = NT <= 2 ? NT : 1;
-        hipLaunchKernelGGL((gemv_q4k_kernel<NTS, false, false, 2>), dim3(gx, n_groups), dim3(64 * waves), lds, st, ka);
+        const bool whole = q4k_whole_buffers(ka, shape.ksplit);
+#define CML_Q4K_LAUNCH(SPR_, WHOLE_, PLAIN_) hipLaunchKernelGGL((gemv_q4k_kernel<NTS, false, false, SPR_, WHOLE_, PLAIN_>), grid, block, lds, st, ka)
+        if (half_tiles) {
+            if (whole) { if (plain) CML_Q4K_LAUNCH(2, true, true); else CML_Q4K_LAUNCH(2, true, false); }
+            else { if (plain) CML_Q4K_LAUNCH(2, false, true); else CML_Q4K_LAUNCH(2, false, false); }
+        } else {
+            if (whole) { if (plain) CML_Q4K_LAUNCH(1, true, true); else CML_Q4K_LAUNCH(1, true, false); }
+            else { if (plain) CML_Q4K_LAUNCH(1, false, true); else CML_Q4K_LAUNCH(1, false, false); }
+        }
+#undef CML_Q4K_LAUNCH
     } else
-        hipLaunchKernelGGL((gemv_q4k_kernel<NT, false>), dim3(gx, n_groups), dim3(64 * waves), lds, st, ka);
+        hipLaunchKernelGGL((gemv_q4k_kernel<NT, false>), grid, block, lds, st, ka);
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }
@@ -604,17 +619,23 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
                        static_cast<size_t>(waves) * 16 * 4;
     if (lds > 64 * 1024) return fail(CML_ERR_UNSUPPORTED, "Q4_K activation of %d super-blocks exceeds the LDS staging limit", ka.n_sb);
     ka.ksplit = shape.ksplit;
+    ka.ksplit_log2 = shape.ksplit >= 8 ? 3 : (shape.ksplit >= 4 ? 2 : (shape.ksplit >= 2 ? 1 : 0));
     ka.tiles_per_wg = shape.tiles_per_wg;
     const dim3 grid(gx, grouped ? (a.group_ids ? a.max_active : a.n_groups) : 1, w2 ? 2 : 1);
-    if (q4k_whole_buffers(ka, shape.ksplit)) {
-        if (half_tiles)
-            hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, 2, true>), grid, dim3(64 * waves), lds, st, ka);
-        else
-            hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, 1, true>), grid, dim3(64 * waves), lds, st, ka);
-    } else if (half_tiles)
-        hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, 2>), grid, dim3(64 * waves), lds, st, ka);
-    else
-        hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true>), grid, dim3(64 * waves), lds, st, ka);
+    {
+        const bool whole = q4k_whole_buffers(ka, shape.ksplit);
+        const bool plain = !grouped && !w2 && !env_int("CAMELID_HIP_Q4K_GENERAL_ENTRY", 0);
+        const dim3 block(64 * waves);
+#define CML_Q4K_LAUNCH(SPR_, WHOLE_, PLAIN_) hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, SPR_, WHOLE_, PLAIN_>), grid, block, lds, st, ka)
+        if (half_tiles) {
+            if (whole) { if (plain) CML_Q4K_LAUNCH(2, true, true); else CML_Q4K_LAUNCH(2, true, false); }
+            else { if (plain) CML_Q4K_LAUNCH(2, false, true); else CML_Q4K_LAUNCH(2, false, false); }
+        } else {
+            if (whole) { if (plain) CML_Q4K_LAUNCH(1, true, true); else CML_Q4K_LAUNCH(1, true, false); }
+            else { if (plain) CML_Q4K_LAUNCH(1, false, true); else CML_Q4K_LAUNCH(1, false, false); }
+        }
+#undef CML_Q4K_LAUNCH
+    }
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }

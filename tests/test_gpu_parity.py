@@ -214,6 +214,9 @@ def test_q4k_gemv_every_configuration_agrees():
                 with G.env(CAMELID_HIP_Q4K_CLAMPED_LOADS=1):
                     assert G.same_bits(G.gpu_gemm(w, s, q), got)
                     assert G.same_bits(G.gpu_gemm(w, s2, q2), two)
+                with G.env(CAMELID_HIP_Q4K_GENERAL_ENTRY=1):   # the kernel entry that also serves expert groups
+                    assert G.same_bits(G.gpu_gemm(w, s, q), got)
+                    assert G.same_bits(G.gpu_gemm(w, s2, q2), two)
             assert G.same_bits(two[0], got) and not G.same_bits(two[1], got)
         assert G.same_bits(per_rpw[0], per_rpw[1])
 
@@ -320,6 +323,8 @@ def test_q4k_fused_quantize_matvec_is_the_two_step_path(rows, cols):
                     with G.env(CAMELID_HIP_Q4K_FUSED_TILES_PER_WG=tpw, CAMELID_HIP_Q4K_KSPLIT=ks, CAMELID_HIP_Q4K_ROWS_PER_WAVE=rpw):
                         with G.env(CAMELID_HIP_FUSED_QUANT=2):   # also where the shape policy would not fuse
                             fused = G.gpu_matmul_f32(w, x)
+                            with G.env(CAMELID_HIP_Q4K_GENERAL_ENTRY=1):
+                                assert G.same_bits(G.gpu_matmul_f32(w, x), fused)
                         with G.env(CAMELID_HIP_FUSED_QUANT=0, CAMELID_HIP_Q4K_ROWS_PER_WAVE=16):
                             two_step = G.gpu_matmul_f32(w, x)
                     assert G.same_bits(fused, two_step)
