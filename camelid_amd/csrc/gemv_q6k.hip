@@ -45,7 +45,8 @@ struct Q6KArgs {
     const int32_t *group_rows;
     const int32_t *group_ids;
     int n_groups;
-    int ksplit;
+    int ksplit;       // 1, 2 or 4 waves per row tile
+    int ksplit_log2;
 };
 
 template <int U_>
@@ -156,12 +157,13 @@ __global__ __launch_bounds__(256) void gemv_q6k_kernel(Q6KArgs a) {
     }
 
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    // the K split is a power of two: shifts, not divisions, on the way to the first load
     const int W = a.ksplit;
-    const int tiles_per_wg = 4 / W;
-    const int tile_in_wg = wave / W, kpart = wave - tile_in_wg * W;
+    const int tiles_per_wg = 4 >> a.ksplit_log2;
+    const int tile_in_wg = wave >> a.ksplit_log2, kpart = wave & (W - 1);
     const int tile = blockIdx.x * tiles_per_wg + tile_in_wg;
-    const int s0 = static_cast<int>(static_cast<int64_t>(kpart) * n_sb / W);
-    const int s1 = static_cast<int>(static_cast<int64_t>(kpart + 1) * n_sb / W);
+    const int s0 = (kpart * n_sb) >> a.ksplit_log2;  // == kpart * n_sb / W
+    const int s1 = ((kpart + 1) * n_sb) >> a.ksplit_log2;
     const int r = lane / LPS, l = lane - r * LPS;
     const int row = tile * RPW + r;
     const bool live = row < a.rows;
@@ -183,16 +185,42 @@ __global__ __launch_bounds__(256) void gemv_q6k_kernel(Q6KArgs a) {
             return a.group_rows ? a.group_rows[j] : j;
         };
         if (p0 > 0) __syncthreads();  // the previous pass's readers are done
+        Q6KRegs<U> ra, rb;
+        bool ra_loaded = false;
         if constexpr (!GROUPED) {
             const uint4 *src = reinterpret_cast<const uint4 *>(a.q);
             uint4 *dst = reinterpret_cast<uint4 *>(ys);
             const int n16 = NT * n_sb * 16;
-            for (int i = tid; i < n16; i += 256) {
-                const uint4 v = src[i];
-                dst[i] = v;
-                bsum16[i] = bytesum16(v);
+            if (NT == 1 && n16 <= 4 * 256) {  // uniform
+                // The activation loads go out first, the first weight buffer right behind them, and
+                // only then is the activation written to LDS: the weight requests are in flight
+                // while it is staged (a wave's loads return in order).
+                uint4 sv[4];
+#pragma unroll
+                for (int k = 0; k < 4; k++) sv[k] = src[min(tid + k * 256, n16 - 1)];
+                const float yd0 = a.yd[min(tid, n_sb - 1)];
+                __builtin_amdgcn_sched_barrier(0);
+                q6k_load(ra, ql, qh, sc, dp, l, s0, s1);
+                ra_loaded = true;
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    const int i = tid + k * 256;
+                    if (i < n16) {
+                        dst[i] = sv[k];
+                        bsum16[i] = bytesum16(sv[k]);
+                    }
+                }
+                if (tid < n_sb) yds[tid] = yd0;
+                for (int i = tid + 256; i < n_sb; i += 256) yds[i] = a.yd[i];
+            } else {
+                for (int i = tid; i < n16; i += 256) {
+                    const uint4 v = src[i];
+                    dst[i] = v;
+                    bsum16[i] = bytesum16(v);
+                }
+                for (int i = tid; i < NT * n_sb; i += 256) yds[i] = a.yd[i];
             }
-            for (int i = tid; i < NT * n_sb; i += 256) yds[i] = a.yd[i];
         } else {
             uint4 *dst = reinterpret_cast<uint4 *>(ys);
             const int c16 = n_sb * 16;
@@ -215,8 +243,7 @@ __global__ __launch_bounds__(256) void gemv_q6k_kernel(Q6KArgs a) {
 #pragma unroll
         for (int t = 0; t < NT; t++) acc[t] = 0.0f;
 
-        Q6KRegs<U> ra, rb;
-        q6k_load(ra, ql, qh, sc, dp, l, s0, s1);
+        if (!ra_loaded) q6k_load(ra, ql, qh, sc, dp, l, s0, s1);
         __builtin_amdgcn_sched_barrier(0);
         // Two register buffers alternate; the last one is consumed without issuing
         // further loads.
@@ -325,6 +352,7 @@ int launch_gemv_q6k(const MatArgs &a, hipStream_t st) {
     ka.group_ids = a.group_ids;
     ka.n_groups = a.n_groups;
     ka.ksplit = pick_ksplit_q6k(ka.rows, ka.n_sb);
+    ka.ksplit_log2 = ka.ksplit >= 4 ? 2 : (ka.ksplit >= 2 ? 1 : 0);
     if (grouped) {
         if (a.band_rows <= 0 || a.band_rows * a.n_groups != w->rows)
             return fail(CML_ERR_SHAPE, "%d bands of %lld rows do not cover %lld rows", a.n_groups, (long long)a.band_rows, (long long)w->rows);
