@@ -173,10 +173,27 @@ __global__ __launch_bounds__(256) void gemm_b32_mfma_kernel(B32MfmaArgs a) {
 
     // activation scales: xss[block][token]
     const int nb = n_slabs * 8;
-    for (int i = tid; i < nb * NTOK; i += nthreads) {
-        const int b = i / NTOK, t = i - b * NTOK;
-        xss[i] = a.xs[act_row(t) * nb + b];
+    // The first values per thread go to registers now and to LDS after the weight and activation
+    // loads below have been issued: storing them here would put a whole memory round trip in front
+    // of the first weight request.
+    constexpr int kScaleRegs = 4;
+    float scale_reg[kScaleRegs];
+    const int n_scales = nb * NTOK;
+#pragma unroll
+    for (int k = 0; k < kScaleRegs; k++) {
+        const int i = min(tid + k * nthreads, n_scales - 1);
+        { const int b = i / NTOK, t = i - b * NTOK; scale_reg[k] = a.xs[act_row(t) * nb + b]; }
     }
+    auto store_scales = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int k = 0; k < kScaleRegs; k++) {
+            const int i = tid + k * nthreads;
+            if (i < n_scales) xss[i] = scale_reg[k];
+        }
+        for (int i = tid + kScaleRegs * nthreads; i < n_scales; i += nthreads) {
+        { const int b = i / NTOK, t = i - b * NTOK; xss[i] = a.xs[act_row(t) * nb + b]; }
+        }
+    };
 
     // Staging: each thread owns kPer fixed (token, piece) pairs; only the slab moves.  Piece pc =
     // half h = pc & 1 of block pc >> 1.  Destination order inside a slab: [pair of blocks][octet
@@ -248,6 +265,7 @@ __global__ __launch_bounds__(256) void gemm_b32_mfma_kernel(B32MfmaArgs a) {
     stage_load(0);
 #pragma unroll
     for (int i = 0; i < RING; i++) load_slot(ring[i], i);
+    store_scales();
     stage_store(buf0, bs0);
     __syncthreads();
 
