@@ -55,6 +55,8 @@ CONFIGS = {
     "q6k_128256x3072_n1": ("Q6_K", 128256, 3072, 1),
     "q4_0_128256x3072_n1": ("Q4_0", 128256, 3072, 1),
     "q4k_14336x4096_n2": ("Q4_K", 14336, 4096, 2),
+    "q4k_14336x4096_n3": ("Q4_K", 14336, 4096, 3),
+    "q4k_4096x14336_n3": ("Q4_K", 4096, 14336, 3),
     "q4k_14336x4096_n4": ("Q4_K", 14336, 4096, 4),
     "q4k_14336x4096_n8": ("Q4_K", 14336, 4096, 8),
     "q4k_14336x4096_n16": ("Q4_K", 14336, 4096, 16),

@@ -496,14 +496,24 @@ int cml_argmax_f32(const float *logits_dev, int64_t n_rows, int64_t n, uint32_t 
 
 // ---- matvec / matmul --------------------------------------------------------------------------------
 
+// The packed-dot kernels serve 8, 4, 2 or 1 tokens per pass over the weight: 3, 5, 6 and 7 tokens
+// are two or three passes, and one pass of the matrix-core kernel beats them even below the batch
+// size from which it wins pass for pass (measured: Q4_0 128256x3072, 3 tokens 73 -> 55 us; Q4_K
+// 14336x4096, 3 tokens 17.0 -> 12.0 us).  A forced threshold (the tuning knobs) is taken as is.
+static bool mfma_pays(int64_t n, int min_tokens, const char *knob) {
+    if (n >= min_tokens) return true;
+    if (env_int(knob, 0) > 0) return false;
+    return n == 3 || (n >= 5 && n <= 7);
+}
+
 static int dispatch(const MatArgs &a, hipStream_t st) {
     int rc;
     switch (a.w->fmt) {
         case CML_Q4_K:
             // int8 matrix cores for the batched shapes (speculative-verify / prefill); packed dot below.
-            // Measured on MI355X at 14336x4096: the matrix-core kernel takes 11.5-12 us for any batch
-            // up to 16 tokens, the packed-dot kernel 8.9 / 12.1 / 18.9 us for 1 / 2 / 4 tokens.
-            if (!a.group_offsets && !a.ints && a.n_tokens >= env_int("CAMELID_HIP_Q4K_MFMA_MIN_TOKENS", 4))
+            // Measured on MI355X at 14336x4096: the matrix-core kernel takes 12 us for any batch up to
+            // 16 tokens, the packed-dot kernel 7.2 / 9.9 us for 1 / 2 tokens and two launches for 3.
+            if (!a.group_offsets && !a.ints && a.n_tokens >= env_int("CAMELID_HIP_Q4K_MFMA_MIN_TOKENS", 3))
                 rc = launch_gemm_q4k_mfma(a, st);
             else
                 rc = launch_gemv_q4k(a, st);
@@ -511,13 +521,13 @@ static int dispatch(const MatArgs &a, hipStream_t st) {
         case CML_Q8_0:
         case CML_Q4_0:
             // the same split for the 32-value-block formats (rows of whole 256-value slabs)
-            if (!a.group_offsets && !a.ints && a.n_tokens >= b32_mfma_min_tokens(a.w->rows) && b32_mfma_usable(a.w))
+            if (!a.group_offsets && !a.ints && mfma_pays(a.n_tokens, b32_mfma_min_tokens(a.w->rows), "CAMELID_HIP_B32_MFMA_MIN_TOKENS") && b32_mfma_usable(a.w))
                 rc = launch_gemm_b32_mfma(a, st);
             else
                 rc = a.w->fmt == CML_Q8_0 ? launch_gemv_q8_0(a, st) : launch_gemv_q4_0(a, st);
             break;
         case CML_Q6_K:
-            if (!a.group_offsets && !a.ints && a.n_tokens >= q6k_mfma_min_tokens(a.w->rows, a.w->nb))
+            if (!a.group_offsets && !a.ints && mfma_pays(a.n_tokens, q6k_mfma_min_tokens(a.w->rows, a.w->nb), "CAMELID_HIP_Q6K_MFMA_MIN_TOKENS"))
                 rc = launch_gemm_q6k_mfma(a, st);
             else
                 rc = launch_gemv_q6k(a, st);

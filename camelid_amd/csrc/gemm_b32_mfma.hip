@@ -420,7 +420,7 @@ bool b32_mfma_usable(const cml_weight *w) {
 int b32_mfma_min_tokens(int64_t rows) {
     const int forced = env_int("CAMELID_HIP_B32_MFMA_MIN_TOKENS", 0);
     if (forced > 0) return forced;
-    return (rows + 15) / 16 >= 2048 ? 5 : 9;
+    return (rows + 15) / 16 >= 2048 ? 4 : 9;  // 128256 x 3072 Q4_0, 4 tokens: 54.6 us against 61.8 us for the packed dot
 }
 
 // Q8_0 / Q4_0 matmul on the matrix cores: plain calls, or grouped by expert (mixture of experts).
