@@ -133,7 +133,8 @@ __device__ __forceinline__ void b32_mfma_operands(const B32SlabWeights<FMT> &r, 
 // KC = slabs per phase (LDS holds two phases of NTOK tokens), RING = weight slabs a wave keeps in
 // flight in registers.
 // A workgroup's 4 waves are 4/TB consecutive row tiles x TB token blocks of 16*GPW tokens.
-template <int FMT, int GPW, int TB, int KC, int RING>
+// PLAIN: the entry of a call without expert groups (no group tables to read before the first request).
+template <int FMT, int GPW, int TB, int KC, int RING, bool PLAIN = false>
 __global__ __launch_bounds__(256) void gemm_b32_mfma_kernel(B32MfmaArgs a) {
     constexpr int NTOK = 16 * GPW * TB;              // tokens staged per workgroup
     constexpr int RT = 4 / TB;                       // row tiles per workgroup
@@ -157,7 +158,7 @@ __global__ __launch_bounds__(256) void gemm_b32_mfma_kernel(B32MfmaArgs a) {
     const int rt = wave / TB, tb = wave - rt * TB;
     const int tile = blockIdx.x * RT + rt;
     const int row = tile * 16 + n;
-    const bool grouped = a.group_offsets != nullptr;
+    const bool grouped = !PLAIN && a.group_offsets != nullptr;
     const int64_t band = grouped ? (a.group_ids ? a.group_ids[blockIdx.z] : static_cast<int>(blockIdx.z)) : 0;
     if (band < 0) return;  // a z-slot past the groups in use
     const int a0 = grouped ? a.group_offsets[band] : 0;  // first assignment of this group
@@ -168,6 +169,7 @@ __global__ __launch_bounds__(256) void gemm_b32_mfma_kernel(B32MfmaArgs a) {
     // activation row of local token t (tokens past the end repeat the last one; their cells are not stored)
     auto act_row = [&](int t) __attribute__((always_inline)) -> int64_t {
         const int j = a0 + tok0 + min(t, n_here - 1);
+        if (PLAIN) return j;
         return a.group_rows ? a.group_rows[j] : j;
     };
 
@@ -349,8 +351,8 @@ __global__ __launch_bounds__(256) void gemm_b32_mfma_kernel(B32MfmaArgs a) {
     }
 }
 
-template <int FMT, int GPW, int TB, int KC, int RING>
-static int launch_b32_mfma_g(const B32MfmaArgs &ka, int n_groups, hipStream_t st) {
+template <int FMT, int GPW, int TB, int KC, int RING, bool PLAIN>
+static int launch_b32_mfma_gp(const B32MfmaArgs &ka, int n_groups, hipStream_t st) {
     constexpr int NTOK = 16 * GPW * TB, RT = 4 / TB;
     const int n_tiles = (ka.rows + 15) / 16;
     const unsigned gx = static_cast<unsigned>((n_tiles + RT - 1) / RT);
@@ -360,13 +362,23 @@ static int launch_b32_mfma_g(const B32MfmaArgs &ka, int n_groups, hipStream_t st
     if (lds > 160 * 1024) return fail(CML_ERR_UNSUPPORTED, "matrix-core path: %d blocks per row exceed the LDS budget", ka.n_slabs * 8);
     static bool raised = false;  // per instantiation: allow more than 64 KB of dynamic LDS once
     if (!raised) {
-        CML_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_b32_mfma_kernel<FMT, GPW, TB, KC, RING>),
+        CML_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_b32_mfma_kernel<FMT, GPW, TB, KC, RING, PLAIN>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
         raised = true;
     }
-    hipLaunchKernelGGL((gemm_b32_mfma_kernel<FMT, GPW, TB, KC, RING>), dim3(gx, gy, n_groups), dim3(256), lds, st, ka);
+    hipLaunchKernelGGL((gemm_b32_mfma_kernel<FMT, GPW, TB, KC, RING, PLAIN>), dim3(gx, gy, n_groups), dim3(256), lds, st, ka);
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
+}
+
+template <int FMT, int GPW, int TB, int KC, int RING>
+static int launch_b32_mfma_g(const B32MfmaArgs &ka, int n_groups, hipStream_t st) {
+    // Measured per variant, same box, alternating runs: the plain entry gains 0.5-2 % everywhere
+    // (Q4_K 4 %) except the 16-token Q8_0 shape, which it slows from 11.3 to 11.9 us -- same
+    // register count, a different schedule; that one keeps the general entry.
+    constexpr bool kPlainPays = !(FMT == CML_Q8_0 && GPW == 1 && TB == 1);
+    return (kPlainPays && ka.group_offsets == nullptr && !env_int("CAMELID_HIP_MFMA_GENERAL_ENTRY", 0)) ? launch_b32_mfma_gp<FMT, GPW, TB, KC, RING, true>(ka, n_groups, st)
+                                       : launch_b32_mfma_gp<FMT, GPW, TB, KC, RING, false>(ka, n_groups, st);
 }
 
 // Phase length and ring depth.  Short phases keep the LDS footprint small, so that several

@@ -108,7 +108,8 @@ __device__ __forceinline__ uint32_t q6_center(uint32_t codes) {
 // KS > 1: KS waves per row tile, each walking one part of K (the matvec kernel's split points);
 // their partial chains are added left to right through LDS at the end.  SPLIT: the same split
 // reproduced inside one lane (for split factors that are not run as waves).
-template <int GPW, int TB, bool SPLIT, int KC, int RING, int KS = 1>
+// PLAIN: the entry of a call without expert groups (no group tables to read before the first request).
+template <int GPW, int TB, bool SPLIT, int KC, int RING, int KS = 1, bool PLAIN = false>
 __global__ __launch_bounds__(256) void gemm_q6k_mfma_kernel(Q6KMfmaArgs a) {
     static_assert(!(SPLIT && KS > 1), "K is split across waves or inside the lane, not both");
     constexpr int NTOK = 16 * GPW * TB;              // tokens staged per workgroup
@@ -134,7 +135,7 @@ __global__ __launch_bounds__(256) void gemm_q6k_mfma_kernel(Q6KMfmaArgs a) {
     const int n_loc = s_end - s_begin, n_max = (n_sb + KS - 1) / KS;
     const int tile = blockIdx.x * RT + rt;
     const int row = tile * 16 + n;
-    const bool grouped = a.group_offsets != nullptr;
+    const bool grouped = !PLAIN && a.group_offsets != nullptr;
     const int64_t band = grouped ? (a.group_ids ? a.group_ids[blockIdx.z] : static_cast<int>(blockIdx.z)) : 0;
     if (band < 0) return;  // a z-slot past the groups in use
     const int a0 = grouped ? a.group_offsets[band] : 0;  // first assignment of this group
@@ -145,6 +146,7 @@ __global__ __launch_bounds__(256) void gemm_q6k_mfma_kernel(Q6KMfmaArgs a) {
     // activation row of local token t (tokens past the end repeat the last one; their cells are not stored)
     auto act_row = [&](int t) __attribute__((always_inline)) -> int64_t {
         const int j = a0 + tok0 + min(t, n_here - 1);
+        if (PLAIN) return j;
         return a.group_rows ? a.group_rows[j] : j;
     };
 
@@ -353,8 +355,8 @@ __global__ __launch_bounds__(256) void gemm_q6k_mfma_kernel(Q6KMfmaArgs a) {
 
 int q6k_ksplit_for(int64_t rows, int64_t n_sb);  // gemv_q6k.hip: the matvec kernel's K-split policy
 
-template <int GPW, int TB, bool SPLIT, int KC, int RING, int KS = 1>
-static int launch_q6k_mfma_g(const Q6KMfmaArgs &ka, int n_groups, hipStream_t st) {
+template <int GPW, int TB, bool SPLIT, int KC, int RING, int KS, bool PLAIN>
+static int launch_q6k_mfma_gp(const Q6KMfmaArgs &ka, int n_groups, hipStream_t st) {
     constexpr int NTOK = 16 * GPW * TB, RT = 4 / (TB * KS);
     const int n_tiles = (ka.rows + 15) / 16;
     const unsigned gx = static_cast<unsigned>((n_tiles + RT - 1) / RT);
@@ -363,13 +365,19 @@ static int launch_q6k_mfma_g(const Q6KMfmaArgs &ka, int n_groups, hipStream_t st
     if (lds > 160 * 1024) return fail(CML_ERR_UNSUPPORTED, "Q6_K matrix-core path: %d super-blocks exceed the LDS budget", ka.n_sb);
     static bool raised = false;  // per instantiation: allow more than 64 KB of dynamic LDS once
     if (!raised) {
-        CML_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q6k_mfma_kernel<GPW, TB, SPLIT, KC, RING, KS>),
+        CML_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q6k_mfma_kernel<GPW, TB, SPLIT, KC, RING, KS, PLAIN>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
         raised = true;
     }
-    hipLaunchKernelGGL((gemm_q6k_mfma_kernel<GPW, TB, SPLIT, KC, RING, KS>), dim3(gx, gy, n_groups), dim3(256), lds, st, ka);
+    hipLaunchKernelGGL((gemm_q6k_mfma_kernel<GPW, TB, SPLIT, KC, RING, KS, PLAIN>), dim3(gx, gy, n_groups), dim3(256), lds, st, ka);
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
+}
+
+template <int GPW, int TB, bool SPLIT, int KC, int RING, int KS = 1>
+static int launch_q6k_mfma_g(const Q6KMfmaArgs &ka, int n_groups, hipStream_t st) {
+    return (ka.group_offsets == nullptr && !env_int("CAMELID_HIP_MFMA_GENERAL_ENTRY", 0)) ? launch_q6k_mfma_gp<GPW, TB, SPLIT, KC, RING, KS, true>(ka, n_groups, st)
+                                       : launch_q6k_mfma_gp<GPW, TB, SPLIT, KC, RING, KS, false>(ka, n_groups, st);
 }
 
 // Phase length and ring depth: short phases and a shallow ring let several workgroups share a
