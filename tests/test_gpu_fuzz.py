@@ -1,0 +1,50 @@
+"""Random shapes through the plain matvec / small-batch entry points: every format, ragged row
+counts, 1..9 tokens, a band view that starts inside a tile -- bit for bit against the oracle in
+the exact order, within 1e-5 max-rel under the default K-split policy."""
+import numpy as np
+import pytest
+
+import oracle
+from camelid_amd import binding as B
+from camelid_amd.binding import Weight, lib
+from tests import gpu_util as G
+
+pytestmark = pytest.mark.gpu
+
+EXACT = {oracle.Q8_0: oracle.ORDER_PRIMARY, oracle.Q4_0: oracle.ORDER_PRIMARY,
+         oracle.Q4_K: oracle.ORDER_PRIMARY, oracle.Q6_K: oracle.ORDER_ALT}
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _init():
+    assert lib().cml_available() == 1
+    B.init(0)
+    yield
+
+
+@pytest.mark.parametrize("seed", [3, 17])
+def test_random_shapes_match_the_oracle(seed):
+    rng = np.random.default_rng(seed)
+    for case in range(48):
+        fmt = [oracle.Q8_0, oracle.Q4_0, oracle.Q4_K, oracle.Q6_K][case % 4]
+        unit = 256 if fmt in (oracle.Q4_K, oracle.Q6_K) else 32
+        rows = int(rng.integers(1, 700))
+        cols = unit * int(rng.integers(1, 24 if unit == 256 else 160))
+        n = int(rng.choice([1, 1, 2, 3, 5, 9]))
+        G.say(f"fuzz seed={seed} case={case} fmt={fmt} {rows}x{cols} n={n}")
+        wire = G.synth_weight(fmt, rows, cols, seed=1000 * seed + case)
+        w = Weight.upload(fmt, rows, cols, wire)
+        x = rng.standard_normal((n, cols)).astype(np.float32)
+        s, q = oracle.quantize_activation(fmt, x)
+        want = oracle.matmul(fmt, wire, cols, x, order=EXACT[fmt], threads=8)
+        with G.env(CAMELID_HIP_EXACT_ORDER="1"):
+            got = G.gpu_gemm(w, s, q).reshape(n, rows)
+            assert G.same_bits(got, want), (case, fmt, rows, cols, n)
+            if n == 1:
+                assert G.same_bits(G.gpu_matmul_f32(w, x[0]), want[0]), (case, fmt, rows, cols)
+            if rows > 40:   # a band of rows that starts inside a tile
+                start, count = int(rng.integers(1, 30)), int(rng.integers(1, rows - 30))
+                band = w.slice(start, count)
+                assert G.same_bits(G.gpu_gemm(band, s, q).reshape(n, count), want[:, start:start + count]), (case, start, count)
+        default = G.gpu_gemm(w, s, q).reshape(n, rows)   # default K-split policy
+        assert G.max_rel(default, want) <= 1e-5, (case, fmt, rows, cols, n)
