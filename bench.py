@@ -19,6 +19,7 @@ import argparse
 import ctypes as C
 import json
 import os
+import re
 import sys
 import time
 
@@ -64,6 +65,10 @@ CONFIGS = {
     "q4k_4096x14336_n16": ("Q4_K", 4096, 14336, 16),
     "q4k_4096x14336_n64": ("Q4_K", 4096, 14336, 64),
     # batches on the other formats (speculative verify / prefill widths); not BASELINE configurations
+    "q8_0_14336x4096_n1": ("Q8_0", 14336, 4096, 1),
+    "q8_0_14336x4096_n2": ("Q8_0", 14336, 4096, 2),
+    "q8_0_128256x3072_n1": ("Q8_0", 128256, 3072, 1),
+    "q8_0_8192x2048_n2": ("Q8_0", 8192, 2048, 2),
     "q8_0_8192x2048_n4": ("Q8_0", 8192, 2048, 4),
     "q8_0_8192x2048_n8": ("Q8_0", 8192, 2048, 8),
     "q4_0_128256x3072_n4": ("Q4_0", 128256, 3072, 4),
@@ -371,7 +376,9 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--config", default="q4k_14336x4096_n1", choices=sorted(CONFIGS) + sorted(MOE_CONFIGS) + sorted(PRODUCER_CONFIGS))
+    ap.add_argument("--config", default="q4k_14336x4096_n1",
+                    help="one of: " + ", ".join(sorted(CONFIGS) + sorted(MOE_CONFIGS) + sorted(PRODUCER_CONFIGS))
+                    + "; or any <format>_<rows>x<cols>_n<tokens>, e.g. q8_0_14336x4352_n1")
     ap.add_argument("--copies", type=int, default=0, help="distinct weight copies to rotate over (0 = enough for ~600 MB)")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="time budget of the CPU baseline leg (0 = skip)")
     ap.add_argument("--seed", type=int, default=1234)
@@ -397,7 +404,15 @@ def main() -> int:
         return bench_producer(args.config, max(1, args.steps), max(0, args.warmup), args.seed)
     if args.config in MOE_CONFIGS:
         return bench_moe(args.config, max(1, args.steps), max(0, args.warmup), args.seed, args.cpu_seconds)
-    fmt_name, rows, cols, n = CONFIGS[args.config]
+    if args.config in CONFIGS:
+        fmt_name, rows, cols, n = CONFIGS[args.config]
+    else:
+        m = re.fullmatch(r"(q8_0|q4_0|q4k|q6k)_(\d+)x(\d+)_n(\d+)", args.config)
+        if not m:
+            print(f"unknown --config {args.config}", file=sys.stderr)
+            return 2
+        fmt_name = {"q8_0": "Q8_0", "q4_0": "Q4_0", "q4k": "Q4_K", "q6k": "Q6_K"}[m.group(1)]
+        rows, cols, n = int(m.group(2)), int(m.group(3)), int(m.group(4))
     fmt = B.FORMATS[fmt_name]
     K, W = max(1, args.steps), max(0, args.warmup)
 

@@ -86,6 +86,10 @@ __device__ __forceinline__ int row_shr_i32(int v) {
     static_assert(N >= 1 && N <= 15, "row_shr distance");
     return __builtin_amdgcn_update_dpp(0, v, 0x110 + N, 0xf, 0xf, true);
 }
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
 template <int N>
 __device__ __forceinline__ float row_shr_f32(float v) {
     return __builtin_bit_cast(float, row_shr_i32<N>(__builtin_bit_cast(int, v)));
@@ -139,9 +143,12 @@ __device__ __forceinline__ int q8_0_round(float v) {
 // packed; `scale` is the same in all eight lanes.  All eight lanes of a group must call it together.
 __device__ __forceinline__ uint32_t q8_0_quantize_lane8(const float4 v, float &scale) {
     float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-    amax = fmaxf(amax, __shfl_xor(amax, 1));
-    amax = fmaxf(amax, __shfl_xor(amax, 2));
-    amax = fmaxf(amax, __shfl_xor(amax, 4));
+    // maximum over the aligned group of eight lanes by data-parallel-primitive moves (no LDS
+    // crossbar round trips): lanes 1 and 2 apart inside each quad, then the other quad of the
+    // group through the mirror of the half row (lane i <-> 7 - i, which holds that quad's maximum)
+    amax = fmaxf(amax, dpp_f32<0xB1>(amax));   // quad_perm [1,0,3,2]
+    amax = fmaxf(amax, dpp_f32<0x4E>(amax));   // quad_perm [2,3,0,1]
+    amax = fmaxf(amax, dpp_f32<0x141>(amax));  // row_half_mirror
     const float u = amax / 127.0f;
     const float inv = (u == 0.0f) ? 0.0f : 1.0f / u;
     // f32 -> f16 round-to-nearest-even -> f32 (reference f32_to_f16_bits, src/inference.rs:27062-27096)

@@ -45,6 +45,9 @@ struct B32Args {
     int early_loads;  // issue the first weight loads ahead of the fused quantizer
 };
 
+#ifndef CML_B32_U
+#define CML_B32_U 2
+#endif
 template <int FMT, int UU = 2>
 struct B32Regs {
     static constexpr int U = UU;  // steps in flight per buffer
@@ -52,6 +55,41 @@ struct B32Regs {
     uint4 qb[U];  // Q8_0 only
     uint32_t d[U];
 };
+
+// Q8_0 rows of 16 lanes ("paired" mapping): a step is 16 blocks = 512 contiguous bytes of the row,
+// and each of the two load instructions takes 256 contiguous bytes of it -- lane l the 16 bytes at
+// l*16 and at 256 + l*16 -- so every instruction consumes whole 128-byte lines exactly once (two
+// lanes share a block: lanes 2j, 2j+1 hold the halves of block j, then of block 8+j).  The two
+// half-block integer sums meet by one lane swap (exact integers: the order inside a block is free);
+// the even lane then carries block j's term, the odd lane block 8+j's, and the ordered fold visits
+// even lanes first.  The one-block-per-lane mapping had each instruction touch half of every line.
+template <int FMT, int P>
+inline constexpr bool kB32Paired =
+#ifdef CML_Q8_0_BLOCK_PER_LANE
+    false;
+#else
+    (FMT == CML_Q8_0 && P == 16);
+#endif
+
+__device__ __forceinline__ int quad_swap1_i32(int v) {  // lanes 2j <-> 2j+1
+    return __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xf, 0xf, true);
+}
+
+// The block whose term lane l carries in step `s` of a paired row, and the two blocks it loads halves of.
+__device__ __forceinline__ int paired_block(int s, int l, int which) { return s * 16 + which * 8 + (l >> 1); }
+
+// Ordered fold for the paired mapping: terms of lanes 0, 2, .., 14 (blocks 0..7 of the step), then
+// of lanes 1, 3, .., 15 (blocks 8..15); lane 15 returns the chain.
+template <int K = 0>
+__device__ __forceinline__ float paired_fold_ordered(float acc, float term) {
+    if constexpr (K == 15) {
+        return acc + term;
+    } else {
+        constexpr int src = (K < 8) ? 2 * K : 2 * (K - 8) + 1;  // lane whose term is the K-th block's
+        acc = acc + row_shr_f32<15 - src>(term);
+        return paired_fold_ordered<K + 1>(acc, term);
+    }
+}
 
 template <int FMT, int P, int U>
 __device__ __forceinline__ void b32_load(B32Regs<FMT, U> &r, const uint8_t *qrow, const uint8_t *srow, int l,
@@ -61,6 +99,15 @@ __device__ __forceinline__ void b32_load(B32Regs<FMT, U> &r, const uint8_t *qrow
     // keeps the next buffer's loads in flight under the current arithmetic.
 #pragma unroll
     for (int u = 0; u < U; u++) {
+        if constexpr (kB32Paired<FMT, P>) {
+            const int s = min(step + u, n_steps - 1);
+            const int ba = min(paired_block(s, l, 0), nb - 1), bb = min(paired_block(s, l, 1), nb - 1);
+            const int half = (l & 1) * 16;
+            r.qa[u] = ldg16_stream(qrow + static_cast<int64_t>(ba) * 32 + half);
+            r.qb[u] = ldg16_stream(qrow + static_cast<int64_t>(bb) * 32 + half);
+            r.d[u] = ldg2(srow + static_cast<int64_t>((l & 1) ? bb : ba) * 2);
+            continue;
+        }
         const int b = min(min(step + u, n_steps - 1) * P + l, nb - 1);
         if constexpr (FMT == CML_Q8_0) {
             // two loads per 32-byte block: each touches half of every line, so the lines must
@@ -84,6 +131,32 @@ __device__ __forceinline__ void b32_compute(const B32Regs<FMT, U> &r, int l, int
                                             int32_t *ints_row) {
 #pragma unroll
     for (int u = 0; u < U; u++) {
+        if constexpr (kB32Paired<FMT, P>) {
+            const int s = min(step + u, n_steps - 1);
+            const int ba = min(paired_block(s, l, 0), nb - 1), bb = min(paired_block(s, l, 1), nb - 1);
+            const int odd = l & 1;
+            const int b_raw = paired_block(step + u, l, odd);
+            const bool valid = (step + u < n_steps) && (b_raw < nb);
+            const int b = odd ? bb : ba;
+            const float dw = f16_bits_to_f32(r.d[u]);
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                const int8_t *y = ys + static_cast<int64_t>(t) * nb * 32 + odd * 16;
+                const uint4 ya = *reinterpret_cast<const uint4 *>(y + ba * 32);
+                const uint4 yb = *reinterpret_cast<const uint4 *>(y + bb * 32);
+                int pa = dot16(r.qa[u], ya, 0), pb = dot16(r.qb[u], yb, 0);
+                pa += quad_swap1_i32(pa);
+                pb += quad_swap1_i32(pb);
+                const int isum = odd ? pb : pa;
+                float term = (static_cast<float>(isum) * dw) * xss[t * nb + b];
+                term = valid ? term : 0.0f;
+                acc[t] = paired_fold_ordered(acc[t], term);
+                if constexpr (INTS) {
+                    if (ints_row != nullptr && valid) ints_row[b] = isum;
+                }
+            }
+            continue;
+        }
         const int b_raw = (step + u) * P + l;
         const bool valid = (step + u < n_steps) && (b_raw < nb);
         const int b = min(min(step + u, n_steps - 1) * P + l, nb - 1);
@@ -118,7 +191,7 @@ __device__ __forceinline__ void b32_compute(const B32Regs<FMT, U> &r, int l, int
 
 // `ra` arrives loaded with steps 0..U-1 (b32_load) -- the caller may have issued those loads well
 // before, e.g. ahead of its prologue.
-template <int FMT, int P, int NT, bool INTS, int U = 2>
+template <int FMT, int P, int NT, bool INTS, int U = CML_B32_U>
 __device__ __forceinline__ void b32_row_pass_from(B32Regs<FMT, U> &ra, const uint8_t *qrow, const uint8_t *srow, int l, int nb,
                                                   const int8_t *ys, const int *bsum, const float *xss, float (&acc)[NT],
                                                   int32_t *ints_row) {
@@ -148,7 +221,7 @@ __device__ __forceinline__ void b32_row_pass_from(B32Regs<FMT, U> &ra, const uin
 
 // One pass over a row's blocks for NT staged activation rows: two register buffers alternate,
 // the last one is consumed without issuing further loads.
-template <int FMT, int P, int NT, bool INTS, int U = 2>
+template <int FMT, int P, int NT, bool INTS, int U = CML_B32_U>
 __device__ __forceinline__ void b32_row_pass(const uint8_t *qrow, const uint8_t *srow, int l, int nb, const int8_t *ys,
                                              const int *bsum, const float *xss, float (&acc)[NT], int32_t *ints_row) {
     const int n_steps = (nb + P - 1) / P;
@@ -187,7 +260,7 @@ __global__ __launch_bounds__(256) void gemv_b32_kernel(B32Args a) {
     const uint8_t *srow = a.scales + arow * a.s_stride;
     const bool leader = (l == P - 1);
     const int n_steps = (nb + P - 1) / P;
-    constexpr int UE = 2;  // steps loaded ahead of the fused quantizer (4 measured slower)
+    constexpr int UE = CML_B32_U;  // steps loaded ahead of the fused quantizer (4 measured slower)
     B32Regs<FMT, UE> ra;
     bool preloaded = false;
 
@@ -206,16 +279,22 @@ __global__ __launch_bounds__(256) void gemv_b32_kernel(B32Args a) {
             preloaded = true;
             __builtin_amdgcn_sched_barrier(0);
             uint32_t *ys32 = reinterpret_cast<uint32_t *>(ys);
+            // straight-line: the four blocks of a thread are independent chains the scheduler can
+            // interleave; only the LDS stores are predicated (whole blocks of eight lanes are in or
+            // out together, and a clamped load duplicates the last block's values)
+            uint32_t packed[NX];
+            float scale[NX];
+#pragma unroll
+            for (int j = 0; j < NX; j++) packed[j] = q8_0_quantize_lane8(xv[j], scale[j]);
 #pragma unroll
             for (int j = 0; j < NX; j++) {
                 const int i = tid + 256 * j;
-                if (i < n4) {  // whole blocks of eight lanes enter and leave together
-                    float scale;
-                    const uint32_t packed = q8_0_quantize_lane8(xv[j], scale);
-                    ys32[i] = packed;
-                    if ((i & 7) == 0) xss[i >> 3] = scale;
+                int sum = 0;
+                if constexpr (FMT == CML_Q4_0) sum = group_sum_to_last<8>(sdot4(packed[j], 0x01010101u, 0));
+                if (i < n4) {
+                    ys32[i] = packed[j];
+                    if ((i & 7) == 0) xss[i >> 3] = scale[j];
                     if constexpr (FMT == CML_Q4_0) {
-                        const int sum = group_sum_to_last<8>(sdot4(packed, 0x01010101u, 0));
                         if ((i & 7) == 7) bsum[i >> 3] = sum;
                     }
                 }
