@@ -45,9 +45,6 @@ struct B32Args {
     int early_loads;  // issue the first weight loads ahead of the fused quantizer
 };
 
-#ifndef CML_B32_U
-#define CML_B32_U 2
-#endif
 template <int FMT, int UU = 2>
 struct B32Regs {
     static constexpr int U = UU;  // steps in flight per buffer
@@ -191,7 +188,7 @@ __device__ __forceinline__ void b32_compute(const B32Regs<FMT, U> &r, int l, int
 
 // `ra` arrives loaded with steps 0..U-1 (b32_load) -- the caller may have issued those loads well
 // before, e.g. ahead of its prologue.
-template <int FMT, int P, int NT, bool INTS, int U = CML_B32_U>
+template <int FMT, int P, int NT, bool INTS, int U = 2>
 __device__ __forceinline__ void b32_row_pass_from(B32Regs<FMT, U> &ra, const uint8_t *qrow, const uint8_t *srow, int l, int nb,
                                                   const int8_t *ys, const int *bsum, const float *xss, float (&acc)[NT],
                                                   int32_t *ints_row) {
@@ -221,7 +218,7 @@ __device__ __forceinline__ void b32_row_pass_from(B32Regs<FMT, U> &ra, const uin
 
 // One pass over a row's blocks for NT staged activation rows: two register buffers alternate,
 // the last one is consumed without issuing further loads.
-template <int FMT, int P, int NT, bool INTS, int U = CML_B32_U>
+template <int FMT, int P, int NT, bool INTS, int U = 2>
 __device__ __forceinline__ void b32_row_pass(const uint8_t *qrow, const uint8_t *srow, int l, int nb, const int8_t *ys,
                                              const int *bsum, const float *xss, float (&acc)[NT], int32_t *ints_row) {
     const int n_steps = (nb + P - 1) / P;
@@ -234,8 +231,9 @@ __device__ __forceinline__ void b32_row_pass(const uint8_t *qrow, const uint8_t 
 // FUSEQ (single token): the activation arrives as f32 and every workgroup quantizes it to Q8_0
 // itself, eight lanes per block, straight into the LDS staging area -- the arithmetic of
 // quantize_q8_0_kernel without the launch and the round trip through memory.
-template <int FMT, int P, int NT, bool INTS, bool FUSEQ = false>
-__global__ __launch_bounds__(256) void gemv_b32_kernel(B32Args a) {
+template <int FMT, int P, int NT, bool INTS, bool FUSEQ = false, int WAVES = 4, int NXQ = 0, int U = 2>
+__global__ __launch_bounds__(WAVES * 64) void gemv_b32_kernel(B32Args a) {
+    constexpr int T = WAVES * 64;  // threads of a workgroup; its activation prologue is shared by WAVES * (64 / P) rows
     static_assert(!FUSEQ || (NT == 1 && !INTS), "the fused quantizer serves single-token calls");
     constexpr int RPW = kWave / P;
     extern __shared__ uint4 smem[];
@@ -253,27 +251,29 @@ __global__ __launch_bounds__(256) void gemv_b32_kernel(B32Args a) {
 
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int r = lane / P, l = lane - r * P;
-    const int row = (blockIdx.x * 4 + wave) * RPW + r;
+    const int row = (blockIdx.x * WAVES + wave) * RPW + r;
     const bool live = row < a.rows;
     const int64_t arow = band * a.rows + (live ? row : a.rows - 1);
     const uint8_t *qrow = a.quants + arow * a.q_stride;
     const uint8_t *srow = a.scales + arow * a.s_stride;
     const bool leader = (l == P - 1);
     const int n_steps = (nb + P - 1) / P;
-    constexpr int UE = CML_B32_U;  // steps loaded ahead of the fused quantizer (4 measured slower)
+    constexpr int UE = U;  // steps per register buffer, also loaded ahead of the prologue
     B32Regs<FMT, UE> ra;
     bool preloaded = false;
 
     if constexpr (FUSEQ) {
         const float4 *x4 = reinterpret_cast<const float4 *>(a.x);
-        constexpr int NX = 4;  // float4 per thread held in registers: rows of up to 128 blocks
-        if (nb <= NX * 32 && a.early_loads) {  // uniform
+        // NXQ > 0 (the launcher's promise that nb * 8 <= T * NXQ): the thread holds NXQ float4 of
+        // the activation in registers -- rows of up to 128 blocks
+        constexpr int NX = NXQ > 0 ? NXQ : 1;
+        if constexpr (NXQ > 0) {
             // The token's f32 loads go out first, the row's first weight steps right behind them, and
             // the quantizer then waits for the f32 values only (a wave's loads return in order).
             const int n4 = nb * 8;
             float4 xv[NX];
 #pragma unroll
-            for (int j = 0; j < NX; j++) xv[j] = x4[min(tid + 256 * j, n4 - 1)];
+            for (int j = 0; j < NX; j++) xv[j] = x4[min(tid + T * j, n4 - 1)];
             __builtin_amdgcn_sched_barrier(0);
             b32_load<FMT, P, UE>(ra, qrow, srow, l, 0, n_steps, nb);
             preloaded = true;
@@ -288,7 +288,7 @@ __global__ __launch_bounds__(256) void gemv_b32_kernel(B32Args a) {
             for (int j = 0; j < NX; j++) packed[j] = q8_0_quantize_lane8(xv[j], scale[j]);
 #pragma unroll
             for (int j = 0; j < NX; j++) {
-                const int i = tid + 256 * j;
+                const int i = tid + T * j;
                 int sum = 0;
                 if constexpr (FMT == CML_Q4_0) sum = group_sum_to_last<8>(sdot4(packed[j], 0x01010101u, 0));
                 if (i < n4) {
@@ -300,13 +300,13 @@ __global__ __launch_bounds__(256) void gemv_b32_kernel(B32Args a) {
                 }
             }
         } else {
-            b32_stage_quantized_from<FMT>([&](int i) { return x4[i]; }, nb, tid, ys, xss, bsum);
+            b32_stage_quantized_from<FMT, T>([&](int i) { return x4[i]; }, nb, tid, ys, xss, bsum);
         }
     } else {
         const uint4 *src = reinterpret_cast<const uint4 *>(q);
         uint4 *dst = reinterpret_cast<uint4 *>(ys);
         const int n16 = NT * nb * 2;  // even: lanes 2k, 2k+1 are in or out together
-        if (NT == 1 && n16 <= 256 && a.early_loads) {  // uniform: one 16-byte piece and one scale per thread at most
+        if (NT == 1 && n16 <= T && a.early_loads) {  // uniform: one 16-byte piece and one scale per thread at most
             // the same order of issue for a quantized activation: its loads, the first weight steps, then the staging
             const uint4 v = src[min(tid, n16 - 1)];
             const float sc = xs[min(tid, nb - 1)];
@@ -324,7 +324,7 @@ __global__ __launch_bounds__(256) void gemv_b32_kernel(B32Args a) {
             }
             if (tid < nb) xss[tid] = sc;
         } else {
-            for (int i = tid; i < n16; i += 256) {
+            for (int i = tid; i < n16; i += T) {
                 const uint4 v = src[i];
                 dst[i] = v;
                 if constexpr (FMT == CML_Q4_0) {
@@ -333,7 +333,7 @@ __global__ __launch_bounds__(256) void gemv_b32_kernel(B32Args a) {
                     if (i & 1) bsum[i >> 1] = s;
                 }
             }
-            for (int i = tid; i < NT * nb; i += 256) xss[i] = xs[i];
+            for (int i = tid; i < NT * nb; i += T) xss[i] = xs[i];
         }
     }
     __syncthreads();
@@ -350,7 +350,7 @@ __global__ __launch_bounds__(256) void gemv_b32_kernel(B32Args a) {
     if (preloaded) {
         b32_row_pass_from<FMT, P, NT, INTS, UE>(ra, qrow, srow, l, nb, ys, bsum, xss, acc, ints_row);
     } else {
-        b32_row_pass<FMT, P, NT, INTS>(qrow, srow, l, nb, ys, bsum, xss, acc, ints_row);
+        b32_row_pass<FMT, P, NT, INTS, U>(qrow, srow, l, nb, ys, bsum, xss, acc, ints_row);
     }
 
     if (leader && live) {
@@ -363,6 +363,18 @@ __global__ __launch_bounds__(256) void gemv_b32_kernel(B32Args a) {
     }
 }
 
+// Steps per register buffer.  Long rows of a matrix with few of them leave one or two waves per
+// SIMD, and then the bytes each wave keeps in flight decide the rate: four steps per buffer
+// instead of two (Q4_0 4096 x 14336: 10.5 -> 9.5 us).  With more waves the deeper buffers only
+// cost registers (14336 x 4096: 15.3 -> 16.4 us).
+static int b32_depth(int rows, int lanes_per_row, int nb) {
+    const int u = env_int("CAMELID_HIP_B32_DEPTH", 0);
+    if (u == 2 || u == 4) return u;
+    const int waves = (rows + 64 / lanes_per_row - 1) / (64 / lanes_per_row);
+    const int n_steps = (nb + lanes_per_row - 1) / lanes_per_row;
+    return (waves <= 2048 && n_steps >= 16) ? 4 : 2;
+}
+
 template <int FMT, int P, int NT>
 static int launch_b32_nt(const B32Args &ba, int n_bands, bool ints, hipStream_t st) {
     const int rows_per_wg = 4 * (64 / P);
@@ -371,6 +383,8 @@ static int launch_b32_nt(const B32Args &ba, int n_bands, bool ints, hipStream_t 
     if (lds > 64 * 1024) return fail(CML_ERR_UNSUPPORTED, "activation of %d blocks x %d tokens exceeds the LDS staging limit", ba.nb, NT);
     if (ints && NT == 1)
         hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, true>), dim3(gx, n_bands), dim3(256), lds, st, ba);
+    else if (NT <= 2 && n_bands == 1 && b32_depth(ba.rows, P, ba.nb) == 4)
+        hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, (NT <= 2 ? NT : 1), false, false, 4, 0, 4>), dim3(gx, n_bands), dim3(256), lds, st, ba);
     else
         hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, NT, false>), dim3(gx, n_bands), dim3(256), lds, st, ba);
     CML_HIP_TRY(hipGetLastError());
@@ -428,11 +442,35 @@ static int launch_b32_f32_p(const cml_weight *w, const float *x, float *out, hip
     ba.x = x;
     ba.out = out;
     ba.early_loads = env_int("CAMELID_HIP_B32_EARLY_LOADS", 1);
-    const int rows_per_wg = 4 * (64 / P);
-    const unsigned gx = static_cast<unsigned>((ba.rows + rows_per_wg - 1) / rows_per_wg);
     const size_t lds = static_cast<size_t>(ba.nb) * (32 + 4 + 4);
     if (lds > 64 * 1024) return fail(CML_ERR_UNSUPPORTED, "activation of %d blocks exceeds the LDS staging limit", ba.nb);
-    hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, true>), dim3(gx, 1), dim3(256), lds, st, ba);
+    // Every workgroup quantizes the whole activation for itself; with eight waves twice the rows
+    // share that prologue.  Worth it while the matrix still gives every compute unit a workgroup.
+    int waves = env_int("CAMELID_HIP_B32_FUSED_WAVES", 0);
+    if (waves != 4 && waves != 8) waves = (ba.rows >= 128 * 8 * (64 / P)) ? 8 : 4;
+    const int rows_per_wg = waves * (64 / P);
+    const unsigned gx = static_cast<unsigned>((ba.rows + rows_per_wg - 1) / rows_per_wg);
+    // float4 of the activation per thread: 1, 2 or 4 in registers; longer rows (or the knob) take the staged path
+    const int n4 = ba.nb * 8, threads = waves * 64;
+    int nxq = !ba.early_loads ? 0 : n4 <= threads ? 1 : n4 <= 2 * threads ? 2 : n4 <= 4 * threads ? 4 : 0;
+    if (waves == 8 && nxq == 4) nxq = 0;  // 2048 float4 would be 256 blocks; eight waves are launched for at most 128
+#define CML_B32_FUSED(W_, N_) \
+    hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, true, W_, N_>), dim3(gx, 1), dim3(W_ * 64), lds, st, ba)
+    const bool deep = nxq == 0 && b32_depth(ba.rows, P, ba.nb) == 4;
+    if (deep) {
+        if (waves == 8) hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, true, 8, 0, 4>), dim3(gx, 1), dim3(512), lds, st, ba);
+        else hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, true, 4, 0, 4>), dim3(gx, 1), dim3(256), lds, st, ba);
+    } else if (waves == 8) {
+        if (nxq == 1) CML_B32_FUSED(8, 1);
+        else if (nxq == 2) CML_B32_FUSED(8, 2);
+        else CML_B32_FUSED(8, 0);
+    } else {
+        if (nxq == 1) CML_B32_FUSED(4, 1);
+        else if (nxq == 2) CML_B32_FUSED(4, 2);
+        else if (nxq == 4) CML_B32_FUSED(4, 4);
+        else CML_B32_FUSED(4, 0);
+    }
+#undef CML_B32_FUSED
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }
@@ -481,11 +519,11 @@ struct B32GroupArgs {
 
 // Quantize one row of nb blocks to Q8_0 straight into the LDS staging area, eight lanes per block;
 // value4(i) yields the row's i-th float4.
-template <int FMT, typename F>
+template <int FMT, int T = 256, typename F>
 __device__ __forceinline__ void b32_stage_quantized_from(F value4, int nb, int tid, int8_t *ys, float *xss, int *bsum) {
     uint32_t *ys32 = reinterpret_cast<uint32_t *>(ys);
     const int n4 = nb * 8;  // a multiple of 8: the eight lanes of a block enter and leave together
-    for (int i = tid; i < n4; i += 256) {
+    for (int i = tid; i < n4; i += T) {
         float scale;
         const uint32_t packed = q8_0_quantize_lane8(value4(i), scale);
         ys32[i] = packed;

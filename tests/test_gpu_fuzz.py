@@ -48,3 +48,25 @@ def test_random_shapes_match_the_oracle(seed):
                 assert G.same_bits(G.gpu_gemm(band, s, q).reshape(n, count), want[:, start:start + count]), (case, start, count)
         default = G.gpu_gemm(w, s, q).reshape(n, rows)   # default K-split policy
         assert G.max_rel(default, want) <= 1e-5, (case, fmt, rows, cols, n)
+
+
+@pytest.mark.parametrize("fmt", [oracle.Q8_0, oracle.Q4_0])
+def test_block32_launch_shapes_agree(fmt):
+    """The 32-value-block matvec under each of its launch shapes (4 or 8 waves per workgroup for
+    the fused quantizer, 2 or 4 steps per register buffer, 8 or 16 lanes per row): the same bits."""
+    lanes_knob = "CAMELID_HIP_Q8_0_LANES" if fmt == oracle.Q8_0 else "CAMELID_HIP_Q4_0_LANES"
+    rng = np.random.default_rng(5)
+    for rows, cols in [(77, 32), (1000, 2048), (530, 4096), (300, 8192 + 64), (64, 14336)]:
+        wire = G.synth_weight(fmt, rows, cols, seed=rows + cols)
+        w = Weight.upload(fmt, rows, cols, wire)
+        x = rng.standard_normal((2, cols)).astype(np.float32)
+        s, q = oracle.quantize_activation(fmt, x)
+        want = oracle.matmul(fmt, wire, cols, x, order=EXACT[fmt], threads=8)
+        for waves in ("4", "8"):
+            for depth in ("2", "4"):
+                for lanes in ("8", "16"):
+                    G.say(f"block32 {fmt} {rows}x{cols} waves={waves} depth={depth} lanes={lanes}")
+                    with G.env(CAMELID_HIP_EXACT_ORDER="1", CAMELID_HIP_B32_FUSED_WAVES=waves, CAMELID_HIP_B32_DEPTH=depth, **{lanes_knob: lanes}):
+                        assert G.same_bits(G.gpu_matmul_f32(w, x[0]), want[0]), (rows, cols, waves, depth, lanes)
+                        assert G.same_bits(G.gpu_gemm(w, s[:1], q[:1]).reshape(rows), want[0]), (rows, cols, depth, lanes)
+                        assert G.same_bits(G.gpu_gemm(w, s, q).reshape(2, rows), want), (rows, cols, depth, lanes)
