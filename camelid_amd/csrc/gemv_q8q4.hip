@@ -385,6 +385,10 @@ static int launch_b32_nt(const B32Args &ba, int n_bands, bool ints, hipStream_t 
         hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, true>), dim3(gx, n_bands), dim3(256), lds, st, ba);
     else if (NT <= 2 && n_bands == 1 && b32_depth(ba.rows, P, ba.nb) == 4)
         hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, (NT <= 2 ? NT : 1), false, false, 4, 0, 4>), dim3(gx, n_bands), dim3(256), lds, st, ba);
+    else if (NT <= 2 && n_bands == 1 && env_int("CAMELID_HIP_B32_WAVES", ba.rows >= 384 * 8 * (64 / P) ? 8 : 4) == 8)
+        // eight-wave workgroups where they still come to 1.5 per compute unit (Q8_0 14336 x 4096: 14.0 -> 12.5 us;
+        // 11008 x 4096, 1.3 per compute unit: 6.1 -> 6.9)
+        hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, (NT <= 2 ? NT : 1), false, false, 8, 0, 2>), dim3((gx + 1) / 2, n_bands), dim3(512), lds, st, ba);
     else
         hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, NT, false>), dim3(gx, n_bands), dim3(256), lds, st, ba);
     CML_HIP_TRY(hipGetLastError());
@@ -447,19 +451,33 @@ static int launch_b32_f32_p(const cml_weight *w, const float *x, float *out, hip
     // Every workgroup quantizes the whole activation for itself; with eight waves twice the rows
     // share that prologue.  Worth it while the matrix still gives every compute unit a workgroup.
     int waves = env_int("CAMELID_HIP_B32_FUSED_WAVES", 0);
-    if (waves != 4 && waves != 8) waves = (ba.rows >= 128 * 8 * (64 / P)) ? 8 : 4;
+    if (waves != 2 && waves != 4 && waves != 8 && waves != 16) {
+        waves = (ba.rows >= 128 * 8 * (64 / P)) ? 8 : 4;
+        // Q8_0 rows of 4096 values (the longest the register prologue takes) on tall matrices: sixteen
+        // waves (16384 x 4096: 14.2 -> 12.7 us, 32000 x 4096: 24.7 -> 22.3); slower for Q4_0 and shorter rows
+        if (FMT == CML_Q8_0 && ba.nb == 128 && ba.rows >= 224 * 16 * (64 / P)) waves = 16;
+    }
     const int rows_per_wg = waves * (64 / P);
     const unsigned gx = static_cast<unsigned>((ba.rows + rows_per_wg - 1) / rows_per_wg);
     // float4 of the activation per thread: 1, 2 or 4 in registers; longer rows (or the knob) take the staged path
     const int n4 = ba.nb * 8, threads = waves * 64;
     int nxq = !ba.early_loads ? 0 : n4 <= threads ? 1 : n4 <= 2 * threads ? 2 : n4 <= 4 * threads ? 4 : 0;
     if (waves == 8 && nxq == 4) nxq = 0;  // 2048 float4 would be 256 blocks; eight waves are launched for at most 128
+    if (waves == 16 && nxq != 1) nxq = 0;
+    if (waves == 2 && nxq != 0) nxq = 4;  // one register variant for the short workgroup
 #define CML_B32_FUSED(W_, N_) \
     hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, true, W_, N_>), dim3(gx, 1), dim3(W_ * 64), lds, st, ba)
     const bool deep = nxq == 0 && b32_depth(ba.rows, P, ba.nb) == 4;
     if (deep) {
-        if (waves == 8) hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, true, 8, 0, 4>), dim3(gx, 1), dim3(512), lds, st, ba);
+        if (waves == 2) hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, true, 2, 0, 4>), dim3(gx, 1), dim3(128), lds, st, ba);
+        else if (waves == 8) hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, true, 8, 0, 4>), dim3(gx, 1), dim3(512), lds, st, ba);
         else hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, true, 4, 0, 4>), dim3(gx, 1), dim3(256), lds, st, ba);
+    } else if (waves == 16) {
+        if (nxq == 1) CML_B32_FUSED(16, 1);
+        else CML_B32_FUSED(16, 0);
+    } else if (waves == 2) {
+        if (nxq == 4) CML_B32_FUSED(2, 4);
+        else CML_B32_FUSED(2, 0);
     } else if (waves == 8) {
         if (nxq == 1) CML_B32_FUSED(8, 1);
         else if (nxq == 2) CML_B32_FUSED(8, 2);

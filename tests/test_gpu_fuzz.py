@@ -62,11 +62,11 @@ def test_block32_launch_shapes_agree(fmt):
         x = rng.standard_normal((2, cols)).astype(np.float32)
         s, q = oracle.quantize_activation(fmt, x)
         want = oracle.matmul(fmt, wire, cols, x, order=EXACT[fmt], threads=8)
-        for waves in ("4", "8"):
+        for waves in ("2", "4", "8", "16"):
             for depth in ("2", "4"):
                 for lanes in ("8", "16"):
                     G.say(f"block32 {fmt} {rows}x{cols} waves={waves} depth={depth} lanes={lanes}")
-                    with G.env(CAMELID_HIP_EXACT_ORDER="1", CAMELID_HIP_B32_FUSED_WAVES=waves, CAMELID_HIP_B32_DEPTH=depth, **{lanes_knob: lanes}):
+                    with G.env(CAMELID_HIP_EXACT_ORDER="1", CAMELID_HIP_B32_FUSED_WAVES=waves, CAMELID_HIP_B32_WAVES=("8" if waves == "8" else "4"), CAMELID_HIP_B32_DEPTH=depth, **{lanes_knob: lanes}):
                         assert G.same_bits(G.gpu_matmul_f32(w, x[0]), want[0]), (rows, cols, waves, depth, lanes)
                         assert G.same_bits(G.gpu_gemm(w, s[:1], q[:1]).reshape(rows), want[0]), (rows, cols, depth, lanes)
                         assert G.same_bits(G.gpu_gemm(w, s, q).reshape(2, rows), want), (rows, cols, depth, lanes)
