@@ -629,11 +629,13 @@ int cml_matmul_f32(const cml_weight *w, const float *x_dev, int64_t n_tokens, fl
                                          ((static_cast<size_t>(n_tokens) * w->cols + 255) & ~size_t(255)));
     hipStream_t st = as_stream(stream);
     const int fuse = env_int("CAMELID_HIP_FUSED_QUANT", 1);  // 0 = never, 1 = by shape, 2 = whenever possible
-    if (w->fmt == CML_Q4_K && n_tokens == 1 && (fuse == 2 || (fuse == 1 && w->nb <= 16))) {
+    const bool fuse_two = n_tokens == 2 && env_int("CAMELID_HIP_FUSED_QUANT_TWO", 1) && !env_int("CAMELID_HIP_Q4K_GENERAL_ENTRY", 0);
+    if (w->fmt == CML_Q4_K && (n_tokens == 1 || fuse_two) && (fuse == 2 || (fuse == 1 && w->nb <= 16))) {
         // decode at hidden sizes up to 4096: one launch quantizes the activation in every workgroup
-        // (one pass of its four waves) and runs the matvec; longer rows would need several
-        // quantizer passes per workgroup and measure no faster than the two launches below
-        const int frc = launch_gemv_q4k_f32(w, x_dev, out_dev, st);
+        // (one pass of its four waves; two passes for a pair of tokens) and runs the matvec; longer
+        // rows would need several quantizer passes per workgroup and measure no faster than the
+        // two launches below
+        const int frc = launch_gemv_q4k_f32(w, x_dev, out_dev, st, static_cast<int>(n_tokens));
         if (frc == CML_OK) g_runs.fetch_add(1, std::memory_order_relaxed);
         return frc;
     }

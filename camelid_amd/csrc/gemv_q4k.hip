@@ -239,7 +239,8 @@ __device__ __forceinline__ void q4k_compute(const Q4KRegs<U> &r, const Q4KLane &
 // The plain entry has none of it, and the K split (a power of two) is shifts.
 template <int NT, bool INTS, bool FUSEQ = false, int SPR = 1, bool WHOLE = false, bool PLAIN = false>
 __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
-    static_assert(!FUSEQ || (NT == 1 && !INTS), "the fused quantizer serves single-token calls");
+    static_assert(!FUSEQ || ((NT == 1 || (NT == 2 && PLAIN)) && !INTS),
+                  "the fused quantizer serves single-token calls and plain two-token calls (contiguous f32 rows)");
     static_assert(SPR == 1 || SPR == 2, "groups per row");
     constexpr int RPW = kWave / (LPS * SPR);  // rows per wave tile
     constexpr int U = 4 / SPR;                // buffer entries per group: a buffer always holds 4 super-blocks of a row
@@ -314,8 +315,11 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
             const int nw = nthreads >> 6;
             const int qrow = lane >> 4, ql = lane & 15;
             const float4 *x4 = reinterpret_cast<const float4 *>(a.x + act_row(0) * n_sb * 256);
+            // NT = 2 (plain call): the two f32 rows are contiguous and so are their staging areas, so
+            // the tokens are simply 2 * n_sb super-blocks in a row.
+            const int tq = NT * n_sb;
             auto load_pass = [&](float4 (&xv)[4], int base) {
-                const int sbk = min(base + qrow, n_sb - 1);
+                const int sbk = min(base + qrow, tq - 1);
 #pragma unroll
                 for (int k = 0; k < 4; k++) xv[k] = x4[sbk * 64 + ql * 4 + k];
             };
@@ -324,7 +328,7 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
                 float dv;
                 int bs;
                 const uint4 packed = q8k_quantize_row16(xv, lane, dv, bs);
-                if (sbk < n_sb) {
+                if (sbk < tq) {
                     reinterpret_cast<uint4 *>(ys)[sbk * 16 + ql] = packed;
                     if (ql & 1) bsum[sbk * 8 + (ql >> 1)] = bs;
                     if (ql == 0) yds[sbk] = dv;
@@ -337,7 +341,7 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
             __builtin_amdgcn_sched_barrier(0);
             for (int base = 4 * wave;;) {
                 const int next = base + 4 * nw;
-                if (next >= n_sb) {
+                if (next >= tq) {
                     quantize_pass(xa, base);
                     break;
                 }
@@ -605,7 +609,8 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
     Q4KShape shape = pick_shape(ka.rows, ka.n_sb);
     const int64_t tiles16 = (ka.rows + ka.row_skip + 15) / 16;
     const int64_t slots = static_cast<int64_t>(grouped ? (a.group_ids ? a.max_active : a.n_groups) : 1) * (w2 ? 2 : 1);
-    const bool half_tiles = q4k_rows_per_wave(tiles16, shape.ksplit, slots) == 8;
+    const bool two = !grouped && !w2 && a.n_tokens == 2;  // plain call with two contiguous f32 rows
+    const bool half_tiles = !two && q4k_rows_per_wave(tiles16, shape.ksplit, slots) == 8;
     const int64_t tiles = half_tiles ? 2 * tiles16 : tiles16;
     int tpw = env_int("CAMELID_HIP_Q4K_FUSED_TILES_PER_WG", 0);
     // 4 waves share the quantizing.  Measured with 8-row tiles at 14336 x 4096 (1792 tiles): 2 waves
@@ -615,8 +620,8 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
     shape.tiles_per_wg = tpw;
     const int waves = shape.ksplit * shape.tiles_per_wg;
     const unsigned gx = static_cast<unsigned>((tiles + shape.tiles_per_wg - 1) / shape.tiles_per_wg);
-    const size_t lds = static_cast<size_t>(ka.n_sb) * (256 + 32) + ((static_cast<size_t>(ka.n_sb) + 3) & ~size_t(3)) * 4 +
-                       static_cast<size_t>(waves) * 16 * 4;
+    const size_t nt = two ? 2 : 1;
+    const size_t lds = nt * ka.n_sb * (256 + 32) + ((nt * ka.n_sb + 3) & ~size_t(3)) * 4 + static_cast<size_t>(waves) * nt * 16 * 4;
     if (lds > 64 * 1024) return fail(CML_ERR_UNSUPPORTED, "Q4_K activation of %d super-blocks exceeds the LDS staging limit", ka.n_sb);
     ka.ksplit = shape.ksplit;
     ka.ksplit_log2 = shape.ksplit >= 8 ? 3 : (shape.ksplit >= 4 ? 2 : (shape.ksplit >= 2 ? 1 : 0));
@@ -627,7 +632,11 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
         const bool plain = !grouped && !w2 && !env_int("CAMELID_HIP_Q4K_GENERAL_ENTRY", 0);
         const dim3 block(64 * waves);
 #define CML_Q4K_LAUNCH(SPR_, WHOLE_, PLAIN_) hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, SPR_, WHOLE_, PLAIN_>), grid, block, lds, st, ka)
-        if (half_tiles) {
+        if (two) {
+            // both tokens in one pass over the weight, 16-row waves as in the two-token matvec
+            if (whole) hipLaunchKernelGGL((gemv_q4k_kernel<2, false, true, 1, true, true>), grid, block, lds, st, ka);
+            else hipLaunchKernelGGL((gemv_q4k_kernel<2, false, true, 1, false, true>), grid, block, lds, st, ka);
+        } else if (half_tiles) {
             if (whole) { if (plain) CML_Q4K_LAUNCH(2, true, true); else CML_Q4K_LAUNCH(2, true, false); }
             else { if (plain) CML_Q4K_LAUNCH(2, false, true); else CML_Q4K_LAUNCH(2, false, false); }
         } else {
@@ -640,11 +649,11 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
     return CML_OK;
 }
 
-int launch_gemv_q4k_f32(const cml_weight *w, const float *x, float *out, hipStream_t st) {
+int launch_gemv_q4k_f32(const cml_weight *w, const float *x, float *out, hipStream_t st, int n_tokens) {
     MatArgs a{};
     a.w = w;
     a.out = out;
-    a.n_tokens = 1;
+    a.n_tokens = n_tokens;  // 1, or 2 contiguous rows of x -> out[2][rows]
     a.n_groups = 1;
     return launch_q4k_f32(a, nullptr, nullptr, x, st);
 }

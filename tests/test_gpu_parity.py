@@ -335,6 +335,39 @@ def test_q4k_fused_quantize_matvec_is_the_two_step_path(rows, cols):
             assert G.same_bits(got, want)
 
 
+@pytest.mark.parametrize("rows,cols", [(190, 3072), (64, 256), (333, 4096), (40, 14336), (77, 1280)])
+def test_q4k_fused_two_tokens_is_the_two_step_path(rows, cols):
+    """Two-token cml_matmul_f32 on Q4_K quantizes both rows inside the matvec kernel: the bits of
+    quantize_q8_k + matmul, and of the oracle, for every workgroup shape and K split."""
+    fmt = oracle.Q4_K
+    rng = np.random.default_rng(7200 + rows)
+    wire = G.synth_weight(fmt, rows, cols, seed=7250 + rows)
+    w = Weight.upload(fmt, rows, cols, wire)
+    acts = _activation_cases(cols, rng)
+    acts[0, :256] = 0.0
+    acts[1, -256:] = 0.0
+    acts[2, 17:21] = [1.5 * 3 / 127, 2.5 * 3 / 127, -0.5 * 3 / 127, 0.5 * 3 / 127]
+    for pair in ((0, 1), (2, 0), (1, 2)):
+        x = np.ascontiguousarray(acts[list(pair)])
+        for tpw in (0, 1, 3, 8):
+            for ks in (0, 1, 2):
+                if ks > cols // 256:
+                    continue
+                G.say(f"Q4_K fused two tokens {rows}x{cols} pair={pair} tiles_per_wg={tpw} ksplit={ks}")
+                with G.env(CAMELID_HIP_Q4K_FUSED_TILES_PER_WG=tpw, CAMELID_HIP_Q4K_KSPLIT=ks):
+                    with G.env(CAMELID_HIP_FUSED_QUANT=2):
+                        fused = G.gpu_matmul_f32(w, x)
+                        with G.env(CAMELID_HIP_Q4K_CLAMPED_LOADS=1):
+                            assert G.same_bits(G.gpu_matmul_f32(w, x), fused)
+                    with G.env(CAMELID_HIP_FUSED_QUANT=0):
+                        two_step = G.gpu_matmul_f32(w, x)
+                assert G.same_bits(fused, two_step), (pair, tpw, ks)
+        with G.env(CAMELID_HIP_EXACT_ORDER="1", CAMELID_HIP_FUSED_QUANT=2):
+            got = G.gpu_matmul_f32(w, x)
+        want = oracle.matmul(fmt, wire, cols, x, order=EXACT_ORDER[fmt], threads=8)
+        assert G.same_bits(got, want)
+
+
 @pytest.mark.parametrize("name,fmt", [("Q8_0", oracle.Q8_0), ("Q4_0", oracle.Q4_0)])
 @pytest.mark.parametrize("rows,cols", [(190, 2048), (33, 32), (70, 3072 + 32), (16, 14336)])
 def test_b32_fused_quantize_matvec_is_the_two_step_path(name, fmt, rows, cols):
