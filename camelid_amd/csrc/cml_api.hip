@@ -639,12 +639,12 @@ int cml_matmul_f32(const cml_weight *w, const float *x_dev, int64_t n_tokens, fl
         if (frc == CML_OK) g_runs.fetch_add(1, std::memory_order_relaxed);
         return frc;
     }
-    if ((w->fmt == CML_Q8_0 || w->fmt == CML_Q4_0) && n_tokens == 1 &&
+    if ((w->fmt == CML_Q8_0 || w->fmt == CML_Q4_0) && (n_tokens == 1 || fuse_two) &&
         (fuse == 2 || (fuse == 1 && w->cols <= 8192 && w->rows <= 32768))) {
         // the same for the 32-value block formats, whose workgroups cover only 16 or 32 rows: worth
         // it where the launch is the larger cost (8192x2048: 7.6 -> 5.9 us per step), not on a
         // vocabulary-sized matrix (128256x3072: 39.5 -> 42.4 us)
-        const int frc = launch_gemv_b32_f32(w, x_dev, out_dev, st);
+        const int frc = launch_gemv_b32_f32(w, x_dev, out_dev, st, static_cast<int>(n_tokens));
         if (frc == CML_OK) g_runs.fetch_add(1, std::memory_order_relaxed);
         return frc;
     }

@@ -114,7 +114,7 @@ int launch_gemv_q4k(const MatArgs &a, hipStream_t st);
 int launch_gemv_q4k_f32_grouped_pair(const MatArgs &a, const cml_weight *w2, float *out2, const float *x, hipStream_t st);
 
 int launch_gemv_q4k_f32(const cml_weight *w, const float *x, float *out, hipStream_t st, int n_tokens = 1);  // quantize + matvec, one or two tokens
-int launch_gemv_b32_f32(const cml_weight *w, const float *x, float *out, hipStream_t st);  // Q8_0 / Q4_0: quantize + matvec, one token
+int launch_gemv_b32_f32(const cml_weight *w, const float *x, float *out, hipStream_t st, int n_tokens = 1);  // quantize + matvec, one or two tokens
 // Where a grouped matvec takes its activation rows from instead of MatArgs::q / scales:
 //   kind 1: ONE f32 token x, quantized inside the kernel, read by every assignment
 //   kind 2 / 3: assignment j's row is silu / gelu_tanh of x[j] times u[j] (f32 rows `stride` apart), quantized in the kernel

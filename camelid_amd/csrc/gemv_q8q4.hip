@@ -234,7 +234,7 @@ __device__ __forceinline__ void b32_row_pass(const uint8_t *qrow, const uint8_t 
 template <int FMT, int P, int NT, bool INTS, bool FUSEQ = false, int WAVES = 4, int NXQ = 0, int U = 2>
 __global__ __launch_bounds__(WAVES * 64) void gemv_b32_kernel(B32Args a) {
     constexpr int T = WAVES * 64;  // threads of a workgroup; its activation prologue is shared by WAVES * (64 / P) rows
-    static_assert(!FUSEQ || (NT == 1 && !INTS), "the fused quantizer serves single-token calls");
+    static_assert(!FUSEQ || (NT <= 2 && !INTS), "the fused quantizer serves one token, or two contiguous f32 rows");
     constexpr int RPW = kWave / P;
     extern __shared__ uint4 smem[];
     const int nb = a.nb;
@@ -270,7 +270,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_b32_kernel(B32Args a) {
         if constexpr (NXQ > 0) {
             // The token's f32 loads go out first, the row's first weight steps right behind them, and
             // the quantizer then waits for the f32 values only (a wave's loads return in order).
-            const int n4 = nb * 8;
+            const int n4 = NT * nb * 8;  // two tokens: contiguous rows, contiguous staging areas
             float4 xv[NX];
 #pragma unroll
             for (int j = 0; j < NX; j++) xv[j] = x4[min(tid + T * j, n4 - 1)];
@@ -300,7 +300,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_b32_kernel(B32Args a) {
                 }
             }
         } else {
-            b32_stage_quantized_from<FMT, T>([&](int i) { return x4[i]; }, nb, tid, ys, xss, bsum);
+            b32_stage_quantized_from<FMT, T>([&](int i) { return x4[i]; }, NT * nb, tid, ys, xss, bsum);
         }
     } else {
         const uint4 *src = reinterpret_cast<const uint4 *>(q);
@@ -435,7 +435,7 @@ static int launch_b32_p(const MatArgs &a, hipStream_t st) {
 
 // Single token, f32 activation in: quantize + matvec in one launch.
 template <int FMT, int P>
-static int launch_b32_f32_p(const cml_weight *w, const float *x, float *out, hipStream_t st) {
+static int launch_b32_f32_p(const cml_weight *w, const float *x, float *out, hipStream_t st, int n_tokens) {
     B32Args ba{};
     ba.quants = w->planes.p[0];
     ba.q_stride = w->planes.row_stride[0];
@@ -446,7 +446,8 @@ static int launch_b32_f32_p(const cml_weight *w, const float *x, float *out, hip
     ba.x = x;
     ba.out = out;
     ba.early_loads = env_int("CAMELID_HIP_B32_EARLY_LOADS", 1);
-    const size_t lds = static_cast<size_t>(ba.nb) * (32 + 4 + 4);
+    const bool two = n_tokens == 2;
+    const size_t lds = static_cast<size_t>(two ? 2 : 1) * ba.nb * (32 + 4 + 4);
     if (lds > 64 * 1024) return fail(CML_ERR_UNSUPPORTED, "activation of %d blocks exceeds the LDS staging limit", ba.nb);
     // Every workgroup quantizes the whole activation for itself; with eight waves twice the rows
     // share that prologue.  Worth it while the matrix still gives every compute unit a workgroup.
@@ -457,18 +458,32 @@ static int launch_b32_f32_p(const cml_weight *w, const float *x, float *out, hip
         // waves (16384 x 4096: 14.2 -> 12.7 us, 32000 x 4096: 24.7 -> 22.3); slower for Q4_0 and shorter rows
         if (FMT == CML_Q8_0 && ba.nb == 128 && ba.rows >= 224 * 16 * (64 / P)) waves = 16;
     }
+    if (two && waves != 4) waves = 8;  // the two-token variants: four or eight waves
     const int rows_per_wg = waves * (64 / P);
     const unsigned gx = static_cast<unsigned>((ba.rows + rows_per_wg - 1) / rows_per_wg);
     // float4 of the activation per thread: 1, 2 or 4 in registers; longer rows (or the knob) take the staged path
-    const int n4 = ba.nb * 8, threads = waves * 64;
+    const int n4 = (two ? 2 : 1) * ba.nb * 8, threads = waves * 64;
     int nxq = !ba.early_loads ? 0 : n4 <= threads ? 1 : n4 <= 2 * threads ? 2 : n4 <= 4 * threads ? 4 : 0;
-    if (waves == 8 && nxq == 4) nxq = 0;  // 2048 float4 would be 256 blocks; eight waves are launched for at most 128
+    if (waves == 8 && nxq == 4 && !two) nxq = 0;  // 2048 float4 would be 256 blocks; eight waves are launched for at most 128
     if (waves == 16 && nxq != 1) nxq = 0;
     if (waves == 2 && nxq != 0) nxq = 4;  // one register variant for the short workgroup
 #define CML_B32_FUSED(W_, N_) \
     hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, true, W_, N_>), dim3(gx, 1), dim3(W_ * 64), lds, st, ba)
-    const bool deep = nxq == 0 && b32_depth(ba.rows, P, ba.nb) == 4;
-    if (deep) {
+    const bool deep = !two && nxq == 0 && b32_depth(ba.rows, P, ba.nb) == 4;
+    if (two) {
+#define CML_B32_FUSED2(W_, N_) \
+    hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 2, false, true, W_, N_>), dim3(gx, 1), dim3(W_ * 64), lds, st, ba)
+        if (waves == 8) {
+            if (nxq == 1 || nxq == 2) CML_B32_FUSED2(8, 2);
+            else if (nxq == 4) CML_B32_FUSED2(8, 4);
+            else CML_B32_FUSED2(8, 0);
+        } else {
+            if (nxq == 1 || nxq == 2) CML_B32_FUSED2(4, 2);
+            else if (nxq == 4) CML_B32_FUSED2(4, 4);
+            else CML_B32_FUSED2(4, 0);
+        }
+#undef CML_B32_FUSED2
+    } else if (deep) {
         if (waves == 2) hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, true, 2, 0, 4>), dim3(gx, 1), dim3(128), lds, st, ba);
         else if (waves == 8) hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, true, 8, 0, 4>), dim3(gx, 1), dim3(512), lds, st, ba);
         else hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, true, 4, 0, 4>), dim3(gx, 1), dim3(256), lds, st, ba);
@@ -493,13 +508,13 @@ static int launch_b32_f32_p(const cml_weight *w, const float *x, float *out, hip
     return CML_OK;
 }
 
-int launch_gemv_b32_f32(const cml_weight *w, const float *x, float *out, hipStream_t st) {
+int launch_gemv_b32_f32(const cml_weight *w, const float *x, float *out, hipStream_t st, int n_tokens) {
     if (w->rows == 0) return CML_OK;
     const bool q8 = w->fmt == CML_Q8_0;
     int p = env_int(q8 ? "CAMELID_HIP_Q8_0_LANES" : "CAMELID_HIP_Q4_0_LANES", 0);
     if (p != 8 && p != 16) p = (w->nb <= 8) ? 8 : 16;
-    if (q8) return p == 8 ? launch_b32_f32_p<CML_Q8_0, 8>(w, x, out, st) : launch_b32_f32_p<CML_Q8_0, 16>(w, x, out, st);
-    return p == 8 ? launch_b32_f32_p<CML_Q4_0, 8>(w, x, out, st) : launch_b32_f32_p<CML_Q4_0, 16>(w, x, out, st);
+    if (q8) return p == 8 ? launch_b32_f32_p<CML_Q8_0, 8>(w, x, out, st, n_tokens) : launch_b32_f32_p<CML_Q8_0, 16>(w, x, out, st, n_tokens);
+    return p == 8 ? launch_b32_f32_p<CML_Q4_0, 8>(w, x, out, st, n_tokens) : launch_b32_f32_p<CML_Q4_0, 16>(w, x, out, st, n_tokens);
 }
 
 // ---- grouped (mixture-of-experts) dispatch ------------------------------------------------------

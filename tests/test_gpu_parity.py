@@ -397,6 +397,35 @@ def test_b32_fused_quantize_matvec_is_the_two_step_path(name, fmt, rows, cols):
             assert G.same_bits(fused, want)
 
 
+@pytest.mark.parametrize("name,fmt", [("Q8_0", oracle.Q8_0), ("Q4_0", oracle.Q4_0)])
+@pytest.mark.parametrize("rows,cols", [(190, 2048), (33, 32), (70, 3072 + 32), (5000, 1024), (16, 8192), (333, 4096), (14336, 4096)])
+def test_b32_fused_two_tokens_is_the_two_step_path(name, fmt, rows, cols):
+    """Two-token cml_matmul_f32 on Q8_0 / Q4_0 weights quantizes both rows inside the matvec
+    kernel: the bits of quantize_q8_0 + matmul and of the oracle, for every lane mapping and
+    workgroup size."""
+    rng = np.random.default_rng(7500 + rows + fmt)
+    wire = G.synth_weight(fmt, rows, cols, seed=7600 + rows + fmt)
+    w = Weight.upload(fmt, rows, cols, wire)
+    acts = _activation_cases(cols, rng)
+    acts[0, :32] = 0.0
+    acts[0, 1:7] = [2.5, 0.5, -0.5, -2.5, 1.5, -1.5]
+    acts[2, -32:] = 0.0
+    lanes_env = "CAMELID_HIP_Q8_0_LANES" if fmt == oracle.Q8_0 else "CAMELID_HIP_Q4_0_LANES"
+    for pair in ((0, 2), (2, 1)):
+        x = np.ascontiguousarray(acts[list(pair)])
+        want = oracle.matmul(fmt, wire, cols, x, order=EXACT_ORDER[fmt], threads=8)
+        for lanes in (0, 8, 16):
+            for waves in (0, 4, 8):
+                G.say(f"{name} fused two tokens {rows}x{cols} pair={pair} lanes={lanes} waves={waves}")
+                with G.env(CAMELID_HIP_B32_FUSED_WAVES=waves, **{lanes_env: lanes}):
+                    with G.env(CAMELID_HIP_FUSED_QUANT=2):
+                        fused = G.gpu_matmul_f32(w, x)
+                    with G.env(CAMELID_HIP_FUSED_QUANT=0):
+                        two_step = G.gpu_matmul_f32(w, x)
+                assert G.same_bits(fused, two_step), (pair, lanes, waves)
+                assert G.same_bits(fused, want), (pair, lanes, waves)
+
+
 # ----------------------------------------------------- errors and the seam ----
 
 def test_error_paths_return_status_codes():
