@@ -230,7 +230,9 @@ int cml_block_dots(const cml_weight *w, const int8_t *q_dev, int32_t *ints_dev, 
 /* f32 activations in, f32 out: quantize (Q8_0 or Q8_K by weight family) into
  * the caller's workspace, then gemv/gemm (reference WireQuant::matvec,
  * src/gemma4_runtime.rs:826-856).  workspace_dev needs
- * cml_matmul_workspace_bytes(fmt, cols, n_tokens) bytes. */
+ * cml_matmul_workspace_bytes(fmt, cols, n_tokens) bytes.  Calls with one or two
+ * tokens on short rows quantize inside the matvec kernel (one launch, the
+ * workspace is left untouched); the result bits do not depend on which way ran. */
 size_t cml_matmul_workspace_bytes(int fmt, int64_t cols, int64_t n_tokens);
 int cml_matmul_f32(const cml_weight *w, const float *x_dev, int64_t n_tokens, float *out_dev,
                    void *workspace_dev, size_t workspace_bytes, cml_stream_t stream);
