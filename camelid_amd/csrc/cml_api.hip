@@ -639,6 +639,14 @@ int cml_matmul_f32(const cml_weight *w, const float *x_dev, int64_t n_tokens, fl
         if (frc == CML_OK) g_runs.fetch_add(1, std::memory_order_relaxed);
         return frc;
     }
+    if (w->fmt == CML_Q6_K && (n_tokens == 1 || fuse_two) && env_int("CAMELID_HIP_Q6K_FUSED_QUANT", 1) &&
+        (fuse == 2 || (fuse == 1 && w->nb <= 16 && w->rows <= 32768))) {
+        // the same for Q6_K: 4096 x 4096 7.0 -> 5.5 us, 14336 x 4096 12.3 -> 10.8; not on a vocabulary
+        // head, whose 4008 workgroups would each quantize the row (128256 x 3072: 49.2 -> 49.6, two tokens 53.3 -> 57.2)
+        const int frc = launch_gemv_q6k_f32(w, x_dev, out_dev, st, static_cast<int>(n_tokens));
+        if (frc == CML_OK) g_runs.fetch_add(1, std::memory_order_relaxed);
+        return frc;
+    }
     if ((w->fmt == CML_Q8_0 || w->fmt == CML_Q4_0) && (n_tokens == 1 || fuse_two) &&
         (fuse == 2 || (fuse == 1 && w->cols <= 8192 && w->rows <= 32768))) {
         // the same for the 32-value block formats, whose workgroups cover only 16 or 32 rows: worth

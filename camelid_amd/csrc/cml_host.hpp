@@ -114,6 +114,7 @@ int launch_gemv_q4k(const MatArgs &a, hipStream_t st);
 int launch_gemv_q4k_f32_grouped_pair(const MatArgs &a, const cml_weight *w2, float *out2, const float *x, hipStream_t st);
 
 int launch_gemv_q4k_f32(const cml_weight *w, const float *x, float *out, hipStream_t st, int n_tokens = 1);  // quantize + matvec, one or two tokens
+int launch_gemv_q6k_f32(const cml_weight *w, const float *x, float *out, hipStream_t st, int n_tokens = 1);  // Q6_K: quantize + matvec, one or two tokens
 int launch_gemv_b32_f32(const cml_weight *w, const float *x, float *out, hipStream_t st, int n_tokens = 1);  // quantize + matvec, one or two tokens
 // Where a grouped matvec takes its activation rows from instead of MatArgs::q / scales:
 //   kind 1: ONE f32 token x, quantized inside the kernel, read by every assignment

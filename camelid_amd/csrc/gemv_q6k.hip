@@ -31,6 +31,7 @@ struct Q6KArgs {
     int rows, n_sb;
     const int8_t *q;
     const float *yd;
+    const float *x;  // fused-quantizer launches: the NT f32 activation rows, contiguous
     float *out;
     const float *residual;
     int32_t *ints;  // [rows][n_sb] or null
@@ -133,9 +134,10 @@ __device__ __forceinline__ void q6k_compute(const Q6KRegs<U> &r, int l, int sb, 
 // U = super-blocks per register buffer: 2, or 4 for weights with thousands of row tiles (an LM
 // head), where the deeper queue per wave pays (128256 x 3072: 49.3 -> 47.1 us; at 4096 x 14336 it
 // costs 1 us).
-template <int NT, bool INTS, bool GROUPED = false, int U = 2>
+template <int NT, bool INTS, bool GROUPED = false, int U = 2, bool FUSEQ = false>
 __global__ __launch_bounds__(256) void gemv_q6k_kernel(Q6KArgs a) {
     static_assert(!(GROUPED && INTS), "block-int diagnostics are for plain calls");
+    static_assert(!FUSEQ || (NT <= 2 && !INTS && !GROUPED), "the fused quantizer serves plain calls of one or two tokens");
     constexpr int LPS = 8, RPW = kWave / LPS;
     extern __shared__ uint4 smem[];
     const int n_sb = a.n_sb;
@@ -191,7 +193,43 @@ __global__ __launch_bounds__(256) void gemv_q6k_kernel(Q6KArgs a) {
             const uint4 *src = reinterpret_cast<const uint4 *>(a.q);
             uint4 *dst = reinterpret_cast<uint4 *>(ys);
             const int n16 = NT * n_sb * 16;
-            if (NT == 1 && n16 <= 4 * 256) {  // uniform
+            if constexpr (FUSEQ) {
+                // The activation arrives as f32 and every workgroup quantizes it to Q8_K itself (the
+                // arithmetic of quantize_q8_k_kernel, a 16-lane row per super-block, four per wave
+                // pass), under the first weight loads: no second launch, no trip through memory.
+                // Two tokens are simply 2 * n_sb super-blocks in a row (rows and staging areas contiguous).
+                const int tq = NT * n_sb;
+                const int qrow = lane >> 4, ql16 = lane & 15;
+                const float4 *x4 = reinterpret_cast<const float4 *>(a.x);
+                auto load_pass = [&](float4 (&xv)[4], int base) {
+                    const int sbk = min(base + qrow, tq - 1);
+#pragma unroll
+                    for (int k = 0; k < 4; k++) xv[k] = x4[sbk * 64 + ql16 * 4 + k];
+                };
+                auto quantize_pass = [&](const float4 (&xv)[4], int base) {
+                    const int sbk = base + qrow;
+                    float dv;
+                    int bs;
+                    const uint4 packed = q8k_quantize_row16(xv, lane, dv, bs);
+                    if (sbk < tq) {
+                        dst[sbk * 16 + ql16] = packed;
+                        bsum16[sbk * 16 + ql16] = bytesum16(packed);
+                        if (ql16 == 0) yds[sbk] = dv;
+                    }
+                };
+                float4 xa[4];
+                load_pass(xa, 4 * wave);
+                __builtin_amdgcn_sched_barrier(0);
+                q6k_load(ra, ql, qh, sc, dp, l, s0, s1);
+                ra_loaded = true;
+                __builtin_amdgcn_sched_barrier(0);
+                for (int base = 4 * wave;;) {
+                    quantize_pass(xa, base);
+                    base += 16;
+                    if (base >= tq) break;  // uniform per wave
+                    load_pass(xa, base);
+                }
+            } else if (NT == 1 && n16 <= 4 * 256) {  // uniform
                 // The activation loads go out first, the first weight buffer right behind them, and
                 // only then is the activation written to LDS: the weight requests are in flight
                 // while it is staged (a wave's loads return in order).
@@ -394,5 +432,36 @@ int launch_gemv_q6k(const MatArgs &a, hipStream_t st) {
 }
 
 int launch_gemm_q6k(const MatArgs &a, hipStream_t st) { return launch_gemv_q6k(a, st); }
+
+// One or two tokens, f32 activation in: quantize + matvec in one launch (plain call).
+int launch_gemv_q6k_f32(const cml_weight *w, const float *x, float *out, hipStream_t st, int n_tokens) {
+    if (w->rows == 0) return CML_OK;
+    if (n_tokens != 1 && n_tokens != 2) return fail(CML_ERR_UNSUPPORTED, "the fused Q6_K launch takes one or two tokens");
+    Q6KArgs ka{};
+    ka.ql = w->planes.p[0]; ka.ql_stride = w->planes.row_stride[0];
+    ka.qh = w->planes.p[1]; ka.qh_stride = w->planes.row_stride[1];
+    ka.sc = w->planes.p[2]; ka.sc_stride = w->planes.row_stride[2];
+    ka.d = w->planes.p[3];  ka.d_stride = w->planes.row_stride[3];
+    ka.rows = static_cast<int>(w->rows);
+    ka.n_sb = static_cast<int>(w->nb);
+    ka.x = x;
+    ka.out = out;
+    ka.n_groups = 1;
+    ka.ksplit = pick_ksplit_q6k(ka.rows, ka.n_sb);
+    ka.ksplit_log2 = ka.ksplit >= 4 ? 2 : (ka.ksplit >= 2 ? 1 : 0);
+    const int tiles_per_wg = 4 / ka.ksplit;
+    const int64_t tiles = (ka.rows + 7) / 8;
+    const unsigned gx = static_cast<unsigned>((tiles + tiles_per_wg - 1) / tiles_per_wg);
+    const size_t lds = q6k_lds_bytes(n_tokens, ka.n_sb);
+    if (lds > 64 * 1024) return fail(CML_ERR_UNSUPPORTED, "Q6_K activation of %d super-blocks exceeds the LDS staging limit", ka.n_sb);
+    if (n_tokens == 2)
+        hipLaunchKernelGGL((gemv_q6k_kernel<2, false, false, 2, true>), dim3(gx, 1), dim3(256), lds, st, ka);
+    else if (tiles >= env_int("CAMELID_HIP_Q6K_DEEP_MIN_TILES", 2048))
+        hipLaunchKernelGGL((gemv_q6k_kernel<1, false, false, 4, true>), dim3(gx, 1), dim3(256), lds, st, ka);
+    else
+        hipLaunchKernelGGL((gemv_q6k_kernel<1, false, false, 2, true>), dim3(gx, 1), dim3(256), lds, st, ka);
+    CML_HIP_TRY(hipGetLastError());
+    return CML_OK;
+}
 
 }  // namespace cml

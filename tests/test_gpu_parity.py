@@ -368,6 +368,39 @@ def test_q4k_fused_two_tokens_is_the_two_step_path(rows, cols):
         assert G.same_bits(got, want)
 
 
+@pytest.mark.parametrize("rows,cols", [(190, 3072), (61, 256), (333, 4096), (20, 14336), (2100, 1280)])
+def test_q6k_fused_quantize_matvec_is_the_two_step_path(rows, cols):
+    """One- and two-token cml_matmul_f32 on Q6_K quantizes inside the matvec kernel: the bits of
+    quantize_q8_k + matmul for every K split and buffer depth, and of the oracle."""
+    fmt = oracle.Q6_K
+    rng = np.random.default_rng(7700 + rows)
+    wire = G.synth_weight(fmt, rows, cols, seed=7750 + rows)
+    w = Weight.upload(fmt, rows, cols, wire)
+    acts = _activation_cases(cols, rng)
+    acts[0, :256] = 0.0
+    acts[0, 5], acts[0, 9] = 3.0, -3.0
+    acts[1, 17:21] = [1.5 * 3 / 127, 2.5 * 3 / 127, -0.5 * 3 / 127, 0.5 * 3 / 127]
+    acts[2, -256:] = 0.0
+    for sel in ((0,), (1,), (2, 0), (1, 2)):
+        x = np.ascontiguousarray(acts[list(sel)])
+        xin = x[0] if len(sel) == 1 else x
+        for ks in (0, 1, 2, 4):
+            if ks > cols // 256:
+                continue
+            for deep in (2048, 1):
+                G.say(f"Q6_K fused quantize+matvec {rows}x{cols} rows={sel} ksplit={ks} deep_min_tiles={deep}")
+                with G.env(CAMELID_HIP_Q6K_KSPLIT=ks, CAMELID_HIP_Q6K_DEEP_MIN_TILES=deep):
+                    with G.env(CAMELID_HIP_FUSED_QUANT=2):
+                        fused = G.gpu_matmul_f32(w, xin)
+                    with G.env(CAMELID_HIP_FUSED_QUANT=0):
+                        two_step = G.gpu_matmul_f32(w, xin)
+                assert G.same_bits(fused, two_step), (sel, ks, deep)
+        with G.env(CAMELID_HIP_EXACT_ORDER="1", CAMELID_HIP_FUSED_QUANT=2):
+            got = G.gpu_matmul_f32(w, xin)
+        want = oracle.matmul(fmt, wire, cols, x, order=EXACT_ORDER[fmt], threads=8)
+        assert G.same_bits(got.reshape(want.shape), want)
+
+
 @pytest.mark.parametrize("name,fmt", [("Q8_0", oracle.Q8_0), ("Q4_0", oracle.Q4_0)])
 @pytest.mark.parametrize("rows,cols", [(190, 2048), (33, 32), (70, 3072 + 32), (16, 14336)])
 def test_b32_fused_quantize_matvec_is_the_two_step_path(name, fmt, rows, cols):
