@@ -630,17 +630,17 @@ int cml_matmul_f32(const cml_weight *w, const float *x_dev, int64_t n_tokens, fl
     hipStream_t st = as_stream(stream);
     const int fuse = env_int("CAMELID_HIP_FUSED_QUANT", 1);  // 0 = never, 1 = by shape, 2 = whenever possible
     const bool fuse_two = n_tokens == 2 && env_int("CAMELID_HIP_FUSED_QUANT_TWO", 1) && !env_int("CAMELID_HIP_Q4K_GENERAL_ENTRY", 0);
-    if (w->fmt == CML_Q4_K && (n_tokens == 1 || fuse_two) && (fuse == 2 || (fuse == 1 && w->nb <= 16))) {
-        // decode at hidden sizes up to 4096: one launch quantizes the activation in every workgroup
-        // (one pass of its four waves; two passes for a pair of tokens) and runs the matvec; longer
-        // rows would need several quantizer passes per workgroup and measure no faster than the
-        // two launches below
+    if (w->fmt == CML_Q4_K && (n_tokens == 1 || fuse_two) && (fuse == 2 || (fuse == 1 && w->nb <= 32))) {
+        // rows of up to 8192 values: one launch quantizes the activation in every workgroup (one or
+        // two passes of its four waves; twice that for a pair of tokens) and runs the matvec
+        // (4096 x 8192: 7.1 -> 6.6 us, 2048 x 8192: 6.3 -> 4.7); at 14336 values the passes cost
+        // what the second launch does (4096 x 14336: 9.6 -> 10.0) and the two launches below stay
         const int frc = launch_gemv_q4k_f32(w, x_dev, out_dev, st, static_cast<int>(n_tokens));
         if (frc == CML_OK) g_runs.fetch_add(1, std::memory_order_relaxed);
         return frc;
     }
     if (w->fmt == CML_Q6_K && (n_tokens == 1 || fuse_two) && env_int("CAMELID_HIP_Q6K_FUSED_QUANT", 1) &&
-        (fuse == 2 || (fuse == 1 && w->nb <= 16 && w->rows <= 32768))) {
+        (fuse == 2 || (fuse == 1 && w->nb <= 32 && w->rows <= 32768))) {
         // the same for Q6_K: 4096 x 4096 7.0 -> 5.5 us, 14336 x 4096 12.3 -> 10.8; not on a vocabulary
         // head, whose 4008 workgroups would each quantize the row (128256 x 3072: 49.2 -> 49.6, two tokens 53.3 -> 57.2)
         const int frc = launch_gemv_q6k_f32(w, x_dev, out_dev, st, static_cast<int>(n_tokens));
