@@ -65,7 +65,7 @@ inline constexpr bool kB32Paired =
 #ifdef CML_Q8_0_BLOCK_PER_LANE
     false;
 #else
-    (FMT == CML_Q8_0 && P == 16);
+    (FMT == CML_Q8_0 && P >= 16);
 #endif
 
 __device__ __forceinline__ int quad_swap1_i32(int v) {  // lanes 2j <-> 2j+1
@@ -73,7 +73,8 @@ __device__ __forceinline__ int quad_swap1_i32(int v) {  // lanes 2j <-> 2j+1
 }
 
 // The block whose term lane l carries in step `s` of a paired row, and the two blocks it loads halves of.
-__device__ __forceinline__ int paired_block(int s, int l, int which) { return s * 16 + which * 8 + (l >> 1); }
+template <int P>
+__device__ __forceinline__ int paired_block(int s, int l, int which) { return s * P + which * (P / 2) + (l >> 1); }
 
 // Ordered fold for the paired mapping: terms of lanes 0, 2, .., 14 (blocks 0..7 of the step), then
 // of lanes 1, 3, .., 15 (blocks 8..15); lane 15 returns the chain.
@@ -88,6 +89,50 @@ __device__ __forceinline__ float paired_fold_ordered(float acc, float term) {
     }
 }
 
+
+// ---- rows wider than one 16-lane DPP row (P = 32 or 64 lanes per matrix row) ----
+// For matrices with few, long rows: the block terms are independent, only the chain is ordered, so
+// more lanes per row multiply the waves without touching a bit.  The chain runs through the R =
+// P / 16 DPP rows of a group one after the other: every DPP row folds its sixteen terms onto the
+// running sum (only the row whose turn it is holds the right one), and that row's last lane hands
+// the sum to the whole group.  After the last hand-over every lane of the group holds the chain.
+template <int P>
+__device__ __forceinline__ float wide_carry(float t, int rho) {
+    static_assert(P == 32 || P == 64, "lanes per row");
+    const int ti = __builtin_bit_cast(int, t);
+    if constexpr (P == 64) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_readlane(ti, 16 * rho + 15));
+    } else {
+        const int lo = __builtin_amdgcn_readlane(ti, 16 * rho + 15), hi = __builtin_amdgcn_readlane(ti, 32 + 16 * rho + 15);
+        return __builtin_bit_cast(float, (threadIdx.x & 32) ? hi : lo);
+    }
+}
+template <int P>
+__device__ __forceinline__ float wide_fold_ordered(float acc, float term) {  // lane l carries block l of the step
+#pragma unroll
+    for (int rho = 0; rho < P / 16; rho++) acc = wide_carry<P>(group_fold_ordered<16>(acc, term), rho);
+    return acc;
+}
+template <int ODD, int K = 0>
+__device__ __forceinline__ float paired_half_fold(float acc, float term) {  // lanes ODD, ODD + 2, .., ODD + 14 of a DPP row
+    if constexpr (K == 8) {
+        return acc;
+    } else {
+        constexpr int shift = 15 - (2 * K + ODD);
+        if constexpr (shift == 0) acc = acc + term;
+        else acc = acc + row_shr_f32<shift>(term);
+        return paired_half_fold<ODD, K + 1>(acc, term);
+    }
+}
+template <int P>
+__device__ __forceinline__ float wide_paired_fold_ordered(float acc, float term) {  // even lanes: blocks 0..P/2-1, odd lanes: the rest
+#pragma unroll
+    for (int rho = 0; rho < P / 16; rho++) acc = wide_carry<P>(paired_half_fold<0>(acc, term), rho);
+#pragma unroll
+    for (int rho = 0; rho < P / 16; rho++) acc = wide_carry<P>(paired_half_fold<1>(acc, term), rho);
+    return acc;
+}
+
 template <int FMT, int P, int U>
 __device__ __forceinline__ void b32_load(B32Regs<FMT, U> &r, const uint8_t *qrow, const uint8_t *srow, int l,
                                          int step, int n_steps, int nb) {
@@ -98,7 +143,7 @@ __device__ __forceinline__ void b32_load(B32Regs<FMT, U> &r, const uint8_t *qrow
     for (int u = 0; u < U; u++) {
         if constexpr (kB32Paired<FMT, P>) {
             const int s = min(step + u, n_steps - 1);
-            const int ba = min(paired_block(s, l, 0), nb - 1), bb = min(paired_block(s, l, 1), nb - 1);
+            const int ba = min(paired_block<P>(s, l, 0), nb - 1), bb = min(paired_block<P>(s, l, 1), nb - 1);
             const int half = (l & 1) * 16;
             r.qa[u] = ldg16_stream(qrow + static_cast<int64_t>(ba) * 32 + half);
             r.qb[u] = ldg16_stream(qrow + static_cast<int64_t>(bb) * 32 + half);
@@ -130,9 +175,9 @@ __device__ __forceinline__ void b32_compute(const B32Regs<FMT, U> &r, int l, int
     for (int u = 0; u < U; u++) {
         if constexpr (kB32Paired<FMT, P>) {
             const int s = min(step + u, n_steps - 1);
-            const int ba = min(paired_block(s, l, 0), nb - 1), bb = min(paired_block(s, l, 1), nb - 1);
+            const int ba = min(paired_block<P>(s, l, 0), nb - 1), bb = min(paired_block<P>(s, l, 1), nb - 1);
             const int odd = l & 1;
-            const int b_raw = paired_block(step + u, l, odd);
+            const int b_raw = paired_block<P>(step + u, l, odd);
             const bool valid = (step + u < n_steps) && (b_raw < nb);
             const int b = odd ? bb : ba;
             const float dw = f16_bits_to_f32(r.d[u]);
@@ -147,7 +192,8 @@ __device__ __forceinline__ void b32_compute(const B32Regs<FMT, U> &r, int l, int
                 const int isum = odd ? pb : pa;
                 float term = (static_cast<float>(isum) * dw) * xss[t * nb + b];
                 term = valid ? term : 0.0f;
-                acc[t] = paired_fold_ordered(acc[t], term);
+                if constexpr (P > 16) acc[t] = wide_paired_fold_ordered<P>(acc[t], term);
+                else acc[t] = paired_fold_ordered(acc[t], term);
                 if constexpr (INTS) {
                     if (ints_row != nullptr && valid) ints_row[b] = isum;
                 }
@@ -178,7 +224,8 @@ __device__ __forceinline__ void b32_compute(const B32Regs<FMT, U> &r, int l, int
             if constexpr (FMT == CML_Q4_0) isum -= 8 * bsum[t * nb + b];
             float term = (static_cast<float>(isum) * dw) * xss[t * nb + b];
             term = valid ? term : 0.0f;
-            acc[t] = group_fold_ordered<P>(acc[t], term);
+            if constexpr (P > 16) acc[t] = wide_fold_ordered<P>(acc[t], term);
+            else acc[t] = group_fold_ordered<P>(acc[t], term);
             if constexpr (INTS) {
                 if (ints_row != nullptr && valid) ints_row[b] = isum;
             }
@@ -363,6 +410,23 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_b32_kernel(B32Args a) {
     }
 }
 
+// Lanes per matrix row of a single-token matvec: 16 (8 for very short rows); 32 where 16 would
+// leave at most 1024 waves (matrices of up to 4096 rows), 64 at most 512 (up to 2048 rows of at
+// least 4096 values).  Measured over rows 1024..5632 x values 2048..14336, both formats: e.g.
+// Q8_0 2048 x 8192 9.4 / 7.8 / 7.2 us with 16 / 32 / 64 lanes, Q4_0 4096 x 4096 4.8 / 4.2 / 5.3,
+// Q4_0 5632 x 4096 4.9 / 5.9 / 6.7.
+static int b32_lanes(int fmt, int64_t rows, int64_t nb) {
+    int p = env_int(fmt == CML_Q8_0 ? "CAMELID_HIP_Q8_0_LANES" : "CAMELID_HIP_Q4_0_LANES", 0);
+    if (p == 8 || p == 16 || p == 32 || p == 64) return p;
+    p = nb <= 8 ? 8 : 16;
+    if (p == 16 && env_int("CAMELID_HIP_B32_WIDE_ROWS", 1)) {
+        const int64_t waves16 = (rows + 3) / 4;
+        if (waves16 <= 512 && nb >= 128) p = 64;
+        else if (waves16 <= 1024 && nb >= 64) p = 32;
+    }
+    return p;
+}
+
 // Steps per register buffer.  Long rows of a matrix with few of them leave one or two waves per
 // SIMD, and then the bytes each wave keeps in flight decide the rate: four steps per buffer
 // instead of two (Q4_0 4096 x 14336: 10.5 -> 9.5 us).  With more waves the deeper buffers only
@@ -459,6 +523,7 @@ static int launch_b32_f32_p(const cml_weight *w, const float *x, float *out, hip
         if (FMT == CML_Q8_0 && ba.nb == 128 && ba.rows >= 224 * 16 * (64 / P)) waves = 16;
     }
     if (two && waves != 4) waves = 8;  // the two-token variants: four or eight waves
+    if (P > 16) waves = 8;
     const int rows_per_wg = waves * (64 / P);
     const unsigned gx = static_cast<unsigned>((ba.rows + rows_per_wg - 1) / rows_per_wg);
     // float4 of the activation per thread: 1, 2 or 4 in registers; longer rows (or the knob) take the staged path
@@ -470,6 +535,14 @@ static int launch_b32_f32_p(const cml_weight *w, const float *x, float *out, hip
 #define CML_B32_FUSED(W_, N_) \
     hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, true, W_, N_>), dim3(gx, 1), dim3(W_ * 64), lds, st, ba)
     const bool deep = !two && nxq == 0 && b32_depth(ba.rows, P, ba.nb) == 4;
+    if constexpr (P > 16) {
+        // wide rows: eight-wave workgroups only (the launcher below sets them), single token
+        if (two || waves != 8) return fail(CML_ERR_UNSUPPORTED, "rows of %d lanes take one token and eight-wave workgroups", P);
+        if (deep) hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, true, 8, 0, 4>), dim3(gx, 1), dim3(512), lds, st, ba);
+        else if (nxq == 1) CML_B32_FUSED(8, 1);
+        else if (nxq == 2) CML_B32_FUSED(8, 2);
+        else CML_B32_FUSED(8, 0);
+    } else
     if (two) {
 #define CML_B32_FUSED2(W_, N_) \
     hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 2, false, true, W_, N_>), dim3(gx, 1), dim3(W_ * 64), lds, st, ba)
@@ -511,10 +584,14 @@ static int launch_b32_f32_p(const cml_weight *w, const float *x, float *out, hip
 int launch_gemv_b32_f32(const cml_weight *w, const float *x, float *out, hipStream_t st, int n_tokens) {
     if (w->rows == 0) return CML_OK;
     const bool q8 = w->fmt == CML_Q8_0;
-    int p = env_int(q8 ? "CAMELID_HIP_Q8_0_LANES" : "CAMELID_HIP_Q4_0_LANES", 0);
-    if (p != 8 && p != 16) p = (w->nb <= 8) ? 8 : 16;
-    if (q8) return p == 8 ? launch_b32_f32_p<CML_Q8_0, 8>(w, x, out, st, n_tokens) : launch_b32_f32_p<CML_Q8_0, 16>(w, x, out, st, n_tokens);
-    return p == 8 ? launch_b32_f32_p<CML_Q4_0, 8>(w, x, out, st, n_tokens) : launch_b32_f32_p<CML_Q4_0, 16>(w, x, out, st, n_tokens);
+    int p = b32_lanes(w->fmt, w->rows, w->nb);
+    if (n_tokens != 1 && p > 16) p = 16;
+    switch (p) {
+        case 8: return q8 ? launch_b32_f32_p<CML_Q8_0, 8>(w, x, out, st, n_tokens) : launch_b32_f32_p<CML_Q4_0, 8>(w, x, out, st, n_tokens);
+        case 32: return q8 ? launch_b32_f32_p<CML_Q8_0, 32>(w, x, out, st, n_tokens) : launch_b32_f32_p<CML_Q4_0, 32>(w, x, out, st, n_tokens);
+        case 64: return q8 ? launch_b32_f32_p<CML_Q8_0, 64>(w, x, out, st, n_tokens) : launch_b32_f32_p<CML_Q4_0, 64>(w, x, out, st, n_tokens);
+        default: return q8 ? launch_b32_f32_p<CML_Q8_0, 16>(w, x, out, st, n_tokens) : launch_b32_f32_p<CML_Q4_0, 16>(w, x, out, st, n_tokens);
+    }
 }
 
 // ---- grouped (mixture-of-experts) dispatch ------------------------------------------------------
@@ -734,13 +811,45 @@ int launch_gemv_b32_grouped(const MatArgs &a, const GroupedPrologue &pro, hipStr
     return p == 8 ? launch_b32_grouped_p<CML_Q4_0, 8>(a, pro, st) : launch_b32_grouped_p<CML_Q4_0, 16>(a, pro, st);
 }
 
+// One token, quantized activation in, rows of 32 or 64 lanes: eight-wave workgroups.
+template <int FMT, int P>
+static int launch_b32_wide(const MatArgs &a, hipStream_t st) {
+    const cml_weight *w = a.w;
+    B32Args ba{};
+    ba.quants = w->planes.p[0];
+    ba.q_stride = w->planes.row_stride[0];
+    ba.scales = w->planes.p[1];
+    ba.s_stride = w->planes.row_stride[1];
+    ba.rows = static_cast<int>(w->rows);
+    ba.nb = static_cast<int>(w->nb);
+    ba.residual = a.residual;
+    ba.q = a.q;
+    ba.xs = a.scales;
+    ba.out = a.out;
+    ba.early_loads = env_int("CAMELID_HIP_B32_EARLY_LOADS", 1);
+    ba.out_slot_stride = ba.rows;
+    const int rows_per_wg = 8 * (64 / P);
+    const unsigned gx = static_cast<unsigned>((ba.rows + rows_per_wg - 1) / rows_per_wg);
+    const size_t lds = static_cast<size_t>(ba.nb) * (32 + 4 + 4);
+    if (lds > 64 * 1024) return fail(CML_ERR_UNSUPPORTED, "activation of %d blocks exceeds the LDS staging limit", ba.nb);
+    if (b32_depth(ba.rows, P, ba.nb) == 4)
+        hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, false, 8, 0, 4>), dim3(gx, 1), dim3(512), lds, st, ba);
+    else
+        hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, false, 8, 0, 2>), dim3(gx, 1), dim3(512), lds, st, ba);
+    CML_HIP_TRY(hipGetLastError());
+    return CML_OK;
+}
+
 template <int FMT>
 static int launch_b32(const MatArgs &a, hipStream_t st) {
     if (a.w->rows == 0 || a.n_tokens == 0) return CML_OK;
     if (a.group_offsets) return launch_gemv_b32_grouped(a, GroupedPrologue{}, st);
-    // 16 lanes per row by default; 8 when rows are short enough that half the lanes would idle.
-    int p = env_int(FMT == CML_Q8_0 ? "CAMELID_HIP_Q8_0_LANES" : "CAMELID_HIP_Q4_0_LANES", 0);
-    if (p != 8 && p != 16) p = (a.w->nb <= 8) ? 8 : 16;
+    // 16 lanes per row by default; 8 when rows are short enough that half the lanes would idle;
+    // 32 or 64 for a single token on a matrix of few, long rows.
+    int p = b32_lanes(FMT, a.w->rows, a.w->nb);
+    if (p > 16 && (a.n_tokens != 1 || a.ints != nullptr)) p = 16;
+    if (p == 32) return launch_b32_wide<FMT, 32>(a, st);
+    if (p == 64) return launch_b32_wide<FMT, 64>(a, st);
     return p == 8 ? launch_b32_p<FMT, 8>(a, st) : launch_b32_p<FMT, 16>(a, st);
 }
 

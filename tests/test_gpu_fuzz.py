@@ -64,7 +64,7 @@ def test_block32_launch_shapes_agree(fmt):
         want = oracle.matmul(fmt, wire, cols, x, order=EXACT[fmt], threads=8)
         for waves in ("2", "4", "8", "16"):
             for depth in ("2", "4"):
-                for lanes in ("8", "16"):
+                for lanes in ("8", "16", "32", "64"):
                     G.say(f"block32 {fmt} {rows}x{cols} waves={waves} depth={depth} lanes={lanes}")
                     with G.env(CAMELID_HIP_EXACT_ORDER="1", CAMELID_HIP_B32_FUSED_WAVES=waves, CAMELID_HIP_B32_WAVES=("8" if waves == "8" else "4"), CAMELID_HIP_B32_DEPTH=depth, **{lanes_knob: lanes}):
                         assert G.same_bits(G.gpu_matmul_f32(w, x[0]), want[0]), (rows, cols, waves, depth, lanes)

@@ -417,7 +417,7 @@ def test_b32_fused_quantize_matvec_is_the_two_step_path(name, fmt, rows, cols):
     acts[1, 3] = np.nan
     lanes_env = "CAMELID_HIP_Q8_0_LANES" if fmt == oracle.Q8_0 else "CAMELID_HIP_Q4_0_LANES"
     for i, x in enumerate(acts):
-        for lanes in (0, 8, 16):
+        for lanes in (0, 8, 16, 32, 64):
             G.say(f"{name} fused quantize+matvec {rows}x{cols} act={i} lanes={lanes}")
             with G.env(**{lanes_env: lanes}):
                 with G.env(CAMELID_HIP_FUSED_QUANT=2):
