@@ -40,6 +40,7 @@
 // activation rows in LDS: the weight is streamed once per NT tokens and every
 // (row, token) cell is the NT = 1 result exactly.
 #include <algorithm>
+#include <cmath>
 
 #include "cml_device.hpp"
 #include "cml_host.hpp"
@@ -510,7 +511,16 @@ int q4k_ksplit_for(int64_t rows, int64_t n_sb) { return pick_shape(rows, n_sb).k
 static int q4k_rows_per_wave(int64_t tiles16, int ksplit, int64_t slots) {
     const int forced = env_int("CAMELID_HIP_Q4K_ROWS_PER_WAVE", 0);
     if (forced == 8 || forced == 16) return forced;
-    return tiles16 * ksplit * slots <= 1024 ? 8 : 16;
+    const int64_t waves16 = tiles16 * ksplit * slots;
+    if (waves16 <= 1024) return 8;
+    // Taller matrices: 16-row waves, unless their workgroups (four waves) fall unevenly on the 256
+    // compute units and the 8-row ones clearly less so -- 20000 x 4096 is 313 workgroups, 1.2 per
+    // unit, so some units carry two: 11.5 us against 9.9 with 625 half-size workgroups.
+    auto imbalance = [](int64_t waves) {
+        const double per_cu = static_cast<double>((waves + 3) / 4) / 256.0;
+        return std::ceil(per_cu) / per_cu;
+    };
+    return imbalance(2 * waves16) + 0.1 < imbalance(waves16) ? 8 : 16;
 }
 
 // Every K part a whole number of 4-super-block buffers and a stride of less than 2 GiB: the

@@ -8,14 +8,15 @@
 // The kernels keep exactly that association: one f32 chain per row, blocks
 // added left to right.
 //
-// Mapping.  Weights are in the plane layout (quants | f16 scales), so a lane
-// loads one whole block with aligned 128-bit loads (2 for Q8_0, 1 for Q4_0) and
-// its scale with a 16-bit load.  P lanes (16 or 8) share a row and take P
-// consecutive blocks per step; the per-block terms are then folded into the
-// row's accumulator in block order with DPP row_shr reads (the last lane of
-// the group owns the chain).  A wave covers 64/P rows; a 256-thread workgroup
-// 4 x 64/P rows.  Activations (int8 + per-block f32 scale, and for Q4_0 the
-// per-block sums that carry the -8 bias) are staged once per workgroup in LDS.
+// Mapping.  Weights are in the plane layout (quants | f16 scales).  P lanes (8, 16, 32 or 64)
+// share a row and take P consecutive blocks per step with aligned 128-bit loads -- Q4_0 one block
+// per lane, Q8_0 with P >= 16 two lanes per block (see kB32Paired), Q8_0 with 8 lanes one block per
+// lane in two loads -- and the block's scale with a 16-bit load.  The per-block terms are folded
+// into the row's accumulator in block order with DPP row_shr reads (the last lane of a 16-lane DPP
+// row owns the chain; rows of 32 / 64 lanes hand it from one DPP row to the next).  A wave covers
+// 64/P rows, a workgroup 2, 4, 8 or 16 waves.  Activations (int8 + per-block f32 scale, and for
+// Q4_0 the per-block sums that carry the -8 bias) are staged once per workgroup in LDS, or
+// quantized there from f32 by the workgroup itself (FUSEQ: one or two tokens).
 #include "cml_device.hpp"
 #include "cml_host.hpp"
 
@@ -53,20 +54,15 @@ struct B32Regs {
     uint32_t d[U];
 };
 
-// Q8_0 rows of 16 lanes ("paired" mapping): a step is 16 blocks = 512 contiguous bytes of the row,
-// and each of the two load instructions takes 256 contiguous bytes of it -- lane l the 16 bytes at
-// l*16 and at 256 + l*16 -- so every instruction consumes whole 128-byte lines exactly once (two
+// Q8_0 rows of P >= 16 lanes ("paired" mapping; written out for P = 16): a step is 16 blocks = 512
+// contiguous bytes of the row, and each of the two load instructions takes 256 contiguous bytes of
+// it -- lane l the 16 bytes at l*16 and at 256 + l*16 -- so every instruction consumes whole 128-byte lines exactly once (two
 // lanes share a block: lanes 2j, 2j+1 hold the halves of block j, then of block 8+j).  The two
 // half-block integer sums meet by one lane swap (exact integers: the order inside a block is free);
 // the even lane then carries block j's term, the odd lane block 8+j's, and the ordered fold visits
 // even lanes first.  The one-block-per-lane mapping had each instruction touch half of every line.
 template <int FMT, int P>
-inline constexpr bool kB32Paired =
-#ifdef CML_Q8_0_BLOCK_PER_LANE
-    false;
-#else
-    (FMT == CML_Q8_0 && P >= 16);
-#endif
+inline constexpr bool kB32Paired = (FMT == CML_Q8_0 && P >= 16);
 
 __device__ __forceinline__ int quad_swap1_i32(int v) {  // lanes 2j <-> 2j+1
     return __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xf, 0xf, true);
