@@ -40,12 +40,12 @@ INT8_PEAK_TOPS = 5000.0  # MI355X published dense int8 matrix-core rate
 # run, so the figures measured for the committed kernels are carried here; null where not measured.
 MEASURED_TRAFFIC_BYTES: dict = {
     # profiles/hbm_traffic_fetch_write_size.txt (copy yardstick: FETCH_SIZE x 2.000, WRITE_SIZE x 1.000)
-    "q4k_14336x4096_n1": 33371998,       # 1.008 x algorithmic
-    "q4k_14336x4096_n16": 34829086,      # 1.018 x
-    "q4k_14336x4096_n64": 39155342,      # 1.038 x
-    "q6k_128256x3072_n1": 323917431,     # 1.001 x
-    "q4_0_128256x3072_n16": 252080618,   # 1.087 x
-    "q6k_128256x3072_n16": 356182086,    # 1.074 x
+    "q4k_14336x4096_n1": 33371997,       # 1.008 x algorithmic
+    "q4k_14336x4096_n16": 34829074,      # 1.018 x
+    "q4k_14336x4096_n64": 39155356,      # 1.038 x
+    "q6k_128256x3072_n1": 323916630,     # 1.001 x
+    "q4_0_128256x3072_n16": 252016327,   # 1.087 x
+    "q6k_128256x3072_n16": 356013774,    # 1.074 x
 }
 
 # name -> (format, rows, cols, tokens): BASELINE.json's configurations.
