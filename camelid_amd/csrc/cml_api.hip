@@ -517,6 +517,12 @@ static int dispatch(const MatArgs &a, hipStream_t st) {
                 rc = launch_gemm_q4k_mfma(a, st);
             else
                 rc = launch_gemv_q4k(a, st);
+            if (rc == CML_ERR_UNSUPPORTED && !a.group_offsets && a.n_tokens > 1) {
+                // rows too long for the matrix-core kernel's LDS staging (it refuses before it
+                // launches anything): the packed-dot kernel serves them in passes of fewer tokens
+                clear_error();
+                rc = launch_gemv_q4k(a, st);
+            }
             break;
         case CML_Q8_0:
         case CML_Q4_0:
@@ -525,12 +531,20 @@ static int dispatch(const MatArgs &a, hipStream_t st) {
                 rc = launch_gemm_b32_mfma(a, st);
             else
                 rc = a.w->fmt == CML_Q8_0 ? launch_gemv_q8_0(a, st) : launch_gemv_q4_0(a, st);
+            if (rc == CML_ERR_UNSUPPORTED && !a.group_offsets && a.n_tokens > 1) {
+                clear_error();
+                rc = a.w->fmt == CML_Q8_0 ? launch_gemv_q8_0(a, st) : launch_gemv_q4_0(a, st);
+            }
             break;
         case CML_Q6_K:
             if (!a.group_offsets && !a.ints && mfma_pays(a.n_tokens, q6k_mfma_min_tokens(a.w->rows, a.w->nb), "CAMELID_HIP_Q6K_MFMA_MIN_TOKENS"))
                 rc = launch_gemm_q6k_mfma(a, st);
             else
                 rc = launch_gemv_q6k(a, st);
+            if (rc == CML_ERR_UNSUPPORTED && !a.group_offsets && a.n_tokens > 1) {
+                clear_error();
+                rc = launch_gemv_q6k(a, st);
+            }
             break;
         default: return fail(CML_ERR_INVALID, "unknown weight format %d", a.w->fmt);
     }

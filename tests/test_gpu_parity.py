@@ -645,3 +645,18 @@ def test_long_rows_in_small_batches_fit_the_staging_limit(name, fmt):
                    CAMELID_HIP_Q6K_MFMA_MIN_TOKENS=1 << 30, CAMELID_HIP_EXACT_ORDER="1"):
             got = G.gpu_gemm(w, s, q)
         check_outputs(fmt, wire, cols, s, q, got, expect_exact=True)
+
+
+@pytest.mark.parametrize("name,fmt", FMTS)
+def test_rows_too_long_for_the_matrix_core_staging_fall_back_to_the_packed_dot(name, fmt):
+    """16384-value rows with 64 tokens: where the matrix-core kernel's LDS staging does not hold the
+    batch, the call is served by the packed-dot kernel in passes of fewer tokens, not refused."""
+    rows, cols, n = 24, 16384, 64
+    wire = G.synth_weight(fmt, rows, cols, seed=950 + fmt)
+    w = Weight.upload(fmt, rows, cols, wire)
+    x = np.random.default_rng(951).standard_normal((n, cols)).astype(np.float32)
+    s, q = oracle.quantize_activation(fmt, x)
+    G.say(f"{name} {rows}x{cols} n={n} default dispatch")
+    with G.env(CAMELID_HIP_EXACT_ORDER="1"):
+        got = G.gpu_gemm(w, s, q)
+    check_outputs(fmt, wire, cols, s, q, got, expect_exact=True)
