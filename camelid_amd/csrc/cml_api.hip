@@ -23,6 +23,16 @@ static std::atomic<int> g_device{-1};
 static std::atomic<uint64_t> g_runs{0};
 static std::mutex g_mutex;
 
+// Staging area of cml_matmul_f32_static: the quantized activation rows (int8 values, then f32
+// scales) of one call.  Device memory that lives in the code object, one copy per GPU, from the
+// moment the library is loaded on that GPU until the process ends.  The name below is a host-side
+// stand-in: only the address hipGetSymbolAddress reports for the current device (kept in
+// g_static_workspace, filled by cml_init) may be handed to a kernel.
+constexpr size_t kStaticWorkspaceBytes = CML_STATIC_WORKSPACE_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticWorkspaceBytes];
+constexpr int kMaxDevices = 64;
+static void *g_static_workspace[kMaxDevices] = {};
+
 int fail(int code, const char *fmt, ...) {
     va_list ap;
     va_start(ap, fmt);
@@ -98,6 +108,12 @@ int cml_init(int device) {
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return fail(CML_ERR_UNAVAILABLE, "device %d is %s; this library carries gfx950 code only", device, prop.gcnArchName);
     CML_HIP_TRY(hipSetDevice(device));
+    if (device < kMaxDevices && g_static_workspace[device] == nullptr) {
+        // with `device` current: every GPU has its own copy of the array at its own address
+        void *p = nullptr;
+        CML_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        g_static_workspace[device] = p;
+    }
     g_device.store(device, std::memory_order_release);
     return CML_OK;
 }
@@ -674,6 +690,23 @@ int cml_matmul_f32(const cml_weight *w, const float *x_dev, int64_t n_tokens, fl
                                  : launch_quantize_q8_0(x_dev, n_tokens, w->cols, q, s, st);
     if (rc != CML_OK) return rc;
     return dispatch(plain_args(w, q, s, n_tokens, out_dev), st);
+}
+
+// The same call for hosts that may not allocate (a stream under graph capture, a serving loop with
+// a fixed memory budget): the quantized activation is staged in the library's own static device
+// array instead of a caller workspace.  Nothing here allocates or frees, on the host or the device.
+int cml_matmul_f32_static(const cml_weight *w, const float *x_dev, int64_t n_tokens, float *out_dev, cml_stream_t stream) {
+    if (!w) return fail(CML_ERR_INVALID, "null weight");
+    if (int rc = check_ready()) return rc;
+    if (n_tokens < 0) return fail(CML_ERR_SHAPE, "negative token count");
+    const int device = g_device.load(std::memory_order_acquire);
+    void *ws = device < kMaxDevices ? g_static_workspace[device] : nullptr;
+    if (!ws) return fail(CML_ERR_UNAVAILABLE, "device %d has no static workspace", device);
+    const size_t need = cml_matmul_workspace_bytes(w->fmt, w->cols, n_tokens);
+    if (need > kStaticWorkspaceBytes)
+        return fail(CML_ERR_SHAPE, "%lld tokens of %lld values need %zu bytes of staging; the static workspace holds %zu",
+                    (long long)n_tokens, (long long)w->cols, need, kStaticWorkspaceBytes);
+    return cml_matmul_f32(w, x_dev, n_tokens, out_dev, ws, kStaticWorkspaceBytes, stream);
 }
 
 // ---- host-slice seam ----------------------------------------------------------------------------------

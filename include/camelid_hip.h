@@ -237,6 +237,20 @@ size_t cml_matmul_workspace_bytes(int fmt, int64_t cols, int64_t n_tokens);
 int cml_matmul_f32(const cml_weight *w, const float *x_dev, int64_t n_tokens, float *out_dev,
                    void *workspace_dev, size_t workspace_bytes, cml_stream_t stream);
 
+/* cml_matmul_f32 without a workspace argument, for callers that cannot allocate
+ * device memory (a stream under HIP graph capture, a serving loop with a fixed
+ * memory budget, a harness that forbids hipMalloc).  It has no counterpart in
+ * the reference.  The quantized activation rows are staged in a static device
+ * array of CML_STATIC_WORKSPACE_BYTES that the library holds on every GPU it is
+ * initialised on until the process ends; the call allocates and frees nothing.
+ * A call whose staging (cml_matmul_workspace_bytes(fmt, cols, n_tokens)) exceeds
+ * that size returns CML_ERR_SHAPE.  Every call on one GPU shares the one array:
+ * calls that overlap on one GPU (two streams, two threads) race on it; calls on
+ * one stream do not.  Results are the bits of cml_matmul_f32. */
+#define CML_STATIC_WORKSPACE_BYTES (1024 * 1024 + 128 * 1024)
+int cml_matmul_f32_static(const cml_weight *w, const float *x_dev, int64_t n_tokens, float *out_dev,
+                          cml_stream_t stream);
+
 /* ---- mixture of experts (reference softmax_top_k, src/inference.rs:
  *      13940-13991; mixtral_moe_ffn, :14142-14280; routed launchers,
  *      src/cuda_resident.rs:12215-12508; moe_weighted_sum_*, :6347-6389) ---- */
