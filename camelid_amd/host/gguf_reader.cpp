@@ -203,7 +203,8 @@ GgufFile read_metadata_with_len(const std::string &path, uint64_t file_len) {
         uint64_t offset;
     };
     std::vector<Raw> raw;
-    raw.reserve(static_cast<size_t>(f.tensor_count));
+    // no reserve from the file's own count: a crafted header must fail as InvalidGguf when the
+    // entries run out, not as a length_error (the reference pushes one by one, src/gguf/reader.rs:444-470)
     for (int64_t i = 0; i < f.tensor_count; i++) {
         Raw r;
         r.name = c.string();

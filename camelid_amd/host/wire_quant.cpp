@@ -388,8 +388,28 @@ std::vector<float> WireQuant::dequantize_elements(size_t start, size_t len) cons
                            "tensor " + name_ + ": elements [" + std::to_string(start) + ", " + std::to_string(start + len) + ") leave the tensor");
     std::vector<float> out(len);
     if (len == 0) return out;
-    // decode the rows that cover the range (one block per row when the row length is still unknown)
-    const size_t in_dim = weight_ ? cols_ : values_per_block(format_);
+    if (!weight_) {
+        // The row length is not known yet (it is fixed by the first matvec) and this call must
+        // not fix it: decode from a temporary upload of just the covering blocks, seen as rows of
+        // one block, and leave the host bytes and the resident state as they are (the reference's
+        // dequantize_elements has no side effect either, src/gemma4_runtime.rs:1154).
+        const size_t bv = values_per_block(format_), bb = bytes_per_block(format_);
+        const size_t b0 = start / bv, b1 = (start + len + bv - 1) / bv;
+        ensure_device();
+        cml_weight *tmp = nullptr;
+        dev(cml_weight_upload(ggml_type_id(format_), static_cast<int64_t>(b1 - b0), static_cast<int64_t>(bv), wire_.data() + b0 * bb,
+                              (b1 - b0) * bb, &tmp),
+            "cml_weight_upload");
+        float *od = static_cast<float *>(out_.reserve((b1 - b0) * bv * sizeof(float)));
+        const int rc = cml_dequantize(tmp, od, nullptr);
+        const int rc2 = rc ? rc : cml_stream_sync(nullptr);
+        cml_weight_free(tmp);
+        dev(rc2, "cml_dequantize");
+        dev(cml_memcpy_d2h(out.data(), od + (start - b0 * bv), len * sizeof(float), nullptr), "cml_memcpy_d2h");
+        return out;
+    }
+    // decode the rows that cover the range
+    const size_t in_dim = cols_;
     const size_t r0 = start / in_dim, r1 = (start + len + in_dim - 1) / in_dim;
     const cml_weight *w = band(in_dim, r0, r1 - r0);
     float *od = static_cast<float *>(out_.reserve((r1 - r0) * in_dim * sizeof(float)));

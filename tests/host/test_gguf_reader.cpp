@@ -3,6 +3,7 @@
 // Expectations follow the reference's tests: tests/nvfp4_wire_lane_refusals.rs:60-80 (sidecar
 // file parses: v3, gemma4, three named tensors, NVFP4 first), tests/invariant_matrix_binding.rs:
 // 561-610 (type id 99 and a first dimension of 48 refuse at parse, with those messages).
+#include <cstring>
 #include <cstdint>
 #include <fstream>
 #include <vector>
@@ -196,6 +197,12 @@ int main(int argc, char **argv) {
         cut.resize(cut.size() - 40);
         write_file(tmp + "/cut.gguf", cut);
         CHECK(error_of([&] { read_metadata(tmp + "/cut.gguf"); }, BackendError::Kind::InvalidGguf).find("beyond end of file") != std::string::npos);
+        // a header that claims 2^62 tensors: refused as an invalid file when the entries run out
+        auto huge = bytes;
+        const uint64_t claimed = uint64_t(1) << 62;
+        std::memcpy(huge.data() + 8, &claimed, 8);   // magic (4) + version (4), then the tensor count
+        write_file(tmp + "/huge_count.gguf", huge);
+        error_of([&] { read_metadata(tmp + "/huge_count.gguf"); }, BackendError::Kind::InvalidGguf);
         std::vector<TensorSpec> dup = {{"w", {32}, 8, std::vector<uint8_t>(34, 0)}, {"w", {32}, 8, std::vector<uint8_t>(34, 0)}};
         write_file(tmp + "/dup.gguf", build(dup, 32));
         CHECK(error_of([&] { read_metadata(tmp + "/dup.gguf"); }, BackendError::Kind::InvalidGguf).find("duplicate tensor name") != std::string::npos);

@@ -160,6 +160,26 @@ int main(int argc, char **argv) {
             orc_dequant(c.fmt, wire.data(), ref.size() / c.block_values, ref.data());
             for (size_t i = 0; i < deq.size(); i++) CHECK(bits_of(deq[i]) == bits_of(ref[in_dim + 7 + i]));
         }
+        // ---- decode before the first matvec (an embedding lookup, then the tied output head):
+        //      decoding must not fix the row length or drop the host bytes ----
+        {
+            const size_t in_dim = 512, out_dim = 9;
+            say(std::string(c.name) + ": from_wire, dequantize_elements, then matvec with the real row length");
+            const auto wire = synth_wire(out_dim * in_dim / c.block_values, c.block_bytes, c.f16_offs);
+            const WireQuant wq = WireQuant::from_wire(c.format, wire.data(), wire.size(), in_dim * out_dim, "token_embd.weight");
+            std::vector<float> ref(in_dim * out_dim);
+            orc_dequant(c.fmt, wire.data(), ref.size() / c.block_values, ref.data());
+            const auto row3 = wq.dequantize_elements(3 * in_dim, in_dim);   // one embedding row
+            for (size_t i = 0; i < row3.size(); i++) CHECK(bits_of(row3[i]) == bits_of(ref[3 * in_dim + i]));
+            const auto odd = wq.dequantize_elements(in_dim - 5, 300);       // a range that straddles blocks and rows
+            for (size_t i = 0; i < odd.size(); i++) CHECK(bits_of(odd[i]) == bits_of(ref[in_dim - 5 + i]));
+            const auto x = activation(in_dim, 0.5f);
+            const auto got = wq.matvec(in_dim, out_dim, x.data());
+            const auto dot = oracle_rows(c, wire, in_dim, 0, out_dim, x, exact_order(c.fmt));
+            for (size_t o = 0; o < out_dim; o++) CHECK_MSG(bits_of(got[o]) == bits_of(dot[o]), "%s matvec after a decode, row %zu", c.name, o);
+            const auto again = wq.dequantize_elements(3 * in_dim, in_dim);  // and from the resident weight afterwards
+            for (size_t i = 0; i < again.size(); i++) CHECK(bits_of(again[i]) == bits_of(ref[3 * in_dim + i]));
+        }
         // ---- batched == single, row band == rows of the full matvec (reference :22626-22677) ----
         {
             const size_t in_dim = 256, out_dim = 6;
