@@ -9,10 +9,14 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <algorithm>
 #include <atomic>
 #include <mutex>
-#include <vector>
+#include <new>
+#include <string>
 #include <unordered_map>
+#include <utility>
+#include <vector>
 
 #include "cml_host.hpp"
 
@@ -45,10 +49,41 @@ void clear_error() { g_error[0] = '\0'; }
 
 bool ready() { return g_device.load(std::memory_order_acquire) >= 0; }
 
+// Tuning knobs (CAMELID_HIP_*) are read from the environment ONCE, into a snapshot taken by
+// cml_init and again by cml_reload_env (reference: every CAMELID_* knob sits in a OnceLock,
+// src/inference.rs:23679-23692).  A launch only walks the snapshot -- normally empty -- and never
+// calls getenv, so it neither pays for it nor races with a setenv in another thread.
+struct EnvSnapshot {
+    std::vector<std::pair<std::string, int>> knobs;  // names without the CAMELID_HIP_ prefix
+};
+static std::atomic<const EnvSnapshot *> g_env{nullptr};
+extern "C" char **environ;
+
+static void load_env_snapshot() {
+    auto *snap = new EnvSnapshot();
+    static const char prefix[] = "CAMELID_HIP_";
+    for (char **e = environ; e && *e; e++) {
+        if (strncmp(*e, prefix, sizeof(prefix) - 1) != 0) continue;
+        const char *eq = strchr(*e, '=');
+        if (!eq || !eq[1]) continue;  // unset or empty: the default applies
+        snap->knobs.emplace_back(std::string(static_cast<const char *>(*e) + sizeof(prefix) - 1, eq), atoi(eq + 1));
+    }
+    // superseded snapshots are kept: a launch on another thread may still be reading one, and
+    // reloads only happen in tests
+    g_env.store(snap, std::memory_order_release);
+}
+
 int env_int(const char *name, int dflt) {
-    const char *v = getenv(name);
-    if (!v || !*v) return dflt;
-    return atoi(v);
+    const EnvSnapshot *snap = g_env.load(std::memory_order_acquire);
+    if (!snap) {  // before cml_init (library gating only)
+        const char *v = getenv(name);
+        return (!v || !*v) ? dflt : atoi(v);
+    }
+    if (snap->knobs.empty()) return dflt;
+    const char *key = name + 12;  // every knob name starts with CAMELID_HIP_
+    for (const auto &kv : snap->knobs)
+        if (kv.first == key) return kv.second;
+    return dflt;
 }
 
 // Environment masking is checked before any driver call (reference
@@ -73,6 +108,57 @@ static int check_ready() {
 
 using namespace cml;
 
+// Nothing may unwind through the C boundary: an entry point whose body can allocate host memory
+// (containers, std::string) runs it inside this guard and reports an allocation failure as a status.
+#define CML_NOTHROW_BEGIN try {
+#define CML_NOTHROW_END                                                        \
+    }                                                                          \
+    catch (const std::bad_alloc &) {                                           \
+        return fail(CML_ERR_OOM, "host allocation failed");                    \
+    }                                                                          \
+    catch (...) {                                                              \
+        return fail(CML_ERR_INVALID, "unexpected C++ exception at the C boundary"); \
+    }
+
+// Read-only yardstick: every lane keeps `in_flight` 16-byte non-temporal loads out over a grid-stride
+// walk of the buffer and stores nothing (what a launch that only reads can reach on this chip).
+template <int INFL>
+__global__ void __launch_bounds__(256) read_kernel(const uint4 *__restrict__ src, size_t n16, uint32_t *sink) {
+    typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+    const v4u *p = reinterpret_cast<const v4u *>(src);
+    const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+    size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    v4u acc = {0, 0, 0, 0};
+    for (; i + (INFL - 1) * stride < n16; i += INFL * stride) {
+        v4u v[INFL];
+#pragma unroll
+        for (int k = 0; k < INFL; k++) v[k] = __builtin_nontemporal_load(p + i + k * stride);
+#pragma unroll
+        for (int k = 0; k < INFL; k++) acc ^= v[k];
+    }
+    for (; i < n16; i += stride) acc ^= __builtin_nontemporal_load(p + i);
+    if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x12345679u && sink) sink[0] = 1;  // keeps the loads alive
+}
+
+namespace {
+struct CacheKey {
+    const void *ptr;
+    size_t len;
+    int fmt;
+    bool operator==(const CacheKey &o) const { return ptr == o.ptr && len == o.len && fmt == o.fmt; }
+};
+struct CacheHash {
+    size_t operator()(const CacheKey &k) const {
+        return std::hash<const void *>()(k.ptr) ^ (std::hash<size_t>()(k.len) * 1315423911u) ^ static_cast<size_t>(k.fmt);
+    }
+};
+// State of the host-slice seam, all under g_mutex: weights cached on the device by (pointer,
+// length, format) and one grow-only device buffer for the activations and outputs of a call.
+std::unordered_map<CacheKey, cml_weight *, CacheHash> g_weight_cache;
+uint8_t *g_seam_buf = nullptr;
+size_t g_seam_bytes = 0;
+}  // namespace
+
 extern "C" {
 
 int cml_block_values(int fmt) { return geometry(fmt).block_values; }
@@ -96,6 +182,9 @@ int cml_init(int device) {
     clear_error();
     if (masked_by_env()) return fail(CML_ERR_UNAVAILABLE, "GPU use is masked by the environment");
     std::lock_guard<std::mutex> lock(g_mutex);
+    CML_NOTHROW_BEGIN
+    if (!g_env.load(std::memory_order_acquire)) load_env_snapshot();
+    CML_NOTHROW_END
     int n = 0;
     if (hipGetDeviceCount(&n) != hipSuccess || n <= 0) {
         (void)hipGetLastError();
@@ -120,7 +209,23 @@ int cml_init(int device) {
 
 void cml_shutdown(void) {
     std::lock_guard<std::mutex> lock(g_mutex);
+    if (ready()) {
+        // what the library itself owns on the device: the seam's cached weights and its staging buffer
+        for (auto &kv : g_weight_cache) cml_weight_free(kv.second);
+        g_weight_cache.clear();
+        if (g_seam_buf) (void)hipFree(g_seam_buf);
+        g_seam_buf = nullptr;
+        g_seam_bytes = 0;
+    }
     g_device.store(-1, std::memory_order_release);
+}
+
+int cml_reload_env(void) {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    CML_NOTHROW_BEGIN
+    load_env_snapshot();
+    CML_NOTHROW_END
+    return CML_OK;
 }
 
 const char *cml_last_error(void) { return g_error; }
@@ -138,8 +243,7 @@ int cml_dev_alloc(size_t nbytes, void **out_dev) {
 }
 
 int cml_dev_free(void *ptr_dev) {
-    if (!ptr_dev) return CML_OK;
-    if (int rc = check_ready()) return rc;
+    if (!ptr_dev) return CML_OK;  // also after cml_shutdown: the caller's buffers outlive it
     CML_HIP_TRY(hipFree(ptr_dev));
     return CML_OK;
 }
@@ -187,6 +291,33 @@ int cml_copy_dev(void *dst_dev, const void *src_dev, size_t nbytes, cml_stream_t
     hipLaunchKernelGGL(copy_kernel, dim3(blocks), dim3(256), 0, as_stream(stream), (uint4 *)dst_dev, (const uint4 *)src_dev, n16);
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
+}
+
+int cml_calibrate_read(const void *src_dev, size_t nbytes, int in_flight, int workgroups, cml_stream_t stream) {
+    if (int rc = check_ready()) return rc;
+    if (nbytes == 0) return CML_OK;
+    if (!src_dev) return fail(CML_ERR_INVALID, "null pointer");
+    if ((nbytes | reinterpret_cast<uintptr_t>(src_dev)) & 15) return fail(CML_ERR_INVALID, "cml_calibrate_read needs a 16-byte aligned pointer and size");
+    const size_t n16 = nbytes / 16;
+    if (workgroups <= 0) workgroups = 2048;
+    const dim3 grid(static_cast<unsigned>(std::min<size_t>((n16 + 255) / 256, static_cast<size_t>(workgroups)))), block(256);
+    const uint4 *src = static_cast<const uint4 *>(src_dev);
+    switch (in_flight) {
+        case 1: hipLaunchKernelGGL(read_kernel<1>, grid, block, 0, as_stream(stream), src, n16, nullptr); break;
+        case 2: hipLaunchKernelGGL(read_kernel<2>, grid, block, 0, as_stream(stream), src, n16, nullptr); break;
+        case 8: hipLaunchKernelGGL(read_kernel<8>, grid, block, 0, as_stream(stream), src, n16, nullptr); break;
+        case 4: hipLaunchKernelGGL(read_kernel<4>, grid, block, 0, as_stream(stream), src, n16, nullptr); break;
+        default: return fail(CML_ERR_INVALID, "in_flight must be 1, 2, 4 or 8");
+    }
+    CML_HIP_TRY(hipGetLastError());
+    return CML_OK;
+}
+
+int cml_calibrate_weight_loads(const cml_weight *w, void *scratch_dev, cml_stream_t stream) {
+    if (!w) return fail(CML_ERR_INVALID, "null weight");
+    if (int rc = check_ready()) return rc;
+    if (w->fmt != CML_Q4_K) return fail(CML_ERR_UNSUPPORTED, "the loads-only twin exists for the Q4_K matvec");
+    return launch_gemv_q4k_loads_only(w, static_cast<float *>(scratch_dev), as_stream(stream));
 }
 
 int cml_stream_sync(cml_stream_t stream) {
@@ -527,9 +658,11 @@ static int dispatch(const MatArgs &a, hipStream_t st) {
     switch (a.w->fmt) {
         case CML_Q4_K:
             // int8 matrix cores for the batched shapes (speculative-verify / prefill); packed dot below.
+            // (A residual only comes with single-token calls; the matrix-core kernels do not add one,
+            // so such a call stays on the packed-dot kernel whatever the thresholds say.)
             // Measured on MI355X at 14336x4096: the matrix-core kernel takes 12 us for any batch up to
             // 16 tokens, the packed-dot kernel 7.2 / 9.9 us for 1 / 2 tokens and two launches for 3.
-            if (!a.group_offsets && !a.ints && a.n_tokens >= env_int("CAMELID_HIP_Q4K_MFMA_MIN_TOKENS", 3))
+            if (!a.group_offsets && !a.ints && !a.residual && a.n_tokens >= env_int("CAMELID_HIP_Q4K_MFMA_MIN_TOKENS", 3))
                 rc = launch_gemm_q4k_mfma(a, st);
             else
                 rc = launch_gemv_q4k(a, st);
@@ -543,7 +676,7 @@ static int dispatch(const MatArgs &a, hipStream_t st) {
         case CML_Q8_0:
         case CML_Q4_0:
             // the same split for the 32-value-block formats (rows of whole 256-value slabs)
-            if (!a.group_offsets && !a.ints && mfma_pays(a.n_tokens, b32_mfma_min_tokens(a.w->rows), "CAMELID_HIP_B32_MFMA_MIN_TOKENS") && b32_mfma_usable(a.w))
+            if (!a.group_offsets && !a.ints && !a.residual && mfma_pays(a.n_tokens, b32_mfma_min_tokens(a.w->rows), "CAMELID_HIP_B32_MFMA_MIN_TOKENS") && b32_mfma_usable(a.w))
                 rc = launch_gemm_b32_mfma(a, st);
             else
                 rc = a.w->fmt == CML_Q8_0 ? launch_gemv_q8_0(a, st) : launch_gemv_q4_0(a, st);
@@ -553,7 +686,8 @@ static int dispatch(const MatArgs &a, hipStream_t st) {
             }
             break;
         case CML_Q6_K:
-            if (!a.group_offsets && !a.ints && mfma_pays(a.n_tokens, q6k_mfma_min_tokens(a.w->rows, a.w->nb), "CAMELID_HIP_Q6K_MFMA_MIN_TOKENS"))
+            if (!a.group_offsets && !a.ints && !a.residual && !q6k_lane_order() &&
+                mfma_pays(a.n_tokens, q6k_mfma_min_tokens(a.w->rows, a.w->nb), "CAMELID_HIP_Q6K_MFMA_MIN_TOKENS"))
                 rc = launch_gemm_q6k_mfma(a, st);
             else
                 rc = launch_gemv_q6k(a, st);
@@ -669,7 +803,7 @@ int cml_matmul_f32(const cml_weight *w, const float *x_dev, int64_t n_tokens, fl
         if (frc == CML_OK) g_runs.fetch_add(1, std::memory_order_relaxed);
         return frc;
     }
-    if (w->fmt == CML_Q6_K && (n_tokens == 1 || fuse_two) && env_int("CAMELID_HIP_Q6K_FUSED_QUANT", 1) &&
+    if (w->fmt == CML_Q6_K && (n_tokens == 1 || fuse_two) && env_int("CAMELID_HIP_Q6K_FUSED_QUANT", 1) && !q6k_lane_order() &&
         (fuse == 2 || (fuse == 1 && w->nb <= 32 && w->rows <= 32768))) {
         // the same for Q6_K: 4096 x 4096 7.0 -> 5.5 us, 14336 x 4096 12.3 -> 10.8; not on a vocabulary
         // head, whose 4008 workgroups would each quantize the row (128256 x 3072: 49.2 -> 49.6, two tokens 53.3 -> 57.2)
@@ -711,21 +845,6 @@ int cml_matmul_f32_static(const cml_weight *w, const float *x_dev, int64_t n_tok
 
 // ---- host-slice seam ----------------------------------------------------------------------------------
 
-namespace {
-struct CacheKey {
-    const void *ptr;
-    size_t len;
-    int fmt;
-    bool operator==(const CacheKey &o) const { return ptr == o.ptr && len == o.len && fmt == o.fmt; }
-};
-struct CacheHash {
-    size_t operator()(const CacheKey &k) const {
-        return std::hash<const void *>()(k.ptr) ^ (std::hash<size_t>()(k.len) * 1315423911u) ^ static_cast<size_t>(k.fmt);
-    }
-};
-std::unordered_map<CacheKey, cml_weight *, CacheHash> g_weight_cache;
-}  // namespace
-
 // Activations down, one dispatch, outputs up; synchronous.  g_mutex is held by the caller.
 static int run_host_seam(const cml_weight *w, const float *input_scales, const int8_t *input_quants, int64_t input_rows, float *output) {
     const int64_t per = is_k_family(w->fmt) ? 256 : 32;
@@ -733,22 +852,25 @@ static int run_host_seam(const cml_weight *w, const float *input_scales, const i
     const size_t sb = static_cast<size_t>(input_rows) * (w->cols / per) * sizeof(float);
     const size_t ob = static_cast<size_t>(input_rows) * w->rows * sizeof(float);
     const size_t q_off = 0, s_off = (qb + 255) & ~size_t(255), o_off = s_off + ((sb + 255) & ~size_t(255));
-    uint8_t *buf = nullptr;
-    CML_HIP_TRY(hipMalloc(reinterpret_cast<void **>(&buf), o_off + ob));
-    int rc = CML_OK;
-    hipError_t e = hipMemcpy(buf + q_off, input_quants, qb, hipMemcpyHostToDevice);
-    if (e == hipSuccess) e = hipMemcpy(buf + s_off, input_scales, sb, hipMemcpyHostToDevice);
-    if (e != hipSuccess) rc = fail(CML_ERR_HIP, "hipMemcpy failed: %s", hipGetErrorString(e));
-    if (rc == CML_OK)
-        rc = dispatch(plain_args(w, reinterpret_cast<int8_t *>(buf + q_off), reinterpret_cast<float *>(buf + s_off),
-                                 input_rows, reinterpret_cast<float *>(buf + o_off)),
-                      nullptr);
-    if (rc == CML_OK) {
-        e = hipMemcpy(output, buf + o_off, ob, hipMemcpyDeviceToHost);  // synchronises the null stream
-        if (e != hipSuccess) rc = fail(CML_ERR_HIP, "device run failed: %s", hipGetErrorString(e));
+    if (o_off + ob > g_seam_bytes) {  // grow-only: a decode loop allocates on its first call, then never again
+        if (g_seam_buf) (void)hipFree(g_seam_buf);
+        g_seam_buf = nullptr;
+        g_seam_bytes = 0;
+        const size_t want = ((o_off + ob) * 5 / 4 + 4095) & ~size_t(4095);
+        CML_HIP_TRY(hipMalloc(reinterpret_cast<void **>(&g_seam_buf), want));
+        g_seam_bytes = want;
     }
-    (void)hipFree(buf);
-    return rc;
+    uint8_t *buf = g_seam_buf;
+    hipError_t e = hipMemcpyAsync(buf + q_off, input_quants, qb, hipMemcpyHostToDevice, nullptr);
+    if (e == hipSuccess) e = hipMemcpyAsync(buf + s_off, input_scales, sb, hipMemcpyHostToDevice, nullptr);
+    if (e != hipSuccess) return fail(CML_ERR_HIP, "hipMemcpy failed: %s", hipGetErrorString(e));
+    if (int rc = dispatch(plain_args(w, reinterpret_cast<int8_t *>(buf + q_off), reinterpret_cast<float *>(buf + s_off),
+                                     input_rows, reinterpret_cast<float *>(buf + o_off)),
+                          nullptr))
+        return rc;
+    e = hipMemcpy(output, buf + o_off, ob, hipMemcpyDeviceToHost);  // synchronises the null stream
+    if (e != hipSuccess) return fail(CML_ERR_HIP, "device run failed: %s", hipGetErrorString(e));
+    return CML_OK;
 }
 
 int cml_try_linear_rows(int fmt, const float *input_scales, const int8_t *input_quants, const uint8_t *weight_wire,
@@ -763,14 +885,21 @@ int cml_try_linear_rows(int fmt, const float *input_scales, const int8_t *input_
     std::lock_guard<std::mutex> lock(g_mutex);
     cml_weight *w = nullptr;
     const CacheKey key{weight_wire, weight_nbytes, fmt};
+    CML_NOTHROW_BEGIN
     auto it = g_weight_cache.find(key);
     if (it != g_weight_cache.end()) {
         w = it->second;
         if (w->rows != weight_rows || w->cols != cols) return fail(CML_ERR_SHAPE, "cached weight has another shape");
     } else {
         if (int rc = cml_weight_upload(fmt, weight_rows, cols, weight_wire, weight_nbytes, &w)) return rc;
-        g_weight_cache.emplace(key, w);
+        try {
+            g_weight_cache.emplace(key, w);
+        } catch (...) {
+            cml_weight_free(w);
+            throw;
+        }
     }
+    CML_NOTHROW_END
     return run_host_seam(w, input_scales, input_quants, input_rows, output);
 }
 
@@ -786,6 +915,7 @@ int cml_try_q8_0_block_linear_row(const float *input_scales, const int8_t *input
     std::lock_guard<std::mutex> lock(g_mutex);
     cml_weight *w = nullptr;
     const CacheKey key{weight_block_bytes, weight_nbytes, -36};  // the in-memory block layout, not a wire format
+    CML_NOTHROW_BEGIN
     auto it = g_weight_cache.find(key);
     if (it != g_weight_cache.end()) {
         w = it->second;
@@ -795,8 +925,14 @@ int cml_try_q8_0_block_linear_row(const float *input_scales, const int8_t *input
         if (!q8_0_blocks_to_wire(weight_block_bytes, n_blocks, wire.data()))
             return fail(CML_ERR_UNSUPPORTED, "a block scale is not an f16 value: these blocks did not come from Q8_0 wire bytes");
         if (int rc = cml_weight_upload(CML_Q8_0, rows, blocks_per_row * 32, wire.data(), wire.size(), &w)) return rc;
-        g_weight_cache.emplace(key, w);
+        try {
+            g_weight_cache.emplace(key, w);
+        } catch (...) {
+            cml_weight_free(w);
+            throw;
+        }
     }
+    CML_NOTHROW_END
     return run_host_seam(w, input_scales, input_quants, 1, output);
 }
 

@@ -54,6 +54,7 @@ struct cml_weight {
     size_t allocation_bytes;
 };
 
+
 namespace cml {
 
 // Plane sizes for `rows` rows; returns the number of planes.
@@ -114,6 +115,7 @@ int launch_gemv_q4k(const MatArgs &a, hipStream_t st);
 int launch_gemv_q4k_f32_grouped_pair(const MatArgs &a, const cml_weight *w2, float *out2, const float *x, hipStream_t st);
 
 int launch_gemv_q4k_f32(const cml_weight *w, const float *x, float *out, hipStream_t st, int n_tokens = 1);  // quantize + matvec, one or two tokens
+int launch_gemv_q4k_loads_only(const cml_weight *w, float *out, hipStream_t st);  // calibration: the single-token launch's loads alone
 int launch_gemv_q6k_f32(const cml_weight *w, const float *x, float *out, hipStream_t st, int n_tokens = 1);  // Q6_K: quantize + matvec, one or two tokens
 int launch_gemv_b32_f32(const cml_weight *w, const float *x, float *out, hipStream_t st, int n_tokens = 1);  // quantize + matvec, one or two tokens
 // Where a grouped matvec takes its activation rows from instead of MatArgs::q / scales:
@@ -141,6 +143,7 @@ int launch_gemm_q4_0(const MatArgs &a, hipStream_t st);
 int launch_gemm_q6k(const MatArgs &a, hipStream_t st);
 int launch_gemm_q6k_mfma(const MatArgs &a, hipStream_t st);  // Q6_K on the matrix cores; plain or grouped
 int q6k_mfma_min_tokens(int64_t rows, int64_t n_sb);         // batch size from which it pays
+bool q6k_lane_order();                                       // CAMELID_HIP_Q6K_LANE_ORDER: the reference CPU lanes' 8-lane order, bit for bit
 
 // Integer tuning knob read once from the environment (0 when unset).
 int env_int(const char *name, int dflt);

@@ -25,6 +25,13 @@
 
 namespace cml {
 
+// LDS written by some lanes of a wave and read by others of the same wave.
+__device__ __forceinline__ void wave_barrier_lds() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 struct Q6KArgs {
     const uint8_t *ql, *qh, *sc, *d;
     int64_t ql_stride, qh_stride, sc_stride, d_stride;
@@ -372,10 +379,109 @@ static int launch_q6k_nt(const Q6KArgs &ka, int n_bands, bool ints, bool grouped
     return CML_OK;
 }
 
+// ---- the 8-lane order of the reference CPU lanes, bit for bit ------------------------------------
+//
+// q6_k_wire_row_dot (src/inference.rs:25535-25581, the Q6_K row dot both CPU lanes call) keeps
+// eight integer lanes per super-block, lane l taking the values whose index is l modulo 8
+// (aux32[l] += sc_j * y * a over j < 16 and both 8-value halves of group j), and eight f32 lane
+// sums  sums[l] += (d_w * yd) * (float)aux32[l]  over the super-blocks in order, folded left to
+// right at the end.  A 4-wide packed dot cannot keep those lanes apart, so the kernels above match
+// this order to 1e-5 only.  This kernel reproduces it exactly and is selected by
+// CAMELID_HIP_Q6K_LANE_ORDER=1 for every plain Q6_K call (one launch per token batch; speed is
+// secondary here: byte loads, one wave per row).  Lane = 8 * g + l: eight super-blocks g in
+// flight per pass, their integers independent; the f32 sums are then advanced in super-block
+// order by the lanes of g = 0 through LDS.
+__global__ __launch_bounds__(256) void gemv_q6k_lanes_kernel(Q6KArgs a, int64_t cols) {
+    extern __shared__ uint4 smem[];
+    int8_t *ys = reinterpret_cast<int8_t *>(smem);                              // [n_sb*256]
+    float *yds = reinterpret_cast<float *>(ys + a.n_sb * 256);                  // [n_sb]
+    float *xch = yds + ((a.n_sb + 3) & ~3);                                     // [4 waves][64]
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int token = blockIdx.y;
+    const int8_t *q = a.q + static_cast<int64_t>(token) * cols;
+    for (int i = tid; i < a.n_sb * 16; i += 256) reinterpret_cast<uint4 *>(ys)[i] = reinterpret_cast<const uint4 *>(q)[i];
+    for (int i = tid; i < a.n_sb; i += 256) yds[i] = a.yd[static_cast<int64_t>(token) * a.n_sb + i];
+    __syncthreads();
+    const int row = blockIdx.x * 4 + wave;
+    if (row >= a.rows) return;  // whole waves leave; no barrier follows
+    const int g = lane >> 3, l = lane & 7;
+    const uint8_t *ql = a.ql + static_cast<int64_t>(row) * a.ql_stride;
+    const uint8_t *qh = a.qh + static_cast<int64_t>(row) * a.qh_stride;
+    const int8_t *sc = reinterpret_cast<const int8_t *>(a.sc + static_cast<int64_t>(row) * a.sc_stride);
+    const uint8_t *dw = a.d + static_cast<int64_t>(row) * a.d_stride;
+    float *mine = xch + wave * 64;
+    float sum_l = 0.0f;  // lanes of g == 0: sums[l]
+    for (int sb0 = 0; sb0 < a.n_sb; sb0 += 8) {
+        const int sb = sb0 + g;
+        float term = 0.0f;
+        if (sb < a.n_sb) {
+            int aux = 0;
+#pragma unroll
+            for (int hh = 0; hh < 2; hh++) {
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    const int ll = l + 8 * k;  // position inside the 32-value region
+                    const int lo_b = ql[sb * 128 + 64 * hh + ll], hi_b = ql[sb * 128 + 64 * hh + 32 + ll], hb = qh[sb * 64 + 32 * hh + ll];
+                    const int code[4] = {(lo_b & 15) | ((hb & 3) << 4), (hi_b & 15) | (((hb >> 2) & 3) << 4),
+                                         (lo_b >> 4) | (((hb >> 4) & 3) << 4), (hi_b >> 4) | (((hb >> 6) & 3) << 4)};
+#pragma unroll
+                    for (int region = 0; region < 4; region++) {
+                        const int v = 128 * hh + 32 * region + ll;
+                        const int scale = sc[sb * 16 + (v >> 4)];
+                        aux += scale * (static_cast<int>(ys[sb * 256 + v]) * (code[region] - 32));
+                    }
+                }
+            }
+            const float dd = f16_bits_to_f32(ldg2(dw + sb * 2)) * yds[sb];
+            term = dd * static_cast<float>(aux);
+        }
+        mine[lane] = term;
+        wave_barrier_lds();
+        if (g == 0) {
+            const int n = min(8, a.n_sb - sb0);
+            for (int k = 0; k < n; k++) sum_l = sum_l + mine[8 * k + l];
+        }
+        wave_barrier_lds();
+    }
+    if (g == 0) mine[l] = sum_l;
+    wave_barrier_lds();
+    if (lane == 0) {
+        float total = 0.0f;
+        for (int k = 0; k < 8; k++) total = total + mine[k];
+        if (a.residual) total = total + a.residual[row];
+        a.out[static_cast<int64_t>(token) * a.rows + row] = total;
+    }
+}
+
+static int launch_gemv_q6k_lanes(const MatArgs &a, hipStream_t st) {
+    const cml_weight *w = a.w;
+    Q6KArgs ka{};
+    ka.ql = w->planes.p[0]; ka.ql_stride = w->planes.row_stride[0];
+    ka.qh = w->planes.p[1]; ka.qh_stride = w->planes.row_stride[1];
+    ka.sc = w->planes.p[2]; ka.sc_stride = w->planes.row_stride[2];
+    ka.d = w->planes.p[3];  ka.d_stride = w->planes.row_stride[3];
+    ka.rows = static_cast<int>(w->rows);
+    ka.n_sb = static_cast<int>(w->nb);
+    ka.q = a.q;
+    ka.yd = a.scales;
+    ka.out = a.out;
+    ka.residual = a.residual;
+    const size_t lds = static_cast<size_t>(ka.n_sb) * 256 + ((static_cast<size_t>(ka.n_sb) + 3) & ~size_t(3)) * 4 + 4 * 64 * 4;
+    if (lds > 64 * 1024) return fail(CML_ERR_UNSUPPORTED, "Q6_K activation of %d super-blocks exceeds the LDS staging limit", ka.n_sb);
+    if (a.n_tokens > 65535) return fail(CML_ERR_UNSUPPORTED, "at most 65535 tokens per call in the lane-order mode");
+    hipLaunchKernelGGL(gemv_q6k_lanes_kernel, dim3(static_cast<unsigned>((ka.rows + 3) / 4), static_cast<unsigned>(a.n_tokens)), dim3(256), lds, st,
+                       ka, static_cast<int64_t>(w->cols));
+    CML_HIP_TRY(hipGetLastError());
+    return CML_OK;
+}
+
+bool q6k_lane_order() { return env_int("CAMELID_HIP_Q6K_LANE_ORDER", 0) != 0; }
+
 int launch_gemv_q6k(const MatArgs &a, hipStream_t st) {
     const cml_weight *w = a.w;
     if (w->rows == 0 || a.n_tokens == 0) return CML_OK;
     const bool grouped = a.group_offsets != nullptr || a.group_ids != nullptr;
+    if (!grouped && !a.ints && q6k_lane_order()) return launch_gemv_q6k_lanes(a, st);
     Q6KArgs ka{};
     ka.ql = w->planes.p[0]; ka.ql_stride = w->planes.row_stride[0];
     ka.qh = w->planes.p[1]; ka.qh_stride = w->planes.row_stride[1];

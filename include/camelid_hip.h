@@ -24,7 +24,18 @@
  *   - all pointers named *_dev are device addresses on the initialised GPU;
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream);
  *     calls only enqueue work, except where a host pointer is read or written;
- *   - one GPU; no collectives.
+ *   - one GPU; no collectives;
+ *   - threads: the host-slice seam (cml_try_*) serialises its callers on one
+ *     process-wide lock, as the reference's backend does (src/cuda.rs:691-699).
+ *     The resident entry points (quantize / gemv / gemm / matmul / moe / producers)
+ *     take no lock: they only enqueue kernels on the caller's stream and keep no
+ *     shared mutable state (cml_matmul_f32_static excepted, see there), so any
+ *     number of threads may call them, each on its own stream, on weights that
+ *     nobody frees meanwhile.  cml_init / cml_shutdown / cml_reload_env must not
+ *     run concurrently with anything else;
+ *   - tuning knobs (environment variables named CAMELID_HIP_*) are read once, by
+ *     cml_init, the way the reference reads its CAMELID_* knobs once per process
+ *     (src/inference.rs:23679-23692); cml_reload_env() reads them again.
  *
  * Tensor conventions (reference src/tensor/mod.rs:79-89, src/inference.rs:
  * 23728-23749): a weight is `rows` output rows of `cols` contraction values,
@@ -72,7 +83,13 @@ typedef void *cml_graph_t;            /* an instantiated hipGraphExec_t */
 int cml_available(void);
 /* Select the device (CAMELID_HIP_DEVICE overrides when device < 0). Idempotent. */
 int cml_init(int device);
+/* Frees what the library itself holds on the device (the seam's weight cache and
+ * staging buffer); handles and buffers the caller created stay the caller's to
+ * free, before or after (cml_weight_free, cml_dev_free). */
 void cml_shutdown(void);
+/* Takes a new snapshot of the CAMELID_HIP_* environment variables (tests change
+ * them between calls; a production host never needs this). */
+int cml_reload_env(void);
 /* Message for the last non-zero status returned to this thread ("" if none). */
 const char *cml_last_error(void);
 /* Number of gemv/gemm launches completed by this process: proves the device
@@ -92,6 +109,18 @@ int cml_memset_dev(void *dst_dev, int value, size_t nbytes, cml_stream_t stream)
  * size; may be captured).  Also the yardstick bench.py reads byte counters and
  * matvec bandwidth against: it moves nbytes in, nbytes out and nothing else. */
 int cml_copy_dev(void *dst_dev, const void *src_dev, size_t nbytes, cml_stream_t stream);
+/* Two more yardsticks for the roofline reading of the matvec kernels (bench.py --calibrate-read /
+ * roofline.shape_ceiling); neither has a counterpart in the reference.
+ * cml_calibrate_read: a launch that only READS nbytes (16-byte aligned), every lane keeping
+ * in_flight (1, 2, 4 or 8) 16-byte non-temporal loads out over a grid-stride walk with `workgroups`
+ * workgroups of 256 lanes (0 = 2048), and stores nothing.
+ * cml_calibrate_weight_loads: the plain single-token Q4_K matvec launch for `w` -- same grid, same
+ * lane addresses, same load instructions and register buffers -- with the activation, the
+ * arithmetic and the stores taken out (scratch_dev: 4 writable bytes, never written in practice).
+ * What these two take for a weight's bytes is what the SHAPE allows a single launch on this chip;
+ * what the real kernel takes beyond that is the kernel's own cost. */
+int cml_calibrate_read(const void *src_dev, size_t nbytes, int in_flight, int workgroups, cml_stream_t stream);
+int cml_calibrate_weight_loads(const cml_weight *w, void *scratch_dev, cml_stream_t stream);
 int cml_stream_sync(cml_stream_t stream);
 /* Streams (default priority), timing events and captured launch sequences, for
  * hosts that drive a decode loop through this library alone.  The reference's
@@ -215,6 +244,18 @@ int cml_argmax_f32(const float *logits_dev, int64_t n_rows, int64_t n, uint32_t 
  * src/cuda_resident.rs:334-413). */
 int cml_gemv(const cml_weight *w, const int8_t *q_dev, const float *scales_dev, float *out_dev,
              const float *residual_dev, cml_stream_t stream);
+/* Accumulation order of cml_gemv / cml_gemm / cml_matmul_f32 (every path gives the
+ * same bits for one weight, whatever the token count):
+ *   Q8_0, Q4_0: the reference's block-order chain, always (src/inference.rs:22729-22798).
+ *   Q4_K: the fused per-super-block chain of q4_k_dot_arm (src/diffusion_gemma/
+ *         refmath.rs:504-562).  By default a weight with few row tiles and long rows
+ *         (an FFN down projection, e.g. 4096 x 14336) has its K range cut into 2 / 4 / 8
+ *         parts whose partial chains are added left to right: within 1e-5 (typically
+ *         1e-7) of the reference chain, not its bits.  CAMELID_HIP_EXACT_ORDER=1
+ *         forbids the cut: then every Q4_K result is the reference chain bit for bit.
+ *   Q6_K: the fused chain of q6_k_dot_arm (refmath.rs:678-721), K cut as for Q4_K;
+ *         within 1e-5 of the 8-lane order of q6_k_wire_row_dot (src/inference.rs:
+ *         25535-25581). */
 /* n_tokens activation rows; out_dev[t*rows + row].  A few tokens run on the
  * packed-dot kernel (up to 8 per pass over the weight), larger batches on the
  * int8 matrix cores (all four formats; Q8_0 / Q4_0 rows must be whole multiples
@@ -333,6 +374,10 @@ int cml_quantize_weights_host(int fmt, const float *src, size_t n_values, uint8_
  *      Returns 0 when the device produced `output`, non-zero when the caller
  *      must run its CPU path.  Weights are cached on the device keyed by
  *      (pointer, length), so they must stay alive and unchanged. ------------ */
+/* The reference signature also passes `weight_scales: &[f32]` (src/cuda.rs:1044-1052,
+ * the f16 scales of weight_bytes widened by the caller); the wire bytes already hold
+ * them, so a binding drops that slice, and passes the format id the reference leaves
+ * implicit (its seam is Q8_0 only; this one takes all four formats). */
 int cml_try_linear_rows(int fmt, const float *input_scales, const int8_t *input_quants,
                         const uint8_t *weight_wire, size_t weight_nbytes, int64_t input_rows,
                         int64_t weight_rows, int64_t cols, float *output);

@@ -19,6 +19,8 @@ def say(msg: str) -> None:
 
 @contextmanager
 def env(**kv):
+    """Tuning knobs for the calls inside the block.  The library reads its environment once, so
+    it is told to read it again on the way in and on the way out."""
     old = {k: os.environ.get(k) for k in kv}
     try:
         for k, v in kv.items():
@@ -26,6 +28,7 @@ def env(**kv):
                 os.environ.pop(k, None)
             else:
                 os.environ[k] = str(v)
+        check(lib().cml_reload_env(), "cml_reload_env")
         yield
     finally:
         for k, v in old.items():
@@ -33,6 +36,7 @@ def env(**kv):
                 os.environ.pop(k, None)
             else:
                 os.environ[k] = v
+        check(lib().cml_reload_env(), "cml_reload_env")
 
 
 def is_k(fmt: int) -> bool:

@@ -53,7 +53,14 @@ def test_c2_q4_k_down_4096x14336():
 
 
 def test_c3_q6_k_lm_head_128256x3072():
-    _case(B.CML_Q6_K, 128256, 3072, seed=1004, exact=True)
+    w, wire, x = _case(B.CML_Q6_K, 128256, 3072, seed=1004, exact=True)
+    # the order the reference's CPU lanes run (8 lanes by index mod 8, q6_k_wire_row_dot): bit for bit
+    # under its own switch
+    G.say("Q6_K 128256x3072 in the 8-lane order")
+    with G.env(CAMELID_HIP_Q6K_LANE_ORDER="1"):
+        got = G.gpu_matmul_f32(w, x)
+    want = oracle.matmul(B.CML_Q6_K, wire, 3072, x, order=oracle.ORDER_PRIMARY, threads=16)
+    assert G.same_bits(got, want)
 
 
 def test_c3_q4_0_lm_head_128256x3072():

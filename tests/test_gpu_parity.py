@@ -660,3 +660,61 @@ def test_rows_too_long_for_the_matrix_core_staging_fall_back_to_the_packed_dot(n
     with G.env(CAMELID_HIP_EXACT_ORDER="1"):
         got = G.gpu_gemm(w, s, q)
     check_outputs(fmt, wire, cols, s, q, got, expect_exact=True)
+
+
+@pytest.mark.parametrize("rows,cols", [(130, 1024), (33, 256), (61, 9 * 256), (300, 14336), (5, 16 * 256)])
+def test_q6k_lane_order_is_the_reference_cpu_chain_bit_for_bit(rows, cols):
+    """CAMELID_HIP_Q6K_LANE_ORDER=1: every plain Q6_K call (one token, a batch, a row band, with a
+    residual, f32 or quantized activations in) returns the bits of q6_k_wire_row_dot's 8-lane order
+    (reference src/inference.rs:25535-25581), the order both of the reference's CPU lanes run."""
+    fmt = B.CML_Q6_K
+    rng = np.random.default_rng(rows + cols)
+    wire = G.synth_weight(fmt, rows, cols, seed=rows * 3 + cols)
+    w = Weight.upload(fmt, rows, cols, wire)
+    x = rng.standard_normal((5, cols)).astype(np.float32)
+    x[1, :256] = 0.0
+    s, q = oracle.quantize_activation(fmt, x)
+    want = oracle.matmul_q(fmt, wire, cols, s, q, order=oracle.ORDER_PRIMARY, threads=8)
+    res = rng.standard_normal(rows).astype(np.float32)
+    G.say(f"Q6_K lane order {rows}x{cols}")
+    with G.env(CAMELID_HIP_Q6K_LANE_ORDER="1"):
+        assert G.same_bits(G.gpu_gemm(w, s[0], q[0]), want[0])
+        assert G.same_bits(G.gpu_gemm(w, s[0], q[0], residual=res), want[0] + res)
+        assert G.same_bits(G.gpu_gemm(w, s, q), want)
+        assert G.same_bits(G.gpu_matmul_f32(w, x[2]), want[2])
+        assert G.same_bits(G.gpu_matmul_f32(w, x), want)
+        if rows > 20:
+            band = w.slice(3, rows - 7)
+            assert G.same_bits(G.gpu_gemm(band, s, q), want[:, 3:rows - 4])
+    # without the switch: the fused chain, within tolerance of it
+    assert G.max_rel(G.gpu_gemm(w, s, q), want) <= TOL
+
+
+@pytest.mark.parametrize("rows,cols", [(512, 4096), (47, 4096), (3000, 4096), (9000, 4096), (14336, 4096), (4096, 14336),
+                                       (300, 14336), (100, 8192), (1000, 2048), (70, 7 * 256), (33, 1024)])
+def test_q4k_single_token_entry_points_give_the_same_bits(rows, cols):
+    """A single-token Q4_K call through both entry points (quantized activation in, f32 activation
+    in), with a residual, and on a row band that starts inside a 16-row tile: the oracle's fused
+    order bit for bit with the K cut forbidden, and one set of bits under the default policy, which
+    cuts K for weights of few row tiles."""
+    fmt = B.CML_Q4_K
+    rng = np.random.default_rng(rows * 5 + cols)
+    wire = G.synth_weight(fmt, rows, cols, seed=rows + 3 * cols)
+    w = Weight.upload(fmt, rows, cols, wire)
+    x = rng.standard_normal(cols).astype(np.float32)
+    x[:256] = 0.0
+    s, q = oracle.quantize_activation(fmt, x)
+    want = oracle.matmul(fmt, wire, cols, x, order=oracle.ORDER_PRIMARY, threads=8)
+    res = rng.standard_normal(rows).astype(np.float32)
+    band = w.slice(5, rows - 9) if rows > 20 else None
+    G.say(f"Q4_K single token on {rows}x{cols}")
+    default_bits = G.gpu_gemm(w, s, q)
+    assert G.max_rel(default_bits, want) <= TOL
+    assert G.same_bits(G.gpu_matmul_f32(w, x), default_bits)
+    with G.env(CAMELID_HIP_EXACT_ORDER="1"):
+        assert G.same_bits(G.gpu_gemm(w, s, q), want)
+        assert G.same_bits(G.gpu_gemm(w, s, q, residual=res), want + res)
+        assert G.same_bits(G.gpu_matmul_f32(w, x), want)
+        if band is not None:
+            assert G.same_bits(G.gpu_gemm(band, s, q), want[5:rows - 4])
+            assert G.same_bits(G.gpu_matmul_f32(band, x), want[5:rows - 4])
