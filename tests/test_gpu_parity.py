@@ -559,6 +559,31 @@ def test_q4k_matrix_core_cells_are_bitwise_the_gemv(rows, cols):
         check_outputs(fmt, wire, cols, s, q, got, expect_exact=True)
 
 
+@pytest.mark.parametrize("rows,cols", [(200, 2 * 256), (75, 7 * 256), (1000, 15 * 256), (14336, 4096), (97, 4096)])
+def test_q4k_two_waves_per_tile_keep_one_chain(rows, cols):
+    """Up to 16 tokens against rows of 2..16 super-blocks with no K cut: two waves share a row tile
+    and split K, the chain stays one chain -- the oracle's order bit for bit, the same bits as one
+    wave per tile (CAMELID_HIP_Q4K_MFMA_PAIR=0), also on a row band that starts inside a tile."""
+    fmt = B.CML_Q4_K
+    rng = np.random.default_rng(rows * 7 + cols)
+    wire = G.synth_weight(fmt, rows, cols, seed=rows + cols)
+    w = Weight.upload(fmt, rows, cols, wire)
+    band = w.slice(5, rows - 9)
+    for n in (3, 9, 16):
+        x = rng.standard_normal((n, cols)).astype(np.float32)
+        s, q = oracle.quantize_activation(fmt, x)
+        want = oracle.matmul_q(fmt, wire, cols, s, q, order=oracle.ORDER_PRIMARY, threads=8)
+        G.say(f"Q4_K two waves per tile {rows}x{cols} n={n}")
+        with G.env(CAMELID_HIP_EXACT_ORDER="1"):
+            got = G.gpu_gemm(w, s, q)
+            got_band = G.gpu_gemm(band, s, q)
+            with G.env(CAMELID_HIP_EXACT_ORDER="1", CAMELID_HIP_Q4K_MFMA_PAIR=0):
+                one_wave = G.gpu_gemm(w, s, q)
+        assert G.same_bits(got, want)
+        assert G.same_bits(got, one_wave)
+        assert G.same_bits(got_band, want[:, 5:rows - 4])
+
+
 @pytest.mark.parametrize("name,fmt", [("Q8_0", oracle.Q8_0), ("Q4_0", oracle.Q4_0)])
 @pytest.mark.parametrize("rows,cols", [(130, 1024), (2049, 5 * 256), (77, 12 * 256), (16, 256)])
 def test_b32_matrix_core_cells_are_bitwise_the_gemv(name, fmt, rows, cols):
