@@ -320,9 +320,12 @@ static int launch_quantize_act(int act, const float *x, int64_t n, int64_t cols,
 // out[t][c] = ((0 + y[a(t,0)][c]*w[t][0]) + y[a(t,1)][c]*w[t][1]) + ...  (reference
 // src/inference.rs:14255-14257: `output += expert_out * weight`, routed order,
 // multiply and add rounded separately).
+// slot_expert (single-token decode without a grouping pass: slot s IS assignment s): the routed
+// expert of every slot; a slot whose id is outside [0, n_experts) was served by nobody and is skipped.
 __global__ __launch_bounds__(256) void moe_weighted_sum_kernel(const float *__restrict__ y, const int32_t *__restrict__ slot_to_assign,
                                                                const float *__restrict__ weight, int k, int64_t hidden,
-                                                               int64_t n_assign, float *__restrict__ out) {
+                                                               int64_t n_assign, float *__restrict__ out,
+                                                               const int32_t *__restrict__ slot_expert, int n_experts) {
     const int64_t c = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     const int64_t t = blockIdx.y;
     if (c >= hidden) return;
@@ -337,6 +340,10 @@ __global__ __launch_bounds__(256) void moe_weighted_sum_kernel(const float *__re
             const int64_t slot = t * k + min(s, k - 1);
             const int64_t a = slot_to_assign ? slot_to_assign[slot] : slot;
             ok[j] = s < k && a >= 0 && a < n_assign;  // a dropped slot (expert id out of range) or a malformed map is skipped
+            if (slot_expert) {
+                const int e = slot_expert[slot];
+                ok[j] = ok[j] && e >= 0 && e < n_experts;
+            }
             yv[j] = y[(ok[j] ? a : 0) * hidden + c];
             wv[j] = weight[slot];
         }
@@ -469,7 +476,7 @@ int cml_moe_weighted_sum(const float *y_dev, const int32_t *route_to_assignment_
     if (n_tokens == 0) return CML_OK;
     if (!y_dev || !weight_dev || !out_dev) return fail(CML_ERR_INVALID, "null pointer");
     hipLaunchKernelGGL(moe_weighted_sum_kernel, dim3(static_cast<unsigned>((hidden + 255) / 256), static_cast<unsigned>(n_tokens)), dim3(256), 0,
-                       as_stream(stream), y_dev, route_to_assignment_dev, weight_dev, k, hidden, n_tokens * k, out_dev);
+                       as_stream(stream), y_dev, route_to_assignment_dev, weight_dev, k, hidden, n_tokens * k, out_dev, nullptr, 0);
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }
@@ -592,7 +599,8 @@ int cml_moe_ffn_ex(const cml_weight *gate, const cml_weight *up, const cml_weigh
         if (int rc = launch_expert_matmul(a, st)) return rc;
     }
     hipLaunchKernelGGL(moe_weighted_sum_kernel, dim3(static_cast<unsigned>((hidden + 255) / 256), static_cast<unsigned>(n_tokens)), dim3(256), 0, st,
-                       ws.y, direct ? nullptr : ws.slot_to_assign, weight_dev, k, hidden, static_cast<int64_t>(n_slots), out_dev);
+                       ws.y, direct ? nullptr : ws.slot_to_assign, weight_dev, k, hidden, static_cast<int64_t>(n_slots), out_dev,
+                       direct ? idx_dev : nullptr, n_experts);
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }

@@ -184,6 +184,47 @@ def test_moe_ffn_is_the_sum_of_single_expert_calls():
     assert G.max_rel(got, want) <= 2e-6   # silu's expf is the only difference
 
 
+@pytest.mark.parametrize("fmt,fmt_down,hidden,ff", [(B.CML_Q4_K, B.CML_Q4_K, 512, 1024), (B.CML_Q4_0, B.CML_Q8_0, 352, 96)])
+@pytest.mark.parametrize("T", [1, 3])
+def test_moe_ffn_skips_slots_with_expert_ids_out_of_range(fmt, fmt_down, hidden, ff, T):
+    """A routed slot whose expert id is outside [0, n_experts) is served by nobody and adds nothing:
+    the same bits as the call with that slot left out (decode and batched paths; the workspace
+    starts poisoned so that a slot's stale output would show)."""
+    E, k = 8, 3
+    gate_up, down = _experts_fused(fmt, fmt_down, E, hidden, ff, 700)
+    wgu = Weight.upload(fmt, E * 2 * ff, hidden, gate_up)
+    wd = Weight.upload(fmt_down, E * hidden, ff, down)
+    rng = np.random.default_rng(701 + T)
+    x = rng.standard_normal((T, hidden)).astype(np.float32)
+    idx = np.stack([rng.permutation(E)[:k] for _ in range(T)]).astype(np.int32)
+    w = rng.random((T, k)).astype(np.float32)
+    for bad in (E + 5, -1):
+        idx_bad = idx.copy()
+        idx_bad[:, 1] = bad
+        G.say(f"moe ffn with expert id {bad} in slot 1, fmt={fmt}/{fmt_down} T={T}")
+        got = _moe_poisoned(wgu, wd, E, k, idx_bad, w, x)
+        want = _moe_poisoned(wgu, wd, E, k - 1, np.ascontiguousarray(idx[:, [0, 2]]), np.ascontiguousarray(w[:, [0, 2]]), x)
+        assert np.isfinite(got).all()
+        assert G.same_bits(got, want)
+
+
+def _moe_poisoned(wgu, wd, E, k, idx, w, x):
+    T, hidden = x.shape
+    ff = wd.cols
+    xd = DeviceBuffer.from_numpy(x)
+    out = DeviceBuffer(T * hidden * 4)
+    out.fill(0xFF)
+    ws_bytes = lib().cml_moe_workspace_bytes(wgu.fmt, hidden, ff, T, k, E)
+    ws = DeviceBuffer(ws_bytes)
+    ws.fill(0xFF)    # NaN patterns wherever a float is read without having been written
+    idx_dev = DeviceBuffer.from_numpy(np.ascontiguousarray(idx, np.int32))
+    w_dev = DeviceBuffer.from_numpy(np.ascontiguousarray(w, np.float32))
+    check(lib().cml_moe_ffn_ex(wgu.handle, None, wd.handle, E, k, idx_dev.ptr, w_dev.ptr, xd.ptr, T, out.ptr, ws.ptr, ws_bytes,
+                               GLU_GELU_TANH, None), "cml_moe_ffn_ex")
+    check(lib().cml_stream_sync(None))
+    return out.to_numpy(np.float32, (T, hidden))
+
+
 @pytest.mark.parametrize("T", [1, 32])
 def test_c5_mixtral_shaped_moe(T):
     """8 experts, gate/up 14336x4096 and down 4096x14336 in Q4_K, top-2 routing."""
