@@ -40,8 +40,8 @@ INT8_PEAK_TOPS = 5000.0  # MI355X published dense int8 matrix-core rate
 # run, so the figures measured for the committed kernels are carried here; null where not measured.
 MEASURED_TRAFFIC_BYTES: dict = {
     # profiles/hbm_traffic_fetch_write_size.txt (copy yardstick: FETCH_SIZE x 2.000, WRITE_SIZE x 1.000)
-    "q4k_14336x4096_n1": 33371997,       # 1.008 x algorithmic
-    "q4k_14336x4096_n16": 34829074,      # 1.018 x
+    "q4k_14336x4096_n1": 33374720,       # 1.008 x algorithmic
+    "q4k_14336x4096_n16": 34686362,      # 1.014 x
     "q4k_14336x4096_n64": 39155356,      # 1.038 x
     "q6k_128256x3072_n1": 323916630,     # 1.001 x
     "q4_0_128256x3072_n16": 252016327,   # 1.087 x
@@ -630,8 +630,11 @@ def main() -> int:
         ceiling["us_per_launch"] = floor_us
         ceiling["gbs"] = round(alg_bytes / floor_us / 1e3, 2)
         ceiling["frac"] = round(alg_bytes / floor_us / 1e3 / HBM_PEAK_GBS, 4)
-        ceiling["note"] = ("launches with this weight's bytes and no arithmetic, same graph replay and rotation: "
-                           "the part of the distance to the roofline that belongs to the shape, not to the kernel")
+        ceiling["note"] = ("launches that only read this weight's bytes (the matvec's own load instructions with nothing "
+                           "behind them; the best of four plain grid-stride read launches), same graph replay and rotation. "
+                           "Measured reference points, not bounds: for a launch of tens of MB they show how much of the "
+                           "distance to the roofline the launch itself costs; on matrices of hundreds of MB the matvec's "
+                           "tiled, non-temporal access pattern outruns the plain read")
     check(L.cml_stream_sync(stream))
     result = out.to_numpy(np.float32, (n, rows))
     if not np.all(np.isfinite(result)):

@@ -134,13 +134,13 @@ __device__ __forceinline__ void b32_mfma_operands(const B32SlabWeights<FMT> &r, 
 // flight in registers.
 // A workgroup's 4 waves are 4/TB consecutive row tiles x TB token blocks of 16*GPW tokens.
 // PLAIN: the entry of a call without expert groups (no group tables to read before the first request).
-template <int FMT, int GPW, int TB, int KC, int RING, bool PLAIN = false>
-__global__ __launch_bounds__(256) void gemm_b32_mfma_kernel(B32MfmaArgs a) {
+template <int FMT, int GPW, int TB, int KC, int RING, bool PLAIN = false, int WAVES = 4>
+__global__ __launch_bounds__(64 * WAVES) void gemm_b32_mfma_kernel(B32MfmaArgs a) {
     constexpr int NTOK = 16 * GPW * TB;              // tokens staged per workgroup
-    constexpr int RT = 4 / TB;                       // row tiles per workgroup
+    constexpr int RT = WAVES / TB;                   // row tiles per workgroup
     constexpr int kBufBytes = KC * NTOK * kB32SlabRow;
     constexpr int kBsInts = KC * 8 * NTOK;           // per buffer: -8 * block sums, [slab][block][token]
-    constexpr int nthreads = 256;
+    constexpr int nthreads = 64 * WAVES;
     constexpr int kPer = NTOK * 16 / nthreads;       // 16-byte pieces of one slab of all tokens, per thread
     static_assert(RING % KC == 0 && kPer >= 1, "phase / staging shape");
     extern __shared__ uint4 smem[];
@@ -351,9 +351,9 @@ __global__ __launch_bounds__(256) void gemm_b32_mfma_kernel(B32MfmaArgs a) {
     }
 }
 
-template <int FMT, int GPW, int TB, int KC, int RING, bool PLAIN>
+template <int FMT, int GPW, int TB, int KC, int RING, bool PLAIN, int WAVES = 4>
 static int launch_b32_mfma_gp(const B32MfmaArgs &ka, int n_groups, hipStream_t st) {
-    constexpr int NTOK = 16 * GPW * TB, RT = 4 / TB;
+    constexpr int NTOK = 16 * GPW * TB, RT = WAVES / TB;
     const int n_tiles = (ka.rows + 15) / 16;
     const unsigned gx = static_cast<unsigned>((n_tiles + RT - 1) / RT);
     const unsigned gy = static_cast<unsigned>((ka.n_tokens + NTOK - 1) / NTOK);
@@ -362,11 +362,11 @@ static int launch_b32_mfma_gp(const B32MfmaArgs &ka, int n_groups, hipStream_t s
     if (lds > 160 * 1024) return fail(CML_ERR_UNSUPPORTED, "matrix-core path: %d blocks per row exceed the LDS budget", ka.n_slabs * 8);
     static bool raised = false;  // per instantiation: allow more than 64 KB of dynamic LDS once
     if (!raised) {
-        CML_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_b32_mfma_kernel<FMT, GPW, TB, KC, RING, PLAIN>),
+        CML_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_b32_mfma_kernel<FMT, GPW, TB, KC, RING, PLAIN, WAVES>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
         raised = true;
     }
-    hipLaunchKernelGGL((gemm_b32_mfma_kernel<FMT, GPW, TB, KC, RING, PLAIN>), dim3(gx, gy, n_groups), dim3(256), lds, st, ka);
+    hipLaunchKernelGGL((gemm_b32_mfma_kernel<FMT, GPW, TB, KC, RING, PLAIN, WAVES>), dim3(gx, gy, n_groups), dim3(64 * WAVES), lds, st, ka);
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }
@@ -392,6 +392,13 @@ static int launch_b32_mfma_p(const B32MfmaArgs &ka, int n_groups, hipStream_t st
     int deep = env_int("CAMELID_HIP_B32_MFMA_DEEP", -1);
     if (deep != 0 && deep != 1) deep = (ka.rows + 15) / 16 < 2048 ? 1 : 0;
     if constexpr (NTOK == 16) {
+        // Q8_0 with at most 512 row tiles: workgroups of two waves instead of four, so that every compute
+        // unit gets one (measured, 16 tokens: 8192 x 2048 11.4 -> 10.6 us, 4096 x 4096 17.5 -> 15.6; Q4_0
+        // 4096 x 4096 18.6 -> 19.9, so Q4_0 keeps four).  A wave still walks a whole row tile alone: the
+        // serial chain of one f32 step per 32-value block is what bounds these launches.
+        const int two = env_int("CAMELID_HIP_B32_MFMA_TWO_WAVES", -1);
+        if (deep && ka.group_offsets == nullptr && (two == 1 || (two != 0 && FMT == CML_Q8_0 && (ka.rows + 15) / 16 <= 512)))
+            return launch_b32_mfma_gp<FMT, GPW, TB, 8, 8, true, 2>(ka, n_groups, st);
         return deep ? launch_b32_mfma_g<FMT, GPW, TB, 8, 8>(ka, n_groups, st) : launch_b32_mfma_g<FMT, GPW, TB, 2, 2>(ka, n_groups, st);
     } else if constexpr (NTOK == 32) {
         return deep ? launch_b32_mfma_g<FMT, GPW, TB, 4, 4>(ka, n_groups, st) : launch_b32_mfma_g<FMT, GPW, TB, 2, 2>(ka, n_groups, st);
