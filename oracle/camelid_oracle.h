@@ -26,9 +26,15 @@
  *                                against dequantized activations (the reference
  *                                tests' own criterion), cross-variant agreement.
  *                                The *bitwise* value of the final f32 has no
- *                                stored vector in the reference: the order of
- *                                operations is transcribed, not pinned
- *                                ("parity unpinned" for the last-ulp value).
+ *                                stored vector in the reference; its association
+ *                                is held by an independent evaluator instead
+ *                                (tests/test_oracle_association.py: integers from
+ *                                the numpy decoders, every float step in exact
+ *                                rationals with an explicit round to binary32),
+ *                                on inputs where the plausible wrong orders give
+ *                                other bits.  What stays transcription: that the
+ *                                formula written into that evaluator is the one
+ *                                in the Rust source.
  *   softmax_top_k, router_     : closed forms and brute force on small inputs;
  *   softmax_top_k                libm expf may differ from Rust's by 1 ulp.
  *   gelu_tanh_mul, silu_mul    : f64 evaluation of the formula within 1e-6; libm
