@@ -803,6 +803,13 @@ int cml_matmul_f32(const cml_weight *w, const float *x_dev, int64_t n_tokens, fl
         if (frc == CML_OK) g_runs.fetch_add(1, std::memory_order_relaxed);
         return frc;
     }
+    if (w->fmt == CML_Q4_K && n_tokens >= 3 && fuse != 0 && env_int("CAMELID_HIP_FUSED_QUANT_BATCH", 1)) {
+        // 3 to 6 tokens on the matrix cores: the workgroups quantize the few rows themselves (14336 x 4096,
+        // 4 tokens: 12.4 -> 11.0 us per step); more tokens cost every workgroup more than the launch saves
+        const int frc = launch_gemm_q4k_mfma_f32(w, x_dev, n_tokens, out_dev, st);
+        if (frc == CML_OK) g_runs.fetch_add(1, std::memory_order_relaxed);
+        if (frc != -1) return frc;
+    }
     if (w->fmt == CML_Q6_K && (n_tokens == 1 || fuse_two) && env_int("CAMELID_HIP_Q6K_FUSED_QUANT", 1) && !q6k_lane_order() &&
         (fuse == 2 || (fuse == 1 && w->nb <= 32 && w->rows <= 32768))) {
         // the same for Q6_K: 4096 x 4096 7.0 -> 5.5 us, 14336 x 4096 12.3 -> 10.8; not on a vocabulary

@@ -115,6 +115,7 @@ int launch_gemv_q4k(const MatArgs &a, hipStream_t st);
 int launch_gemv_q4k_f32_grouped_pair(const MatArgs &a, const cml_weight *w2, float *out2, const float *x, hipStream_t st);
 
 int launch_gemv_q4k_f32(const cml_weight *w, const float *x, float *out, hipStream_t st, int n_tokens = 1);  // quantize + matvec, one or two tokens
+int launch_gemm_q4k_mfma_f32(const cml_weight *w, const float *x, int64_t n_tokens, float *out, hipStream_t st);  // 3..8 tokens, quantize inside; -1: not served
 int launch_gemv_q4k_loads_only(const cml_weight *w, float *out, hipStream_t st);  // calibration: the single-token launch's loads alone
 int launch_gemv_q6k_f32(const cml_weight *w, const float *x, float *out, hipStream_t st, int n_tokens = 1);  // Q6_K: quantize + matvec, one or two tokens
 int launch_gemv_b32_f32(const cml_weight *w, const float *x, float *out, hipStream_t st, int n_tokens = 1);  // quantize + matvec, one or two tokens

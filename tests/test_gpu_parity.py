@@ -368,6 +368,38 @@ def test_q4k_fused_two_tokens_is_the_two_step_path(rows, cols):
         assert G.same_bits(got, want)
 
 
+@pytest.mark.parametrize("rows,cols", [(190, 3072), (64, 512), (333, 4096), (14336, 4096), (77, 1280)])
+def test_q4k_fused_quantize_small_batches_are_the_two_step_path(rows, cols):
+    """3 to 8 f32 rows against a Q4_K weight run as ONE launch (the matrix-core kernel quantizes them
+    itself): bit for bit the quantize launch + matmul, on rows with zero blocks, equal magnitudes of
+    both signs and exact rounding ties, for a full weight and a band that starts inside a tile."""
+    fmt = B.CML_Q4_K
+    rng = np.random.default_rng(rows + cols)
+    wire = G.synth_weight(fmt, rows, cols, seed=rows * 11 + cols)
+    w = Weight.upload(fmt, rows, cols, wire)
+    band = w.slice(3, rows - 7) if rows > 20 else None
+    for n in (3, 4, 5, 6, 8):                 # 8: served when CAMELID_HIP_FUSED_QUANT_BATCH_MAX allows it
+        x = rng.standard_normal((n, cols)).astype(np.float32)
+        x[0, :256] = 0.0                      # an empty super-block
+        x[1, 256:512] = np.float32(0.5)       # every value the maximum
+        x[n - 1, 0] = -x[n - 1, 1]            # two first holders of the maximum, opposite signs
+        x[2, :256] = np.round(x[2, :256] * 4) / 4
+        G.say(f"Q4_K fused quantize, {n} tokens, {rows}x{cols}")
+        s, q = oracle.quantize_activation(fmt, x)
+        with G.env(CAMELID_HIP_EXACT_ORDER="1", CAMELID_HIP_FUSED_QUANT_BATCH_MAX=8):
+            got = G.gpu_matmul_f32(w, x)
+            two_step = G.gpu_gemm(w, s, q)
+            with G.env(CAMELID_HIP_EXACT_ORDER="1", CAMELID_HIP_FUSED_QUANT_BATCH=0):
+                unfused = G.gpu_matmul_f32(w, x)
+            if band is not None:
+                got_band = G.gpu_matmul_f32(band, x)
+        assert G.same_bits(got, two_step)
+        assert G.same_bits(got, unfused)
+        check_outputs(fmt, wire, cols, s, q, got, expect_exact=True)
+        if band is not None:
+            assert G.same_bits(got_band, got[:, 3:rows - 4])
+
+
 @pytest.mark.parametrize("rows,cols", [(190, 3072), (61, 256), (333, 4096), (20, 14336), (2100, 1280)])
 def test_q6k_fused_quantize_matvec_is_the_two_step_path(rows, cols):
     """One- and two-token cml_matmul_f32 on Q6_K quantizes inside the matvec kernel: the bits of
