@@ -662,7 +662,7 @@ static int dispatch(const MatArgs &a, hipStream_t st) {
             // so such a call stays on the packed-dot kernel whatever the thresholds say.)
             // Measured on MI355X at 14336x4096: the matrix-core kernel takes 12 us for any batch up to
             // 16 tokens, the packed-dot kernel 7.2 / 9.9 us for 1 / 2 tokens and two launches for 3.
-            if (!a.group_offsets && !a.ints && !a.residual && a.n_tokens >= env_int("CAMELID_HIP_Q4K_MFMA_MIN_TOKENS", 3))
+            if (!a.group_offsets && !a.ints && !a.residual && !q4k_lane_order() && a.n_tokens >= env_int("CAMELID_HIP_Q4K_MFMA_MIN_TOKENS", 3))
                 rc = launch_gemm_q4k_mfma(a, st);
             else
                 rc = launch_gemv_q4k(a, st);
@@ -794,7 +794,7 @@ int cml_matmul_f32(const cml_weight *w, const float *x_dev, int64_t n_tokens, fl
     hipStream_t st = as_stream(stream);
     const int fuse = env_int("CAMELID_HIP_FUSED_QUANT", 1);  // 0 = never, 1 = by shape, 2 = whenever possible
     const bool fuse_two = n_tokens == 2 && env_int("CAMELID_HIP_FUSED_QUANT_TWO", 1) && !env_int("CAMELID_HIP_Q4K_GENERAL_ENTRY", 0);
-    if (w->fmt == CML_Q4_K && (n_tokens == 1 || fuse_two) && (fuse == 2 || (fuse == 1 && w->nb <= 32))) {
+    if (w->fmt == CML_Q4_K && !q4k_lane_order() && (n_tokens == 1 || fuse_two) && (fuse == 2 || (fuse == 1 && w->nb <= 32))) {
         // rows of up to 8192 values: one launch quantizes the activation in every workgroup (one or
         // two passes of its four waves; twice that for a pair of tokens) and runs the matvec
         // (4096 x 8192: 7.1 -> 6.6 us, 2048 x 8192: 6.3 -> 4.7); at 14336 values the passes cost
@@ -803,7 +803,7 @@ int cml_matmul_f32(const cml_weight *w, const float *x_dev, int64_t n_tokens, fl
         if (frc == CML_OK) g_runs.fetch_add(1, std::memory_order_relaxed);
         return frc;
     }
-    if (w->fmt == CML_Q4_K && n_tokens >= 3 && fuse != 0 && env_int("CAMELID_HIP_FUSED_QUANT_BATCH", 1)) {
+    if (w->fmt == CML_Q4_K && !q4k_lane_order() && n_tokens >= 3 && fuse != 0 && env_int("CAMELID_HIP_FUSED_QUANT_BATCH", 1)) {
         // 3 to 6 tokens on the matrix cores: the workgroups quantize the few rows themselves (14336 x 4096,
         // 4 tokens: 12.4 -> 11.0 us per step); more tokens cost every workgroup more than the launch saves
         const int frc = launch_gemm_q4k_mfma_f32(w, x_dev, n_tokens, out_dev, st);

@@ -144,6 +144,7 @@ int launch_gemm_q4_0(const MatArgs &a, hipStream_t st);
 int launch_gemm_q6k(const MatArgs &a, hipStream_t st);
 int launch_gemm_q6k_mfma(const MatArgs &a, hipStream_t st);  // Q6_K on the matrix cores; plain or grouped
 int q6k_mfma_min_tokens(int64_t rows, int64_t n_sb);         // batch size from which it pays
+bool q4k_lane_order();                                       // CAMELID_HIP_Q4K_LANE_ORDER: the reference wire row dot's generic 8-lane order, bit for bit
 bool q6k_lane_order();                                       // CAMELID_HIP_Q6K_LANE_ORDER: the reference CPU lanes' 8-lane order, bit for bit
 
 // Integer tuning knob read once from the environment (0 when unset).

@@ -710,10 +710,131 @@ int launch_gemv_q4k_f32_grouped_pair(const MatArgs &a, const cml_weight *w2, flo
     return launch_q4k_f32(a, w2, out2, x, st);
 }
 
+// ---- the generic 8-lane order of the reference's wire row dot, bit for bit ----------------------
+//
+// q4_k_wire_row_dot (src/inference.rs:25806-25889, the Q4_K row dot of the Gemma-4 wire lane and
+// the oracle of the reference's CUDA matvec) is not the fused chain the kernels above keep: per
+// super-block it takes eight integer lanes by value index modulo 8
+// (aux32[l] += scale_j * y * a), sums[l] += (d * yd) * (float)aux32[l] with multiply and add
+// rounded separately, sumf -= (dmin * yd) * (float)sumi for the mins, and returns
+// sumf + (((0 + sums[0]) + sums[1]) + ...).  The kernels above match it to 1e-5; this one
+// reproduces it exactly and serves every plain Q4_K call under CAMELID_HIP_Q4K_LANE_ORDER=1
+// (speed is secondary: byte loads from the tiled layout, one wave per row).  Lane = 8 * g + l:
+// eight super-blocks g per pass, their integers independent; the f32 sums are then advanced in
+// super-block order by the lanes of g = 0 through LDS.
+__device__ __forceinline__ void q4k_wave_lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+__global__ __launch_bounds__(256) void gemv_q4k_lanes_kernel(const uint8_t *__restrict__ wbase, int64_t sb_stride, int rows, int row_skip,
+                                                             int n_sb, const int8_t *__restrict__ q, const float *__restrict__ yd,
+                                                             float *__restrict__ out, const float *__restrict__ residual) {
+    extern __shared__ uint4 smem[];
+    int8_t *ys = reinterpret_cast<int8_t *>(smem);                        // [n_sb*256]
+    float *yds = reinterpret_cast<float *>(ys + n_sb * 256);              // [n_sb]
+    float *xch = yds + ((n_sb + 3) & ~3);                                 // [4 waves][64 lane terms + 8 mins terms]
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int token = blockIdx.y;
+    const int8_t *qt = q + static_cast<int64_t>(token) * n_sb * 256;
+    for (int i = tid; i < n_sb * 16; i += 256) reinterpret_cast<uint4 *>(ys)[i] = reinterpret_cast<const uint4 *>(qt)[i];
+    for (int i = tid; i < n_sb; i += 256) yds[i] = yd[static_cast<int64_t>(token) * n_sb + i];
+    __syncthreads();
+    const int row = blockIdx.x * 4 + wave;
+    if (row >= rows) return;  // whole waves leave; no workgroup barrier follows
+    const int g = lane >> 3, l = lane & 7;
+    const int lrow = row + row_skip;  // row in the tiled layout
+    const uint8_t *tile = wbase + static_cast<int64_t>(lrow >> 4) * kQ4KChunk;
+    const int rl = lrow & 15;
+    float *mine = xch + wave * 72;
+    float sum_l = 0.0f;   // lanes of g == 0: sums[l]
+    float sumf = 0.0f;    // lane 0: the mins chain
+    for (int sb0 = 0; sb0 < n_sb; sb0 += 8) {
+        const int sb = sb0 + g;
+        float term = 0.0f, mterm = 0.0f;
+        if (sb < n_sb) {
+            const uint8_t *chunk = tile + static_cast<int64_t>(sb) * sb_stride;
+            const uint4 hdr = *reinterpret_cast<const uint4 *>(chunk + rl * 16);
+            uint32_t sc03, sc47, m03, m47;
+            q4k_unpack_scales(hdr.y, hdr.z, hdr.w, sc03, sc47, m03, m47);
+            const int8_t *y = ys + sb * 256;
+            int aux = 0;
+#pragma unroll
+            for (int j = 0; j < 8; j++) {  // sub-block j: chunk j / 2, low (even j) or high nibbles
+                const int scale = static_cast<int>(((j < 4 ? sc03 : sc47) >> (8 * (j & 3))) & 0xff);
+                int part = 0;
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    const int jj = 8 * k + l;  // byte of the chunk
+                    const uint8_t byte = chunk[(jj < 16 ? 256 : 1280) + rl * 64 + (j >> 1) * 16 + (jj & 15)];
+                    const int a4 = (j & 1) ? (byte >> 4) : (byte & 15);
+                    part += static_cast<int>(y[32 * j + jj]) * a4;
+                }
+                aux += scale * part;
+            }
+            // the mins: lane l takes the 16-value sums j = l and l + 8, the eight lanes' parts are added (exact integers)
+            int sumi = 0;
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const int j = l + 8 * h;
+                int bs = 0;
+#pragma unroll
+                for (int t = 0; t < 16; t++) bs += y[16 * j + t];
+                const int g8 = j >> 1;
+                sumi += bs * static_cast<int>(((g8 < 4 ? m03 : m47) >> (8 * (g8 & 3))) & 0xff);
+            }
+            sumi += __shfl_xor(sumi, 1);
+            sumi += __shfl_xor(sumi, 2);
+            sumi += __shfl_xor(sumi, 4);
+            const float d = f16_bits_to_f32(hdr.x & 0xffffu), dmin = f16_bits_to_f32(hdr.x >> 16);
+            const float ydv = yds[sb];
+            const float dd = d * ydv;
+            term = dd * static_cast<float>(aux);
+            mterm = (dmin * ydv) * static_cast<float>(sumi);
+        }
+        mine[lane] = term;
+        if (l == 0) mine[64 + g] = mterm;
+        q4k_wave_lds_sync();
+        if (g == 0) {
+            const int n = min(8, n_sb - sb0);
+            for (int k = 0; k < n; k++) {
+                sum_l = sum_l + mine[8 * k + l];
+                sumf = sumf - mine[64 + k];  // only lane 0's copy is used
+            }
+        }
+        q4k_wave_lds_sync();
+    }
+    if (g == 0) mine[l] = sum_l;
+    q4k_wave_lds_sync();
+    if (lane == 0) {
+        float lanes = 0.0f;
+        for (int k = 0; k < 8; k++) lanes = lanes + mine[k];
+        float total = sumf + lanes;
+        if (residual) total = total + residual[row];
+        out[static_cast<int64_t>(token) * rows + row] = total;
+    }
+}
+
+bool q4k_lane_order() { return env_int("CAMELID_HIP_Q4K_LANE_ORDER", 0) != 0; }
+
+static int launch_gemv_q4k_lanes(const MatArgs &a, hipStream_t st) {
+    const cml_weight *w = a.w;
+    const int n_sb = static_cast<int>(w->nb);
+    const size_t lds = static_cast<size_t>(n_sb) * 256 + ((static_cast<size_t>(n_sb) + 3) & ~size_t(3)) * 4 + 4 * 72 * 4;
+    if (lds > 64 * 1024) return fail(CML_ERR_UNSUPPORTED, "Q4_K activation of %d super-blocks exceeds the LDS staging limit", n_sb);
+    if (a.n_tokens > 65535) return fail(CML_ERR_UNSUPPORTED, "at most 65535 tokens per call in the lane-order mode");
+    hipLaunchKernelGGL(gemv_q4k_lanes_kernel, dim3(static_cast<unsigned>((w->rows + 3) / 4), static_cast<unsigned>(a.n_tokens)), dim3(256), lds, st,
+                       w->planes.p[0], w->planes.row_stride[0], static_cast<int>(w->rows), w->row_skip, n_sb, a.q, a.scales, a.out, a.residual);
+    CML_HIP_TRY(hipGetLastError());
+    return CML_OK;
+}
+
 int launch_gemv_q4k(const MatArgs &a, hipStream_t st) {
     const cml_weight *w = a.w;
     if (w->rows == 0 || a.n_tokens == 0) return CML_OK;
     const bool grouped = a.group_offsets != nullptr || a.group_ids != nullptr;
+    if (!grouped && !a.ints && q4k_lane_order()) return launch_gemv_q4k_lanes(a, st);
     Q4KArgs ka{};
     ka.w = w->planes.p[0];
     ka.sb_stride = w->planes.row_stride[0];

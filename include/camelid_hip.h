@@ -253,9 +253,14 @@ int cml_gemv(const cml_weight *w, const int8_t *q_dev, const float *scales_dev, 
  *         parts whose partial chains are added left to right: within 1e-5 (typically
  *         1e-7) of the reference chain, not its bits.  CAMELID_HIP_EXACT_ORDER=1
  *         forbids the cut: then every Q4_K result is the reference chain bit for bit.
+ *         The other Q4_K order of the reference, the generic 8-lane one of
+ *         q4_k_wire_row_dot (src/inference.rs:25806-25889, the Gemma-4 wire lane), is
+ *         matched within 1e-5 by default and bit for bit under
+ *         CAMELID_HIP_Q4K_LANE_ORDER=1 (plain calls; slower).
  *   Q6_K: the fused chain of q6_k_dot_arm (refmath.rs:678-721), K cut as for Q4_K;
  *         within 1e-5 of the 8-lane order of q6_k_wire_row_dot (src/inference.rs:
- *         25535-25581). */
+ *         25535-25581), which CAMELID_HIP_Q6K_LANE_ORDER=1 reproduces bit for bit
+ *         (plain calls; slower). */
 /* n_tokens activation rows; out_dev[t*rows + row].  A few tokens run on the
  * packed-dot kernel (up to 8 per pass over the weight), larger batches on the
  * int8 matrix cores (all four formats; Q8_0 / Q4_0 rows must be whole multiples

@@ -43,7 +43,13 @@ def test_c1_q8_0_8192x2048():
 
 
 def test_c2_q4_k_gate_up_14336x4096():
-    _case(B.CML_Q4_K, 14336, 4096, seed=1002, exact=True)
+    w, wire, x = _case(B.CML_Q4_K, 14336, 4096, seed=1002, exact=True)
+    # the generic 8-lane order of the reference's wire row dot (q4_k_wire_row_dot): bit for bit under its own switch
+    G.say("Q4_K 14336x4096 in the 8-lane order")
+    with G.env(CAMELID_HIP_Q4K_LANE_ORDER="1"):
+        got = G.gpu_matmul_f32(w, x)
+    want = oracle.matmul(B.CML_Q4_K, wire, 4096, x, order=oracle.ORDER_ALT, threads=16)
+    assert G.same_bits(got, want)
 
 
 def test_c2_q4_k_down_4096x14336():

@@ -747,6 +747,41 @@ def test_q6k_lane_order_is_the_reference_cpu_chain_bit_for_bit(rows, cols):
     assert G.max_rel(G.gpu_gemm(w, s, q), want) <= TOL
 
 
+@pytest.mark.parametrize("rows,cols", [(130, 1024), (33, 256), (61, 9 * 256), (300, 14336), (5, 16 * 256), (2000, 4096)])
+def test_q4k_lane_order_is_the_reference_wire_row_dot_bit_for_bit(rows, cols):
+    """CAMELID_HIP_Q4K_LANE_ORDER=1: every plain Q4_K call (one token, a batch, a row band that
+    starts inside a tile, with a residual, f32 or quantized activations in) returns the bits of
+    q4_k_wire_row_dot's generic 8-lane order (reference src/inference.rs:25806-25889), the order of
+    the Gemma-4 wire lane; the default kernels keep the fused order of q4_k_dot_arm."""
+    fmt = B.CML_Q4_K
+    rng = np.random.default_rng(rows + cols)
+    wire = G.synth_weight(fmt, rows, cols, seed=rows * 3 + cols)
+    w = Weight.upload(fmt, rows, cols, wire)
+    x = rng.standard_normal((5, cols)).astype(np.float32)
+    x[1, :256] = 0.0
+    s, q = oracle.quantize_activation(fmt, x)
+    want = oracle.matmul_q(fmt, wire, cols, s, q, order=oracle.ORDER_ALT, threads=8)
+    fused = oracle.matmul_q(fmt, wire, cols, s, q, order=oracle.ORDER_PRIMARY, threads=8)
+    res = rng.standard_normal(rows).astype(np.float32)
+    G.say(f"Q4_K lane order {rows}x{cols}")
+    with G.env(CAMELID_HIP_Q4K_LANE_ORDER="1"):
+        assert G.same_bits(G.gpu_gemm(w, s[0], q[0]), want[0])
+        assert G.same_bits(G.gpu_gemm(w, s[0], q[0], residual=res), want[0] + res)
+        assert G.same_bits(G.gpu_gemm(w, s, q), want)
+        assert G.same_bits(G.gpu_matmul_f32(w, x[2]), want[2])
+        assert G.same_bits(G.gpu_matmul_f32(w, x), want)
+        if rows > 20:
+            band = w.slice(3, rows - 7)
+            assert G.same_bits(G.gpu_gemm(band, s, q), want[:, 3:rows - 4])
+    # without the switch: the fused chain (exactly, with the K cut forbidden), within tolerance of the 8-lane order
+    with G.env(CAMELID_HIP_EXACT_ORDER="1"):
+        got = G.gpu_gemm(w, s, q)
+    assert G.same_bits(got, fused)
+    assert G.max_rel(got, want) <= TOL
+    if cols >= 1024:
+        assert not G.same_bits(fused, want)    # the two orders do differ on this input
+
+
 @pytest.mark.parametrize("rows,cols", [(512, 4096), (47, 4096), (3000, 4096), (9000, 4096), (14336, 4096), (4096, 14336),
                                        (300, 14336), (100, 8192), (1000, 2048), (70, 7 * 256), (33, 1024)])
 def test_q4k_single_token_entry_points_give_the_same_bits(rows, cols):
