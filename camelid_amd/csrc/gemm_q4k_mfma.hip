@@ -356,20 +356,23 @@ int q4k_ksplit_for(int64_t rows, int64_t n_sb);  // gemv_q4k.hip: the matvec ker
 // With one wave per row tile a 14336 x 4096 weight is 896 waves -- fewer than the chip has SIMDs,
 // each alone on its SIMD, so nothing runs while a wave waits for memory or for its own matrix-core
 // results.  Here two waves share a row tile and split K at `s_mid`; the reference's chain over the
-// super-blocks of a row stays ONE chain, in order: the second wave computes the exact integers
-// (P, S) of its super-blocks and leaves them in LDS with the row's d / dmin; the first wave chains
-// its own super-blocks meanwhile, and after one barrier both continue through the second wave's
-// terms -- the first wave for two of a lane's four cells, the second (seeded with the first
-// wave's sums) for the other two.  Same integers, same f32 operations in the same order as the
-// kernel above: bit for bit.
+// super-blocks of a row stays ONE chain, in order.  The first wave chains its super-blocks as the
+// kernel above does.  The second cannot start its chain before the first has ended, but
+// everything of a step that does not depend on the running sum it does at once: the exact
+// integers (P, S) from the matrix cores, their conversion, the products yd * d and yd * dmin --
+// the four operands of the two fused steps per super-block and cell, kept in registers.  After
+// one barrier it takes the first wave's sums from LDS and runs the chain itself: sixteen dependent
+// operations per cell.  Same integers, same f32 operations in the same order as the kernel
+// above: bit for bit.
 // The whole quantized activation (16 tokens x 4096 values) is staged once, before the only other
 // barrier; a workgroup is 8 waves = 4 row tiles, one per compute unit.  Each lane loads only the
 // nibble bytes it contracts itself (3 KB of requests per 2304-byte tile entry instead of 5 KB).
 // Measured at 14336 x 4096, cache-cold, us per launch: 16 tokens 11.7 -> 10.3, 4 tokens 11.4 -> 9.9.
 // Where the time goes (per-wave time stamps, medians): activation staged and first weights in at
 // 2.7 us, eight steps of 0.5-1.0 us (the first four wait for memory: all of a wave's first half
-// is requested at once), 0.9 us at the barrier for the slowest wave of the workgroup, 1.0 us for
-// the rest of the chain and the store.
+// is requested at once), 0.9 us at the barrier for the slowest wave of the workgroup, then the
+// chain, the store and the end of the launch.  (Parking the second wave's integers in LDS and
+// splitting the rest of the chain between both waves measured the same 10.3 us with more code.)
 struct Q4KMfmaPairArgs {
     const uint8_t *w;   // tiled layout [super-block][tile][2304 B]
     int64_t sb_stride;
@@ -385,8 +388,7 @@ struct Q4KMfmaPairArgs {
 constexpr int kPairSb = 16;    // most super-blocks per row
 constexpr int kPairPart = 8;   // most super-blocks per wave
 constexpr int kPairTiles = 4;  // row tiles per workgroup
-constexpr size_t kPairLds = static_cast<size_t>(kPairSb) * 16 * kSlabRow + kPairSb * 16 * 4 +
-                            static_cast<size_t>(kPairTiles) * kPairPart * (2 * 64 * 16 + 16 * 8) + kPairTiles * 64 * 8;
+constexpr size_t kPairLds = static_cast<size_t>(kPairSb) * 16 * kSlabRow + kPairSb * 16 * 4 + kPairTiles * 64 * 16;
 
 // FUSEQ (a few tokens): the f32 activation is quantized to Q8_K by the workgroup itself, a 16-lane
 // row per (token, super-block) with the device function the quantizer launch uses -- the same bytes
@@ -398,9 +400,7 @@ __global__ __launch_bounds__(512) void gemm_q4k_mfma_pair_kernel(Q4KMfmaPairArgs
     extern __shared__ uint4 smem[];
     uint8_t *act = reinterpret_cast<uint8_t *>(smem);                            // [kPairSb][16 tokens][kSlabRow]
     float *yds = reinterpret_cast<float *>(act + kPairSb * 16 * kSlabRow);        // [kPairSb][16 tokens]
-    v4i *terms = reinterpret_cast<v4i *>(yds + kPairSb * 16);                     // [tile][kPairPart][cells 0,1 | cells 2,3][lane]: P, S, P, S
-    float2 *dsc = reinterpret_cast<float2 *>(terms + kPairTiles * kPairPart * 2 * 64);  // [tile][kPairPart][row]: d, dmin
-    float2 *handoff = dsc + kPairTiles * kPairPart * 16;                          // [tile][lane]: the first wave's chains of cells 2 and 3
+    float4 *handoff = reinterpret_cast<float4 *>(yds + kPairSb * 16);             // [tile][lane]: the first wave's four chains
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
@@ -500,12 +500,11 @@ __global__ __launch_bounds__(512) void gemm_q4k_mfma_pair_kernel(Q4KMfmaPairArgs
 
     // Cell j of this lane: token 4 * kq + j of the tile's row n.
     float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-    auto chain_cell = [&](int j, float yv, int P, int S, float dw, float dminw) __attribute__((always_inline)) {
-        const float Dd = yv * dw;
-        const float Mm = yv * dminw;
-        acc[j] = __builtin_fmaf(-Mm, static_cast<float>(P), acc[j]);
-        acc[j] = __builtin_fmaf(Dd, static_cast<float>(S), acc[j]);
-    };
+    // The second wave cannot chain yet (its chain starts where the first wave's ends), but everything
+    // of a step that does not depend on the running sum can be done now: it keeps, per super-block
+    // and cell, the four operands of the two fused steps.  What is left for after the barrier is
+    // the chain itself, sixteen dependent operations per cell.
+    float keep[kPairPart][4][4];  // {-(yd * dmin), float(P), yd * d, float(S)}
 
 #pragma unroll
     for (int i = 0; i < kPairPart; i++) {
@@ -541,54 +540,52 @@ __global__ __launch_bounds__(512) void gemm_q4k_mfma_pair_kernel(Q4KMfmaPairArgs
                 }
             }
             const v4i S = Slo + Shi * 8;
-            if (kd == 0) {
-                const float4 ydv = *reinterpret_cast<const float4 *>(yds + sb * 16 + cell_tok);
-                chain_cell(0, ydv.x, P[0], S[0], dw, dminw);
-                chain_cell(1, ydv.y, P[1], S[1], dw, dminw);
-                chain_cell(2, ydv.z, P[2], S[2], dw, dminw);
-                chain_cell(3, ydv.w, P[3], S[3], dw, dminw);
-            } else {
-                // the exact integers of this super-block, with the row's d and dmin: cells 0 and 1 for
-                // the first wave, cells 2 and 3 for this one after the barrier
-                terms[((rt * kPairPart + i) * 2) * 64 + lane] = v4i{P[0], S[0], P[1], S[1]};
-                terms[((rt * kPairPart + i) * 2 + 1) * 64 + lane] = v4i{P[2], S[2], P[3], S[3]};
-                if (kq == 0) dsc[(rt * kPairPart + i) * 16 + n] = make_float2(dw, dminw);
+            const float4 ydv = *reinterpret_cast<const float4 *>(yds + sb * 16 + cell_tok);
+            const float yv[4] = {ydv.x, ydv.y, ydv.z, ydv.w};
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float Dd = yv[j] * dw;
+                const float Mm = yv[j] * dminw;
+                if (kd == 0) {
+                    acc[j] = __builtin_fmaf(-Mm, static_cast<float>(P[j]), acc[j]);
+                    acc[j] = __builtin_fmaf(Dd, static_cast<float>(S[j]), acc[j]);
+                } else {
+                    keep[i][j][0] = -Mm;
+                    keep[i][j][1] = static_cast<float>(P[j]);
+                    keep[i][j][2] = Dd;
+                    keep[i][j][3] = static_cast<float>(S[j]);
+                }
             }
         }
         if (i + 4 < kPairPart) load_slot(ring[i & 3], i + 4);
     }
-    // the first wave hands the chains of cells 2 and 3 to the second
-    if (kd == 0) handoff[rt * 64 + lane] = make_float2(acc[2], acc[3]);
+    // the first wave hands its chains to the second and is done
+    if (kd == 0) handoff[rt * 64 + lane] = make_float4(acc[0], acc[1], acc[2], acc[3]);
     __syncthreads();
-
-    // The rest of every chain, the second wave's super-blocks in order: cells 0 and 1 in the first
-    // wave, cells 2 and 3 in the second.  One small rolled loop for both: this is code no wave has
-    // run yet, reached by all of them at once, and every instruction line of it is a fetch the
-    // whole workgroup waits for (an unrolled version of these 16 steps took 0.85 us).
-    float c0 = kd ? 0.0f : acc[0], c1 = kd ? 0.0f : acc[1];
-    if (kd) {
-        const float2 h = handoff[rt * 64 + lane];
-        c0 = h.x;
-        c1 = h.y;
+    if (kd == 0) return;
+    {
+        const float4 h = handoff[rt * 64 + lane];
+        acc[0] = h.x;
+        acc[1] = h.y;
+        acc[2] = h.z;
+        acc[3] = h.w;
     }
-    const v4i *tp = terms + ((rt * kPairPart) * 2 + kd) * 64 + lane;
-    const float2 *dp = dsc + (rt * kPairPart) * 16 + n;
-    const float *yp = yds + a.s_mid * 16 + cell_tok + 2 * kd;
-#pragma unroll 1
-    for (int i = 0; i < n_sb - a.s_mid; i++) {
-        const v4i t = tp[i * 128];
-        const float2 ds = dp[i * 16];
-        const float2 yv = *reinterpret_cast<const float2 *>(yp + i * 16);
-        c0 = __builtin_fmaf(-(yv.x * ds.y), static_cast<float>(t[0]), c0);
-        c0 = __builtin_fmaf(yv.x * ds.x, static_cast<float>(t[1]), c0);
-        c1 = __builtin_fmaf(-(yv.y * ds.y), static_cast<float>(t[2]), c1);
-        c1 = __builtin_fmaf(yv.y * ds.x, static_cast<float>(t[3]), c1);
+#pragma unroll
+    for (int i = 0; i < kPairPart; i++) {
+        if (i < n_loc) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                acc[j] = __builtin_fmaf(keep[i][j][0], keep[i][j][1], acc[j]);
+                acc[j] = __builtin_fmaf(keep[i][j][2], keep[i][j][3], acc[j]);
+            }
+        }
     }
     if (tile < n_tiles && row >= 0 && row < a.rows) {
-        const int t = cell_tok + 2 * kd;
-        float *o = a.out + static_cast<int64_t>(tok0 + t) * a.rows + row;
-        if (t < n_here) o[0] = c0;
-        if (t + 1 < n_here) o[a.rows] = c1;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int t = cell_tok + j;
+            if (t < n_here) a.out[static_cast<int64_t>(tok0 + t) * a.rows + row] = acc[j];
+        }
     }
 }
 
