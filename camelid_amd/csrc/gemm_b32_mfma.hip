@@ -351,6 +351,188 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_b32_mfma_kernel(B32MfmaArgs a
     }
 }
 
+// ---- up to 16 tokens, short rows, few row tiles: KD waves per row tile ------------------------------
+//
+// A matrix of 512 row tiles is 512 waves for the kernel above, each walking its tile's blocks alone
+// on its SIMD: 24 thousand cycles per wave of which the vector and matrix instructions are a
+// third -- the rest is one instruction waiting for the one before it (counters: 1561 vector
+// instructions, 64 matrix instructions, 4900 cycles of s_waitcnt in 24461).  What is ordered in
+// the reference's sum is only the chain  acc = acc + term_b  over the blocks of a row; a block's
+// term  (float(isum) * d_w) * d_x  does not depend on the running sum.  So KD waves share a row
+// tile, each taking one run of the row's 256-value slabs (all of them requested at entry): wave 0
+// chains its terms as it goes, the others keep theirs in registers, and the running sums are
+// handed from wave to wave through LDS behind KD - 1 barriers, each wave adding its terms in
+// block order -- the reference's association bit for bit, with KD times the waves.
+// SPW = most slabs per wave (rows of up to KD * SPW slabs), TPW = row tiles per workgroup (they share the staged activation).
+template <int FMT, int KD, int SPW, int TPW>
+__global__ __launch_bounds__(64 * KD * TPW) void gemm_b32_mfma_kpar_kernel(B32MfmaArgs a) {
+    constexpr int nthreads = 64 * KD * TPW;
+    constexpr int kStage = 256 * KD * SPW / nthreads;  // 16-byte activation pieces per thread for the longest row
+    static_assert(kStage >= 1 && 256 % nthreads == 0 || nthreads % 256 == 0, "staging passes are whole slabs or whole fractions of one");
+    extern __shared__ uint4 smem[];
+    const int n_slabs = a.n_slabs, nb = n_slabs * 8;
+    uint8_t *act = reinterpret_cast<uint8_t *>(smem);                                   // [n_slabs][16 tokens][kB32SlabRow]
+    int *bs = reinterpret_cast<int *>(act + n_slabs * 16 * kB32SlabRow);                // Q4_0: [nb][16 tokens] -8 * block sums
+    float *xss = reinterpret_cast<float *>(bs + (FMT == CML_Q4_0 ? nb * 16 : 0));       // [nb][16 tokens]
+    float4 *handoff_all = reinterpret_cast<float4 *>(xss + nb * 16);                    // [TPW][64 lanes]
+
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    const int kd = wave % KD, tw = wave / KD;
+    float4 *handoff = handoff_all + tw * 64;
+    const int n = lane & 15, kq = lane >> 4;
+    const int n_tiles = (a.rows + 15) / 16;
+    const int tile = blockIdx.x * TPW + tw;
+    const int row = tile * 16 + n;
+    const int tok0 = blockIdx.y * 16;
+    const int n_here = min(16, a.n_tokens - tok0);
+    auto act_row = [&](int t) __attribute__((always_inline)) -> int64_t { return tok0 + min(t, n_here - 1); };
+    // this wave's slabs: [s_begin, s_begin + n_loc), at most SPW
+    const int s_begin = kd * n_slabs / KD, n_loc = (kd + 1) * n_slabs / KD - s_begin;
+
+    // activation pieces first (cache hits; the stores below then never wait behind a weight load)
+    v4i_b32 sreg[kStage];
+#pragma unroll
+    for (int k = 0; k < kStage; k++) {
+        const int i = tid + k * nthreads;  // piece (slab, token, pc)
+        if (i < n_slabs * 256) {
+            const int slab = i >> 8, t = (i >> 4) & 15, pc = i & 15;
+            sreg[k] = reinterpret_cast<const v4i_b32 *>(a.q + (act_row(t) * n_slabs + slab) * 256)[pc];
+        }
+    }
+    const int64_t arow = min(row, a.rows - 1);
+    const uint8_t *qlane = a.quants + arow * a.q_stride + 16 * kq;
+    const uint8_t *srow = a.scales + arow * a.s_stride;
+    B32SlabWeights<FMT> ring[SPW];
+#pragma unroll
+    for (int i = 0; i < SPW; i++)
+        if (i < n_loc) b32_mfma_load<FMT>(ring[i], qlane, srow, s_begin + i);  // wave-uniform
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int k = 0; k < kStage; k++) {
+        const int i = tid + k * nthreads;
+        const int slab = i >> 8, t = (i >> 4) & 15, pc = i & 15, blk = pc >> 1, h = pc & 1;
+        if (i >= n_slabs * 256) continue;
+        if (slab < n_slabs) {
+            uint8_t *dst = act + (slab * 16 + t) * kB32SlabRow;
+            const v4i_b32 v = sreg[k];
+            if constexpr (FMT == CML_Q8_0) {
+                dst += (blk >> 1) * 64 + h * 16 + (blk & 1) * 8;
+                *reinterpret_cast<v2i_b32 *>(dst) = v2i_b32{v.x, v.y};
+                *reinterpret_cast<v2i_b32 *>(dst + 32) = v2i_b32{v.z, v.w};
+            } else {
+                dst += (blk >> 1) * 64 + (blk & 1) * 8 + h * 4;
+                *reinterpret_cast<int *>(dst) = v.x;
+                *reinterpret_cast<int *>(dst + 16) = v.y;
+                *reinterpret_cast<int *>(dst + 32) = v.z;
+                *reinterpret_cast<int *>(dst + 48) = v.w;
+            }
+        }
+        if constexpr (FMT == CML_Q4_0) {
+            // the block's -8 * sum of activations: the two halves sit in adjacent lanes, which swap partial sums
+            const v4i_b32 v = sreg[k];
+            int sum = sdot4(static_cast<uint32_t>(v.x), 0x01010101u, 0);
+            sum = sdot4(static_cast<uint32_t>(v.y), 0x01010101u, sum);
+            sum = sdot4(static_cast<uint32_t>(v.z), 0x01010101u, sum);
+            sum = sdot4(static_cast<uint32_t>(v.w), 0x01010101u, sum);
+            sum += __builtin_amdgcn_update_dpp(0, sum, 0xB1 /* quad_perm [1,0,3,2] */, 0xf, 0xf, false);
+            if (slab < n_slabs) bs[(slab * 8 + blk) * 16 + t] = -8 * sum;
+        }
+    }
+    for (int i = tid; i < nb * 16; i += nthreads) {
+        const int b = i >> 4, t = i & 15;
+        xss[i] = a.xs[act_row(t) * nb + b];
+    }
+    __syncthreads();
+
+    const int a_off = n * kB32SlabRow + 16 * kq;
+    const int cell_tok = 4 * kq;
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    float keep[SPW][8][4];
+#pragma unroll
+    for (int i = 0; i < SPW; i++) {
+        if (i < n_loc) {
+            const int slab = s_begin + i;
+            const B32SlabWeights<FMT> &w0 = ring[i];
+            const uint32_t dwords[4] = {w0.d.x, w0.d.y, w0.d.z, w0.d.w};
+            long bw8[8];
+            b32_mfma_operands<FMT>(w0, bw8);
+            const uint8_t *abase = act + slab * (16 * kB32SlabRow) + a_off;
+#pragma unroll
+            for (int pr = 0; pr < 4; pr++) {
+                const v4i_b32 av = *reinterpret_cast<const v4i_b32 *>(abase + 64 * pr);
+                const long a2[2] = {
+                    static_cast<long>(static_cast<unsigned long long>(static_cast<uint32_t>(av.x)) | (static_cast<unsigned long long>(static_cast<uint32_t>(av.y)) << 32)),
+                    static_cast<long>(static_cast<unsigned long long>(static_cast<uint32_t>(av.z)) | (static_cast<unsigned long long>(static_cast<uint32_t>(av.w)) << 32))};
+                const float dw[2] = {f16_bits_to_f32(dwords[pr] & 0xffffu), f16_bits_to_f32(dwords[pr] >> 16)};
+#pragma unroll
+                for (int e = 0; e < 2; e++) {
+                    const int b = 2 * pr + e;
+                    v4i_b32 c = {0, 0, 0, 0};
+                    if constexpr (FMT == CML_Q4_0) c = *reinterpret_cast<const v4i_b32 *>(bs + (slab * 8 + b) * 16 + cell_tok);
+                    const v4i_b32 d = __builtin_amdgcn_mfma_i32_16x16x32_i8(a2[e], bw8[b], c, 0, 0, 0);
+                    const float4 xv = *reinterpret_cast<const float4 *>(xss + (slab * 8 + b) * 16 + cell_tok);
+                    const float t4[4] = {(static_cast<float>(d[0]) * dw[e]) * xv.x, (static_cast<float>(d[1]) * dw[e]) * xv.y,
+                                         (static_cast<float>(d[2]) * dw[e]) * xv.z, (static_cast<float>(d[3]) * dw[e]) * xv.w};
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        if (kd == 0) acc[j] = acc[j] + t4[j];
+                        else keep[i][b][j] = t4[j];
+                    }
+                }
+            }
+        }
+    }
+    // the running sums go from wave to wave, each adding its blocks in order
+#pragma unroll
+    for (int stage = 1; stage < KD; stage++) {
+        if (kd == stage - 1) handoff[lane] = make_float4(acc[0], acc[1], acc[2], acc[3]);
+        __syncthreads();
+        if (kd == stage) {
+            const float4 h = handoff[lane];
+            acc[0] = h.x;
+            acc[1] = h.y;
+            acc[2] = h.z;
+            acc[3] = h.w;
+#pragma unroll
+            for (int i = 0; i < SPW; i++) {
+                if (i < n_loc) {
+#pragma unroll
+                    for (int b = 0; b < 8; b++)
+#pragma unroll
+                        for (int j = 0; j < 4; j++) acc[j] = acc[j] + keep[i][b][j];
+                }
+            }
+        }
+        // (the next stage's writer is the wave that has just read the slot: no second barrier)
+    }
+    if (kd == KD - 1 && tile < n_tiles && row < a.rows) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int t = cell_tok + j;
+            if (t < n_here) a.out[static_cast<int64_t>(tok0 + t) * a.rows + row] = acc[j];
+        }
+    }
+}
+
+template <int FMT, int KD, int SPW, int TPW>
+static int launch_b32_mfma_kpar(const B32MfmaArgs &ka, hipStream_t st) {
+    const int n_tiles = (ka.rows + 15) / 16;
+    const int nb = ka.n_slabs * 8;
+    const size_t lds = static_cast<size_t>(ka.n_slabs) * 16 * kB32SlabRow + (FMT == CML_Q4_0 ? static_cast<size_t>(nb) * 16 * 4 : 0) +
+                       static_cast<size_t>(nb) * 16 * 4 + TPW * 64 * 16;
+    static bool raised = false;
+    if (!raised) {
+        CML_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_b32_mfma_kpar_kernel<FMT, KD, SPW, TPW>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        raised = true;
+    }
+    hipLaunchKernelGGL((gemm_b32_mfma_kpar_kernel<FMT, KD, SPW, TPW>),
+                       dim3(static_cast<unsigned>((n_tiles + TPW - 1) / TPW), static_cast<unsigned>((ka.n_tokens + 15) / 16)), dim3(64 * KD * TPW), lds, st, ka);
+    CML_HIP_TRY(hipGetLastError());
+    return CML_OK;
+}
+
 template <int FMT, int GPW, int TB, int KC, int RING, bool PLAIN, int WAVES = 4>
 static int launch_b32_mfma_gp(const B32MfmaArgs &ka, int n_groups, hipStream_t st) {
     constexpr int NTOK = 16 * GPW * TB, RT = WAVES / TB;
@@ -412,6 +594,35 @@ static int launch_b32_mfma_fmt(const B32MfmaArgs &ka, int n_groups, bool grouped
     // Workgroup shape: token groups per wave x token blocks across waves.  Default: one wave per
     // row tile with 16 / 32 / 64 tokens; a matrix with fewer row tiles than the chip has SIMDs
     // spreads the tokens of a tile over 2 or 4 waves instead.
+    // Up to 16 tokens, rows of at most 16 slabs, few row tiles: several waves per row tile, one chain.
+    // Workgroup shapes by measurement (16 tokens, kernel us cache-cold, against the kernel below):
+    //   rows of <= 8 slabs:  <= 256 tiles: 8 waves per tile (4096 x 2048 Q8_0 10.0 -> 6.0);
+    //                        <= 768 tiles: 4 waves per tile, 2 tiles per workgroup (8192 x 2048 Q8_0 10.6 -> 8.0, Q4_0 11.8 -> 7.0);
+    //                        more tiles: no gain (16384 x 2048 12.3 -> 12.2), the kernel below stays;
+    //   rows of 9..16 slabs: the staged activation fills half of a compute unit's LDS, one workgroup per unit:
+    //                        <= 256 tiles: 8 waves per tile (4096 x 4096 Q8_0 15.6 -> 10.8, Q4_0 18.6 -> 8.8);
+    //                        <= 512 tiles: the same, 2 tiles per workgroup (8192 x 4096 Q8_0 16.9 -> 14.3, Q4_0 19.1 -> 11.1);
+    //                        896 tiles lose (14336 x 4096 20.6 -> 26.0).
+    const int kpar = env_int("CAMELID_HIP_B32_MFMA_KPAR", -1);
+    const int tiles = (ka.rows + 15) / 16;
+    if (!grouped && ka.n_tokens <= 16 && env_int("CAMELID_HIP_B32_MFMA_SHAPE", 0) == 0 && kpar != 0) {
+        if (ka.n_slabs >= 4 && ka.n_slabs <= 8) {
+            if (kpar == 1) return launch_b32_mfma_kpar<FMT, 4, 2, 1>(ka, st);
+            if (kpar == 2) return launch_b32_mfma_kpar<FMT, 4, 2, 2>(ka, st);
+            if (kpar == 3) return launch_b32_mfma_kpar<FMT, 8, 1, 1>(ka, st);
+            if (kpar == 4) return launch_b32_mfma_kpar<FMT, 8, 1, 2>(ka, st);
+            if (tiles <= 256) return launch_b32_mfma_kpar<FMT, 8, 1, 1>(ka, st);
+            if (tiles <= 768) return launch_b32_mfma_kpar<FMT, 4, 2, 2>(ka, st);
+        } else if (ka.n_slabs > 8 && ka.n_slabs <= 16) {
+            if (kpar == 1) return launch_b32_mfma_kpar<FMT, 4, 4, 1>(ka, st);
+            if (kpar == 2) return launch_b32_mfma_kpar<FMT, 8, 2, 1>(ka, st);
+            if (kpar == 3) return launch_b32_mfma_kpar<FMT, 8, 2, 2>(ka, st);
+            if (tiles <= 256) return launch_b32_mfma_kpar<FMT, 8, 2, 1>(ka, st);
+            if (tiles <= 512) return launch_b32_mfma_kpar<FMT, 8, 2, 2>(ka, st);
+        } else if (ka.n_slabs >= 2 && ka.n_slabs < 4 && (kpar > 0 || tiles <= 768)) {
+            return launch_b32_mfma_kpar<FMT, 2, 2, 1>(ka, st);
+        }
+    }
     switch (env_int("CAMELID_HIP_B32_MFMA_SHAPE", 0)) {
         case 1: return launch_b32_mfma_p<FMT, 1, 1>(ka, n_groups, st);   // 16 tokens, 1 wave per row tile
         case 2: return launch_b32_mfma_p<FMT, 2, 1>(ka, n_groups, st);   // 32 tokens, 1 wave per row tile

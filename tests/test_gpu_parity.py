@@ -642,6 +642,30 @@ def test_b32_matrix_core_cells_are_bitwise_the_gemv(name, fmt, rows, cols):
 
 
 @pytest.mark.parametrize("name,fmt", [("Q8_0", oracle.Q8_0), ("Q4_0", oracle.Q4_0)])
+@pytest.mark.parametrize("rows,cols", [(130, 2 * 256), (45, 3 * 256), (2049, 5 * 256), (500, 8 * 256), (77, 12 * 256),
+                                       (4100, 16 * 256), (16, 4 * 256)])
+def test_b32_waves_sharing_a_row_tile_keep_the_block_order(name, fmt, rows, cols):
+    """Up to 16 tokens on a matrix of few row tiles: 2, 4 or 8 waves share a row tile, each taking a
+    run of the row's slabs, and hand the running sums on in order -- the block-order chain of the
+    reference bit for bit, in every workgroup shape (CAMELID_HIP_B32_MFMA_KPAR = 1..4; 0 = one wave
+    per tile), on ragged row counts and with a token count that leaves cells unused."""
+    rng = np.random.default_rng(rows * 3 + cols + fmt)
+    wire = G.synth_weight(fmt, rows, cols, seed=rows + cols * 7 + fmt)
+    w = Weight.upload(fmt, rows, cols, wire)
+    for n in (3, 9, 16):
+        x = rng.standard_normal((n, cols)).astype(np.float32)
+        x[n - 1, :64] = 0.0
+        s, q = oracle.quantize_activation(fmt, x)
+        want = oracle.matmul_q(fmt, wire, cols, s, q, order=oracle.ORDER_PRIMARY, threads=8)
+        with G.env(CAMELID_HIP_B32_MFMA_MIN_TOKENS=1):
+            for variant in (-1, 0, 1, 2, 3, 4):
+                G.say(f"{name} waves per tile, {rows}x{cols} n={n} variant={variant}")
+                with G.env(CAMELID_HIP_B32_MFMA_MIN_TOKENS=1, CAMELID_HIP_B32_MFMA_KPAR=variant):
+                    got = G.gpu_gemm(w, s, q)
+                assert G.same_bits(got, want)
+
+
+@pytest.mark.parametrize("name,fmt", [("Q8_0", oracle.Q8_0), ("Q4_0", oracle.Q4_0)])
 def test_b32_rows_that_are_not_whole_slabs_take_the_packed_dot_kernel(name, fmt):
     rows, cols, n = 40, 352, 9     # 11 blocks: not a multiple of 8
     wire = G.synth_weight(fmt, rows, cols, seed=77 + fmt)
