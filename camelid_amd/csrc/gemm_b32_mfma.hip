@@ -368,7 +368,7 @@ template <int FMT, int KD, int SPW, int TPW>
 __global__ __launch_bounds__(64 * KD * TPW) void gemm_b32_mfma_kpar_kernel(B32MfmaArgs a) {
     constexpr int nthreads = 64 * KD * TPW;
     constexpr int kStage = 256 * KD * SPW / nthreads;  // 16-byte activation pieces per thread for the longest row
-    static_assert(kStage >= 1 && 256 % nthreads == 0 || nthreads % 256 == 0, "staging passes are whole slabs or whole fractions of one");
+    static_assert(kStage >= 1 && kStage * nthreads == 256 * KD * SPW, "the threads of a workgroup stage the longest row in whole passes");
     extern __shared__ uint4 smem[];
     const int n_slabs = a.n_slabs, nb = n_slabs * 8;
     uint8_t *act = reinterpret_cast<uint8_t *>(smem);                                   // [n_slabs][16 tokens][kB32SlabRow]

@@ -673,7 +673,6 @@ __global__ __launch_bounds__(256) void gemv_b32_grouped_kernel(B32GroupArgs a) {
     const uint8_t *qrow = a.quants + arow * a.q_stride;
     const uint8_t *srow = a.scales + arow * a.s_stride;
     const bool leader = (l == P - 1);
-    const int n_steps = (nb + P - 1) / P;
 
     // Stage the activation rows of assignments a0+c0 .. (nt of them, `staged` slots filled).
     auto stage = [&](int c0, int nt, int staged) {

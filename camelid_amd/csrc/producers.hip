@@ -100,7 +100,7 @@ __device__ __forceinline__ float ordered_sum_nonneg(const float4 *xs4, int c4, i
     __shared__ int s_head[kSumThreads];      // first thread of the group ending at thread t
     __shared__ int s_count[kSumWaves];       // groups per wave
     __shared__ uint16_t s_list[kSumWaves][64];  // the last threads of a wave's groups, in order
-    const int lane = tid & 63, wave = tid >> 6, rl = lane & 15, row = lane >> 4;
+    const int lane = tid & 63, wave = tid >> 6, row = lane >> 4;
     const float4 *mine = xs4 + tid * c4;
 
     // 1. chunk sums and their exclusive scan (the association of this approximation is free):
