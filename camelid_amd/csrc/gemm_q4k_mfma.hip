@@ -17,16 +17,18 @@
 // packed 16-bit multiply per four weights (a byte pair times a digit never
 // carries into its neighbour), independent of the token count.
 //
-// Instruction: v_mfma_i32_16x16x64_i8, K = 64 = one 32-byte chunk of the block
-// (its low nibbles = sub-block 2c, its high nibbles = sub-block 2c+1):
-//     A[t][k]  = y_t[64c + k]                          16 tokens, from LDS
-//     B[k][n]  = digit-scaled nibble k of row n        16 rows, built in registers
-//     D[t][n] += ...                                   over the 4 chunks
-// Lane L supplies A-row t = L%16 and B-column n = L%16 at k = 16*(L/16)..+15 (its
-// piece a or b of the chunk, low or high nibbles: ONE sub-block per lane and
-// chunk, hence one scale digit pair), and receives D[4*(L/16)+v][L%16], v < 4:
-// four tokens of one weight row, whose f32 chains live in that lane, in
-// super-block order.
+// Instruction: v_mfma_i32_16x16x64_i8.  One instruction contracts 64 values of ONE nibble plane
+// (low nibbles = the even sub-block of a 32-byte chunk, high nibbles = the odd one) taken from two
+// chunks, ch = 2q + half for q = 0, 1 -- the contraction index may be assigned freely as long as
+// both operands agree, and the sum is an exact integer:
+//     A[t][k]  = y_t[64ch + 32plane + 16p + j]         16 tokens, from LDS
+//     B[k][n]  = digit-scaled nibble `plane` of byte j of piece p of chunk ch of row n
+//     D[t][n] += ...                                   over the 4 steps (q, plane) of a super-block
+// Lane L supplies A-row t = L%16 and B-column n = L%16 at k = 16*(L/16)..+15, where L/16 = 2*half + p:
+// piece p (a or b) of chunk ch -- so a lane loads the 16 bytes of ONE piece of TWO chunks, both
+// nibbles of every byte are its own (one sub-block per lane and step, hence one scale digit pair),
+// and the 64 lanes of a load cover 1024 distinct bytes.  It receives D[4*(L/16)+v][L%16], v < 4:
+// four tokens of one weight row, whose f32 chains live in that lane, in super-block order.
 //
 // A workgroup is 4 waves: 4/TB consecutive 16-row tiles x TB token blocks of
 // 16*GPW tokens, sharing the staged activations of NTOK = 16*GPW*TB tokens.  K is
@@ -75,15 +77,15 @@ struct Q4KMfmaArgs {
 
 struct MfmaWeights {
     uint4 hdr;
-    uint4 piece[4];  // this lane's 16 nibble bytes of each of the 4 chunks
+    uint4 piece[2];  // this lane's 16 nibble bytes of the two chunks it contracts (both nibbles of every byte are its own)
 };
 
-// hdr_ptr / piece_ptr already include the lane's offsets inside a chunk; `off` = sb * sb_stride.
+// hdr_ptr / piece_ptr already include the lane's offsets inside a tile entry; `off` = sb * sb_stride.
 __device__ __forceinline__ void mfma_load_weights(MfmaWeights &r, const uint8_t *hdr_ptr, const uint8_t *piece_ptr,
                                                   int64_t off) {
     r.hdr = ldg16(hdr_ptr + off);
-#pragma unroll
-    for (int c = 0; c < 4; c++) r.piece[c] = ldg16(piece_ptr + off + c * 16);
+    r.piece[0] = ldg16(piece_ptr + off);
+    r.piece[1] = ldg16(piece_ptr + off + 32);
 }
 
 __device__ __forceinline__ v4i as_v4i(const uint4 &v) {
@@ -186,13 +188,15 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
 
     // Lane constants.
     const uint8_t *w_hdr = wtile + n * 16;
-    const uint8_t *w_piece = wtile + ((kq & 1) ? 1280 : 256) + n * 64;   // piece a (values 0..15) or b (16..31) of chunk 0
-    const int nib_shift = 4 * half;                                       // low nibbles = sub-block 2c, high = 2c+1
-    // A operand: this lane is token (lane & 15) of a group, bytes 16*kq..+15 of a chunk.
-    const int a_off = (lane & 15) * kSlabRow + 16 * kq;  // + 64c, + token-group and slot offsets
+    // A matrix instruction contracts 64 values of ONE nibble plane of two 32-byte chunks, ch = 2 * q + half
+    // (q = 0, 1): the lane needs piece a (values 0..15) or b (16..31) of those two chunks only, and the 64
+    // lanes of a load cover 1024 distinct bytes of the tile entry.
+    const uint8_t *w_piece = wtile + ((kq & 1) ? 1280 : 256) + n * 64 + half * 16;
+    // A operand: this lane is token (lane & 15) of a group; step (q, plane) takes bytes 128q + 64half + 32plane + 16(kq&1) .. +15.
+    const int a_off = (lane & 15) * kSlabRow + 64 * half + 16 * (kq & 1);  // + 128q + 32plane, + token-group and slot offsets
     // D values v = 0..3 of this lane: tokens 4*kq + v of the group, weight row n.
     const int cell_tok = 4 * kq;
-    const int sc_shift = 8 * half;                  // byte `half` / `2+half` of the scale words
+    const int sc_shift = 16 * half;                 // scales of sub-blocks 2*half, 2*half+1 (and +4) within their words
 
     // A wave streams its tile through a ring of RING register slots: slot i is
     // refilled with super-block sb + RING right after super-block sb has been
@@ -232,28 +236,31 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
             part++;
             next_cut = (part + 1) * n_sb / a.ksplit;
         }
-        // this row's scales and mins of the sub-blocks {half, 2+half, 4+half, 6+half}
+        // this row's scales and mins of the sub-blocks {2half, 2half+1, 4+2half, 5+2half}
         // (reference q4_k_scale_min, src/tensor/mod.rs:5997-6006)
         uint32_t sc03, sc47, m03, m47;
         q4k_unpack_scales(w0.hdr.y, w0.hdr.z, w0.hdr.w, sc03, sc47, m03, m47);
         const float dw = f16_bits_to_f32(w0.hdr.x & 0xffffu);
         const float dminw = f16_bits_to_f32(w0.hdr.x >> 16);
-        v4i blo[4], bhi[4], bm[4];
+        v4i blo[4], bhi[4], bm[4];  // step c = 2 * q + plane
 #pragma unroll
-        for (int c = 0; c < 4; c++) {
-            const uint32_t scw = (c < 2) ? sc03 : sc47, mw = (c < 2) ? m03 : m47;
-            const int sh = sc_shift + 16 * (c & 1);
-            const uint32_t scale = (scw >> sh) & 0xff;
-            const uint32_t lo = scale & 7u, hi = scale >> 3;
-            const uint32_t lo2 = lo | (lo << 16), hi2 = hi | (hi << 16);
-            const uint32_t m = (mw >> sh) & 0xff;
-            const int m4 = static_cast<int>(__builtin_amdgcn_perm(m, m, 0u));  // byte 0 (m < 64) in all four bytes
-            bm[c] = v4i{m4, m4, m4, m4};
-            const uint4 &pc = w0.piece[c];
-            const uint32_t n0 = (pc.x >> nib_shift) & 0x0f0f0f0fu, n1 = (pc.y >> nib_shift) & 0x0f0f0f0fu;
-            const uint32_t n2 = (pc.z >> nib_shift) & 0x0f0f0f0fu, n3 = (pc.w >> nib_shift) & 0x0f0f0f0fu;
-            blo[c] = v4i{scale_bytes(n0, lo2), scale_bytes(n1, lo2), scale_bytes(n2, lo2), scale_bytes(n3, lo2)};
-            bhi[c] = v4i{scale_bytes(n0, hi2), scale_bytes(n1, hi2), scale_bytes(n2, hi2), scale_bytes(n3, hi2)};
+        for (int q = 0; q < 2; q++) {
+            const uint32_t scw = (q ? sc47 : sc03) >> sc_shift, mw = (q ? m47 : m03) >> sc_shift;
+            const uint4 &pc = w0.piece[q];
+#pragma unroll
+            for (int plane = 0; plane < 2; plane++) {  // low nibbles = sub-block 2 * ch, high = 2 * ch + 1
+                const int c = 2 * q + plane;
+                const uint32_t scale = (scw >> (8 * plane)) & 0xff;
+                const uint32_t lo = scale & 7u, hi = scale >> 3;
+                const uint32_t lo2 = lo | (lo << 16), hi2 = hi | (hi << 16);
+                const uint32_t m = (mw >> (8 * plane)) & 0xff;
+                const int m4 = static_cast<int>(__builtin_amdgcn_perm(m, m, 0u));  // byte 0 (m < 64) in all four bytes
+                bm[c] = v4i{m4, m4, m4, m4};
+                const uint32_t n0 = (pc.x >> (4 * plane)) & 0x0f0f0f0fu, n1 = (pc.y >> (4 * plane)) & 0x0f0f0f0fu;
+                const uint32_t n2 = (pc.z >> (4 * plane)) & 0x0f0f0f0fu, n3 = (pc.w >> (4 * plane)) & 0x0f0f0f0fu;
+                blo[c] = v4i{scale_bytes(n0, lo2), scale_bytes(n1, lo2), scale_bytes(n2, lo2), scale_bytes(n3, lo2)};
+                bhi[c] = v4i{scale_bytes(n0, hi2), scale_bytes(n1, hi2), scale_bytes(n2, hi2), scale_bytes(n3, hi2)};
+            }
         }
         const float *ydp = yds + sb * NTOK + tb * (16 * GPW) + cell_tok;
 #pragma unroll
@@ -262,7 +269,7 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
             v4i Slo = {0, 0, 0, 0}, Shi = {0, 0, 0, 0}, P = {0, 0, 0, 0};
 #pragma unroll
             for (int c = 0; c < 4; c++) {
-                const v4i av = *reinterpret_cast<const v4i *>(ybase + 64 * c);
+                const v4i av = *reinterpret_cast<const v4i *>(ybase + 128 * (c >> 1) + 32 * (c & 1));
                 Slo = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, blo[c], Slo, 0, 0, 0);
                 Shi = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, bhi[c], Shi, 0, 0, 0);
                 P = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, bm[c], P, 0, 0, 0);
