@@ -320,22 +320,28 @@ def bench_moe(name: str, K: int, W: int, seed: int, cpu_seconds: float) -> int:
     for i in range(W):
         step(i)
     check(L.cml_stream_sync(stream))
-    g = capture(stream, step, K)
     timers = [timer] + [Timer(stream) for _ in range(31)]
-    ms = time_graph_median(stream, g, timers)[0] / K
+    # per step = (median 2K-step replay - median K-step replay) / K: the constant a replay pays for being launched drops out
+    g = capture(stream, step, K)
+    t_k = time_graph_median(stream, g, timers)[0]
+    g2 = capture(stream, step, 2 * K)
+    ms = (time_graph_median(stream, g2, timers)[0] - t_k) / K
     check(L.cml_stream_sync(stream))
     if not np.all(np.isfinite(out.to_numpy(np.float32, (T, hidden)))):
         print("non-finite output", file=sys.stderr)
         return 4
     gbs = alg_bytes / (ms * 1e-3) / 1e9
     if gemma:
-        # route, plan, [quantize,] gate|up, gelu*up->Q8_0, down, weighted sum
-        launches, kernel = (6 if T == 1 else 7), "gemv_b32_grouped_kernel (2 launches of the step)"
+        # one token: route, gate|up (quantizes the token itself), down (gelu*up->Q8_0 in its prologue), weighted sum;
+        # more: route, plan, quantize, gate|up, gelu*up->Q8_0, down, weighted sum
+        launches, kernel = (4 if T == 1 else 7), "gemv_b32_grouped_kernel (2 launches of the step)"
         what = "route (full softmax) + fused gate|up matvec + gelu_tanh*up->Q8_0 + down matvec + weighted sum, graph replay"
     else:
-        # route, plan, [quantize,] gate, up (one launch at 1 token), silu*up->Q8_K, down, weighted sum
-        launches, kernel = (6 if T == 1 else 8), "gemv_q4k_kernel / gemm_q4k_mfma_kernel grouped by expert (2-3 launches of the step)"
-        what = "route + gate/up matvecs + silu*up->Q8_K + down matvec + weighted sum, graph replay"
+        # one token: route, gate and up in one launch (quantizes the token itself), silu*up->Q8_K, down + weighted sum in one launch;
+        # more: route, plan, quantize, gate, up, silu*up->Q8_K, down, weighted sum
+        launches, kernel = (4 if T == 1 else 8), "gemv_q4k_kernel / gemm_q4k_mfma_kernel grouped by expert (2-3 launches of the step)"
+        what = ("route + gate/up matvecs + silu*up->Q8_K + down matvec + weighted sum (one token: folded into the down launch), "
+                "graph replay")
     line = {
         "metric": f"{fmt_name} mixture-of-experts FFN µs + achieved HBM GB/s, {E} experts top-{k}, {ff}x{hidden}, {T} token(s)",
         "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": W,
@@ -419,9 +425,11 @@ def time_read_only(stream, timers, nbytes: int, K: int, in_flight: int, groups: 
 
     for i in range(8):
         step(i)
-    g, g2 = capture(stream, step, K), capture(stream, step, 2 * K)
-    ms = (time_graph_median(stream, g2, timers)[0] - time_graph_median(stream, g, timers)[0]) / K
+    g = capture(stream, step, K)
+    t_k = time_graph_median(stream, g, timers)[0]
     check(L.cml_graph_destroy(g))
+    g2 = capture(stream, step, 2 * K)
+    ms = (time_graph_median(stream, g2, timers)[0] - t_k) / K
     check(L.cml_graph_destroy(g2))
     return ms * 1e3, bufs
 

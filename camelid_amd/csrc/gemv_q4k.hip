@@ -710,6 +710,152 @@ int launch_gemv_q4k_f32_grouped_pair(const MatArgs &a, const cml_weight *w2, flo
     return launch_q4k_f32(a, w2, out2, x, st);
 }
 
+// ---- mixture-of-experts decode: down projection of the routed experts + weighted sum, one launch ----
+//
+// One token, k routed experts, Q4_K down matrices stacked by expert.  The separate path is a launch
+// with grid.y = routed slot that writes y[slot][row], then a launch that mixes
+// out[row] = ((0 + y[0][row] * w[0]) + y[1][row] * w[1]) + ...  (reference src/inference.rs:14255-14257).
+// Here a workgroup owns one 16-row tile for ALL slots: its waves are slot x K part (the K cut of
+// the shape policy, as in the kernel above), every wave computes what its twin in the separate
+// launch computes, and after the one barrier the first 16 threads add each slot's partial chains
+// left to right and mix the slots in routed order -- the same operations in the same order,
+// without the second launch and without y going through memory.  Same number of waves per
+// launch as before (slots x parts x tiles); a slot whose expert id is out of range takes no part.
+struct MoeDownSumArgs {
+    const uint8_t *w;         // stacked experts, tiled layout
+    int64_t sb_stride;
+    int rows;                 // rows of one expert (a multiple of 16)
+    int n_sb, n_experts, n_slots;
+    int ksplit, ksplit_log2;
+    const int32_t *idx;       // [n_slots] routed expert of each slot
+    const float *weight;      // [n_slots]
+    const int8_t *q;          // [n_slots][n_sb*256]: every slot's own activation
+    const float *yd;          // [n_slots][n_sb]
+    float *out;               // [rows]
+};
+
+__global__ __launch_bounds__(512) void moe_down_sum_q4k_kernel(MoeDownSumArgs a) {
+    constexpr int U = 4;
+    using Regs = Q4KRegs<U>;
+    extern __shared__ uint4 smem[];
+    const int n_sb = a.n_sb, S = a.n_slots, W = a.ksplit;
+    int8_t *ys = reinterpret_cast<int8_t *>(smem);                     // [S][n_sb*256]
+    int *bsum = reinterpret_cast<int *>(ys + S * n_sb * 256);          // [S][n_sb*8]
+    float *yds = reinterpret_cast<float *>(bsum + S * n_sb * 8);       // [S][n_sb]
+    float *part = yds + ((S * n_sb + 3) & ~3);                         // [S][W][16]
+
+    const int tid = threadIdx.x, nthreads = blockDim.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    const int slot = wave >> a.ksplit_log2, kpart = wave & (W - 1);
+    const int expert = a.idx[slot];
+    const bool served = expert >= 0 && expert < a.n_experts;   // wave-uniform
+    const int tile = blockIdx.x;
+    const int s0 = (kpart * n_sb) >> a.ksplit_log2, s1 = ((kpart + 1) * n_sb) >> a.ksplit_log2;
+    const int r = lane / LPS, l = lane - r * LPS;
+    const uint8_t *wtile = a.w + (static_cast<int64_t>(served ? expert : 0) * (a.rows / 16) + tile) * kQ4KChunk;
+    const int piece = r * LPS + l;
+    Q4KLane ln;
+    ln.c = l;
+    ln.sh = (ln.c & 1) * 16;
+    ln.upper = ln.c >= 2;
+    auto load_buffer = [&](Regs &dst, int sb) __attribute__((always_inline)) { q4k_load<U, 1>(dst, wtile, a.sb_stride, r, piece, sb, s1); };
+
+    // every slot's activation row into LDS, with the 32-value sums; the first weight buffer goes out
+    // behind the first activation loads
+    Regs ra, rb;
+    const int c16 = n_sb * 16, n16 = S * c16;
+    uint4 *dst = reinterpret_cast<uint4 *>(ys);
+    const uint4 *src = reinterpret_cast<const uint4 *>(a.q);
+    uint4 first = src[min(tid, n16 - 1)];
+    __builtin_amdgcn_sched_barrier(0);
+    if (served) load_buffer(ra, s0);
+    __builtin_amdgcn_sched_barrier(0);
+    for (int i = tid; i < n16 + (n16 & 1); i += nthreads) {  // lanes 2k, 2k+1 stay together for the pair sum
+        const uint4 v = i == tid ? first : src[min(i, n16 - 1)];
+        int sum = bytesum16(v);
+        sum += row_shr_i32<1>(sum);
+        if (i < n16) {
+            dst[i] = v;
+            if (i & 1) bsum[i >> 1] = sum;
+        }
+    }
+    for (int i = tid; i < S * n_sb; i += nthreads) yds[i] = a.yd[i];
+    __syncthreads();
+
+    float acc[1] = {0.0f};
+    if (served) {
+        const int8_t *ys_s = ys + slot * n_sb * 256;
+        const int *bsum_s = bsum + slot * n_sb * 8;
+        const float *yds_s = yds + slot * n_sb;
+        for (int sb = s0;;) {
+            if (sb + U >= s1) {
+                q4k_compute<1, false, U, 1>(ra, ln, sb, s1, ys_s, bsum_s, yds_s, n_sb, acc, nullptr);
+                break;
+            }
+            load_buffer(rb, sb + U);
+            __builtin_amdgcn_sched_barrier(0);
+            q4k_compute<1, false, U, 1>(ra, ln, sb, s1, ys_s, bsum_s, yds_s, n_sb, acc, nullptr);
+            __builtin_amdgcn_sched_barrier(0);
+            sb += U;
+            if (sb + U >= s1) {
+                q4k_compute<1, false, U, 1>(rb, ln, sb, s1, ys_s, bsum_s, yds_s, n_sb, acc, nullptr);
+                break;
+            }
+            load_buffer(ra, sb + U);
+            __builtin_amdgcn_sched_barrier(0);
+            q4k_compute<1, false, U, 1>(rb, ln, sb, s1, ys_s, bsum_s, yds_s, n_sb, acc, nullptr);
+            __builtin_amdgcn_sched_barrier(0);
+            sb += U;
+        }
+    }
+    if (l == LPS - 1) part[wave * 16 + r] = acc[0];
+    __syncthreads();
+    if (tid < 16) {
+        const int row = tile * 16 + tid;
+        float mix = 0.0f;
+        for (int s = 0; s < S; s++) {
+            const int e = a.idx[s];
+            if (e < 0 || e >= a.n_experts) continue;  // nobody served this slot
+            float v = part[(s * W) * 16 + tid];
+            for (int k = 1; k < W; k++) v = v + part[(s * W + k) * 16 + tid];
+            mix = mix + v * a.weight[s];
+        }
+        if (row < a.rows) a.out[row] = mix;
+    }
+}
+
+int q4k_moe_down_sum_waves(int64_t rows_per_expert, int64_t n_sb, int n_slots) { return pick_shape(rows_per_expert, n_sb).ksplit * n_slots; }
+
+// -1: the shape is not one this launch serves (the caller runs the separate launches).
+int launch_moe_down_sum_q4k(const cml_weight *down, int n_experts, int n_slots, const int32_t *idx, const float *weight, const int8_t *q,
+                            const float *yd, float *out, hipStream_t st) {
+    const int64_t rows = down->rows / n_experts;
+    if (rows % 16 != 0 || down->row_skip != 0 || n_slots < 1) return -1;
+    const Q4KShape shape = pick_shape(rows, down->nb);
+    const int waves = shape.ksplit * n_slots;
+    const int n_sb = static_cast<int>(down->nb);
+    const size_t lds = static_cast<size_t>(n_slots) * n_sb * (256 + 32) + ((static_cast<size_t>(n_slots) * n_sb + 3) & ~size_t(3)) * 4 +
+                       static_cast<size_t>(waves) * 16 * 4;
+    if (waves > 8 || lds > 64 * 1024) return -1;  // eight waves: the register budget of the two buffers without spills
+    MoeDownSumArgs a{};
+    a.w = down->planes.p[0];
+    a.sb_stride = down->planes.row_stride[0];
+    a.rows = static_cast<int>(rows);
+    a.n_sb = n_sb;
+    a.n_experts = n_experts;
+    a.n_slots = n_slots;
+    a.ksplit = shape.ksplit;
+    a.ksplit_log2 = shape.ksplit >= 8 ? 3 : (shape.ksplit >= 4 ? 2 : (shape.ksplit >= 2 ? 1 : 0));
+    a.idx = idx;
+    a.weight = weight;
+    a.q = q;
+    a.yd = yd;
+    a.out = out;
+    hipLaunchKernelGGL(moe_down_sum_q4k_kernel, dim3(static_cast<unsigned>(rows / 16)), dim3(64 * waves), lds, st, a);
+    CML_HIP_TRY(hipGetLastError());
+    return CML_OK;
+}
+
 // ---- the generic 8-lane order of the reference's wire row dot, bit for bit ----------------------
 //
 // q4_k_wire_row_dot (src/inference.rs:25806-25889, the Q4_K row dot of the Gemma-4 wire lane and

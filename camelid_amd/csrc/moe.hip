@@ -596,6 +596,12 @@ int cml_moe_ffn_ex(const cml_weight *gate, const cml_weight *up, const cml_weigh
         if (int rc = launch_gemv_b32_grouped(a, gated, st)) return rc;
     } else {
         if (int rc = launch_glu_quantize(glu, act_mid, ws.g, u_rows, n_slots, ff, glu_stride, ws.hq, ws.hd, st)) return rc;
+        if (q4k_direct && down->fmt == CML_Q4_K && env_int("CAMELID_HIP_MOE_FOLD_SUM", 1)) {
+            // decode: the routed experts' down projections and the weighted sum in one launch (a workgroup
+            // owns a row tile for all slots); -1 = a shape that launch does not serve
+            const int rc = launch_moe_down_sum_q4k(down, n_experts, n_slots, idx_dev, weight_dev, ws.hq, ws.hd, out_dev, st);
+            if (rc != -1) return rc;
+        }
         if (int rc = launch_expert_matmul(a, st)) return rc;
     }
     hipLaunchKernelGGL(moe_weighted_sum_kernel, dim3(static_cast<unsigned>((hidden + 255) / 256), static_cast<unsigned>(n_tokens)), dim3(256), 0, st,

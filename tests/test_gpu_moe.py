@@ -208,6 +208,35 @@ def test_moe_ffn_skips_slots_with_expert_ids_out_of_range(fmt, fmt_down, hidden,
         assert G.same_bits(got, want)
 
 
+@pytest.mark.parametrize("E,k,hidden,ff", [(8, 2, 512, 1024), (8, 3, 4096, 14336 // 4), (16, 4, 1024, 2048), (4, 1, 256, 768)])
+def test_moe_decode_down_projection_with_the_weighted_sum_folded_in(E, k, hidden, ff):
+    """One token, Q4_K experts: the down projections of the routed experts and the weighted sum run as
+    one launch (a workgroup owns a row tile for all slots) -- bit for bit the separate launches
+    (CAMELID_HIP_MOE_FOLD_SUM=0), under the default K cut and with it forbidden, also when a slot's
+    expert id is out of range."""
+    gate_up, down = _experts_fused(B.CML_Q4_K, B.CML_Q4_K, E, hidden, ff, 800 + E)
+    wgu = Weight.upload(B.CML_Q4_K, E * 2 * ff, hidden, gate_up)
+    wd = Weight.upload(B.CML_Q4_K, E * hidden, ff, down)
+    rng = np.random.default_rng(801 + hidden)
+    x = rng.standard_normal((1, hidden)).astype(np.float32)
+    idx = rng.permutation(E)[:k].astype(np.int32).reshape(1, k)
+    w = rng.random((1, k)).astype(np.float32)
+    for exact in ("0", "1"):
+        for bad in (False, True):
+            if bad and k < 2:
+                continue
+            ids = idx.copy()
+            if bad:
+                ids[0, k - 1] = E + 3
+            G.say(f"moe decode, folded sum, E={E} k={k} {hidden}x{ff} exact={exact} bad={bad}")
+            with G.env(CAMELID_HIP_EXACT_ORDER=exact):
+                folded = _moe_poisoned(wgu, wd, E, k, ids, w, x)
+                with G.env(CAMELID_HIP_EXACT_ORDER=exact, CAMELID_HIP_MOE_FOLD_SUM=0):
+                    separate = _moe_poisoned(wgu, wd, E, k, ids, w, x)
+            assert np.isfinite(folded).all()
+            assert G.same_bits(folded, separate)
+
+
 def _moe_poisoned(wgu, wd, E, k, idx, w, x):
     T, hidden = x.shape
     ff = wd.cols
