@@ -61,8 +61,10 @@ CONFIGS = {
     "q4k_14336x4096_n4": ("Q4_K", 14336, 4096, 4),
     "q4k_14336x4096_n8": ("Q4_K", 14336, 4096, 8),
     "q4k_14336x4096_n16": ("Q4_K", 14336, 4096, 16),
+    "q4k_14336x4096_n32": ("Q4_K", 14336, 4096, 32),
     "q4k_14336x4096_n64": ("Q4_K", 14336, 4096, 64),
     "q4k_4096x14336_n16": ("Q4_K", 4096, 14336, 16),
+    "q4k_4096x14336_n32": ("Q4_K", 4096, 14336, 32),
     "q4k_4096x14336_n64": ("Q4_K", 4096, 14336, 64),
     # batches on the other formats (speculative verify / prefill widths); not BASELINE configurations
     "q8_0_14336x4096_n1": ("Q8_0", 14336, 4096, 1),

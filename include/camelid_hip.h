@@ -277,7 +277,8 @@ int cml_block_dots(const cml_weight *w, const int8_t *q_dev, int32_t *ints_dev, 
  * the caller's workspace, then gemv/gemm (reference WireQuant::matvec,
  * src/gemma4_runtime.rs:826-856).  workspace_dev needs
  * cml_matmul_workspace_bytes(fmt, cols, n_tokens) bytes.  Calls with one or two
- * tokens on short rows quantize inside the matvec kernel (one launch, the
+ * tokens on short rows, and Q4_K calls with three to six tokens on rows of up
+ * to 4096 values, quantize inside the product kernel (one launch, the
  * workspace is left untouched); the result bits do not depend on which way ran. */
 size_t cml_matmul_workspace_bytes(int fmt, int64_t cols, int64_t n_tokens);
 int cml_matmul_f32(const cml_weight *w, const float *x_dev, int64_t n_tokens, float *out_dev,
