@@ -94,6 +94,35 @@ __device__ __forceinline__ v4i as_v4i(const uint4 &v) {
 }
 
 typedef unsigned short us2 __attribute__((ext_vector_type(2)));
+typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+// P = sum_g m_g * sum_{t<32} y[32g+t] on the matrix cores without an int8 operand of replicated
+// mins: the sums of the activation's sixteen 16-value runs (at most 16 * 127 = 2032 in magnitude:
+// exact in f16) are staged beside the activation, the 6-bit mins are exact in f16, so ONE
+// v_mfma_f32_16x16x16_f16 over k = run index gives P in f32 -- every product and every partial sum
+// an integer below 2^24, hence exact whatever the order -- where four int8 instructions and
+// their four replicated operands were needed, and the int -> float conversion falls away.
+// Lane (n, kq) supplies runs 4 * kq .. + 3: the mins of sub-blocks 2 * kq and 2 * kq + 1, twice each.
+__device__ __forceinline__ v4h q4k_min_operand(uint32_t m03, uint32_t m47, int kq) {
+    const uint32_t mw = ((kq & 2) ? m47 : m03) >> (16 * (kq & 1));
+    const _Float16 ma = static_cast<_Float16>(static_cast<float>(mw & 0xffu));
+    const _Float16 mb = static_cast<_Float16>(static_cast<float>((mw >> 8) & 0xffu));
+    return v4h{ma, ma, mb, mb};
+}
+
+// The sum of a 16-byte piece of int8 activation as f16 (exact).
+__device__ __forceinline__ _Float16 run_sum_f16(const uint4 &piece) { return static_cast<_Float16>(static_cast<float>(bytesum16(piece))); }
+
+// The two 3-bit digits of the scales in bytes 0 and 1 of `scw`, each replicated into both 16-bit halves of a word
+// (operands of scale_bytes): lo2[plane], hi2[plane].
+__device__ __forceinline__ void q4k_digit_words(uint32_t scw, uint32_t (&lo2)[2], uint32_t (&hi2)[2]) {
+    const uint32_t lo = scw & 0x07070707u, hi = (scw >> 3) & 0x07070707u;
+    lo2[0] = __builtin_amdgcn_perm(lo, lo, 0x0c000c00u);
+    lo2[1] = __builtin_amdgcn_perm(lo, lo, 0x0c010c01u);
+    hi2[0] = __builtin_amdgcn_perm(hi, hi, 0x0c000c00u);
+    hi2[1] = __builtin_amdgcn_perm(hi, hi, 0x0c010c01u);
+}
 
 // Four bytes (each < 16) times one digit (< 8, replicated in both 16-bit halves of `digit2`).
 __device__ __forceinline__ int scale_bytes(uint32_t bytes, uint32_t digit2) {
@@ -108,7 +137,13 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
     // super-blocks per phase and K part (a buffer holds up to 128 token-super-blocks)
     constexpr int KC = (128 / (NTOK * KS)) > 0 ? 128 / (NTOK * KS) : 1;
     constexpr int RT = 4 / (TB * KS);                // row tiles per workgroup
-    constexpr int kBufBytes = KS * KC * NTOK * kSlabRow;
+    // P through one f16 matrix instruction on staged run sums (q4k_min_operand) where it pays: two token groups per
+    // wave, no K parts (14336 x 4096, 32 tokens: 13.8 -> 13.0 us).  Elsewhere the staging costs what the instructions
+    // save or more (64 tokens 19.1 -> 20.1 us, expert groups 194.7 -> 196.7 us per layer), and with K parts the 32
+    // bytes per token and slab are the difference between two workgroups per compute unit and one (27.4 -> 37.8 us).
+    constexpr bool kF16P = GPW == 2 && KS == 1;
+    constexpr int kActBytes = KS * KC * NTOK * kSlabRow;  // activation slabs of one phase
+    constexpr int kBufBytes = kActBytes + (kF16P ? KS * KC * NTOK * 32 : 0);  // + the sums of their 16-value runs, f16 [slab][token][16]
     constexpr int nthreads = 256;
     constexpr int kPieces = NTOK * 16;               // 16-byte pieces of one super-block of all tokens
     constexpr int kPer = kPieces / nthreads;         // 1, 2 or 4
@@ -117,7 +152,7 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
     constexpr int RING = (GPW == 1 && KS == 1) ? 8 : 4;
     static_assert(RING % KC == 0 && kPer >= 1 && RT >= 1, "phase / staging shape");
     extern __shared__ uint4 smem[];
-    uint8_t *buf0 = reinterpret_cast<uint8_t *>(smem);  // [KC][NTOK][kSlabRow]
+    uint8_t *buf0 = reinterpret_cast<uint8_t *>(smem);  // [KC][NTOK][kSlabRow], then [KC][NTOK][16] f16
     uint8_t *buf1 = buf0 + kBufBytes;
     float *yds = reinterpret_cast<float *>(buf1 + kBufBytes);  // [n_sb][NTOK]
 
@@ -183,7 +218,13 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
 #pragma unroll
         for (int s = 0; s < KS * KC; s++)
 #pragma unroll
-            for (int k = 0; k < kPer; k++) *reinterpret_cast<v4i *>(buf + s * (NTOK * kSlabRow) + stage_dst[k]) = sreg[s][k];
+            for (int k = 0; k < kPer; k++) {
+                *reinterpret_cast<v4i *>(buf + s * (NTOK * kSlabRow) + stage_dst[k]) = sreg[s][k];
+                // thread tid + k * nthreads holds piece (token, piece) = that index: run sums are [slab][token][piece]
+                if constexpr (kF16P)
+                    reinterpret_cast<_Float16 *>(buf + kActBytes)[s * (NTOK * 16) + tid + k * nthreads] =
+                        run_sum_f16(make_uint4(sreg[s][k][0], sreg[s][k][1], sreg[s][k][2], sreg[s][k][3]));
+            }
     };
 
     // Lane constants.
@@ -224,7 +265,10 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
     int next_cut = a.ksplit <= 1 ? n_sb : n_sb / a.ksplit;  // first super-block of part 1
 
     // One super-block of this wave's tile against its token block.
-    auto step = [&](const MfmaWeights &w0, int sb, const uint8_t *slot) __attribute__((always_inline)) {
+    auto step = [&](const MfmaWeights &w0, int sb, const uint8_t *buf, int slab) __attribute__((always_inline)) {
+        const uint8_t *slot = buf + slab * (NTOK * kSlabRow);
+        // run sums of this wave's first token group: token n's runs 4 * kq .. + 3
+        const _Float16 *runs = reinterpret_cast<const _Float16 *>(buf + kActBytes) + (slab * NTOK + tb * (16 * GPW) + n) * 16 + 4 * kq;
         if (SPLIT && sb == next_cut) {  // the matvec kernel's K-split point: close the partial chain
 #pragma unroll
             for (int g = 0; g < GPW; g++)
@@ -255,26 +299,30 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
         q4k_unpack_scales(w0.hdr.y, w0.hdr.z, w0.hdr.w, sc03, sc47, m03, m47);
         const float dw = f16_bits_to_f32(w0.hdr.x & 0xffffu);
         const float dminw = f16_bits_to_f32(w0.hdr.x >> 16);
-        v4i blo[4], bhi[4], bm[4];  // step c = 2 * q + plane
+        v4i blo[4], bhi[4], bm[kF16P ? 1 : 4];  // step c = 2 * q + plane
+        const v4h bp = q4k_min_operand(m03, m47, kq);
 #pragma unroll
         for (int q = 0; q < 2; q++) {
-            const uint32_t scw = (q ? sc47 : sc03) >> sc_shift, mw = (q ? m47 : m03) >> sc_shift;
+            uint32_t lo2[2], hi2[2];
+            q4k_digit_words((q ? sc47 : sc03) >> sc_shift, lo2, hi2);
             const uint4 &pc = w0.piece[q];
 #pragma unroll
             for (int plane = 0; plane < 2; plane++) {  // low nibbles = sub-block 2 * ch, high = 2 * ch + 1
                 const int c = 2 * q + plane;
-                const uint32_t scale = (scw >> (8 * plane)) & 0xff;
-                const uint32_t lo = scale & 7u, hi = scale >> 3;
-                const uint32_t lo2 = lo | (lo << 16), hi2 = hi | (hi << 16);
-                const uint32_t m = (mw >> (8 * plane)) & 0xff;
-                const int m4 = static_cast<int>(__builtin_amdgcn_perm(m, m, 0u));  // byte 0 (m < 64) in all four bytes
-                bm[c] = v4i{m4, m4, m4, m4};
                 const uint32_t n0 = (pc.x >> (4 * plane)) & 0x0f0f0f0fu, n1 = (pc.y >> (4 * plane)) & 0x0f0f0f0fu;
                 const uint32_t n2 = (pc.z >> (4 * plane)) & 0x0f0f0f0fu, n3 = (pc.w >> (4 * plane)) & 0x0f0f0f0fu;
-                blo[c] = v4i{scale_bytes(n0, lo2), scale_bytes(n1, lo2), scale_bytes(n2, lo2), scale_bytes(n3, lo2)};
-                bhi[c] = v4i{scale_bytes(n0, hi2), scale_bytes(n1, hi2), scale_bytes(n2, hi2), scale_bytes(n3, hi2)};
+                blo[c] = v4i{scale_bytes(n0, lo2[plane]), scale_bytes(n1, lo2[plane]), scale_bytes(n2, lo2[plane]), scale_bytes(n3, lo2[plane])};
+                bhi[c] = v4i{scale_bytes(n0, hi2[plane]), scale_bytes(n1, hi2[plane]), scale_bytes(n2, hi2[plane]), scale_bytes(n3, hi2[plane])};
+                if constexpr (!kF16P) {  // the sub-block's min in all 16 bytes: P as a third int8 contraction
+                    const uint32_t m = (((q ? m47 : m03) >> sc_shift) >> (8 * plane)) & 0xff;
+                    const int m4 = static_cast<int>(__builtin_amdgcn_perm(m, m, 0u));
+                    bm[c] = v4i{m4, m4, m4, m4};
+                }
             }
         }
+        auto min_sums = [&](int g) __attribute__((always_inline)) -> v4f {  // P of token group g, exact (see q4k_min_operand)
+            return __builtin_amdgcn_mfma_f32_16x16x16f16(*reinterpret_cast<const v4h *>(runs + g * (16 * 16)), bp, v4f{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+        };
         const float *ydp = yds + sb * NTOK + tb * (16 * GPW) + cell_tok;
         if constexpr (kPipelined) {
             // Several token groups per wave, and nothing else on the SIMD to cover a wait: the group loop
@@ -283,7 +331,8 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
             // matrix instructions of group g + 1 -- so an LDS round trip or a matrix result is never
             // waited for with an idle wave.  Two groups per wave: 14336 x 4096, 32 tokens 14.5 -> 13.8 us; 4096 x 14336, 32 tokens
             // 20.1 -> 19.2 us, 64 tokens 27.8 -> 27.4 us.
-            v4i Slo[2], Shi[2], P[2];
+            v4i Slo[2], Shi[2];
+            v4f P[2];
             auto chain = [&](int g) __attribute__((always_inline)) {
                 const float4 ydv = *reinterpret_cast<const float4 *>(ydp + 16 * g);
                 const float yv[4] = {ydv.x, ydv.y, ydv.z, ydv.w};
@@ -292,7 +341,7 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
                     const int s_cell = Slo[g & 1][j] + 8 * Shi[g & 1][j];
                     const float Dd = yv[j] * dw;
                     const float Mm = yv[j] * dminw;
-                    acc[g][j] = __builtin_fmaf(-Mm, static_cast<float>(P[g & 1][j]), acc[g][j]);
+                    acc[g][j] = __builtin_fmaf(-Mm, P[g & 1][j], acc[g][j]);
                     acc[g][j] = __builtin_fmaf(Dd, static_cast<float>(s_cell), acc[g][j]);
                 }
             };
@@ -302,13 +351,15 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
                 __builtin_amdgcn_sched_barrier(0);
                 Slo[g & 1] = v4i{0, 0, 0, 0};
                 Shi[g & 1] = v4i{0, 0, 0, 0};
-                P[g & 1] = v4i{0, 0, 0, 0};
+                v4i Pi = {0, 0, 0, 0};
+                if constexpr (kF16P) P[g & 1] = min_sums(g);
 #pragma unroll
                 for (int c = 0; c < 4; c++) {
                     Slo[g & 1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(av[g & 1][c], blo[c], Slo[g & 1], 0, 0, 0);
                     Shi[g & 1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(av[g & 1][c], bhi[c], Shi[g & 1], 0, 0, 0);
-                    P[g & 1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(av[g & 1][c], bm[c], P[g & 1], 0, 0, 0);
+                    if constexpr (!kF16P) Pi = __builtin_amdgcn_mfma_i32_16x16x64_i8(av[g & 1][c], bm[c], Pi, 0, 0, 0);
                 }
+                if constexpr (!kF16P) P[g & 1] = v4f{static_cast<float>(Pi[0]), static_cast<float>(Pi[1]), static_cast<float>(Pi[2]), static_cast<float>(Pi[3])};
                 if (g > 0) chain(g - 1);
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -317,13 +368,14 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
 #pragma unroll
             for (int g = 0; g < GPW; g++) {
                 load_a(av[0], g);
-                v4i Slo = {0, 0, 0, 0}, Shi = {0, 0, 0, 0}, P = {0, 0, 0, 0};
+                v4i Slo = {0, 0, 0, 0}, Shi = {0, 0, 0, 0}, Pi = {0, 0, 0, 0};
 #pragma unroll
                 for (int c = 0; c < 4; c++) {
                     Slo = __builtin_amdgcn_mfma_i32_16x16x64_i8(av[0][c], blo[c], Slo, 0, 0, 0);
                     Shi = __builtin_amdgcn_mfma_i32_16x16x64_i8(av[0][c], bhi[c], Shi, 0, 0, 0);
-                    P = __builtin_amdgcn_mfma_i32_16x16x64_i8(av[0][c], bm[c], P, 0, 0, 0);
+                    Pi = __builtin_amdgcn_mfma_i32_16x16x64_i8(av[0][c], bm[c], Pi, 0, 0, 0);
                 }
+                const v4f P = {static_cast<float>(Pi[0]), static_cast<float>(Pi[1]), static_cast<float>(Pi[2]), static_cast<float>(Pi[3])};
                 const float4 ydv = *reinterpret_cast<const float4 *>(ydp + 16 * g);
                 const float yv[4] = {ydv.x, ydv.y, ydv.z, ydv.w};
 #pragma unroll
@@ -331,7 +383,7 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
                     const int s_cell = Slo[j] + 8 * Shi[j];
                     const float Dd = yv[j] * dw;
                     const float Mm = yv[j] * dminw;
-                    acc[g][j] = __builtin_fmaf(-Mm, static_cast<float>(P[j]), acc[g][j]);
+                    acc[g][j] = __builtin_fmaf(-Mm, P[j], acc[g][j]);
                     acc[g][j] = __builtin_fmaf(Dd, static_cast<float>(s_cell), acc[g][j]);
                 }
             }
@@ -354,7 +406,7 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
                 stage_load(loc + KC);
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if (loc < n_loc) step(ring[i], s_begin + loc, cur + (ks * KC + i % KC) * (NTOK * kSlabRow));
+            if (loc < n_loc) step(ring[i], s_begin + loc, cur, ks * KC + i % KC);
             // many-token steps fill the register file on their own: keep the scheduler from
             // overlapping two of them (measured: it spills and loses more than it hides)
             if constexpr (GPW > 1) __builtin_amdgcn_sched_barrier(0);
@@ -446,7 +498,7 @@ struct Q4KMfmaPairArgs {
 constexpr int kPairSb = 16;    // most super-blocks per row
 constexpr int kPairPart = 8;   // most super-blocks per wave
 constexpr int kPairTiles = 4;  // row tiles per workgroup
-constexpr size_t kPairLds = static_cast<size_t>(kPairSb) * 16 * kSlabRow + kPairSb * 16 * 4 + kPairTiles * 64 * 16;
+constexpr size_t kPairLds = static_cast<size_t>(kPairSb) * 16 * kSlabRow + kPairSb * 16 * 4 + kPairTiles * 64 * 16 + kPairSb * 16 * 32;
 
 // FUSEQ (a few tokens): the f32 activation is quantized to Q8_K by the workgroup itself, a 16-lane
 // row per (token, super-block) with the device function the quantizer launch uses -- the same bytes
@@ -459,6 +511,7 @@ __global__ __launch_bounds__(512) void gemm_q4k_mfma_pair_kernel(Q4KMfmaPairArgs
     uint8_t *act = reinterpret_cast<uint8_t *>(smem);                            // [kPairSb][16 tokens][kSlabRow]
     float *yds = reinterpret_cast<float *>(act + kPairSb * 16 * kSlabRow);        // [kPairSb][16 tokens]
     float4 *handoff = reinterpret_cast<float4 *>(yds + kPairSb * 16);             // [tile][lane]: the first wave's four chains
+    _Float16 *runs = reinterpret_cast<_Float16 *>(handoff + kPairTiles * 64);     // [kPairSb][16 tokens][16]: sums of the 16-value runs
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
@@ -542,6 +595,7 @@ __global__ __launch_bounds__(512) void gemm_q4k_mfma_pair_kernel(Q4KMfmaPairArgs
                 const int t = b >> 4, sb = b & 15;
                 if (t < n_here && sb < n_sb) {
                     *reinterpret_cast<uint4 *>(act + (sb * 16 + t) * kSlabRow + ql * 16) = packed;
+                    runs[(sb * 16 + t) * 16 + ql] = run_sum_f16(packed);
                     if (ql == 0) yds[sb * 16 + t] = dv;
                 }
             }
@@ -551,6 +605,7 @@ __global__ __launch_bounds__(512) void gemm_q4k_mfma_pair_kernel(Q4KMfmaPairArgs
         for (int k = 0; k < 8; k++) {
             const int i = tid + k * 512;  // slots past n_sb receive a copy of the last super-block; nobody reads them
             *reinterpret_cast<v4i *>(act + ((i >> 8) * 16 + ((i >> 4) & 15)) * kSlabRow + (i & 15) * 16) = sreg[k];
+            runs[i] = run_sum_f16(make_uint4(sreg[k][0], sreg[k][1], sreg[k][2], sreg[k][3]));  // i = (sb * 16 + token) * 16 + piece
         }
         if (tid < 256) yds[tid] = yd_mine;
     }
@@ -574,27 +629,23 @@ __global__ __launch_bounds__(512) void gemm_q4k_mfma_pair_kernel(Q4KMfmaPairArgs
             const float dw = f16_bits_to_f32(w0.hdr.x & 0xffffu);
             const float dminw = f16_bits_to_f32(w0.hdr.x >> 16);
             const uint8_t *ybase = act + sb * (16 * kSlabRow) + a_off;
-            v4i Slo = {0, 0, 0, 0}, Shi = {0, 0, 0, 0}, P = {0, 0, 0, 0};
+            v4i Slo = {0, 0, 0, 0}, Shi = {0, 0, 0, 0};
+            const v4f P = __builtin_amdgcn_mfma_f32_16x16x16f16(*reinterpret_cast<const v4h *>(runs + (sb * 16 + n) * 16 + 4 * kq),
+                                                                q4k_min_operand(m03, m47, kq), v4f{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
 #pragma unroll
             for (int q = 0; q < 2; q++) {
-                const uint32_t scw = (q ? sc47 : sc03) >> sc_shift, mw = (q ? m47 : m03) >> sc_shift;
+                uint32_t lo2[2], hi2[2];
+                q4k_digit_words((q ? sc47 : sc03) >> sc_shift, lo2, hi2);
                 const uint4 &pc = w0.piece[q];
 #pragma unroll
                 for (int plane = 0; plane < 2; plane++) {  // low nibbles = sub-block 2 * ch, high = 2 * ch + 1
-                    const uint32_t scale = (scw >> (8 * plane)) & 0xff;
-                    const uint32_t lo = scale & 7u, hi = scale >> 3;
-                    const uint32_t lo2 = lo | (lo << 16), hi2 = hi | (hi << 16);
-                    const uint32_t m = (mw >> (8 * plane)) & 0xff;
-                    const int m4 = static_cast<int>(__builtin_amdgcn_perm(m, m, 0u));
                     const uint32_t n0 = (pc.x >> (4 * plane)) & 0x0f0f0f0fu, n1 = (pc.y >> (4 * plane)) & 0x0f0f0f0fu;
                     const uint32_t n2 = (pc.z >> (4 * plane)) & 0x0f0f0f0fu, n3 = (pc.w >> (4 * plane)) & 0x0f0f0f0fu;
-                    const v4i blo = {scale_bytes(n0, lo2), scale_bytes(n1, lo2), scale_bytes(n2, lo2), scale_bytes(n3, lo2)};
-                    const v4i bhi = {scale_bytes(n0, hi2), scale_bytes(n1, hi2), scale_bytes(n2, hi2), scale_bytes(n3, hi2)};
-                    const v4i bm = {m4, m4, m4, m4};
+                    const v4i blo = {scale_bytes(n0, lo2[plane]), scale_bytes(n1, lo2[plane]), scale_bytes(n2, lo2[plane]), scale_bytes(n3, lo2[plane])};
+                    const v4i bhi = {scale_bytes(n0, hi2[plane]), scale_bytes(n1, hi2[plane]), scale_bytes(n2, hi2[plane]), scale_bytes(n3, hi2[plane])};
                     const v4i av = *reinterpret_cast<const v4i *>(ybase + 128 * q + 32 * plane);
                     Slo = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, blo, Slo, 0, 0, 0);
                     Shi = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, bhi, Shi, 0, 0, 0);
-                    P = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, bm, P, 0, 0, 0);
                 }
             }
             const v4i S = Slo + Shi * 8;
@@ -605,11 +656,11 @@ __global__ __launch_bounds__(512) void gemm_q4k_mfma_pair_kernel(Q4KMfmaPairArgs
                 const float Dd = yv[j] * dw;
                 const float Mm = yv[j] * dminw;
                 if (kd == 0) {
-                    acc[j] = __builtin_fmaf(-Mm, static_cast<float>(P[j]), acc[j]);
+                    acc[j] = __builtin_fmaf(-Mm, P[j], acc[j]);
                     acc[j] = __builtin_fmaf(Dd, static_cast<float>(S[j]), acc[j]);
                 } else {
                     keep[i][j][0] = -Mm;
-                    keep[i][j][1] = static_cast<float>(P[j]);
+                    keep[i][j][1] = P[j];
                     keep[i][j][2] = Dd;
                     keep[i][j][3] = static_cast<float>(S[j]);
                 }
@@ -705,7 +756,7 @@ static int launch_mfma_split(const Q4KMfmaArgs &ka, int n_groups, hipStream_t st
     const int n_tiles = (ka.rows + ka.row_skip + 15) / 16;
     const unsigned gx = static_cast<unsigned>((n_tiles + RT - 1) / RT);
     const unsigned gy = static_cast<unsigned>((ka.n_tokens + NTOK - 1) / NTOK);
-    const size_t lds = 2 * static_cast<size_t>(KS * KC * NTOK) * kSlabRow + static_cast<size_t>(ka.n_sb) * NTOK * 4;
+    const size_t lds = 2 * static_cast<size_t>(KS * KC * NTOK) * (kSlabRow + ((GPW == 2 && KS == 1) ? 32 : 0)) + static_cast<size_t>(ka.n_sb) * NTOK * 4;
     if (lds > 160 * 1024) return fail(CML_ERR_UNSUPPORTED, "Q4_K matrix-core path: %d super-blocks exceed the LDS budget", ka.n_sb);
     static bool raised = false;  // per instantiation: allow more than 64 KB of dynamic LDS once
     if (!raised) {
