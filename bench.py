@@ -40,9 +40,9 @@ INT8_PEAK_TOPS = 5000.0  # MI355X published dense int8 matrix-core rate
 # run, so the figures measured for the committed kernels are carried here; null where not measured.
 MEASURED_TRAFFIC_BYTES: dict = {
     # profiles/hbm_traffic_fetch_write_size.txt (copy yardstick: FETCH_SIZE x 2.000, WRITE_SIZE x 1.000)
-    "q4k_14336x4096_n1": 33374720,       # 1.008 x algorithmic
-    "q4k_14336x4096_n16": 34686362,      # 1.014 x
-    "q4k_14336x4096_n64": 39155356,      # 1.038 x
+    "q4k_14336x4096_n1": 33370112,       # 1.008 x algorithmic
+    "q4k_14336x4096_n16": 34694144,      # 1.014 x
+    "q4k_14336x4096_n64": 39146496,      # 1.037 x
     "q6k_128256x3072_n1": 323916630,     # 1.001 x
     "q4_0_128256x3072_n16": 252016327,   # 1.087 x
     "q6k_128256x3072_n16": 356013774,    # 1.074 x
@@ -123,8 +123,20 @@ class Timer:
         return float(ms.value)
 
 
+EAGER = False   # --eager: plain stream launches in place of graph replays
+
+
+class EagerSteps:
+    """Stands in for a captured graph under --eager: `count` calls of fn(i) as plain stream launches."""
+
+    def __init__(self, fn, count: int):
+        self.fn, self.count = fn, count
+
+
 def capture(stream, fn, count: int):
     """Capture `count` calls of fn(i) on `stream` into one replayable graph."""
+    if EAGER:
+        return EagerSteps(fn, count)
     L = lib()
     check(L.cml_graph_begin_capture(stream), "begin capture")
     for i in range(count):
@@ -134,12 +146,25 @@ def capture(stream, fn, count: int):
     return g
 
 
+def destroy_graph(graph) -> None:
+    if not isinstance(graph, EagerSteps):
+        check(lib().cml_graph_destroy(graph))
+
+
+def launch_graph(graph, stream) -> None:
+    if isinstance(graph, EagerSteps):
+        for i in range(graph.count):
+            graph.fn(i)
+    else:
+        check(lib().cml_graph_launch(graph, stream))
+
+
 def time_graph(stream, graph, timer: Timer, replays: int = 1) -> float:
     L = lib()
     check(L.cml_stream_sync(stream))
     timer.start()
     for _ in range(replays):
-        check(L.cml_graph_launch(graph, stream))
+        launch_graph(graph, stream)
     return timer.stop_ms()
 
 
@@ -155,12 +180,12 @@ def time_graph_median(stream, graph, timers: list) -> tuple:
     L = lib()
     one = max(time_graph(stream, graph, timers[0]), 1e-3)
     for _ in range(min(4000, int(SETTLE_MS / one) + 1)):
-        check(L.cml_graph_launch(graph, stream))
+        launch_graph(graph, stream)
     check(L.cml_stream_sync(stream))
     n = max(5, min(len(timers), int(SAMPLE_MS / one) + 1))
     for t in timers[:n]:
         check(L.cml_event_record(t.e0, stream))
-        check(L.cml_graph_launch(graph, stream))
+        launch_graph(graph, stream)
         check(L.cml_event_record(t.e1, stream))
     check(L.cml_stream_sync(stream))
     ms = []
@@ -429,10 +454,10 @@ def time_read_only(stream, timers, nbytes: int, K: int, in_flight: int, groups: 
         step(i)
     g = capture(stream, step, K)
     t_k = time_graph_median(stream, g, timers)[0]
-    check(L.cml_graph_destroy(g))
+    destroy_graph(g)
     g2 = capture(stream, step, 2 * K)
     ms = (time_graph_median(stream, g2, timers)[0] - t_k) / K
-    check(L.cml_graph_destroy(g2))
+    destroy_graph(g2)
     return ms * 1e3, bufs
 
 
@@ -496,6 +521,9 @@ def main() -> int:
     ap.add_argument("--copies", type=int, default=0, help="distinct weight copies to rotate over (0 = enough for ~600 MB)")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="time budget of the CPU baseline leg (0 = skip)")
     ap.add_argument("--seed", type=int, default=1234)
+    ap.add_argument("--eager", action="store_true",
+                    help="plain stream launches in place of graph replays: for profilers that cannot follow a graph launch "
+                         "(kernel durations are the same; per-step times then include the host's launch cost)")
     ap.add_argument("--cold-only", action="store_true",
                     help="skip the cache-warm leg and the eager loop (every launch of the dominant kernel is then "
                          "cache-cold, so a profiler's average duration is comparable with roofline.us_per_launch)")
@@ -505,6 +533,8 @@ def main() -> int:
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="BYTES",
                     help="instead of a matvec, time a plain device copy of BYTES (the yardstick for byte counters)")
     args = ap.parse_args()
+    global EAGER
+    EAGER = args.eager
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no collectives and every box here has one GPU; "
               f"--gpus {args.gpus} is not supported", file=sys.stderr)
@@ -566,7 +596,7 @@ def main() -> int:
     # pay the same constant, so the K steps themselves are the difference of the two medians.
     g_twice = capture(stream, step, 2 * K)
     ms_twice, _ = time_graph_median(stream, g_twice, timers)
-    check(L.cml_graph_destroy(g_twice))
+    destroy_graph(g_twice)
     ms_per_step = (ms_twice - ms_total) / K
     replay_overhead_us = max(0.0, (2 * ms_total - ms_twice) * 1e3)
     # the same K steps launched one by one from Python, for the record
@@ -610,7 +640,7 @@ def main() -> int:
         t_k = time_graph_median(stream, g_k, timers)[0]
         g_2k = capture(stream, fn, 2 * K)
         t_2k = time_graph_median(stream, g_2k, timers)[0]
-        check(L.cml_graph_destroy(g_2k))
+        destroy_graph(g_2k)
         return (t_2k - t_k) / K
 
     kern_ms = per_step(gemv_cold, g_cold)
