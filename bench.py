@@ -365,8 +365,8 @@ def bench_moe(name: str, K: int, W: int, seed: int, cpu_seconds: float) -> int:
         what = "route (full softmax) + fused gate|up matvec + gelu_tanh*up->Q8_0 + down matvec + weighted sum, graph replay"
     else:
         # one token: route, gate and up in one launch (quantizes the token itself), silu*up->Q8_K, down + weighted sum in one launch;
-        # more: route, plan, quantize, gate, up, silu*up->Q8_K, down, weighted sum
-        launches, kernel = (4 if T == 1 else 8), "gemv_q4k_kernel / gemm_q4k_mfma_kernel grouped by expert (2-3 launches of the step)"
+        # more: route, plan, quantize, gate and up in one launch, silu*up->Q8_K, down, weighted sum
+        launches, kernel = (4 if T == 1 else 7), "gemv_q4k_kernel / gemm_q4k_mfma_kernel grouped by expert (2-3 launches of the step)"
         what = ("route + gate/up matvecs + silu*up->Q8_K + down matvec + weighted sum (one token: folded into the down launch), "
                 "graph replay")
     line = {

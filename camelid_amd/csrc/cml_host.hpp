@@ -108,6 +108,10 @@ struct MatArgs {
     int64_t n_assign_total;        // all assignments of a grouped call (0 = unknown): sizes the expected group
     int n_groups;
     int64_t band_rows;
+    // Grouped Q4_K matrix-core calls only: a second stacked weight of the same shape against the same
+    // activations, its cells to out2, in the same launch (gate and up of an expert layer).
+    const cml_weight *w2;
+    float *out2;
 };
 
 int launch_gemv_q4k(const MatArgs &a, hipStream_t st);

@@ -73,6 +73,11 @@ struct Q4KMfmaArgs {
     const int32_t *group_offsets;
     const int32_t *group_rows;
     const int32_t *group_ids;  // z-slot -> group (-1: unused slot), or null (the z-slot is the group)
+    // Pair launch (grouped calls only): a second stacked weight of the same shape against the same activations,
+    // written to out2 (gate and up of an expert layer in ONE launch: blockIdx.z = 2 * slot + which, so the two
+    // kernels' last, partly filled rounds of workgroups become one).
+    const uint8_t *w2;
+    float *out2;
 };
 
 struct MfmaWeights {
@@ -170,14 +175,17 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
     const int tile = blockIdx.x * RT + rt;
     const int row = tile * 16 + n - a.row_skip;
     const bool grouped = !PLAIN && a.group_offsets != nullptr;
-    const int64_t band = grouped ? (a.group_ids ? a.group_ids[blockIdx.z] : static_cast<int>(blockIdx.z)) : 0;
+    const bool pair = !PLAIN && a.w2 != nullptr;
+    const int zslot = pair ? static_cast<int>(blockIdx.z >> 1) : static_cast<int>(blockIdx.z);
+    const bool second = pair && (blockIdx.z & 1);
+    const int64_t band = grouped ? (a.group_ids ? a.group_ids[zslot] : zslot) : 0;
     if (band < 0) return;  // a z-slot past the groups in use
     const int a0 = grouped ? a.group_offsets[band] : 0;                      // first assignment of this group
     const int n_assign = grouped ? a.group_offsets[band + 1] - a0 : a.n_tokens;
     const int tok0 = blockIdx.y * NTOK;                    // first token (assignment of the group) of this workgroup
     if (tok0 >= n_assign) return;                          // nothing routed here: the whole workgroup leaves
     const int n_here = min(NTOK, n_assign - tok0);
-    const uint8_t *wtile = a.w + (band * (a.rows / 16) + min(tile, n_tiles - 1)) * 2304;
+    const uint8_t *wtile = (second ? a.w2 : a.w) + (band * (a.rows / 16) + min(tile, n_tiles - 1)) * 2304;
     // activation row of local token t (tokens past the end repeat the last one; their cells are not stored)
     auto act_row = [&](int t) __attribute__((always_inline)) -> int64_t {
         const int j = a0 + tok0 + min(t, n_here - 1);
@@ -453,7 +461,7 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
                 const int t = tb * (16 * GPW) + 16 * g + cell_tok + j;
                 if (t < n_here) {
                     const float v = (part == 0) ? acc[g][j] : total[g][j] + acc[g][j];
-                    a.out[static_cast<int64_t>(a0 + tok0 + t) * a.rows + row] = v;
+                    (second ? a.out2 : a.out)[static_cast<int64_t>(a0 + tok0 + t) * a.rows + row] = v;
                 }
             }
     }
@@ -806,7 +814,14 @@ int launch_gemm_q4k_mfma(const MatArgs &a, hipStream_t st) {
     ka.group_offsets = a.group_offsets;
     ka.group_rows = a.group_rows;
     ka.group_ids = a.group_ids;
-    const int ng = grouped ? (a.group_ids ? a.max_active : a.n_groups) : 1;
+    if (a.w2) {
+        if (!grouped || a.w2->fmt != w->fmt || a.w2->rows != w->rows || a.w2->nb != w->nb || a.w2->row_skip != 0 ||
+            a.w2->planes.row_stride[0] != w->planes.row_stride[0])
+            return fail(CML_ERR_SHAPE, "the two weights of a pair launch differ in shape");
+        ka.w2 = a.w2->planes.p[0];
+        ka.out2 = a.out2;
+    }
+    const int ng = (grouped ? (a.group_ids ? a.max_active : a.n_groups) : 1) * (a.w2 ? 2 : 1);
     // Workgroup shape: tokens staged per workgroup x how they are split over waves.  Default: one
     // wave per row tile, 16 / 32 / 64 tokens per workgroup by batch size; more tokens = more
     // workgroup columns (grid.y), each a pass over the weight.  The other shapes stay selectable

@@ -574,6 +574,14 @@ int cml_moe_ffn_ex(const cml_weight *gate, const cml_weight *up, const cml_weigh
         if (int rc = launch_gemv_q4k_f32_grouped_pair(a, up, up ? ws.u : nullptr, x_dev, st)) return rc;
     } else if (fused_gate_up) {
         if (int rc = launch_expert_matmul(a, st)) return rc;
+    } else if (gate->fmt == CML_Q4_K && a.n_tokens >= env_int("CAMELID_HIP_Q4K_MFMA_MIN_TOKENS", 4) && env_int("CAMELID_HIP_MOE_PAIR_LAUNCH", 1)) {
+        // gate and up on the matrix cores as ONE launch: twice the workgroups in one grid, one partly
+        // filled last round of them instead of two
+        a.w2 = up;
+        a.out2 = ws.u;
+        if (int rc = launch_gemm_q4k_mfma(a, st)) return rc;
+        a.w2 = nullptr;
+        a.out2 = nullptr;
     } else {
         if (int rc = launch_expert_matmul(a, st)) return rc;
         a.w = up;

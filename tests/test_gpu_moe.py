@@ -254,6 +254,28 @@ def _moe_poisoned(wgu, wd, E, k, idx, w, x):
     return out.to_numpy(np.float32, (T, hidden))
 
 
+@pytest.mark.parametrize("E,k,hidden,ff,T", [(8, 2, 512, 1024, 7), (8, 2, 1024, 2048, 40), (4, 3, 256, 768, 16), (16, 4, 512, 512, 33)])
+def test_moe_gate_and_up_in_one_launch_give_the_bits_of_two(E, k, hidden, ff, T):
+    """Batches on Q4_K experts with gate and up as separate tensors: both projections run as one
+    matrix-core launch (twice the workgroups in one grid) -- bit for bit the two launches
+    (CAMELID_HIP_MOE_PAIR_LAUNCH=0)."""
+    gate, up, down = _experts(E, hidden, ff, 970 + E)
+    wg = Weight.upload(B.CML_Q4_K, E * ff, hidden, gate)
+    wu = Weight.upload(B.CML_Q4_K, E * ff, hidden, up)
+    wd = Weight.upload(B.CML_Q4_K, E * hidden, ff, down)
+    rng = np.random.default_rng(971 + T)
+    x = rng.standard_normal((T, hidden)).astype(np.float32)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    logits[:, 1] -= 50.0    # an expert nobody routes to
+    idx_dev, w_dev, _, _ = gpu_route(logits, k)
+    G.say(f"moe gate|up pair launch, E={E} k={k} {hidden}x{ff} T={T}")
+    one = gpu_moe(wg, wu, wd, E, k, idx_dev, w_dev, x)
+    with G.env(CAMELID_HIP_MOE_PAIR_LAUNCH=0):
+        two = gpu_moe(wg, wu, wd, E, k, idx_dev, w_dev, x)
+    assert np.isfinite(one).all()
+    assert G.same_bits(one, two)
+
+
 @pytest.mark.parametrize("T", [1, 32])
 def test_c5_mixtral_shaped_moe(T):
     """8 experts, gate/up 14336x4096 and down 4096x14336 in Q4_K, top-2 routing."""
