@@ -78,6 +78,7 @@ struct Q4KMfmaArgs {
     // kernels' last, partly filled rounds of workgroups become one).
     const uint8_t *w2;
     float *out2;
+    int stage_once;  // rows that fit both activation buffers are staged in the prologue, once
 };
 
 struct MfmaWeights {
@@ -135,7 +136,7 @@ __device__ __forceinline__ int scale_bytes(uint32_t bytes, uint32_t digit2) {
     return __builtin_bit_cast(int, p);
 }
 
-template <int GPW, int TB, bool SPLIT, int KS = 1, bool PLAIN = false>
+template <int GPW, int TB, bool SPLIT, int KS = 1, bool PLAIN = false, bool ONCE = false>
 __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
     static_assert(!(SPLIT && KS > 1), "K is split across waves or inside the lane, not both");
     constexpr int NTOK = 16 * GPW * TB;              // tokens staged per workgroup
@@ -154,6 +155,7 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
     constexpr int kPer = kPieces / nthreads;         // 1, 2 or 4
     // weight super-blocks a wave keeps in flight (register ring): a 16-token step is short, so it
     // takes 8 to cover the HBM latency; steps over more tokens are longer and 4 are enough
+    // (staged-once mode with the whole row of 16 requested in the prologue: the 32-token expert layer 174 -> 179 us)
     constexpr int RING = (GPW == 1 && KS == 1) ? 8 : 4;
     static_assert(RING % KC == 0 && kPer >= 1 && RT >= 1, "phase / staging shape");
     extern __shared__ uint4 smem[];
@@ -211,8 +213,9 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
         stage_src[k] = reinterpret_cast<const v4i *>(a.q + act_row(t) * n_sb * 256) + piece;
         stage_dst[k] = t * kSlabRow + piece * 16;
     }
-    v4i sreg[KS * KC][kPer];
-    auto stage_load = [&](int p0) __attribute__((always_inline)) {  // of every K part, the KC super-blocks starting at its p0-th
+    typedef v4i StageRegs[KS * KC][kPer];
+    StageRegs sreg;
+    auto stage_load_to = [&](StageRegs &sreg, int p0) __attribute__((always_inline)) {  // of every K part, the KC super-blocks starting at its p0-th
 #pragma unroll
         for (int kp = 0; kp < KS; kp++)
 #pragma unroll
@@ -222,7 +225,8 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
                 for (int k = 0; k < kPer; k++) sreg[kp * KC + s][k] = stage_src[k][off];
             }
     };
-    auto stage_store = [&](uint8_t *buf) __attribute__((always_inline)) {
+    auto stage_load = [&](int p0) __attribute__((always_inline)) { stage_load_to(sreg, p0); };
+    auto stage_store_from = [&](const StageRegs &sreg, uint8_t *buf) __attribute__((always_inline)) {
 #pragma unroll
         for (int s = 0; s < KS * KC; s++)
 #pragma unroll
@@ -234,6 +238,7 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
                         run_sum_f16(make_uint4(sreg[s][k][0], sreg[s][k][1], sreg[s][k][2], sreg[s][k][3]));
             }
     };
+    auto stage_store = [&](uint8_t *buf) __attribute__((always_inline)) { stage_store_from(sreg, buf); };
 
     // Lane constants.
     const uint8_t *w_hdr = wtile + n * 16;
@@ -258,10 +263,32 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
         mfma_load_weights(r, w_hdr, w_piece, min(s_begin + loc, s_end - 1) * a.sb_stride);
     };
 
-    stage_load(0);
+    // ONCE (the launcher's choice for rows of up to 2 * KC super-blocks; one 16-token group per wave, no K parts): both buffers together hold the
+    // whole activation, so it is staged ONCE -- no barrier in the middle of the walk (0.9 us per workgroup waiting
+    // for its slowest wave, per-wave time stamps) and no re-read of clamped slabs in the last phase.  buf1 follows
+    // buf0, so slab s of the row sits where phase s / KC would have put it.
+    static_assert(!ONCE || (GPW == 1 && KS == 1 && TB == 1 && !kF16P), "staged-once mode: one token group per wave, no K parts");
+    if constexpr (ONCE) {
+        // (half of the weight ring is requested behind the activation, the other half once the staging registers are free)
+        StageRegs second;
+        stage_load(0);
+        stage_load_to(second, KC);
 #pragma unroll
-    for (int i = 0; i < RING; i++) load_slot(ring[i], i);
-    stage_store(buf0);
+        for (int i = 0; i < RING / 2; i++)
+            if (i < n_loc) load_slot(ring[i], i);
+        __builtin_amdgcn_sched_barrier(0);
+        stage_store(buf0);
+        stage_store_from(second, buf1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = RING / 2; i < RING; i++)
+            if (i < n_loc) load_slot(ring[i], i);
+    } else {
+        stage_load(0);
+#pragma unroll
+        for (int i = 0; i < RING; i++) load_slot(ring[i], i);
+        stage_store(buf0);
+    }
     __syncthreads();
 
     float acc[GPW][4], total[GPW][4];
@@ -410,18 +437,22 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
 #pragma unroll
         for (int i = 0; i < RING; i++) {
             const int loc = l0 + i;
-            if (i % KC == 0) {
+            if (i % KC == 0 && !ONCE) {
                 stage_load(loc + KC);
                 __builtin_amdgcn_sched_barrier(0);
             }
             if (loc < n_loc) step(ring[i], s_begin + loc, cur, ks * KC + i % KC);
             // many-token steps fill the register file on their own: keep the scheduler from
             // overlapping two of them (measured: it spills and loses more than it hides)
-            if constexpr (GPW > 1) __builtin_amdgcn_sched_barrier(0);
+            // (staged-once mode has no barrier between steps: without this fence the scheduler interleaves several
+            // steps and needs more registers than two waves per SIMD leave)
+            if constexpr (GPW > 1 || ONCE) __builtin_amdgcn_sched_barrier(0);
             if constexpr (decltype(refill)::value) load_slot(ring[i], loc + RING);
             if (i % KC == KC - 1) {
-                stage_store(nxt);
-                __syncthreads();  // next phase complete in `nxt`, everyone done with `cur`
+                if constexpr (!ONCE) {
+                    stage_store(nxt);
+                    __syncthreads();  // next phase complete in `nxt`, everyone done with `cur`
+                }
                 uint8_t *t = cur;
                 cur = nxt;
                 nxt = t;
@@ -766,6 +797,19 @@ static int launch_mfma_split(const Q4KMfmaArgs &ka, int n_groups, hipStream_t st
     const unsigned gy = static_cast<unsigned>((ka.n_tokens + NTOK - 1) / NTOK);
     const size_t lds = 2 * static_cast<size_t>(KS * KC * NTOK) * (kSlabRow + ((GPW == 2 && KS == 1) ? 32 : 0)) + static_cast<size_t>(ka.n_sb) * NTOK * 4;
     if (lds > 160 * 1024) return fail(CML_ERR_UNSUPPORTED, "Q4_K matrix-core path: %d super-blocks exceed the LDS budget", ka.n_sb);
+    if constexpr (GPW == 1 && TB == 1 && KS == 1) {
+        if (ka.n_sb <= 2 * KC && ka.stage_once) {  // the whole activation fits the two buffers: staged once
+            static bool raised_once = false;
+            if (!raised_once) {
+                CML_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_mfma_kernel<GPW, TB, SPLIT, KS, PLAIN, true>),
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+                raised_once = true;
+            }
+            hipLaunchKernelGGL((gemm_q4k_mfma_kernel<GPW, TB, SPLIT, KS, PLAIN, true>), dim3(gx, gy, n_groups), dim3(256), lds, st, ka);
+            CML_HIP_TRY(hipGetLastError());
+            return CML_OK;
+        }
+    }
     static bool raised = false;  // per instantiation: allow more than 64 KB of dynamic LDS once
     if (!raised) {
         CML_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_mfma_kernel<GPW, TB, SPLIT, KS, PLAIN>),
@@ -814,6 +858,7 @@ int launch_gemm_q4k_mfma(const MatArgs &a, hipStream_t st) {
     ka.group_offsets = a.group_offsets;
     ka.group_rows = a.group_rows;
     ka.group_ids = a.group_ids;
+    ka.stage_once = env_int("CAMELID_HIP_Q4K_MFMA_STAGE_ONCE", 1);
     if (a.w2) {
         if (!grouped || a.w2->fmt != w->fmt || a.w2->rows != w->rows || a.w2->nb != w->nb || a.w2->row_skip != 0 ||
             a.w2->planes.row_stride[0] != w->planes.row_stride[0])
