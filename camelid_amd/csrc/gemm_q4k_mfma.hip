@@ -147,7 +147,7 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
     // wave, no K parts (14336 x 4096, 32 tokens: 13.8 -> 13.0 us).  Elsewhere the staging costs what the instructions
     // save or more (64 tokens 19.1 -> 20.1 us, expert groups 194.7 -> 196.7 us per layer), and with K parts the 32
     // bytes per token and slab are the difference between two workgroups per compute unit and one (27.4 -> 37.8 us).
-    constexpr bool kF16P = GPW == 2 && KS == 1;
+    constexpr bool kF16P = (GPW == 2 && KS == 1) || ONCE;  // (staged once, the run sums cost one pass in the prologue)
     constexpr int kActBytes = KS * KC * NTOK * kSlabRow;  // activation slabs of one phase
     constexpr int kBufBytes = kActBytes + (kF16P ? KS * KC * NTOK * 32 : 0);  // + the sums of their 16-value runs, f16 [slab][token][16]
     constexpr int nthreads = 256;
@@ -267,7 +267,7 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
     // whole activation, so it is staged ONCE -- no barrier in the middle of the walk (0.9 us per workgroup waiting
     // for its slowest wave, per-wave time stamps) and no re-read of clamped slabs in the last phase.  buf1 follows
     // buf0, so slab s of the row sits where phase s / KC would have put it.
-    static_assert(!ONCE || (GPW == 1 && KS == 1 && TB == 1 && !kF16P), "staged-once mode: one token group per wave, no K parts");
+    static_assert(!ONCE || (GPW == 1 && KS == 1 && TB == 1), "staged-once mode: one token group per wave, no K parts");
     if constexpr (ONCE) {
         // (half of the weight ring is requested behind the activation, the other half once the staging registers are free)
         StageRegs second;
@@ -404,13 +404,15 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
             for (int g = 0; g < GPW; g++) {
                 load_a(av[0], g);
                 v4i Slo = {0, 0, 0, 0}, Shi = {0, 0, 0, 0}, Pi = {0, 0, 0, 0};
+                v4f P;
+                if constexpr (kF16P) P = min_sums(g);
 #pragma unroll
                 for (int c = 0; c < 4; c++) {
                     Slo = __builtin_amdgcn_mfma_i32_16x16x64_i8(av[0][c], blo[c], Slo, 0, 0, 0);
                     Shi = __builtin_amdgcn_mfma_i32_16x16x64_i8(av[0][c], bhi[c], Shi, 0, 0, 0);
-                    Pi = __builtin_amdgcn_mfma_i32_16x16x64_i8(av[0][c], bm[c], Pi, 0, 0, 0);
+                    if constexpr (!kF16P) Pi = __builtin_amdgcn_mfma_i32_16x16x64_i8(av[0][c], bm[c], Pi, 0, 0, 0);
                 }
-                const v4f P = {static_cast<float>(Pi[0]), static_cast<float>(Pi[1]), static_cast<float>(Pi[2]), static_cast<float>(Pi[3])};
+                if constexpr (!kF16P) P = v4f{static_cast<float>(Pi[0]), static_cast<float>(Pi[1]), static_cast<float>(Pi[2]), static_cast<float>(Pi[3])};
                 const float4 ydv = *reinterpret_cast<const float4 *>(ydp + 16 * g);
                 const float yv[4] = {ydv.x, ydv.y, ydv.z, ydv.w};
 #pragma unroll
@@ -799,13 +801,14 @@ static int launch_mfma_split(const Q4KMfmaArgs &ka, int n_groups, hipStream_t st
     if (lds > 160 * 1024) return fail(CML_ERR_UNSUPPORTED, "Q4_K matrix-core path: %d super-blocks exceed the LDS budget", ka.n_sb);
     if constexpr (GPW == 1 && TB == 1 && KS == 1) {
         if (ka.n_sb <= 2 * KC && ka.stage_once) {  // the whole activation fits the two buffers: staged once
+            const size_t lds_once = lds + 2 * static_cast<size_t>(KC * NTOK) * 32;  // + the run sums
             static bool raised_once = false;
             if (!raised_once) {
                 CML_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_mfma_kernel<GPW, TB, SPLIT, KS, PLAIN, true>),
                                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
                 raised_once = true;
             }
-            hipLaunchKernelGGL((gemm_q4k_mfma_kernel<GPW, TB, SPLIT, KS, PLAIN, true>), dim3(gx, gy, n_groups), dim3(256), lds, st, ka);
+            hipLaunchKernelGGL((gemm_q4k_mfma_kernel<GPW, TB, SPLIT, KS, PLAIN, true>), dim3(gx, gy, n_groups), dim3(256), lds_once, st, ka);
             CML_HIP_TRY(hipGetLastError());
             return CML_OK;
         }
