@@ -250,7 +250,10 @@ __device__ __forceinline__ void q4k_compute(const Q4KRegs<U> &r, const Q4KLane &
 // integer divisions that was about 600 instructions and four scalar-load round trips before the
 // first weight request -- 0.8 us of a kernel that lives for eight (14336 x 4096: 8.05 -> 7.25 us).
 // The plain entry has none of it, and the K split (a power of two) is shifts.
-template <int NT, bool INTS, bool FUSEQ = false, int SPR = 1, bool WHOLE = false, bool PLAIN = false, bool LOADONLY = false>
+//
+// DIRECT: the decode launch of an expert layer (one shared f32 token, y-slot = routed assignment, z = which of up to
+// two weights) with its mode known at compile time, for the same reason (one-token MoE layer 44.1 -> 42.6 us).
+template <int NT, bool INTS, bool FUSEQ = false, int SPR = 1, bool WHOLE = false, bool PLAIN = false, bool LOADONLY = false, bool DIRECT = false>
 __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
     static_assert(!FUSEQ || ((NT == 1 || (NT == 2 && PLAIN)) && !INTS),
                   "the fused quantizer serves single-token calls and plain two-token calls (contiguous f32 rows)");
@@ -268,14 +271,15 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
 
     const int tid = threadIdx.x;
     const int nthreads = blockDim.x;
-    const bool direct = !PLAIN && a.group_offsets == nullptr && a.group_ids != nullptr;
-    const bool grouped = !PLAIN && a.group_offsets != nullptr;
-    const int64_t band = (grouped || direct) ? (a.group_ids ? a.group_ids[blockIdx.y] : static_cast<int>(blockIdx.y)) : 0;
+    static_assert(!(DIRECT && PLAIN), "a direct launch is a grouped one");
+    const bool direct = DIRECT || (!PLAIN && a.group_offsets == nullptr && a.group_ids != nullptr);
+    const bool grouped = !DIRECT && !PLAIN && a.group_offsets != nullptr;
+    const int64_t band = DIRECT ? a.group_ids[blockIdx.y] : (grouped || direct) ? (a.group_ids ? a.group_ids[blockIdx.y] : static_cast<int>(blockIdx.y)) : 0;
     if (band < 0 || (direct && band >= a.n_groups)) return;  // a y-slot past the groups in use, or an id out of range
-    const int a0 = grouped ? a.group_offsets[band] : (direct ? static_cast<int>(blockIdx.y) : 0);  // first assignment of this group
-    const int n_assign = grouped ? a.group_offsets[band + 1] - a0 : (direct ? 1 : NT);
+    const int a0 = DIRECT ? static_cast<int>(blockIdx.y) : grouped ? a.group_offsets[band] : (direct ? static_cast<int>(blockIdx.y) : 0);  // first assignment of this group
+    const int n_assign = DIRECT ? 1 : grouped ? a.group_offsets[band + 1] - a0 : (direct ? 1 : NT);
     if (n_assign <= 0) return;  // an expert nobody routed to: the whole workgroup leaves
-    const bool second = !PLAIN && gridDim.z > 1 && blockIdx.z == 1;
+    const bool second = DIRECT ? blockIdx.z == 1 : (!PLAIN && gridDim.z > 1 && blockIdx.z == 1);
     const uint8_t *w = (second ? a.w2 : a.w) + band * (a.rows / 16) * kQ4KChunk;
 
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
@@ -316,7 +320,7 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
         auto act_row = [&](int t) -> int64_t {
             const int j = a0 + min(p0 + t, n_assign - 1);
             if (PLAIN) return j;
-            if (a.shared_act) return 0;
+            if (DIRECT || a.shared_act) return 0;
             return a.group_rows ? a.group_rows[j] : j;
         };
         Regs ra, rb;
@@ -671,6 +675,12 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
             // both tokens in one pass over the weight, 16-row waves as in the two-token matvec
             if (whole) hipLaunchKernelGGL((gemv_q4k_kernel<2, false, true, 1, true, true>), grid, block, lds, st, ka);
             else hipLaunchKernelGGL((gemv_q4k_kernel<2, false, true, 1, false, true>), grid, block, lds, st, ka);
+        } else if (!plain && ka.shared_act && ka.group_ids && !env_int("CAMELID_HIP_Q4K_GENERAL_ENTRY", 0)) {
+            // the decode launch of an expert layer: its own entry
+#define CML_Q4K_DIRECT(SPR_, WHOLE_) hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, SPR_, WHOLE_, false, false, true>), grid, block, lds, st, ka)
+            if (half_tiles) { if (whole) CML_Q4K_DIRECT(2, true); else CML_Q4K_DIRECT(2, false); }
+            else { if (whole) CML_Q4K_DIRECT(1, true); else CML_Q4K_DIRECT(1, false); }
+#undef CML_Q4K_DIRECT
         } else if (half_tiles) {
             if (whole) { if (plain) CML_Q4K_LAUNCH(2, true, true); else CML_Q4K_LAUNCH(2, true, false); }
             else { if (plain) CML_Q4K_LAUNCH(2, false, true); else CML_Q4K_LAUNCH(2, false, false); }
