@@ -196,6 +196,35 @@ def time_graph_median(stream, graph, timers: list) -> tuple:
     return float(np.median(ms)), n
 
 
+LAUNCH_CAL_STEPS = 64   # the constant a replay pays for being launched is measured on graphs of at most this many steps
+
+
+def steps_ms(stream, fn, K: int, timers: list) -> tuple:
+    """(ms per step, ms of the K-step replay, launch constant in ms, replays timed) for K calls of fn(i)
+    replayed as ONE graph.  A replay pays a constant for being launched (a few microseconds: 5 % of a
+    20-step graph, nothing of a 2000-step one); it is measured as 2 * T(K0) - T(2 * K0) on graphs of
+    K0 = min(K, 64) and 2 * K0 steps and taken off the K-step replay.  For K <= 64 that is the
+    difference of the two medians, (T(2K) - T(K)) / K; a long graph is timed as what it is, K steps in
+    a row, and not by the difference of two long replays (whose second half runs a few per cent
+    slower on some boxes once the chip has been kept busy for tens of milliseconds -- a difference
+    of long replays reports that half alone)."""
+    k0 = min(K, LAUNCH_CAL_STEPS)
+    g0 = capture(stream, fn, k0)
+    t0, n0 = time_graph_median(stream, g0, timers)
+    g1 = capture(stream, fn, 2 * k0)
+    t1, _ = time_graph_median(stream, g1, timers)
+    destroy_graph(g1)
+    const_ms = max(0.0, 2.0 * t0 - t1)
+    if k0 == K:
+        total, n = t0, n0
+    else:
+        gk = capture(stream, fn, K)
+        total, n = time_graph_median(stream, gk, timers)
+        destroy_graph(gk)
+    destroy_graph(g0)
+    return (total - const_ms) / K, total, const_ms, n
+
+
 def cpu_topology() -> dict:
     """Logical and physical core counts and the CPU model string of this host (from /proc/cpuinfo)."""
     logical = os.cpu_count() or 1
@@ -348,11 +377,7 @@ def bench_moe(name: str, K: int, W: int, seed: int, cpu_seconds: float) -> int:
         step(i)
     check(L.cml_stream_sync(stream))
     timers = [timer] + [Timer(stream) for _ in range(31)]
-    # per step = (median 2K-step replay - median K-step replay) / K: the constant a replay pays for being launched drops out
-    g = capture(stream, step, K)
-    t_k = time_graph_median(stream, g, timers)[0]
-    g2 = capture(stream, step, 2 * K)
-    ms = (time_graph_median(stream, g2, timers)[0] - t_k) / K
+    ms = steps_ms(stream, step, K, timers)[0]
     check(L.cml_stream_sync(stream))
     if not np.all(np.isfinite(out.to_numpy(np.float32, (T, hidden)))):
         print("non-finite output", file=sys.stderr)
@@ -426,8 +451,7 @@ def bench_producer(name: str, K: int, W: int, seed: int) -> int:
 
     for i in range(W):
         step(i)
-    g = capture(stream, step, K)
-    ms = time_graph_median(stream, g, [timer] + [Timer(stream) for _ in range(31)])[0] / K
+    ms = steps_ms(stream, step, K, [timer] + [Timer(stream) for _ in range(31)])[0]
     alg = T * cols * 5 + cols * 4 + T * (cols // 256) * 4
     print(json.dumps({"metric": f"rms_norm + Q8_K quantize µs, {cols} values x {T} token(s)", "value": round(ms * 1e3, 3), "unit": "us",
                       "higher_is_better": False, "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": round(ms, 6),
@@ -452,12 +476,7 @@ def time_read_only(stream, timers, nbytes: int, K: int, in_flight: int, groups: 
 
     for i in range(8):
         step(i)
-    g = capture(stream, step, K)
-    t_k = time_graph_median(stream, g, timers)[0]
-    destroy_graph(g)
-    g2 = capture(stream, step, 2 * K)
-    ms = (time_graph_median(stream, g2, timers)[0] - t_k) / K
-    destroy_graph(g2)
+    ms = steps_ms(stream, step, K, timers)[0]
     return ms * 1e3, bufs
 
 
@@ -500,8 +519,7 @@ def calibrate_copy(nbytes: int, K: int, W: int) -> int:
 
     for i in range(W):
         step(i)
-    g = capture(stream, step, K)
-    ms = time_graph_median(stream, g, [timer] + [Timer(stream) for _ in range(31)])[0] / K
+    ms = steps_ms(stream, step, K, [timer] + [Timer(stream) for _ in range(31)])[0]
     check(L.cml_stream_sync(stream))
     gbs = 2 * nbytes / (ms * 1e-3) / 1e9
     print(json.dumps({"metric": "plain device copy (read + write)", "value": round(gbs, 2), "unit": "GB/s",
@@ -589,16 +607,8 @@ def main() -> int:
     # steps K.  A replay of few steps is shorter than the GPU's clock ramp, so the graph is first
     # replayed untimed, then several replays are timed and the median replay is reported.
     timers = [timer] + [Timer(stream) for _ in range(63)]
-    g_steps = capture(stream, step, K)
-    ms_total, replays = time_graph_median(stream, g_steps, timers)
-    # A replay also pays a constant for being launched (a few microseconds between two replays):
-    # 5 % of a 20-step graph, nothing of a 2000-step one.  The same steps captured twice over (2K)
-    # pay the same constant, so the K steps themselves are the difference of the two medians.
-    g_twice = capture(stream, step, 2 * K)
-    ms_twice, _ = time_graph_median(stream, g_twice, timers)
-    destroy_graph(g_twice)
-    ms_per_step = (ms_twice - ms_total) / K
-    replay_overhead_us = max(0.0, (2 * ms_total - ms_twice) * 1e3)
+    ms_per_step, ms_total, const_ms, replays = steps_ms(stream, step, K, timers)
+    replay_overhead_us = const_ms * 1e3
     # the same K steps launched one by one from Python, for the record
     check(L.cml_stream_sync(stream))
     eager_us = None
@@ -634,19 +644,13 @@ def main() -> int:
         else:
             check(L.cml_gemm(weights[0].handle, qd.ptr, sd.ptr, n, out.ptr, stream), "cml_gemm")
 
-    g_cold = capture(stream, gemv_cold, K)
-    g_warm = capture(stream, gemv_warm, K)
-    def per_step(fn, g_k):
-        t_k = time_graph_median(stream, g_k, timers)[0]
-        g_2k = capture(stream, fn, 2 * K)
-        t_2k = time_graph_median(stream, g_2k, timers)[0]
-        destroy_graph(g_2k)
-        return (t_2k - t_k) / K
+    def per_step(fn):
+        return steps_ms(stream, fn, K, timers)[0]
 
-    kern_ms = per_step(gemv_cold, g_cold)
+    kern_ms = per_step(gemv_cold)
     warm_ms = None
     if not args.cold_only:
-        warm_ms = per_step(gemv_warm, g_warm)
+        warm_ms = per_step(gemv_warm)
     # what the SHAPE allows a single launch: the matvec's own loads with nothing behind them (Q4_K),
     # and the best of a few read-only launches over the same number of bytes
     ceiling = None
@@ -658,8 +662,7 @@ def main() -> int:
             def loads_only(i):
                 check(L.cml_calibrate_weight_loads(weights[i % copies].handle, scratch.ptr, stream), "cml_calibrate_weight_loads")
 
-            g_loads = capture(stream, loads_only, K)
-            ceiling["matvec_loads_only_us"] = round(per_step(loads_only, g_loads) * 1e3, 3)
+            ceiling["matvec_loads_only_us"] = round(per_step(loads_only) * 1e3, 3)
         best_us, bufs = None, None
         for groups, in_flight in ((2048, 4), (4096, 4), (8192, 4), (2048, 8)):
             us, bufs = time_read_only(stream, timers, wire.nbytes // 16 * 16, K, in_flight, groups, bufs)
@@ -698,9 +701,10 @@ def main() -> int:
                    "step": "quantize activation + fused dequantize-matvec (cml_matmul_f32), graph replay",
                    "launches_per_step": 1 if fused else 2,
                    "replays": replays,
-                   "timing": f"graphs of {K} and {2 * K} steps, each replayed untimed for {SETTLE_MS:.0f} ms of GPU time, then {replays} "
-                             "replays timed back to back between their own HIP events; ms_per_step = (median 2K-step replay - "
-                             "median K-step replay) / K, which leaves out the constant a replay pays for being launched",
+                   "timing": f"a graph of {K} steps replayed untimed for {SETTLE_MS:.0f} ms of GPU time, then {replays} replays timed back "
+                             "to back between their own HIP events; ms_per_step = (median replay - launch constant) / K, the "
+                             f"constant a replay pays for being launched measured as 2 T(k) - T(2k) on graphs of k = {min(K, LAUNCH_CAL_STEPS)} "
+                             "and 2k steps (for K <= 64 that is (T(2K) - T(K)) / K)",
                    "replay_launch_overhead_us": round(replay_overhead_us, 3),
                    "k_step_replay_ms": round(ms_total, 6),
                    "eager_python_us_per_call": None if eager_us is None else round(eager_us, 3)},
