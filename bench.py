@@ -648,6 +648,12 @@ def main() -> int:
         return steps_ms(stream, fn, K, timers)[0]
 
     kern_ms = per_step(gemv_cold)
+    # where the step quantizes in the kernel: the same matvec on an activation quantized ONCE beforehand,
+    # the way the reference shares one quantized activation between the projections that read it
+    # (SharedActivation, src/gemma4_runtime.rs:1288-1340) -- what a second projection of the same input costs
+    shared_ms = None
+    if fused and not args.cold_only:
+        shared_ms = per_step(lambda i: check(L.cml_gemm(weights[i % copies].handle, qd.ptr, sd.ptr, n, out.ptr, stream), "cml_gemm"))
     warm_ms = None
     if not args.cold_only:
         warm_ms = per_step(gemv_warm)
@@ -716,6 +722,7 @@ def main() -> int:
                      "us_per_launch": round(kern_ms * 1e3, 3),
                      "cache_warm_us_per_launch": None if warm_ms is None else round(warm_ms * 1e3, 3),
                      "cache_warm_gbs": None if warm_ms is None else round(alg_bytes / (warm_ms * 1e-3) / 1e9, 2),
+                     "shared_activation_us_per_launch": None if shared_ms is None else round(shared_ms * 1e3, 3),
                      "shape_ceiling": ceiling},
     }
     if n >= 8:
