@@ -41,6 +41,7 @@
 // (row, token) cell is the NT = 1 result exactly.
 #include <algorithm>
 #include <cmath>
+#include <type_traits>
 
 #include "cml_device.hpp"
 #include "cml_host.hpp"
@@ -253,13 +254,17 @@ __device__ __forceinline__ void q4k_compute(const Q4KRegs<U> &r, const Q4KLane &
 //
 // DIRECT: the decode launch of an expert layer (one shared f32 token, y-slot = routed assignment, z = which of up to
 // two weights) with its mode known at compile time, for the same reason (one-token MoE layer 44.1 -> 42.6 us).
-template <int NT, bool INTS, bool FUSEQ = false, int SPR = 1, bool WHOLE = false, bool PLAIN = false, bool LOADONLY = false, bool DIRECT = false>
+template <int NT, bool INTS, bool FUSEQ = false, int SPR = 1, bool WHOLE = false, bool PLAIN = false, bool LOADONLY = false, bool DIRECT = false,
+          int RING = 0>
 __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
     static_assert(!FUSEQ || ((NT == 1 || (NT == 2 && PLAIN)) && !INTS),
                   "the fused quantizer serves single-token calls and plain two-token calls (contiguous f32 rows)");
     static_assert(SPR == 1 || SPR == 2, "groups per row");
     constexpr int RPW = kWave / (LPS * SPR);  // rows per wave tile
-    constexpr int U = 4 / SPR;                // buffer entries per group: a buffer always holds 4 super-blocks of a row
+    static_assert(RING == 0 || ((RING == 3 || RING == 4) && SPR == 2 && WHOLE && PLAIN), "the ring serves plain calls with 8-row waves and needs no clamping");
+    constexpr int NB = RING ? RING : 1;  // ring slots
+    constexpr int PRE = RING ? 2 : 1;  // slots requested before the activation is staged (the rest right after)
+    constexpr int U = RING ? 1 : 4 / SPR;  // buffer entries per group: two buffers of 4 super-blocks of a row, or a ring of 2-super-block ones
     constexpr int UB = U * SPR;
     using Regs = Q4KRegs<U>;
     extern __shared__ uint4 smem[];
@@ -324,7 +329,13 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
             return a.group_rows ? a.group_rows[j] : j;
         };
         Regs ra, rb;
+        Regs ring[NB];
+        auto ring_prologue = [&]() __attribute__((always_inline)) {
+#pragma unroll
+            for (int k = 0; k < PRE; k++) load_buffer(ring[k], s0 + k * UB);
+        };
         if constexpr (LOADONLY) {
+            if constexpr (RING) ring_prologue(); else
             load_buffer(ra, s0);
         } else if constexpr (FUSEQ) {
             // f32 loads of the first batch, the first weight buffer right behind
@@ -356,6 +367,7 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
             float4 xa[4], xb[4];
             load_pass(xa, 4 * wave);
             __builtin_amdgcn_sched_barrier(0);
+            if constexpr (RING) ring_prologue(); else
             load_buffer(ra, s0);
             __builtin_amdgcn_sched_barrier(0);
             for (int base = 4 * wave;;) {
@@ -391,6 +403,7 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
             }
 
             __builtin_amdgcn_sched_barrier(0);
+            if constexpr (RING) ring_prologue(); else
             load_buffer(ra, s0);
             __builtin_amdgcn_sched_barrier(0);
 
@@ -434,6 +447,54 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
         // the current one is consumed.  The last buffer is consumed without issuing
         // anything, so no load is wasted; sched_barrier keeps the loads ahead of
         // the arithmetic they overlap with.
+        if constexpr (RING) {
+            // A ring of three 2-super-block buffers instead of two 4-super-block ones: fewer bytes
+            // in flight per wave (6 super-blocks of a row against 8), but a slot is requested again
+            // after two super-blocks' arithmetic instead of four, so the wave's requests never drop
+            // to half (14336 x 4096: 7.21 -> 6.78 us; two slots 7.3-7.4, four 6.81, five 7.05, six
+            // 7.27; three slots with all three requested before the quantizer 6.92).  The part
+            // holds n >= 3 steps of two super-blocks (the launcher checks).  Whole turns of the
+            // ring run in a loop; the last 3..5 steps are straight-line code per remainder, so
+            // that every wait counts exactly the loads behind the buffer it needs -- a load
+            // under a condition would make each later wait assume it had not been issued.
+            auto compute = [&](const Regs &b, int step) __attribute__((always_inline)) {
+                q4k_compute<NT, INTS, U, SPR, WHOLE, LOADONLY>(b, ln, s0 + step * UB + h, s1, ys, bsum, yds, n_sb, acc, ints_row);
+                __builtin_amdgcn_sched_barrier(0);
+            };
+            auto request = [&](Regs &b, int step) __attribute__((always_inline)) {
+                load_buffer(b, s0 + step * UB);
+                __builtin_amdgcn_sched_barrier(0);
+            };
+#pragma unroll
+            for (int j = PRE; j < NB; j++) request(ring[j], j);
+            const int n = (s1 - s0) / UB;
+            int k = 0;
+            for (; k + 2 * NB <= n; k += NB) {
+#pragma unroll
+                for (int j = 0; j < NB; j++) {
+                    compute(ring[j], k + j);
+                    request(ring[j], k + NB + j);
+                }
+            }
+            auto tail = [&](auto extra) __attribute__((always_inline)) {  // `extra` steps are not requested yet
+                constexpr int E = decltype(extra)::value;
+#pragma unroll
+                for (int j = 0; j < NB; j++) {
+                    compute(ring[j], k + j);
+                    if (j < E) request(ring[j], k + NB + j);
+                }
+#pragma unroll
+                for (int j = 0; j < E; j++) compute(ring[j], k + NB + j);
+            };
+            switch (n - k - NB) {
+                case 0: tail(std::integral_constant<int, 0>{}); break;
+                case 1: tail(std::integral_constant<int, 1>{}); break;
+                case 2: tail(std::integral_constant<int, 2>{}); break;
+                default:
+                    if constexpr (NB > 3) tail(std::integral_constant<int, 3>{});
+                    break;
+            }
+        } else
         for (int sb = s0;;) {
             if (sb + UB >= s1) {
                 q4k_compute<NT, INTS, U, SPR, WHOLE, LOADONLY>(ra, ln, sb + h, s1, ys, bsum, yds, n_sb, acc, ints_row);
@@ -553,6 +614,13 @@ static bool q4k_whole_buffers(const Q4KArgs &ka, int ksplit) {
     return ka.n_sb % (4 * ksplit) == 0 && ka.sb_stride < (int64_t(1) << 31);
 }
 
+// The three-slot ring of 2-super-block buffers (8-row waves): every K part an even number of
+// super-blocks, at least six, and a stride of less than 2 GiB.
+static bool q4k_ring(const Q4KArgs &ka, int ksplit) {
+    if (!env_int("CAMELID_HIP_Q4K_RING", 1) || env_int("CAMELID_HIP_Q4K_CLAMPED_LOADS", 0)) return false;
+    return ka.n_sb % (2 * ksplit) == 0 && ka.n_sb / (2 * ksplit) >= 3 && ka.sb_stride < (int64_t(1) << 31);
+}
+
 template <int NT>
 static int launch_q4k_nt(Q4KArgs ka, const Q4KShape &shape, int n_groups, bool ints, hipStream_t st) {
     const int waves = shape.ksplit * shape.tiles_per_wg;
@@ -575,7 +643,9 @@ static int launch_q4k_nt(Q4KArgs ka, const Q4KShape &shape, int n_groups, bool i
         constexpr int NTS = NT <= 2 ? NT : 1;
         const bool whole = q4k_whole_buffers(ka, shape.ksplit);
 #define CML_Q4K_LAUNCH(SPR_, WHOLE_, PLAIN_) hipLaunchKernelGGL((gemv_q4k_kernel<NTS, false, false, SPR_, WHOLE_, PLAIN_>), grid, block, lds, st, ka)
-        if (half_tiles) {
+        if (half_tiles && plain && q4k_ring(ka, shape.ksplit)) {
+            hipLaunchKernelGGL((gemv_q4k_kernel<1, false, false, 2, true, true, false, false, 3>), grid, block, lds, st, ka);
+        } else if (half_tiles) {
             if (whole) { if (plain) CML_Q4K_LAUNCH(2, true, true); else CML_Q4K_LAUNCH(2, true, false); }
             else { if (plain) CML_Q4K_LAUNCH(2, false, true); else CML_Q4K_LAUNCH(2, false, false); }
         } else {
@@ -662,13 +732,15 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
     const dim3 grid(gx, grouped ? (a.group_ids ? a.max_active : a.n_groups) : 1, w2 ? 2 : 1);
     {
         const bool whole = q4k_whole_buffers(ka, shape.ksplit);
+        const bool ring = q4k_ring(ka, shape.ksplit);
         const bool plain = !grouped && !w2 && !env_int("CAMELID_HIP_Q4K_GENERAL_ENTRY", 0);
         const dim3 block(64 * waves);
 #define CML_Q4K_LAUNCH(SPR_, WHOLE_, PLAIN_) hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, SPR_, WHOLE_, PLAIN_>), grid, block, lds, st, ka)
         if (loads_only) {
             // calibration: the plain single-token launch with its loads and nothing else
 #define CML_Q4K_LOADS(SPR_, WHOLE_) hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, SPR_, WHOLE_, true, true>), grid, block, lds, st, ka)
-            if (half_tiles) { if (whole) CML_Q4K_LOADS(2, true); else CML_Q4K_LOADS(2, false); }
+            if (half_tiles && ring) hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, 2, true, true, true, false, 3>), grid, block, lds, st, ka);
+            else if (half_tiles) { if (whole) CML_Q4K_LOADS(2, true); else CML_Q4K_LOADS(2, false); }
             else { if (whole) CML_Q4K_LOADS(1, true); else CML_Q4K_LOADS(1, false); }
 #undef CML_Q4K_LOADS
         } else if (two) {
@@ -681,6 +753,8 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
             if (half_tiles) { if (whole) CML_Q4K_DIRECT(2, true); else CML_Q4K_DIRECT(2, false); }
             else { if (whole) CML_Q4K_DIRECT(1, true); else CML_Q4K_DIRECT(1, false); }
 #undef CML_Q4K_DIRECT
+        } else if (half_tiles && ring && plain) {
+            hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, 2, true, true, false, false, 3>), grid, block, lds, st, ka);
         } else if (half_tiles) {
             if (whole) { if (plain) CML_Q4K_LAUNCH(2, true, true); else CML_Q4K_LAUNCH(2, true, false); }
             else { if (plain) CML_Q4K_LAUNCH(2, false, true); else CML_Q4K_LAUNCH(2, false, false); }
@@ -744,8 +818,12 @@ struct MoeDownSumArgs {
     float *out;               // [rows]
 };
 
+template <bool RING>
 __global__ __launch_bounds__(512) void moe_down_sum_q4k_kernel(MoeDownSumArgs a) {
-    constexpr int U = 4;
+    // RING: three 2-super-block buffers instead of two 4-super-block ones, as in the matvec above
+    // (every K part an even number of super-blocks, at least six: the launcher checks)
+    constexpr int U = RING ? 2 : 4;
+    constexpr int NB = 3;
     using Regs = Q4KRegs<U>;
     extern __shared__ uint4 smem[];
     const int n_sb = a.n_sb, S = a.n_slots, W = a.ksplit;
@@ -768,17 +846,30 @@ __global__ __launch_bounds__(512) void moe_down_sum_q4k_kernel(MoeDownSumArgs a)
     ln.c = l;
     ln.sh = (ln.c & 1) * 16;
     ln.upper = ln.c >= 2;
-    auto load_buffer = [&](Regs &dst, int sb) __attribute__((always_inline)) { q4k_load<U, 1>(dst, wtile, a.sb_stride, r, piece, sb, s1); };
+    auto load_buffer = [&](Regs &dst, int sb) __attribute__((always_inline)) {
+        if constexpr (RING)
+            q4k_load_whole<U, 1>(dst, wtile + static_cast<int64_t>(sb) * a.sb_stride, a.sb_stride, static_cast<uint32_t>(r) * 16, static_cast<uint32_t>(piece) * 16);
+        else
+            q4k_load<U, 1>(dst, wtile, a.sb_stride, r, piece, sb, s1);
+    };
 
     // every slot's activation row into LDS, with the 32-value sums; the first weight buffer goes out
     // behind the first activation loads
     Regs ra, rb;
+    Regs ring[RING ? NB : 1];
     const int c16 = n_sb * 16, n16 = S * c16;
     uint4 *dst = reinterpret_cast<uint4 *>(ys);
     const uint4 *src = reinterpret_cast<const uint4 *>(a.q);
     uint4 first = src[min(tid, n16 - 1)];
     __builtin_amdgcn_sched_barrier(0);
-    if (served) load_buffer(ra, s0);
+    if (served) {
+        if constexpr (RING) {
+            load_buffer(ring[0], s0);
+            load_buffer(ring[1], s0 + U);
+        } else {
+            load_buffer(ra, s0);
+        }
+    }
     __builtin_amdgcn_sched_barrier(0);
     for (int i = tid; i < n16 + (n16 & 1); i += nthreads) {  // lanes 2k, 2k+1 stay together for the pair sum
         const uint4 v = i == tid ? first : src[min(i, n16 - 1)];
@@ -797,6 +888,41 @@ __global__ __launch_bounds__(512) void moe_down_sum_q4k_kernel(MoeDownSumArgs a)
         const int8_t *ys_s = ys + slot * n_sb * 256;
         const int *bsum_s = bsum + slot * n_sb * 8;
         const float *yds_s = yds + slot * n_sb;
+        if constexpr (RING) {
+            auto compute = [&](const Regs &b, int step) __attribute__((always_inline)) {
+                q4k_compute<1, false, U, 1, true>(b, ln, s0 + step * U, s1, ys_s, bsum_s, yds_s, n_sb, acc, nullptr);
+                __builtin_amdgcn_sched_barrier(0);
+            };
+            auto request = [&](Regs &b, int step) __attribute__((always_inline)) {
+                load_buffer(b, s0 + step * U);
+                __builtin_amdgcn_sched_barrier(0);
+            };
+            request(ring[2], 2);
+            const int n = (s1 - s0) / U;
+            int k = 0;
+            for (; k + 2 * NB <= n; k += NB) {
+#pragma unroll
+                for (int j = 0; j < NB; j++) {
+                    compute(ring[j], k + j);
+                    request(ring[j], k + NB + j);
+                }
+            }
+            auto tail = [&](auto extra) __attribute__((always_inline)) {  // `extra` steps are not requested yet
+                constexpr int E = decltype(extra)::value;
+#pragma unroll
+                for (int j = 0; j < NB; j++) {
+                    compute(ring[j], k + j);
+                    if (j < E) request(ring[j], k + NB + j);
+                }
+#pragma unroll
+                for (int j = 0; j < E; j++) compute(ring[j], k + NB + j);
+            };
+            switch (n - k - NB) {
+                case 0: tail(std::integral_constant<int, 0>{}); break;
+                case 1: tail(std::integral_constant<int, 1>{}); break;
+                default: tail(std::integral_constant<int, 2>{}); break;
+            }
+        } else
         for (int sb = s0;;) {
             if (sb + U >= s1) {
                 q4k_compute<1, false, U, 1>(ra, ln, sb, s1, ys_s, bsum_s, yds_s, n_sb, acc, nullptr);
@@ -861,7 +987,10 @@ int launch_moe_down_sum_q4k(const cml_weight *down, int n_experts, int n_slots, 
     a.q = q;
     a.yd = yd;
     a.out = out;
-    hipLaunchKernelGGL(moe_down_sum_q4k_kernel, dim3(static_cast<unsigned>(rows / 16)), dim3(64 * waves), lds, st, a);
+    const bool ring = env_int("CAMELID_HIP_Q4K_RING", 1) && !env_int("CAMELID_HIP_Q4K_CLAMPED_LOADS", 0) && n_sb % (2 * shape.ksplit) == 0 &&
+                      n_sb / (2 * shape.ksplit) >= 3 && a.sb_stride < (int64_t(1) << 31);
+    if (ring) hipLaunchKernelGGL(moe_down_sum_q4k_kernel<true>, dim3(static_cast<unsigned>(rows / 16)), dim3(64 * waves), lds, st, a);
+    else hipLaunchKernelGGL(moe_down_sum_q4k_kernel<false>, dim3(static_cast<unsigned>(rows / 16)), dim3(64 * waves), lds, st, a);
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }
