@@ -261,7 +261,7 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
                   "the fused quantizer serves single-token calls and plain two-token calls (contiguous f32 rows)");
     static_assert(SPR == 1 || SPR == 2, "groups per row");
     constexpr int RPW = kWave / (LPS * SPR);  // rows per wave tile
-    static_assert(RING == 0 || ((RING == 3 || RING == 4) && SPR == 2 && WHOLE && PLAIN), "the ring serves plain calls with 8-row waves and needs no clamping");
+    static_assert(RING == 0 || (RING >= 3 && RING <= 6 && WHOLE && PLAIN), "the ring serves plain calls and needs no clamping");
     constexpr int NB = RING ? RING : 1;  // ring slots
     constexpr int PRE = RING ? 2 : 1;  // slots requested before the activation is staged (the rest right after)
     constexpr int U = RING ? 1 : 4 / SPR;  // buffer entries per group: two buffers of 4 super-blocks of a row, or a ring of 2-super-block ones
@@ -448,15 +448,18 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
         // anything, so no load is wasted; sched_barrier keeps the loads ahead of
         // the arithmetic they overlap with.
         if constexpr (RING) {
-            // A ring of three 2-super-block buffers instead of two 4-super-block ones: fewer bytes
-            // in flight per wave (6 super-blocks of a row against 8), but a slot is requested again
-            // after two super-blocks' arithmetic instead of four, so the wave's requests never drop
-            // to half (14336 x 4096: 7.21 -> 6.78 us; two slots 7.3-7.4, four 6.81, five 7.05, six
-            // 7.27; three slots with all three requested before the quantizer 6.92).  The part
-            // holds n >= 3 steps of two super-blocks (the launcher checks).  Whole turns of the
-            // ring run in a loop; the last 3..5 steps are straight-line code per remainder, so
-            // that every wait counts exactly the loads behind the buffer it needs -- a load
-            // under a condition would make each later wait assume it had not been issued.
+            // A ring of NB small buffers (one super-block per 4-lane group and step: two
+            // super-blocks of a row for 8-row waves, one for 16-row waves) instead of two
+            // 4-super-block ones.  Fewer bytes are in flight per wave, but a slot is requested
+            // again after one step's arithmetic instead of four super-blocks', so the wave's
+            // requests never drop to half.  14336 x 4096, 8-row waves: 7.21 -> 6.78 us with three
+            // slots (two slots 7.3-7.4, four 6.81, five 7.05, six 7.27; all three requested before
+            // the quantizer 6.92, one 7.00).  16-row waves (two-token calls): four slots, 9.60 ->
+            // 8.87 us (three 8.99, five 8.88, six 8.98).  The part holds n >= NB steps (the
+            // launcher checks).  Whole turns of the ring run in a loop; the last NB..2NB-1 steps
+            // are straight-line code per remainder, so that every wait counts exactly the loads
+            // behind the buffer it needs -- a load under a condition would make each later wait
+            // assume it had not been issued.
             auto compute = [&](const Regs &b, int step) __attribute__((always_inline)) {
                 q4k_compute<NT, INTS, U, SPR, WHOLE, LOADONLY>(b, ln, s0 + step * UB + h, s1, ys, bsum, yds, n_sb, acc, ints_row);
                 __builtin_amdgcn_sched_barrier(0);
@@ -490,9 +493,9 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
                 case 0: tail(std::integral_constant<int, 0>{}); break;
                 case 1: tail(std::integral_constant<int, 1>{}); break;
                 case 2: tail(std::integral_constant<int, 2>{}); break;
-                default:
-                    if constexpr (NB > 3) tail(std::integral_constant<int, 3>{});
-                    break;
+                case 3: if constexpr (NB > 3) tail(std::integral_constant<int, 3>{}); break;
+                case 4: if constexpr (NB > 4) tail(std::integral_constant<int, 4>{}); break;
+                default: if constexpr (NB > 5) tail(std::integral_constant<int, 5>{}); break;
             }
         } else
         for (int sb = s0;;) {
@@ -614,11 +617,13 @@ static bool q4k_whole_buffers(const Q4KArgs &ka, int ksplit) {
     return ka.n_sb % (4 * ksplit) == 0 && ka.sb_stride < (int64_t(1) << 31);
 }
 
-// The three-slot ring of 2-super-block buffers (8-row waves): every K part an even number of
-// super-blocks, at least six, and a stride of less than 2 GiB.
-static bool q4k_ring(const Q4KArgs &ka, int ksplit) {
+// The ring of small register buffers applies (plain calls): 8-row waves (spr = 2) walk a K part in
+// steps of two super-blocks through three slots, 16-row waves (spr = 1) in steps of one through
+// four; the part must hold at least one full ring of whole steps, the stride less than 2 GiB.
+static bool q4k_ring(const Q4KArgs &ka, int ksplit, int spr = 2) {
     if (!env_int("CAMELID_HIP_Q4K_RING", 1) || env_int("CAMELID_HIP_Q4K_CLAMPED_LOADS", 0)) return false;
-    return ka.n_sb % (2 * ksplit) == 0 && ka.n_sb / (2 * ksplit) >= 3 && ka.sb_stride < (int64_t(1) << 31);
+    const int slots = spr == 2 ? 3 : 4;
+    return ka.n_sb % (spr * ksplit) == 0 && ka.n_sb / (spr * ksplit) >= slots && ka.sb_stride < (int64_t(1) << 31);
 }
 
 template <int NT>
@@ -645,6 +650,8 @@ static int launch_q4k_nt(Q4KArgs ka, const Q4KShape &shape, int n_groups, bool i
 #define CML_Q4K_LAUNCH(SPR_, WHOLE_, PLAIN_) hipLaunchKernelGGL((gemv_q4k_kernel<NTS, false, false, SPR_, WHOLE_, PLAIN_>), grid, block, lds, st, ka)
         if (half_tiles && plain && q4k_ring(ka, shape.ksplit)) {
             hipLaunchKernelGGL((gemv_q4k_kernel<1, false, false, 2, true, true, false, false, 3>), grid, block, lds, st, ka);
+        } else if (!half_tiles && plain && q4k_ring(ka, shape.ksplit, 1)) {
+            hipLaunchKernelGGL((gemv_q4k_kernel<NTS, false, false, 1, true, true, false, false, 4>), grid, block, lds, st, ka);
         } else if (half_tiles) {
             if (whole) { if (plain) CML_Q4K_LAUNCH(2, true, true); else CML_Q4K_LAUNCH(2, true, false); }
             else { if (plain) CML_Q4K_LAUNCH(2, false, true); else CML_Q4K_LAUNCH(2, false, false); }
@@ -740,12 +747,14 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
             // calibration: the plain single-token launch with its loads and nothing else
 #define CML_Q4K_LOADS(SPR_, WHOLE_) hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, SPR_, WHOLE_, true, true>), grid, block, lds, st, ka)
             if (half_tiles && ring) hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, 2, true, true, true, false, 3>), grid, block, lds, st, ka);
+            else if (!half_tiles && q4k_ring(ka, shape.ksplit, 1)) hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, 1, true, true, true, false, 4>), grid, block, lds, st, ka);
             else if (half_tiles) { if (whole) CML_Q4K_LOADS(2, true); else CML_Q4K_LOADS(2, false); }
             else { if (whole) CML_Q4K_LOADS(1, true); else CML_Q4K_LOADS(1, false); }
 #undef CML_Q4K_LOADS
         } else if (two) {
             // both tokens in one pass over the weight, 16-row waves as in the two-token matvec
-            if (whole) hipLaunchKernelGGL((gemv_q4k_kernel<2, false, true, 1, true, true>), grid, block, lds, st, ka);
+            if (q4k_ring(ka, shape.ksplit, 1)) hipLaunchKernelGGL((gemv_q4k_kernel<2, false, true, 1, true, true, false, false, 4>), grid, block, lds, st, ka);
+            else if (whole) hipLaunchKernelGGL((gemv_q4k_kernel<2, false, true, 1, true, true>), grid, block, lds, st, ka);
             else hipLaunchKernelGGL((gemv_q4k_kernel<2, false, true, 1, false, true>), grid, block, lds, st, ka);
         } else if (!plain && ka.shared_act && ka.group_ids && !env_int("CAMELID_HIP_Q4K_GENERAL_ENTRY", 0)) {
             // the decode launch of an expert layer: its own entry
@@ -755,6 +764,8 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
 #undef CML_Q4K_DIRECT
         } else if (half_tiles && ring && plain) {
             hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, 2, true, true, false, false, 3>), grid, block, lds, st, ka);
+        } else if (!half_tiles && plain && q4k_ring(ka, shape.ksplit, 1)) {
+            hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, 1, true, true, false, false, 4>), grid, block, lds, st, ka);
         } else if (half_tiles) {
             if (whole) { if (plain) CML_Q4K_LAUNCH(2, true, true); else CML_Q4K_LAUNCH(2, true, false); }
             else { if (plain) CML_Q4K_LAUNCH(2, false, true); else CML_Q4K_LAUNCH(2, false, false); }
