@@ -271,11 +271,57 @@ __device__ __forceinline__ void b32_row_pass(const uint8_t *qrow, const uint8_t 
     b32_row_pass_from<FMT, P, NT, INTS, U>(ra, qrow, srow, l, nb, ys, bsum, xss, acc, ints_row);
 }
 
+// The same pass through a ring of NB one-step buffers: a slot is requested again after ONE step's
+// arithmetic, so the wave's requests in flight never drop to half as they do between two U-step
+// buffers.  `ring[0..PRE-1]` arrive loaded with steps 0..PRE-1; n_steps >= NB (the launcher checks).
+// Whole turns run in a loop, the last NB..2NB-1 steps are straight-line code per remainder so
+// that every wait counts exactly the loads behind the buffer it needs.
+template <int FMT, int P, int NT, int NB, int PRE>
+__device__ __forceinline__ void b32_row_pass_ring(B32Regs<FMT, 1> (&ring)[NB], const uint8_t *qrow, const uint8_t *srow, int l, int nb,
+                                                  const int8_t *ys, const int *bsum, const float *xss, float (&acc)[NT]) {
+    const int n = (nb + P - 1) / P;
+    auto compute = [&](const B32Regs<FMT, 1> &b, int step) __attribute__((always_inline)) {
+        b32_compute<FMT, P, NT, false, 1>(b, l, step, n, nb, ys, bsum, xss, acc, nullptr);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    auto request = [&](B32Regs<FMT, 1> &b, int step) __attribute__((always_inline)) {
+        b32_load<FMT, P, 1>(b, qrow, srow, l, step, n, nb);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+#pragma unroll
+    for (int j = PRE; j < NB; j++) request(ring[j], j);
+    int k = 0;
+    for (; k + 2 * NB <= n; k += NB) {
+#pragma unroll
+        for (int j = 0; j < NB; j++) {
+            compute(ring[j], k + j);
+            request(ring[j], k + NB + j);
+        }
+    }
+    auto tail = [&](auto extra) __attribute__((always_inline)) {  // `extra` steps are not requested yet
+        constexpr int E = decltype(extra)::value;
+#pragma unroll
+        for (int j = 0; j < NB; j++) {
+            compute(ring[j], k + j);
+            if (j < E) request(ring[j], k + NB + j);
+        }
+#pragma unroll
+        for (int j = 0; j < E; j++) compute(ring[j], k + NB + j);
+    };
+    switch (n - k - NB) {
+        case 0: tail(std::integral_constant<int, 0>{}); break;
+        case 1: tail(std::integral_constant<int, 1>{}); break;
+        default: tail(std::integral_constant<int, 2>{}); break;
+    }
+}
+
 // FUSEQ (single token): the activation arrives as f32 and every workgroup quantizes it to Q8_0
 // itself, eight lanes per block, straight into the LDS staging area -- the arithmetic of
 // quantize_q8_0_kernel without the launch and the round trip through memory.
-template <int FMT, int P, int NT, bool INTS, bool FUSEQ = false, int WAVES = 4, int NXQ = 0, int U = 2>
+template <int FMT, int P, int NT, bool INTS, bool FUSEQ = false, int WAVES = 4, int NXQ = 0, int U = 2, int RING = 0>
 __global__ __launch_bounds__(WAVES * 64) void gemv_b32_kernel(B32Args a) {
+    static_assert(RING == 0 || (RING == 3 && FUSEQ && NXQ > 0 && !INTS), "the ring serves the fused single-launch calls with the activation in registers");
+    constexpr int NB = RING ? RING : 1, PRE = RING ? 2 : 1;
     constexpr int T = WAVES * 64;  // threads of a workgroup; its activation prologue is shared by WAVES * (64 / P) rows
     static_assert(!FUSEQ || (NT <= 2 && !INTS), "the fused quantizer serves one token, or two contiguous f32 rows");
     constexpr int RPW = kWave / P;
@@ -303,6 +349,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_b32_kernel(B32Args a) {
     const int n_steps = (nb + P - 1) / P;
     constexpr int UE = U;  // steps per register buffer, also loaded ahead of the prologue
     B32Regs<FMT, UE> ra;
+    B32Regs<FMT, 1> ring[NB];
     bool preloaded = false;
 
     if constexpr (FUSEQ) {
@@ -318,7 +365,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_b32_kernel(B32Args a) {
 #pragma unroll
             for (int j = 0; j < NX; j++) xv[j] = x4[min(tid + T * j, n4 - 1)];
             __builtin_amdgcn_sched_barrier(0);
-            b32_load<FMT, P, UE>(ra, qrow, srow, l, 0, n_steps, nb);
+            if constexpr (RING) {
+#pragma unroll
+                for (int j = 0; j < PRE; j++) b32_load<FMT, P, 1>(ring[j], qrow, srow, l, j, n_steps, nb);
+            } else {
+                b32_load<FMT, P, UE>(ra, qrow, srow, l, 0, n_steps, nb);
+            }
             preloaded = true;
             __builtin_amdgcn_sched_barrier(0);
             uint32_t *ys32 = reinterpret_cast<uint32_t *>(ys);
@@ -390,7 +442,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_b32_kernel(B32Args a) {
 #pragma unroll
     for (int t = 0; t < NT; t++) acc[t] = 0.0f;
 
-    if (preloaded) {
+    if constexpr (RING) {
+        b32_row_pass_ring<FMT, P, NT, NB, PRE>(ring, qrow, srow, l, nb, ys, bsum, xss, acc);
+    } else if (preloaded) {
         b32_row_pass_from<FMT, P, NT, INTS, UE>(ra, qrow, srow, l, nb, ys, bsum, xss, acc, ints_row);
     } else {
         b32_row_pass<FMT, P, NT, INTS, U>(qrow, srow, l, nb, ys, bsum, xss, acc, ints_row);
@@ -563,7 +617,13 @@ static int launch_b32_f32_p(const cml_weight *w, const float *x, float *out, hip
         if (nxq == 4) CML_B32_FUSED(2, 4);
         else CML_B32_FUSED(2, 0);
     } else if (waves == 8) {
-        if (nxq == 1) CML_B32_FUSED(8, 1);
+        // Q8_0 rows of 16 lanes: a ring of three one-step buffers instead of two two-step ones
+        // (8192 x 2048: 4.80 -> 4.61 us; four slots 5.2; Q4_0 14336 x 4096 7.22 / 7.20 / 7.8 with
+        // none / three / four, so Q4_0 keeps the two buffers; sixteen-wave workgroups gain nothing)
+        const bool ring = FMT == CML_Q8_0 && P == 16 && (ba.nb + P - 1) / P >= 3 && env_int("CAMELID_HIP_B32_RING", 1);
+        if (ring && nxq == 1) hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, true, 8, 1, 2, 3>), dim3(gx, 1), dim3(512), lds, st, ba);
+        else if (ring && nxq == 2) hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, true, 8, 2, 2, 3>), dim3(gx, 1), dim3(512), lds, st, ba);
+        else if (nxq == 1) CML_B32_FUSED(8, 1);
         else if (nxq == 2) CML_B32_FUSED(8, 2);
         else CML_B32_FUSED(8, 0);
     } else {
