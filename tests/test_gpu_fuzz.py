@@ -72,3 +72,44 @@ def test_block32_launch_shapes_agree(fmt):
                         assert G.same_bits(G.gpu_matmul_f32(w, x[0]), want[0]), (rows, cols, waves, depth, lanes)
                         assert G.same_bits(G.gpu_gemm(w, s[:1], q[:1]).reshape(rows), want[0]), (rows, cols, depth, lanes)
                         assert G.same_bits(G.gpu_gemm(w, s, q).reshape(2, rows), want), (rows, cols, depth, lanes)
+
+
+def test_register_buffer_rings_cover_every_remainder():
+    """The single-token matvecs that walk a row through a ring of small register buffers (Q4_K: three
+    2-super-block slots under 8-row waves, four 1-super-block slots under 16-row waves; Q8_0:
+    three one-step slots) against the oracle in the exact order, for every remainder of the row
+    length modulo the ring, with the ring and without it (CAMELID_HIP_Q4K_RING / _B32_RING = 0),
+    quantized and f32 activations, one and two tokens, K cut 1 and 2."""
+    rng = np.random.default_rng(41)
+    cases = [(oracle.Q4_K, 200, 256 * nsb) for nsb in (6, 8, 10, 12, 14, 16, 18, 20)]   # 8-row waves: 3..10 steps of two
+    cases += [(oracle.Q4_K, 136, 256 * nsb) for nsb in (4, 5, 6, 7, 8, 9, 11)]           # two tokens: 16-row waves, steps of one
+    cases += [(oracle.Q8_0, 4200, 512 * steps) for steps in (3, 4, 5, 6, 7, 8)]          # 16-lane rows, eight-wave workgroups
+    for fmt, rows, cols in cases:
+        wire = G.synth_weight(fmt, rows, cols, seed=rows + cols)
+        w = Weight.upload(fmt, rows, cols, wire)
+        x = rng.standard_normal((2, cols)).astype(np.float32)
+        s, q = oracle.quantize_activation(fmt, x)
+        want = oracle.matmul(fmt, wire, cols, x, order=EXACT[fmt], threads=8)
+        for ring in ("1", "0"):
+            for ksplit in ("1", "2"):
+                if fmt != oracle.Q4_K and ksplit != "1":
+                    continue
+                G.say(f"ring fmt={fmt} {rows}x{cols} ring={ring} ksplit={ksplit}")
+                with G.env(CAMELID_HIP_Q4K_RING=ring, CAMELID_HIP_B32_RING=ring, CAMELID_HIP_Q4K_KSPLIT=ksplit):
+                    one = G.gpu_matmul_f32(w, x[0])
+                    two = G.gpu_matmul_f32(w, x)
+                    pre = G.gpu_gemm(w, s[:1], q[:1]).reshape(rows)
+                    pre2 = G.gpu_gemm(w, s, q).reshape(2, rows)
+                if ksplit == "1":
+                    assert G.same_bits(one, want[0]), (fmt, rows, cols, ring)
+                    assert G.same_bits(two, want), (fmt, rows, cols, ring)
+                    assert G.same_bits(pre, want[0]), (fmt, rows, cols, ring)
+                    assert G.same_bits(pre2, want), (fmt, rows, cols, ring)
+                else:
+                    for got, ref in ((one, want[0]), (two, want), (pre, want[0]), (pre2, want)):
+                        assert G.max_rel(got, ref) <= 1e-5, (fmt, rows, cols, ring, ksplit)
+                    if ring == "1":
+                        cut = (one, two, pre, pre2)
+                    else:   # the K cut decides the association, the ring does not
+                        for got, ref in zip((one, two, pre, pre2), cut):
+                            assert G.same_bits(got, ref), (fmt, rows, cols, "ring on/off under the K cut")
