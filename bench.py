@@ -40,7 +40,7 @@ INT8_PEAK_TOPS = 5000.0  # MI355X published dense int8 matrix-core rate
 # run, so the figures measured for the committed kernels are carried here; null where not measured.
 MEASURED_TRAFFIC_BYTES: dict = {
     # profiles/hbm_traffic_fetch_write_size.txt (copy yardstick: FETCH_SIZE x 2.000, WRITE_SIZE x 1.000)
-    "q4k_14336x4096_n1": 33418240,       # 1.009 x algorithmic
+    "q4k_14336x4096_n1": 33383424,       # 1.008 x algorithmic
     "q4k_14336x4096_n16": 34694144,      # 1.014 x
     "q4k_14336x4096_n64": 39150592,      # 1.037 x
     "q6k_128256x3072_n1": 323916630,     # 1.001 x
