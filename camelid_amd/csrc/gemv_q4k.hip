@@ -661,6 +661,9 @@ static int launch_q4k_nt(Q4KArgs ka, const Q4KShape &shape, int n_groups, bool i
 #define CML_Q4K_LAUNCH(SPR_, WHOLE_, PLAIN_) hipLaunchKernelGGL((gemv_q4k_kernel<NTS, false, false, SPR_, WHOLE_, PLAIN_>), grid, block, lds, st, ka)
         if (half_tiles && plain && q4k_ring(ka, shape.ksplit) && ka.n_sb == 16 * shape.ksplit) {
             hipLaunchKernelGGL((gemv_q4k_kernel<1, false, false, 2, true, true, false, false, 3, 8>), grid, block, lds, st, ka);
+        } else if (half_tiles && plain && q4k_ring(ka, shape.ksplit) && ka.n_sb == 14 * shape.ksplit) {
+            // K parts of 3584 values (14336 cut four ways, or rows of 3584): seven steps
+            hipLaunchKernelGGL((gemv_q4k_kernel<1, false, false, 2, true, true, false, false, 3, 7>), grid, block, lds, st, ka);
         } else if (half_tiles && plain && q4k_ring(ka, shape.ksplit)) {
             hipLaunchKernelGGL((gemv_q4k_kernel<1, false, false, 2, true, true, false, false, 3>), grid, block, lds, st, ka);
         } else if (!half_tiles && plain && q4k_ring(ka, shape.ksplit, 1)) {
@@ -779,6 +782,8 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
         } else if (half_tiles && ring && plain && ka.n_sb == 16 * shape.ksplit) {
             // rows (K parts) of 4096 values: eight steps, the walk unrolled
             hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, 2, true, true, false, false, 3, 8>), grid, block, lds, st, ka);
+        } else if (half_tiles && ring && plain && ka.n_sb == 14 * shape.ksplit) {
+            hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, 2, true, true, false, false, 3, 7>), grid, block, lds, st, ka);  // rows of 3584 values
         } else if (half_tiles && ring && plain) {
             hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, 2, true, true, false, false, 3>), grid, block, lds, st, ka);
         } else if (!half_tiles && plain && q4k_ring(ka, shape.ksplit, 1)) {
