@@ -851,7 +851,7 @@ struct MoeDownSumArgs {
     float *out;               // [rows]
 };
 
-template <bool RING>
+template <bool RING, int NSTEPS = 0>
 __global__ __launch_bounds__(512) void moe_down_sum_q4k_kernel(MoeDownSumArgs a) {
     // RING: three 2-super-block buffers instead of two 4-super-block ones, as in the matvec above
     // (every K part an even number of super-blocks, at least six: the launcher checks)
@@ -931,6 +931,14 @@ __global__ __launch_bounds__(512) void moe_down_sum_q4k_kernel(MoeDownSumArgs a)
                 __builtin_amdgcn_sched_barrier(0);
             };
             request(ring[2], 2);
+            if constexpr (NSTEPS > 0) {  // the part's length known at compile time: the walk unrolled
+                static_assert(NSTEPS >= NB, "a part holds at least one full ring");
+#pragma unroll
+                for (int i = 0; i < NSTEPS; i++) {
+                    compute(ring[i % NB], i);
+                    if (i + NB < NSTEPS) request(ring[i % NB], i + NB);
+                }
+            } else {
             const int n = (s1 - s0) / U;
             int k = 0;
             for (; k + 2 * NB <= n; k += NB) {
@@ -954,6 +962,7 @@ __global__ __launch_bounds__(512) void moe_down_sum_q4k_kernel(MoeDownSumArgs a)
                 case 0: tail(std::integral_constant<int, 0>{}); break;
                 case 1: tail(std::integral_constant<int, 1>{}); break;
                 default: tail(std::integral_constant<int, 2>{}); break;
+            }
             }
         } else
         for (int sb = s0;;) {
@@ -1022,7 +1031,9 @@ int launch_moe_down_sum_q4k(const cml_weight *down, int n_experts, int n_slots, 
     a.out = out;
     const bool ring = env_int("CAMELID_HIP_Q4K_RING", 1) && !env_int("CAMELID_HIP_Q4K_CLAMPED_LOADS", 0) && n_sb % (2 * shape.ksplit) == 0 &&
                       n_sb / (2 * shape.ksplit) >= 3 && a.sb_stride < (int64_t(1) << 31);
-    if (ring) hipLaunchKernelGGL(moe_down_sum_q4k_kernel<true>, dim3(static_cast<unsigned>(rows / 16)), dim3(64 * waves), lds, st, a);
+    if (ring && n_sb == 14 * shape.ksplit)  // K parts of 3584 values (Mixtral's 14336 cut four ways): seven steps
+        hipLaunchKernelGGL((moe_down_sum_q4k_kernel<true, 7>), dim3(static_cast<unsigned>(rows / 16)), dim3(64 * waves), lds, st, a);
+    else if (ring) hipLaunchKernelGGL(moe_down_sum_q4k_kernel<true>, dim3(static_cast<unsigned>(rows / 16)), dim3(64 * waves), lds, st, a);
     else hipLaunchKernelGGL(moe_down_sum_q4k_kernel<false>, dim3(static_cast<unsigned>(rows / 16)), dim3(64 * waves), lds, st, a);
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
