@@ -261,7 +261,7 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
                   "the fused quantizer serves single-token calls and plain two-token calls (contiguous f32 rows)");
     static_assert(SPR == 1 || SPR == 2, "groups per row");
     constexpr int RPW = kWave / (LPS * SPR);  // rows per wave tile
-    static_assert(RING == 0 || (RING >= 3 && RING <= 6 && WHOLE && PLAIN), "the ring serves plain calls and needs no clamping");
+    static_assert(RING == 0 || (RING >= 3 && RING <= 6 && WHOLE && (PLAIN || DIRECT)), "the ring serves plain and direct calls and needs no clamping");
     constexpr int NB = RING ? RING : 1;  // ring slots
     constexpr int PRE = RING ? 2 : 1;  // slots requested before the activation is staged (the rest right after)
     constexpr int U = RING ? 1 : 4 / SPR;  // buffer entries per group: two buffers of 4 super-blocks of a row, or a ring of 2-super-block ones
@@ -776,7 +776,9 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
         } else if (!plain && ka.shared_act && ka.group_ids && !env_int("CAMELID_HIP_Q4K_GENERAL_ENTRY", 0)) {
             // the decode launch of an expert layer: its own entry
 #define CML_Q4K_DIRECT(SPR_, WHOLE_) hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, SPR_, WHOLE_, false, false, true>), grid, block, lds, st, ka)
-            if (half_tiles) { if (whole) CML_Q4K_DIRECT(2, true); else CML_Q4K_DIRECT(2, false); }
+            if (half_tiles && ring && ka.n_sb == 16 * shape.ksplit && env_int("CAMELID_HIP_Q4K_DIRECT_RING", 1))
+                hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, 2, true, false, false, true, 3, 8>), grid, block, lds, st, ka);
+            else if (half_tiles) { if (whole) CML_Q4K_DIRECT(2, true); else CML_Q4K_DIRECT(2, false); }
             else { if (whole) CML_Q4K_DIRECT(1, true); else CML_Q4K_DIRECT(1, false); }
 #undef CML_Q4K_DIRECT
         } else if (half_tiles && ring && plain && ka.n_sb == 16 * shape.ksplit) {
