@@ -637,6 +637,42 @@ static bool q4k_ring(const Q4KArgs &ka, int ksplit, int spr = 2) {
     return ka.n_sb % (spr * ksplit) == 0 && ka.n_sb / (spr * ksplit) >= slots && ka.sb_stride < (int64_t(1) << 31);
 }
 
+// A plain ring launch.  Part lengths that common models have get the walk unrolled (NSTEPS known
+// at compile time: no loop, no per-remainder tails -- the two-token call on rows of 4096 values
+// 8.87 -> 8.44 us, the single-token one 6.89 -> 6.81); every other length runs the loop.
+// 8-row waves (SPR = 2, three slots) step two super-blocks at a time: rows / K parts of 3072, 3584
+// and 4096 values are 6, 7 and 8 steps; 16-row waves (SPR = 1, four slots) step one: 12, 14, 16.
+template <int NT, bool FUSEQ, int SPR, bool LOADONLY = false>
+static void launch_q4k_ring(const Q4KArgs &ka, int ksplit, dim3 grid, dim3 block, size_t lds, hipStream_t st) {
+    constexpr int SLOTS = SPR == 2 ? 3 : 4;
+    const int steps = ka.n_sb / (SPR * ksplit);
+#define CML_Q4K_RING(N_) hipLaunchKernelGGL((gemv_q4k_kernel<NT, false, FUSEQ, SPR, true, true, LOADONLY, false, SLOTS, N_>), grid, block, lds, st, ka)
+    if constexpr (LOADONLY && SPR == 2) {
+        if (steps == 8) CML_Q4K_RING(8);
+        else CML_Q4K_RING(0);
+    } else if constexpr (LOADONLY) {
+        CML_Q4K_RING(0);
+    } else if constexpr (SPR == 2) {
+        switch (steps) {
+            case 6: CML_Q4K_RING(6); break;
+            case 7: CML_Q4K_RING(7); break;
+            case 8: CML_Q4K_RING(8); break;
+            default: CML_Q4K_RING(0); break;
+        }
+    } else if constexpr (NT == 2 && FUSEQ) {
+        switch (steps) {
+            case 12: CML_Q4K_RING(12); break;
+            case 14: CML_Q4K_RING(14); break;
+            case 16: CML_Q4K_RING(16); break;
+            default: CML_Q4K_RING(0); break;
+        }
+    } else {
+        if (steps == 16) CML_Q4K_RING(16);
+        else CML_Q4K_RING(0);
+    }
+#undef CML_Q4K_RING
+}
+
 template <int NT>
 static int launch_q4k_nt(Q4KArgs ka, const Q4KShape &shape, int n_groups, bool ints, hipStream_t st) {
     const int waves = shape.ksplit * shape.tiles_per_wg;
@@ -659,15 +695,10 @@ static int launch_q4k_nt(Q4KArgs ka, const Q4KShape &shape, int n_groups, bool i
         constexpr int NTS = NT <= 2 ? NT : 1;
         const bool whole = q4k_whole_buffers(ka, shape.ksplit);
 #define CML_Q4K_LAUNCH(SPR_, WHOLE_, PLAIN_) hipLaunchKernelGGL((gemv_q4k_kernel<NTS, false, false, SPR_, WHOLE_, PLAIN_>), grid, block, lds, st, ka)
-        if (half_tiles && plain && q4k_ring(ka, shape.ksplit) && ka.n_sb == 16 * shape.ksplit) {
-            hipLaunchKernelGGL((gemv_q4k_kernel<1, false, false, 2, true, true, false, false, 3, 8>), grid, block, lds, st, ka);
-        } else if (half_tiles && plain && q4k_ring(ka, shape.ksplit) && ka.n_sb == 14 * shape.ksplit) {
-            // K parts of 3584 values (14336 cut four ways, or rows of 3584): seven steps
-            hipLaunchKernelGGL((gemv_q4k_kernel<1, false, false, 2, true, true, false, false, 3, 7>), grid, block, lds, st, ka);
-        } else if (half_tiles && plain && q4k_ring(ka, shape.ksplit)) {
-            hipLaunchKernelGGL((gemv_q4k_kernel<1, false, false, 2, true, true, false, false, 3>), grid, block, lds, st, ka);
+        if (half_tiles && plain && q4k_ring(ka, shape.ksplit)) {
+            launch_q4k_ring<1, false, 2>(ka, shape.ksplit, grid, block, lds, st);
         } else if (!half_tiles && plain && q4k_ring(ka, shape.ksplit, 1)) {
-            hipLaunchKernelGGL((gemv_q4k_kernel<NTS, false, false, 1, true, true, false, false, 4>), grid, block, lds, st, ka);
+            launch_q4k_ring<NTS, false, 1>(ka, shape.ksplit, grid, block, lds, st);
         } else if (half_tiles) {
             if (whole) { if (plain) CML_Q4K_LAUNCH(2, true, true); else CML_Q4K_LAUNCH(2, true, false); }
             else { if (plain) CML_Q4K_LAUNCH(2, false, true); else CML_Q4K_LAUNCH(2, false, false); }
@@ -762,15 +793,14 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
         if (loads_only) {
             // calibration: the plain single-token launch with its loads and nothing else
 #define CML_Q4K_LOADS(SPR_, WHOLE_) hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, SPR_, WHOLE_, true, true>), grid, block, lds, st, ka)
-            if (half_tiles && ring && ka.n_sb == 16 * shape.ksplit) hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, 2, true, true, true, false, 3, 8>), grid, block, lds, st, ka);
-            else if (half_tiles && ring) hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, 2, true, true, true, false, 3>), grid, block, lds, st, ka);
-            else if (!half_tiles && q4k_ring(ka, shape.ksplit, 1)) hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, 1, true, true, true, false, 4>), grid, block, lds, st, ka);
+            if (half_tiles && ring) launch_q4k_ring<1, true, 2, true>(ka, shape.ksplit, grid, block, lds, st);
+            else if (!half_tiles && q4k_ring(ka, shape.ksplit, 1)) launch_q4k_ring<1, true, 1, true>(ka, shape.ksplit, grid, block, lds, st);
             else if (half_tiles) { if (whole) CML_Q4K_LOADS(2, true); else CML_Q4K_LOADS(2, false); }
             else { if (whole) CML_Q4K_LOADS(1, true); else CML_Q4K_LOADS(1, false); }
 #undef CML_Q4K_LOADS
         } else if (two) {
             // both tokens in one pass over the weight, 16-row waves as in the two-token matvec
-            if (q4k_ring(ka, shape.ksplit, 1)) hipLaunchKernelGGL((gemv_q4k_kernel<2, false, true, 1, true, true, false, false, 4>), grid, block, lds, st, ka);
+            if (q4k_ring(ka, shape.ksplit, 1)) launch_q4k_ring<2, true, 1>(ka, shape.ksplit, grid, block, lds, st);
             else if (whole) hipLaunchKernelGGL((gemv_q4k_kernel<2, false, true, 1, true, true>), grid, block, lds, st, ka);
             else hipLaunchKernelGGL((gemv_q4k_kernel<2, false, true, 1, false, true>), grid, block, lds, st, ka);
         } else if (!plain && ka.shared_act && ka.group_ids && !env_int("CAMELID_HIP_Q4K_GENERAL_ENTRY", 0)) {
@@ -781,15 +811,10 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
             else if (half_tiles) { if (whole) CML_Q4K_DIRECT(2, true); else CML_Q4K_DIRECT(2, false); }
             else { if (whole) CML_Q4K_DIRECT(1, true); else CML_Q4K_DIRECT(1, false); }
 #undef CML_Q4K_DIRECT
-        } else if (half_tiles && ring && plain && ka.n_sb == 16 * shape.ksplit) {
-            // rows (K parts) of 4096 values: eight steps, the walk unrolled
-            hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, 2, true, true, false, false, 3, 8>), grid, block, lds, st, ka);
-        } else if (half_tiles && ring && plain && ka.n_sb == 14 * shape.ksplit) {
-            hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, 2, true, true, false, false, 3, 7>), grid, block, lds, st, ka);  // rows of 3584 values
         } else if (half_tiles && ring && plain) {
-            hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, 2, true, true, false, false, 3>), grid, block, lds, st, ka);
+            launch_q4k_ring<1, true, 2>(ka, shape.ksplit, grid, block, lds, st);
         } else if (!half_tiles && plain && q4k_ring(ka, shape.ksplit, 1)) {
-            hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, 1, true, true, false, false, 4>), grid, block, lds, st, ka);
+            launch_q4k_ring<1, true, 1>(ka, shape.ksplit, grid, block, lds, st);
         } else if (half_tiles) {
             if (whole) { if (plain) CML_Q4K_LAUNCH(2, true, true); else CML_Q4K_LAUNCH(2, true, false); }
             else { if (plain) CML_Q4K_LAUNCH(2, false, true); else CML_Q4K_LAUNCH(2, false, false); }

@@ -82,7 +82,7 @@ def test_register_buffer_rings_cover_every_remainder():
     quantized and f32 activations, one and two tokens, K cut 1 and 2."""
     rng = np.random.default_rng(41)
     cases = [(oracle.Q4_K, 200, 256 * nsb) for nsb in (6, 8, 10, 12, 14, 16, 18, 20, 28, 32)]   # 8-row waves: 3..16 steps of two
-    cases += [(oracle.Q4_K, 136, 256 * nsb) for nsb in (4, 5, 6, 7, 8, 9, 11)]           # two tokens: 16-row waves, steps of one
+    cases += [(oracle.Q4_K, 136, 256 * nsb) for nsb in (4, 5, 6, 7, 8, 9, 11, 12, 14, 16)]           # two tokens: 16-row waves, steps of one
     cases += [(oracle.Q8_0, 4200, 512 * steps) for steps in (3, 4, 5, 6, 7, 8)]          # 16-lane rows, eight-wave workgroups
     for fmt, rows, cols in cases:
         wire = G.synth_weight(fmt, rows, cols, seed=rows + cols)
