@@ -361,6 +361,9 @@ def bench_moe(name: str, K: int, W: int, seed: int, cpu_seconds: float) -> int:
     ws = DeviceBuffer(ws_bytes)
     timer = Timer(stream)
 
+    # CAMELID_BENCH_MOE_TWO_CALLS=1: the Mixtral-shaped step as cml_moe_route_top_k + cml_moe_ffn (the routing always a launch of its own)
+    two_calls = os.environ.get("CAMELID_BENCH_MOE_TWO_CALLS", "0") == "1"
+
     def step(i):
         gate, up, down = layers[i % n_layers]
         if gemma:
@@ -368,10 +371,14 @@ def bench_moe(name: str, K: int, W: int, seed: int, cpu_seconds: float) -> int:
                   "cml_moe_route_softmax_top_k")
             check(L.cml_moe_ffn_ex(gate.handle, None, down.handle, E, k, idx.ptr, wts.ptr, xd.ptr, T, out.ptr,
                                    ws.ptr, ws_bytes, 1, stream), "cml_moe_ffn_ex")
-        else:
+        elif two_calls:
             check(L.cml_moe_route_top_k(ld[i % n_sets].ptr, T, E, k, idx.ptr, wts.ptr, stream), "cml_moe_route_top_k")
             check(L.cml_moe_ffn(gate.handle, up.handle, down.handle, E, k, idx.ptr, wts.ptr, xd.ptr, T, out.ptr,
                                 ws.ptr, ws_bytes, stream), "cml_moe_ffn")
+        else:
+            # router logits in: routing and expert lane as one call (one token: routed inside the gate|up launch)
+            check(L.cml_moe_ffn_logits(gate.handle, up.handle, down.handle, E, k, ld[i % n_sets].ptr, xd.ptr, T, out.ptr,
+                                       ws.ptr, ws_bytes, stream), "cml_moe_ffn_logits")
 
     for i in range(W):
         step(i)
@@ -389,11 +396,12 @@ def bench_moe(name: str, K: int, W: int, seed: int, cpu_seconds: float) -> int:
         launches, kernel = (4 if T == 1 else 7), "gemv_b32_grouped_kernel (2 launches of the step)"
         what = "route (full softmax) + fused gate|up matvec + gelu_tanh*up->Q8_0 + down matvec + weighted sum, graph replay"
     else:
-        # one token: route, gate and up in one launch (quantizes the token itself), silu*up->Q8_K, down + weighted sum in one launch;
+        # one token: gate and up in one launch (routes and quantizes the token itself), silu*up->Q8_K, down + weighted sum in one launch;
         # more: route, plan, quantize, gate and up in one launch, silu*up->Q8_K, down, weighted sum
-        launches, kernel = (4 if T == 1 else 7), "gemv_q4k_kernel / gemm_q4k_mfma_kernel grouped by expert (2-3 launches of the step)"
-        what = ("route + gate/up matvecs + silu*up->Q8_K + down matvec + weighted sum (one token: folded into the down launch), "
-                "graph replay")
+        routed_in_launch = T == 1 and not two_calls and os.environ.get("CAMELID_HIP_MOE_FOLD_ROUTE", "1") != "0"
+        launches, kernel = ((3 if routed_in_launch else 4) if T == 1 else 7), "gemv_q4k_kernel / gemm_q4k_mfma_kernel grouped by expert (2-3 launches of the step)"
+        what = ("route + gate/up matvecs + silu*up->Q8_K + down matvec + weighted sum (cml_moe_ffn_logits; one token: the routing inside "
+                "the gate|up launch, the weighted sum inside the down launch), graph replay")
     line = {
         "metric": f"{fmt_name} mixture-of-experts FFN µs + achieved HBM GB/s, {E} experts top-{k}, {ff}x{hidden}, {T} token(s)",
         "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": W,

@@ -226,6 +226,68 @@ __device__ __forceinline__ int row_allor(int v) {
     return v;
 }
 
+// ---- mixture-of-experts routing by one wave ------------------------------------------------------
+// f32::total_cmp as an integer key (larger key = greater value).
+__device__ __forceinline__ int total_key(float v) {
+    const int b = __builtin_bit_cast(int, v);
+    return b ^ static_cast<int>(static_cast<unsigned>(b >> 31) >> 1);
+}
+
+// Maximum over the 64 lanes of a wave, returned in every lane (all lanes must be active).
+__device__ __forceinline__ int wave_allmax_i32(int v) {
+    v = max(v, row_ror_i32<1>(v));
+    v = max(v, row_ror_i32<2>(v));
+    v = max(v, row_ror_i32<4>(v));
+    v = max(v, row_ror_i32<8>(v));
+    return max(max(__builtin_amdgcn_readlane(v, 0), __builtin_amdgcn_readlane(v, 16)),
+               max(__builtin_amdgcn_readlane(v, 32), __builtin_amdgcn_readlane(v, 48)));
+}
+
+// Mixtral routing of ONE token by one whole wave (reference softmax_top_k, src/inference.rs:
+// 13940-13991): top-k by logit (total order, descending, ties to the lower index), softmax over the
+// selected in selection order, renormalised, re-sorted by weight (descending, ties to the lower
+// index).  n_experts <= 128 (lane l holds experts l and l + 64 during the selection), k <= 64.
+// On return lane s < k holds the s-th SELECTED expert, its weight and the rank it takes in the
+// routed order; the short sequential parts run redundantly in every lane.
+// moe_route_wave_values: the same on logits the caller has loaded (l0 = logit of expert `lane`, l1 of
+// expert lane + 64; lanes past n_experts pass anything).
+__device__ __forceinline__ void moe_route_wave_values(float l0, float l1, int n_experts, int k, int lane, int &sel_e, float &w, int &rank) {
+    bool v0 = lane < n_experts, v1 = lane + 64 < n_experts;
+    const int k0 = total_key(l0), k1 = total_key(l1);
+    sel_e = 0;
+    float sel_v = 0.0f;
+    for (int s = 0; s < k; s++) {  // top-k by logit (total order, descending), ties to the lower index
+        const int m = wave_allmax_i32(max(v0 ? k0 : INT32_MIN, v1 ? k1 : INT32_MIN));
+        const unsigned long long b0 = __builtin_amdgcn_ballot_w64(v0 && k0 == m), b1 = __builtin_amdgcn_ballot_w64(v1 && k1 == m);
+        const int e = b0 ? __builtin_ctzll(b0) : (b1 ? 64 + __builtin_ctzll(b1) : 0);
+        const int from = __builtin_amdgcn_readlane(__builtin_bit_cast(int, e < 64 ? l0 : l1), e & 63);
+        if (e == lane) v0 = false;
+        if (e == lane + 64) v1 = false;
+        if (lane == s) {
+            sel_e = e;
+            sel_v = __builtin_bit_cast(float, from);
+        }
+    }
+    float mx = -INFINITY;
+    for (int s = 0; s < k; s++) mx = fmaxf(mx, __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sel_v), s)));
+    const float wv = (lane < k && fabsf(sel_v) < INFINITY) ? expf(sel_v - mx) : 0.0f;  // is_finite: NaN and inf give 0
+    float sum = 0.0f;
+    for (int s = 0; s < k; s++) sum = sum + __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wv), s));
+    w = sum > 0.0f ? wv / sum : 1.0f / static_cast<float>(k);
+    // re-sort by weight (descending), ties to the lower index: the rank of (w, index) in that total order
+    const int wk = total_key(w);
+    rank = 0;
+    for (int s = 0; s < k; s++) {
+        const int ok = total_key(__builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, w), s)));
+        const int oe = __builtin_amdgcn_readlane(sel_e, s);
+        rank += (ok > wk || (ok == wk && oe < sel_e)) ? 1 : 0;
+    }
+}
+__device__ __forceinline__ void moe_route_wave(const float *lg, int n_experts, int k, int lane, int &sel_e, float &w, int &rank) {
+    const float l0 = lane < n_experts ? lg[lane] : 0.0f, l1 = lane + 64 < n_experts ? lg[lane + 64] : 0.0f;
+    moe_route_wave_values(l0, l1, n_experts, k, lane, sel_e, w, rank);
+}
+
 // ---- gated activations ------------------------------------------------------------------------
 // GLU 0: silu(g) * u = (g / (1 + exp(-g))) * u (reference CpuTensor::silu_mul).
 // GLU 1: gelu_pytorch_tanh(g) * u = (0.5 * g * (1 + tanh(C * (g + 0.044715 * g * g * g)))) * u,

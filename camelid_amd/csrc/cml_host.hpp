@@ -112,11 +112,20 @@ struct MatArgs {
     // activations, its cells to out2, in the same launch (gate and up of an expert layer).
     const cml_weight *w2;
     float *out2;
+    // Direct Q4_K decode launch only: route the token inside the launch (Mixtral routing of the
+    // n_groups logits, top route_k), y-slot = routed rank; experts and weights in routed order are
+    // left in route_idx / route_w.  Null = the caller has routed (group_ids).
+    const float *route_logits;
+    int route_k;
+    int32_t *route_idx;
+    float *route_w;
 };
 
 int launch_gemv_q4k(const MatArgs &a, hipStream_t st);
 // quantize + matvec for two stacked expert weights of one shape in one launch; a.q / a.scales unused, x = f32 rows
 int launch_gemv_q4k_f32_grouped_pair(const MatArgs &a, const cml_weight *w2, float *out2, const float *x, hipStream_t st);
+// whether that launch, as a direct call on these two weights, can route the token itself (a.route_logits)
+bool gemv_q4k_direct_can_route(const cml_weight *w, int64_t band_rows, int n_slots, bool pair);
 
 int launch_gemv_q4k_f32(const cml_weight *w, const float *x, float *out, hipStream_t st, int n_tokens = 1);  // quantize + matvec, one or two tokens
 int launch_gemm_q4k_mfma_f32(const cml_weight *w, const float *x, int64_t n_tokens, float *out, hipStream_t st);  // 3..8 tokens, quantize inside; -1: not served

@@ -76,6 +76,13 @@ struct Q4KArgs {
     // row 0 (shared_act: every assignment reads the one token) or row y.
     int n_groups;
     int shared_act;
+    // Direct call that routes the token itself (ROUTE): the n_groups router logits of the one token;
+    // y-slot y serves the expert of routed rank y (Mixtral routing, top route_k), and the first
+    // workgroup leaves experts and weights in routed order for the launches behind this one.
+    const float *route_logits;
+    int route_k;
+    int32_t *route_idx;  // [route_k]
+    float *route_w;      // [route_k]
     // Pair launch (gridDim.z == 2): blockIdx.z = 1 works on a second weight of the same shape
     // against the same activations and writes out2 (gate and up projections in one launch).
     const uint8_t *w2;
@@ -255,8 +262,9 @@ __device__ __forceinline__ void q4k_compute(const Q4KRegs<U> &r, const Q4KLane &
 // DIRECT: the decode launch of an expert layer (one shared f32 token, y-slot = routed assignment, z = which of up to
 // two weights) with its mode known at compile time, for the same reason (one-token MoE layer 44.1 -> 42.6 us).
 template <int NT, bool INTS, bool FUSEQ = false, int SPR = 1, bool WHOLE = false, bool PLAIN = false, bool LOADONLY = false, bool DIRECT = false,
-          int RING = 0, int NSTEPS = 0>
+          int RING = 0, int NSTEPS = 0, bool ROUTE = false>
 __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
+    static_assert(!ROUTE || DIRECT, "only the direct launch routes");
     static_assert(!FUSEQ || ((NT == 1 || (NT == 2 && PLAIN)) && !INTS),
                   "the fused quantizer serves single-token calls and plain two-token calls (contiguous f32 rows)");
     static_assert(SPR == 1 || SPR == 2, "groups per row");
@@ -279,7 +287,34 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
     static_assert(!(DIRECT && PLAIN), "a direct launch is a grouped one");
     const bool direct = DIRECT || (!PLAIN && a.group_offsets == nullptr && a.group_ids != nullptr);
     const bool grouped = !DIRECT && !PLAIN && a.group_offsets != nullptr;
-    const int64_t band = DIRECT ? a.group_ids[blockIdx.y] : (grouped || direct) ? (a.group_ids ? a.group_ids[blockIdx.y] : static_cast<int>(blockIdx.y)) : 0;
+    int64_t band;
+    float4 x_early[4];  // ROUTE: the wave's first quantizer pass of the token, requested before the routing
+    if constexpr (ROUTE) {
+        // every wave routes the token for itself (no barrier, nothing shared): a few dozen vector
+        // instructions and one expf in front of the first weight request, instead of a launch
+        // (the logits are requested first, the wave's share of the f32 token right behind them: the
+        // selection runs while the token is on its way)
+        const int rl0 = tid & 63;
+        const float rl_lo = rl0 < a.n_groups ? a.route_logits[rl0] : 0.0f, rl_hi = rl0 + 64 < a.n_groups ? a.route_logits[rl0 + 64] : 0.0f;
+        __builtin_amdgcn_sched_barrier(0);
+        {
+            const int sbk = min(4 * (tid >> 6) + (rl0 >> 4), a.n_sb - 1);
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++) x_early[kk] = reinterpret_cast<const float4 *>(a.x)[sbk * 64 + (rl0 & 15) * 4 + kk];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        int sel_e, rank;
+        float rw;
+        moe_route_wave_values(rl_lo, rl_hi, a.n_groups, a.route_k, rl0, sel_e, rw, rank);
+        const unsigned long long mine = __builtin_amdgcn_ballot_w64(rl0 < a.route_k && rank == static_cast<int>(blockIdx.y));
+        band = __builtin_amdgcn_readlane(sel_e, mine ? __builtin_ctzll(mine) : 0);
+        if (blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && tid < a.route_k) {
+            a.route_idx[rank] = sel_e;
+            a.route_w[rank] = rw;
+        }
+    } else {
+        band = DIRECT ? a.group_ids[blockIdx.y] : (grouped || direct) ? (a.group_ids ? a.group_ids[blockIdx.y] : static_cast<int>(blockIdx.y)) : 0;
+    }
     if (band < 0 || (direct && band >= a.n_groups)) return;  // a y-slot past the groups in use, or an id out of range
     const int a0 = DIRECT ? static_cast<int>(blockIdx.y) : grouped ? a.group_offsets[band] : (direct ? static_cast<int>(blockIdx.y) : 0);  // first assignment of this group
     const int n_assign = DIRECT ? 1 : grouped ? a.group_offsets[band + 1] - a0 : (direct ? 1 : NT);
@@ -365,7 +400,12 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
                 }
             };
             float4 xa[4], xb[4];
-            load_pass(xa, 4 * wave);
+            if constexpr (ROUTE) {
+#pragma unroll
+                for (int kk = 0; kk < 4; kk++) xa[kk] = x_early[kk];
+            } else {
+                load_pass(xa, 4 * wave);
+            }
             __builtin_amdgcn_sched_barrier(0);
             if constexpr (RING) ring_prologue(); else
             load_buffer(ra, s0);
@@ -756,6 +796,10 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
     ka.group_ids = a.group_ids;
     ka.n_groups = a.n_groups;
     ka.shared_act = grouped && !a.group_offsets;  // direct call: the one f32 token
+    ka.route_logits = a.route_logits;
+    ka.route_k = a.route_k;
+    ka.route_idx = a.route_idx;
+    ka.route_w = a.route_w;
     if (w2) {
         if (w2->fmt != w->fmt || w2->rows != w->rows || w2->nb != w->nb || w2->row_skip != w->row_skip ||
             w2->planes.row_stride[0] != w->planes.row_stride[0])
@@ -806,7 +850,10 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
         } else if (!plain && ka.shared_act && ka.group_ids && !env_int("CAMELID_HIP_Q4K_GENERAL_ENTRY", 0)) {
             // the decode launch of an expert layer: its own entry
 #define CML_Q4K_DIRECT(SPR_, WHOLE_) hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, SPR_, WHOLE_, false, false, true>), grid, block, lds, st, ka)
-            if (half_tiles && ring && ka.n_sb == 16 * shape.ksplit && env_int("CAMELID_HIP_Q4K_DIRECT_RING", 1))
+            if (ka.route_logits) {
+                if (!(half_tiles && ring && ka.n_sb == 16 * shape.ksplit)) return fail(CML_ERR_UNSUPPORTED, "the routing launch serves rows of 4096 values under 8-row waves");
+                hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, 2, true, false, false, true, 3, 8, true>), grid, block, lds, st, ka);
+            } else if (half_tiles && ring && ka.n_sb == 16 * shape.ksplit && env_int("CAMELID_HIP_Q4K_DIRECT_RING", 1))
                 hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, 2, true, false, false, true, 3, 8>), grid, block, lds, st, ka);
             else if (half_tiles) { if (whole) CML_Q4K_DIRECT(2, true); else CML_Q4K_DIRECT(2, false); }
             else { if (whole) CML_Q4K_DIRECT(1, true); else CML_Q4K_DIRECT(1, false); }
@@ -826,6 +873,20 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
     }
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
+}
+
+// The conditions under which the direct launch above takes the routing variant, for the caller
+// that has to decide between it and a routing launch of its own.
+bool gemv_q4k_direct_can_route(const cml_weight *w, int64_t band_rows, int n_slots, bool pair) {
+    if (w->fmt != CML_Q4_K || band_rows <= 0 || band_rows % 16 != 0 || w->row_skip != 0 || n_slots < 1 || n_slots > 64) return false;
+    if (env_int("CAMELID_HIP_Q4K_GENERAL_ENTRY", 0)) return false;
+    Q4KArgs ka{};
+    ka.n_sb = static_cast<int>(w->nb);
+    ka.sb_stride = w->planes.row_stride[0];
+    const Q4KShape shape = pick_shape(band_rows, ka.n_sb);
+    const int64_t tiles16 = (band_rows + 15) / 16;
+    const bool half_tiles = q4k_rows_per_wave(tiles16, shape.ksplit, static_cast<int64_t>(n_slots) * (pair ? 2 : 1)) == 8;
+    return half_tiles && q4k_ring(ka, shape.ksplit) && ka.n_sb == 16 * shape.ksplit;
 }
 
 // Calibration: the launch of a plain single-token Q4_K matvec (same grid, same lanes, same

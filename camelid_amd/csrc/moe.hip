@@ -22,12 +22,6 @@ namespace cml {
 
 constexpr int kMaxExperts = 128;
 
-// f32::total_cmp as an integer key (larger key = greater value).
-__device__ __forceinline__ int total_key(float v) {
-    const int b = __builtin_bit_cast(int, v);
-    return b ^ static_cast<int>(static_cast<unsigned>(b >> 31) >> 1);
-}
-
 // One thread per token.  reference softmax_top_k, src/inference.rs:13940-13991.
 __global__ __launch_bounds__(64) void moe_route_kernel(const float *__restrict__ logits, int64_t n_tokens, int n_experts,
                                                        int k, int32_t *__restrict__ idx_out, float *__restrict__ w_out) {
@@ -90,16 +84,6 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const float *__restrict__
     }
 }
 
-// Maximum over the 64 lanes of a wave, returned in every lane (all lanes must be active).
-__device__ __forceinline__ int wave_allmax_i32(int v) {
-    v = max(v, row_ror_i32<1>(v));
-    v = max(v, row_ror_i32<2>(v));
-    v = max(v, row_ror_i32<4>(v));
-    v = max(v, row_ror_i32<8>(v));
-    return max(max(__builtin_amdgcn_readlane(v, 0), __builtin_amdgcn_readlane(v, 16)),
-               max(__builtin_amdgcn_readlane(v, 32), __builtin_amdgcn_readlane(v, 48)));
-}
-
 // The same routing with one wave per token (k <= 64), lane l holding experts l and l + 64 during the
 // selection and the l-th selected expert afterwards; the short sequential parts (maximum and sum over
 // the k selected, in selection order) run redundantly in every lane.  Same arithmetic, value for
@@ -110,38 +94,9 @@ __global__ __launch_bounds__(256) void moe_route_wave_kernel(const float *__rest
     const int64_t t_raw = static_cast<int64_t>(blockIdx.x) * 4 + wave;
     const bool live = t_raw < n_tokens;
     const int64_t t = live ? t_raw : n_tokens - 1;  // spare waves repeat the last token and store nothing
-    const float *lg = logits + t * n_experts;
-    bool v0 = lane < n_experts, v1 = lane + 64 < n_experts;
-    const float l0 = v0 ? lg[lane] : 0.0f, l1 = v1 ? lg[lane + 64] : 0.0f;
-    const int k0 = total_key(l0), k1 = total_key(l1);
-    int sel_e = 0;
-    float sel_v = 0.0f;
-    for (int s = 0; s < k; s++) {  // top-k by logit (total order, descending), ties to the lower index
-        const int m = wave_allmax_i32(max(v0 ? k0 : INT32_MIN, v1 ? k1 : INT32_MIN));
-        const unsigned long long b0 = __builtin_amdgcn_ballot_w64(v0 && k0 == m), b1 = __builtin_amdgcn_ballot_w64(v1 && k1 == m);
-        const int e = b0 ? __builtin_ctzll(b0) : (b1 ? 64 + __builtin_ctzll(b1) : 0);
-        const int from = __builtin_amdgcn_readlane(__builtin_bit_cast(int, e < 64 ? l0 : l1), e & 63);
-        if (e == lane) v0 = false;
-        if (e == lane + 64) v1 = false;
-        if (lane == s) {
-            sel_e = e;
-            sel_v = __builtin_bit_cast(float, from);
-        }
-    }
-    float mx = -INFINITY;
-    for (int s = 0; s < k; s++) mx = fmaxf(mx, __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sel_v), s)));
-    const float wv = (lane < k && fabsf(sel_v) < INFINITY) ? expf(sel_v - mx) : 0.0f;  // is_finite: NaN and inf give 0
-    float sum = 0.0f;
-    for (int s = 0; s < k; s++) sum = sum + __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wv), s));
-    const float w = sum > 0.0f ? wv / sum : 1.0f / static_cast<float>(k);
-    // re-sort by weight (descending), ties to the lower index: the rank of (w, index) in that total order
-    const int wk = total_key(w);
-    int rank = 0;
-    for (int s = 0; s < k; s++) {
-        const int ok = total_key(__builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, w), s)));
-        const int oe = __builtin_amdgcn_readlane(sel_e, s);
-        rank += (ok > wk || (ok == wk && oe < sel_e)) ? 1 : 0;
-    }
+    int sel_e, rank;
+    float w;
+    moe_route_wave(logits + t * n_experts, n_experts, k, lane, sel_e, w, rank);
     if (live && lane < k) {
         idx_out[t * k + rank] = sel_e;
         w_out[t * k + rank] = w;
@@ -360,6 +315,8 @@ struct MoeWorkspace {
     int32_t *offsets, *assign_token, *slot_to_assign, *group_ids;
     float *g, *u, *y, *hd;
     int8_t *hq;
+    int32_t *route_idx;  // routing results of the entry that takes logits
+    float *route_w;
     size_t total;
 };
 
@@ -384,6 +341,8 @@ static MoeWorkspace carve(void *base, int64_t hidden, int64_t ff, int64_t n_toke
     w.hq = reinterpret_cast<int8_t *>(take(A * ff));
     w.hd = reinterpret_cast<float *>(take(A * ((ff + 31) / 32) * 4));
     w.y = reinterpret_cast<float *>(take(A * hidden * 4));
+    w.route_idx = reinterpret_cast<int32_t *>(take(A * 4));
+    w.route_w = reinterpret_cast<float *>(take(A * 4));
     w.total = at;
     return w;
 }
@@ -494,9 +453,10 @@ int cml_moe_ffn(const cml_weight *gate, const cml_weight *up, const cml_weight *
                           CML_GLU_SILU, stream);
 }
 
-int cml_moe_ffn_ex(const cml_weight *gate, const cml_weight *up, const cml_weight *down, int n_experts, int k,
-                   const int32_t *idx_dev, const float *weight_dev, const float *x_dev, int64_t n_tokens, float *out_dev,
-                   void *workspace_dev, size_t workspace_bytes, int glu, cml_stream_t stream) {
+// logits_dev non-null: the call routes itself (Mixtral routing) into the workspace; idx_dev / weight_dev are ignored.
+static int moe_ffn_impl(const cml_weight *gate, const cml_weight *up, const cml_weight *down, int n_experts, int k,
+                        const int32_t *idx_dev, const float *weight_dev, const float *logits_dev, const float *x_dev, int64_t n_tokens,
+                        float *out_dev, void *workspace_dev, size_t workspace_bytes, int glu, cml_stream_t stream) {
     if (!ready()) return fail(CML_ERR_UNAVAILABLE, "cml_init has not succeeded");
     if (!gate || !down) return fail(CML_ERR_INVALID, "null weight");
     if (glu != CML_GLU_SILU && glu != CML_GLU_GELU_TANH) return fail(CML_ERR_INVALID, "unknown expert activation %d", glu);
@@ -514,7 +474,7 @@ int cml_moe_ffn_ex(const cml_weight *gate, const cml_weight *up, const cml_weigh
     if (hidden % (act_in == 2 ? 256 : 32) || ff % (act_mid == 2 ? 256 : 32))
         return fail(CML_ERR_SHAPE, "hidden and ff must be whole blocks of the expert formats");
     if (n_tokens == 0) return CML_OK;
-    if (!idx_dev || !weight_dev || !x_dev || !out_dev || !workspace_dev) return fail(CML_ERR_INVALID, "null pointer");
+    if ((!logits_dev && (!idx_dev || !weight_dev)) || !x_dev || !out_dev || !workspace_dev) return fail(CML_ERR_INVALID, "null pointer");
     if ((reinterpret_cast<uintptr_t>(x_dev) & 15u) || (reinterpret_cast<uintptr_t>(workspace_dev) & 255u))
         return fail(CML_ERR_INVALID, "x must be 16-byte and the workspace 256-byte aligned");
     const MoeWorkspace ws = carve(workspace_dev, hidden, ff, n_tokens, k, n_experts);
@@ -537,6 +497,19 @@ int cml_moe_ffn_ex(const cml_weight *gate, const cml_weight *up, const cml_weigh
     // much to re-quantize in every workgroup).
     const bool q4k_direct = fused_decode && act_in == 2 && act_mid == 2;
     const bool direct = b32_direct || q4k_direct;
+    // Routing: inside the gate|up launch where that launch can do it (one token, Q4_K experts, rows of
+    // 4096 values: every wave routes the token itself and the first workgroup leaves the result for
+    // the launches behind it), a launch of its own otherwise.
+    bool route_in_launch = false;
+    if (logits_dev) {
+        idx_dev = ws.route_idx;
+        weight_dev = ws.route_w;
+        route_in_launch = q4k_direct && k <= 64 && env_int("CAMELID_HIP_MOE_FOLD_ROUTE", 1) &&
+                          gemv_q4k_direct_can_route(gate, fused_gate_up ? 2 * ff : ff, n_slots, up != nullptr);
+        if (!route_in_launch) {
+            if (int rc = cml_moe_route_top_k(logits_dev, n_tokens, n_experts, k, ws.route_idx, ws.route_w, stream)) return rc;
+        }
+    }
     if (!fused_decode) {
         if (int rc = launch_quantize_act(act_in, x_dev, n_tokens, hidden, ws.xq, ws.xd, st)) return rc;
     }
@@ -571,7 +544,14 @@ int cml_moe_ffn_ex(const cml_weight *gate, const cml_weight *up, const cml_weigh
             if (int rc = launch_gemv_b32_grouped(a, token, st)) return rc;
         }
     } else if (fused_decode) {
+        if (route_in_launch) {
+            a.route_logits = logits_dev;
+            a.route_k = k;
+            a.route_idx = ws.route_idx;
+            a.route_w = ws.route_w;
+        }
         if (int rc = launch_gemv_q4k_f32_grouped_pair(a, up, up ? ws.u : nullptr, x_dev, st)) return rc;
+        a.route_logits = nullptr;
     } else if (fused_gate_up) {
         if (int rc = launch_expert_matmul(a, st)) return rc;
     } else if (gate->fmt == CML_Q4_K && a.n_tokens >= env_int("CAMELID_HIP_Q4K_MFMA_MIN_TOKENS", 4) && env_int("CAMELID_HIP_MOE_PAIR_LAUNCH", 1)) {
@@ -617,6 +597,22 @@ int cml_moe_ffn_ex(const cml_weight *gate, const cml_weight *up, const cml_weigh
                        direct ? idx_dev : nullptr, n_experts);
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
+}
+
+int cml_moe_ffn_ex(const cml_weight *gate, const cml_weight *up, const cml_weight *down, int n_experts, int k,
+                   const int32_t *idx_dev, const float *weight_dev, const float *x_dev, int64_t n_tokens, float *out_dev,
+                   void *workspace_dev, size_t workspace_bytes, int glu, cml_stream_t stream) {
+    return moe_ffn_impl(gate, up, down, n_experts, k, idx_dev, weight_dev, nullptr, x_dev, n_tokens, out_dev, workspace_dev, workspace_bytes, glu,
+                        stream);
+}
+
+int cml_moe_ffn_logits(const cml_weight *gate, const cml_weight *up, const cml_weight *down, int n_experts, int k,
+                       const float *logits_dev, const float *x_dev, int64_t n_tokens, float *out_dev, void *workspace_dev,
+                       size_t workspace_bytes, cml_stream_t stream) {
+    if (!up) return fail(CML_ERR_INVALID, "null weight");
+    if (!logits_dev && n_tokens > 0) return fail(CML_ERR_INVALID, "null pointer");
+    return moe_ffn_impl(gate, up, down, n_experts, k, nullptr, nullptr, logits_dev, x_dev, n_tokens, out_dev, workspace_dev, workspace_bytes,
+                        CML_GLU_SILU, stream);
 }
 
 }  // extern "C"

@@ -337,6 +337,19 @@ int cml_moe_ffn_ex(const cml_weight *gate, const cml_weight *up, const cml_weigh
                    int64_t n_tokens, float *out_dev, void *workspace_dev, size_t workspace_bytes,
                    int glu, cml_stream_t stream);
 
+/* cml_moe_route_top_k and cml_moe_ffn as one call: logits_dev f32[n_tokens *
+ * n_experts] are the router's outputs (what the reference's mixtral_moe_ffn
+ * has after its router projection, src/inference.rs:14168-14172; routing and
+ * expert lane :14173-14280).  Same results, bit for bit, as the two calls.  One
+ * token on Q4_K experts with rows of 4096 values is routed inside the gate|up
+ * launch (three launches per layer instead of four); every other shape runs
+ * the routing launch first.  The routed experts and weights are kept in the
+ * workspace. */
+int cml_moe_ffn_logits(const cml_weight *gate, const cml_weight *up, const cml_weight *down,
+                       int n_experts, int k, const float *logits_dev, const float *x_dev,
+                       int64_t n_tokens, float *out_dev, void *workspace_dev, size_t workspace_bytes,
+                       cml_stream_t stream);
+
 /* The pieces cml_moe_ffn is made of, for callers that schedule the expert
  * lane themselves.
  * cml_moe_plan groups the n_tokens*k routed slots by expert, keeping (token,

@@ -66,6 +66,23 @@ def gpu_moe(gate, up, down, E, k, idx_dev, w_dev, x, glu=None):
     return out.to_numpy(np.float32, (T, hidden))
 
 
+def gpu_moe_logits(gate, up, down, E, k, logits, x):
+    """cml_moe_ffn_logits: routing and expert lane in one call; the workspace is poisoned first."""
+    T, hidden = x.shape
+    ff = down.cols
+    xd = DeviceBuffer.from_numpy(x)
+    ld = DeviceBuffer.from_numpy(np.ascontiguousarray(logits, np.float32))
+    out = DeviceBuffer(T * hidden * 4)
+    out.fill(0xFF)
+    ws_bytes = lib().cml_moe_workspace_bytes(gate.fmt, hidden, ff, T, k, E)
+    ws = DeviceBuffer(ws_bytes)
+    ws.fill(0xFF)
+    check(lib().cml_moe_ffn_logits(gate.handle, up.handle, down.handle, E, k, ld.ptr, xd.ptr, T, out.ptr, ws.ptr, ws_bytes, None),
+          "cml_moe_ffn_logits")
+    check(lib().cml_stream_sync(None))
+    return out.to_numpy(np.float32, (T, hidden))
+
+
 def test_route_top_k_matches_oracle():
     rng = np.random.default_rng(300)
     logits = rng.standard_normal((257, 8)).astype(np.float32)
@@ -130,6 +147,47 @@ def test_moe_ffn_small_matches_oracle(T):
     assert G.max_rel(got, want) <= 1e-5
     got2 = gpu_moe(wg, wu, wd, E, k, idx_dev, w_dev, x)   # default K-split policy
     assert G.max_rel(got2, want) <= 1e-5
+
+
+@pytest.mark.parametrize("T", [1, 3, 9])
+@pytest.mark.parametrize("E,k,hidden,ff", [(8, 2, 512, 1024), (16, 4, 1024, 512), (5, 5, 256, 256)])
+def test_moe_ffn_logits_is_route_then_ffn(E, k, hidden, ff, T):
+    """cml_moe_ffn_logits on shapes its gate|up launch does not route itself: a routing launch into the
+    workspace, then the expert lane -- the bits of cml_moe_route_top_k followed by cml_moe_ffn; infinite
+    and NaN logits included."""
+    gate, up, down = _experts(E, hidden, ff, 340 + E)
+    rng = np.random.default_rng(341 + T)
+    x = rng.standard_normal((T, hidden)).astype(np.float32)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    logits[0, 1] = np.inf
+    if T > 1:
+        logits[1, 0] = np.nan
+        logits[T - 1, :] = 0.25   # every expert ties
+    wg = Weight.upload(B.CML_Q4_K, E * ff, hidden, gate)
+    wu = Weight.upload(B.CML_Q4_K, E * ff, hidden, up)
+    wd = Weight.upload(B.CML_Q4_K, E * hidden, ff, down)
+    G.say(f"moe ffn from logits E={E} k={k} {hidden}x{ff} T={T}")
+    want = gpu_moe(wg, wu, wd, E, k, *gpu_route(logits, k)[:2], x)
+    assert G.same_bits(gpu_moe_logits(wg, wu, wd, E, k, logits, x), want)
+
+
+def test_moe_ffn_logits_rejects_bad_arguments():
+    E, k, hidden, ff = 4, 2, 256, 256
+    gate, up, down = _experts(E, hidden, ff, 350)
+    wg = Weight.upload(B.CML_Q4_K, E * ff, hidden, gate)
+    wu = Weight.upload(B.CML_Q4_K, E * ff, hidden, up)
+    wd = Weight.upload(B.CML_Q4_K, E * hidden, ff, down)
+    x = DeviceBuffer.from_numpy(np.zeros((1, hidden), np.float32))
+    lg = DeviceBuffer.from_numpy(np.zeros((1, E), np.float32))
+    out = DeviceBuffer(hidden * 4)
+    ws_bytes = lib().cml_moe_workspace_bytes(B.CML_Q4_K, hidden, ff, 1, k, E)
+    ws = DeviceBuffer(ws_bytes)
+    L = lib()
+    assert L.cml_moe_ffn_logits(wg.handle, wu.handle, wd.handle, E, k, None, x.ptr, 1, out.ptr, ws.ptr, ws_bytes, None) == 2
+    assert L.cml_moe_ffn_logits(wg.handle, None, wd.handle, E, k, lg.ptr, x.ptr, 1, out.ptr, ws.ptr, ws_bytes, None) == 2
+    assert L.cml_moe_ffn_logits(wg.handle, wu.handle, wd.handle, E, E + 1, lg.ptr, x.ptr, 1, out.ptr, ws.ptr, ws_bytes, None) == 3
+    assert L.cml_moe_ffn_logits(wg.handle, wu.handle, wd.handle, E, k, lg.ptr, x.ptr, 1, out.ptr, ws.ptr, ws_bytes - 256, None) == 3
+    assert L.cml_moe_ffn_logits(wg.handle, wu.handle, wd.handle, E, k, lg.ptr, x.ptr, 0, out.ptr, ws.ptr, ws_bytes, None) == 0
 
 
 @pytest.mark.parametrize("T", [1, 2, 5, 32])
@@ -291,6 +349,16 @@ def test_c5_mixtral_shaped_moe(T):
     idx_dev, w_dev, idx, w = gpu_route(logits, k)
     G.say(f"C5 Mixtral-shaped MoE T={T}: device run")
     got = gpu_moe(wg, wu, wd, E, k, idx_dev, w_dev, x)
+    # routing and expert lane as one call (one token: routed inside the gate|up launch): the same bits,
+    # also with the routing as a launch of its own and on logits that tie
+    G.say(f"C5 Mixtral-shaped MoE T={T}: the entry that takes logits")
+    assert G.same_bits(gpu_moe_logits(wg, wu, wd, E, k, logits, x), got)
+    with G.env(CAMELID_HIP_MOE_FOLD_ROUTE="0"):
+        assert G.same_bits(gpu_moe_logits(wg, wu, wd, E, k, logits, x), got)
+    tied = logits.copy()
+    tied[:, 5] = tied[:, 2]
+    tied[:, 7] = tied[:, 2]
+    assert G.same_bits(gpu_moe_logits(wg, wu, wd, E, k, tied, x), gpu_moe(wg, wu, wd, E, k, *gpu_route(tied, k)[:2], x))
     tt = min(T, 4)   # the oracle walks 3 full expert matvecs per (token, expert): bound the CPU work
     want = oracle.moe_ffn(B.CML_Q4_K, gate, up, down, E, k, hidden, ff, logits[:tt], x[:tt], threads=16)
     assert G.max_rel(got[:tt], want) <= 1e-5
