@@ -434,6 +434,66 @@ def bench_moe(name: str, K: int, W: int, seed: int, cpu_seconds: float) -> int:
     return 0
 
 
+PAIR_CONFIGS = {
+    # name -> (format, rows, cols): one token against TWO weights of one shape that read it (gate and up of a dense FFN)
+    "q4k_pair_14336x4096": ("Q4_K", 14336, 4096),
+    "q4k_pair_4096x4096": ("Q4_K", 4096, 4096),
+}
+
+
+def bench_pair(name: str, K: int, W: int, seed: int) -> int:
+    """cml_matmul_f32_pair: one f32 token, two weights, one launch where the shape is served; beside it
+    the same step as two cml_matmul_f32 calls."""
+    L = lib()
+    fmt_name, rows, cols = PAIR_CONFIGS[name]
+    fmt = B.FORMATS[fmt_name]
+    wire_a, wire_b = synth_weight(fmt, rows, cols, seed), synth_weight(fmt, rows, cols, seed + 7)
+    copies = max(2, min(32, -(-600_000_000 // (2 * wire_a.nbytes))))
+    wa = [Weight.upload(fmt, rows, cols, wire_a) for _ in range(copies)]
+    wb = [Weight.upload(fmt, rows, cols, wire_b) for _ in range(copies)]
+    x = np.random.default_rng(seed + 1).standard_normal((1, cols)).astype(np.float32)
+    alg = 2 * wire_a.nbytes + 4 * cols + 2 * 4 * rows
+    stream = C.c_void_p()
+    check(L.cml_stream_create(C.byref(stream)))
+    xd = DeviceBuffer.from_numpy(x)
+    ws_bytes = L.cml_matmul_workspace_bytes(fmt, cols, 1)
+    ws = DeviceBuffer(ws_bytes)
+    oa, ob = DeviceBuffer(rows * 4), DeviceBuffer(rows * 4)
+
+    def pair(i):
+        check(L.cml_matmul_f32_pair(wa[i % copies].handle, wb[i % copies].handle, xd.ptr, oa.ptr, ob.ptr, ws.ptr, ws_bytes, stream),
+              "cml_matmul_f32_pair")
+
+    def two(i):
+        check(L.cml_matmul_f32(wa[i % copies].handle, xd.ptr, 1, oa.ptr, ws.ptr, ws_bytes, stream), "cml_matmul_f32")
+        check(L.cml_matmul_f32(wb[i % copies].handle, xd.ptr, 1, ob.ptr, ws.ptr, ws_bytes, stream), "cml_matmul_f32")
+
+    for i in range(W):
+        pair(i)
+    check(L.cml_stream_sync(stream))
+    timers = [Timer(stream) for _ in range(32)]
+    ms = steps_ms(stream, pair, K, timers)[0]
+    ms_two = steps_ms(stream, two, K, timers)[0]
+    check(L.cml_stream_sync(stream))
+    got = oa.to_numpy(np.float32, (rows,))
+    if not np.all(np.isfinite(got)):
+        print("non-finite output", file=sys.stderr)
+        return 4
+    gbs = alg / (ms * 1e-3) / 1e9
+    print(json.dumps({
+        "metric": f"{fmt_name} matvec pair (one token, two weights) µs + achieved HBM GB/s, 2 x {rows}x{cols}",
+        "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": round(ms, 6),
+        "us_per_call": round(ms * 1e3, 3), "pct_of_hbm_peak": round(100.0 * gbs / HBM_PEAK_GBS, 2), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
+        "config": {"workload": name, "format": fmt_name, "rows": rows, "cols": cols, "tokens": 1, "weights": 2,
+                   "algorithmic_bytes_per_call": alg, "weight_copies_rotated": copies,
+                   "step": "cml_matmul_f32_pair: quantize the token + both fused dequantize-matvecs, graph replay",
+                   "as_two_calls_us": round(ms_two * 1e3, 3)},
+        "roofline": {"bound": "hbm", "kernel": "gemv_q4k_kernel, grid.z = 2 (one launch)", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "us_per_launch": round(ms * 1e3, 3)}}, ensure_ascii=False))
+    return 0
+
+
 PRODUCER_CONFIGS = {
     # name -> (cols, tokens): rms_norm fused with the Q8_K quantizer, the step upstream of a projection
     "rmsnorm_q8k_4096_t1": (4096, 1),
@@ -542,7 +602,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--config", default="q4k_14336x4096_n1",
-                    help="one of: " + ", ".join(sorted(CONFIGS) + sorted(MOE_CONFIGS) + sorted(PRODUCER_CONFIGS))
+                    help="one of: " + ", ".join(sorted(CONFIGS) + sorted(MOE_CONFIGS) + sorted(PAIR_CONFIGS) + sorted(PRODUCER_CONFIGS))
                     + "; or any <format>_<rows>x<cols>_n<tokens>, e.g. q8_0_14336x4352_n1")
     ap.add_argument("--copies", type=int, default=0, help="distinct weight copies to rotate over (0 = enough for ~600 MB)")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="time budget of the CPU baseline leg (0 = skip)")
@@ -577,6 +637,8 @@ def main() -> int:
         return calibrate_copy(args.calibrate_copy, max(1, args.steps), max(0, args.warmup))
     if args.config in PRODUCER_CONFIGS:
         return bench_producer(args.config, max(1, args.steps), max(0, args.warmup), args.seed)
+    if args.config in PAIR_CONFIGS:
+        return bench_pair(args.config, max(1, args.steps), max(0, args.warmup), args.seed)
     if args.config in MOE_CONFIGS:
         return bench_moe(args.config, max(1, args.steps), max(0, args.warmup), args.seed, args.cpu_seconds)
     if args.config in CONFIGS:

@@ -833,6 +833,30 @@ int cml_matmul_f32(const cml_weight *w, const float *x_dev, int64_t n_tokens, fl
     return dispatch(plain_args(w, q, s, n_tokens, out_dev), st);
 }
 
+// One token against TWO weights of one shape that read the same activation (gate and up of a dense
+// FFN): Q4_K rows of up to 8192 values run as one launch that quantizes the token once per
+// workgroup and streams both weights (grid.z = 2); every other case is two cml_matmul_f32 calls.
+// Same bits as the two calls.
+int cml_matmul_f32_pair(const cml_weight *w_a, const cml_weight *w_b, const float *x_dev, float *out_a_dev, float *out_b_dev,
+                        void *workspace_dev, size_t workspace_bytes, cml_stream_t stream) {
+    if (!w_a || !w_b) return fail(CML_ERR_INVALID, "null weight");
+    if (int rc = check_ready()) return rc;
+    if (w_a->cols != w_b->cols) return fail(CML_ERR_SHAPE, "the two weights read activations of %lld and %lld values", (long long)w_a->cols, (long long)w_b->cols);
+    if (!x_dev || !out_a_dev || !out_b_dev || !workspace_dev) return fail(CML_ERR_INVALID, "null pointer");
+    if (misaligned16(x_dev) || misaligned16(workspace_dev)) return fail(CML_ERR_INVALID, "activations and workspace must be 16-byte aligned");
+    const bool same_shape = w_a->fmt == w_b->fmt && w_a->rows == w_b->rows && w_a->nb == w_b->nb && w_a->row_skip == w_b->row_skip &&
+                            w_a->planes.row_stride[0] == w_b->planes.row_stride[0];
+    const int fuse = env_int("CAMELID_HIP_FUSED_QUANT", 1);
+    if (same_shape && w_a->rows > 0 && w_a->fmt == CML_Q4_K && !q4k_lane_order() && (fuse == 2 || (fuse == 1 && w_a->nb <= 32)) &&
+        env_int("CAMELID_HIP_PAIR_LAUNCH", 1)) {
+        const int frc = launch_gemv_q4k_f32_pair(w_a, w_b, x_dev, out_a_dev, out_b_dev, as_stream(stream));
+        if (frc == CML_OK) g_runs.fetch_add(2, std::memory_order_relaxed);
+        return frc;
+    }
+    if (int rc = cml_matmul_f32(w_a, x_dev, 1, out_a_dev, workspace_dev, workspace_bytes, stream)) return rc;
+    return cml_matmul_f32(w_b, x_dev, 1, out_b_dev, workspace_dev, workspace_bytes, stream);
+}
+
 // The same call for hosts that may not allocate (a stream under graph capture, a serving loop with
 // a fixed memory budget): the quantized activation is staged in the library's own static device
 // array instead of a caller workspace.  Nothing here allocates or frees, on the host or the device.

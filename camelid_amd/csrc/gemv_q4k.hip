@@ -262,8 +262,9 @@ __device__ __forceinline__ void q4k_compute(const Q4KRegs<U> &r, const Q4KLane &
 // DIRECT: the decode launch of an expert layer (one shared f32 token, y-slot = routed assignment, z = which of up to
 // two weights) with its mode known at compile time, for the same reason (one-token MoE layer 44.1 -> 42.6 us).
 template <int NT, bool INTS, bool FUSEQ = false, int SPR = 1, bool WHOLE = false, bool PLAIN = false, bool LOADONLY = false, bool DIRECT = false,
-          int RING = 0, int NSTEPS = 0, bool ROUTE = false>
+          int RING = 0, int NSTEPS = 0, bool ROUTE = false, bool PAIR = false>
 __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
+    static_assert(!PAIR || (PLAIN && FUSEQ && NT == 1), "a plain pair: one f32 token against two weights of one shape (grid.z = 2)");
     static_assert(!ROUTE || DIRECT, "only the direct launch routes");
     static_assert(!FUSEQ || ((NT == 1 || (NT == 2 && PLAIN)) && !INTS),
                   "the fused quantizer serves single-token calls and plain two-token calls (contiguous f32 rows)");
@@ -319,7 +320,7 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
     const int a0 = DIRECT ? static_cast<int>(blockIdx.y) : grouped ? a.group_offsets[band] : (direct ? static_cast<int>(blockIdx.y) : 0);  // first assignment of this group
     const int n_assign = DIRECT ? 1 : grouped ? a.group_offsets[band + 1] - a0 : (direct ? 1 : NT);
     if (n_assign <= 0) return;  // an expert nobody routed to: the whole workgroup leaves
-    const bool second = DIRECT ? blockIdx.z == 1 : (!PLAIN && gridDim.z > 1 && blockIdx.z == 1);
+    const bool second = (DIRECT || PAIR) ? blockIdx.z == 1 : (!PLAIN && gridDim.z > 1 && blockIdx.z == 1);
     const uint8_t *w = (second ? a.w2 : a.w) + band * (a.rows / 16) * kQ4KChunk;
 
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
@@ -682,11 +683,11 @@ static bool q4k_ring(const Q4KArgs &ka, int ksplit, int spr = 2) {
 // 8.87 -> 8.44 us, the single-token one 6.89 -> 6.81); every other length runs the loop.
 // 8-row waves (SPR = 2, three slots) step two super-blocks at a time: rows / K parts of 3072, 3584
 // and 4096 values are 6, 7 and 8 steps; 16-row waves (SPR = 1, four slots) step one: 12, 14, 16.
-template <int NT, bool FUSEQ, int SPR, bool LOADONLY = false>
+template <int NT, bool FUSEQ, int SPR, bool LOADONLY = false, bool PAIR = false>
 static void launch_q4k_ring(const Q4KArgs &ka, int ksplit, dim3 grid, dim3 block, size_t lds, hipStream_t st) {
     constexpr int SLOTS = SPR == 2 ? 3 : 4;
     const int steps = ka.n_sb / (SPR * ksplit);
-#define CML_Q4K_RING(N_) hipLaunchKernelGGL((gemv_q4k_kernel<NT, false, FUSEQ, SPR, true, true, LOADONLY, false, SLOTS, N_>), grid, block, lds, st, ka)
+#define CML_Q4K_RING(N_) hipLaunchKernelGGL((gemv_q4k_kernel<NT, false, FUSEQ, SPR, true, true, LOADONLY, false, SLOTS, N_, false, PAIR>), grid, block, lds, st, ka)
     if constexpr (LOADONLY && SPR == 2) {
         if (steps == 8) CML_Q4K_RING(8);
         else CML_Q4K_RING(0);
@@ -858,6 +859,10 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
             else if (half_tiles) { if (whole) CML_Q4K_DIRECT(2, true); else CML_Q4K_DIRECT(2, false); }
             else { if (whole) CML_Q4K_DIRECT(1, true); else CML_Q4K_DIRECT(1, false); }
 #undef CML_Q4K_DIRECT
+        } else if (!grouped && w2 && half_tiles && ring && !env_int("CAMELID_HIP_Q4K_GENERAL_ENTRY", 0)) {
+            launch_q4k_ring<1, true, 2, false, true>(ka, shape.ksplit, grid, block, lds, st);  // a plain pair: grid.z = 2
+        } else if (!grouped && w2 && !half_tiles && q4k_ring(ka, shape.ksplit, 1) && !env_int("CAMELID_HIP_Q4K_GENERAL_ENTRY", 0)) {
+            launch_q4k_ring<1, true, 1, false, true>(ka, shape.ksplit, grid, block, lds, st);
         } else if (half_tiles && ring && plain) {
             launch_q4k_ring<1, true, 2>(ka, shape.ksplit, grid, block, lds, st);
         } else if (!half_tiles && plain && q4k_ring(ka, shape.ksplit, 1)) {
@@ -899,6 +904,16 @@ int launch_gemv_q4k_loads_only(const cml_weight *w, float *out, hipStream_t st) 
     a.n_tokens = 1;
     a.n_groups = 1;
     return launch_q4k_f32(a, nullptr, nullptr, nullptr, st, true);
+}
+
+// One f32 token against two weights of one shape (the gate and up projections of a dense FFN) in one launch.
+int launch_gemv_q4k_f32_pair(const cml_weight *w, const cml_weight *w2, const float *x, float *out, float *out2, hipStream_t st) {
+    MatArgs a{};
+    a.w = w;
+    a.out = out;
+    a.n_tokens = 1;
+    a.n_groups = 1;
+    return launch_q4k_f32(a, w2, out2, x, st);
 }
 
 int launch_gemv_q4k_f32(const cml_weight *w, const float *x, float *out, hipStream_t st, int n_tokens) {

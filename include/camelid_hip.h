@@ -284,6 +284,17 @@ size_t cml_matmul_workspace_bytes(int fmt, int64_t cols, int64_t n_tokens);
 int cml_matmul_f32(const cml_weight *w, const float *x_dev, int64_t n_tokens, float *out_dev,
                    void *workspace_dev, size_t workspace_bytes, cml_stream_t stream);
 
+/* cml_matmul_f32 for ONE token against TWO weights that read the same
+ * activation -- the gate and up projections of a dense FFN, which the reference
+ * runs as two matvecs on one shared quantized activation (SharedActivation,
+ * src/gemma4_runtime.rs:1288-1340; gate / up at :5591-5592 and :5965-5966).  Q4_K weights of one shape with rows of up to 8192 values run
+ * as one launch (the token quantized once per workgroup, both weights
+ * streamed); every other pair is two cml_matmul_f32 calls.  Same bits as the
+ * two calls.  workspace as for cml_matmul_f32 with n_tokens = 1. */
+int cml_matmul_f32_pair(const cml_weight *w_a, const cml_weight *w_b, const float *x_dev,
+                        float *out_a_dev, float *out_b_dev, void *workspace_dev,
+                        size_t workspace_bytes, cml_stream_t stream);
+
 /* cml_matmul_f32 without a workspace argument, for callers that cannot allocate
  * device memory (a stream under HIP graph capture, a serving loop with a fixed
  * memory budget, a harness that forbids hipMalloc).  It has no counterpart in

@@ -834,3 +834,44 @@ def test_q4k_single_token_entry_points_give_the_same_bits(rows, cols):
         if band is not None:
             assert G.same_bits(G.gpu_gemm(band, s, q), want[5:rows - 4])
             assert G.same_bits(G.gpu_matmul_f32(band, x), want[5:rows - 4])
+
+
+@pytest.mark.parametrize("name,fmt,rows,cols", [("Q4_K", B.CML_Q4_K, 14336, 4096), ("Q4_K", B.CML_Q4_K, 200, 4096), ("Q4_K", B.CML_Q4_K, 1000, 3584),
+                                                ("Q4_K", B.CML_Q4_K, 530, 2304), ("Q4_K", B.CML_Q4_K, 4096, 14336), ("Q4_K", B.CML_Q4_K, 17000, 1024),
+                                                ("Q6_K", B.CML_Q6_K, 300, 1024), ("Q8_0", B.CML_Q8_0, 700, 2048), ("Q4_0", B.CML_Q4_0, 64, 96)])
+def test_matmul_f32_pair_is_two_single_calls(name, fmt, rows, cols):
+    """cml_matmul_f32_pair (one token, two weights that read it: gate and up of a dense FFN): the bits
+    of two cml_matmul_f32 calls -- where it runs as one launch (Q4_K, with and without the ring of
+    register buffers, 8- and 16-row waves), where it does not (other formats, long rows), and with
+    the one-launch path switched off; weights of different shapes are two calls."""
+    rng = np.random.default_rng(rows + cols)
+    wa = Weight.upload(fmt, rows, cols, G.synth_weight(fmt, rows, cols, seed=rows + 1))
+    wb = Weight.upload(fmt, rows, cols, G.synth_weight(fmt, rows, cols, seed=rows + 2))
+    x = rng.standard_normal(cols).astype(np.float32)
+
+    def pair(w1, w2):
+        ws_bytes = lib().cml_matmul_workspace_bytes(fmt, cols, 1)
+        xd = DeviceBuffer.from_numpy(x.reshape(1, -1))
+        ws = DeviceBuffer(max(ws_bytes, 16))
+        o1, o2 = DeviceBuffer(w1.rows * 4), DeviceBuffer(w2.rows * 4)
+        o1.fill(0xFF)
+        o2.fill(0xFF)
+        check(lib().cml_matmul_f32_pair(w1.handle, w2.handle, xd.ptr, o1.ptr, o2.ptr, ws.ptr, ws_bytes, None), "cml_matmul_f32_pair")
+        check(lib().cml_stream_sync(None))
+        return o1.to_numpy(np.float32, (w1.rows,)), o2.to_numpy(np.float32, (w2.rows,))
+
+    G.say(f"pair {name} {rows}x{cols}")
+    want_a, want_b = G.gpu_matmul_f32(wa, x), G.gpu_matmul_f32(wb, x)
+    for knobs in ({}, {"CAMELID_HIP_Q4K_RING": "0"}, {"CAMELID_HIP_PAIR_LAUNCH": "0"}, {"CAMELID_HIP_Q4K_ROWS_PER_WAVE": "16"}, {"CAMELID_HIP_Q4K_ROWS_PER_WAVE": "8"}):
+        with G.env(**knobs):
+            got_a, got_b = pair(wa, wb)
+        assert G.same_bits(got_a, want_a), (name, rows, cols, knobs)
+        assert G.same_bits(got_b, want_b), (name, rows, cols, knobs)
+    if rows > 40:   # a second weight of another shape: two calls
+        band = wb.slice(16, rows - 32)
+        got_a, got_c = pair(wa, band)
+        assert G.same_bits(got_a, want_a) and G.same_bits(got_c, want_b[16:rows - 16])
+    L = lib()
+    d = DeviceBuffer(64)
+    assert L.cml_matmul_f32_pair(wa.handle, None, d.ptr, d.ptr, d.ptr, d.ptr, 64, None) == 2
+    assert L.cml_matmul_f32_pair(wa.handle, wb.handle, None, d.ptr, d.ptr, d.ptr, 64, None) == 2
