@@ -359,6 +359,11 @@ def test_c5_mixtral_shaped_moe(T):
     tied[:, 5] = tied[:, 2]
     tied[:, 7] = tied[:, 2]
     assert G.same_bits(gpu_moe_logits(wg, wu, wd, E, k, tied, x), gpu_moe(wg, wu, wd, E, k, *gpu_route(tied, k)[:2], x))
+    odd = logits.copy()
+    odd[:, 1] = np.inf
+    odd[:, 6] = np.nan
+    odd[:, 0] = -np.inf
+    assert G.same_bits(gpu_moe_logits(wg, wu, wd, E, k, odd, x), gpu_moe(wg, wu, wd, E, k, *gpu_route(odd, k)[:2], x))
     tt = min(T, 4)   # the oracle walks 3 full expert matvecs per (token, expert): bound the CPU work
     want = oracle.moe_ffn(B.CML_Q4_K, gate, up, down, E, k, hidden, ff, logits[:tt], x[:tt], threads=16)
     assert G.max_rel(got[:tt], want) <= 1e-5
