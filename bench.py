@@ -438,6 +438,8 @@ PAIR_CONFIGS = {
     # name -> (format, rows, cols): one token against TWO weights of one shape that read it (gate and up of a dense FFN)
     "q4k_pair_14336x4096": ("Q4_K", 14336, 4096),
     "q4k_pair_4096x4096": ("Q4_K", 4096, 4096),
+    "q8_0_pair_8192x2048": ("Q8_0", 8192, 2048),
+    "q4_0_pair_14336x4096": ("Q4_0", 14336, 4096),
 }
 
 
@@ -489,7 +491,7 @@ def bench_pair(name: str, K: int, W: int, seed: int) -> int:
                    "algorithmic_bytes_per_call": alg, "weight_copies_rotated": copies,
                    "step": "cml_matmul_f32_pair: quantize the token + both fused dequantize-matvecs, graph replay",
                    "as_two_calls_us": round(ms_two * 1e3, 3)},
-        "roofline": {"bound": "hbm", "kernel": "gemv_q4k_kernel, grid.z = 2 (one launch)", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS,
+        "roofline": {"bound": "hbm", "kernel": "the single-token matvec kernel of the format, grid.z = 2 (one launch)", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "us_per_launch": round(ms * 1e3, 3)}}, ensure_ascii=False))
     return 0
 

@@ -853,6 +853,12 @@ int cml_matmul_f32_pair(const cml_weight *w_a, const cml_weight *w_b, const floa
         if (frc == CML_OK) g_runs.fetch_add(2, std::memory_order_relaxed);
         return frc;
     }
+    if (same_shape && w_a->rows > 0 && (w_a->fmt == CML_Q8_0 || w_a->fmt == CML_Q4_0) && w_a->planes.row_stride[1] == w_b->planes.row_stride[1] &&
+        (fuse == 2 || (fuse == 1 && w_a->cols <= 8192 && w_a->rows <= 32768)) && env_int("CAMELID_HIP_PAIR_LAUNCH", 1)) {
+        const int frc = launch_gemv_b32_f32_pair(w_a, w_b, x_dev, out_a_dev, out_b_dev, as_stream(stream));
+        if (frc == CML_OK) g_runs.fetch_add(2, std::memory_order_relaxed);
+        if (frc != -1) return frc;
+    }
     if (int rc = cml_matmul_f32(w_a, x_dev, 1, out_a_dev, workspace_dev, workspace_bytes, stream)) return rc;
     return cml_matmul_f32(w_b, x_dev, 1, out_b_dev, workspace_dev, workspace_bytes, stream);
 }

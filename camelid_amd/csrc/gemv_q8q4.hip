@@ -44,6 +44,10 @@ struct B32Args {
     int64_t act_slot_stride;
     int64_t out_slot_stride;
     int early_loads;  // issue the first weight loads ahead of the fused quantizer
+    // PAIR (grid.z = 2): blockIdx.z = 1 works on a second weight of the same shape against the same token
+    const uint8_t *quants2;
+    const uint8_t *scales2;
+    float *out2;
 };
 
 template <int FMT, int UU = 2>
@@ -318,8 +322,9 @@ __device__ __forceinline__ void b32_row_pass_ring(B32Regs<FMT, 1> (&ring)[NB], c
 // FUSEQ (single token): the activation arrives as f32 and every workgroup quantizes it to Q8_0
 // itself, eight lanes per block, straight into the LDS staging area -- the arithmetic of
 // quantize_q8_0_kernel without the launch and the round trip through memory.
-template <int FMT, int P, int NT, bool INTS, bool FUSEQ = false, int WAVES = 4, int NXQ = 0, int U = 2, int RING = 0>
+template <int FMT, int P, int NT, bool INTS, bool FUSEQ = false, int WAVES = 4, int NXQ = 0, int U = 2, int RING = 0, bool PAIR = false>
 __global__ __launch_bounds__(WAVES * 64) void gemv_b32_kernel(B32Args a) {
+    static_assert(!PAIR || (FUSEQ && NT == 1 && !INTS), "a pair: one f32 token against two weights of one shape");
     static_assert(RING == 0 || (RING == 3 && FUSEQ && NXQ > 0 && !INTS), "the ring serves the fused single-launch calls with the activation in registers");
     constexpr int NB = RING ? RING : 1, PRE = RING ? 2 : 1;
     constexpr int T = WAVES * 64;  // threads of a workgroup; its activation prologue is shared by WAVES * (64 / P) rows
@@ -336,15 +341,16 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_b32_kernel(B32Args a) {
     const int64_t band = a.band_ids ? a.band_ids[slot] : 0;
     const int8_t *q = a.q + static_cast<int64_t>(slot) * a.act_slot_stride * nb * 32;
     const float *xs = a.xs + static_cast<int64_t>(slot) * a.act_slot_stride * nb;
-    float *out = a.out + static_cast<int64_t>(slot) * a.out_slot_stride;
+    float *out = (PAIR && blockIdx.z == 1 ? a.out2 : a.out) + static_cast<int64_t>(slot) * a.out_slot_stride;
 
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int r = lane / P, l = lane - r * P;
     const int row = (blockIdx.x * WAVES + wave) * RPW + r;
     const bool live = row < a.rows;
     const int64_t arow = band * a.rows + (live ? row : a.rows - 1);
-    const uint8_t *qrow = a.quants + arow * a.q_stride;
-    const uint8_t *srow = a.scales + arow * a.s_stride;
+    const bool second = PAIR && blockIdx.z == 1;
+    const uint8_t *qrow = (second ? a.quants2 : a.quants) + arow * a.q_stride;
+    const uint8_t *srow = (second ? a.scales2 : a.scales) + arow * a.s_stride;
     const bool leader = (l == P - 1);
     const int n_steps = (nb + P - 1) / P;
     constexpr int UE = U;  // steps per register buffer, also loaded ahead of the prologue
@@ -549,8 +555,14 @@ static int launch_b32_p(const MatArgs &a, hipStream_t st) {
 
 // Single token, f32 activation in: quantize + matvec in one launch.
 template <int FMT, int P>
-static int launch_b32_f32_p(const cml_weight *w, const float *x, float *out, hipStream_t st, int n_tokens) {
+static int launch_b32_f32_p(const cml_weight *w, const float *x, float *out, hipStream_t st, int n_tokens, const cml_weight *w2 = nullptr,
+                            float *out2 = nullptr) {
     B32Args ba{};
+    if (w2) {
+        ba.quants2 = w2->planes.p[0];
+        ba.scales2 = w2->planes.p[1];
+        ba.out2 = out2;
+    }
     ba.quants = w->planes.p[0];
     ba.q_stride = w->planes.row_stride[0];
     ba.scales = w->planes.p[1];
@@ -582,6 +594,22 @@ static int launch_b32_f32_p(const cml_weight *w, const float *x, float *out, hip
     if (waves == 8 && nxq == 4 && !two) nxq = 0;  // 2048 float4 would be 256 blocks; eight waves are launched for at most 128
     if (waves == 16 && nxq != 1) nxq = 0;
     if (waves == 2 && nxq != 0) nxq = 4;  // one register variant for the short workgroup
+    if (w2) {
+        // one token, two weights (grid.z = 2): the 16-lane, eight-wave launches with the token in registers; -1 = not served
+        if constexpr (P == 16) {
+            if (two || waves != 8 || (nxq != 1 && nxq != 2)) return -1;
+            const bool ring = FMT == CML_Q8_0 && (ba.nb + P - 1) / P >= 3 && env_int("CAMELID_HIP_B32_RING", 1);
+            const dim3 grid2(gx, 1, 2);
+            if (ring && nxq == 1) hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, true, 8, 1, 2, 3, true>), grid2, dim3(512), lds, st, ba);
+            else if (ring) hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, true, 8, 2, 2, 3, true>), grid2, dim3(512), lds, st, ba);
+            else if (nxq == 1) hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, true, 8, 1, 2, 0, true>), grid2, dim3(512), lds, st, ba);
+            else hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, true, 8, 2, 2, 0, true>), grid2, dim3(512), lds, st, ba);
+            CML_HIP_TRY(hipGetLastError());
+            return CML_OK;
+        } else {
+            return -1;
+        }
+    }
 #define CML_B32_FUSED(W_, N_) \
     hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, true, W_, N_>), dim3(gx, 1), dim3(W_ * 64), lds, st, ba)
     const bool deep = !two && nxq == 0 && b32_depth(ba.rows, P, ba.nb) == 4;
@@ -635,6 +663,13 @@ static int launch_b32_f32_p(const cml_weight *w, const float *x, float *out, hip
 #undef CML_B32_FUSED
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
+}
+
+// One f32 token against two weights of one shape in one launch; -1 = a shape that launch does not serve.
+int launch_gemv_b32_f32_pair(const cml_weight *w, const cml_weight *w2, const float *x, float *out, float *out2, hipStream_t st) {
+    if (w->rows == 0) return CML_OK;
+    if (b32_lanes(w->fmt, w->rows, w->nb) != 16) return -1;
+    return w->fmt == CML_Q8_0 ? launch_b32_f32_p<CML_Q8_0, 16>(w, x, out, st, 1, w2, out2) : launch_b32_f32_p<CML_Q4_0, 16>(w, x, out, st, 1, w2, out2);
 }
 
 int launch_gemv_b32_f32(const cml_weight *w, const float *x, float *out, hipStream_t st, int n_tokens) {

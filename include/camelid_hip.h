@@ -287,10 +287,12 @@ int cml_matmul_f32(const cml_weight *w, const float *x_dev, int64_t n_tokens, fl
 /* cml_matmul_f32 for ONE token against TWO weights that read the same
  * activation -- the gate and up projections of a dense FFN, which the reference
  * runs as two matvecs on one shared quantized activation (SharedActivation,
- * src/gemma4_runtime.rs:1288-1340; gate / up at :5591-5592 and :5965-5966).  Q4_K weights of one shape with rows of up to 8192 values run
- * as one launch (the token quantized once per workgroup, both weights
- * streamed); every other pair is two cml_matmul_f32 calls.  Same bits as the
- * two calls.  workspace as for cml_matmul_f32 with n_tokens = 1. */
+ * src/gemma4_runtime.rs:1288-1340; gate / up at :5591-5592 and :5965-5966).
+ * Two weights of one shape run as ONE launch (the token quantized once per
+ * workgroup, both weights streamed) for Q4_K rows of up to 8192 values and for
+ * Q8_0 / Q4_0 matrices of 4096 to 32768 rows of up to 4096 values; every other
+ * pair is two cml_matmul_f32 calls.  Same bits as the two calls.  workspace as
+ * for cml_matmul_f32 with n_tokens = 1. */
 int cml_matmul_f32_pair(const cml_weight *w_a, const cml_weight *w_b, const float *x_dev,
                         float *out_a_dev, float *out_b_dev, void *workspace_dev,
                         size_t workspace_bytes, cml_stream_t stream);

@@ -838,11 +838,14 @@ def test_q4k_single_token_entry_points_give_the_same_bits(rows, cols):
 
 @pytest.mark.parametrize("name,fmt,rows,cols", [("Q4_K", B.CML_Q4_K, 14336, 4096), ("Q4_K", B.CML_Q4_K, 200, 4096), ("Q4_K", B.CML_Q4_K, 1000, 3584),
                                                 ("Q4_K", B.CML_Q4_K, 530, 2304), ("Q4_K", B.CML_Q4_K, 4096, 14336), ("Q4_K", B.CML_Q4_K, 17000, 1024),
-                                                ("Q6_K", B.CML_Q6_K, 300, 1024), ("Q8_0", B.CML_Q8_0, 700, 2048), ("Q4_0", B.CML_Q4_0, 64, 96)])
+                                                ("Q6_K", B.CML_Q6_K, 300, 1024), ("Q8_0", B.CML_Q8_0, 700, 2048), ("Q4_0", B.CML_Q4_0, 64, 96),
+                                                ("Q8_0", B.CML_Q8_0, 8192, 2048), ("Q8_0", B.CML_Q8_0, 4099, 4096), ("Q4_0", B.CML_Q4_0, 4100, 4096),
+                                                ("Q4_0", B.CML_Q4_0, 5000, 1056), ("Q8_0", B.CML_Q8_0, 4500, 96)])
 def test_matmul_f32_pair_is_two_single_calls(name, fmt, rows, cols):
     """cml_matmul_f32_pair (one token, two weights that read it: gate and up of a dense FFN): the bits
     of two cml_matmul_f32 calls -- where it runs as one launch (Q4_K, with and without the ring of
-    register buffers, 8- and 16-row waves), where it does not (other formats, long rows), and with
+    register buffers, 8- and 16-row waves; Q8_0 / Q4_0 on at least 4096 rows of 16 lanes), where it
+    does not (Q6_K, few rows, long rows), and with
     the one-launch path switched off; weights of different shapes are two calls."""
     rng = np.random.default_rng(rows + cols)
     wa = Weight.upload(fmt, rows, cols, G.synth_weight(fmt, rows, cols, seed=rows + 1))
@@ -862,7 +865,8 @@ def test_matmul_f32_pair_is_two_single_calls(name, fmt, rows, cols):
 
     G.say(f"pair {name} {rows}x{cols}")
     want_a, want_b = G.gpu_matmul_f32(wa, x), G.gpu_matmul_f32(wb, x)
-    for knobs in ({}, {"CAMELID_HIP_Q4K_RING": "0"}, {"CAMELID_HIP_PAIR_LAUNCH": "0"}, {"CAMELID_HIP_Q4K_ROWS_PER_WAVE": "16"}, {"CAMELID_HIP_Q4K_ROWS_PER_WAVE": "8"}):
+    for knobs in ({}, {"CAMELID_HIP_Q4K_RING": "0", "CAMELID_HIP_B32_RING": "0"}, {"CAMELID_HIP_PAIR_LAUNCH": "0"}, {"CAMELID_HIP_Q4K_ROWS_PER_WAVE": "16"},
+                  {"CAMELID_HIP_Q4K_ROWS_PER_WAVE": "8"}):
         with G.env(**knobs):
             got_a, got_b = pair(wa, wb)
         assert G.same_bits(got_a, want_a), (name, rows, cols, knobs)
