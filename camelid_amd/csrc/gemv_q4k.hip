@@ -261,6 +261,16 @@ __device__ __forceinline__ void q4k_compute(const Q4KRegs<U> &r, const Q4KLane &
 //
 // DIRECT: the decode launch of an expert layer (one shared f32 token, y-slot = routed assignment, z = which of up to
 // two weights) with its mode known at compile time, for the same reason (one-token MoE layer 44.1 -> 42.6 us).
+//
+// RING = number of slots (0: two alternating 4-super-block register buffers): the K part walked through a ring of small
+// register buffers, one super-block per 4-lane group and step; NSTEPS > 0: the part's length in steps known at compile
+// time, the walk unrolled.  See the walk below for why and the measurements.
+//
+// ROUTE (with DIRECT): the launch routes the token itself from the router's logits (Mixtral routing by every wave,
+// moe_route_wave_values); y-slot = routed rank; the first workgroup leaves experts and weights in routed order.
+//
+// PAIR (with PLAIN): grid.z = 2, blockIdx.z = 1 streams a second weight of the same shape against the same token
+// (gate and up of a dense FFN in one launch).
 template <int NT, bool INTS, bool FUSEQ = false, int SPR = 1, bool WHOLE = false, bool PLAIN = false, bool LOADONLY = false, bool DIRECT = false,
           int RING = 0, int NSTEPS = 0, bool ROUTE = false, bool PAIR = false>
 __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
