@@ -18,7 +18,7 @@ FORMATS = {"Q4_0": CML_Q4_0, "Q8_0": CML_Q8_0, "Q4_K": CML_Q4_K, "Q6_K": CML_Q6_
 EXPORTS = [
     "cml_available", "cml_init", "cml_shutdown", "cml_reload_env", "cml_last_error", "cml_run_count",
     "cml_block_values", "cml_block_bytes",
-    "cml_dev_alloc", "cml_dev_free", "cml_memcpy_h2d", "cml_memcpy_d2h", "cml_memset_dev", "cml_copy_dev", "cml_calibrate_read", "cml_calibrate_weight_loads", "cml_stream_sync",
+    "cml_dev_alloc", "cml_dev_free", "cml_memcpy_h2d", "cml_memcpy_d2h", "cml_memset_dev", "cml_copy_dev", "cml_calibrate_read", "cml_calibrate_weight_loads", "cml_calibrate_matvec_ablation", "cml_stream_sync",
     "cml_stream_create", "cml_stream_destroy", "cml_event_create", "cml_event_record", "cml_event_elapsed_ms",
     "cml_event_destroy", "cml_graph_begin_capture", "cml_graph_end_capture", "cml_graph_launch", "cml_graph_destroy",
     "cml_weight_upload", "cml_weight_upload_dev", "cml_weight_slice", "cml_weight_info",
@@ -69,6 +69,7 @@ def lib() -> C.CDLL:
     L.cml_copy_dev.argtypes = [vp, vp, sz, vp]
     L.cml_calibrate_read.argtypes = [vp, sz, i32, i32, vp]
     L.cml_calibrate_weight_loads.argtypes = [vp, vp, vp]
+    L.cml_calibrate_matvec_ablation.argtypes = [vp, vp, vp, i32, vp]
     L.cml_stream_sync.argtypes = [vp]
     L.cml_stream_create.argtypes = [pp]
     L.cml_stream_destroy.argtypes = [vp]

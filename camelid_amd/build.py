@@ -49,9 +49,17 @@ FLAGS = [
 ]
 
 
+# Per-file flags.  gemv_q4k.hip: kernels whose arguments are plain scalars get them preloaded into
+# SGPRs by the command processor (no scalar-load round trip before a wave's first address); kernels
+# that take a struct by value are unaffected.
+FILE_FLAGS = {
+    "gemv_q4k.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
+}
+
+
 def _compile(src: str, extra: list[str]) -> str:
     obj = os.path.join(OBJ, os.path.splitext(src)[0] + ".o")
-    cmd = [HIPCC, *FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = [HIPCC, *FLAGS, *FILE_FLAGS.get(src, []), *extra, "-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{r.stdout}\n{r.stderr}")

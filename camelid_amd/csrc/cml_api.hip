@@ -320,6 +320,13 @@ int cml_calibrate_weight_loads(const cml_weight *w, void *scratch_dev, cml_strea
     return launch_gemv_q4k_loads_only(w, static_cast<float *>(scratch_dev), as_stream(stream));
 }
 
+int cml_calibrate_matvec_ablation(const cml_weight *w, const float *x_dev, float *out_dev, int mask, cml_stream_t stream) {
+    if (!w || !x_dev || !out_dev) return fail(CML_ERR_INVALID, "null pointer");
+    if (int rc = check_ready()) return rc;
+    if (w->fmt != CML_Q4_K) return fail(CML_ERR_UNSUPPORTED, "the ablated launches exist for the Q4_K matvec");
+    return launch_gemv_q4k_ablated(w, x_dev, out_dev, mask, as_stream(stream));
+}
+
 int cml_stream_sync(cml_stream_t stream) {
     if (int rc = check_ready()) return rc;
     CML_HIP_TRY(hipStreamSynchronize(as_stream(stream)));

@@ -354,6 +354,74 @@ __device__ __forceinline__ uint4 q8k_quantize_row16(const float4 (&v)[4], int la
     return packed;
 }
 
+// The same quantizer with a 32-lane half wave per super-block (one wave does two super-blocks in
+// one pass): lane l of a half holds values 8l..8l+7 (v[0], v[1]).  Returns the 8 quants packed in
+// value order; `d` is the same in every lane of the half; lanes with (l & 3) == 3 get in `bsum`
+// the sum of the 32 quants of group l / 4.  Same arithmetic, value for value, as
+// q8k_quantize_wave.  The signed value of the first strictly greatest |v| is found without a
+// per-element search in the common case: with hi / lo the lane's signed extremes, the holders of
+// the maximum magnitude are the lanes with hi == amax (a positive holder) or -lo == amax (a
+// negative one); unless a half has both kinds the sign is the one kind present.  A half that has
+// both takes the element-by-element search (wave-uniform branch).  Must be called by all 64 lanes.
+__device__ __forceinline__ uint2 q8k_quantize_row32(const float4 (&v)[2], int lane, float &d, int &bsum) {
+    const float vals[8] = {v[0].x, v[0].y, v[0].z, v[0].w, v[1].x, v[1].y, v[1].z, v[1].w};
+    float hi = vals[0], lo = vals[0];  // fmaxf / fminf drop NaNs
+#pragma unroll
+    for (int j = 1; j < 8; j++) {
+        hi = fmaxf(hi, vals[j]);
+        lo = fminf(lo, vals[j]);
+    }
+    const float lmax = fmaxf(fmaxf(hi, -lo), 0.0f);  // the trailing 0 turns an all-NaN lane into 0
+    // non-negative floats order like their bit patterns: integer maxima fold into the DPP moves
+    int m = __builtin_bit_cast(int, lmax);
+    m = max(m, row_ror_i32<1>(m));
+    m = max(m, row_ror_i32<2>(m));
+    m = max(m, row_ror_i32<4>(m));
+    m = max(m, row_ror_i32<8>(m));
+    {
+        typedef unsigned int v2u_dev __attribute__((ext_vector_type(2)));
+        const v2u_dev r = __builtin_amdgcn_permlane16_swap(static_cast<unsigned>(m), static_cast<unsigned>(m), false, false);
+        m = max(static_cast<int>(r.x), static_cast<int>(r.y));  // both 16-lane rows of the half
+    }
+    const float amax = __builtin_bit_cast(float, m);
+    const bool empty = m == 0;
+    const unsigned long long bp = __builtin_amdgcn_ballot_w64(hi == amax), bn = __builtin_amdgcn_ballot_w64(-lo == amax);
+    const uint32_t bp0 = static_cast<uint32_t>(bp), bp1 = static_cast<uint32_t>(bp >> 32);
+    const uint32_t bn0 = static_cast<uint32_t>(bn), bn1 = static_cast<uint32_t>(bn >> 32);
+    const bool upper = (lane & 32) != 0;
+    float vmax = ((upper ? bn1 : bn0) != 0u) ? -amax : amax;
+    if ((bp0 != 0u && bn0 != 0u) || (bp1 != 0u && bn1 != 0u)) {
+        // equal magnitudes of both signs in one super-block: the first holder decides (lowest lane of
+        // the half, lowest value in the lane)
+        const uint32_t holders = upper ? (bp1 | bn1) : (bp0 | bn0);
+        const bool first = holders != 0u && (lane & 31) == __builtin_ctz(holders);
+        float mine = vals[7];
+#pragma unroll
+        for (int j = 6; j >= 0; j--) mine = (fabsf(vals[j]) == amax) ? vals[j] : mine;
+        int sv = row_allor(first ? __builtin_bit_cast(int, mine) : 0);
+        typedef unsigned int v2u_dev __attribute__((ext_vector_type(2)));
+        const v2u_dev r = __builtin_amdgcn_permlane16_swap(static_cast<unsigned>(sv), static_cast<unsigned>(sv), false, false);
+        sv = static_cast<int>(r.x | r.y);
+        vmax = __builtin_bit_cast(float, sv);
+    }
+    const float iscale = -127.0f / vmax;
+    uint32_t pk[2];
+#pragma unroll
+    for (int k = 0; k < 2; k++) {
+        const int q0 = min(nearest_int_magic(iscale * vals[4 * k + 0]), 127);
+        const int q1 = min(nearest_int_magic(iscale * vals[4 * k + 1]), 127);
+        const int q2 = min(nearest_int_magic(iscale * vals[4 * k + 2]), 127);
+        const int q3 = min(nearest_int_magic(iscale * vals[4 * k + 3]), 127);
+        pk[k] = empty ? 0u : pack4(q0, q1, q2, q3);
+    }
+    d = empty ? 0.0f : 1.0f / iscale;
+    int s = sdot4(pk[1], 0x01010101u, sdot4(pk[0], 0x01010101u, 0));
+    s += row_shr_i32<1>(s);
+    s += row_shr_i32<2>(s);
+    bsum = s;
+    return make_uint2(pk[0], pk[1]);
+}
+
 // ---- GGUF Q4_K scale/min words ------------------------------------------------
 
 // The 12 scale bytes of a Q4_K super-block as three little-endian words

@@ -621,6 +621,149 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
     }
 }
 
+// ---- the single-token launch of whole rows: eight-wave workgroups, scalar arguments ------------
+//
+// The plain fused single-token matvec of rows of 2 * NSTEPS super-blocks with no K cut (the decode
+// shape: 14336 x 4096).  Arithmetic and association are exactly those of
+// gemv_q4k_kernel<1, .., SPR = 2, RING = 3> above (same loads, same q4k_compute, same chain); the
+// launch is rebuilt around its two ends, which is where a kernel that lives for six microseconds
+// loses against its own weight stream:
+//   * eight waves per workgroup -- 224 workgroups for 14336 rows, one per compute unit and two
+//     waves per SIMD everywhere, instead of 448 four-wave ones of which most units got two and a
+//     quarter got one; a unit's second workgroup had its f32 activation queued behind the first
+//     one's weight requests in the unit's in-order memory pipe (0.7-1.0 us late);
+//   * an execution barrier between the activation requests and the weight requests, so that in that
+//     pipe every wave's share of the activation is ahead of every weight request of the workgroup;
+//   * the quantizer with a 32-lane half wave per super-block: the eight waves quantize the sixteen
+//     super-blocks of a row in ONE pass, eight values per lane, about half the instructions per wave
+//     of the 16-lane form (q8k_quantize_row32);
+//   * scalar kernel arguments (twelve dwords, preloaded into SGPRs where the firmware does that)
+//     and statically sized LDS: no scalar-load round trip and no size arithmetic before the first
+//     address.
+// Measured on 14336 x 4096, same box, same run: 6.84 -> 6.65 us.  With the activation taken out
+// altogether (no f32 loads, no quantizer, no barriers: ABLATE = 1) the launch takes the same time,
+// so nothing is left in the prologue; without the output store (4) 6.30; without arithmetic and
+// store (the weight requests alone, 7) 6.0-6.06.  What remains above the bare request stream is the
+// drain -- the last step's arithmetic after the last bytes arrive, and the store's way to L2.
+//
+// ABLATE (timing experiments, reachable only through cml_calibrate_matvec_ablation; results are
+// wrong): 1 = no activation, 2 = no arithmetic, 4 = no store.
+template <int NSTEPS, int ABLATE = 0>
+__global__ __launch_bounds__(512) void gemv_q4k_cu_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ out,
+                                                          const float *__restrict__ residual, uint32_t sb_stride, int rows, int row_skip,
+                                                          int tiles16) {
+    constexpr int WAVES = 8;
+    constexpr int NSB = 2 * NSTEPS;  // super-blocks per row
+    constexpr int NB = 3, PRE = 2;   // ring slots; slots requested before the quantizer
+    static_assert(NSTEPS >= NB && NSB <= 2 * WAVES, "one quantizer pass covers the row");
+    constexpr bool NOACT = (ABLATE & 1) != 0, NOMATH = (ABLATE & 2) != 0, NOSTORE = (ABLATE & 4) != 0;
+    using Regs = Q4KRegs<1>;
+    __shared__ __attribute__((aligned(16))) int8_t ys[NSB * 256];
+    __shared__ int bsum[NSB * 8];
+    __shared__ float yds[NSB];
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+
+    // the f32 activation: wave w quantizes super-blocks 2w and 2w + 1, a half wave each
+    const int half = lane >> 5, ql = lane & 31;
+    const int sbk = 2 * wave + half;
+    float4 xv[2];
+    if constexpr (!NOACT) {
+        const float4 *x4 = reinterpret_cast<const float4 *>(x) + min(sbk, NSB - 1) * 64 + ql * 2;
+        xv[0] = x4[0];
+        xv[1] = x4[1];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (!NOACT) __builtin_amdgcn_s_barrier();  // execution only: every activation request of the workgroup is out
+    __builtin_amdgcn_sched_barrier(0);
+
+    const int tile = blockIdx.x * WAVES + wave;  // 8-row half tile
+    const int g = lane / LPS, l = lane - g * LPS;
+    const int r = g >> 1, h = g & 1;
+    const int row = tile * 8 + r - row_skip;  // negative for the skipped head of a view's first tile
+    const bool live = row >= 0 && row < rows;
+    const int rl = (tile & 1) * 8 + r;        // row in the 16-row layout tile
+    // half tiles past the end (grid rounding) re-read the last tile and store nothing
+    const uint8_t *wtile = w + static_cast<int64_t>(min(tile >> 1, tiles16 - 1)) * kQ4KChunk;
+    const uint32_t hoff = static_cast<uint32_t>(h) * sb_stride;
+    const uint32_t hdr_off = hoff + rl * 16, q_off = hoff + (rl * LPS + l) * 16;
+    Regs ring[NB];
+    auto request = [&](Regs &b, int step) __attribute__((always_inline)) {
+        q4k_load_whole<1, 2>(b, wtile + static_cast<int64_t>(2 * step) * sb_stride, sb_stride, hdr_off, q_off);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+#pragma unroll
+    for (int k = 0; k < PRE; k++) request(ring[k], k);
+
+    if constexpr (!NOACT) {
+        // Every wave runs the quantizer (a wave without a super-block of its own redoes the last one and
+        // stores nothing): the f32 loads above are then used unconditionally, and the compiler cannot
+        // sink them into a conditional block behind the weight requests.
+        const bool mine = NSB == 2 * WAVES || sbk < NSB;
+        float dv;
+        int bs;
+        const uint2 packed = q8k_quantize_row32(xv, lane, dv, bs);
+        if (mine) {
+            reinterpret_cast<uint2 *>(ys)[sbk * 32 + ql] = packed;
+            if ((ql & 3) == 3) bsum[sbk * 8 + (ql >> 2)] = bs;
+            if (ql == 0) yds[sbk] = dv;
+        }
+        __syncthreads();
+    }
+
+    Q4KLane ln;
+    ln.c = l;
+    ln.sh = (l & 1) * 16;
+    ln.upper = l >= 2;
+    float acc[1] = {0.0f};
+    auto compute = [&](const Regs &b, int step) __attribute__((always_inline)) {
+        q4k_compute<1, false, 1, 2, true, NOMATH>(b, ln, 2 * step + h, NSB, ys, bsum, yds, NSB, acc, nullptr);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+#pragma unroll
+    for (int j = PRE; j < NB; j++) request(ring[j], j);
+#pragma unroll
+    for (int i = 0; i < NSTEPS; i++) {
+        compute(ring[i % NB], i);
+        if (i + NB < NSTEPS) request(ring[i % NB], i + NB);
+    }
+    if constexpr (NOSTORE) {
+        // keeps the arithmetic alive; the condition does not hold for weights written by this library's upload
+        if (__builtin_bit_cast(uint32_t, acc[0]) == 0x12345679u) out[0] = 1.0f;
+        return;
+    }
+    if (l == LPS - 1 && h == 1 && live) {  // the second group's last lane ran the row's chain
+        float v = acc[0];
+        if (residual) v = v + residual[row];
+        out[row] = v;
+    }
+}
+
+// Whether the launch above serves this call: rows of 4096 values, no K cut (the shape policy gives
+// that from 12288 rows on, i.e. at least 192 eight-wave workgroups), a stride the 32-bit lane
+// offsets can hold.  CAMELID_HIP_Q4K_CU=0 keeps the four-wave launch.
+static bool q4k_cu_serves(const Q4KArgs &ka, int ksplit) {
+    return ksplit == 1 && ka.n_sb == 16 && ka.sb_stride < (int64_t(1) << 31) && env_int("CAMELID_HIP_Q4K_CU", 1) != 0 &&
+           !env_int("CAMELID_HIP_Q4K_CLAMPED_LOADS", 0) && env_int("CAMELID_HIP_Q4K_RING", 1) != 0;
+}
+
+static int launch_q4k_cu(const Q4KArgs &ka, int ablate, hipStream_t st) {
+    if (!(ablate & 1) && !ka.x) return fail(CML_ERR_INVALID, "null activation");  // every variant but the one without the activation reads it
+    const int tiles16 = (ka.rows + ka.row_skip + 15) / 16;
+    const dim3 grid(static_cast<unsigned>((2 * tiles16 + 7) / 8)), block(512);
+    const uint32_t stride = static_cast<uint32_t>(ka.sb_stride);
+#define CML_Q4K_CU(A_) hipLaunchKernelGGL((gemv_q4k_cu_kernel<8, A_>), grid, block, 0, st, ka.w, ka.x, ka.out, ka.residual, stride, ka.rows, ka.row_skip, tiles16)
+    switch (ablate) {
+        case 0: CML_Q4K_CU(0); break;
+        case 1: CML_Q4K_CU(1); break;
+        case 4: CML_Q4K_CU(4); break;
+        case 7: CML_Q4K_CU(7); break;
+        default: return fail(CML_ERR_INVALID, "ablation mask must be 1, 4 or 7");
+    }
+#undef CML_Q4K_CU
+    return CML_OK;
+}
+
 // Launch shape.  `ksplit` depends on the weight shape only, so gemv and gemm
 // give every cell the same association; 1 (the reference's own) whenever the
 // row count alone yields about one wave per SIMD (1024 on this chip).
@@ -788,7 +931,10 @@ static int launch_q4k_pick_nt(const Q4KArgs &ka, const Q4KShape &shape, int n_gr
 // Grouped call (group_offsets set): every group dots its assignments' activation rows
 // (group_rows) one at a time.  `w2`/`out2` non-null: a second weight of the same shape in the
 // same launch (grid.z = 2).
-static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, const float *x, hipStream_t st, bool loads_only = false) {
+// ablate: 0 = the real launch; 7 = its weight requests alone (x may be null); 1 / 4 = without the activation / without the
+// store (the eight-wave launch only) -- the calibration entries' timing experiments.
+static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, const float *x, hipStream_t st, int ablate = 0) {
+    const bool loads_only = ablate != 0;
     const cml_weight *w = a.w;
     const bool grouped = a.group_offsets != nullptr || a.group_ids != nullptr;
     if (w->rows == 0) return CML_OK;
@@ -845,7 +991,11 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
         const bool plain = !grouped && !w2 && !env_int("CAMELID_HIP_Q4K_GENERAL_ENTRY", 0);
         const dim3 block(64 * waves);
 #define CML_Q4K_LAUNCH(SPR_, WHOLE_, PLAIN_) hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, SPR_, WHOLE_, PLAIN_>), grid, block, lds, st, ka)
-        if (loads_only) {
+        if (loads_only && half_tiles && ring && plain && q4k_cu_serves(ka, shape.ksplit)) {
+            if (int rc = launch_q4k_cu(ka, ablate, st)) return rc;
+        } else if (loads_only && ablate != 7) {
+            return fail(CML_ERR_UNSUPPORTED, "this ablation exists for the eight-wave single-token launch (rows of 4096 values, no K cut)");
+        } else if (loads_only) {
             // calibration: the plain single-token launch with its loads and nothing else
 #define CML_Q4K_LOADS(SPR_, WHOLE_) hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, SPR_, WHOLE_, true, true>), grid, block, lds, st, ka)
             if (half_tiles && ring) launch_q4k_ring<1, true, 2, true>(ka, shape.ksplit, grid, block, lds, st);
@@ -873,6 +1023,8 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
             launch_q4k_ring<1, true, 2, false, true>(ka, shape.ksplit, grid, block, lds, st);  // a plain pair: grid.z = 2
         } else if (!grouped && w2 && !half_tiles && q4k_ring(ka, shape.ksplit, 1) && !env_int("CAMELID_HIP_Q4K_GENERAL_ENTRY", 0)) {
             launch_q4k_ring<1, true, 1, false, true>(ka, shape.ksplit, grid, block, lds, st);
+        } else if (half_tiles && ring && plain && q4k_cu_serves(ka, shape.ksplit)) {
+            if (int rc = launch_q4k_cu(ka, 0, st)) return rc;  // rows of 4096 values, no K cut: eight-wave workgroups
         } else if (half_tiles && ring && plain) {
             launch_q4k_ring<1, true, 2>(ka, shape.ksplit, grid, block, lds, st);
         } else if (!half_tiles && plain && q4k_ring(ka, shape.ksplit, 1)) {
@@ -913,7 +1065,20 @@ int launch_gemv_q4k_loads_only(const cml_weight *w, float *out, hipStream_t st) 
     a.out = out;
     a.n_tokens = 1;
     a.n_groups = 1;
-    return launch_q4k_f32(a, nullptr, nullptr, nullptr, st, true);
+    return launch_q4k_f32(a, nullptr, nullptr, nullptr, st, 7);
+}
+
+// Calibration: the eight-wave single-token launch with parts taken out (mask 1 = no activation, 4 = no store,
+// 7 = the weight requests alone).  `out` must hold the weight's rows; its contents are meaningless afterwards.
+int launch_gemv_q4k_ablated(const cml_weight *w, const float *x, float *out, int mask, hipStream_t st) {
+    if (w->rows == 0) return CML_OK;
+    if (mask != 1 && mask != 4 && mask != 7) return fail(CML_ERR_INVALID, "ablation mask must be 1, 4 or 7");
+    MatArgs a{};
+    a.w = w;
+    a.out = out;
+    a.n_tokens = 1;
+    a.n_groups = 1;
+    return launch_q4k_f32(a, nullptr, nullptr, x, st, mask);
 }
 
 // One f32 token against two weights of one shape (the gate and up projections of a dense FFN) in one launch.

@@ -121,6 +121,12 @@ int cml_copy_dev(void *dst_dev, const void *src_dev, size_t nbytes, cml_stream_t
  * what the real kernel takes beyond that is the kernel's own cost. */
 int cml_calibrate_read(const void *src_dev, size_t nbytes, int in_flight, int workgroups, cml_stream_t stream);
 int cml_calibrate_weight_loads(const cml_weight *w, void *scratch_dev, cml_stream_t stream);
+/* cml_calibrate_matvec_ablation: the single-token Q4_K launch of cml_matmul_f32 for `w` with parts
+ * taken out, to time what each part costs: mask 1 = no activation (no f32 loads, no quantizer, no
+ * barrier), 4 = no output store, 7 = the weight requests alone.  Served
+ * for the shapes the eight-wave launch serves (rows of 4096 values, 12288 to 16384 rows);
+ * CML_ERR_UNSUPPORTED otherwise.  out_dev must hold w's rows and is garbage afterwards. */
+int cml_calibrate_matvec_ablation(const cml_weight *w, const float *x_dev, float *out_dev, int mask, cml_stream_t stream);
 int cml_stream_sync(cml_stream_t stream);
 /* Streams (default priority), timing events and captured launch sequences, for
  * hosts that drive a decode loop through this library alone.  The reference's
