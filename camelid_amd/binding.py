@@ -16,7 +16,7 @@ CML_Q4_0, CML_Q8_0, CML_Q4_K, CML_Q6_K = 2, 8, 12, 14
 FORMATS = {"Q4_0": CML_Q4_0, "Q8_0": CML_Q8_0, "Q4_K": CML_Q4_K, "Q6_K": CML_Q6_K}
 
 EXPORTS = [
-    "cml_available", "cml_init", "cml_shutdown", "cml_reload_env", "cml_last_error", "cml_run_count",
+    "cml_available", "cml_init", "cml_shutdown", "cml_reload_env", "cml_last_error", "cml_run_count", "cml_kernel_launches", "cml_kernel_launch_report",
     "cml_block_values", "cml_block_bytes",
     "cml_dev_alloc", "cml_dev_free", "cml_memcpy_h2d", "cml_memcpy_d2h", "cml_memset_dev", "cml_copy_dev", "cml_calibrate_read", "cml_calibrate_weight_loads", "cml_calibrate_matvec_ablation", "cml_stream_sync",
     "cml_stream_create", "cml_stream_destroy", "cml_event_create", "cml_event_record", "cml_event_elapsed_ms",
@@ -58,6 +58,10 @@ def lib() -> C.CDLL:
     L.cml_available.restype = i32
     L.cml_init.argtypes = [i32]
     L.cml_last_error.restype = C.c_char_p
+    L.cml_kernel_launches.argtypes = [C.c_char_p]
+    L.cml_kernel_launches.restype = C.c_uint64
+    L.cml_kernel_launch_report.argtypes = [C.c_char_p, sz]
+    L.cml_kernel_launch_report.restype = sz
     L.cml_run_count.restype = C.c_uint64
     L.cml_block_values.argtypes = [i32]
     L.cml_block_bytes.argtypes = [i32]

@@ -49,6 +49,17 @@ void clear_error() { g_error[0] = '\0'; }
 
 bool ready() { return g_device.load(std::memory_order_acquire) >= 0; }
 
+static std::atomic<LaunchCounter *> g_counters{nullptr};
+
+LaunchCounter::LaunchCounter(const std::string &nm) : LaunchCounter(strdup(nm.c_str())) {}
+
+LaunchCounter::LaunchCounter(const char *nm) : name(nm ? nm : "?") {
+    LaunchCounter *head = g_counters.load(std::memory_order_acquire);
+    do {
+        next = head;
+    } while (!g_counters.compare_exchange_weak(head, this, std::memory_order_release, std::memory_order_acquire));
+}
+
 // Tuning knobs (CAMELID_HIP_*) are read from the environment ONCE, into a snapshot taken by
 // cml_init and again by cml_reload_env (reference: every CAMELID_* knob sits in a OnceLock,
 // src/inference.rs:23679-23692).  A launch only walks the snapshot -- normally empty -- and never
@@ -230,6 +241,31 @@ int cml_reload_env(void) {
 
 const char *cml_last_error(void) { return g_error; }
 uint64_t cml_run_count(void) { return g_runs.load(std::memory_order_relaxed); }
+
+uint64_t cml_kernel_launches(const char *prefix) {
+    const size_t len = prefix ? strlen(prefix) : 0;
+    uint64_t total = 0;
+    for (const LaunchCounter *c = g_counters.load(std::memory_order_acquire); c; c = c->next)
+        if (len == 0 || strncmp(c->name, prefix, len) == 0) total += c->n.load(std::memory_order_relaxed);
+    return total;
+}
+
+size_t cml_kernel_launch_report(char *buf, size_t cap) {
+    // "name count\n" per counter; returns the size the whole report needs (with its terminator)
+    size_t need = 1, at = 0;
+    for (const LaunchCounter *c = g_counters.load(std::memory_order_acquire); c; c = c->next) {
+        char line[160];
+        const int n = snprintf(line, sizeof(line), "%s %llu\n", c->name, static_cast<unsigned long long>(c->n.load(std::memory_order_relaxed)));
+        if (n <= 0) continue;
+        need += static_cast<size_t>(n);
+        if (buf && at + static_cast<size_t>(n) < cap) {
+            memcpy(buf + at, line, static_cast<size_t>(n));
+            at += static_cast<size_t>(n);
+        }
+    }
+    if (buf && cap) buf[at] = '\0';
+    return need;
+}
 
 // ---- device memory plumbing ------------------------------------------------------------------------
 

@@ -6,6 +6,7 @@
 #include <stdint.h>
 #include <stdio.h>
 
+#include <atomic>
 #include <string>
 
 #include "../../include/camelid_hip.h"
@@ -27,6 +28,24 @@ bool ready();  // cml_init succeeded and the device is current
     } while (0)
 
 inline hipStream_t as_stream(cml_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+// Which kernel family served a call (reference: the engaged counters its tests read to prove that a
+// dispatch fired, src/inference.rs:23740, 24596-24603; src/cuda.rs:346-358).  Every launcher counts
+// under a dotted name, "<format>.<family>[.<variant>...]"; cml_kernel_launches(prefix) sums the
+// counters whose names start with the prefix.  One relaxed atomic add per launch.
+struct LaunchCounter {
+    const char *name;
+    std::atomic<uint64_t> n{0};
+    LaunchCounter *next = nullptr;
+    explicit LaunchCounter(const char *nm);         // links itself into the registry; nm must outlive the process (a literal)
+    explicit LaunchCounter(const std::string &nm);  // the same for a name built at the first launch (kept for good)
+};
+// name_ may be any expression (evaluated once, at the site's first launch)
+#define CML_COUNT_LAUNCH(name_)                               \
+    do {                                                      \
+        static ::cml::LaunchCounter cml_counter_(name_);      \
+        cml_counter_.n.fetch_add(1, std::memory_order_relaxed); \
+    } while (0)
 
 struct Geometry {
     int block_values;

@@ -37,6 +37,9 @@
 // RING slabs per wave.
 #include <type_traits>
 
+#include <atomic>
+#include <string>
+
 #include "cml_device.hpp"
 #include "cml_host.hpp"
 
@@ -521,14 +524,16 @@ static int launch_b32_mfma_kpar(const B32MfmaArgs &ka, hipStream_t st) {
     const int nb = ka.n_slabs * 8;
     const size_t lds = static_cast<size_t>(ka.n_slabs) * 16 * kB32SlabRow + (FMT == CML_Q4_0 ? static_cast<size_t>(nb) * 16 * 4 : 0) +
                        static_cast<size_t>(nb) * 16 * 4 + TPW * 64 * 16;
-    static bool raised = false;
-    if (!raised) {
+    static std::atomic<bool> raised{false};  // setting the attribute twice from two threads is harmless
+    if (!raised.load(std::memory_order_acquire)) {
         CML_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_b32_mfma_kpar_kernel<FMT, KD, SPW, TPW>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-        raised = true;
+        raised.store(true, std::memory_order_release);
     }
     hipLaunchKernelGGL((gemm_b32_mfma_kpar_kernel<FMT, KD, SPW, TPW>),
                        dim3(static_cast<unsigned>((n_tiles + TPW - 1) / TPW), static_cast<unsigned>((ka.n_tokens + 15) / 16)), dim3(64 * KD * TPW), lds, st, ka);
+    // "<format>.mfma.kpar.k<waves per row tile>s<slabs per wave>t<tiles per workgroup>"
+    CML_COUNT_LAUNCH(std::string(FMT == CML_Q8_0 ? "q8_0" : "q4_0") + ".mfma.kpar.k" + std::to_string(KD) + "s" + std::to_string(SPW) + "t" + std::to_string(TPW));
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }
@@ -542,13 +547,16 @@ static int launch_b32_mfma_gp(const B32MfmaArgs &ka, int n_groups, hipStream_t s
     const size_t lds = 2 * static_cast<size_t>(KC * NTOK) * kB32SlabRow + (FMT == CML_Q4_0 ? 2 * static_cast<size_t>(KC * NTOK) * 8 * 4 : 0) +
                        static_cast<size_t>(ka.n_slabs) * 8 * NTOK * 4;
     if (lds > 160 * 1024) return fail(CML_ERR_UNSUPPORTED, "matrix-core path: %d blocks per row exceed the LDS budget", ka.n_slabs * 8);
-    static bool raised = false;  // per instantiation: allow more than 64 KB of dynamic LDS once
-    if (!raised) {
+    static std::atomic<bool> raised{false};  // per instantiation: allow more than 64 KB of dynamic LDS once
+    if (!raised.load(std::memory_order_acquire)) {
         CML_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_b32_mfma_kernel<FMT, GPW, TB, KC, RING, PLAIN, WAVES>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-        raised = true;
+        raised.store(true, std::memory_order_release);
     }
     hipLaunchKernelGGL((gemm_b32_mfma_kernel<FMT, GPW, TB, KC, RING, PLAIN, WAVES>), dim3(gx, gy, n_groups), dim3(64 * WAVES), lds, st, ka);
+    // "<format>.mfma.tile.g<token groups per wave>t<waves over tokens>.w<waves>.r<ring depth>[.grouped]"
+    CML_COUNT_LAUNCH(std::string(FMT == CML_Q8_0 ? "q8_0" : "q4_0") + ".mfma.tile.g" + std::to_string(GPW) + "t" + std::to_string(TB) + ".w" +
+                     std::to_string(WAVES) + ".r" + std::to_string(RING) + (PLAIN ? "" : ".grouped"));
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }

@@ -46,6 +46,9 @@
 // chain restarts at the split points).
 #include <type_traits>
 
+#include <atomic>
+#include <string>
+
 #include "cml_device.hpp"
 #include "cml_host.hpp"
 
@@ -754,14 +757,15 @@ static int launch_mfma_pair(const Q4KMfmaArgs &ka, const float *x, hipStream_t s
     pa.n_tokens = ka.n_tokens;
     pa.s_mid = (ka.n_sb + 1) / 2;
     const int n_tiles = (ka.rows + ka.row_skip + 15) / 16;
-    static bool raised = false;
-    if (!raised) {
+    static std::atomic<bool> raised{false};  // setting the attribute twice from two threads is harmless
+    if (!raised.load(std::memory_order_acquire)) {
         CML_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_mfma_pair_kernel<FUSEQ>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-        raised = true;
+        raised.store(true, std::memory_order_release);
     }
     const dim3 grid(static_cast<unsigned>((n_tiles + kPairTiles - 1) / kPairTiles), static_cast<unsigned>((ka.n_tokens + 15) / 16));
     hipLaunchKernelGGL(gemm_q4k_mfma_pair_kernel<FUSEQ>, grid, dim3(512), kPairLds, st, pa);
+    if constexpr (FUSEQ) CML_COUNT_LAUNCH("q4k.mfma.pair.fused"); else CML_COUNT_LAUNCH("q4k.mfma.pair");
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }
@@ -790,6 +794,18 @@ int launch_gemm_q4k_mfma_f32(const cml_weight *w, const float *x, int64_t n_toke
     return launch_mfma_pair<true>(ka, x, st);
 }
 
+// Counter name of a general-kernel instantiation: "q4k.mfma.tile" (one wave per row tile), ".ksplit<KS>" (K parts of a
+// tile on KS waves) or ".serial_split" (the K cut walked inside the lane), then the workgroup shape g<token groups per
+// wave>t<waves over tokens>, ".grouped" for expert-grouped calls and ".once" where the activation is staged once.
+static std::string q4k_mfma_name(int gpw, int tb, bool split, int ks, bool plain, bool once) {
+    std::string n = "q4k.mfma.";
+    n += ks > 1 ? "ksplit" + std::to_string(ks) : (split ? "serial_split" : "tile");
+    n += ".g" + std::to_string(gpw) + "t" + std::to_string(tb);
+    if (!plain) n += ".grouped";
+    if (once) n += ".once";
+    return n;
+}
+
 template <int GPW, int TB, bool SPLIT, int KS = 1, bool PLAIN = false>
 static int launch_mfma_split(const Q4KMfmaArgs &ka, int n_groups, hipStream_t st) {
     constexpr int NTOK = 16 * GPW * TB, RT = 4 / (TB * KS);
@@ -802,24 +818,26 @@ static int launch_mfma_split(const Q4KMfmaArgs &ka, int n_groups, hipStream_t st
     if constexpr (GPW == 1 && TB == 1 && KS == 1) {
         if (ka.n_sb <= 2 * KC && ka.stage_once) {  // the whole activation fits the two buffers: staged once
             const size_t lds_once = lds + 2 * static_cast<size_t>(KC * NTOK) * 32;  // + the run sums
-            static bool raised_once = false;
-            if (!raised_once) {
+            static std::atomic<bool> raised_once{false};
+            if (!raised_once.load(std::memory_order_acquire)) {
                 CML_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_mfma_kernel<GPW, TB, SPLIT, KS, PLAIN, true>),
                                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-                raised_once = true;
+                raised_once.store(true, std::memory_order_release);
             }
             hipLaunchKernelGGL((gemm_q4k_mfma_kernel<GPW, TB, SPLIT, KS, PLAIN, true>), dim3(gx, gy, n_groups), dim3(256), lds_once, st, ka);
+            CML_COUNT_LAUNCH(q4k_mfma_name(GPW, TB, SPLIT, KS, PLAIN, true));
             CML_HIP_TRY(hipGetLastError());
             return CML_OK;
         }
     }
-    static bool raised = false;  // per instantiation: allow more than 64 KB of dynamic LDS once
-    if (!raised) {
+    static std::atomic<bool> raised{false};  // per instantiation: allow more than 64 KB of dynamic LDS once
+    if (!raised.load(std::memory_order_acquire)) {
         CML_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_mfma_kernel<GPW, TB, SPLIT, KS, PLAIN>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-        raised = true;
+        raised.store(true, std::memory_order_release);
     }
     hipLaunchKernelGGL((gemm_q4k_mfma_kernel<GPW, TB, SPLIT, KS, PLAIN>), dim3(gx, gy, n_groups), dim3(256), lds, st, ka);
+    CML_COUNT_LAUNCH(q4k_mfma_name(GPW, TB, SPLIT, KS, PLAIN, false));
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }

@@ -33,6 +33,9 @@
 // the matvec result bit for bit.
 #include <type_traits>
 
+#include <atomic>
+#include <string>
+
 #include "cml_device.hpp"
 #include "cml_host.hpp"
 
@@ -363,13 +366,16 @@ static int launch_q6k_mfma_gp(const Q6KMfmaArgs &ka, int n_groups, hipStream_t s
     const unsigned gy = static_cast<unsigned>((ka.n_tokens + NTOK - 1) / NTOK);
     const size_t lds = 2 * static_cast<size_t>(KS * KC * NTOK) * kQ6SlabRow + static_cast<size_t>(ka.n_sb) * NTOK * 4;
     if (lds > 160 * 1024) return fail(CML_ERR_UNSUPPORTED, "Q6_K matrix-core path: %d super-blocks exceed the LDS budget", ka.n_sb);
-    static bool raised = false;  // per instantiation: allow more than 64 KB of dynamic LDS once
-    if (!raised) {
+    static std::atomic<bool> raised{false};  // per instantiation: allow more than 64 KB of dynamic LDS once
+    if (!raised.load(std::memory_order_acquire)) {
         CML_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q6k_mfma_kernel<GPW, TB, SPLIT, KC, RING, KS, PLAIN>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-        raised = true;
+        raised.store(true, std::memory_order_release);
     }
     hipLaunchKernelGGL((gemm_q6k_mfma_kernel<GPW, TB, SPLIT, KC, RING, KS, PLAIN>), dim3(gx, gy, n_groups), dim3(256), lds, st, ka);
+    // "q6k.mfma.<tile | ksplit<KS> | serial_split>.g<token groups per wave>t<waves over tokens>.r<ring depth>[.grouped]"
+    CML_COUNT_LAUNCH(std::string("q6k.mfma.") + (KS > 1 ? "ksplit" + std::to_string(KS) : std::string(SPLIT ? "serial_split" : "tile")) + ".g" +
+                     std::to_string(GPW) + "t" + std::to_string(TB) + ".r" + std::to_string(RING) + (PLAIN ? "" : ".grouped"));
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }

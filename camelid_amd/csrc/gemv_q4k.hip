@@ -761,6 +761,8 @@ static int launch_q4k_cu(const Q4KArgs &ka, int ablate, hipStream_t st) {
         default: return fail(CML_ERR_INVALID, "ablation mask must be 1, 4 or 7");
     }
 #undef CML_Q4K_CU
+    if (ablate) CML_COUNT_LAUNCH("q4k.calibrate.wg8");
+    else CML_COUNT_LAUNCH("q4k.dot.wg8.fused");
     return CML_OK;
 }
 
@@ -865,6 +867,10 @@ static void launch_q4k_ring(const Q4KArgs &ka, int ksplit, dim3 grid, dim3 block
         else CML_Q4K_RING(0);
     }
 #undef CML_Q4K_RING
+    if constexpr (LOADONLY) CML_COUNT_LAUNCH("q4k.calibrate.ring");
+    else if constexpr (PAIR) CML_COUNT_LAUNCH("q4k.dot.ring.fused.pair");
+    else if constexpr (FUSEQ) CML_COUNT_LAUNCH("q4k.dot.ring.fused");
+    else CML_COUNT_LAUNCH("q4k.dot.ring");
 }
 
 template <int NT>
@@ -882,9 +888,11 @@ static int launch_q4k_nt(Q4KArgs ka, const Q4KShape &shape, int n_groups, bool i
     ka.tiles_per_wg = shape.tiles_per_wg;
     const bool plain = !ka.group_offsets && !ka.group_ids && !env_int("CAMELID_HIP_Q4K_GENERAL_ENTRY", 0);
     const dim3 grid(gx, n_groups), block(64 * waves);
-    if (ints && NT == 1)
+    const bool grouped_call = ka.group_offsets || ka.group_ids;
+    if (ints && NT == 1) {
         hipLaunchKernelGGL((gemv_q4k_kernel<1, true>), grid, block, lds, st, ka);
-    else if (NT <= 2) {
+        CML_COUNT_LAUNCH("q4k.dot.ints");
+    } else if (NT <= 2) {
         // one or two tokens: 8-row waves, unclamped loads and the short entry where they apply
         constexpr int NTS = NT <= 2 ? NT : 1;
         const bool whole = q4k_whole_buffers(ka, shape.ksplit);
@@ -896,13 +904,17 @@ static int launch_q4k_nt(Q4KArgs ka, const Q4KShape &shape, int n_groups, bool i
         } else if (half_tiles) {
             if (whole) { if (plain) CML_Q4K_LAUNCH(2, true, true); else CML_Q4K_LAUNCH(2, true, false); }
             else { if (plain) CML_Q4K_LAUNCH(2, false, true); else CML_Q4K_LAUNCH(2, false, false); }
+            if (grouped_call) CML_COUNT_LAUNCH("q4k.dot.buffers.grouped"); else CML_COUNT_LAUNCH("q4k.dot.buffers");
         } else {
             if (whole) { if (plain) CML_Q4K_LAUNCH(1, true, true); else CML_Q4K_LAUNCH(1, true, false); }
             else { if (plain) CML_Q4K_LAUNCH(1, false, true); else CML_Q4K_LAUNCH(1, false, false); }
+            if (grouped_call) CML_COUNT_LAUNCH("q4k.dot.buffers.grouped"); else CML_COUNT_LAUNCH("q4k.dot.buffers");
         }
 #undef CML_Q4K_LAUNCH
-    } else
+    } else {
         hipLaunchKernelGGL((gemv_q4k_kernel<NT, false>), grid, block, lds, st, ka);
+        if (grouped_call) CML_COUNT_LAUNCH("q4k.dot.buffers.grouped"); else CML_COUNT_LAUNCH("q4k.dot.buffers");
+    }
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }
@@ -1000,24 +1012,29 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
 #define CML_Q4K_LOADS(SPR_, WHOLE_) hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, SPR_, WHOLE_, true, true>), grid, block, lds, st, ka)
             if (half_tiles && ring) launch_q4k_ring<1, true, 2, true>(ka, shape.ksplit, grid, block, lds, st);
             else if (!half_tiles && q4k_ring(ka, shape.ksplit, 1)) launch_q4k_ring<1, true, 1, true>(ka, shape.ksplit, grid, block, lds, st);
-            else if (half_tiles) { if (whole) CML_Q4K_LOADS(2, true); else CML_Q4K_LOADS(2, false); }
-            else { if (whole) CML_Q4K_LOADS(1, true); else CML_Q4K_LOADS(1, false); }
+            else if (half_tiles) { if (whole) CML_Q4K_LOADS(2, true); else CML_Q4K_LOADS(2, false); CML_COUNT_LAUNCH("q4k.calibrate.buffers"); }
+            else { if (whole) CML_Q4K_LOADS(1, true); else CML_Q4K_LOADS(1, false); CML_COUNT_LAUNCH("q4k.calibrate.buffers"); }
 #undef CML_Q4K_LOADS
         } else if (two) {
             // both tokens in one pass over the weight, 16-row waves as in the two-token matvec
             if (q4k_ring(ka, shape.ksplit, 1)) launch_q4k_ring<2, true, 1>(ka, shape.ksplit, grid, block, lds, st);
-            else if (whole) hipLaunchKernelGGL((gemv_q4k_kernel<2, false, true, 1, true, true>), grid, block, lds, st, ka);
-            else hipLaunchKernelGGL((gemv_q4k_kernel<2, false, true, 1, false, true>), grid, block, lds, st, ka);
+            else {
+                if (whole) hipLaunchKernelGGL((gemv_q4k_kernel<2, false, true, 1, true, true>), grid, block, lds, st, ka);
+                else hipLaunchKernelGGL((gemv_q4k_kernel<2, false, true, 1, false, true>), grid, block, lds, st, ka);
+                CML_COUNT_LAUNCH("q4k.dot.buffers.fused");
+            }
         } else if (!plain && ka.shared_act && ka.group_ids && !env_int("CAMELID_HIP_Q4K_GENERAL_ENTRY", 0)) {
             // the decode launch of an expert layer: its own entry
 #define CML_Q4K_DIRECT(SPR_, WHOLE_) hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, SPR_, WHOLE_, false, false, true>), grid, block, lds, st, ka)
             if (ka.route_logits) {
                 if (!(half_tiles && ring && ka.n_sb == 16 * shape.ksplit)) return fail(CML_ERR_UNSUPPORTED, "the routing launch serves rows of 4096 values under 8-row waves");
                 hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, 2, true, false, false, true, 3, 8, true>), grid, block, lds, st, ka);
-            } else if (half_tiles && ring && ka.n_sb == 16 * shape.ksplit && env_int("CAMELID_HIP_Q4K_DIRECT_RING", 1))
+                CML_COUNT_LAUNCH("q4k.dot.direct.ring.route");
+            } else if (half_tiles && ring && ka.n_sb == 16 * shape.ksplit && env_int("CAMELID_HIP_Q4K_DIRECT_RING", 1)) {
                 hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, 2, true, false, false, true, 3, 8>), grid, block, lds, st, ka);
-            else if (half_tiles) { if (whole) CML_Q4K_DIRECT(2, true); else CML_Q4K_DIRECT(2, false); }
-            else { if (whole) CML_Q4K_DIRECT(1, true); else CML_Q4K_DIRECT(1, false); }
+                CML_COUNT_LAUNCH("q4k.dot.direct.ring");
+            } else if (half_tiles) { if (whole) CML_Q4K_DIRECT(2, true); else CML_Q4K_DIRECT(2, false); CML_COUNT_LAUNCH("q4k.dot.direct.buffers"); }
+            else { if (whole) CML_Q4K_DIRECT(1, true); else CML_Q4K_DIRECT(1, false); CML_COUNT_LAUNCH("q4k.dot.direct.buffers"); }
 #undef CML_Q4K_DIRECT
         } else if (!grouped && w2 && half_tiles && ring && !env_int("CAMELID_HIP_Q4K_GENERAL_ENTRY", 0)) {
             launch_q4k_ring<1, true, 2, false, true>(ka, shape.ksplit, grid, block, lds, st);  // a plain pair: grid.z = 2
@@ -1032,9 +1049,11 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
         } else if (half_tiles) {
             if (whole) { if (plain) CML_Q4K_LAUNCH(2, true, true); else CML_Q4K_LAUNCH(2, true, false); }
             else { if (plain) CML_Q4K_LAUNCH(2, false, true); else CML_Q4K_LAUNCH(2, false, false); }
+            if (plain) CML_COUNT_LAUNCH("q4k.dot.buffers.fused"); else if (w2) CML_COUNT_LAUNCH("q4k.dot.buffers.fused.pair"); else CML_COUNT_LAUNCH("q4k.dot.buffers.fused.grouped");
         } else {
             if (whole) { if (plain) CML_Q4K_LAUNCH(1, true, true); else CML_Q4K_LAUNCH(1, true, false); }
             else { if (plain) CML_Q4K_LAUNCH(1, false, true); else CML_Q4K_LAUNCH(1, false, false); }
+            if (plain) CML_COUNT_LAUNCH("q4k.dot.buffers.fused"); else if (w2) CML_COUNT_LAUNCH("q4k.dot.buffers.fused.pair"); else CML_COUNT_LAUNCH("q4k.dot.buffers.fused.grouped");
         }
 #undef CML_Q4K_LAUNCH
     }
@@ -1313,6 +1332,7 @@ int launch_moe_down_sum_q4k(const cml_weight *down, int n_experts, int n_slots, 
         hipLaunchKernelGGL((moe_down_sum_q4k_kernel<true, 7>), dim3(static_cast<unsigned>(rows / 16)), dim3(64 * waves), lds, st, a);
     else if (ring) hipLaunchKernelGGL(moe_down_sum_q4k_kernel<true>, dim3(static_cast<unsigned>(rows / 16)), dim3(64 * waves), lds, st, a);
     else hipLaunchKernelGGL(moe_down_sum_q4k_kernel<false>, dim3(static_cast<unsigned>(rows / 16)), dim3(64 * waves), lds, st, a);
+    if (ring) CML_COUNT_LAUNCH("q4k.down_sum.ring"); else CML_COUNT_LAUNCH("q4k.down_sum.buffers");
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }
@@ -1433,6 +1453,7 @@ static int launch_gemv_q4k_lanes(const MatArgs &a, hipStream_t st) {
     if (a.n_tokens > 65535) return fail(CML_ERR_UNSUPPORTED, "at most 65535 tokens per call in the lane-order mode");
     hipLaunchKernelGGL(gemv_q4k_lanes_kernel, dim3(static_cast<unsigned>((w->rows + 3) / 4), static_cast<unsigned>(a.n_tokens)), dim3(256), lds, st,
                        w->planes.p[0], w->planes.row_stride[0], static_cast<int>(w->rows), w->row_skip, n_sb, a.q, a.scales, a.out, a.residual);
+    CML_COUNT_LAUNCH("q4k.lanes");
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }

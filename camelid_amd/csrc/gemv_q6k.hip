@@ -367,14 +367,19 @@ static int launch_q6k_nt(const Q6KArgs &ka, int n_bands, bool ints, bool grouped
     const unsigned gx = static_cast<unsigned>((tiles + tiles_per_wg - 1) / tiles_per_wg);
     const size_t lds = q6k_lds_bytes(NT, ka.n_sb);
     if (lds > 64 * 1024) return fail(CML_ERR_UNSUPPORTED, "Q6_K activation of %d super-blocks x %d tokens exceeds the LDS staging limit", ka.n_sb, NT);
-    if (grouped)
+    if (grouped) {
         hipLaunchKernelGGL((gemv_q6k_kernel<NT, false, true>), dim3(gx, n_bands), dim3(256), lds, st, ka);
-    else if (ints && NT == 1)
+        CML_COUNT_LAUNCH("q6k.dot.grouped");
+    } else if (ints && NT == 1) {
         hipLaunchKernelGGL((gemv_q6k_kernel<1, true>), dim3(gx, n_bands), dim3(256), lds, st, ka);
-    else if (NT == 1 && tiles >= env_int("CAMELID_HIP_Q6K_DEEP_MIN_TILES", 2048))
+        CML_COUNT_LAUNCH("q6k.dot.ints");
+    } else if (NT == 1 && tiles >= env_int("CAMELID_HIP_Q6K_DEEP_MIN_TILES", 2048)) {
         hipLaunchKernelGGL((gemv_q6k_kernel<1, false, false, 4>), dim3(gx, n_bands), dim3(256), lds, st, ka);
-    else
+        CML_COUNT_LAUNCH("q6k.dot.deep");
+    } else {
         hipLaunchKernelGGL((gemv_q6k_kernel<NT, false>), dim3(gx, n_bands), dim3(256), lds, st, ka);
+        CML_COUNT_LAUNCH("q6k.dot.buffers");
+    }
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }
@@ -471,6 +476,7 @@ static int launch_gemv_q6k_lanes(const MatArgs &a, hipStream_t st) {
     if (a.n_tokens > 65535) return fail(CML_ERR_UNSUPPORTED, "at most 65535 tokens per call in the lane-order mode");
     hipLaunchKernelGGL(gemv_q6k_lanes_kernel, dim3(static_cast<unsigned>((ka.rows + 3) / 4), static_cast<unsigned>(a.n_tokens)), dim3(256), lds, st,
                        ka, static_cast<int64_t>(w->cols));
+    CML_COUNT_LAUNCH("q6k.lanes");
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }
@@ -560,12 +566,16 @@ int launch_gemv_q6k_f32(const cml_weight *w, const float *x, float *out, hipStre
     const unsigned gx = static_cast<unsigned>((tiles + tiles_per_wg - 1) / tiles_per_wg);
     const size_t lds = q6k_lds_bytes(n_tokens, ka.n_sb);
     if (lds > 64 * 1024) return fail(CML_ERR_UNSUPPORTED, "Q6_K activation of %d super-blocks exceeds the LDS staging limit", ka.n_sb);
-    if (n_tokens == 2)
+    if (n_tokens == 2) {
         hipLaunchKernelGGL((gemv_q6k_kernel<2, false, false, 2, true>), dim3(gx, 1), dim3(256), lds, st, ka);
-    else if (tiles >= env_int("CAMELID_HIP_Q6K_DEEP_MIN_TILES", 2048))
+        CML_COUNT_LAUNCH("q6k.dot.buffers.fused");
+    } else if (tiles >= env_int("CAMELID_HIP_Q6K_DEEP_MIN_TILES", 2048)) {
         hipLaunchKernelGGL((gemv_q6k_kernel<1, false, false, 4, true>), dim3(gx, 1), dim3(256), lds, st, ka);
-    else
+        CML_COUNT_LAUNCH("q6k.dot.deep.fused");
+    } else {
         hipLaunchKernelGGL((gemv_q6k_kernel<1, false, false, 2, true>), dim3(gx, 1), dim3(256), lds, st, ka);
+        CML_COUNT_LAUNCH("q6k.dot.buffers.fused");
+    }
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }

@@ -17,6 +17,8 @@
 // 64/P rows, a workgroup 2, 4, 8 or 16 waves.  Activations (int8 + per-block f32 scale, and for
 // Q4_0 the per-block sums that carry the -8 bias) are staged once per workgroup in LDS, or
 // quantized there from f32 by the workgroup itself (FUSEQ: one or two tokens).
+#include <string>
+
 #include "cml_device.hpp"
 #include "cml_host.hpp"
 
@@ -495,22 +497,34 @@ static int b32_depth(int rows, int lanes_per_row, int nb) {
     return (waves <= 2048 && n_steps >= 16) ? 4 : 2;
 }
 
+
+// Counter names of this file: "<format>.dot.p<lanes per row>.<variant>" (launch-counter registry, cml_kernel_launches).
+template <int FMT, int P>
+static std::string b32_counter(const char *variant) {
+    return std::string(FMT == CML_Q8_0 ? "q8_0" : "q4_0") + ".dot.p" + std::to_string(P) + "." + variant;
+}
+
 template <int FMT, int P, int NT>
 static int launch_b32_nt(const B32Args &ba, int n_bands, bool ints, hipStream_t st) {
     const int rows_per_wg = 4 * (64 / P);
     const unsigned gx = static_cast<unsigned>((ba.rows + rows_per_wg - 1) / rows_per_wg);
     const size_t lds = static_cast<size_t>(NT) * ba.nb * (32 + 4 + 4);
     if (lds > 64 * 1024) return fail(CML_ERR_UNSUPPORTED, "activation of %d blocks x %d tokens exceeds the LDS staging limit", ba.nb, NT);
-    if (ints && NT == 1)
+    if (ints && NT == 1) {
         hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, true>), dim3(gx, n_bands), dim3(256), lds, st, ba);
-    else if (NT <= 2 && n_bands == 1 && b32_depth(ba.rows, P, ba.nb) == 4)
+        CML_COUNT_LAUNCH((b32_counter<FMT, P>("ints")));
+    } else if (NT <= 2 && n_bands == 1 && b32_depth(ba.rows, P, ba.nb) == 4) {
         hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, (NT <= 2 ? NT : 1), false, false, 4, 0, 4>), dim3(gx, n_bands), dim3(256), lds, st, ba);
-    else if (NT <= 2 && n_bands == 1 && env_int("CAMELID_HIP_B32_WAVES", ba.rows >= 384 * 8 * (64 / P) ? 8 : 4) == 8)
+        CML_COUNT_LAUNCH((b32_counter<FMT, P>("w4.deep")));
+    } else if (NT <= 2 && n_bands == 1 && env_int("CAMELID_HIP_B32_WAVES", ba.rows >= 384 * 8 * (64 / P) ? 8 : 4) == 8) {
         // eight-wave workgroups where they still come to 1.5 per compute unit (Q8_0 14336 x 4096: 14.0 -> 12.5 us;
         // 11008 x 4096, 1.3 per compute unit: 6.1 -> 6.9)
         hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, (NT <= 2 ? NT : 1), false, false, 8, 0, 2>), dim3((gx + 1) / 2, n_bands), dim3(512), lds, st, ba);
-    else
+        CML_COUNT_LAUNCH((b32_counter<FMT, P>("w8")));
+    } else {
         hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, NT, false>), dim3(gx, n_bands), dim3(256), lds, st, ba);
+        CML_COUNT_LAUNCH((b32_counter<FMT, P>("w4")));
+    }
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }
@@ -604,6 +618,7 @@ static int launch_b32_f32_p(const cml_weight *w, const float *x, float *out, hip
             else if (ring) hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, true, 8, 2, 2, 3, true>), grid2, dim3(512), lds, st, ba);
             else if (nxq == 1) hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, true, 8, 1, 2, 0, true>), grid2, dim3(512), lds, st, ba);
             else hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, true, 8, 2, 2, 0, true>), grid2, dim3(512), lds, st, ba);
+            if (ring) CML_COUNT_LAUNCH((b32_counter<FMT, P>("w8.ring.fused.pair"))); else CML_COUNT_LAUNCH((b32_counter<FMT, P>("w8.fused.pair")));
             CML_HIP_TRY(hipGetLastError());
             return CML_OK;
         } else {
@@ -661,6 +676,17 @@ static int launch_b32_f32_p(const cml_weight *w, const float *x, float *out, hip
         else CML_B32_FUSED(4, 0);
     }
 #undef CML_B32_FUSED
+    {
+        const bool ring_taken = !two && !deep && waves == 8 && FMT == CML_Q8_0 && P == 16 && (ba.nb + P - 1) / P >= 3 && env_int("CAMELID_HIP_B32_RING", 1) &&
+                                (nxq == 1 || nxq == 2);
+        if (two) { if (waves == 8) CML_COUNT_LAUNCH((b32_counter<FMT, P>("w8.fused.two"))); else CML_COUNT_LAUNCH((b32_counter<FMT, P>("w4.fused.two"))); }
+        else if (ring_taken) CML_COUNT_LAUNCH((b32_counter<FMT, P>("w8.ring.fused")));
+        else if (deep) { if (waves == 2) CML_COUNT_LAUNCH((b32_counter<FMT, P>("w2.deep.fused"))); else if (waves == 8) CML_COUNT_LAUNCH((b32_counter<FMT, P>("w8.deep.fused"))); else CML_COUNT_LAUNCH((b32_counter<FMT, P>("w4.deep.fused"))); }
+        else if (waves == 16) CML_COUNT_LAUNCH((b32_counter<FMT, P>("w16.fused")));
+        else if (waves == 8) CML_COUNT_LAUNCH((b32_counter<FMT, P>("w8.fused")));
+        else if (waves == 2) CML_COUNT_LAUNCH((b32_counter<FMT, P>("w2.fused")));
+        else CML_COUNT_LAUNCH((b32_counter<FMT, P>("w4.fused")));
+    }
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }
@@ -869,6 +895,14 @@ static int launch_b32_grouped_u(const MatArgs &a, const GroupedPrologue &pro, hi
             else hipLaunchKernelGGL((gemv_b32_grouped_kernel<FMT, P, 4, 0, U>), grid, dim3(256), lds, st, ga);
             break;
     }
+    switch (pro.kind) {  // "<format>.dot.p<lanes>.grouped[.token | .silu | .gelu | .one]": the prologue a grouped launch ran
+        case 1: CML_COUNT_LAUNCH((b32_counter<FMT, P>("grouped.token"))); break;
+        case 2: CML_COUNT_LAUNCH((b32_counter<FMT, P>("grouped.silu"))); break;
+        case 3: CML_COUNT_LAUNCH((b32_counter<FMT, P>("grouped.gelu"))); break;
+        default:
+            if (one) CML_COUNT_LAUNCH((b32_counter<FMT, P>("grouped.one"))); else CML_COUNT_LAUNCH((b32_counter<FMT, P>("grouped")));
+            break;
+    }
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }
@@ -926,6 +960,7 @@ static int launch_b32_wide(const MatArgs &a, hipStream_t st) {
         hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, false, 8, 0, 4>), dim3(gx, 1), dim3(512), lds, st, ba);
     else
         hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, false, 8, 0, 2>), dim3(gx, 1), dim3(512), lds, st, ba);
+    CML_COUNT_LAUNCH((b32_counter<FMT, P>("w8.wide")));
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }

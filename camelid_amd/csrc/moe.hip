@@ -364,9 +364,11 @@ int cml_moe_route_top_k(const float *logits_dev, int64_t n_tokens, int n_experts
     if (k <= 64) {
         hipLaunchKernelGGL(moe_route_wave_kernel, dim3(static_cast<unsigned>((n_tokens + 3) / 4)), dim3(256), 0, as_stream(stream), logits_dev,
                            n_tokens, n_experts, k, idx_dev, weight_dev);
+        CML_COUNT_LAUNCH("moe.route.wave");
     } else {
         hipLaunchKernelGGL(moe_route_kernel, dim3(static_cast<unsigned>((n_tokens + 63) / 64)), dim3(64), 0, as_stream(stream), logits_dev,
                            n_tokens, n_experts, k, idx_dev, weight_dev);
+        CML_COUNT_LAUNCH("moe.route.thread");
     }
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
@@ -383,6 +385,7 @@ int cml_moe_route_softmax_top_k(const float *logits_dev, int64_t n_tokens, int n
     const unsigned grid = static_cast<unsigned>((n_tokens + 3) / 4);
     hipLaunchKernelGGL(moe_route_softmax_kernel, dim3(grid), dim3(256), 0, as_stream(stream), logits_dev, n_tokens, n_experts, k,
                        down_scale_dev, idx_dev, weight_dev);
+    CML_COUNT_LAUNCH("moe.route.softmax");
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }
@@ -396,6 +399,7 @@ int cml_moe_plan(const int32_t *idx_dev, int64_t n_tokens, int k, int n_experts,
     if (n_tokens > 0 && (!idx_dev || !token_ids_dev || !route_to_assignment_dev)) return fail(CML_ERR_INVALID, "null pointer");
     hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(kPlanThreads), 0, as_stream(stream), idx_dev, static_cast<int>(n_tokens * k), n_experts, k,
                        token_offsets_dev, token_ids_dev, route_to_assignment_dev, union_experts_dev);
+    CML_COUNT_LAUNCH("moe.plan");
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }
@@ -436,6 +440,7 @@ int cml_moe_weighted_sum(const float *y_dev, const int32_t *route_to_assignment_
     if (!y_dev || !weight_dev || !out_dev) return fail(CML_ERR_INVALID, "null pointer");
     hipLaunchKernelGGL(moe_weighted_sum_kernel, dim3(static_cast<unsigned>((hidden + 255) / 256), static_cast<unsigned>(n_tokens)), dim3(256), 0,
                        as_stream(stream), y_dev, route_to_assignment_dev, weight_dev, k, hidden, n_tokens * k, out_dev, nullptr, 0);
+    CML_COUNT_LAUNCH("moe.weighted_sum");
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }
@@ -516,6 +521,7 @@ static int moe_ffn_impl(const cml_weight *gate, const cml_weight *up, const cml_
     if (!direct) {
         hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(kPlanThreads), 0, st, idx_dev, n_slots, n_experts, k, ws.offsets, ws.assign_token,
                            ws.slot_to_assign, ws.group_ids);
+        CML_COUNT_LAUNCH("moe.plan");
         CML_HIP_TRY(hipGetLastError());
     }
 
@@ -595,6 +601,7 @@ static int moe_ffn_impl(const cml_weight *gate, const cml_weight *up, const cml_
     hipLaunchKernelGGL(moe_weighted_sum_kernel, dim3(static_cast<unsigned>((hidden + 255) / 256), static_cast<unsigned>(n_tokens)), dim3(256), 0, st,
                        ws.y, direct ? nullptr : ws.slot_to_assign, weight_dev, k, hidden, static_cast<int64_t>(n_slots), out_dev,
                        direct ? idx_dev : nullptr, n_experts);
+    CML_COUNT_LAUNCH("moe.weighted_sum");
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }

@@ -380,6 +380,7 @@ int launch_rms_norm_quantize(int act, const float *x, const float *weight, float
         case 3: hipLaunchKernelGGL(rms_norm_quantize_kernel<3>, grid, block, lds, st, x, weight, eps, c, normed, q, scales); break;
         default: hipLaunchKernelGGL(rms_norm_quantize_kernel<2>, grid, block, lds, st, x, weight, eps, c, normed, q, scales); break;
     }
+    CML_COUNT_LAUNCH("producer.rms_norm");
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }
@@ -433,12 +434,14 @@ int launch_glu_quantize(int glu, int act, const float *g, const float *u, int64_
         const int bpr = static_cast<int>(cols / 32);
         if (glu == 0) hipLaunchKernelGGL(glu_quantize_q8_0_kernel<0>, grid, dim3(256), 0, st, g, u, n_blocks, bpr, in_stride, q, scales);
         else hipLaunchKernelGGL(glu_quantize_q8_0_kernel<1>, grid, dim3(256), 0, st, g, u, n_blocks, bpr, in_stride, q, scales);
+        CML_COUNT_LAUNCH("producer.glu.q8_0");
     } else {
         const int64_t n_sb = n_tokens * (cols / 256);
         const dim3 grid(static_cast<unsigned>((n_sb + 3) / 4));
         const int spr = static_cast<int>(cols / 256);
         if (glu == 0) hipLaunchKernelGGL(glu_quantize_q8k_kernel<0>, grid, dim3(256), 0, st, g, u, n_sb, spr, in_stride, q, scales);
         else hipLaunchKernelGGL(glu_quantize_q8k_kernel<1>, grid, dim3(256), 0, st, g, u, n_sb, spr, in_stride, q, scales);
+        CML_COUNT_LAUNCH("producer.glu.q8_k");
     }
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;

@@ -54,6 +54,7 @@ int launch_quantize_q8_0(const float *x, int64_t n_tokens, int64_t cols, int8_t 
     const int64_t threads = n_blocks * 8;
     const unsigned grid = static_cast<unsigned>((threads + 255) / 256);
     hipLaunchKernelGGL(quantize_q8_0_kernel, dim3(grid), dim3(256), 0, st, x, n_blocks, q, s);
+    CML_COUNT_LAUNCH("quantize.q8_0");
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }
@@ -63,6 +64,7 @@ int launch_quantize_q8_k(const float *x, int64_t n_tokens, int64_t cols, int8_t 
     if (n_sb == 0) return CML_OK;
     const unsigned grid = static_cast<unsigned>((n_sb + 3) / 4);
     hipLaunchKernelGGL(quantize_q8_k_kernel, dim3(grid), dim3(256), 0, st, x, n_sb, q, d);
+    CML_COUNT_LAUNCH("quantize.q8_k");
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }

@@ -95,6 +95,17 @@ const char *cml_last_error(void);
 /* Number of gemv/gemm launches completed by this process: proves the device
  * lane ran (reference cuda_q8_run_count, src/cuda.rs:350-358). */
 uint64_t cml_run_count(void);
+/* Launches, by kernel family, since the library was loaded: the sum of the counters whose dotted
+ * name starts with `prefix` (null or "" = all).  Names are "<format>.<family>[.<variant>...]",
+ * e.g. "q4k.dot.wg8", "q4k.dot.ring.fused", "q4k.mfma.pair", "q8_0.mfma.kpar", "q6k.lanes",
+ * "moe.plan": a test (or a host) reads the counter before and after a call to prove WHICH kernel
+ * served it -- several kernels give the same bits, so results alone cannot (reference: the
+ * engaged counters of src/inference.rs:23740, 24596-24603 and the test that reads them,
+ * src/inference/tests.rs:7158-7196; cuda_q8_run_count, src/cuda.rs:346-358).
+ * cml_kernel_launch_report writes "name count" lines for every counter that has fired into buf
+ * (at most cap bytes, always terminated) and returns the size the whole report needs. */
+uint64_t cml_kernel_launches(const char *prefix);
+size_t cml_kernel_launch_report(char *buf, size_t cap);
 /* Block geometry helpers: 0 for an unknown format. */
 int cml_block_values(int fmt);
 int cml_block_bytes(int fmt);

@@ -39,6 +39,38 @@ def env(**kv):
         check(lib().cml_reload_env(), "cml_reload_env")
 
 
+def launch_counts() -> dict:
+    """{counter name: launches so far} from the library's kernel-family counters."""
+    L = lib()
+    need = L.cml_kernel_launch_report(None, 0)
+    buf = C.create_string_buffer(int(need) + 256)
+    L.cml_kernel_launch_report(buf, len(buf))
+    out = {}
+    for line in buf.value.decode().splitlines():
+        name, _, n = line.rpartition(" ")
+        out[name] = out.get(name, 0) + int(n)
+    return out
+
+
+@contextmanager
+def engaged(*expect, none=()):
+    """The calls inside the block launch at least one kernel whose counter name matches each regular
+    expression of `expect`, and none whose name matches one of `none` (re.search on the dotted
+    names).  Several kernels of this library return the same bits, so a comparison of results cannot
+    tell which one served a call: this can (the reference's tests read its engaged counters for
+    the same reason, src/inference/tests.rs:7158-7196)."""
+    import re
+    before = launch_counts()
+    yield
+    after = launch_counts()
+    fired = {k: v - before.get(k, 0) for k, v in after.items() if v > before.get(k, 0)}
+    for pat in expect:
+        assert any(re.search(pat, k) for k in fired), f"no kernel matching {pat!r} ran; launched: {fired}"
+    for pat in none:
+        hit = {k: v for k, v in fired.items() if re.search(pat, k)}
+        assert not hit, f"kernels matching {pat!r} ran: {hit}"
+
+
 def is_k(fmt: int) -> bool:
     return fmt in (B.CML_Q4_K, B.CML_Q6_K)
 

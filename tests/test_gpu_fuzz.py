@@ -95,7 +95,16 @@ def test_register_buffer_rings_cover_every_remainder():
                 if fmt != oracle.Q4_K and ksplit != "1":
                     continue
                 G.say(f"ring fmt={fmt} {rows}x{cols} ring={ring} ksplit={ksplit}")
-                with G.env(CAMELID_HIP_Q4K_RING=ring, CAMELID_HIP_B32_RING=ring, CAMELID_HIP_Q4K_KSPLIT=ksplit):
+                # the kernels that must (not) have served these calls: with the ring on and no K cut every test row is
+                # a whole number of ring steps; with it off no ring kernel may run
+                tag = "q4k" if fmt == oracle.Q4_K else "q8_0"
+                if ring == "0":
+                    proof = G.engaged(rf"^{tag}\.dot\.", none=(rf"^{tag}\.dot\..*ring", r"^q4k\.dot\.wg8"))
+                elif ksplit == "1":
+                    proof = G.engaged(rf"^{tag}\.dot\..*ring")
+                else:
+                    proof = G.engaged(rf"^{tag}\.dot\.")
+                with G.env(CAMELID_HIP_Q4K_RING=ring, CAMELID_HIP_B32_RING=ring, CAMELID_HIP_Q4K_KSPLIT=ksplit), proof:
                     one = G.gpu_matmul_f32(w, x[0])
                     two = G.gpu_matmul_f32(w, x)
                     pre = G.gpu_gemm(w, s[:1], q[:1]).reshape(rows)

@@ -335,6 +335,59 @@ def test_q4k_fused_quantize_matvec_is_the_two_step_path(rows, cols):
             assert G.same_bits(got, want)
 
 
+@pytest.mark.parametrize("rows", [12288, 14336, 14327, 16384])
+def test_q4k_eight_wave_launch_is_the_four_wave_launch_and_the_two_step_path(rows):
+    """Rows of 4096 values on 12288 to 16384 rows (no K cut): cml_matmul_f32 runs the eight-wave launch
+    whose quantizer gives a 32-lane half wave to each super-block.  Same bits as the four-wave ring launch
+    (CAMELID_HIP_Q4K_CU=0, 16-lane quantizer rows), as quantize_q8_k followed by the matvec, and as the
+    oracle, on activations built to break a quantizer: zero super-blocks, the maximum magnitude held by both
+    signs (first holder positive, first holder negative, inside one lane, in different lanes, in the two
+    16-lane rows of a half wave, in the two halves), exact rounding ties, a super-block of equal values, NaNs;
+    also on a row band that starts inside a 16-row tile.  The counters prove which launch ran."""
+    fmt, cols = oracle.Q4_K, 4096
+    rng = np.random.default_rng(8000 + rows)
+    wire = G.synth_weight(fmt, rows, cols, seed=8100 + rows)
+    w = Weight.upload(fmt, rows, cols, wire)
+    acts = rng.standard_normal((6, cols)).astype(np.float32)
+    a = acts[0]
+    a[0:256] = 0.0                                    # an all-zero super-block
+    a[256 + 5], a[256 + 6] = 3.5, -3.5                # both signs in one lane (values 8l..8l+7), positive first
+    a[512 + 6], a[512 + 5] = 3.5, -3.5                # ... negative first
+    a[768 + 3], a[768 + 100] = -4.0, 4.0              # different lanes of one 16-lane row, negative first
+    a[1024 + 3], a[1024 + 200] = 4.0, -4.0            # the two 16-lane rows of a half wave, positive first
+    a[1280 + 130], a[1280 + 255] = -4.5, 4.5          # upper row only, negative first
+    a[1536:1792] = 2.0                                # a super-block of equal values
+    a[1792:2048] = -2.0
+    a[2048 + 7] = 127.0
+    a[2048 + 8:2048 + 12] = [0.5, 1.5, -0.5, -2.5]    # exact .5 ties under iscale = -1
+    a[2304 + 0], a[2304 + 255] = -6.0, 6.0            # first and last value of a super-block
+    b = acts[1]
+    b[3], b[300], b[1000] = np.nan, np.nan, np.nan    # NaNs are skipped by the maximum scan
+    b[256 * 5:256 * 6] = np.nan                       # a whole super-block of NaNs
+    acts[2, :] = 0.0                                  # everything zero
+    acts[3, 1::2] = -acts[3, ::2]                     # every magnitude twice, alternating signs
+    acts[4] = np.round(acts[4] * 8) / 8               # many repeated magnitudes
+    band = w.slice(5, rows - 9)
+    s_all, q_all = oracle.quantize_activation(fmt, np.nan_to_num(acts))
+    for i, x in enumerate(acts):
+        G.say(f"Q4_K eight-wave launch {rows}x4096 act={i}")
+        with G.engaged(r"^q4k\.dot\.wg8\.fused$", none=(r"^q4k\.dot\.ring", r"^q4k\.dot\.buffers", r"^quantize\.")):
+            got = G.gpu_matmul_f32(w, x)
+            got_band = G.gpu_matmul_f32(band, x)
+        with G.env(CAMELID_HIP_Q4K_CU=0), G.engaged(r"^q4k\.dot\.ring\.fused$", none=(r"^q4k\.dot\.wg8",)):
+            four = G.gpu_matmul_f32(w, x)
+        with G.env(CAMELID_HIP_FUSED_QUANT=0), G.engaged(r"^quantize\.q8_k$", r"^q4k\.dot\.ring$", none=(r"^q4k\.dot\.wg8", r"fused")):
+            two_step = G.gpu_matmul_f32(w, x)
+        assert G.same_bits(got, four), (rows, i)
+        assert G.same_bits(got, two_step), (rows, i)
+        assert G.same_bits(got_band, got[5:rows - 4]), (rows, i)
+        if i != 1:   # the oracle's comparison has no meaning for NaN inputs; the two-step bits above cover them
+            want = oracle.matmul(fmt, wire, cols, x[None, :], order=EXACT_ORDER[fmt], threads=16)[0]
+            assert G.same_bits(got, want), (rows, i)
+            d_gpu, q_gpu = G.gpu_quantize(True, x)
+            assert np.array_equal(q_gpu, q_all[i]) and np.array_equal(d_gpu.view(np.uint32), s_all[i].view(np.uint32))
+
+
 @pytest.mark.parametrize("rows,cols", [(190, 3072), (64, 256), (333, 4096), (40, 14336), (77, 1280)])
 def test_q4k_fused_two_tokens_is_the_two_step_path(rows, cols):
     """Two-token cml_matmul_f32 on Q4_K quantizes both rows inside the matvec kernel: the bits of
@@ -563,6 +616,10 @@ def test_q8_0_block_seam_takes_in_memory_blocks():
 
 # ------------------------------------------------- matrix-core path (n >= 16) ----
 
+# CAMELID_HIP_*_MFMA_SHAPE -> the workgroup shape in the kernel-family counter names
+# (g<token groups per wave>t<waves over the tokens of a row tile>)
+MFMA_SHAPES = {1: "g1t1", 2: "g2t1", 3: "g4t1", 4: "g1t2", 5: "g2t2", 6: "g1t4"}
+
 # (4096, 4096) and (2000, 18*256): the matvec kernel splits K four ways (even and uneven parts);
 # (1600, 9*256) and (6400, 8*256): two ways; (300, 56*256): eight ways (reproduced inside the lane)
 @pytest.mark.parametrize("rows,cols", [(130, 1024), (2049, 5 * 256), (300, 56 * 256), (16, 256), (4096, 4096), (2000, 18 * 256),
@@ -577,12 +634,14 @@ def test_q4k_matrix_core_cells_are_bitwise_the_gemv(rows, cols):
         s, q = oracle.quantize_activation(fmt, x)
         for shape in (0, 1, 2, 3, 4, 5, 6):   # 0 = the default workgroup shape, 1..6 = every other one
             G.say(f"Q4_K matrix-core {rows}x{cols} n={n} shape={shape}")
-            with G.env(CAMELID_HIP_Q4K_MFMA_SHAPE=shape):
+            # which kernel must have run: any matrix-core one by default, the named workgroup shape otherwise
+            want_kernel = r"^q4k\.mfma\." if shape == 0 else r"^q4k\.mfma\.(tile|serial_split)\." + MFMA_SHAPES[shape] + r"(\.|$)"
+            with G.env(CAMELID_HIP_Q4K_MFMA_SHAPE=shape), G.engaged(want_kernel, none=(r"^q4k\.dot\.",)):
                 got = G.gpu_gemm(w, s, q)                      # default K-split policy, reproduced across waves or in-lane
             if shape == 0:
-                with G.env(CAMELID_HIP_Q4K_MFMA_SERIAL_SPLIT=1):
+                with G.env(CAMELID_HIP_Q4K_MFMA_SERIAL_SPLIT=1), G.engaged(r"^q4k\.mfma\.", none=(r"^q4k\.mfma\.ksplit", r"^q4k\.dot\.")):
                     assert G.same_bits(got, G.gpu_gemm(w, s, q))
-            with G.env(CAMELID_HIP_Q4K_MFMA_MIN_TOKENS=1 << 30):
+            with G.env(CAMELID_HIP_Q4K_MFMA_MIN_TOKENS=1 << 30), G.engaged(r"^q4k\.dot\.", none=(r"^q4k\.mfma\.",)):
                 ref = G.gpu_gemm(w, s, q)                      # the packed-dot kernel on the same inputs
             assert G.same_bits(got, ref)
             check_outputs(fmt, wire, cols, s, q, got, expect_exact=False)
@@ -607,9 +666,10 @@ def test_q4k_two_waves_per_tile_keep_one_chain(rows, cols):
         want = oracle.matmul_q(fmt, wire, cols, s, q, order=oracle.ORDER_PRIMARY, threads=8)
         G.say(f"Q4_K two waves per tile {rows}x{cols} n={n}")
         with G.env(CAMELID_HIP_EXACT_ORDER="1"):
-            got = G.gpu_gemm(w, s, q)
-            got_band = G.gpu_gemm(band, s, q)
-            with G.env(CAMELID_HIP_EXACT_ORDER="1", CAMELID_HIP_Q4K_MFMA_PAIR=0):
+            with G.engaged(r"^q4k\.mfma\.pair$", none=(r"^q4k\.mfma\.(tile|serial_split|ksplit)", r"^q4k\.dot\.")):
+                got = G.gpu_gemm(w, s, q)
+                got_band = G.gpu_gemm(band, s, q)
+            with G.env(CAMELID_HIP_EXACT_ORDER="1", CAMELID_HIP_Q4K_MFMA_PAIR=0), G.engaged(r"^q4k\.mfma\.tile\.g1t1", none=(r"^q4k\.mfma\.pair", r"^q4k\.dot\.")):
                 one_wave = G.gpu_gemm(w, s, q)
         assert G.same_bits(got, want)
         assert G.same_bits(got, one_wave)
@@ -630,12 +690,16 @@ def test_b32_matrix_core_cells_are_bitwise_the_gemv(name, fmt, rows, cols):
             x[1] = 0.0              # an all-zero token: scale 0, sums 0
             x[2, :32] = -x[2, :32].max() * 4   # a block at the negative extreme
         s, q = oracle.quantize_activation(fmt, x)
-        with G.env(CAMELID_HIP_B32_MFMA_MIN_TOKENS=1 << 30):
+        tag = name.lower()
+        with G.env(CAMELID_HIP_B32_MFMA_MIN_TOKENS=1 << 30), G.engaged(rf"^{tag}\.dot\.", none=(rf"^{tag}\.mfma\.",)):
             ref = G.gpu_gemm(w, s, q)                      # the packed-dot kernel on the same inputs
         for shape in (0, 1, 2, 3, 4, 5, 6):   # 0 = the default workgroup shape, 1..6 = every other one
             G.say(f"{name} matrix-core {rows}x{cols} n={n} shape={shape}")
             for deep in (0, 1):          # short phases / shallow ring, long phases / deep ring
-                with G.env(CAMELID_HIP_B32_MFMA_SHAPE=shape, CAMELID_HIP_B32_MFMA_DEEP=deep):
+                # MIN_TOKENS=1: the matrix-core kernels also below the batch size from which they pay
+                want_kernel = rf"^{tag}\.mfma\." if shape == 0 else rf"^{tag}\.mfma\.tile\." + MFMA_SHAPES[shape] + r"\.w\d+\." + ("r[48]" if deep else "r2")
+                with G.env(CAMELID_HIP_B32_MFMA_SHAPE=shape, CAMELID_HIP_B32_MFMA_DEEP=deep, CAMELID_HIP_B32_MFMA_MIN_TOKENS=1), \
+                        G.engaged(want_kernel, none=(rf"^{tag}\.dot\.",)):
                     got = G.gpu_gemm(w, s, q)
                 assert G.same_bits(got, ref)
         check_outputs(fmt, wire, cols, s, q, got, expect_exact=True)
@@ -658,9 +722,19 @@ def test_b32_waves_sharing_a_row_tile_keep_the_block_order(name, fmt, rows, cols
         s, q = oracle.quantize_activation(fmt, x)
         want = oracle.matmul_q(fmt, wire, cols, s, q, order=oracle.ORDER_PRIMARY, threads=8)
         with G.env(CAMELID_HIP_B32_MFMA_MIN_TOKENS=1):
+            tag, slabs = name.lower(), cols // 256
             for variant in (-1, 0, 1, 2, 3, 4):
                 G.say(f"{name} waves per tile, {rows}x{cols} n={n} variant={variant}")
-                with G.env(CAMELID_HIP_B32_MFMA_MIN_TOKENS=1, CAMELID_HIP_B32_MFMA_KPAR=variant):
+                # the kernel each variant selects for rows of this many slabs (launch_b32_mfma_fmt); every test matrix
+                # has few enough row tiles for the default (-1) to share tiles as well
+                if variant == 0:
+                    want_kernel, never = rf"^{tag}\.mfma\.tile\.", (rf"^{tag}\.mfma\.kpar", rf"^{tag}\.dot\.")
+                else:
+                    table = ({1: "k4s2t1", 2: "k4s2t2", 3: "k8s1t1", 4: "k8s1t2"} if 4 <= slabs <= 8 else
+                             {1: "k4s4t1", 2: "k8s2t1", 3: "k8s2t2"} if 8 < slabs <= 16 else {1: "k2s2t1", 2: "k2s2t1", 3: "k2s2t1", 4: "k2s2t1"})
+                    want_kernel = rf"^{tag}\.mfma\.kpar\." + table.get(variant, r"k\d")
+                    never = (rf"^{tag}\.mfma\.tile\.", rf"^{tag}\.dot\.")
+                with G.env(CAMELID_HIP_B32_MFMA_MIN_TOKENS=1, CAMELID_HIP_B32_MFMA_KPAR=variant), G.engaged(want_kernel, none=never):
                     got = G.gpu_gemm(w, s, q)
                 assert G.same_bits(got, want)
 
@@ -694,15 +768,18 @@ def test_q6k_matrix_core_cells_are_bitwise_the_gemv(rows, cols):
             x[1] = 0.0
             x[2, :256] = -np.abs(x[2, :256]).max() * 4   # a super-block at the negative extreme
         s, q = oracle.quantize_activation(fmt, x)
-        with G.env(CAMELID_HIP_Q6K_MFMA_MIN_TOKENS=1 << 30):
+        with G.env(CAMELID_HIP_Q6K_MFMA_MIN_TOKENS=1 << 30), G.engaged(r"^q6k\.dot\.", none=(r"^q6k\.mfma\.",)):
             ref = G.gpu_gemm(w, s, q)                      # the packed-dot kernel on the same inputs
         for shape in (0, 1, 2, 3, 4, 6):
             for deep in (0, 1):
                 G.say(f"Q6_K matrix-core {rows}x{cols} n={n} shape={shape} deep={deep}")
-                with G.env(CAMELID_HIP_Q6K_MFMA_SHAPE=shape, CAMELID_HIP_Q6K_MFMA_DEEP=deep, CAMELID_HIP_Q6K_MFMA_MIN_TOKENS=1):
+                want_kernel = r"^q6k\.mfma\." if shape == 0 else r"^q6k\.mfma\.(tile|serial_split)\." + MFMA_SHAPES[shape] + r"\." + ("r4" if deep else "r2")
+                with G.env(CAMELID_HIP_Q6K_MFMA_SHAPE=shape, CAMELID_HIP_Q6K_MFMA_DEEP=deep, CAMELID_HIP_Q6K_MFMA_MIN_TOKENS=1), \
+                        G.engaged(want_kernel, none=(r"^q6k\.dot\.",)):
                     got = G.gpu_gemm(w, s, q)
                 assert G.same_bits(got, ref)
-        with G.env(CAMELID_HIP_Q6K_MFMA_SERIAL_SPLIT=1, CAMELID_HIP_Q6K_MFMA_MIN_TOKENS=1):   # the split inside the lane
+        with G.env(CAMELID_HIP_Q6K_MFMA_SERIAL_SPLIT=1, CAMELID_HIP_Q6K_MFMA_MIN_TOKENS=1), \
+                G.engaged(r"^q6k\.mfma\.", none=(r"^q6k\.mfma\.ksplit", r"^q6k\.dot\.")):   # the split inside the lane
             assert G.same_bits(G.gpu_gemm(w, s, q), ref)
         check_outputs(fmt, wire, cols, s, q, got, expect_exact=False)
         with G.env(CAMELID_HIP_EXACT_ORDER="1", CAMELID_HIP_Q6K_MFMA_MIN_TOKENS=1):
