@@ -956,3 +956,84 @@ def test_matmul_f32_pair_is_two_single_calls(name, fmt, rows, cols):
     d = DeviceBuffer(64)
     assert L.cml_matmul_f32_pair(wa.handle, None, d.ptr, d.ptr, d.ptr, d.ptr, 64, None) == 2
     assert L.cml_matmul_f32_pair(wa.handle, wb.handle, None, d.ptr, d.ptr, d.ptr, 64, None) == 2
+
+
+# ------------------------------------------------- the top of the integer range ----
+
+def _saturated_weight(fmt, rows, cols, rng):
+    """Wire rows whose every block sits at the top (or bottom) of what the format can encode, with
+    small random f16 scales so that the f32 results stay finite."""
+    nb = cols // oracle.block_values(fmt)
+    bb = oracle.block_bytes(fmt)
+    blk = np.empty((rows, nb, bb), np.uint8)
+
+    def f16_bytes(lo, hi, shape):
+        return rng.uniform(lo, hi, shape).astype(np.float16).view(np.uint8).reshape(*shape, 2)
+
+    if fmt == B.CML_Q4_K:
+        blk[:, :, 16:] = rng.integers(0xcc, 0x100, (rows, nb, 128), dtype=np.uint8)   # nibbles 12..15
+        blk[:, :, 4:16] = 0xff                                                        # 6-bit scales and mins all 63
+        blk[:, :, 0:2] = f16_bytes(0.001, 0.004, (rows, nb))
+        blk[:, :, 2:4] = f16_bytes(0.01, 0.04, (rows, nb))
+    elif fmt == B.CML_Q6_K:
+        top = rng.integers(0, 2, (rows, nb, 1), dtype=np.uint8)                       # a super-block of all 63 or all 0 codes (+31 / -32)
+        blk[:, :, 0:192] = np.where(top == 1, 0xff, 0x00)
+        blk[:, :, 192:208] = rng.choice(np.array([127, -128, -127], np.int8), (rows, nb, 16)).view(np.uint8)
+        blk[:, :, 208:210] = f16_bytes(0.0005, 0.002, (rows, nb))
+    elif fmt == B.CML_Q8_0:
+        blk[:, :, 0:2] = f16_bytes(0.01, 0.05, (rows, nb))
+        blk[:, :, 2:] = rng.choice(np.array([127, -128], np.int8), (rows, nb, 32)).view(np.uint8)
+    else:
+        blk[:, :, 0:2] = f16_bytes(0.01, 0.05, (rows, nb))
+        blk[:, :, 2:] = rng.choice(np.array([0x00, 0xff, 0xf0, 0x0f], np.uint8), (rows, nb, 16))   # nibbles 0 or 15: -8 or +7
+    return np.ascontiguousarray(blk.reshape(-1))
+
+
+@pytest.mark.parametrize("name,fmt", FMTS)
+def test_saturated_blocks_and_activations_keep_every_bit(name, fmt):
+    """Weights and activations at the top of the integer range -- 6-bit scales all 63 with nibbles 12..15,
+    Q6_K codes all 63 or all 0 under int8 scales of +127 / -128, int8 weights of +127 / -128, activations of
+    +127, of -128 (which no quantizer produces but a caller of cml_gemv may pass), of the weight's sign and
+    of 125..127 -- through cml_block_dots, cml_gemv and cml_gemm at 2, 3, 16 and 64 tokens, in both
+    accumulation orders of the K-quants: the oracle's bits.  The super-block integers pass 2^24 here, so
+    their conversion to f32 rounds; 24-bit multiplies, digit-split scales and half-precision run sums inside
+    the kernels would show up as wrong bits exactly on such inputs."""
+    rng = np.random.default_rng(900 + fmt)
+    bv = oracle.block_values(fmt)
+    is_k = G.is_k(fmt)
+    lane_knob = {B.CML_Q4_K: "CAMELID_HIP_Q4K_LANE_ORDER", B.CML_Q6_K: "CAMELID_HIP_Q6K_LANE_ORDER"}.get(fmt)
+    # the order the fast kernels keep, and the one the lane-order kernels keep
+    fast_order = EXACT_ORDER[fmt]
+    lane_order = (oracle.ORDER_ALT if fast_order == oracle.ORDER_PRIMARY else oracle.ORDER_PRIMARY) if is_k else None
+    for rows, nbr in ((37, 3), (300, 16), (130, 8 if not is_k else 5)):
+        cols = nbr * (256 if is_k else 256)   # Q8_0 / Q4_0: whole 256-value slabs, so that the matrix-core kernels serve them
+        wire = _saturated_weight(fmt, rows, cols, rng)
+        w = Weight.upload(fmt, rows, cols, wire)
+        n_max = 64
+        q = np.empty((n_max, cols), np.int8)
+        q[0] = 127
+        q[1] = -128
+        q[2] = rng.integers(125, 128, cols)
+        q[3] = np.where(rng.integers(0, 2, cols) == 1, 127, -128)
+        q[4:] = rng.choice(np.array([127, -128, -127, 126], np.int8), (n_max - 4, cols))
+        s = rng.uniform(0.01, 0.05, (n_max, cols // (256 if is_k else 32))).astype(np.float32)
+        G.say(f"{name} saturated {rows}x{cols}: block integers")
+        for t in (0, 1, 3):
+            assert np.array_equal(G.gpu_block_dots(w, q[t]), oracle.block_ints(fmt, wire, cols, q[t])), (name, rows, cols, t)
+        for n in (1, 2, 3, 16, 64):
+            want = oracle.matmul_q(fmt, wire, cols, s[:n], q[:n], order=fast_order, threads=8)
+            G.say(f"{name} saturated {rows}x{cols} n={n}")
+            with G.env(CAMELID_HIP_EXACT_ORDER="1"):
+                got = G.gpu_gemm(w, s[0], q[0]) if n == 1 else G.gpu_gemm(w, s[:n], q[:n])
+                assert G.same_bits(got.reshape(n, rows), want), (name, rows, cols, n, "fast kernels")
+                if n >= 3:   # the packed-dot kernel on the same batch
+                    knob = {B.CML_Q4_K: "CAMELID_HIP_Q4K_MFMA_MIN_TOKENS", B.CML_Q6_K: "CAMELID_HIP_Q6K_MFMA_MIN_TOKENS"}.get(fmt, "CAMELID_HIP_B32_MFMA_MIN_TOKENS")
+                    with G.env(CAMELID_HIP_EXACT_ORDER="1", **{knob: 1 << 30}), G.engaged(r"\.dot\.", none=(r"\.mfma\.",)):
+                        assert G.same_bits(G.gpu_gemm(w, s[:n], q[:n]), want), (name, rows, cols, n, "packed dot")
+                    with G.env(CAMELID_HIP_EXACT_ORDER="1", **{knob: 1}), G.engaged(r"\.mfma\.", none=(r"\.dot\.",)):
+                        assert G.same_bits(G.gpu_gemm(w, s[:n], q[:n]), want), (name, rows, cols, n, "matrix cores")
+            if lane_knob and n <= 3:
+                want_lane = oracle.matmul_q(fmt, wire, cols, s[:n], q[:n], order=lane_order, threads=8)
+                with G.env(**{lane_knob: 1}), G.engaged(r"\.lanes$"):
+                    got = G.gpu_gemm(w, s[0], q[0]) if n == 1 else G.gpu_gemm(w, s[:n], q[:n])
+                assert G.same_bits(got.reshape(n, rows), want_lane), (name, rows, cols, n, "lane order")
