@@ -23,7 +23,7 @@ EXPORTS = [
     "cml_event_destroy", "cml_graph_begin_capture", "cml_graph_end_capture", "cml_graph_launch", "cml_graph_destroy",
     "cml_weight_upload", "cml_weight_upload_dev", "cml_weight_slice", "cml_weight_info",
     "cml_weight_download", "cml_weight_free",
-    "cml_quantize_q8_0", "cml_quantize_q8_k", "cml_rms_norm_quantize", "cml_sum_squares_f32", "cml_silu_mul_quantize", "cml_glu_quantize", "cml_embed_gather", "cml_argmax_f32", "cml_dequantize",
+    "cml_quantize_q8_0", "cml_quantize_q8_k", "cml_rms_norm_quantize", "cml_rms_inv_norm_quantize", "cml_sum_squares_f32", "cml_silu_mul_quantize", "cml_glu_quantize", "cml_embed_gather", "cml_argmax_f32", "cml_dequantize",
     "cml_gemv", "cml_gemm", "cml_block_dots", "cml_matmul_workspace_bytes", "cml_matmul_f32", "cml_matmul_f32_pair", "cml_matmul_f32_static",
     "cml_moe_route_top_k", "cml_moe_route_softmax_top_k", "cml_moe_workspace_bytes", "cml_moe_ffn", "cml_moe_ffn_ex", "cml_moe_ffn_logits",
     "cml_moe_plan", "cml_moe_gemv_routed", "cml_moe_weighted_sum",
@@ -95,6 +95,7 @@ def lib() -> C.CDLL:
     L.cml_quantize_q8_0.argtypes = [vp, i64, i64, vp, vp, vp]
     L.cml_quantize_q8_k.argtypes = [vp, i64, i64, vp, vp, vp]
     L.cml_rms_norm_quantize.argtypes = [i32, vp, vp, C.c_float, i64, i64, vp, vp, vp, vp]
+    L.cml_rms_inv_norm_quantize.argtypes = [i32, vp, vp, C.c_float, i64, vp, vp, vp]
     L.cml_sum_squares_f32.argtypes = [vp, i64, i64, vp, vp]
     L.cml_silu_mul_quantize.argtypes = [i32, vp, vp, i64, i64, vp, vp, vp]
     L.cml_embed_gather.argtypes = [vp, vp, i64, vp, vp]

@@ -640,6 +640,19 @@ int cml_sum_squares_f32(const float *x_dev, int64_t n_rows, int64_t cols, float 
     return launch_rms_norm_quantize(3, x_dev, nullptr, 0.0f, n_rows, cols, out_dev, nullptr, nullptr, as_stream(stream));
 }
 
+int cml_rms_inv_norm_quantize(int act, const float *x_dev, const float *weight_dev, float rms_inv, int64_t cols, int8_t *q_dev,
+                              float *scales_dev, cml_stream_t stream) {
+    if (int rc = check_ready()) return rc;
+    if (act != CML_ACT_Q8_0 && act != CML_ACT_Q8_K) return fail(CML_ERR_INVALID, "activation format %d is not a quantized one", act);
+    const int64_t unit = act == CML_ACT_Q8_K ? 256 : 32;
+    if (cols < 0 || cols % unit != 0) return fail(CML_ERR_SHAPE, "cols %lld is not a multiple of %lld", (long long)cols, (long long)unit);
+    if (cols == 0) return CML_OK;
+    if (!x_dev || !weight_dev || !q_dev || !scales_dev) return fail(CML_ERR_INVALID, "null pointer");
+    if (misaligned16(x_dev) || misaligned16(weight_dev) || (reinterpret_cast<uintptr_t>(q_dev) & 3u))
+        return fail(CML_ERR_INVALID, "x and weight must be 16-byte and q 4-byte aligned");
+    return launch_rms_inv_norm_quantize(act, x_dev, weight_dev, rms_inv, cols, q_dev, scales_dev, as_stream(stream));
+}
+
 int cml_silu_mul_quantize(int act, const float *gate_dev, const float *up_dev, int64_t n_tokens, int64_t cols, int8_t *q_dev,
                           float *scales_dev, cml_stream_t stream) {
     return cml_glu_quantize(CML_GLU_SILU, act, gate_dev, up_dev, n_tokens, cols, q_dev, scales_dev, stream);

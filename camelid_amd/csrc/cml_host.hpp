@@ -88,6 +88,8 @@ bool q8_0_blocks_to_wire(const uint8_t *blocks, size_t n_blocks, uint8_t *wire);
 int launch_quantize_q8_0(const float *x, int64_t n_tokens, int64_t cols, int8_t *q, float *s, hipStream_t st);
 int launch_quantize_q8_k(const float *x, int64_t n_tokens, int64_t cols, int8_t *q, float *d, hipStream_t st);
 
+int launch_rms_inv_norm_quantize(int act, const float *x, const float *weight, float rms_inv, int64_t cols, int8_t *q, float *scales, hipStream_t st);
+
 // producers.hip: act = 0 (f32 only), 1 (Q8_0), 2 (Q8_K)
 int launch_rms_norm_quantize(int act, const float *x, const float *weight, float eps, int64_t n_tokens, int64_t cols,
                              float *normed, int8_t *q, float *scales, hipStream_t st);

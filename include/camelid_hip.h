@@ -211,6 +211,13 @@ enum { CML_ACT_F32 = 0, CML_ACT_Q8_0 = 1, CML_ACT_Q8_K = 2 };
 int cml_rms_norm_quantize(int act, const float *x_dev, const float *weight_dev, float eps,
                           int64_t n_tokens, int64_t cols, float *normed_dev, int8_t *q_dev,
                           float *scales_dev, cml_stream_t stream);
+/* The same norm with the inverse root-mean-square supplied by the host (reference
+ * rms_inv_norm_quantize_q8_0 / _q8k, src/cuda_resident.rs:272-315, 4272-4291: the CPU router has
+ * already scanned the row and hands over its exact sequential (mean_square + eps)^-0.5): one row,
+ * value[i] = (x[i] * rms_inv) * weight[i], each multiply rounded, then the quantizer above.
+ * act is CML_ACT_Q8_0 (cols a multiple of 32) or CML_ACT_Q8_K (a multiple of 256). */
+int cml_rms_inv_norm_quantize(int act, const float *x_dev, const float *weight_dev, float rms_inv,
+                              int64_t cols, int8_t *q_dev, float *scales_dev, cml_stream_t stream);
 /* The first pass of the norm on its own: out_dev[r] = (((0 + x[r][0]^2) + x[r][1]^2) + ...) in f32,
  * every product and every sum rounded, in index order -- the bits of the scalar
  * loop (reference rms_norm's ordered sum, src/cuda_resident.rs:124-131;

@@ -141,6 +141,37 @@ def test_rms_norm_quantize_is_the_composed_result(cols):
         assert np.array_equal(q3, q) and np.array_equal(s3.view(np.uint32), s.view(np.uint32))
 
 
+@pytest.mark.parametrize("cols", [256, 2816, 4096, 14336])
+def test_rms_inv_norm_quantize_with_the_hosts_inverse(cols):
+    """The norm with the inverse root-mean-square handed over by the host (the reference's CPU router has
+    scanned the row already): value = (x * rms_inv) * weight with both multiplies rounded, then the
+    quantizer -- the bits of the numpy float32 expression followed by the oracle's quantizer, on rows
+    with zero blocks, rounding ties and the maximum held by both signs."""
+    x, w = _rows(3, cols, 960 + cols)
+    x[0, :256] = 0.0
+    x[1, 5], x[1, 9] = 7.0, -7.0
+    w[5], w[9] = 1.0, 1.0
+    for r in range(3):
+        # the host's scan: the sequential f32 sum of squares, (mean + eps)^-0.5 (reference src/tensor/mod.rs:2707-2760)
+        acc = np.float32(0.0)
+        for v in x[r]:
+            acc = np.float32(acc + np.float32(v * v))
+        rms_inv = np.float32(1.0) / np.sqrt(np.float32(acc / np.float32(cols) + np.float32(1e-6)), dtype=np.float32)
+        value = ((x[r] * rms_inv).astype(np.float32) * w).astype(np.float32)
+        for act, per in ((ACT_Q8_0, 32), (ACT_Q8_K, 256)):
+            G.say(f"rms_inv_norm_quantize cols={cols} row={r} act={act}")
+            xd, wd = DeviceBuffer.from_numpy(x[r]), DeviceBuffer.from_numpy(w)
+            qd, sd = DeviceBuffer(cols), DeviceBuffer(cols // per * 4)
+            with G.engaged(r"^producer\.rms_inv_norm\." + ("q8_0" if act == ACT_Q8_0 else "q8_k")):
+                check(lib().cml_rms_inv_norm_quantize(act, xd.ptr, wd.ptr, float(rms_inv), cols, qd.ptr, sd.ptr, None), "cml_rms_inv_norm_quantize")
+            check(lib().cml_stream_sync(None))
+            q, s = qd.to_numpy(np.int8, (cols,)), sd.to_numpy(np.float32, (cols // per,))
+            so, qo = (oracle.quantize_q8_0 if act == ACT_Q8_0 else oracle.quantize_q8_k)(value)
+            assert np.array_equal(q, qo) and np.array_equal(s.view(np.uint32), so.view(np.uint32))
+    assert lib().cml_rms_inv_norm_quantize(ACT_Q8_K, xd.ptr, wd.ptr, 1.0, 100, qd.ptr, sd.ptr, None) != 0   # not whole super-blocks
+    assert lib().cml_rms_inv_norm_quantize(ACT_F32, xd.ptr, wd.ptr, 1.0, cols, qd.ptr, sd.ptr, None) != 0   # nothing to quantize into
+
+
 def test_silu_mul_quantize():
     rng = np.random.default_rng(990)
     for n, cols in ((1, 14336), (3, 2048), (5, 256)):
