@@ -496,6 +496,72 @@ def bench_pair(name: str, K: int, W: int, seed: int) -> int:
     return 0
 
 
+MULTI_CONFIGS = {
+    # name -> (format, [rows of each weight], cols): one token against several weights that read it
+    "q4k_qkv_4096": ("Q4_K", [4096, 1024, 1024], 4096),           # q | k | v of a Llama-3-8B attention block (grouped-query: 8 KV heads)
+    "q4k_qkv_gate_up_4096": ("Q4_K", [14336, 14336], 4096),       # gate | up through the same entry
+    "q4k_qkv_3584": ("Q4_K", [3584, 512, 512], 3584),             # Qwen2.5-7B-shaped q | k | v
+}
+
+
+def bench_multi(name: str, K: int, W: int, seed: int) -> int:
+    """cml_matmul_f32_multi: one f32 token, several weights, one launch where the set is served; beside it the
+    same step as one cml_matmul_f32 call per weight."""
+    L = lib()
+    fmt_name, rows_list, cols = MULTI_CONFIGS[name]
+    fmt = B.FORMATS[fmt_name]
+    n = len(rows_list)
+    wires = [synth_weight(fmt, r, cols, seed + 11 * j) for j, r in enumerate(rows_list)]
+    total = sum(w.nbytes for w in wires)
+    copies = max(2, min(32, -(-600_000_000 // total)))
+    sets = [[Weight.upload(fmt, r, cols, wires[j]) for j, r in enumerate(rows_list)] for _ in range(copies)]
+    x = np.random.default_rng(seed + 1).standard_normal((1, cols)).astype(np.float32)
+    alg = total + 4 * cols + 4 * sum(rows_list)
+    stream = C.c_void_p()
+    check(L.cml_stream_create(C.byref(stream)))
+    xd = DeviceBuffer.from_numpy(x)
+    ws_bytes = L.cml_matmul_workspace_bytes(fmt, cols, 1)
+    ws = DeviceBuffer(ws_bytes)
+    outs = [DeviceBuffer(r * 4) for r in rows_list]
+    optrs = (C.c_void_p * n)(*[o.ptr for o in outs])
+    handles = [(C.c_void_p * n)(*[w.handle for w in st]) for st in sets]
+
+    def multi(i):
+        check(L.cml_matmul_f32_multi(handles[i % copies], n, xd.ptr, optrs, ws.ptr, ws_bytes, stream), "cml_matmul_f32_multi")
+
+    def singles(i):
+        for j, w in enumerate(sets[i % copies]):
+            check(L.cml_matmul_f32(w.handle, xd.ptr, 1, outs[j].ptr, ws.ptr, ws_bytes, stream), "cml_matmul_f32")
+
+    for i in range(W):
+        multi(i)
+    check(L.cml_stream_sync(stream))
+    timers = [Timer(stream) for _ in range(32)]
+    before = L.cml_kernel_launches(b"")
+    multi(0)
+    launches = L.cml_kernel_launches(b"") - before
+    ms = steps_ms(stream, multi, K, timers)[0]
+    ms_single = steps_ms(stream, singles, K, timers)[0]
+    check(L.cml_stream_sync(stream))
+    if not all(np.all(np.isfinite(o.to_numpy(np.float32, (r,)))) for o, r in zip(outs, rows_list)):
+        print("non-finite output", file=sys.stderr)
+        return 4
+    gbs = alg / (ms * 1e-3) / 1e9
+    print(json.dumps({
+        "metric": f"{fmt_name} matvec of {n} weights off one token µs + achieved HBM GB/s, rows {rows_list} x {cols}",
+        "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": round(ms, 6),
+        "us_per_call": round(ms * 1e3, 3), "pct_of_hbm_peak": round(100.0 * gbs / HBM_PEAK_GBS, 2), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
+        "config": {"workload": name, "format": fmt_name, "rows": rows_list, "cols": cols, "tokens": 1, "weights": n,
+                   "algorithmic_bytes_per_call": alg, "weight_copies_rotated": copies, "launches_per_step": int(launches),
+                   "step": "cml_matmul_f32_multi: quantize the token + every fused dequantize-matvec, graph replay",
+                   "as_single_calls_us": round(ms_single * 1e3, 3)},
+        "roofline": {"bound": "hbm", "kernel": "the single-token Q4_K matvec kernel, the weights' workgroups end to end in one launch",
+                     "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "us_per_launch": round(ms * 1e3, 3)}}, ensure_ascii=False))
+    return 0
+
+
 PRODUCER_CONFIGS = {
     # name -> (cols, tokens): rms_norm fused with the Q8_K quantizer, the step upstream of a projection
     "rmsnorm_q8k_4096_t1": (4096, 1),
@@ -604,7 +670,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--config", default="q4k_14336x4096_n1",
-                    help="one of: " + ", ".join(sorted(CONFIGS) + sorted(MOE_CONFIGS) + sorted(PAIR_CONFIGS) + sorted(PRODUCER_CONFIGS))
+                    help="one of: " + ", ".join(sorted(CONFIGS) + sorted(MOE_CONFIGS) + sorted(PAIR_CONFIGS) + sorted(MULTI_CONFIGS) + sorted(PRODUCER_CONFIGS))
                     + "; or any <format>_<rows>x<cols>_n<tokens>, e.g. q8_0_14336x4352_n1")
     ap.add_argument("--copies", type=int, default=0, help="distinct weight copies to rotate over (0 = enough for ~600 MB)")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="time budget of the CPU baseline leg (0 = skip)")
@@ -641,6 +707,8 @@ def main() -> int:
         return bench_producer(args.config, max(1, args.steps), max(0, args.warmup), args.seed)
     if args.config in PAIR_CONFIGS:
         return bench_pair(args.config, max(1, args.steps), max(0, args.warmup), args.seed)
+    if args.config in MULTI_CONFIGS:
+        return bench_multi(args.config, max(1, args.steps), max(0, args.warmup), args.seed)
     if args.config in MOE_CONFIGS:
         return bench_moe(args.config, max(1, args.steps), max(0, args.warmup), args.seed, args.cpu_seconds)
     if args.config in CONFIGS:

@@ -24,7 +24,7 @@ EXPORTS = [
     "cml_weight_upload", "cml_weight_upload_dev", "cml_weight_slice", "cml_weight_info",
     "cml_weight_download", "cml_weight_free",
     "cml_quantize_q8_0", "cml_quantize_q8_k", "cml_rms_norm_quantize", "cml_rms_inv_norm_quantize", "cml_sum_squares_f32", "cml_silu_mul_quantize", "cml_glu_quantize", "cml_embed_gather", "cml_argmax_f32", "cml_dequantize",
-    "cml_gemv", "cml_gemm", "cml_block_dots", "cml_matmul_workspace_bytes", "cml_matmul_f32", "cml_matmul_f32_pair", "cml_matmul_f32_static",
+    "cml_gemv", "cml_gemm", "cml_block_dots", "cml_matmul_workspace_bytes", "cml_matmul_f32", "cml_matmul_f32_pair", "cml_matmul_f32_multi", "cml_matmul_f32_static",
     "cml_moe_route_top_k", "cml_moe_route_softmax_top_k", "cml_moe_workspace_bytes", "cml_moe_ffn", "cml_moe_ffn_ex", "cml_moe_ffn_logits",
     "cml_moe_plan", "cml_moe_gemv_routed", "cml_moe_weighted_sum",
     "cml_quantize_weights_host", "cml_try_linear_rows", "cml_try_q8_0_block_linear_row",
@@ -109,6 +109,7 @@ def lib() -> C.CDLL:
     L.cml_matmul_f32.argtypes = [vp, vp, i64, vp, vp, sz, vp]
     L.cml_matmul_f32_static.argtypes = [vp, vp, i64, vp, vp]
     L.cml_matmul_f32_pair.argtypes = [vp, vp, vp, vp, vp, vp, sz, vp]
+    L.cml_matmul_f32_multi.argtypes = [vp, i32, vp, vp, vp, sz, vp]
     L.cml_moe_route_top_k.argtypes = [vp, i64, i32, i32, vp, vp, vp]
     L.cml_moe_workspace_bytes.argtypes = [i32, i64, i64, i64, i32, i32]
     L.cml_moe_workspace_bytes.restype = sz

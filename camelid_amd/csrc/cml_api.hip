@@ -919,6 +919,46 @@ int cml_matmul_f32_pair(const cml_weight *w_a, const cml_weight *w_b, const floa
     return cml_matmul_f32(w_b, x_dev, 1, out_b_dev, workspace_dev, workspace_bytes, stream);
 }
 
+// One token against SEVERAL weights that read the same activation (the q, k and v projections of an attention block,
+// gate and up of an FFN: the projections the reference hangs off one SharedActivation, src/gemma4_runtime.rs:1288-1340).
+// Groups of up to four Q4_K weights of one row length and one K cut run as one launch; everything else as calls of
+// their own.  Same bits as n cml_matmul_f32 calls.
+int cml_matmul_f32_multi(const cml_weight *const *weights, int n_weights, const float *x_dev, float *const *outs_dev, void *workspace_dev,
+                         size_t workspace_bytes, cml_stream_t stream) {
+    if (n_weights < 0) return fail(CML_ERR_SHAPE, "negative weight count");
+    if (n_weights == 0) return CML_OK;
+    if (!weights || !outs_dev) return fail(CML_ERR_INVALID, "null pointer");
+    if (int rc = check_ready()) return rc;
+    for (int j = 0; j < n_weights; j++) {
+        if (!weights[j] || !outs_dev[j]) return fail(CML_ERR_INVALID, "null weight or output %d", j);
+        if (weights[j]->cols != weights[0]->cols)
+            return fail(CML_ERR_SHAPE, "weights 0 and %d read activations of %lld and %lld values", j, (long long)weights[0]->cols, (long long)weights[j]->cols);
+    }
+    if (!x_dev || !workspace_dev) return fail(CML_ERR_INVALID, "null pointer");
+    if (misaligned16(x_dev) || misaligned16(workspace_dev)) return fail(CML_ERR_INVALID, "activations and workspace must be 16-byte aligned");
+    const int fuse = env_int("CAMELID_HIP_FUSED_QUANT", 1);
+    int j = 0;
+    while (j < n_weights) {
+        // the longest run of up to four weights, starting here, that one launch serves
+        int served = 0;
+        if (weights[j]->fmt == CML_Q4_K && !q4k_lane_order() && (fuse == 2 || (fuse == 1 && weights[j]->nb <= 32))) {
+            for (int take = std::min(4, n_weights - j); take >= 2 && !served; take--) {
+                const int frc = launch_gemv_q4k_f32_multi(weights + j, take, x_dev, outs_dev + j, as_stream(stream));
+                if (frc == CML_OK) served = take;
+                else if (frc != -1) return frc;
+            }
+        }
+        if (served) {
+            g_runs.fetch_add(static_cast<uint64_t>(served), std::memory_order_relaxed);
+            j += served;
+            continue;
+        }
+        if (int rc = cml_matmul_f32(weights[j], x_dev, 1, outs_dev[j], workspace_dev, workspace_bytes, stream)) return rc;
+        j++;
+    }
+    return CML_OK;
+}
+
 // The same call for hosts that may not allocate (a stream under graph capture, a serving loop with
 // a fixed memory budget): the quantized activation is staged in the library's own static device
 // array instead of a caller workspace.  Nothing here allocates or frees, on the host or the device.

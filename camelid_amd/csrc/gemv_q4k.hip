@@ -90,6 +90,14 @@ struct Q4KArgs {
     int ksplit;        // waves sharing one row tile (1, 2, 4 or 8)
     int ksplit_log2;
     int tiles_per_wg;  // row tiles per workgroup; blockDim.x = 64 * ksplit * tiles_per_wg
+    // Multi launch (MULTI): up to four weights of one row length and one K cut against the same token, their workgroups
+    // laid end to end along grid.x; weight j serves workgroups [wg_end[j-1], wg_end[j]) and writes outm[j].
+    const uint8_t *wm[4];
+    float *outm[4];
+    int64_t stridem[4];
+    int rowsm[4];
+    int skipm[4];
+    int wg_end[4];
 };
 
 constexpr int kQ4KStageRegs = 4;  // activation chunks a thread holds in registers during the prologue
@@ -271,10 +279,27 @@ __device__ __forceinline__ void q4k_compute(const Q4KRegs<U> &r, const Q4KLane &
 //
 // PAIR (with PLAIN): grid.z = 2, blockIdx.z = 1 streams a second weight of the same shape against the same token
 // (gate and up of a dense FFN in one launch).
+//
+// MULTI (with PLAIN): up to four weights of one row length and one K cut but different row counts against the same
+// token (the q, k and v projections of an attention block), their workgroups end to end along grid.x.
 template <int NT, bool INTS, bool FUSEQ = false, int SPR = 1, bool WHOLE = false, bool PLAIN = false, bool LOADONLY = false, bool DIRECT = false,
-          int RING = 0, int NSTEPS = 0, bool ROUTE = false, bool PAIR = false>
-__global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
+          int RING = 0, int NSTEPS = 0, bool ROUTE = false, bool PAIR = false, bool MULTI = false>
+__global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a_in) {
     static_assert(!PAIR || (PLAIN && FUSEQ && NT == 1), "a plain pair: one f32 token against two weights of one shape (grid.z = 2)");
+    static_assert(!MULTI || (PLAIN && FUSEQ && NT == 1 && !PAIR && !LOADONLY), "a multi launch: one f32 token against several plain weights");
+    Q4KArgs a = a_in;
+    int bx = blockIdx.x;  // workgroup index within its weight
+    if constexpr (MULTI) {
+        // which weight this workgroup belongs to (wave-uniform selects: no indexed access to the argument block)
+        const int j = (bx >= a_in.wg_end[0]) + (bx >= a_in.wg_end[1]) + (bx >= a_in.wg_end[2]);
+        auto pick = [&](auto v0, auto v1, auto v2, auto v3) { return j == 0 ? v0 : (j == 1 ? v1 : (j == 2 ? v2 : v3)); };
+        a.w = pick(a_in.wm[0], a_in.wm[1], a_in.wm[2], a_in.wm[3]);
+        a.out = pick(a_in.outm[0], a_in.outm[1], a_in.outm[2], a_in.outm[3]);
+        a.sb_stride = pick(a_in.stridem[0], a_in.stridem[1], a_in.stridem[2], a_in.stridem[3]);
+        a.rows = pick(a_in.rowsm[0], a_in.rowsm[1], a_in.rowsm[2], a_in.rowsm[3]);
+        a.row_skip = pick(a_in.skipm[0], a_in.skipm[1], a_in.skipm[2], a_in.skipm[3]);
+        bx -= pick(0, a_in.wg_end[0], a_in.wg_end[1], a_in.wg_end[2]);
+    }
     static_assert(!ROUTE || DIRECT, "only the direct launch routes");
     static_assert(!FUSEQ || ((NT == 1 || (NT == 2 && PLAIN)) && !INTS),
                   "the fused quantizer serves single-token calls and plain two-token calls (contiguous f32 rows)");
@@ -336,7 +361,7 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int W = a.ksplit;  // 1, 2, 4 or 8
     const int tile_in_wg = wave >> a.ksplit_log2, kpart = wave & (W - 1);
-    const int tile = blockIdx.x * a.tiles_per_wg + tile_in_wg;
+    const int tile = bx * a.tiles_per_wg + tile_in_wg;
     const int s0 = (kpart * n_sb) >> a.ksplit_log2;  // == kpart * n_sb / W
     const int s1 = ((kpart + 1) * n_sb) >> a.ksplit_log2;
     const int g = lane / LPS, l = lane - g * LPS;
@@ -609,7 +634,7 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a) {
                 const int rr = i % RPW;
                 const int t = (i / RPW) % NT;
                 const int tw = i / (RPW * NT);
-                const int orow = (blockIdx.x * a.tiles_per_wg + tw) * RPW + rr - a.row_skip;
+                const int orow = (bx * a.tiles_per_wg + tw) * RPW + rr - a.row_skip;
                 if (orow < 0 || orow >= a.rows || t >= n_here) continue;
                 float v = part[((tw * W) * NT + t) * RPW + rr];
                 for (int k = 1; k < W; k++) v = v + part[((tw * W + k) * NT + t) * RPW + rr];
@@ -838,12 +863,15 @@ static bool q4k_ring(const Q4KArgs &ka, int ksplit, int spr = 2) {
 // 8.87 -> 8.44 us, the single-token one 6.89 -> 6.81); every other length runs the loop.
 // 8-row waves (SPR = 2, three slots) step two super-blocks at a time: rows / K parts of 3072, 3584
 // and 4096 values are 6, 7 and 8 steps; 16-row waves (SPR = 1, four slots) step one: 12, 14, 16.
-template <int NT, bool FUSEQ, int SPR, bool LOADONLY = false, bool PAIR = false>
+template <int NT, bool FUSEQ, int SPR, bool LOADONLY = false, bool PAIR = false, bool MULTI = false>
 static void launch_q4k_ring(const Q4KArgs &ka, int ksplit, dim3 grid, dim3 block, size_t lds, hipStream_t st) {
     constexpr int SLOTS = SPR == 2 ? 3 : 4;
     const int steps = ka.n_sb / (SPR * ksplit);
-#define CML_Q4K_RING(N_) hipLaunchKernelGGL((gemv_q4k_kernel<NT, false, FUSEQ, SPR, true, true, LOADONLY, false, SLOTS, N_, false, PAIR>), grid, block, lds, st, ka)
-    if constexpr (LOADONLY && SPR == 2) {
+#define CML_Q4K_RING(N_) hipLaunchKernelGGL((gemv_q4k_kernel<NT, false, FUSEQ, SPR, true, true, LOADONLY, false, SLOTS, N_, false, PAIR, MULTI>), grid, block, lds, st, ka)
+    if constexpr (MULTI) {
+        if (steps == 8) CML_Q4K_RING(8);
+        else CML_Q4K_RING(0);
+    } else if constexpr (LOADONLY && SPR == 2) {
         if (steps == 8) CML_Q4K_RING(8);
         else CML_Q4K_RING(0);
     } else if constexpr (LOADONLY) {
@@ -868,6 +896,7 @@ static void launch_q4k_ring(const Q4KArgs &ka, int ksplit, dim3 grid, dim3 block
     }
 #undef CML_Q4K_RING
     if constexpr (LOADONLY) CML_COUNT_LAUNCH("q4k.calibrate.ring");
+    else if constexpr (MULTI) CML_COUNT_LAUNCH("q4k.dot.ring.fused.multi");
     else if constexpr (PAIR) CML_COUNT_LAUNCH("q4k.dot.ring.fused.pair");
     else if constexpr (FUSEQ) CML_COUNT_LAUNCH("q4k.dot.ring.fused");
     else CML_COUNT_LAUNCH("q4k.dot.ring");
@@ -1108,6 +1137,68 @@ int launch_gemv_q4k_f32_pair(const cml_weight *w, const cml_weight *w2, const fl
     a.n_tokens = 1;
     a.n_groups = 1;
     return launch_q4k_f32(a, w2, out2, x, st);
+}
+
+// One f32 token against up to four Q4_K weights of one row length (any row counts) in ONE launch: the workgroups of the
+// weights lie end to end along grid.x, every workgroup quantizes the token once, and each weight keeps the K cut its
+// shape has in a call of its own -- so every output is that call's bits.  -1 = not a set this launch serves (formats,
+// row lengths or K cuts differ, rows too long to quantize in the kernel): the caller makes the calls one by one.
+int launch_gemv_q4k_f32_multi(const cml_weight *const *ws, int n, const float *x, float *const *outs, hipStream_t st) {
+    if (n < 2 || n > 4) return -1;
+    if (env_int("CAMELID_HIP_Q4K_GENERAL_ENTRY", 0) || !env_int("CAMELID_HIP_MULTI_LAUNCH", 1)) return -1;
+    const int n_sb = static_cast<int>(ws[0]->nb);
+    int ksplit = 0;
+    int64_t tiles16_all = 0;
+    for (int j = 0; j < n; j++) {
+        if (ws[j]->fmt != CML_Q4_K || ws[j]->nb != ws[0]->nb || ws[j]->rows <= 0 || ws[j]->planes.row_stride[0] >= (int64_t(1) << 31)) return -1;
+        const int ks = pick_shape(ws[j]->rows, n_sb).ksplit;
+        if (j && ks != ksplit) return -1;
+        ksplit = ks;
+        tiles16_all += (ws[j]->rows + ws[j]->row_skip + 15) / 16;
+    }
+    Q4KArgs ka{};
+    ka.n_sb = n_sb;
+    ka.x = x;
+    ka.ksplit = ksplit;
+    ka.ksplit_log2 = ksplit >= 8 ? 3 : (ksplit >= 4 ? 2 : (ksplit >= 2 ? 1 : 0));
+    ka.tiles_per_wg = std::max(1, 4 / ksplit);
+    const int waves = ksplit * ka.tiles_per_wg;
+    // 8-row waves (two lane groups per row) unless the launch is tall enough for 16-row ones; the choice changes no bit
+    const bool half_tiles = q4k_rows_per_wave(tiles16_all, ksplit, 1) == 8;
+    int wg = 0;
+    for (int j = 0; j < 4; j++) {
+        const cml_weight *w = ws[std::min(j, n - 1)];
+        ka.wm[j] = w->planes.p[0];
+        ka.outm[j] = outs[std::min(j, n - 1)];
+        ka.stridem[j] = w->planes.row_stride[0];
+        ka.rowsm[j] = static_cast<int>(w->rows);
+        ka.skipm[j] = w->row_skip;
+        if (j < n) {
+            const int64_t tiles16 = (w->rows + w->row_skip + 15) / 16;
+            const int64_t tiles = half_tiles ? 2 * tiles16 : tiles16;
+            wg += static_cast<int>((tiles + ka.tiles_per_wg - 1) / ka.tiles_per_wg);
+        }
+        ka.wg_end[j] = j < n ? wg : INT32_MAX;
+    }
+    ka.sb_stride = ka.stridem[0];  // the shape helpers below read these two; every weight passes the same checks
+    ka.rows = ka.rowsm[0];
+    const size_t lds = static_cast<size_t>(n_sb) * (256 + 32) + ((static_cast<size_t>(n_sb) + 3) & ~size_t(3)) * 4 + static_cast<size_t>(waves) * 16 * 4;
+    if (lds > 64 * 1024) return -1;
+    const dim3 grid(static_cast<unsigned>(wg)), block(64 * waves);
+    const bool whole = q4k_whole_buffers(ka, ksplit);
+    if (half_tiles && q4k_ring(ka, ksplit)) {
+        launch_q4k_ring<1, true, 2, false, false, true>(ka, ksplit, grid, block, lds, st);
+    } else if (!half_tiles && q4k_ring(ka, ksplit, 1)) {
+        launch_q4k_ring<1, true, 1, false, false, true>(ka, ksplit, grid, block, lds, st);
+    } else {
+#define CML_Q4K_MULTI(SPR_, WHOLE_) hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, SPR_, WHOLE_, true, false, false, 0, 0, false, false, true>), grid, block, lds, st, ka)
+        if (half_tiles) { if (whole) CML_Q4K_MULTI(2, true); else CML_Q4K_MULTI(2, false); }
+        else { if (whole) CML_Q4K_MULTI(1, true); else CML_Q4K_MULTI(1, false); }
+#undef CML_Q4K_MULTI
+        CML_COUNT_LAUNCH("q4k.dot.buffers.fused.multi");
+    }
+    CML_HIP_TRY(hipGetLastError());
+    return CML_OK;
 }
 
 int launch_gemv_q4k_f32(const cml_weight *w, const float *x, float *out, hipStream_t st, int n_tokens) {

@@ -1037,3 +1037,75 @@ def test_saturated_blocks_and_activations_keep_every_bit(name, fmt):
                 with G.env(**{lane_knob: 1}), G.engaged(r"\.lanes$"):
                     got = G.gpu_gemm(w, s[0], q[0]) if n == 1 else G.gpu_gemm(w, s[:n], q[:n])
                 assert G.same_bits(got.reshape(n, rows), want_lane), (name, rows, cols, n, "lane order")
+
+
+# ------------------------------------------------- several projections of one token, one launch ----
+
+def _multi(ws, x, stream=None):
+    """cml_matmul_f32_multi through the C ABI: host arrays of weight handles and output pointers."""
+    n = len(ws)
+    cols = ws[0].cols
+    ws_bytes = lib().cml_matmul_workspace_bytes(ws[0].fmt, cols, 1)
+    xd = DeviceBuffer.from_numpy(np.ascontiguousarray(x, np.float32).reshape(1, -1))
+    wsp = DeviceBuffer(max(ws_bytes, 16))
+    outs = [DeviceBuffer(max(w.rows * 4, 16)) for w in ws]
+    for o in outs:
+        o.fill(0xFF)
+    handles = (C.c_void_p * n)(*[w.handle for w in ws])
+    optrs = (C.c_void_p * n)(*[o.ptr for o in outs])
+    check(lib().cml_matmul_f32_multi(handles, n, xd.ptr, optrs, wsp.ptr, ws_bytes, stream), "cml_matmul_f32_multi")
+    check(lib().cml_stream_sync(stream))
+    return [o.to_numpy(np.float32, (w.rows,)) for o, w in zip(outs, ws)]
+
+
+@pytest.mark.parametrize("case", ["qkv_4096", "gate_up_14336", "ragged_2304", "three_3584", "mixed_cut", "five", "q6k", "bands"])
+def test_matmul_f32_multi_is_the_single_calls(case):
+    """cml_matmul_f32_multi: several weights that read one token (q | k | v of an attention block, gate | up of an FFN).
+    Runs of up to four Q4_K weights with one K cut go out as one launch -- the counters prove it -- and every
+    output is the bits of a cml_matmul_f32 call of its own; sets the one launch does not serve (different K cuts,
+    another format) fall back to single calls with the same results."""
+    fmt = B.CML_Q4_K
+    shapes, cols, one_launch = {
+        "qkv_4096": ([4096, 1024, 1024], 4096, 1),          # K cut 4 for all three: the two-buffer kernel
+        "gate_up_14336": ([14336, 14336], 4096, 1),         # no K cut: the ring kernel
+        "ragged_2304": ([200, 77, 530, 16], 2304, 1),       # ragged row counts, 9 super-blocks
+        "three_3584": ([1000, 333, 4100], 3584, 1),
+        "mixed_cut": ([14336, 4096], 4096, 0),              # K cuts 1 and 4: two calls
+        "five": ([512, 256, 256, 128, 640], 2048, 2),       # four in one launch, the fifth alone
+        "q6k": ([300, 200], 1024, 0),
+        "bands": ([700, 300, 650], 4096, 1),
+    }[case]
+    if case == "q6k":
+        fmt = B.CML_Q6_K
+    rng = np.random.default_rng(sum(shapes) + cols)
+    ws = [Weight.upload(fmt, r, cols, G.synth_weight(fmt, r, cols, seed=r + cols + j)) for j, r in enumerate(shapes)]
+    if case == "bands":   # views that start inside a 16-row tile
+        ws = [ws[0].slice(5, 600), ws[1].slice(0, 300), ws[2].slice(17, 601)]
+    x = rng.standard_normal(cols).astype(np.float32)
+    x[:256] = 0.0
+    G.say(f"multi {case}: single calls")
+    want = [G.gpu_matmul_f32(w, x) for w in ws]
+    G.say(f"multi {case}: one call")
+    if case == "q6k":
+        proof = G.engaged(r"^q6k\.dot\.", none=(r"multi",))
+    elif one_launch == 0:
+        proof = G.engaged(r"^q4k\.dot\.", none=(r"multi",))
+    else:
+        proof = G.engaged(r"^q4k\.dot\.(ring|buffers)\.fused\.multi$")
+    before = G.launch_counts()
+    with proof:
+        got = _multi(ws, x)
+    after = G.launch_counts()
+    launches = sum(after.values()) - sum(before.values())
+    assert launches == {"five": 2}.get(case, 1 if one_launch else launches), (case, launches)
+    for j, (g, wnt) in enumerate(zip(got, want)):
+        assert G.same_bits(g, wnt), (case, j)
+    with G.env(CAMELID_HIP_MULTI_LAUNCH=0), G.engaged(none=(r"multi",)):
+        got = _multi(ws, x)
+    for j, (g, wnt) in enumerate(zip(got, want)):
+        assert G.same_bits(g, wnt), (case, j, "single calls inside")
+    if fmt == B.CML_Q4_K:
+        with G.env(CAMELID_HIP_EXACT_ORDER="1"):
+            got = _multi(ws, x)
+            for j, (g, w) in enumerate(zip(got, ws)):
+                assert G.same_bits(g, G.gpu_matmul_f32(w, x)), (case, j, "exact order")
