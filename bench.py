@@ -133,6 +133,19 @@ class EagerSteps:
         self.fn, self.count = fn, count
 
 
+def launch_report() -> dict:
+    """{kernel-family counter: launches so far} (cml_kernel_launch_report)."""
+    L = lib()
+    need = int(L.cml_kernel_launch_report(None, 0))
+    buf = C.create_string_buffer(need + 256)
+    L.cml_kernel_launch_report(buf, len(buf))
+    out = {}
+    for line in buf.value.decode().splitlines():
+        name, _, count = line.rpartition(" ")
+        out[name] = out.get(name, 0) + int(count)
+    return out
+
+
 def capture(stream, fn, count: int):
     """Capture `count` calls of fn(i) on `stream` into one replayable graph."""
     if EAGER:
@@ -769,8 +782,13 @@ def main() -> int:
     # Decode at the usual hidden sizes runs quantize + matvec as ONE kernel (Q4_K up to 4096 values
     # per row, Q8_0 / Q4_0 up to 8192 values and 32768 rows): there the step itself is the dominant kernel's launch.
     # Elsewhere it is the matvec on quantized activations.
-    fused = n == 1 and os.environ.get("CAMELID_HIP_FUSED_QUANT", "1") != "0" and (
-        (fmt_name == "Q4_K" and cols <= 4096) or (fmt_name in ("Q8_0", "Q4_0") and cols <= 8192 and rows <= 32768))
+    # The library's launch counters say which it is: one launch per step = the step is the dominant kernel's launch.
+    launches_before, report_before = L.cml_kernel_launches(b""), launch_report()
+    step(0)
+    launches_per_step = int(L.cml_kernel_launches(b"") - launches_before)
+    report_after = launch_report()
+    kernels_of_step = sorted(k for k, v in report_after.items() if v > report_before.get(k, 0))
+    fused = n == 1 and launches_per_step == 1
 
     def gemv_cold(i):
         if fused:
@@ -855,7 +873,8 @@ def main() -> int:
         "config": {"workload": args.config, "format": fmt_name, "rows": rows, "cols": cols, "tokens": n,
                    "algorithmic_bytes_per_call": alg_bytes, "weight_copies_rotated": copies,
                    "step": "quantize activation + fused dequantize-matvec (cml_matmul_f32), graph replay",
-                   "launches_per_step": 1 if fused else 2,
+                   "launches_per_step": launches_per_step,
+                   "kernels": kernels_of_step,
                    "replays": replays,
                    "timing": f"a graph of {K} steps replayed untimed for {SETTLE_MS:.0f} ms of GPU time, then {replays} replays timed back "
                              "to back between their own HIP events; ms_per_step = (median replay - launch constant) / K, the "

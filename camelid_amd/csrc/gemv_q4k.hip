@@ -764,6 +764,126 @@ __global__ __launch_bounds__(512) void gemv_q4k_cu_kernel(const uint8_t *__restr
     }
 }
 
+// The same launch for a weight whose shape the policy cuts K for (few row tiles, long rows: the FFN down projection,
+// 4096 x 14336): a workgroup's eight waves are 8 / KS half tiles x KS parts of NSTEPS steps each, the workgroup
+// quantizes the WHOLE row once (56 super-blocks: 28 pairs over the eight waves, four passes of the 32-lane quantizer
+// with every f32 request out before the first weight request), every wave then walks its own part, and the KS partial
+// chains of a row are added left to right through LDS -- the association of gemv_q4k_kernel under the same K cut, so
+// the same bits.  The two-launch form (a quantizing launch, then the matvec) takes 9.1 us per step at 4096 x 14336 for
+// a 7.1 us matvec; the four-wave kernel with the quantizer inside took 10.0 (512 workgroups each quantizing the row).
+template <int KS, int NSTEPS>
+__global__ __launch_bounds__(512) void gemv_q4k_cu_kcut_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ out,
+                                                               const float *__restrict__ residual, uint32_t sb_stride, int rows, int row_skip,
+                                                               int tiles16) {
+    constexpr int WAVES = 8, TPW = WAVES / KS;   // half tiles per workgroup
+    constexpr int NSB = KS * 2 * NSTEPS;         // super-blocks per row
+    constexpr int PAIRS = NSB / 2, PASSES = (PAIRS + WAVES - 1) / WAVES;
+    constexpr int NB = 3, PRE = 2;
+    static_assert((KS == 2 || KS == 4) && NSTEPS >= NB, "K parts of at least one full ring");
+    using Regs = Q4KRegs<1>;
+    __shared__ __attribute__((aligned(16))) int8_t ys[NSB * 256];
+    __shared__ int bsum[NSB * 8];
+    __shared__ float yds[NSB];
+    __shared__ float part[WAVES * 8];
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+
+    // the f32 activation: pass p of wave w quantizes the super-block pair w + 8 p, a half wave per super-block
+    const int half = lane >> 5, ql = lane & 31;
+    float4 xv[PASSES][2];
+#pragma unroll
+    for (int p = 0; p < PASSES; p++) {
+        const int sbk = 2 * min(wave + WAVES * p, PAIRS - 1) + half;
+        const float4 *x4 = reinterpret_cast<const float4 *>(x) + sbk * 64 + ql * 2;
+        xv[p][0] = x4[0];
+        xv[p][1] = x4[1];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();  // execution only: every activation request of the workgroup is out
+    __builtin_amdgcn_sched_barrier(0);
+
+    const int tile_in_wg = wave / KS, kpart = wave - tile_in_wg * KS;
+    const int tile = blockIdx.x * TPW + tile_in_wg;  // 8-row half tile
+    const int s0 = kpart * 2 * NSTEPS;               // first super-block of this wave's part
+    const int g = lane / LPS, l = lane - g * LPS;
+    const int r = g >> 1, h = g & 1;
+    const int rl = (tile & 1) * 8 + r;
+    const uint8_t *wtile = w + static_cast<int64_t>(min(tile >> 1, tiles16 - 1)) * kQ4KChunk;
+    const uint32_t hoff = static_cast<uint32_t>(h) * sb_stride;
+    const uint32_t hdr_off = hoff + rl * 16, q_off = hoff + (rl * LPS + l) * 16;
+    Regs ring[NB];
+    auto request = [&](Regs &b, int step) __attribute__((always_inline)) {
+        q4k_load_whole<1, 2>(b, wtile + static_cast<int64_t>(s0 + 2 * step) * sb_stride, sb_stride, hdr_off, q_off);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+#pragma unroll
+    for (int k = 0; k < PRE; k++) request(ring[k], k);
+
+    // every wave runs every pass (a wave without a pair of its own in the last pass redoes the last pair and stores
+    // nothing): the f32 loads above are then used unconditionally and stay ahead of the weight requests
+#pragma unroll
+    for (int p = 0; p < PASSES; p++) {
+        const int pair = wave + WAVES * p;
+        const bool mine = WAVES * (p + 1) <= PAIRS || pair < PAIRS;
+        const int sbk = 2 * min(pair, PAIRS - 1) + half;
+        float dv;
+        int bs;
+        const uint2 packed = q8k_quantize_row32(xv[p], lane, dv, bs);
+        if (mine) {
+            reinterpret_cast<uint2 *>(ys)[sbk * 32 + ql] = packed;
+            if ((ql & 3) == 3) bsum[sbk * 8 + (ql >> 2)] = bs;
+            if (ql == 0) yds[sbk] = dv;
+        }
+    }
+    __syncthreads();
+
+    Q4KLane ln;
+    ln.c = l;
+    ln.sh = (l & 1) * 16;
+    ln.upper = l >= 2;
+    float acc[1] = {0.0f};
+    auto compute = [&](const Regs &b, int step) __attribute__((always_inline)) {
+        q4k_compute<1, false, 1, 2, true, false>(b, ln, s0 + 2 * step + h, NSB, ys, bsum, yds, NSB, acc, nullptr);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+#pragma unroll
+    for (int j = PRE; j < NB; j++) request(ring[j], j);
+#pragma unroll
+    for (int i = 0; i < NSTEPS; i++) {
+        compute(ring[i % NB], i);
+        if (i + NB < NSTEPS) request(ring[i % NB], i + NB);
+    }
+    if (l == LPS - 1 && h == 1) part[wave * 8 + r] = acc[0];
+    __syncthreads();
+    if (tid < TPW * 8) {
+        const int tw = tid >> 3, rr = tid & 7;
+        const int orow = (blockIdx.x * TPW + tw) * 8 + rr - row_skip;
+        if (orow >= 0 && orow < rows) {
+            float v = part[(tw * KS) * 8 + rr];
+#pragma unroll
+            for (int k = 1; k < KS; k++) v = v + part[(tw * KS + k) * 8 + rr];
+            if (residual) v = v + residual[orow];
+            out[orow] = v;
+        }
+    }
+}
+
+// The K-cut form serves rows of 14336 values cut four ways (seven steps per part).
+static bool q4k_cu_kcut_serves(const Q4KArgs &ka, int ksplit) {
+    return ksplit == 4 && ka.n_sb == 56 && ka.sb_stride < (int64_t(1) << 31) && env_int("CAMELID_HIP_Q4K_CU", 1) != 0 &&
+           !env_int("CAMELID_HIP_Q4K_CLAMPED_LOADS", 0) && env_int("CAMELID_HIP_Q4K_RING", 1) != 0;
+}
+
+static int launch_q4k_cu_kcut(const Q4KArgs &ka, hipStream_t st) {
+    if (!ka.x) return fail(CML_ERR_INVALID, "null activation");
+    const int tiles16 = (ka.rows + ka.row_skip + 15) / 16;
+    const dim3 grid(static_cast<unsigned>((2 * tiles16 + 1) / 2)), block(512);  // two half tiles per workgroup
+    hipLaunchKernelGGL((gemv_q4k_cu_kcut_kernel<4, 7>), grid, block, 0, st, ka.w, ka.x, ka.out, ka.residual, static_cast<uint32_t>(ka.sb_stride), ka.rows,
+                       ka.row_skip, tiles16);
+    CML_COUNT_LAUNCH("q4k.dot.wg8.kcut.fused");
+    return CML_OK;
+}
+
 // Whether the launch above serves this call: rows of 4096 values, no K cut (the shape policy gives
 // that from 12288 rows on, i.e. at least 192 eight-wave workgroups), a stride the 32-bit lane
 // offsets can hold.  CAMELID_HIP_Q4K_CU=0 keeps the four-wave launch.
@@ -840,6 +960,18 @@ static int q4k_rows_per_wave(int64_t tiles16, int ksplit, int64_t slots) {
         return std::ceil(per_cu) / per_cu;
     };
     return imbalance(2 * waves16) + 0.1 < imbalance(waves16) ? 8 : 16;
+}
+
+// A single f32 token on this weight runs as ONE launch although its rows are longer than the in-kernel quantizer of
+// the four-wave launches takes (the caller's decision between one launch and quantize-then-matvec).
+bool gemv_q4k_long_rows_fuse(const cml_weight *w) {
+    if (w->fmt != CML_Q4_K || w->rows <= 0) return false;
+    Q4KArgs ka{};
+    ka.n_sb = static_cast<int>(w->nb);
+    ka.sb_stride = w->planes.row_stride[0];
+    const int64_t tiles16 = (w->rows + w->row_skip + 15) / 16;
+    const int ks = pick_shape(w->rows, ka.n_sb).ksplit;
+    return q4k_cu_kcut_serves(ka, ks) && q4k_rows_per_wave(tiles16, ks, 1) == 8 && !env_int("CAMELID_HIP_Q4K_GENERAL_ENTRY", 0);
 }
 
 // Every K part a whole number of 4-super-block buffers and a stride of less than 2 GiB: the
@@ -1069,6 +1201,8 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
             launch_q4k_ring<1, true, 2, false, true>(ka, shape.ksplit, grid, block, lds, st);  // a plain pair: grid.z = 2
         } else if (!grouped && w2 && !half_tiles && q4k_ring(ka, shape.ksplit, 1) && !env_int("CAMELID_HIP_Q4K_GENERAL_ENTRY", 0)) {
             launch_q4k_ring<1, true, 1, false, true>(ka, shape.ksplit, grid, block, lds, st);
+        } else if (half_tiles && plain && !two && q4k_cu_kcut_serves(ka, shape.ksplit)) {
+            if (int rc = launch_q4k_cu_kcut(ka, st)) return rc;  // rows of 14336 values cut four ways: eight-wave workgroups, the row quantized once each
         } else if (half_tiles && ring && plain && q4k_cu_serves(ka, shape.ksplit)) {
             if (int rc = launch_q4k_cu(ka, 0, st)) return rc;  // rows of 4096 values, no K cut: eight-wave workgroups
         } else if (half_tiles && ring && plain) {
