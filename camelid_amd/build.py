@@ -49,12 +49,8 @@ FLAGS = [
 ]
 
 
-# Per-file flags.  gemv_q4k.hip: kernels whose arguments are plain scalars get them preloaded into
-# SGPRs by the command processor (no scalar-load round trip before a wave's first address); kernels
-# that take a struct by value are unaffected.
-FILE_FLAGS = {
-    "gemv_q4k.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
-}
+# Per-file flags (none at present).
+FILE_FLAGS: dict = {}
 
 
 def _compile(src: str, extra: list[str]) -> str:

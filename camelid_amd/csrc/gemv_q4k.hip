@@ -662,9 +662,11 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a_in) {
 //   * the quantizer with a 32-lane half wave per super-block: the eight waves quantize the sixteen
 //     super-blocks of a row in ONE pass, eight values per lane, about half the instructions per wave
 //     of the 16-lane form (q8k_quantize_row32);
-//   * scalar kernel arguments (twelve dwords, preloaded into SGPRs where the firmware does that)
-//     and statically sized LDS: no scalar-load round trip and no size arithmetic before the first
-//     address.
+//   * a 48-byte argument block and statically sized LDS: one scalar load and no size arithmetic
+//     before the first address.  (Plain scalar arguments preloaded into SGPRs by the command
+//     processor, -amdgpu-kernarg-preload-count, measured the same time to within noise, and
+//     rocprofv3 could not follow graph replays of that form of the kernel; the argument block is a
+//     struct by value like every other kernel's here.)
 // Measured on 14336 x 4096, same box, same run: 6.84 -> 6.65 us.  With the activation taken out
 // altogether (no f32 loads, no quantizer, no barriers: ABLATE = 1) the launch takes the same time,
 // so nothing is left in the prologue; without the output store (4) 6.30; without arithmetic and
@@ -673,10 +675,24 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(Q4KArgs a_in) {
 //
 // ABLATE (timing experiments, reachable only through cml_calibrate_matvec_ablation; results are
 // wrong): 1 = no activation, 2 = no arithmetic, 4 = no store.
+struct Q4KCuArgs {
+    const uint8_t *w;       // tiled layout, as Q4KArgs::w
+    const float *x;         // the f32 token
+    float *out;             // [rows]
+    const float *residual;  // [rows] or null
+    uint32_t sb_stride;     // bytes between consecutive super-blocks of one tile (below 2 GiB)
+    int rows, row_skip;     // as Q4KArgs
+    int tiles16;            // 16-row layout tiles that hold the rows
+};
+
 template <int NSTEPS, int ABLATE = 0>
-__global__ __launch_bounds__(512) void gemv_q4k_cu_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ out,
-                                                          const float *__restrict__ residual, uint32_t sb_stride, int rows, int row_skip,
-                                                          int tiles16) {
+__global__ __launch_bounds__(512) void gemv_q4k_cu_kernel(Q4KCuArgs a) {
+    const uint8_t *__restrict__ w = a.w;
+    const float *__restrict__ x = a.x;
+    float *__restrict__ out = a.out;
+    const float *__restrict__ residual = a.residual;
+    const uint32_t sb_stride = a.sb_stride;
+    const int rows = a.rows, row_skip = a.row_skip, tiles16 = a.tiles16;
     constexpr int WAVES = 8;
     constexpr int NSB = 2 * NSTEPS;  // super-blocks per row
     constexpr int NB = 3, PRE = 2;   // ring slots; slots requested before the quantizer
@@ -772,9 +788,13 @@ __global__ __launch_bounds__(512) void gemv_q4k_cu_kernel(const uint8_t *__restr
 // the same bits.  The two-launch form (a quantizing launch, then the matvec) takes 9.1 us per step at 4096 x 14336 for
 // a 7.1 us matvec; the four-wave kernel with the quantizer inside took 10.0 (512 workgroups each quantizing the row).
 template <int KS, int NSTEPS>
-__global__ __launch_bounds__(512) void gemv_q4k_cu_kcut_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ out,
-                                                               const float *__restrict__ residual, uint32_t sb_stride, int rows, int row_skip,
-                                                               int tiles16) {
+__global__ __launch_bounds__(512) void gemv_q4k_cu_kcut_kernel(Q4KCuArgs a) {
+    const uint8_t *__restrict__ w = a.w;
+    const float *__restrict__ x = a.x;
+    float *__restrict__ out = a.out;
+    const float *__restrict__ residual = a.residual;
+    const uint32_t sb_stride = a.sb_stride;
+    const int rows = a.rows, row_skip = a.row_skip, tiles16 = a.tiles16;
     constexpr int WAVES = 8, TPW = WAVES / KS;   // half tiles per workgroup
     constexpr int NSB = KS * 2 * NSTEPS;         // super-blocks per row
     constexpr int PAIRS = NSB / 2, PASSES = (PAIRS + WAVES - 1) / WAVES;
@@ -878,8 +898,8 @@ static int launch_q4k_cu_kcut(const Q4KArgs &ka, hipStream_t st) {
     if (!ka.x) return fail(CML_ERR_INVALID, "null activation");
     const int tiles16 = (ka.rows + ka.row_skip + 15) / 16;
     const dim3 grid(static_cast<unsigned>((2 * tiles16 + 1) / 2)), block(512);  // two half tiles per workgroup
-    hipLaunchKernelGGL((gemv_q4k_cu_kcut_kernel<4, 7>), grid, block, 0, st, ka.w, ka.x, ka.out, ka.residual, static_cast<uint32_t>(ka.sb_stride), ka.rows,
-                       ka.row_skip, tiles16);
+    const Q4KCuArgs ca{ka.w, ka.x, ka.out, ka.residual, static_cast<uint32_t>(ka.sb_stride), ka.rows, ka.row_skip, tiles16};
+    hipLaunchKernelGGL((gemv_q4k_cu_kcut_kernel<4, 7>), grid, block, 0, st, ca);
     CML_COUNT_LAUNCH("q4k.dot.wg8.kcut.fused");
     return CML_OK;
 }
@@ -896,8 +916,8 @@ static int launch_q4k_cu(const Q4KArgs &ka, int ablate, hipStream_t st) {
     if (!(ablate & 1) && !ka.x) return fail(CML_ERR_INVALID, "null activation");  // every variant but the one without the activation reads it
     const int tiles16 = (ka.rows + ka.row_skip + 15) / 16;
     const dim3 grid(static_cast<unsigned>((2 * tiles16 + 7) / 8)), block(512);
-    const uint32_t stride = static_cast<uint32_t>(ka.sb_stride);
-#define CML_Q4K_CU(A_) hipLaunchKernelGGL((gemv_q4k_cu_kernel<8, A_>), grid, block, 0, st, ka.w, ka.x, ka.out, ka.residual, stride, ka.rows, ka.row_skip, tiles16)
+    const Q4KCuArgs ca{ka.w, ka.x, ka.out, ka.residual, static_cast<uint32_t>(ka.sb_stride), ka.rows, ka.row_skip, tiles16};
+#define CML_Q4K_CU(A_) hipLaunchKernelGGL((gemv_q4k_cu_kernel<8, A_>), grid, block, 0, st, ca)
     switch (ablate) {
         case 0: CML_Q4K_CU(0); break;
         case 1: CML_Q4K_CU(1); break;
