@@ -556,7 +556,17 @@ static int moe_ffn_impl(const cml_weight *gate, const cml_weight *up, const cml_
             a.route_idx = ws.route_idx;
             a.route_w = ws.route_w;
         }
-        if (int rc = launch_gemv_q4k_f32_grouped_pair(a, up, up ? ws.u : nullptr, x_dev, st)) return rc;
+        int rc = launch_gemv_q4k_f32_grouped_pair(a, up, up ? ws.u : nullptr, x_dev, st);
+        if (rc == CML_ERR_UNSUPPORTED && route_in_launch) {
+            // the launch decided against routing inside it (its own shape checks are the authority): route in a
+            // launch of its own and run the gate|up launch on the routed slots
+            clear_error();
+            route_in_launch = false;
+            a.route_logits = nullptr;
+            if (int rrc = cml_moe_route_top_k(logits_dev, n_tokens, n_experts, k, ws.route_idx, ws.route_w, stream)) return rrc;
+            rc = launch_gemv_q4k_f32_grouped_pair(a, up, up ? ws.u : nullptr, x_dev, st);
+        }
+        if (rc) return rc;
         a.route_logits = nullptr;
     } else if (fused_gate_up) {
         if (int rc = launch_expert_matmul(a, st)) return rc;

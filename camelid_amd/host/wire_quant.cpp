@@ -396,15 +396,15 @@ std::vector<float> WireQuant::dequantize_elements(size_t start, size_t len) cons
         const size_t bv = values_per_block(format_), bb = bytes_per_block(format_);
         const size_t b0 = start / bv, b1 = (start + len + bv - 1) / bv;
         ensure_device();
-        cml_weight *tmp = nullptr;
+        cml_weight *raw = nullptr;
         dev(cml_weight_upload(ggml_type_id(format_), static_cast<int64_t>(b1 - b0), static_cast<int64_t>(bv), wire_.data() + b0 * bb,
-                              (b1 - b0) * bb, &tmp),
+                              (b1 - b0) * bb, &raw),
             "cml_weight_upload");
+        // freed on every way out of this block, an exception from reserve() or dev() included
+        const std::unique_ptr<cml_weight, void (*)(cml_weight *)> tmp(raw, cml_weight_free);
         float *od = static_cast<float *>(out_.reserve((b1 - b0) * bv * sizeof(float)));
-        const int rc = cml_dequantize(tmp, od, nullptr);
-        const int rc2 = rc ? rc : cml_stream_sync(nullptr);
-        cml_weight_free(tmp);
-        dev(rc2, "cml_dequantize");
+        dev(cml_dequantize(tmp.get(), od, nullptr), "cml_dequantize");
+        dev(cml_stream_sync(nullptr), "cml_stream_sync");
         dev(cml_memcpy_d2h(out.data(), od + (start - b0 * bv), len * sizeof(float), nullptr), "cml_memcpy_d2h");
         return out;
     }

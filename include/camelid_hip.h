@@ -28,10 +28,11 @@
  *   - threads: the host-slice seam (cml_try_*) serialises its callers on one
  *     process-wide lock, as the reference's backend does (src/cuda.rs:691-699).
  *     The resident entry points (quantize / gemv / gemm / matmul / moe / producers)
- *     take no lock: they only enqueue kernels on the caller's stream and keep no
- *     shared mutable state (cml_matmul_f32_static excepted, see there), so any
- *     number of threads may call them, each on its own stream, on weights that
- *     nobody frees meanwhile.  cml_init / cml_shutdown / cml_reload_env must not
+ *     take no lock: they only enqueue kernels on the caller's stream; what they
+ *     share is atomic (the launch counters, and one flag per kernel that needs
+ *     more than 64 KB of LDS, set the first time it is launched) -- and the static
+ *     array of cml_matmul_f32_static, see there -- so any number of threads may
+ *     call them, each on its own stream, on weights that nobody frees meanwhile.  cml_init / cml_shutdown / cml_reload_env must not
  *     run concurrently with anything else;
  *   - tuning knobs (environment variables named CAMELID_HIP_*) are read once, by
  *     cml_init, the way the reference reads its CAMELID_* knobs once per process
@@ -314,9 +315,11 @@ int cml_matmul_f32(const cml_weight *w, const float *x_dev, int64_t n_tokens, fl
  * src/gemma4_runtime.rs:1288-1340; gate / up at :5591-5592 and :5965-5966).
  * Two weights of one shape run as ONE launch (the token quantized once per
  * workgroup, both weights streamed) for Q4_K rows of up to 8192 values and for
- * Q8_0 / Q4_0 matrices of 4096 to 32768 rows of up to 4096 values; every other
- * pair is two cml_matmul_f32 calls.  Same bits as the two calls.  workspace as
- * for cml_matmul_f32 with n_tokens = 1. */
+ * Q8_0 / Q4_0 matrices of 4096 to 32768 rows of up to 4096 values where the
+ * single call runs eight-wave workgroups with 16 lanes per row (the launcher
+ * decides: not, for one, Q8_0 rows of 4096 values on 14336 rows or more, which
+ * run sixteen-wave workgroups); every other pair is two cml_matmul_f32 calls.
+ * Same bits as the two calls.  workspace as for cml_matmul_f32 with n_tokens = 1. */
 int cml_matmul_f32_pair(const cml_weight *w_a, const cml_weight *w_b, const float *x_dev,
                         float *out_a_dev, float *out_b_dev, void *workspace_dev,
                         size_t workspace_bytes, cml_stream_t stream);

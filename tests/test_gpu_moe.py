@@ -171,6 +171,55 @@ def test_moe_ffn_logits_is_route_then_ffn(E, k, hidden, ff, T):
     assert G.same_bits(gpu_moe_logits(wg, wu, wd, E, k, logits, x), want)
 
 
+def _stacked_from_one(base, E, block_bytes, scale0):
+    """E experts from one expert's wire bytes, made distinct cheaply: expert e carries its own f16 super-block
+    scale d in every block (the first two bytes of a Q4_K block), so which expert served a slot shows in every output."""
+    out = np.tile(base, E).reshape(E, -1, block_bytes)
+    for e in range(E):
+        out[e, :, 0:2] = np.frombuffer(np.float16(scale0 * (1.0 + 0.03 * e)).tobytes(), np.uint8)
+    return out.reshape(-1)
+
+
+# The gate|up launch routes the token itself where it runs 8-row waves, which the launch policy picks while the routed slots
+# of both projections stay below about 4.5 sixteen-row waves per SIMD quarter (top-2 and top-3 at these sizes); with top-4
+# and top-8 it runs 16-row waves, whose launch has no routing variant, and a routing launch goes first.
+@pytest.mark.parametrize("E,k,ff,in_launch", [(72, 3, 12288, True), (100, 2, 14336, True), (8, 3, 12288, True), (72, 4, 12288, False),
+                                              (100, 8, 12800, False)])
+def test_moe_ffn_logits_routes_inside_the_launch_like_the_routing_launch(E, k, ff, in_launch):
+    """One token on Q4_K experts whose gate / up bands take no K cut (12288 rows of 4096 values): the gate|up
+    launch routes the token itself (every wave, from the logits).  More than 64 experts (both halves of a lane's
+    pair), top-3 / 4 / 8, logits that tie, infinities and NaNs: the bits of the routing launch followed by the
+    expert lane (CAMELID_HIP_MOE_FOLD_ROUTE=0), and the counters say which ran."""
+    hidden = 4096
+    g1, u1, d1 = _experts(1, hidden, ff, 360 + E + k)
+    gate, up, down = (_stacked_from_one(t, E, 144, 0.004) for t in (g1, u1, d1))
+    wg = Weight.upload(B.CML_Q4_K, E * ff, hidden, gate)
+    wu = Weight.upload(B.CML_Q4_K, E * ff, hidden, up)
+    wd = Weight.upload(B.CML_Q4_K, E * hidden, ff, down)
+    del gate, up, down
+    rng = np.random.default_rng(361 + E)
+    x = rng.standard_normal((1, hidden)).astype(np.float32)
+    base = rng.standard_normal((1, E)).astype(np.float32)
+    tied = base.copy()
+    tied[0, E // 2:] = tied[0, 1]            # many experts tie, across lane 64 where there are that many
+    tied[0, 3] = tied[0, 1]
+    odd = base.copy()
+    odd[0, 0], odd[0, E - 1], odd[0, E // 2] = np.nan, np.inf, -np.inf
+    outs = []
+    for i, logits in enumerate((base, tied, odd, np.full((1, E), 0.25, np.float32))):
+        G.say(f"moe ffn routed in the launch E={E} k={k} case={i}")
+        proof = (G.engaged(r"^q4k\.dot\.direct\.ring\.route$", none=(r"^moe\.route",)) if in_launch else
+                 G.engaged(r"^moe\.route", r"^q4k\.dot\.direct", none=(r"\.route$",)))
+        with proof:
+            got = gpu_moe_logits(wg, wu, wd, E, k, logits, x)
+        with G.env(CAMELID_HIP_MOE_FOLD_ROUTE="0"), G.engaged(r"^moe\.route", r"^q4k\.dot\.direct", none=(r"\.route$",)):
+            want = gpu_moe_logits(wg, wu, wd, E, k, logits, x)
+        assert G.same_bits(got, want), (E, k, i)
+        assert G.same_bits(got, gpu_moe(wg, wu, wd, E, k, *gpu_route(logits, k)[:2], x)), (E, k, i)
+        outs.append(got)
+    assert not G.same_bits(outs[0], outs[3])   # the routing does change the result: the experts differ
+
+
 def test_moe_ffn_logits_rejects_bad_arguments():
     E, k, hidden, ff = 4, 2, 256, 256
     gate, up, down = _experts(E, hidden, ff, 350)
