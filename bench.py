@@ -34,18 +34,20 @@ from camelid_amd.binding import DeviceBuffer, Weight, check, lib  # noqa: E402
 HBM_PEAK_GBS = 8000.0    # MI355X published HBM3E bandwidth
 INT8_PEAK_TOPS = 5000.0  # MI355X published dense int8 matrix-core rate
 
-# HBM bytes per launch of the dominant kernel, from hardware counters: FETCH_SIZE + WRITE_SIZE of
-# `rocprofv3 --pmc` runs of this file, each scaled by what the same counter reads for
-# `--calibrate-copy` (a plain copy of known size).  Counters cannot be read from inside the timed
-# run, so the figures measured for the committed kernels are carried here; null where not measured.
-MEASURED_TRAFFIC_BYTES: dict = {
-    # profiles/hbm_traffic_fetch_write_size.txt (copy yardstick: FETCH_SIZE x 2.000, WRITE_SIZE x 1.000)
-    "q4k_14336x4096_n1": 33383424,       # 1.008 x algorithmic
-    "q4k_14336x4096_n16": 34694144,      # 1.014 x
-    "q4k_14336x4096_n64": 39150592,      # 1.037 x
-    "q6k_128256x3072_n1": 323916630,     # 1.001 x
-    "q4_0_128256x3072_n16": 252016327,   # 1.087 x
-    "q6k_128256x3072_n16": 356013774,    # 1.074 x
+# HBM bytes per launch of the dominant kernel, from hardware counters: FETCH_SIZE + WRITE_SIZE of `rocprofv3 --pmc`
+# runs of this file, each scaled by what the same counter reads for `--calibrate-copy` (a plain copy of known size).
+# Counters cannot be read from inside the timed run, so a line carries the reading together with where it was taken
+# (`roofline.traffic_source`: the summary under profiles/ and the kernel symbol it was read for) -- a reading of another
+# kernel, or none, shows as such instead of posing as this run's.  Configurations without a reading report null.
+TRAFFIC_SOURCE = "profiles/hbm_traffic_fetch_write_size.txt"
+TRAFFIC_READINGS: dict = {
+    # config -> (bytes per launch, kernel-family counter the step must have fired for the reading to apply, kernel symbol)
+    "q4k_14336x4096_n1": (33338368, "q4k.dot.wg8.fused", "gemv_q4k_cu_kernel<8, 0>"),            # 1.007 x algorithmic
+    "q4k_14336x4096_n16": (34694144, "q4k.mfma.pair", "gemm_q4k_mfma_pair_kernel<false>"),       # 1.014 x
+    "q4k_14336x4096_n64": (39150592, "q4k.mfma.tile.g4t1", "gemm_q4k_mfma_kernel<4, 1, ...>"),   # 1.037 x
+    "q6k_128256x3072_n1": (323916630, "q6k.dot.deep", "gemv_q6k_kernel<1, false, false, 4>"),    # 1.001 x
+    "q4_0_128256x3072_n16": (252016327, "q4_0.mfma.tile", "gemm_b32_mfma_kernel<2, ...>"),       # 1.096 x
+    "q6k_128256x3072_n16": (356013774, "q6k.mfma.tile", "gemm_q6k_mfma_kernel<...>"),            # 1.074 x
 }
 
 # name -> (format, rows, cols, tokens): BASELINE.json's configurations.
@@ -859,6 +861,15 @@ def main() -> int:
         return 4
 
     achieved = alg_bytes / (kern_ms * 1e-3) / 1e9
+    # the counter reading for this configuration, if one was taken and this run launched the kernel it was taken for
+    traffic_bytes, traffic_source = None, None
+    reading = TRAFFIC_READINGS.get(args.config)
+    if reading is not None:
+        if any(k.startswith(reading[1]) for k in kernels_of_step) or any(k.startswith(reading[1]) for k in launch_report()):
+            traffic_bytes = reading[0]
+            traffic_source = {"file": TRAFFIC_SOURCE, "kernel": reading[2], "counters": "FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 (copy-kernel yardstick), KiB per dispatch"}
+        else:
+            traffic_source = {"file": TRAFFIC_SOURCE, "kernel": reading[2], "note": "reading not applied: this run launched other kernels"}
     line = {
         "metric": "Q4_K matvec µs + achieved HBM GB/s (% of peak), 14336x4096, batch 1"
                   if args.config == "q4k_14336x4096_n1" else f"{fmt_name} matvec µs + achieved HBM GB/s, {rows}x{cols}, batch {n}",
@@ -882,12 +893,13 @@ def main() -> int:
                              "and 2k steps (for K <= 64 that is (T(2K) - T(K)) / K)",
                    "replay_launch_overhead_us": round(replay_overhead_us, 3),
                    "k_step_replay_ms": round(ms_total, 6),
+                   "raw_us_per_step": round(ms_total / K * 1e3, 3),   # the K-step replay divided by K, nothing taken off
                    "eager_python_us_per_call": None if eager_us is None else round(eager_us, 3)},
         "roofline": {"bound": "hbm",
                      "kernel": f"gemv_{fmt_name.lower()} with the activation quantizer fused in (cml_matmul_f32, one launch)" if fused
                      else f"gemv_{fmt_name.lower()} (cml_gemm on quantized activations)",
                      "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.config),
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic_bytes, "traffic_source": traffic_source,
                      "us_per_launch": round(kern_ms * 1e3, 3),
                      "cache_warm_us_per_launch": None if warm_ms is None else round(warm_ms * 1e3, 3),
                      "cache_warm_gbs": None if warm_ms is None else round(alg_bytes / (warm_ms * 1e-3) / 1e9, 2),

@@ -117,28 +117,6 @@ int cml_dev_free(void *ptr_dev);
 int cml_memcpy_h2d(void *dst_dev, const void *src_host, size_t nbytes, cml_stream_t stream);
 int cml_memcpy_d2h(void *dst_host, const void *src_dev, size_t nbytes, cml_stream_t stream);
 int cml_memset_dev(void *dst_dev, int value, size_t nbytes, cml_stream_t stream);
-/* Device-to-device streaming copy by a plain kernel (16-byte aligned pointers and
- * size; may be captured).  Also the yardstick bench.py reads byte counters and
- * matvec bandwidth against: it moves nbytes in, nbytes out and nothing else. */
-int cml_copy_dev(void *dst_dev, const void *src_dev, size_t nbytes, cml_stream_t stream);
-/* Two more yardsticks for the roofline reading of the matvec kernels (bench.py --calibrate-read /
- * roofline.shape_ceiling); neither has a counterpart in the reference.
- * cml_calibrate_read: a launch that only READS nbytes (16-byte aligned), every lane keeping
- * in_flight (1, 2, 4 or 8) 16-byte non-temporal loads out over a grid-stride walk with `workgroups`
- * workgroups of 256 lanes (0 = 2048), and stores nothing.
- * cml_calibrate_weight_loads: the plain single-token Q4_K matvec launch for `w` -- same grid, same
- * lane addresses, same load instructions and register buffers -- with the activation, the
- * arithmetic and the stores taken out (scratch_dev: 4 writable bytes, never written in practice).
- * What these two take for a weight's bytes is what the SHAPE allows a single launch on this chip;
- * what the real kernel takes beyond that is the kernel's own cost. */
-int cml_calibrate_read(const void *src_dev, size_t nbytes, int in_flight, int workgroups, cml_stream_t stream);
-int cml_calibrate_weight_loads(const cml_weight *w, void *scratch_dev, cml_stream_t stream);
-/* cml_calibrate_matvec_ablation: the single-token Q4_K launch of cml_matmul_f32 for `w` with parts
- * taken out, to time what each part costs: mask 1 = no activation (no f32 loads, no quantizer, no
- * barrier), 4 = no output store, 7 = the weight requests alone.  Served
- * for the shapes the eight-wave launch serves (rows of 4096 values, 12288 to 16384 rows);
- * CML_ERR_UNSUPPORTED otherwise.  out_dev must hold w's rows and is garbage afterwards. */
-int cml_calibrate_matvec_ablation(const cml_weight *w, const float *x_dev, float *out_dev, int mask, cml_stream_t stream);
 int cml_stream_sync(cml_stream_t stream);
 /* Streams (default priority), timing events and captured launch sequences, for
  * hosts that drive a decode loop through this library alone.  The reference's
@@ -462,6 +440,34 @@ int cml_try_linear_rows(int fmt, const float *input_scales, const int8_t *input_
 int cml_try_q8_0_block_linear_row(const float *input_scales, const int8_t *input_quants,
                                   const uint8_t *weight_block_bytes, size_t weight_nbytes,
                                   int64_t rows, int64_t blocks_per_row, float *output);
+
+/* ==== Diagnostics: measurement yardsticks of bench.py ==========================================
+ * None of these has a counterpart in the reference and a production host never calls them:
+ * they exist so that the roofline reading of the matvec kernels (bench.py: roofline.shape_ceiling,
+ * --calibrate-copy, --calibrate-read) rests on launches anybody can re-run, not on constants.
+ * They share the library's launch path and may be captured into graphs; they change no state. */
+/* Device-to-device streaming copy by a plain kernel (16-byte aligned pointers and
+ * size; may be captured).  Also the yardstick bench.py reads byte counters and
+ * matvec bandwidth against: it moves nbytes in, nbytes out and nothing else. */
+int cml_copy_dev(void *dst_dev, const void *src_dev, size_t nbytes, cml_stream_t stream);
+/* Two more yardsticks for the roofline reading of the matvec kernels (bench.py --calibrate-read /
+ * roofline.shape_ceiling); neither has a counterpart in the reference.
+ * cml_calibrate_read: a launch that only READS nbytes (16-byte aligned), every lane keeping
+ * in_flight (1, 2, 4 or 8) 16-byte non-temporal loads out over a grid-stride walk with `workgroups`
+ * workgroups of 256 lanes (0 = 2048), and stores nothing.
+ * cml_calibrate_weight_loads: the plain single-token Q4_K matvec launch for `w` -- same grid, same
+ * lane addresses, same load instructions and register buffers -- with the activation, the
+ * arithmetic and the stores taken out (scratch_dev: 4 writable bytes, never written in practice).
+ * What these two take for a weight's bytes is what the SHAPE allows a single launch on this chip;
+ * what the real kernel takes beyond that is the kernel's own cost. */
+int cml_calibrate_read(const void *src_dev, size_t nbytes, int in_flight, int workgroups, cml_stream_t stream);
+int cml_calibrate_weight_loads(const cml_weight *w, void *scratch_dev, cml_stream_t stream);
+/* cml_calibrate_matvec_ablation: the single-token Q4_K launch of cml_matmul_f32 for `w` with parts
+ * taken out, to time what each part costs: mask 1 = no activation (no f32 loads, no quantizer, no
+ * barrier), 4 = no output store, 7 = the weight requests alone.  Served
+ * for the shapes the eight-wave launch serves (rows of 4096 values, 12288 to 16384 rows);
+ * CML_ERR_UNSUPPORTED otherwise.  out_dev must hold w's rows and is garbage afterwards. */
+int cml_calibrate_matvec_ablation(const cml_weight *w, const float *x_dev, float *out_dev, int mask, cml_stream_t stream);
 
 #ifdef __cplusplus
 }
