@@ -860,6 +860,14 @@ int cml_matmul_f32(const cml_weight *w, const float *x_dev, int64_t n_tokens, fl
         if (frc == CML_OK) g_runs.fetch_add(1, std::memory_order_relaxed);
         return frc;
     }
+    if (w->fmt == CML_Q4_K && !q4k_lane_order() && (n_tokens == 3 || n_tokens == 4) && fuse != 0 && w->nb <= 32 &&
+        !env_int("CAMELID_HIP_Q4K_GENERAL_ENTRY", 0)) {
+        // three or four tokens on rows of 4096 values with no K cut: the eight-wave packed-dot launch replays each
+        // step's unpacked weight against the tokens (one launch, quantizer inside); -1 = not such a shape
+        const int frc = launch_gemv_q4k_f32(w, x_dev, out_dev, st, static_cast<int>(n_tokens));
+        if (frc == CML_OK) g_runs.fetch_add(1, std::memory_order_relaxed);
+        if (frc != -1) return frc;
+    }
     if (w->fmt == CML_Q4_K && !q4k_lane_order() && n_tokens >= 3 && fuse != 0 && env_int("CAMELID_HIP_FUSED_QUANT_BATCH", 1)) {
         // 3 to 6 tokens on the matrix cores: the workgroups quantize the few rows themselves (14336 x 4096,
         // 4 tokens: 12.4 -> 11.0 us per step); more tokens cost every workgroup more than the launch saves

@@ -685,7 +685,12 @@ struct Q4KCuArgs {
     int tiles16;            // 16-row layout tiles that hold the rows
 };
 
-template <int NSTEPS, int ABLATE = 0>
+// NT (1 to 4) tokens: the f32 rows are contiguous ([NT][row length]), pass p of the quantizer takes token p, the
+// unpacked weight of a step is replayed against the NT staged rows from registers, and token t writes out[t][rows]
+// -- every cell the one-token result, bit for bit (the same q4k_compute).  The weight streams once for the NT tokens
+// and the vector work per step grows by about 60 instructions per token, which the stream hides up to three
+// tokens and nearly at four.
+template <int NSTEPS, int ABLATE = 0, int NT = 1>
 __global__ __launch_bounds__(512) void gemv_q4k_cu_kernel(Q4KCuArgs a) {
     const uint8_t *__restrict__ w = a.w;
     const float *__restrict__ x = a.x;
@@ -696,23 +701,27 @@ __global__ __launch_bounds__(512) void gemv_q4k_cu_kernel(Q4KCuArgs a) {
     constexpr int WAVES = 8;
     constexpr int NSB = 2 * NSTEPS;  // super-blocks per row
     constexpr int NB = 3, PRE = 2;   // ring slots; slots requested before the quantizer
-    static_assert(NSTEPS >= NB && NSB <= 2 * WAVES, "one quantizer pass covers the row");
+    static_assert(NSTEPS >= NB && NSB <= 2 * WAVES, "one quantizer pass covers a row");
+    static_assert(NT >= 1 && NT <= 4 && (NT == 1 || ABLATE == 0), "up to four tokens; the ablations are one-token launches");
     constexpr bool NOACT = (ABLATE & 1) != 0, NOMATH = (ABLATE & 2) != 0, NOSTORE = (ABLATE & 4) != 0;
     using Regs = Q4KRegs<1>;
-    __shared__ __attribute__((aligned(16))) int8_t ys[NSB * 256];
-    __shared__ int bsum[NSB * 8];
-    __shared__ float yds[NSB];
+    __shared__ __attribute__((aligned(16))) int8_t ys[NT * NSB * 256];
+    __shared__ int bsum[NT * NSB * 8];
+    __shared__ float yds[NT * NSB];
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
 
-    // the f32 activation: wave w quantizes super-blocks 2w and 2w + 1, a half wave each
+    // the f32 activation: wave w quantizes super-blocks 2w and 2w + 1 of every token, a half wave each
     const int half = lane >> 5, ql = lane & 31;
     const int sbk = 2 * wave + half;
-    float4 xv[2];
+    float4 xv[NT][2];
     if constexpr (!NOACT) {
-        const float4 *x4 = reinterpret_cast<const float4 *>(x) + min(sbk, NSB - 1) * 64 + ql * 2;
-        xv[0] = x4[0];
-        xv[1] = x4[1];
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            const float4 *x4 = reinterpret_cast<const float4 *>(x) + (t * NSB + min(sbk, NSB - 1)) * 64 + ql * 2;
+            xv[t][0] = x4[0];
+            xv[t][1] = x4[1];
+        }
     }
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (!NOACT) __builtin_amdgcn_s_barrier();  // execution only: every activation request of the workgroup is out
@@ -741,13 +750,17 @@ __global__ __launch_bounds__(512) void gemv_q4k_cu_kernel(Q4KCuArgs a) {
         // stores nothing): the f32 loads above are then used unconditionally, and the compiler cannot
         // sink them into a conditional block behind the weight requests.
         const bool mine = NSB == 2 * WAVES || sbk < NSB;
-        float dv;
-        int bs;
-        const uint2 packed = q8k_quantize_row32(xv, lane, dv, bs);
-        if (mine) {
-            reinterpret_cast<uint2 *>(ys)[sbk * 32 + ql] = packed;
-            if ((ql & 3) == 3) bsum[sbk * 8 + (ql >> 2)] = bs;
-            if (ql == 0) yds[sbk] = dv;
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            float dv;
+            int bs;
+            const uint2 packed = q8k_quantize_row32(xv[t], lane, dv, bs);
+            if (mine) {
+                const int at = t * NSB + sbk;
+                reinterpret_cast<uint2 *>(ys)[at * 32 + ql] = packed;
+                if ((ql & 3) == 3) bsum[at * 8 + (ql >> 2)] = bs;
+                if (ql == 0) yds[at] = dv;
+            }
         }
         __syncthreads();
     }
@@ -756,9 +769,11 @@ __global__ __launch_bounds__(512) void gemv_q4k_cu_kernel(Q4KCuArgs a) {
     ln.c = l;
     ln.sh = (l & 1) * 16;
     ln.upper = l >= 2;
-    float acc[1] = {0.0f};
+    float acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++) acc[t] = 0.0f;
     auto compute = [&](const Regs &b, int step) __attribute__((always_inline)) {
-        q4k_compute<1, false, 1, 2, true, NOMATH>(b, ln, 2 * step + h, NSB, ys, bsum, yds, NSB, acc, nullptr);
+        q4k_compute<NT, false, 1, 2, true, NOMATH>(b, ln, 2 * step + h, NSB, ys, bsum, yds, NSB, acc, nullptr);
         __builtin_amdgcn_sched_barrier(0);
     };
 #pragma unroll
@@ -773,10 +788,13 @@ __global__ __launch_bounds__(512) void gemv_q4k_cu_kernel(Q4KCuArgs a) {
         if (__builtin_bit_cast(uint32_t, acc[0]) == 0x12345679u) out[0] = 1.0f;
         return;
     }
-    if (l == LPS - 1 && h == 1 && live) {  // the second group's last lane ran the row's chain
-        float v = acc[0];
-        if (residual) v = v + residual[row];
-        out[row] = v;
+    if (l == LPS - 1 && h == 1 && live) {  // the second group's last lane ran the row's chains
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            float v = acc[t];
+            if (NT == 1 && residual) v = v + residual[row];
+            out[static_cast<int64_t>(t) * rows + row] = v;
+        }
     }
 }
 
@@ -912,12 +930,28 @@ static bool q4k_cu_serves(const Q4KArgs &ka, int ksplit) {
            !env_int("CAMELID_HIP_Q4K_CLAMPED_LOADS", 0) && env_int("CAMELID_HIP_Q4K_RING", 1) != 0;
 }
 
-static int launch_q4k_cu(const Q4KArgs &ka, int ablate, hipStream_t st) {
+// Most tokens the eight-wave launch replays per step (CAMELID_HIP_Q4K_CU_TOKENS, 1 to 4).  Measured at 14336 x 4096, us
+// per step against what served the call before: 2 tokens 7.20 (8.46, the 16-row-wave ring launch), 3 tokens 8.83 (9.71,
+// the matrix-core launch with the quantizer inside), 4 tokens 14.5 (10.3: the vector work no longer hides).  Default 3.
+static int q4k_cu_max_tokens() { return std::min(4, std::max(1, env_int("CAMELID_HIP_Q4K_CU_TOKENS", 3))); }
+
+static int launch_q4k_cu(const Q4KArgs &ka, int ablate, hipStream_t st, int n_tokens = 1) {
     if (!(ablate & 1) && !ka.x) return fail(CML_ERR_INVALID, "null activation");  // every variant but the one without the activation reads it
     const int tiles16 = (ka.rows + ka.row_skip + 15) / 16;
     const dim3 grid(static_cast<unsigned>((2 * tiles16 + 7) / 8)), block(512);
     const Q4KCuArgs ca{ka.w, ka.x, ka.out, ka.residual, static_cast<uint32_t>(ka.sb_stride), ka.rows, ka.row_skip, tiles16};
 #define CML_Q4K_CU(A_) hipLaunchKernelGGL((gemv_q4k_cu_kernel<8, A_>), grid, block, 0, st, ca)
+    if (n_tokens > 1) {
+        if (ablate) return fail(CML_ERR_INVALID, "the ablations are one-token launches");
+        switch (n_tokens) {
+            case 2: hipLaunchKernelGGL((gemv_q4k_cu_kernel<8, 0, 2>), grid, block, 0, st, ca); break;
+            case 3: hipLaunchKernelGGL((gemv_q4k_cu_kernel<8, 0, 3>), grid, block, 0, st, ca); break;
+            case 4: hipLaunchKernelGGL((gemv_q4k_cu_kernel<8, 0, 4>), grid, block, 0, st, ca); break;
+            default: return fail(CML_ERR_INVALID, "the eight-wave launch takes up to four tokens");
+        }
+        CML_COUNT_LAUNCH("q4k.dot.wg8.fused.tokens");
+        return CML_OK;
+    }
     switch (ablate) {
         case 0: CML_Q4K_CU(0); break;
         case 1: CML_Q4K_CU(1); break;
@@ -1196,6 +1230,11 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
             else if (half_tiles) { if (whole) CML_Q4K_LOADS(2, true); else CML_Q4K_LOADS(2, false); CML_COUNT_LAUNCH("q4k.calibrate.buffers"); }
             else { if (whole) CML_Q4K_LOADS(1, true); else CML_Q4K_LOADS(1, false); CML_COUNT_LAUNCH("q4k.calibrate.buffers"); }
 #undef CML_Q4K_LOADS
+        } else if (plain && a.n_tokens >= 2 && a.n_tokens <= q4k_cu_max_tokens() && q4k_rows_per_wave(tiles16, shape.ksplit, 1) == 8 &&
+                   q4k_ring(ka, shape.ksplit) && q4k_cu_serves(ka, shape.ksplit)) {
+            if (int rc = launch_q4k_cu(ka, 0, st, static_cast<int>(a.n_tokens))) return rc;  // a few tokens replayed against each step's weight
+        } else if (!grouped && !w2 && a.n_tokens > 2) {
+            return -1;  // more than two tokens of a plain call: only the eight-wave launch above takes them
         } else if (two) {
             // both tokens in one pass over the weight, 16-row waves as in the two-token matvec
             if (q4k_ring(ka, shape.ksplit, 1)) launch_q4k_ring<2, true, 1>(ka, shape.ksplit, grid, block, lds, st);
@@ -1359,7 +1398,7 @@ int launch_gemv_q4k_f32(const cml_weight *w, const float *x, float *out, hipStre
     MatArgs a{};
     a.w = w;
     a.out = out;
-    a.n_tokens = n_tokens;  // 1, or 2 contiguous rows of x -> out[2][rows]
+    a.n_tokens = n_tokens;  // 1, or 2 (3, 4: -1 where the eight-wave launch does not serve the shape) contiguous rows of x -> out[n][rows]
     a.n_groups = 1;
     return launch_q4k_f32(a, nullptr, nullptr, x, st);
 }

@@ -388,6 +388,36 @@ def test_q4k_eight_wave_launch_is_the_four_wave_launch_and_the_two_step_path(row
             assert np.array_equal(q_gpu, q_all[i]) and np.array_equal(d_gpu.view(np.uint32), s_all[i].view(np.uint32))
 
 
+@pytest.mark.parametrize("rows", [12288, 14336, 14327])
+def test_q4k_eight_wave_launch_replays_a_few_tokens(rows):
+    """Two, three (and, under its knob, four) tokens on the eight-wave launch: the weight of a step unpacked once and
+    replayed against every token's staged row.  Each cell is the single-token call's bits and the oracle's, the
+    counters show the launch, and with it switched off (CAMELID_HIP_Q4K_CU_TOKENS=1) the former paths give the same
+    bits: the 16-row-wave ring launch for two tokens, the matrix-core launch for three and four."""
+    fmt, cols = oracle.Q4_K, 4096
+    rng = np.random.default_rng(8400 + rows)
+    wire = G.synth_weight(fmt, rows, cols, seed=8500 + rows)
+    w = Weight.upload(fmt, rows, cols, wire)
+    x = rng.standard_normal((4, cols)).astype(np.float32)
+    x[1, :512] = 0.0
+    x[2, 1::2] = -x[2, ::2]
+    x[3, 7], x[3, 1000] = 9.0, -9.0
+    singles = np.stack([G.gpu_matmul_f32(w, x[t]) for t in range(4)])
+    want = oracle.matmul(fmt, wire, cols, x, order=EXACT_ORDER[fmt], threads=16)
+    assert G.same_bits(singles, want)
+    for n in (2, 3, 4):
+        G.say(f"Q4_K eight-wave launch {rows}x4096, {n} tokens")
+        with G.env(CAMELID_HIP_Q4K_CU_TOKENS=4), G.engaged(r"^q4k\.dot\.wg8\.fused\.tokens$", none=(r"^q4k\.mfma", r"^q4k\.dot\.ring", r"^quantize\.")):
+            got = G.gpu_matmul_f32(w, x[:n])
+        assert G.same_bits(got, singles[:n]), (rows, n)
+        former = r"^q4k\.dot\.ring\.fused$" if n == 2 else r"^q4k\.mfma\.pair\.fused$"
+        with G.env(CAMELID_HIP_Q4K_CU_TOKENS=1), G.engaged(former, none=(r"^q4k\.dot\.wg8",)):
+            assert G.same_bits(G.gpu_matmul_f32(w, x[:n]), singles[:n]), (rows, n, "former path")
+        default_kernel = r"^q4k\.dot\.wg8\.fused\.tokens$" if n <= 3 else r"^q4k\.mfma\.pair\.fused$"
+        with G.engaged(default_kernel):
+            assert G.same_bits(G.gpu_matmul_f32(w, x[:n]), singles[:n]), (rows, n, "default")
+
+
 @pytest.mark.parametrize("rows", [4096, 3100, 6100])
 def test_q4k_eight_wave_launch_under_the_k_cut_is_the_two_launch_path(rows):
     """Rows of 14336 values on 3072 to 6128 rows (the FFN down projection: the shape policy cuts K four ways):
