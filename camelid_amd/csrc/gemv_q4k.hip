@@ -242,12 +242,21 @@ __device__ __forceinline__ void q4k_compute(const Q4KRegs<U> &r, const Q4KLane &
             }
             acc[t] = __builtin_fmaf(-M, static_cast<float>(p_total), acc[t]);
             acc[t] = __builtin_fmaf(D, static_cast<float>(s_total), acc[t]);
+            // The chain advances HERE.  Its only reader is the store of the one lane per row that owns it, under a
+            // condition, and without this the compiler sinks every fused step of the row into that block: the
+            // operands of all steps (eight registers per step and token) stay live to the end, and the whole dependent
+            // chain -- 32 operations for a row of 4096 values -- runs after the last weight bytes have arrived,
+            // where nothing is left to overlap it.
+            asm volatile("" : "+v"(acc[t]));
             if constexpr (INTS) {
                 if (ints_row != nullptr && valid) {
                     ints_row[2 * i] = s_total;
                     ints_row[2 * i + 1] = p_total;
                 }
             }
+            // one-entry buffers replayed against three or four tokens (the eight-wave launch): token by token, or the
+            // scheduler holds every token's staged row in registers at once and the kernel no longer fits two waves per SIMD
+            if constexpr (U == 1 && NT >= 3) __builtin_amdgcn_sched_barrier(0);
         }
     }
 }
@@ -761,6 +770,7 @@ __global__ __launch_bounds__(512) void gemv_q4k_cu_kernel(Q4KCuArgs a) {
                 if ((ql & 3) == 3) bsum[at * 8 + (ql >> 2)] = bs;
                 if (ql == 0) yds[at] = dv;
             }
+            if constexpr (NT >= 3) __builtin_amdgcn_sched_barrier(0);  // one token's pass at a time: the passes interleaved need too many registers
         }
         __syncthreads();
     }
