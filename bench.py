@@ -413,7 +413,7 @@ def bench_moe(name: str, K: int, W: int, seed: int, cpu_seconds: float) -> int:
     else:
         # one token: gate and up in one launch (routes and quantizes the token itself), silu*up->Q8_K, down + weighted sum in one launch;
         # more: route, plan, quantize, gate and up in one launch, silu*up->Q8_K, down, weighted sum
-        routed_in_launch = T == 1 and not two_calls and os.environ.get("CAMELID_HIP_MOE_FOLD_ROUTE", "1") != "0"
+        routed_in_launch = T == 1 and not two_calls and not (os.environ.get("CAMELID_HIP_TUNING", "0") not in ("", "0") and os.environ.get("CAMELID_HIP_MOE_FOLD_ROUTE", "1") == "0")
         launches, kernel = ((3 if routed_in_launch else 4) if T == 1 else 7), "gemv_q4k_kernel / gemm_q4k_mfma_kernel grouped by expert (2-3 launches of the step)"
         what = ("route + gate/up matvecs + silu*up->Q8_K + down matvec + weighted sum (cml_moe_ffn_logits; one token: the routing inside "
                 "the gate|up launch, the weighted sum inside the down launch), graph replay")

@@ -60,10 +60,16 @@ LaunchCounter::LaunchCounter(const char *nm) : name(nm ? nm : "?") {
     } while (!g_counters.compare_exchange_weak(head, this, std::memory_order_release, std::memory_order_acquire));
 }
 
-// Tuning knobs (CAMELID_HIP_*) are read from the environment ONCE, into a snapshot taken by
+// Knobs (CAMELID_HIP_*) are read from the environment ONCE, into a snapshot taken by
 // cml_init and again by cml_reload_env (reference: every CAMELID_* knob sits in a OnceLock,
 // src/inference.rs:23679-23692).  A launch only walks the snapshot -- normally empty -- and never
 // calls getenv, so it neither pays for it nor races with a setenv in another thread.
+// Two kinds.  The few knobs that choose WHAT is computed or where (the device, and which of the
+// reference's accumulation orders the results follow) are always honoured.  Everything else chooses
+// among kernels that give the same bits -- launch shapes, ring depths, thresholds: the switches
+// of this library's own tests and measurements -- and is honoured only when CAMELID_HIP_TUNING=1 is set
+// with it, so that a stray variable in a production host's environment cannot move a call onto a
+// slower kernel.
 struct EnvSnapshot {
     std::vector<std::pair<std::string, int>> knobs;  // names without the CAMELID_HIP_ prefix
 };
@@ -73,11 +79,17 @@ extern "C" char **environ;
 static void load_env_snapshot() {
     auto *snap = new EnvSnapshot();
     static const char prefix[] = "CAMELID_HIP_";
+    static const char *const always[] = {"DEVICE", "EXACT_ORDER", "Q4K_LANE_ORDER", "Q6K_LANE_ORDER"};
+    const char *tuning_env = getenv("CAMELID_HIP_TUNING");
+    const bool tuning = tuning_env && atoi(tuning_env) != 0;
     for (char **e = environ; e && *e; e++) {
         if (strncmp(*e, prefix, sizeof(prefix) - 1) != 0) continue;
         const char *eq = strchr(*e, '=');
         if (!eq || !eq[1]) continue;  // unset or empty: the default applies
-        snap->knobs.emplace_back(std::string(static_cast<const char *>(*e) + sizeof(prefix) - 1, eq), atoi(eq + 1));
+        std::string key(static_cast<const char *>(*e) + sizeof(prefix) - 1, eq);
+        bool take = tuning;
+        for (const char *a : always) take = take || key == a;
+        if (take) snap->knobs.emplace_back(std::move(key), atoi(eq + 1));
     }
     // superseded snapshots are kept: a launch on another thread may still be reading one, and
     // reloads only happen in tests

@@ -34,9 +34,15 @@
  *     array of cml_matmul_f32_static, see there -- so any number of threads may
  *     call them, each on its own stream, on weights that nobody frees meanwhile.  cml_init / cml_shutdown / cml_reload_env must not
  *     run concurrently with anything else;
- *   - tuning knobs (environment variables named CAMELID_HIP_*) are read once, by
+ *   - knobs (environment variables named CAMELID_HIP_*) are read once, by
  *     cml_init, the way the reference reads its CAMELID_* knobs once per process
- *     (src/inference.rs:23679-23692); cml_reload_env() reads them again.
+ *     (src/inference.rs:23679-23692); cml_reload_env() reads them again.  Four
+ *     are always honoured because they choose what is computed or where:
+ *     CAMELID_HIP_DEVICE, CAMELID_HIP_EXACT_ORDER, CAMELID_HIP_Q4K_LANE_ORDER,
+ *     CAMELID_HIP_Q6K_LANE_ORDER.  All others choose among kernels that give the
+ *     same bits (launch shapes, ring depths, thresholds: the switches of this
+ *     library's tests and measurements) and are ignored unless
+ *     CAMELID_HIP_TUNING=1 is set as well.
  *
  * Tensor conventions (reference src/tensor/mod.rs:79-89, src/inference.rs:
  * 23728-23749): a weight is `rows` output rows of `cols` contraction values,

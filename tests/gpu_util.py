@@ -19,8 +19,10 @@ def say(msg: str) -> None:
 
 @contextmanager
 def env(**kv):
-    """Tuning knobs for the calls inside the block.  The library reads its environment once, so
+    """Knobs for the calls inside the block.  The library reads its environment once, so
     it is told to read it again on the way in and on the way out."""
+    kv = dict(kv)
+    kv.setdefault("CAMELID_HIP_TUNING", "1")  # launch-shape knobs are honoured only with this switch
     old = {k: os.environ.get(k) for k in kv}
     try:
         for k, v in kv.items():

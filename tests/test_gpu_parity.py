@@ -335,6 +335,25 @@ def test_q4k_fused_quantize_matvec_is_the_two_step_path(rows, cols):
             assert G.same_bits(got, want)
 
 
+def test_launch_shape_knobs_need_the_tuning_switch():
+    """A knob that only chooses among kernels of equal bits is honoured when CAMELID_HIP_TUNING=1 is set
+    with it and ignored otherwise (a stray variable cannot move a production call onto another kernel);
+    the knobs that choose the accumulation order are honoured on their own.  The counters say which
+    kernel ran."""
+    fmt, rows, cols = oracle.Q4_K, 12288, 4096
+    w = Weight.upload(fmt, rows, cols, G.synth_weight(fmt, rows, cols, seed=8801))
+    x = np.random.default_rng(8802).standard_normal(cols).astype(np.float32)
+    with G.engaged(r"^q4k\.dot\.wg8\.fused$"):
+        want = G.gpu_matmul_f32(w, x)
+    with G.env(CAMELID_HIP_Q4K_CU=0, CAMELID_HIP_TUNING=0), G.engaged(r"^q4k\.dot\.wg8\.fused$", none=(r"^q4k\.dot\.ring",)):
+        assert G.same_bits(G.gpu_matmul_f32(w, x), want)
+    with G.env(CAMELID_HIP_Q4K_CU=0, CAMELID_HIP_TUNING=1), G.engaged(r"^q4k\.dot\.ring\.fused$", none=(r"^q4k\.dot\.wg8",)):
+        assert G.same_bits(G.gpu_matmul_f32(w, x), want)
+    # an order knob without the switch: the 8-lane order of the reference's generic CPU lane
+    with G.env(CAMELID_HIP_Q4K_LANE_ORDER=1, CAMELID_HIP_TUNING=0), G.engaged(r"^q4k\.lanes$", none=(r"^q4k\.dot\.",)):
+        G.gpu_matmul_f32(w, x)
+
+
 @pytest.mark.parametrize("rows", [12288, 14336, 14327, 16384])
 def test_q4k_eight_wave_launch_is_the_four_wave_launch_and_the_two_step_path(rows):
     """Rows of 4096 values on 12288 to 16384 rows (no K cut): cml_matmul_f32 runs the eight-wave launch
