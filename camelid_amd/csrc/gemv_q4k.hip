@@ -932,44 +932,66 @@ static int launch_q4k_cu_kcut(const Q4KArgs &ka, hipStream_t st) {
     return CML_OK;
 }
 
-// Whether the launch above serves this call: rows of 4096 values, no K cut (the shape policy gives
-// that from 12288 rows on, i.e. at least 192 eight-wave workgroups), a stride the 32-bit lane
-// offsets can hold.  CAMELID_HIP_Q4K_CU=0 keeps the four-wave launch.
-static bool q4k_cu_serves(const Q4KArgs &ka, int ksplit) {
-    return ksplit == 1 && ka.n_sb == 16 && ka.sb_stride < (int64_t(1) << 31) && env_int("CAMELID_HIP_Q4K_CU", 1) != 0 &&
-           !env_int("CAMELID_HIP_Q4K_CLAMPED_LOADS", 0) && env_int("CAMELID_HIP_Q4K_RING", 1) != 0;
+// Whether the launch above serves this call: rows of 6 to 16 super-blocks (an even count: 1536 to 4096 values), no
+// K cut (the shape policy gives that from 12288 rows on, i.e. at least 192 eight-wave workgroups), a stride the
+// 32-bit lane offsets can hold.  One and two tokens only while the launch is at most one workgroup per compute unit
+// (16384 rows): beyond that the four-wave workgroups spread more evenly (18944 x 3584: 8.77 us against 9.33 with
+// eight waves; three tokens 13.3 against 16.0 for what served them before, so those stay).
+// CAMELID_HIP_Q4K_CU=0 keeps the four-wave launch.
+constexpr int kComputeUnits = 256;  // MI355X
+static bool q4k_cu_serves(const Q4KArgs &ka, int ksplit, int n_tokens = 1) {
+    const int workgroups = (2 * ((ka.rows + ka.row_skip + 15) / 16) + 7) / 8;
+    return ksplit == 1 && (n_tokens >= 3 || workgroups <= kComputeUnits) && ka.n_sb <= 16 && ka.n_sb >= 6 && (ka.n_sb & 1) == 0 &&
+           ka.sb_stride < (int64_t(1) << 31) && env_int("CAMELID_HIP_Q4K_CU", 1) != 0 && !env_int("CAMELID_HIP_Q4K_CLAMPED_LOADS", 0) &&
+           env_int("CAMELID_HIP_Q4K_RING", 1) != 0;
 }
 
 // Most tokens the eight-wave launch replays per step (CAMELID_HIP_Q4K_CU_TOKENS, 1 to 4).  Measured at 14336 x 4096, us
 // per step against what served the call before: 2 tokens 7.20 (8.46, the 16-row-wave ring launch), 3 tokens 8.83 (9.71,
 // the matrix-core launch with the quantizer inside), 4 tokens 14.5 (10.3: the vector work no longer hides).  Default 3.
-static int q4k_cu_max_tokens() { return std::min(4, std::max(1, env_int("CAMELID_HIP_Q4K_CU_TOKENS", 3))); }
+static int q4k_cu_max_tokens(int n_sb) { return std::min(n_sb == 16 ? 4 : 3, std::max(1, env_int("CAMELID_HIP_Q4K_CU_TOKENS", 3))); }
 
 static int launch_q4k_cu(const Q4KArgs &ka, int ablate, hipStream_t st, int n_tokens = 1) {
     if (!(ablate & 1) && !ka.x) return fail(CML_ERR_INVALID, "null activation");  // every variant but the one without the activation reads it
     const int tiles16 = (ka.rows + ka.row_skip + 15) / 16;
     const dim3 grid(static_cast<unsigned>((2 * tiles16 + 7) / 8)), block(512);
     const Q4KCuArgs ca{ka.w, ka.x, ka.out, ka.residual, static_cast<uint32_t>(ka.sb_stride), ka.rows, ka.row_skip, tiles16};
-#define CML_Q4K_CU(A_) hipLaunchKernelGGL((gemv_q4k_cu_kernel<8, A_>), grid, block, 0, st, ca)
+    // rows of 2 * NSTEPS super-blocks: one instantiation per row length (1536 to 4096 values)
+#define CML_Q4K_CU_STEPS(NT_)                                                                                 \
+    switch (ka.n_sb) {                                                                                        \
+        case 16: hipLaunchKernelGGL((gemv_q4k_cu_kernel<8, 0, NT_>), grid, block, 0, st, ca); break;          \
+        case 14: hipLaunchKernelGGL((gemv_q4k_cu_kernel<7, 0, NT_>), grid, block, 0, st, ca); break;          \
+        case 12: hipLaunchKernelGGL((gemv_q4k_cu_kernel<6, 0, NT_>), grid, block, 0, st, ca); break;          \
+        case 10: hipLaunchKernelGGL((gemv_q4k_cu_kernel<5, 0, NT_>), grid, block, 0, st, ca); break;          \
+        case 8: hipLaunchKernelGGL((gemv_q4k_cu_kernel<4, 0, NT_>), grid, block, 0, st, ca); break;           \
+        case 6: hipLaunchKernelGGL((gemv_q4k_cu_kernel<3, 0, NT_>), grid, block, 0, st, ca); break;           \
+        default: return fail(CML_ERR_UNSUPPORTED, "the eight-wave launch takes rows of 6 to 16 super-blocks");  \
+    }
     if (n_tokens > 1) {
         if (ablate) return fail(CML_ERR_INVALID, "the ablations are one-token launches");
         switch (n_tokens) {
-            case 2: hipLaunchKernelGGL((gemv_q4k_cu_kernel<8, 0, 2>), grid, block, 0, st, ca); break;
-            case 3: hipLaunchKernelGGL((gemv_q4k_cu_kernel<8, 0, 3>), grid, block, 0, st, ca); break;
-            case 4: hipLaunchKernelGGL((gemv_q4k_cu_kernel<8, 0, 4>), grid, block, 0, st, ca); break;
+            case 2: CML_Q4K_CU_STEPS(2); break;
+            case 3: CML_Q4K_CU_STEPS(3); break;
+            case 4:
+                if (ka.n_sb != 16) return fail(CML_ERR_INVALID, "four tokens: rows of 16 super-blocks only");
+                hipLaunchKernelGGL((gemv_q4k_cu_kernel<8, 0, 4>), grid, block, 0, st, ca);
+                break;
             default: return fail(CML_ERR_INVALID, "the eight-wave launch takes up to four tokens");
         }
         CML_COUNT_LAUNCH("q4k.dot.wg8.fused.tokens");
         return CML_OK;
     }
+    if (ablate && ka.n_sb != 16) return fail(CML_ERR_UNSUPPORTED, "the ablations exist for rows of 4096 values");
+#define CML_Q4K_CU(A_) hipLaunchKernelGGL((gemv_q4k_cu_kernel<8, A_>), grid, block, 0, st, ca)
     switch (ablate) {
-        case 0: CML_Q4K_CU(0); break;
+        case 0: CML_Q4K_CU_STEPS(1); break;
         case 1: CML_Q4K_CU(1); break;
         case 4: CML_Q4K_CU(4); break;
         case 7: CML_Q4K_CU(7); break;
         default: return fail(CML_ERR_INVALID, "ablation mask must be 1, 4 or 7");
     }
 #undef CML_Q4K_CU
+#undef CML_Q4K_CU_STEPS
     if (ablate) CML_COUNT_LAUNCH("q4k.calibrate.wg8");
     else CML_COUNT_LAUNCH("q4k.dot.wg8.fused");
     return CML_OK;
@@ -1228,7 +1250,7 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
         const bool plain = !grouped && !w2 && !env_int("CAMELID_HIP_Q4K_GENERAL_ENTRY", 0);
         const dim3 block(64 * waves);
 #define CML_Q4K_LAUNCH(SPR_, WHOLE_, PLAIN_) hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, SPR_, WHOLE_, PLAIN_>), grid, block, lds, st, ka)
-        if (loads_only && half_tiles && ring && plain && q4k_cu_serves(ka, shape.ksplit)) {
+        if (loads_only && half_tiles && ring && plain && q4k_cu_serves(ka, shape.ksplit) && ka.n_sb == 16) {
             if (int rc = launch_q4k_cu(ka, ablate, st)) return rc;
         } else if (loads_only && ablate != 7) {
             return fail(CML_ERR_UNSUPPORTED, "this ablation exists for the eight-wave single-token launch (rows of 4096 values, no K cut)");
@@ -1240,8 +1262,8 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
             else if (half_tiles) { if (whole) CML_Q4K_LOADS(2, true); else CML_Q4K_LOADS(2, false); CML_COUNT_LAUNCH("q4k.calibrate.buffers"); }
             else { if (whole) CML_Q4K_LOADS(1, true); else CML_Q4K_LOADS(1, false); CML_COUNT_LAUNCH("q4k.calibrate.buffers"); }
 #undef CML_Q4K_LOADS
-        } else if (plain && a.n_tokens >= 2 && a.n_tokens <= q4k_cu_max_tokens() && q4k_rows_per_wave(tiles16, shape.ksplit, 1) == 8 &&
-                   q4k_ring(ka, shape.ksplit) && q4k_cu_serves(ka, shape.ksplit)) {
+        } else if (plain && a.n_tokens >= 2 && a.n_tokens <= q4k_cu_max_tokens(ka.n_sb) && q4k_rows_per_wave(tiles16, shape.ksplit, 1) == 8 &&
+                   q4k_ring(ka, shape.ksplit) && q4k_cu_serves(ka, shape.ksplit, static_cast<int>(a.n_tokens))) {
             if (int rc = launch_q4k_cu(ka, 0, st, static_cast<int>(a.n_tokens))) return rc;  // a few tokens replayed against each step's weight
         } else if (!grouped && !w2 && a.n_tokens > 2) {
             return -1;  // more than two tokens of a plain call: only the eight-wave launch above takes them

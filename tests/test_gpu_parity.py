@@ -437,6 +437,34 @@ def test_q4k_eight_wave_launch_replays_a_few_tokens(rows):
             assert G.same_bits(G.gpu_matmul_f32(w, x[:n]), singles[:n]), (rows, n, "default")
 
 
+@pytest.mark.parametrize("rows,cols", [(12800, 1536), (12304, 2048), (13000, 2560), (12320, 3072), (16384, 3584)])
+def test_q4k_eight_wave_launch_serves_rows_of_six_to_sixteen_super_blocks(rows, cols):
+    """The eight-wave launch on the other row lengths it is built for (1536 to 3584 values: 6 to 14 super-blocks, an
+    even count), one to three tokens: the bits of the four-wave / matrix-core paths it replaces and of the oracle,
+    also on a row band; the counters show the launch."""
+    fmt = oracle.Q4_K
+    rng = np.random.default_rng(8600 + cols)
+    wire = G.synth_weight(fmt, rows, cols, seed=8700 + cols)
+    w = Weight.upload(fmt, rows, cols, wire)
+    x = rng.standard_normal((3, cols)).astype(np.float32)
+    x[1, :256] = 0.0
+    x[2, 5], x[2, cols - 3] = 7.0, -7.0
+    want = oracle.matmul(fmt, wire, cols, x, order=EXACT_ORDER[fmt], threads=16)
+    band = w.slice(3, rows - 20)
+    for n in (1, 2, 3):
+        G.say(f"Q4_K eight-wave launch {rows}x{cols}, {n} tokens")
+        kernel = r"^q4k\.dot\.wg8\.fused$" if n == 1 else r"^q4k\.dot\.wg8\.fused\.tokens$"
+        with G.engaged(kernel, none=(r"^q4k\.mfma", r"^q4k\.dot\.ring", r"^q4k\.dot\.buffers", r"^quantize\.")):
+            got = G.gpu_matmul_f32(w, x[:n] if n > 1 else x[0])
+            got_band = G.gpu_matmul_f32(band, x[:n] if n > 1 else x[0])
+        got = np.asarray(got).reshape(n, rows)
+        assert G.same_bits(got, want[:n]), (rows, cols, n)
+        assert G.same_bits(np.asarray(got_band).reshape(n, rows - 20), got[:, 3:rows - 17]), (rows, cols, n, "band")
+        with G.env(CAMELID_HIP_Q4K_CU=0), G.engaged(none=(r"^q4k\.dot\.wg8",)):
+            former = np.asarray(G.gpu_matmul_f32(w, x[:n] if n > 1 else x[0])).reshape(n, rows)
+        assert G.same_bits(former, got), (rows, cols, n, "former path")
+
+
 @pytest.mark.parametrize("rows", [4096, 3100, 6100])
 def test_q4k_eight_wave_launch_under_the_k_cut_is_the_two_launch_path(rows):
     """Rows of 14336 values on 3072 to 6128 rows (the FFN down projection: the shape policy cuts K four ways):
