@@ -946,9 +946,10 @@ static bool q4k_cu_serves(const Q4KArgs &ka, int ksplit, int n_tokens = 1) {
            env_int("CAMELID_HIP_Q4K_RING", 1) != 0;
 }
 
-// Most tokens the eight-wave launch replays per step (CAMELID_HIP_Q4K_CU_TOKENS, 1 to 4).  Measured at 14336 x 4096, us
-// per step against what served the call before: 2 tokens 7.20 (8.46, the 16-row-wave ring launch), 3 tokens 8.83 (9.71,
-// the matrix-core launch with the quantizer inside), 4 tokens 14.5 (10.3: the vector work no longer hides).  Default 3.
+// Most tokens the eight-wave launch replays per step (CAMELID_HIP_Q4K_CU_TOKENS, 1 to 4; four only on rows of 4096 values).
+// Measured at 14336 x 4096, us per step against what served the call before: 2 tokens 7.0 (8.46, the 16-row-wave ring launch),
+// 3 tokens 8.6 (9.71, the matrix-core launch with the quantizer inside), 4 tokens 10.4 (10.3: the vector work no longer hides
+// behind the stream).  Default 3.
 static int q4k_cu_max_tokens(int n_sb) { return std::min(n_sb == 16 ? 4 : 3, std::max(1, env_int("CAMELID_HIP_Q4K_CU_TOKENS", 3))); }
 
 static int launch_q4k_cu(const Q4KArgs &ka, int ablate, hipStream_t st, int n_tokens = 1) {
