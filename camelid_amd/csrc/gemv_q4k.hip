@@ -815,12 +815,17 @@ __global__ __launch_bounds__(512) void gemv_q4k_cu_kernel(Q4KCuArgs a) {
 // chains of a row are added left to right through LDS -- the association of gemv_q4k_kernel under the same K cut, so
 // the same bits.  The two-launch form (a quantizing launch, then the matvec) takes 9.1 us per step at 4096 x 14336 for
 // a 7.1 us matvec; the four-wave kernel with the quantizer inside took 10.0 (512 workgroups each quantizing the row).
-// Of this launch's 7.64 us the activation path is 0.97 (6.66 without it: every workgroup quantizes all 14336 values, four
-// quantizer passes per wave against one in the uncut launch, where they hide), the combine and store 0.38 (7.26 without),
-// the weight requests alone 6.02.
+// With the whole row quantized before the walk the launch takes 7.64 us, of which the activation path is 0.97 (6.66
+// without it: every workgroup quantizes all 14336 values, four quantizer passes per wave against one in the uncut launch,
+// where they hide), the combine and store 0.38 (7.26 without), the weight requests alone 6.02; STAGED brings it to 7.19.
 // ABLATE: as in gemv_q4k_cu_kernel (timing experiments; results are wrong).
-template <int KS, int NSTEPS, int ABLATE = 0>
+// STAGED: the quantizer passes are interleaved with the walk.  Pass p quantizes, for every K part, the two super-block
+// pairs its steps 2p and 2p + 1 read (the part's two waves take one pair each), so after pass 0 and one barrier every
+// wave starts walking, and pass p + 1 runs between the requests and the arithmetic of steps 2p, 2p + 1: the weight
+// stream never waits for a whole row to be quantized.
+template <int KS, int NSTEPS, int ABLATE = 0, bool STAGED = false>
 __global__ __launch_bounds__(512) void gemv_q4k_cu_kcut_kernel(Q4KCuArgs a) {
+    static_assert(!STAGED || (KS == 4 && NSTEPS == 7), "the staged quantizer: four K parts of seven steps, two waves each");
     constexpr bool NOACT = (ABLATE & 1) != 0, NOMATH = (ABLATE & 2) != 0, NOSTORE = (ABLATE & 4) != 0;
     const uint8_t *__restrict__ w = a.w;
     const float *__restrict__ x = a.x;
@@ -843,13 +848,22 @@ __global__ __launch_bounds__(512) void gemv_q4k_cu_kcut_kernel(Q4KCuArgs a) {
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
 
-    // the f32 activation: pass p of wave w quantizes the super-block pair w + 8 p, a half wave per super-block
+    // the f32 activation: pass p of wave w quantizes the super-block pair w + 8 p (STAGED: pair 2p + (w / KS) of K part
+    // w % KS), a half wave per super-block
     const int half = lane >> 5, ql = lane & 31;
+    auto pair_of = [&](int p) __attribute__((always_inline)) -> int {
+        if constexpr (STAGED) return NSTEPS * (wave % KS) + min(2 * p + wave / KS, NSTEPS - 1);
+        else return min(wave + WAVES * p, PAIRS - 1);
+    };
+    auto pair_mine = [&](int p) __attribute__((always_inline)) -> bool {
+        if constexpr (STAGED) return 2 * p + wave / KS < NSTEPS;
+        else return WAVES * (p + 1) <= PAIRS || wave + WAVES * p < PAIRS;
+    };
     float4 xv[PASSES][2];
     if constexpr (!NOACT) {
 #pragma unroll
         for (int p = 0; p < PASSES; p++) {
-            const int sbk = 2 * min(wave + WAVES * p, PAIRS - 1) + half;
+            const int sbk = 2 * pair_of(p) + half;
             const float4 *x4 = reinterpret_cast<const float4 *>(x) + sbk * 64 + ql * 2;
             xv[p][0] = x4[0];
             xv[p][1] = x4[1];
@@ -878,20 +892,24 @@ __global__ __launch_bounds__(512) void gemv_q4k_cu_kcut_kernel(Q4KCuArgs a) {
 
     // every wave runs every pass (a wave without a pair of its own in the last pass redoes the last pair and stores
     // nothing): the f32 loads above are then used unconditionally and stay ahead of the weight requests
+    auto quantize_pass = [&](int p) __attribute__((always_inline)) {
+        const int sbk = 2 * pair_of(p) + half;
+        float dv;
+        int bs;
+        const uint2 packed = q8k_quantize_row32(xv[p], lane, dv, bs);
+        if (pair_mine(p)) {
+            reinterpret_cast<uint2 *>(ys)[sbk * 32 + ql] = packed;
+            if ((ql & 3) == 3) bsum[sbk * 8 + (ql >> 2)] = bs;
+            if (ql == 0) yds[sbk] = dv;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
     if constexpr (!NOACT) {
+        if constexpr (STAGED) {
+            quantize_pass(0);
+        } else {
 #pragma unroll
-        for (int p = 0; p < PASSES; p++) {
-            const int pair = wave + WAVES * p;
-            const bool mine = WAVES * (p + 1) <= PAIRS || pair < PAIRS;
-            const int sbk = 2 * min(pair, PAIRS - 1) + half;
-            float dv;
-            int bs;
-            const uint2 packed = q8k_quantize_row32(xv[p], lane, dv, bs);
-            if (mine) {
-                reinterpret_cast<uint2 *>(ys)[sbk * 32 + ql] = packed;
-                if ((ql & 3) == 3) bsum[sbk * 8 + (ql >> 2)] = bs;
-                if (ql == 0) yds[sbk] = dv;
-            }
+            for (int p = 0; p < PASSES; p++) quantize_pass(p);
         }
         __syncthreads();
     }
@@ -909,6 +927,12 @@ __global__ __launch_bounds__(512) void gemv_q4k_cu_kcut_kernel(Q4KCuArgs a) {
     for (int j = PRE; j < NB; j++) request(ring[j], j);
 #pragma unroll
     for (int i = 0; i < NSTEPS; i++) {
+        if constexpr (STAGED && !NOACT) {
+            // before steps 2p - 2 and 2p - 1: pass p, for steps 2p and 2p + 1; a barrier before step 2p makes it visible
+            // (the pass behind the step's re-request instead of ahead of the step: 7.62 us against 7.19-7.3)
+            if (i % 2 == 0 && i / 2 + 1 < PASSES) quantize_pass(i / 2 + 1);
+            if (i % 2 == 0 && i > 0) __syncthreads();
+        }
         compute(ring[i % NB], i);
         if (i + NB < NSTEPS) request(ring[i % NB], i + NB);
     }
@@ -944,13 +968,22 @@ static int launch_q4k_cu_kcut(const Q4KArgs &ka, hipStream_t st, int ablate = 0)
     const dim3 grid(static_cast<unsigned>((2 * tiles16 + 1) / 2)), block(512);  // two half tiles per workgroup
     const Q4KCuArgs ca{ka.w, ka.x, ka.out, ka.residual, static_cast<uint32_t>(ka.sb_stride), ka.rows, ka.row_skip, tiles16};
     switch (ablate) {
-        case 0: hipLaunchKernelGGL((gemv_q4k_cu_kcut_kernel<4, 7>), grid, block, 0, st, ca); break;
+        case 0:
+            // CAMELID_HIP_Q4K_KCUT_STAGED=0: the whole row quantized before the walk (7.63 us against 7.19 at 4096 x 14336)
+            if (env_int("CAMELID_HIP_Q4K_KCUT_STAGED", 1)) {
+                hipLaunchKernelGGL((gemv_q4k_cu_kcut_kernel<4, 7, 0, true>), grid, block, 0, st, ca);
+                CML_COUNT_LAUNCH("q4k.dot.wg8.kcut.fused");
+            } else {
+                hipLaunchKernelGGL((gemv_q4k_cu_kcut_kernel<4, 7>), grid, block, 0, st, ca);
+                CML_COUNT_LAUNCH("q4k.dot.wg8.kcut.fused.whole_row");
+            }
+            return CML_OK;
         case 1: hipLaunchKernelGGL((gemv_q4k_cu_kcut_kernel<4, 7, 1>), grid, block, 0, st, ca); break;
         case 4: hipLaunchKernelGGL((gemv_q4k_cu_kcut_kernel<4, 7, 4>), grid, block, 0, st, ca); break;
         case 7: hipLaunchKernelGGL((gemv_q4k_cu_kcut_kernel<4, 7, 7>), grid, block, 0, st, ca); break;
         default: return fail(CML_ERR_INVALID, "ablation mask must be 1, 4 or 7");
     }
-    if (ablate) CML_COUNT_LAUNCH("q4k.calibrate.wg8.kcut"); else CML_COUNT_LAUNCH("q4k.dot.wg8.kcut.fused");
+    CML_COUNT_LAUNCH("q4k.calibrate.wg8.kcut");
     return CML_OK;
 }
 

@@ -495,7 +495,10 @@ def test_q4k_eight_wave_launch_under_the_k_cut_is_the_two_launch_path(rows):
             got_band = G.gpu_matmul_f32(band, x)
         with G.env(CAMELID_HIP_Q4K_CU=0), G.engaged(r"^quantize\.q8_k$", r"^q4k\.dot\.", none=(r"^q4k\.dot\.wg8",)):
             two_launches = G.gpu_matmul_f32(w, x)
+        with G.env(CAMELID_HIP_Q4K_KCUT_STAGED=0), G.engaged(r"^q4k\.dot\.wg8\.kcut\.fused\.whole_row$", none=(r"^q4k\.dot\.wg8\.kcut\.fused$",)):
+            whole_row = G.gpu_matmul_f32(w, x)   # the row quantized before the walk instead of pass by pass along it
         assert G.same_bits(got, two_launches), (rows, i)
+        assert G.same_bits(got, whole_row), (rows, i)
         assert G.same_bits(got_band, got[5:rows - 4]), (rows, i)
         if i != 1:
             want = oracle.matmul(fmt, wire, cols, x[None, :], order=EXACT_ORDER[fmt], threads=16)[0]
