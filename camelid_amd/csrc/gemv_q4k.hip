@@ -1522,8 +1522,13 @@ struct MoeDownSumArgs {
     float *out;               // [rows]
 };
 
-template <bool RING, int NSTEPS = 0>
+// OWN (parts of at most 16 super-blocks): every wave stages the activation of its own (slot, K part) and nothing else --
+// four 16-byte loads per lane, all requested ahead of the first weight requests, written to the wave's own stretch of
+// LDS -- so no workgroup barrier stands before the walk (the shared staging loop made three dependent trips to
+// memory, then a barrier for the slowest of eight waves).
+template <bool RING, int NSTEPS = 0, bool OWN = false>
 __global__ __launch_bounds__(512) void moe_down_sum_q4k_kernel(MoeDownSumArgs a) {
+    static_assert(!OWN || RING, "own staging rides with the ring walk");
     // RING: three 2-super-block buffers instead of two 4-super-block ones, as in the matvec above
     // (every K part an even number of super-blocks, at least six: the launcher checks)
     constexpr int U = RING ? 2 : 4;
@@ -1564,6 +1569,34 @@ __global__ __launch_bounds__(512) void moe_down_sum_q4k_kernel(MoeDownSumArgs a)
     const int c16 = n_sb * 16, n16 = S * c16;
     uint4 *dst = reinterpret_cast<uint4 *>(ys);
     const uint4 *src = reinterpret_cast<const uint4 *>(a.q);
+    if constexpr (OWN) {
+        const int base16 = (slot * n_sb + s0) * 16, n_loc16 = (s1 - s0) * 16;  // this wave's stretch: at most 256 pieces
+        uint4 v[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) v[k] = src[base16 + min(lane + 64 * k, n_loc16 - 1)];
+        const float yd_mine = a.yd[slot * n_sb + s0 + min(lane, s1 - s0 - 1)];
+        __builtin_amdgcn_sched_barrier(0);
+        if (served) {
+            load_buffer(ring[0], s0);
+            load_buffer(ring[1], s0 + U);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int i = lane + 64 * k;  // lanes 2j, 2j+1 hold the halves of a 32-value group
+            int sum = bytesum16(v[k]);
+            sum += row_shr_i32<1>(sum);
+            if (i < n_loc16) {
+                dst[base16 + i] = v[k];
+                if (i & 1) bsum[(base16 + i) >> 1] = sum;
+            }
+        }
+        if (lane < s1 - s0) yds[slot * n_sb + s0 + lane] = yd_mine;
+        // written and read by this wave alone
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    } else {
     uint4 first = src[min(tid, n16 - 1)];
     __builtin_amdgcn_sched_barrier(0);
     if (served) {
@@ -1586,6 +1619,7 @@ __global__ __launch_bounds__(512) void moe_down_sum_q4k_kernel(MoeDownSumArgs a)
     }
     for (int i = tid; i < S * n_sb; i += nthreads) yds[i] = a.yd[i];
     __syncthreads();
+    }
 
     float acc[1] = {0.0f};
     if (served) {
@@ -1702,7 +1736,9 @@ int launch_moe_down_sum_q4k(const cml_weight *down, int n_experts, int n_slots, 
     a.out = out;
     const bool ring = env_int("CAMELID_HIP_Q4K_RING", 1) && !env_int("CAMELID_HIP_Q4K_CLAMPED_LOADS", 0) && n_sb % (2 * shape.ksplit) == 0 &&
                       n_sb / (2 * shape.ksplit) >= 3 && a.sb_stride < (int64_t(1) << 31);
-    if (ring && n_sb == 14 * shape.ksplit)  // K parts of 3584 values (Mixtral's 14336 cut four ways): seven steps
+    if (ring && n_sb == 14 * shape.ksplit && env_int("CAMELID_HIP_MOE_DOWN_OWN_STAGING", 1))  // K parts of 3584 values (Mixtral's 14336 cut four ways): seven steps
+        hipLaunchKernelGGL((moe_down_sum_q4k_kernel<true, 7, true>), dim3(static_cast<unsigned>(rows / 16)), dim3(64 * waves), lds, st, a);
+    else if (ring && n_sb == 14 * shape.ksplit)
         hipLaunchKernelGGL((moe_down_sum_q4k_kernel<true, 7>), dim3(static_cast<unsigned>(rows / 16)), dim3(64 * waves), lds, st, a);
     else if (ring) hipLaunchKernelGGL(moe_down_sum_q4k_kernel<true>, dim3(static_cast<unsigned>(rows / 16)), dim3(64 * waves), lds, st, a);
     else hipLaunchKernelGGL(moe_down_sum_q4k_kernel<false>, dim3(static_cast<unsigned>(rows / 16)), dim3(64 * waves), lds, st, a);
