@@ -597,6 +597,9 @@ static int launch_b32_f32_p(const cml_weight *w, const float *x, float *out, hip
         // Q8_0 rows of 4096 values (the longest the register prologue takes) on tall matrices: sixteen
         // waves (16384 x 4096: 14.2 -> 12.7 us, 32000 x 4096: 24.7 -> 22.3); slower for Q4_0 and shorter rows
         if (FMT == CML_Q8_0 && ba.nb == 128 && ba.rows >= 224 * 16 * (64 / P)) waves = 16;
+        // Q4_0 on a vocabulary-sized matrix: sixteen waves halve the number of workgroups that each quantize the
+        // token (128256 x 3072: 34.1 -> 33.3 us; Q8_0 there is the same 59.2 us with 4, 8 or 16)
+        if (FMT == CML_Q4_0 && ba.nb <= 128 && ba.rows >= 65536) waves = 16;
     }
     if (two && waves != 4) waves = 8;  // the two-token variants: four or eight waves
     if (P > 16) waves = 8;
