@@ -247,6 +247,9 @@ private:
     std::string name_;
     std::vector<uint8_t> wire_;  // kept until the first use fixes the column count
     mutable cml_weight *weight_ = nullptr;
+    // before the row length is known: the tensor resident as rows of ONE block each, for dequantize_elements
+    // (an embedding table is only ever read that way); released when a matvec fixes the row length
+    mutable cml_weight *block_view_ = nullptr;
     mutable size_t cols_ = 0;
     mutable std::map<std::pair<size_t, size_t>, cml_weight *> bands_;
     mutable DeviceScratch out_, q_, s_;

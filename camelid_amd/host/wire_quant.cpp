@@ -199,6 +199,8 @@ void WireQuant::release() {
     bands_.clear();
     if (weight_) cml_weight_free(weight_);
     weight_ = nullptr;
+    if (block_view_) cml_weight_free(block_view_);
+    block_view_ = nullptr;
 }
 
 WireQuant &WireQuant::operator=(WireQuant &&o) noexcept {
@@ -209,9 +211,11 @@ WireQuant &WireQuant::operator=(WireQuant &&o) noexcept {
         name_ = std::move(o.name_);
         wire_ = std::move(o.wire_);
         weight_ = o.weight_;
+        block_view_ = o.block_view_;
         cols_ = o.cols_;
         bands_ = std::move(o.bands_);
         o.weight_ = nullptr;
+        o.block_view_ = nullptr;
         o.bands_.clear();
     }
     return *this;
@@ -231,6 +235,8 @@ size_t WireQuant::rows_for(size_t in_dim) const {
         dev(cml_weight_upload(ggml_type_id(format_), static_cast<int64_t>(rows), static_cast<int64_t>(in_dim), wire_.data(), wire_.size(), &weight_),
             "cml_weight_upload");
         cols_ = in_dim;
+        if (block_view_) cml_weight_free(block_view_);  // the row layout serves dequantize_elements from here on
+        block_view_ = nullptr;
         auto *self = const_cast<WireQuant *>(this);
         self->wire_.clear();
         self->wire_.shrink_to_fit();
@@ -389,18 +395,21 @@ std::vector<float> WireQuant::dequantize_elements(size_t start, size_t len) cons
     std::vector<float> out(len);
     if (len == 0) return out;
     if (!weight_) {
-        // The row length is not known yet (it is fixed by the first matvec) and this call must
-        // not fix it: decode from a temporary upload of just the covering blocks, seen as rows of
-        // one block, and leave the host bytes and the resident state as they are (the reference's
-        // dequantize_elements has no side effect either, src/gemma4_runtime.rs:1154).
+        // The row length is not known yet (it is fixed by the first matvec) and this call must not fix it (the
+        // reference's dequantize_elements has no side effect either, src/gemma4_runtime.rs:1154).  The tensor goes to
+        // the device ONCE, seen as rows of one block each, and stays there: a token's embedding row is then a row
+        // band of that view -- no allocation, upload or free per call (an embedding table is read this way for every
+        // token and never gets a matvec).
         const size_t bv = values_per_block(format_), bb = bytes_per_block(format_);
         const size_t b0 = start / bv, b1 = (start + len + bv - 1) / bv;
         ensure_device();
+        if (!block_view_)
+            dev(cml_weight_upload(ggml_type_id(format_), static_cast<int64_t>(wire_.size() / bb), static_cast<int64_t>(bv), wire_.data(),
+                                  wire_.size(), &block_view_),
+                "cml_weight_upload");
         cml_weight *raw = nullptr;
-        dev(cml_weight_upload(ggml_type_id(format_), static_cast<int64_t>(b1 - b0), static_cast<int64_t>(bv), wire_.data() + b0 * bb,
-                              (b1 - b0) * bb, &raw),
-            "cml_weight_upload");
-        // freed on every way out of this block, an exception from reserve() or dev() included
+        dev(cml_weight_slice(block_view_, static_cast<int64_t>(b0), static_cast<int64_t>(b1 - b0), &raw), "cml_weight_slice");
+        // the view handle is released on every way out of this block, an exception from reserve() or dev() included
         const std::unique_ptr<cml_weight, void (*)(cml_weight *)> tmp(raw, cml_weight_free);
         float *od = static_cast<float *>(out_.reserve((b1 - b0) * bv * sizeof(float)));
         dev(cml_dequantize(tmp.get(), od, nullptr), "cml_dequantize");
