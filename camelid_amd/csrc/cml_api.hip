@@ -74,6 +74,7 @@ struct EnvSnapshot {
     std::vector<std::pair<std::string, int>> knobs;  // names without the CAMELID_HIP_ prefix
 };
 static std::atomic<const EnvSnapshot *> g_env{nullptr};
+static std::vector<const EnvSnapshot *> g_env_retired;  // guarded by g_mutex
 extern "C" char **environ;
 
 static void load_env_snapshot() {
@@ -91,9 +92,10 @@ static void load_env_snapshot() {
         for (const char *a : always) take = take || key == a;
         if (take) snap->knobs.emplace_back(std::move(key), atoi(eq + 1));
     }
-    // superseded snapshots are kept: a launch on another thread may still be reading one, and
-    // reloads only happen in tests
-    g_env.store(snap, std::memory_order_release);
+    // a superseded snapshot is not freed here -- a launch on another thread may still be walking it -- but
+    // retired, and freed by cml_shutdown, which by contract runs alone (callers hold g_mutex)
+    const EnvSnapshot *old = g_env.exchange(snap, std::memory_order_acq_rel);
+    if (old) g_env_retired.push_back(old);
 }
 
 int env_int(const char *name, int dflt) {
@@ -240,6 +242,8 @@ void cml_shutdown(void) {
         g_seam_buf = nullptr;
         g_seam_bytes = 0;
     }
+    for (const EnvSnapshot *e : g_env_retired) delete e;  // snapshots superseded by cml_reload_env
+    g_env_retired.clear();
     g_device.store(-1, std::memory_order_release);
 }
 
