@@ -51,6 +51,41 @@ TRAFFIC_READINGS: dict = {
     "q6k_128256x3072_n16": (356138676, "q6k.mfma.tile", "gemm_q6k_mfma_kernel<1, 1, false, 2, 2, 1, true>"),      # 1.074 x
 }
 
+# rocprofv3 --kernel-trace averages of the dominant kernel, read at run time from the committed summaries (never copied
+# into this file): config -> (summary under profiles/, kernel symbol prefix, launch-counter prefix the step must have fired).
+ROCPROF_SUMMARIES: dict = {
+    "q4k_14336x4096_n1": ("profiles/gemv_q4k_fused_quantize_14336x4096_n1.txt", "void cml::gemv_q4k_cu_kernel<8, 0, 1>", "q4k.dot.wg8.fused"),
+    "q4k_4096x14336_n1": ("profiles/gemv_q4k_4096x14336_n1.txt", "void cml::gemv_q4k_cu_kcut_kernel<4, 7", "q4k.dot.wg8.kcut.fused"),
+    "q4k_14336x4096_n16": ("profiles/gemm_q4k_mfma_14336x4096_n16.txt", "void cml::gemm_q4k_mfma_pair_kernel<false>", "q4k.mfma.pair"),
+    "q4k_14336x4096_n64": ("profiles/gemm_q4k_mfma_14336x4096_n64.txt", "void cml::gemm_q4k_mfma_kernel<4, 1,", "q4k.mfma.tile.g4t1"),
+    "q8_0_8192x2048_n1": ("profiles/gemv_q8_0_8192x2048_n1.txt", "void cml::gemv_b32_kernel<", "q8_0.dot."),
+    "q6k_128256x3072_n1": ("profiles/gemv_q6k_128256x3072_n1.txt", "void cml::gemv_q6k_kernel<", "q6k.dot."),
+    "q4_0_128256x3072_n1": ("profiles/gemv_q4_0_128256x3072_n1.txt", "void cml::gemv_b32_kernel<", "q4_0.dot."),
+}
+
+
+def rocprof_summary(config: str, kernels_of_step) -> dict | None:
+    """The profiler's average duration of this configuration's dominant kernel, from the committed summary, with its source;
+    None when there is no summary, or when this run launched another kernel family than the summary was taken for."""
+    entry = ROCPROF_SUMMARIES.get(config)
+    if entry is None or not any(k.startswith(entry[2]) for k in kernels_of_step):
+        return None
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), entry[0])
+    try:
+        best = None
+        for line in open(path):
+            if line.startswith('"' + entry[1]):
+                cells = line.rsplit('",', 1)[1].split(",")   # Calls, TotalDurationNs, AverageNs, ...
+                calls, avg = int(cells[0]), float(cells[2])
+                if best is None or calls > best[0]:
+                    best = (calls, avg, line.split('",', 1)[0].strip('"'))
+        if best is None:
+            return None
+        return {"us_per_launch": round(best[1] / 1e3, 3), "calls": best[0], "file": entry[0], "kernel": best[2]}
+    except OSError:
+        return None
+
+
 # name -> (format, rows, cols, tokens): BASELINE.json's configurations.
 CONFIGS = {
     "q4k_14336x4096_n1": ("Q4_K", 14336, 4096, 1),   # the metric's configuration (Llama-3-8B FFN gate/up)
@@ -902,6 +937,7 @@ def main() -> int:
                      "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic_bytes, "traffic_source": traffic_source,
                      "us_per_launch": round(kern_ms * 1e3, 3),
+                     "rocprofv3": rocprof_summary(args.config, kernels_of_step),
                      "cache_warm_us_per_launch": None if warm_ms is None else round(warm_ms * 1e3, 3),
                      "cache_warm_gbs": None if warm_ms is None else round(alg_bytes / (warm_ms * 1e-3) / 1e9, 2),
                      "shared_activation_us_per_launch": None if shared_ms is None else round(shared_ms * 1e3, 3),
