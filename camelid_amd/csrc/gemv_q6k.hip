@@ -344,6 +344,114 @@ __global__ __launch_bounds__(256) void gemv_q6k_kernel(Q6KArgs a) {
     }
 }
 
+// ---- one token on a weight whose shape the policy cuts K for: eight-wave workgroups, one launch ----
+//
+// Few row tiles, long rows -- the FFN down projection in Q6_K (4096 x 14336: 56 super-blocks cut four ways).  The
+// two-launch form (a quantizing launch, then gemv_q6k_kernel) takes 12.3 us per step for a 10.1 us matvec.  Here a
+// workgroup's eight waves are 8 / KS row tiles (8 rows each) x KS parts of NSTEPS super-blocks; the arithmetic is
+// q6k_load / q6k_compute, one super-block per step, and the KS partial chains of a row are added left to right
+// through LDS -- the association of gemv_q6k_kernel under the same cut, so the same bits.  The workgroup quantizes
+// the row ONCE, a 32-lane half wave per super-block, pass by pass ALONG the walk: pass p produces, for every K part,
+// the four super-blocks its steps 4p .. 4p + 3 read (the part's two waves take two each), so the walk starts after
+// one pass and the others run between steps, with a barrier ahead of the first step that reads a pass.  Every f32
+// request is out before the first weight request (an execution barrier), and the weights stream through a ring of
+// NB one-super-block buffers.
+template <int KS, int NSTEPS, int NB = 4>
+__global__ __launch_bounds__(512) void gemv_q6k_cu_kcut_kernel(Q6KArgs a) {
+    constexpr int WAVES = 8, LPS = 8, RPW = kWave / LPS, TPW = WAVES / KS, NSB = KS * NSTEPS, PRE = 2;
+    constexpr int PER_PASS = 2 * TPW;                       // super-blocks a pass gives every part
+    constexpr int PASSES = (NSTEPS + PER_PASS - 1) / PER_PASS;
+    static_assert(NSTEPS >= NB && WAVES % KS == 0, "K parts of at least one full ring");
+    __shared__ __attribute__((aligned(16))) int8_t ys[NSB * 256];
+    __shared__ int bsum16[NSB * 16];
+    __shared__ float yds[NSB];
+    __shared__ float part[WAVES * RPW];
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    const int tile_in_wg = wave / KS, kpart = wave - tile_in_wg * KS;
+    const int s0 = kpart * NSTEPS;  // first super-block of this wave's part
+
+    // the f32 activation: in pass p this wave's halves take super-blocks PER_PASS * p + 2 * tile_in_wg + {0, 1} of its part
+    const int half = lane >> 5, ql32 = lane & 31;
+    auto unit_of = [&](int p) __attribute__((always_inline)) -> int { return PER_PASS * p + 2 * tile_in_wg + half; };
+    float4 xv[PASSES][2];
+#pragma unroll
+    for (int p = 0; p < PASSES; p++) {
+        const float4 *x4 = reinterpret_cast<const float4 *>(a.x) + (s0 + min(unit_of(p), NSTEPS - 1)) * 64 + ql32 * 2;
+        xv[p][0] = x4[0];
+        xv[p][1] = x4[1];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();  // execution only: every activation request of the workgroup is out
+    __builtin_amdgcn_sched_barrier(0);
+
+    const int r = lane / LPS, l = lane - r * LPS;
+    const int row = (blockIdx.x * TPW + tile_in_wg) * RPW + r;
+    const bool live = row < a.rows;
+    const int64_t arow = live ? row : a.rows - 1;  // rows past the end (grid rounding) re-read the last row and store nothing
+    const uint8_t *ql = a.ql + arow * a.ql_stride;
+    const uint8_t *qh = a.qh + arow * a.qh_stride;
+    const uint8_t *sc = a.sc + arow * a.sc_stride;
+    const uint8_t *dp = a.d + arow * a.d_stride;
+    Q6KRegs<1> ring[NB];
+    auto request = [&](Q6KRegs<1> &b, int step) __attribute__((always_inline)) {
+        q6k_load(b, ql, qh, sc, dp, l, s0 + step, s0 + NSTEPS);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+#pragma unroll
+    for (int k = 0; k < PRE; k++) request(ring[k], k);
+
+    // every wave runs every pass (a half without a super-block of its own in the last pass redoes the part's last one
+    // and stores nothing): the f32 loads above are used unconditionally and stay ahead of the weight requests
+    auto quantize_pass = [&](int p) __attribute__((always_inline)) {
+        const int u = unit_of(p);
+        float dv;
+        int bs;
+        const uint2 packed = q8k_quantize_row32(xv[p], lane, dv, bs);
+        int s16 = sdot4(packed.y, 0x01010101u, sdot4(packed.x, 0x01010101u, 0));
+        s16 += row_shr_i32<1>(s16);  // odd lanes: the sum of 16 consecutive quants
+        if (u < NSTEPS) {
+            const int sbk = s0 + u;
+            reinterpret_cast<uint2 *>(ys)[sbk * 32 + ql32] = packed;
+            if (ql32 & 1) bsum16[sbk * 16 + (ql32 >> 1)] = s16;
+            if (ql32 == 0) yds[sbk] = dv;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    quantize_pass(0);
+    __syncthreads();
+
+    float acc[1] = {0.0f};
+    auto compute = [&](const Q6KRegs<1> &b, int step) __attribute__((always_inline)) {
+        q6k_compute<1, false, 1>(b, l, s0 + step, s0 + NSTEPS, ys, bsum16, yds, NSB, acc, nullptr);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+#pragma unroll
+    for (int j = PRE; j < NB; j++) request(ring[j], j);
+#pragma unroll
+    for (int i = 0; i < NSTEPS; i++) {
+        if (i % PER_PASS == 0) {  // the first step that reads pass i / PER_PASS: the next pass goes ahead of it
+            if (i / PER_PASS + 1 < PASSES) quantize_pass(i / PER_PASS + 1);
+            if (i > 0) __syncthreads();
+        }
+        compute(ring[i % NB], i);
+        if (i + NB < NSTEPS) request(ring[i % NB], i + NB);
+    }
+    if (l == LPS - 1) part[wave * RPW + r] = acc[0];
+    __syncthreads();
+    if (tid < TPW * RPW) {
+        const int tw = tid / RPW, rr = tid - tw * RPW;
+        const int orow = (blockIdx.x * TPW + tw) * RPW + rr;
+        if (orow < a.rows) {
+            float v = part[(tw * KS) * RPW + rr];
+#pragma unroll
+            for (int k = 1; k < KS; k++) v = v + part[(tw * KS + k) * RPW + rr];
+            if (a.residual) v = v + a.residual[orow];
+            a.out[orow] = v;
+        }
+    }
+}
+
 static int pick_ksplit_q6k(int64_t rows, int64_t n_sb) {
     const int forced = env_int("CAMELID_HIP_Q6K_KSPLIT", 0);
     if ((forced == 1 || forced == 2 || forced == 4) && forced <= n_sb) return forced;
@@ -355,6 +463,12 @@ static int pick_ksplit_q6k(int64_t rows, int64_t n_sb) {
 }
 
 int q6k_ksplit_for(int64_t rows, int64_t n_sb) { return pick_ksplit_q6k(rows, n_sb); }
+
+// The K-cut eight-wave launch serves rows of 14336 values cut four ways (CAMELID_HIP_Q6K_CU=0: the two-launch form).
+static bool q6k_cu_kcut_serves(int64_t rows, int64_t n_sb) {
+    return n_sb == 56 && pick_ksplit_q6k(rows, n_sb) == 4 && env_int("CAMELID_HIP_Q6K_CU", 1) != 0;
+}
+bool gemv_q6k_long_rows_fuse(const cml_weight *w) { return w->fmt == CML_Q6_K && q6k_cu_kcut_serves(w->rows, w->nb); }
 
 static size_t q6k_lds_bytes(int nt, int n_sb) {
     return static_cast<size_t>(nt) * n_sb * (256 + 64) + ((static_cast<size_t>(nt) * n_sb + 3) & ~size_t(3)) * 4 + 4 * nt * 8 * 4;
@@ -566,6 +680,13 @@ int launch_gemv_q6k_f32(const cml_weight *w, const float *x, float *out, hipStre
     const unsigned gx = static_cast<unsigned>((tiles + tiles_per_wg - 1) / tiles_per_wg);
     const size_t lds = q6k_lds_bytes(n_tokens, ka.n_sb);
     if (lds > 64 * 1024) return fail(CML_ERR_UNSUPPORTED, "Q6_K activation of %d super-blocks exceeds the LDS staging limit", ka.n_sb);
+    if (n_tokens == 1 && q6k_cu_kcut_serves(ka.rows, ka.n_sb)) {
+        // (ring of 3 / 4 / 5 / 6 one-super-block buffers: 10.61 / 10.42 / 10.86 / 11.32 us at 4096 x 14336)
+        hipLaunchKernelGGL((gemv_q6k_cu_kcut_kernel<4, 14>), dim3(static_cast<unsigned>((tiles + 1) / 2)), dim3(512), 0, st, ka);
+        CML_COUNT_LAUNCH("q6k.dot.wg8.kcut.fused");
+        CML_HIP_TRY(hipGetLastError());
+        return CML_OK;
+    }
     if (n_tokens == 2) {
         hipLaunchKernelGGL((gemv_q6k_kernel<2, false, false, 2, true>), dim3(gx, 1), dim3(256), lds, st, ka);
         CML_COUNT_LAUNCH("q6k.dot.buffers.fused");

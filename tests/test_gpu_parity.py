@@ -505,6 +505,44 @@ def test_q4k_eight_wave_launch_under_the_k_cut_is_the_two_launch_path(rows):
             assert G.max_rel(got, want) <= TOL, (rows, i)
 
 
+@pytest.mark.parametrize("rows", [4096, 3100, 6100])
+def test_q6k_eight_wave_launch_under_the_k_cut_is_the_two_launch_path(rows):
+    """Q6_K rows of 14336 values on up to 6136 rows (the FFN down projection: the shape policy cuts K four ways):
+    cml_matmul_f32 with one token runs ONE launch whose eight-wave workgroups quantize the row once each, pass by
+    pass along the walk.  Same bits as the quantizing launch followed by the four-wave matvec (CAMELID_HIP_Q6K_CU=0)
+    on activations built to break a quantizer, and with a residual-free row count that is not a multiple of the
+    workgroup's 16 rows; within 1e-5 of the oracle's uncut chain."""
+    fmt, cols = oracle.Q6_K, 14336
+    rng = np.random.default_rng(9200 + rows)
+    wire = G.synth_weight(fmt, rows, cols, seed=9300 + rows)
+    w = Weight.upload(fmt, rows, cols, wire)
+    acts = rng.standard_normal((4, cols)).astype(np.float32)
+    a = acts[0]
+    a[0:256] = 0.0
+    a[256 + 5], a[256 + 6] = 3.5, -3.5
+    a[512 + 6], a[512 + 5] = 3.5, -3.5
+    a[768 + 3], a[768 + 100] = -4.0, 4.0
+    a[1024 + 3], a[1024 + 200] = 4.0, -4.0
+    a[13 * 1024 + 130], a[13 * 1024 + 255] = -4.5, 4.5
+    a[-256:] = 2.0                                    # the last super-block: equal values
+    acts[1, 3], acts[1, 9000] = np.nan, np.nan
+    acts[1, 256 * 55:] = np.nan
+    acts[2, 1::2] = -acts[2, ::2]
+    band = w.slice(5, rows - 9)
+    for i, x in enumerate(acts):
+        G.say(f"Q6_K eight-wave K-cut launch {rows}x14336 act={i}")
+        with G.engaged(r"^q6k\.dot\.wg8\.kcut\.fused$", none=(r"^q6k\.dot\.buffers", r"^q6k\.dot\.deep", r"^quantize\.")):
+            got = G.gpu_matmul_f32(w, x)
+            got_band = G.gpu_matmul_f32(band, x)
+        with G.env(CAMELID_HIP_Q6K_CU=0), G.engaged(r"^quantize\.q8_k$", r"^q6k\.dot\.", none=(r"^q6k\.dot\.wg8",)):
+            two_launches = G.gpu_matmul_f32(w, x)
+        assert G.same_bits(got, two_launches), (rows, i)
+        assert G.same_bits(got_band, got[5:rows - 4]), (rows, i)
+        if i != 1:
+            want = oracle.matmul(fmt, wire, cols, x[None, :], order=EXACT_ORDER[fmt], threads=16)[0]
+            assert G.max_rel(got, want) <= TOL, (rows, i)
+
+
 @pytest.mark.parametrize("rows,cols", [(190, 3072), (64, 256), (333, 4096), (40, 14336), (77, 1280)])
 def test_q4k_fused_two_tokens_is_the_two_step_path(rows, cols):
     """Two-token cml_matmul_f32 on Q4_K quantizes both rows inside the matvec kernel: the bits of
