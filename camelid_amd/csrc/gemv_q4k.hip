@@ -699,15 +699,14 @@ struct Q4KCuArgs {
 // -- every cell the one-token result, bit for bit (the same q4k_compute).  The weight streams once for the NT tokens
 // and the vector work per step grows by about 60 instructions per token, which the stream hides up to three
 // tokens and nearly at four.
-template <int NSTEPS, int ABLATE = 0, int NT = 1>
-__global__ __launch_bounds__(512) void gemv_q4k_cu_kernel(Q4KCuArgs a) {
+template <int NSTEPS, int ABLATE = 0, int NT = 1, int WAVES = 8>
+__global__ __launch_bounds__(WAVES * 64) void gemv_q4k_cu_kernel(Q4KCuArgs a) {
     const uint8_t *__restrict__ w = a.w;
     const float *__restrict__ x = a.x;
     float *__restrict__ out = a.out;
     const float *__restrict__ residual = a.residual;
     const uint32_t sb_stride = a.sb_stride;
     const int rows = a.rows, row_skip = a.row_skip, tiles16 = a.tiles16;
-    constexpr int WAVES = 8;
     constexpr int NSB = 2 * NSTEPS;  // super-blocks per row
     constexpr int NB = 3, PRE = 2;   // ring slots; slots requested before the quantizer
     static_assert(NSTEPS >= NB && NSB <= 2 * WAVES, "one quantizer pass covers a row");
@@ -990,13 +989,31 @@ static int launch_q4k_cu_kcut(const Q4KArgs &ka, hipStream_t st, int ablate = 0)
 // Whether the launch above serves this call: rows of 6 to 16 super-blocks (an even count: 1536 to 4096 values), no
 // K cut (the shape policy gives that from 12288 rows on, i.e. at least 192 eight-wave workgroups), a stride the
 // 32-bit lane offsets can hold.  One and two tokens only while the launch is at most one workgroup per compute unit
-// (16384 rows): beyond that the four-wave workgroups spread more evenly (18944 x 3584: 8.77 us against 9.33 with
-// eight waves; three tokens 13.3 against 16.0 for what served them before, so those stay).
+// (with more than 256 workgroups some units carry two: 18944 x 3584 with eight waves 9.33 us against 8.77 for the
+// four-wave workgroups), which wider workgroups keep up to 24576 rows.
 // CAMELID_HIP_Q4K_CU=0 keeps the four-wave launch.
 constexpr int kComputeUnits = 256;  // MI355X
+// Waves per workgroup of that launch, 0 when it does not serve the row count: the smallest of 8, 10 and 12 (three
+// tokens: and 16) that keeps the launch within one workgroup per compute unit -- wider than eight for rows of 14 or 16
+// super-blocks and up to three tokens; three tokens take eight waves at any row count beyond.  Measured, us per step,
+// wide against what served the shape before: 18944 x 3584 (ten waves) 7.56 / 8.24 / 10.1 for one / two / three tokens
+// against 8.68 / 11.07 / 13.27; 24576 x 4096 (twelve) 9.87 / 10.67 / 11.9 against 10.09 / 12.44 / 14.75; sixteen waves
+// at 28672 and 32000 x 4096 lose to the 16-row waves for one and two tokens (11.7 against 11.25, 12.57 against 12.2,
+// 13.6 against 13.1) and win for three (14.3 and 15.2 against 15.1 and 15.5 with eight waves, 18.2 and 18.6 before).
+// CAMELID_HIP_Q4K_CU_WAVES considers that width only.
+static int q4k_cu_waves(const Q4KArgs &ka, int n_tokens) {
+    const int half_tiles = 2 * ((ka.rows + ka.row_skip + 15) / 16);
+    const int only = env_int("CAMELID_HIP_Q4K_CU_WAVES", 0);
+    for (int wv : {8, 10, 12, 16}) {
+        if (only && wv != only) continue;
+        if (wv > 8 && (ka.n_sb < 14 || n_tokens > 3)) break;
+        if (wv == 16 && n_tokens < 3) break;
+        if ((half_tiles + wv - 1) / wv <= kComputeUnits) return wv;
+    }
+    return n_tokens >= 3 ? 8 : 0;
+}
 static bool q4k_cu_serves(const Q4KArgs &ka, int ksplit, int n_tokens = 1) {
-    const int workgroups = (2 * ((ka.rows + ka.row_skip + 15) / 16) + 7) / 8;
-    return ksplit == 1 && (n_tokens >= 3 || workgroups <= kComputeUnits) && ka.n_sb <= 16 && ka.n_sb >= 6 && (ka.n_sb & 1) == 0 &&
+    return ksplit == 1 && ka.n_sb <= 16 && ka.n_sb >= 6 && (ka.n_sb & 1) == 0 && q4k_cu_waves(ka, n_tokens) != 0 &&
            ka.sb_stride < (int64_t(1) << 31) && env_int("CAMELID_HIP_Q4K_CU", 1) != 0 && !env_int("CAMELID_HIP_Q4K_CLAMPED_LOADS", 0) &&
            env_int("CAMELID_HIP_Q4K_RING", 1) != 0;
 }
@@ -1022,6 +1039,28 @@ static int launch_q4k_cu(const Q4KArgs &ka, int ablate, hipStream_t st, int n_to
         case 8: hipLaunchKernelGGL((gemv_q4k_cu_kernel<4, 0, NT_>), grid, block, 0, st, ca); break;           \
         case 6: hipLaunchKernelGGL((gemv_q4k_cu_kernel<3, 0, NT_>), grid, block, 0, st, ca); break;           \
         default: return fail(CML_ERR_UNSUPPORTED, "the eight-wave launch takes rows of 6 to 16 super-blocks");  \
+    }
+    const int waves = ablate ? 8 : q4k_cu_waves(ka, n_tokens);
+    if (waves > 8) {  // more than 256 eight-wave workgroups: wider ones, still one per compute unit
+#define CML_Q4K_CU_WIDE(NS_, NT_, WV_) \
+    hipLaunchKernelGGL((gemv_q4k_cu_kernel<NS_, 0, NT_, WV_>), dim3(static_cast<unsigned>((2 * tiles16 + WV_ - 1) / WV_)), dim3(WV_ * 64), 0, st, ca)
+#define CML_Q4K_CU_WIDE_WAVES(NS_, NT_)                                                  \
+    switch (waves) {                                                                     \
+        case 10: CML_Q4K_CU_WIDE(NS_, NT_, 10); break;                                   \
+        case 12: CML_Q4K_CU_WIDE(NS_, NT_, 12); break;                                   \
+        default: CML_Q4K_CU_WIDE(NS_, NT_, 16); break;                                   \
+    }
+        if (ka.n_sb == 16 && n_tokens == 1) { CML_Q4K_CU_WIDE_WAVES(8, 1) }
+        else if (ka.n_sb == 16 && n_tokens == 2) { CML_Q4K_CU_WIDE_WAVES(8, 2) }
+        else if (ka.n_sb == 16) { CML_Q4K_CU_WIDE_WAVES(8, 3) }
+        else if (n_tokens == 1) { CML_Q4K_CU_WIDE_WAVES(7, 1) }
+        else if (n_tokens == 2) { CML_Q4K_CU_WIDE_WAVES(7, 2) }
+        else { CML_Q4K_CU_WIDE_WAVES(7, 3) }
+#undef CML_Q4K_CU_WIDE_WAVES
+#undef CML_Q4K_CU_WIDE
+        if (n_tokens > 1) CML_COUNT_LAUNCH("q4k.dot.wg8.fused.tokens.wide");
+        else CML_COUNT_LAUNCH("q4k.dot.wg8.fused.wide");
+        return CML_OK;
     }
     if (n_tokens > 1) {
         if (ablate) return fail(CML_ERR_INVALID, "the ablations are one-token launches");
@@ -1320,7 +1359,8 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
             else if (half_tiles) { if (whole) CML_Q4K_LOADS(2, true); else CML_Q4K_LOADS(2, false); CML_COUNT_LAUNCH("q4k.calibrate.buffers"); }
             else { if (whole) CML_Q4K_LOADS(1, true); else CML_Q4K_LOADS(1, false); CML_COUNT_LAUNCH("q4k.calibrate.buffers"); }
 #undef CML_Q4K_LOADS
-        } else if (plain && a.n_tokens >= 2 && a.n_tokens <= q4k_cu_max_tokens(ka.n_sb) && q4k_rows_per_wave(tiles16, shape.ksplit, 1) == 8 &&
+        } else if (plain && a.n_tokens >= 2 && a.n_tokens <= q4k_cu_max_tokens(ka.n_sb) &&
+                   (a.n_tokens >= 3 || q4k_rows_per_wave(tiles16, shape.ksplit, 1) == 8) &&  // three tokens: at any row count (128256 x 4096: 55.0 us against 66.7)
                    q4k_ring(ka, shape.ksplit) && q4k_cu_serves(ka, shape.ksplit, static_cast<int>(a.n_tokens))) {
             if (int rc = launch_q4k_cu(ka, 0, st, static_cast<int>(a.n_tokens))) return rc;  // a few tokens replayed against each step's weight
         } else if (!grouped && !w2 && a.n_tokens > 2) {

@@ -465,6 +465,39 @@ def test_q4k_eight_wave_launch_serves_rows_of_six_to_sixteen_super_blocks(rows, 
         assert G.same_bits(former, got), (rows, cols, n, "former path")
 
 
+@pytest.mark.parametrize("rows,cols,tokens,kernel", [
+    (18944, 3584, (1, 2, 3), "wide"),     # ten waves per workgroup
+    (24570, 4096, (1, 2, 3), "wide"),     # twelve, the last 16-row tile partly filled
+    (28672, 4096, (3,), "wide"),          # sixteen: three tokens only
+    (40000, 4096, (3,), "eight"),         # three tokens beyond one workgroup per compute unit: eight waves
+])
+def test_q4k_wide_workgroups_beyond_one_eight_wave_workgroup_per_unit(rows, cols, tokens, kernel):
+    """More than 16384 rows of 14 or 16 super-blocks: the one-workgroup-per-compute-unit launch with ten, twelve or
+    sixteen waves per workgroup (and three tokens on eight waves at any row count).  The bits of the oracle and of
+    the four-wave / matrix-core paths that served these shapes before, also on a row band; the counters show the launch."""
+    fmt = oracle.Q4_K
+    rng = np.random.default_rng(8800 + rows)
+    wire = G.synth_weight(fmt, rows, cols, seed=8900 + rows)
+    w = Weight.upload(fmt, rows, cols, wire)
+    x = rng.standard_normal((3, cols)).astype(np.float32)
+    x[1, :256] = 0.0
+    x[2, 5], x[2, cols - 3] = 7.0, -7.0
+    want = oracle.matmul(fmt, wire, cols, x, order=EXACT_ORDER[fmt], threads=16)
+    band = w.slice(3, rows - 20)
+    for n in tokens:
+        G.say(f"Q4_K wide workgroups {rows}x{cols}, {n} tokens")
+        name = r"^q4k\.dot\.wg8\.fused" + (r"\.tokens" if n > 1 else "") + (r"\.wide$" if kernel == "wide" else "$")
+        with G.engaged(name, none=(r"^q4k\.mfma", r"^q4k\.dot\.ring", r"^q4k\.dot\.buffers", r"^quantize\.")):
+            got = G.gpu_matmul_f32(w, x[:n] if n > 1 else x[0])
+            got_band = G.gpu_matmul_f32(band, x[:n] if n > 1 else x[0])
+        got = np.asarray(got).reshape(n, rows)
+        assert G.same_bits(got, want[:n]), (rows, cols, n)
+        assert G.same_bits(np.asarray(got_band).reshape(n, rows - 20), got[:, 3:rows - 17]), (rows, cols, n, "band")
+        with G.env(CAMELID_HIP_Q4K_CU=0), G.engaged(none=(r"^q4k\.dot\.wg8",)):
+            former = np.asarray(G.gpu_matmul_f32(w, x[:n] if n > 1 else x[0])).reshape(n, rows)
+        assert G.same_bits(former, got), (rows, cols, n, "former path")
+
+
 @pytest.mark.parametrize("rows", [4096, 3100, 6100])
 def test_q4k_eight_wave_launch_under_the_k_cut_is_the_two_launch_path(rows):
     """Rows of 14336 values on 3072 to 6128 rows (the FFN down projection: the shape policy cuts K four ways):
