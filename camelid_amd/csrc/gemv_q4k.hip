@@ -709,7 +709,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_cu_kernel(Q4KCuArgs a) {
     const int rows = a.rows, row_skip = a.row_skip, tiles16 = a.tiles16;
     constexpr int NSB = 2 * NSTEPS;  // super-blocks per row
     constexpr int NB = 3, PRE = 2;   // ring slots; slots requested before the quantizer
-    static_assert(NSTEPS >= NB && NSB <= 2 * WAVES, "one quantizer pass covers a row");
+    constexpr int PASSES = (NSB + 2 * WAVES - 1) / (2 * WAVES);  // quantizer passes per token: 2 * WAVES super-blocks each
+    static_assert(NSTEPS >= NB && PASSES <= 2, "at most two quantizer passes cover a row");
     static_assert(NT >= 1 && NT <= 4 && (NT == 1 || ABLATE == 0), "up to four tokens; the ablations are one-token launches");
     constexpr bool NOACT = (ABLATE & 1) != 0, NOMATH = (ABLATE & 2) != 0, NOSTORE = (ABLATE & 4) != 0;
     using Regs = Q4KRegs<1>;
@@ -719,16 +720,19 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_cu_kernel(Q4KCuArgs a) {
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
 
-    // the f32 activation: wave w quantizes super-blocks 2w and 2w + 1 of every token, a half wave each
+    // the f32 activation: pass p of wave w quantizes super-blocks 2 (w + WAVES p) and the next of every token, a half wave each
     const int half = lane >> 5, ql = lane & 31;
-    const int sbk = 2 * wave + half;
-    float4 xv[NT][2];
+    float4 xv[NT][PASSES][2];
     if constexpr (!NOACT) {
 #pragma unroll
         for (int t = 0; t < NT; t++) {
-            const float4 *x4 = reinterpret_cast<const float4 *>(x) + (t * NSB + min(sbk, NSB - 1)) * 64 + ql * 2;
-            xv[t][0] = x4[0];
-            xv[t][1] = x4[1];
+#pragma unroll
+            for (int p = 0; p < PASSES; p++) {
+                const int sbk = 2 * (wave + WAVES * p) + half;
+                const float4 *x4 = reinterpret_cast<const float4 *>(x) + (t * NSB + min(sbk, NSB - 1)) * 64 + ql * 2;
+                xv[t][p][0] = x4[0];
+                xv[t][p][1] = x4[1];
+            }
         }
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -757,19 +761,23 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_cu_kernel(Q4KCuArgs a) {
         // Every wave runs the quantizer (a wave without a super-block of its own redoes the last one and
         // stores nothing): the f32 loads above are then used unconditionally, and the compiler cannot
         // sink them into a conditional block behind the weight requests.
-        const bool mine = NSB == 2 * WAVES || sbk < NSB;
 #pragma unroll
         for (int t = 0; t < NT; t++) {
-            float dv;
-            int bs;
-            const uint2 packed = q8k_quantize_row32(xv[t], lane, dv, bs);
-            if (mine) {
-                const int at = t * NSB + sbk;
-                reinterpret_cast<uint2 *>(ys)[at * 32 + ql] = packed;
-                if ((ql & 3) == 3) bsum[at * 8 + (ql >> 2)] = bs;
-                if (ql == 0) yds[at] = dv;
+#pragma unroll
+            for (int p = 0; p < PASSES; p++) {
+                const int sbk = 2 * (wave + WAVES * p) + half;
+                const bool mine = NSB == 2 * WAVES * PASSES || sbk < NSB;
+                float dv;
+                int bs;
+                const uint2 packed = q8k_quantize_row32(xv[t][p], lane, dv, bs);
+                if (mine) {
+                    const int at = t * NSB + sbk;
+                    reinterpret_cast<uint2 *>(ys)[at * 32 + ql] = packed;
+                    if ((ql & 3) == 3) bsum[at * 8 + (ql >> 2)] = bs;
+                    if (ql == 0) yds[at] = dv;
+                }
+                if constexpr (NT * PASSES >= 3) __builtin_amdgcn_sched_barrier(0);  // one pass at a time: the passes interleaved need too many registers
             }
-            if constexpr (NT >= 3) __builtin_amdgcn_sched_barrier(0);  // one token's pass at a time: the passes interleaved need too many registers
         }
         __syncthreads();
     }
@@ -986,11 +994,15 @@ static int launch_q4k_cu_kcut(const Q4KArgs &ka, hipStream_t st, int ablate = 0)
     return CML_OK;
 }
 
-// Whether the launch above serves this call: rows of 6 to 16 super-blocks (an even count: 1536 to 4096 values), no
-// K cut (the shape policy gives that from 12288 rows on, i.e. at least 192 eight-wave workgroups), a stride the
-// 32-bit lane offsets can hold.  One and two tokens only while the launch is at most one workgroup per compute unit
-// (with more than 256 workgroups some units carry two: 18944 x 3584 with eight waves 9.33 us against 8.77 for the
-// four-wave workgroups), which wider workgroups keep up to 24576 rows.
+// Whether the launch above serves this call: rows of 6 to 16 super-blocks (an even count: 1536 to 4096 values) or of
+// 20, 24 or 32 (5120, 6144, 8192 values: two quantizer passes), no K cut (the shape policy gives that from 12288 rows
+// on, i.e. at least 192 eight-wave workgroups), a stride the 32-bit lane offsets can hold.  One and two tokens only
+// while the launch is at most one workgroup per compute unit (with more than 256 workgroups some units carry two:
+// 18944 x 3584 with eight waves 9.33 us against 8.77 for the four-wave workgroups), which wider workgroups keep up to
+// 24576 rows.  The longer rows, us per step against the four-wave / matrix-core launches that served them: 13824 x 5120
+// 7.65 / 8.99 / 11.5 for one / two / three tokens against 8.62 / 10.66 / 17.2; 17920 x 5120 (ten waves) 9.45 against
+// 10.74; 16384 x 6144 9.94 against 10.5; 14336 x 8192 11.27 against 12.2; 28672 x 8192, three tokens, 27.3 against 32.5.
+// Seven waves per workgroup on 14336 x 4096 (256 workgroups instead of 224): 6.72 against 6.56.
 // CAMELID_HIP_Q4K_CU=0 keeps the four-wave launch.
 constexpr int kComputeUnits = 256;  // MI355X
 // Waves per workgroup of that launch, 0 when it does not serve the row count: the smallest of 8, 10 and 12 (three
@@ -1006,14 +1018,15 @@ static int q4k_cu_waves(const Q4KArgs &ka, int n_tokens) {
     const int only = env_int("CAMELID_HIP_Q4K_CU_WAVES", 0);
     for (int wv : {8, 10, 12, 16}) {
         if (only && wv != only) continue;
-        if (wv > 8 && (ka.n_sb < 14 || n_tokens > 3)) break;
+        if (wv > 8 && (ka.n_sb < 14 || ka.n_sb > 20 || n_tokens > 3)) break;
         if (wv == 16 && n_tokens < 3) break;
         if ((half_tiles + wv - 1) / wv <= kComputeUnits) return wv;
     }
     return n_tokens >= 3 ? 8 : 0;
 }
 static bool q4k_cu_serves(const Q4KArgs &ka, int ksplit, int n_tokens = 1) {
-    return ksplit == 1 && ka.n_sb <= 16 && ka.n_sb >= 6 && (ka.n_sb & 1) == 0 && q4k_cu_waves(ka, n_tokens) != 0 &&
+    const bool length = (ka.n_sb <= 16 && ka.n_sb >= 6 && (ka.n_sb & 1) == 0) || ka.n_sb == 20 || ka.n_sb == 24 || ka.n_sb == 32;
+    return ksplit == 1 && length && q4k_cu_waves(ka, n_tokens) != 0 &&
            ka.sb_stride < (int64_t(1) << 31) && env_int("CAMELID_HIP_Q4K_CU", 1) != 0 && !env_int("CAMELID_HIP_Q4K_CLAMPED_LOADS", 0) &&
            env_int("CAMELID_HIP_Q4K_RING", 1) != 0;
 }
@@ -1032,13 +1045,16 @@ static int launch_q4k_cu(const Q4KArgs &ka, int ablate, hipStream_t st, int n_to
     // rows of 2 * NSTEPS super-blocks: one instantiation per row length (1536 to 4096 values)
 #define CML_Q4K_CU_STEPS(NT_)                                                                                 \
     switch (ka.n_sb) {                                                                                        \
+        case 32: hipLaunchKernelGGL((gemv_q4k_cu_kernel<16, 0, NT_>), grid, block, 0, st, ca); break;         \
+        case 24: hipLaunchKernelGGL((gemv_q4k_cu_kernel<12, 0, NT_>), grid, block, 0, st, ca); break;         \
+        case 20: hipLaunchKernelGGL((gemv_q4k_cu_kernel<10, 0, NT_>), grid, block, 0, st, ca); break;         \
         case 16: hipLaunchKernelGGL((gemv_q4k_cu_kernel<8, 0, NT_>), grid, block, 0, st, ca); break;          \
         case 14: hipLaunchKernelGGL((gemv_q4k_cu_kernel<7, 0, NT_>), grid, block, 0, st, ca); break;          \
         case 12: hipLaunchKernelGGL((gemv_q4k_cu_kernel<6, 0, NT_>), grid, block, 0, st, ca); break;          \
         case 10: hipLaunchKernelGGL((gemv_q4k_cu_kernel<5, 0, NT_>), grid, block, 0, st, ca); break;          \
         case 8: hipLaunchKernelGGL((gemv_q4k_cu_kernel<4, 0, NT_>), grid, block, 0, st, ca); break;           \
         case 6: hipLaunchKernelGGL((gemv_q4k_cu_kernel<3, 0, NT_>), grid, block, 0, st, ca); break;           \
-        default: return fail(CML_ERR_UNSUPPORTED, "the eight-wave launch takes rows of 6 to 16 super-blocks");  \
+        default: return fail(CML_ERR_UNSUPPORTED, "the eight-wave launch takes rows of 6 to 16, 20, 24 or 32 super-blocks");  \
     }
     const int waves = ablate ? 8 : q4k_cu_waves(ka, n_tokens);
     if (waves > 8) {  // more than 256 eight-wave workgroups: wider ones, still one per compute unit
@@ -1050,7 +1066,10 @@ static int launch_q4k_cu(const Q4KArgs &ka, int ablate, hipStream_t st, int n_to
         case 12: CML_Q4K_CU_WIDE(NS_, NT_, 12); break;                                   \
         default: CML_Q4K_CU_WIDE(NS_, NT_, 16); break;                                   \
     }
-        if (ka.n_sb == 16 && n_tokens == 1) { CML_Q4K_CU_WIDE_WAVES(8, 1) }
+        if (ka.n_sb == 20 && n_tokens == 1) { CML_Q4K_CU_WIDE_WAVES(10, 1) }
+        else if (ka.n_sb == 20 && n_tokens == 2) { CML_Q4K_CU_WIDE_WAVES(10, 2) }
+        else if (ka.n_sb == 20) { CML_Q4K_CU_WIDE_WAVES(10, 3) }
+        else if (ka.n_sb == 16 && n_tokens == 1) { CML_Q4K_CU_WIDE_WAVES(8, 1) }
         else if (ka.n_sb == 16 && n_tokens == 2) { CML_Q4K_CU_WIDE_WAVES(8, 2) }
         else if (ka.n_sb == 16) { CML_Q4K_CU_WIDE_WAVES(8, 3) }
         else if (n_tokens == 1) { CML_Q4K_CU_WIDE_WAVES(7, 1) }

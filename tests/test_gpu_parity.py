@@ -437,10 +437,11 @@ def test_q4k_eight_wave_launch_replays_a_few_tokens(rows):
             assert G.same_bits(G.gpu_matmul_f32(w, x[:n]), singles[:n]), (rows, n, "default")
 
 
-@pytest.mark.parametrize("rows,cols", [(12800, 1536), (12304, 2048), (13000, 2560), (12320, 3072), (16384, 3584)])
+@pytest.mark.parametrize("rows,cols", [(12800, 1536), (12304, 2048), (13000, 2560), (12320, 3072), (16384, 3584),
+                                       (13824, 5120), (12800, 6144), (12330, 8192)])
 def test_q4k_eight_wave_launch_serves_rows_of_six_to_sixteen_super_blocks(rows, cols):
     """The eight-wave launch on the other row lengths it is built for (1536 to 3584 values: 6 to 14 super-blocks, an
-    even count), one to three tokens: the bits of the four-wave / matrix-core paths it replaces and of the oracle,
+    even count; 5120, 6144 and 8192 values: 20, 24 and 32 super-blocks, quantized in two passes), one to three tokens: the bits of the four-wave / matrix-core paths it replaces and of the oracle,
     also on a row band; the counters show the launch."""
     fmt = oracle.Q4_K
     rng = np.random.default_rng(8600 + cols)
@@ -468,6 +469,7 @@ def test_q4k_eight_wave_launch_serves_rows_of_six_to_sixteen_super_blocks(rows, 
 @pytest.mark.parametrize("rows,cols,tokens,kernel", [
     (18944, 3584, (1, 2, 3), "wide"),     # ten waves per workgroup
     (24570, 4096, (1, 2, 3), "wide"),     # twelve, the last 16-row tile partly filled
+    (17920, 5120, (1, 2, 3), "wide"),     # ten, two quantizer passes
     (28672, 4096, (3,), "wide"),          # sixteen: three tokens only
     (40000, 4096, (3,), "eight"),         # three tokens beyond one workgroup per compute unit: eight waves
 ])
