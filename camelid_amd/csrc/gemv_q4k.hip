@@ -830,9 +830,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_cu_kernel(Q4KCuArgs a) {
 // pairs its steps 2p and 2p + 1 read (the part's two waves take one pair each), so after pass 0 and one barrier every
 // wave starts walking, and pass p + 1 runs between the requests and the arithmetic of steps 2p, 2p + 1: the weight
 // stream never waits for a whole row to be quantized.
-template <int KS, int NSTEPS, int ABLATE = 0, bool STAGED = false>
-__global__ __launch_bounds__(512) void gemv_q4k_cu_kcut_kernel(Q4KCuArgs a) {
-    static_assert(!STAGED || (KS == 4 && NSTEPS == 7), "the staged quantizer: four K parts of seven steps, two waves each");
+template <int KS, int NSTEPS, int ABLATE = 0, bool STAGED = false, int WAVES = 8>
+__global__ __launch_bounds__(WAVES * 64) void gemv_q4k_cu_kcut_kernel(Q4KCuArgs a) {
+    static_assert(!STAGED || (KS == 4 && NSTEPS == 7 && WAVES == 8), "the staged quantizer: four K parts of seven steps, two waves each");
     constexpr bool NOACT = (ABLATE & 1) != 0, NOMATH = (ABLATE & 2) != 0, NOSTORE = (ABLATE & 4) != 0;
     const uint8_t *__restrict__ w = a.w;
     const float *__restrict__ x = a.x;
@@ -840,13 +840,13 @@ __global__ __launch_bounds__(512) void gemv_q4k_cu_kcut_kernel(Q4KCuArgs a) {
     const float *__restrict__ residual = a.residual;
     const uint32_t sb_stride = a.sb_stride;
     const int rows = a.rows, row_skip = a.row_skip, tiles16 = a.tiles16;
-    constexpr int WAVES = 8, TPW = WAVES / KS;   // half tiles per workgroup
+    constexpr int TPW = WAVES / KS;              // half tiles per workgroup
     constexpr int NSB = KS * 2 * NSTEPS;         // super-blocks per row
     constexpr int PAIRS = NSB / 2, PASSES = (PAIRS + WAVES - 1) / WAVES;
     // (more slots requested ahead of the quantizer are slower: 3 of 3 7.87 us, 4 of 4 7.85, 5 of 5 8.1, all 7 9.45 against 7.64 --
     // requests for several far-apart super-blocks per wave at once break up the front the grid sweeps the matrix with)
-    constexpr int NB = 3, PRE = 2;
-    static_assert((KS == 2 || KS == 4) && NSTEPS >= NB, "K parts of at least one full ring");
+    constexpr int NB = NSTEPS < 3 ? NSTEPS : 3, PRE = 2;
+    static_assert((KS == 2 || KS == 4) && WAVES % KS == 0 && NSTEPS >= 2, "K parts of at least two steps");
     using Regs = Q4KRegs<1>;
     __shared__ __attribute__((aligned(16))) int8_t ys[NSB * 256];
     __shared__ int bsum[NSB * 8];
@@ -963,17 +963,57 @@ __global__ __launch_bounds__(512) void gemv_q4k_cu_kcut_kernel(Q4KCuArgs a) {
     }
 }
 
-// The K-cut form serves rows of 14336 values cut four ways (seven steps per part).
-static bool q4k_cu_kcut_serves(const Q4KArgs &ka, int ksplit) {
-    return ksplit == 4 && ka.n_sb == 56 && ka.sb_stride < (int64_t(1) << 31) && env_int("CAMELID_HIP_Q4K_CU", 1) != 0 &&
-           !env_int("CAMELID_HIP_Q4K_CLAMPED_LOADS", 0) && env_int("CAMELID_HIP_Q4K_RING", 1) != 0;
+constexpr int kComputeUnits = 256;  // MI355X
+
+// The K-cut form serves rows of 14336 values cut four ways (seven steps per part, the staged quantizer) and the
+// shorter rows the policy cuts: four ways into parts of 2, 3 or 4 steps (rows of 4096, 6144, 8192 values on up to 6128
+// rows), two ways into parts of 3, 4, 5, 6 or 8 steps (3072, 4096, 5120, 6144, 8192 values on up to 12272 rows); sixteen
+// waves per workgroup where eight would need more than one workgroup per compute unit.  Returns the waves per
+// workgroup, 0 when the form does not serve.  CAMELID_HIP_Q4K_KCUT_SHORT=0 leaves the shorter rows to the four-wave launch.
+static int q4k_cu_kcut_waves(const Q4KArgs &ka, int ksplit) {
+    if (ka.sb_stride >= (int64_t(1) << 31) || env_int("CAMELID_HIP_Q4K_CU", 1) == 0 || env_int("CAMELID_HIP_Q4K_CLAMPED_LOADS", 0) ||
+        env_int("CAMELID_HIP_Q4K_RING", 1) == 0)
+        return 0;
+    if (ksplit == 4 && ka.n_sb == 56) return 8;
+    if ((ksplit != 2 && ksplit != 4) || ka.n_sb % (2 * ksplit) != 0 || !env_int("CAMELID_HIP_Q4K_KCUT_SHORT", 1)) return 0;
+    const int nsteps = ka.n_sb / (2 * ksplit);
+    if (ksplit == 4 ? (nsteps < 2 || nsteps > 4) : (nsteps < 3 || nsteps == 7 || nsteps > 8)) return 0;
+    const int only = env_int("CAMELID_HIP_Q4K_KCUT_WAVES", 0);
+    if (only == 8 || only == 16) return only;
+    const int tpw8 = 8 / ksplit;  // half tiles per eight-wave workgroup
+    return ((ka.rows + ka.row_skip + 15) / 16 * 2 + tpw8 - 1) / tpw8 <= kComputeUnits ? 8 : 16;
 }
+static bool q4k_cu_kcut_serves(const Q4KArgs &ka, int ksplit) { return q4k_cu_kcut_waves(ka, ksplit) != 0; }
 
 static int launch_q4k_cu_kcut(const Q4KArgs &ka, hipStream_t st, int ablate = 0) {
     if (!(ablate & 1) && !ka.x) return fail(CML_ERR_INVALID, "null activation");
     const int tiles16 = (ka.rows + ka.row_skip + 15) / 16;
-    const dim3 grid(static_cast<unsigned>((2 * tiles16 + 1) / 2)), block(512);  // two half tiles per workgroup
     const Q4KCuArgs ca{ka.w, ka.x, ka.out, ka.residual, static_cast<uint32_t>(ka.sb_stride), ka.rows, ka.row_skip, tiles16};
+    if (ka.n_sb != 56) {
+        if (ablate) return fail(CML_ERR_UNSUPPORTED, "the K-cut ablations exist for rows of 14336 values");
+        const int ks = ka.ksplit, waves = q4k_cu_kcut_waves(ka, ks), tpw = waves / ks;  // half tiles per workgroup
+        const dim3 grid(static_cast<unsigned>((2 * tiles16 + tpw - 1) / tpw)), block(64 * waves);
+#define CML_Q4K_KCUT(KS_, NS_)                                                                              \
+    case KS_ * 100 + NS_:                                                                                   \
+        if (waves == 8) hipLaunchKernelGGL((gemv_q4k_cu_kcut_kernel<KS_, NS_>), grid, block, 0, st, ca);    \
+        else hipLaunchKernelGGL((gemv_q4k_cu_kcut_kernel<KS_, NS_, 0, false, 16>), grid, block, 0, st, ca); \
+        break;
+        switch (ks * 100 + ka.n_sb / (2 * ks)) {
+            CML_Q4K_KCUT(4, 2)
+            CML_Q4K_KCUT(4, 3)
+            CML_Q4K_KCUT(4, 4)
+            CML_Q4K_KCUT(2, 3)
+            CML_Q4K_KCUT(2, 4)
+            CML_Q4K_KCUT(2, 5)
+            CML_Q4K_KCUT(2, 6)
+            CML_Q4K_KCUT(2, 8)
+            default: return fail(CML_ERR_UNSUPPORTED, "no K-cut form for %d super-blocks cut %d ways", ka.n_sb, ks);
+        }
+#undef CML_Q4K_KCUT
+        CML_COUNT_LAUNCH("q4k.dot.wg8.kcut.fused.short");
+        return CML_OK;
+    }
+    const dim3 grid(static_cast<unsigned>((2 * tiles16 + 1) / 2)), block(512);  // two half tiles per workgroup
     switch (ablate) {
         case 0:
             // CAMELID_HIP_Q4K_KCUT_STAGED=0: the whole row quantized before the walk (7.63 us against 7.19 at 4096 x 14336)
@@ -1004,7 +1044,6 @@ static int launch_q4k_cu_kcut(const Q4KArgs &ka, hipStream_t st, int ablate = 0)
 // 10.74; 16384 x 6144 9.94 against 10.5; 14336 x 8192 11.27 against 12.2; 28672 x 8192, three tokens, 27.3 against 32.5.
 // Seven waves per workgroup on 14336 x 4096 (256 workgroups instead of 224): 6.72 against 6.56.
 // CAMELID_HIP_Q4K_CU=0 keeps the four-wave launch.
-constexpr int kComputeUnits = 256;  // MI355X
 // Waves per workgroup of that launch, 0 when it does not serve the row count: the smallest of 8, 10 and 12 (three
 // tokens: and 16) that keeps the launch within one workgroup per compute unit -- wider than eight for rows of 14 or 16
 // super-blocks and up to three tokens; three tokens take eight waves at any row count beyond.  Measured, us per step,

@@ -540,6 +540,46 @@ def test_q4k_eight_wave_launch_under_the_k_cut_is_the_two_launch_path(rows):
             assert G.max_rel(got, want) <= TOL, (rows, i)
 
 
+@pytest.mark.parametrize("rows,cols", [
+    (4096, 4096), (5003, 4096), (4096, 6144), (3080, 8192),                       # cut four ways: parts of 2, 2, 3, 4 steps
+    (8192, 3072), (11008, 4096), (9216, 5120), (6150, 6144), (10240, 8192),       # cut two ways: parts of 3, 4, 5, 6, 8 steps
+])
+def test_q4k_eight_wave_launch_under_the_k_cut_on_shorter_rows(rows, cols):
+    """Rows of 3072 to 8192 values on fewer than 12288 rows (attention projections, smaller FFN matrices: the shape
+    policy cuts K two or four ways): one launch of eight- or sixteen-wave workgroups that quantize the row once each.
+    Same bits as the four-wave launch it replaces (CAMELID_HIP_Q4K_KCUT_SHORT=0), whatever the workgroup width, on
+    activations built to break a quantizer and on a row band; within 1e-5 of the oracle's uncut chain."""
+    fmt = oracle.Q4_K
+    rng = np.random.default_rng(9400 + rows + cols)
+    wire = G.synth_weight(fmt, rows, cols, seed=9500 + rows + cols)
+    w = Weight.upload(fmt, rows, cols, wire)
+    acts = rng.standard_normal((3, cols)).astype(np.float32)
+    a = acts[0]
+    a[0:256] = 0.0
+    a[256 + 5], a[256 + 6] = 3.5, -3.5
+    a[512 + 6], a[512 + 5] = 3.5, -3.5
+    a[768 + 3], a[768 + 100] = -4.0, 4.0
+    a[-256:] = 2.0
+    acts[1, 3], acts[1, cols - 300] = np.nan, np.nan
+    acts[2, 1::2] = -acts[2, ::2]
+    band = w.slice(5, rows - 9)
+    for i, x in enumerate(acts):
+        G.say(f"Q4_K K-cut launch on shorter rows {rows}x{cols} act={i}")
+        with G.engaged(r"^q4k\.dot\.wg8\.kcut\.fused\.short$", none=(r"^q4k\.dot\.ring", r"^q4k\.dot\.buffers", r"^quantize\.")):
+            got = G.gpu_matmul_f32(w, x)
+            got_band = G.gpu_matmul_f32(band, x)
+        with G.env(CAMELID_HIP_Q4K_KCUT_SHORT=0), G.engaged(r"^q4k\.dot\.", none=(r"^q4k\.dot\.wg8",)):
+            four_wave = G.gpu_matmul_f32(w, x)
+        assert G.same_bits(got, four_wave), (rows, cols, i)
+        assert G.same_bits(got_band, got[5:rows - 4]), (rows, cols, i)
+        for width in (8, 16):
+            with G.env(CAMELID_HIP_Q4K_KCUT_WAVES=width), G.engaged(r"^q4k\.dot\.wg8\.kcut\.fused\.short$"):
+                assert G.same_bits(G.gpu_matmul_f32(w, x), got), (rows, cols, i, width)
+        if i != 1:
+            want = oracle.matmul(fmt, wire, cols, x[None, :], order=EXACT_ORDER[fmt], threads=16)[0]
+            assert G.max_rel(got, want) <= TOL, (rows, cols, i)
+
+
 @pytest.mark.parametrize("rows", [4096, 3100, 6100])
 def test_q6k_eight_wave_launch_under_the_k_cut_is_the_two_launch_path(rows):
     """Q6_K rows of 14336 values on up to 6136 rows (the FFN down projection: the shape policy cuts K four ways):
