@@ -722,7 +722,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--config", default="q4k_14336x4096_n1",
                     help="one of: " + ", ".join(sorted(CONFIGS) + sorted(MOE_CONFIGS) + sorted(PAIR_CONFIGS) + sorted(MULTI_CONFIGS) + sorted(PRODUCER_CONFIGS))
-                    + "; or any <format>_<rows>x<cols>_n<tokens>, e.g. q8_0_14336x4352_n1")
+                    + "; or any <format>_<rows>x<cols>_n<tokens>, <format>_pair_<rows>x<cols>, <format>_multi_<rows>+<rows>[+...]x<cols>, "
+                      "e.g. q8_0_14336x4352_n1, q4k_pair_11008x4096, q4k_multi_4096+1024+1024x4096")
     ap.add_argument("--copies", type=int, default=0, help="distinct weight copies to rotate over (0 = enough for ~600 MB)")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="time budget of the CPU baseline leg (0 = skip)")
     ap.add_argument("--seed", type=int, default=1234)
@@ -756,6 +757,13 @@ def main() -> int:
         return calibrate_copy(args.calibrate_copy, max(1, args.steps), max(0, args.warmup))
     if args.config in PRODUCER_CONFIGS:
         return bench_producer(args.config, max(1, args.steps), max(0, args.warmup), args.seed)
+    fmt_names = {"q8_0": "Q8_0", "q4_0": "Q4_0", "q4k": "Q4_K", "q6k": "Q6_K"}
+    m = re.fullmatch(r"(q8_0|q4_0|q4k|q6k)_pair_(\d+)x(\d+)", args.config)
+    if m and args.config not in PAIR_CONFIGS:
+        PAIR_CONFIGS[args.config] = (fmt_names[m.group(1)], int(m.group(2)), int(m.group(3)))
+    m = re.fullmatch(r"(q8_0|q4_0|q4k|q6k)_multi_(\d+(?:\+\d+){1,3})x(\d+)", args.config)
+    if m:
+        MULTI_CONFIGS[args.config] = (fmt_names[m.group(1)], [int(r) for r in m.group(2).split("+")], int(m.group(3)))
     if args.config in PAIR_CONFIGS:
         return bench_pair(args.config, max(1, args.steps), max(0, args.warmup), args.seed)
     if args.config in MULTI_CONFIGS:

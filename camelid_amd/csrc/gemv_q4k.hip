@@ -694,6 +694,17 @@ struct Q4KCuArgs {
     int tiles16;            // 16-row layout tiles that hold the rows
 };
 
+// The K-cut form against up to four weights of one row length and one K cut (any row counts) in one launch: their
+// workgroups lie end to end along grid.x, every workgroup quantizes the token once.
+struct Q4KCuMultiArgs {
+    const float *x;          // the f32 token
+    const uint8_t *wm[4];    // tiled layouts
+    float *outm[4];          // [rowsm[j]] each
+    uint32_t stridem[4];     // bytes between consecutive super-blocks of one tile
+    int rowsm[4], skipm[4], tiles16m[4];
+    int wg_end[4];           // workgroups of weights 0 .. j (INT32_MAX beyond the last weight)
+};
+
 // NT (1 to 4) tokens: the f32 rows are contiguous ([NT][row length]), pass p of the quantizer takes token p, the
 // unpacked weight of a step is replayed against the NT staged rows from registers, and token t writes out[t][rows]
 // -- every cell the one-token result, bit for bit (the same q4k_compute).  The weight streams once for the NT tokens
@@ -830,16 +841,37 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_cu_kernel(Q4KCuArgs a) {
 // pairs its steps 2p and 2p + 1 read (the part's two waves take one pair each), so after pass 0 and one barrier every
 // wave starts walking, and pass p + 1 runs between the requests and the arithmetic of steps 2p, 2p + 1: the weight
 // stream never waits for a whole row to be quantized.
-template <int KS, int NSTEPS, int ABLATE = 0, bool STAGED = false, int WAVES = 8>
-__global__ __launch_bounds__(WAVES * 64) void gemv_q4k_cu_kcut_kernel(Q4KCuArgs a) {
+template <int KS, int NSTEPS, int ABLATE = 0, bool STAGED = false, int WAVES = 8, bool MULTI = false>
+__global__ __launch_bounds__(WAVES * 64) void gemv_q4k_cu_kcut_kernel(std::conditional_t<MULTI, Q4KCuMultiArgs, Q4KCuArgs> a) {
     static_assert(!STAGED || (KS == 4 && NSTEPS == 7 && WAVES == 8), "the staged quantizer: four K parts of seven steps, two waves each");
+    static_assert(!MULTI || (ABLATE == 0 && !STAGED), "the multi launch: the plain short form");
     constexpr bool NOACT = (ABLATE & 1) != 0, NOMATH = (ABLATE & 2) != 0, NOSTORE = (ABLATE & 4) != 0;
-    const uint8_t *__restrict__ w = a.w;
+    const uint8_t *__restrict__ w;
     const float *__restrict__ x = a.x;
-    float *__restrict__ out = a.out;
-    const float *__restrict__ residual = a.residual;
-    const uint32_t sb_stride = a.sb_stride;
-    const int rows = a.rows, row_skip = a.row_skip, tiles16 = a.tiles16;
+    float *__restrict__ out;
+    const float *__restrict__ residual;
+    uint32_t sb_stride;
+    int rows, row_skip, tiles16;
+    int bx = blockIdx.x;  // workgroup index within its weight
+    if constexpr (MULTI) {
+        // which weight this workgroup belongs to (wave-uniform selects: no indexed access to the argument block)
+        const int j = (bx >= a.wg_end[0]) + (bx >= a.wg_end[1]) + (bx >= a.wg_end[2]);
+        auto pick = [&](auto v0, auto v1, auto v2, auto v3) { return j == 0 ? v0 : (j == 1 ? v1 : (j == 2 ? v2 : v3)); };
+        w = pick(a.wm[0], a.wm[1], a.wm[2], a.wm[3]);
+        out = pick(a.outm[0], a.outm[1], a.outm[2], a.outm[3]);
+        residual = nullptr;
+        sb_stride = pick(a.stridem[0], a.stridem[1], a.stridem[2], a.stridem[3]);
+        rows = pick(a.rowsm[0], a.rowsm[1], a.rowsm[2], a.rowsm[3]);
+        row_skip = pick(a.skipm[0], a.skipm[1], a.skipm[2], a.skipm[3]);
+        tiles16 = pick(a.tiles16m[0], a.tiles16m[1], a.tiles16m[2], a.tiles16m[3]);
+        bx -= pick(0, a.wg_end[0], a.wg_end[1], a.wg_end[2]);
+    } else {
+        w = a.w;
+        out = a.out;
+        residual = a.residual;
+        sb_stride = a.sb_stride;
+        rows = a.rows, row_skip = a.row_skip, tiles16 = a.tiles16;
+    }
     constexpr int TPW = WAVES / KS;              // half tiles per workgroup
     constexpr int NSB = KS * 2 * NSTEPS;         // super-blocks per row
     constexpr int PAIRS = NSB / 2, PASSES = (PAIRS + WAVES - 1) / WAVES;
@@ -881,7 +913,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_cu_kcut_kernel(Q4KCuArgs 
     }
 
     const int tile_in_wg = wave / KS, kpart = wave - tile_in_wg * KS;
-    const int tile = blockIdx.x * TPW + tile_in_wg;  // 8-row half tile
+    const int tile = bx * TPW + tile_in_wg;  // 8-row half tile
     const int s0 = kpart * 2 * NSTEPS;               // first super-block of this wave's part
     const int g = lane / LPS, l = lane - g * LPS;
     const int r = g >> 1, h = g & 1;
@@ -952,7 +984,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_cu_kcut_kernel(Q4KCuArgs 
     __syncthreads();
     if (tid < TPW * 8) {
         const int tw = tid >> 3, rr = tid & 7;
-        const int orow = (blockIdx.x * TPW + tw) * 8 + rr - row_skip;
+        const int orow = (bx * TPW + tw) * 8 + rr - row_skip;
         if (orow >= 0 && orow < rows) {
             float v = part[(tw * KS) * 8 + rr];
 #pragma unroll
@@ -1031,6 +1063,59 @@ static int launch_q4k_cu_kcut(const Q4KArgs &ka, hipStream_t st, int ablate = 0)
         default: return fail(CML_ERR_INVALID, "ablation mask must be 1, 4 or 7");
     }
     CML_COUNT_LAUNCH("q4k.calibrate.wg8.kcut");
+    return CML_OK;
+}
+
+// The short K-cut forms against two to four weights of one row length and one K cut in ONE launch (the q, k and v
+// projections of an attention block): every output is its own call's bits.  -1 = not a set this launch serves.
+// Against the four-wave multi launch: 4096 + 1024 + 1024 rows of 4096 values 4.96 us against 5.38, 6144 + 1024 + 1024
+// of 6144 9.22 against 10.0, three times 4096 x 4096 6.83 against 6.84.  A pair of equal weights through it gains
+// nothing (11008 x 4096 9.82 against 9.91, 4096 x 4096 5.38 against 5.25), so pairs stay on the four-wave pair launch.
+// CAMELID_HIP_Q4K_KCUT_MULTI=0 keeps the four-wave multi launch.
+static int launch_q4k_cu_kcut_multi(const cml_weight *const *ws, int n, const float *x, float *const *outs, int ksplit, hipStream_t st) {
+    if (n < 2 || n > 4 || ws[0]->nb == 56) return -1;
+    int64_t tiles16_all = 0;
+    for (int j = 0; j < n; j++) tiles16_all += (ws[j]->rows + ws[j]->row_skip + 15) / 16;
+    if (tiles16_all * 16 > INT32_MAX) return -1;
+    Q4KArgs probe{};
+    probe.n_sb = static_cast<int>(ws[0]->nb);
+    probe.rows = static_cast<int>(tiles16_all * 16);
+    for (int j = 0; j < n; j++) probe.sb_stride = std::max<int64_t>(probe.sb_stride, ws[j]->planes.row_stride[0]);
+    if (!q4k_cu_kcut_waves(probe, ksplit)) return -1;
+    if (!x) return fail(CML_ERR_INVALID, "null activation");
+    constexpr int waves = 8;         // sixteen-wave workgroups are slower here at every set measured
+    const int tpw = waves / ksplit;  // half tiles per workgroup
+    Q4KCuMultiArgs ma{};
+    ma.x = x;
+    int wg = 0;
+    for (int j = 0; j < 4; j++) {
+        const cml_weight *w = ws[std::min(j, n - 1)];
+        ma.wm[j] = static_cast<const uint8_t *>(w->planes.p[0]);
+        ma.outm[j] = outs[std::min(j, n - 1)];
+        ma.stridem[j] = static_cast<uint32_t>(w->planes.row_stride[0]);
+        ma.rowsm[j] = static_cast<int>(w->rows);
+        ma.skipm[j] = w->row_skip;
+        ma.tiles16m[j] = static_cast<int>((w->rows + w->row_skip + 15) / 16);
+        if (j < n) wg += (2 * ma.tiles16m[j] + tpw - 1) / tpw;
+        ma.wg_end[j] = j < n ? wg : INT32_MAX;
+    }
+    const dim3 grid(static_cast<unsigned>(wg)), block(64 * waves);
+#define CML_Q4K_KCUT(KS_, NS_) \
+    case KS_ * 100 + NS_: hipLaunchKernelGGL((gemv_q4k_cu_kcut_kernel<KS_, NS_, 0, false, 8, true>), grid, block, 0, st, ma); break;
+    switch (ksplit * 100 + probe.n_sb / (2 * ksplit)) {
+        CML_Q4K_KCUT(4, 2)
+        CML_Q4K_KCUT(4, 3)
+        CML_Q4K_KCUT(4, 4)
+        CML_Q4K_KCUT(2, 3)
+        CML_Q4K_KCUT(2, 4)
+        CML_Q4K_KCUT(2, 5)
+        CML_Q4K_KCUT(2, 6)
+        CML_Q4K_KCUT(2, 8)
+        default: return -1;
+    }
+#undef CML_Q4K_KCUT
+    CML_COUNT_LAUNCH("q4k.dot.wg8.kcut.fused.multi");
+    CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }
 
@@ -1536,6 +1621,10 @@ int launch_gemv_q4k_f32_multi(const cml_weight *const *ws, int n, const float *x
         if (j && ks != ksplit) return -1;
         ksplit = ks;
         tiles16_all += (ws[j]->rows + ws[j]->row_skip + 15) / 16;
+    }
+    if (env_int("CAMELID_HIP_Q4K_KCUT_MULTI", 1)) {
+        const int rc = launch_q4k_cu_kcut_multi(ws, n, x, outs, ksplit, st);
+        if (rc != -1) return rc;
     }
     Q4KArgs ka{};
     ka.n_sb = n_sb;

@@ -1288,7 +1288,8 @@ def _multi(ws, x, stream=None):
     return [o.to_numpy(np.float32, (w.rows,)) for o, w in zip(outs, ws)]
 
 
-@pytest.mark.parametrize("case", ["qkv_4096", "gate_up_14336", "ragged_2304", "three_3584", "mixed_cut", "five", "q6k", "bands"])
+@pytest.mark.parametrize("case", ["qkv_4096", "gate_up_14336", "ragged_2304", "three_3584", "mixed_cut", "five", "q6k", "bands",
+                                  "cut4_8192", "cut2_4096"])
 def test_matmul_f32_multi_is_the_single_calls(case):
     """cml_matmul_f32_multi: several weights that read one token (q | k | v of an attention block, gate | up of an FFN).
     Runs of up to four Q4_K weights with one K cut go out as one launch -- the counters prove it -- and every
@@ -1296,7 +1297,9 @@ def test_matmul_f32_multi_is_the_single_calls(case):
     another format) fall back to single calls with the same results."""
     fmt = B.CML_Q4_K
     shapes, cols, one_launch = {
-        "qkv_4096": ([4096, 1024, 1024], 4096, 1),          # K cut 4 for all three: the two-buffer kernel
+        "qkv_4096": ([4096, 1024, 1024], 4096, 1),          # K cut 4 for all three: the eight-wave K-cut form
+        "cut4_8192": ([4000, 3100, 5000], 8192, 1),         # K cut 4, parts of four steps
+        "cut2_4096": ([8192, 6144, 7001], 4096, 1),         # K cut 2, parts of four steps
         "gate_up_14336": ([14336, 14336], 4096, 1),         # no K cut: the ring kernel
         "ragged_2304": ([200, 77, 530, 16], 2304, 1),       # ragged row counts, 9 super-blocks
         "three_3584": ([1000, 333, 4100], 3584, 1),
@@ -1320,6 +1323,8 @@ def test_matmul_f32_multi_is_the_single_calls(case):
         proof = G.engaged(r"^q6k\.dot\.", none=(r"multi",))
     elif one_launch == 0:
         proof = G.engaged(r"^q4k\.dot\.", none=(r"multi",))
+    elif case in ("qkv_4096", "bands", "cut4_8192", "cut2_4096"):
+        proof = G.engaged(r"^q4k\.dot\.wg8\.kcut\.fused\.multi$", none=(r"^q4k\.dot\.(ring|buffers)",))
     else:
         proof = G.engaged(r"^q4k\.dot\.(ring|buffers)\.fused\.multi$")
     before = G.launch_counts()
@@ -1334,6 +1339,11 @@ def test_matmul_f32_multi_is_the_single_calls(case):
         got = _multi(ws, x)
     for j, (g, wnt) in enumerate(zip(got, want)):
         assert G.same_bits(g, wnt), (case, j, "single calls inside")
+    if fmt == B.CML_Q4_K and one_launch:
+        with G.env(CAMELID_HIP_Q4K_KCUT_MULTI=0), G.engaged(r"^q4k\.dot\.(ring|buffers)\.fused\.multi$", none=(r"^q4k\.dot\.wg8",)):
+            got = _multi(ws, x)
+        for j, (g, wnt) in enumerate(zip(got, want)):
+            assert G.same_bits(g, wnt), (case, j, "four-wave multi launch")
     if fmt == B.CML_Q4_K:
         with G.env(CAMELID_HIP_EXACT_ORDER="1"):
             got = _multi(ws, x)
