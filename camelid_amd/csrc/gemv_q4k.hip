@@ -995,25 +995,163 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_cu_kcut_kernel(std::condi
     }
 }
 
+// The K-cut form for rows the cut does not divide into whole two-super-block steps (rows of 43 super-blocks cut four
+// ways: parts of 10, 11, 11, 11; an odd part length; 5120 values cut four ways: parts of 5).  The parts are those of
+// gemv_q4k_kernel, [k n / KS, (k + 1) n / KS), so the association and the bits are the same.  Every part runs MAXSTEPS
+// steps: all but the last lie wholly inside every part (whole loads, no masks), the last one may be half or wholly
+// outside its part (clamped loads, masked terms).  The quantizer is staged as in the 14336-value form: the wave of
+// half tile t and part k quantizes the super-blocks of step TPW p + t of part k in pass p, a barrier in front of
+// step TPW p makes them visible, and pass p + 1 runs ahead of that step's arithmetic.
+struct Q4KCuAnyArgs {
+    Q4KCuArgs one;
+    int n_sb;  // super-blocks per row
+};
+
+template <int KS, int MAXSTEPS, int WAVES = 8>
+__global__ __launch_bounds__(WAVES * 64) void gemv_q4k_cu_kcut_any_kernel(Q4KCuAnyArgs aa) {
+    const Q4KCuArgs &a = aa.one;
+    const uint8_t *__restrict__ w = a.w;
+    const float *__restrict__ x = a.x;
+    float *__restrict__ out = a.out;
+    const float *__restrict__ residual = a.residual;
+    const uint32_t sb_stride = a.sb_stride;
+    const int rows = a.rows, row_skip = a.row_skip, tiles16 = a.tiles16, n_sb = aa.n_sb;
+    constexpr int TPW = WAVES / KS;  // half tiles per workgroup = waves per K part
+    static_assert(WAVES % KS == 0 && WAVES >= 8 && WAVES <= 16, "whole half tiles per workgroup");
+    constexpr int PASSES = (MAXSTEPS + TPW - 1) / TPW;
+    constexpr int NB = MAXSTEPS < 3 ? MAXSTEPS : 3, PRE = 2;
+    static_assert((KS == 2 || KS == 4) && MAXSTEPS >= 2, "K parts of at least two steps");
+    using Regs = Q4KRegs<1>;
+    extern __shared__ uint4 smem_any[];
+    int8_t *ys = reinterpret_cast<int8_t *>(smem_any);           // [n_sb * 256]
+    int *bsum = reinterpret_cast<int *>(ys + n_sb * 256);        // [n_sb * 8]
+    float *yds = reinterpret_cast<float *>(bsum + n_sb * 8);     // [n_sb]
+    float *part = yds + ((n_sb + 3) & ~3);                       // [WAVES * 8]
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    const int tile_in_wg = wave / KS, kpart = wave - tile_in_wg * KS;
+    const int s0 = (kpart * n_sb) / KS, s1 = ((kpart + 1) * n_sb) / KS;  // this wave's part
+
+    // the f32 activation: pass p of this wave takes the two super-blocks of step TPW p + tile_in_wg of its own part
+    const int half = lane >> 5, ql = lane & 31;
+    auto pass_sb = [&](int p) __attribute__((always_inline)) -> int { return s0 + 2 * (TPW * p + tile_in_wg) + half; };
+    float4 xv[PASSES][2];
+#pragma unroll
+    for (int p = 0; p < PASSES; p++) {
+        const float4 *x4 = reinterpret_cast<const float4 *>(x) + min(pass_sb(p), n_sb - 1) * 64 + ql * 2;
+        xv[p][0] = x4[0];
+        xv[p][1] = x4[1];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();  // execution only: every activation request of the workgroup is out
+    __builtin_amdgcn_sched_barrier(0);
+
+    const int tile = blockIdx.x * TPW + tile_in_wg;  // 8-row half tile
+    const int g = lane / LPS, l = lane - g * LPS;
+    const int r = g >> 1, h = g & 1;
+    const int rl = (tile & 1) * 8 + r;
+    const uint8_t *wtile = w + static_cast<int64_t>(min(tile >> 1, tiles16 - 1)) * kQ4KChunk;
+    const uint32_t hoff = static_cast<uint32_t>(h) * sb_stride;
+    const uint32_t hdr_off = hoff + rl * 16, q_off = hoff + (rl * LPS + l) * 16;
+    Regs ring[NB];
+    auto request = [&](Regs &b, int step) __attribute__((always_inline)) {
+        if (step < MAXSTEPS - 1) q4k_load_whole<1, 2>(b, wtile + static_cast<int64_t>(s0 + 2 * step) * sb_stride, sb_stride, hdr_off, q_off);
+        else q4k_load<1, 2>(b, wtile, sb_stride, rl, rl * LPS + l, s0 + 2 * step + h, s1);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+#pragma unroll
+    for (int k = 0; k < PRE; k++) request(ring[k], k);
+
+    // every wave runs every pass (super-blocks outside its part are redone from clamped values and not stored)
+    auto quantize_pass = [&](int p) __attribute__((always_inline)) {
+        const int sbk = pass_sb(p);
+        float dv;
+        int bs;
+        const uint2 packed = q8k_quantize_row32(xv[p], lane, dv, bs);
+        if (sbk < s1) {
+            reinterpret_cast<uint2 *>(ys)[sbk * 32 + ql] = packed;
+            if ((ql & 3) == 3) bsum[sbk * 8 + (ql >> 2)] = bs;
+            if (ql == 0) yds[sbk] = dv;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    quantize_pass(0);
+    __syncthreads();
+
+    Q4KLane ln;
+    ln.c = l;
+    ln.sh = (l & 1) * 16;
+    ln.upper = l >= 2;
+    float acc[1] = {0.0f};
+    auto compute = [&](const Regs &b, int step) __attribute__((always_inline)) {
+        if (step < MAXSTEPS - 1) q4k_compute<1, false, 1, 2, true>(b, ln, s0 + 2 * step + h, s1, ys, bsum, yds, n_sb, acc, nullptr);
+        else q4k_compute<1, false, 1, 2, false>(b, ln, s0 + 2 * step + h, s1, ys, bsum, yds, n_sb, acc, nullptr);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+#pragma unroll
+    for (int j = PRE; j < NB; j++) request(ring[j], j);
+#pragma unroll
+    for (int i = 0; i < MAXSTEPS; i++) {
+        if (i % TPW == 0 && i / TPW + 1 < PASSES) quantize_pass(i / TPW + 1);
+        if (i % TPW == 0 && i > 0) __syncthreads();
+        compute(ring[i % NB], i);
+        if (i + NB < MAXSTEPS) request(ring[i % NB], i + NB);
+    }
+    if (l == LPS - 1 && h == 1) part[wave * 8 + r] = acc[0];
+    __syncthreads();
+    if (tid < TPW * 8) {
+        const int tw = tid >> 3, rr = tid & 7;
+        const int orow = (blockIdx.x * TPW + tw) * 8 + rr - row_skip;
+        if (orow >= 0 && orow < rows) {
+            float v = part[(tw * KS) * 8 + rr];
+#pragma unroll
+            for (int k = 1; k < KS; k++) v = v + part[(tw * KS + k) * 8 + rr];
+            if (residual) v = v + residual[orow];
+            out[orow] = v;
+        }
+    }
+}
+
 constexpr int kComputeUnits = 256;  // MI355X
+
+// Steps per part of the form for uneven parts (gemv_q4k_cu_kcut_any_kernel), 0 where the whole-step forms or none
+// serve: rows the cut leaves no whole number of two-super-block steps, or longer parts than the whole-step forms take
+// (4096 x 11008: 43 super-blocks four ways, 8.20 -> 6.29 us; 5120 x 5120: 20 four ways, 7.2 -> 4.69; 5120 x 13824: 54,
+// 11.6 -> 8.76; 3584 x 18944: 74, 10.76 -> 8.64; 4096 x 10240 7.70 -> 5.89).  CAMELID_HIP_Q4K_KCUT_ANY=0 leaves them
+// to the four-wave launches.
+static int q4k_cu_kcut_any_steps(const Q4KArgs &ka, int ksplit) {
+    if (!env_int("CAMELID_HIP_Q4K_KCUT_ANY", 1) || (ksplit == 4 && ka.n_sb == 56)) return 0;
+    const int longest = (ka.n_sb + ksplit - 1) / ksplit, steps = (longest + 1) / 2;
+    const bool whole_steps = ka.n_sb % (2 * ksplit) == 0;
+    if (ksplit == 4) return (whole_steps ? steps > 4 && steps <= 10 : steps >= 3 && steps <= 10) ? steps : 0;
+    if (ksplit == 2) return (whole_steps ? steps == 7 : steps >= 3 && steps <= 7) ? steps : 0;  // (28 steps, 8192 x 28672: 90-124 us against 26.6, the unrolled walk spills)
+    return 0;
+}
 
 // The K-cut form serves rows of 14336 values cut four ways (seven steps per part, the staged quantizer) and the
 // shorter rows the policy cuts: four ways into parts of 2, 3 or 4 steps (rows of 4096, 6144, 8192 values on up to 6128
-// rows), two ways into parts of 3, 4, 5, 6 or 8 steps (3072, 4096, 5120, 6144, 8192 values on up to 12272 rows); sixteen
-// waves per workgroup where eight would need more than one workgroup per compute unit.  Returns the waves per
-// workgroup, 0 when the form does not serve.  CAMELID_HIP_Q4K_KCUT_SHORT=0 leaves the shorter rows to the four-wave launch.
+// rows), two ways into parts of 3, 4, 5, 6 or 8 steps (3072, 4096, 5120, 6144, 8192 values on up to 12272 rows), and
+// what q4k_cu_kcut_any_steps lists; twelve (then sixteen) waves per workgroup where eight would need more than one
+// workgroup per compute unit -- twelve always suffice below 12288 rows, and beat sixteen wherever both were measured
+// (9216 x 5120: 8.13 / 5.97 / 6.75 us with 8 / 12 / 16 waves against 7.38 for the four-wave launch; 11008 x 4096:
+// 6.64 / 5.75 / 6.13 against 6.54; 5120 x 8192: 7.29 / 5.83 / 6.17 against 8.02).  Returns the waves per workgroup,
+// 0 when the form does not serve.  CAMELID_HIP_Q4K_KCUT_SHORT=0 leaves all but the 14336-value rows to the four-wave launch.
 static int q4k_cu_kcut_waves(const Q4KArgs &ka, int ksplit) {
     if (ka.sb_stride >= (int64_t(1) << 31) || env_int("CAMELID_HIP_Q4K_CU", 1) == 0 || env_int("CAMELID_HIP_Q4K_CLAMPED_LOADS", 0) ||
         env_int("CAMELID_HIP_Q4K_RING", 1) == 0)
         return 0;
     if (ksplit == 4 && ka.n_sb == 56) return 8;
-    if ((ksplit != 2 && ksplit != 4) || ka.n_sb % (2 * ksplit) != 0 || !env_int("CAMELID_HIP_Q4K_KCUT_SHORT", 1)) return 0;
+    if ((ksplit != 2 && ksplit != 4) || !env_int("CAMELID_HIP_Q4K_KCUT_SHORT", 1)) return 0;
+    if (q4k_cu_kcut_any_steps(ka, ksplit)) return 8;
+    if (ka.n_sb % (2 * ksplit) != 0) return 0;
     const int nsteps = ka.n_sb / (2 * ksplit);
     if (ksplit == 4 ? (nsteps < 2 || nsteps > 4) : (nsteps < 3 || nsteps == 7 || nsteps > 8)) return 0;
     const int only = env_int("CAMELID_HIP_Q4K_KCUT_WAVES", 0);
-    if (only == 8 || only == 16) return only;
-    const int tpw8 = 8 / ksplit;  // half tiles per eight-wave workgroup
-    return ((ka.rows + ka.row_skip + 15) / 16 * 2 + tpw8 - 1) / tpw8 <= kComputeUnits ? 8 : 16;
+    if (only == 8 || only == 12 || only == 16) return only;
+    const int half_tiles = (ka.rows + ka.row_skip + 15) / 16 * 2;
+    int waves = 8;
+    while (waves < 16 && (half_tiles + waves / ksplit - 1) / (waves / ksplit) > kComputeUnits) waves += 4;
+    return waves;
 }
 static bool q4k_cu_kcut_serves(const Q4KArgs &ka, int ksplit) { return q4k_cu_kcut_waves(ka, ksplit) != 0; }
 
@@ -1021,6 +1159,45 @@ static int launch_q4k_cu_kcut(const Q4KArgs &ka, hipStream_t st, int ablate = 0)
     if (!(ablate & 1) && !ka.x) return fail(CML_ERR_INVALID, "null activation");
     const int tiles16 = (ka.rows + ka.row_skip + 15) / 16;
     const Q4KCuArgs ca{ka.w, ka.x, ka.out, ka.residual, static_cast<uint32_t>(ka.sb_stride), ka.rows, ka.row_skip, tiles16};
+    if (const int any_steps = q4k_cu_kcut_any_steps(ka, ka.ksplit)) {
+        if (ablate) return fail(CML_ERR_UNSUPPORTED, "the K-cut ablations exist for rows of 14336 values");
+        // eight waves, or twelve / sixteen where eight would need more than one workgroup per compute unit
+        const int ks = ka.ksplit;
+        int waves = env_int("CAMELID_HIP_Q4K_KCUT_WAVES", 0);
+        if (waves != 8 && waves != 12 && waves != 16) {
+            waves = 8;
+            while (waves < 16 && (2 * tiles16 + waves / ks - 1) / (waves / ks) > kComputeUnits) waves += 4;
+        }
+        const int tpw = waves / ks;
+        const dim3 grid(static_cast<unsigned>((2 * tiles16 + tpw - 1) / tpw)), block(64 * waves);
+        const size_t lds = static_cast<size_t>(ka.n_sb) * (256 + 32) + ((static_cast<size_t>(ka.n_sb) + 3) & ~size_t(3)) * 4 + 16 * 8 * 4;
+        const Q4KCuAnyArgs aa{ca, ka.n_sb};
+#define CML_Q4K_KCUT_ANY(KS_, NS_)                                                                                        \
+    case KS_ * 100 + NS_:                                                                                                 \
+        if (waves == 8) hipLaunchKernelGGL((gemv_q4k_cu_kcut_any_kernel<KS_, NS_, 8>), grid, block, lds, st, aa);         \
+        else if (waves == 12) hipLaunchKernelGGL((gemv_q4k_cu_kcut_any_kernel<KS_, NS_, 12>), grid, block, lds, st, aa);  \
+        else hipLaunchKernelGGL((gemv_q4k_cu_kcut_any_kernel<KS_, NS_, 16>), grid, block, lds, st, aa);                   \
+        break;
+        switch (ks * 100 + any_steps) {
+            CML_Q4K_KCUT_ANY(4, 3)
+            CML_Q4K_KCUT_ANY(4, 4)
+            CML_Q4K_KCUT_ANY(4, 5)
+            CML_Q4K_KCUT_ANY(4, 6)
+            CML_Q4K_KCUT_ANY(4, 7)
+            CML_Q4K_KCUT_ANY(4, 8)
+            CML_Q4K_KCUT_ANY(4, 9)
+            CML_Q4K_KCUT_ANY(4, 10)
+            CML_Q4K_KCUT_ANY(2, 3)
+            CML_Q4K_KCUT_ANY(2, 4)
+            CML_Q4K_KCUT_ANY(2, 5)
+            CML_Q4K_KCUT_ANY(2, 6)
+            CML_Q4K_KCUT_ANY(2, 7)
+            default: return fail(CML_ERR_UNSUPPORTED, "no K-cut form for %d super-blocks cut %d ways", ka.n_sb, ks);
+        }
+#undef CML_Q4K_KCUT_ANY
+        CML_COUNT_LAUNCH("q4k.dot.wg8.kcut.fused.uneven");
+        return CML_OK;
+    }
     if (ka.n_sb != 56) {
         if (ablate) return fail(CML_ERR_UNSUPPORTED, "the K-cut ablations exist for rows of 14336 values");
         const int ks = ka.ksplit, waves = q4k_cu_kcut_waves(ka, ks), tpw = waves / ks;  // half tiles per workgroup
@@ -1028,6 +1205,7 @@ static int launch_q4k_cu_kcut(const Q4KArgs &ka, hipStream_t st, int ablate = 0)
 #define CML_Q4K_KCUT(KS_, NS_)                                                                              \
     case KS_ * 100 + NS_:                                                                                   \
         if (waves == 8) hipLaunchKernelGGL((gemv_q4k_cu_kcut_kernel<KS_, NS_>), grid, block, 0, st, ca);    \
+        else if (waves == 12) hipLaunchKernelGGL((gemv_q4k_cu_kcut_kernel<KS_, NS_, 0, false, 12>), grid, block, 0, st, ca); \
         else hipLaunchKernelGGL((gemv_q4k_cu_kcut_kernel<KS_, NS_, 0, false, 16>), grid, block, 0, st, ca); \
         break;
         switch (ks * 100 + ka.n_sb / (2 * ks)) {
@@ -1081,9 +1259,9 @@ static int launch_q4k_cu_kcut_multi(const cml_weight *const *ws, int n, const fl
     probe.n_sb = static_cast<int>(ws[0]->nb);
     probe.rows = static_cast<int>(tiles16_all * 16);
     for (int j = 0; j < n; j++) probe.sb_stride = std::max<int64_t>(probe.sb_stride, ws[j]->planes.row_stride[0]);
-    if (!q4k_cu_kcut_waves(probe, ksplit)) return -1;
+    if (!q4k_cu_kcut_waves(probe, ksplit) || q4k_cu_kcut_any_steps(probe, ksplit)) return -1;  // the whole-step forms only
     if (!x) return fail(CML_ERR_INVALID, "null activation");
-    constexpr int waves = 8;         // sixteen-wave workgroups are slower here at every set measured
+    constexpr int waves = 8;         // twelve- and sixteen-wave workgroups are slower here at every set measured (q | k | v: 5.70 and 5.27 us against 4.96)
     const int tpw = waves / ksplit;  // half tiles per workgroup
     Q4KCuMultiArgs ma{};
     ma.x = x;

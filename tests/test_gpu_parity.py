@@ -543,10 +543,14 @@ def test_q4k_eight_wave_launch_under_the_k_cut_is_the_two_launch_path(rows):
 @pytest.mark.parametrize("rows,cols", [
     (4096, 4096), (5003, 4096), (4096, 6144), (3080, 8192),                       # cut four ways: parts of 2, 2, 3, 4 steps
     (8192, 3072), (11008, 4096), (9216, 5120), (6150, 6144), (10240, 8192),       # cut two ways: parts of 3, 4, 5, 6, 8 steps
+    # parts that are no whole number of two-super-block steps, or longer than the forms above take
+    (4096, 11008), (5120, 5120), (5125, 13824), (3584, 18944), (3584, 3584), (4100, 10240), (8192, 7168), (3300, 2304),
+    (5000, 16384), (4096, 20480),
 ])
 def test_q4k_eight_wave_launch_under_the_k_cut_on_shorter_rows(rows, cols):
-    """Rows of 3072 to 8192 values on fewer than 12288 rows (attention projections, smaller FFN matrices: the shape
-    policy cuts K two or four ways): one launch of eight- or sixteen-wave workgroups that quantize the row once each.
+    """Rows of 2304 to 20480 values on fewer than 12288 rows (attention projections, smaller FFN matrices, the down
+    projections of 11008-, 13824- and 18944-wide FFNs: the shape policy cuts K two or four ways, into parts that need
+    not be whole steps or equal): one launch of eight-, twelve- or sixteen-wave workgroups that quantize the row once each.
     Same bits as the four-wave launch it replaces (CAMELID_HIP_Q4K_KCUT_SHORT=0), whatever the workgroup width, on
     activations built to break a quantizer and on a row band; within 1e-5 of the oracle's uncut chain."""
     fmt = oracle.Q4_K
@@ -565,15 +569,15 @@ def test_q4k_eight_wave_launch_under_the_k_cut_on_shorter_rows(rows, cols):
     band = w.slice(5, rows - 9)
     for i, x in enumerate(acts):
         G.say(f"Q4_K K-cut launch on shorter rows {rows}x{cols} act={i}")
-        with G.engaged(r"^q4k\.dot\.wg8\.kcut\.fused\.short$", none=(r"^q4k\.dot\.ring", r"^q4k\.dot\.buffers", r"^quantize\.")):
+        with G.engaged(r"^q4k\.dot\.wg8\.kcut\.fused\.(short|uneven)$", none=(r"^q4k\.dot\.ring", r"^q4k\.dot\.buffers", r"^quantize\.")):
             got = G.gpu_matmul_f32(w, x)
             got_band = G.gpu_matmul_f32(band, x)
         with G.env(CAMELID_HIP_Q4K_KCUT_SHORT=0), G.engaged(r"^q4k\.dot\.", none=(r"^q4k\.dot\.wg8",)):
             four_wave = G.gpu_matmul_f32(w, x)
         assert G.same_bits(got, four_wave), (rows, cols, i)
         assert G.same_bits(got_band, got[5:rows - 4]), (rows, cols, i)
-        for width in (8, 16):
-            with G.env(CAMELID_HIP_Q4K_KCUT_WAVES=width), G.engaged(r"^q4k\.dot\.wg8\.kcut\.fused\.short$"):
+        for width in (8, 12, 16):
+            with G.env(CAMELID_HIP_Q4K_KCUT_WAVES=width), G.engaged(r"^q4k\.dot\.wg8\.kcut\.fused\.(short|uneven)$"):
                 assert G.same_bits(G.gpu_matmul_f32(w, x), got), (rows, cols, i, width)
         if i != 1:
             want = oracle.matmul(fmt, wire, cols, x[None, :], order=EXACT_ORDER[fmt], threads=16)[0]
