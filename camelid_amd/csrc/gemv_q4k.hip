@@ -1120,7 +1120,9 @@ constexpr int kComputeUnits = 256;  // MI355X
 // 11.6 -> 8.76; 3584 x 18944: 74, 10.76 -> 8.64; 4096 x 10240 7.70 -> 5.89).  CAMELID_HIP_Q4K_KCUT_ANY=0 leaves them
 // to the four-wave launches.
 static int q4k_cu_kcut_any_steps(const Q4KArgs &ka, int ksplit) {
-    if (!env_int("CAMELID_HIP_Q4K_KCUT_ANY", 1) || (ksplit == 4 && ka.n_sb == 56)) return 0;
+    if (!env_int("CAMELID_HIP_Q4K_KCUT_ANY", 1)) return 0;
+    if (ksplit == 4 && ka.n_sb == 56)  // rows of 14336 values: the form of its own while that is one workgroup per compute unit
+        return (ka.rows + ka.row_skip + 15) / 16 > kComputeUnits && env_int("CAMELID_HIP_Q4K_KCUT_ANY", 1) != 2 ? 7 : 0;
     const int longest = (ka.n_sb + ksplit - 1) / ksplit, steps = (longest + 1) / 2;
     const bool whole_steps = ka.n_sb % (2 * ksplit) == 0;
     if (ksplit == 4) return (whole_steps ? steps > 4 && steps <= 10 : steps >= 3 && steps <= 10) ? steps : 0;
@@ -1159,8 +1161,7 @@ static int launch_q4k_cu_kcut(const Q4KArgs &ka, hipStream_t st, int ablate = 0)
     if (!(ablate & 1) && !ka.x) return fail(CML_ERR_INVALID, "null activation");
     const int tiles16 = (ka.rows + ka.row_skip + 15) / 16;
     const Q4KCuArgs ca{ka.w, ka.x, ka.out, ka.residual, static_cast<uint32_t>(ka.sb_stride), ka.rows, ka.row_skip, tiles16};
-    if (const int any_steps = q4k_cu_kcut_any_steps(ka, ka.ksplit)) {
-        if (ablate) return fail(CML_ERR_UNSUPPORTED, "the K-cut ablations exist for rows of 14336 values");
+    if (const int any_steps = ablate ? 0 : q4k_cu_kcut_any_steps(ka, ka.ksplit)) {
         // eight waves, or twelve / sixteen where eight would need more than one workgroup per compute unit
         const int ks = ka.ksplit;
         int waves = env_int("CAMELID_HIP_Q4K_KCUT_WAVES", 0);

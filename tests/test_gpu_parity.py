@@ -525,15 +525,21 @@ def test_q4k_eight_wave_launch_under_the_k_cut_is_the_two_launch_path(rows):
     band = w.slice(5, rows - 9)
     for i, x in enumerate(acts):
         G.say(f"Q4_K eight-wave K-cut launch {rows}x14336 act={i}")
-        with G.engaged(r"^q4k\.dot\.wg8\.kcut\.fused$", none=(r"^q4k\.dot\.ring", r"^q4k\.dot\.buffers", r"^quantize\.")):
+        # up to 4096 rows (one eight-wave workgroup per compute unit) the form of its own, beyond twelve-wave workgroups of the general one
+        kernel = r"^q4k\.dot\.wg8\.kcut\.fused$" if rows <= 4096 else r"^q4k\.dot\.wg8\.kcut\.fused\.uneven$"
+        with G.engaged(kernel, none=(r"^q4k\.dot\.ring", r"^q4k\.dot\.buffers", r"^quantize\.")):
             got = G.gpu_matmul_f32(w, x)
             got_band = G.gpu_matmul_f32(band, x)
         with G.env(CAMELID_HIP_Q4K_CU=0), G.engaged(r"^quantize\.q8_k$", r"^q4k\.dot\.", none=(r"^q4k\.dot\.wg8",)):
             two_launches = G.gpu_matmul_f32(w, x)
-        with G.env(CAMELID_HIP_Q4K_KCUT_STAGED=0), G.engaged(r"^q4k\.dot\.wg8\.kcut\.fused\.whole_row$", none=(r"^q4k\.dot\.wg8\.kcut\.fused$",)):
+        with G.env(CAMELID_HIP_Q4K_KCUT_STAGED=0, CAMELID_HIP_Q4K_KCUT_ANY=2), \
+                G.engaged(r"^q4k\.dot\.wg8\.kcut\.fused\.whole_row$", none=(r"^q4k\.dot\.wg8\.kcut\.fused$",)):
             whole_row = G.gpu_matmul_f32(w, x)   # the row quantized before the walk instead of pass by pass along it
+        with G.env(CAMELID_HIP_Q4K_KCUT_ANY=2), G.engaged(r"^q4k\.dot\.wg8\.kcut\.fused$"):
+            own_form = G.gpu_matmul_f32(w, x)
         assert G.same_bits(got, two_launches), (rows, i)
         assert G.same_bits(got, whole_row), (rows, i)
+        assert G.same_bits(got, own_form), (rows, i)
         assert G.same_bits(got_band, got[5:rows - 4]), (rows, i)
         if i != 1:
             want = oracle.matmul(fmt, wire, cols, x[None, :], order=EXACT_ORDER[fmt], threads=16)[0]
