@@ -356,20 +356,29 @@ __global__ __launch_bounds__(256) void gemv_q6k_kernel(Q6KArgs a) {
 // one pass and the others run between steps, with a barrier ahead of the first step that reads a pass.  Every f32
 // request is out before the first weight request (an execution barrier), and the weights stream through a ring of
 // NB one-super-block buffers.
-template <int KS, int NSTEPS, int NB = 4>
-__global__ __launch_bounds__(512) void gemv_q6k_cu_kcut_kernel(Q6KArgs a) {
-    constexpr int WAVES = 8, LPS = 8, RPW = kWave / LPS, TPW = WAVES / KS, NSB = KS * NSTEPS, PRE = 2;
+// ANY: the row length is the launch's (n_sb super-blocks, staged in dynamic LDS), the parts are those of
+// gemv_q6k_kernel, [k n / KS, (k + 1) n / KS) -- unequal when KS does not divide n -- and NSTEPS is the longest part:
+// steps past a shorter part's end re-read its last super-block and add nothing.
+template <int KS, int NSTEPS, int NB = 4, int WAVES = 8, bool ANY = false>
+__global__ __launch_bounds__(WAVES * 64) void gemv_q6k_cu_kcut_kernel(Q6KArgs a) {
+    constexpr int LPS = 8, RPW = kWave / LPS, TPW = WAVES / KS, PRE = 2;
     constexpr int PER_PASS = 2 * TPW;                       // super-blocks a pass gives every part
     constexpr int PASSES = (NSTEPS + PER_PASS - 1) / PER_PASS;
     static_assert(NSTEPS >= NB && WAVES % KS == 0, "K parts of at least one full ring");
-    __shared__ __attribute__((aligned(16))) int8_t ys[NSB * 256];
-    __shared__ int bsum16[NSB * 16];
-    __shared__ float yds[NSB];
+    const int NSB = ANY ? a.n_sb : KS * NSTEPS;
+    __shared__ __attribute__((aligned(16))) int8_t ys_fixed[ANY ? 16 : KS * NSTEPS * 256];
+    __shared__ int bsum16_fixed[ANY ? 1 : KS * NSTEPS * 16];
+    __shared__ float yds_fixed[ANY ? 1 : KS * NSTEPS];
     __shared__ float part[WAVES * RPW];
+    extern __shared__ uint4 smem_q6k_any[];
+    int8_t *ys = ANY ? reinterpret_cast<int8_t *>(smem_q6k_any) : ys_fixed;
+    int *bsum16 = ANY ? reinterpret_cast<int *>(ys + NSB * 256) : bsum16_fixed;
+    float *yds = ANY ? reinterpret_cast<float *>(bsum16 + NSB * 16) : yds_fixed;
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int tile_in_wg = wave / KS, kpart = wave - tile_in_wg * KS;
-    const int s0 = kpart * NSTEPS;  // first super-block of this wave's part
+    const int s0 = ANY ? (kpart * NSB) / KS : kpart * NSTEPS;  // first super-block of this wave's part
+    const int s1 = ANY ? ((kpart + 1) * NSB) / KS : s0 + NSTEPS;
 
     // the f32 activation: in pass p this wave's halves take super-blocks PER_PASS * p + 2 * tile_in_wg + {0, 1} of its part
     const int half = lane >> 5, ql32 = lane & 31;
@@ -377,7 +386,7 @@ __global__ __launch_bounds__(512) void gemv_q6k_cu_kcut_kernel(Q6KArgs a) {
     float4 xv[PASSES][2];
 #pragma unroll
     for (int p = 0; p < PASSES; p++) {
-        const float4 *x4 = reinterpret_cast<const float4 *>(a.x) + (s0 + min(unit_of(p), NSTEPS - 1)) * 64 + ql32 * 2;
+        const float4 *x4 = reinterpret_cast<const float4 *>(a.x) + min(s0 + unit_of(p), s1 - 1) * 64 + ql32 * 2;
         xv[p][0] = x4[0];
         xv[p][1] = x4[1];
     }
@@ -395,7 +404,7 @@ __global__ __launch_bounds__(512) void gemv_q6k_cu_kcut_kernel(Q6KArgs a) {
     const uint8_t *dp = a.d + arow * a.d_stride;
     Q6KRegs<1> ring[NB];
     auto request = [&](Q6KRegs<1> &b, int step) __attribute__((always_inline)) {
-        q6k_load(b, ql, qh, sc, dp, l, s0 + step, s0 + NSTEPS);
+        q6k_load(b, ql, qh, sc, dp, l, s0 + step, s1);
         __builtin_amdgcn_sched_barrier(0);
     };
 #pragma unroll
@@ -410,7 +419,7 @@ __global__ __launch_bounds__(512) void gemv_q6k_cu_kcut_kernel(Q6KArgs a) {
         const uint2 packed = q8k_quantize_row32(xv[p], lane, dv, bs);
         int s16 = sdot4(packed.y, 0x01010101u, sdot4(packed.x, 0x01010101u, 0));
         s16 += row_shr_i32<1>(s16);  // odd lanes: the sum of 16 consecutive quants
-        if (u < NSTEPS) {
+        if (s0 + u < s1) {
             const int sbk = s0 + u;
             reinterpret_cast<uint2 *>(ys)[sbk * 32 + ql32] = packed;
             if (ql32 & 1) bsum16[sbk * 16 + (ql32 >> 1)] = s16;
@@ -423,7 +432,7 @@ __global__ __launch_bounds__(512) void gemv_q6k_cu_kcut_kernel(Q6KArgs a) {
 
     float acc[1] = {0.0f};
     auto compute = [&](const Q6KRegs<1> &b, int step) __attribute__((always_inline)) {
-        q6k_compute<1, false, 1>(b, l, s0 + step, s0 + NSTEPS, ys, bsum16, yds, NSB, acc, nullptr);
+        q6k_compute<1, false, 1>(b, l, s0 + step, s1, ys, bsum16, yds, NSB, acc, nullptr);
         __builtin_amdgcn_sched_barrier(0);
     };
 #pragma unroll
@@ -468,7 +477,22 @@ int q6k_ksplit_for(int64_t rows, int64_t n_sb) { return pick_ksplit_q6k(rows, n_
 static bool q6k_cu_kcut_serves(int64_t rows, int64_t n_sb) {
     return n_sb == 56 && pick_ksplit_q6k(rows, n_sb) == 4 && env_int("CAMELID_HIP_Q6K_CU", 1) != 0;
 }
-bool gemv_q6k_long_rows_fuse(const cml_weight *w) { return w->fmt == CML_Q6_K && q6k_cu_kcut_serves(w->rows, w->nb); }
+// Steps per part (the longest part's super-blocks) of the general K-cut form, 0 where it does not serve.
+// CAMELID_HIP_Q6K_KCUT_ANY=0 leaves these shapes to the four-wave launches.
+static int q6k_cu_kcut_any_steps(int64_t rows, int64_t n_sb) {
+    if (!env_int("CAMELID_HIP_Q6K_KCUT_ANY", 1) || !env_int("CAMELID_HIP_Q6K_CU", 1)) return 0;
+    const int ks = pick_ksplit_q6k(rows, n_sb);
+    if (ks != 2 && ks != 4) return 0;
+    const int steps = static_cast<int>((n_sb + ks - 1) / ks);
+    for (int served : {4, 5, 6, 8, 11, 14, 19, 7, 10, 12, 16}) {
+        const bool four_ways = served == 5 || served == 11 || served == 14 || served == 19, two_ways = served == 7 || served == 10 || served == 12 || served == 16;
+        if (steps == served && !(ks == 4 && two_ways) && !(ks == 2 && four_ways)) return steps;
+    }
+    return 0;
+}
+bool gemv_q6k_long_rows_fuse(const cml_weight *w) {
+    return w->fmt == CML_Q6_K && (q6k_cu_kcut_serves(w->rows, w->nb) || q6k_cu_kcut_any_steps(w->rows, w->nb) != 0);
+}
 
 static size_t q6k_lds_bytes(int nt, int n_sb) {
     return static_cast<size_t>(nt) * n_sb * (256 + 64) + ((static_cast<size_t>(nt) * n_sb + 3) & ~size_t(3)) * 4 + 4 * nt * 8 * 4;
@@ -680,10 +704,45 @@ int launch_gemv_q6k_f32(const cml_weight *w, const float *x, float *out, hipStre
     const unsigned gx = static_cast<unsigned>((tiles + tiles_per_wg - 1) / tiles_per_wg);
     const size_t lds = q6k_lds_bytes(n_tokens, ka.n_sb);
     if (lds > 64 * 1024) return fail(CML_ERR_UNSUPPORTED, "Q6_K activation of %d super-blocks exceeds the LDS staging limit", ka.n_sb);
-    if (n_tokens == 1 && q6k_cu_kcut_serves(ka.rows, ka.n_sb)) {
+    if (n_tokens == 1 && q6k_cu_kcut_serves(ka.rows, ka.n_sb) && tiles <= 2 * 256) {
         // (ring of 3 / 4 / 5 / 6 one-super-block buffers: 10.61 / 10.42 / 10.86 / 11.32 us at 4096 x 14336)
         hipLaunchKernelGGL((gemv_q6k_cu_kcut_kernel<4, 14>), dim3(static_cast<unsigned>((tiles + 1) / 2)), dim3(512), 0, st, ka);
         CML_COUNT_LAUNCH("q6k.dot.wg8.kcut.fused");
+        CML_HIP_TRY(hipGetLastError());
+        return CML_OK;
+    }
+    if (const int any_steps = n_tokens == 1 ? q6k_cu_kcut_any_steps(ka.rows, ka.n_sb) : 0) {
+        // the general K-cut form: eight waves, or twelve where eight would need more than one workgroup per compute unit
+        const int ks = ka.ksplit;
+        int waves = env_int("CAMELID_HIP_Q6K_KCUT_WAVES", 0);
+        if (waves != 8 && waves != 12) waves = (tiles + 8 / ks - 1) / (8 / ks) <= 256 ? 8 : 12;
+        const int tpw = waves / ks;
+        const dim3 grid(static_cast<unsigned>((tiles + tpw - 1) / tpw)), block(64 * waves);
+        const size_t lds_any = static_cast<size_t>(ka.n_sb) * (256 + 64 + 4);
+#define CML_Q6K_KCUT_ANY(KS_, NS_)                                                                                          \
+    case KS_ * 100 + NS_:                                                                                                   \
+        if (waves == 8) hipLaunchKernelGGL((gemv_q6k_cu_kcut_kernel<KS_, NS_, 4, 8, true>), grid, block, lds_any, st, ka);   \
+        else hipLaunchKernelGGL((gemv_q6k_cu_kcut_kernel<KS_, NS_, 4, 12, true>), grid, block, lds_any, st, ka);             \
+        break;
+        switch (ks * 100 + any_steps) {
+            CML_Q6K_KCUT_ANY(4, 4)
+            CML_Q6K_KCUT_ANY(4, 5)
+            CML_Q6K_KCUT_ANY(4, 6)
+            CML_Q6K_KCUT_ANY(4, 8)
+            CML_Q6K_KCUT_ANY(4, 11)
+            CML_Q6K_KCUT_ANY(4, 14)
+            CML_Q6K_KCUT_ANY(4, 19)
+            CML_Q6K_KCUT_ANY(2, 4)
+            CML_Q6K_KCUT_ANY(2, 6)
+            CML_Q6K_KCUT_ANY(2, 7)
+            CML_Q6K_KCUT_ANY(2, 8)
+            CML_Q6K_KCUT_ANY(2, 10)
+            CML_Q6K_KCUT_ANY(2, 12)
+            CML_Q6K_KCUT_ANY(2, 16)
+            default: return fail(CML_ERR_UNSUPPORTED, "no Q6_K K-cut form for %d super-blocks cut %d ways", ka.n_sb, ks);
+        }
+#undef CML_Q6K_KCUT_ANY
+        CML_COUNT_LAUNCH("q6k.dot.wg8.kcut.fused.any");
         CML_HIP_TRY(hipGetLastError());
         return CML_OK;
     }

@@ -616,7 +616,9 @@ def test_q6k_eight_wave_launch_under_the_k_cut_is_the_two_launch_path(rows):
     band = w.slice(5, rows - 9)
     for i, x in enumerate(acts):
         G.say(f"Q6_K eight-wave K-cut launch {rows}x14336 act={i}")
-        with G.engaged(r"^q6k\.dot\.wg8\.kcut\.fused$", none=(r"^q6k\.dot\.buffers", r"^q6k\.dot\.deep", r"^quantize\.")):
+        # up to 4096 rows (one eight-wave workgroup per compute unit) the form of its own, beyond twelve-wave workgroups of the general one
+        kernel = r"^q6k\.dot\.wg8\.kcut\.fused$" if rows <= 4096 else r"^q6k\.dot\.wg8\.kcut\.fused\.any$"
+        with G.engaged(kernel, none=(r"^q6k\.dot\.buffers", r"^q6k\.dot\.deep", r"^quantize\.")):
             got = G.gpu_matmul_f32(w, x)
             got_band = G.gpu_matmul_f32(band, x)
         with G.env(CAMELID_HIP_Q6K_CU=0), G.engaged(r"^quantize\.q8_k$", r"^q6k\.dot\.", none=(r"^q6k\.dot\.wg8",)):
@@ -626,6 +628,46 @@ def test_q6k_eight_wave_launch_under_the_k_cut_is_the_two_launch_path(rows):
         if i != 1:
             want = oracle.matmul(fmt, wire, cols, x[None, :], order=EXACT_ORDER[fmt], threads=16)[0]
             assert G.max_rel(got, want) <= TOL, (rows, i)
+
+
+@pytest.mark.parametrize("rows,cols", [
+    (4096, 4096), (5003, 5120), (4096, 6144), (3080, 8192), (4096, 11008), (5125, 13824), (3584, 18944),   # cut four ways
+    (8192, 2048), (6200, 3072), (3584, 3584), (11008, 4096), (9216, 5120), (6200, 6144), (8200, 8192),      # cut two ways
+])
+def test_q6k_eight_wave_launch_under_the_k_cut_on_other_rows(rows, cols):
+    """Q6_K rows of 2048 to 18944 values on fewer than 12288 rows (the shape policy cuts K two or four ways, into
+    parts that need not be equal): one launch of eight- or twelve-wave workgroups that quantize the row once each.
+    Same bits as the four-wave launches they replace (CAMELID_HIP_Q6K_KCUT_ANY=0), whatever the workgroup width,
+    on activations built to break a quantizer and on a row band; within 1e-5 of the oracle's uncut chain."""
+    fmt = oracle.Q6_K
+    rng = np.random.default_rng(9600 + rows + cols)
+    wire = G.synth_weight(fmt, rows, cols, seed=9700 + rows + cols)
+    w = Weight.upload(fmt, rows, cols, wire)
+    acts = rng.standard_normal((3, cols)).astype(np.float32)
+    a = acts[0]
+    a[0:256] = 0.0
+    a[256 + 5], a[256 + 6] = 3.5, -3.5
+    a[512 + 6], a[512 + 5] = 3.5, -3.5
+    a[768 + 3], a[768 + 100] = -4.0, 4.0
+    a[-256:] = 2.0
+    acts[1, 3], acts[1, cols - 300] = np.nan, np.nan
+    acts[2, 1::2] = -acts[2, ::2]
+    band = w.slice(5, rows - 9)
+    for i, x in enumerate(acts):
+        G.say(f"Q6_K K-cut launch {rows}x{cols} act={i}")
+        with G.engaged(r"^q6k\.dot\.wg8\.kcut\.fused\.any$", none=(r"^q6k\.dot\.buffers", r"^q6k\.dot\.deep", r"^quantize\.")):
+            got = G.gpu_matmul_f32(w, x)
+            got_band = G.gpu_matmul_f32(band, x)
+        with G.env(CAMELID_HIP_Q6K_KCUT_ANY=0), G.engaged(r"^q6k\.dot\.", none=(r"^q6k\.dot\.wg8",)):
+            four_wave = G.gpu_matmul_f32(w, x)
+        assert G.same_bits(got, four_wave), (rows, cols, i)
+        assert G.same_bits(got_band, got[5:rows - 4]), (rows, cols, i)
+        for width in (8, 12):
+            with G.env(CAMELID_HIP_Q6K_KCUT_WAVES=width), G.engaged(r"^q6k\.dot\.wg8\.kcut\.fused\.any$"):
+                assert G.same_bits(G.gpu_matmul_f32(w, x), got), (rows, cols, i, width)
+        if i != 1:
+            want = oracle.matmul(fmt, wire, cols, x[None, :], order=EXACT_ORDER[fmt], threads=16)[0]
+            assert G.max_rel(got, want) <= TOL, (rows, cols, i)
 
 
 @pytest.mark.parametrize("rows,cols", [(190, 3072), (64, 256), (333, 4096), (40, 14336), (77, 1280)])
