@@ -482,6 +482,13 @@ static bool q6k_cu_kcut_serves(int64_t rows, int64_t n_sb) {
 static int q6k_cu_kcut_any_steps(int64_t rows, int64_t n_sb) {
     if (!env_int("CAMELID_HIP_Q6K_KCUT_ANY", 1) || !env_int("CAMELID_HIP_Q6K_CU", 1)) return 0;
     const int ks = pick_ksplit_q6k(rows, n_sb);
+    if (ks == 1) {
+        // no K cut: while twelve-wave workgroups still come to one per compute unit.  us per step against the four-wave
+        // launches: 14336 x 4096 10.27 / 10.78, 18944 x 3584 (ten waves) 12.12 / 14.46, 16384 x 4096 10.6 / 11.18,
+        // 12288 x 4096 9.9 / 10.5, 13824 x 5120 13.65 / 13.85, 24576 x 4096 (twelve) 14.8 / 15.05
+        const bool length = n_sb == 12 || n_sb == 14 || n_sb == 16 || n_sb == 20 || n_sb == 24 || n_sb == 32;
+        return length && (rows + 7) / 8 <= 12 * 256 ? static_cast<int>(n_sb) : 0;
+    }
     if (ks != 2 && ks != 4) return 0;
     const int steps = static_cast<int>((n_sb + ks - 1) / ks);
     for (int served : {4, 5, 6, 8, 11, 14, 19, 7, 10, 12, 16}) {
@@ -715,7 +722,10 @@ int launch_gemv_q6k_f32(const cml_weight *w, const float *x, float *out, hipStre
         // the general K-cut form: eight waves, or twelve where eight would need more than one workgroup per compute unit
         const int ks = ka.ksplit;
         int waves = env_int("CAMELID_HIP_Q6K_KCUT_WAVES", 0);
-        if (waves != 8 && waves != 12) waves = (tiles + 8 / ks - 1) / (8 / ks) <= 256 ? 8 : 12;
+        if (waves != 8 && waves != 12 && !(waves == 10 && ks == 1)) {
+            waves = 8;
+            while (waves < 12 && (tiles + waves / ks - 1) / (waves / ks) > 256) waves += ks == 1 ? 2 : 4;
+        }
         const int tpw = waves / ks;
         const dim3 grid(static_cast<unsigned>((tiles + tpw - 1) / tpw)), block(64 * waves);
         const size_t lds_any = static_cast<size_t>(ka.n_sb) * (256 + 64 + 4);
@@ -739,6 +749,20 @@ int launch_gemv_q6k_f32(const cml_weight *w, const float *x, float *out, hipStre
             CML_Q6K_KCUT_ANY(2, 10)
             CML_Q6K_KCUT_ANY(2, 12)
             CML_Q6K_KCUT_ANY(2, 16)
+            // no K cut (12288 to 24576 rows): the same launch, every wave a row tile of its own
+#define CML_Q6K_CU_ANY(NS_)                                                                                                \
+    case 100 + NS_:                                                                                                        \
+        if (waves == 8) hipLaunchKernelGGL((gemv_q6k_cu_kcut_kernel<1, NS_, 4, 8, true>), grid, block, lds_any, st, ka);    \
+        else if (waves == 10) hipLaunchKernelGGL((gemv_q6k_cu_kcut_kernel<1, NS_, 4, 10, true>), grid, block, lds_any, st, ka); \
+        else hipLaunchKernelGGL((gemv_q6k_cu_kcut_kernel<1, NS_, 4, 12, true>), grid, block, lds_any, st, ka);              \
+        break;
+            CML_Q6K_CU_ANY(12)
+            CML_Q6K_CU_ANY(14)
+            CML_Q6K_CU_ANY(16)
+            CML_Q6K_CU_ANY(20)
+            CML_Q6K_CU_ANY(24)
+            CML_Q6K_CU_ANY(32)
+#undef CML_Q6K_CU_ANY
             default: return fail(CML_ERR_UNSUPPORTED, "no Q6_K K-cut form for %d super-blocks cut %d ways", ka.n_sb, ks);
         }
 #undef CML_Q6K_KCUT_ANY

@@ -633,10 +633,12 @@ def test_q6k_eight_wave_launch_under_the_k_cut_is_the_two_launch_path(rows):
 @pytest.mark.parametrize("rows,cols", [
     (4096, 4096), (5003, 5120), (4096, 6144), (3080, 8192), (4096, 11008), (5125, 13824), (3584, 18944),   # cut four ways
     (8192, 2048), (6200, 3072), (3584, 3584), (11008, 4096), (9216, 5120), (6200, 6144), (8200, 8192),      # cut two ways
+    (14336, 4096), (18944, 3584), (13000, 5120), (12300, 3072), (24570, 4096), (12400, 8192),                # no cut
 ])
 def test_q6k_eight_wave_launch_under_the_k_cut_on_other_rows(rows, cols):
     """Q6_K rows of 2048 to 18944 values on fewer than 12288 rows (the shape policy cuts K two or four ways, into
-    parts that need not be equal): one launch of eight- or twelve-wave workgroups that quantize the row once each.
+    parts that need not be equal), and rows of 3072 to 8192 values on 12288 to 24576 rows (no cut): one launch of
+    eight-, ten- or twelve-wave workgroups, at most one per compute unit, that quantize the row once each.
     Same bits as the four-wave launches they replace (CAMELID_HIP_Q6K_KCUT_ANY=0), whatever the workgroup width,
     on activations built to break a quantizer and on a row band; within 1e-5 of the oracle's uncut chain."""
     fmt = oracle.Q6_K
