@@ -601,6 +601,19 @@ static int launch_b32_f32_p(const cml_weight *w, const float *x, float *out, hip
         // token (128256 x 3072: 34.1 -> 33.3 us; Q8_0 there is the same 59.2 us with 4, 8 or 16)
         if (FMT == CML_Q4_0 && ba.nb <= 128 && ba.rows >= 65536) waves = 16;
     }
+    // Rows of more than 4096 values (the token is staged through LDS by every workgroup), one token, 16 lanes per row:
+    // sixteen waves once eight-wave workgroups would outnumber the compute units (Q8_0 14336 x 8192: 30.0 -> 23.3 us,
+    // 28672 x 8192 52.4 -> 42.2, 10240 x 8192 25.6 -> 18.4; Q4_0 14336 x 8192 15.9 -> 14.5, 9216 x 5120 9.23 -> 8.49);
+    // Q8_0 rows of 8192 values on up to 8192 rows: four waves and two-step buffers (8192 x 8192: 19.3 -> 16.2 us,
+    // 6144 x 8192 15.6 -> 13.5; shorter rows and Q4_0 keep eight: 8192 x 6144 11.1 against 11.9, Q4_0 8192 x 8192 10.95 against 12.6)
+    bool shallow = false;
+    if (P == 16 && !two && !w2 && ba.nb > 128 && !env_int("CAMELID_HIP_B32_FUSED_WAVES", 0) && env_int("CAMELID_HIP_B32_LONG_ROW_WAVES", 1)) {
+        if (ba.rows > 256 * 8 * (64 / P)) {
+            if (FMT == CML_Q4_0 || ba.nb >= 256 || ba.rows < 16384) waves = 16;  // (Q8_0 16384 x 6144 and 32000 x 5120: 1 % slower with sixteen)
+        } else if (FMT == CML_Q8_0 && ba.nb >= 256) {
+            waves = 4, shallow = true;
+        }
+    }
     if (two && waves != 4) waves = 8;  // the two-token variants: four or eight waves
     if (P > 16) waves = 8;
     const int rows_per_wg = waves * (64 / P);
@@ -630,7 +643,7 @@ static int launch_b32_f32_p(const cml_weight *w, const float *x, float *out, hip
     }
 #define CML_B32_FUSED(W_, N_) \
     hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, true, W_, N_>), dim3(gx, 1), dim3(W_ * 64), lds, st, ba)
-    const bool deep = !two && nxq == 0 && b32_depth(ba.rows, P, ba.nb) == 4;
+    const bool deep = !two && nxq == 0 && !shallow && b32_depth(ba.rows, P, ba.nb) == 4;
     if constexpr (P > 16) {
         // wide rows: eight-wave workgroups only (the launcher below sets them), single token
         if (two || waves != 8) return fail(CML_ERR_UNSUPPORTED, "rows of %d lanes take one token and eight-wave workgroups", P);
@@ -655,6 +668,7 @@ static int launch_b32_f32_p(const cml_weight *w, const float *x, float *out, hip
     } else if (deep) {
         if (waves == 2) hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, true, 2, 0, 4>), dim3(gx, 1), dim3(128), lds, st, ba);
         else if (waves == 8) hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, true, 8, 0, 4>), dim3(gx, 1), dim3(512), lds, st, ba);
+        else if (waves == 16) hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, true, 16, 0, 4>), dim3(gx, 1), dim3(1024), lds, st, ba);
         else hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, true, 4, 0, 4>), dim3(gx, 1), dim3(256), lds, st, ba);
     } else if (waves == 16) {
         if (nxq == 1) CML_B32_FUSED(16, 1);
@@ -684,7 +698,7 @@ static int launch_b32_f32_p(const cml_weight *w, const float *x, float *out, hip
                                 (nxq == 1 || nxq == 2);
         if (two) { if (waves == 8) CML_COUNT_LAUNCH((b32_counter<FMT, P>("w8.fused.two"))); else CML_COUNT_LAUNCH((b32_counter<FMT, P>("w4.fused.two"))); }
         else if (ring_taken) CML_COUNT_LAUNCH((b32_counter<FMT, P>("w8.ring.fused")));
-        else if (deep) { if (waves == 2) CML_COUNT_LAUNCH((b32_counter<FMT, P>("w2.deep.fused"))); else if (waves == 8) CML_COUNT_LAUNCH((b32_counter<FMT, P>("w8.deep.fused"))); else CML_COUNT_LAUNCH((b32_counter<FMT, P>("w4.deep.fused"))); }
+        else if (deep) { if (waves == 2) CML_COUNT_LAUNCH((b32_counter<FMT, P>("w2.deep.fused"))); else if (waves == 8) CML_COUNT_LAUNCH((b32_counter<FMT, P>("w8.deep.fused"))); else if (waves == 16) CML_COUNT_LAUNCH((b32_counter<FMT, P>("w16.deep.fused"))); else CML_COUNT_LAUNCH((b32_counter<FMT, P>("w4.deep.fused"))); }
         else if (waves == 16) CML_COUNT_LAUNCH((b32_counter<FMT, P>("w16.fused")));
         else if (waves == 8) CML_COUNT_LAUNCH((b32_counter<FMT, P>("w8.fused")));
         else if (waves == 2) CML_COUNT_LAUNCH((b32_counter<FMT, P>("w2.fused")));

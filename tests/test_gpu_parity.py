@@ -800,6 +800,42 @@ def test_b32_fused_quantize_matvec_is_the_two_step_path(name, fmt, rows, cols):
 
 
 @pytest.mark.parametrize("name,fmt", [("Q8_0", oracle.Q8_0), ("Q4_0", oracle.Q4_0)])
+@pytest.mark.parametrize("rows,cols", [(9001, 5120), (8192, 8192), (10250, 8192), (6000, 8192)])
+def test_b32_fused_launch_shapes_on_rows_longer_than_4096_values(name, fmt, rows, cols):
+    """Single-token cml_matmul_f32 on Q8_0 / Q4_0 rows of more than 4096 values (every workgroup stages the token
+    through LDS): sixteen-wave workgroups beyond 8192 rows, four-wave ones with two-step buffers for Q8_0 rows of
+    8192 values on up to 8192 rows, eight-wave ones otherwise.  The counters show which launch ran; each gives the
+    oracle's bits and those of quantize + matvec, as does every workgroup width and buffer depth the knobs select."""
+    rng = np.random.default_rng(9800 + rows + fmt)
+    wire = G.synth_weight(fmt, rows, cols, seed=9900 + rows + fmt)
+    w = Weight.upload(fmt, rows, cols, wire)
+    x = rng.standard_normal(cols).astype(np.float32)
+    x[:64] = 0.0
+    x[64:70] = [2.5, 0.5, -0.5, -2.5, 1.5, -1.5]
+    want = oracle.matmul(fmt, wire, cols, x[None, :], order=EXACT_ORDER[fmt], threads=16)[0]
+    fam = "q8_0" if fmt == oracle.Q8_0 else "q4_0"
+    if rows > 8192:
+        kernel = rf"^{fam}\.dot\.p16\.w16\.fused$"
+    elif fmt == oracle.Q8_0 and cols >= 8192:
+        kernel = rf"^{fam}\.dot\.p16\.w4\.fused$"
+    else:
+        kernel = rf"^{fam}\.dot\.p16\.w8\.(deep\.)?fused$"
+    G.say(f"{name} {rows}x{cols}: default launch")
+    with G.engaged(kernel, none=(r"^quantize\.",)):
+        got = G.gpu_matmul_f32(w, x)
+    assert G.same_bits(got, want), (name, rows, cols)
+    with G.env(CAMELID_HIP_FUSED_QUANT=0), G.engaged(r"^quantize\.q8_0$"):
+        assert G.same_bits(G.gpu_matmul_f32(w, x), want), (name, rows, cols, "two launches")
+    with G.env(CAMELID_HIP_B32_LONG_ROW_WAVES=0), G.engaged(rf"^{fam}\.dot\.p16\.w8\.(deep\.)?fused$"):
+        assert G.same_bits(G.gpu_matmul_f32(w, x), want), (name, rows, cols, "eight waves")
+    for waves in (4, 8, 16):
+        for depth in (2, 4):
+            G.say(f"{name} {rows}x{cols}: waves={waves} depth={depth}")
+            with G.env(CAMELID_HIP_B32_FUSED_WAVES=waves, CAMELID_HIP_B32_DEPTH=depth), G.engaged(rf"^{fam}\.dot\.p16\.w{waves}\."):
+                assert G.same_bits(G.gpu_matmul_f32(w, x), want), (name, rows, cols, waves, depth)
+
+
+@pytest.mark.parametrize("name,fmt", [("Q8_0", oracle.Q8_0), ("Q4_0", oracle.Q4_0)])
 @pytest.mark.parametrize("rows,cols", [(190, 2048), (33, 32), (70, 3072 + 32), (5000, 1024), (16, 8192), (333, 4096), (14336, 4096)])
 def test_b32_fused_two_tokens_is_the_two_step_path(name, fmt, rows, cols):
     """Two-token cml_matmul_f32 on Q8_0 / Q4_0 weights quantizes both rows inside the matvec
