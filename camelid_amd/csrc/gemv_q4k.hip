@@ -1669,7 +1669,7 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
 #define CML_Q4K_LAUNCH(SPR_, WHOLE_, PLAIN_) hipLaunchKernelGGL((gemv_q4k_kernel<1, false, true, SPR_, WHOLE_, PLAIN_>), grid, block, lds, st, ka)
         if (loads_only && half_tiles && ring && plain && q4k_cu_serves(ka, shape.ksplit) && ka.n_sb == 16) {
             if (int rc = launch_q4k_cu(ka, ablate, st)) return rc;
-        } else if (loads_only && half_tiles && plain && q4k_cu_kcut_serves(ka, shape.ksplit)) {
+        } else if (loads_only && half_tiles && plain && q4k_cu_kcut_serves(ka, shape.ksplit) && ka.n_sb == 56 && !q4k_cu_kcut_any_steps(ka, shape.ksplit)) {
             if (int rc = launch_q4k_cu_kcut(ka, st, ablate)) return rc;
         } else if (loads_only && ablate != 7) {
             return fail(CML_ERR_UNSUPPORTED, "this ablation exists for the eight-wave single-token launch (rows of 4096 values, no K cut)");

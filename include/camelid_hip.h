@@ -472,7 +472,8 @@ int cml_calibrate_weight_loads(const cml_weight *w, void *scratch_dev, cml_strea
  * taken out, to time what each part costs: mask 1 = no activation (no f32 loads, no quantizer, no
  * barrier), 4 = no output store, 7 = the weight requests alone.  Served for rows of 4096 values on
  * 12288 to 16384 rows (the eight-wave launch) and for rows of 14336 values on 3072 to 6128 rows (its
- * K-cut form); CML_ERR_UNSUPPORTED otherwise.  out_dev must hold w's rows and is garbage afterwards. */
+ * eight-wave K-cut form, which is also what cml_matmul_f32 launches up to 4096 rows; beyond it launches
+ * twelve-wave workgroups); CML_ERR_UNSUPPORTED otherwise.  out_dev must hold w's rows and is garbage afterwards. */
 int cml_calibrate_matvec_ablation(const cml_weight *w, const float *x_dev, float *out_dev, int mask, cml_stream_t stream);
 
 #ifdef __cplusplus

@@ -799,6 +799,26 @@ def test_b32_fused_quantize_matvec_is_the_two_step_path(name, fmt, rows, cols):
             assert G.same_bits(fused, want)
 
 
+@pytest.mark.parametrize("rows,cols", [(14336, 4096), (4096, 14336), (5120, 14336), (4096, 4096), (4096, 11008), (11008, 4096),
+                                       (18944, 3584), (13824, 5120), (200, 2304), (32000, 4096)])
+def test_q4k_loads_only_twin_runs_for_every_single_token_launch_shape(rows, cols):
+    """cml_calibrate_weight_loads (the matvec's weight requests and nothing else, what bench.py prices a shape's
+    ceiling with) is served whatever launch cml_matmul_f32 picks for the shape, and leaves the weight intact."""
+    fmt = oracle.Q4_K
+    wire = G.synth_weight(fmt, rows, cols, seed=9950 + rows + cols)
+    w = Weight.upload(fmt, rows, cols, wire)
+    x = np.random.default_rng(9960 + rows).standard_normal(cols).astype(np.float32)
+    before = G.gpu_matmul_f32(w, x)
+    scratch = DeviceBuffer(256)
+    stream = C.c_void_p()
+    check(lib().cml_stream_create(C.byref(stream)))
+    G.say(f"Q4_K loads-only twin {rows}x{cols}")
+    with G.engaged(r"^q4k\.calibrate\."):
+        check(lib().cml_calibrate_weight_loads(w.handle, scratch.ptr, stream), "cml_calibrate_weight_loads")
+        check(lib().cml_stream_sync(stream))
+    assert G.same_bits(G.gpu_matmul_f32(w, x), before)
+
+
 @pytest.mark.parametrize("name,fmt", [("Q8_0", oracle.Q8_0), ("Q4_0", oracle.Q4_0)])
 @pytest.mark.parametrize("rows,cols", [(9001, 5120), (8192, 8192), (10250, 8192), (6000, 8192)])
 def test_b32_fused_launch_shapes_on_rows_longer_than_4096_values(name, fmt, rows, cols):
