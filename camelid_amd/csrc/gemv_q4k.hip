@@ -878,7 +878,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_cu_kcut_kernel(std::condi
     // (more slots requested ahead of the quantizer are slower: 3 of 3 7.87 us, 4 of 4 7.85, 5 of 5 8.1, all 7 9.45 against 7.64 --
     // requests for several far-apart super-blocks per wave at once break up the front the grid sweeps the matrix with)
     constexpr int NB = NSTEPS < 3 ? NSTEPS : 3, PRE = 2;
-    static_assert((KS == 2 || KS == 4) && WAVES % KS == 0 && NSTEPS >= 2, "K parts of at least two steps");
+    static_assert((KS == 2 || KS == 4 || KS == 8) && WAVES % KS == 0 && NSTEPS >= 2, "K parts of at least two steps");
     using Regs = Q4KRegs<1>;
     __shared__ __attribute__((aligned(16))) int8_t ys[NSB * 256];
     __shared__ int bsum[NSB * 8];
@@ -1020,7 +1020,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_cu_kcut_any_kernel(Q4KCuA
     static_assert(WAVES % KS == 0 && WAVES >= 8 && WAVES <= 16, "whole half tiles per workgroup");
     constexpr int PASSES = (MAXSTEPS + TPW - 1) / TPW;
     constexpr int NB = MAXSTEPS < 3 ? MAXSTEPS : 3, PRE = 2;
-    static_assert((KS == 2 || KS == 4) && MAXSTEPS >= 2, "K parts of at least two steps");
+    static_assert((KS == 2 || KS == 4 || KS == 8) && MAXSTEPS >= 2, "K parts of at least two steps");
     using Regs = Q4KRegs<1>;
     extern __shared__ uint4 smem_any[];
     int8_t *ys = reinterpret_cast<int8_t *>(smem_any);           // [n_sb * 256]
@@ -1127,6 +1127,7 @@ static int q4k_cu_kcut_any_steps(const Q4KArgs &ka, int ksplit) {
     const bool whole_steps = ka.n_sb % (2 * ksplit) == 0;
     if (ksplit == 4) return (whole_steps ? steps > 4 && steps <= 10 : steps >= 3 && steps <= 10) ? steps : 0;
     if (ksplit == 2) return (whole_steps ? steps == 7 : steps >= 3 && steps <= 7) ? steps : 0;  // (28 steps, 8192 x 28672: 90-124 us against 26.6, the unrolled walk spills)
+    if (ksplit == 8) return (whole_steps ? steps > 4 && steps <= 6 : steps >= 3 && steps <= 6) ? steps : 0;
     return 0;
 }
 
@@ -1143,16 +1144,18 @@ static int q4k_cu_kcut_waves(const Q4KArgs &ka, int ksplit) {
         env_int("CAMELID_HIP_Q4K_RING", 1) == 0)
         return 0;
     if (ksplit == 4 && ka.n_sb == 56) return 8;
-    if ((ksplit != 2 && ksplit != 4) || !env_int("CAMELID_HIP_Q4K_KCUT_SHORT", 1)) return 0;
+    if ((ksplit != 2 && ksplit != 4 && ksplit != 8) || !env_int("CAMELID_HIP_Q4K_KCUT_SHORT", 1)) return 0;
+    // fewer than 96 eight-wave workgroups leave too many compute units idle (2048 x 2048, 64 of them: 2.95 us against 2.88)
+    if (((ka.rows + ka.row_skip + 15) / 16 * 2 + 8 / ksplit - 1) / (8 / ksplit) < 96) return 0;
     if (q4k_cu_kcut_any_steps(ka, ksplit)) return 8;
     if (ka.n_sb % (2 * ksplit) != 0) return 0;
     const int nsteps = ka.n_sb / (2 * ksplit);
-    if (ksplit == 4 ? (nsteps < 2 || nsteps > 4) : (nsteps < 3 || nsteps == 7 || nsteps > 8)) return 0;
+    if (ksplit == 2 ? (nsteps < 2 || nsteps == 7 || nsteps > 8) : (nsteps < 2 || nsteps > 4)) return 0;
     const int only = env_int("CAMELID_HIP_Q4K_KCUT_WAVES", 0);
-    if (only == 8 || only == 12 || only == 16) return only;
+    if (only == 8 || only == 16 || (only == 12 && ksplit != 8)) return only;  // whole half tiles per workgroup: eight parts take 8 or 16 waves
     const int half_tiles = (ka.rows + ka.row_skip + 15) / 16 * 2;
     int waves = 8;
-    while (waves < 16 && (half_tiles + waves / ksplit - 1) / (waves / ksplit) > kComputeUnits) waves += 4;
+    while (waves < 16 && (half_tiles + waves / ksplit - 1) / (waves / ksplit) > kComputeUnits) waves += ksplit == 8 ? 8 : 4;
     return waves;
 }
 static bool q4k_cu_kcut_serves(const Q4KArgs &ka, int ksplit) { return q4k_cu_kcut_waves(ka, ksplit) != 0; }
@@ -1167,8 +1170,9 @@ static int launch_q4k_cu_kcut(const Q4KArgs &ka, hipStream_t st, int ablate = 0)
         int waves = env_int("CAMELID_HIP_Q4K_KCUT_WAVES", 0);
         if (waves != 8 && waves != 12 && waves != 16) {
             waves = 8;
-            while (waves < 16 && (2 * tiles16 + waves / ks - 1) / (waves / ks) > kComputeUnits) waves += 4;
+            while (waves < 16 && (2 * tiles16 + waves / ks - 1) / (waves / ks) > kComputeUnits) waves += ks == 8 ? 8 : 4;
         }
+        if (ks == 8 && waves == 12) waves = 16;
         const int tpw = waves / ks;
         const dim3 grid(static_cast<unsigned>((2 * tiles16 + tpw - 1) / tpw)), block(64 * waves);
         const size_t lds = static_cast<size_t>(ka.n_sb) * (256 + 32) + ((static_cast<size_t>(ka.n_sb) + 3) & ~size_t(3)) * 4 + 16 * 8 * 4;
@@ -1193,6 +1197,16 @@ static int launch_q4k_cu_kcut(const Q4KArgs &ka, hipStream_t st, int ablate = 0)
             CML_Q4K_KCUT_ANY(2, 5)
             CML_Q4K_KCUT_ANY(2, 6)
             CML_Q4K_KCUT_ANY(2, 7)
+#define CML_Q4K_KCUT_ANY8(NS_)                                                                                      \
+    case 8 * 100 + NS_:                                                                                             \
+        if (waves == 8) hipLaunchKernelGGL((gemv_q4k_cu_kcut_any_kernel<8, NS_, 8>), grid, block, lds, st, aa);     \
+        else hipLaunchKernelGGL((gemv_q4k_cu_kcut_any_kernel<8, NS_, 16>), grid, block, lds, st, aa);               \
+        break;
+            CML_Q4K_KCUT_ANY8(3)
+            CML_Q4K_KCUT_ANY8(4)
+            CML_Q4K_KCUT_ANY8(5)
+            CML_Q4K_KCUT_ANY8(6)
+#undef CML_Q4K_KCUT_ANY8
             default: return fail(CML_ERR_UNSUPPORTED, "no K-cut form for %d super-blocks cut %d ways", ka.n_sb, ks);
         }
 #undef CML_Q4K_KCUT_ANY
@@ -1213,11 +1227,21 @@ static int launch_q4k_cu_kcut(const Q4KArgs &ka, hipStream_t st, int ablate = 0)
             CML_Q4K_KCUT(4, 2)
             CML_Q4K_KCUT(4, 3)
             CML_Q4K_KCUT(4, 4)
+            CML_Q4K_KCUT(2, 2)
             CML_Q4K_KCUT(2, 3)
             CML_Q4K_KCUT(2, 4)
             CML_Q4K_KCUT(2, 5)
             CML_Q4K_KCUT(2, 6)
             CML_Q4K_KCUT(2, 8)
+#define CML_Q4K_KCUT8(NS_)                                                                                \
+    case 8 * 100 + NS_:                                                                                   \
+        if (waves == 8) hipLaunchKernelGGL((gemv_q4k_cu_kcut_kernel<8, NS_>), grid, block, 0, st, ca);    \
+        else hipLaunchKernelGGL((gemv_q4k_cu_kcut_kernel<8, NS_, 0, false, 16>), grid, block, 0, st, ca); \
+        break;
+            CML_Q4K_KCUT8(2)
+            CML_Q4K_KCUT8(3)
+            CML_Q4K_KCUT8(4)
+#undef CML_Q4K_KCUT8
             default: return fail(CML_ERR_UNSUPPORTED, "no K-cut form for %d super-blocks cut %d ways", ka.n_sb, ks);
         }
 #undef CML_Q4K_KCUT
@@ -1285,11 +1309,15 @@ static int launch_q4k_cu_kcut_multi(const cml_weight *const *ws, int n, const fl
         CML_Q4K_KCUT(4, 2)
         CML_Q4K_KCUT(4, 3)
         CML_Q4K_KCUT(4, 4)
+        CML_Q4K_KCUT(2, 2)
         CML_Q4K_KCUT(2, 3)
         CML_Q4K_KCUT(2, 4)
         CML_Q4K_KCUT(2, 5)
         CML_Q4K_KCUT(2, 6)
         CML_Q4K_KCUT(2, 8)
+        CML_Q4K_KCUT(8, 2)
+        CML_Q4K_KCUT(8, 3)
+        CML_Q4K_KCUT(8, 4)
         default: return -1;
     }
 #undef CML_Q4K_KCUT
@@ -1472,6 +1500,8 @@ bool gemv_q4k_long_rows_fuse(const cml_weight *w) {
     Q4KArgs ka{};
     ka.n_sb = static_cast<int>(w->nb);
     ka.sb_stride = w->planes.row_stride[0];
+    ka.rows = static_cast<int>(w->rows);
+    ka.row_skip = w->row_skip;
     const int64_t tiles16 = (w->rows + w->row_skip + 15) / 16;
     const int ks = pick_shape(w->rows, ka.n_sb).ksplit;
     return q4k_cu_kcut_serves(ka, ks) && q4k_rows_per_wave(tiles16, ks, 1) == 8 && !env_int("CAMELID_HIP_Q4K_GENERAL_ENTRY", 0);

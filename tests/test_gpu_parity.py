@@ -552,6 +552,8 @@ def test_q4k_eight_wave_launch_under_the_k_cut_is_the_two_launch_path(rows):
     # parts that are no whole number of two-super-block steps, or longer than the forms above take
     (4096, 11008), (5120, 5120), (5125, 13824), (3584, 18944), (3584, 3584), (4100, 10240), (8192, 7168), (3300, 2304),
     (5000, 16384), (4096, 20480),
+    # cut eight ways (fewer than 3072 rows), and rows of 2048 values cut two ways
+    (2048, 8192), (2050, 14336), (2048, 11008), (2560, 10240), (3000, 12288), (8192, 2048), (2048, 5632),
 ])
 def test_q4k_eight_wave_launch_under_the_k_cut_on_shorter_rows(rows, cols):
     """Rows of 2304 to 20480 values on fewer than 12288 rows (attention projections, smaller FFN matrices, the down
@@ -1433,7 +1435,7 @@ def test_matmul_f32_multi_is_the_single_calls(case):
         proof = G.engaged(r"^q6k\.dot\.", none=(r"multi",))
     elif one_launch == 0:
         proof = G.engaged(r"^q4k\.dot\.", none=(r"multi",))
-    elif case in ("qkv_4096", "bands", "cut4_8192", "cut2_4096"):
+    elif case in ("qkv_4096", "cut4_8192", "cut2_4096"):   # ("bands" is too small for eight-wave workgroups to fill the chip)
         proof = G.engaged(r"^q4k\.dot\.wg8\.kcut\.fused\.multi$", none=(r"^q4k\.dot\.(ring|buffers)",))
     else:
         proof = G.engaged(r"^q4k\.dot\.(ring|buffers)\.fused\.multi$")
