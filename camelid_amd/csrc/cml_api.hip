@@ -867,8 +867,8 @@ int cml_matmul_f32(const cml_weight *w, const float *x_dev, int64_t n_tokens, fl
     const int fuse = env_int("CAMELID_HIP_FUSED_QUANT", 1);  // 0 = never, 1 = by shape, 2 = whenever possible
     const bool fuse_two = n_tokens == 2 && env_int("CAMELID_HIP_FUSED_QUANT_TWO", 1) && !env_int("CAMELID_HIP_Q4K_GENERAL_ENTRY", 0);
     if (w->fmt == CML_Q4_K && !q4k_lane_order() && (n_tokens == 1 || fuse_two) &&
-        (fuse == 2 || (fuse == 1 && (w->nb <= 32 || (n_tokens == 1 && gemv_q4k_long_rows_fuse(w)))))) {
-        // rows of up to 8192 values: one launch quantizes the activation in every workgroup (one or
+        (fuse == 2 || (fuse == 1 && (w->nb <= 32 || gemv_q4k_long_rows_fuse(w, static_cast<int>(n_tokens)))))) {
+        // rows of up to 8192 values (and the longer rows the one-launch K-cut forms serve): one launch quantizes the activation in every workgroup (one or
         // two passes of its four waves; twice that for a pair of tokens) and runs the matvec
         // (4096 x 8192: 7.1 -> 6.6 us, 2048 x 8192: 6.3 -> 4.7); at 14336 values the passes cost
         // what the second launch does (4096 x 14336: 9.6 -> 10.0) and the two launches below stay
@@ -876,8 +876,8 @@ int cml_matmul_f32(const cml_weight *w, const float *x_dev, int64_t n_tokens, fl
         if (frc == CML_OK) g_runs.fetch_add(1, std::memory_order_relaxed);
         return frc;
     }
-    if (w->fmt == CML_Q4_K && !q4k_lane_order() && (n_tokens == 3 || n_tokens == 4) && fuse != 0 && w->nb <= 32 &&
-        !env_int("CAMELID_HIP_Q4K_GENERAL_ENTRY", 0)) {
+    if (w->fmt == CML_Q4_K && !q4k_lane_order() && (n_tokens == 3 || n_tokens == 4) && fuse != 0 &&
+        (w->nb <= 32 || gemv_q4k_long_rows_fuse(w, static_cast<int>(n_tokens))) && !env_int("CAMELID_HIP_Q4K_GENERAL_ENTRY", 0)) {
         // three or four tokens on rows of 4096 values with no K cut: the eight-wave packed-dot launch replays each
         // step's unpacked weight against the tokens (one launch, quantizer inside); -1 = not such a shape
         const int frc = launch_gemv_q4k_f32(w, x_dev, out_dev, st, static_cast<int>(n_tokens));

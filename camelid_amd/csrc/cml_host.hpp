@@ -147,7 +147,7 @@ int launch_gemv_q4k(const MatArgs &a, hipStream_t st);
 int launch_gemv_q4k_f32_grouped_pair(const MatArgs &a, const cml_weight *w2, float *out2, const float *x, hipStream_t st);
 int launch_gemv_q4k_f32_pair(const cml_weight *w, const cml_weight *w2, const float *x, float *out, float *out2, hipStream_t st);
 bool gemv_q6k_long_rows_fuse(const cml_weight *w);  // the same for Q6_K
-bool gemv_q4k_long_rows_fuse(const cml_weight *w);  // a single f32 token on this weight is one launch although its rows exceed 8192 values
+bool gemv_q4k_long_rows_fuse(const cml_weight *w, int n_tokens = 1);  // a single f32 token on this weight is one launch although its rows exceed 8192 values
 int launch_gemv_q4k_f32_multi(const cml_weight *const *ws, int n, const float *x, float *const *outs, hipStream_t st);  // -1: not served
 // whether that launch, as a direct call on these two weights, can route the token itself (a.route_logits)
 bool gemv_q4k_direct_can_route(const cml_weight *w, int64_t band_rows, int n_slots, bool pair);

@@ -1007,7 +1007,9 @@ struct Q4KCuAnyArgs {
     int n_sb;  // super-blocks per row
 };
 
-template <int KS, int MAXSTEPS, int WAVES = 8>
+// NT (1 to 3) tokens: contiguous f32 rows in, out[t][rows]; every pass quantizes its super-blocks of all the tokens,
+// and a step's unpacked weight is replayed against them -- every cell the one-token launch's bits.
+template <int KS, int MAXSTEPS, int WAVES = 8, int NT = 1>
 __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_cu_kcut_any_kernel(Q4KCuAnyArgs aa) {
     const Q4KCuArgs &a = aa.one;
     const uint8_t *__restrict__ w = a.w;
@@ -1021,12 +1023,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_cu_kcut_any_kernel(Q4KCuA
     constexpr int PASSES = (MAXSTEPS + TPW - 1) / TPW;
     constexpr int NB = MAXSTEPS < 3 ? MAXSTEPS : 3, PRE = 2;
     static_assert((KS == 2 || KS == 4 || KS == 8) && MAXSTEPS >= 2, "K parts of at least two steps");
+    static_assert(NT >= 1 && NT <= 3, "one to three tokens");
     using Regs = Q4KRegs<1>;
     extern __shared__ uint4 smem_any[];
-    int8_t *ys = reinterpret_cast<int8_t *>(smem_any);           // [n_sb * 256]
-    int *bsum = reinterpret_cast<int *>(ys + n_sb * 256);        // [n_sb * 8]
-    float *yds = reinterpret_cast<float *>(bsum + n_sb * 8);     // [n_sb]
-    float *part = yds + ((n_sb + 3) & ~3);                       // [WAVES * 8]
+    int8_t *ys = reinterpret_cast<int8_t *>(smem_any);               // [NT][n_sb * 256]
+    int *bsum = reinterpret_cast<int *>(ys + NT * n_sb * 256);       // [NT][n_sb * 8]
+    float *yds = reinterpret_cast<float *>(bsum + NT * n_sb * 8);    // [NT][n_sb]
+    float *part = yds + ((NT * n_sb + 3) & ~3);                      // [WAVES][NT][8]
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int tile_in_wg = wave / KS, kpart = wave - tile_in_wg * KS;
@@ -1035,12 +1038,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_cu_kcut_any_kernel(Q4KCuA
     // the f32 activation: pass p of this wave takes the two super-blocks of step TPW p + tile_in_wg of its own part
     const int half = lane >> 5, ql = lane & 31;
     auto pass_sb = [&](int p) __attribute__((always_inline)) -> int { return s0 + 2 * (TPW * p + tile_in_wg) + half; };
-    float4 xv[PASSES][2];
+    float4 xv[PASSES][NT][2];
 #pragma unroll
     for (int p = 0; p < PASSES; p++) {
-        const float4 *x4 = reinterpret_cast<const float4 *>(x) + min(pass_sb(p), n_sb - 1) * 64 + ql * 2;
-        xv[p][0] = x4[0];
-        xv[p][1] = x4[1];
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            const float4 *x4 = reinterpret_cast<const float4 *>(x) + (t * n_sb + min(pass_sb(p), n_sb - 1)) * 64 + ql * 2;
+            xv[p][t][0] = x4[0];
+            xv[p][t][1] = x4[1];
+        }
     }
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_barrier();  // execution only: every activation request of the workgroup is out
@@ -1065,15 +1071,19 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_cu_kcut_any_kernel(Q4KCuA
     // every wave runs every pass (super-blocks outside its part are redone from clamped values and not stored)
     auto quantize_pass = [&](int p) __attribute__((always_inline)) {
         const int sbk = pass_sb(p);
-        float dv;
-        int bs;
-        const uint2 packed = q8k_quantize_row32(xv[p], lane, dv, bs);
-        if (sbk < s1) {
-            reinterpret_cast<uint2 *>(ys)[sbk * 32 + ql] = packed;
-            if ((ql & 3) == 3) bsum[sbk * 8 + (ql >> 2)] = bs;
-            if (ql == 0) yds[sbk] = dv;
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            float dv;
+            int bs;
+            const uint2 packed = q8k_quantize_row32(xv[p][t], lane, dv, bs);
+            if (sbk < s1) {
+                const int at = t * n_sb + sbk;
+                reinterpret_cast<uint2 *>(ys)[at * 32 + ql] = packed;
+                if ((ql & 3) == 3) bsum[at * 8 + (ql >> 2)] = bs;
+                if (ql == 0) yds[at] = dv;
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
-        __builtin_amdgcn_sched_barrier(0);
     };
     quantize_pass(0);
     __syncthreads();
@@ -1082,10 +1092,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_cu_kcut_any_kernel(Q4KCuA
     ln.c = l;
     ln.sh = (l & 1) * 16;
     ln.upper = l >= 2;
-    float acc[1] = {0.0f};
+    float acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++) acc[t] = 0.0f;
     auto compute = [&](const Regs &b, int step) __attribute__((always_inline)) {
-        if (step < MAXSTEPS - 1) q4k_compute<1, false, 1, 2, true>(b, ln, s0 + 2 * step + h, s1, ys, bsum, yds, n_sb, acc, nullptr);
-        else q4k_compute<1, false, 1, 2, false>(b, ln, s0 + 2 * step + h, s1, ys, bsum, yds, n_sb, acc, nullptr);
+        if (step < MAXSTEPS - 1) q4k_compute<NT, false, 1, 2, true>(b, ln, s0 + 2 * step + h, s1, ys, bsum, yds, n_sb, acc, nullptr);
+        else q4k_compute<NT, false, 1, 2, false>(b, ln, s0 + 2 * step + h, s1, ys, bsum, yds, n_sb, acc, nullptr);
         __builtin_amdgcn_sched_barrier(0);
     };
 #pragma unroll
@@ -1097,17 +1109,20 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_cu_kcut_any_kernel(Q4KCuA
         compute(ring[i % NB], i);
         if (i + NB < MAXSTEPS) request(ring[i % NB], i + NB);
     }
-    if (l == LPS - 1 && h == 1) part[wave * 8 + r] = acc[0];
+    if (l == LPS - 1 && h == 1) {
+#pragma unroll
+        for (int t = 0; t < NT; t++) part[(wave * NT + t) * 8 + r] = acc[t];
+    }
     __syncthreads();
-    if (tid < TPW * 8) {
-        const int tw = tid >> 3, rr = tid & 7;
+    if (tid < TPW * NT * 8) {
+        const int rr = tid & 7, t = (tid >> 3) % NT, tw = (tid >> 3) / NT;
         const int orow = (blockIdx.x * TPW + tw) * 8 + rr - row_skip;
         if (orow >= 0 && orow < rows) {
-            float v = part[(tw * KS) * 8 + rr];
+            float v = part[((tw * KS) * NT + t) * 8 + rr];
 #pragma unroll
-            for (int k = 1; k < KS; k++) v = v + part[(tw * KS + k) * 8 + rr];
-            if (residual) v = v + residual[orow];
-            out[orow] = v;
+            for (int k = 1; k < KS; k++) v = v + part[((tw * KS + k) * NT + t) * 8 + rr];
+            if (NT == 1 && residual) v = v + residual[orow];
+            out[static_cast<int64_t>(t) * rows + orow] = v;
         }
     }
 }
@@ -1266,6 +1281,72 @@ static int launch_q4k_cu_kcut(const Q4KArgs &ka, hipStream_t st, int ablate = 0)
         default: return fail(CML_ERR_INVALID, "ablation mask must be 1, 4 or 7");
     }
     CML_COUNT_LAUNCH("q4k.calibrate.wg8.kcut");
+    return CML_OK;
+}
+
+// Two or three tokens under a K cut: the general K-cut form replays each step's unpacked weight against the tokens
+// (one launch, every cell the one-token bits).  Steps per part, 0 where it does not serve (the row lengths of the
+// instantiations below; the tokens' staging must fit LDS; not below 96 workgroups).  Before: two tokens ran on
+// 16-row waves that quantize both rows in every four-wave workgroup (or, beyond 8192 values, after a quantizing
+// launch), three on the matrix cores -- 4096 x 14336: 10.7 / 15.2 us for two / three tokens, 4096 x 4096 5.1 / 7.7.
+// CAMELID_HIP_Q4K_KCUT_TOKENS=0 keeps those.
+static int q4k_cu_kcut_tokens_steps(const Q4KArgs &ka, int ksplit, int n_tokens) {
+    if (n_tokens < 2 || n_tokens > 3 || !env_int("CAMELID_HIP_Q4K_KCUT_TOKENS", 1) || !env_int("CAMELID_HIP_Q4K_KCUT_SHORT", 1)) return 0;
+    if (ka.sb_stride >= (int64_t(1) << 31) || env_int("CAMELID_HIP_Q4K_CU", 1) == 0 || env_int("CAMELID_HIP_Q4K_CLAMPED_LOADS", 0) ||
+        env_int("CAMELID_HIP_Q4K_RING", 1) == 0)
+        return 0;
+    if (ksplit != 2 && ksplit != 4 && ksplit != 8) return 0;
+    if (((ka.rows + ka.row_skip + 15) / 16 * 2 + 8 / ksplit - 1) / (8 / ksplit) < 96) return 0;
+    const size_t lds = static_cast<size_t>(n_tokens) * ka.n_sb * (256 + 32) + ((static_cast<size_t>(n_tokens) * ka.n_sb + 3) & ~size_t(3)) * 4 + 16 * 3 * 8 * 4;
+    if (lds > 64 * 1024) return 0;
+    const int steps = ((ka.n_sb + ksplit - 1) / ksplit + 1) / 2;
+    const bool served = ksplit == 4 ? (steps == 2 || steps == 3 || steps == 4 || steps == 6 || steps == 7 || steps == 10)
+                      : ksplit == 2 ? (steps == 3 || steps == 4 || steps == 5 || steps == 7)
+                                    : (steps == 2 || steps == 3 || steps == 4);
+    return served ? steps : 0;
+}
+
+static int launch_q4k_cu_kcut_tokens(const Q4KArgs &ka, int n_tokens, hipStream_t st) {
+    if (!ka.x) return fail(CML_ERR_INVALID, "null activation");
+    const int ks = ka.ksplit, steps = q4k_cu_kcut_tokens_steps(ka, ks, n_tokens);
+    const int tiles16 = (ka.rows + ka.row_skip + 15) / 16;
+    int waves = 8;
+    if ((2 * tiles16 + 8 / ks - 1) / (8 / ks) > kComputeUnits) waves = ks == 8 ? 16 : 12;
+    const int only = env_int("CAMELID_HIP_Q4K_KCUT_WAVES", 0);
+    if (only == 8 || (only == 12 && ks != 8) || (only == 16 && ks == 8)) waves = only;
+    const int tpw = waves / ks;
+    const dim3 grid(static_cast<unsigned>((2 * tiles16 + tpw - 1) / tpw)), block(64 * waves);
+    const size_t lds = static_cast<size_t>(n_tokens) * ka.n_sb * (256 + 32) + ((static_cast<size_t>(n_tokens) * ka.n_sb + 3) & ~size_t(3)) * 4 +
+                       static_cast<size_t>(waves) * n_tokens * 8 * 4;
+    const Q4KCuAnyArgs aa{Q4KCuArgs{ka.w, ka.x, ka.out, nullptr, static_cast<uint32_t>(ka.sb_stride), ka.rows, ka.row_skip, tiles16}, ka.n_sb};
+#define CML_Q4K_KCUT_TOK(KS_, NS_, WIDE_)                                                                                                  \
+    case KS_ * 100 + NS_:                                                                                                                  \
+        if (n_tokens == 2) {                                                                                                               \
+            if (waves == 8) hipLaunchKernelGGL((gemv_q4k_cu_kcut_any_kernel<KS_, NS_, 8, 2>), grid, block, lds, st, aa);                   \
+            else hipLaunchKernelGGL((gemv_q4k_cu_kcut_any_kernel<KS_, NS_, WIDE_, 2>), grid, block, lds, st, aa);                          \
+        } else {                                                                                                                           \
+            if (waves == 8) hipLaunchKernelGGL((gemv_q4k_cu_kcut_any_kernel<KS_, NS_, 8, 3>), grid, block, lds, st, aa);                   \
+            else hipLaunchKernelGGL((gemv_q4k_cu_kcut_any_kernel<KS_, NS_, WIDE_, 3>), grid, block, lds, st, aa);                          \
+        }                                                                                                                                  \
+        break;
+    switch (ks * 100 + steps) {
+        CML_Q4K_KCUT_TOK(4, 2, 12)
+        CML_Q4K_KCUT_TOK(4, 3, 12)
+        CML_Q4K_KCUT_TOK(4, 4, 12)
+        CML_Q4K_KCUT_TOK(4, 6, 12)
+        CML_Q4K_KCUT_TOK(4, 7, 12)
+        CML_Q4K_KCUT_TOK(4, 10, 12)
+        CML_Q4K_KCUT_TOK(2, 3, 12)
+        CML_Q4K_KCUT_TOK(2, 4, 12)
+        CML_Q4K_KCUT_TOK(2, 5, 12)
+        CML_Q4K_KCUT_TOK(2, 7, 12)
+        CML_Q4K_KCUT_TOK(8, 2, 16)
+        CML_Q4K_KCUT_TOK(8, 3, 16)
+        CML_Q4K_KCUT_TOK(8, 4, 16)
+        default: return fail(CML_ERR_UNSUPPORTED, "no K-cut form for %d tokens on %d super-blocks cut %d ways", n_tokens, ka.n_sb, ks);
+    }
+#undef CML_Q4K_KCUT_TOK
+    CML_COUNT_LAUNCH("q4k.dot.wg8.kcut.fused.tokens");
     return CML_OK;
 }
 
@@ -1495,8 +1576,17 @@ static int q4k_rows_per_wave(int64_t tiles16, int ksplit, int64_t slots) {
 
 // A single f32 token on this weight runs as ONE launch although its rows are longer than the in-kernel quantizer of
 // the four-wave launches takes (the caller's decision between one launch and quantize-then-matvec).
-bool gemv_q4k_long_rows_fuse(const cml_weight *w) {
+bool gemv_q4k_long_rows_fuse(const cml_weight *w, int n_tokens) {
     if (w->fmt != CML_Q4_K || w->rows <= 0) return false;
+    if (n_tokens == 2 || n_tokens == 3) {
+        Q4KArgs ka{};
+        ka.n_sb = static_cast<int>(w->nb);
+        ka.sb_stride = w->planes.row_stride[0];
+        ka.rows = static_cast<int>(w->rows);
+        ka.row_skip = w->row_skip;
+        return q4k_cu_kcut_tokens_steps(ka, pick_shape(w->rows, ka.n_sb).ksplit, n_tokens) != 0 && !env_int("CAMELID_HIP_Q4K_GENERAL_ENTRY", 0);
+    }
+    if (n_tokens != 1) return false;
     Q4KArgs ka{};
     ka.n_sb = static_cast<int>(w->nb);
     ka.sb_stride = w->planes.row_stride[0];
@@ -1715,8 +1805,10 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
                    (a.n_tokens >= 3 || q4k_rows_per_wave(tiles16, shape.ksplit, 1) == 8) &&  // three tokens: at any row count (128256 x 4096: 55.0 us against 66.7)
                    q4k_ring(ka, shape.ksplit) && q4k_cu_serves(ka, shape.ksplit, static_cast<int>(a.n_tokens))) {
             if (int rc = launch_q4k_cu(ka, 0, st, static_cast<int>(a.n_tokens))) return rc;  // a few tokens replayed against each step's weight
+        } else if (plain && (a.n_tokens == 2 || a.n_tokens == 3) && q4k_cu_kcut_tokens_steps(ka, shape.ksplit, static_cast<int>(a.n_tokens))) {
+            if (int rc = launch_q4k_cu_kcut_tokens(ka, static_cast<int>(a.n_tokens), st)) return rc;  // two or three tokens under a K cut
         } else if (!grouped && !w2 && a.n_tokens > 2) {
-            return -1;  // more than two tokens of a plain call: only the eight-wave launch above takes them
+            return -1;  // more than two tokens of a plain call: only the eight-wave launches above take them
         } else if (two) {
             // both tokens in one pass over the weight, 16-row waves as in the two-token matvec
             if (q4k_ring(ka, shape.ksplit, 1)) launch_q4k_ring<2, true, 1>(ka, shape.ksplit, grid, block, lds, st);

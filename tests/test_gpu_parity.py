@@ -592,6 +592,41 @@ def test_q4k_eight_wave_launch_under_the_k_cut_on_shorter_rows(rows, cols):
             assert G.max_rel(got, want) <= TOL, (rows, cols, i)
 
 
+@pytest.mark.parametrize("rows,cols", [(4096, 4096), (4096, 14336), (11008, 4096), (4096, 11008), (5120, 5120), (2048, 8192),
+                                       (5003, 8192), (9216, 5120), (3584, 18944), (8192, 3072)])
+def test_q4k_k_cut_launch_replays_two_and_three_tokens(rows, cols):
+    """Two and three tokens on a weight whose shape the policy cuts K for: one launch of the general K-cut form, each
+    step's unpacked weight replayed against every token's staged row.  Every cell is the single-token call's bits,
+    also on a row band; the counters show the launch, and with it switched off (CAMELID_HIP_Q4K_KCUT_TOKENS=0) the
+    former paths (16-row waves for two tokens, the matrix cores for three) give the same bits."""
+    fmt = oracle.Q4_K
+    rng = np.random.default_rng(10100 + rows + cols)
+    wire = G.synth_weight(fmt, rows, cols, seed=10200 + rows + cols)
+    w = Weight.upload(fmt, rows, cols, wire)
+    x = rng.standard_normal((3, cols)).astype(np.float32)
+    x[0, :256] = 0.0
+    x[1, 1::2] = -x[1, ::2]
+    x[2, 5], x[2, cols - 3] = 7.0, -7.0
+    x[2, 300] = np.nan
+    singles = np.stack([G.gpu_matmul_f32(w, x[t]) for t in range(3)])
+    band = w.slice(5, rows - 9)
+    for n in (2, 3):
+        if n * (cols // 256) * 292 + 1536 > 64 * 1024:
+            continue   # the tokens' staging does not fit LDS: the former paths serve the call
+        G.say(f"Q4_K K-cut launch {rows}x{cols}, {n} tokens")
+        with G.engaged(r"^q4k\.dot\.wg8\.kcut\.fused\.tokens$", none=(r"^q4k\.mfma", r"^q4k\.dot\.ring", r"^q4k\.dot\.buffers", r"^quantize\.")):
+            got = np.asarray(G.gpu_matmul_f32(w, x[:n])).reshape(n, rows)
+            got_band = np.asarray(G.gpu_matmul_f32(band, x[:n])).reshape(n, rows - 9)
+        assert G.same_bits(got, singles[:n]), (rows, cols, n)
+        assert G.same_bits(got_band, got[:, 5:rows - 4]), (rows, cols, n, "band")
+        with G.env(CAMELID_HIP_Q4K_KCUT_TOKENS=0), G.engaged(none=(r"^q4k\.dot\.wg8\.kcut\.fused\.tokens$",)):
+            former = np.asarray(G.gpu_matmul_f32(w, x[:n])).reshape(n, rows)
+        assert G.same_bits(former, got), (rows, cols, n, "former path")
+        for width in (8, 12, 16):
+            with G.env(CAMELID_HIP_Q4K_KCUT_WAVES=width), G.engaged(r"^q4k\.dot\.wg8\.kcut\.fused\.tokens$"):
+                assert G.same_bits(np.asarray(G.gpu_matmul_f32(w, x[:n])).reshape(n, rows), got), (rows, cols, n, width)
+
+
 @pytest.mark.parametrize("rows", [4096, 3100, 6100])
 def test_q6k_eight_wave_launch_under_the_k_cut_is_the_two_launch_path(rows):
     """Q6_K rows of 14336 values on up to 6136 rows (the FFN down projection: the shape policy cuts K four ways):
