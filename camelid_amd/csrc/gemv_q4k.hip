@@ -1023,7 +1023,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_cu_kcut_any_kernel(Q4KCuA
     constexpr int PASSES = (MAXSTEPS + TPW - 1) / TPW;
     constexpr int NB = MAXSTEPS < 3 ? MAXSTEPS : 3, PRE = 2;
     static_assert((KS == 2 || KS == 4 || KS == 8) && MAXSTEPS >= 2, "K parts of at least two steps");
-    static_assert(NT >= 1 && NT <= 3, "one to three tokens");
+    static_assert(NT >= 1 && NT <= 4, "one to four tokens");
     using Regs = Q4KRegs<1>;
     extern __shared__ uint4 smem_any[];
     int8_t *ys = reinterpret_cast<int8_t *>(smem_any);               // [NT][n_sb * 256]
@@ -1284,25 +1284,28 @@ static int launch_q4k_cu_kcut(const Q4KArgs &ka, hipStream_t st, int ablate = 0)
     return CML_OK;
 }
 
-// Two or three tokens under a K cut: the general K-cut form replays each step's unpacked weight against the tokens
+// Two to four tokens under a K cut: the general K-cut form replays each step's unpacked weight against the tokens
 // (one launch, every cell the one-token bits).  Steps per part, 0 where it does not serve (the row lengths of the
 // instantiations below; the tokens' staging must fit LDS; not below 96 workgroups).  Before: two tokens ran on
 // 16-row waves that quantize both rows in every four-wave workgroup (or, beyond 8192 values, after a quantizing
 // launch), three on the matrix cores -- 4096 x 14336: 10.7 / 15.2 us for two / three tokens, 4096 x 4096 5.1 / 7.7.
 // CAMELID_HIP_Q4K_KCUT_TOKENS=0 keeps those.
 static int q4k_cu_kcut_tokens_steps(const Q4KArgs &ka, int ksplit, int n_tokens) {
-    if (n_tokens < 2 || n_tokens > 3 || !env_int("CAMELID_HIP_Q4K_KCUT_TOKENS", 1) || !env_int("CAMELID_HIP_Q4K_KCUT_SHORT", 1)) return 0;
+    if (n_tokens < 2 || n_tokens > 4 || !env_int("CAMELID_HIP_Q4K_KCUT_TOKENS", 1) || !env_int("CAMELID_HIP_Q4K_KCUT_SHORT", 1)) return 0;
     if (ka.sb_stride >= (int64_t(1) << 31) || env_int("CAMELID_HIP_Q4K_CU", 1) == 0 || env_int("CAMELID_HIP_Q4K_CLAMPED_LOADS", 0) ||
         env_int("CAMELID_HIP_Q4K_RING", 1) == 0)
         return 0;
     if (ksplit != 2 && ksplit != 4 && ksplit != 8) return 0;
     if (((ka.rows + ka.row_skip + 15) / 16 * 2 + 8 / ksplit - 1) / (8 / ksplit) < 96) return 0;
-    const size_t lds = static_cast<size_t>(n_tokens) * ka.n_sb * (256 + 32) + ((static_cast<size_t>(n_tokens) * ka.n_sb + 3) & ~size_t(3)) * 4 + 16 * 3 * 8 * 4;
+    const size_t lds = static_cast<size_t>(n_tokens) * ka.n_sb * (256 + 32) + ((static_cast<size_t>(n_tokens) * ka.n_sb + 3) & ~size_t(3)) * 4 + 16 * 4 * 8 * 4;
     if (lds > 64 * 1024) return 0;
     const int steps = ((ka.n_sb + ksplit - 1) / ksplit + 1) / 2;
     const bool served = ksplit == 4 ? (steps == 2 || steps == 3 || steps == 4 || steps == 6 || steps == 7 || steps == 10)
                       : ksplit == 2 ? (steps == 3 || steps == 4 || steps == 5 || steps == 7)
                                     : (steps == 2 || steps == 3 || steps == 4);
+    // four tokens: parts of up to four steps (4096 x 4096 6.15 us against 7.76 on the matrix cores, 11008 x 4096 9.77 against 13.1,
+    // 2048 x 8192 8.5 against 19.4; 4096 x 11008, six steps, 14.3 against 12.9)
+    if (n_tokens == 4 && steps > 4) return 0;
     return served ? steps : 0;
 }
 
@@ -1324,6 +1327,9 @@ static int launch_q4k_cu_kcut_tokens(const Q4KArgs &ka, int n_tokens, hipStream_
         if (n_tokens == 2) {                                                                                                               \
             if (waves == 8) hipLaunchKernelGGL((gemv_q4k_cu_kcut_any_kernel<KS_, NS_, 8, 2>), grid, block, lds, st, aa);                   \
             else hipLaunchKernelGGL((gemv_q4k_cu_kcut_any_kernel<KS_, NS_, WIDE_, 2>), grid, block, lds, st, aa);                          \
+        } else if (n_tokens == 4) {                                                                                                        \
+            if (waves == 8) hipLaunchKernelGGL((gemv_q4k_cu_kcut_any_kernel<KS_, NS_, 8, 4>), grid, block, lds, st, aa);                   \
+            else hipLaunchKernelGGL((gemv_q4k_cu_kcut_any_kernel<KS_, NS_, WIDE_, 4>), grid, block, lds, st, aa);                          \
         } else {                                                                                                                           \
             if (waves == 8) hipLaunchKernelGGL((gemv_q4k_cu_kcut_any_kernel<KS_, NS_, 8, 3>), grid, block, lds, st, aa);                   \
             else hipLaunchKernelGGL((gemv_q4k_cu_kcut_any_kernel<KS_, NS_, WIDE_, 3>), grid, block, lds, st, aa);                          \
@@ -1578,7 +1584,7 @@ static int q4k_rows_per_wave(int64_t tiles16, int ksplit, int64_t slots) {
 // the four-wave launches takes (the caller's decision between one launch and quantize-then-matvec).
 bool gemv_q4k_long_rows_fuse(const cml_weight *w, int n_tokens) {
     if (w->fmt != CML_Q4_K || w->rows <= 0) return false;
-    if (n_tokens == 2 || n_tokens == 3) {
+    if (n_tokens >= 2 && n_tokens <= 4) {
         Q4KArgs ka{};
         ka.n_sb = static_cast<int>(w->nb);
         ka.sb_stride = w->planes.row_stride[0];
@@ -1805,7 +1811,7 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
                    (a.n_tokens >= 3 || q4k_rows_per_wave(tiles16, shape.ksplit, 1) == 8) &&  // three tokens: at any row count (128256 x 4096: 55.0 us against 66.7)
                    q4k_ring(ka, shape.ksplit) && q4k_cu_serves(ka, shape.ksplit, static_cast<int>(a.n_tokens))) {
             if (int rc = launch_q4k_cu(ka, 0, st, static_cast<int>(a.n_tokens))) return rc;  // a few tokens replayed against each step's weight
-        } else if (plain && (a.n_tokens == 2 || a.n_tokens == 3) && q4k_cu_kcut_tokens_steps(ka, shape.ksplit, static_cast<int>(a.n_tokens))) {
+        } else if (plain && a.n_tokens >= 2 && a.n_tokens <= 4 && q4k_cu_kcut_tokens_steps(ka, shape.ksplit, static_cast<int>(a.n_tokens))) {
             if (int rc = launch_q4k_cu_kcut_tokens(ka, static_cast<int>(a.n_tokens), st)) return rc;  // two or three tokens under a K cut
         } else if (!grouped && !w2 && a.n_tokens > 2) {
             return -1;  // more than two tokens of a plain call: only the eight-wave launches above take them

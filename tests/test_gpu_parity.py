@@ -595,7 +595,7 @@ def test_q4k_eight_wave_launch_under_the_k_cut_on_shorter_rows(rows, cols):
 @pytest.mark.parametrize("rows,cols", [(4096, 4096), (4096, 14336), (11008, 4096), (4096, 11008), (5120, 5120), (2048, 8192),
                                        (5003, 8192), (9216, 5120), (3584, 18944), (8192, 3072)])
 def test_q4k_k_cut_launch_replays_two_and_three_tokens(rows, cols):
-    """Two and three tokens on a weight whose shape the policy cuts K for: one launch of the general K-cut form, each
+    """Two and three (on parts of up to four steps: four) tokens on a weight whose shape the policy cuts K for: one launch of the general K-cut form, each
     step's unpacked weight replayed against every token's staged row.  Every cell is the single-token call's bits,
     also on a row band; the counters show the launch, and with it switched off (CAMELID_HIP_Q4K_KCUT_TOKENS=0) the
     former paths (16-row waves for two tokens, the matrix cores for three) give the same bits."""
@@ -603,14 +603,15 @@ def test_q4k_k_cut_launch_replays_two_and_three_tokens(rows, cols):
     rng = np.random.default_rng(10100 + rows + cols)
     wire = G.synth_weight(fmt, rows, cols, seed=10200 + rows + cols)
     w = Weight.upload(fmt, rows, cols, wire)
-    x = rng.standard_normal((3, cols)).astype(np.float32)
+    x = rng.standard_normal((4, cols)).astype(np.float32)
     x[0, :256] = 0.0
     x[1, 1::2] = -x[1, ::2]
     x[2, 5], x[2, cols - 3] = 7.0, -7.0
     x[2, 300] = np.nan
-    singles = np.stack([G.gpu_matmul_f32(w, x[t]) for t in range(3)])
+    singles = np.stack([G.gpu_matmul_f32(w, x[t]) for t in range(4)])
     band = w.slice(5, rows - 9)
-    for n in (2, 3):
+    four = (rows, cols) in ((4096, 4096), (11008, 4096), (5120, 5120), (2048, 8192), (5003, 8192), (8192, 3072))   # parts of up to four steps
+    for n in (2, 3, 4) if four else (2, 3):
         if n * (cols // 256) * 292 + 1536 > 64 * 1024:
             continue   # the tokens' staging does not fit LDS: the former paths serve the call
         G.say(f"Q4_K K-cut launch {rows}x{cols}, {n} tokens")
