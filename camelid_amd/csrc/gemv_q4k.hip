@@ -1544,7 +1544,12 @@ static Q4KShape pick_shape(int64_t rows, int64_t n_sb) {
     if ((forced == 1 || forced == 2 || forced == 4 || forced == 8) && forced <= n_sb) {
         ks = forced;
     } else if (!env_int("CAMELID_HIP_EXACT_ORDER", 0)) {
-        while (ks < 8 && tiles * ks < 768 && n_sb / (ks * 2) >= 4) ks *= 2;
+        // At most four parts: the matrix-core kernels run a cut of two or four as that many waves per row tile, but walk
+        // an eight-way cut inside the lane, one wave per row tile -- 128 waves for 2048 rows (2048 x 8192, 64 tokens:
+        // 38.9 us with eight parts, 13.9 with four; 16 tokens on 2560 x 10240 23.2 against 12.2).  A single token pays
+        // 0.3 to 0.4 us for it on those shapes (2048 x 8192: 3.88 -> 4.21 us).  CAMELID_HIP_Q4K_MAX_KSPLIT=8 restores eight.
+        const int most = env_int("CAMELID_HIP_Q4K_MAX_KSPLIT", 4) == 8 ? 8 : 4;
+        while (ks < most && tiles * ks < 768 && n_sb / (ks * 2) >= 4) ks *= 2;
     }
     s.ksplit = ks;
     int tpw = env_int("CAMELID_HIP_Q4K_TILES_PER_WG", 0);

@@ -575,21 +575,29 @@ def test_q4k_eight_wave_launch_under_the_k_cut_on_shorter_rows(rows, cols):
     acts[1, 3], acts[1, cols - 300] = np.nan, np.nan
     acts[2, 1::2] = -acts[2, ::2]
     band = w.slice(5, rows - 9)
+    # below 3072 rows the policy would cut long rows eight ways; it stops at four by default and the eight-way forms stay selectable
+    for most in ((4, 8) if rows < 3072 else (4,)):
+        with G.env(CAMELID_HIP_Q4K_MAX_KSPLIT=most):
+            _check_q4k_k_cut_forms(fmt, wire, w, band, acts, rows, cols, most)
+
+
+def _check_q4k_k_cut_forms(fmt, wire, w, band, acts, rows, cols, most):
+    served = r"^q4k\.dot\.wg8\.kcut\.fused(\.(short|uneven))?$"   # (rows of 14336 values cut four ways: the form of their own)
     for i, x in enumerate(acts):
-        G.say(f"Q4_K K-cut launch on shorter rows {rows}x{cols} act={i}")
-        with G.engaged(r"^q4k\.dot\.wg8\.kcut\.fused\.(short|uneven)$", none=(r"^q4k\.dot\.ring", r"^q4k\.dot\.buffers", r"^quantize\.")):
+        G.say(f"Q4_K K-cut launch on shorter rows {rows}x{cols} act={i} at most {most} parts")
+        with G.engaged(served, none=(r"^q4k\.dot\.ring", r"^q4k\.dot\.buffers", r"^quantize\.")):
             got = G.gpu_matmul_f32(w, x)
             got_band = G.gpu_matmul_f32(band, x)
-        with G.env(CAMELID_HIP_Q4K_KCUT_SHORT=0), G.engaged(r"^q4k\.dot\.", none=(r"^q4k\.dot\.wg8",)):
+        with G.env(CAMELID_HIP_Q4K_KCUT_SHORT=0, CAMELID_HIP_Q4K_CU=0), G.engaged(r"^q4k\.dot\.", none=(r"^q4k\.dot\.wg8",)):
             four_wave = G.gpu_matmul_f32(w, x)
-        assert G.same_bits(got, four_wave), (rows, cols, i)
-        assert G.same_bits(got_band, got[5:rows - 4]), (rows, cols, i)
+        assert G.same_bits(got, four_wave), (rows, cols, i, most)
+        assert G.same_bits(got_band, got[5:rows - 4]), (rows, cols, i, most)
         for width in (8, 12, 16):
-            with G.env(CAMELID_HIP_Q4K_KCUT_WAVES=width), G.engaged(r"^q4k\.dot\.wg8\.kcut\.fused\.(short|uneven)$"):
-                assert G.same_bits(G.gpu_matmul_f32(w, x), got), (rows, cols, i, width)
+            with G.env(CAMELID_HIP_Q4K_KCUT_WAVES=width), G.engaged(served):
+                assert G.same_bits(G.gpu_matmul_f32(w, x), got), (rows, cols, i, most, width)
         if i != 1:
             want = oracle.matmul(fmt, wire, cols, x[None, :], order=EXACT_ORDER[fmt], threads=16)[0]
-            assert G.max_rel(got, want) <= TOL, (rows, cols, i)
+            assert G.max_rel(got, want) <= TOL, (rows, cols, i, most)
 
 
 @pytest.mark.parametrize("rows,cols", [(4096, 4096), (4096, 14336), (11008, 4096), (4096, 11008), (5120, 5120), (2048, 8192),
