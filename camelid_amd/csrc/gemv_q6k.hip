@@ -359,21 +359,24 @@ __global__ __launch_bounds__(256) void gemv_q6k_kernel(Q6KArgs a) {
 // ANY: the row length is the launch's (n_sb super-blocks, staged in dynamic LDS), the parts are those of
 // gemv_q6k_kernel, [k n / KS, (k + 1) n / KS) -- unequal when KS does not divide n -- and NSTEPS is the longest part:
 // steps past a shorter part's end re-read its last super-block and add nothing.
-template <int KS, int NSTEPS, int NB = 4, int WAVES = 8, bool ANY = false>
+// NT = 2 (with ANY): two contiguous f32 rows in, out[2][rows]; every pass quantizes its super-blocks of both tokens and a
+// step's unpacked weight is replayed against them -- each cell the one-token launch's bits.
+template <int KS, int NSTEPS, int NB = 4, int WAVES = 8, bool ANY = false, int NT = 1>
 __global__ __launch_bounds__(WAVES * 64) void gemv_q6k_cu_kcut_kernel(Q6KArgs a) {
     constexpr int LPS = 8, RPW = kWave / LPS, TPW = WAVES / KS, PRE = 2;
     constexpr int PER_PASS = 2 * TPW;                       // super-blocks a pass gives every part
     constexpr int PASSES = (NSTEPS + PER_PASS - 1) / PER_PASS;
     static_assert(NSTEPS >= NB && WAVES % KS == 0, "K parts of at least one full ring");
+    static_assert(NT == 1 || (ANY && NT == 2), "two tokens: the general form");
     const int NSB = ANY ? a.n_sb : KS * NSTEPS;
     __shared__ __attribute__((aligned(16))) int8_t ys_fixed[ANY ? 16 : KS * NSTEPS * 256];
     __shared__ int bsum16_fixed[ANY ? 1 : KS * NSTEPS * 16];
     __shared__ float yds_fixed[ANY ? 1 : KS * NSTEPS];
-    __shared__ float part[WAVES * RPW];
+    __shared__ float part[WAVES * NT * RPW];
     extern __shared__ uint4 smem_q6k_any[];
     int8_t *ys = ANY ? reinterpret_cast<int8_t *>(smem_q6k_any) : ys_fixed;
-    int *bsum16 = ANY ? reinterpret_cast<int *>(ys + NSB * 256) : bsum16_fixed;
-    float *yds = ANY ? reinterpret_cast<float *>(bsum16 + NSB * 16) : yds_fixed;
+    int *bsum16 = ANY ? reinterpret_cast<int *>(ys + NT * NSB * 256) : bsum16_fixed;
+    float *yds = ANY ? reinterpret_cast<float *>(bsum16 + NT * NSB * 16) : yds_fixed;
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int tile_in_wg = wave / KS, kpart = wave - tile_in_wg * KS;
@@ -383,12 +386,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q6k_cu_kcut_kernel(Q6KArgs a)
     // the f32 activation: in pass p this wave's halves take super-blocks PER_PASS * p + 2 * tile_in_wg + {0, 1} of its part
     const int half = lane >> 5, ql32 = lane & 31;
     auto unit_of = [&](int p) __attribute__((always_inline)) -> int { return PER_PASS * p + 2 * tile_in_wg + half; };
-    float4 xv[PASSES][2];
+    float4 xv[PASSES][NT][2];
 #pragma unroll
     for (int p = 0; p < PASSES; p++) {
-        const float4 *x4 = reinterpret_cast<const float4 *>(a.x) + min(s0 + unit_of(p), s1 - 1) * 64 + ql32 * 2;
-        xv[p][0] = x4[0];
-        xv[p][1] = x4[1];
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            const float4 *x4 = reinterpret_cast<const float4 *>(a.x) + (t * NSB + min(s0 + unit_of(p), s1 - 1)) * 64 + ql32 * 2;
+            xv[p][t][0] = x4[0];
+            xv[p][t][1] = x4[1];
+        }
     }
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_barrier();  // execution only: every activation request of the workgroup is out
@@ -414,25 +420,30 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q6k_cu_kcut_kernel(Q6KArgs a)
     // and stores nothing): the f32 loads above are used unconditionally and stay ahead of the weight requests
     auto quantize_pass = [&](int p) __attribute__((always_inline)) {
         const int u = unit_of(p);
-        float dv;
-        int bs;
-        const uint2 packed = q8k_quantize_row32(xv[p], lane, dv, bs);
-        int s16 = sdot4(packed.y, 0x01010101u, sdot4(packed.x, 0x01010101u, 0));
-        s16 += row_shr_i32<1>(s16);  // odd lanes: the sum of 16 consecutive quants
-        if (s0 + u < s1) {
-            const int sbk = s0 + u;
-            reinterpret_cast<uint2 *>(ys)[sbk * 32 + ql32] = packed;
-            if (ql32 & 1) bsum16[sbk * 16 + (ql32 >> 1)] = s16;
-            if (ql32 == 0) yds[sbk] = dv;
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            float dv;
+            int bs;
+            const uint2 packed = q8k_quantize_row32(xv[p][t], lane, dv, bs);
+            int s16 = sdot4(packed.y, 0x01010101u, sdot4(packed.x, 0x01010101u, 0));
+            s16 += row_shr_i32<1>(s16);  // odd lanes: the sum of 16 consecutive quants
+            if (s0 + u < s1) {
+                const int sbk = t * NSB + s0 + u;
+                reinterpret_cast<uint2 *>(ys)[sbk * 32 + ql32] = packed;
+                if (ql32 & 1) bsum16[sbk * 16 + (ql32 >> 1)] = s16;
+                if (ql32 == 0) yds[sbk] = dv;
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
-        __builtin_amdgcn_sched_barrier(0);
     };
     quantize_pass(0);
     __syncthreads();
 
-    float acc[1] = {0.0f};
+    float acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++) acc[t] = 0.0f;
     auto compute = [&](const Q6KRegs<1> &b, int step) __attribute__((always_inline)) {
-        q6k_compute<1, false, 1>(b, l, s0 + step, s1, ys, bsum16, yds, NSB, acc, nullptr);
+        q6k_compute<NT, false, 1>(b, l, s0 + step, s1, ys, bsum16, yds, NSB, acc, nullptr);
         __builtin_amdgcn_sched_barrier(0);
     };
 #pragma unroll
@@ -446,17 +457,20 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q6k_cu_kcut_kernel(Q6KArgs a)
         compute(ring[i % NB], i);
         if (i + NB < NSTEPS) request(ring[i % NB], i + NB);
     }
-    if (l == LPS - 1) part[wave * RPW + r] = acc[0];
+    if (l == LPS - 1) {
+#pragma unroll
+        for (int t = 0; t < NT; t++) part[(wave * NT + t) * RPW + r] = acc[t];
+    }
     __syncthreads();
-    if (tid < TPW * RPW) {
-        const int tw = tid / RPW, rr = tid - tw * RPW;
+    if (tid < TPW * NT * RPW) {
+        const int rr = tid % RPW, t = (tid / RPW) % NT, tw = tid / (RPW * NT);
         const int orow = (blockIdx.x * TPW + tw) * RPW + rr;
         if (orow < a.rows) {
-            float v = part[(tw * KS) * RPW + rr];
+            float v = part[((tw * KS) * NT + t) * RPW + rr];
 #pragma unroll
-            for (int k = 1; k < KS; k++) v = v + part[(tw * KS + k) * RPW + rr];
-            if (a.residual) v = v + a.residual[orow];
-            a.out[orow] = v;
+            for (int k = 1; k < KS; k++) v = v + part[((tw * KS + k) * NT + t) * RPW + rr];
+            if (NT == 1 && a.residual) v = v + a.residual[orow];
+            a.out[static_cast<int64_t>(t) * a.rows + orow] = v;
         }
     }
 }
@@ -717,6 +731,44 @@ int launch_gemv_q6k_f32(const cml_weight *w, const float *x, float *out, hipStre
         CML_COUNT_LAUNCH("q6k.dot.wg8.kcut.fused");
         CML_HIP_TRY(hipGetLastError());
         return CML_OK;
+    }
+    if (const int two_steps = (n_tokens == 2 && env_int("CAMELID_HIP_Q6K_KCUT_TOKENS", 1)) ? q6k_cu_kcut_any_steps(ka.rows, ka.n_sb) : 0) {
+        // two tokens on the general K-cut form (4096 x 4096: 6.65 us before on the four-wave launch that quantizes both rows in every workgroup)
+        const int ks = ka.ksplit;
+        int waves = 8;
+        while (waves < 12 && (tiles + waves / ks - 1) / (waves / ks) > 256) waves += ks == 1 ? 2 : 4;
+        const int tpw = waves / ks;
+        const dim3 grid(static_cast<unsigned>((tiles + tpw - 1) / tpw)), block(64 * waves);
+        const size_t lds_two = 2 * static_cast<size_t>(ka.n_sb) * (256 + 64 + 4);
+        bool launched = lds_two <= 64 * 1024;
+        if (launched) {
+#define CML_Q6K_KCUT_TWO(KS_, NS_, W2_)                                                                                              \
+    case KS_ * 100 + NS_:                                                                                                            \
+        if (waves == 8) hipLaunchKernelGGL((gemv_q6k_cu_kcut_kernel<KS_, NS_, 4, 8, true, 2>), grid, block, lds_two, st, ka);         \
+        else if (waves == W2_) hipLaunchKernelGGL((gemv_q6k_cu_kcut_kernel<KS_, NS_, 4, W2_, true, 2>), grid, block, lds_two, st, ka); \
+        else launched = false;                                                                                                       \
+        break;
+            switch (ks * 100 + two_steps) {
+                CML_Q6K_KCUT_TWO(4, 4, 12)
+                CML_Q6K_KCUT_TWO(4, 5, 12)
+                CML_Q6K_KCUT_TWO(4, 8, 12)
+                CML_Q6K_KCUT_TWO(4, 11, 12)
+                CML_Q6K_KCUT_TWO(4, 14, 12)
+                CML_Q6K_KCUT_TWO(2, 4, 12)
+                CML_Q6K_KCUT_TWO(2, 6, 12)
+                CML_Q6K_KCUT_TWO(2, 8, 12)
+                CML_Q6K_KCUT_TWO(2, 10, 12)
+                CML_Q6K_KCUT_TWO(1, 14, 10)
+                CML_Q6K_KCUT_TWO(1, 16, 10)
+                default: launched = false; break;
+            }
+#undef CML_Q6K_KCUT_TWO
+        }
+        if (launched) {
+            CML_COUNT_LAUNCH("q6k.dot.wg8.kcut.fused.two");
+            CML_HIP_TRY(hipGetLastError());
+            return CML_OK;
+        }
     }
     if (const int any_steps = n_tokens == 1 ? q6k_cu_kcut_any_steps(ka.rows, ka.n_sb) : 0) {
         // the general K-cut form: eight waves, or twelve where eight would need more than one workgroup per compute unit

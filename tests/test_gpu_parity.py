@@ -718,6 +718,33 @@ def test_q6k_eight_wave_launch_under_the_k_cut_on_other_rows(rows, cols):
             assert G.max_rel(got, want) <= TOL, (rows, cols, i)
 
 
+@pytest.mark.parametrize("rows,cols", [(4096, 4096), (5003, 5120), (3080, 8192), (8192, 2048), (6200, 3072), (11008, 4096), (9216, 5120),
+                                       (14336, 4096), (18944, 3584)])
+def test_q6k_k_cut_launch_replays_two_tokens(rows, cols):
+    """Two tokens on the Q6_K one-workgroup-per-unit launch (rows of up to 8192 values): each step's unpacked weight
+    replayed against both staged rows.  Every cell is the single-token call's bits, also on a row band; the counters
+    show the launch, and with it switched off (CAMELID_HIP_Q6K_KCUT_TOKENS=0) the four-wave launch gives the same bits."""
+    fmt = oracle.Q6_K
+    rng = np.random.default_rng(10300 + rows + cols)
+    wire = G.synth_weight(fmt, rows, cols, seed=10400 + rows + cols)
+    w = Weight.upload(fmt, rows, cols, wire)
+    x = rng.standard_normal((2, cols)).astype(np.float32)
+    x[0, :256] = 0.0
+    x[1, 1::2] = -x[1, ::2]
+    x[1, 300] = np.nan
+    singles = np.stack([G.gpu_matmul_f32(w, x[t]) for t in range(2)])
+    band = w.slice(8, rows - 16)   # (Q6_K views start on a row of the 8-row tiles or anywhere: the planes are row-major)
+    G.say(f"Q6_K K-cut launch {rows}x{cols}, two tokens")
+    with G.engaged(r"^q6k\.dot\.wg8\.kcut\.fused\.two$", none=(r"^q6k\.dot\.buffers", r"^q6k\.mfma", r"^quantize\.")):
+        got = np.asarray(G.gpu_matmul_f32(w, x)).reshape(2, rows)
+        got_band = np.asarray(G.gpu_matmul_f32(band, x)).reshape(2, rows - 16)
+    assert G.same_bits(got, singles), (rows, cols)
+    assert G.same_bits(got_band, got[:, 8:rows - 8]), (rows, cols, "band")
+    with G.env(CAMELID_HIP_Q6K_KCUT_TOKENS=0), G.engaged(none=(r"^q6k\.dot\.wg8\.kcut\.fused\.two$",)):
+        former = np.asarray(G.gpu_matmul_f32(w, x)).reshape(2, rows)
+    assert G.same_bits(former, got), (rows, cols, "former path")
+
+
 @pytest.mark.parametrize("rows,cols", [(190, 3072), (64, 256), (333, 4096), (40, 14336), (77, 1280)])
 def test_q4k_fused_two_tokens_is_the_two_step_path(rows, cols):
     """Two-token cml_matmul_f32 on Q4_K quantizes both rows inside the matvec kernel: the bits of
