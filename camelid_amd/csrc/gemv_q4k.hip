@@ -1452,8 +1452,14 @@ static bool q4k_cu_serves(const Q4KArgs &ka, int ksplit, int n_tokens = 1) {
 // Most tokens the eight-wave launch replays per step (CAMELID_HIP_Q4K_CU_TOKENS, 1 to 4; four only on rows of 4096 values).
 // Measured at 14336 x 4096, us per step against what served the call before: 2 tokens 7.0 (8.46, the 16-row-wave ring launch),
 // 3 tokens 8.6 (9.71, the matrix-core launch with the quantizer inside), 4 tokens 10.4 (10.3: the vector work no longer hides
-// behind the stream).  Default 3.
-static int q4k_cu_max_tokens(int n_sb) { return std::min(n_sb == 16 ? 4 : 3, std::max(1, env_int("CAMELID_HIP_Q4K_CU_TOKENS", 3))); }
+// behind the stream).  Default 3; 4 on rows of 3584 or 4096 values from 24576 rows on, where the matrix-core launch streams
+// less well than this one (4 tokens on 128256 x 4096: 66.8 us against 75.2, 65536 x 4096 35.7 against 39.9, 32000 x 4096
+// 19.3 against 20.7).
+static int q4k_cu_max_tokens(int n_sb, int rows) {
+    const int knob = env_int("CAMELID_HIP_Q4K_CU_TOKENS", 0);
+    const int most = knob >= 1 ? knob : (rows >= 24576 ? 4 : 3);
+    return std::min((n_sb == 16 || n_sb == 14) ? 4 : 3, most);
+}
 
 static int launch_q4k_cu(const Q4KArgs &ka, int ablate, hipStream_t st, int n_tokens = 1) {
     if (!(ablate & 1) && !ka.x) return fail(CML_ERR_INVALID, "null activation");  // every variant but the one without the activation reads it
@@ -1505,8 +1511,9 @@ static int launch_q4k_cu(const Q4KArgs &ka, int ablate, hipStream_t st, int n_to
             case 2: CML_Q4K_CU_STEPS(2); break;
             case 3: CML_Q4K_CU_STEPS(3); break;
             case 4:
-                if (ka.n_sb != 16) return fail(CML_ERR_INVALID, "four tokens: rows of 16 super-blocks only");
-                hipLaunchKernelGGL((gemv_q4k_cu_kernel<8, 0, 4>), grid, block, 0, st, ca);
+                if (ka.n_sb == 16) hipLaunchKernelGGL((gemv_q4k_cu_kernel<8, 0, 4>), grid, block, 0, st, ca);
+                else if (ka.n_sb == 14) hipLaunchKernelGGL((gemv_q4k_cu_kernel<7, 0, 4>), grid, block, 0, st, ca);
+                else return fail(CML_ERR_INVALID, "four tokens: rows of 14 or 16 super-blocks only");
                 break;
             default: return fail(CML_ERR_INVALID, "the eight-wave launch takes up to four tokens");
         }
@@ -1812,7 +1819,7 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
             else if (half_tiles) { if (whole) CML_Q4K_LOADS(2, true); else CML_Q4K_LOADS(2, false); CML_COUNT_LAUNCH("q4k.calibrate.buffers"); }
             else { if (whole) CML_Q4K_LOADS(1, true); else CML_Q4K_LOADS(1, false); CML_COUNT_LAUNCH("q4k.calibrate.buffers"); }
 #undef CML_Q4K_LOADS
-        } else if (plain && a.n_tokens >= 2 && a.n_tokens <= q4k_cu_max_tokens(ka.n_sb) &&
+        } else if (plain && a.n_tokens >= 2 && a.n_tokens <= q4k_cu_max_tokens(ka.n_sb, ka.rows) &&
                    (a.n_tokens >= 3 || q4k_rows_per_wave(tiles16, shape.ksplit, 1) == 8) &&  // three tokens: at any row count (128256 x 4096: 55.0 us against 66.7)
                    q4k_ring(ka, shape.ksplit) && q4k_cu_serves(ka, shape.ksplit, static_cast<int>(a.n_tokens))) {
             if (int rc = launch_q4k_cu(ka, 0, st, static_cast<int>(a.n_tokens))) return rc;  // a few tokens replayed against each step's weight

@@ -471,7 +471,8 @@ def test_q4k_eight_wave_launch_serves_rows_of_six_to_sixteen_super_blocks(rows, 
     (24570, 4096, (1, 2, 3), "wide"),     # twelve, the last 16-row tile partly filled
     (17920, 5120, (1, 2, 3), "wide"),     # ten, two quantizer passes
     (28672, 4096, (3,), "wide"),          # sixteen: three tokens only
-    (40000, 4096, (3,), "eight"),         # three tokens beyond one workgroup per compute unit: eight waves
+    (40000, 4096, (3, 4), "eight"),       # three and (from 24576 rows on) four tokens beyond one workgroup per compute unit: eight waves
+    (24600, 3584, (4,), "eight"),
 ])
 def test_q4k_wide_workgroups_beyond_one_eight_wave_workgroup_per_unit(rows, cols, tokens, kernel):
     """More than 16384 rows of 14 or 16 super-blocks: the one-workgroup-per-compute-unit launch with ten, twelve or
@@ -481,7 +482,7 @@ def test_q4k_wide_workgroups_beyond_one_eight_wave_workgroup_per_unit(rows, cols
     rng = np.random.default_rng(8800 + rows)
     wire = G.synth_weight(fmt, rows, cols, seed=8900 + rows)
     w = Weight.upload(fmt, rows, cols, wire)
-    x = rng.standard_normal((3, cols)).astype(np.float32)
+    x = rng.standard_normal((4, cols)).astype(np.float32)
     x[1, :256] = 0.0
     x[2, 5], x[2, cols - 3] = 7.0, -7.0
     want = oracle.matmul(fmt, wire, cols, x, order=EXACT_ORDER[fmt], threads=16)
