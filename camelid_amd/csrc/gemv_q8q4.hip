@@ -480,6 +480,7 @@ static int b32_lanes(int fmt, int64_t rows, int64_t nb) {
     if (p == 16 && env_int("CAMELID_HIP_B32_WIDE_ROWS", 1)) {
         const int64_t waves16 = (rows + 3) / 4;
         if (waves16 <= 512 && nb >= 128) p = 64;
+        else if (fmt == CML_Q8_0 && nb == 128 && rows > 3584 && rows <= 4096) p = 64;  // Q8_0 4096 x 4096: 6.26 -> 5.66 us (3200 x 4096, 4096 x 5120 ... 8192 lose with 64)
         else if (waves16 <= 1024 && nb >= 64) p = 32;
     }
     return p;
