@@ -621,10 +621,14 @@ static int launch_b32_f32_p(const cml_weight *w, const float *x, float *out, hip
     const unsigned gx = static_cast<unsigned>((ba.rows + rows_per_wg - 1) / rows_per_wg);
     // float4 of the activation per thread: 1, 2 or 4 in registers; longer rows (or the knob) take the staged path
     const int n4 = (two ? 2 : 1) * ba.nb * 8, threads = waves * 64;
-    int nxq = !ba.early_loads ? 0 : n4 <= threads ? 1 : n4 <= 2 * threads ? 2 : n4 <= 4 * threads ? 4 : 0;
-    if (waves == 8 && nxq == 4 && !two) nxq = 0;  // 2048 float4 would be 256 blocks; eight waves are launched for at most 128
-    if (waves == 16 && nxq != 1) nxq = 0;
-    if (waves == 2 && nxq != 0) nxq = 4;  // one register variant for the short workgroup
+    int nxq = !ba.early_loads ? 0 : n4 <= threads ? 1 : n4 <= 2 * threads ? 2 : n4 <= 4 * threads ? 4 : n4 <= 8 * threads ? 8 : 0;
+    // (the token held in registers -- its requests out ahead of the first weight requests -- instead of staged through a loop
+    // that the weight requests wait behind: Q8_0 2048 x 8192 7.14 -> 6.29 us, 4096 x 8192 9.86 -> 8.58; Q4_0 8192 x 8192 11.2 -> 9.8)
+    const int nxq_most = env_int("CAMELID_HIP_B32_NXQ_MOST", 8);
+    if (nxq > nxq_most) nxq = 0;
+    if (two && nxq == 8) nxq = 0;
+    if (waves == 16 && nxq > 2) nxq = 0;
+    if (waves == 2) nxq = (nxq >= 1 && nxq <= 4) ? 4 : 0;  // one register variant for the short workgroup
     if (w2) {
         // one token, two weights (grid.z = 2): the 16-lane, eight-wave launches with the token in registers; -1 = not served
         if constexpr (P == 16) {
@@ -651,6 +655,8 @@ static int launch_b32_f32_p(const cml_weight *w, const float *x, float *out, hip
         if (deep) hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, true, 8, 0, 4>), dim3(gx, 1), dim3(512), lds, st, ba);
         else if (nxq == 1) CML_B32_FUSED(8, 1);
         else if (nxq == 2) CML_B32_FUSED(8, 2);
+        else if (nxq == 4) CML_B32_FUSED(8, 4);
+        else if (nxq == 8) CML_B32_FUSED(8, 8);
         else CML_B32_FUSED(8, 0);
     } else
     if (two) {
@@ -673,6 +679,7 @@ static int launch_b32_f32_p(const cml_weight *w, const float *x, float *out, hip
         else hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, true, 4, 0, 4>), dim3(gx, 1), dim3(256), lds, st, ba);
     } else if (waves == 16) {
         if (nxq == 1) CML_B32_FUSED(16, 1);
+        else if (nxq == 2) CML_B32_FUSED(16, 2);
         else CML_B32_FUSED(16, 0);
     } else if (waves == 2) {
         if (nxq == 4) CML_B32_FUSED(2, 4);
@@ -686,11 +693,14 @@ static int launch_b32_f32_p(const cml_weight *w, const float *x, float *out, hip
         else if (ring && nxq == 2) hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, true, 8, 2, 2, 3>), dim3(gx, 1), dim3(512), lds, st, ba);
         else if (nxq == 1) CML_B32_FUSED(8, 1);
         else if (nxq == 2) CML_B32_FUSED(8, 2);
+        else if (nxq == 4) CML_B32_FUSED(8, 4);
+        else if (nxq == 8) CML_B32_FUSED(8, 8);
         else CML_B32_FUSED(8, 0);
     } else {
         if (nxq == 1) CML_B32_FUSED(4, 1);
         else if (nxq == 2) CML_B32_FUSED(4, 2);
         else if (nxq == 4) CML_B32_FUSED(4, 4);
+        else if (nxq == 8) CML_B32_FUSED(4, 8);
         else CML_B32_FUSED(4, 0);
     }
 #undef CML_B32_FUSED

@@ -922,11 +922,17 @@ def test_b32_fused_launch_shapes_on_rows_longer_than_4096_values(name, fmt, rows
         assert G.same_bits(G.gpu_matmul_f32(w, x), want), (name, rows, cols, "two launches")
     with G.env(CAMELID_HIP_B32_LONG_ROW_WAVES=0), G.engaged(rf"^{fam}\.dot\.p16\.w8\.(deep\.)?fused$"):
         assert G.same_bits(G.gpu_matmul_f32(w, x), want), (name, rows, cols, "eight waves")
+    for most in (1, 2, 4, 8):   # how many float4 of the token a thread may hold in registers (beyond: staged through a loop)
+        G.say(f"{name} {rows}x{cols}: at most {most} float4 of the token per thread")
+        with G.env(CAMELID_HIP_B32_NXQ_MOST=most), G.engaged(rf"^{fam}\.dot\.p16\."):
+            assert G.same_bits(G.gpu_matmul_f32(w, x), want), (name, rows, cols, "registers", most)
     for waves in (4, 8, 16):
         for depth in (2, 4):
             G.say(f"{name} {rows}x{cols}: waves={waves} depth={depth}")
-            with G.env(CAMELID_HIP_B32_FUSED_WAVES=waves, CAMELID_HIP_B32_DEPTH=depth), G.engaged(rf"^{fam}\.dot\.p16\.w{waves}\."):
-                assert G.same_bits(G.gpu_matmul_f32(w, x), want), (name, rows, cols, waves, depth)
+            for most in (8, 1):
+                with G.env(CAMELID_HIP_B32_FUSED_WAVES=waves, CAMELID_HIP_B32_DEPTH=depth, CAMELID_HIP_B32_NXQ_MOST=most), \
+                        G.engaged(rf"^{fam}\.dot\.p16\.w{waves}\."):
+                    assert G.same_bits(G.gpu_matmul_f32(w, x), want), (name, rows, cols, waves, depth, most)
 
 
 @pytest.mark.parametrize("name,fmt", [("Q8_0", oracle.Q8_0), ("Q4_0", oracle.Q4_0)])
