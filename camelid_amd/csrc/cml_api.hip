@@ -900,7 +900,7 @@ int cml_matmul_f32(const cml_weight *w, const float *x_dev, int64_t n_tokens, fl
         return frc;
     }
     if ((w->fmt == CML_Q8_0 || w->fmt == CML_Q4_0) && (n_tokens == 1 || fuse_two) &&
-        (fuse == 2 || (fuse == 1 && w->cols <= 8192 && (n_tokens == 1 || w->rows <= 32768)))) {
+        (fuse == 2 || (fuse == 1 && (w->cols <= 8192 || (n_tokens == 1 && gemv_b32_long_rows_fuse(w))) && (n_tokens == 1 || w->rows <= 32768)))) {
         // the same for the 32-value block formats (8192x2048: 7.6 -> 5.9 us per step).  One token: on every row
         // count -- with eight- and sixteen-wave workgroups the quantizer hides on a vocabulary head too (128256 x 3072:
         // Q8_0 62.3 -> 59.7 us, Q4_0 35.7 -> 34.4; 151936 x 3584 Q8_0 83.5 -> 81.4).  Two tokens: up to 32768 rows

@@ -146,7 +146,8 @@ int launch_gemv_q4k(const MatArgs &a, hipStream_t st);
 // quantize + matvec for two stacked expert weights of one shape in one launch; a.q / a.scales unused, x = f32 rows
 int launch_gemv_q4k_f32_grouped_pair(const MatArgs &a, const cml_weight *w2, float *out2, const float *x, hipStream_t st);
 int launch_gemv_q4k_f32_pair(const cml_weight *w, const cml_weight *w2, const float *x, float *out, float *out2, hipStream_t st);
-bool gemv_q6k_long_rows_fuse(const cml_weight *w);  // the same for Q6_K
+bool gemv_q6k_long_rows_fuse(const cml_weight *w);
+bool gemv_b32_long_rows_fuse(const cml_weight *w);  // the same for Q8_0 / Q4_0 rows of more than 8192 values  // the same for Q6_K
 bool gemv_q4k_long_rows_fuse(const cml_weight *w, int n_tokens = 1);  // a single f32 token on this weight is one launch although its rows exceed 8192 values
 int launch_gemv_q4k_f32_multi(const cml_weight *const *ws, int n, const float *x, float *const *outs, hipStream_t st);  // -1: not served
 // whether that launch, as a direct call on these two weights, can route the token itself (a.route_logits)

@@ -568,6 +568,66 @@ static int launch_b32_p(const MatArgs &a, hipStream_t st) {
     return CML_OK;
 }
 
+// Workgroup width of the fused (f32 token in) launch, how many float4 of the token a thread holds in registers
+// (0 = the token is staged through a loop) and whether the two-step buffers are kept where the depth rule would take four.
+struct B32FusedShape {
+    int waves, nxq;
+    bool shallow;
+};
+static B32FusedShape b32_fused_shape(int fmt, int P, int rows, int nb, bool two, bool pair, bool early_loads) {
+    // Every workgroup quantizes the whole activation for itself; with eight waves twice the rows
+    // share that prologue.  Worth it while the matrix still gives every compute unit a workgroup.
+    int waves = env_int("CAMELID_HIP_B32_FUSED_WAVES", 0);
+    if (waves != 2 && waves != 4 && waves != 8 && waves != 16) {
+        waves = (rows >= 128 * 8 * (64 / P)) ? 8 : 4;
+        // Q8_0 rows of 4096 values (the longest the register prologue takes) on tall matrices: sixteen
+        // waves (16384 x 4096: 14.2 -> 12.7 us, 32000 x 4096: 24.7 -> 22.3); slower for Q4_0 and shorter rows
+        if (fmt == CML_Q8_0 && nb == 128 && rows >= 224 * 16 * (64 / P)) waves = 16;
+        // Q4_0 on a vocabulary-sized matrix: sixteen waves halve the number of workgroups that each quantize the
+        // token (128256 x 3072: 34.1 -> 33.3 us; Q8_0 there is the same 59.2 us with 4, 8 or 16)
+        if (fmt == CML_Q4_0 && nb <= 128 && rows >= 65536) waves = 16;
+    }
+    // Rows of more than 4096 values (the token is staged through LDS by every workgroup), one token, 16 lanes per row:
+    // sixteen waves once eight-wave workgroups would outnumber the compute units (Q8_0 14336 x 8192: 30.0 -> 23.3 us,
+    // 28672 x 8192 52.4 -> 42.2, 10240 x 8192 25.6 -> 18.4; Q4_0 14336 x 8192 15.9 -> 14.5, 9216 x 5120 9.23 -> 8.49);
+    // Q8_0 rows of 8192 values on up to 8192 rows: four waves and two-step buffers (8192 x 8192: 19.3 -> 16.2 us,
+    // 6144 x 8192 15.6 -> 13.5; shorter rows and Q4_0 keep eight: 8192 x 6144 11.1 against 11.9, Q4_0 8192 x 8192 10.95 against 12.6)
+    bool shallow = false;
+    if (P == 16 && !two && !pair && nb > 128 && !env_int("CAMELID_HIP_B32_FUSED_WAVES", 0) && env_int("CAMELID_HIP_B32_LONG_ROW_WAVES", 1)) {
+        if (rows > 256 * 8 * (64 / P)) {
+            if (fmt == CML_Q4_0 || nb >= 256 || rows < 16384) waves = 16;  // (Q8_0 16384 x 6144 and 32000 x 5120: 1 % slower with sixteen)
+        } else if (fmt == CML_Q8_0 && nb >= 256) {
+            waves = 4, shallow = true;
+        }
+    }
+    if (two && waves != 4) waves = 8;  // the two-token variants: four or eight waves
+    if (P > 16) waves = 8;
+    // float4 of the activation per thread: 1, 2 or 4 in registers; longer rows (or the knob) take the staged path
+    const int n4 = (two ? 2 : 1) * nb * 8, threads = waves * 64;
+    int nxq = !early_loads ? 0 : n4 <= threads ? 1 : n4 <= 2 * threads ? 2 : n4 <= 4 * threads ? 4 : n4 <= 8 * threads ? 8 : 0;
+    // (the token held in registers -- its requests out ahead of the first weight requests -- instead of staged through a loop
+    // that the weight requests wait behind: Q8_0 2048 x 8192 7.14 -> 6.29 us, 4096 x 8192 9.86 -> 8.58; Q4_0 8192 x 8192 11.2 -> 9.8)
+    const int nxq_most = env_int("CAMELID_HIP_B32_NXQ_MOST", 8);
+    if (nxq > nxq_most) nxq = 0;
+    if (two && nxq == 8) nxq = 0;
+    if (waves == 16 && nxq > 2) nxq = 0;
+    if (waves == 2) nxq = (nxq >= 1 && nxq <= 4) ? 4 : 0;  // one register variant for the short workgroup
+    return B32FusedShape{waves, nxq, shallow};
+}
+
+// A single f32 token on this weight runs as ONE launch although its rows are longer than 8192 values: where the
+// launch holds the token in registers (rows of up to 16384 values on eight-wave workgroups).  Against a quantizing
+// launch followed by the matvec: Q8_0 4096 x 14336 13.5 us against 14.65, 4096 x 11008 12.96 against 14.92, 2048 x 11008
+// 8.67 against 10.09; Q4_0 8192 x 14336 14.66 against 17.0, 5120 x 13824 13.0 against 14.4, 4096 x 14336 10.57 against 11.09.
+// Where the token would be staged through a loop the two launches are as fast or faster (Q8_0 8192 x 14336 24.8 against 23.9,
+// 8192 x 28672 47.9 against 44.4).
+bool gemv_b32_long_rows_fuse(const cml_weight *w) {
+    if ((w->fmt != CML_Q8_0 && w->fmt != CML_Q4_0) || w->rows <= 0 || !env_int("CAMELID_HIP_B32_LONG_ROWS_FUSE", 1)) return false;
+    if (static_cast<size_t>(w->nb) * (32 + 4 + 4) > 64 * 1024) return false;
+    const int p = b32_lanes(w->fmt, w->rows, w->nb);
+    return b32_fused_shape(w->fmt, p, static_cast<int>(w->rows), static_cast<int>(w->nb), false, false, env_int("CAMELID_HIP_B32_EARLY_LOADS", 1) != 0).nxq > 0;
+}
+
 // Single token, f32 activation in: quantize + matvec in one launch.
 template <int FMT, int P>
 static int launch_b32_f32_p(const cml_weight *w, const float *x, float *out, hipStream_t st, int n_tokens, const cml_weight *w2 = nullptr,
@@ -590,45 +650,11 @@ static int launch_b32_f32_p(const cml_weight *w, const float *x, float *out, hip
     const bool two = n_tokens == 2;
     const size_t lds = static_cast<size_t>(two ? 2 : 1) * ba.nb * (32 + 4 + 4);
     if (lds > 64 * 1024) return fail(CML_ERR_UNSUPPORTED, "activation of %d blocks exceeds the LDS staging limit", ba.nb);
-    // Every workgroup quantizes the whole activation for itself; with eight waves twice the rows
-    // share that prologue.  Worth it while the matrix still gives every compute unit a workgroup.
-    int waves = env_int("CAMELID_HIP_B32_FUSED_WAVES", 0);
-    if (waves != 2 && waves != 4 && waves != 8 && waves != 16) {
-        waves = (ba.rows >= 128 * 8 * (64 / P)) ? 8 : 4;
-        // Q8_0 rows of 4096 values (the longest the register prologue takes) on tall matrices: sixteen
-        // waves (16384 x 4096: 14.2 -> 12.7 us, 32000 x 4096: 24.7 -> 22.3); slower for Q4_0 and shorter rows
-        if (FMT == CML_Q8_0 && ba.nb == 128 && ba.rows >= 224 * 16 * (64 / P)) waves = 16;
-        // Q4_0 on a vocabulary-sized matrix: sixteen waves halve the number of workgroups that each quantize the
-        // token (128256 x 3072: 34.1 -> 33.3 us; Q8_0 there is the same 59.2 us with 4, 8 or 16)
-        if (FMT == CML_Q4_0 && ba.nb <= 128 && ba.rows >= 65536) waves = 16;
-    }
-    // Rows of more than 4096 values (the token is staged through LDS by every workgroup), one token, 16 lanes per row:
-    // sixteen waves once eight-wave workgroups would outnumber the compute units (Q8_0 14336 x 8192: 30.0 -> 23.3 us,
-    // 28672 x 8192 52.4 -> 42.2, 10240 x 8192 25.6 -> 18.4; Q4_0 14336 x 8192 15.9 -> 14.5, 9216 x 5120 9.23 -> 8.49);
-    // Q8_0 rows of 8192 values on up to 8192 rows: four waves and two-step buffers (8192 x 8192: 19.3 -> 16.2 us,
-    // 6144 x 8192 15.6 -> 13.5; shorter rows and Q4_0 keep eight: 8192 x 6144 11.1 against 11.9, Q4_0 8192 x 8192 10.95 against 12.6)
-    bool shallow = false;
-    if (P == 16 && !two && !w2 && ba.nb > 128 && !env_int("CAMELID_HIP_B32_FUSED_WAVES", 0) && env_int("CAMELID_HIP_B32_LONG_ROW_WAVES", 1)) {
-        if (ba.rows > 256 * 8 * (64 / P)) {
-            if (FMT == CML_Q4_0 || ba.nb >= 256 || ba.rows < 16384) waves = 16;  // (Q8_0 16384 x 6144 and 32000 x 5120: 1 % slower with sixteen)
-        } else if (FMT == CML_Q8_0 && ba.nb >= 256) {
-            waves = 4, shallow = true;
-        }
-    }
-    if (two && waves != 4) waves = 8;  // the two-token variants: four or eight waves
-    if (P > 16) waves = 8;
+    const B32FusedShape fs = b32_fused_shape(FMT, P, ba.rows, ba.nb, two, w2 != nullptr, ba.early_loads != 0);
+    const int waves = fs.waves, nxq = fs.nxq;
+    const bool shallow = fs.shallow;
     const int rows_per_wg = waves * (64 / P);
     const unsigned gx = static_cast<unsigned>((ba.rows + rows_per_wg - 1) / rows_per_wg);
-    // float4 of the activation per thread: 1, 2 or 4 in registers; longer rows (or the knob) take the staged path
-    const int n4 = (two ? 2 : 1) * ba.nb * 8, threads = waves * 64;
-    int nxq = !ba.early_loads ? 0 : n4 <= threads ? 1 : n4 <= 2 * threads ? 2 : n4 <= 4 * threads ? 4 : n4 <= 8 * threads ? 8 : 0;
-    // (the token held in registers -- its requests out ahead of the first weight requests -- instead of staged through a loop
-    // that the weight requests wait behind: Q8_0 2048 x 8192 7.14 -> 6.29 us, 4096 x 8192 9.86 -> 8.58; Q4_0 8192 x 8192 11.2 -> 9.8)
-    const int nxq_most = env_int("CAMELID_HIP_B32_NXQ_MOST", 8);
-    if (nxq > nxq_most) nxq = 0;
-    if (two && nxq == 8) nxq = 0;
-    if (waves == 16 && nxq > 2) nxq = 0;
-    if (waves == 2) nxq = (nxq >= 1 && nxq <= 4) ? 4 : 0;  // one register variant for the short workgroup
     if (w2) {
         // one token, two weights (grid.z = 2): the 16-lane, eight-wave launches with the token in registers; -1 = not served
         if constexpr (P == 16) {

@@ -894,6 +894,36 @@ def test_q4k_loads_only_twin_runs_for_every_single_token_launch_shape(rows, cols
 
 
 @pytest.mark.parametrize("name,fmt", [("Q8_0", oracle.Q8_0), ("Q4_0", oracle.Q4_0)])
+@pytest.mark.parametrize("rows,cols", [(4096, 14336), (2050, 11008), (8192, 14336), (5120, 13824), (3000, 16384)])
+def test_b32_rows_longer_than_8192_values_run_as_one_launch_where_the_token_fits_registers(name, fmt, rows, cols):
+    """Single-token cml_matmul_f32 on Q8_0 / Q4_0 rows of 8193 to 16384 values: one launch (the quantizer inside, the
+    token in registers) wherever the launch shape holds the token in registers, else a quantizing launch and the
+    matvec -- the counters show which; both give the oracle's bits."""
+    rng = np.random.default_rng(10500 + rows + fmt)
+    wire = G.synth_weight(fmt, rows, cols, seed=10600 + rows + fmt)
+    w = Weight.upload(fmt, rows, cols, wire)
+    x = rng.standard_normal(cols).astype(np.float32)
+    x[:64] = 0.0
+    x[64:70] = [2.5, 0.5, -0.5, -2.5, 1.5, -1.5]
+    x[-32:] = 3.0
+    want = oracle.matmul(fmt, wire, cols, x[None, :], order=EXACT_ORDER[fmt], threads=16)[0]
+    G.say(f"{name} {rows}x{cols}: default")
+    before = G.launch_counts()
+    got = G.gpu_matmul_f32(w, x)
+    after = G.launch_counts()
+    fired = {k: v - before.get(k, 0) for k, v in after.items() if v > before.get(k, 0)}
+    assert G.same_bits(got, want), (name, rows, cols, fired)
+    one_launch = not any(k.startswith("quantize.") for k in fired)
+    # Q8_0 on 4097 to 8192 rows of at least 8192 values runs four-wave workgroups, which stage the token: two launches
+    expect_one = not (fmt == oracle.Q8_0 and 4096 < rows <= 8192)
+    assert one_launch == expect_one, (name, rows, cols, fired)
+    with G.env(CAMELID_HIP_B32_LONG_ROWS_FUSE=0), G.engaged(r"^quantize\.q8_0$"):
+        assert G.same_bits(G.gpu_matmul_f32(w, x), want), (name, rows, cols, "two launches")
+    with G.env(CAMELID_HIP_FUSED_QUANT=2), G.engaged(none=(r"^quantize\.",)):
+        assert G.same_bits(G.gpu_matmul_f32(w, x), want), (name, rows, cols, "one launch forced")
+
+
+@pytest.mark.parametrize("name,fmt", [("Q8_0", oracle.Q8_0), ("Q4_0", oracle.Q4_0)])
 @pytest.mark.parametrize("rows,cols", [(9001, 5120), (8192, 8192), (10250, 8192), (6000, 8192)])
 def test_b32_fused_launch_shapes_on_rows_longer_than_4096_values(name, fmt, rows, cols):
     """Single-token cml_matmul_f32 on Q8_0 / Q4_0 rows of more than 4096 values (every workgroup stages the token
