@@ -361,12 +361,13 @@ __global__ __launch_bounds__(256) void gemv_q6k_kernel(Q6KArgs a) {
 // steps past a shorter part's end re-read its last super-block and add nothing.
 // NT = 2 (with ANY): two contiguous f32 rows in, out[2][rows]; every pass quantizes its super-blocks of both tokens and a
 // step's unpacked weight is replayed against them -- each cell the one-token launch's bits.
-template <int KS, int NSTEPS, int NB = 4, int WAVES = 8, bool ANY = false, int NT = 1>
+template <int KS, int NSTEPS, int NB = 4, int WAVES = 8, bool ANY = false, int NT = 1, int U = 1>
 __global__ __launch_bounds__(WAVES * 64) void gemv_q6k_cu_kcut_kernel(Q6KArgs a) {
     constexpr int LPS = 8, RPW = kWave / LPS, TPW = WAVES / KS, PRE = 2;
     constexpr int PER_PASS = 2 * TPW;                       // super-blocks a pass gives every part
     constexpr int PASSES = (NSTEPS + PER_PASS - 1) / PER_PASS;
-    static_assert(NSTEPS >= NB && WAVES % KS == 0, "K parts of at least one full ring");
+    constexpr int USTEPS = (NSTEPS + U - 1) / U;  // ring steps: U super-blocks of a row each
+    static_assert(USTEPS >= NB && WAVES % KS == 0 && PER_PASS % U == 0, "K parts of at least one full ring; whole steps per quantizer pass");
     static_assert(NT == 1 || (ANY && NT == 2), "two tokens: the general form");
     const int NSB = ANY ? a.n_sb : KS * NSTEPS;
     __shared__ __attribute__((aligned(16))) int8_t ys_fixed[ANY ? 16 : KS * NSTEPS * 256];
@@ -408,9 +409,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q6k_cu_kcut_kernel(Q6KArgs a)
     const uint8_t *qh = a.qh + arow * a.qh_stride;
     const uint8_t *sc = a.sc + arow * a.sc_stride;
     const uint8_t *dp = a.d + arow * a.d_stride;
-    Q6KRegs<1> ring[NB];
-    auto request = [&](Q6KRegs<1> &b, int step) __attribute__((always_inline)) {
-        q6k_load(b, ql, qh, sc, dp, l, s0 + step, s1);
+    Q6KRegs<U> ring[NB];
+    auto request = [&](Q6KRegs<U> &b, int step) __attribute__((always_inline)) {
+        q6k_load(b, ql, qh, sc, dp, l, s0 + U * step, s1);
         __builtin_amdgcn_sched_barrier(0);
     };
 #pragma unroll
@@ -442,20 +443,20 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q6k_cu_kcut_kernel(Q6KArgs a)
     float acc[NT];
 #pragma unroll
     for (int t = 0; t < NT; t++) acc[t] = 0.0f;
-    auto compute = [&](const Q6KRegs<1> &b, int step) __attribute__((always_inline)) {
-        q6k_compute<NT, false, 1>(b, l, s0 + step, s1, ys, bsum16, yds, NSB, acc, nullptr);
+    auto compute = [&](const Q6KRegs<U> &b, int step) __attribute__((always_inline)) {
+        q6k_compute<NT, false, U>(b, l, s0 + U * step, s1, ys, bsum16, yds, NSB, acc, nullptr);
         __builtin_amdgcn_sched_barrier(0);
     };
 #pragma unroll
     for (int j = PRE; j < NB; j++) request(ring[j], j);
 #pragma unroll
-    for (int i = 0; i < NSTEPS; i++) {
-        if (i % PER_PASS == 0) {  // the first step that reads pass i / PER_PASS: the next pass goes ahead of it
-            if (i / PER_PASS + 1 < PASSES) quantize_pass(i / PER_PASS + 1);
+    for (int i = 0; i < USTEPS; i++) {
+        if ((U * i) % PER_PASS == 0) {  // the first step that reads pass U i / PER_PASS: the next pass goes ahead of it
+            if ((U * i) / PER_PASS + 1 < PASSES) quantize_pass((U * i) / PER_PASS + 1);
             if (i > 0) __syncthreads();
         }
         compute(ring[i % NB], i);
-        if (i + NB < NSTEPS) request(ring[i % NB], i + NB);
+        if (i + NB < USTEPS) request(ring[i % NB], i + NB);
     }
     if (l == LPS - 1) {
 #pragma unroll
@@ -802,8 +803,17 @@ int launch_gemv_q6k_f32(const cml_weight *w, const float *x, float *out, hipStre
             CML_Q6K_KCUT_ANY(2, 12)
             CML_Q6K_KCUT_ANY(2, 16)
             // no K cut (12288 to 24576 rows): the same launch, every wave a row tile of its own
+            // two super-blocks of a row per ring step (256 contiguous bytes of each plane row per request), three slots: 13824 x 5120
+            // 13.6 -> 12.7 us, 14336 x 8192 20.0 -> 18.8, 18944 x 3584 12.05 -> 11.8; rows of 4096 values keep four one-super-block slots
+            // (16384 x 4096 10.55 against 10.6).  CAMELID_HIP_Q6K_CU_U2=0: one super-block per step everywhere.
 #define CML_Q6K_CU_ANY(NS_)                                                                                                \
     case 100 + NS_:                                                                                                        \
+        if (NS_ != 16 && env_int("CAMELID_HIP_Q6K_CU_U2", 1)) {                                                            \
+            if (waves == 8) hipLaunchKernelGGL((gemv_q6k_cu_kcut_kernel<1, NS_, 3, 8, true, 1, 2>), grid, block, lds_any, st, ka);        \
+            else if (waves == 10) hipLaunchKernelGGL((gemv_q6k_cu_kcut_kernel<1, NS_, 3, 10, true, 1, 2>), grid, block, lds_any, st, ka); \
+            else hipLaunchKernelGGL((gemv_q6k_cu_kcut_kernel<1, NS_, 3, 12, true, 1, 2>), grid, block, lds_any, st, ka);                  \
+            break;                                                                                                         \
+        }                                                                                                                  \
         if (waves == 8) hipLaunchKernelGGL((gemv_q6k_cu_kcut_kernel<1, NS_, 4, 8, true>), grid, block, lds_any, st, ka);    \
         else if (waves == 10) hipLaunchKernelGGL((gemv_q6k_cu_kcut_kernel<1, NS_, 4, 10, true>), grid, block, lds_any, st, ka); \
         else hipLaunchKernelGGL((gemv_q6k_cu_kcut_kernel<1, NS_, 4, 12, true>), grid, block, lds_any, st, ka);              \

@@ -712,8 +712,9 @@ def test_q6k_eight_wave_launch_under_the_k_cut_on_other_rows(rows, cols):
         assert G.same_bits(got, four_wave), (rows, cols, i)
         assert G.same_bits(got_band, got[5:rows - 4]), (rows, cols, i)
         for width in (8, 12):
-            with G.env(CAMELID_HIP_Q6K_KCUT_WAVES=width), G.engaged(r"^q6k\.dot\.wg8\.kcut\.fused\.any$"):
-                assert G.same_bits(G.gpu_matmul_f32(w, x), got), (rows, cols, i, width)
+            for two_per_step in (1, 0):   # (the no-cut form: two super-blocks of a row per ring step, or one)
+                with G.env(CAMELID_HIP_Q6K_KCUT_WAVES=width, CAMELID_HIP_Q6K_CU_U2=two_per_step), G.engaged(r"^q6k\.dot\.wg8\.kcut\.fused\.any$"):
+                    assert G.same_bits(G.gpu_matmul_f32(w, x), got), (rows, cols, i, width, two_per_step)
         if i != 1:
             want = oracle.matmul(fmt, wire, cols, x[None, :], order=EXACT_ORDER[fmt], threads=16)[0]
             assert G.max_rel(got, want) <= TOL, (rows, cols, i)
