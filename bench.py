@@ -552,6 +552,8 @@ MULTI_CONFIGS = {
     "q4k_qkv_4096": ("Q4_K", [4096, 1024, 1024], 4096),           # q | k | v of a Llama-3-8B attention block (grouped-query: 8 KV heads)
     "q4k_qkv_gate_up_4096": ("Q4_K", [14336, 14336], 4096),       # gate | up through the same entry
     "q4k_qkv_3584": ("Q4_K", [3584, 512, 512], 3584),             # Qwen2.5-7B-shaped q | k | v
+    "q8_0_qkv_4096": ("Q8_0", [4096, 1024, 1024], 4096),          # the same attention block in the 32-value block formats
+    "q4_0_qkv_4096": ("Q4_0", [4096, 1024, 1024], 4096),
 }
 
 

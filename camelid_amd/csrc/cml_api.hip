@@ -974,6 +974,14 @@ int cml_matmul_f32_multi(const cml_weight *const *weights, int n_weights, const 
                 else if (frc != -1) return frc;
             }
         }
+        if (!served && (weights[j]->fmt == CML_Q8_0 || weights[j]->fmt == CML_Q4_0) && (fuse == 2 || (fuse == 1 && weights[j]->cols <= 8192))) {
+            // the same for the 32-value block formats (q | k | v of one attention block)
+            for (int take = std::min(4, n_weights - j); take >= 2 && !served; take--) {
+                const int frc = launch_gemv_b32_f32_multi(weights + j, take, x_dev, outs_dev + j, as_stream(stream));
+                if (frc == CML_OK) served = take;
+                else if (frc != -1) return frc;
+            }
+        }
         if (served) {
             g_runs.fetch_add(static_cast<uint64_t>(served), std::memory_order_relaxed);
             j += served;

@@ -52,6 +52,18 @@ struct B32Args {
     float *out2;
 };
 
+// One f32 token against up to four weights of one format and row length (any row counts) in one launch: their
+// workgroups lie end to end along grid.x, every workgroup quantizes the token once.
+struct B32MultiArgs {
+    B32Args base;             // everything the weights share (nb, x, early_loads)
+    const uint8_t *quantsm[4];
+    const uint8_t *scalesm[4];
+    int64_t q_stridem[4], s_stridem[4];
+    float *outm[4];
+    int rowsm[4];
+    int wg_end[4];            // workgroups of weights 0 .. j (INT32_MAX beyond the last weight)
+};
+
 template <int FMT, int UU = 2>
 struct B32Regs {
     static constexpr int U = UU;  // steps in flight per buffer
@@ -324,9 +336,30 @@ __device__ __forceinline__ void b32_row_pass_ring(B32Regs<FMT, 1> (&ring)[NB], c
 // FUSEQ (single token): the activation arrives as f32 and every workgroup quantizes it to Q8_0
 // itself, eight lanes per block, straight into the LDS staging area -- the arithmetic of
 // quantize_q8_0_kernel without the launch and the round trip through memory.
-template <int FMT, int P, int NT, bool INTS, bool FUSEQ = false, int WAVES = 4, int NXQ = 0, int U = 2, int RING = 0, bool PAIR = false>
-__global__ __launch_bounds__(WAVES * 64) void gemv_b32_kernel(B32Args a) {
+template <int FMT, int P, int NT, bool INTS, bool FUSEQ = false, int WAVES = 4, int NXQ = 0, int U = 2, int RING = 0, bool PAIR = false, bool MULTI = false>
+__global__ __launch_bounds__(WAVES * 64) void gemv_b32_kernel(std::conditional_t<MULTI, B32MultiArgs, B32Args> a_in) {
     static_assert(!PAIR || (FUSEQ && NT == 1 && !INTS), "a pair: one f32 token against two weights of one shape");
+    static_assert(!MULTI || (FUSEQ && NT == 1 && !INTS && !PAIR), "a multi launch: one f32 token against several weights");
+    B32Args a_sel;        // MULTI: the shared arguments with this workgroup's weight filled in
+    int bx = blockIdx.x;  // workgroup index within its weight
+    if constexpr (MULTI) {
+        B32Args &a = a_sel;
+        a = a_in.base;
+        // which weight this workgroup belongs to (wave-uniform selects: no indexed access to the argument block)
+        const int j = (bx >= a_in.wg_end[0]) + (bx >= a_in.wg_end[1]) + (bx >= a_in.wg_end[2]);
+        auto pick = [&](auto v0, auto v1, auto v2, auto v3) { return j == 0 ? v0 : (j == 1 ? v1 : (j == 2 ? v2 : v3)); };
+        a.quants = pick(a_in.quantsm[0], a_in.quantsm[1], a_in.quantsm[2], a_in.quantsm[3]);
+        a.scales = pick(a_in.scalesm[0], a_in.scalesm[1], a_in.scalesm[2], a_in.scalesm[3]);
+        a.q_stride = pick(a_in.q_stridem[0], a_in.q_stridem[1], a_in.q_stridem[2], a_in.q_stridem[3]);
+        a.s_stride = pick(a_in.s_stridem[0], a_in.s_stridem[1], a_in.s_stridem[2], a_in.s_stridem[3]);
+        a.out = pick(a_in.outm[0], a_in.outm[1], a_in.outm[2], a_in.outm[3]);
+        a.rows = pick(a_in.rowsm[0], a_in.rowsm[1], a_in.rowsm[2], a_in.rowsm[3]);
+        bx -= pick(0, a_in.wg_end[0], a_in.wg_end[1], a_in.wg_end[2]);
+    }
+    const B32Args &a = [&]() -> const B32Args & {
+        if constexpr (MULTI) return a_sel;
+        else return a_in;
+    }();
     static_assert(RING == 0 || (RING == 3 && FUSEQ && NXQ > 0 && !INTS), "the ring serves the fused single-launch calls with the activation in registers");
     constexpr int NB = RING ? RING : 1, PRE = RING ? 2 : 1;
     constexpr int T = WAVES * 64;  // threads of a workgroup; its activation prologue is shared by WAVES * (64 / P) rows
@@ -347,7 +380,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_b32_kernel(B32Args a) {
 
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int r = lane / P, l = lane - r * P;
-    const int row = (blockIdx.x * WAVES + wave) * RPW + r;
+    const int row = (bx * WAVES + wave) * RPW + r;
     const bool live = row < a.rows;
     const int64_t arow = band * a.rows + (live ? row : a.rows - 1);
     const bool second = PAIR && blockIdx.z == 1;
@@ -750,6 +783,74 @@ int launch_gemv_b32_f32_pair(const cml_weight *w, const cml_weight *w2, const fl
     if (w->rows == 0) return CML_OK;
     if (b32_lanes(w->fmt, w->rows, w->nb) != 16) return -1;
     return w->fmt == CML_Q8_0 ? launch_b32_f32_p<CML_Q8_0, 16>(w, x, out, st, 1, w2, out2) : launch_b32_f32_p<CML_Q4_0, 16>(w, x, out, st, 1, w2, out2);
+}
+
+// One f32 token against two to four Q8_0 or Q4_0 weights of one row length in ONE launch (the q, k and v projections of
+// an attention block): the eight-wave launches with the token in registers; every output is its own call's bits
+// (the row chain does not depend on the launch shape).  -1 = not a set this launch serves.
+// CAMELID_HIP_B32_MULTI=0: the caller makes the calls one by one.
+template <int FMT, int P>
+static int launch_b32_multi_p(const cml_weight *const *ws, int n, const float *x, float *const *outs, int nxq, hipStream_t st) {
+    B32MultiArgs ma{};
+    ma.base.nb = static_cast<int>(ws[0]->nb);
+    ma.base.x = x;
+    ma.base.early_loads = 1;
+    constexpr int rows_per_wg = 8 * (64 / P);
+    int wg = 0;
+    for (int j = 0; j < 4; j++) {
+        const cml_weight *w = ws[std::min(j, n - 1)];
+        ma.quantsm[j] = w->planes.p[0];
+        ma.q_stridem[j] = w->planes.row_stride[0];
+        ma.scalesm[j] = w->planes.p[1];
+        ma.s_stridem[j] = w->planes.row_stride[1];
+        ma.outm[j] = outs[std::min(j, n - 1)];
+        ma.rowsm[j] = static_cast<int>(w->rows);
+        if (j < n) wg += (ma.rowsm[j] + rows_per_wg - 1) / rows_per_wg;
+        ma.wg_end[j] = j < n ? wg : INT32_MAX;
+    }
+    const size_t lds = static_cast<size_t>(ma.base.nb) * (32 + 4 + 4);
+    const dim3 grid(static_cast<unsigned>(wg)), block(512);
+#define CML_B32_MULTI(N_) hipLaunchKernelGGL((gemv_b32_kernel<FMT, P, 1, false, true, 8, N_, 2, 0, false, true>), grid, block, lds, st, ma)
+    switch (nxq) {
+        case 1: CML_B32_MULTI(1); break;
+        case 2: CML_B32_MULTI(2); break;
+        case 4: CML_B32_MULTI(4); break;
+        case 8: CML_B32_MULTI(8); break;
+        default: return -1;
+    }
+#undef CML_B32_MULTI
+    CML_COUNT_LAUNCH((b32_counter<FMT, P>("w8.fused.multi")));
+    CML_HIP_TRY(hipGetLastError());
+    return CML_OK;
+}
+
+int launch_gemv_b32_f32_multi(const cml_weight *const *ws, int n, const float *x, float *const *outs, hipStream_t st) {
+    if (n < 2 || n > 4 || !env_int("CAMELID_HIP_B32_MULTI", 1) || !env_int("CAMELID_HIP_MULTI_LAUNCH", 1)) return -1;
+    const int fmt = ws[0]->fmt;
+    if (fmt != CML_Q8_0 && fmt != CML_Q4_0) return -1;
+    int64_t rows_all = 0;
+    for (int j = 0; j < n; j++) {
+        if (ws[j]->fmt != fmt || ws[j]->nb != ws[0]->nb || ws[j]->rows <= 0) return -1;
+        rows_all += ws[j]->rows;
+    }
+    if (rows_all > INT32_MAX || static_cast<size_t>(ws[0]->nb) * (32 + 4 + 4) > 64 * 1024) return -1;
+    if (!x) return fail(CML_ERR_INVALID, "null activation");
+    const int p = b32_lanes(fmt, rows_all, ws[0]->nb);
+    const B32FusedShape fs = b32_fused_shape(fmt, p, static_cast<int>(rows_all), static_cast<int>(ws[0]->nb), false, false, true);
+    // the eight-wave launches with the token in registers (a set whose total shape takes another launch: single calls)
+    int nxq = fs.nxq;
+    if (fs.waves != 8) {
+        const int n4 = static_cast<int>(ws[0]->nb) * 8;
+        nxq = n4 <= 512 ? 1 : n4 <= 1024 ? 2 : n4 <= 2048 ? 4 : n4 <= 4096 ? 8 : 0;
+    }
+    if (nxq == 0) return -1;
+    const bool q8 = fmt == CML_Q8_0;
+    switch (p) {
+        case 8: return q8 ? launch_b32_multi_p<CML_Q8_0, 8>(ws, n, x, outs, nxq, st) : launch_b32_multi_p<CML_Q4_0, 8>(ws, n, x, outs, nxq, st);
+        case 32: return q8 ? launch_b32_multi_p<CML_Q8_0, 32>(ws, n, x, outs, nxq, st) : launch_b32_multi_p<CML_Q4_0, 32>(ws, n, x, outs, nxq, st);
+        case 64: return q8 ? launch_b32_multi_p<CML_Q8_0, 64>(ws, n, x, outs, nxq, st) : launch_b32_multi_p<CML_Q4_0, 64>(ws, n, x, outs, nxq, st);
+        default: return q8 ? launch_b32_multi_p<CML_Q8_0, 16>(ws, n, x, outs, nxq, st) : launch_b32_multi_p<CML_Q4_0, 16>(ws, n, x, outs, nxq, st);
+    }
 }
 
 int launch_gemv_b32_f32(const cml_weight *w, const float *x, float *out, hipStream_t st, int n_tokens) {

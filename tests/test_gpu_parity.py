@@ -1510,7 +1510,8 @@ def _multi(ws, x, stream=None):
 
 
 @pytest.mark.parametrize("case", ["qkv_4096", "gate_up_14336", "ragged_2304", "three_3584", "mixed_cut", "five", "q6k", "bands",
-                                  "cut4_8192", "cut2_4096"])
+                                  "cut4_8192", "cut2_4096", "q8_0_qkv_4096", "q4_0_qkv_3584", "q8_0_ragged_2048", "q4_0_pair_8192",
+                                  "q4_0_gate_up_14336", "q8_0_tiny"])
 def test_matmul_f32_multi_is_the_single_calls(case):
     """cml_matmul_f32_multi: several weights that read one token (q | k | v of an attention block, gate | up of an FFN).
     Runs of up to four Q4_K weights with one K cut go out as one launch -- the counters prove it -- and every
@@ -1528,9 +1529,19 @@ def test_matmul_f32_multi_is_the_single_calls(case):
         "five": ([512, 256, 256, 128, 640], 2048, 2),       # four in one launch, the fifth alone
         "q6k": ([300, 200], 1024, 0),
         "bands": ([700, 300, 650], 4096, 1),
+        "q8_0_qkv_4096": ([4096, 1024, 1024], 4096, 1),     # the 32-value block formats: one launch too
+        "q4_0_qkv_3584": ([3584, 512, 512], 3584, 1),
+        "q8_0_ragged_2048": ([200, 77, 530, 16], 2048, 1),
+        "q4_0_pair_8192": ([4096, 1030], 8192, 1),
+        "q4_0_gate_up_14336": ([14336, 14336], 4096, 1),
+        "q8_0_tiny": ([40, 24], 64, 1),
     }[case]
     if case == "q6k":
         fmt = B.CML_Q6_K
+    elif case.startswith("q8_0"):
+        fmt = B.CML_Q8_0
+    elif case.startswith("q4_0"):
+        fmt = B.CML_Q4_0
     rng = np.random.default_rng(sum(shapes) + cols)
     ws = [Weight.upload(fmt, r, cols, G.synth_weight(fmt, r, cols, seed=r + cols + j)) for j, r in enumerate(shapes)]
     if case == "bands":   # views that start inside a 16-row tile
@@ -1542,6 +1553,8 @@ def test_matmul_f32_multi_is_the_single_calls(case):
     G.say(f"multi {case}: one call")
     if case == "q6k":
         proof = G.engaged(r"^q6k\.dot\.", none=(r"multi",))
+    elif fmt in (B.CML_Q8_0, B.CML_Q4_0):
+        proof = G.engaged(r"^q[48]_0\.dot\.p\d+\.w8\.fused\.multi$", none=(r"^quantize\.",))
     elif one_launch == 0:
         proof = G.engaged(r"^q4k\.dot\.", none=(r"multi",))
     elif case in ("qkv_4096", "cut4_8192", "cut2_4096"):   # ("bands" is too small for eight-wave workgroups to fill the chip)
