@@ -42,13 +42,13 @@ INT8_PEAK_TOPS = 5000.0  # MI355X published dense int8 matrix-core rate
 TRAFFIC_SOURCE = "profiles/hbm_traffic_fetch_write_size.txt"
 TRAFFIC_READINGS: dict = {
     # config -> (bytes per launch, kernel-family counter the step must have fired for the reading to apply, kernel symbol)
-    "q4k_14336x4096_n1": (33337928, "q4k.dot.wg8.fused", "gemv_q4k_cu_kernel<8, 0, 1, 8>"),                       # 1.007 x algorithmic
-    "q4k_4096x14336_n1": (33677871, "q4k.dot.wg8.kcut.fused", "gemv_q4k_cu_kcut_kernel<4, 7, 0, true, 8, false>"),  # 1.017 x
-    "q4k_14336x4096_n16": (34691633, "q4k.mfma.pair", "gemm_q4k_mfma_pair_kernel<false>"),                        # 1.014 x
-    "q4k_14336x4096_n64": (39147971, "q4k.mfma.tile.g4t1", "gemm_q4k_mfma_kernel<4, 1, false, 1, true, false>"),  # 1.037 x
-    "q6k_128256x3072_n1": (323895279, "q6k.dot.deep", "gemv_q6k_kernel<1, false, false, 4, false>"),              # 1.001 x
-    "q4_0_128256x3072_n16": (252013735, "q4_0.mfma.tile", "gemm_b32_mfma_kernel<2, 1, 1, 2, 2, true, 4>"),        # 1.096 x
-    "q6k_128256x3072_n16": (356106585, "q6k.mfma.tile", "gemm_q6k_mfma_kernel<1, 1, false, 2, 2, 1, true>"),      # 1.074 x
+    "q4k_14336x4096_n1": (33323600, "q4k.dot.wg8.fused", "gemv_q4k_cu_kernel<8, 0, 1, 8>"),                       # 1.007 x algorithmic
+    "q4k_4096x14336_n1": (33677877, "q4k.dot.wg8.kcut.fused", "gemv_q4k_cu_kcut_kernel<4, 7, 0, true, 8, false>"),  # 1.017 x
+    "q4k_14336x4096_n16": (34691593, "q4k.mfma.pair", "gemm_q4k_mfma_pair_kernel<false>"),                        # 1.014 x
+    "q4k_14336x4096_n64": (39147913, "q4k.mfma.tile.g4t1", "gemm_q4k_mfma_kernel<4, 1, false, 1, true, false>"),  # 1.037 x
+    "q6k_128256x3072_n1": (323896969, "q6k.dot.deep", "gemv_q6k_kernel<1, false, false, 4, false>"),              # 1.001 x
+    "q4_0_128256x3072_n16": (252021326, "q4_0.mfma.tile", "gemm_b32_mfma_kernel<2, 1, 1, 2, 2, true, 4>"),        # 1.096 x
+    "q6k_128256x3072_n16": (356232056, "q6k.mfma.tile", "gemm_q6k_mfma_kernel<1, 1, false, 2, 2, 1, true>"),      # 1.074 x
 }
 
 # rocprofv3 --kernel-trace averages of the dominant kernel, read at run time from the committed summaries (never copied
