@@ -937,7 +937,13 @@ int cml_matmul_f32_pair(const cml_weight *w_a, const cml_weight *w_b, const floa
     }
     if (same_shape && w_a->rows > 0 && (w_a->fmt == CML_Q8_0 || w_a->fmt == CML_Q4_0) && w_a->planes.row_stride[1] == w_b->planes.row_stride[1] &&
         (fuse == 2 || (fuse == 1 && w_a->cols <= 8192 && w_a->rows <= 32768)) && env_int("CAMELID_HIP_PAIR_LAUNCH", 1)) {
-        const int frc = launch_gemv_b32_f32_pair(w_a, w_b, x_dev, out_a_dev, out_b_dev, as_stream(stream));
+        int frc = launch_gemv_b32_f32_pair(w_a, w_b, x_dev, out_a_dev, out_b_dev, as_stream(stream));
+        if (frc == -1) {
+            // a shape the pair launch (16 lanes per row, up to two float4 of the token per thread) does not take: the multi launch
+            const cml_weight *const ws[2] = {w_a, w_b};
+            float *const outs[2] = {out_a_dev, out_b_dev};
+            frc = launch_gemv_b32_f32_multi(ws, 2, x_dev, outs, as_stream(stream));
+        }
         if (frc == CML_OK) g_runs.fetch_add(2, std::memory_order_relaxed);
         if (frc != -1) return frc;
     }

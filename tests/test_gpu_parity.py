@@ -1368,7 +1368,9 @@ def test_q4k_single_token_entry_points_give_the_same_bits(rows, cols):
                                                 ("Q4_K", B.CML_Q4_K, 530, 2304), ("Q4_K", B.CML_Q4_K, 4096, 14336), ("Q4_K", B.CML_Q4_K, 17000, 1024),
                                                 ("Q6_K", B.CML_Q6_K, 300, 1024), ("Q8_0", B.CML_Q8_0, 700, 2048), ("Q4_0", B.CML_Q4_0, 64, 96),
                                                 ("Q8_0", B.CML_Q8_0, 8192, 2048), ("Q8_0", B.CML_Q8_0, 4099, 4096), ("Q4_0", B.CML_Q4_0, 4100, 4096),
-                                                ("Q4_0", B.CML_Q4_0, 5000, 1056), ("Q8_0", B.CML_Q8_0, 4500, 96)])
+                                                ("Q4_0", B.CML_Q4_0, 5000, 1056), ("Q8_0", B.CML_Q8_0, 4500, 96),
+                                                # shapes the b32 pair launch does not take: served by the multi launch of two weights
+                                                ("Q8_0", B.CML_Q8_0, 4096, 4096), ("Q4_0", B.CML_Q4_0, 6000, 5120), ("Q4_0", B.CML_Q4_0, 3000, 8192)])
 def test_matmul_f32_pair_is_two_single_calls(name, fmt, rows, cols):
     """cml_matmul_f32_pair (one token, two weights that read it: gate and up of a dense FFN): the bits
     of two cml_matmul_f32 calls -- where it runs as one launch (Q4_K, with and without the ring of
@@ -1393,8 +1395,12 @@ def test_matmul_f32_pair_is_two_single_calls(name, fmt, rows, cols):
 
     G.say(f"pair {name} {rows}x{cols}")
     want_a, want_b = G.gpu_matmul_f32(wa, x), G.gpu_matmul_f32(wb, x)
+    if (name, rows, cols) in (("Q8_0", 4096, 4096), ("Q4_0", 6000, 5120), ("Q4_0", 3000, 8192)):
+        with G.engaged(r"^q[48]_0\.dot\.p\d+\.w8\.fused\.multi$", none=(r"^quantize\.", r"pair")):
+            got_a, got_b = pair(wa, wb)
+        assert G.same_bits(got_a, want_a) and G.same_bits(got_b, want_b), (name, rows, cols, "multi launch of two")
     for knobs in ({}, {"CAMELID_HIP_Q4K_RING": "0", "CAMELID_HIP_B32_RING": "0"}, {"CAMELID_HIP_PAIR_LAUNCH": "0"}, {"CAMELID_HIP_Q4K_ROWS_PER_WAVE": "16"},
-                  {"CAMELID_HIP_Q4K_ROWS_PER_WAVE": "8"}):
+                  {"CAMELID_HIP_Q4K_ROWS_PER_WAVE": "8"}, {"CAMELID_HIP_B32_MULTI": "0"}):
         with G.env(**knobs):
             got_a, got_b = pair(wa, wb)
         assert G.same_bits(got_a, want_a), (name, rows, cols, knobs)
