@@ -554,6 +554,7 @@ MULTI_CONFIGS = {
     "q4k_qkv_3584": ("Q4_K", [3584, 512, 512], 3584),             # Qwen2.5-7B-shaped q | k | v
     "q8_0_qkv_4096": ("Q8_0", [4096, 1024, 1024], 4096),          # the same attention block in the 32-value block formats
     "q4_0_qkv_4096": ("Q4_0", [4096, 1024, 1024], 4096),
+    "q6k_qkv_4096": ("Q6_K", [4096, 1024, 1024], 4096),
 }
 
 

@@ -947,6 +947,15 @@ int cml_matmul_f32_pair(const cml_weight *w_a, const cml_weight *w_b, const floa
         if (frc == CML_OK) g_runs.fetch_add(2, std::memory_order_relaxed);
         if (frc != -1) return frc;
     }
+    if (same_shape && w_a->rows > 0 && w_a->fmt == CML_Q6_K && !q6k_lane_order() && env_int("CAMELID_HIP_Q6K_FUSED_QUANT", 1) &&
+        (fuse == 2 || (fuse == 1 && w_a->nb <= 32)) && env_int("CAMELID_HIP_PAIR_LAUNCH", 1)) {
+        // Q6_K: the multi launch of two weights (gate and up of 14336 x 4096: 21.2 -> 19.0 us)
+        const cml_weight *const ws[2] = {w_a, w_b};
+        float *const outs[2] = {out_a_dev, out_b_dev};
+        const int frc = launch_gemv_q6k_f32_multi(ws, 2, x_dev, outs, as_stream(stream));
+        if (frc == CML_OK) g_runs.fetch_add(2, std::memory_order_relaxed);
+        if (frc != -1) return frc;
+    }
     if (int rc = cml_matmul_f32(w_a, x_dev, 1, out_a_dev, workspace_dev, workspace_bytes, stream)) return rc;
     return cml_matmul_f32(w_b, x_dev, 1, out_b_dev, workspace_dev, workspace_bytes, stream);
 }
@@ -984,6 +993,15 @@ int cml_matmul_f32_multi(const cml_weight *const *weights, int n_weights, const 
             // the same for the 32-value block formats (q | k | v of one attention block)
             for (int take = std::min(4, n_weights - j); take >= 2 && !served; take--) {
                 const int frc = launch_gemv_b32_f32_multi(weights + j, take, x_dev, outs_dev + j, as_stream(stream));
+                if (frc == CML_OK) served = take;
+                else if (frc != -1) return frc;
+            }
+        }
+        if (!served && weights[j]->fmt == CML_Q6_K && !q6k_lane_order() && env_int("CAMELID_HIP_Q6K_FUSED_QUANT", 1) &&
+            (fuse == 2 || (fuse == 1 && weights[j]->nb <= 32))) {
+            // and for Q6_K sets whose shapes take one K cut
+            for (int take = std::min(4, n_weights - j); take >= 2 && !served; take--) {
+                const int frc = launch_gemv_q6k_f32_multi(weights + j, take, x_dev, outs_dev + j, as_stream(stream));
                 if (frc == CML_OK) served = take;
                 else if (frc != -1) return frc;
             }

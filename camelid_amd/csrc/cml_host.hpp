@@ -162,7 +162,8 @@ int launch_gemv_q4k_loads_only(const cml_weight *w, float *out, hipStream_t st);
 int launch_gemv_q4k_ablated(const cml_weight *w, const float *x, float *out, int mask, hipStream_t st);  // calibration: parts of the launch taken out
 int launch_gemv_q6k_f32(const cml_weight *w, const float *x, float *out, hipStream_t st, int n_tokens = 1);  // Q6_K: quantize + matvec, one or two tokens
 int launch_gemv_b32_f32(const cml_weight *w, const float *x, float *out, hipStream_t st, int n_tokens = 1);
-int launch_gemv_b32_f32_multi(const cml_weight *const *ws, int n, const float *x, float *const *outs, hipStream_t st);  // -1 = not served  // quantize + matvec, one or two tokens
+int launch_gemv_b32_f32_multi(const cml_weight *const *ws, int n, const float *x, float *const *outs, hipStream_t st);  // -1 = not served
+int launch_gemv_q6k_f32_multi(const cml_weight *const *ws, int n, const float *x, float *const *outs, hipStream_t st);  // -1 = not served  // quantize + matvec, one or two tokens
 int launch_gemv_b32_f32_pair(const cml_weight *w, const cml_weight *w2, const float *x, float *out, float *out2, hipStream_t st);  // -1: not served
 // Where a grouped matvec takes its activation rows from instead of MatArgs::q / scales:
 //   kind 1: ONE f32 token x, quantized inside the kernel, read by every assignment

@@ -21,6 +21,8 @@
 #include "cml_device.hpp"
 #include "cml_host.hpp"
 
+#include <type_traits>
+
 #pragma clang fp contract(off)
 
 namespace cml {
@@ -55,6 +57,17 @@ struct Q6KArgs {
     int n_groups;
     int ksplit;       // 1, 2 or 4 waves per row tile
     int ksplit_log2;
+};
+
+// One f32 token against up to four Q6_K weights of one row length and one K cut (any row counts) in one launch of the
+// one-workgroup-per-unit form: their workgroups lie end to end along grid.x, every workgroup quantizes the token once.
+struct Q6KMultiArgs {
+    Q6KArgs base;  // what the weights share (n_sb, x, ksplit)
+    const uint8_t *qlm[4], *qhm[4], *scm[4], *dm[4];
+    int64_t ql_stridem[4], qh_stridem[4], sc_stridem[4], d_stridem[4];
+    float *outm[4];
+    int rowsm[4];
+    int wg_end[4];  // workgroups of weights 0 .. j (INT32_MAX beyond the last weight)
 };
 
 template <int U_>
@@ -361,8 +374,33 @@ __global__ __launch_bounds__(256) void gemv_q6k_kernel(Q6KArgs a) {
 // steps past a shorter part's end re-read its last super-block and add nothing.
 // NT = 2 (with ANY): two contiguous f32 rows in, out[2][rows]; every pass quantizes its super-blocks of both tokens and a
 // step's unpacked weight is replayed against them -- each cell the one-token launch's bits.
-template <int KS, int NSTEPS, int NB = 4, int WAVES = 8, bool ANY = false, int NT = 1, int U = 1>
-__global__ __launch_bounds__(WAVES * 64) void gemv_q6k_cu_kcut_kernel(Q6KArgs a) {
+template <int KS, int NSTEPS, int NB = 4, int WAVES = 8, bool ANY = false, int NT = 1, int U = 1, bool MULTI = false>
+__global__ __launch_bounds__(WAVES * 64) void gemv_q6k_cu_kcut_kernel(std::conditional_t<MULTI, Q6KMultiArgs, Q6KArgs> a_in) {
+    static_assert(!MULTI || (ANY && NT == 1), "the multi launch: the general form, one token");
+    Q6KArgs a_sel;        // MULTI: the shared arguments with this workgroup's weight filled in
+    int bx = blockIdx.x;  // workgroup index within its weight
+    if constexpr (MULTI) {
+        Q6KArgs &a = a_sel;
+        a = a_in.base;
+        // which weight this workgroup belongs to (wave-uniform selects: no indexed access to the argument block)
+        const int j = (bx >= a_in.wg_end[0]) + (bx >= a_in.wg_end[1]) + (bx >= a_in.wg_end[2]);
+        auto pick = [&](auto v0, auto v1, auto v2, auto v3) { return j == 0 ? v0 : (j == 1 ? v1 : (j == 2 ? v2 : v3)); };
+        a.ql = pick(a_in.qlm[0], a_in.qlm[1], a_in.qlm[2], a_in.qlm[3]);
+        a.qh = pick(a_in.qhm[0], a_in.qhm[1], a_in.qhm[2], a_in.qhm[3]);
+        a.sc = pick(a_in.scm[0], a_in.scm[1], a_in.scm[2], a_in.scm[3]);
+        a.d = pick(a_in.dm[0], a_in.dm[1], a_in.dm[2], a_in.dm[3]);
+        a.ql_stride = pick(a_in.ql_stridem[0], a_in.ql_stridem[1], a_in.ql_stridem[2], a_in.ql_stridem[3]);
+        a.qh_stride = pick(a_in.qh_stridem[0], a_in.qh_stridem[1], a_in.qh_stridem[2], a_in.qh_stridem[3]);
+        a.sc_stride = pick(a_in.sc_stridem[0], a_in.sc_stridem[1], a_in.sc_stridem[2], a_in.sc_stridem[3]);
+        a.d_stride = pick(a_in.d_stridem[0], a_in.d_stridem[1], a_in.d_stridem[2], a_in.d_stridem[3]);
+        a.out = pick(a_in.outm[0], a_in.outm[1], a_in.outm[2], a_in.outm[3]);
+        a.rows = pick(a_in.rowsm[0], a_in.rowsm[1], a_in.rowsm[2], a_in.rowsm[3]);
+        bx -= pick(0, a_in.wg_end[0], a_in.wg_end[1], a_in.wg_end[2]);
+    }
+    const Q6KArgs &a = [&]() -> const Q6KArgs & {
+        if constexpr (MULTI) return a_sel;
+        else return a_in;
+    }();
     constexpr int LPS = 8, RPW = kWave / LPS, TPW = WAVES / KS, PRE = 2;
     constexpr int PER_PASS = 2 * TPW;                       // super-blocks a pass gives every part
     constexpr int PASSES = (NSTEPS + PER_PASS - 1) / PER_PASS;
@@ -402,7 +440,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q6k_cu_kcut_kernel(Q6KArgs a)
     __builtin_amdgcn_sched_barrier(0);
 
     const int r = lane / LPS, l = lane - r * LPS;
-    const int row = (blockIdx.x * TPW + tile_in_wg) * RPW + r;
+    const int row = (bx * TPW + tile_in_wg) * RPW + r;
     const bool live = row < a.rows;
     const int64_t arow = live ? row : a.rows - 1;  // rows past the end (grid rounding) re-read the last row and store nothing
     const uint8_t *ql = a.ql + arow * a.ql_stride;
@@ -465,7 +503,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q6k_cu_kcut_kernel(Q6KArgs a)
     __syncthreads();
     if (tid < TPW * NT * RPW) {
         const int rr = tid % RPW, t = (tid / RPW) % NT, tw = tid / (RPW * NT);
-        const int orow = (blockIdx.x * TPW + tw) * RPW + rr;
+        const int orow = (bx * TPW + tw) * RPW + rr;
         if (orow < a.rows) {
             float v = part[((tw * KS) * NT + t) * RPW + rr];
 #pragma unroll
@@ -514,6 +552,65 @@ static int q6k_cu_kcut_any_steps(int64_t rows, int64_t n_sb) {
 }
 bool gemv_q6k_long_rows_fuse(const cml_weight *w) {
     return w->fmt == CML_Q6_K && (q6k_cu_kcut_serves(w->rows, w->nb) || q6k_cu_kcut_any_steps(w->rows, w->nb) != 0);
+}
+
+// One f32 token against two to four Q6_K weights of one row length whose shapes take the same K cut, in ONE launch of
+// the one-workgroup-per-unit form (eight waves); every output is its own call's bits.  -1 = not a set this launch
+// serves.  CAMELID_HIP_Q6K_MULTI=0: the caller makes the calls one by one.
+int launch_gemv_q6k_f32_multi(const cml_weight *const *ws, int n, const float *x, float *const *outs, hipStream_t st) {
+    if (n < 2 || n > 4 || !env_int("CAMELID_HIP_Q6K_MULTI", 1) || !env_int("CAMELID_HIP_MULTI_LAUNCH", 1)) return -1;
+    const int64_t n_sb = ws[0]->nb;
+    int ks = 0, steps = 0;
+    for (int j = 0; j < n; j++) {
+        if (ws[j]->fmt != CML_Q6_K || ws[j]->nb != n_sb || ws[j]->rows <= 0) return -1;
+        const int k = pick_ksplit_q6k(ws[j]->rows, n_sb), st_j = q6k_cu_kcut_any_steps(ws[j]->rows, n_sb);
+        if (st_j == 0 || (j && (k != ks || st_j != steps))) return -1;
+        ks = k;
+        steps = st_j;
+    }
+    if (!x) return fail(CML_ERR_INVALID, "null activation");
+    Q6KMultiArgs ma{};
+    ma.base.n_sb = static_cast<int>(n_sb);
+    ma.base.x = x;
+    ma.base.n_groups = 1;
+    ma.base.ksplit = ks;
+    ma.base.ksplit_log2 = ks >= 4 ? 2 : (ks >= 2 ? 1 : 0);
+    const int tpw = 8 / ks;  // 8-row tiles per eight-wave workgroup
+    int wg = 0;
+    for (int j = 0; j < 4; j++) {
+        const cml_weight *w = ws[std::min(j, n - 1)];
+        ma.qlm[j] = w->planes.p[0]; ma.ql_stridem[j] = w->planes.row_stride[0];
+        ma.qhm[j] = w->planes.p[1]; ma.qh_stridem[j] = w->planes.row_stride[1];
+        ma.scm[j] = w->planes.p[2]; ma.sc_stridem[j] = w->planes.row_stride[2];
+        ma.dm[j] = w->planes.p[3];  ma.d_stridem[j] = w->planes.row_stride[3];
+        ma.outm[j] = outs[std::min(j, n - 1)];
+        ma.rowsm[j] = static_cast<int>(w->rows);
+        if (j < n) wg += static_cast<int>(((w->rows + 7) / 8 + tpw - 1) / tpw);
+        ma.wg_end[j] = j < n ? wg : INT32_MAX;
+    }
+    const dim3 grid(static_cast<unsigned>(wg)), block(512);
+    const size_t lds = static_cast<size_t>(n_sb) * (256 + 64 + 4);
+#define CML_Q6K_MULTI(KS_, NS_) \
+    case KS_ * 100 + NS_: hipLaunchKernelGGL((gemv_q6k_cu_kcut_kernel<KS_, NS_, 4, 8, true, 1, 1, true>), grid, block, lds, st, ma); break;
+    switch (ks * 100 + steps) {
+        CML_Q6K_MULTI(4, 4)
+        CML_Q6K_MULTI(4, 5)
+        CML_Q6K_MULTI(4, 6)
+        CML_Q6K_MULTI(4, 8)
+        CML_Q6K_MULTI(2, 4)
+        CML_Q6K_MULTI(2, 6)
+        CML_Q6K_MULTI(2, 7)
+        CML_Q6K_MULTI(2, 8)
+        CML_Q6K_MULTI(1, 12)
+        CML_Q6K_MULTI(1, 14)
+        CML_Q6K_MULTI(1, 16)
+        CML_Q6K_MULTI(1, 20)
+        default: return -1;
+    }
+#undef CML_Q6K_MULTI
+    CML_COUNT_LAUNCH("q6k.dot.wg8.kcut.fused.multi");
+    CML_HIP_TRY(hipGetLastError());
+    return CML_OK;
 }
 
 static size_t q6k_lds_bytes(int nt, int n_sb) {

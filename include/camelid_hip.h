@@ -322,8 +322,8 @@ int cml_matmul_f32_pair(const cml_weight *w_a, const cml_weight *w_b, const floa
  * gate and up of an FFN -- the projections the reference runs off one SharedActivation,
  * src/gemma4_runtime.rs:1288-1340; the per-layer dispatch_gemv calls of the device lane,
  * src/cuda_resident.rs:18161-19525): outs_dev[j][rows_j] = weights[j] x.  All weights read rows of
- * the same length; runs of up to four Q4_K weights whose shapes take the same K cut, and of up to
- * four Q8_0 or Q4_0 weights, go out as ONE launch (their workgroups end to end, the token quantized
+ * the same length; runs of up to four Q4_K or Q6_K weights whose shapes take the same K cut, and of
+ * up to four Q8_0 or Q4_0 weights, go out as ONE launch (their workgroups end to end, the token quantized
  * once per workgroup), everything else as calls of its own.  The bits of n cml_matmul_f32 calls either way.  workspace as for
  * cml_matmul_f32 with one token.  weights / outs_dev are host arrays of n pointers. */
 int cml_matmul_f32_multi(const cml_weight *const *weights, int n_weights, const float *x_dev,

@@ -1370,7 +1370,8 @@ def test_q4k_single_token_entry_points_give_the_same_bits(rows, cols):
                                                 ("Q8_0", B.CML_Q8_0, 8192, 2048), ("Q8_0", B.CML_Q8_0, 4099, 4096), ("Q4_0", B.CML_Q4_0, 4100, 4096),
                                                 ("Q4_0", B.CML_Q4_0, 5000, 1056), ("Q8_0", B.CML_Q8_0, 4500, 96),
                                                 # shapes the b32 pair launch does not take: served by the multi launch of two weights
-                                                ("Q8_0", B.CML_Q8_0, 4096, 4096), ("Q4_0", B.CML_Q4_0, 6000, 5120), ("Q4_0", B.CML_Q4_0, 3000, 8192)])
+                                                ("Q8_0", B.CML_Q8_0, 4096, 4096), ("Q4_0", B.CML_Q4_0, 6000, 5120), ("Q4_0", B.CML_Q4_0, 3000, 8192),
+                                                ("Q6_K", B.CML_Q6_K, 14336, 4096), ("Q6_K", B.CML_Q6_K, 4100, 4096)])
 def test_matmul_f32_pair_is_two_single_calls(name, fmt, rows, cols):
     """cml_matmul_f32_pair (one token, two weights that read it: gate and up of a dense FFN): the bits
     of two cml_matmul_f32 calls -- where it runs as one launch (Q4_K, with and without the ring of
@@ -1399,8 +1400,12 @@ def test_matmul_f32_pair_is_two_single_calls(name, fmt, rows, cols):
         with G.engaged(r"^q[48]_0\.dot\.p\d+\.w8\.fused\.multi$", none=(r"^quantize\.", r"pair")):
             got_a, got_b = pair(wa, wb)
         assert G.same_bits(got_a, want_a) and G.same_bits(got_b, want_b), (name, rows, cols, "multi launch of two")
+    if name == "Q6_K" and rows >= 4096:
+        with G.engaged(r"^q6k\.dot\.wg8\.kcut\.fused\.multi$", none=(r"^quantize\.",)):
+            got_a, got_b = pair(wa, wb)
+        assert G.same_bits(got_a, want_a) and G.same_bits(got_b, want_b), (name, rows, cols, "multi launch of two")
     for knobs in ({}, {"CAMELID_HIP_Q4K_RING": "0", "CAMELID_HIP_B32_RING": "0"}, {"CAMELID_HIP_PAIR_LAUNCH": "0"}, {"CAMELID_HIP_Q4K_ROWS_PER_WAVE": "16"},
-                  {"CAMELID_HIP_Q4K_ROWS_PER_WAVE": "8"}, {"CAMELID_HIP_B32_MULTI": "0"}):
+                  {"CAMELID_HIP_Q4K_ROWS_PER_WAVE": "8"}, {"CAMELID_HIP_B32_MULTI": "0"}, {"CAMELID_HIP_Q6K_MULTI": "0"}):
         with G.env(**knobs):
             got_a, got_b = pair(wa, wb)
         assert G.same_bits(got_a, want_a), (name, rows, cols, knobs)
@@ -1517,7 +1522,7 @@ def _multi(ws, x, stream=None):
 
 @pytest.mark.parametrize("case", ["qkv_4096", "gate_up_14336", "ragged_2304", "three_3584", "mixed_cut", "five", "q6k", "bands",
                                   "cut4_8192", "cut2_4096", "q8_0_qkv_4096", "q4_0_qkv_3584", "q8_0_ragged_2048", "q4_0_pair_8192",
-                                  "q4_0_gate_up_14336", "q8_0_tiny"])
+                                  "q4_0_gate_up_14336", "q8_0_tiny", "q6k_qkv_4096", "q6k_gate_up_14336", "q6k_mixed_cut", "q6k_qkv_3584"])
 def test_matmul_f32_multi_is_the_single_calls(case):
     """cml_matmul_f32_multi: several weights that read one token (q | k | v of an attention block, gate | up of an FFN).
     Runs of up to four Q4_K weights with one K cut go out as one launch -- the counters prove it -- and every
@@ -1541,8 +1546,12 @@ def test_matmul_f32_multi_is_the_single_calls(case):
         "q4_0_pair_8192": ([4096, 1030], 8192, 1),
         "q4_0_gate_up_14336": ([14336, 14336], 4096, 1),
         "q8_0_tiny": ([40, 24], 64, 1),
+        "q6k_qkv_4096": ([4096, 1030, 1024], 4096, 1),      # Q6_K sets with one K cut: one launch of the one-workgroup-per-unit form
+        "q6k_gate_up_14336": ([14336, 14336], 4096, 1),
+        "q6k_qkv_3584": ([3584, 512, 512], 3584, 1),
+        "q6k_mixed_cut": ([8192, 1024], 4096, 0),           # K cuts 2 and 4: two calls
     }[case]
-    if case == "q6k":
+    if case.startswith("q6k"):
         fmt = B.CML_Q6_K
     elif case.startswith("q8_0"):
         fmt = B.CML_Q8_0
@@ -1557,7 +1566,9 @@ def test_matmul_f32_multi_is_the_single_calls(case):
     G.say(f"multi {case}: single calls")
     want = [G.gpu_matmul_f32(w, x) for w in ws]
     G.say(f"multi {case}: one call")
-    if case == "q6k":
+    if fmt == B.CML_Q6_K and one_launch:
+        proof = G.engaged(r"^q6k\.dot\.wg8\.kcut\.fused\.multi$", none=(r"^quantize\.",))
+    elif fmt == B.CML_Q6_K:
         proof = G.engaged(r"^q6k\.dot\.", none=(r"multi",))
     elif fmt in (B.CML_Q8_0, B.CML_Q4_0):
         proof = G.engaged(r"^q[48]_0\.dot\.p\d+\.w8\.fused\.multi$", none=(r"^quantize\.",))
