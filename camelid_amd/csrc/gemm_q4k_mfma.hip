@@ -82,6 +82,9 @@ struct Q4KMfmaArgs {
     const uint8_t *w2;
     float *out2;
     int stage_once;  // rows that fit both activation buffers are staged in the prologue, once
+    // Staged-once mode: a workgroup walks every gridDim.x-th group of row tiles (of both weights of a pair launch,
+    // the second weight's groups following the first's) against the activation it staged, the weight ring running
+    // on across the group boundaries; blockIdx.z is then the group slot alone.
 };
 
 struct MfmaWeights {
@@ -90,11 +93,22 @@ struct MfmaWeights {
 };
 
 // hdr_ptr / piece_ptr already include the lane's offsets inside a tile entry; `off` = sb * sb_stride.
+// STREAM: non-temporal loads, for launches that read every weight byte once (staged-once mode: one token column
+// per weight, or per expert; the 32-token Mixtral-shaped layer 173 -> 165 us).  Launches with several token columns
+// read the weight once per column and want the later columns served by the caches (4096 x 14336, 64 tokens:
+// 30.8 us with plain loads, 32.4 non-temporal).
+template <bool STREAM = false>
 __device__ __forceinline__ void mfma_load_weights(MfmaWeights &r, const uint8_t *hdr_ptr, const uint8_t *piece_ptr,
                                                   int64_t off) {
-    r.hdr = ldg16(hdr_ptr + off);
-    r.piece[0] = ldg16(piece_ptr + off);
-    r.piece[1] = ldg16(piece_ptr + off + 32);
+    if constexpr (STREAM) {
+        r.hdr = ldg16_stream(hdr_ptr + off);
+        r.piece[0] = ldg16_stream(piece_ptr + off);
+        r.piece[1] = ldg16_stream(piece_ptr + off + 32);
+    } else {
+        r.hdr = ldg16(hdr_ptr + off);
+        r.piece[0] = ldg16(piece_ptr + off);
+        r.piece[1] = ldg16(piece_ptr + off + 32);
+    }
 }
 
 __device__ __forceinline__ v4i as_v4i(const uint4 &v) {
@@ -139,7 +153,7 @@ __device__ __forceinline__ int scale_bytes(uint32_t bytes, uint32_t digit2) {
     return __builtin_bit_cast(int, p);
 }
 
-template <int GPW, int TB, bool SPLIT, int KS = 1, bool PLAIN = false, bool ONCE = false>
+template <int GPW, int TB, bool SPLIT, int KS = 1, bool PLAIN = false, bool ONCE = false, int NSB = 0>
 __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
     static_assert(!(SPLIT && KS > 1), "K is split across waves or inside the lane, not both");
     constexpr int NTOK = 16 * GPW * TB;              // tokens staged per workgroup
@@ -161,6 +175,8 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
     // (staged-once mode with the whole row of 16 requested in the prologue: the 32-token expert layer 174 -> 179 us)
     constexpr int RING = (GPW == 1 && KS == 1) ? 8 : 4;
     static_assert(RING % KC == 0 && kPer >= 1 && RT >= 1, "phase / staging shape");
+    // NSB: the row length in super-blocks where the launcher knows it at compile time (staged-once mode; 0 = any)
+    static_assert(NSB == 0 || (ONCE && NSB % RING == 0 && NSB <= 2 * KC), "row length known at compile time: whole rounds of the ring");
     extern __shared__ uint4 smem[];
     uint8_t *buf0 = reinterpret_cast<uint8_t *>(smem);  // [KC][NTOK][kSlabRow], then [KC][NTOK][16] f16
     uint8_t *buf1 = buf0 + kBufBytes;
@@ -177,12 +193,20 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
     const int s_begin = KS > 1 ? ks * n_sb / KS : 0, s_end = KS > 1 ? (ks + 1) * n_sb / KS : n_sb;
     const int n_loc = s_end - s_begin, n_max = (n_sb + KS - 1) / KS;
     const int n_tiles = (a.rows + a.row_skip + 15) / 16;
-    const int tile = blockIdx.x * RT + rt;
-    const int row = tile * 16 + n - a.row_skip;
     const bool grouped = !PLAIN && a.group_offsets != nullptr;
     const bool pair = !PLAIN && a.w2 != nullptr;
-    const int zslot = pair ? static_cast<int>(blockIdx.z >> 1) : static_cast<int>(blockIdx.z);
-    const bool second = pair && (blockIdx.z & 1);
+    // Staged-once mode: this workgroup's units are u0, u0 + ustride, ... of the launch's list -- the groups of RT
+    // row tiles of the weight, then (pair launch) those of the second weight; strided by the grid, so that at any
+    // moment neighbouring workgroups read neighbouring tile entries and the launch sweeps the weight as one front.
+    // Otherwise one unit, and a pair launch keeps the weight in the low bit of blockIdx.z.
+    const int units_per_w = (n_tiles + RT - 1) / RT;
+    const int u0 = static_cast<int>(blockIdx.x), ustride = static_cast<int>(gridDim.x);
+    const int n_units = ONCE ? ((pair ? 2 * units_per_w : units_per_w) - 1 - u0) / ustride + 1 : 1;
+    const int zslot = (pair && !ONCE) ? static_cast<int>(blockIdx.z >> 1) : static_cast<int>(blockIdx.z);
+    // the unit being consumed: its weight, row tile and this lane's output row
+    bool second = ONCE ? (pair && u0 >= units_per_w) : (pair && (blockIdx.z & 1));
+    int tile = (u0 - (ONCE && second ? units_per_w : 0)) * RT + rt;
+    int row = tile * 16 + n - a.row_skip;
     const int64_t band = grouped ? (a.group_ids ? a.group_ids[zslot] : zslot) : 0;
     if (band < 0) return;  // a z-slot past the groups in use
     const int a0 = grouped ? a.group_offsets[band] : 0;                      // first assignment of this group
@@ -190,7 +214,11 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
     const int tok0 = blockIdx.y * NTOK;                    // first token (assignment of the group) of this workgroup
     if (tok0 >= n_assign) return;                          // nothing routed here: the whole workgroup leaves
     const int n_here = min(NTOK, n_assign - tok0);
-    const uint8_t *wtile = (second ? a.w2 : a.w) + (band * (a.rows / 16) + min(tile, n_tiles - 1)) * 2304;
+    // tile entry of super-block 0 of row tile `t` of this group's band (tiles past the end read the last one; their cells are not stored)
+    auto tile_entry = [&](bool of_second, int t) __attribute__((always_inline)) -> const uint8_t * {
+        return (of_second ? a.w2 : a.w) + (band * (a.rows / 16) + min(t, n_tiles - 1)) * 2304;
+    };
+    const uint8_t *wtile = tile_entry(second, tile);
     // activation row of local token t (tokens past the end repeat the last one; their cells are not stored)
     auto act_row = [&](int t) __attribute__((always_inline)) -> int64_t {
         const int j = a0 + tok0 + min(t, n_here - 1);
@@ -244,11 +272,14 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
     auto stage_store = [&](uint8_t *buf) __attribute__((always_inline)) { stage_store_from(sreg, buf); };
 
     // Lane constants.
-    const uint8_t *w_hdr = wtile + n * 16;
+    const int hdr_off = n * 16;
     // A matrix instruction contracts 64 values of ONE nibble plane of two 32-byte chunks, ch = 2 * q + half
     // (q = 0, 1): the lane needs piece a (values 0..15) or b (16..31) of those two chunks only, and the 64
     // lanes of a load cover 1024 distinct bytes of the tile entry.
-    const uint8_t *w_piece = wtile + ((kq & 1) ? 1280 : 256) + n * 64 + half * 16;
+    const int piece_off = ((kq & 1) ? 1280 : 256) + n * 64 + half * 16;
+    // (staged-once mode: the unit being REQUESTED, which runs ahead of the one being consumed)
+    const uint8_t *w_hdr = wtile + hdr_off;
+    const uint8_t *w_piece = wtile + piece_off;
     // A operand: this lane is token (lane & 15) of a group; step (q, plane) takes bytes 128q + 64half + 32plane + 16(kq&1) .. +15.
     const int a_off = (lane & 15) * kSlabRow + 64 * half + 16 * (kq & 1);  // + 128q + 32plane, + token-group and slot offsets
     // D values v = 0..3 of this lane: tokens 4*kq + v of the group, weight row n.
@@ -263,9 +294,27 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
     MfmaWeights ring[RING];
     // `loc` counts super-blocks inside this wave's part of K
     auto load_slot = [&](MfmaWeights &r, int loc) __attribute__((always_inline)) {
-        mfma_load_weights(r, w_hdr, w_piece, min(s_begin + loc, s_end - 1) * a.sb_stride);
+        mfma_load_weights<!PLAIN>(r, w_hdr, w_piece, min(s_begin + loc, s_end - 1) * a.sb_stride);
     };
-
+    // Staged-once mode: the next super-block of the walk over this workgroup's units.  The request itself is
+    // unconditional (past the end of the walk the last super-block is requested again: a cache hit, at most
+    // RING - 1 times per wave and only for walks that are no whole number of rounds), so the ring's loads stay
+    // straight-line code and the waits on them exact; only the bookkeeping, uniform over the wave, branches.
+    int pf_sb = 0, pf_unit = 0;
+    auto request_next = [&](MfmaWeights &r) __attribute__((always_inline)) {
+        mfma_load_weights<true>(r, w_hdr, w_piece, pf_sb * a.sb_stride);
+        if (pf_sb + 1 < n_sb) {
+            ++pf_sb;
+        } else if (pf_unit + 1 < n_units) {
+            pf_sb = 0;
+            ++pf_unit;
+            const int u = u0 + pf_unit * ustride;
+            const bool s2 = pair && u >= units_per_w;
+            const uint8_t *wt = tile_entry(s2, (u - (s2 ? units_per_w : 0)) * RT + rt);
+            w_hdr = wt + hdr_off;
+            w_piece = wt + piece_off;
+        }
+    };
     // ONCE (the launcher's choice for rows of up to 2 * KC super-blocks; one 16-token group per wave, no K parts): both buffers together hold the
     // whole activation, so it is staged ONCE -- no barrier in the middle of the walk (0.9 us per workgroup waiting
     // for its slowest wave, per-wave time stamps) and no re-read of clamped slabs in the last phase.  buf1 follows
@@ -273,19 +322,21 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
     static_assert(!ONCE || (GPW == 1 && KS == 1 && TB == 1), "staged-once mode: one token group per wave, no K parts");
     if constexpr (ONCE) {
         // (half of the weight ring is requested behind the activation, the other half once the staging registers are free)
-        StageRegs second;
+        StageRegs sreg2;
         stage_load(0);
-        stage_load_to(second, KC);
+        stage_load_to(sreg2, KC);
+        auto request_first = [&](MfmaWeights &r, int i) __attribute__((always_inline)) {
+            if constexpr (NSB > 0) mfma_load_weights<true>(r, w_hdr, w_piece, i * a.sb_stride);
+            else request_next(r);
+        };
 #pragma unroll
-        for (int i = 0; i < RING / 2; i++)
-            if (i < n_loc) load_slot(ring[i], i);
+        for (int i = 0; i < RING / 2; i++) request_first(ring[i], i);
         __builtin_amdgcn_sched_barrier(0);
         stage_store(buf0);
-        stage_store_from(second, buf1);
+        stage_store_from(sreg2, buf1);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int i = RING / 2; i < RING; i++)
-            if (i < n_loc) load_slot(ring[i], i);
+        for (int i = RING / 2; i < RING; i++) request_first(ring[i], i);
     } else {
         stage_load(0);
 #pragma unroll
@@ -442,28 +493,133 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
 #pragma unroll
         for (int i = 0; i < RING; i++) {
             const int loc = l0 + i;
-            if (i % KC == 0 && !ONCE) {
+            if (i % KC == 0) {
                 stage_load(loc + KC);
                 __builtin_amdgcn_sched_barrier(0);
             }
             if (loc < n_loc) step(ring[i], s_begin + loc, cur, ks * KC + i % KC);
             // many-token steps fill the register file on their own: keep the scheduler from
             // overlapping two of them (measured: it spills and loses more than it hides)
-            // (staged-once mode has no barrier between steps: without this fence the scheduler interleaves several
-            // steps and needs more registers than two waves per SIMD leave)
-            if constexpr (GPW > 1 || ONCE) __builtin_amdgcn_sched_barrier(0);
+            if constexpr (GPW > 1) __builtin_amdgcn_sched_barrier(0);
             if constexpr (decltype(refill)::value) load_slot(ring[i], loc + RING);
             if (i % KC == KC - 1) {
-                if constexpr (!ONCE) {
-                    stage_store(nxt);
-                    __syncthreads();  // next phase complete in `nxt`, everyone done with `cur`
-                }
+                stage_store(nxt);
+                __syncthreads();  // next phase complete in `nxt`, everyone done with `cur`
                 uint8_t *t = cur;
                 cur = nxt;
                 nxt = t;
             }
         }
     };
+    // the cells of the unit just walked: tokens cell_tok .. + 3 of each group, weight row `row`
+    auto store_cells = [&]() __attribute__((always_inline)) {
+        if (tile < n_tiles && row >= 0 && row < a.rows) {
+#pragma unroll
+            for (int g = 0; g < GPW; g++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const int t = tb * (16 * GPW) + 16 * g + cell_tok + j;
+                    if (t < n_here) {
+                        const float v = (part == 0) ? acc[g][j] : total[g][j] + acc[g][j];
+                        (second ? a.out2 : a.out)[static_cast<int64_t>(a0 + tok0 + t) * a.rows + row] = v;
+                    }
+                }
+        }
+    };
+    if constexpr (ONCE) {
+        // One walk over the super-blocks of all of this workgroup's units: the ring is refilled across the unit
+        // boundaries, so the activation is staged and the stream started once per workgroup, not once per unit.
+        // Slab s of the row sits in buf0 (s < KC) or buf1.
+        const int walk = n_units * n_sb;
+        int sb = 0, unit = 0;
+        // The chains advance inside their step: their only reader is the conditional store that closes a unit, and
+        // without this the compiler sinks the fused steps of a whole round into that block -- every step's integers
+        // stay live (spilled to the accumulation registers) and the dependent chains run where nothing overlaps them.
+        auto pin_chains = [&]() __attribute__((always_inline)) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) asm volatile("" : "+v"(acc[0][j]));
+        };
+        auto walk_step = [&](const MfmaWeights &w0) __attribute__((always_inline)) {
+            step(w0, sb, sb >= KC ? buf1 : buf0, sb >= KC ? sb - KC : sb);
+            pin_chains();
+            // (no barrier between steps here: without this fence the scheduler interleaves several steps
+            // and needs more registers than two waves per SIMD leave)
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        auto close_unit = [&]() __attribute__((always_inline)) {
+            if (++sb == n_sb) {  // the unit's rows are complete
+                store_cells();
+                sb = 0;
+                ++unit;
+                const int u = u0 + unit * ustride;
+                second = pair && u >= units_per_w;
+                tile = (u - (second ? units_per_w : 0)) * RT + rt;
+                row = tile * 16 + n - a.row_skip;
+                part = 0;
+                next_cut = a.ksplit <= 1 ? n_sb : n_sb / a.ksplit;
+#pragma unroll
+                for (int j = 0; j < 4; j++) acc[0][j] = total[0][j] = 0.0f;
+            }
+        };
+        if constexpr (NSB > 0) {
+            // Rows of NSB super-blocks: the walk of a unit is straight-line code (slab addresses and ring slots known
+            // at compile time); step s requests step s + RING, which for the last RING steps lies in the next unit.
+            for (int k = 0; k < n_units; ++k) {
+                auto fixed_step = [&](int s0) __attribute__((always_inline)) {
+                    step(ring[s0 % RING], s0, s0 >= KC ? buf1 : buf0, s0 % KC);
+                    pin_chains();
+                    __builtin_amdgcn_sched_barrier(0);
+                };
+#pragma unroll
+                for (int s0 = 0; s0 < NSB - RING; s0++) {
+                    fixed_step(s0);
+                    mfma_load_weights<true>(ring[s0 % RING], w_hdr, w_piece, (s0 + RING) * a.sb_stride);
+                }
+                // The last RING steps request the next unit's first super-blocks.  After the last unit the requests
+                // still go out -- every lane to the weight's first bytes, one cache line -- rather than sit in a
+                // branch of their own: two arms with the same steps are merged above the branch by the compiler,
+                // and with them the waits for all of the arm's ring slots (four steps' data awaited at once).
+                const bool more = k + 1 < n_units;
+                int64_t next_stride = 0;
+                if (more) {
+                    const int u = u0 + (k + 1) * ustride;
+                    const bool s2 = pair && u >= units_per_w;
+                    const uint8_t *wt = tile_entry(s2, (u - (s2 ? units_per_w : 0)) * RT + rt);
+                    w_hdr = wt + hdr_off;
+                    w_piece = wt + piece_off;
+                    next_stride = a.sb_stride;
+                } else {
+                    w_hdr = w_piece = a.w;
+                }
+#pragma unroll
+                for (int s0 = NSB - RING; s0 < NSB; s0++) {
+                    fixed_step(s0);
+                    mfma_load_weights<true>(ring[s0 % RING], w_hdr, w_piece, (s0 + RING - NSB) * next_stride);
+                }
+                sb = NSB - 1;
+                close_unit();
+            }
+            return;
+        }
+        // Every round but the last refills the ring, all of its steps lie inside the walk; the last one only drains it.
+        int l0 = 0;
+        for (; l0 + RING < walk; l0 += RING) {
+#pragma unroll
+            for (int i = 0; i < RING; i++) {
+                walk_step(ring[i]);
+                request_next(ring[i]);
+                close_unit();
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < RING; i++) {
+            if (l0 + i < walk) {
+                walk_step(ring[i]);
+                close_unit();
+            }
+        }
+        return;
+    }
     int l0 = 0;
     for (; l0 + RING < n_max; l0 += RING) round(l0, std::true_type{});
     round(l0, std::false_type{});
@@ -489,18 +645,7 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
             }
     }
 
-    if (tile < n_tiles && row >= 0 && row < a.rows) {
-#pragma unroll
-        for (int g = 0; g < GPW; g++)
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const int t = tb * (16 * GPW) + 16 * g + cell_tok + j;
-                if (t < n_here) {
-                    const float v = (part == 0) ? acc[g][j] : total[g][j] + acc[g][j];
-                    (second ? a.out2 : a.out)[static_cast<int64_t>(a0 + tok0 + t) * a.rows + row] = v;
-                }
-            }
-    }
+    store_cells();
 }
 
 int q4k_ksplit_for(int64_t rows, int64_t n_sb);  // gemv_q4k.hip: the matvec kernel's K-split policy
@@ -796,7 +941,9 @@ int launch_gemm_q4k_mfma_f32(const cml_weight *w, const float *x, int64_t n_toke
 
 // Counter name of a general-kernel instantiation: "q4k.mfma.tile" (one wave per row tile), ".ksplit<KS>" (K parts of a
 // tile on KS waves) or ".serial_split" (the K cut walked inside the lane), then the workgroup shape g<token groups per
-// wave>t<waves over tokens>, ".grouped" for expert-grouped calls and ".once" where the activation is staged once.
+// wave>t<waves over tokens>, ".grouped" for expert-grouped calls and ".once" where the activation is staged once
+// (then ".k<super-blocks per row>" where the walk knows the row length at compile time, ".units" where a workgroup
+// walks more than one group of row tiles).
 static std::string q4k_mfma_name(int gpw, int tb, bool split, int ks, bool plain, bool once) {
     std::string n = "q4k.mfma.";
     n += ks > 1 ? "ksplit" + std::to_string(ks) : (split ? "serial_split" : "tile");
@@ -804,6 +951,33 @@ static std::string q4k_mfma_name(int gpw, int tb, bool split, int ks, bool plain
     if (!plain) n += ".grouped";
     if (once) n += ".once";
     return n;
+}
+
+// Staged-once mode (one 16-token group per wave, rows of up to 16 super-blocks): a unit is four row tiles, a
+// workgroup walks every gridDim.x-th unit.  Units per workgroup: enough that the whole launch is resident at once,
+// two workgroups per compute unit (what the LDS lets a unit hold) -- the staging and the start of the stream are
+// paid once per workgroup's share of the weight, and there is no partly filled last round of workgroups (the
+// 32-token Mixtral-shaped layer, gate and up in one launch: 3584 workgroups of one unit 178 us per layer, 1792 of
+// two 170, 896 of four 178, 512 of seven 165).
+template <bool SPLIT, bool PLAIN, int NSB>
+static int launch_mfma_once(const Q4KMfmaArgs &ka, int n_tiles, int pair_f, int slots, unsigned gy, int64_t columns, size_t lds, hipStream_t st) {
+    static std::atomic<bool> raised{false};  // per instantiation: allow more than 64 KB of dynamic LDS once
+    if (!raised.load(std::memory_order_acquire)) {
+        CML_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_mfma_kernel<1, 1, SPLIT, 1, PLAIN, true, NSB>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        raised.store(true, std::memory_order_release);
+    }
+    const int64_t units_all = static_cast<int64_t>((n_tiles + 3) / 4) * pair_f;
+    int units = env_int("CAMELID_HIP_Q4K_MFMA_UNITS", 0);
+    if (units <= 0) units = static_cast<int>(std::min<int64_t>(16, std::max<int64_t>(1, (units_all * slots * columns + 511) / 512)));
+    units = static_cast<int>(std::min<int64_t>(units, units_all));
+    const unsigned gxu = static_cast<unsigned>((units_all + units - 1) / units);
+    hipLaunchKernelGGL((gemm_q4k_mfma_kernel<1, 1, SPLIT, 1, PLAIN, true, NSB>), dim3(gxu, gy, slots), dim3(256), lds, st, ka);
+    // (a counter's name is built once per site: one site per name)
+    if (units > 1) CML_COUNT_LAUNCH(q4k_mfma_name(1, 1, SPLIT, 1, PLAIN, true) + (NSB ? ".k" + std::to_string(NSB) : "") + ".units");
+    else CML_COUNT_LAUNCH(q4k_mfma_name(1, 1, SPLIT, 1, PLAIN, true) + (NSB ? ".k" + std::to_string(NSB) : ""));
+    CML_HIP_TRY(hipGetLastError());
+    return CML_OK;
 }
 
 template <int GPW, int TB, bool SPLIT, int KS = 1, bool PLAIN = false>
@@ -818,16 +992,13 @@ static int launch_mfma_split(const Q4KMfmaArgs &ka, int n_groups, hipStream_t st
     if constexpr (GPW == 1 && TB == 1 && KS == 1) {
         if (ka.n_sb <= 2 * KC && ka.stage_once) {  // the whole activation fits the two buffers: staged once
             const size_t lds_once = lds + 2 * static_cast<size_t>(KC * NTOK) * 32;  // + the run sums
-            static std::atomic<bool> raised_once{false};
-            if (!raised_once.load(std::memory_order_acquire)) {
-                CML_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_mfma_kernel<GPW, TB, SPLIT, KS, PLAIN, true>),
-                                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-                raised_once.store(true, std::memory_order_release);
-            }
-            hipLaunchKernelGGL((gemm_q4k_mfma_kernel<GPW, TB, SPLIT, KS, PLAIN, true>), dim3(gx, gy, n_groups), dim3(256), lds_once, st, ka);
-            CML_COUNT_LAUNCH(q4k_mfma_name(GPW, TB, SPLIT, KS, PLAIN, true));
-            CML_HIP_TRY(hipGetLastError());
-            return CML_OK;
+            const int pair_f = ka.w2 ? 2 : 1, slots = n_groups / pair_f;
+            const int64_t columns = ka.group_offsets ? 1 : gy;  // (a grouped call counts one token column per group: the others leave at once)
+            // rows of 2048 or 4096 values: the walk of a unit as straight-line code
+            const bool fixed = env_int("CAMELID_HIP_Q4K_MFMA_FIXED_ROWS", 1);
+            if (fixed && ka.n_sb == 16) return launch_mfma_once<SPLIT, PLAIN, 16>(ka, n_tiles, pair_f, slots, gy, columns, lds_once, st);
+            if (fixed && ka.n_sb == 8) return launch_mfma_once<SPLIT, PLAIN, 8>(ka, n_tiles, pair_f, slots, gy, columns, lds_once, st);
+            return launch_mfma_once<SPLIT, PLAIN, 0>(ka, n_tiles, pair_f, slots, gy, columns, lds_once, st);
         }
     }
     static std::atomic<bool> raised{false};  // per instantiation: allow more than 64 KB of dynamic LDS once

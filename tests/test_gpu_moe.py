@@ -383,6 +383,45 @@ def test_moe_gate_and_up_in_one_launch_give_the_bits_of_two(E, k, hidden, ff, T)
     assert G.same_bits(one, two)
 
 
+@pytest.mark.parametrize("E,k,hidden,ff,T", [(8, 2, 4096, 1024, 40), (8, 2, 2048, 2048, 16), (8, 3, 3072, 2048, 33), (8, 2, 4096, 2048, 9)])
+def test_moe_staged_once_walks_of_several_units_give_the_bits_of_one_unit_each(E, k, hidden, ff, T):
+    """The expert-grouped matrix-core launch on rows of up to 16 super-blocks stages the activation once per
+    workgroup and walks several groups of row tiles against it (gate and up in one list, the ring refilled
+    across the group boundaries); rows of 2048 and 4096 values take the walk with the row length known at
+    compile time.  Every shape of that launch -- one unit per workgroup, three, the launcher's own choice, the
+    general walk, the phased staging -- gives the same bits, and so do gate and up as two launches."""
+    gate, up, down = _experts(E, hidden, ff, 1170 + E)
+    wg = Weight.upload(B.CML_Q4_K, E * ff, hidden, gate)
+    wu = Weight.upload(B.CML_Q4_K, E * ff, hidden, up)
+    wd = Weight.upload(B.CML_Q4_K, E * hidden, ff, down)
+    rng = np.random.default_rng(1171 + T)
+    x = rng.standard_normal((T, hidden)).astype(np.float32)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    logits[:, 1] -= 50.0    # an expert nobody routes to
+    idx_dev, w_dev, _, _ = gpu_route(logits, k)
+    fixed = {4096: r"\.k16", 2048: r"\.k8"}.get(hidden)
+    G.say(f"moe staged-once unit walk, E={E} k={k} {hidden}x{ff} T={T}")
+    with G.env(CAMELID_HIP_TUNING=1, CAMELID_HIP_Q4K_MFMA_UNITS=1), G.engaged(r"^q4k\.mfma\.(tile|serial_split)\.g1t1\.grouped\.once", none=(r"\.units$",)):
+        one = gpu_moe(wg, wu, wd, E, k, idx_dev, w_dev, x)
+    assert np.isfinite(one).all()
+    with G.env(CAMELID_HIP_TUNING=1, CAMELID_HIP_Q4K_MFMA_UNITS=3), G.engaged(r"^q4k\.mfma\.(tile|serial_split)\.g1t1\.grouped\.once.*\.units$"):
+        three = gpu_moe(wg, wu, wd, E, k, idx_dev, w_dev, x)
+    assert G.same_bits(one, three)
+    with G.engaged(r"^q4k\.mfma\.(tile|serial_split)\.g1t1\.grouped\.once" + (fixed or "")):
+        auto = gpu_moe(wg, wu, wd, E, k, idx_dev, w_dev, x)
+    assert G.same_bits(one, auto)
+    with G.env(CAMELID_HIP_TUNING=1, CAMELID_HIP_Q4K_MFMA_FIXED_ROWS=0, CAMELID_HIP_Q4K_MFMA_UNITS=5), \
+            G.engaged(r"^q4k\.mfma\.(tile|serial_split)\.g1t1\.grouped\.once\.units$"):
+        general = gpu_moe(wg, wu, wd, E, k, idx_dev, w_dev, x)
+    assert G.same_bits(one, general)
+    with G.env(CAMELID_HIP_MOE_PAIR_LAUNCH=0):
+        two = gpu_moe(wg, wu, wd, E, k, idx_dev, w_dev, x)
+    assert G.same_bits(one, two)
+    with G.env(CAMELID_HIP_TUNING=1, CAMELID_HIP_Q4K_MFMA_STAGE_ONCE=0), G.engaged(r"^q4k\.mfma\.(tile|serial_split)\.g1t1\.grouped$"):
+        phased = gpu_moe(wg, wu, wd, E, k, idx_dev, w_dev, x)
+    assert G.same_bits(one, phased)
+
+
 @pytest.mark.parametrize("T", [1, 32])
 def test_c5_mixtral_shaped_moe(T):
     """8 experts, gate/up 14336x4096 and down 4096x14336 in Q4_K, top-2 routing."""

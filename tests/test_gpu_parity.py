@@ -1101,7 +1101,7 @@ def test_q4k_matrix_core_cells_are_bitwise_the_gemv(rows, cols):
         check_outputs(fmt, wire, cols, s, q, got, expect_exact=True)
 
 
-@pytest.mark.parametrize("rows,cols", [(200, 2 * 256), (75, 7 * 256), (1000, 15 * 256), (14336, 4096), (97, 4096)])
+@pytest.mark.parametrize("rows,cols", [(200, 2 * 256), (75, 7 * 256), (1000, 15 * 256), (14336, 4096), (97, 4096), (300, 8 * 256)])
 def test_q4k_two_waves_per_tile_keep_one_chain(rows, cols):
     """Up to 16 tokens against rows of 2..16 super-blocks with no K cut: two waves share a row tile
     and split K, the chain stays one chain -- the oracle's order bit for bit, the same bits as one
@@ -1122,9 +1122,21 @@ def test_q4k_two_waves_per_tile_keep_one_chain(rows, cols):
                 got_band = G.gpu_gemm(band, s, q)
             with G.env(CAMELID_HIP_EXACT_ORDER="1", CAMELID_HIP_Q4K_MFMA_PAIR=0), G.engaged(r"^q4k\.mfma\.tile\.g1t1", none=(r"^q4k\.mfma\.pair", r"^q4k\.dot\.")):
                 one_wave = G.gpu_gemm(w, s, q)
+            # one wave per tile walking three groups of row tiles per workgroup (a last group partly past the end of
+            # the weight, a band that starts inside a tile), with the row length known at compile time or not
+            with G.env(CAMELID_HIP_EXACT_ORDER="1", CAMELID_HIP_Q4K_MFMA_PAIR=0, CAMELID_HIP_Q4K_MFMA_UNITS=3), \
+                    G.engaged(r"^q4k\.mfma\.tile\.g1t1\.once.*\.units$" if rows > 64 else r"^q4k\.mfma\.tile\.g1t1\.once"):
+                walk = G.gpu_gemm(w, s, q)
+                walk_band = G.gpu_gemm(band, s, q)
+            with G.env(CAMELID_HIP_EXACT_ORDER="1", CAMELID_HIP_Q4K_MFMA_PAIR=0, CAMELID_HIP_Q4K_MFMA_UNITS=2, CAMELID_HIP_Q4K_MFMA_FIXED_ROWS=0), \
+                    G.engaged(r"^q4k\.mfma\.tile\.g1t1\.once", none=(r"\.k(8|16)",)):
+                walk_any = G.gpu_gemm(w, s, q)
         assert G.same_bits(got, want)
         assert G.same_bits(got, one_wave)
         assert G.same_bits(got_band, want[:, 5:rows - 4])
+        assert G.same_bits(walk, want)
+        assert G.same_bits(walk_band, want[:, 5:rows - 4])
+        assert G.same_bits(walk_any, want)
 
 
 @pytest.mark.parametrize("name,fmt", [("Q8_0", oracle.Q8_0), ("Q4_0", oracle.Q4_0)])
