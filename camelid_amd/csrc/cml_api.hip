@@ -876,7 +876,13 @@ int cml_matmul_f32(const cml_weight *w, const float *x_dev, int64_t n_tokens, fl
         if (frc == CML_OK) g_runs.fetch_add(1, std::memory_order_relaxed);
         return frc;
     }
-    if (w->fmt == CML_Q4_K && !q4k_lane_order() && (n_tokens == 3 || n_tokens == 4) && fuse != 0 &&
+    // (not on a vocabulary-sized weight: there the matrix-core kernel that walks the weight with one resident
+    // workgroup per compute unit takes 55 us for 3 to 8 tokens at 128256 x 4096, quantizing launch included,
+    // against 58 / 68 us here for 3 / 4; at 24576 x 4096 this launch is ahead, 11.9 against 17 us for 3)
+    const int64_t q4k_sbs = w->rows * w->nb;
+    const bool tall_for_tokens = w->nb <= 16 && q4k_sbs >= (n_tokens == 4 ? int64_t(49152) * 16 : int64_t(98304) * 16) &&
+                                 env_int("CAMELID_HIP_Q4K_TALL_TOKENS_MFMA", 1);
+    if (w->fmt == CML_Q4_K && !q4k_lane_order() && (n_tokens == 3 || n_tokens == 4) && fuse != 0 && !tall_for_tokens &&
         (w->nb <= 32 || gemv_q4k_long_rows_fuse(w, static_cast<int>(n_tokens))) && !env_int("CAMELID_HIP_Q4K_GENERAL_ENTRY", 0)) {
         // three or four tokens on rows of 4096 values with no K cut: the eight-wave packed-dot launch replays each
         // step's unpacked weight against the tokens (one launch, quantizer inside); -1 = not such a shape

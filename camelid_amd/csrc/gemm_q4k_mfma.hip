@@ -916,9 +916,14 @@ static int launch_mfma_pair(const Q4KMfmaArgs &ka, const float *x, hipStream_t s
 }
 
 // Which plain calls the pair kernel serves: one column of up to 16 tokens against rows of 2..16
-// super-blocks that the shape policy does not cut.
+// super-blocks that the shape policy does not cut, on weights of up to 16384 rows -- about one of its workgroups
+// per compute unit.  A taller weight queues several of them per unit, each staging the whole activation again and
+// filling its ring from nothing; there the staged-once kernel walks the weight with one resident workgroup per
+// unit (16 tokens, us per step: 24576 x 4096 20.7 -> 17.5, 32000 x 4096 22.4 -> 19.0, 65536 x 4096 41.2 -> 31.5,
+// 128256 x 4096 76.4 -> 59.0, 128256 x 2048 51.6 -> 33.5, 151936 x 3584 82.8 -> 71.9; 14336 x 4096 12.4 either way).
 static bool mfma_pair_serves(int64_t rows, int64_t n_sb, int64_t n_tokens) {
     return n_tokens <= 16 && n_sb <= kPairSb && n_sb >= 2 && q4k_ksplit_for(rows, n_sb) == 1 &&
+           rows <= env_int("CAMELID_HIP_Q4K_MFMA_PAIR_MAX_ROWS", 16384) &&
            env_int("CAMELID_HIP_Q4K_MFMA_SHAPE", 0) == 0 && env_int("CAMELID_HIP_Q4K_MFMA_PAIR", 1);
 }
 
@@ -969,7 +974,15 @@ static int launch_mfma_once(const Q4KMfmaArgs &ka, int n_tiles, int pair_f, int 
     }
     const int64_t units_all = static_cast<int64_t>((n_tiles + 3) / 4) * pair_f;
     int units = env_int("CAMELID_HIP_Q4K_MFMA_UNITS", 0);
-    if (units <= 0) units = static_cast<int>(std::min<int64_t>(16, std::max<int64_t>(1, (units_all * slots * columns + 511) / 512)));
+    if (units <= 0) {
+        // expert groups: two workgroups per compute unit; a plain call: one (128256 x 4096, 16 tokens, 2004 units:
+        // 1 / 2 / 4 / 8 / 16 per workgroup 68.5 / 64.8 / 61.4 / 59.0 / 89.6 us; 65536 x 4096: 35.3 / 33.3 / 31.5 / 47.7 / 85.6)
+        const int64_t resident = ka.group_offsets ? 512 : 256;
+        units = static_cast<int>(std::min<int64_t>(16, std::max<int64_t>(1, (units_all * slots * columns + resident - 1) / resident)));
+        // the walk that does not know the row length at compile time pays for its bookkeeping beyond two units
+        // (151936 x 3584, 16 tokens: 75.2 / 71.9 / 74.2 / 88.7 us for 1 / 2 / 4 / 8)
+        if (NSB == 0 && !ka.group_offsets) units = std::min(units, 2);
+    }
     units = static_cast<int>(std::min<int64_t>(units, units_all));
     const unsigned gxu = static_cast<unsigned>((units_all + units - 1) / units);
     hipLaunchKernelGGL((gemm_q4k_mfma_kernel<1, 1, SPLIT, 1, PLAIN, true, NSB>), dim3(gxu, gy, slots), dim3(256), lds, st, ka);
