@@ -294,7 +294,7 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
     MfmaWeights ring[RING];
     // `loc` counts super-blocks inside this wave's part of K
     auto load_slot = [&](MfmaWeights &r, int loc) __attribute__((always_inline)) {
-        mfma_load_weights<!PLAIN>(r, w_hdr, w_piece, min(s_begin + loc, s_end - 1) * a.sb_stride);
+        mfma_load_weights<false>(r, w_hdr, w_piece, min(s_begin + loc, s_end - 1) * a.sb_stride);
     };
     // Staged-once mode: the next super-block of the walk over this workgroup's units.  The request itself is
     // unconditional (past the end of the walk the last super-block is requested again: a cache hit, at most
