@@ -361,6 +361,8 @@ MOE_CONFIGS = {
     # Mixtral-8x7B-shaped expert FFN in Q4_K: separate gate / up tensors, top-k softmax routing, silu
     "moe_q4k_8x14336x4096_t1": ("mixtral", "Q4_K", 8, 2, 4096, 14336, 1),
     "moe_q4k_8x14336x4096_t32": ("mixtral", "Q4_K", 8, 2, 4096, 14336, 32),
+    "moe_q4k_8x14336x4096_t64": ("mixtral", "Q4_K", 8, 2, 4096, 14336, 64),   # short prefill: 16 assignments per expert on average
+    "moe_q4k_8x14336x4096_t128": ("mixtral", "Q4_K", 8, 2, 4096, 14336, 128),
     # Gemma-4 26B-shaped expert lane in Q4_0: fused gate|up tensor, full-softmax routing with
     # per-expert down scales, gelu_tanh
     "moe_q4_0_128x704x2816_t1": ("gemma4", "Q4_0", 128, 8, 2816, 704, 1),

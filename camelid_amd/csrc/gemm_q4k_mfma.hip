@@ -173,14 +173,17 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
     // weight super-blocks a wave keeps in flight (register ring): a 16-token step is short, so it
     // takes 8 to cover the HBM latency; steps over more tokens are longer and 4 are enough
     // (staged-once mode with the whole row of 16 requested in the prologue: the 32-token expert layer 174 -> 179 us)
-    constexpr int RING = (GPW == 1 && KS == 1) ? 8 : 4;
-    static_assert(RING % KC == 0 && kPer >= 1 && RT >= 1, "phase / staging shape");
+    // (staged-once mode with two token groups per wave: one workgroup per compute unit, one wave per SIMD -- eight slots fit)
+    constexpr int RING = ((GPW == 1 && KS == 1) || ONCE) ? 8 : 4;
+    static_assert((ONCE || RING % KC == 0) && kPer >= 1 && RT >= 1, "phase / staging shape");
+    // staged-once mode holds a row of up to 16 super-blocks as kOnceChunks chunks of KC slabs, each laid out like a phase buffer
+    constexpr int kOnceChunks = 16 / KC;
     // NSB: the row length in super-blocks where the launcher knows it at compile time (staged-once mode; 0 = any)
-    static_assert(NSB == 0 || (ONCE && NSB % RING == 0 && NSB <= 2 * KC), "row length known at compile time: whole rounds of the ring");
+    static_assert(NSB == 0 || (ONCE && NSB % RING == 0 && NSB <= 16), "row length known at compile time: whole rounds of the ring");
     extern __shared__ uint4 smem[];
     uint8_t *buf0 = reinterpret_cast<uint8_t *>(smem);  // [KC][NTOK][kSlabRow], then [KC][NTOK][16] f16
     uint8_t *buf1 = buf0 + kBufBytes;
-    float *yds = reinterpret_cast<float *>(buf1 + kBufBytes);  // [n_sb][NTOK]
+    float *yds = reinterpret_cast<float *>(buf0 + (ONCE ? kOnceChunks : 2) * kBufBytes);  // [n_sb][NTOK]
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
@@ -315,13 +318,13 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
             w_piece = wt + piece_off;
         }
     };
-    // ONCE (the launcher's choice for rows of up to 2 * KC super-blocks; one 16-token group per wave, no K parts): both buffers together hold the
+    // ONCE (the launcher's choice for rows of up to 16 super-blocks; one or two 16-token groups per wave, no K parts): the LDS holds the
     // whole activation, so it is staged ONCE -- no barrier in the middle of the walk (0.9 us per workgroup waiting
-    // for its slowest wave, per-wave time stamps) and no re-read of clamped slabs in the last phase.  buf1 follows
-    // buf0, so slab s of the row sits where phase s / KC would have put it.
-    static_assert(!ONCE || (GPW == 1 && KS == 1 && TB == 1), "staged-once mode: one token group per wave, no K parts");
+    // for its slowest wave, per-wave time stamps) and no re-read of clamped slabs in the last phase.  The chunks of
+    // KC slabs follow one another, so slab s of the row sits where phase s / KC would have put it.
+    static_assert(!ONCE || (GPW <= 2 && KS == 1 && TB == 1), "staged-once mode: one or two token groups per wave, no K parts");
     if constexpr (ONCE) {
-        // (half of the weight ring is requested behind the activation, the other half once the staging registers are free)
+        // (half of the weight ring is requested behind the first two chunks of the activation, the other half once the staging registers are free)
         StageRegs sreg2;
         stage_load(0);
         stage_load_to(sreg2, KC);
@@ -337,6 +340,16 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int i = RING / 2; i < RING; i++) request_first(ring[i], i);
+        // the chunks past the first two (32 tokens: chunks of four slabs), where the row has them
+#pragma unroll
+        for (int c = 2; c < kOnceChunks; c += 2) {
+            if (c * KC < n_sb) {
+                stage_load(c * KC);
+                stage_load_to(sreg2, (c + 1) * KC);
+                stage_store(buf0 + c * kBufBytes);
+                stage_store_from(sreg2, buf0 + (c + 1) * kBufBytes);
+            }
+        }
     } else {
         stage_load(0);
 #pragma unroll
@@ -529,7 +542,7 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
     if constexpr (ONCE) {
         // One walk over the super-blocks of all of this workgroup's units: the ring is refilled across the unit
         // boundaries, so the activation is staged and the stream started once per workgroup, not once per unit.
-        // Slab s of the row sits in buf0 (s < KC) or buf1.
+        // Slab s of the row sits in chunk s / KC.
         const int walk = n_units * n_sb;
         int sb = 0, unit = 0;
         // The chains advance inside their step: their only reader is the conditional store that closes a unit, and
@@ -537,10 +550,12 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
         // stay live (spilled to the accumulation registers) and the dependent chains run where nothing overlaps them.
         auto pin_chains = [&]() __attribute__((always_inline)) {
 #pragma unroll
-            for (int j = 0; j < 4; j++) asm volatile("" : "+v"(acc[0][j]));
+            for (int g = 0; g < GPW; g++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) asm volatile("" : "+v"(acc[g][j]));
         };
         auto walk_step = [&](const MfmaWeights &w0) __attribute__((always_inline)) {
-            step(w0, sb, sb >= KC ? buf1 : buf0, sb >= KC ? sb - KC : sb);
+            step(w0, sb, buf0 + (sb / KC) * kBufBytes, sb % KC);
             pin_chains();
             // (no barrier between steps here: without this fence the scheduler interleaves several steps
             // and needs more registers than two waves per SIMD leave)
@@ -558,7 +573,9 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
                 part = 0;
                 next_cut = a.ksplit <= 1 ? n_sb : n_sb / a.ksplit;
 #pragma unroll
-                for (int j = 0; j < 4; j++) acc[0][j] = total[0][j] = 0.0f;
+                for (int g = 0; g < GPW; g++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++) acc[g][j] = total[g][j] = 0.0f;
             }
         };
         if constexpr (NSB > 0) {
@@ -566,7 +583,7 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
             // at compile time); step s requests step s + RING, which for the last RING steps lies in the next unit.
             for (int k = 0; k < n_units; ++k) {
                 auto fixed_step = [&](int s0) __attribute__((always_inline)) {
-                    step(ring[s0 % RING], s0, s0 >= KC ? buf1 : buf0, s0 % KC);
+                    step(ring[s0 % RING], s0, buf0 + (s0 / KC) * kBufBytes, s0 % KC);
                     pin_chains();
                     __builtin_amdgcn_sched_barrier(0);
                 };
@@ -964,11 +981,11 @@ static std::string q4k_mfma_name(int gpw, int tb, bool split, int ks, bool plain
 // paid once per workgroup's share of the weight, and there is no partly filled last round of workgroups (the
 // 32-token Mixtral-shaped layer, gate and up in one launch: 3584 workgroups of one unit 178 us per layer, 1792 of
 // two 170, 896 of four 178, 512 of seven 165).
-template <bool SPLIT, bool PLAIN, int NSB>
+template <bool SPLIT, bool PLAIN, int NSB, int GPW = 1>
 static int launch_mfma_once(const Q4KMfmaArgs &ka, int n_tiles, int pair_f, int slots, unsigned gy, int64_t columns, size_t lds, hipStream_t st) {
     static std::atomic<bool> raised{false};  // per instantiation: allow more than 64 KB of dynamic LDS once
     if (!raised.load(std::memory_order_acquire)) {
-        CML_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_mfma_kernel<1, 1, SPLIT, 1, PLAIN, true, NSB>),
+        CML_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_mfma_kernel<GPW, 1, SPLIT, 1, PLAIN, true, NSB>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
         raised.store(true, std::memory_order_release);
     }
@@ -977,7 +994,8 @@ static int launch_mfma_once(const Q4KMfmaArgs &ka, int n_tiles, int pair_f, int 
     if (units <= 0) {
         // expert groups: two workgroups per compute unit; a plain call: one (128256 x 4096, 16 tokens, 2004 units:
         // 1 / 2 / 4 / 8 / 16 per workgroup 68.5 / 64.8 / 61.4 / 59.0 / 89.6 us; 65536 x 4096: 35.3 / 33.3 / 31.5 / 47.7 / 85.6)
-        const int64_t resident = ka.group_offsets ? 512 : 256;
+        // (two token groups per wave fill a compute unit's LDS with one workgroup)
+        const int64_t resident = (ka.group_offsets && GPW == 1) ? 512 : 256;
         units = static_cast<int>(std::min<int64_t>(16, std::max<int64_t>(1, (units_all * slots * columns + resident - 1) / resident)));
         // the walk that does not know the row length at compile time pays for its bookkeeping beyond two units
         // (151936 x 3584, 16 tokens: 75.2 / 71.9 / 74.2 / 88.7 us for 1 / 2 / 4 / 8)
@@ -985,10 +1003,10 @@ static int launch_mfma_once(const Q4KMfmaArgs &ka, int n_tiles, int pair_f, int 
     }
     units = static_cast<int>(std::min<int64_t>(units, units_all));
     const unsigned gxu = static_cast<unsigned>((units_all + units - 1) / units);
-    hipLaunchKernelGGL((gemm_q4k_mfma_kernel<1, 1, SPLIT, 1, PLAIN, true, NSB>), dim3(gxu, gy, slots), dim3(256), lds, st, ka);
+    hipLaunchKernelGGL((gemm_q4k_mfma_kernel<GPW, 1, SPLIT, 1, PLAIN, true, NSB>), dim3(gxu, gy, slots), dim3(256), lds, st, ka);
     // (a counter's name is built once per site: one site per name)
-    if (units > 1) CML_COUNT_LAUNCH(q4k_mfma_name(1, 1, SPLIT, 1, PLAIN, true) + (NSB ? ".k" + std::to_string(NSB) : "") + ".units");
-    else CML_COUNT_LAUNCH(q4k_mfma_name(1, 1, SPLIT, 1, PLAIN, true) + (NSB ? ".k" + std::to_string(NSB) : ""));
+    if (units > 1) CML_COUNT_LAUNCH(q4k_mfma_name(GPW, 1, SPLIT, 1, PLAIN, true) + (NSB ? ".k" + std::to_string(NSB) : "") + ".units");
+    else CML_COUNT_LAUNCH(q4k_mfma_name(GPW, 1, SPLIT, 1, PLAIN, true) + (NSB ? ".k" + std::to_string(NSB) : ""));
     CML_HIP_TRY(hipGetLastError());
     return CML_OK;
 }
@@ -1002,16 +1020,20 @@ static int launch_mfma_split(const Q4KMfmaArgs &ka, int n_groups, hipStream_t st
     const unsigned gy = static_cast<unsigned>((ka.n_tokens + NTOK - 1) / NTOK);
     const size_t lds = 2 * static_cast<size_t>(KS * KC * NTOK) * (kSlabRow + ((GPW == 2 && KS == 1) ? 32 : 0)) + static_cast<size_t>(ka.n_sb) * NTOK * 4;
     if (lds > 160 * 1024) return fail(CML_ERR_UNSUPPORTED, "Q4_K matrix-core path: %d super-blocks exceed the LDS budget", ka.n_sb);
-    if constexpr (GPW == 1 && TB == 1 && KS == 1) {
-        if (ka.n_sb <= 2 * KC && ka.stage_once) {  // the whole activation fits the two buffers: staged once
-            const size_t lds_once = lds + 2 * static_cast<size_t>(KC * NTOK) * 32;  // + the run sums
+    if constexpr ((GPW == 1 || GPW == 2) && TB == 1 && KS == 1) {
+        // Rows of up to 16 super-blocks: the whole activation fits the LDS and is staged once.  One token group per
+        // wave: always.  Two (17 to 32 tokens; 155 KB, one workgroup per compute unit): expert groups, and plain calls
+        // on weights of more than 16384 rows, where the launch walks the weight with resident workgroups.
+        const bool two_groups_pay = ka.group_offsets != nullptr || n_tiles > 1024;
+        if (ka.n_sb <= 16 && ka.stage_once && (GPW == 1 || (two_groups_pay && env_int("CAMELID_HIP_Q4K_MFMA_ONCE_TWO_GROUPS", 1)))) {
+            const size_t lds_once = static_cast<size_t>(16) * NTOK * (kSlabRow + 32) + static_cast<size_t>(ka.n_sb) * NTOK * 4;  // slabs + run sums, scales
             const int pair_f = ka.w2 ? 2 : 1, slots = n_groups / pair_f;
             const int64_t columns = ka.group_offsets ? 1 : gy;  // (a grouped call counts one token column per group: the others leave at once)
             // rows of 2048 or 4096 values: the walk of a unit as straight-line code
             const bool fixed = env_int("CAMELID_HIP_Q4K_MFMA_FIXED_ROWS", 1);
-            if (fixed && ka.n_sb == 16) return launch_mfma_once<SPLIT, PLAIN, 16>(ka, n_tiles, pair_f, slots, gy, columns, lds_once, st);
-            if (fixed && ka.n_sb == 8) return launch_mfma_once<SPLIT, PLAIN, 8>(ka, n_tiles, pair_f, slots, gy, columns, lds_once, st);
-            return launch_mfma_once<SPLIT, PLAIN, 0>(ka, n_tiles, pair_f, slots, gy, columns, lds_once, st);
+            if (fixed && ka.n_sb == 16) return launch_mfma_once<SPLIT, PLAIN, 16, GPW>(ka, n_tiles, pair_f, slots, gy, columns, lds_once, st);
+            if (fixed && ka.n_sb == 8) return launch_mfma_once<SPLIT, PLAIN, 8, GPW>(ka, n_tiles, pair_f, slots, gy, columns, lds_once, st);
+            return launch_mfma_once<SPLIT, PLAIN, 0, GPW>(ka, n_tiles, pair_f, slots, gy, columns, lds_once, st);
         }
     }
     static std::atomic<bool> raised{false};  // per instantiation: allow more than 64 KB of dynamic LDS once
@@ -1097,7 +1119,14 @@ int launch_gemm_q4k_mfma(const MatArgs &a, hipStream_t st) {
         case 6: return launch_mfma<1, 4>(ka, ng, st);   // 64 tokens, 4 waves per row tile
         default: break;
     }
-    if (grouped) return launch_mfma<1, 1>(ka, ng, st);  // assignments per expert are few and uneven: the smallest tile wastes least
+    if (grouped) {
+        // assignments per expert are few and uneven: the smallest tile wastes least -- until most experts hold more
+        // than 16 and a second token column would read their weights a second time
+        const int slots = std::max(1, ng / (a.w2 ? 2 : 1));
+        if (ka.n_sb <= 16 && a.n_tokens > 16 && a.n_assign_total > 12 * static_cast<int64_t>(slots) && env_int("CAMELID_HIP_Q4K_MFMA_ONCE_TWO_GROUPS", 1))
+            return launch_mfma<2, 1>(ka, ng, st);
+        return launch_mfma<1, 1>(ka, ng, st);
+    }
     if (a.n_tokens > 32) return launch_mfma<4, 1>(ka, ng, st);
     if (a.n_tokens > 16) return launch_mfma<2, 1>(ka, ng, st);
     return launch_mfma<1, 1>(ka, ng, st);

@@ -383,7 +383,7 @@ def test_moe_gate_and_up_in_one_launch_give_the_bits_of_two(E, k, hidden, ff, T)
     assert G.same_bits(one, two)
 
 
-@pytest.mark.parametrize("E,k,hidden,ff,T", [(8, 2, 4096, 1024, 40), (8, 2, 2048, 2048, 16), (8, 3, 3072, 2048, 33), (8, 2, 4096, 2048, 9)])
+@pytest.mark.parametrize("E,k,hidden,ff,T", [(8, 2, 4096, 1024, 40), (8, 2, 2048, 2048, 16), (8, 3, 3072, 2048, 30), (8, 2, 4096, 2048, 9)])
 def test_moe_staged_once_walks_of_several_units_give_the_bits_of_one_unit_each(E, k, hidden, ff, T):
     """The expert-grouped matrix-core launch on rows of up to 16 super-blocks stages the activation once per
     workgroup and walks several groups of row tiles against it (gate and up in one list, the ring refilled
@@ -420,6 +420,37 @@ def test_moe_staged_once_walks_of_several_units_give_the_bits_of_one_unit_each(E
     with G.env(CAMELID_HIP_TUNING=1, CAMELID_HIP_Q4K_MFMA_STAGE_ONCE=0), G.engaged(r"^q4k\.mfma\.(tile|serial_split)\.g1t1\.grouped$"):
         phased = gpu_moe(wg, wu, wd, E, k, idx_dev, w_dev, x)
     assert G.same_bits(one, phased)
+
+
+@pytest.mark.parametrize("E,k,hidden,ff,T", [(8, 2, 4096, 1024, 64), (4, 2, 2048, 2048, 70), (8, 3, 3072, 2048, 40)])
+def test_moe_experts_with_more_than_16_assignments_take_two_token_groups_per_wave(E, k, hidden, ff, T):
+    """Once the experts of a batch hold more than 16 assignments on average, the staged-once launch gives a wave
+    two 16-token groups (one pass over an expert's weights serves 32 assignments; one workgroup per compute unit):
+    the same bits as one group per wave with a second token column, and as gate and up in two launches."""
+    gate, up, down = _experts(E, hidden, ff, 1270 + E)
+    wg = Weight.upload(B.CML_Q4_K, E * ff, hidden, gate)
+    wu = Weight.upload(B.CML_Q4_K, E * ff, hidden, up)
+    wd = Weight.upload(B.CML_Q4_K, E * hidden, ff, down)
+    rng = np.random.default_rng(1271 + T)
+    x = rng.standard_normal((T, hidden)).astype(np.float32)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    logits[:, 0] += 1.5     # a crowded expert (more than 32 assignments at the larger T), an idle one
+    logits[:, 1] -= 50.0
+    idx_dev, w_dev, _, _ = gpu_route(logits, k)
+    G.say(f"moe two token groups per wave, E={E} k={k} {hidden}x{ff} T={T}")
+    with G.engaged(r"^q4k\.mfma\.(tile|serial_split)\.g2t1\.grouped\.once"):
+        two_groups = gpu_moe(wg, wu, wd, E, k, idx_dev, w_dev, x)
+    assert np.isfinite(two_groups).all()
+    with G.env(CAMELID_HIP_TUNING=1, CAMELID_HIP_Q4K_MFMA_ONCE_TWO_GROUPS=0), \
+            G.engaged(r"^q4k\.mfma\.(tile|serial_split)\.g1t1\.grouped\.once", none=(r"\.g2t1",)):
+        one_group = gpu_moe(wg, wu, wd, E, k, idx_dev, w_dev, x)
+    assert G.same_bits(two_groups, one_group)
+    with G.env(CAMELID_HIP_TUNING=1, CAMELID_HIP_Q4K_MFMA_UNITS=3, CAMELID_HIP_Q4K_MFMA_FIXED_ROWS=0):
+        general = gpu_moe(wg, wu, wd, E, k, idx_dev, w_dev, x)
+    assert G.same_bits(two_groups, general)
+    with G.env(CAMELID_HIP_MOE_PAIR_LAUNCH=0):
+        two_launches = gpu_moe(wg, wu, wd, E, k, idx_dev, w_dev, x)
+    assert G.same_bits(two_groups, two_launches)
 
 
 @pytest.mark.parametrize("T", [1, 32])

@@ -1139,14 +1139,15 @@ def test_q4k_two_waves_per_tile_keep_one_chain(rows, cols):
         assert G.same_bits(walk_any, want)
 
 
-@pytest.mark.parametrize("rows,cols,tokens", [(16400, 2048, (9, 16)), (20000, 14 * 256, (5, 16)), (49168, 4096, (3, 4, 7))])
+@pytest.mark.parametrize("rows,cols,tokens", [(16400, 2048, (9, 16, 17, 32)), (20000, 14 * 256, (5, 16, 25)), (49168, 4096, (3, 4, 7, 31))])
 def test_q4k_tall_weights_take_the_resident_walk(rows, cols, tokens):
     """Up to 16 tokens against a Q4_K weight of more than 16384 rows (no K cut): one wave per row tile, the
     activation staged once per workgroup, the launch sized to about one resident workgroup per compute unit that
     walks its share of the weight -- from f32 rows (cml_matmul_f32: the quantizing launch, then this one) the
     oracle's chain bit for bit, and the bits of the two-waves-per-tile kernel that serves shorter weights.  Four
     tokens on a vocabulary-sized weight come here too (three on a weight of this size stay on the packed-dot
-    launch); the last group of row tiles lies partly past the end of the weight."""
+    launch), and 17 to 32 tokens as two token groups per wave; the last group of row tiles lies partly past the
+    end of the weight."""
     fmt = B.CML_Q4_K
     rng = np.random.default_rng(rows + cols)
     wire = G.synth_weight(fmt, rows, cols, seed=rows * 3 + cols)
@@ -1156,12 +1157,14 @@ def test_q4k_tall_weights_take_the_resident_walk(rows, cols, tokens):
         s, q = oracle.quantize_activation(fmt, x)
         want = oracle.matmul_q(fmt, wire, cols, s, q, order=oracle.ORDER_PRIMARY, threads=8)
         G.say(f"Q4_K tall weight {rows}x{cols} n={n}")
-        walk = r"^q4k\.dot\.wg8\.fused\.tokens$" if n == 3 else r"^q4k\.mfma\.tile\.g1t1\.once"
+        walk = r"^q4k\.dot\.wg8\.fused\.tokens$" if n == 3 else (r"^q4k\.mfma\.tile\.g1t1\.once" if n <= 16 else r"^q4k\.mfma\.tile\.g2t1\.once")
         with G.env(CAMELID_HIP_EXACT_ORDER="1"):
             with G.engaged(walk, none=(r"^q4k\.mfma\.pair",)):
                 got = G.gpu_matmul_f32(w, x)
-            with G.env(CAMELID_HIP_EXACT_ORDER="1", CAMELID_HIP_Q4K_MFMA_PAIR_MAX_ROWS=1 << 30, CAMELID_HIP_Q4K_TALL_TOKENS_MFMA=0), \
-                    G.engaged(r"^q4k\.mfma\.pair" if n > 4 else r"^q4k\.(dot\.wg8\.fused\.tokens|mfma\.pair)"):
+            # the launches that served these calls before: two waves per tile up to 16 tokens, the phased kernel beyond
+            with G.env(CAMELID_HIP_EXACT_ORDER="1", CAMELID_HIP_Q4K_MFMA_PAIR_MAX_ROWS=1 << 30, CAMELID_HIP_Q4K_TALL_TOKENS_MFMA=0,
+                       CAMELID_HIP_Q4K_MFMA_ONCE_TWO_GROUPS=0), \
+                    G.engaged(r"^q4k\.mfma\.tile\.g2t1$" if n > 16 else (r"^q4k\.mfma\.pair" if n > 4 else r"^q4k\.(dot\.wg8\.fused\.tokens|mfma\.pair)")):
                 former = G.gpu_matmul_f32(w, x)
         assert G.same_bits(got, want)
         assert G.same_bits(got, former)
