@@ -898,9 +898,11 @@ int cml_matmul_f32(const cml_weight *w, const float *x_dev, int64_t n_tokens, fl
         if (frc != -1) return frc;
     }
     if (w->fmt == CML_Q6_K && (n_tokens == 1 || fuse_two) && env_int("CAMELID_HIP_Q6K_FUSED_QUANT", 1) && !q6k_lane_order() &&
-        (fuse == 2 || (fuse == 1 && ((w->nb <= 32 && w->rows <= 32768) || (n_tokens == 1 && gemv_q6k_long_rows_fuse(w)))))) {
-        // the same for Q6_K: 4096 x 4096 7.0 -> 5.5 us, 14336 x 4096 12.3 -> 10.8; not on a vocabulary
-        // head, whose 4008 workgroups would each quantize the row (128256 x 3072: 49.2 -> 49.6, two tokens 53.3 -> 57.2)
+        (fuse == 2 || (fuse == 1 && ((w->nb <= 32 && w->rows <= (n_tokens == 1 ? 98304 : 32768)) || (n_tokens == 1 && gemv_q6k_long_rows_fuse(w)))))) {
+        // the same for Q6_K: 4096 x 4096 7.0 -> 5.5 us, 14336 x 4096 12.3 -> 10.8, 65536 x 4096 36.1 -> 34.5; not on
+        // the largest vocabulary heads, whose 4008 workgroups would each quantize the row (128256 x 3072: 49.5 either
+        // way, 128256 x 4096 67.5 / 67.3; two tokens 53.3 -> 57.2).  A launch of about the resident workgroups, each
+        // quantizing once and walking every n-th group of row tiles, measured slower there (50.7 - 53.7 us for 512 - 2048).
         const int frc = launch_gemv_q6k_f32(w, x_dev, out_dev, st, static_cast<int>(n_tokens));
         if (frc == CML_OK) g_runs.fetch_add(1, std::memory_order_relaxed);
         return frc;

@@ -174,7 +174,8 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
     // takes 8 to cover the HBM latency; steps over more tokens are longer and 4 are enough
     // (staged-once mode with the whole row of 16 requested in the prologue: the 32-token expert layer 174 -> 179 us)
     // (staged-once mode with two token groups per wave: one workgroup per compute unit, one wave per SIMD -- eight slots fit)
-    constexpr int RING = ((GPW == 1 && KS == 1) || ONCE) ? 8 : 4;
+    // (rows of 12 / 14 super-blocks known at compile time: six / seven slots, so that a row is two rounds of the ring)
+    constexpr int RING = NSB == 12 ? 6 : NSB == 14 ? 7 : ((GPW == 1 && KS == 1) || ONCE) ? 8 : 4;
     static_assert((ONCE || RING % KC == 0) && kPer >= 1 && RT >= 1, "phase / staging shape");
     // staged-once mode holds a row of up to 16 super-blocks as kOnceChunks chunks of KC slabs, each laid out like a phase buffer
     constexpr int kOnceChunks = 16 / KC;
@@ -1024,14 +1025,16 @@ static int launch_mfma_split(const Q4KMfmaArgs &ka, int n_groups, hipStream_t st
         // Rows of up to 16 super-blocks: the whole activation fits the LDS and is staged once.  One token group per
         // wave: always.  Two (17 to 32 tokens; 155 KB, one workgroup per compute unit): expert groups, and plain calls
         // on weights of more than 16384 rows, where the launch walks the weight with resident workgroups.
-        const bool two_groups_pay = ka.group_offsets != nullptr || n_tiles > 1024;
+        const bool two_groups_pay = ka.group_offsets != nullptr || n_tiles > env_int("CAMELID_HIP_Q4K_MFMA_ONCE_TWO_GROUPS_MIN_TILES", 1024);
         if (ka.n_sb <= 16 && ka.stage_once && (GPW == 1 || (two_groups_pay && env_int("CAMELID_HIP_Q4K_MFMA_ONCE_TWO_GROUPS", 1)))) {
             const size_t lds_once = static_cast<size_t>(16) * NTOK * (kSlabRow + 32) + static_cast<size_t>(ka.n_sb) * NTOK * 4;  // slabs + run sums, scales
             const int pair_f = ka.w2 ? 2 : 1, slots = n_groups / pair_f;
             const int64_t columns = ka.group_offsets ? 1 : gy;  // (a grouped call counts one token column per group: the others leave at once)
-            // rows of 2048 or 4096 values: the walk of a unit as straight-line code
+            // rows of 2048, 3072, 3584 or 4096 values: the walk of a unit as straight-line code
             const bool fixed = env_int("CAMELID_HIP_Q4K_MFMA_FIXED_ROWS", 1);
             if (fixed && ka.n_sb == 16) return launch_mfma_once<SPLIT, PLAIN, 16, GPW>(ka, n_tiles, pair_f, slots, gy, columns, lds_once, st);
+            if (fixed && ka.n_sb == 14) return launch_mfma_once<SPLIT, PLAIN, 14, GPW>(ka, n_tiles, pair_f, slots, gy, columns, lds_once, st);
+            if (fixed && ka.n_sb == 12) return launch_mfma_once<SPLIT, PLAIN, 12, GPW>(ka, n_tiles, pair_f, slots, gy, columns, lds_once, st);
             if (fixed && ka.n_sb == 8) return launch_mfma_once<SPLIT, PLAIN, 8, GPW>(ka, n_tiles, pair_f, slots, gy, columns, lds_once, st);
             return launch_mfma_once<SPLIT, PLAIN, 0, GPW>(ka, n_tiles, pair_f, slots, gy, columns, lds_once, st);
         }
