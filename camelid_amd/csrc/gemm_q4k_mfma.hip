@@ -175,12 +175,13 @@ __global__ __launch_bounds__(256) void gemm_q4k_mfma_kernel(Q4KMfmaArgs a) {
     // (staged-once mode with the whole row of 16 requested in the prologue: the 32-token expert layer 174 -> 179 us)
     // (staged-once mode with two token groups per wave: one workgroup per compute unit, one wave per SIMD -- eight slots fit)
     // (rows of 12 / 14 super-blocks known at compile time: six / seven slots, so that a row is two rounds of the ring)
-    constexpr int RING = NSB == 12 ? 6 : NSB == 14 ? 7 : ((GPW == 1 && KS == 1) || ONCE) ? 8 : 4;
+    constexpr int RING = NSB == 12 ? 6 : NSB == 14 ? 7 : NSB == 20 ? 10 : ((GPW == 1 && KS == 1) || ONCE) ? 8 : 4;
     static_assert((ONCE || RING % KC == 0) && kPer >= 1 && RT >= 1, "phase / staging shape");
     // staged-once mode holds a row of up to 16 super-blocks as kOnceChunks chunks of KC slabs, each laid out like a phase buffer
-    constexpr int kOnceChunks = 16 / KC;
+    // (one token group per wave: also rows of 20 / 24 / 32 super-blocks -- 32 x 16 tokens fill a compute unit's LDS like 16 x 32)
+    constexpr int kOnceChunks = (NSB > 16 ? 32 : 16) / KC;
     // NSB: the row length in super-blocks where the launcher knows it at compile time (staged-once mode; 0 = any)
-    static_assert(NSB == 0 || (ONCE && NSB % RING == 0 && NSB <= 16), "row length known at compile time: whole rounds of the ring");
+    static_assert(NSB == 0 || (ONCE && NSB % RING == 0 && (NSB <= 16 || (NSB <= 32 && GPW == 1))), "row length known at compile time: whole rounds of the ring");
     extern __shared__ uint4 smem[];
     uint8_t *buf0 = reinterpret_cast<uint8_t *>(smem);  // [KC][NTOK][kSlabRow], then [KC][NTOK][16] f16
     uint8_t *buf1 = buf0 + kBufBytes;
@@ -1037,6 +1038,16 @@ static int launch_mfma_split(const Q4KMfmaArgs &ka, int n_groups, hipStream_t st
             if (fixed && ka.n_sb == 12) return launch_mfma_once<SPLIT, PLAIN, 12, GPW>(ka, n_tiles, pair_f, slots, gy, columns, lds_once, st);
             if (fixed && ka.n_sb == 8) return launch_mfma_once<SPLIT, PLAIN, 8, GPW>(ka, n_tiles, pair_f, slots, gy, columns, lds_once, st);
             return launch_mfma_once<SPLIT, PLAIN, 0, GPW>(ka, n_tiles, pair_f, slots, gy, columns, lds_once, st);
+        }
+        // Rows of 5120 / 6144 / 8192 values on a tall plain weight, up to 16 tokens: the same walk with 32 slabs of LDS
+        // (one workgroup per compute unit); 128256 x 8192 at 16 tokens 132.9 -> 110.4 us, 152064 x 5120 108.0 -> 88.2, 32000 x 5120 26.9 -> 23.7.
+        if constexpr (GPW == 1 && PLAIN) {
+            if (ka.stage_once && n_tiles > env_int("CAMELID_HIP_Q4K_MFMA_ONCE_LONG_MIN_TILES", 1024) && (ka.n_sb == 20 || ka.n_sb == 24 || ka.n_sb == 32)) {
+                const size_t lds_long = static_cast<size_t>(32) * NTOK * (kSlabRow + 32) + static_cast<size_t>(ka.n_sb) * NTOK * 4;
+                if (ka.n_sb == 20) return launch_mfma_once<SPLIT, PLAIN, 20, 1>(ka, n_tiles, 1, 1, gy, gy, lds_long, st);
+                if (ka.n_sb == 24) return launch_mfma_once<SPLIT, PLAIN, 24, 1>(ka, n_tiles, 1, 1, gy, gy, lds_long, st);
+                return launch_mfma_once<SPLIT, PLAIN, 32, 1>(ka, n_tiles, 1, 1, gy, gy, lds_long, st);
+            }
         }
     }
     static std::atomic<bool> raised{false};  // per instantiation: allow more than 64 KB of dynamic LDS once

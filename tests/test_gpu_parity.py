@@ -1170,6 +1170,31 @@ def test_q4k_tall_weights_take_the_resident_walk(rows, cols, tokens):
         assert G.same_bits(got, former)
 
 
+@pytest.mark.parametrize("rows,cols", [(16700, 20 * 256), (3001, 24 * 256), (2000, 32 * 256)])
+def test_q4k_tall_weights_with_long_rows_take_the_resident_walk(rows, cols):
+    """Up to 16 tokens against a tall Q4_K weight whose rows are 5120 / 6144 / 8192 values: the staged-once walk
+    with 32 slabs of LDS (one resident workgroup per compute unit) -- the oracle's chain bit for bit, and the
+    bits of the phased kernel that served these shapes.  (The smaller weights here are sent to it by its knob.)"""
+    fmt = B.CML_Q4_K
+    rng = np.random.default_rng(rows + cols)
+    wire = G.synth_weight(fmt, rows, cols, seed=rows * 5 + cols)
+    w = Weight.upload(fmt, rows, cols, wire)
+    min_tiles = 1024 if rows > 16384 else 1
+    for n in (4, 16):
+        x = rng.standard_normal((n, cols)).astype(np.float32)
+        s, q = oracle.quantize_activation(fmt, x)
+        want = oracle.matmul_q(fmt, wire, cols, s, q, order=oracle.ORDER_PRIMARY, threads=8)
+        G.say(f"Q4_K tall weight, long rows {rows}x{cols} n={n}")
+        with G.env(CAMELID_HIP_EXACT_ORDER="1", CAMELID_HIP_Q4K_MFMA_ONCE_LONG_MIN_TILES=min_tiles, CAMELID_HIP_Q4K_MFMA_MIN_TOKENS=3), \
+                G.engaged(rf"^q4k\.mfma\.tile\.g1t1\.once\.k{cols // 256}"):
+            got = G.gpu_gemm(w, s, q)
+        with G.env(CAMELID_HIP_EXACT_ORDER="1", CAMELID_HIP_Q4K_MFMA_ONCE_LONG_MIN_TILES=1 << 30, CAMELID_HIP_Q4K_MFMA_MIN_TOKENS=3), \
+                G.engaged(r"^q4k\.mfma\.tile\.g1t1$"):
+            former = G.gpu_gemm(w, s, q)
+        assert G.same_bits(got, want)
+        assert G.same_bits(got, former)
+
+
 @pytest.mark.parametrize("name,fmt", [("Q8_0", oracle.Q8_0), ("Q4_0", oracle.Q4_0)])
 @pytest.mark.parametrize("rows,cols", [(130, 1024), (2049, 5 * 256), (77, 12 * 256), (16, 256)])
 def test_b32_matrix_core_cells_are_bitwise_the_gemv(name, fmt, rows, cols):
