@@ -363,6 +363,9 @@ MOE_CONFIGS = {
     "moe_q4k_8x14336x4096_t32": ("mixtral", "Q4_K", 8, 2, 4096, 14336, 32),
     "moe_q4k_8x14336x4096_t64": ("mixtral", "Q4_K", 8, 2, 4096, 14336, 64),   # short prefill: 16 assignments per expert on average
     "moe_q4k_8x14336x4096_t128": ("mixtral", "Q4_K", 8, 2, 4096, 14336, 128),
+    # Mixtral-8x22B-shaped: hidden 6144 (rows of 24 super-blocks), ff 16384
+    "moe_q4k_8x16384x6144_t1": ("mixtral", "Q4_K", 8, 2, 6144, 16384, 1),
+    "moe_q4k_8x16384x6144_t32": ("mixtral", "Q4_K", 8, 2, 6144, 16384, 32),
     # Gemma-4 26B-shaped expert lane in Q4_0: fused gate|up tensor, full-softmax routing with
     # per-expert down scales, gelu_tanh
     "moe_q4_0_128x704x2816_t1": ("gemma4", "Q4_0", 128, 8, 2816, 704, 1),

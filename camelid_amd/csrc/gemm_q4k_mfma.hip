@@ -997,7 +997,7 @@ static int launch_mfma_once(const Q4KMfmaArgs &ka, int n_tiles, int pair_f, int 
         // expert groups: two workgroups per compute unit; a plain call: one (128256 x 4096, 16 tokens, 2004 units:
         // 1 / 2 / 4 / 8 / 16 per workgroup 68.5 / 64.8 / 61.4 / 59.0 / 89.6 us; 65536 x 4096: 35.3 / 33.3 / 31.5 / 47.7 / 85.6)
         // (two token groups per wave fill a compute unit's LDS with one workgroup)
-        const int64_t resident = (ka.group_offsets && GPW == 1) ? 512 : 256;
+        const int64_t resident = (ka.group_offsets && GPW == 1 && NSB <= 16) ? 512 : 256;
         units = static_cast<int>(std::min<int64_t>(16, std::max<int64_t>(1, (units_all * slots * columns + resident - 1) / resident)));
         // the walk that does not know the row length at compile time pays for its bookkeeping beyond two units
         // (151936 x 3584, 16 tokens: 75.2 / 71.9 / 74.2 / 88.7 us for 1 / 2 / 4 / 8)
@@ -1041,12 +1041,16 @@ static int launch_mfma_split(const Q4KMfmaArgs &ka, int n_groups, hipStream_t st
         }
         // Rows of 5120 / 6144 / 8192 values on a tall plain weight, up to 16 tokens: the same walk with 32 slabs of LDS
         // (one workgroup per compute unit); 128256 x 8192 at 16 tokens 132.9 -> 110.4 us, 152064 x 5120 108.0 -> 88.2, 32000 x 5120 26.9 -> 23.7.
-        if constexpr (GPW == 1 && PLAIN) {
-            if (ka.stage_once && n_tiles > env_int("CAMELID_HIP_Q4K_MFMA_ONCE_LONG_MIN_TILES", 1024) && (ka.n_sb == 20 || ka.n_sb == 24 || ka.n_sb == 32)) {
+        // (expert groups with such rows as well: gate and up of a Mixtral-8x22B-shaped layer, hidden 6144)
+        if constexpr (GPW == 1) {
+            const bool tall_or_grouped = ka.group_offsets != nullptr || n_tiles > env_int("CAMELID_HIP_Q4K_MFMA_ONCE_LONG_MIN_TILES", 1024);
+            if (ka.stage_once && tall_or_grouped && (ka.n_sb == 20 || ka.n_sb == 24 || ka.n_sb == 32) && env_int("CAMELID_HIP_Q4K_MFMA_ONCE_LONG_ROWS", 1)) {
                 const size_t lds_long = static_cast<size_t>(32) * NTOK * (kSlabRow + 32) + static_cast<size_t>(ka.n_sb) * NTOK * 4;
-                if (ka.n_sb == 20) return launch_mfma_once<SPLIT, PLAIN, 20, 1>(ka, n_tiles, 1, 1, gy, gy, lds_long, st);
-                if (ka.n_sb == 24) return launch_mfma_once<SPLIT, PLAIN, 24, 1>(ka, n_tiles, 1, 1, gy, gy, lds_long, st);
-                return launch_mfma_once<SPLIT, PLAIN, 32, 1>(ka, n_tiles, 1, 1, gy, gy, lds_long, st);
+                const int pair_f = ka.w2 ? 2 : 1, slots = n_groups / pair_f;
+                const int64_t columns = ka.group_offsets ? 1 : gy;
+                if (ka.n_sb == 20) return launch_mfma_once<SPLIT, PLAIN, 20, 1>(ka, n_tiles, pair_f, slots, gy, columns, lds_long, st);
+                if (ka.n_sb == 24) return launch_mfma_once<SPLIT, PLAIN, 24, 1>(ka, n_tiles, pair_f, slots, gy, columns, lds_long, st);
+                return launch_mfma_once<SPLIT, PLAIN, 32, 1>(ka, n_tiles, pair_f, slots, gy, columns, lds_long, st);
             }
         }
     }

@@ -453,6 +453,32 @@ def test_moe_experts_with_more_than_16_assignments_take_two_token_groups_per_wav
     assert G.same_bits(two_groups, two_launches)
 
 
+@pytest.mark.parametrize("E,k,hidden,ff,T", [(8, 2, 6144, 1024, 24), (8, 2, 5120, 1024, 9), (8, 2, 8192, 1024, 40)])
+def test_moe_experts_with_long_rows_take_the_staged_once_walk(E, k, hidden, ff, T):
+    """Expert groups whose gate / up rows are 5120, 6144 or 8192 values (a Mixtral-8x22B-shaped layer has 6144):
+    the staged-once launch with 32 slabs of LDS, one workgroup per compute unit -- the bits of the phased
+    launch, with one or three groups of row tiles per workgroup."""
+    gate, up, down = _experts(E, hidden, ff, 1370 + E)
+    wg = Weight.upload(B.CML_Q4_K, E * ff, hidden, gate)
+    wu = Weight.upload(B.CML_Q4_K, E * ff, hidden, up)
+    wd = Weight.upload(B.CML_Q4_K, E * hidden, ff, down)
+    rng = np.random.default_rng(1371 + T)
+    x = rng.standard_normal((T, hidden)).astype(np.float32)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    logits[:, 1] -= 50.0    # an expert nobody routes to
+    idx_dev, w_dev, _, _ = gpu_route(logits, k)
+    G.say(f"moe long rows, E={E} k={k} {hidden}x{ff} T={T}")
+    with G.engaged(rf"^q4k\.mfma\.(tile|serial_split)\.g1t1\.grouped\.once\.k{hidden // 256}"):
+        walk = gpu_moe(wg, wu, wd, E, k, idx_dev, w_dev, x)
+    assert np.isfinite(walk).all()
+    with G.env(CAMELID_HIP_TUNING=1, CAMELID_HIP_Q4K_MFMA_ONCE_LONG_ROWS=0), G.engaged(r"^q4k\.mfma\.(tile|serial_split)\.g1t1\.grouped$"):
+        phased = gpu_moe(wg, wu, wd, E, k, idx_dev, w_dev, x)
+    assert G.same_bits(walk, phased)
+    with G.env(CAMELID_HIP_TUNING=1, CAMELID_HIP_Q4K_MFMA_UNITS=3), G.engaged(rf"\.once\.k{hidden // 256}\.units$"):
+        three = gpu_moe(wg, wu, wd, E, k, idx_dev, w_dev, x)
+    assert G.same_bits(walk, three)
+
+
 @pytest.mark.parametrize("T", [1, 32])
 def test_c5_mixtral_shaped_moe(T):
     """8 experts, gate/up 14336x4096 and down 4096x14336 in Q4_K, top-2 routing."""
