@@ -1039,11 +1039,12 @@ static int launch_mfma_split(const Q4KMfmaArgs &ka, int n_groups, hipStream_t st
             if (fixed && ka.n_sb == 8) return launch_mfma_once<SPLIT, PLAIN, 8, GPW>(ka, n_tiles, pair_f, slots, gy, columns, lds_once, st);
             return launch_mfma_once<SPLIT, PLAIN, 0, GPW>(ka, n_tiles, pair_f, slots, gy, columns, lds_once, st);
         }
-        // Rows of 5120 / 6144 / 8192 values on a tall plain weight, up to 16 tokens: the same walk with 32 slabs of LDS
+        // Rows of 5120 / 6144 / 8192 values, up to 16 tokens: the same walk with 32 slabs of LDS
         // (one workgroup per compute unit); 128256 x 8192 at 16 tokens 132.9 -> 110.4 us, 152064 x 5120 108.0 -> 88.2, 32000 x 5120 26.9 -> 23.7.
         // (expert groups with such rows as well: gate and up of a Mixtral-8x22B-shaped layer, hidden 6144)
         if constexpr (GPW == 1) {
-            const bool tall_or_grouped = ka.group_offsets != nullptr || n_tiles > env_int("CAMELID_HIP_Q4K_MFMA_ONCE_LONG_MIN_TILES", 1024);
+            // (plain calls: at any row count the shape policy leaves uncut -- 13824 x 5120 at 16 tokens 17.8 -> 15.8 us, 14336 x 8192 24.8 -> 19.6)
+            const bool tall_or_grouped = ka.group_offsets != nullptr || n_tiles > env_int("CAMELID_HIP_Q4K_MFMA_ONCE_LONG_MIN_TILES", 0);
             if (ka.stage_once && tall_or_grouped && (ka.n_sb == 20 || ka.n_sb == 24 || ka.n_sb == 32) && env_int("CAMELID_HIP_Q4K_MFMA_ONCE_LONG_ROWS", 1)) {
                 const size_t lds_long = static_cast<size_t>(32) * NTOK * (kSlabRow + 32) + static_cast<size_t>(ka.n_sb) * NTOK * 4;
                 const int pair_f = ka.w2 ? 2 : 1, slots = n_groups / pair_f;
