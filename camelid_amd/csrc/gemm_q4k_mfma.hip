@@ -81,10 +81,11 @@ struct Q4KMfmaArgs {
     // kernels' last, partly filled rounds of workgroups become one).
     const uint8_t *w2;
     float *out2;
-    int stage_once;  // rows that fit both activation buffers are staged in the prologue, once
-    // Staged-once mode: a workgroup walks every gridDim.x-th group of row tiles (of both weights of a pair launch,
-    // the second weight's groups following the first's) against the activation it staged, the weight ring running
-    // on across the group boundaries; blockIdx.z is then the group slot alone.
+    // Rows whose whole activation fits the LDS are staged in the prologue, once.  A workgroup of such a launch walks
+    // every gridDim.x-th group of row tiles (of both weights of a pair launch, the second weight's groups following
+    // the first's) against the activation it staged, the weight ring running on across the group boundaries;
+    // blockIdx.z is then the group slot alone.
+    int stage_once;
 };
 
 struct MfmaWeights {
