@@ -44,6 +44,14 @@
 // through LDS at the end -- which is also what fills the chip when there are
 // fewer row tiles than SIMDs -- or, for other split factors, inside the lane (the
 // chain restarts at the split points).
+//
+// Staged-once mode (ONCE): where the whole activation of a workgroup's tokens fits the LDS -- 16 tokens x up to 32
+// super-blocks, or 32 tokens x up to 16 -- it is staged in the prologue and the walk has no barrier.  Such a launch
+// is sized to be resident at once (two workgroups per compute unit for expert groups with 16 tokens per wave, one
+// otherwise) and each workgroup walks every gridDim.x-th group of four row tiles, the register ring refilled across
+// the groups: the staging and the start of the weight stream are paid once per workgroup, and the launch sweeps the
+// weight as one contiguous front.  It serves expert-grouped gate|up launches and plain calls of up to 32 tokens on
+// weights of more than 16384 rows (up to 16 tokens: any uncut weight with rows of 5120 / 6144 / 8192 values).
 #include <type_traits>
 
 #include <atomic>
