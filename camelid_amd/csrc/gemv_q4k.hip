@@ -1788,7 +1788,13 @@ static int launch_q4k_f32(const MatArgs &a, const cml_weight *w2, float *out2, c
     // 4 waves share the quantizing.  Measured with 8-row tiles at 14336 x 4096 (1792 tiles): 2 waves
     // 9.6 us, 4 waves 8.7, 8 waves 9.1; 7 waves -- one workgroup for each of the 256 compute units
     // on paper -- 9.1, and 5 or 6 waves 12.7 / 13.2: workgroups do not land one per unit.
-    if (tpw < 1 || tpw * shape.ksplit > 8) tpw = std::max(1, 4 / shape.ksplit);
+    if (tpw < 1 || tpw * shape.ksplit > 8) {
+        tpw = std::max(1, 4 / shape.ksplit);
+        // The decode launch of an expert layer (routed slots x gate and up in one grid): seven-wave workgroups where
+        // they divide the half tiles -- 14336 rows are 256 of them per matrix, and the 1024 workgroups of the
+        // Mixtral-shaped layer are four per compute unit, all resident (38.9 -> 38.1 us per token).
+        if (ka.shared_act && a.group_ids && half_tiles && shape.ksplit == 1 && tiles % 7 == 0 && env_int("CAMELID_HIP_Q4K_DIRECT_SEVEN_WAVES", 1)) tpw = 7;
+    }
     shape.tiles_per_wg = tpw;
     const int waves = shape.ksplit * shape.tiles_per_wg;
     const unsigned gx = static_cast<unsigned>((tiles + shape.tiles_per_wg - 1) / shape.tiles_per_wg);
