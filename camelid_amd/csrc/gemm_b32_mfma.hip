@@ -285,59 +285,38 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_b32_mfma_kernel(B32MfmaArgs a
         const uint32_t dwords[4] = {w0.d.x, w0.d.y, w0.d.z, w0.d.w};
         long bw8[8];
         b32_mfma_operands<FMT>(w0, bw8);
-        if constexpr (GPW == 1) {
-            // One token group per wave: the slab's eight matrix instructions go out back to back (they do not depend
-            // on one another), then the eight f32 steps run in block order -- the same operations in the same order
-            // per cell, without a wait on the matrix core in front of every step (16 tokens: Q4_0 128256 x 3072
-            // 61.7 -> 60.9 us, 32000 x 4096 39.7 -> 37.8, 14336 x 4096 21.7 -> 20.8; Q8_0 128256 x 3072 97.8 -> 95.0).
-            v4i_b32 d8[8];
-#pragma unroll
-            for (int pr = 0; pr < 4; pr++) {
-                const v4i_b32 av = *reinterpret_cast<const v4i_b32 *>(act + tb * (16 * kB32SlabRow) + a_off + 64 * pr);
-                const long a2[2] = {
-                    static_cast<long>(static_cast<unsigned long long>(static_cast<uint32_t>(av.x)) | (static_cast<unsigned long long>(static_cast<uint32_t>(av.y)) << 32)),
-                    static_cast<long>(static_cast<unsigned long long>(static_cast<uint32_t>(av.z)) | (static_cast<unsigned long long>(static_cast<uint32_t>(av.w)) << 32))};
-#pragma unroll
-                for (int e = 0; e < 2; e++) {
-                    const int b = 2 * pr + e;
-                    v4i_b32 c = {0, 0, 0, 0};
-                    if constexpr (FMT == CML_Q4_0) c = *reinterpret_cast<const v4i_b32 *>(bs + b * NTOK + 16 * tb + cell_tok);
-                    d8[b] = __builtin_amdgcn_mfma_i32_16x16x32_i8(a2[e], bw8[b], c, 0, 0, 0);
-                }
-            }
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int b = 0; b < 8; b++) {
-                const float dwb = f16_bits_to_f32((dwords[b >> 1] >> (16 * (b & 1))) & 0xffffu);
-                const float4 xv = *reinterpret_cast<const float4 *>(xss + (slab * 8 + b) * NTOK + 16 * tb + cell_tok);
-                acc[0][0] = acc[0][0] + (static_cast<float>(d8[b][0]) * dwb) * xv.x;
-                acc[0][1] = acc[0][1] + (static_cast<float>(d8[b][1]) * dwb) * xv.y;
-                acc[0][2] = acc[0][2] + (static_cast<float>(d8[b][2]) * dwb) * xv.z;
-                acc[0][3] = acc[0][3] + (static_cast<float>(d8[b][3]) * dwb) * xv.w;
-            }
-            return;
-        }
-#pragma unroll
-        for (int pr = 0; pr < 4; pr++) {
-            const long bw[2] = {bw8[2 * pr], bw8[2 * pr + 1]};
-            const float dw[2] = {f16_bits_to_f32(dwords[pr] & 0xffffu), f16_bits_to_f32(dwords[pr] >> 16)};
+        {
+            // Per token group: the slab's eight matrix instructions go out back to back (they do not depend on one
+            // another), then the eight f32 steps run in block order -- the same operations in the same order per
+            // cell, without a wait on the matrix core in front of every step (16 tokens: Q4_0 128256 x 3072
+            // 61.7 -> 60.9 us, 32000 x 4096 39.7 -> 37.8, 14336 x 4096 21.7 -> 20.8; Q8_0 128256 x 3072 97.8 -> 95.0;
+            // Q4_0 128256 x 3072 at 32 / 64 tokens 97.9 -> 85.2 / 181.5 -> 158.6).
 #pragma unroll
             for (int g = 0; g < GPW; g++) {
-                const v4i_b32 av = *reinterpret_cast<const v4i_b32 *>(act + (tb * GPW + g) * (16 * kB32SlabRow) + a_off + 64 * pr);
-                const long a2[2] = {
-                    static_cast<long>(static_cast<unsigned long long>(static_cast<uint32_t>(av.x)) | (static_cast<unsigned long long>(static_cast<uint32_t>(av.y)) << 32)),
-                    static_cast<long>(static_cast<unsigned long long>(static_cast<uint32_t>(av.z)) | (static_cast<unsigned long long>(static_cast<uint32_t>(av.w)) << 32))};
+                v4i_b32 d8[8];
 #pragma unroll
-                for (int e = 0; e < 2; e++) {
-                    const int b = 2 * pr + e;
-                    v4i_b32 c = {0, 0, 0, 0};
-                    if constexpr (FMT == CML_Q4_0) c = *reinterpret_cast<const v4i_b32 *>(bs + b * NTOK + 16 * (tb * GPW + g) + cell_tok);
-                    const v4i_b32 d = __builtin_amdgcn_mfma_i32_16x16x32_i8(a2[e], bw[e], c, 0, 0, 0);
+                for (int pr = 0; pr < 4; pr++) {
+                    const v4i_b32 av = *reinterpret_cast<const v4i_b32 *>(act + (tb * GPW + g) * (16 * kB32SlabRow) + a_off + 64 * pr);
+                    const long a2[2] = {
+                        static_cast<long>(static_cast<unsigned long long>(static_cast<uint32_t>(av.x)) | (static_cast<unsigned long long>(static_cast<uint32_t>(av.y)) << 32)),
+                        static_cast<long>(static_cast<unsigned long long>(static_cast<uint32_t>(av.z)) | (static_cast<unsigned long long>(static_cast<uint32_t>(av.w)) << 32))};
+#pragma unroll
+                    for (int e = 0; e < 2; e++) {
+                        const int b = 2 * pr + e;
+                        v4i_b32 c = {0, 0, 0, 0};
+                        if constexpr (FMT == CML_Q4_0) c = *reinterpret_cast<const v4i_b32 *>(bs + b * NTOK + 16 * (tb * GPW + g) + cell_tok);
+                        d8[b] = __builtin_amdgcn_mfma_i32_16x16x32_i8(a2[e], bw8[b], c, 0, 0, 0);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int b = 0; b < 8; b++) {
+                    const float dwb = f16_bits_to_f32((dwords[b >> 1] >> (16 * (b & 1))) & 0xffffu);
                     const float4 xv = *reinterpret_cast<const float4 *>(xss + (slab * 8 + b) * NTOK + 16 * (tb * GPW + g) + cell_tok);
-                    acc[g][0] = acc[g][0] + (static_cast<float>(d[0]) * dw[e]) * xv.x;
-                    acc[g][1] = acc[g][1] + (static_cast<float>(d[1]) * dw[e]) * xv.y;
-                    acc[g][2] = acc[g][2] + (static_cast<float>(d[2]) * dw[e]) * xv.z;
-                    acc[g][3] = acc[g][3] + (static_cast<float>(d[3]) * dw[e]) * xv.w;
+                    acc[g][0] = acc[g][0] + (static_cast<float>(d8[b][0]) * dwb) * xv.x;
+                    acc[g][1] = acc[g][1] + (static_cast<float>(d8[b][1]) * dwb) * xv.y;
+                    acc[g][2] = acc[g][2] + (static_cast<float>(d8[b][2]) * dwb) * xv.z;
+                    acc[g][3] = acc[g][3] + (static_cast<float>(d8[b][3]) * dwb) * xv.w;
                 }
             }
         }
